@@ -1,0 +1,465 @@
+"""ctypes view of oracle/libtsoracle.so (the CPU restatement of the reference path).
+
+Test infrastructure only: imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py as the checker.  The product package never imports it.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_DIR, "libtsoracle.so")
+
+F32, F16, Q8_0, Q4_K, BF16, MXFP4 = 0, 1, 8, 12, 30, 39
+
+
+def build():
+    subprocess.check_call(["make", "-C", _DIR, "-s", "-B"])
+
+
+class Shaping(C.Structure):
+    _fields_ = [
+        ("temperature", C.c_double),
+        ("top_k", C.c_uint32),
+        ("has_top_p", C.c_int32),
+        ("top_p", C.c_double),
+        ("repetition_penalty", C.c_double),
+        ("has_seed", C.c_int32),
+        ("seed", C.c_uint64),
+        ("presence_penalty", C.c_double),
+        ("frequency_penalty", C.c_double),
+        ("has_min_p", C.c_int32),
+        ("min_p", C.c_double),
+    ]
+
+
+def shaping(temperature=0.0, top_k=0, top_p=None, repetition_penalty=1.0, seed=None,
+            presence_penalty=0.0, frequency_penalty=0.0, min_p=None):
+    s = Shaping()
+    s.temperature = temperature
+    s.top_k = top_k
+    s.has_top_p = top_p is not None
+    s.top_p = top_p or 0.0
+    s.repetition_penalty = repetition_penalty
+    s.has_seed = seed is not None
+    s.seed = seed or 0
+    s.presence_penalty = presence_penalty
+    s.frequency_penalty = frequency_penalty
+    s.has_min_p = min_p is not None
+    s.min_p = min_p or 0.0
+    return s
+
+
+class RoundResult(C.Structure):
+    _fields_ = [
+        ("accepted", C.c_int32),
+        ("committed", C.c_int32),
+        ("next", C.c_int32),
+        ("stopped", C.c_int32),
+        ("draw_step", C.c_uint64),
+        ("path", C.c_int32 * 17),
+        ("path_len", C.c_int32),
+    ]
+
+    def as_dict(self):
+        return dict(accepted=self.accepted, committed=self.committed, next=self.next,
+                    stopped=self.stopped, draw_step=self.draw_step,
+                    path=list(self.path[: self.path_len]))
+
+
+class Tensor(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int32), ("rows", C.c_int64), ("cols", C.c_int64)]
+
+
+class Layer(C.Structure):
+    _fields_ = [(n, Tensor) for n in
+                ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up",
+                 "w_down")]
+
+
+class ModelDesc(C.Structure):
+    _fields_ = [
+        ("n_layers", C.c_int32), ("hidden", C.c_int32), ("n_q_heads", C.c_int32),
+        ("n_kv_heads", C.c_int32), ("head_dim", C.c_int32), ("ffn", C.c_int32),
+        ("vocab", C.c_int32), ("max_context", C.c_int32),
+        ("rms_eps", C.c_float), ("rope_theta", C.c_float), ("attn_scale", C.c_float),
+        ("rope_factors", C.POINTER(C.c_float)),
+        ("round_kv_f16", C.c_int32), ("threads", C.c_int32),
+        ("embed", Tensor), ("final_norm", Tensor), ("lm_head", Tensor),
+        ("layers", C.POINTER(Layer)),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        L.tso_f32_to_f16.argtypes = [C.c_float]
+        L.tso_f32_to_f16.restype = C.c_uint16
+        L.tso_f16_to_f32.argtypes = [C.c_uint16]
+        L.tso_f16_to_f32.restype = C.c_float
+        L.tso_f32_to_bf16.argtypes = [C.c_float]
+        L.tso_f32_to_bf16.restype = C.c_uint16
+        L.tso_bf16_to_f32.argtypes = [C.c_uint16]
+        L.tso_bf16_to_f32.restype = C.c_float
+        L.tso_row_bytes.argtypes = [C.c_int, C.c_int64]
+        L.tso_row_bytes.restype = C.c_int64
+        L.tso_mxfp4_scale.argtypes = [C.c_uint8]
+        L.tso_mxfp4_scale.restype = C.c_float
+        L.tso_silu.argtypes = [C.c_float]
+        L.tso_silu.restype = C.c_float
+        L.tso_mix.argtypes = [C.c_uint64]
+        L.tso_mix.restype = C.c_uint64
+        L.tso_derive_step_value.argtypes = [C.c_uint64, C.c_uint64]
+        L.tso_derive_step_value.restype = C.c_uint64
+        L.tso_to_unit_interval.argtypes = [C.c_uint64]
+        L.tso_to_unit_interval.restype = C.c_double
+        L.tso_dist_probability.restype = C.c_double
+        L.tso_dist_draw.restype = C.c_uint32
+        L.tso_model_create.restype = C.c_void_p
+        L.tso_model_position.restype = C.c_int64
+        L.tso_model_k.restype = C.POINTER(C.c_float)
+        L.tso_model_v.restype = C.POINTER(C.c_float)
+        L.tso_last_error.restype = C.c_char_p
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def last_error():
+    return lib().tso_last_error().decode()
+
+
+# ---------------------------------------------------------------- conversions
+def f32_to_f16_bits(x):
+    x = np.asarray(x, np.float32)
+    f = np.vectorize(lambda v: lib().tso_f32_to_f16(float(v)), otypes=[np.uint16])
+    return f(x)
+
+
+def row_bytes(dtype, n):
+    return lib().tso_row_bytes(dtype, n)
+
+
+def quantize(dtype, w):
+    """w: [rows, cols] fp32 -> uint8 [rows, row_bytes]."""
+    w = np.ascontiguousarray(w, np.float32)
+    rows, cols = w.shape
+    if dtype == F32:
+        return w.view(np.uint8).reshape(rows, cols * 4).copy()
+    if dtype == F16:
+        return w.astype(np.float16).view(np.uint8).reshape(rows, cols * 2).copy()
+    if dtype == BF16:
+        out = np.empty((rows, cols), np.uint16)
+        flat = w.reshape(-1)
+        o = out.reshape(-1)
+        for i in range(flat.size):
+            o[i] = lib().tso_f32_to_bf16(float(flat[i]))
+        return out.view(np.uint8).reshape(rows, cols * 2)
+    fn = {Q8_0: lib().tso_quantize_q8_0, Q4_K: lib().tso_quantize_q4_k,
+          MXFP4: lib().tso_quantize_mxfp4}[dtype]
+    rb = row_bytes(dtype, cols)
+    out = np.empty((rows, rb), np.uint8)
+    for r in range(rows):
+        fn(_p(w[r]), C.c_int64(cols), C.c_void_p(out[r].ctypes.data))
+    return out
+
+
+def dequantize(dtype, b, cols):
+    b = np.ascontiguousarray(b, np.uint8)
+    if b.ndim == 1:
+        b = b.reshape(1, -1)
+    rows = b.shape[0]
+    out = np.empty((rows, cols), np.float32)
+    for r in range(rows):
+        lib().tso_dequantize_row(C.c_int(dtype), C.c_void_p(b[r].ctypes.data), C.c_int64(cols),
+                                 C.c_void_p(out[r].ctypes.data))
+    return out
+
+
+def gemv(dtype, wbytes, rows, cols, x):
+    wbytes = np.ascontiguousarray(wbytes, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty(rows, np.float32)
+    lib().tso_gemv(C.c_int(dtype), _p(wbytes), C.c_int64(rows), C.c_int64(cols), _p(x), _p(y))
+    return y
+
+
+# ---------------------------------------------------------------------- ops
+def rms_norm(x, w, eps):
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    y = np.empty_like(x)
+    lib().tso_rms_norm(_p(x), _p(w), C.c_int64(x.size), C.c_float(eps), _p(y))
+    return y
+
+
+def rope_neox(x, num_tokens, num_heads, head_dim, rotated_pairs, position, theta):
+    x = np.array(x, np.float32, copy=True)
+    lib().tso_rope_neox(_p(x), num_tokens, num_heads, head_dim, rotated_pairs, C.c_int64(position),
+                        C.c_float(theta))
+    return x
+
+
+def rope_neox_freqs(x, num_tokens, num_heads, head_dim, rotated_pairs, position, freqs):
+    x = np.array(x, np.float32, copy=True)
+    freqs = np.ascontiguousarray(freqs, np.float32)
+    lib().tso_rope_neox_freqs(_p(x), num_tokens, num_heads, head_dim, rotated_pairs,
+                              C.c_int64(position), _p(freqs))
+    return x
+
+
+def llama3_rope_factors(rotary_dim, base, factor, low, high, original_context):
+    out = np.empty(max(rotary_dim // 2, 1), np.float32)
+    rc = lib().tso_llama3_rope_factors(rotary_dim, C.c_double(base), C.c_double(factor),
+                                       C.c_double(low), C.c_double(high),
+                                       C.c_double(original_context), _p(out))
+    return None if rc < 0 else out
+
+
+def rope_frequencies_with_factors(rotary_dim, base, factors):
+    factors = np.ascontiguousarray(factors, np.float32)
+    out = np.empty(rotary_dim // 2, np.float32)
+    lib().tso_rope_frequencies_with_factors(rotary_dim, C.c_float(base), _p(factors), _p(out))
+    return out
+
+
+def causal_attention(q, k, v, head_dim, nq, nkv, seq_len, window=0, scale=0.0, sinks=None):
+    q = np.ascontiguousarray(q, np.float32)
+    k = np.ascontiguousarray(k, np.float32)
+    v = np.ascontiguousarray(v, np.float32)
+    out = np.empty(nq * head_dim, np.float32)
+    sp = _p(np.ascontiguousarray(sinks, np.float32)) if sinks is not None else None
+    lib().tso_causal_attention(_p(q), _p(k), _p(v), head_dim, nq, nkv, C.c_int64(seq_len),
+                               C.c_int64(window), C.c_float(scale), sp, _p(out))
+    return out
+
+
+# ----------------------------------------------------------------- selection
+def _hist(history):
+    h = np.ascontiguousarray(history if history is not None else [], np.int32)
+    return h, _p(h), C.c_int64(h.size)
+
+
+def _logits_bits(logits):
+    a = np.asarray(logits)
+    if a.dtype == np.uint16:
+        return np.ascontiguousarray(a)
+    return np.ascontiguousarray(a.astype(np.float16)).view(np.uint16)
+
+
+def select(logits, cfg, history=None, position=0):
+    lb = _logits_bits(logits)
+    h, hp, hn = _hist(history)
+    out = C.c_int32()
+    rc = lib().tso_select(_p(lb), C.c_int64(lb.size), C.byref(cfg), hp, hn, C.c_uint64(position),
+                          C.byref(out))
+    if rc < 0:
+        raise ValueError(last_error())
+    return out.value
+
+
+def shaped_distribution(logits, cfg, history=None, position=0):
+    lb = _logits_bits(logits)
+    h, hp, hn = _hist(history)
+    sup = np.empty(lb.size, np.uint32)
+    pr = np.empty(lb.size, np.float64)
+    n = C.c_int64()
+    rc = lib().tso_shaped_distribution(_p(lb), C.c_int64(lb.size), C.byref(cfg), hp, hn,
+                                       C.c_uint64(position), _p(sup), _p(pr), C.byref(n))
+    if rc < 0:
+        raise ValueError(last_error())
+    return sup[: n.value].copy(), pr[: n.value].copy()
+
+
+def dist_probability(support, probs, token):
+    s = np.ascontiguousarray(support, np.uint32)
+    p = np.ascontiguousarray(probs, np.float64)
+    return lib().tso_dist_probability(_p(s), _p(p), C.c_int64(s.size), C.c_uint32(token))
+
+
+def dist_draw(support, probs, seed, position):
+    s = np.ascontiguousarray(support, np.uint32)
+    p = np.ascontiguousarray(probs, np.float64)
+    return lib().tso_dist_draw(_p(s), _p(p), C.c_int64(s.size), C.c_uint64(seed), C.c_uint64(position))
+
+
+def residual(p, q):
+    ps, pp = np.ascontiguousarray(p[0], np.uint32), np.ascontiguousarray(p[1], np.float64)
+    qs, qp = np.ascontiguousarray(q[0], np.uint32), np.ascontiguousarray(q[1], np.float64)
+    os_ = np.empty(ps.size, np.uint32)
+    op = np.empty(ps.size, np.float64)
+    n = C.c_int64()
+    rc = lib().tso_residual(_p(ps), _p(pp), C.c_int64(ps.size), _p(qs), _p(qp), C.c_int64(qs.size),
+                            _p(os_), _p(op), C.byref(n))
+    if rc == 0:
+        return None
+    return os_[: n.value].copy(), op[: n.value].copy()
+
+
+def draft_chain(draft_logits, cfg, history=None, generated=0, draw_step=0):
+    lb = _logits_bits(draft_logits)
+    k, vocab = lb.shape
+    h, hp, hn = _hist(history)
+    ds = C.c_uint64(draw_step)
+    props = np.empty(k, np.int32)
+    rc = lib().tso_draft_chain(_p(lb), k, C.c_int64(vocab), C.byref(cfg), hp, hn,
+                               C.c_uint64(generated), C.byref(ds), _p(props))
+    if rc < 0:
+        raise ValueError(last_error())
+    return props, ds.value
+
+
+def chain_round(target_logits, draft_logits, proposals, cfg, history=None, generated=0,
+                max_new_tokens=1 << 40, stop_tokens=None, draw_step=0):
+    tb = _logits_bits(target_logits)
+    k = len(proposals)
+    vocab = tb.shape[1]
+    db = _logits_bits(draft_logits) if draft_logits is not None else None
+    h, hp, hn = _hist(history)
+    pr = np.ascontiguousarray(proposals, np.int32)
+    st = np.ascontiguousarray(stop_tokens if stop_tokens is not None else [], np.int32)
+    out = RoundResult()
+    rc = lib().tso_chain_round(_p(tb), _p(db) if db is not None else None, _p(pr), k,
+                               C.c_int64(vocab), C.byref(cfg), hp, hn, C.c_uint64(generated),
+                               C.c_uint64(max_new_tokens), _p(st), int(st.size),
+                               C.c_uint64(draw_step), C.byref(out))
+    if rc < 0:
+        raise ValueError(last_error())
+    return out.as_dict()
+
+
+def tree_round_greedy(target_logits, feed, parent, cfg, history=None, generated=0,
+                      max_new_tokens=1 << 40, stop_tokens=None):
+    tb = _logits_bits(target_logits)
+    m, vocab = tb.shape
+    h, hp, hn = _hist(history)
+    fd = np.ascontiguousarray(feed, np.int32)
+    pa = np.ascontiguousarray(parent, np.int32)
+    st = np.ascontiguousarray(stop_tokens if stop_tokens is not None else [], np.int32)
+    out = RoundResult()
+    rc = lib().tso_tree_round_greedy(_p(tb), _p(fd), _p(pa), m, C.c_int64(vocab), C.byref(cfg), hp,
+                                     hn, C.c_uint64(generated), C.c_uint64(max_new_tokens), _p(st),
+                                     int(st.size), C.byref(out))
+    if rc < 0:
+        raise ValueError(last_error())
+    return out.as_dict()
+
+
+def tree_round_sampled(target_logits, draft_logits, feed, parent, cfg, history=None, generated=0,
+                       draw_step=0):
+    tb = _logits_bits(target_logits)
+    db = _logits_bits(draft_logits)
+    m, vocab = tb.shape
+    h, hp, hn = _hist(history)
+    fd = np.ascontiguousarray(feed, np.int32)
+    pa = np.ascontiguousarray(parent, np.int32)
+    out = RoundResult()
+    rc = lib().tso_tree_round_sampled(_p(tb), _p(db), _p(fd), _p(pa), m, C.c_int64(vocab),
+                                      C.byref(cfg), hp, hn, C.c_uint64(generated),
+                                      C.c_uint64(draw_step), C.byref(out))
+    if rc < 0:
+        raise ValueError(last_error())
+    return out.as_dict()
+
+
+# --------------------------------------------------------------------- model
+def _tensor(entry):
+    """entry: None | (dtype, uint8 array [rows, row_bytes], rows, cols)."""
+    t = Tensor()
+    if entry is None:
+        return t
+    dtype, data, rows, cols = entry
+    t.data = data.ctypes.data
+    t.dtype = dtype
+    t.rows = rows
+    t.cols = cols
+    return t
+
+
+class Model:
+    """Oracle target model over host weight bytes.
+
+    `weights` is the dict produced by turbospark_amd.synth / tests: keys embed, final_norm,
+    lm_head (optional) and layers (list of dicts with attn_norm, wq, wk, wv, wo,
+    [q_norm, k_norm], ffn_norm, w_gate, w_up, w_down); every tensor is
+    (dtype, uint8 ndarray, rows, cols).  The arrays must outlive the model.
+    """
+
+    def __init__(self, cfg, weights, round_kv_f16=True, threads=1):
+        self._keep = weights
+        n = cfg["n_layers"]
+        self._layers = (Layer * n)()
+        for i, lw in enumerate(weights["layers"]):
+            for name, _ in Layer._fields_:
+                setattr(self._layers[i], name, _tensor(lw.get(name)))
+        d = ModelDesc()
+        for key in ("n_layers", "hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab",
+                    "max_context"):
+            setattr(d, key, cfg[key])
+        d.rms_eps = cfg.get("rms_eps", 1e-5)
+        d.rope_theta = cfg.get("rope_theta", 10000.0)
+        d.attn_scale = cfg.get("attn_scale", 0.0)
+        self._factors = None
+        if cfg.get("rope_factors") is not None:
+            self._factors = np.ascontiguousarray(cfg["rope_factors"], np.float32)
+            d.rope_factors = self._factors.ctypes.data_as(C.POINTER(C.c_float))
+        d.round_kv_f16 = int(round_kv_f16)
+        d.threads = threads
+        d.embed = _tensor(weights["embed"])
+        d.final_norm = _tensor(weights["final_norm"])
+        d.lm_head = _tensor(weights.get("lm_head"))
+        d.layers = C.cast(self._layers, C.POINTER(Layer))
+        self.cfg = cfg
+        self._h = C.c_void_p(lib().tso_model_create(C.byref(d)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().tso_model_destroy(self._h)
+            self._h = None
+
+    @property
+    def position(self):
+        return lib().tso_model_position(self._h)
+
+    def reset(self):
+        lib().tso_model_reset(self._h)
+
+    def rewind_to(self, position):
+        lib().tso_model_rewind_to(self._h, C.c_int64(position))
+
+    def verify(self, feed, base, parent=None, want_f32=False, n_layers_run=-1):
+        feed = np.ascontiguousarray(feed, np.int32)
+        m = feed.size
+        vocab = self.cfg["vocab"]
+        f16 = np.empty((m, vocab), np.uint16)
+        f32 = np.empty((m, vocab), np.float32) if want_f32 else None
+        pa = np.ascontiguousarray(parent, np.int32) if parent is not None else None
+        rc = lib().tso_model_verify(self._h, _p(feed), _p(pa) if pa is not None else None, m,
+                                    C.c_int64(base), _p(f16), _p(f32) if want_f32 else None,
+                                    n_layers_run)
+        if rc < 0:
+            raise ValueError(last_error())
+        return (f16, f32) if want_f32 else f16
+
+    def kv(self, layer):
+        c = self.cfg
+        n = c["max_context"] * c["n_kv_heads"] * c["head_dim"]
+        shape = (c["max_context"], c["n_kv_heads"], c["head_dim"])
+        k = np.ctypeslib.as_array(lib().tso_model_k(self._h, layer), shape=(n,)).reshape(shape)
+        v = np.ctypeslib.as_array(lib().tso_model_v(self._h, layer), shape=(n,)).reshape(shape)
+        return k, v
+
+    def compact_tree(self, base, path):
+        p = np.ascontiguousarray(path, np.uint32)
+        lib().tso_model_compact_tree(self._h, C.c_int64(base), _p(p), int(p.size))

@@ -1,0 +1,248 @@
+// Llama-style target forward of the CPU oracle (test infrastructure only).
+//
+// The reference has no verify pass for this family (real_forward_traits.rs:323-328); it is
+// composed here from the per-token decode graph (families/llama/mod.rs:197-316,
+// attn.rs:152-369, dense.rs:45-120) under the batched-verify contract of
+// families/qwen/batched.rs:92-456: M rows at positions base..base+M, K/V of row m stored at
+// cache position base+m before any row attends, row m sees [0, base+m] (chain) or the
+// committed prefix plus its root path (tree, batched_layers.rs:216-228,373-408).
+// All arithmetic is the fp32 of crates/compute; the only fp16 roundings are the K/V cache
+// store (optional) and the logits store, the two dtype boundaries the engine fixes.
+#include "tsoracle.h"
+
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+void tso_set_error(const std::string& s);
+
+struct tso_model {
+    tso_model_desc d;
+    std::vector<tso_layer> layers;
+    std::vector<float> rope_freqs;  // non-empty when rope_factors given
+    std::vector<std::vector<float>> k, v;  // per layer [max_context][nkv*hd]
+    int64_t position = 0;
+};
+
+namespace {
+
+// Y[m][r] = sum_k dequant(W[r])[k] * X[m][k]; each (m, r) is the sequential fp32 sum of
+// dequant_*_gemv (q4_k.rs:207-220).  The row is dequantized once and reused for all m,
+// which changes no bit of any result.
+void gemm_rows(const tso_tensor& w, const float* x, int m_rows, float* y, int threads) {
+    int64_t rows = w.rows, cols = w.cols;
+    int64_t rb = tso_row_bytes(w.dtype, cols);
+    const uint8_t* base = (const uint8_t*)w.data;
+#pragma omp parallel num_threads(threads)
+    {
+        std::vector<float> deq((size_t)cols);
+#pragma omp for schedule(static)
+        for (int64_t r = 0; r < rows; r++) {
+            tso_dequantize_row(w.dtype, base + r * rb, cols, deq.data());
+            for (int m = 0; m < m_rows; m++) {
+                const float* xv = x + (int64_t)m * cols;
+                float acc = 0.0f;
+                for (int64_t kk = 0; kk < cols; kk++) acc += deq[kk] * xv[kk];
+                y[(int64_t)m * rows + r] = acc;
+            }
+        }
+    }
+}
+
+std::vector<float> norm_weight(const tso_tensor& t) {
+    std::vector<float> w((size_t)t.cols);
+    tso_dequantize_row(t.dtype, (const uint8_t*)t.data, t.cols, w.data());
+    return w;
+}
+
+inline float round_f16(float x) { return tso_f16_to_f32(tso_f32_to_f16(x)); }
+
+}  // namespace
+
+extern "C" tso_model* tso_model_create(const tso_model_desc* desc) {
+    tso_model* m = new tso_model();
+    m->d = *desc;
+    m->layers.assign(desc->layers, desc->layers + desc->n_layers);
+    m->d.layers = m->layers.data();
+    if (m->d.threads < 1) m->d.threads = 1;
+    int64_t stride = (int64_t)desc->n_kv_heads * desc->head_dim;
+    m->k.resize(desc->n_layers);
+    m->v.resize(desc->n_layers);
+    for (int l = 0; l < desc->n_layers; l++) {
+        m->k[l].assign((size_t)(desc->max_context * stride), 0.0f);
+        m->v[l].assign((size_t)(desc->max_context * stride), 0.0f);
+    }
+    if (desc->rope_factors) {
+        m->rope_freqs.resize(desc->head_dim / 2);
+        tso_rope_frequencies_with_factors(desc->head_dim, desc->rope_theta, desc->rope_factors,
+                                          m->rope_freqs.data());
+        m->d.rope_factors = nullptr;
+    }
+    return m;
+}
+
+extern "C" void tso_model_destroy(tso_model* m) { delete m; }
+extern "C" void tso_model_reset(tso_model* m) { m->position = 0; }
+extern "C" int64_t tso_model_position(const tso_model* m) { return m->position; }
+// kv_cache_rewind.rs:46-55: a cursor move; rows are addressed by absolute position and
+// nothing is erased.
+extern "C" void tso_model_rewind_to(tso_model* m, int64_t position) { m->position = position; }
+extern "C" float* tso_model_k(tso_model* m, int layer) { return m->k[layer].data(); }
+extern "C" float* tso_model_v(tso_model* m, int layer) { return m->v[layer].data(); }
+
+extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32_t* parent,
+                                int M, int64_t base, uint16_t* logits_f16, float* logits_f32,
+                                int n_layers_run) {
+    const tso_model_desc& d = mdl->d;
+    // batched.rs:106-185 refusals
+    if (M <= 0) {
+        tso_set_error("verify: empty feed");
+        return -1;
+    }
+    if (base != mdl->position) {
+        tso_set_error("verify: start position does not match the KV cursor");
+        return -2;
+    }
+    if (base + M > d.max_context) {
+        tso_set_error("verify: block would write past the KV capacity");
+        return -3;
+    }
+    for (int m = 0; m < M; m++)
+        if (feed[m] < 0 || feed[m] >= d.vocab) {
+            tso_set_error("verify: token id outside the vocabulary");
+            return -4;
+        }
+    std::vector<int> depth(M, 0);
+    if (parent) {
+        if (parent[0] != -1) {
+            tso_set_error("verify_tree: slot 0 must be the anchor (parent -1)");
+            return -5;
+        }
+        for (int s = 1; s < M; s++) {
+            if (parent[s] < 0 || parent[s] >= s) {
+                tso_set_error("verify_tree: parent[s] must be in [0, s)");
+                return -5;
+            }
+            depth[s] = depth[parent[s]] + 1;
+        }
+    } else {
+        for (int m = 0; m < M; m++) depth[m] = m;
+    }
+
+    const int H = d.hidden, nq = d.n_q_heads, nkv = d.n_kv_heads, hd = d.head_dim, F = d.ffn;
+    const int qd = nq * hd, kvd = nkv * hd;
+    const int T = d.threads;
+    std::vector<float> x((size_t)M * H), xn((size_t)M * H);
+    // embed lookup (real_forward_dispatch.rs:154): one dequantized row per token
+    {
+        int64_t rb = tso_row_bytes(d.embed.dtype, H);
+        for (int m = 0; m < M; m++)
+            tso_dequantize_row(d.embed.dtype, (const uint8_t*)d.embed.data + (int64_t)feed[m] * rb, H,
+                               &x[(size_t)m * H]);
+    }
+    std::vector<float> q((size_t)M * qd), kk((size_t)M * kvd), vv((size_t)M * kvd),
+        att((size_t)M * qd), proj((size_t)M * H), gate((size_t)M * F), up((size_t)M * F);
+
+    int L = n_layers_run < 0 ? d.n_layers : std::min(n_layers_run, (int)d.n_layers);
+    for (int l = 0; l < L; l++) {
+        const tso_layer& ly = d.layers[l];
+        std::vector<float> wn = norm_weight(ly.attn_norm);
+        for (int m = 0; m < M; m++)
+            tso_rms_norm(&x[(size_t)m * H], wn.data(), H, d.rms_eps, &xn[(size_t)m * H]);
+        gemm_rows(ly.wq, xn.data(), M, q.data(), T);
+        gemm_rows(ly.wk, xn.data(), M, kk.data(), T);
+        gemm_rows(ly.wv, xn.data(), M, vv.data(), T);
+        if (ly.q_norm.data) {  // per-head q/k RMSNorm (families/llama/state.rs:344-347)
+            std::vector<float> qw = norm_weight(ly.q_norm), kw = norm_weight(ly.k_norm);
+            std::vector<float> tmp(hd);
+            for (int m = 0; m < M; m++) {
+                for (int h = 0; h < nq; h++) {
+                    float* p = &q[(size_t)m * qd + (size_t)h * hd];
+                    tso_rms_norm(p, qw.data(), hd, d.rms_eps, tmp.data());
+                    std::memcpy(p, tmp.data(), sizeof(float) * hd);
+                }
+                for (int h = 0; h < nkv; h++) {
+                    float* p = &kk[(size_t)m * kvd + (size_t)h * hd];
+                    tso_rms_norm(p, kw.data(), hd, d.rms_eps, tmp.data());
+                    std::memcpy(p, tmp.data(), sizeof(float) * hd);
+                }
+            }
+        }
+        float* kc = mdl->k[l].data();
+        float* vc = mdl->v[l].data();
+        for (int m = 0; m < M; m++) {
+            int64_t pos = base + depth[m];
+            if (!mdl->rope_freqs.empty()) {
+                tso_rope_neox_freqs(&q[(size_t)m * qd], 1, nq, hd, hd / 2, pos, mdl->rope_freqs.data());
+                tso_rope_neox_freqs(&kk[(size_t)m * kvd], 1, nkv, hd, hd / 2, pos, mdl->rope_freqs.data());
+            } else {
+                tso_rope_neox(&q[(size_t)m * qd], 1, nq, hd, hd / 2, pos, d.rope_theta);
+                tso_rope_neox(&kk[(size_t)m * kvd], 1, nkv, hd, hd / 2, pos, d.rope_theta);
+            }
+            // K,V land in the cache slot of row m (batched_layers.rs:84-113)
+            float* kd = kc + (base + m) * kvd;
+            float* vd = vc + (base + m) * kvd;
+            for (int i = 0; i < kvd; i++) {
+                kd[i] = d.round_kv_f16 ? round_f16(kk[(size_t)m * kvd + i]) : kk[(size_t)m * kvd + i];
+                vd[i] = d.round_kv_f16 ? round_f16(vv[(size_t)m * kvd + i]) : vv[(size_t)m * kvd + i];
+            }
+        }
+#pragma omp parallel for num_threads(T) schedule(static)
+        for (int m = 0; m < M; m++) {
+            if (!parent) {
+                tso_causal_attention(&q[(size_t)m * qd], kc, vc, hd, nq, nkv, base + m + 1, 0,
+                                     d.attn_scale, nullptr, &att[(size_t)m * qd]);
+            } else {
+                int64_t path[64];
+                int n = 0;
+                for (int s = m; s >= 0; s = parent[s]) path[n++] = base + s;
+                for (int i = 0; i < n / 2; i++) std::swap(path[i], path[n - 1 - i]);
+                tso_attention_core(&q[(size_t)m * qd], kc, vc, hd, nq, nkv, 0, base, path, n,
+                                   d.attn_scale, nullptr, &att[(size_t)m * qd]);
+            }
+        }
+        gemm_rows(ly.wo, att.data(), M, proj.data(), T);
+        for (size_t i = 0; i < (size_t)M * H; i++) x[i] = x[i] + proj[i];
+
+        std::vector<float> wf = norm_weight(ly.ffn_norm);
+        for (int m = 0; m < M; m++)
+            tso_rms_norm(&x[(size_t)m * H], wf.data(), H, d.rms_eps, &xn[(size_t)m * H]);
+        gemm_rows(ly.w_gate, xn.data(), M, gate.data(), T);
+        gemm_rows(ly.w_up, xn.data(), M, up.data(), T);
+        for (size_t i = 0; i < (size_t)M * F; i++) gate[i] = tso_silu(gate[i]) * up[i];
+        gemm_rows(ly.w_down, gate.data(), M, proj.data(), T);
+        for (size_t i = 0; i < (size_t)M * H; i++) x[i] = x[i] + proj[i];
+    }
+
+    // head (verify_layers.rs:270-333): final norm, lm_head, raw logits (mod.rs:421-423)
+    std::vector<float> wfin = norm_weight(d.final_norm);
+    for (int m = 0; m < M; m++)
+        tso_rms_norm(&x[(size_t)m * H], wfin.data(), H, d.rms_eps, &xn[(size_t)m * H]);
+    const tso_tensor& head = d.lm_head.data ? d.lm_head : d.embed;
+    std::vector<float> logits((size_t)M * d.vocab);
+    gemm_rows(head, xn.data(), M, logits.data(), T);
+    if (logits_f32) std::memcpy(logits_f32, logits.data(), logits.size() * sizeof(float));
+    if (logits_f16)
+        for (size_t i = 0; i < logits.size(); i++) logits_f16[i] = tso_f32_to_f16(logits[i]);
+    mdl->position = base + M;
+    return 0;
+}
+
+// families/qwen/dflash_tree.rs:106-207: gather the accepted path's rows into consecutive
+// slots; safe in place because path[i] >= i.
+extern "C" void tso_model_compact_tree(tso_model* m, int64_t base, const uint32_t* path, int n) {
+    int64_t stride = (int64_t)m->d.n_kv_heads * m->d.head_dim;
+    for (int l = 0; l < m->d.n_layers; l++)
+        for (int i = 0; i < n; i++) {
+            if ((int64_t)path[i] == i) continue;
+            std::memmove(&m->k[l][(base + i) * stride], &m->k[l][(base + path[i]) * stride],
+                         sizeof(float) * stride);
+            std::memmove(&m->v[l][(base + i) * stride], &m->v[l][(base + path[i]) * stride],
+                         sizeof(float) * stride);
+        }
+}

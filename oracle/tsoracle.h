@@ -1,0 +1,213 @@
+/*
+ * tsoracle.h -- CPU restatement of the reference's speculative-verify path.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT THE PRODUCT.  Nothing under turbospark_amd/
+ * may include, link or call it.  It exists so the HIP path has something to be
+ * compared against: plain scalar C++ that follows the reference's own CPU
+ * sources function by function (each function cites the file:line it restates),
+ * compiled with -ffp-contract=off so no multiply-add is fused that the Rust
+ * original keeps separate.
+ *
+ * Pinned parts (what proves each restatement, besides reading it):
+ *   - Q4_K decode / scale unpack ....... the reference's hand-packed superblock literal
+ *   - Q8_0, Q4_K encode ................ round-trip bounds, idempotence, zero blocks
+ *   - MXFP4 decode ..................... ggml-produced bytes -> floats fixture, all 256 scale bytes
+ *   - rope / llama-3 factors ........... the reference's literal factor profile + closed forms
+ *   - attention, rms_norm .............. closed-form small cases and brute-force restatements
+ *   - whole fp32 Llama-style forward ... MLX known-answer logits (three fixtures), 2e-4
+ *   - residual, shaped distribution .... the reference's exact unit cases; brute-force enumeration
+ *   - greedy tree walk ................. the reference's unit case
+ *   - mix / derive_step_value .......... the published splitmix64 output vectors (the reference
+ *                                        only tests invariants; its mixer is that textbook routine)
+ *   - rejection round .................. distributional law (first emitted token ~ target p,
+ *                                        acceptance rate = sum min(p,q)) over thousands of seeds
+ * PARITY UNPINNED (no golden value exists anywhere in the reference):
+ *   - tso_tree_round_sampled: multi-branch rejection sampling on a tree is not
+ *     defined by the reference at all; the definition here is this project's own
+ *     (checked only against the chain round on chain-shaped trees and in law).
+ *   - tso_quantize_mxfp4: the reference has no MXFP4 encoder; checked by brute force
+ *     against "nearest codebook value under the tightest covering exponent".
+ */
+#ifndef TSORACLE_H
+#define TSORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Weight storage types; values are the ggml type ids the reference's GGUF
+ * intake uses, so a tensor description reads the same on both sides. */
+enum {
+    TSO_F32 = 0,
+    TSO_F16 = 1,
+    TSO_Q8_0 = 8,
+    TSO_Q4_K = 12,
+    TSO_BF16 = 30,
+    TSO_MXFP4 = 39,
+};
+
+/* ---- scalar conversions ------------------------------------------------ */
+uint16_t tso_f32_to_f16(float x);   /* IEEE round-to-nearest-even, as the `half` crate */
+float tso_f16_to_f32(uint16_t h);
+uint16_t tso_f32_to_bf16(float x);  /* crates/compute/src/quant.rs:28-39 */
+float tso_bf16_to_f32(uint16_t b);  /* crates/compute/src/quant.rs:14-17 */
+
+/* ---- block formats ----------------------------------------------------- */
+int64_t tso_row_bytes(int dtype, int64_t n);
+void tso_quantize_q8_0(const float* row, int64_t n, uint8_t* out);
+void tso_dequantize_q8_0(const uint8_t* blocks, int64_t n, float* out);
+void tso_quantize_q4_k(const float* row, int64_t n, uint8_t* out);
+void tso_dequantize_q4_k(const uint8_t* blocks, int64_t n, float* out);
+void tso_q4_k_scale_min(int j, const uint8_t* packed12, uint8_t* sc, uint8_t* mn);
+float tso_mxfp4_scale(uint8_t e);
+void tso_dequantize_mxfp4(const uint8_t* blocks, int64_t n, float* out);
+void tso_quantize_mxfp4(const float* row, int64_t n, uint8_t* out); /* ours: reference has no encoder */
+void tso_dequantize_row(int dtype, const uint8_t* row, int64_t n, float* out);
+/* y[r] = sum_k dequant(W[r,:])[k] * x[k], sequential fp32 sum (q4_k.rs:207-220). */
+void tso_gemv(int dtype, const uint8_t* w, int64_t rows, int64_t cols, const float* x, float* y);
+
+/* ---- ops --------------------------------------------------------------- */
+void tso_rms_norm(const float* x, const float* w, int64_t n, float eps, float* y);
+void tso_rope_neox(float* x, int num_tokens, int num_heads, int head_dim, int rotated_pairs,
+                   int64_t position, float theta);
+void tso_rope_neox_freqs(float* x, int num_tokens, int num_heads, int head_dim, int rotated_pairs,
+                         int64_t position, const float* freqs);
+int tso_llama3_rope_factors(int rotary_dim, double base, double factor, double low_freq_factor,
+                            double high_freq_factor, double original_context, float* out);
+void tso_rope_frequencies_with_factors(int rotary_dim, float base, const float* factors, float* out);
+/* window <= 0: full; sinks NULL: none; scale <= 0: 1/sqrt(head_dim). */
+void tso_causal_attention(const float* q, const float* k, const float* v, int head_dim, int nq,
+                          int nkv, int64_t seq_len, int64_t window, float scale, const float* sinks,
+                          float* out);
+void tso_attention_core(const float* q, const float* k, const float* v, int head_dim, int nq,
+                        int nkv, int64_t kv_start, int64_t prefix_end, const int64_t* extra,
+                        int n_extra, float scale, const float* sinks, float* out);
+float tso_silu(float x);
+
+/* ---- selection --------------------------------------------------------- */
+typedef struct {
+    double temperature;
+    uint32_t top_k;
+    int32_t has_top_p;
+    double top_p;
+    double repetition_penalty;
+    int32_t has_seed; /* benchmarks always pass a seed; 0 here is refused */
+    uint64_t seed;
+    double presence_penalty;
+    double frequency_penalty;
+    int32_t has_min_p;
+    double min_p;
+} tso_shaping;
+
+uint64_t tso_mix(uint64_t x);
+uint64_t tso_derive_step_value(uint64_t seed, uint64_t position);
+double tso_to_unit_interval(uint64_t v);
+/* Returns 0 on success, <0 on the reference's refusals (empty domain, non-finite). */
+int tso_select(const uint16_t* logits, int64_t vocab, const tso_shaping* cfg, const int32_t* history,
+               int64_t n_history, uint64_t position, int32_t* out_token);
+/* support/probs must hold `vocab` entries. */
+int tso_shaped_distribution(const uint16_t* logits, int64_t vocab, const tso_shaping* cfg,
+                            const int32_t* history, int64_t n_history, uint64_t position,
+                            uint32_t* support, double* probs, int64_t* n_out);
+double tso_dist_probability(const uint32_t* support, const double* probs, int64_t n, uint32_t token);
+uint32_t tso_dist_draw(const uint32_t* support, const double* probs, int64_t n, uint64_t seed,
+                       uint64_t position);
+/* Returns 1 and fills out (capacity np) when mass survives, 0 for the None case. */
+int tso_residual(const uint32_t* ps, const double* pp, int64_t np, const uint32_t* qs,
+                 const double* qp, int64_t nq, uint32_t* out_support, double* out_probs,
+                 int64_t* n_out);
+
+/* ---- one speculative round's host half -------------------------------- */
+typedef struct {
+    int32_t accepted;       /* proposals accepted this round */
+    int32_t committed;      /* tokens pushed to history this round (excludes a stopping token) */
+    int32_t next;           /* corrected / bonus token; -1 when the round stopped */
+    int32_t stopped;        /* 0 none, 1 stop token, 2 budget */
+    uint64_t draw_step;     /* counter after the round */
+    int32_t path[17];       /* tree rounds: accepted slots, path[0] = 0 */
+    int32_t path_len;
+} tso_round_result;
+
+/* Draft half of a sampled chain round (speculative.rs:606-660): draws k proposals,
+ * one from each row of draft_logits, then advances draw_step once more for the
+ * row-only step.  Greedy: argmax per row, draw_step untouched. */
+int tso_draft_chain(const uint16_t* draft_logits, int k, int64_t vocab, const tso_shaping* cfg,
+                    const int32_t* history, int64_t n_history, uint64_t generated,
+                    uint64_t* draw_step, int32_t* proposals);
+/* Acceptance + bonus (speculative.rs:694-754, 861-879).  target_logits is (k+1) x vocab.
+ * stop_tokens may be NULL.  max_new_tokens bounds `generated` as the sink does. */
+int tso_chain_round(const uint16_t* target_logits, const uint16_t* draft_logits,
+                    const int32_t* proposals, int k, int64_t vocab, const tso_shaping* cfg,
+                    const int32_t* history, int64_t n_history, uint64_t generated,
+                    uint64_t max_new_tokens, const int32_t* stop_tokens, int n_stop,
+                    uint64_t draw_step, tso_round_result* out);
+/* Greedy tree walk (speculative.rs:494-550); parent[] are SLOT parents, parent[0] = -1. */
+int tso_tree_round_greedy(const uint16_t* target_logits, const int32_t* feed, const int32_t* parent,
+                          int m, int64_t vocab, const tso_shaping* cfg, const int32_t* history,
+                          int64_t n_history, uint64_t generated, uint64_t max_new_tokens,
+                          const int32_t* stop_tokens, int n_stop, tso_round_result* out);
+/* Multi-branch rejection on a tree.  NOT IN THE REFERENCE -- this project's definition:
+ * at each accepted node, children are tried in slot order; child c (token x, drawn from
+ * the drafter row q of its parent) is accepted iff r*q(x) <= p(x) with a fresh uniform;
+ * on rejection p <- normalise(max(p - q, 0)) and the next sibling is tried; when all
+ * siblings are rejected (or there are none) the next token is drawn from the current p.
+ * draft_logits is m x vocab: row s is the drafter distribution the children of slot s
+ * were drawn from. */
+int tso_tree_round_sampled(const uint16_t* target_logits, const uint16_t* draft_logits,
+                           const int32_t* feed, const int32_t* parent, int m, int64_t vocab,
+                           const tso_shaping* cfg, const int32_t* history, int64_t n_history,
+                           uint64_t generated, uint64_t draw_step, tso_round_result* out);
+
+/* ---- Llama-style target model ------------------------------------------ */
+typedef struct {
+    const void* data; /* row-major, one byte run per output row */
+    int32_t dtype;
+    int64_t rows, cols;
+} tso_tensor;
+
+typedef struct {
+    tso_tensor attn_norm, wq, wk, wv, wo, q_norm, k_norm; /* q_norm/k_norm data NULL when absent */
+    tso_tensor ffn_norm, w_gate, w_up, w_down;
+} tso_layer;
+
+typedef struct {
+    int32_t n_layers, hidden, n_q_heads, n_kv_heads, head_dim, ffn, vocab, max_context;
+    float rms_eps, rope_theta, attn_scale; /* attn_scale <= 0: 1/sqrt(head_dim) */
+    const float* rope_factors;             /* NULL or head_dim/2 per-pair divisors */
+    int32_t round_kv_f16;                  /* store K,V through fp16 (the engine's cache dtype) */
+    int32_t threads;                       /* OpenMP threads for the row loops; 1 = scalar reference */
+    tso_tensor embed, final_norm, lm_head; /* lm_head.data NULL => tied to embed */
+    const tso_layer* layers;
+} tso_model_desc;
+
+typedef struct tso_model tso_model;
+tso_model* tso_model_create(const tso_model_desc* desc);
+void tso_model_destroy(tso_model* m);
+void tso_model_reset(tso_model* m);
+int64_t tso_model_position(const tso_model* m);
+void tso_model_rewind_to(tso_model* m, int64_t position); /* kv_cache_rewind.rs:46-55 */
+/* Raw access to the fp32 KV store of one layer: [position][kv_head][head_dim]. */
+float* tso_model_k(tso_model* m, int layer);
+float* tso_model_v(tso_model* m, int layer);
+/* One batched pass over `m_rows` fed tokens at base (batched.rs:92-456 semantics for a
+ * pure-attention target).  parent NULL => chain (row i at position base+i, sees [0, base+i]).
+ * parent given => tree (row s rotated at base+depth[s], sees [0,base) + its root path; K/V of
+ * slot s stored at cache position base+s).  logits_f16 (m_rows x vocab) and logits_f32 are
+ * both optional.  n_layers_run < 0 => all layers (a positive value runs a prefix of the
+ * stack and then the head; used only to bound the timed CPU baseline sample).
+ * Advances the cursor by m_rows. */
+int tso_model_verify(tso_model* m, const int32_t* feed, const int32_t* parent, int m_rows,
+                     int64_t base, uint16_t* logits_f16, float* logits_f32, int n_layers_run);
+/* Tree compaction (families/qwen/dflash_tree.rs:106-207): move the K/V rows of slots
+ * path[0..n) to cache positions base..base+n. */
+void tso_model_compact_tree(tso_model* m, int64_t base, const uint32_t* path, int n);
+
+const char* tso_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
