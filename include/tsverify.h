@@ -1,0 +1,196 @@
+/*
+ * tsverify.h -- C ABI of the MI355X speculative-decoding verify engine.
+ *
+ * One handle (tsv_ctx) is one target model resident in HBM plus its fp16 KV cache:
+ * the drop-in for the reference's `SpeculativeProducer` on a pure-attention target
+ * (crates/runtime/src/producer.rs:164-387).  Each entry point names the trait method
+ * (or reference function) it replaces.  Conventions are the reference's own outbound
+ * C ABI conventions (crates/ffi/include/turbospark.h:10-34): int32 status (0 = OK),
+ * a thread-local last-error string, borrowed const inputs, opaque handles, no
+ * unwinding across the boundary, one generation at a time per handle.
+ *
+ * All pointers are plain host pointers unless a parameter says "device".
+ */
+#ifndef TSVERIFY_H
+#define TSVERIFY_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TSV_MAX_ROWS 16 /* rows one verify pass takes (reference: MAX_BATCH_ROWS, crates/gpu/src/dequant_int4_batch.rs:50) */
+
+/* Status codes. */
+enum {
+    TSV_OK = 0,
+    TSV_ERR_INVALID = -1,     /* a refusal by name: bad argument, cursor mismatch, unsupported shaping */
+    TSV_ERR_DEVICE = -2,      /* a HIP call failed */
+    TSV_ERR_UNSUPPORTED = -3, /* a shape or dtype this build has no kernel for */
+};
+
+/* Weight storage types; the values are ggml type ids, as in the reference's GGUF intake. */
+enum {
+    TSV_F32 = 0,
+    TSV_F16 = 1,
+    TSV_Q8_0 = 8,  /* 34 B / 32 elems  (crates/compute/src/quant_gguf/q8_0.rs) */
+    TSV_Q4_K = 12, /* 144 B / 256 elems (crates/compute/src/quant_gguf/q4_k.rs) */
+    TSV_BF16 = 30,
+};
+
+/* A host tensor in GGUF layout: one byte run per output row, rows x cols elements. */
+typedef struct {
+    const void* data;
+    int32_t dtype;
+    int64_t rows, cols;
+} tsv_tensor;
+
+/* One decoder layer (crates/runtime/src/families/llama/{attn,dense}.rs).  q_norm/k_norm
+ * (per-head RMSNorm, qwen3 style) have data == NULL when absent. */
+typedef struct {
+    tsv_tensor attn_norm, wq, wk, wv, wo, q_norm, k_norm;
+    tsv_tensor ffn_norm, w_gate, w_up, w_down;
+} tsv_layer;
+
+typedef struct {
+    int32_t n_layers, hidden, n_q_heads, n_kv_heads, head_dim, ffn, vocab, max_context;
+    float rms_eps, rope_theta, attn_scale; /* attn_scale <= 0 means 1/sqrt(head_dim) */
+    const float* rope_factors;             /* NULL, or head_dim/2 llama-3 per-pair divisors */
+    tsv_tensor embed, final_norm, lm_head; /* lm_head.data NULL: tied to embed */
+    const tsv_layer* layers;
+} tsv_model_desc;
+
+typedef struct tsv_ctx tsv_ctx;
+
+/* Shaping configuration: crates/selection/src/shaping.rs:44-123 (`ShapingConfig`). */
+typedef struct {
+    double temperature;
+    uint32_t top_k;
+    int32_t has_top_p;
+    double top_p;
+    double repetition_penalty;
+    int32_t has_seed;
+    uint64_t seed;
+    double presence_penalty;
+    double frequency_penalty;
+    int32_t has_min_p;
+    double min_p;
+} tsv_shaping;
+
+/* A rollback point: `SpeculativeProducer::Checkpoint` (real_forward_rollback.rs:19-28)
+ * for a target with no recurrent state. */
+typedef struct {
+    int64_t position;
+} tsv_point;
+
+/* One round handed to the fused entry point. */
+typedef struct {
+    const int32_t* feed;   /* feed[0] = the confirmed token, feed[1..m) = proposals / tree nodes */
+    const int32_t* parent; /* NULL: chain.  Else slot parents, parent[0] = -1, parent[s] < s */
+    int32_t m;             /* rows, 1..TSV_MAX_ROWS */
+    int64_t base;          /* position of feed[0]; must equal the KV cursor */
+    tsv_shaping shaping;
+    /* Drafter logits, fp16, host or device memory.  Chain: (m-1) x vocab, row i is the
+     * distribution proposal i was drawn from.  Tree: m x vocab, row s is the distribution
+     * the children of slot s were drawn from.  NULL at temperature 0. */
+    const uint16_t* draft_logits;
+    uint64_t draw_step; /* the loop's monotone uniform counter (speculative.rs:396-402) */
+    const int32_t* stop_tokens;
+    int32_t n_stop;
+    uint64_t generated;      /* tokens reported so far (TokenSink::generated) */
+    uint64_t max_new_tokens; /* budget; 0 = unbounded */
+    uint16_t* logits_out;    /* optional: m x vocab fp16 copy of the verify logits */
+} tsv_round;
+
+typedef struct {
+    int32_t accepted;  /* proposals (tree: nodes) accepted */
+    int32_t committed; /* tokens pushed to history (a stopping token is counted, not pushed) */
+    int32_t next;      /* corrected / bonus token, -1 if the round stopped */
+    int32_t stopped;   /* 0 no, 1 stop token, 2 budget */
+    uint64_t draw_step;
+    int32_t path[TSV_MAX_ROWS + 1]; /* accepted slots, path[0] = 0 (chain: 0,1,..,accepted) */
+    int32_t path_len;
+    int64_t kv_position; /* KV cursor after truncation: base + committed + 1 */
+    /* Smallest relative distance of any f64 comparison this round (acceptance tests and
+     * the cumulative draw) from flipping; decisions are bit-stable against host libm /
+     * summation-order differences while this is >> 1e-12. */
+    double min_margin;
+} tsv_round_result;
+
+/* ---- lifetime ------------------------------------------------------------- */
+/* Uploads and re-tiles the weights, allocates the KV cache.  Replaces
+ * `RealForwardRunner::open` for the scope of this path. */
+int32_t tsv_open(const tsv_model_desc* desc, tsv_ctx** out);
+void tsv_close(tsv_ctx* ctx);
+/* Copies the calling thread's last error text (NUL-terminated) into buf; returns its length. */
+int32_t tsv_last_error(char* buf, int32_t cap);
+/* The HIP stream every kernel of this handle is launched on (a hipStream_t). */
+void* tsv_stream(tsv_ctx* ctx);
+
+/* ---- LogitProducer (producer.rs:17-104) ------------------------------------ */
+int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset */
+int64_t tsv_kv_position(const tsv_ctx* ctx);   /* kv.position() */
+/* LogitProducer::produce: one token at `position`; logits: vocab fp16. */
+int32_t tsv_produce(tsv_ctx* ctx, int32_t token, int64_t position, uint16_t* logits);
+/* produce_prefill / ChunkedPrefillRunner::prefill_chunk: feeds n tokens from pos0 in
+ * passes of TSV_MAX_ROWS rows; logits (nullable) receives the LAST token's row. */
+int32_t tsv_prefill(tsv_ctx* ctx, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits);
+
+/* ---- SpeculativeProducer (producer.rs:164-387) ------------------------------ */
+int32_t tsv_checkpoint(tsv_ctx* ctx, tsv_point* out);              /* checkpoint() */
+int32_t tsv_rollback(tsv_ctx* ctx, const tsv_point* point);        /* rollback() */
+/* rollback_retaining(point, keep_rows): new KV length = point + keep_rows. */
+int32_t tsv_rollback_retaining(tsv_ctx* ctx, const tsv_point* point, int32_t keep_rows);
+int32_t tsv_commit_pending(tsv_ctx* ctx, int32_t keep_rows); /* no-op without recurrent state */
+int32_t tsv_discard_pending(tsv_ctx* ctx);
+/* verify(feed, base, logits): m rows at base..base+m, row i sees [0, base+i].
+ * logits nullable (m x vocab fp16): NULL keeps them on the device for tsv_accept. */
+int32_t tsv_verify(tsv_ctx* ctx, const int32_t* feed, int32_t m, int64_t base, uint16_t* logits);
+/* verify_tree(feed, parent, base, logits): row s rotated at base+depth[s], sees the
+ * prefix plus its root path; K/V of slot s stored at cache position base+s. */
+int32_t tsv_verify_tree(tsv_ctx* ctx, const int32_t* feed, const int32_t* parent, int32_t m,
+                        int64_t base, uint16_t* logits);
+/* compact_tree(base, path): gather the accepted path's K/V rows to base..base+n. */
+int32_t tsv_compact_tree(tsv_ctx* ctx, int64_t base, const uint32_t* path, int32_t n);
+
+/* ---- acceptance on the device ----------------------------------------------- */
+/* The host half of a round (speculative.rs:694-754, 861-879; tree: 494-550) run as
+ * kernels over the logits the last verify left on the device, followed by the KV
+ * truncation (and, for a tree, compaction).  Uses round->{parent,m,base,shaping,
+ * draft_logits,draw_step,stop_tokens,generated,max_new_tokens}; feed must be the feed
+ * of that verify. */
+int32_t tsv_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result* out);
+/* verify + accept + truncate in one call: the whole verify step. */
+int32_t tsv_verify_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result* out);
+/* Draft half of a sampled chain round (speculative.rs:606-660): draws k proposals, one
+ * from each row of draft_logits (k x vocab fp16, host or device), advancing *draw_step by
+ * k + 1; greedy: argmax per row. */
+int32_t tsv_draft_chain(tsv_ctx* ctx, const uint16_t* draft_logits, int32_t k,
+                        const tsv_shaping* shaping, uint64_t* draw_step, int32_t* proposals);
+
+/* ---- install-time helpers (host) --------------------------------------------- */
+/* The reference's quantize-on-install encoders (q8_0.rs:56-77, q4_k.rs:126-204). */
+int64_t tsv_row_bytes(int32_t dtype, int64_t cols);
+int32_t tsv_quantize_rows(int32_t dtype, const float* src, int64_t rows, int64_t cols, void* dst);
+/* Seeded synthetic tensor: rows x cols of N(0, sigma) from a counter-based generator
+ * keyed by (seed, stream), quantized to dtype row by row (the random-init installs of
+ * crates/repack/src/synthetic_*.rs).  dst holds rows * tsv_row_bytes(dtype, cols) bytes. */
+int32_t tsv_synth_tensor(int32_t dtype, uint64_t seed, uint64_t stream, float sigma, int64_t rows,
+                         int64_t cols, void* dst);
+
+/* ---- introspection for tests -------------------------------------------------- */
+/* Copies layer `layer`'s K and V rows [pos0, pos0+n) to host as fp16 in the reference
+ * layout [position][kv_head][head_dim] (crates/gpu/src/kv_cache.rs:1-10). */
+int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v);
+/* One quantized small-M matmul through the same kernels the forward uses:
+ * y[m][r] = sum_k W[r][k] x[m][k]; x is m x cols fp32 (rounded to fp16 on entry), y is
+ * m x rows fp32.  W host tensor in GGUF layout (re-tiled per call).  `splits` <= 0 picks
+ * the engine's own split-K factor. */
+int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,80 @@
+"""GPU parity of the dequant-fused small-M matmul against the oracle's dequantize-then-dot.
+
+Mirrors crates/gpu/tests/dequant_q4_k_gemv_parity.rs (bound scale*1e-2 + n*1e-4, :34-45) and
+dequant_kquant_gemm_parity.rs (every width 1..16; a row's result must not depend on how many
+rows ride with it)."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from tests.test_oracle_quant import lcg_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dtype, rows, cols, seed):
+    from turbospark_amd import ffi
+    w = lcg_weights(rows * cols, seed).reshape(rows, cols) * 0.05
+    entry = ffi.quantize(dtype, w)
+    x = lcg_weights(16 * cols, seed + 1).reshape(16, cols)
+    x16 = x.astype(np.float16).astype(np.float32)  # the kernel's operand precision
+    want = np.stack([ob.gemv(dtype, entry[1], rows, cols, x16[b]) for b in range(16)])
+    return entry, x, x16, want
+
+
+@pytest.mark.parametrize("dtype,rows,cols", [(12, 64, 512), (12, 48, 2048), (8, 64, 512), (8, 32, 1408)])
+def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
+    from turbospark_amd import ffi
+    entry, x, x16, want = _case(dtype, rows, cols, 31)
+    scale = np.abs(want).max()
+    bound = scale * 1e-2 + cols * 1e-4
+    first = None
+    for m in range(1, 17):
+        got = ffi.matmul(entry, x[:m])
+        assert got.shape == (m, rows)
+        err = np.abs(got - want[:m]).max()
+        assert err <= bound, (m, err, bound)
+        # much tighter than the reference's bound: fp32 accumulation of exact products
+        assert err <= scale * 2e-4 + 1e-5, (m, err)
+        if first is None:
+            first = got[0].copy()
+        # row invariance: row 0 is bit-identical whatever rides with it
+        assert np.array_equal(got[0], first), m
+
+
+@pytest.mark.parametrize("dtype", [12, 8])
+def test_split_k_changes_nothing_but_rounding_and_is_deterministic(dtype):
+    from turbospark_amd import ffi
+    entry, x, x16, want = _case(dtype, 32, 2048, 77)
+    a = ffi.matmul(entry, x[:5], splits=1)
+    b = ffi.matmul(entry, x[:5], splits=4)
+    c = ffi.matmul(entry, x[:5], splits=4)
+    assert np.array_equal(b, c)
+    assert np.abs(a - b).max() <= np.abs(want).max() * 1e-5 + 1e-6
+    assert np.abs(a - want[:5]).max() <= np.abs(want).max() * 2e-4 + 1e-5
+
+
+def test_q4k_hand_packed_superblock_through_the_kernel(golden):
+    """The reference's literal superblock (quant_gguf.rs:226-267) as a 16-row weight matrix:
+    one-hot activations read the decoded weights back out of the kernel."""
+    import json, os
+    from turbospark_amd import ffi
+    g = json.load(open(os.path.join(golden, "q4k_handpacked.json")))
+    quants = [(e * 7 + 3) % 16 for e in range(256)]
+    body = bytearray(g["D_BITS"] + g["DMIN_BITS"] + g["PACKED"])
+    for grp in range(4):
+        for l in range(32):
+            at = grp * 64 + l
+            body.append(quants[at] | (quants[at + 32] << 4))
+    blk = np.frombuffer(bytes(body), np.uint8)
+    raw = np.tile(blk, (16, 1))
+    entry = (ffi.Q4_K, np.ascontiguousarray(raw), 16, 256)
+    want = np.array([g["d"] * g["LS"][e // 32] * quants[e] - g["dmin"] * g["LM"][e // 32] for e in range(256)],
+                    np.float32)
+    for e0 in range(0, 256, 16):
+        x = np.zeros((16, 256), np.float32)
+        for b in range(16):
+            x[b, e0 + b] = 1.0
+        got = ffi.matmul(entry, x)
+        for b in range(16):
+            assert np.all(got[b] == want[e0 + b]), (e0 + b, got[b, 0], want[e0 + b])

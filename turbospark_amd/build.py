@@ -1,0 +1,53 @@
+"""Builds turbospark_amd/libtsverify.so (HIP kernels + C ABI) for gfx950 with hipcc."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libtsverify.so")
+SOURCES = ["gemm.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip"]
+# host_utils.hip is host-only code; clang 22 -O3 does not terminate on it, -O2 does.
+OPT = {"host_utils.hip": "-O2"}
+FLAGS = [
+    "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # packed-fp32 VALU forms are switched off for every kernel in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-pthread",
+]
+
+
+def build(verbose=False):
+    objs = []
+    procs = []
+    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    for src in SOURCES:
+        obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+        cmd = ["hipcc", OPT.get(src, "-O3"), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        objs.append(obj)
+    failed = False
+    for src, p in procs:
+        try:
+            out, _ = p.communicate(timeout=900)
+        except subprocess.TimeoutExpired:
+            p.kill()
+            out, _ = p.communicate()
+            out += b"\n(compiler killed after 900 s)"
+            p.returncode = -9
+        text = out.decode(errors="replace")
+        if p.returncode != 0:
+            failed = True
+            sys.stderr.write(f"--- {src} failed ---\n{text}\n")
+        elif verbose and text.strip():
+            print(f"--- {src} ---\n{text}")
+    if failed:
+        raise RuntimeError("hipcc failed")
+    subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-pthread", *objs, "-o", LIB])
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

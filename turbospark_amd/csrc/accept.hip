@@ -1,0 +1,649 @@
+// Device-side acceptance for a speculative round: softmax statistics, greedy / rejection
+// sampling acceptance, the residual or bonus draw, and the round's bookkeeping.
+//
+// Restates on the GPU what the reference runs on the host in f64
+// (crates/runtime/src/speculative.rs:694-754,861-879; crates/selection/src/choose.rs:111-338,
+// distribution.rs:61-126, derive.rs:19-45) so a round returns a few dozen bytes instead of
+// m x vocab fp16 logits.
+//
+// Arithmetic: every probability is computed in f64 with the reference's operation sequence
+//   e = exp(f64(w) - max);  p = e / sum;  weight = pow(p / top, 1/T);  prob = weight / total
+// but `sum` and `total` are parallel (fixed-order, deterministic) reductions rather than one
+// sequential loop, and the cumulative draw walks rank order (logit descending, index ascending)
+// through a 65536-bin histogram keyed by the fp16 logit -- exp is monotone, so rank-by-exp is
+// rank-by-logit -- instead of sorting the vocabulary.  Integer outputs can therefore differ
+// from the host sequence only when a comparison is within ~1e-13 of flipping; every comparison's
+// distance from flipping is folded into `min_margin` so a caller can see that it never was.
+// Bin masses are accumulated as 2^-62 fixed point with integer atomics: order independent,
+// hence bit-reproducible run to run.
+#include "tsv_internal.h"
+
+namespace tsv {
+
+namespace {
+
+constexpr int NSEG = 64;          // index segments per vocabulary row
+constexpr int MAX_DIST_ROWS = 32;  // target rows + drafter rows
+constexpr int MAX_JOBS = 16;
+constexpr double FIX = 4611686018427387904.0;  // 2^62
+
+struct RowStat {
+    double mx, sum, total, top;
+};
+
+// Scratch layout inside AcceptScratch::stats (doubles):
+//   [0, 4*32)                         RowStat per distribution row
+//   pmax / psum / ptot partials follow
+struct Layout {
+    RowStat* stat;
+    double* pmax;  // [rows][NSEG]
+    double* psum;
+    double* ptot;
+    double* segtot;  // [jobs][NSEG] residual mass per segment
+};
+__host__ __device__ inline Layout layout(double* base) {
+    Layout l;
+    l.stat = (RowStat*)base;
+    l.pmax = base + 4 * MAX_DIST_ROWS;
+    l.psum = l.pmax + MAX_DIST_ROWS * NSEG;
+    l.ptot = l.psum + MAX_DIST_ROWS * NSEG;
+    l.segtot = l.ptot + MAX_DIST_ROWS * NSEG;
+    return l;
+}
+
+struct Job {
+    int32_t mode;  // 0 none, 1 draw from p, 2 draw from residual(p, q)
+    int32_t row_p, row_q;
+    double u;
+};
+
+struct Decision {
+    Job job;
+    int32_t accepted, committed, stopped, pad;
+    uint64_t draw_step;
+    double margin;
+};
+
+__device__ __forceinline__ float h2f(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+
+// crates/selection/src/derive.rs:19-45
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+__device__ __forceinline__ double unit_draw(uint64_t seed, uint64_t position) {
+    const uint64_t v = mix64(seed ^ (position * 0x9E3779B97F4A7C15ull));
+    return (double)(v >> 11) * (1.0 / 9007199254740992.0);
+}
+
+// Rank key of an fp16 logit: 0 for the largest value, ascending as the logit falls; +0 and
+// -0 share a key (they have the same exp, so the reference breaks their tie by index).
+__device__ __forceinline__ uint32_t rank_key(uint16_t b) {
+    if (b == 0x8000u) b = 0;
+    const uint32_t asc = (b & 0x8000u) ? (uint32_t)(~b & 0xFFFFu) : (uint32_t)(b | 0x8000u);
+    return 0xFFFFu - asc;
+}
+
+// choose.rs:296-319 for one candidate of a row whose statistics are known
+__device__ __forceinline__ double prob_of(uint16_t bits, const RowStat& s, double inv_t) {
+    const double e = exp((double)h2f(bits) - s.mx);
+    const double p = e / s.sum;
+    return pow(p / s.top, inv_t) / s.total;
+}
+
+template <typename T>
+__device__ __forceinline__ T shfl_xor_t(T v, int o) {
+    static_assert(sizeof(T) == 8, "64-bit only");
+    uint64_t u = __builtin_bit_cast(uint64_t, v);
+    uint32_t lo = __shfl_xor((uint32_t)u, o), hi = __shfl_xor((uint32_t)(u >> 32), o);
+    return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+}
+
+// Deterministic block sum: xor-butterfly inside a wave, then the waves in index order.
+__device__ double block_sum_f64(double v, double* red) {
+    for (int o = 32; o > 0; o >>= 1) v += shfl_xor_t(v, o);
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (int i = 0; i < nw; i++) t += red[i];
+    return t;
+}
+
+__device__ __forceinline__ const uint16_t* row_ptr(const uint16_t* target, const uint16_t* draft, int m,
+                                                   int vocab, int row) {
+    return row < m ? target + (long)row * vocab : draft + (long)(row - m) * vocab;
+}
+
+// ---- statistics, three short passes over every distribution row -------------------------
+__global__ __launch_bounds__(256) void k_row_max(const uint16_t* target, const uint16_t* draft, int m,
+                                                 int vocab, double* scratch, int32_t* err) {
+    __shared__ double red[4];
+    const int row = blockIdx.y, seg = blockIdx.x;
+    const uint16_t* p = row_ptr(target, draft, m, vocab, row);
+    const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    float mx = -INFINITY;
+    bool bad = false;
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const uint16_t b = p[v];
+        bad |= (b & 0x7C00u) == 0x7C00u;
+        mx = fmaxf(mx, h2f(b));
+    }
+    if (bad) atomicOr(err, 1);
+    double d = (double)mx;
+    for (int o = 32; o > 0; o >>= 1) d = fmax(d, shfl_xor_t(d, o));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = d;
+    __syncthreads();
+    if (threadIdx.x == 0) layout(scratch).pmax[row * NSEG + seg] = fmax(fmax(red[0], red[1]), fmax(red[2], red[3]));
+}
+
+__global__ __launch_bounds__(256) void k_row_sum(const uint16_t* target, const uint16_t* draft, int m,
+                                                 int vocab, double* scratch) {
+    __shared__ double red[4];
+    const int row = blockIdx.y, seg = blockIdx.x;
+    Layout L = layout(scratch);
+    double mx = -INFINITY;
+    for (int s = 0; s < NSEG; s++) mx = fmax(mx, L.pmax[row * NSEG + s]);
+    const uint16_t* p = row_ptr(target, draft, m, vocab, row);
+    const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    double acc = 0.0;
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) acc += exp((double)h2f(p[v]) - mx);
+    acc = block_sum_f64(acc, red);
+    if (threadIdx.x == 0) {
+        L.psum[row * NSEG + seg] = acc;
+        if (seg == 0) L.stat[row].mx = mx;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const uint16_t* draft, int m,
+                                                   int vocab, double* scratch, double inv_t) {
+    __shared__ double red[4];
+    const int row = blockIdx.y, seg = blockIdx.x;
+    Layout L = layout(scratch);
+    double mx = -INFINITY, sum = 0.0;
+    for (int s = 0; s < NSEG; s++) {
+        mx = fmax(mx, L.pmax[row * NSEG + s]);
+        sum += L.psum[row * NSEG + s];
+    }
+    const double top = 1.0 / sum;  // the arg-max candidate has e == exp(0) == 1
+    const uint16_t* p = row_ptr(target, draft, m, vocab, row);
+    const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    double acc = 0.0;
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const double e = exp((double)h2f(p[v]) - mx);
+        acc += pow((e / sum) / top, inv_t);
+    }
+    acc = block_sum_f64(acc, red);
+    if (threadIdx.x == 0) {
+        L.ptot[row * NSEG + seg] = acc;
+        if (seg == 0) {
+            L.stat[row].sum = sum;
+            L.stat[row].top = top;
+        }
+    }
+}
+
+__device__ RowStat load_stat(const Layout& L, int row) {
+    RowStat s;
+    double mx = -INFINITY, sum = 0.0, tot = 0.0;
+    for (int i = 0; i < NSEG; i++) {
+        mx = fmax(mx, L.pmax[row * NSEG + i]);
+        sum += L.psum[row * NSEG + i];
+        tot += L.ptot[row * NSEG + i];
+    }
+    s.mx = mx;
+    s.sum = sum;
+    s.top = 1.0 / sum;
+    s.total = tot;
+    return s;
+}
+
+__device__ __forceinline__ void fold_margin(double& margin, double a, double b) {
+    const double scale = fmax(fabs(a), fabs(b));
+    const double rel = scale > 0.0 ? fabs(a - b) / scale : 0.0;
+    margin = fmin(margin, rel);
+}
+
+// TokenSink::commit restricted to what a token-id interface can see
+// (crates/runtime/src/token_sink.rs:64-124): 0 continue, 1 stop token, 2 budget.
+__device__ int sink_commit(const AcceptParams& ap, int32_t token, uint64_t& generated, int32_t& committed) {
+    generated += 1;
+    for (int i = 0; i < ap.n_stop; i++)
+        if (ap.stop_tokens[i] == token) return 1;
+    if (ap.max_new_tokens != 0 && generated >= ap.max_new_tokens) return 2;
+    committed += 1;
+    return 0;
+}
+
+// speculative.rs:694-754: the sequential walk over the proposals of a sampled chain round.
+__device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t* target,
+                                         const uint16_t* draft, const Layout& L) {
+    Decision d;
+    d.job.mode = 0;
+    d.job.row_p = d.job.row_q = 0;
+    d.job.u = 0.0;
+    d.accepted = d.committed = d.stopped = d.pad = 0;
+    d.margin = 1.0;
+    uint64_t ds = ap.draw_step, gen = ap.generated;
+    const double inv_t = 1.0 / ap.temperature;
+    int reject = -1;
+    for (int i = 0; i < ap.k; i++) {
+        const int32_t x = ap.feed[i + 1];
+        const RowStat sp = load_stat(L, i), sq = load_stat(L, ap.m + i);
+        const double px = prob_of(target[(long)i * ap.vocab + x], sp, inv_t);
+        const double qx = prob_of(draft[(long)i * ap.vocab + x], sq, inv_t);
+        const double r = unit_draw(ap.seed, ds);
+        ds += 1;
+        fold_margin(d.margin, r * qx, px);
+        if (r * qx <= px) {
+            d.accepted += 1;
+            if ((d.stopped = sink_commit(ap, x, gen, d.committed))) break;
+        } else {
+            reject = i;
+            break;
+        }
+    }
+    if (!d.stopped) {
+        d.job.u = unit_draw(ap.seed, ds);
+        ds += 1;
+        if (reject >= 0) {
+            d.job.mode = 2;
+            d.job.row_p = reject;
+            d.job.row_q = ap.m + reject;
+        } else {
+            d.job.mode = 1;
+            d.job.row_p = d.accepted;
+        }
+    }
+    d.draw_step = ds;
+    return d;
+}
+
+// ---- masses + rank histogram --------------------------------------------------------------
+// kind 0: the job comes out of the chain decision (every workgroup re-derives it: a few
+// dozen f64 ops).  kind 1: jobs are "draw from drafter row j at position draw_step + j".
+__global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const uint16_t* draft,
+                                                   const AcceptParams* app, double* scratch, double* work,
+                                                   unsigned long long* hist, Decision* dec_out, int kind) {
+    __shared__ Decision dec;
+    __shared__ double red[4];
+    const AcceptParams& ap = *app;
+    const int seg = blockIdx.x, jobi = blockIdx.y;
+    Layout L = layout(scratch);
+    if (threadIdx.x == 0) {
+        if (kind == 0) {
+            dec = decide_chain_sampled(ap, target, draft, L);
+        } else {
+            dec.job.mode = 1;
+            dec.job.row_p = ap.m + jobi;
+            dec.job.row_q = 0;
+            dec.job.u = unit_draw(ap.seed, ap.draw_step + jobi);
+            dec.accepted = dec.committed = dec.stopped = 0;
+            dec.draw_step = ap.draw_step;
+            dec.margin = 1.0;
+        }
+        if (seg == 0) dec_out[jobi] = dec;
+    }
+    __syncthreads();
+    const Job job = dec.job;
+    if (job.mode == 0) return;
+    const int vocab = ap.vocab;
+    const double inv_t = 1.0 / ap.temperature;
+    const RowStat sp = load_stat(L, job.row_p);
+    RowStat sq = sp;
+    if (job.mode == 2) sq = load_stat(L, job.row_q);
+    const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, job.row_p);
+    const uint16_t* lq = row_ptr(target, draft, ap.m, vocab, job.row_q);
+    double* wp = work + (long)jobi * 2 * vocab;
+    double* wr = wp + vocab;
+    unsigned long long* hp = hist + (long)jobi * 2 * 65536;
+    unsigned long long* hr = hp + 65536;
+    const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    double racc = 0.0;
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const uint16_t b = lp[v];
+        const double pv = prob_of(b, sp, inv_t);
+        const uint32_t key = rank_key(b);
+        wp[v] = pv;
+        atomicAdd(hp + key, (unsigned long long)(pv * FIX));
+        if (job.mode == 2) {
+            const double mv = fmax(pv - prob_of(lq[v], sq, inv_t), 0.0);
+            wr[v] = mv;
+            racc += mv;
+            if (mv > 0.0) atomicAdd(hr + key, (unsigned long long)(mv * FIX));
+        }
+    }
+    if (job.mode == 2) {
+        racc = block_sum_f64(racc, red);
+        if (threadIdx.x == 0) L.segtot[jobi * NSEG + seg] = racc;
+    }
+}
+
+// ---- the cumulative walk --------------------------------------------------------------------
+// One workgroup per job.  Finds the rank bin in which the cumulative mass first exceeds the
+// uniform (exact integer prefix over the fixed-point bins, cleared as they are read), then
+// walks that bin's candidates in index order in f64.
+__global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uint16_t* draft,
+                                               const AcceptParams* app, double* scratch, const double* work,
+                                               unsigned long long* hist, const Decision* dec_in,
+                                               AcceptResult* res, int32_t* tokens_out, const int32_t* err,
+                                               int kind) {
+    __shared__ unsigned long long wsum[16];
+    __shared__ double dsum[16];
+    __shared__ unsigned long long s_total, s_before;
+    __shared__ int s_bin, s_last_bin, s_token, s_fallback;
+    __shared__ double s_cum_before, s_cum_at;
+    const AcceptParams& ap = *app;
+    const int jobi = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const Decision dec = dec_in[jobi];
+    Layout L = layout(scratch);
+    const int vocab = ap.vocab;
+    int token = -1;
+    double margin = dec.margin;
+
+    if (dec.job.mode != 0) {
+        int mode = dec.job.mode;
+        double R = 1.0;
+        if (mode == 2) {
+            R = 0.0;
+            for (int s = 0; s < NSEG; s++) R += L.segtot[jobi * NSEG + s];
+            if (R < 1e-12) mode = 1;  // distribution.rs:96-126: residual underflow -> plain p draw
+        }
+        unsigned long long* hp = hist + (long)jobi * 2 * 65536;
+        unsigned long long* hsel = mode == 2 ? hp + 65536 : hp;
+        const double* w = work + (long)jobi * 2 * vocab + (mode == 2 ? vocab : 0);
+        const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, dec.job.row_p);
+
+        // 64 consecutive bins per thread; integer sums are exact and order independent
+        unsigned long long loc = 0;
+        for (int i = 0; i < 64; i++) loc += hsel[tid * 64 + i];
+        unsigned long long inc = loc;
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t lo = __shfl_up((uint32_t)inc, o), hi = __shfl_up((uint32_t)(inc >> 32), o);
+            const unsigned long long up = ((unsigned long long)hi << 32) | lo;
+            if (lane >= o) inc += up;
+        }
+        if (lane == 63) wsum[wave] = inc;
+        if (tid == 0) {
+            s_bin = -1;
+            s_last_bin = -1;
+            s_token = -1;
+            s_fallback = 0;
+        }
+        __syncthreads();
+        unsigned long long wbase = 0, total = 0;
+        for (int i = 0; i < 16; i++) {
+            if (i < wave) wbase += wsum[i];
+            total += wsum[i];
+        }
+        const unsigned long long excl = wbase + inc - loc;
+        // target in fixed point: u * total (the bins hold unnormalised mass in residual mode)
+        const unsigned long long tgt = (unsigned long long)(dec.job.u * (double)total);
+        if (loc > 0) atomicMax(&s_last_bin, tid * 64 + 63);
+        if (excl <= tgt && tgt < excl + loc) {
+            unsigned long long c = excl;
+            for (int i = 0; i < 64; i++) {
+                const unsigned long long hv = hsel[tid * 64 + i];
+                if (tgt < c + hv) {
+                    s_bin = tid * 64 + i;
+                    s_before = c;
+                    break;
+                }
+                c += hv;
+            }
+        }
+        if (tid == 0) s_total = total;
+        __syncthreads();
+        int bin = s_bin;
+        if (bin < 0) {
+            // rounding at the tail: the reference falls back to the LAST surviving candidate
+            // (choose.rs:333-338).  Last occupied bin, last matching index.
+            const int lb = s_last_bin;  // upper end of the last occupied 64-bin group
+            if (tid * 64 + 63 == lb) {
+                int bb = lb;
+                while (bb > tid * 64 && hsel[bb] == 0) bb--;
+                s_bin = bb;
+                s_before = total;
+                s_fallback = 1;
+            }
+            __syncthreads();
+            bin = s_bin;
+        }
+        const bool fallback = s_fallback != 0;
+        // walk the bin in index order: contiguous index chunk per thread
+        const int per = (vocab + 1023) / 1024, v0 = tid * per, v1 = min(v0 + per, vocab);
+        double lsum = 0.0;
+        int lastv = -1;
+        for (int v = v0; v < v1; v++)
+            if ((int)rank_key(lp[v]) == bin) {
+                const double wv = mode == 2 ? w[v] / R : w[v];
+                if (mode != 2 || wv > 0.0) {
+                    lsum += wv;
+                    lastv = v;
+                }
+            }
+        double incd = lsum;
+        for (int o = 1; o < 64; o <<= 1) {
+            uint64_t u = __builtin_bit_cast(uint64_t, incd);
+            uint32_t lo = __shfl_up((uint32_t)u, o), hi = __shfl_up((uint32_t)(u >> 32), o);
+            const double up = __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+            if (lane >= o) incd += up;
+        }
+        if (lane == 63) dsum[wave] = incd;
+        __syncthreads();
+        double dbase = 0.0;
+        for (int i = 0; i < wave; i++) dbase += dsum[i];
+        const double norm = (double)s_total;  // fixed-point total <-> 1.0 (p mode) or R (residual)
+        const double cum0 = (double)s_before / norm;  // cumulative mass before this bin
+        const double before = cum0 + (dbase + incd - lsum);
+        if (fallback) {
+            if (lastv >= 0) atomicMax(&s_token, lastv);
+        } else {
+            const double u = dec.job.u;
+            if (lsum > 0.0 && !(u < before) && u < before + lsum) {
+                double c = before;
+                for (int v = v0; v < v1; v++)
+                    if ((int)rank_key(lp[v]) == bin) {
+                        const double wv = mode == 2 ? w[v] / R : w[v];
+                        if (mode == 2 && !(wv > 0.0)) continue;
+                        if (u < c + wv) {
+                            s_token = v;
+                            s_cum_before = c;
+                            s_cum_at = c + wv;
+                            break;
+                        }
+                        c += wv;
+                    }
+            }
+        }
+        __syncthreads();
+        token = s_token;
+        if (token < 0) {
+            // the f64 walk and the fixed-point bin search disagreed by a rounding: the uniform
+            // sits on a bin edge.  Take the bin's first (u below) or last candidate and report
+            // a zero margin.
+            if (lastv >= 0) atomicMax(&s_token, lastv);
+            __syncthreads();
+            token = s_token;
+            margin = 0.0;
+        } else if (!fallback) {
+            margin = fmin(margin, fmin(dec.job.u - s_cum_before, s_cum_at - dec.job.u));
+        }
+        // clear both histograms of this job for the next round (every read is behind a barrier)
+        __syncthreads();
+        for (int i = tid; i < 2 * 65536; i += 1024) hp[i] = 0;
+    }
+
+    if (tid == 0) {
+        if (kind == 1) {
+            tokens_out[jobi] = token;
+            if (jobi == 0) res->error = *err;
+            // margins of the k draws are folded on the host side from res->min_margin
+            atomicMin((unsigned long long*)&res->min_margin, __builtin_bit_cast(unsigned long long, margin));
+        } else {
+            res->accepted = dec.accepted;
+            res->committed = dec.committed;
+            res->stopped = dec.stopped;
+            res->next = dec.stopped ? -1 : token;
+            res->draw_step = dec.draw_step;
+            res->path_len = dec.accepted + 1;
+            for (int i = 0; i <= dec.accepted; i++) res->path[i] = i;
+            res->min_margin = margin;
+            res->error = *err;
+        }
+    }
+}
+
+// ---- greedy --------------------------------------------------------------------------------
+// choose.rs:277-285: first maximum.  One workgroup per target row.
+__global__ __launch_bounds__(1024) void k_argmax(const uint16_t* target, int vocab, int32_t* out, int32_t* err) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    const uint16_t* p = target + (long)blockIdx.x * vocab;
+    float best = -INFINITY;
+    int idx = 0x7FFFFFFF;
+    bool bad = false;
+    for (int v = threadIdx.x; v < vocab; v += 1024) {
+        const uint16_t b = p[v];
+        bad |= (b & 0x7C00u) == 0x7C00u;
+        const float f = h2f(b);
+        if (f > best || (f == best && v < idx)) {
+            best = f;
+            idx = v;
+        }
+    }
+    if (bad) atomicOr(err, 1);
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o);
+        const int oi = __shfl_xor(idx, o);
+        if (ob > best || (ob == best && oi < idx)) {
+            best = ob;
+            idx = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        bv[threadIdx.x >> 6] = best;
+        bi[threadIdx.x >> 6] = idx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 16; i++)
+            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) {
+                best = bv[i];
+                idx = bi[i];
+            }
+        out[blockIdx.x] = idx;
+    }
+}
+
+// speculative.rs:736-754 (chain) and 494-550 (tree walk) at temperature 0.
+__global__ void k_walk_greedy(const AcceptParams* app, const int32_t* amax, AcceptResult* res, const int32_t* err) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const AcceptParams& ap = *app;
+    uint64_t gen = ap.generated;
+    int32_t committed = 0, stopped = 0, next = -1;
+    int at = 0, plen = 1;
+    res->path[0] = 0;
+    for (;;) {
+        const int32_t want = amax[at];
+        int hit = -1;
+        if (ap.tree) {
+            for (int s = 1; s < ap.m; s++)
+                if (ap.parent[s] == at && ap.feed[s] == want) {
+                    hit = s;
+                    break;
+                }
+        } else if (at + 1 < ap.m && ap.feed[at + 1] == want) {
+            hit = at + 1;
+        }
+        if (hit < 0) {
+            next = want;
+            break;
+        }
+        res->path[plen++] = hit;
+        at = hit;
+        if ((stopped = sink_commit(ap, want, gen, committed))) break;
+    }
+    res->accepted = plen - 1;
+    res->committed = committed;
+    res->stopped = stopped;
+    res->next = stopped ? -1 : next;
+    res->draw_step = ap.draw_step;
+    res->path_len = plen;
+    res->min_margin = 1.0;
+    res->error = *err;
+}
+
+__global__ void k_clear_result(AcceptResult* res, int32_t* err) {
+    if (threadIdx.x == 0) {
+        *err = 0;
+        res->error = 0;
+        res->min_margin = 1.0;
+    }
+}
+
+}  // namespace
+
+// scratch.counters: [0] error flag, [16..32) greedy arg-max per row; decisions live after the
+// statistics block; histograms and work arrays are separate allocations in AcceptScratch.
+size_t accept_stats_doubles() { return 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG + MAX_JOBS * 16; }
+
+static Decision* decisions(const AcceptScratch& sc) {
+    return (Decision*)(sc.stats + 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG);
+}
+
+int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
+                  const AcceptParams& ap, const AcceptScratch& sc) {
+    int32_t* err = (int32_t*)sc.counters;
+    int32_t* amax = (int32_t*)sc.counters + 16;
+    hipLaunchKernelGGL(k_clear_result, dim3(1), dim3(64), 0, s, sc.result, err);
+    if (!ap.sampled) {
+        hipLaunchKernelGGL(k_argmax, dim3(ap.m), dim3(1024), 0, s, target, ap.vocab, amax, err);
+        hipLaunchKernelGGL(k_walk_greedy, dim3(1), dim3(64), 0, s, ap_dev, amax, sc.result, err);
+        TSV_HIP(hipGetLastError());
+        return TSV_OK;
+    }
+    if (ap.tree) {
+        set_error("sampled acceptance over a tree is not built yet (the reference has none: speculative.rs:390-392)");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    const int rows = ap.m + ap.k;
+    const double inv_t = 1.0 / ap.temperature;
+    hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err);
+    hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
+    hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, inv_t);
+    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, 1), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), 0);
+    hipLaunchKernelGGL(k_pick, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), sc.result, (int32_t*)nullptr, err, 0);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+// Draft half of a chain round: proposals[j] = q_j.draw(seed, draw_step + j) (speculative.rs:636-648),
+// or the arg-max at temperature 0.  ap_dev: m = 0, k = rows, draw_step = first position.
+int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev, const AcceptParams& ap,
+                       const AcceptScratch& sc, int32_t* proposals_dev) {
+    int32_t* err = (int32_t*)sc.counters;
+    hipLaunchKernelGGL(k_clear_result, dim3(1), dim3(64), 0, s, sc.result, err);
+    if (!ap.sampled) {
+        hipLaunchKernelGGL(k_argmax, dim3(ap.k), dim3(1024), 0, s, draft, ap.vocab, proposals_dev, err);
+        TSV_HIP(hipGetLastError());
+        return TSV_OK;
+    }
+    const double inv_t = 1.0 / ap.temperature;
+    hipLaunchKernelGGL(k_row_max, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, err);
+    hipLaunchKernelGGL(k_row_sum, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats);
+    hipLaunchKernelGGL(k_row_total, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, inv_t);
+    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), 1);
+    hipLaunchKernelGGL(k_pick, dim3(ap.k), dim3(1024), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), sc.result, proposals_dev, err, 1);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+}  // namespace tsv

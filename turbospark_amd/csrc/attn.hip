@@ -1,0 +1,238 @@
+// Flash-decoding split-KV GQA attention for a verify pass on gfx950.
+//
+// Replaces the reference's per-row loop of split-KV decode dispatches
+// (crates/runtime/src/families/qwen/batched_layers.rs:409-430 over
+// crates/gpu/src/attention_decode.rs:1092-1363, tree variant :1153-1230); arithmetic contract
+// crates/compute/src/attention.rs:53-137.  Differences by design:
+//  * ALL rows of the pass (and all q heads of a GQA group) share ONE read of K and V: the
+//    (row, q-head-in-group) pairs are the 16-wide N operand of the MFMA, so the KV bytes are
+//    read once per layer instead of once per row;
+//  * the causal / tree mask over the drafted suffix is a 16-bit ancestor set per row;
+//  * S^T = K Q^T is computed with v_mfma_f32_16x16x32_f16 (K positions as the M operand), whose
+//    accumulator layout (lane: row j, positions 4*kg..4*kg+3) is exactly the B-operand layout
+//    of v_mfma_f32_16x16x16_f16, so O^T += V^T P^T needs no data movement; V is stored in the
+//    cache pre-arranged as that MFMA's A fragments.
+#include "tsv_internal.h"
+
+namespace tsv {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+int attn_chunks(int nkv) {
+    int n = 256 / nkv;
+    if (n < 1) n = 1;
+    if (n > 64) n = 64;
+    return n;
+}
+
+template <int HD, int RT>
+__global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) {
+    constexpr int KS = HD / 32;  // K steps of the score MFMA
+    constexpr int VT = HD / 16;  // output tiles along head_dim
+    constexpr int PER_LANE = RT * VT * 4 + 2 * RT;
+    __shared__ float xch[64 * PER_LANE];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 15, kg = lane >> 4;
+    const int chunk = blockIdx.x, h = blockIdx.y, rt0 = blockIdx.z * RT;
+    const VerifyParams* vp = a.vp;
+    const int M = vp->m, base = vp->base, kvlen = base + M;
+    const int nblk = (kvlen + 15) >> 4;
+    const int bpc = (nblk + a.nch - 1) / a.nch;
+    const int b0 = chunk * bpc, b1 = min(b0 + bpc, nblk);
+    const float scale = a.scale;
+
+    // query fragments and per-row ancestor sets
+    uint4 qf[RT][KS];
+    uint32_t anc[RT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const int r = (rt0 + t) * 16 + j;
+        anc[t] = 0xFFFFu;
+        if (r < R) {
+            const int mrow = r / G, g = r - mrow * G;
+            anc[t] = vp->anc[mrow];
+            const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
+#pragma unroll
+            for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
+        } else {
+#pragma unroll
+            for (int s = 0; s < KS; s++) qf[t][s] = make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    float mrun[RT], lrun[RT];
+    float4v O[RT][VT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        mrun[t] = -INFINITY;
+        lrun[t] = 0.f;
+#pragma unroll
+        for (int d = 0; d < VT; d++) O[t][d] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const _Float16* kbase = (const _Float16*)a.kc + (long)h * a.max_ctx * HD;
+    const _Float16* vbase = (const _Float16*)a.vc + (long)h * (a.max_ctx >> 4) * (HD * 16);
+    for (int b = b0 + wave; b < b1; b += 4) {
+        const int p0 = b << 4;
+        uint4 kf[KS];
+        uint2 vf[VT];
+        const _Float16* kp = kbase + (long)(p0 + j) * HD + 8 * kg;
+#pragma unroll
+        for (int s = 0; s < KS; s++) kf[s] = *(const uint4*)(kp + 32 * s);
+        const _Float16* vpn = vbase + (long)b * (HD * 16) + lane * 4;
+#pragma unroll
+        for (int d = 0; d < VT; d++) vf[d] = *(const uint2*)(vpn + d * 256);
+        const bool tail = p0 + 16 > base;
+#pragma unroll
+        for (int t = 0; t < RT; t++) {
+            float4v S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; s++)
+                S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, kf[s]),
+                                                           __builtin_bit_cast(half8, qf[t][s]), S, 0, 0, 0);
+            float sc[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                sc[i] = S[i] * scale;
+                if (tail) {
+                    const int slot = p0 + 4 * kg + i - base;
+                    const bool ok = slot < 0 || (slot < M && ((anc[t] >> slot) & 1u));
+                    if (!ok) sc[i] = -INFINITY;
+                }
+            }
+            float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            mb = fmaxf(mb, __shfl_xor(mb, 16));
+            mb = fmaxf(mb, __shfl_xor(mb, 32));
+            const float mnew = fmaxf(mrun[t], mb);
+            float alpha = 1.f;
+            half4 P = {0, 0, 0, 0};
+            if (mnew > -INFINITY) {
+                alpha = __expf(mrun[t] - mnew);
+                float ps = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float p = __expf(sc[i] - mnew);
+                    ps += p;
+                    P[i] = (_Float16)p;
+                }
+                lrun[t] = lrun[t] * alpha + ps;
+                mrun[t] = mnew;
+            }
+#pragma unroll
+            for (int d = 0; d < VT; d++) {
+                O[t][d] *= alpha;
+                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, vf[d]), P, O[t][d], 0, 0, 0);
+            }
+        }
+    }
+
+    // fold the four waves' running (m, l, O) into wave 0, one wave at a time
+    for (int w = 1; w < 4; w++) {
+        if (wave == w) {
+            float* dst = xch + lane * PER_LANE;
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                dst[2 * t] = mrun[t];
+                dst[2 * t + 1] = lrun[t];
+#pragma unroll
+                for (int d = 0; d < VT; d++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) dst[2 * RT + (t * VT + d) * 4 + i] = O[t][d][i];
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+            const float* src = xch + lane * PER_LANE;
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                const float m1 = src[2 * t], l1 = src[2 * t + 1];
+                const float mnew = fmaxf(mrun[t], m1);
+                if (mnew > -INFINITY) {
+                    const float a0 = __expf(mrun[t] - mnew), a1 = __expf(m1 - mnew);
+                    lrun[t] = lrun[t] * a0 + l1 * a1;
+#pragma unroll
+                    for (int d = 0; d < VT; d++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            O[t][d][i] = O[t][d][i] * a0 + src[2 * RT + (t * VT + d) * 4 + i] * a1;
+                    mrun[t] = mnew;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        float l = lrun[t];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        const int r = (rt0 + t) * 16 + j;
+        if (r >= R) continue;
+        const long slot = ((long)h * a.nch + chunk) * R + r;
+        if (kg == 0) {
+            a.part_ml[slot * 2] = mrun[t];
+            a.part_ml[slot * 2 + 1] = l;
+        }
+        float* o = a.part_o + slot * HD + 4 * kg;
+#pragma unroll
+        for (int d = 0; d < VT; d++) *(float4v*)(o + 16 * d) = O[t][d];
+    }
+}
+
+__device__ __forceinline__ int frag_index_a(int k, int row) {
+    const int sub = k >> 5, e = k & 31, kg = e >> 3, o = e & 7;
+    const int p = (o & 4) | ((o & 1) << 1) | ((o >> 1) & 1);
+    return ((sub * 4 + kg) * 16 + row) * 8 + p;
+}
+
+// Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
+// m* = max m_c, D = sum l_c e^{m_c-m*}, O = sum O_c e^{m_c-m*}, out = O / D) and store the row
+// as fp16 activation fragments of the output projection (K index = q_head*hd + d).
+__global__ void k_attn_combine(AttnArgs a, int G, int R) {
+    const int m = blockIdx.x, qh = blockIdx.y, d = threadIdx.x;
+    const int hd = a.hd;
+    if (d >= hd) return;
+    const int h = qh / G, g = qh - h * G, r = m * G + g;
+    float mx = -INFINITY;
+    for (int c = 0; c < a.nch; c++) mx = fmaxf(mx, a.part_ml[(((long)h * a.nch + c) * R + r) * 2]);
+    float den = 0.f, num = 0.f;
+    for (int c = 0; c < a.nch; c++) {
+        const long slot = ((long)h * a.nch + c) * R + r;
+        const float mc = a.part_ml[slot * 2];
+        if (mc == -INFINITY) continue;
+        const float w = __expf(mc - mx);
+        den += a.part_ml[slot * 2 + 1] * w;
+        num += a.part_o[slot * hd + d] * w;
+    }
+    ((_Float16*)a.xfrag)[frag_index_a(qh * hd + d, m)] = (_Float16)(num / den);
+}
+
+template <int HD>
+static int launch_hd(hipStream_t s, const AttnArgs& a, int m, int G, int R) {
+    const int trt = (R + 15) / 16;
+    if (trt <= 1) {
+        hipLaunchKernelGGL((k_attn_partial<HD, 1>), dim3(a.nch, a.nkv, 1), dim3(256), 0, s, a, G, R);
+    } else if (trt <= 2) {
+        hipLaunchKernelGGL((k_attn_partial<HD, 2>), dim3(a.nch, a.nkv, 1), dim3(256), 0, s, a, G, R);
+    } else {
+        hipLaunchKernelGGL((k_attn_partial<HD, 4>), dim3(a.nch, a.nkv, (trt + 3) / 4), dim3(256), 0, s, a, G, R);
+    }
+    TSV_HIP(hipGetLastError());
+    hipLaunchKernelGGL(k_attn_combine, dim3(m, a.nq), dim3(HD), 0, s, a, G, R);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+int launch_attention(hipStream_t s, const AttnArgs& a, int m) {
+    const int G = a.nq / a.nkv, R = m * G;
+    if (a.hd == 128) return launch_hd<128>(s, a, m, G, R);
+    if (a.hd == 64) return launch_hd<64>(s, a, m, G, R);
+    set_error("attention: head_dim must be 64 or 128");
+    return TSV_ERR_UNSUPPORTED;
+}
+
+}  // namespace tsv

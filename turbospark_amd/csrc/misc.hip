@@ -1,0 +1,239 @@
+// Small per-row kernels of the verify pass: embedding lookup, residual-add + RMSNorm,
+// q/k rotation + KV-cache store, KV row gather / read-back.
+#include "tsv_internal.h"
+
+namespace tsv {
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+
+__device__ __forceinline__ int frag_index(int k, int row) {
+    // fp16 activation fragments: [k/32][kg = (k%32)/8][16 rows][8], with the order inside each
+    // 8-slice the weight unpack produces ([0,2,1,3,4,6,5,7]).
+    const int sub = k >> 5, e = k & 31, kg = e >> 3, o = e & 7;
+    const int p = (o & 4) | ((o & 1) << 1) | ((o >> 1) & 1);
+    return ((sub * 4 + kg) * 16 + row) * 8 + p;
+}
+
+// ---------------------------------------------------------------- embedding lookup
+// One dequantized table row per fed token (crates/runtime/src/real_forward_dispatch.rs:154),
+// arithmetic of dequantize_q4_k / dequantize_q8_0.
+__global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, float* __restrict__ x,
+                        const VerifyParams* __restrict__ vp) {
+    const int m = blockIdx.x;
+    if (m >= vp->m) return;
+    const long tok = vp->feed[m];
+    for (int e = threadIdx.x; e < hidden; e += blockDim.x) {
+        float v;
+        if (dtype == TSV_Q4_K) {
+            const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 144;
+            const float d = f16_bits_to_f32(*(const uint16_t*)blk);
+            const float dmin = f16_bits_to_f32(*(const uint16_t*)(blk + 2));
+            const uint8_t* packed = blk + 4;
+            const int w = e & 255, g = w >> 6, hi = (w >> 5) & 1, l = w & 31, j = 2 * g + hi;
+            int sc, mn;
+            if (j < 4) {
+                sc = packed[j] & 63;
+                mn = packed[j + 4] & 63;
+            } else {
+                sc = (packed[j + 4] & 0xF) | ((packed[j - 4] >> 6) << 4);
+                mn = (packed[j + 4] >> 4) | ((packed[j] >> 6) << 4);
+            }
+            const uint8_t byte = blk[16 + 32 * g + l];
+            const int q = hi ? (byte >> 4) : (byte & 0xF);
+            const float dl = d * (float)sc, ml = dmin * (float)mn;
+            v = __fsub_rn(__fmul_rn(dl, (float)q), ml);
+        } else if (dtype == TSV_Q8_0) {
+            const uint8_t* blk = raw + (tok * (hidden / 32) + (e >> 5)) * 34;
+            const float d = f16_bits_to_f32(*(const uint16_t*)blk);
+            v = (float)(int8_t)blk[2 + (e & 31)] * d;
+        } else if (dtype == TSV_F16) {
+            v = f16_bits_to_f32(((const uint16_t*)raw)[tok * hidden + e]);
+        } else if (dtype == TSV_BF16) {
+            v = __uint_as_float((uint32_t)((const uint16_t*)raw)[tok * hidden + e] << 16);
+        } else {
+            v = ((const float*)raw)[tok * hidden + e];
+        }
+        x[(long)m * hidden + e] = v;
+    }
+}
+
+int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
+                 const VerifyParams* vp, int m) {
+    hipLaunchKernelGGL(k_embed, dim3(m), dim3(256), 0, s, raw, dtype, hidden, x, vp);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+// ---------------------------------------------------------------- residual add + RMSNorm
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; i++) t += red[i];
+    __syncthreads();
+    return t;
+}
+
+// x[m] += sum over split-K partials of the previous matmul (fixed order: deterministic), then
+// y = x * w / sqrt(mean x^2 + eps) (crates/compute/src/rms_norm.rs:5-14) stored as the next
+// matmul's fp16 activation fragments.  One workgroup per row.
+__global__ __launch_bounds__(256) void k_addnorm(float* __restrict__ x, const float* __restrict__ partial,
+                                                 int splits, int ldp, const float* __restrict__ w,
+                                                 float eps, int hidden, _Float16* __restrict__ xfrag) {
+    __shared__ float red[8];
+    const int m = blockIdx.x;
+    float* xr = x + (long)m * hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+        float v = xr[i];
+        for (int s = 0; s < splits; s++) v += partial[((long)s * 16 + m) * ldp + i];
+        xr[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += 256)
+        xfrag[frag_index(i, m)] = (_Float16)(xr[i] * w[i] * inv);
+}
+
+int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
+                   float eps, int hidden, uint4* xfrag, int m) {
+    hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(256), 0, s, x, partial, splits, ldp, w, eps, hidden,
+                       (_Float16*)xfrag);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+__global__ void k_f32_to_xfrag(const float* __restrict__ x, int k, _Float16* __restrict__ xfrag) {
+    const int m = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < k) xfrag[frag_index(i, m)] = (_Float16)x[(long)m * k + i];
+}
+
+int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m) {
+    hipLaunchKernelGGL(k_f32_to_xfrag, dim3((k + 255) / 256, m), dim3(256), 0, s, x, k, (_Float16*)xfrag);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+// ---------------------------------------------------------------- rope + KV store
+// One wave per (row, head): sums the split-K partials of the fused q/k/v projection, applies
+// the optional per-head RMSNorm (families/llama/state.rs:344-347) and the NeoX rotation
+// (crates/compute/src/rope.rs:208-256: pairs (i, i + hd/2), angle = position * freq_i), then
+// stores q as fp16 rows and K/V straight into the cache slot of that row
+// (families/qwen/batched_layers.rs:84-113).  V is stored in 16-position blocks laid out as
+// MFMA A-fragments: [hd/16][lane = (pos%16/4)*16 + d%16][pos%4].
+__global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
+    const int m = blockIdx.x, head = blockIdx.y;
+    const VerifyParams* vp = a.vp;
+    if (m >= vp->m) return;
+    const int hd = a.hd, half = hd >> 1, i = threadIdx.x;
+    const int kind = head < a.nq ? 0 : head < a.nq + a.nkv ? 1 : 2;
+    const int h = kind == 0 ? head : kind == 1 ? head - a.nq : head - a.nq - a.nkv;
+    const int col = head * hd;  // q heads, then k heads, then v heads: the fused projection's row order
+    float x0 = 0.f, x1 = 0.f;
+    if (i < half) {
+        for (int s = 0; s < a.splits; s++) {
+            const float* p = a.qkv + ((long)s * 16 + m) * a.ldq + col;
+            x0 += p[i];
+            x1 += p[i + half];
+        }
+    }
+    const float* nw = kind == 0 ? a.q_norm : kind == 1 ? a.k_norm : nullptr;
+    if (nw) {
+        float ss = i < half ? x0 * x0 + x1 * x1 : 0.f;
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        const float inv = 1.0f / sqrtf(ss / (float)hd + a.eps);
+        if (i < half) {
+            x0 = x0 * nw[i] * inv;
+            x1 = x1 * nw[i + half] * inv;
+        }
+    }
+    if (i >= half) return;
+    if (kind != 2) {
+        const float angle = (float)vp->pos[m] * a.freqs[i];
+        float sn, cs;
+        sincosf(angle, &sn, &cs);
+        const float r0 = x0 * cs - x1 * sn;
+        const float r1 = x0 * sn + x1 * cs;
+        x0 = r0;
+        x1 = r1;
+    }
+    const _Float16 h0 = (_Float16)x0, h1 = (_Float16)x1;
+    if (kind == 0) {
+        _Float16* q = (_Float16*)a.q16 + ((long)m * a.nq + h) * hd;
+        q[i] = h0;
+        q[i + half] = h1;
+    } else {
+        const int pos = vp->base + m;  // the cache slot of row m
+        if (kind == 1) {
+            _Float16* k = (_Float16*)a.kc + ((long)h * a.max_ctx + pos) * hd;
+            k[i] = h0;
+            k[i + half] = h1;
+        } else {
+            _Float16* v = (_Float16*)a.vc + ((long)h * (a.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
+            const int po = pos & 15, kg = po >> 2, pi = po & 3;
+            const int d0 = i, d1 = i + half;
+            v[(((d0 >> 4) * 64) + kg * 16 + (d0 & 15)) * 4 + pi] = h0;
+            v[(((d1 >> 4) * 64) + kg * 16 + (d1 & 15)) * 4 + pi] = h1;
+        }
+    }
+}
+
+int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m) {
+    hipLaunchKernelGGL(k_rope_kv, dim3(m, a.nq + 2 * a.nkv), dim3(64), 0, s, a);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+// ---------------------------------------------------------------- KV row gather / read
+__device__ __forceinline__ long v_index(int h, int pos, int d, int hd, int max_ctx) {
+    const int po = pos & 15;
+    return ((long)h * (max_ctx >> 4) + (pos >> 4)) * (hd * 16) +
+           ((((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3));
+}
+
+// Tree compaction (families/qwen/dflash_tree.rs:106-207): rows of slots path[0..n) move to
+// base..base+n.  path is strictly increasing with path[i] >= i, so walking i upward never
+// overwrites a row that is still to be read.  One workgroup per kv head, sequential over i.
+__global__ void k_kv_gather(uint16_t* kc, uint16_t* vc, int hd, int max_ctx, const int32_t* path, int n,
+                            int base) {
+    const int h = blockIdx.x, d = threadIdx.x;
+    for (int i = 0; i < n; i++) {
+        const int src = base + path[i], dst = base + i;
+        if (src == dst) continue;
+        if (d < hd) {
+            kc[((long)h * max_ctx + dst) * hd + d] = kc[((long)h * max_ctx + src) * hd + d];
+            vc[v_index(h, dst, d, hd, max_ctx)] = vc[v_index(h, src, d, hd, max_ctx)];
+        }
+    }
+}
+
+int launch_kv_gather(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx,
+                     const int32_t* path_dev, int n, int base) {
+    hipLaunchKernelGGL(k_kv_gather, dim3(nkv), dim3(128), 0, s, kc, vc, hd, max_ctx, path_dev, n, base);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+__global__ void k_kv_read(const uint16_t* kc, const uint16_t* vc, int nkv, int hd, int max_ctx, int pos0,
+                          uint16_t* k_out, uint16_t* v_out) {
+    const int p = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    if (d >= hd) return;
+    const long o = ((long)p * nkv + h) * hd + d;
+    k_out[o] = kc[((long)h * max_ctx + pos0 + p) * hd + d];
+    v_out[o] = vc[v_index(h, pos0 + p, d, hd, max_ctx)];
+}
+
+int launch_kv_read(hipStream_t s, const uint16_t* kc, const uint16_t* vc, int nkv, int hd, int max_ctx,
+                   int pos0, int n, uint16_t* k_out, uint16_t* v_out) {
+    hipLaunchKernelGGL(k_kv_read, dim3(n, nkv), dim3(128), 0, s, kc, vc, nkv, hd, max_ctx, pos0, k_out, v_out);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+}  // namespace tsv

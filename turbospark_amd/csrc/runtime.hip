@@ -1,0 +1,800 @@
+// Host runtime of libtsverify: the handle, weight upload / re-tiling, the KV arena, the launch
+// sequence of one verify pass, and the C ABI.
+//
+// The pass composes the reference's Llama-family decode graph row-wise
+// (crates/runtime/src/families/llama/mod.rs:197-316, attn.rs:152-369, dense.rs:45-120) under the
+// batched-verify contract of crates/runtime/src/families/qwen/batched.rs:92-456.  Residual
+// stream and all intermediates are fp32; fp16 appears where the engine's storage dtype is
+// fixed (KV cache, logits) and as the MFMA operand type of the matmuls.
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#include "tsv_internal.h"
+
+using namespace tsv;
+
+namespace {
+
+struct LayerW {
+    TiledW qkv, wo, gate_up, down;
+    float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    uint16_t *kc = nullptr, *vc = nullptr;
+};
+
+int dtype_fmt(int dtype) { return dtype == TSV_Q4_K ? FMT_Q4K : dtype == TSV_Q8_0 ? FMT_Q80 : -1; }
+
+}  // namespace
+
+struct tsv_ctx {
+    int n_layers = 0, hidden = 0, nq = 0, nkv = 0, hd = 0, ffn = 0, vocab = 0, max_context = 0, ctx_alloc = 0;
+    float eps = 0, attn_scale = 0;
+    hipStream_t stream = nullptr;
+    std::vector<LayerW> layers;
+    TiledW head;
+    uint8_t* embed_raw = nullptr;
+    int embed_dtype = 0;
+    float* final_norm = nullptr;
+    float* freqs = nullptr;
+    // scratch
+    float* x = nullptr;
+    uint4 *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
+    float* partial = nullptr;
+    size_t partial_floats = 0;
+    uint16_t* q16 = nullptr;
+    float *part_o = nullptr, *part_ml = nullptr;
+    int nch = 0;
+    uint16_t* logits = nullptr;       // [16][vocab] fp16, device
+    uint16_t* draft_stage = nullptr;  // [16][vocab] fp16, device
+    VerifyParams *vp_dev = nullptr, *vp_host = nullptr;
+    AcceptParams *ap_dev = nullptr, *ap_host = nullptr;
+    AcceptResult* res_host = nullptr;
+    int32_t *tok_dev = nullptr, *tok_host = nullptr;
+    AcceptScratch sc{};
+    std::vector<void*> allocs;
+    int64_t position = 0;
+    int last_m = 0;
+    int64_t last_base = -1;
+};
+
+namespace {
+
+template <class T>
+int dev_alloc(tsv_ctx* c, T** p, size_t bytes, bool zero = false) {
+    void* q = nullptr;
+    TSV_HIP(hipMalloc(&q, bytes ? bytes : 16));
+    c->allocs.push_back(q);
+    if (zero) TSV_HIP(hipMemsetAsync(q, 0, bytes, c->stream));
+    *p = (T*)q;
+    return TSV_OK;
+}
+
+float to_f32(const tsv_tensor& t, int64_t i) {
+    switch (t.dtype) {
+        case TSV_F32: return ((const float*)t.data)[i];
+        case TSV_F16: {
+            _Float16 h;
+            std::memcpy(&h, (const uint16_t*)t.data + i, 2);
+            return (float)h;
+        }
+        case TSV_BF16: {
+            uint32_t u = (uint32_t)((const uint16_t*)t.data)[i] << 16;
+            float f;
+            std::memcpy(&f, &u, 4);
+            return f;
+        }
+    }
+    return 0.f;
+}
+
+int upload_vector(tsv_ctx* c, const tsv_tensor& t, int64_t n, float** out, const char* what) {
+    if (!t.data || t.rows * t.cols != n || (t.dtype != TSV_F32 && t.dtype != TSV_F16 && t.dtype != TSV_BF16)) {
+        set_error(std::string(what) + ": expected an f32/f16/bf16 vector of the model's width");
+        return TSV_ERR_INVALID;
+    }
+    std::vector<float> h((size_t)n);
+    for (int64_t i = 0; i < n; i++) h[i] = to_f32(t, i);
+    int rc = dev_alloc(c, out, (size_t)n * 4);
+    if (rc) return rc;
+    TSV_HIP(hipMemcpy(*out, h.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    return TSV_OK;
+}
+
+struct Stager {
+    uint8_t* dev = nullptr;
+    size_t cap = 0;
+};
+
+int stage_raw(tsv_ctx* c, Stager& st, const tsv_tensor& t) {
+    const int64_t rb = row_bytes(t.dtype, t.cols);
+    const size_t bytes = (size_t)(rb * t.rows);
+    if (bytes > st.cap) {
+        if (st.dev) TSV_HIP(hipFree(st.dev));
+        st.dev = nullptr;
+        TSV_HIP(hipMalloc((void**)&st.dev, bytes));
+        st.cap = bytes;
+    }
+    TSV_HIP(hipMemcpyAsync(st.dev, t.data, bytes, hipMemcpyHostToDevice, c->stream));
+    return TSV_OK;
+}
+
+int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* what) {
+    const int fmt = dtype_fmt(t.dtype);
+    if (!t.data || t.rows != rows || t.cols != cols) {
+        set_error(std::string(what) + ": shape does not match the model description");
+        return TSV_ERR_INVALID;
+    }
+    if (fmt < 0) {
+        set_error(std::string(what) + ": matmul weights must be Q4_K or Q8_0 in this build");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    if (cols % fmt_chunk_elems(fmt) || rows % 16) {
+        set_error(std::string(what) + ": K must be whole 256 (Q4_K) / 128 (Q8_0) chunks and rows a multiple of 16");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    return TSV_OK;
+}
+
+// Allocates a tiled matrix of `total_rows` rows and re-tiles `parts` into it: concatenated
+// (interleave == false) or with their 16-row tiles alternating (gate / up).
+int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_parts, bool interleave, TiledW* out) {
+    const int fmt = dtype_fmt(parts[0]->dtype);
+    int64_t total_rows = 0;
+    for (int i = 0; i < n_parts; i++) {
+        if (dtype_fmt(parts[i]->dtype) != fmt || parts[i]->cols != parts[0]->cols) {
+            set_error("fused projection parts must share dtype and K");
+            return TSV_ERR_INVALID;
+        }
+        total_rows += parts[i]->rows;
+    }
+    out->fmt = fmt;
+    out->k = (int)parts[0]->cols;
+    out->kchunks = out->k / fmt_chunk_elems(fmt);
+    out->n_rows = (int)total_rows;
+    out->n_tiles = (int)((total_rows + 15) / 16);
+    out->bytes = (size_t)out->n_tiles * out->kchunks * fmt_tile_bytes(fmt);
+    int rc = dev_alloc(c, &out->tiles, out->bytes);
+    if (rc) return rc;
+    int tile_off = 0;
+    for (int i = 0; i < n_parts; i++) {
+        if ((rc = stage_raw(c, st, *parts[i]))) return rc;
+        rc = launch_repack(c->stream, fmt, st.dev, (int)parts[i]->rows, out->k, out->tiles, out->kchunks,
+                           interleave ? n_parts : 1, interleave ? i : tile_off);
+        if (rc) return rc;
+        TSV_HIP(hipStreamSynchronize(c->stream));  // the stager is reused by the next part
+        tile_off += (int)(parts[i]->rows / 16);
+    }
+    return TSV_OK;
+}
+
+int splits_for(const TiledW& w, int m, int epi) { return epi == EPI_PARTIAL ? gemm_default_splits(w, m) : 1; }
+
+size_t partial_need(const TiledW& w) {
+    size_t need = 0;
+    for (int m : {4, 8, 16}) {
+        size_t s = (size_t)splits_for(w, m, EPI_PARTIAL) * 16 * (size_t)w.n_tiles * 16;
+        if (s > need) need = s;
+    }
+    return need;
+}
+
+int is_device_pointer(const void* p) {
+    hipPointerAttribute_t a;
+    hipError_t e = hipPointerGetAttributes(&a, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return a.type == hipMemoryTypeDevice;
+}
+
+int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
+    if (!(s.temperature >= 0.0) || !std::isfinite(s.temperature)) {
+        set_error("temperature must be finite and non-negative");
+        return TSV_ERR_INVALID;
+    }
+    if (s.temperature == 0.0) return TSV_OK;
+    if (!s.has_seed) {
+        set_error("a sampled round needs an explicit seed");
+        return TSV_ERR_INVALID;
+    }
+    if (sampled_supported_only &&
+        (s.top_k != 0 || s.has_top_p || s.has_min_p || s.repetition_penalty != 1.0 || s.presence_penalty != 0.0 ||
+         s.frequency_penalty != 0.0)) {
+        set_error("device acceptance: top-k / top-p / min-p / penalties are not built; use temperature only");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    return TSV_OK;
+}
+
+// One verify pass: enqueue everything on the handle's stream; no synchronisation.
+int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m, int64_t base) {
+    // batched.rs:106-185 refusals
+    if (!feed || m < 1) {
+        set_error("verify: empty feed");
+        return TSV_ERR_INVALID;
+    }
+    if (m > TSV_MAX_ROWS) {
+        set_error("verify: more rows than one pass takes (16)");
+        return TSV_ERR_INVALID;
+    }
+    if (base != c->position) {
+        set_error("verify: start position does not match the KV cursor");
+        return TSV_ERR_INVALID;
+    }
+    if (base + m > c->max_context) {
+        set_error("verify: block would write past the KV capacity");
+        return TSV_ERR_INVALID;
+    }
+    VerifyParams vp;
+    std::memset(&vp, 0, sizeof vp);
+    vp.m = m;
+    vp.base = (int32_t)base;
+    int depth[TSV_MAX_ROWS] = {0};
+    for (int i = 0; i < m; i++) {
+        if (feed[i] < 0 || feed[i] >= c->vocab) {
+            set_error("verify: token id outside the vocabulary");
+            return TSV_ERR_INVALID;
+        }
+        vp.feed[i] = feed[i];
+        if (parent) {
+            if (i == 0 ? parent[0] != -1 : (parent[i] < 0 || parent[i] >= i)) {
+                set_error("verify_tree: parent[0] must be -1 and parent[s] in [0, s)");
+                return TSV_ERR_INVALID;
+            }
+            depth[i] = i == 0 ? 0 : depth[parent[i]] + 1;
+            vp.anc[i] = (i == 0 ? 0u : vp.anc[parent[i]]) | (1u << i);
+        } else {
+            depth[i] = i;
+            vp.anc[i] = (2u << i) - 1u;
+        }
+        vp.pos[i] = (int32_t)base + depth[i];
+    }
+    hipStream_t s = c->stream;
+    // the pinned staging copy must not be rewritten while an earlier copy is still in flight
+    TSV_HIP(hipStreamSynchronize(s));
+    *c->vp_host = vp;
+    TSV_HIP(hipMemcpyAsync(c->vp_dev, c->vp_host, sizeof vp, hipMemcpyHostToDevice, s));
+
+    int rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m);
+    if (rc) return rc;
+    int prev_splits = 0;
+    const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
+    for (int l = 0; l < c->n_layers; l++) {
+        LayerW& L = c->layers[l];
+        if ((rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m)))
+            return rc;
+        int sp = splits_for(L.qkv, m, EPI_PARTIAL);
+        if ((rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n))) return rc;
+        RopeKvArgs ra;
+        ra.qkv = c->partial;
+        ra.splits = sp;
+        ra.ldq = qkv_n;
+        ra.freqs = c->freqs;
+        ra.q_norm = L.q_norm;
+        ra.k_norm = L.k_norm;
+        ra.eps = c->eps;
+        ra.q16 = c->q16;
+        ra.kc = L.kc;
+        ra.vc = L.vc;
+        ra.nq = c->nq;
+        ra.nkv = c->nkv;
+        ra.hd = c->hd;
+        ra.max_ctx = c->ctx_alloc;
+        ra.vp = c->vp_dev;
+        if ((rc = launch_rope_kv(s, ra, m))) return rc;
+        AttnArgs aa;
+        aa.q16 = c->q16;
+        aa.kc = L.kc;
+        aa.vc = L.vc;
+        aa.part_o = c->part_o;
+        aa.part_ml = c->part_ml;
+        aa.xfrag = c->xf_b;
+        aa.nq = c->nq;
+        aa.nkv = c->nkv;
+        aa.hd = c->hd;
+        aa.max_ctx = c->ctx_alloc;
+        aa.nch = c->nch;
+        aa.scale = c->attn_scale;
+        aa.vp = c->vp_dev;
+        if ((rc = launch_attention(s, aa, m))) return rc;
+        sp = splits_for(L.wo, m, EPI_PARTIAL);
+        if ((rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden))) return rc;
+        if ((rc = launch_addnorm(s, c->x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m))) return rc;
+        if ((rc = launch_gemm(s, L.gate_up, c->xf_a, c->xf_c, c->vp_dev, m, 1, EPI_SILU, 0, 0))) return rc;
+        sp = splits_for(L.down, m, EPI_PARTIAL);
+        if ((rc = launch_gemm(s, L.down, c->xf_c, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden))) return rc;
+        prev_splits = sp;
+    }
+    if ((rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m)))
+        return rc;
+    if ((rc = launch_gemm(s, c->head, c->xf_a, c->logits, c->vp_dev, m, 1, EPI_LOGITS, c->vocab, c->vocab))) return rc;
+    c->position = base + m;
+    c->last_m = m;
+    c->last_base = base;
+    return TSV_OK;
+}
+
+int finish_verify(tsv_ctx* c, int m, uint16_t* logits_out) {
+    if (logits_out) {
+        TSV_HIP(hipMemcpyAsync(logits_out, c->logits, (size_t)m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
+        TSV_HIP(hipStreamSynchronize(c->stream));
+    }
+    return TSV_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
+    if (!d || !out || !d->layers) {
+        set_error("open: null argument");
+        return TSV_ERR_INVALID;
+    }
+    if (d->head_dim != 64 && d->head_dim != 128) {
+        set_error("open: head_dim must be 64 or 128");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    if (d->n_q_heads % d->n_kv_heads || d->n_q_heads / d->n_kv_heads > 8 || d->hidden % 32 || d->ffn % 32) {
+        set_error("open: unsupported head grouping or widths");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    tsv_ctx* c = new tsv_ctx();
+    auto fail = [&](int rc) {
+        tsv_close(c);
+        return rc;
+    };
+    c->n_layers = d->n_layers;
+    c->hidden = d->hidden;
+    c->nq = d->n_q_heads;
+    c->nkv = d->n_kv_heads;
+    c->hd = d->head_dim;
+    c->ffn = d->ffn;
+    c->vocab = d->vocab;
+    c->max_context = d->max_context;
+    c->ctx_alloc = ((d->max_context + 15) / 16) * 16;
+    c->eps = d->rms_eps;
+    c->attn_scale = d->attn_scale > 0.f ? d->attn_scale : 1.0f / std::sqrt((float)d->head_dim);
+    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
+        set_error("open: cannot create a HIP stream (no GPU?)");
+        delete c;
+        return TSV_ERR_DEVICE;
+    }
+    int rc;
+    Stager st;
+    const int qd = c->nq * c->hd, kvd = c->nkv * c->hd;
+    c->layers.resize(c->n_layers);
+    size_t pneed = 0;
+    for (int l = 0; l < c->n_layers; l++) {
+        const tsv_layer& s = d->layers[l];
+        LayerW& L = c->layers[l];
+        if ((rc = check_matrix(s.wq, qd, c->hidden, "wq")) || (rc = check_matrix(s.wk, kvd, c->hidden, "wk")) ||
+            (rc = check_matrix(s.wv, kvd, c->hidden, "wv")) || (rc = check_matrix(s.wo, c->hidden, qd, "wo")) ||
+            (rc = check_matrix(s.w_gate, c->ffn, c->hidden, "w_gate")) ||
+            (rc = check_matrix(s.w_up, c->ffn, c->hidden, "w_up")) ||
+            (rc = check_matrix(s.w_down, c->hidden, c->ffn, "w_down")))
+            return fail(rc);
+        const tsv_tensor* qkv[3] = {&s.wq, &s.wk, &s.wv};
+        const tsv_tensor* gu[2] = {&s.w_gate, &s.w_up};
+        const tsv_tensor* wo[1] = {&s.wo};
+        const tsv_tensor* dn[1] = {&s.w_down};
+        if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv)) || (rc = make_tiled(c, st, wo, 1, false, &L.wo)) ||
+            (rc = make_tiled(c, st, gu, 2, true, &L.gate_up)) || (rc = make_tiled(c, st, dn, 1, false, &L.down)))
+            return fail(rc);
+        if ((rc = upload_vector(c, s.attn_norm, c->hidden, &L.attn_norm, "attn_norm")) ||
+            (rc = upload_vector(c, s.ffn_norm, c->hidden, &L.ffn_norm, "ffn_norm")))
+            return fail(rc);
+        if (s.q_norm.data) {
+            if ((rc = upload_vector(c, s.q_norm, c->hd, &L.q_norm, "q_norm")) ||
+                (rc = upload_vector(c, s.k_norm, c->hd, &L.k_norm, "k_norm")))
+                return fail(rc);
+        }
+        const size_t kvb = (size_t)c->nkv * c->ctx_alloc * c->hd * 2;
+        if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) return fail(rc);
+        pneed = std::max(pneed, std::max(partial_need(L.qkv), std::max(partial_need(L.wo), partial_need(L.down))));
+    }
+    // embedding table (raw GGUF rows for the lookup) and output head (tiled)
+    const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
+    if (!d->embed.data || d->embed.rows != c->vocab || d->embed.cols != c->hidden || erb < 0) {
+        set_error("open: embedding table shape / dtype");
+        return fail(TSV_ERR_INVALID);
+    }
+    c->embed_dtype = d->embed.dtype;
+    if ((rc = dev_alloc(c, &c->embed_raw, (size_t)(erb * c->vocab)))) return fail(rc);
+    if (hipMemcpy(c->embed_raw, d->embed.data, (size_t)(erb * c->vocab), hipMemcpyHostToDevice) != hipSuccess) {
+        set_error("open: embedding upload failed");
+        return fail(TSV_ERR_DEVICE);
+    }
+    {
+        tsv_tensor head = d->lm_head.data ? d->lm_head : d->embed;
+        // the head's row count need not be a multiple of 16: the last tile is zero padded
+        const int fmt = dtype_fmt(head.dtype);
+        if (head.rows != c->vocab || head.cols != c->hidden || fmt < 0 || c->hidden % fmt_chunk_elems(fmt)) {
+            set_error("open: output head must be a Q4_K / Q8_0 vocab x hidden matrix");
+            return fail(TSV_ERR_UNSUPPORTED);
+        }
+        const tsv_tensor* hp[1] = {&head};
+        if ((rc = make_tiled(c, st, hp, 1, false, &c->head))) return fail(rc);
+    }
+    if (st.dev) (void)hipFree(st.dev);
+    if ((rc = upload_vector(c, d->final_norm, c->hidden, &c->final_norm, "final_norm"))) return fail(rc);
+    {
+        // rope.rs:208-256 (scalar theta: exp(-(2i/hd) * ln theta)) or rope.rs:447-460 (per-pair divisors)
+        std::vector<float> f((size_t)c->hd / 2);
+        for (int i = 0; i < c->hd / 2; i++) {
+            if (d->rope_factors)
+                f[i] = std::pow(d->rope_theta, -((float)(2 * i)) / (float)c->hd) / d->rope_factors[i];
+            else
+                f[i] = std::exp((-((float)(2 * i)) / (float)c->hd) * std::log(d->rope_theta));
+        }
+        if ((rc = dev_alloc(c, &c->freqs, f.size() * 4))) return fail(rc);
+        if (hipMemcpy(c->freqs, f.data(), f.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail(TSV_ERR_DEVICE);
+    }
+    // scratch
+    const int kmax = std::max(std::max(c->hidden, qd), c->ffn);
+    const size_t xfb = (size_t)kmax / 32 * 4 * 16 * 16;
+    c->nch = attn_chunks(c->nkv);
+    const size_t rows_max = (size_t)TSV_MAX_ROWS * (c->nq / c->nkv);
+    c->partial_floats = pneed;
+    if ((rc = dev_alloc(c, &c->x, (size_t)16 * c->hidden * 4, true)) || (rc = dev_alloc(c, &c->xf_a, xfb, true)) ||
+        (rc = dev_alloc(c, &c->xf_b, xfb, true)) || (rc = dev_alloc(c, &c->xf_c, xfb, true)) ||
+        (rc = dev_alloc(c, &c->partial, pneed * 4, true)) || (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
+        (rc = dev_alloc(c, &c->part_o, (size_t)c->nkv * c->nch * rows_max * c->hd * 4, true)) ||
+        (rc = dev_alloc(c, &c->part_ml, (size_t)c->nkv * c->nch * rows_max * 2 * 4, true)) ||
+        (rc = dev_alloc(c, &c->logits, (size_t)16 * c->vocab * 2, true)) ||
+        (rc = dev_alloc(c, &c->draft_stage, (size_t)16 * c->vocab * 2, true)) ||
+        (rc = dev_alloc(c, &c->vp_dev, sizeof(VerifyParams), true)) ||
+        (rc = dev_alloc(c, &c->ap_dev, sizeof(AcceptParams), true)) ||
+        (rc = dev_alloc(c, &c->tok_dev, 64 * 4, true)) ||
+        (rc = dev_alloc(c, &c->sc.stats, accept_stats_doubles() * 8, true)) ||
+        (rc = dev_alloc(c, &c->sc.work, (size_t)16 * 2 * c->vocab * 8, true)) ||
+        (rc = dev_alloc(c, &c->sc.hist, (size_t)16 * 2 * 65536 * 8, true)) ||
+        (rc = dev_alloc(c, &c->sc.counters, 64 * 4, true)) ||
+        (rc = dev_alloc(c, &c->sc.result, sizeof(AcceptResult), true)))
+        return fail(rc);
+    if (hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
+        hipHostMalloc((void**)&c->ap_host, sizeof(AcceptParams)) != hipSuccess ||
+        hipHostMalloc((void**)&c->res_host, sizeof(AcceptResult)) != hipSuccess ||
+        hipHostMalloc((void**)&c->tok_host, 64 * 4) != hipSuccess) {
+        set_error("open: pinned host allocation failed");
+        return fail(TSV_ERR_DEVICE);
+    }
+    if (hipStreamSynchronize(c->stream) != hipSuccess) {
+        set_error("open: device initialisation failed");
+        return fail(TSV_ERR_DEVICE);
+    }
+    *out = c;
+    return TSV_OK;
+}
+
+extern "C" void tsv_close(tsv_ctx* c) {
+    if (!c) return;
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    for (void* p : c->allocs) (void)hipFree(p);
+    if (c->vp_host) (void)hipHostFree(c->vp_host);
+    if (c->ap_host) (void)hipHostFree(c->ap_host);
+    if (c->res_host) (void)hipHostFree(c->res_host);
+    if (c->tok_host) (void)hipHostFree(c->tok_host);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+extern "C" void* tsv_stream(tsv_ctx* c) { return c ? (void*)c->stream : nullptr; }
+
+extern "C" int32_t tsv_reset(tsv_ctx* c) {
+    c->position = 0;
+    c->last_m = 0;
+    return TSV_OK;
+}
+
+extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c->position; }
+
+extern "C" int32_t tsv_verify(tsv_ctx* c, const int32_t* feed, int32_t m, int64_t base, uint16_t* logits) {
+    int rc = enqueue_verify(c, feed, nullptr, m, base);
+    return rc ? rc : finish_verify(c, m, logits);
+}
+
+extern "C" int32_t tsv_verify_tree(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int32_t m, int64_t base,
+                                   uint16_t* logits) {
+    if (!parent) {
+        set_error("verify_tree: null parent array");
+        return TSV_ERR_INVALID;
+    }
+    int rc = enqueue_verify(c, feed, parent, m, base);
+    return rc ? rc : finish_verify(c, m, logits);
+}
+
+extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint16_t* logits) {
+    return tsv_verify(c, &token, 1, position, logits);
+}
+
+extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
+    if (n < 1) {
+        set_error("prefill: empty token list");
+        return TSV_ERR_INVALID;
+    }
+    for (int64_t i = 0; i < n; i += TSV_MAX_ROWS) {
+        const int m = (int)std::min<int64_t>(TSV_MAX_ROWS, n - i);
+        int rc = enqueue_verify(c, ids + i, nullptr, m, pos0 + i);
+        if (rc) return rc;
+        if (i + m >= n && logits) {
+            TSV_HIP(hipMemcpyAsync(logits, c->logits + (size_t)(m - 1) * c->vocab, (size_t)c->vocab * 2,
+                                   hipMemcpyDeviceToHost, c->stream));
+        }
+    }
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {
+    out->position = c->position;
+    return TSV_OK;
+}
+
+// real_forward_rollback.rs:153-209 for a target without recurrent state: kv.rewind_by, a
+// cursor move (kv_cache_rewind.rs:46-55); rows past the cursor become unreachable.
+extern "C" int32_t tsv_rollback(tsv_ctx* c, const tsv_point* p) {
+    if (p->position < 0 || p->position > c->position) {
+        set_error("rollback: point is ahead of the KV cursor");
+        return TSV_ERR_INVALID;
+    }
+    c->position = p->position;
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_rollback_retaining(tsv_ctx* c, const tsv_point* p, int32_t keep_rows) {
+    if (keep_rows < 0 || p->position + keep_rows > c->position) {
+        set_error("rollback_retaining: keep_rows exceeds the rows the last verify wrote");
+        return TSV_ERR_INVALID;
+    }
+    c->position = p->position + keep_rows;
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_commit_pending(tsv_ctx*, int32_t) { return TSV_OK; }
+extern "C" int32_t tsv_discard_pending(tsv_ctx*) { return TSV_OK; }
+
+extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* path, int32_t n) {
+    if (n < 1 || n > TSV_MAX_ROWS || path[0] != 0) {
+        set_error("compact_tree: path must start at slot 0 and hold 1..16 slots");
+        return TSV_ERR_INVALID;
+    }
+    for (int i = 1; i < n; i++)
+        if (path[i] <= path[i - 1] || path[i] >= TSV_MAX_ROWS) {
+            set_error("compact_tree: path must be strictly increasing");
+            return TSV_ERR_INVALID;
+        }
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
+    TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
+    for (auto& L : c->layers) {
+        int rc = launch_kv_gather(c->stream, L.kc, L.vc, c->nkv, c->hd, c->ctx_alloc, c->tok_dev + 32, n, (int)base);
+        if (rc) return rc;
+    }
+    return TSV_OK;
+}
+
+namespace {
+
+int fill_accept(tsv_ctx* c, const tsv_round* r, AcceptParams* ap) {
+    std::memset(ap, 0, sizeof *ap);
+    ap->m = r->m;
+    ap->k = r->m - 1;
+    ap->vocab = c->vocab;
+    ap->tree = r->parent != nullptr;
+    ap->sampled = r->shaping.temperature != 0.0;
+    if (r->n_stop < 0 || r->n_stop > 16) {
+        set_error("accept: at most 16 stop tokens");
+        return TSV_ERR_INVALID;
+    }
+    ap->n_stop = r->n_stop;
+    for (int i = 0; i < r->m; i++) {
+        ap->feed[i] = r->feed[i];
+        ap->parent[i] = r->parent ? r->parent[i] : i - 1;
+    }
+    for (int i = 0; i < r->n_stop; i++) ap->stop_tokens[i] = r->stop_tokens[i];
+    ap->temperature = r->shaping.temperature;
+    ap->seed = r->shaping.seed;
+    ap->draw_step = r->draw_step;
+    ap->generated = r->generated;
+    ap->max_new_tokens = r->max_new_tokens;
+    return TSV_OK;
+}
+
+int stage_draft(tsv_ctx* c, const uint16_t* draft, int rows, const uint16_t** dev) {
+    if (is_device_pointer(draft)) {
+        *dev = draft;
+        return TSV_OK;
+    }
+    TSV_HIP(hipMemcpyAsync(c->draft_stage, draft, (size_t)rows * c->vocab * 2, hipMemcpyHostToDevice, c->stream));
+    *dev = c->draft_stage;
+    return TSV_OK;
+}
+
+int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
+    int rc = check_shaping(r->shaping, true);
+    if (rc) return rc;
+    if (r->m != c->last_m || r->base != c->last_base) {
+        set_error("accept: the round does not describe the last verify pass");
+        return TSV_ERR_INVALID;
+    }
+    const bool sampled = r->shaping.temperature != 0.0;
+    const uint16_t* draft = nullptr;
+    if (sampled) {
+        if (!r->draft_logits) {
+            set_error("accept: a sampled round needs the drafter's logits");
+            return TSV_ERR_INVALID;
+        }
+        if ((rc = stage_draft(c, r->draft_logits, r->parent ? r->m : r->m - 1, &draft))) return rc;
+    }
+    TSV_HIP(hipStreamSynchronize(c->stream));  // pinned parameter block is about to be rewritten
+    if ((rc = fill_accept(c, r, c->ap_host))) return rc;
+    TSV_HIP(hipMemcpyAsync(c->ap_dev, c->ap_host, sizeof(AcceptParams), hipMemcpyHostToDevice, c->stream));
+    if ((rc = launch_accept(c->stream, c->logits, draft, c->ap_dev, *c->ap_host, c->sc))) return rc;
+    TSV_HIP(hipMemcpyAsync(c->res_host, c->sc.result, sizeof(AcceptResult), hipMemcpyDeviceToHost, c->stream));
+    if (r->logits_out)
+        TSV_HIP(hipMemcpyAsync(r->logits_out, c->logits, (size_t)r->m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    const AcceptResult& a = *c->res_host;
+    if (a.error) {
+        set_error("accept: score vector must not contain a non-finite entry");
+        return TSV_ERR_INVALID;
+    }
+    std::memset(out, 0, sizeof *out);
+    out->accepted = a.accepted;
+    out->committed = a.committed;
+    out->next = a.next;
+    out->stopped = a.stopped;
+    out->draw_step = a.draw_step;
+    out->path_len = a.path_len;
+    for (int i = 0; i < a.path_len; i++) out->path[i] = a.path[i];
+    out->min_margin = a.min_margin;
+    // KV truncation.  Rows base..base+committed hold the confirmed token and every committed
+    // proposal; everything after becomes unreachable (speculative.rs:791-814).
+    const int keep = a.committed + 1;
+    if (r->parent && keep > 1) {
+        uint32_t path[TSV_MAX_ROWS + 1];
+        for (int i = 0; i < keep; i++) path[i] = (uint32_t)a.path[i];
+        if ((rc = tsv_compact_tree(c, r->base, path, keep))) return rc;
+    }
+    c->position = r->base + keep;
+    out->kv_position = c->position;
+    return TSV_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t tsv_accept(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
+    if (!c || !r || !out || !r->feed) {
+        set_error("accept: null argument");
+        return TSV_ERR_INVALID;
+    }
+    return accept_impl(c, r, out);
+}
+
+extern "C" int32_t tsv_verify_accept(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
+    if (!c || !r || !out || !r->feed) {
+        set_error("verify_accept: null argument");
+        return TSV_ERR_INVALID;
+    }
+    int rc = check_shaping(r->shaping, true);
+    if (rc) return rc;
+    if ((rc = enqueue_verify(c, r->feed, r->parent, r->m, r->base))) return rc;
+    return accept_impl(c, r, out);
+}
+
+extern "C" int32_t tsv_draft_chain(tsv_ctx* c, const uint16_t* draft_logits, int32_t k, const tsv_shaping* sh,
+                                   uint64_t* draw_step, int32_t* proposals) {
+    if (!c || !draft_logits || !sh || !draw_step || !proposals || k < 1 || k > TSV_MAX_ROWS - 1) {
+        set_error("draft_chain: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    int rc = check_shaping(*sh, true);
+    if (rc) return rc;
+    const uint16_t* draft = nullptr;
+    if ((rc = stage_draft(c, draft_logits, k, &draft))) return rc;
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    AcceptParams* ap = c->ap_host;
+    std::memset(ap, 0, sizeof *ap);
+    ap->m = 0;
+    ap->k = k;
+    ap->vocab = c->vocab;
+    ap->sampled = sh->temperature != 0.0;
+    ap->temperature = sh->temperature;
+    ap->seed = sh->seed;
+    ap->draw_step = *draw_step;
+    TSV_HIP(hipMemcpyAsync(c->ap_dev, ap, sizeof *ap, hipMemcpyHostToDevice, c->stream));
+    if ((rc = launch_draft_chain(c->stream, draft, c->ap_dev, *ap, c->sc, c->tok_dev))) return rc;
+    TSV_HIP(hipMemcpyAsync(c->tok_host, c->tok_dev, (size_t)k * 4, hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipMemcpyAsync(c->res_host, c->sc.result, sizeof(AcceptResult), hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    if (c->res_host->error) {
+        set_error("draft_chain: score vector must not contain a non-finite entry");
+        return TSV_ERR_INVALID;
+    }
+    for (int i = 0; i < k; i++) proposals[i] = c->tok_host[i];
+    if (ap->sampled) *draw_step += (uint64_t)k + 1;  // k draws + the row-only step (speculative.rs:618-624)
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v) {
+    if (layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
+        set_error("read_kv: range outside the cache");
+        return TSV_ERR_INVALID;
+    }
+    const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
+    uint16_t *kd = nullptr, *vd = nullptr;
+    TSV_HIP(hipMalloc((void**)&kd, bytes));
+    TSV_HIP(hipMalloc((void**)&vd, bytes));
+    int rc = launch_kv_read(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->ctx_alloc,
+                            (int)pos0, (int)n, kd, vd);
+    if (!rc) {
+        hipError_t e1 = hipMemcpyAsync(k, kd, bytes, hipMemcpyDeviceToHost, c->stream);
+        hipError_t e2 = hipMemcpyAsync(v, vd, bytes, hipMemcpyDeviceToHost, c->stream);
+        hipError_t e3 = hipStreamSynchronize(c->stream);
+        if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) {
+            set_error("read_kv: copy failed");
+            rc = TSV_ERR_DEVICE;
+        }
+    }
+    (void)hipFree(kd);
+    (void)hipFree(vd);
+    return rc;
+}
+
+extern "C" int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits) {
+    if (!w || !x || !y || m < 1 || m > TSV_MAX_ROWS) {
+        set_error("matmul: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    int rc = check_matrix(*w, w->rows, w->cols, "matmul weight");
+    if (rc) return rc;
+    tsv_ctx tmp;
+    tsv_ctx* c = &tmp;
+    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    Stager st;
+    TiledW tw;
+    const tsv_tensor* parts[1] = {w};
+    VerifyParams vp;
+    std::memset(&vp, 0, sizeof vp);
+    vp.m = m;
+    float *xd = nullptr, *pd = nullptr;
+    uint4* xf = nullptr;
+    VerifyParams* vpd = nullptr;
+    const int k = (int)w->cols, n = (int)w->rows;
+    std::vector<float> part;
+    int sp = 1;
+    rc = make_tiled(c, st, parts, 1, false, &tw);
+    if (!rc) {
+        sp = splits > 0 ? std::min(splits, tw.kchunks) : gemm_default_splits(tw, m);
+        const int kslice = (tw.kchunks + sp - 1) / sp;
+        sp = (tw.kchunks + kslice - 1) / kslice;
+    }
+    if (!rc) rc = dev_alloc(c, &xd, (size_t)m * k * 4);
+    if (!rc) rc = dev_alloc(c, &xf, (size_t)k / 32 * 4 * 16 * 16, true);
+    if (!rc) rc = dev_alloc(c, &pd, (size_t)sp * 16 * n * 4, true);
+    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
+    if (!rc && hipMemcpyAsync(xd, x, (size_t)m * k * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess) rc = TSV_ERR_DEVICE;
+    if (!rc && hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess) rc = TSV_ERR_DEVICE;
+    if (!rc) rc = launch_f32_to_xfrag(c->stream, xd, k, xf, m);
+    if (!rc) rc = launch_gemm(c->stream, tw, xf, pd, vpd, m, sp, EPI_PARTIAL, n, n);
+    if (!rc) {
+        part.resize((size_t)sp * 16 * n);
+        if (hipMemcpyAsync(part.data(), pd, part.size() * 4, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+            hipStreamSynchronize(c->stream) != hipSuccess) {
+            set_error("matmul: device execution failed");
+            rc = TSV_ERR_DEVICE;
+        }
+    }
+    if (!rc)
+        for (int b = 0; b < m; b++)
+            for (int j = 0; j < n; j++) {
+                float acc = 0.f;
+                for (int s = 0; s < sp; s++) acc += part[((size_t)s * 16 + b) * n + j];
+                y[(size_t)b * n + j] = acc;
+            }
+    if (st.dev) (void)hipFree(st.dev);
+    (void)hipStreamSynchronize(c->stream);
+    for (void* p : c->allocs) (void)hipFree(p);
+    (void)hipStreamDestroy(c->stream);
+    return rc;
+}

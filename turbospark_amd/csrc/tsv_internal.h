@@ -1,0 +1,156 @@
+// Internal declarations shared by the HIP translation units of libtsverify.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/tsverify.h"
+
+namespace tsv {
+
+void set_error(const std::string& s);
+const std::string& get_error();
+
+#define TSV_HIP(call)                                                                       \
+    do {                                                                                    \
+        hipError_t e_ = (call);                                                             \
+        if (e_ != hipSuccess) {                                                             \
+            tsv::set_error(std::string(#call) + ": " + hipGetErrorString(e_));              \
+            return TSV_ERR_DEVICE;                                                          \
+        }                                                                                   \
+    } while (0)
+
+// ---------------------------------------------------------------------------------------
+// Device weight layout ("row tiles").  A matrix W[N][K] is cut into tiles of 16 output rows
+// by one K-chunk (256 elements for Q4_K, 128 for Q8_0); tiles are stored [row tile][chunk]
+// so a wave streaming along K for its 16 rows reads one contiguous byte run.  Inside a
+// tile every wave-wide load instruction covers 1 KiB contiguous (64 lanes x 16 B):
+//   Q4_K tile, 2304 B: [half 0..1][lane 0..63][16 B] nibble bytes, then [row 0..15][16 B]
+//                      (f16 d, f16 dmin, 12 packed scale bytes) -- the 144 B of each of the
+//                      16 superblocks, byte for byte, only re-ordered.
+//   Q8_0 tile, 2176 B: [half 0..1][lane][16 B] int8 quants, then [row][4 x f16 d].
+// lane = kg*16 + r: r = row inside the tile, kg = which 8-element K slice of a 32-element
+// sub-block the lane feeds to the MFMA.
+// ---------------------------------------------------------------------------------------
+enum { FMT_Q4K = 0, FMT_Q80 = 1 };
+
+struct TiledW {
+    uint8_t* tiles = nullptr;  // device
+    int fmt = 0;
+    int n_rows = 0;    // real output rows
+    int n_tiles = 0;   // ceil(n_rows / 16)
+    int kchunks = 0;   // K / chunk elems
+    int k = 0;
+    size_t bytes = 0;
+};
+
+inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q4K ? 256 : 128; }
+inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 2304 : 2176; }
+inline int fmt_nsub(int fmt) { return fmt == FMT_Q4K ? 8 : 4; }
+
+// Per-call parameters every kernel of a verify pass reads from device memory, so a captured
+// launch sequence can be replayed at another base position.
+struct VerifyParams {
+    int32_t m;               // rows of this pass
+    int32_t base;            // position of row 0 == KV length before the pass
+    int32_t feed[TSV_MAX_ROWS];
+    int32_t pos[TSV_MAX_ROWS];   // rope position of row i: base + depth[i]
+    uint32_t anc[TSV_MAX_ROWS];  // bit s set: row i attends cache slot base+s
+};
+
+enum { EPI_PARTIAL = 0, EPI_SILU = 1, EPI_LOGITS = 2 };
+
+struct GemmArgs {
+    const uint8_t* w;
+    const uint4* xfrag;  // [K/32][4][16] x 16 B, fp16 activations in fragment order
+    void* out;           // EPI_PARTIAL: float [splits][16][ldo]; EPI_SILU: xfrag of the next matmul;
+                         // EPI_LOGITS: half [m][ldo]
+    const VerifyParams* vp;
+    int n_tiles, kchunks, kslice, splits, ldo, n_valid;
+};
+
+int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
+                  int kchunks, int tile_stride, int tile_offset);
+int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
+                int m, int splits, int epi, int ldo, int n_valid);
+int gemm_default_splits(const TiledW& w, int m);
+
+int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
+                 const VerifyParams* vp, int m);
+int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
+                   float eps, int hidden, uint4* xfrag, int m);
+int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
+
+struct RopeKvArgs {
+    const float* qkv;  // [splits][16][ldq]
+    int splits, ldq;
+    const float* freqs;   // head_dim/2
+    const float* q_norm;  // nullable, head_dim
+    const float* k_norm;
+    float eps;
+    uint16_t* q16;  // [16][nq][hd] fp16
+    uint16_t* kc;   // [nkv][max_ctx][hd]
+    uint16_t* vc;   // [nkv][max_ctx/16][hd/16][64][4]
+    int nq, nkv, hd, max_ctx;
+    const VerifyParams* vp;
+};
+int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m);
+
+struct AttnArgs {
+    const uint16_t* q16;
+    const uint16_t* kc;
+    const uint16_t* vc;
+    float* part_o;   // [nkv][nch][rows][hd]
+    float* part_ml;  // [nkv][nch][rows][2]
+    uint4* xfrag;    // output, K index = qh*hd + d
+    int nq, nkv, hd, max_ctx, nch;
+    float scale;
+    const VerifyParams* vp;
+};
+int launch_attention(hipStream_t s, const AttnArgs& a, int m);
+int attn_chunks(int nkv);
+
+int launch_kv_gather(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx,
+                     const int32_t* path_dev, int n, int base);
+int launch_kv_read(hipStream_t s, const uint16_t* kc, const uint16_t* vc, int nkv, int hd, int max_ctx,
+                   int pos0, int n, uint16_t* k_out, uint16_t* v_out);
+
+// ---- acceptance -------------------------------------------------------------------------
+struct AcceptParams {
+    int32_t m, k;            // rows, proposals (chain: m-1)
+    int32_t vocab;
+    int32_t tree;            // 0 chain, 1 tree
+    int32_t sampled;
+    int32_t n_stop;
+    int32_t feed[TSV_MAX_ROWS];
+    int32_t parent[TSV_MAX_ROWS];
+    int32_t stop_tokens[16];
+    double temperature;
+    uint64_t seed, draw_step, generated, max_new_tokens;
+};
+struct AcceptResult {
+    int32_t accepted, committed, next, stopped;
+    uint64_t draw_step;
+    int32_t path[TSV_MAX_ROWS + 1];
+    int32_t path_len;
+    double min_margin;
+    int32_t error;  // 1: non-finite logit
+};
+struct AcceptScratch {
+    double* stats;       // accept_stats_doubles() doubles: row statistics, partials, decisions
+    double* work;        // [16 jobs][2][vocab] candidate masses (p, residual)
+    uint64_t* hist;      // [16 jobs][2][65536] fixed-point mass per rank bin; zero between calls
+    uint32_t* counters;  // 64 words: error flag, greedy arg-max per row
+    AcceptResult* result;  // device
+};
+size_t accept_stats_doubles();
+int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
+                  const AcceptParams& ap_host, const AcceptScratch& sc);
+int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,
+                       const AcceptParams& ap_host, const AcceptScratch& sc, int32_t* proposals_dev);
+
+// ---- host utilities ----------------------------------------------------------------------
+int64_t row_bytes(int dtype, int64_t cols);
+
+}  // namespace tsv

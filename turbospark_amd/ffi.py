@@ -1,0 +1,207 @@
+"""ctypes binding of include/tsverify.h."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libtsverify.so")
+
+F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
+MAX_ROWS = 16
+
+
+class TsvError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"tsverify error {code}: {text}")
+        self.code = code
+        self.text = text
+
+
+class Tensor(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int32), ("rows", C.c_int64), ("cols", C.c_int64)]
+
+
+class Layer(C.Structure):
+    _fields_ = [(n, Tensor) for n in
+                ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up",
+                 "w_down")]
+
+
+class ModelDesc(C.Structure):
+    _fields_ = [
+        ("n_layers", C.c_int32), ("hidden", C.c_int32), ("n_q_heads", C.c_int32),
+        ("n_kv_heads", C.c_int32), ("head_dim", C.c_int32), ("ffn", C.c_int32),
+        ("vocab", C.c_int32), ("max_context", C.c_int32),
+        ("rms_eps", C.c_float), ("rope_theta", C.c_float), ("attn_scale", C.c_float),
+        ("rope_factors", C.POINTER(C.c_float)),
+        ("embed", Tensor), ("final_norm", Tensor), ("lm_head", Tensor),
+        ("layers", C.POINTER(Layer)),
+    ]
+
+
+class Shaping(C.Structure):
+    _fields_ = [
+        ("temperature", C.c_double), ("top_k", C.c_uint32), ("has_top_p", C.c_int32),
+        ("top_p", C.c_double), ("repetition_penalty", C.c_double), ("has_seed", C.c_int32),
+        ("seed", C.c_uint64), ("presence_penalty", C.c_double), ("frequency_penalty", C.c_double),
+        ("has_min_p", C.c_int32), ("min_p", C.c_double),
+    ]
+
+
+def shaping(temperature=0.0, top_k=0, top_p=None, repetition_penalty=1.0, seed=None,
+            presence_penalty=0.0, frequency_penalty=0.0, min_p=None):
+    """`ShapingConfig::new` (crates/selection/src/shaping.rs:84-123): validated at construction."""
+    if not np.isfinite(temperature) or temperature < 0:
+        raise ValueError(f"temperature must be finite and non-negative, got {temperature}")
+    if top_k > 256:
+        raise ValueError(f"top_k must be between 0 and 256, got {top_k}")
+    if top_p is not None and not (np.isfinite(top_p) and 0.0 < top_p <= 1.0):
+        raise ValueError(f"top_p must be finite and in (0, 1], got {top_p}")
+    if not np.isfinite(repetition_penalty) or repetition_penalty <= 0:
+        raise ValueError("repetition_penalty must be finite and greater than zero")
+    s = Shaping()
+    s.temperature = temperature
+    s.top_k = top_k
+    s.has_top_p = top_p is not None
+    s.top_p = top_p or 0.0
+    s.repetition_penalty = repetition_penalty
+    s.has_seed = seed is not None
+    s.seed = seed or 0
+    s.presence_penalty = presence_penalty
+    s.frequency_penalty = frequency_penalty
+    s.has_min_p = min_p is not None
+    s.min_p = min_p or 0.0
+    return s
+
+
+class Point(C.Structure):
+    _fields_ = [("position", C.c_int64)]
+
+
+class Round(C.Structure):
+    _fields_ = [
+        ("feed", C.POINTER(C.c_int32)), ("parent", C.POINTER(C.c_int32)), ("m", C.c_int32),
+        ("base", C.c_int64), ("shaping", Shaping), ("draft_logits", C.c_void_p),
+        ("draw_step", C.c_uint64), ("stop_tokens", C.POINTER(C.c_int32)), ("n_stop", C.c_int32),
+        ("generated", C.c_uint64), ("max_new_tokens", C.c_uint64), ("logits_out", C.c_void_p),
+    ]
+
+
+class RoundResultC(C.Structure):
+    _fields_ = [
+        ("accepted", C.c_int32), ("committed", C.c_int32), ("next", C.c_int32), ("stopped", C.c_int32),
+        ("draw_step", C.c_uint64), ("path", C.c_int32 * (MAX_ROWS + 1)), ("path_len", C.c_int32),
+        ("kv_position", C.c_int64), ("min_margin", C.c_double),
+    ]
+
+
+EXPORTS = [
+    "tsv_open", "tsv_close", "tsv_last_error", "tsv_stream", "tsv_reset", "tsv_kv_position",
+    "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
+    "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
+    "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
+    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul",
+]
+
+_lib = None
+
+
+def lib():
+    """Loads libtsverify.so.  Fails loudly when it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(hipcc, gfx950).  turbospark_amd has no CPU path.")
+        L = C.CDLL(LIB_PATH)
+        L.tsv_stream.restype = C.c_void_p
+        L.tsv_stream.argtypes = [C.c_void_p]
+        L.tsv_kv_position.restype = C.c_int64
+        L.tsv_kv_position.argtypes = [C.c_void_p]
+        L.tsv_row_bytes.restype = C.c_int64
+        L.tsv_row_bytes.argtypes = [C.c_int32, C.c_int64]
+        L.tsv_close.restype = None
+        L.tsv_close.argtypes = [C.c_void_p]
+        L.tsv_open.argtypes = [C.POINTER(ModelDesc), C.POINTER(C.c_void_p)]
+        L.tsv_reset.argtypes = [C.c_void_p]
+        L.tsv_produce.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
+        L.tsv_prefill.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+        L.tsv_checkpoint.argtypes = [C.c_void_p, C.POINTER(Point)]
+        L.tsv_rollback.argtypes = [C.c_void_p, C.POINTER(Point)]
+        L.tsv_rollback_retaining.argtypes = [C.c_void_p, C.POINTER(Point), C.c_int32]
+        L.tsv_commit_pending.argtypes = [C.c_void_p, C.c_int32]
+        L.tsv_discard_pending.argtypes = [C.c_void_p]
+        L.tsv_verify.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
+        L.tsv_verify_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
+        L.tsv_compact_tree.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int32]
+        L.tsv_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
+        L.tsv_verify_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
+        L.tsv_draft_chain.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(Shaping),
+                                      C.POINTER(C.c_uint64), C.c_void_p]
+        L.tsv_quantize_rows.argtypes = [C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+        L.tsv_synth_tensor.argtypes = [C.c_int32, C.c_uint64, C.c_uint64, C.c_float, C.c_int64, C.c_int64,
+                                       C.c_void_p]
+        L.tsv_read_kv.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
+        L.tsv_matmul.argtypes = [C.POINTER(Tensor), C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
+        L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
+        _lib = L
+    return _lib
+
+
+def last_error():
+    buf = C.create_string_buffer(1024)
+    lib().tsv_last_error(buf, 1024)
+    return buf.value.decode(errors="replace")
+
+
+def check(rc):
+    if rc != 0:
+        raise TsvError(rc, last_error())
+
+
+def tensor(entry):
+    """entry: None | (dtype, uint8 ndarray [rows, row_bytes], rows, cols)."""
+    t = Tensor()
+    if entry is None:
+        return t
+    dtype, data, rows, cols = entry
+    t.data = data.ctypes.data
+    t.dtype = dtype
+    t.rows = rows
+    t.cols = cols
+    return t
+
+
+def row_bytes(dtype, cols):
+    return lib().tsv_row_bytes(dtype, cols)
+
+
+def quantize(dtype, w):
+    """fp32 [rows, cols] -> (dtype, uint8 [rows, row_bytes], rows, cols) with the install-time encoders."""
+    w = np.ascontiguousarray(w, np.float32)
+    rows, cols = w.shape
+    rb = row_bytes(dtype, cols)
+    if rb < 0:
+        raise ValueError("column count is not whole blocks of this dtype")
+    out = np.empty((rows, rb), np.uint8)
+    check(lib().tsv_quantize_rows(dtype, w.ctypes.data, rows, cols, out.ctypes.data))
+    return (dtype, out, rows, cols)
+
+
+def synth_tensor(dtype, seed, stream, sigma, rows, cols):
+    rb = row_bytes(dtype, cols)
+    out = np.empty((rows, rb), np.uint8)
+    check(lib().tsv_synth_tensor(dtype, seed, stream, sigma, rows, cols, out.ctypes.data))
+    return (dtype, out, rows, cols)
+
+
+def matmul(entry, x, splits=0):
+    """y[m][r] = sum_k W[r][k] x[m][k] through the verify pass's own matmul kernel."""
+    x = np.ascontiguousarray(x, np.float32)
+    m = x.shape[0]
+    t = tensor(entry)
+    y = np.empty((m, entry[2]), np.float32)
+    check(lib().tsv_matmul(C.byref(t), x.ctypes.data, m, y.ctypes.data, splits))
+    return y

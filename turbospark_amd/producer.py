@@ -1,0 +1,216 @@
+"""Host-side mirror of the reference's producer traits for the verify path.
+
+`HipVerifier` carries the method names and argument meaning of `LogitProducer` and
+`SpeculativeProducer` (crates/runtime/src/producer.rs:17-104,164-387) over the C ABI of
+libtsverify.so.  Errors surface as `TsvError` carrying the engine's message (the reference
+returns `Result<(), String>`).
+"""
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+
+from . import ffi
+
+
+@dataclass
+class RoundResult:
+    accepted: int
+    committed: int
+    next: int
+    stopped: int
+    draw_step: int
+    path: List[int] = field(default_factory=list)
+    kv_position: int = 0
+    min_margin: float = 1.0
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, np.int32)
+
+
+class HipVerifier:
+    """One target model resident on the GPU with its fp16 KV cache."""
+
+    def __init__(self, cfg, weights):
+        self.cfg = dict(cfg)
+        self._keep = weights
+        n = len(weights["layers"])
+        self._layers = (ffi.Layer * n)()
+        for i, lw in enumerate(weights["layers"]):
+            for name, _ in ffi.Layer._fields_:
+                setattr(self._layers[i], name, ffi.tensor(lw.get(name)))
+        d = ffi.ModelDesc()
+        d.n_layers = n
+        for key in ("hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_context"):
+            setattr(d, key, cfg[key])
+        d.rms_eps = cfg.get("rms_eps", 1e-5)
+        d.rope_theta = cfg.get("rope_theta", 10000.0)
+        d.attn_scale = cfg.get("attn_scale", 0.0)
+        self._factors = None
+        if cfg.get("rope_factors") is not None:
+            self._factors = np.ascontiguousarray(cfg["rope_factors"], np.float32)
+            d.rope_factors = self._factors.ctypes.data_as(C.POINTER(C.c_float))
+        d.embed = ffi.tensor(weights["embed"])
+        d.final_norm = ffi.tensor(weights["final_norm"])
+        d.lm_head = ffi.tensor(weights.get("lm_head"))
+        d.layers = C.cast(self._layers, C.POINTER(ffi.Layer))
+        h = C.c_void_p()
+        ffi.check(ffi.lib().tsv_open(C.byref(d), C.byref(h)))
+        self._h = h
+        self.vocab = cfg["vocab"]
+
+    def close(self):
+        if getattr(self, "_h", None):
+            ffi.lib().tsv_close(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    # ---- LogitProducer ----------------------------------------------------------------
+    def reset(self):
+        ffi.check(ffi.lib().tsv_reset(self._h))
+
+    @property
+    def position(self):
+        return ffi.lib().tsv_kv_position(self._h)
+
+    @property
+    def stream(self):
+        """The hipStream_t (as an integer) every kernel of this handle runs on."""
+        return ffi.lib().tsv_stream(self._h)
+
+    def produce(self, token, position):
+        out = np.empty(self.vocab, np.uint16)
+        ffi.check(ffi.lib().tsv_produce(self._h, int(token), int(position), out.ctypes.data))
+        return out
+
+    def prefill(self, ids, pos0=0, want_logits=True):
+        ids = _i32(ids)
+        out = np.empty(self.vocab, np.uint16) if want_logits else None
+        ffi.check(ffi.lib().tsv_prefill(self._h, ids.ctypes.data, ids.size, int(pos0),
+                                        out.ctypes.data if want_logits else None))
+        return out
+
+    # ---- SpeculativeProducer ----------------------------------------------------------
+    def checkpoint(self):
+        p = ffi.Point()
+        ffi.check(ffi.lib().tsv_checkpoint(self._h, C.byref(p)))
+        return p
+
+    def rollback(self, point):
+        ffi.check(ffi.lib().tsv_rollback(self._h, C.byref(point)))
+
+    def supports_retaining_rollback(self):
+        return True
+
+    def rollback_retaining(self, point, keep_rows):
+        ffi.check(ffi.lib().tsv_rollback_retaining(self._h, C.byref(point), int(keep_rows)))
+
+    def commit_pending(self, keep_rows):
+        ffi.check(ffi.lib().tsv_commit_pending(self._h, int(keep_rows)))
+
+    def discard_pending(self):
+        ffi.check(ffi.lib().tsv_discard_pending(self._h))
+
+    def verify(self, feed, base, want_logits=True):
+        feed = _i32(feed)
+        out = np.empty((feed.size, self.vocab), np.uint16) if want_logits else None
+        ffi.check(ffi.lib().tsv_verify(self._h, feed.ctypes.data, feed.size, int(base),
+                                       out.ctypes.data if want_logits else None))
+        return out
+
+    def verify_tree(self, feed, parent, base, want_logits=True):
+        feed, parent = _i32(feed), _i32(parent)
+        out = np.empty((feed.size, self.vocab), np.uint16) if want_logits else None
+        ffi.check(ffi.lib().tsv_verify_tree(self._h, feed.ctypes.data, parent.ctypes.data, feed.size,
+                                            int(base), out.ctypes.data if want_logits else None))
+        return out
+
+    def compact_tree(self, base, path):
+        p = np.ascontiguousarray(path, np.uint32)
+        ffi.check(ffi.lib().tsv_compact_tree(self._h, int(base), p.ctypes.data, p.size))
+
+    # ---- device-side acceptance -----------------------------------------------------------
+    def _round(self, feed, base, cfg, parent, draft_logits, draw_step, stop_tokens, generated,
+               max_new_tokens, want_logits):
+        keep = {}
+        r = ffi.Round()
+        keep["feed"] = _i32(feed)
+        r.feed = keep["feed"].ctypes.data_as(C.POINTER(C.c_int32))
+        r.m = keep["feed"].size
+        if parent is not None:
+            keep["parent"] = _i32(parent)
+            r.parent = keep["parent"].ctypes.data_as(C.POINTER(C.c_int32))
+        r.base = int(base)
+        r.shaping = cfg
+        if draft_logits is not None:
+            if isinstance(draft_logits, int):
+                r.draft_logits = draft_logits  # a device pointer
+            else:
+                a = np.asarray(draft_logits)
+                if a.dtype != np.uint16:
+                    a = a.astype(np.float16).view(np.uint16)
+                keep["draft"] = np.ascontiguousarray(a)
+                r.draft_logits = keep["draft"].ctypes.data
+        r.draw_step = int(draw_step)
+        if stop_tokens is not None and len(stop_tokens):
+            keep["stop"] = _i32(stop_tokens)
+            r.stop_tokens = keep["stop"].ctypes.data_as(C.POINTER(C.c_int32))
+            r.n_stop = keep["stop"].size
+        r.generated = int(generated)
+        r.max_new_tokens = int(max_new_tokens)
+        if want_logits:
+            keep["logits"] = np.empty((r.m, self.vocab), np.uint16)
+            r.logits_out = keep["logits"].ctypes.data
+        return r, keep
+
+    @staticmethod
+    def _result(c):
+        return RoundResult(c.accepted, c.committed, c.next, c.stopped, c.draw_step,
+                           list(c.path[: c.path_len]), c.kv_position, c.min_margin)
+
+    def accept(self, feed, base, cfg, parent=None, draft_logits=None, draw_step=0, stop_tokens=None,
+               generated=0, max_new_tokens=0):
+        """Acceptance + truncation over the logits the last verify left on the device."""
+        r, keep = self._round(feed, base, cfg, parent, draft_logits, draw_step, stop_tokens, generated,
+                              max_new_tokens, False)
+        out = ffi.RoundResultC()
+        ffi.check(ffi.lib().tsv_accept(self._h, C.byref(r), C.byref(out)))
+        return self._result(out)
+
+    def verify_accept(self, feed, base, cfg, parent=None, draft_logits=None, draw_step=0,
+                      stop_tokens=None, generated=0, max_new_tokens=0, want_logits=False):
+        """The whole verify step: target forward, acceptance, KV truncation."""
+        r, keep = self._round(feed, base, cfg, parent, draft_logits, draw_step, stop_tokens, generated,
+                              max_new_tokens, want_logits)
+        out = ffi.RoundResultC()
+        ffi.check(ffi.lib().tsv_verify_accept(self._h, C.byref(r), C.byref(out)))
+        res = self._result(out)
+        return (res, keep["logits"]) if want_logits else res
+
+    def draft_chain(self, draft_logits, cfg, draw_step=0):
+        """Draw the k proposals of a chain round from the drafter's rows; returns (proposals, draw_step)."""
+        if isinstance(draft_logits, tuple):  # (device pointer, k)
+            ptr, k = draft_logits
+        else:
+            a = np.asarray(draft_logits)
+            if a.dtype != np.uint16:
+                a = a.astype(np.float16).view(np.uint16)
+            a = np.ascontiguousarray(a)
+            ptr, k = a.ctypes.data, a.shape[0]
+        ds = C.c_uint64(int(draw_step))
+        props = np.empty(k, np.int32)
+        ffi.check(ffi.lib().tsv_draft_chain(self._h, ptr, k, C.byref(cfg), C.byref(ds), props.ctypes.data))
+        return props, ds.value
+
+    # ---- test introspection ------------------------------------------------------------------
+    def read_kv(self, layer, pos0, n):
+        c = self.cfg
+        shape = (n, c["n_kv_heads"], c["head_dim"])
+        k = np.empty(shape, np.float16)
+        v = np.empty(shape, np.float16)
+        ffi.check(ffi.lib().tsv_read_kv(self._h, layer, int(pos0), int(n), k.ctypes.data, v.ctypes.data))
+        return k, v

@@ -1,0 +1,39 @@
+"""Seeded random-init target models in GGUF block formats (the reference's synthetic installs,
+crates/repack/src/synthetic_*.rs, for the verify path's benchmark configurations)."""
+import numpy as np
+
+from . import ffi
+
+# BASELINE configurations of the verify path (dense ones).
+CONFIGS = {
+    # tiny Llama-style decoder, the reference's CPU-runnable plumbing case
+    "tiny_q8_0": dict(n_layers=2, hidden=512, n_q_heads=8, n_kv_heads=8, head_dim=64, ffn=1408,
+                      vocab=4096, rms_eps=1e-5, rope_theta=10000.0, dtype=ffi.Q8_0),
+    # a small Q4_K stand-in with the 8B model's head geometry (GQA 4, head_dim 128)
+    "small_q4_k": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
+                       vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
+    # Llama-3-8B shape
+    "llama3_8b_q4_k": dict(n_layers=32, hidden=4096, n_q_heads=32, n_kv_heads=8, head_dim=128,
+                           ffn=14336, vocab=128256, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
+}
+
+
+def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
+    """N(0, sigma) weights quantized to cfg['dtype']; norm weights 1.0.  Returns the weight
+    dictionary both the engine and the test oracle take."""
+    dt = cfg["dtype"]
+    H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
+    qd, kvd = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    ones = lambda n: (ffi.F32, np.ones((1, n), np.float32).view(np.uint8).reshape(1, -1), 1, n)
+    stream = [0]
+
+    def t(rows, cols):
+        stream[0] += 1
+        return ffi.synth_tensor(dt, seed, stream[0], sigma, rows, cols)
+
+    L = cfg["n_layers"] if n_layers is None else n_layers
+    layers = []
+    for _ in range(L):
+        layers.append(dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H), wo=t(H, qd),
+                           ffn_norm=ones(H), w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F)))
+    return dict(embed=t(V, H), final_norm=ones(H), lm_head=t(V, H), layers=layers)
