@@ -190,6 +190,14 @@ int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16
  * the engine's own split-K factor. */
 int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits);
 
+/* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
+ * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache
+ * slot base+i and sees [0, base) plus the slots of its root path (parent NULL: chain).
+ * out: m x nq x hd fp16.  (The per-kernel parity hook of crates/gpu/tests/attention_tree_parity.rs.) */
+int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
+                      int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
+                      uint16_t* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,71 @@
+"""GPU parity of the verify-pass attention kernel against the oracle's causal attention.
+
+Mirrors crates/gpu/tests/attention_tree_parity.rs (identity path == chain row; a branch node ==
+the chain over its root path) and crates/compute/src/attention.rs' reference arithmetic."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(q, k, v, base, parent, scale=0.0):
+    m, nq, hd = q.shape
+    nkv = k.shape[1]
+    out = np.empty((m, nq, hd), np.float32)
+    import ctypes as C
+    for i in range(m):
+        if parent is None:
+            out[i] = ob.causal_attention(q[i], k, v, hd, nq, nkv, base + i + 1, 0, scale).reshape(nq, hd)
+        else:
+            path = []
+            s = i
+            while s >= 0:
+                path.append(base + s)
+                s = parent[s]
+            path = np.array(path[::-1], np.int64)
+            o = np.empty(nq * hd, np.float32)
+            qq = np.ascontiguousarray(q[i], np.float32)
+            kk = np.ascontiguousarray(k, np.float32)
+            vv = np.ascontiguousarray(v, np.float32)
+            ob.lib().tso_attention_core(qq.ctypes.data_as(C.c_void_p), kk.ctypes.data_as(C.c_void_p),
+                                        vv.ctypes.data_as(C.c_void_p), hd, nq, nkv, C.c_int64(0), C.c_int64(base),
+                                        path.ctypes.data_as(C.c_void_p), len(path), C.c_float(scale), None,
+                                        o.ctypes.data_as(C.c_void_p))
+            out[i] = o.reshape(nq, hd)
+    return out
+
+
+def _rand(m, nq, nkv, hd, base, seed):
+    rng = np.random.default_rng(seed)
+    r16 = lambda *s: rng.standard_normal(s).astype(np.float16).astype(np.float32)
+    return r16(m, nq, hd), r16(base + m, nkv, hd), r16(base + m, nkv, hd)
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 8, 64), (4, 1, 128), (32, 8, 128), (16, 2, 64)])
+@pytest.mark.parametrize("m,base", [(1, 0), (1, 37), (4, 0), (5, 0), (8, 0), (16, 0), (5, 200), (16, 1000), (9, 15)])
+def test_chain_attention_matches_the_oracle(nq, nkv, hd, m, base):
+    from turbospark_amd import ffi
+    q, k, v = _rand(m, nq, nkv, hd, base, 100 + m + base)
+    got = ffi.attention(q, k, v, base)
+    want = _oracle(q, k, v, base, None)
+    err = np.abs(got - want).reshape(m, -1).max(1)
+    assert err.max() <= 5e-3 * max(1.0, np.abs(want).max()), err  # Tolerance::FP16_REDUCTION
+
+
+def test_tree_attention_sees_prefix_plus_root_path():
+    from turbospark_amd import ffi
+    parent = [-1, 0, 0, 0, 0, 1, 5, 6, 2, 8, 9, 3, 11, 12, 4, 14]
+    for (nq, nkv, hd, base) in [(4, 1, 128, 37), (32, 8, 128, 300), (8, 8, 64, 0)]:
+        q, k, v = _rand(16, nq, nkv, hd, base, 5)
+        got = ffi.attention(q, k, v, base, parent)
+        want = _oracle(q, k, v, base, parent)
+        assert np.abs(got - want).max() <= 5e-3 * max(1.0, np.abs(want).max())
+        # identity path == chain, bit for bit
+        a = ffi.attention(q[:6], k[:base + 6], v[:base + 6], base)
+        b = ffi.attention(q[:6], k[:base + 6], v[:base + 6], base, [-1, 0, 1, 2, 3, 4])
+        assert np.array_equal(a, b)
+        # the identity map over a branching layout must FAIL at branch nodes
+        c = ffi.attention(q, k, v, base)
+        assert np.abs(c[8] - want[8]).max() > 1e-2

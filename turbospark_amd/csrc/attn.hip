@@ -43,6 +43,7 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
     const int bpc = (nblk + a.nch - 1) / a.nch;
     const int b0 = chunk * bpc, b1 = min(b0 + bpc, nblk);
     const float scale = a.scale;
+    const uint32_t mmask = (1u << M) - 1u;  // slots that exist in this pass
 
     // query fragments and per-row ancestor sets
     uint4 qf[RT][KS];
@@ -93,16 +94,17 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
             for (int s = 0; s < KS; s++)
                 S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, kf[s]),
                                                            __builtin_bit_cast(half8, qf[t][s]), S, 0, 0, 0);
+            // Visibility of this lane's four positions as a 4-bit word, computed without
+            // branches: bit (slot + 16) of `w` says whether cache slot base+slot is visible
+            // (the 16 low bits stand for prefix positions, always visible).
+            uint32_t vis4 = 0xFu;
+            if (tail) {
+                const uint64_t w = ((uint64_t)(anc[t] & mmask) << 16) | 0xFFFFull;
+                vis4 = (uint32_t)(w >> (p0 + 4 * kg - base + 16)) & 0xFu;  // shift in [1, 47]
+            }
             float sc[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                sc[i] = S[i] * scale;
-                if (tail) {
-                    const int slot = p0 + 4 * kg + i - base;
-                    const bool ok = slot < 0 || (slot < M && ((anc[t] >> slot) & 1u));
-                    if (!ok) sc[i] = -INFINITY;
-                }
-            }
+            for (int i = 0; i < 4; i++) sc[i] = ((vis4 >> i) & 1u) ? S[i] * scale : -INFINITY;
             float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             mb = fmaxf(mb, __shfl_xor(mb, 16));
             mb = fmaxf(mb, __shfl_xor(mb, 32));

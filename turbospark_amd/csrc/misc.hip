@@ -229,6 +229,22 @@ __global__ void k_kv_read(const uint16_t* kc, const uint16_t* vc, int nkv, int h
     v_out[o] = vc[v_index(h, pos0 + p, d, hd, max_ctx)];
 }
 
+__global__ void k_kv_fill(uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0,
+                          const uint16_t* k_in, const uint16_t* v_in) {
+    const int p = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    if (d >= hd) return;
+    const long o = ((long)p * nkv + h) * hd + d;
+    kc[((long)h * max_ctx + pos0 + p) * hd + d] = k_in[o];
+    vc[v_index(h, pos0 + p, d, hd, max_ctx)] = v_in[o];
+}
+
+int launch_kv_fill(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0, int n,
+                   const uint16_t* k_in, const uint16_t* v_in) {
+    hipLaunchKernelGGL(k_kv_fill, dim3(n, nkv), dim3(128), 0, s, kc, vc, nkv, hd, max_ctx, pos0, k_in, v_in);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
 int launch_kv_read(hipStream_t s, const uint16_t* kc, const uint16_t* vc, int nkv, int hd, int max_ctx,
                    int pos0, int n, uint16_t* k_out, uint16_t* v_out) {
     hipLaunchKernelGGL(k_kv_read, dim3(n, nkv), dim3(128), 0, s, kc, vc, nkv, hd, max_ctx, pos0, k_out, v_out);

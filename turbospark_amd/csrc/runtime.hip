@@ -207,6 +207,35 @@ int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
     return TSV_OK;
 }
 
+int fill_params(VerifyParams& vp, const int32_t* feed, const int32_t* parent, int m, int64_t base, int vocab) {
+    std::memset(&vp, 0, sizeof vp);
+    vp.m = m;
+    vp.base = (int32_t)base;
+    int depth[TSV_MAX_ROWS] = {0};
+    for (int i = 0; i < m; i++) {
+        if (feed) {
+            if (feed[i] < 0 || feed[i] >= vocab) {
+                set_error("verify: token id outside the vocabulary");
+                return TSV_ERR_INVALID;
+            }
+            vp.feed[i] = feed[i];
+        }
+        if (parent) {
+            if (i == 0 ? parent[0] != -1 : (parent[i] < 0 || parent[i] >= i)) {
+                set_error("verify_tree: parent[0] must be -1 and parent[s] in [0, s)");
+                return TSV_ERR_INVALID;
+            }
+            depth[i] = i == 0 ? 0 : depth[parent[i]] + 1;
+            vp.anc[i] = (i == 0 ? 0u : vp.anc[parent[i]]) | (1u << i);
+        } else {
+            depth[i] = i;
+            vp.anc[i] = (2u << i) - 1u;
+        }
+        vp.pos[i] = (int32_t)base + depth[i];
+    }
+    return TSV_OK;
+}
+
 // One verify pass: enqueue everything on the handle's stream; no synchronisation.
 int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m, int64_t base) {
     // batched.rs:106-185 refusals
@@ -227,29 +256,8 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
         return TSV_ERR_INVALID;
     }
     VerifyParams vp;
-    std::memset(&vp, 0, sizeof vp);
-    vp.m = m;
-    vp.base = (int32_t)base;
-    int depth[TSV_MAX_ROWS] = {0};
-    for (int i = 0; i < m; i++) {
-        if (feed[i] < 0 || feed[i] >= c->vocab) {
-            set_error("verify: token id outside the vocabulary");
-            return TSV_ERR_INVALID;
-        }
-        vp.feed[i] = feed[i];
-        if (parent) {
-            if (i == 0 ? parent[0] != -1 : (parent[i] < 0 || parent[i] >= i)) {
-                set_error("verify_tree: parent[0] must be -1 and parent[s] in [0, s)");
-                return TSV_ERR_INVALID;
-            }
-            depth[i] = i == 0 ? 0 : depth[parent[i]] + 1;
-            vp.anc[i] = (i == 0 ? 0u : vp.anc[parent[i]]) | (1u << i);
-        } else {
-            depth[i] = i;
-            vp.anc[i] = (2u << i) - 1u;
-        }
-        vp.pos[i] = (int32_t)base + depth[i];
-    }
+    int prc = fill_params(vp, feed, parent, m, base, c->vocab);
+    if (prc) return prc;
     hipStream_t s = c->stream;
     // the pinned staging copy must not be rewritten while an earlier copy is still in flight
     TSV_HIP(hipStreamSynchronize(s));
@@ -793,6 +801,76 @@ extern "C" int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, fl
                 y[(size_t)b * n + j] = acc;
             }
     if (st.dev) (void)hipFree(st.dev);
+    (void)hipStreamSynchronize(c->stream);
+    for (void* p : c->allocs) (void)hipFree(p);
+    (void)hipStreamDestroy(c->stream);
+    return rc;
+}
+
+extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
+                                 int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
+                                 uint16_t* out) {
+    if (!q || !k || !v || !out || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0) {
+        set_error("attention: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    tsv_ctx tmp;
+    tsv_ctx* c = &tmp;
+    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    VerifyParams vp;
+    int rc = fill_params(vp, nullptr, parent, m, base, 0);
+    const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv;
+    const size_t kvb = (size_t)nkv * ctx * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
+    uint16_t *kc = nullptr, *vc = nullptr, *kin = nullptr, *vin = nullptr, *q16 = nullptr;
+    float *po = nullptr, *pml = nullptr;
+    uint4* xf = nullptr;
+    VerifyParams* vpd = nullptr;
+    const size_t xfb = (size_t)nq * hd / 32 * 4 * 16 * 16;
+    if (!rc) rc = dev_alloc(c, &kc, kvb, true);
+    if (!rc) rc = dev_alloc(c, &vc, kvb, true);
+    if (!rc) rc = dev_alloc(c, &kin, inb);
+    if (!rc) rc = dev_alloc(c, &vin, inb);
+    if (!rc) rc = dev_alloc(c, &q16, qb);
+    if (!rc) rc = dev_alloc(c, &po, (size_t)nkv * nch * m * G * hd * 4, true);
+    if (!rc) rc = dev_alloc(c, &pml, (size_t)nkv * nch * m * G * 2 * 4, true);
+    if (!rc) rc = dev_alloc(c, &xf, xfb, true);
+    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
+    if (!rc && (hipMemcpyAsync(kin, k, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+                hipMemcpyAsync(vin, v, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+                hipMemcpyAsync(q16, q, qb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+                hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess))
+        rc = TSV_ERR_DEVICE;
+    if (!rc) rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, 0, seq, kin, vin);
+    if (!rc) {
+        AttnArgs aa;
+        aa.q16 = q16;
+        aa.kc = kc;
+        aa.vc = vc;
+        aa.part_o = po;
+        aa.part_ml = pml;
+        aa.xfrag = xf;
+        aa.nq = nq;
+        aa.nkv = nkv;
+        aa.hd = hd;
+        aa.max_ctx = ctx;
+        aa.nch = nch;
+        aa.scale = scale > 0.f ? scale : 1.0f / std::sqrt((float)hd);
+        aa.vp = vpd;
+        rc = launch_attention(c->stream, aa, m);
+    }
+    std::vector<uint16_t> frag(xfb / 2);
+    if (!rc && (hipMemcpyAsync(frag.data(), xf, xfb, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                hipStreamSynchronize(c->stream) != hipSuccess)) {
+        set_error("attention: device execution failed");
+        rc = TSV_ERR_DEVICE;
+    }
+    if (!rc)
+        for (int b = 0; b < m; b++)
+            for (int kk = 0; kk < nq * hd; kk++) {
+                const int sub = kk >> 5, e = kk & 31, kg = e >> 3, o = e & 7;
+                const int p = (o & 4) | ((o & 1) << 1) | ((o >> 1) & 1);
+                out[(size_t)b * nq * hd + kk] = frag[(size_t)((sub * 4 + kg) * 16 + b) * 8 + p];
+            }
     (void)hipStreamSynchronize(c->stream);
     for (void* p : c->allocs) (void)hipFree(p);
     (void)hipStreamDestroy(c->stream);

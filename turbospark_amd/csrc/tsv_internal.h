@@ -113,6 +113,8 @@ int attn_chunks(int nkv);
 
 int launch_kv_gather(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx,
                      const int32_t* path_dev, int n, int base);
+int launch_kv_fill(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0, int n,
+                   const uint16_t* k_in, const uint16_t* v_in);
 int launch_kv_read(hipStream_t s, const uint16_t* kc, const uint16_t* vc, int nkv, int hd, int max_ctx,
                    int pos0, int n, uint16_t* k_out, uint16_t* v_out);
 

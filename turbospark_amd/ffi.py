@@ -101,7 +101,7 @@ EXPORTS = [
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
-    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul",
+    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention",
 ]
 
 _lib = None
@@ -145,6 +145,8 @@ def lib():
                                        C.c_void_p]
         L.tsv_read_kv.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.tsv_matmul.argtypes = [C.POINTER(Tensor), C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
+        L.tsv_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                    C.c_int64, C.c_void_p, C.c_float, C.c_void_p]
         L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
         _lib = L
     return _lib
@@ -205,3 +207,18 @@ def matmul(entry, x, splits=0):
     y = np.empty((m, entry[2]), np.float32)
     check(lib().tsv_matmul(C.byref(t), x.ctypes.data, m, y.ctypes.data, splits))
     return y
+
+
+def attention(q, k, v, base, parent=None, scale=0.0):
+    """q [m, nq, hd], k/v [base+m, nkv, hd] (any float dtype; rounded to fp16) -> fp32 [m, nq, hd]."""
+    q16 = np.ascontiguousarray(np.asarray(q, np.float32).astype(np.float16))
+    k16 = np.ascontiguousarray(np.asarray(k, np.float32).astype(np.float16))
+    v16 = np.ascontiguousarray(np.asarray(v, np.float32).astype(np.float16))
+    m, nq, hd = q16.shape
+    nkv = k16.shape[1]
+    assert k16.shape[0] == base + m
+    out = np.empty((m, nq, hd), np.float16)
+    pa = np.ascontiguousarray(parent, np.int32) if parent is not None else None
+    check(lib().tsv_attention(q16.ctypes.data, k16.ctypes.data, v16.ctypes.data, m, nq, nkv, hd, base,
+                              pa.ctypes.data if pa is not None else None, scale, out.ctypes.data))
+    return out.astype(np.float32)
