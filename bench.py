@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the speculative-decoding verify step on one MI355X.
+
+A "step" is one verify step: the target forward over the k+1 fed rows, device-side acceptance
+and the KV truncation (`HipVerifier.verify_accept`), on a Llama-3-8B-shaped random-init Q4_K
+target with a 4096-token fp16 KV cache, chain draft k=4, rejection sampling at T=0.8 -- the
+configuration the headline metric is quoted on.  Inputs (weights, KV cache, drafter logits,
+proposals) are resident in HBM before the timed region.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # BASELINE configs[1]
+    "llama3_8b_q4_k_k4_ctx4096": dict(model="llama3_8b_q4_k", ctx=4096, k=4, temperature=0.8),
+    # BASELINE configs[0] (the reference's CPU-runnable plumbing case), greedy
+    "tiny_q8_0_k4_ctx256": dict(model="tiny_q8_0", ctx=256, k=4, temperature=0.0),
+    "small_q4_k_k4_ctx256": dict(model="small_q4_k", ctx=256, k=4, temperature=0.8),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(cfg, ctx, m):
+    """Bytes one verify step has to move: every quantized weight once, the KV rows [0, ctx+m)
+    once per layer, m embedding rows, m x vocab fp16 logits, m new KV rows."""
+    from turbospark_amd import ffi
+    H, F, V, L = cfg["hidden"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
+    qd, kvd = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    rb = lambda rows, cols: rows * ffi.row_bytes(cfg["dtype"], cols)
+    per_layer = dict(qkv=rb(qd + 2 * kvd, H), wo=rb(H, qd), gate_up=rb(2 * F, H), down=rb(H, F))
+    head = rb(V, H)
+    weights = L * sum(per_layer.values()) + head
+    kv = L * (ctx + m) * kvd * 2 * 2
+    small = m * ffi.row_bytes(cfg["dtype"], H) + m * V * 2 + L * m * kvd * 2 * 2
+    return dict(per_layer=per_layer, head=head, weights=weights, kv=kv, total=weights + kv + small)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="llama3_8b_q4_k_k4_ctx4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--layers", type=int, default=None, help="debug: build only this many layers")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=20261125)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "
+                 "supported (see DESIGN.md, 'how the path would shard').")
+
+    import turbospark_amd as ts
+    from turbospark_amd import hip, synth
+
+    wl = WORKLOADS[args.workload]
+    cfg = dict(synth.CONFIGS[wl["model"]])
+    if args.layers:
+        cfg["n_layers"] = args.layers
+    k, ctx, T = wl["k"], wl["ctx"], wl["temperature"]
+    m = k + 1
+    cfg["max_context"] = ctx + 32
+    V = cfg["vocab"]
+
+    t0 = time.time()
+    weights = synth.make_weights(cfg, seed=args.seed)
+    log(f"[bench] synthetic {wl['model']} weights ({cfg['n_layers']} layers) in {time.time() - t0:.1f}s")
+    t0 = time.time()
+    eng = ts.HipVerifier(cfg, weights)
+    log(f"[bench] upload + re-tile in {time.time() - t0:.1f}s")
+    rng = np.random.default_rng(args.seed)
+    prompt = rng.integers(0, V, ctx).astype(np.int32)
+    t0 = time.time()
+    eng.prefill(prompt[:-1], 0, want_logits=False)   # the last prompt token is the round's confirmed token
+    log(f"[bench] prefill of {ctx - 1} tokens in {time.time() - t0:.2f}s")
+    base = eng.position
+    point = eng.checkpoint()
+    anchor = int(prompt[-1])
+
+    # drafter logits N(0,1) per round, resident on the device; proposals drawn on the device
+    rounds = args.warmup + args.steps
+    shaping = [ts.shaping(T, seed=args.seed + r) if T > 0 else ts.shaping(0.0) for r in range(rounds)]
+    draft_host = rng.standard_normal((rounds, k, V)).astype(np.float16)
+    draft_dev = hip.DeviceBuffer(draft_host.nbytes).upload(draft_host)
+    row_bytes = k * V * 2
+    feeds, draw_steps = [], []
+    for r in range(rounds):
+        props, ds = eng.draft_chain((draft_dev.address(r * row_bytes), k), shaping[r], 0)
+        feeds.append([anchor] + [int(t) for t in props])
+        draw_steps.append(ds)
+
+    def step(r):
+        res = eng.verify_accept(feeds[r], base, shaping[r],
+                                draft_logits=draft_dev.address(r * row_bytes) if T > 0 else None,
+                                draw_step=draw_steps[r])
+        eng.rollback(point)   # every step verifies at exactly `ctx` tokens of context
+        return res
+
+    for r in range(args.warmup):
+        step(r)
+    stream = eng.stream
+    e0, e1 = hip.Event(), hip.Event()
+    hip.check(hip.rt().hipStreamSynchronize(stream), "sync")
+    e0.record(stream)
+    t0 = time.perf_counter()
+    results = [step(args.warmup + i) for i in range(args.steps)]
+    hip.check(hip.rt().hipStreamSynchronize(stream), "sync")
+    wall = time.perf_counter() - t0
+    e1.record(stream)
+    e1.sync()
+    gpu_ms = e1.ms_since(e0)
+    verified = sum(r.accepted + 1 for r in results)
+    mean_acc = float(np.mean([r.accepted for r in results]))
+    min_margin = min(r.min_margin for r in results)
+    ms_per_step = wall * 1000.0 / args.steps
+
+    # per-kernel-class durations, HIP events around every launch on the engine's stream
+    eng.set_profile(True)
+    nprof = min(5, args.steps)
+    for i in range(nprof):
+        step(args.warmup + i)
+    prof = eng.get_profile()
+    eng.set_profile(False)
+    ab = algorithmic_bytes(cfg, ctx, m)
+    L = cfg["n_layers"]
+    kern = {}
+    for name, nbytes, count in (("qkv", ab["per_layer"]["qkv"], L), ("wo", ab["per_layer"]["wo"], L),
+                                ("gate_up", ab["per_layer"]["gate_up"], L), ("down", ab["per_layer"]["down"], L),
+                                ("head", ab["head"], 1), ("attention", ab["kv"] // L, L)):
+        ms, launches = prof[name]
+        if launches:
+            avg_ms = ms / launches
+            kern[name] = dict(avg_us=round(avg_ms * 1000, 2), GBps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
+                              bytes=int(nbytes), launches_per_step=launches // nprof)
+    gemm_ms = sum(prof[n][0] for n in ("qkv", "wo", "gate_up", "down", "head")) / nprof
+    dom = kern.get("gate_up", {})
+    peak = 8000.0
+    roofline = dict(bound="hbm", kernel="k_gemm<Q4_K> gate/up (silu-mul epilogue)" if cfg["dtype"] == 12 else "k_gemm<Q8_0> gate/up",
+                    achieved=dom.get("GBps"), peak=peak, unit="GB/s",
+                    frac=round(dom.get("GBps", 0.0) / peak, 4), traffic=None,
+                    algorithmic_bytes_per_launch=dom.get("bytes"), avg_launch_us=dom.get("avg_us"),
+                    all_matmuls_GBps=round(ab["weights"] / (gemm_ms * 1e-3) / 1e9, 1) if gemm_ms else None,
+                    step_algorithmic_bytes=int(ab["total"]),
+                    step_frac_of_hbm_roofline=round(ab["total"] / (ms_per_step * 1e-3) / 1e9 / peak, 4),
+                    per_kernel=kern,
+                    profile_ms_per_step={n: round(v[0] / nprof, 4) for n, v in prof.items()})
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(cfg, weights, eng, base, feeds[args.warmup], mean_acc)
+
+    out = {
+        "metric": "verified tokens/s + verify-step latency (8B Q4_K, k=4, 4K ctx); % HBM roofline",
+        "value": round(verified / wall, 2), "unit": "verified tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "q4_k weights x f16 activations, f32 accumulate; f64 acceptance" if cfg["dtype"] == 12 else "q8_0 x f16, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,
+                   "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin},
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+
+
+def cpu_baseline(cfg, weights, eng, base, feed, mean_acc):
+    """The oracle (the CPU restatement of the reference path) timed on this host, one thread, on
+    a bounded sample: the first two layers plus the output head of the same verify step, and
+    the head alone; the full-stack time is extrapolated linearly in the layer count."""
+    from oracle import binding as ob
+    L = cfg["n_layers"]
+    sample_layers = min(2, L)
+    cpu = ob.Model(cfg, weights, round_kv_f16=True, threads=1)
+    for layer in range(sample_layers):
+        kg, vg = eng.read_kv(layer, 0, base)
+        kc, vc = cpu.kv(layer)
+        kc[:base] = kg.astype(np.float32)
+        vc[:base] = vg.astype(np.float32)
+    cpu.rewind_to(base)
+    t0 = time.perf_counter()
+    cpu.verify(feed, base, n_layers_run=0)
+    t_head = time.perf_counter() - t0
+    cpu.rewind_to(base)
+    t0 = time.perf_counter()
+    cpu.verify(feed, base, n_layers_run=sample_layers)
+    t_sample = time.perf_counter() - t0
+    t_full = t_head + (t_sample - t_head) * L / sample_layers
+    return {"value": round((mean_acc + 1.0) / t_full, 4), "unit": "verified tokens/s", "cores": 1, "kind": "port",
+            "sample": f"oracle forward of the same verify step, {sample_layers} of {L} layers + output head "
+                      f"({t_sample:.2f}s) and head alone ({t_head:.2f}s), extrapolated to {L} layers = {t_full:.2f}s; "
+                      "acceptance excluded (ms-scale)",
+            "seconds_per_step_extrapolated": round(t_full, 3)}
+
+
+if __name__ == "__main__":
+    main()

@@ -190,6 +190,14 @@ int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16
  * the engine's own split-K factor. */
 int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits);
 
+/* Per-kernel-class timing with HIP events on the handle's stream (one event pair per launch
+ * while enabled).  Classes, in order: embed, norm, qkv matmul, rope+kv store, attention,
+ * output projection, gate/up matmul, down matmul, output head, acceptance.  tsv_get_profile
+ * sums the elapsed milliseconds and launch counts since the last call and clears them. */
+#define TSV_PROFILE_CLASSES 10
+int32_t tsv_set_profile(tsv_ctx* ctx, int32_t on);
+int32_t tsv_get_profile(tsv_ctx* ctx, float* ms, int32_t* counts, int32_t n_classes);
+
 /* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
  * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache
  * slot base+i and sees [0, base) plus the slots of its root path (parent NULL: chain).

@@ -193,24 +193,38 @@ __device__ __forceinline__ int frag_index_a(int k, int row) {
 
 // Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
 // m* = max m_c, D = sum l_c e^{m_c-m*}, O = sum O_c e^{m_c-m*}, out = O / D) and store the row
-// as fp16 activation fragments of the output projection (K index = q_head*hd + d).
+// as fp16 activation fragments of the output projection (K index = q_head*hd + d).  The first
+// wave turns the (m_c, l_c) pairs into per-chunk weights once; every thread then sums its
+// output element over the chunks with independent loads.
 __global__ void k_attn_combine(AttnArgs a, int G, int R) {
+    __shared__ float wgt[64];
+    __shared__ float s_den;
     const int m = blockIdx.x, qh = blockIdx.y, d = threadIdx.x;
-    const int hd = a.hd;
-    if (d >= hd) return;
+    const int hd = a.hd, nch = a.nch;
     const int h = qh / G, g = qh - h * G, r = m * G + g;
-    float mx = -INFINITY;
-    for (int c = 0; c < a.nch; c++) mx = fmaxf(mx, a.part_ml[(((long)h * a.nch + c) * R + r) * 2]);
-    float den = 0.f, num = 0.f;
-    for (int c = 0; c < a.nch; c++) {
-        const long slot = ((long)h * a.nch + c) * R + r;
-        const float mc = a.part_ml[slot * 2];
-        if (mc == -INFINITY) continue;
-        const float w = __expf(mc - mx);
-        den += a.part_ml[slot * 2 + 1] * w;
-        num += a.part_o[slot * hd + d] * w;
+    if (d < 64) {
+        float mc = -INFINITY, lc = 0.f;
+        if (d < nch) {
+            const long slot = ((long)h * nch + d) * R + r;
+            mc = a.part_ml[slot * 2];
+            lc = a.part_ml[slot * 2 + 1];
+        }
+        float mx = mc;
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        const float w = mc > -INFINITY ? __expf(mc - mx) : 0.f;
+        float den = lc * w;
+        for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+        wgt[d] = w;
+        if (d == 0) s_den = den;
     }
-    ((_Float16*)a.xfrag)[frag_index_a(qh * hd + d, m)] = (_Float16)(num / den);
+    __syncthreads();
+    if (d >= hd) return;
+    const float* po = a.part_o + ((long)h * nch * R + r) * hd + d;
+    const long stride = (long)R * hd;
+    float num = 0.f;
+#pragma unroll 8
+    for (int c = 0; c < nch; c++) num += wgt[c] * po[c * stride];
+    ((_Float16*)a.xfrag)[frag_index_a(qh * hd + d, m)] = (_Float16)(num / s_den);
 }
 
 template <int HD>
@@ -224,7 +238,7 @@ static int launch_hd(hipStream_t s, const AttnArgs& a, int m, int G, int R) {
         hipLaunchKernelGGL((k_attn_partial<HD, 4>), dim3(a.nch, a.nkv, (trt + 3) / 4), dim3(256), 0, s, a, G, R);
     }
     TSV_HIP(hipGetLastError());
-    hipLaunchKernelGGL(k_attn_combine, dim3(m, a.nq), dim3(HD), 0, s, a, G, R);
+    hipLaunchKernelGGL(k_attn_combine, dim3(m, a.nq), dim3(HD < 64 ? 64 : HD), 0, s, a, G, R);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -250,7 +250,7 @@ __device__ __forceinline__ int frag_off(int e, int row) {
 template <class F, int MPAD, int EPI>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     extern __shared__ uint4 lds[];
-    constexpr int STAGES = 3;
+    constexpr int STAGES = 4;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int split = blockIdx.x % a.splits, grp = blockIdx.x / a.splits;
     const int tile = grp * 4 + wave;
@@ -260,10 +260,15 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     const uint8_t* wt = a.w + ((size_t)tile * a.kchunks + c0) * F::TILE_BYTES;
     const int m = a.vp->m;
 
+    // Software pipeline over the K chunks, STAGES tiles in flight per wave.  Every load in the
+    // steady state is unconditional (straight-line code), so the compiler can wait on the oldest
+    // outstanding tile only (s_waitcnt vmcnt(n)) instead of draining the queue.
     typename F::Regs st[STAGES];
+    const int last = max(nc - 1, 0);
+    if (active) {
 #pragma unroll
-    for (int s = 0; s < STAGES; s++)
-        if (active && s < nc) F::load(st[s], wt + (size_t)s * F::TILE_BYTES, lane);
+        for (int s = 0; s < STAGES; s++) F::load(st[s], wt + (size_t)min(s, last) * F::TILE_BYTES, lane);
+    }
 
     // stage this K slice of the activations: [sub][kg][MPAD rows] x 16 B, then their sums
     const int nsub = nc * F::NSUB, sub0 = c0 * F::NSUB;
@@ -289,16 +294,26 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 
     float4v acc = {0.f, 0.f, 0.f, 0.f};
     if (active) {
-        for (int c = 0; c < nc; c += STAGES) {
+        int c = 0;
+        for (; c + 2 * STAGES <= nc; c += STAGES) {
 #pragma unroll
             for (int s = 0; s < STAGES; s++) {
-                if (c + s < nc) {
-                    compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
-                    if (c + s + STAGES < nc)
-                        F::load(st[s], wt + (size_t)(c + s + STAGES) * F::TILE_BYTES, lane);
-                }
+                compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
+                F::load(st[s], wt + (size_t)(c + s + STAGES) * F::TILE_BYTES, lane);
             }
         }
+        // last group that still has tiles to fetch (fewer than STAGES of them)
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) {
+            if (c + s < nc) {
+                compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
+                if (c + s + STAGES < nc) F::load(st[s], wt + (size_t)(c + s + STAGES) * F::TILE_BYTES, lane);
+            }
+        }
+        c += STAGES;
+#pragma unroll
+        for (int s = 0; s < STAGES; s++)
+            if (c + s < nc) compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
     }
 
     const int j = lane & 15, kg = lane >> 4;

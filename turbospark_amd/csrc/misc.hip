@@ -80,29 +80,44 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // x[m] += sum over split-K partials of the previous matmul (fixed order: deterministic), then
 // y = x * w / sqrt(mean x^2 + eps) (crates/compute/src/rms_norm.rs:5-14) stored as the next
-// matmul's fp16 activation fragments.  One workgroup per row.
-__global__ __launch_bounds__(256) void k_addnorm(float* __restrict__ x, const float* __restrict__ partial,
-                                                 int splits, int ldp, const float* __restrict__ w,
-                                                 float eps, int hidden, _Float16* __restrict__ xfrag) {
-    __shared__ float red[8];
+// matmul's fp16 activation fragments.  One workgroup per row, four consecutive elements per
+// thread so every load of a row is issued before the first one is waited on.
+__global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const float* __restrict__ partial,
+                                                  int splits, int ldp, const float* __restrict__ w,
+                                                  float eps, int hidden, _Float16* __restrict__ xfrag) {
+    __shared__ float red[16];
     const int m = blockIdx.x;
-    float* xr = x + (long)m * hidden;
+    float4* xr = (float4*)(x + (long)m * hidden);
+    const float4* wr = (const float4*)w;
+    const int n4 = hidden >> 2;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < hidden; i += 256) {
-        float v = xr[i];
-        for (int s = 0; s < splits; s++) v += partial[((long)s * 16 + m) * ldp + i];
+    for (int i = threadIdx.x; i < n4; i += 1024) {
+        float4 v = xr[i];
+        for (int s = 0; s < splits; s++) {
+            const float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
+            v.x += p.x;
+            v.y += p.y;
+            v.z += p.z;
+            v.w += p.w;
+        }
         xr[i] = v;
-        ss += v * v;
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
-    for (int i = threadIdx.x; i < hidden; i += 256)
-        xfrag[frag_index(i, m)] = (_Float16)(xr[i] * w[i] * inv);
+    for (int i = threadIdx.x; i < n4; i += 1024) {
+        const float4 v = xr[i], g = wr[i];
+        // elements 4i..4i+3 sit in one half of an 8-slice; fragment order there is (0, 2, 1, 3)
+        typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+        half4 h = {(_Float16)(v.x * g.x * inv), (_Float16)(v.z * g.z * inv), (_Float16)(v.y * g.y * inv),
+                   (_Float16)(v.w * g.w * inv)};
+        *(half4*)(xfrag + frag_index(4 * i, m)) = h;
+    }
 }
 
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
                    float eps, int hidden, uint4* xfrag, int m) {
-    hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(256), 0, s, x, partial, splits, ldp, w, eps, hidden,
+    hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
                        (_Float16*)xfrag);
     TSV_HIP(hipGetLastError());
     return TSV_OK;

@@ -55,6 +55,11 @@ struct tsv_ctx {
     int64_t position = 0;
     int last_m = 0;
     int64_t last_base = -1;
+    // per-kernel-class timing (tsv_set_profile): one event pair per launch
+    bool profile = false;
+    std::vector<hipEvent_t> ev;
+    std::vector<int> ev_class;
+    size_t ev_used = 0;
 };
 
 namespace {
@@ -207,6 +212,31 @@ int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
     return TSV_OK;
 }
 
+enum { PC_EMBED = 0, PC_NORM, PC_QKV, PC_ROPE, PC_ATTN, PC_WO, PC_GATEUP, PC_DOWN, PC_HEAD, PC_ACCEPT, PC_COUNT };
+
+struct ProfScope {
+    tsv_ctx* c;
+    ProfScope(tsv_ctx* c_, int cls) : c(c_) {
+        if (!c->profile) return;
+        if (c->ev_used + 2 > c->ev.size()) {
+            for (int i = 0; i < 2; i++) {
+                hipEvent_t e;
+                (void)hipEventCreate(&e);
+                c->ev.push_back(e);
+                c->ev_class.push_back(0);
+            }
+        }
+        c->ev_class[c->ev_used] = cls;
+        (void)hipEventRecord(c->ev[c->ev_used], c->stream);
+    }
+    ~ProfScope() {
+        if (!c->profile) return;
+        (void)hipEventRecord(c->ev[c->ev_used + 1], c->stream);
+        c->ev_used += 2;
+    }
+};
+#define PROF(cls) ProfScope prof_scope_(c, cls)
+
 int fill_params(VerifyParams& vp, const int32_t* feed, const int32_t* parent, int m, int64_t base, int vocab) {
     std::memset(&vp, 0, sizeof vp);
     vp.m = m;
@@ -264,16 +294,27 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     *c->vp_host = vp;
     TSV_HIP(hipMemcpyAsync(c->vp_dev, c->vp_host, sizeof vp, hipMemcpyHostToDevice, s));
 
-    int rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m);
+    int rc;
+    {
+        PROF(PC_EMBED);
+        rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m);
+    }
     if (rc) return rc;
     int prev_splits = 0;
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
-        if ((rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m)))
-            return rc;
+        {
+            PROF(PC_NORM);
+            rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m);
+        }
+        if (rc) return rc;
         int sp = splits_for(L.qkv, m, EPI_PARTIAL);
-        if ((rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n))) return rc;
+        {
+            PROF(PC_QKV);
+            rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n);
+        }
+        if (rc) return rc;
         RopeKvArgs ra;
         ra.qkv = c->partial;
         ra.splits = sp;
@@ -290,7 +331,11 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
         ra.hd = c->hd;
         ra.max_ctx = c->ctx_alloc;
         ra.vp = c->vp_dev;
-        if ((rc = launch_rope_kv(s, ra, m))) return rc;
+        {
+            PROF(PC_ROPE);
+            rc = launch_rope_kv(s, ra, m);
+        }
+        if (rc) return rc;
         AttnArgs aa;
         aa.q16 = c->q16;
         aa.kc = L.kc;
@@ -305,18 +350,45 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
         aa.nch = c->nch;
         aa.scale = c->attn_scale;
         aa.vp = c->vp_dev;
-        if ((rc = launch_attention(s, aa, m))) return rc;
+        {
+            PROF(PC_ATTN);
+            rc = launch_attention(s, aa, m);
+        }
+        if (rc) return rc;
         sp = splits_for(L.wo, m, EPI_PARTIAL);
-        if ((rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden))) return rc;
-        if ((rc = launch_addnorm(s, c->x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m))) return rc;
-        if ((rc = launch_gemm(s, L.gate_up, c->xf_a, c->xf_c, c->vp_dev, m, 1, EPI_SILU, 0, 0))) return rc;
+        {
+            PROF(PC_WO);
+            rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
+        }
+        if (rc) return rc;
+        {
+            PROF(PC_NORM);
+            rc = launch_addnorm(s, c->x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m);
+        }
+        if (rc) return rc;
+        {
+            PROF(PC_GATEUP);
+            rc = launch_gemm(s, L.gate_up, c->xf_a, c->xf_c, c->vp_dev, m, 1, EPI_SILU, 0, 0);
+        }
+        if (rc) return rc;
         sp = splits_for(L.down, m, EPI_PARTIAL);
-        if ((rc = launch_gemm(s, L.down, c->xf_c, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden))) return rc;
+        {
+            PROF(PC_DOWN);
+            rc = launch_gemm(s, L.down, c->xf_c, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
+        }
+        if (rc) return rc;
         prev_splits = sp;
     }
-    if ((rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m)))
-        return rc;
-    if ((rc = launch_gemm(s, c->head, c->xf_a, c->logits, c->vp_dev, m, 1, EPI_LOGITS, c->vocab, c->vocab))) return rc;
+    {
+        PROF(PC_NORM);
+        rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m);
+    }
+    if (rc) return rc;
+    {
+        PROF(PC_HEAD);
+        rc = launch_gemm(s, c->head, c->xf_a, c->logits, c->vp_dev, m, 1, EPI_LOGITS, c->vocab, c->vocab);
+    }
+    if (rc) return rc;
     c->position = base + m;
     c->last_m = m;
     c->last_base = base;
@@ -482,8 +554,35 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
+    for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
+}
+
+extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    c->profile = on != 0;
+    c->ev_used = 0;
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_get_profile(tsv_ctx* c, float* ms, int32_t* counts, int32_t n_classes) {
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    for (int i = 0; i < n_classes; i++) {
+        ms[i] = 0.f;
+        counts[i] = 0;
+    }
+    for (size_t i = 0; i + 1 < c->ev_used; i += 2) {
+        float t = 0.f;
+        TSV_HIP(hipEventElapsedTime(&t, c->ev[i], c->ev[i + 1]));
+        const int cls = c->ev_class[i];
+        if (cls < n_classes) {
+            ms[cls] += t;
+            counts[cls] += 1;
+        }
+    }
+    c->ev_used = 0;
+    return TSV_OK;
 }
 
 extern "C" void* tsv_stream(tsv_ctx* c) { return c ? (void*)c->stream : nullptr; }
@@ -637,7 +736,11 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     TSV_HIP(hipStreamSynchronize(c->stream));  // pinned parameter block is about to be rewritten
     if ((rc = fill_accept(c, r, c->ap_host))) return rc;
     TSV_HIP(hipMemcpyAsync(c->ap_dev, c->ap_host, sizeof(AcceptParams), hipMemcpyHostToDevice, c->stream));
-    if ((rc = launch_accept(c->stream, c->logits, draft, c->ap_dev, *c->ap_host, c->sc))) return rc;
+    {
+        PROF(PC_ACCEPT);
+        rc = launch_accept(c->stream, c->logits, draft, c->ap_dev, *c->ap_host, c->sc);
+    }
+    if (rc) return rc;
     TSV_HIP(hipMemcpyAsync(c->res_host, c->sc.result, sizeof(AcceptResult), hipMemcpyDeviceToHost, c->stream));
     if (r->logits_out)
         TSV_HIP(hipMemcpyAsync(r->logits_out, c->logits, (size_t)r->m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));

@@ -101,7 +101,7 @@ EXPORTS = [
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
-    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention",
+    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile",
 ]
 
 _lib = None
@@ -147,6 +147,8 @@ def lib():
         L.tsv_matmul.argtypes = [C.POINTER(Tensor), C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
         L.tsv_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                     C.c_int64, C.c_void_p, C.c_float, C.c_void_p]
+        L.tsv_set_profile.argtypes = [C.c_void_p, C.c_int32]
+        L.tsv_get_profile.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]
         L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
         _lib = L
     return _lib

@@ -206,6 +206,19 @@ class HipVerifier:
         ffi.check(ffi.lib().tsv_draft_chain(self._h, ptr, k, C.byref(cfg), C.byref(ds), props.ctypes.data))
         return props, ds.value
 
+    PROFILE_CLASSES = ("embed", "norm", "qkv", "rope_kv", "attention", "wo", "gate_up", "down", "head", "accept")
+
+    def set_profile(self, on):
+        ffi.check(ffi.lib().tsv_set_profile(self._h, int(bool(on))))
+
+    def get_profile(self):
+        """{class: (total ms, launches)} since the last call (HIP events around every launch)."""
+        n = len(self.PROFILE_CLASSES)
+        ms = np.zeros(n, np.float32)
+        cnt = np.zeros(n, np.int32)
+        ffi.check(ffi.lib().tsv_get_profile(self._h, ms.ctypes.data, cnt.ctypes.data, n))
+        return {k: (float(ms[i]), int(cnt[i])) for i, k in enumerate(self.PROFILE_CLASSES)}
+
     # ---- test introspection ------------------------------------------------------------------
     def read_kv(self, layer, pos0, n):
         c = self.cfg
