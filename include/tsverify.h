@@ -198,6 +198,13 @@ int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int
 int32_t tsv_set_profile(tsv_ctx* ctx, int32_t on);
 int32_t tsv_get_profile(tsv_ctx* ctx, float* ms, int32_t* counts, int32_t n_classes);
 
+/* Measurement hook (no reference counterpart): average microseconds of `iters` back-to-back
+ * launches of the verify matmul kernel on a rows x cols weight of `dtype` with m activation
+ * rows; epi 0 = split-K partials, 1 = silu(gate)*up over interleaved tiles, 2 = fp16 logits;
+ * `rotate` weight copies are cycled so the bytes come from HBM. */
+int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
+                        int32_t iters, int32_t rotate, float* avg_us);
+
 /* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
  * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache
  * slot base+i and sees [0, base) plus the slots of its root path (parent NULL: chain).

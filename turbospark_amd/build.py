@@ -9,6 +9,8 @@ LIB = os.path.join(HERE, "libtsverify.so")
 SOURCES = ["gemm.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip"]
 # host_utils.hip is host-only code; clang 22 -O3 does not terminate on it, -O2 does.
 OPT = {"host_utils.hip": "-O2"}
+# MFMA results straight into VGPRs (no v_accvgpr_read copies before the scaling FMAs)
+EXTRA = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 FLAGS = [
     "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed-fp32 VALU forms are switched off for every kernel in this library
@@ -23,7 +25,7 @@ def build(verbose=False):
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
     for src in SOURCES:
         obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
-        cmd = ["hipcc", OPT.get(src, "-O3"), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = ["hipcc", OPT.get(src, "-O3"), *FLAGS, *EXTRA.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))

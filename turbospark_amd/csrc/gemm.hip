@@ -19,6 +19,8 @@
 //    ([0,2,1,3,4,6,5,7]); the activations are stored pre-permuted instead of shuffling weights;
 //  * weights are re-tiled once at load so each wave-wide load is 1 KiB contiguous (16 B per
 //    lane); activations for the workgroup's K slice are staged once in LDS and shared by its waves.
+#include <algorithm>
+
 #include "tsv_internal.h"
 
 namespace tsv {
@@ -161,80 +163,107 @@ __device__ __forceinline__ float ubyte(uint32_t v, int i) { return (float)((v >>
 __device__ __forceinline__ half8 as_half8(uint4 v) { return __builtin_bit_cast(half8, v); }
 __device__ __forceinline__ half8 as_half8(u32x4 v) { return __builtin_bit_cast(half8, v); }
 
-template <int MPAD>
-__device__ __forceinline__ void fma_sub(float4v& acc, const float4v& D, float sj, float cj,
-                                        const float* xs, int lsub, int kg) {
-    // activation sums of this lane's four batch rows (rows >= MPAD alias lower rows: their
-    // results are never stored)
-    const float4v x4 = *(const float4v*)(xs + lsub * MPAD + ((4 * kg) & (MPAD - 1)));
-    acc.x += sj * D.x - cj * x4.x;
-    acc.y += sj * D.y - cj * x4.y;
-    acc.z += sj * D.z - cj * x4.z;
-    acc.w += sj * D.w - cj * x4.w;
+// (v & mask) | bits as ONE v_and_or_b32: the instruction can take a single literal / scalar
+// operand, so the second constant is pinned in a vector register.
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits_vgpr) {
+    return (v & mask) | bits_vgpr;
 }
 
-template <int MPAD>
-__device__ __forceinline__ void compute(const Q4K::Regs& r, const uint4* xf, const float* xs, int lc,
-                                        int lane, float4v& acc) {
-    const int kg = lane >> 4, row = lane & (MPAD - 1);
+struct Consts {
+    uint32_t k6400, k5400, k64;
+};
+
+// One Q4_K superblock tile (16 weight rows x 256 K) against the staged activations.
+//   acc  += sum_j d*sc_j * (X_j . (off_j + q_j))          8 x v_mfma_f32_16x16x32_f16 + 4 FMAs each
+//   acc  -= sum_j (d*sc_j*off_j + dmin*m_j) * sum_k X_jk   2 x v_mfma_f32_16x16x4_f32 (fp32 operands,
+//           K index = sub-block: lane group kg supplies sub-blocks kg and 4+kg)
+// Both parts are summed per tile first so the large code offsets cancel before they reach the
+// running accumulator.
+__device__ __forceinline__ void compute(const Q4K::Regs& r, const uint4* xf, const float* xs, int lc, int lane,
+                                        int M, int rowA, const Consts& k, float4v& acc) {
+    const int kg = lane >> 4;
+    float4v t;  // this tile's contribution: starts at the (negative) offset term, ends small
     const float d = h2f_lo(r.s.x), dmin = h2f_hi(r.s.x);
     // 6-bit scale / min unpack (q4_k.rs:43-54), four sub-blocks per 32-bit word
     const uint32_t sl = r.s.y & 0x3F3F3F3Fu, ml = r.s.z & 0x3F3F3F3Fu;
     const uint32_t sh = (r.s.w & 0x0F0F0F0Fu) | ((r.s.y >> 2) & 0x30303030u);
     const uint32_t mh = ((r.s.w >> 4) & 0x0F0F0F0Fu) | ((r.s.z >> 2) & 0x30303030u);
     const float4v zero = {0.f, 0.f, 0.f, 0.f};
+    // min / offset term: this lane's two sub-blocks are kg (from sl/ml) and 4+kg (from sh/mh);
+    // even sub-blocks carry the 1024 code offset, odd ones 64.
+    {
+        const float off = (kg & 1) ? 64.0f : 1024.0f;
+        const float s0 = d * (float)((sl >> (8 * kg)) & 0xFFu), s1 = d * (float)((sh >> (8 * kg)) & 0xFFu);
+        const float c0 = __builtin_fmaf(s0, off, dmin * (float)((ml >> (8 * kg)) & 0xFFu));
+        const float c1 = __builtin_fmaf(s1, off, dmin * (float)((mh >> (8 * kg)) & 0xFFu));
+        const float x0 = xs[(lc * 8 + kg) * M + rowA], x1 = xs[(lc * 8 + 4 + kg) * M + rowA];
+        t = __builtin_amdgcn_mfma_f32_16x16x4f32(x0, -c0, zero, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_16x16x4f32(x1, -c1, t, 0, 0, 0);
+    }
 #pragma unroll
     for (int g = 0; g < 4; g++) {
         const uint32_t w0 = g == 0 ? r.q0.x : g == 1 ? r.q0.z : g == 2 ? r.q1.x : r.q1.z;
         const uint32_t w1 = g == 0 ? r.q0.y : g == 1 ? r.q0.w : g == 2 ? r.q1.y : r.q1.w;
-        const uint32_t sw = g < 2 ? sl : sh, mw = g < 2 ? ml : mh;
+        const uint32_t sw = g < 2 ? sl : sh;
         const int b0 = (2 * g) & 3;
         const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
         // low nibbles: sub-block 2g, codes as 1024+q
         {
-            uint4 b = make_uint4((w0 & 0x000F000Fu) | 0x64006400u, (v0 & 0x000F000Fu) | 0x64006400u,
-                                 (w1 & 0x000F000Fu) | 0x64006400u, (v1 & 0x000F000Fu) | 0x64006400u);
-            const int lsub = lc * 8 + 2 * g;
-            const uint4 a = xf[(lsub * 4 + kg) * MPAD + row];
-            float4v D = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a), as_half8(b), zero, 0, 0, 0);
+            uint4 b = make_uint4(and_or(w0, 0x000F000Fu, k.k6400), and_or(v0, 0x000F000Fu, k.k6400),
+                                 and_or(w1, 0x000F000Fu, k.k6400), and_or(v1, 0x000F000Fu, k.k6400));
+            const uint4 a = xf[((lc * 8 + 2 * g) * 4 + kg) * M + rowA];
+            const float4v D = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a), as_half8(b), zero, 0, 0, 0);
             const float sj = d * ubyte(sw, b0);
-            const float cj = sj * 1024.0f + dmin * ubyte(mw, b0);
-            fma_sub<MPAD>(acc, D, sj, cj, xs, lsub, kg);
+            t.x = __builtin_fmaf(sj, D.x, t.x);
+            t.y = __builtin_fmaf(sj, D.y, t.y);
+            t.z = __builtin_fmaf(sj, D.z, t.z);
+            t.w = __builtin_fmaf(sj, D.w, t.w);
         }
         // high nibbles: sub-block 2g+1, codes as 64+q
         {
-            uint4 b = make_uint4((w0 & 0x00F000F0u) | 0x54005400u, (v0 & 0x00F000F0u) | 0x54005400u,
-                                 (w1 & 0x00F000F0u) | 0x54005400u, (v1 & 0x00F000F0u) | 0x54005400u);
-            const int lsub = lc * 8 + 2 * g + 1;
-            const uint4 a = xf[(lsub * 4 + kg) * MPAD + row];
-            float4v D = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a), as_half8(b), zero, 0, 0, 0);
+            uint4 b = make_uint4(and_or(w0, 0x00F000F0u, k.k5400), and_or(v0, 0x00F000F0u, k.k5400),
+                                 and_or(w1, 0x00F000F0u, k.k5400), and_or(v1, 0x00F000F0u, k.k5400));
+            const uint4 a = xf[((lc * 8 + 2 * g + 1) * 4 + kg) * M + rowA];
+            const float4v D = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a), as_half8(b), zero, 0, 0, 0);
             const float sj = d * ubyte(sw, b0 + 1);
-            const float cj = sj * 64.0f + dmin * ubyte(mw, b0 + 1);
-            fma_sub<MPAD>(acc, D, sj, cj, xs, lsub, kg);
+            t.x = __builtin_fmaf(sj, D.x, t.x);
+            t.y = __builtin_fmaf(sj, D.y, t.y);
+            t.z = __builtin_fmaf(sj, D.z, t.z);
+            t.w = __builtin_fmaf(sj, D.w, t.w);
         }
     }
+    acc += t;
 }
 
-template <int MPAD>
-__device__ __forceinline__ void compute(const Q80::Regs& r, const uint4* xf, const float* xs, int lc,
-                                        int lane, float4v& acc) {
-    const int kg = lane >> 4, row = lane & (MPAD - 1);
+// One Q8_0 tile (16 rows x 128 K = four 32-element blocks).  Codes go in as 1024 + (q + 128);
+// the 1152 offset comes back out through the activation sums on the fp32 matrix pipe.
+__device__ __forceinline__ void compute(const Q80::Regs& r, const uint4* xf, const float* xs, int lc, int lane,
+                                        int M, int rowA, const Consts& k, float4v& acc) {
+    const int kg = lane >> 4;
+    float4v t;
     const float4v zero = {0.f, 0.f, 0.f, 0.f};
-    const uint32_t c64 = 0x64646464u;
+    {
+        const uint32_t sw = kg < 2 ? r.s.x : r.s.y;
+        const float dk = (kg & 1) ? h2f_hi(sw) : h2f_lo(sw);  // block kg's scale
+        t = __builtin_amdgcn_mfma_f32_16x16x4f32(xs[(lc * 4 + kg) * M + rowA], dk * -1152.0f, zero, 0, 0, 0);
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const uint32_t w0 = (j == 0 ? r.q0.x : j == 1 ? r.q0.z : j == 2 ? r.q1.x : r.q1.z) ^ 0x80808080u;
         const uint32_t w1 = (j == 0 ? r.q0.y : j == 1 ? r.q0.w : j == 2 ? r.q1.y : r.q1.w) ^ 0x80808080u;
         // bytes -> fp16 1024 + (q + 128): interleave each byte with 0x64
-        uint4 b = make_uint4(__builtin_amdgcn_perm(c64, w0, 0x04020400u), __builtin_amdgcn_perm(c64, w0, 0x04030401u),
-                             __builtin_amdgcn_perm(c64, w1, 0x04020400u), __builtin_amdgcn_perm(c64, w1, 0x04030401u));
-        const int lsub = lc * 4 + j;
-        const uint4 a = xf[(lsub * 4 + kg) * MPAD + row];
-        float4v D = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a), as_half8(b), zero, 0, 0, 0);
+        uint4 b = make_uint4(__builtin_amdgcn_perm(k.k64, w0, 0x04020400u), __builtin_amdgcn_perm(k.k64, w0, 0x04030401u),
+                             __builtin_amdgcn_perm(k.k64, w1, 0x04020400u), __builtin_amdgcn_perm(k.k64, w1, 0x04030401u));
+        const uint4 a = xf[((lc * 4 + j) * 4 + kg) * M + rowA];
+        const float4v D = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a), as_half8(b), zero, 0, 0, 0);
         const uint32_t sw = j < 2 ? r.s.x : r.s.y;
         const float dj = (j & 1) ? h2f_hi(sw) : h2f_lo(sw);
-        fma_sub<MPAD>(acc, D, dj, dj * 1152.0f, xs, lsub, kg);
+        t.x = __builtin_fmaf(dj, D.x, t.x);
+        t.y = __builtin_fmaf(dj, D.y, t.y);
+        t.z = __builtin_fmaf(dj, D.z, t.z);
+        t.w = __builtin_fmaf(dj, D.w, t.w);
     }
+    acc += t;
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
@@ -247,7 +276,10 @@ __device__ __forceinline__ int frag_off(int e, int row) {
     return (kg * 16 + row) * 8 + p;
 }
 
-template <class F, int MPAD, int EPI>
+// LDS bytes per 32-element sub-block of a K slice for m activation rows: fp16 fragments + fp32 sums.
+__host__ __device__ inline int lds_per_sub(int m) { return 4 * m * 16 + m * 4; }
+
+template <class F, int EPI>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     extern __shared__ uint4 lds[];
     constexpr int STAGES = 4;
@@ -258,7 +290,13 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     const int nc = min(a.kslice, a.kchunks - c0);
     const bool active = tile < a.n_tiles && nc > 0;
     const uint8_t* wt = a.w + ((size_t)tile * a.kchunks + c0) * F::TILE_BYTES;
-    const int m = a.vp->m;
+    const int M = a.vp->m;
+    const int rowA = min(lane & 15, M - 1);  // padding rows of the A operand alias the last real row
+    Consts k;
+    k.k6400 = 0x64006400u;
+    k.k5400 = 0x54005400u;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
 
     // Software pipeline over the K chunks, STAGES tiles in flight per wave.  Every load in the
     // steady state is unconditional (straight-line code), so the compiler can wait on the oldest
@@ -270,21 +308,21 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
         for (int s = 0; s < STAGES; s++) F::load(st[s], wt + (size_t)min(s, last) * F::TILE_BYTES, lane);
     }
 
-    // stage this K slice of the activations: [sub][kg][MPAD rows] x 16 B, then their sums
+    // stage this K slice of the activations: [sub][kg][M rows] x 16 B, then their per-sub-block sums
     const int nsub = nc * F::NSUB, sub0 = c0 * F::NSUB;
     uint4* xf = lds;
-    float* xs = (float*)(lds + a.kslice * F::NSUB * 4 * MPAD);
-    for (int u = tid; u < nsub * 4 * MPAD; u += 256) {
-        const int row = u % MPAD, t = u / MPAD;
+    float* xs = (float*)(lds + a.kslice * F::NSUB * 4 * M);
+    for (int u = tid; u < nsub * 4 * M; u += 256) {
+        const int row = u % M, t = u / M;
         xf[u] = a.xfrag[((size_t)(sub0 * 4 + t)) * 16 + row];
     }
     __syncthreads();
-    for (int v = tid; v < nsub * MPAD; v += 256) {
-        const int row = v % MPAD, ls = v / MPAD;
+    for (int v = tid; v < nsub * M; v += 256) {
+        const int row = v % M, ls = v / M;
         float s = 0.f;
 #pragma unroll
         for (int kg = 0; kg < 4; kg++) {
-            const half8 h = as_half8(xf[(ls * 4 + kg) * MPAD + row]);
+            const half8 h = as_half8(xf[(ls * 4 + kg) * M + row]);
 #pragma unroll
             for (int i = 0; i < 8; i++) s += (float)h[i];
         }
@@ -298,7 +336,7 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
         for (; c + 2 * STAGES <= nc; c += STAGES) {
 #pragma unroll
             for (int s = 0; s < STAGES; s++) {
-                compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
+                compute(st[s], xf, xs, c + s, lane, M, rowA, k, acc);
                 F::load(st[s], wt + (size_t)(c + s + STAGES) * F::TILE_BYTES, lane);
             }
         }
@@ -306,18 +344,19 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
         for (int s = 0; s < STAGES; s++) {
             if (c + s < nc) {
-                compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
+                compute(st[s], xf, xs, c + s, lane, M, rowA, k, acc);
                 if (c + s + STAGES < nc) F::load(st[s], wt + (size_t)(c + s + STAGES) * F::TILE_BYTES, lane);
             }
         }
         c += STAGES;
 #pragma unroll
         for (int s = 0; s < STAGES; s++)
-            if (c + s < nc) compute<MPAD>(st[s], xf, xs, c + s, lane, acc);
+            if (c + s < nc) compute(st[s], xf, xs, c + s, lane, M, rowA, k, acc);
     }
 
     const int j = lane & 15, kg = lane >> 4;
     const int n = tile * 16 + j;
+    const int m = M;
     if (EPI == EPI_PARTIAL) {
         if (!active) return;
         float* out = (float*)a.out + (size_t)split * 16 * a.ldo;
@@ -357,8 +396,7 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 
 int gemm_default_splits(const TiledW& w, int m) {
     // Enough workgroups to cover 256 CUs about twice, K slices no shorter than two chunks,
-    // and an LDS footprint that still lets two workgroups share a CU.
-    const int mpad = m <= 4 ? 4 : m <= 8 ? 8 : 16;
+    // and an LDS footprint that still lets several workgroups share a CU.
     const int groups = (w.n_tiles + 3) / 4;
     int splits = 1;
     while (groups * splits < 448 && w.kchunks / (splits * 2) >= 2 && w.kchunks % (splits * 2) == 0) splits *= 2;
@@ -369,44 +407,37 @@ int gemm_default_splits(const TiledW& w, int m) {
                 splits = s;
                 if (groups * s >= 448) break;
             }
-    const int chunk_bytes = fmt_nsub(w.fmt) * (4 * mpad * 16 + mpad * 4);
-    while ((w.kchunks + splits - 1) / splits * chunk_bytes > 72 * 1024) splits++;
+    const int chunk_bytes = fmt_nsub(w.fmt) * lds_per_sub(m);
+    while ((w.kchunks + splits - 1) / splits * chunk_bytes > 76 * 1024) splits++;
     // normalise: every split non-empty
     const int kslice = (w.kchunks + splits - 1) / splits;
     return (w.kchunks + kslice - 1) / kslice;
 }
 
-template <class F, int MPAD, int EPI>
-static int launch_t(hipStream_t s, const GemmArgs& a, int groups) {
-    const size_t lds = (size_t)a.kslice * F::NSUB * (4 * MPAD * 16 + MPAD * 4);
-    static size_t configured = 0;
-    if (lds > 64 * 1024 && lds > configured) {
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm<F, MPAD, EPI>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)(160 * 1024)));
-        configured = 160 * 1024;
+template <class F, int EPI>
+static int launch_t(hipStream_t s, const GemmArgs& a, int groups, int m) {
+    const size_t lds = std::max<size_t>((size_t)a.kslice * F::NSUB * lds_per_sub(m), 2048);
+    static bool configured = false;
+    if (!configured) {
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm<F, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)(160 * 1024)));
+        configured = true;
     }
     if (lds > 160 * 1024) {
         set_error("matmul: activation slice does not fit LDS; raise the split count");
         return TSV_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL((k_gemm<F, MPAD, EPI>), dim3(groups * a.splits), dim3(256), lds, s, a);
+    hipLaunchKernelGGL((k_gemm<F, EPI>), dim3(groups * a.splits), dim3(256), lds, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
-}
-
-template <class F, int EPI>
-static int launch_m(hipStream_t s, const GemmArgs& a, int groups, int m) {
-    if (m <= 4) return launch_t<F, 4, EPI>(s, a, groups);
-    if (m <= 8) return launch_t<F, 8, EPI>(s, a, groups);
-    return launch_t<F, 16, EPI>(s, a, groups);
 }
 
 template <class F>
 static int launch_f(hipStream_t s, const GemmArgs& a, int groups, int m, int epi) {
     switch (epi) {
-        case EPI_PARTIAL: return launch_m<F, EPI_PARTIAL>(s, a, groups, m);
-        case EPI_SILU: return launch_m<F, EPI_SILU>(s, a, groups, m);
-        default: return launch_m<F, EPI_LOGITS>(s, a, groups, m);
+        case EPI_PARTIAL: return launch_t<F, EPI_PARTIAL>(s, a, groups, m);
+        case EPI_SILU: return launch_t<F, EPI_SILU>(s, a, groups, m);
+        default: return launch_t<F, EPI_LOGITS>(s, a, groups, m);
     }
 }
 

@@ -979,3 +979,99 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     (void)hipStreamDestroy(c->stream);
     return rc;
 }
+
+// Measurement hook: average duration (HIP events on a private stream) of `iters` back-to-back
+// launches of the verify pass's matmul over a rows x cols weight of the given dtype filled with
+// pseudo-random block bytes, m activation rows, epilogue `epi` (0 split-K partials, 1 silu-mul over
+// interleaved gate/up tiles, 2 fp16 logits).  `rotate` distinct weight copies are cycled so the
+// kernel streams from HBM rather than from cache.
+extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
+                                   int32_t iters, int32_t rotate, float* avg_us) {
+    const int fmt = dtype_fmt(dtype);
+    if (fmt < 0 || rows % 16 || cols % fmt_chunk_elems(fmt) || m < 1 || m > TSV_MAX_ROWS || iters < 1 || rotate < 1) {
+        set_error("matmul_time: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    tsv_ctx tmp;
+    tsv_ctx* c = &tmp;
+    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    TiledW w;
+    w.fmt = fmt;
+    w.k = (int)cols;
+    w.kchunks = w.k / fmt_chunk_elems(fmt);
+    w.n_rows = (int)rows;
+    w.n_tiles = (int)(rows / 16);
+    w.bytes = (size_t)w.n_tiles * w.kchunks * fmt_tile_bytes(fmt);
+    std::vector<uint8_t*> copies((size_t)rotate);
+    int rc = TSV_OK;
+    {
+        // block bytes: small fp16 scales (0x2xxx) and arbitrary quants
+        std::vector<uint8_t> host(w.bytes);
+        uint64_t sd = 88172645463325252ull;
+        for (size_t i = 0; i < host.size(); i += 8) {
+            sd ^= sd << 13;
+            sd ^= sd >> 7;
+            sd ^= sd << 17;
+            std::memcpy(&host[i], &sd, std::min<size_t>(8, host.size() - i));
+        }
+        const int tb = fmt_tile_bytes(fmt);
+        for (size_t t = 0; t < w.bytes / tb; t++) {
+            uint8_t* sc = &host[t * tb + 2048];
+            if (fmt == FMT_Q4K)
+                for (int r = 0; r < 16; r++) {
+                    sc[r * 16 + 1] = 0x20;
+                    sc[r * 16 + 3] = 0x20;
+                }
+            else
+                for (int i = 0; i < 64; i++) sc[2 * i + 1] = 0x20;
+        }
+        for (int i = 0; i < rotate && !rc; i++) {
+            rc = dev_alloc(c, &copies[i], w.bytes);
+            if (!rc && hipMemcpy(copies[i], host.data(), w.bytes, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
+        }
+    }
+    VerifyParams vp;
+    std::memset(&vp, 0, sizeof vp);
+    vp.m = m;
+    uint4* xf = nullptr;
+    float* out = nullptr;
+    VerifyParams* vpd = nullptr;
+    int sp = 1;
+    if (!rc) {
+        w.tiles = copies[0];
+        sp = epi == EPI_PARTIAL ? (splits > 0 ? splits : gemm_default_splits(w, m)) : 1;
+        const int kslice = (w.kchunks + sp - 1) / sp;
+        sp = (w.kchunks + kslice - 1) / kslice;
+    }
+    if (!rc) rc = dev_alloc(c, &xf, (size_t)std::max<int64_t>(cols, rows) / 32 * 4 * 16 * 16 + 4096, true);
+    if (!rc) rc = dev_alloc(c, &out, (size_t)sp * 16 * rows * 4 + (size_t)rows * 32 * 2, true);
+    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
+    if (!rc && hipMemcpy(vpd, &vp, sizeof vp, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (!rc && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = TSV_ERR_DEVICE;
+    for (int pass = 0; pass < 2 && !rc; pass++) {  // pass 0 warms up
+        if (pass == 1) (void)hipEventRecord(e0, c->stream);
+        for (int i = 0; i < (pass ? iters : std::min(iters, 3)) && !rc; i++) {
+            w.tiles = copies[(size_t)(i % rotate)];
+            rc = launch_gemm(c->stream, w, xf, epi == EPI_SILU ? (void*)(xf + 64) : (void*)out, vpd, m, sp, epi,
+                             (int)rows, (int)rows);
+        }
+        if (pass == 1) (void)hipEventRecord(e1, c->stream);
+    }
+    if (!rc) {
+        if (hipStreamSynchronize(c->stream) != hipSuccess) {
+            set_error("matmul_time: device execution failed");
+            rc = TSV_ERR_DEVICE;
+        } else {
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            *avg_us = ms * 1000.f / (float)iters;
+        }
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipStreamSynchronize(c->stream);
+    for (void* p : c->allocs) (void)hipFree(p);
+    (void)hipStreamDestroy(c->stream);
+    return rc;
+}
