@@ -46,8 +46,38 @@ def algorithmic_bytes(cfg, ctx, m):
     return dict(per_layer=per_layer, head=head, weights=weights, kv=kv, total=weights + kv + small)
 
 
+def trace_summary(path):
+    """Per-kernel statistics of the verify STEPS in a `rocprofv3 --kernel-trace --output-format csv`
+    trace of this script: only dispatches after the first acceptance-statistics kernel are counted,
+    which leaves out weight re-tiling and the 16-row prefill passes that build the KV cache.
+    Kernels are keyed by name and grid size, so the five matmul shapes show up separately."""
+    import csv
+    rows = list(csv.DictReader(open(path)))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    start = next(i for i, r in enumerate(rows) if "k_row_max" in r["Kernel_Name"])
+    stats = {}
+    for r in rows[start:]:
+        name = r["Kernel_Name"].replace("tsv::", "").replace("(anonymous namespace)::", "")
+        name = name.split("(")[0].replace("void ", "")
+        key = (name, int(r["Grid_Size_X"]) // max(int(r["Workgroup_Size_X"]), 1), int(r["LDS_Block_Size"]))
+        d = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+        st = stats.setdefault(key, [0, 0, 10**12, 0])
+        st[0] += 1
+        st[1] += d
+        st[2] = min(st[2], d)
+        st[3] = max(st[3], d)
+    total = sum(v[1] for v in stats.values())
+    print(f"{'kernel':44s} {'wgs':>6s} {'lds':>7s} {'calls':>7s} {'avg_us':>9s} {'min_us':>9s} {'max_us':>9s} {'share':>7s}")
+    for (name, wgs, lds), v in sorted(stats.items(), key=lambda kv: -kv[1][1]):
+        print(f"{name[:44]:44s} {wgs:6d} {lds:7d} {v[0]:7d} {v[1] / v[0] / 1e3:9.2f} {v[2] / 1e3:9.2f} {v[3] / 1e3:9.2f} "
+              f"{100.0 * v[1] / total:6.2f}%")
+    print(f"total kernel time in verify steps: {total / 1e6:.3f} ms over the traced steps")
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--trace-summary", default=None, metavar="CSV",
+                    help="summarise a rocprofv3 kernel-trace CSV of this script (verify steps only) and exit")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -56,6 +86,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=20261125)
     args = ap.parse_args()
+    if args.trace_summary:
+        trace_summary(args.trace_summary)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "
                  "supported (see DESIGN.md, 'how the path would shard').")

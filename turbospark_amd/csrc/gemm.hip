@@ -279,10 +279,18 @@ __device__ __forceinline__ int frag_off(int e, int row) {
 // LDS bytes per 32-element sub-block of a K slice for m activation rows: fp16 fragments + fp32 sums.
 __host__ __device__ inline int lds_per_sub(int m) { return 4 * m * 16 + m * 4; }
 
+#ifndef TSV_GEMM_STAGES
+#define TSV_GEMM_STAGES 4
+#endif
+#ifndef TSV_GEMM_WAVES
+#define TSV_GEMM_WAVES 2
+#endif
+
 template <class F, int EPI>
-__global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TSV_GEMM_WAVES, TSV_GEMM_WAVES)))
+void k_gemm(GemmArgs a) {
     extern __shared__ uint4 lds[];
-    constexpr int STAGES = 4;
+    constexpr int STAGES = TSV_GEMM_STAGES;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int split = blockIdx.x % a.splits, grp = blockIdx.x / a.splits;
     const int tile = grp * 4 + wave;

@@ -5,7 +5,7 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libtsverify.so")
+LIB_PATH = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
 
 F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
 MAX_ROWS = 16
