@@ -185,15 +185,10 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
     }
 }
 
-__device__ __forceinline__ int frag_index_a(int k, int row) {
-    const int sub = k >> 5, e = k & 31, kg = e >> 3, o = e & 7;
-    const int p = (o & 4) | ((o & 1) << 1) | ((o >> 1) & 1);
-    return ((sub * 4 + kg) * 16 + row) * 8 + p;
-}
-
 // Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
 // m* = max m_c, D = sum l_c e^{m_c-m*}, O = sum O_c e^{m_c-m*}, out = O / D) and store the row
-// as fp16 activation fragments of the output projection (K index = q_head*hd + d).  The first
+// as fp16 activation fragments (and sub-block sums) of the output projection (K index =
+// q_head*hd + d).  The first
 // wave turns the (m_c, l_c) pairs into per-chunk weights once; every thread then sums its
 // output element over the chunks with independent loads.
 __global__ void k_attn_combine(AttnArgs a, int G, int R) {
@@ -224,7 +219,13 @@ __global__ void k_attn_combine(AttnArgs a, int G, int R) {
     float num = 0.f;
 #pragma unroll 8
     for (int c = 0; c < nch; c++) num += wgt[c] * po[c * stride];
-    ((_Float16*)a.xfrag)[frag_index_a(qh * hd + d, m)] = (_Float16)(num / s_den);
+    const _Float16 o16 = (_Float16)(num / s_den);
+    const int kk = qh * hd + d;
+    ((_Float16*)a.xfrag)[frag_index(kk, m)] = o16;
+    // sum of each 32-element sub-block of the output projection's input (32 neighbouring threads)
+    float sum = (float)o16;
+    for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
+    if ((d & 31) == 0) ((float*)((char*)a.xfrag + xfrag_sum_offset(a.nq * hd)))[xsum_index(kk >> 5, m)] = sum;
 }
 
 template <int HD>

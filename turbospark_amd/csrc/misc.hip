@@ -8,14 +8,6 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
-__device__ __forceinline__ int frag_index(int k, int row) {
-    // fp16 activation fragments: [k/32][kg = (k%32)/8][16 rows][8], with the order inside each
-    // 8-slice the weight unpack produces ([0,2,1,3,4,6,5,7]).
-    const int sub = k >> 5, e = k & 31, kg = e >> 3, o = e & 7;
-    const int p = (o & 4) | ((o & 1) << 1) | ((o >> 1) & 1);
-    return ((sub * 4 + kg) * 16 + row) * 8 + p;
-}
-
 // ---------------------------------------------------------------- embedding lookup
 // One dequantized table row per fed token (crates/runtime/src/real_forward_dispatch.rs:154),
 // arithmetic of dequantize_q4_k / dequantize_q8_0.
@@ -80,7 +72,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // x[m] += sum over split-K partials of the previous matmul (fixed order: deterministic), then
 // y = x * w / sqrt(mean x^2 + eps) (crates/compute/src/rms_norm.rs:5-14) stored as the next
-// matmul's fp16 activation fragments.  One workgroup per row, four consecutive elements per
+// matmul's fp16 activation fragments plus the sums of the rounded values over every 32-element
+// sub-block (eight neighbouring threads).  One workgroup per row, four consecutive elements per
 // thread so every load of a row is issued before the first one is waited on.
 __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const float* __restrict__ partial,
                                                   int splits, int ldp, const float* __restrict__ w,
@@ -105,13 +98,19 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
     }
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+    float* sums = (float*)((char*)xfrag + xfrag_sum_offset(hidden));
     for (int i = threadIdx.x; i < n4; i += 1024) {
         const float4 v = xr[i], g = wr[i];
-        // elements 4i..4i+3 sit in one half of an 8-slice; fragment order there is (0, 2, 1, 3)
+        // elements 4i..4i+3 are one K step of the fragment layout, stored in the order (0, 2, 1, 3)
         typedef _Float16 half4 __attribute__((ext_vector_type(4)));
         half4 h = {(_Float16)(v.x * g.x * inv), (_Float16)(v.z * g.z * inv), (_Float16)(v.y * g.y * inv),
                    (_Float16)(v.w * g.w * inv)};
         *(half4*)(xfrag + frag_index(4 * i, m)) = h;
+        float sum = ((float)h.x + (float)h.y) + ((float)h.z + (float)h.w);
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        sum += __shfl_xor(sum, 4);
+        if ((i & 7) == 0) sums[xsum_index(i >> 3, m)] = sum;
     }
 }
 
@@ -126,7 +125,12 @@ int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, in
 __global__ void k_f32_to_xfrag(const float* __restrict__ x, int k, _Float16* __restrict__ xfrag) {
     const int m = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < k) xfrag[frag_index(i, m)] = (_Float16)x[(long)m * k + i];
+    if (i >= k) return;  // k is a multiple of 32: whole sub-blocks leave together
+    const _Float16 h = (_Float16)x[(long)m * k + i];
+    xfrag[frag_index(i, m)] = h;
+    float sum = (float)h;
+    for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
+    if ((i & 31) == 0) ((float*)((char*)xfrag + xfrag_sum_offset(k)))[xsum_index(i >> 5, m)] = sum;
 }
 
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m) {

@@ -133,15 +133,16 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
         set_error(std::string(what) + ": matmul weights must be Q4_K or Q8_0 in this build");
         return TSV_ERR_UNSUPPORTED;
     }
-    if (cols % fmt_chunk_elems(fmt) || rows % 16) {
-        set_error(std::string(what) + ": K must be whole 256 (Q4_K) / 128 (Q8_0) chunks and rows a multiple of 16");
+    if (cols % fmt_chunk_elems(fmt) || rows < 1) {
+        set_error(std::string(what) + ": K must be whole 256 (Q4_K) / 128 (Q8_0) chunks");
         return TSV_ERR_UNSUPPORTED;
     }
     return TSV_OK;
 }
 
-// Allocates a tiled matrix of `total_rows` rows and re-tiles `parts` into it: concatenated
-// (interleave == false) or with their 16-row tiles alternating (gate / up).
+// Allocates a tiled matrix of `total_rows` rows and re-tiles `parts` into it: concatenated row
+// by row (interleave == false) or alternating in runs of 32 rows (gate / up: each 64-row tile
+// holds 32 gate rows in its low lanes and the matching 32 up rows in its high lanes).
 int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_parts, bool interleave, TiledW* out) {
     const int fmt = dtype_fmt(parts[0]->dtype);
     int64_t total_rows = 0;
@@ -150,24 +151,29 @@ int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_par
             set_error("fused projection parts must share dtype and K");
             return TSV_ERR_INVALID;
         }
+        if (interleave && (parts[i]->rows != parts[0]->rows || parts[i]->rows % 32)) {
+            set_error("gate / up projections must have the same row count, a multiple of 32");
+            return TSV_ERR_UNSUPPORTED;
+        }
         total_rows += parts[i]->rows;
     }
     out->fmt = fmt;
     out->k = (int)parts[0]->cols;
     out->kchunks = out->k / fmt_chunk_elems(fmt);
     out->n_rows = (int)total_rows;
-    out->n_tiles = (int)((total_rows + 15) / 16);
+    out->n_tiles = (int)((total_rows + TILE_ROWS - 1) / TILE_ROWS);
     out->bytes = (size_t)out->n_tiles * out->kchunks * fmt_tile_bytes(fmt);
-    int rc = dev_alloc(c, &out->tiles, out->bytes);
+    int rc = dev_alloc(c, &out->tiles, out->bytes, true);  // rows past the last one stay zero blocks
     if (rc) return rc;
-    int tile_off = 0;
+    int row_off = 0;
     for (int i = 0; i < n_parts; i++) {
         if ((rc = stage_raw(c, st, *parts[i]))) return rc;
-        rc = launch_repack(c->stream, fmt, st.dev, (int)parts[i]->rows, out->k, out->tiles, out->kchunks,
-                           interleave ? n_parts : 1, interleave ? i : tile_off);
+        const int rows = (int)parts[i]->rows;
+        rc = interleave ? launch_repack(c->stream, fmt, st.dev, rows, out->k, out->tiles, out->kchunks, 32, 32 * n_parts, 32 * i)
+                        : launch_repack(c->stream, fmt, st.dev, rows, out->k, out->tiles, out->kchunks, rows, 0, row_off);
         if (rc) return rc;
         TSV_HIP(hipStreamSynchronize(c->stream));  // the stager is reused by the next part
-        tile_off += (int)(parts[i]->rows / 16);
+        row_off += rows;
     }
     return TSV_OK;
 }
@@ -177,7 +183,7 @@ int splits_for(const TiledW& w, int m, int epi) { return epi == EPI_PARTIAL ? ge
 size_t partial_need(const TiledW& w) {
     size_t need = 0;
     for (int m : {4, 8, 16}) {
-        size_t s = (size_t)splits_for(w, m, EPI_PARTIAL) * 16 * (size_t)w.n_tiles * 16;
+        size_t s = (size_t)splits_for(w, m, EPI_PARTIAL) * 16 * (size_t)w.n_tiles * TILE_ROWS;
         if (s > need) need = s;
     }
     return need;
@@ -511,7 +517,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     }
     // scratch
     const int kmax = std::max(std::max(c->hidden, qd), c->ffn);
-    const size_t xfb = (size_t)kmax / 32 * 4 * 16 * 16;
+    const size_t xfb = xfrag_bytes(kmax);
     c->nch = attn_chunks(c->nkv);
     const size_t rows_max = (size_t)TSV_MAX_ROWS * (c->nq / c->nkv);
     c->partial_floats = pneed;
@@ -881,7 +887,7 @@ extern "C" int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, fl
         sp = (tw.kchunks + kslice - 1) / kslice;
     }
     if (!rc) rc = dev_alloc(c, &xd, (size_t)m * k * 4);
-    if (!rc) rc = dev_alloc(c, &xf, (size_t)k / 32 * 4 * 16 * 16, true);
+    if (!rc) rc = dev_alloc(c, &xf, xfrag_bytes(k), true);
     if (!rc) rc = dev_alloc(c, &pd, (size_t)sp * 16 * n * 4, true);
     if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
     if (!rc && hipMemcpyAsync(xd, x, (size_t)m * k * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess) rc = TSV_ERR_DEVICE;
@@ -928,7 +934,7 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     float *po = nullptr, *pml = nullptr;
     uint4* xf = nullptr;
     VerifyParams* vpd = nullptr;
-    const size_t xfb = (size_t)nq * hd / 32 * 4 * 16 * 16;
+    const size_t xfb = xfrag_bytes(nq * hd);
     if (!rc) rc = dev_alloc(c, &kc, kvb, true);
     if (!rc) rc = dev_alloc(c, &vc, kvb, true);
     if (!rc) rc = dev_alloc(c, &kin, inb);
@@ -969,11 +975,7 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     }
     if (!rc)
         for (int b = 0; b < m; b++)
-            for (int kk = 0; kk < nq * hd; kk++) {
-                const int sub = kk >> 5, e = kk & 31, kg = e >> 3, o = e & 7;
-                const int p = (o & 4) | ((o & 1) << 1) | ((o >> 1) & 1);
-                out[(size_t)b * nq * hd + kk] = frag[(size_t)((sub * 4 + kg) * 16 + b) * 8 + p];
-            }
+            for (int kk = 0; kk < nq * hd; kk++) out[(size_t)b * nq * hd + kk] = frag[(size_t)frag_index(kk, b)];
     (void)hipStreamSynchronize(c->stream);
     for (void* p : c->allocs) (void)hipFree(p);
     (void)hipStreamDestroy(c->stream);
@@ -988,7 +990,7 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
 extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
                                    int32_t iters, int32_t rotate, float* avg_us) {
     const int fmt = dtype_fmt(dtype);
-    if (fmt < 0 || rows % 16 || cols % fmt_chunk_elems(fmt) || m < 1 || m > TSV_MAX_ROWS || iters < 1 || rotate < 1) {
+    if (fmt < 0 || rows % TILE_ROWS || cols % fmt_chunk_elems(fmt) || m < 1 || m > TSV_MAX_ROWS || iters < 1 || rotate < 1) {
         set_error("matmul_time: bad argument");
         return TSV_ERR_INVALID;
     }
@@ -1000,7 +1002,7 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
     w.k = (int)cols;
     w.kchunks = w.k / fmt_chunk_elems(fmt);
     w.n_rows = (int)rows;
-    w.n_tiles = (int)(rows / 16);
+    w.n_tiles = (int)(rows / TILE_ROWS);
     w.bytes = (size_t)w.n_tiles * w.kchunks * fmt_tile_bytes(fmt);
     std::vector<uint8_t*> copies((size_t)rotate);
     int rc = TSV_OK;
@@ -1016,14 +1018,14 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
         }
         const int tb = fmt_tile_bytes(fmt);
         for (size_t t = 0; t < w.bytes / tb; t++) {
-            uint8_t* sc = &host[t * tb + 2048];
+            uint8_t* sc = &host[t * tb + 8192];
             if (fmt == FMT_Q4K)
-                for (int r = 0; r < 16; r++) {
+                for (int r = 0; r < 64; r++) {
                     sc[r * 16 + 1] = 0x20;
                     sc[r * 16 + 3] = 0x20;
                 }
             else
-                for (int i = 0; i < 64; i++) sc[2 * i + 1] = 0x20;
+                for (int i = 0; i < 256; i++) sc[2 * i + 1] = 0x20;
         }
         for (int i = 0; i < rotate && !rc; i++) {
             rc = dev_alloc(c, &copies[i], w.bytes);
@@ -1043,8 +1045,8 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
         const int kslice = (w.kchunks + sp - 1) / sp;
         sp = (w.kchunks + kslice - 1) / kslice;
     }
-    if (!rc) rc = dev_alloc(c, &xf, (size_t)std::max<int64_t>(cols, rows) / 32 * 4 * 16 * 16 + 4096, true);
-    if (!rc) rc = dev_alloc(c, &out, (size_t)sp * 16 * rows * 4 + (size_t)rows * 32 * 2, true);
+    if (!rc) rc = dev_alloc(c, &xf, xfrag_bytes((int)cols), true);
+    if (!rc) rc = dev_alloc(c, &out, (size_t)sp * 16 * rows * 4 + xfrag_bytes((int)rows), true);
     if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
     if (!rc && hipMemcpy(vpd, &vp, sizeof vp, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -1053,8 +1055,7 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
         if (pass == 1) (void)hipEventRecord(e0, c->stream);
         for (int i = 0; i < (pass ? iters : std::min(iters, 3)) && !rc; i++) {
             w.tiles = copies[(size_t)(i % rotate)];
-            rc = launch_gemm(c->stream, w, xf, epi == EPI_SILU ? (void*)(xf + 64) : (void*)out, vpd, m, sp, epi,
-                             (int)rows, (int)rows);
+            rc = launch_gemm(c->stream, w, xf, (void*)out, vpd, m, sp, epi, (int)rows, (int)rows);
         }
         if (pass == 1) (void)hipEventRecord(e1, c->stream);
     }

@@ -22,16 +22,25 @@ const std::string& get_error();
     } while (0)
 
 // ---------------------------------------------------------------------------------------
-// Device weight layout ("row tiles").  A matrix W[N][K] is cut into tiles of 16 output rows
+// Device weight layout ("row tiles").  A matrix W[N][K] is cut into tiles of 64 output rows
 // by one K-chunk (256 elements for Q4_K, 128 for Q8_0); tiles are stored [row tile][chunk]
-// so a wave streaming along K for its 16 rows reads one contiguous byte run.  Inside a
-// tile every wave-wide load instruction covers 1 KiB contiguous (64 lanes x 16 B):
-//   Q4_K tile, 2304 B: [half 0..1][lane 0..63][16 B] nibble bytes, then [row 0..15][16 B]
-//                      (f16 d, f16 dmin, 12 packed scale bytes) -- the 144 B of each of the
-//                      16 superblocks, byte for byte, only re-ordered.
-//   Q8_0 tile, 2176 B: [half 0..1][lane][16 B] int8 quants, then [row][4 x f16 d].
-// lane = kg*16 + r: r = row inside the tile, kg = which 8-element K slice of a 32-element
-// sub-block the lane feeds to the MFMA.
+// so a wave streaming along K for its 64 rows reads one contiguous byte run.  Lane l of the
+// wave owns weight row l of the tile; every wave-wide load covers 1 KiB contiguous
+// (64 lanes x 16 B):
+//   Q4_K tile, 9216 B: [unit 0..7][lane][16 B] nibble bytes 16*unit.. of the lane's superblock,
+//                      then [lane][16 B] (f16 d, f16 dmin, 12 packed scale bytes) -- the 144 B
+//                      of each of the 64 superblocks, byte for byte, only re-ordered.
+//   Q8_0 tile, 8704 B: [unit 0..7][lane][16 B] int8 quants (unit u = bytes 16*(u%2).. of block
+//                      u/2 of the chunk), then [lane][4 x f16 d].
+// Rows past the matrix's last row are all-zero blocks (scale 0).
+//
+// Activation layout ("fragments").  The <=16 fp16 activation rows of a K-wide matmul input
+// are stored as the A operands of v_mfma_f32_4x4x4_16B_f16, ready to load one 8-byte word per
+// lane: [K/64 pair][row group g = row/4][step b = (k%64)/4][i = row%4][4 halfs], the four halfs
+// in the order the weight unpack produces (k%4 = 0, 2, 1, 3).  Behind the fragments
+// (byte offset xfrag_sum_offset(K)) sit the fp32 sums of the fp16-rounded activations over
+// every 32-element sub-block, [K/256][g][sub%8][i], which the matmul uses to take the
+// integer-code offsets and the Q4_K min term back out.
 // ---------------------------------------------------------------------------------------
 enum { FMT_Q4K = 0, FMT_Q80 = 1 };
 
@@ -39,15 +48,28 @@ struct TiledW {
     uint8_t* tiles = nullptr;  // device
     int fmt = 0;
     int n_rows = 0;    // real output rows
-    int n_tiles = 0;   // ceil(n_rows / 16)
+    int n_tiles = 0;   // ceil(n_rows / 64)
     int kchunks = 0;   // K / chunk elems
     int k = 0;
     size_t bytes = 0;
 };
 
 inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q4K ? 256 : 128; }
-inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 2304 : 2176; }
+inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : 8704; }
 inline int fmt_nsub(int fmt) { return fmt == FMT_Q4K ? 8 : 4; }
+constexpr int TILE_ROWS = 64;
+
+// index (in halfs) of activation element (row, k) in the fragment layout
+__host__ __device__ inline int frag_index(int k, int row) {
+    const int pos = ((k & 1) << 1) | ((k >> 1) & 1);  // k%4 = 0,1,2,3 -> slot 0,2,1,3
+    return ((((k >> 6) * 4 + (row >> 2)) * 16 + ((k >> 2) & 15)) * 4 + (row & 3)) * 4 + pos;
+}
+__host__ __device__ inline size_t xfrag_sum_offset(int k) { return (size_t)((k + 63) / 64) * 2048; }
+__host__ __device__ inline size_t xfrag_bytes(int k) { return xfrag_sum_offset(k) + (size_t)((k + 255) / 256) * 512; }
+// index (in floats) of the sum of sub-block `sub` (= k/32) of `row`
+__host__ __device__ inline int xsum_index(int sub, int row) {
+    return (((sub >> 3) * 4 + (row >> 2)) * 8 + (sub & 7)) * 4 + (row & 3);
+}
 
 // Per-call parameters every kernel of a verify pass reads from device memory, so a captured
 // launch sequence can be replayed at another base position.
@@ -63,15 +85,18 @@ enum { EPI_PARTIAL = 0, EPI_SILU = 1, EPI_LOGITS = 2 };
 
 struct GemmArgs {
     const uint8_t* w;
-    const uint4* xfrag;  // [K/32][4][16] x 16 B, fp16 activations in fragment order
-    void* out;           // EPI_PARTIAL: float [splits][16][ldo]; EPI_SILU: xfrag of the next matmul;
-                         // EPI_LOGITS: half [m][ldo]
+    const uint2* xfrag;  // activation fragments, 8 B per (pair, row group, lane)
+    const float* xsum;   // their sub-block sums
+    void* out;           // EPI_PARTIAL: float [splits][16][ldo]; EPI_SILU: fragments (+ sums) of the
+                         // next matmul; EPI_LOGITS: half [m][ldo]
     const VerifyParams* vp;
-    int n_tiles, kchunks, kslice, splits, ldo, n_valid;
+    int n_tiles, kchunks, kslice, splits, kparts, per, ldo, n_valid;
 };
 
+// Re-tiles n_rows GGUF rows of `raw` into `tiles`; source row r lands in tiled row
+// (r / grp) * stride + offset + r % grp.
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
-                  int kchunks, int tile_stride, int tile_offset);
+                  int kchunks, int grp, int stride, int offset);
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
                 int m, int splits, int epi, int ldo, int n_valid);
 int gemm_default_splits(const TiledW& w, int m);
