@@ -55,6 +55,12 @@ struct tsv_ctx {
     int64_t position = 0;
     int last_m = 0;
     int64_t last_base = -1;
+    // The launch sequence of a pass depends on the row count only (positions, tokens and the
+    // tree shape are read from device memory), so it is captured once per row count into a HIP
+    // graph and replayed: a graph node starts ~1 us sooner after its predecessor than a
+    // stream launch does, and a pass is ~290 dependent launches.
+    bool use_graph = true;
+    hipGraphExec_t pass_graph[TSV_MAX_ROWS + 1] = {};
     // per-kernel-class timing (tsv_set_profile): one event pair per launch
     bool profile = false;
     std::vector<hipEvent_t> ev;
@@ -272,6 +278,8 @@ int fill_params(VerifyParams& vp, const int32_t* feed, const int32_t* parent, in
     return TSV_OK;
 }
 
+int run_pass(tsv_ctx* c, int m);
+
 // One verify pass: enqueue everything on the handle's stream; no synchronisation.
 int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m, int64_t base) {
     // batched.rs:106-185 refusals
@@ -299,7 +307,17 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     TSV_HIP(hipStreamSynchronize(s));
     *c->vp_host = vp;
     TSV_HIP(hipMemcpyAsync(c->vp_dev, c->vp_host, sizeof vp, hipMemcpyHostToDevice, s));
+    int rc = run_pass(c, m);
+    if (rc) return rc;
+    c->position = base + m;
+    c->last_m = m;
+    c->last_base = base;
+    return TSV_OK;
+}
 
+// The kernels of one pass over m rows, in order, on the handle's stream.
+int launch_pass(tsv_ctx* c, int m) {
+    hipStream_t s = c->stream;
     int rc;
     {
         PROF(PC_EMBED);
@@ -394,10 +412,30 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
         PROF(PC_HEAD);
         rc = launch_gemm(s, c->head, c->xf_a, c->logits, c->vp_dev, m, 1, EPI_LOGITS, c->vocab, c->vocab);
     }
-    if (rc) return rc;
-    c->position = base + m;
-    c->last_m = m;
-    c->last_base = base;
+    return rc;
+}
+
+int run_pass(tsv_ctx* c, int m) {
+    if (!c->use_graph || c->profile) return launch_pass(c, m);
+    if (!c->pass_graph[m]) {
+        hipGraph_t g = nullptr;
+        TSV_HIP(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+        const int rc = launch_pass(c, m);
+        const hipError_t e = hipStreamEndCapture(c->stream, &g);
+        if (rc || e != hipSuccess) {
+            if (g) (void)hipGraphDestroy(g);
+            if (!rc) set_error(std::string("verify: graph capture failed: ") + hipGetErrorString(e));
+            return rc ? rc : TSV_ERR_DEVICE;
+        }
+        const hipError_t ei = hipGraphInstantiate(&c->pass_graph[m], g, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(g);
+        if (ei != hipSuccess) {
+            c->pass_graph[m] = nullptr;
+            set_error(std::string("verify: graph instantiation failed: ") + hipGetErrorString(ei));
+            return TSV_ERR_DEVICE;
+        }
+    }
+    TSV_HIP(hipGraphLaunch(c->pass_graph[m], c->stream));
     return TSV_OK;
 }
 
@@ -440,6 +478,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->ctx_alloc = ((d->max_context + 15) / 16) * 16;
     c->eps = d->rms_eps;
     c->attn_scale = d->attn_scale > 0.f ? d->attn_scale : 1.0f / std::sqrt((float)d->head_dim);
+    if (const char* e = getenv("TSV_NO_GRAPH")) c->use_graph = e[0] == '0' || e[0] == '\0';
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("open: cannot create a HIP stream (no GPU?)");
         delete c;
@@ -560,6 +599,8 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
+    for (hipGraphExec_t g : c->pass_graph)
+        if (g) (void)hipGraphExecDestroy(g);
     for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
