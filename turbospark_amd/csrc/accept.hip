@@ -25,6 +25,7 @@ namespace {
 constexpr int NSEG = 64;          // index segments per vocabulary row
 constexpr int MAX_DIST_ROWS = 32;  // target rows + drafter rows
 constexpr int MAX_JOBS = 16;
+constexpr int NSUB = 4;  // workgroups per segment in the mass / histogram pass
 constexpr double FIX = 4611686018427387904.0;  // 2^62
 
 struct RowStat {
@@ -39,7 +40,7 @@ struct Layout {
     double* pmax;  // [rows][NSEG]
     double* psum;
     double* ptot;
-    double* segtot;  // [jobs][NSEG] residual mass per segment
+    double* segtot;  // [jobs][NSEG * NSUB] residual mass per piece of a segment
 };
 __host__ __device__ inline Layout layout(double* base) {
     Layout l;
@@ -86,6 +87,13 @@ __device__ __forceinline__ uint32_t rank_key(uint16_t b) {
     return 0xFFFFu - asc;
 }
 
+// Where the histogram keeps rank bin `key`: the two low 6-bit fields are swapped, so the 64
+// consecutive keys one thread of the cumulative walk owns are 64 words apart and neighbouring
+// threads read neighbouring words.
+__device__ __forceinline__ uint32_t bin_addr(uint32_t key) {
+    return (key & 0xF000u) | ((key & 63u) << 6) | ((key >> 6) & 63u);
+}
+
 // choose.rs:296-319 for one candidate of a row whose statistics are known
 __device__ __forceinline__ double prob_of(uint16_t bits, const RowStat& s, double inv_t) {
     const double e = exp((double)h2f(bits) - s.mx);
@@ -118,11 +126,31 @@ __device__ __forceinline__ const uint16_t* row_ptr(const uint16_t* target, const
     return row < m ? target + (long)row * vocab : draft + (long)(row - m) * vocab;
 }
 
+// Wave-wide fold of a row's NSEG (= wave size) partials: lane s loads segment s, an xor
+// butterfly combines them.  Both lanes of a pair add the same two operands, so every lane ends
+// with the same bits, and every kernel that needs a row's statistics gets them this way.
+__device__ __forceinline__ double wave_max_f64(double v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmax(v, shfl_xor_t(v, o));
+    return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    for (int o = 32; o > 0; o >>= 1) v += shfl_xor_t(v, o);
+    return v;
+}
+static_assert(NSEG == 64, "one lane per segment");
+
 // ---- statistics, three short passes over every distribution row -------------------------
 __global__ __launch_bounds__(256) void k_row_max(const uint16_t* target, const uint16_t* draft, int m,
-                                                 int vocab, double* scratch, int32_t* err) {
+                                                 int vocab, double* scratch, int32_t* err,
+                                                 unsigned long long* hist, int hist_words) {
     __shared__ double red[4];
     const int row = blockIdx.y, seg = blockIdx.x;
+    {
+        // the rank histograms of this round's draws start from zero: every workgroup clears a slice
+        const int nwg = gridDim.x * gridDim.y, wg = blockIdx.y * gridDim.x + blockIdx.x;
+        const int per = (hist_words + nwg - 1) / nwg, h0 = wg * per, h1 = min(h0 + per, hist_words);
+        for (int i = h0 + threadIdx.x; i < h1; i += 256) hist[i] = 0;
+    }
     const uint16_t* p = row_ptr(target, draft, m, vocab, row);
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
     float mx = -INFINITY;
@@ -145,8 +173,7 @@ __global__ __launch_bounds__(256) void k_row_sum(const uint16_t* target, const u
     __shared__ double red[4];
     const int row = blockIdx.y, seg = blockIdx.x;
     Layout L = layout(scratch);
-    double mx = -INFINITY;
-    for (int s = 0; s < NSEG; s++) mx = fmax(mx, L.pmax[row * NSEG + s]);
+    const double mx = wave_max_f64(L.pmax[row * NSEG + (threadIdx.x & 63)]);
     const uint16_t* p = row_ptr(target, draft, m, vocab, row);
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
     double acc = 0.0;
@@ -163,11 +190,8 @@ __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const
     __shared__ double red[4];
     const int row = blockIdx.y, seg = blockIdx.x;
     Layout L = layout(scratch);
-    double mx = -INFINITY, sum = 0.0;
-    for (int s = 0; s < NSEG; s++) {
-        mx = fmax(mx, L.pmax[row * NSEG + s]);
-        sum += L.psum[row * NSEG + s];
-    }
+    const double mx = wave_max_f64(L.pmax[row * NSEG + (threadIdx.x & 63)]);
+    const double sum = wave_sum_f64(L.psum[row * NSEG + (threadIdx.x & 63)]);
     const double top = 1.0 / sum;  // the arg-max candidate has e == exp(0) == 1
     const uint16_t* p = row_ptr(target, draft, m, vocab, row);
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
@@ -186,18 +210,14 @@ __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const
     }
 }
 
+// Called by one whole wave: the finished statistics of `row`, identical in every lane.
 __device__ RowStat load_stat(const Layout& L, int row) {
+    const int lane = threadIdx.x & 63;
     RowStat s;
-    double mx = -INFINITY, sum = 0.0, tot = 0.0;
-    for (int i = 0; i < NSEG; i++) {
-        mx = fmax(mx, L.pmax[row * NSEG + i]);
-        sum += L.psum[row * NSEG + i];
-        tot += L.ptot[row * NSEG + i];
-    }
-    s.mx = mx;
-    s.sum = sum;
-    s.top = 1.0 / sum;
-    s.total = tot;
+    s.mx = wave_max_f64(L.pmax[row * NSEG + lane]);
+    s.sum = wave_sum_f64(L.psum[row * NSEG + lane]);
+    s.top = 1.0 / s.sum;
+    s.total = wave_sum_f64(L.ptot[row * NSEG + lane]);
     return s;
 }
 
@@ -220,7 +240,7 @@ __device__ int sink_commit(const AcceptParams& ap, int32_t token, uint64_t& gene
 
 // speculative.rs:694-754: the sequential walk over the proposals of a sampled chain round.
 __device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t* target,
-                                         const uint16_t* draft, const Layout& L) {
+                                         const uint16_t* draft, const RowStat* stats) {
     Decision d;
     d.job.mode = 0;
     d.job.row_p = d.job.row_q = 0;
@@ -232,7 +252,7 @@ __device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t*
     int reject = -1;
     for (int i = 0; i < ap.k; i++) {
         const int32_t x = ap.feed[i + 1];
-        const RowStat sp = load_stat(L, i), sq = load_stat(L, ap.m + i);
+        const RowStat sp = stats[i], sq = stats[ap.m + i];
         const double px = prob_of(target[(long)i * ap.vocab + x], sp, inv_t);
         const double qx = prob_of(draft[(long)i * ap.vocab + x], sq, inv_t);
         const double r = unit_draw(ap.seed, ds);
@@ -270,12 +290,22 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
                                                    unsigned long long* hist, Decision* dec_out, int kind) {
     __shared__ Decision dec;
     __shared__ double red[4];
+    __shared__ RowStat stats[MAX_DIST_ROWS];
     const AcceptParams& ap = *app;
-    const int seg = blockIdx.x, jobi = blockIdx.y;
+    const int seg = blockIdx.x, jobi = blockIdx.y, sub = blockIdx.z;
     Layout L = layout(scratch);
+    {
+        // every row's statistics, one wave per row at a time
+        const int rows = kind == 0 ? ap.m + ap.k : ap.k;
+        for (int r = threadIdx.x >> 6; r < rows; r += 4) {
+            const RowStat st = load_stat(L, r);
+            if ((threadIdx.x & 63) == 0) stats[r] = st;
+        }
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
         if (kind == 0) {
-            dec = decide_chain_sampled(ap, target, draft, L);
+            dec = decide_chain_sampled(ap, target, draft, stats);
         } else {
             dec.job.mode = 1;
             dec.job.row_p = ap.m + jobi;
@@ -285,16 +315,15 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
             dec.draw_step = ap.draw_step;
             dec.margin = 1.0;
         }
-        if (seg == 0) dec_out[jobi] = dec;
+        if (seg == 0 && sub == 0) dec_out[jobi] = dec;
     }
     __syncthreads();
     const Job job = dec.job;
     if (job.mode == 0) return;
     const int vocab = ap.vocab;
     const double inv_t = 1.0 / ap.temperature;
-    const RowStat sp = load_stat(L, job.row_p);
-    RowStat sq = sp;
-    if (job.mode == 2) sq = load_stat(L, job.row_q);
+    const RowStat sp = stats[job.row_p];
+    const RowStat sq = stats[job.mode == 2 ? job.row_q : job.row_p];
     const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, job.row_p);
     const uint16_t* lq = row_ptr(target, draft, ap.m, vocab, job.row_q);
     double* wp = work + (long)jobi * 2 * vocab;
@@ -303,10 +332,10 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     unsigned long long* hr = hp + 65536;
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
     double racc = 0.0;
-    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+    for (int v = v0 + sub * 256 + threadIdx.x; v < v1; v += 256 * NSUB) {
         const uint16_t b = lp[v];
         const double pv = prob_of(b, sp, inv_t);
-        const uint32_t key = rank_key(b);
+        const uint32_t key = bin_addr(rank_key(b));
         wp[v] = pv;
         atomicAdd(hp + key, (unsigned long long)(pv * FIX));
         if (job.mode == 2) {
@@ -318,7 +347,36 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     }
     if (job.mode == 2) {
         racc = block_sum_f64(racc, red);
-        if (threadIdx.x == 0) L.segtot[jobi * NSEG + seg] = racc;
+        if (threadIdx.x == 0) L.segtot[(jobi * NSEG + seg) * NSUB + sub] = racc;
+    }
+}
+
+// Calls on_match(v) for every index v in [v0, v1) whose logit bits are `want` (or -0 when the
+// bin is the zero bin), eight keys per 16-byte load when the row allows it.
+template <class Fn>
+__device__ __forceinline__ void scan_chunk(const uint16_t* lp, int v0, int v1, uint32_t want, bool zero_bin, bool vec,
+                                           Fn&& on_match) {
+    for (int g = v0; g < v1; g += 8) {
+        uint32_t w[4];
+        if (vec && g + 8 <= v1) {
+            const uint4 q = *(const uint4*)(lp + g);
+            w[0] = q.x;
+            w[1] = q.y;
+            w[2] = q.z;
+            w[3] = q.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t lo = g + 2 * j < v1 ? lp[g + 2 * j] : (want ^ 0x4000u);
+                const uint32_t hi = g + 2 * j + 1 < v1 ? lp[g + 2 * j + 1] : (want ^ 0x4000u);
+                w[j] = lo | (hi << 16);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t bits = (w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+            if (bits == want || (zero_bin && bits == 0x8000u)) on_match(g + j);
+        }
     }
 }
 
@@ -348,8 +406,15 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         int mode = dec.job.mode;
         double R = 1.0;
         if (mode == 2) {
-            R = 0.0;
-            for (int s = 0; s < NSEG; s++) R += L.segtot[jobi * NSEG + s];
+            // residual mass: the pieces' partial sums folded in a fixed order
+            static_assert(NSEG * NSUB == 256, "four waves fold the pieces");
+            if (tid < 256) {
+                const double part = wave_sum_f64(L.segtot[jobi * NSEG * NSUB + tid]);
+                if (lane == 0) dsum[wave] = part;
+            }
+            __syncthreads();
+            R = (dsum[0] + dsum[1]) + (dsum[2] + dsum[3]);
+            __syncthreads();
             if (R < 1e-12) mode = 1;  // distribution.rs:96-126: residual underflow -> plain p draw
         }
         unsigned long long* hp = hist + (long)jobi * 2 * 65536;
@@ -357,9 +422,12 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         const double* w = work + (long)jobi * 2 * vocab + (mode == 2 ? vocab : 0);
         const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, dec.job.row_p);
 
-        // 64 consecutive bins per thread; integer sums are exact and order independent
+        // 64 consecutive rank bins per thread (see bin_addr); integer sums are exact and order
+        // independent
+        const unsigned long long* hmine = hsel + (tid >> 6) * 4096 + (tid & 63);
         unsigned long long loc = 0;
-        for (int i = 0; i < 64; i++) loc += hsel[tid * 64 + i];
+#pragma unroll 16
+        for (int i = 0; i < 64; i++) loc += hmine[i * 64];
         unsigned long long inc = loc;
         for (int o = 1; o < 64; o <<= 1) {
             const uint32_t lo = __shfl_up((uint32_t)inc, o), hi = __shfl_up((uint32_t)(inc >> 32), o);
@@ -386,7 +454,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         if (excl <= tgt && tgt < excl + loc) {
             unsigned long long c = excl;
             for (int i = 0; i < 64; i++) {
-                const unsigned long long hv = hsel[tid * 64 + i];
+                const unsigned long long hv = hmine[i * 64];
                 if (tgt < c + hv) {
                     s_bin = tid * 64 + i;
                     s_before = c;
@@ -404,7 +472,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             const int lb = s_last_bin;  // upper end of the last occupied 64-bin group
             if (tid * 64 + 63 == lb) {
                 int bb = lb;
-                while (bb > tid * 64 && hsel[bb] == 0) bb--;
+                while (bb > tid * 64 && hsel[bin_addr(bb)] == 0) bb--;
                 s_bin = bb;
                 s_before = total;
                 s_fallback = 1;
@@ -414,17 +482,20 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         }
         const bool fallback = s_fallback != 0;
         // walk the bin in index order: contiguous index chunk per thread
-        const int per = (vocab + 1023) / 1024, v0 = tid * per, v1 = min(v0 + per, vocab);
+        const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = tid * per, v1 = min(v0 + per, vocab);
+        const bool vec = ((uintptr_t)lp & 15) == 0;
+        const uint32_t asc = 0xFFFFu - (uint32_t)bin;  // inverse of rank_key
+        const uint32_t want = (asc & 0x8000u) ? (asc & 0x7FFFu) : (~asc & 0xFFFFu);
+        const bool zero_bin = want == 0;
         double lsum = 0.0;
         int lastv = -1;
-        for (int v = v0; v < v1; v++)
-            if ((int)rank_key(lp[v]) == bin) {
-                const double wv = mode == 2 ? w[v] / R : w[v];
-                if (mode != 2 || wv > 0.0) {
-                    lsum += wv;
-                    lastv = v;
-                }
+        scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int v) {
+            const double wv = mode == 2 ? w[v] / R : w[v];
+            if (mode != 2 || wv > 0.0) {
+                lsum += wv;
+                lastv = v;
             }
+        });
         double incd = lsum;
         for (int o = 1; o < 64; o <<= 1) {
             uint64_t u = __builtin_bit_cast(uint64_t, incd);
@@ -445,18 +516,20 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             const double u = dec.job.u;
             if (lsum > 0.0 && !(u < before) && u < before + lsum) {
                 double c = before;
-                for (int v = v0; v < v1; v++)
-                    if ((int)rank_key(lp[v]) == bin) {
-                        const double wv = mode == 2 ? w[v] / R : w[v];
-                        if (mode == 2 && !(wv > 0.0)) continue;
-                        if (u < c + wv) {
-                            s_token = v;
-                            s_cum_before = c;
-                            s_cum_at = c + wv;
-                            break;
-                        }
-                        c += wv;
+                bool found = false;
+                scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int v) {
+                    if (found) return;
+                    const double wv = mode == 2 ? w[v] / R : w[v];
+                    if (mode == 2 && !(wv > 0.0)) return;
+                    if (u < c + wv) {
+                        s_token = v;
+                        s_cum_before = c;
+                        s_cum_at = c + wv;
+                        found = true;
+                        return;
                     }
+                    c += wv;
+                });
             }
         }
         __syncthreads();
@@ -472,9 +545,6 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         } else if (!fallback) {
             margin = fmin(margin, fmin(dec.job.u - s_cum_before, s_cum_at - dec.job.u));
         }
-        // clear both histograms of this job for the next round (every read is behind a barrier)
-        __syncthreads();
-        for (int i = tid; i < 2 * 65536; i += 1024) hp[i] = 0;
     }
 
     if (tid == 0) {
@@ -589,10 +659,12 @@ __global__ void k_clear_result(AcceptResult* res, int32_t* err) {
 
 // scratch.counters: [0] error flag, [16..32) greedy arg-max per row; decisions live after the
 // statistics block; histograms and work arrays are separate allocations in AcceptScratch.
-size_t accept_stats_doubles() { return 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG + MAX_JOBS * 16; }
+size_t accept_stats_doubles() {
+    return 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG * NSUB + MAX_JOBS * 16;
+}
 
 static Decision* decisions(const AcceptScratch& sc) {
-    return (Decision*)(sc.stats + 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG);
+    return (Decision*)(sc.stats + 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG * NSUB);
 }
 
 int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
@@ -612,10 +684,11 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
     }
     const int rows = ap.m + ap.k;
     const double inv_t = 1.0 / ap.temperature;
-    hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err);
+    hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err,
+                       (unsigned long long*)sc.hist, 2 * 65536);
     hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
     hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, inv_t);
-    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, 1), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, 1, NSUB), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), 0);
     hipLaunchKernelGGL(k_pick, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), sc.result, (int32_t*)nullptr, err, 0);
@@ -635,10 +708,11 @@ int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams*
         return TSV_OK;
     }
     const double inv_t = 1.0 / ap.temperature;
-    hipLaunchKernelGGL(k_row_max, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, err);
+    hipLaunchKernelGGL(k_row_max, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, err,
+                       (unsigned long long*)sc.hist, ap.k * 2 * 65536);
     hipLaunchKernelGGL(k_row_sum, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats);
     hipLaunchKernelGGL(k_row_total, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, inv_t);
-    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
+    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, ap.k, NSUB), dim3(256), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), 1);
     hipLaunchKernelGGL(k_pick, dim3(ap.k), dim3(1024), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), sc.result, proposals_dev, err, 1);

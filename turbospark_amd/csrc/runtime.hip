@@ -56,10 +56,11 @@ struct tsv_ctx {
     int last_m = 0;
     int64_t last_base = -1;
     // The launch sequence of a pass depends on the row count only (positions, tokens and the
-    // tree shape are read from device memory), so it is captured once per row count into a HIP
-    // graph and replayed: a graph node starts ~1 us sooner after its predecessor than a
-    // stream launch does, and a pass is ~290 dependent launches.
-    bool use_graph = true;
+    // tree shape are read from device memory), so it can be captured once per row count into a
+    // HIP graph and replayed (environment TSV_GRAPH=1).  Off by default: the pass is bound by
+    // the GPU-side cost of ~290 dependent kernels, not by host launch time, and replay measured
+    // the same step time as plain stream launches.
+    bool use_graph = false;
     hipGraphExec_t pass_graph[TSV_MAX_ROWS + 1] = {};
     // per-kernel-class timing (tsv_set_profile): one event pair per launch
     bool profile = false;
@@ -478,7 +479,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->ctx_alloc = ((d->max_context + 15) / 16) * 16;
     c->eps = d->rms_eps;
     c->attn_scale = d->attn_scale > 0.f ? d->attn_scale : 1.0f / std::sqrt((float)d->head_dim);
-    if (const char* e = getenv("TSV_NO_GRAPH")) c->use_graph = e[0] == '0' || e[0] == '\0';
+    if (const char* e = getenv("TSV_GRAPH")) c->use_graph = e[0] == '1';
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("open: cannot create a HIP stream (no GPU?)");
         delete c;
