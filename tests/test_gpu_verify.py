@@ -11,7 +11,9 @@ def _prompt(n, vocab, seed):
     return np.random.default_rng(seed).integers(0, vocab, n).astype(np.int32)
 
 
-@pytest.mark.parametrize("name,ctx,k", [("tiny_q8_0", 256, 4), ("small_q4_k", 70, 4), ("small_q4_k", 33, 15)])
+@pytest.mark.parametrize("name,ctx,k", [("tiny_q8_0", 256, 4), ("small_q4_k", 70, 4), ("small_q4_k", 33, 15),
+                                        ("xcd_q4_k", 70, 4), ("xcd_q4_k", 33, 7), ("xcd_q4_k", 40, 0),
+                                        ("xcd_q8_0", 70, 4), ("xcd_q4_k", 33, 15)])
 def test_verify_logits_match_the_oracle(name, ctx, k):
     cfg, w, gpu, cpu = gc.build_pair(name, max_context=ctx + 32)
     prompt = _prompt(ctx, cfg["vocab"], 7)
@@ -33,9 +35,10 @@ def test_verify_logits_match_the_oracle(name, ctx, k):
     assert gpu.position == ctx + k + 1
 
 
-def test_a_batched_pass_equals_the_same_tokens_fed_one_at_a_time():
+@pytest.mark.parametrize("name", ["small_q4_k", "xcd_q4_k", "xcd_q8_0"])
+def test_a_batched_pass_equals_the_same_tokens_fed_one_at_a_time(name):
     """crates/runtime/tests/real_forward_qwen35_mtp.rs:962-1032: the row-invariance gate."""
-    cfg, w, gpu, cpu = gc.build_pair("small_q4_k", max_context=96)
+    cfg, w, gpu, cpu = gc.build_pair(name, max_context=96)
     prompt = _prompt(40, cfg["vocab"], 3)
     gpu.prefill(prompt, 0, want_logits=False)
     feed = _prompt(6, cfg["vocab"], 4)
@@ -46,10 +49,11 @@ def test_a_batched_pass_equals_the_same_tokens_fed_one_at_a_time():
     assert np.array_equal(batch, seq)
 
 
-def test_rollback_equals_a_fresh_run():
+@pytest.mark.parametrize("name", ["tiny_q8_0", "xcd_q4_k"])
+def test_rollback_equals_a_fresh_run(name):
     """crates/bench/tests/rollback_probe.rs:1-140: after feeding and rolling back a rejected block,
     the kept continuation's logits equal, by bits, a run that never saw the rejected block."""
-    cfg, w, gpu, cpu = gc.build_pair("tiny_q8_0", max_context=128)
+    cfg, w, gpu, cpu = gc.build_pair(name, max_context=128)
     prompt = _prompt(50, cfg["vocab"], 11)
     rejected = _prompt(5, cfg["vocab"], 12)
     kept = _prompt(5, cfg["vocab"], 13)

@@ -29,16 +29,10 @@
 //    Neither split depends on the number of activation rows, so a row's result is the same
 //    bits whether it is verified alone or in a block.
 #include <algorithm>
-#include <utility>
 
-#include "tsv_internal.h"
+#include "gemm_core.h"
 
 namespace tsv {
-
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // ------------------------------------------------------------------------------- re-tiling
 // One thread per 16-byte unit of a source row's chunk (unit 8 = the scale header).
@@ -100,209 +94,6 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
-
-// ------------------------------------------------------------------------------- helpers
-template <int... I, class Fn>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, Fn&& f) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, class Fn>
-__device__ __forceinline__ void static_for(Fn&& f) {
-    static_for_impl(std::make_integer_sequence<int, N>{}, f);
-}
-
-// D[i] += sum_k A_step[i][k] * B_lane[k]: A taken from block `STEP` of the a operand for all lanes
-template <int STEP>
-__device__ __forceinline__ float4v mfma_f16(u32x2 a, u32x2 b, float4v c) {
-    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4, a), __builtin_bit_cast(half4, b), c, 4, STEP, 0);
-}
-template <int STEP>
-__device__ __forceinline__ float4v mfma_f32(float a, float b, float4v c) {
-    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 4, STEP, 0);
-}
-
-__device__ __forceinline__ float h2f_lo(uint32_t v) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)(v & 0xFFFF));
-}
-__device__ __forceinline__ float h2f_hi(uint32_t v) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)(v >> 16));
-}
-__device__ __forceinline__ float ubyte(uint32_t v, int i) { return (float)((v >> (8 * i)) & 0xFF); }
-
-// (v & mask) | bits as ONE v_and_or_b32: the instruction can take a single literal / scalar
-// operand, so the second constant is pinned in a vector register.
-__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits_vgpr) {
-    return (v & mask) | bits_vgpr;
-}
-
-struct Consts {
-    uint32_t k6400, k5400, k64;
-};
-
-// ------------------------------------------------------------------------------- formats
-struct Q4K {
-    static constexpr int NSUB = 8, NPAIR = 4, TILE_BYTES = 9216;
-    struct Regs {
-        u32x4 q[8];
-        u32x4 s;
-    };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
-        const u32x4* p = (const u32x4*)tile + lane;
-#pragma unroll
-        for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
-        r.s = __builtin_nontemporal_load(p + 512);
-    }
-    // float index of this lane's sub-block sums for row group g of chunk c
-    static __device__ __forceinline__ int xs_index(int c, int g, int lane) { return (c * 4 + g) * 32 + (lane & 31); }
-};
-
-struct Q80 {
-    static constexpr int NSUB = 4, NPAIR = 2, TILE_BYTES = 8704;
-    struct Regs {
-        u32x4 q[8];
-        u32x2 s;
-    };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
-        const u32x4* p = (const u32x4*)tile + lane;
-#pragma unroll
-        for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
-        r.s = __builtin_nontemporal_load((const u32x2*)(tile + 8192) + lane);
-    }
-    // a 128-element chunk is half of a 256-element sum group: its four sub-blocks go to blocks 0..3
-    static __device__ __forceinline__ int xs_index(int c, int g, int lane) {
-        return ((c >> 1) * 4 + g) * 32 + (c & 1) * 16 + (lane & 15);
-    }
-};
-
-template <class F, int NG>
-struct Stage {
-    typename F::Regs w;
-    u32x2 xa[F::NPAIR][NG];
-    float xs[NG];
-};
-
-template <class F, int NG>
-__device__ __forceinline__ void load_stage(Stage<F, NG>& st, const GemmArgs& a, const uint8_t* wt, int c, int lane) {
-    // The loads of one stage stay together and in program order (scheduling fences on both
-    // sides), so "stage s has landed" is one s_waitcnt vmcnt(n) with the same n on every path.
-    __builtin_amdgcn_sched_barrier(0);
-    const u32x2* xp = (const u32x2*)a.xfrag + (size_t)c * F::NPAIR * 256 + lane;
-#pragma unroll
-    for (int p = 0; p < F::NPAIR; p++)
-#pragma unroll
-        for (int g = 0; g < NG; g++) st.xa[p][g] = xp[(p * 4 + g) * 64];
-#pragma unroll
-    for (int g = 0; g < NG; g++) st.xs[g] = a.xsum[F::xs_index(c, g, lane)];
-    F::load(st.w, wt + (size_t)c * F::TILE_BYTES, lane);
-    __builtin_amdgcn_sched_barrier(0);
-}
-
-__device__ __forceinline__ void fma4(float4v& t, float s, const float4v& d) {
-    t.x = __builtin_fmaf(s, d.x, t.x);
-    t.y = __builtin_fmaf(s, d.y, t.y);
-    t.z = __builtin_fmaf(s, d.z, t.z);
-    t.w = __builtin_fmaf(s, d.w, t.w);
-}
-
-// One Q4_K superblock tile (64 weight rows x 256 K) against NG groups of four activation rows.
-//   t  = - sum_j (d*sc_j*off_j + dmin*m_j) * sum_k X_jk       8 fp32 MFMAs per group
-//   t += sum_j d*sc_j * (X_j . (off_j + q_j))                  64 fp16 MFMAs per group
-// Both parts are summed per tile first so the large code offsets cancel before they reach the
-// running accumulator.
-template <int NG>
-__device__ __forceinline__ void compute(const Stage<Q4K, NG>& st, const Consts& k, float4v (&acc)[NG]) {
-    const Q4K::Regs& r = st.w;
-    const float d = h2f_lo(r.s.x), dmin = h2f_hi(r.s.x);
-    // 6-bit scale / min unpack (q4_k.rs:43-54), four sub-blocks per 32-bit word
-    const uint32_t sl = r.s.y & 0x3F3F3F3Fu, ml = r.s.z & 0x3F3F3F3Fu;
-    const uint32_t sh = (r.s.w & 0x0F0F0F0Fu) | ((r.s.y >> 2) & 0x30303030u);
-    const uint32_t mh = ((r.s.w >> 4) & 0x0F0F0F0Fu) | ((r.s.z >> 2) & 0x30303030u);
-    float sc[8], cf[8];
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        sc[j] = d * ubyte(j < 4 ? sl : sh, j & 3);
-        const float mn = dmin * ubyte(j < 4 ? ml : mh, j & 3);
-        // even sub-blocks carry the 1024 code offset, odd ones 64
-        cf[j] = -__builtin_fmaf(sc[j], (j & 1) ? 64.0f : 1024.0f, mn);
-    }
-    float4v t[NG];
-#pragma unroll
-    for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
-    static_for<8>([&](auto J) {
-        constexpr int j = decltype(J)::value;
-#pragma unroll
-        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(st.xs[g], cf[j], t[g]);
-    });
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-        float4v dlo[NG], dhi[NG];
-#pragma unroll
-        for (int g = 0; g < NG; g++) dlo[g] = dhi[g] = float4v{0.f, 0.f, 0.f, 0.f};
-        static_for<8>([&](auto W) {
-            constexpr int w = decltype(W)::value;
-            const uint32_t word = r.q[2 * p + w / 4][w % 4];
-            const uint32_t v = word >> 8;
-            const u32x2 blo = {and_or(word, 0x000F000Fu, k.k6400), and_or(v, 0x000F000Fu, k.k6400)};
-            const u32x2 bhi = {and_or(word, 0x00F000F0u, k.k5400), and_or(v, 0x00F000F0u, k.k5400)};
-#pragma unroll
-            for (int g = 0; g < NG; g++) {
-                dlo[g] = mfma_f16<w>(st.xa[p][g], blo, dlo[g]);
-                dhi[g] = mfma_f16<w + 8>(st.xa[p][g], bhi, dhi[g]);
-            }
-        });
-#pragma unroll
-        for (int g = 0; g < NG; g++) {
-            fma4(t[g], sc[2 * p], dlo[g]);
-            fma4(t[g], sc[2 * p + 1], dhi[g]);
-        }
-    }
-#pragma unroll
-    for (int g = 0; g < NG; g++) acc[g] += t[g];
-}
-
-// One Q8_0 tile (64 rows x 128 K = four 32-element blocks).  Codes go in as 1024 + (q + 128);
-// the 1152 offset comes back out through the activation sums on the fp32 matrix pipe.
-template <int NG>
-__device__ __forceinline__ void compute(const Stage<Q80, NG>& st, const Consts& k, float4v (&acc)[NG]) {
-    const Q80::Regs& r = st.w;
-    float dj[4] = {h2f_lo(r.s.x), h2f_hi(r.s.x), h2f_lo(r.s.y), h2f_hi(r.s.y)};
-    float4v t[NG];
-#pragma unroll
-    for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
-    static_for<4>([&](auto J) {
-        constexpr int j = decltype(J)::value;
-#pragma unroll
-        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(st.xs[g], dj[j] * -1152.0f, t[g]);
-    });
-#pragma unroll
-    for (int p = 0; p < 2; p++) {
-        float4v da[NG], db[NG];
-#pragma unroll
-        for (int g = 0; g < NG; g++) da[g] = db[g] = float4v{0.f, 0.f, 0.f, 0.f};
-        static_for<8>([&](auto W) {
-            constexpr int w = decltype(W)::value;
-            // bytes -> fp16 1024 + (q + 128): interleave each byte with 0x64
-            const uint32_t wa = r.q[4 * p + w / 4][w % 4] ^ 0x80808080u;
-            const uint32_t wb = r.q[4 * p + 2 + w / 4][w % 4] ^ 0x80808080u;
-            const u32x2 ba = {__builtin_amdgcn_perm(k.k64, wa, 0x04020400u), __builtin_amdgcn_perm(k.k64, wa, 0x04030401u)};
-            const u32x2 bb = {__builtin_amdgcn_perm(k.k64, wb, 0x04020400u), __builtin_amdgcn_perm(k.k64, wb, 0x04030401u)};
-#pragma unroll
-            for (int g = 0; g < NG; g++) {
-                da[g] = mfma_f16<w>(st.xa[p][g], ba, da[g]);
-                db[g] = mfma_f16<w + 8>(st.xa[p][g], bb, db[g]);
-            }
-        });
-#pragma unroll
-        for (int g = 0; g < NG; g++) {
-            fma4(t[g], dj[2 * p], da[g]);
-            fma4(t[g], dj[2 * p + 1], db[g]);
-        }
-    }
-#pragma unroll
-    for (int g = 0; g < NG; g++) acc[g] += t[g];
-}
-
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 
 // Stores one row group's finished sums.  v[i] is output column n of activation row 4g+i.
 template <int EPI>
@@ -373,15 +164,17 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     // outstanding tile only (s_waitcnt vmcnt(n)) instead of draining the queue.
     if (nc > 0) {
         Stage<F, NG> st[STAGES];
+        const ActLoader<false> x(a.xfrag, a.xsum);
         const int last = c0 + nc - 1;
+        auto fetch = [&](Stage<F, NG>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
 #pragma unroll
-        for (int s = 0; s < STAGES; s++) load_stage(st[s], a, wt, min(c0 + s, last), lane);
+        for (int s = 0; s < STAGES; s++) fetch(st[s], min(c0 + s, last));
         int c = 0;
         for (; c + 2 * STAGES <= nc; c += STAGES) {
 #pragma unroll
             for (int s = 0; s < STAGES; s++) {
                 compute(st[s], k, acc);
-                load_stage(st[s], a, wt, c0 + c + s + STAGES, lane);
+                fetch(st[s], c0 + c + s + STAGES);
             }
         }
         // last group that still has tiles to fetch (fewer than STAGES of them)
@@ -389,7 +182,7 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
         for (int s = 0; s < STAGES; s++) {
             if (c + s < nc) {
                 compute(st[s], k, acc);
-                if (c + s + STAGES < nc) load_stage(st[s], a, wt, c0 + c + s + STAGES, lane);
+                if (c + s + STAGES < nc) fetch(st[s], c0 + c + s + STAGES);
             }
         }
         c += STAGES;

@@ -1,0 +1,250 @@
+// Device-side core of the dequant-fused small-M matmul: weight-tile formats, the register stage
+// of the software pipeline, and the per-tile MFMA sequences.  Shared by the stand-alone matmul
+// kernel and the fused per-XCD layer kernels.
+#pragma once
+#include <utility>
+
+#include "tsv_internal.h"
+
+namespace tsv {
+
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ------------------------------------------------------------------------------- helpers
+template <int... I, class Fn>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, Fn&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// D[i] += sum_k A_step[i][k] * B_lane[k]: A taken from block `STEP` of the a operand for all lanes
+template <int STEP>
+__device__ __forceinline__ float4v mfma_f16(u32x2 a, u32x2 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4, a), __builtin_bit_cast(half4, b), c, 4, STEP, 0);
+}
+template <int STEP>
+__device__ __forceinline__ float4v mfma_f32(float a, float b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 4, STEP, 0);
+}
+
+__device__ __forceinline__ float h2f_lo(uint32_t v) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(v & 0xFFFF));
+}
+__device__ __forceinline__ float h2f_hi(uint32_t v) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(v >> 16));
+}
+__device__ __forceinline__ float ubyte(uint32_t v, int i) { return (float)((v >> (8 * i)) & 0xFF); }
+
+// (v & mask) | bits as ONE v_and_or_b32: the instruction can take a single literal / scalar
+// operand, so the second constant is pinned in a vector register.
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits_vgpr) {
+    return (v & mask) | bits_vgpr;
+}
+
+struct Consts {
+    uint32_t k6400, k5400, k64;
+};
+
+// ------------------------------------------------------------------------------- formats
+struct Q4K {
+    static constexpr int NSUB = 8, NPAIR = 4, TILE_BYTES = 9216;
+    struct Regs {
+        u32x4 q[8];
+        u32x4 s;
+    };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
+        const u32x4* p = (const u32x4*)tile + lane;
+#pragma unroll
+        for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
+        r.s = __builtin_nontemporal_load(p + 512);
+    }
+    // float index of this lane's sub-block sums for row group g of chunk c
+    static __device__ __forceinline__ int xs_index(int c, int g, int lane) { return (c * 4 + g) * 32 + (lane & 31); }
+};
+
+struct Q80 {
+    static constexpr int NSUB = 4, NPAIR = 2, TILE_BYTES = 8704;
+    struct Regs {
+        u32x4 q[8];
+        u32x2 s;
+    };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
+        const u32x4* p = (const u32x4*)tile + lane;
+#pragma unroll
+        for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
+        r.s = __builtin_nontemporal_load((const u32x2*)(tile + 8192) + lane);
+    }
+    // a 128-element chunk is half of a 256-element sum group: its four sub-blocks go to blocks 0..3
+    static __device__ __forceinline__ int xs_index(int c, int g, int lane) {
+        return ((c >> 1) * 4 + g) * 32 + (c & 1) * 16 + (lane & 15);
+    }
+};
+
+template <class F, int NG>
+struct Stage {
+    typename F::Regs w;
+    u32x2 xa[F::NPAIR][NG];
+    float xs[NG];
+};
+
+// Cache policy of the activation loads: plain, or device-coherent (sc1) for activations that
+// another compute unit wrote earlier in the same kernel (they must not come from this CU's L1).
+template <bool COHERENT>
+struct ActLoader {
+    __amdgpu_buffer_rsrc_t frag, sums;
+    const u32x2* fragp;
+    const float* sump;
+    __device__ __forceinline__ ActLoader(const void* xfrag, const void* xsum) {
+        fragp = (const u32x2*)xfrag;
+        sump = (const float*)xsum;
+        if (COHERENT) {
+            frag = __builtin_amdgcn_make_buffer_rsrc((void*)xfrag, 0, 0x7FFFFFFF, 0x00027000);
+            sums = __builtin_amdgcn_make_buffer_rsrc((void*)xsum, 0, 0x7FFFFFFF, 0x00027000);
+        }
+    }
+    __device__ __forceinline__ u32x2 frag_at(int idx) const {  // idx in 8-byte units
+        if (COHERENT) return __builtin_amdgcn_raw_buffer_load_b64(frag, idx * 8, 0, 16);
+        return fragp[idx];
+    }
+    __device__ __forceinline__ float sum_at(int idx) const {
+        if (COHERENT) return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sums, idx * 4, 0, 16));
+        return sump[idx];
+    }
+};
+
+// activations of K chunk c (chunk index in the activation's own K axis)
+template <class F, int NG, bool COH>
+__device__ __forceinline__ void load_x(Stage<F, NG>& st, const ActLoader<COH>& x, int c, int lane) {
+#pragma unroll
+    for (int p = 0; p < F::NPAIR; p++)
+#pragma unroll
+        for (int g = 0; g < NG; g++) st.xa[p][g] = x.frag_at(((c * F::NPAIR + p) * 4 + g) * 64 + lane);
+#pragma unroll
+    for (int g = 0; g < NG; g++) st.xs[g] = x.sum_at(F::xs_index(c, g, lane));
+}
+
+// The loads of one stage stay together and in program order (scheduling fences on both sides),
+// so "stage s has landed" is one s_waitcnt vmcnt(n) with the same n on every path.
+template <class F, int NG, bool COH>
+__device__ __forceinline__ void load_stage(Stage<F, NG>& st, const ActLoader<COH>& x, const uint8_t* tile_chunk, int c,
+                                           int lane) {
+    __builtin_amdgcn_sched_barrier(0);
+    load_x(st, x, c, lane);
+    F::load(st.w, tile_chunk, lane);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void fma4(float4v& t, float s, const float4v& d) {
+    t.x = __builtin_fmaf(s, d.x, t.x);
+    t.y = __builtin_fmaf(s, d.y, t.y);
+    t.z = __builtin_fmaf(s, d.z, t.z);
+    t.w = __builtin_fmaf(s, d.w, t.w);
+}
+
+// One Q4_K superblock tile (64 weight rows x 256 K) against NG groups of four activation rows.
+//   t  = - sum_j (d*sc_j*off_j + dmin*m_j) * sum_k X_jk       8 fp32 MFMAs per group
+//   t += sum_j d*sc_j * (X_j . (off_j + q_j))                  64 fp16 MFMAs per group
+// Both parts are summed per tile first so the large code offsets cancel before they reach the
+// running accumulator.
+template <int NG>
+__device__ __forceinline__ void compute(const Stage<Q4K, NG>& st, const Consts& k, float4v (&acc)[NG]) {
+    const Q4K::Regs& r = st.w;
+    const float d = h2f_lo(r.s.x), dmin = h2f_hi(r.s.x);
+    // 6-bit scale / min unpack (q4_k.rs:43-54), four sub-blocks per 32-bit word
+    const uint32_t sl = r.s.y & 0x3F3F3F3Fu, ml = r.s.z & 0x3F3F3F3Fu;
+    const uint32_t sh = (r.s.w & 0x0F0F0F0Fu) | ((r.s.y >> 2) & 0x30303030u);
+    const uint32_t mh = ((r.s.w >> 4) & 0x0F0F0F0Fu) | ((r.s.z >> 2) & 0x30303030u);
+    float sc[8], cf[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        sc[j] = d * ubyte(j < 4 ? sl : sh, j & 3);
+        const float mn = dmin * ubyte(j < 4 ? ml : mh, j & 3);
+        // even sub-blocks carry the 1024 code offset, odd ones 64
+        cf[j] = -__builtin_fmaf(sc[j], (j & 1) ? 64.0f : 1024.0f, mn);
+    }
+    float4v t[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
+    static_for<8>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+#pragma unroll
+        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(st.xs[g], cf[j], t[g]);
+    });
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        float4v dlo[NG], dhi[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) dlo[g] = dhi[g] = float4v{0.f, 0.f, 0.f, 0.f};
+        static_for<8>([&](auto W) {
+            constexpr int w = decltype(W)::value;
+            const uint32_t word = r.q[2 * p + w / 4][w % 4];
+            const uint32_t v = word >> 8;
+            const u32x2 blo = {and_or(word, 0x000F000Fu, k.k6400), and_or(v, 0x000F000Fu, k.k6400)};
+            const u32x2 bhi = {and_or(word, 0x00F000F0u, k.k5400), and_or(v, 0x00F000F0u, k.k5400)};
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                dlo[g] = mfma_f16<w>(st.xa[p][g], blo, dlo[g]);
+                dhi[g] = mfma_f16<w + 8>(st.xa[p][g], bhi, dhi[g]);
+            }
+        });
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            fma4(t[g], sc[2 * p], dlo[g]);
+            fma4(t[g], sc[2 * p + 1], dhi[g]);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < NG; g++) acc[g] += t[g];
+}
+
+// One Q8_0 tile (64 rows x 128 K = four 32-element blocks).  Codes go in as 1024 + (q + 128);
+// the 1152 offset comes back out through the activation sums on the fp32 matrix pipe.
+template <int NG>
+__device__ __forceinline__ void compute(const Stage<Q80, NG>& st, const Consts& k, float4v (&acc)[NG]) {
+    const Q80::Regs& r = st.w;
+    float dj[4] = {h2f_lo(r.s.x), h2f_hi(r.s.x), h2f_lo(r.s.y), h2f_hi(r.s.y)};
+    float4v t[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
+    static_for<4>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+#pragma unroll
+        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(st.xs[g], dj[j] * -1152.0f, t[g]);
+    });
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        float4v da[NG], db[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) da[g] = db[g] = float4v{0.f, 0.f, 0.f, 0.f};
+        static_for<8>([&](auto W) {
+            constexpr int w = decltype(W)::value;
+            // bytes -> fp16 1024 + (q + 128): interleave each byte with 0x64
+            const uint32_t wa = r.q[4 * p + w / 4][w % 4] ^ 0x80808080u;
+            const uint32_t wb = r.q[4 * p + 2 + w / 4][w % 4] ^ 0x80808080u;
+            const u32x2 ba = {__builtin_amdgcn_perm(k.k64, wa, 0x04020400u), __builtin_amdgcn_perm(k.k64, wa, 0x04030401u)};
+            const u32x2 bb = {__builtin_amdgcn_perm(k.k64, wb, 0x04020400u), __builtin_amdgcn_perm(k.k64, wb, 0x04030401u)};
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                da[g] = mfma_f16<w>(st.xa[p][g], ba, da[g]);
+                db[g] = mfma_f16<w + 8>(st.xa[p][g], bb, db[g]);
+            }
+        });
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            fma4(t[g], dj[2 * p], da[g]);
+            fma4(t[g], dj[2 * p + 1], db[g]);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < NG; g++) acc[g] += t[g];
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+
+}  // namespace tsv

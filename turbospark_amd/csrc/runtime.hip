@@ -41,6 +41,17 @@ struct tsv_ctx {
     uint4 *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
     float* partial = nullptr;
     size_t partial_floats = 0;
+    // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
+    // sum-of-squares partials, per-XCD partial sums, barrier counters
+    bool fused_ffn = false;
+    float* x2 = nullptr;
+    uint8_t* frag8 = nullptr;
+    size_t frag8_stride = 0;
+    float* ssq8 = nullptr;
+    float* partial8 = nullptr;
+    unsigned *rank_ctr = nullptr, *bar_ctr = nullptr;
+    int* fused_err = nullptr;  // pinned host memory the kernels can write
+    unsigned bar_count = 0;
     uint16_t* q16 = nullptr;
     float *part_o = nullptr, *part_ml = nullptr;
     int nch = 0;
@@ -326,12 +337,14 @@ int launch_pass(tsv_ctx* c, int m) {
     }
     if (rc) return rc;
     int prev_splits = 0;
+    const float* prev_partial = c->partial;
+    float *x = c->x, *x_other = c->x2;  // the fused kernels write the residual rows to the other buffer
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
         {
             PROF(PC_NORM);
-            rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m);
+            rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m);
         }
         if (rc) return rc;
         int sp = splits_for(L.qkv, m, EPI_PARTIAL);
@@ -386,9 +399,46 @@ int launch_pass(tsv_ctx* c, int m) {
             rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
         }
         if (rc) return rc;
+        if (c->fused_ffn) {
+            FfnBlockArgs fa;
+            fa.sync.rank_ctr = c->rank_ctr;
+            fa.sync.bar_ctr = c->bar_ctr;
+            fa.sync.err = c->fused_err;
+            fa.sync.bar_base = c->bar_count;
+            c->bar_count += 32u * (unsigned)fused_ffn_barriers();
+            fa.norm.x_in = x;
+            fa.norm.x_out = x_other;
+            fa.norm.partial = c->partial;
+            fa.norm.n_partials = sp;
+            fa.norm.norm_w = L.ffn_norm;
+            fa.norm.frag = c->frag8;
+            fa.norm.frag_stride = c->frag8_stride;
+            fa.norm.ssq = c->ssq8;
+            fa.norm.hidden = c->hidden;
+            fa.norm.eps = c->eps;
+            fa.vp = c->vp_dev;
+            fa.w_gate_up = L.gate_up.tiles;
+            fa.gu_tiles = L.gate_up.n_tiles;
+            fa.gu_kchunks = L.gate_up.kchunks;
+            fa.frag_c = c->xf_c;
+            fa.ffn = c->ffn;
+            fa.w_down = L.down.tiles;
+            fa.down_tiles = L.down.n_tiles;
+            fa.down_kchunks = L.down.kchunks;
+            fa.partial_out = c->partial8;
+            {
+                PROF(PC_GATEUP);
+                rc = launch_ffn_block(s, L.gate_up.fmt, fa, m);
+            }
+            if (rc) return rc;
+            std::swap(x, x_other);
+            prev_partial = c->partial8;
+            prev_splits = 8;
+            continue;
+        }
         {
             PROF(PC_NORM);
-            rc = launch_addnorm(s, c->x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m);
+            rc = launch_addnorm(s, x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m);
         }
         if (rc) return rc;
         {
@@ -402,11 +452,12 @@ int launch_pass(tsv_ctx* c, int m) {
             rc = launch_gemm(s, L.down, c->xf_c, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
         }
         if (rc) return rc;
+        prev_partial = c->partial;
         prev_splits = sp;
     }
     {
         PROF(PC_NORM);
-        rc = launch_addnorm(s, c->x, c->partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m);
+        rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m);
     }
     if (rc) return rc;
     {
@@ -440,10 +491,22 @@ int run_pass(tsv_ctx* c, int m) {
     return TSV_OK;
 }
 
+// After a stream synchronisation: did a fused kernel give up on a barrier?  Its results are then
+// incomplete; the handle switches to the unfused kernels for good and reports the failure.
+int check_fused(tsv_ctx* c) {
+    if (!c->fused_err || *c->fused_err == 0) return TSV_OK;
+    set_error(*c->fused_err == 2 ? "fused layer kernel: unexpected XCD id; fused path disabled, repeat the call"
+                                 : "fused layer kernel: XCD barrier timed out; fused path disabled, repeat the call");
+    *c->fused_err = 0;
+    c->fused_ffn = false;
+    return TSV_ERR_DEVICE;
+}
+
 int finish_verify(tsv_ctx* c, int m, uint16_t* logits_out) {
     if (logits_out) {
         TSV_HIP(hipMemcpyAsync(logits_out, c->logits, (size_t)m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
         TSV_HIP(hipStreamSynchronize(c->stream));
+        return check_fused(c);
     }
     return TSV_OK;
 }
@@ -577,6 +640,33 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->sc.counters, 64 * 4, true)) ||
         (rc = dev_alloc(c, &c->sc.result, sizeof(AcceptResult), true)))
         return fail(rc);
+    {
+        // per-XCD fused kernels: every layer must fit their sharding; they need all 256
+        // workgroups resident at once (cooperative launch) and a fresh barrier base per launch
+        // (so not inside a captured graph)
+        bool ok = !c->use_graph;
+        if (const char* e = getenv("TSV_FUSED")) ok = ok && e[0] != '0';
+        int coop = 0, ncu = 0;
+        if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, 0) != hipSuccess) coop = 0;
+        if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) ncu = 0;
+        ok = ok && coop && ncu == 256;
+        for (const LayerW& L : c->layers) ok = ok && fused_ffn_supported(L.gate_up, L.down, c->hidden, c->ffn);
+        if (ok) {
+            c->frag8_stride = (xfrag_bytes(c->hidden) + 255) & ~(size_t)255;
+            if ((rc = dev_alloc(c, &c->x2, (size_t)16 * c->hidden * 4, true)) ||
+                (rc = dev_alloc(c, &c->frag8, 8 * c->frag8_stride, true)) ||
+                (rc = dev_alloc(c, &c->ssq8, (size_t)8 * 16 * 32 * 4, true)) ||
+                (rc = dev_alloc(c, &c->partial8, (size_t)8 * 16 * c->hidden * 4, true)) ||
+                (rc = dev_alloc(c, &c->rank_ctr, 8 * 64 * 4, true)) || (rc = dev_alloc(c, &c->bar_ctr, 8 * 64 * 4, true)))
+                return fail(rc);
+            if (hipHostMalloc((void**)&c->fused_err, sizeof(int)) != hipSuccess) {
+                set_error("open: pinned host allocation failed");
+                return fail(TSV_ERR_DEVICE);
+            }
+            *c->fused_err = 0;
+            c->fused_ffn = true;
+        }
+    }
     if (hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
         hipHostMalloc((void**)&c->ap_host, sizeof(AcceptParams)) != hipSuccess ||
         hipHostMalloc((void**)&c->res_host, sizeof(AcceptResult)) != hipSuccess ||
@@ -600,6 +690,7 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
+    if (c->fused_err) (void)hipHostFree(c->fused_err);
     for (hipGraphExec_t g : c->pass_graph)
         if (g) (void)hipGraphExecDestroy(g);
     for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
@@ -677,7 +768,7 @@ extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_
         }
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
-    return TSV_OK;
+    return check_fused(c);
 }
 
 extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {
@@ -793,6 +884,7 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     if (r->logits_out)
         TSV_HIP(hipMemcpyAsync(r->logits_out, c->logits, (size_t)r->m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipStreamSynchronize(c->stream));
+    if ((rc = check_fused(c))) return rc;
     const AcceptResult& a = *c->res_host;
     if (a.error) {
         set_error("accept: score vector must not contain a non-finite entry");

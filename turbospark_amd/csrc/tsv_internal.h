@@ -101,6 +101,44 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
                 int m, int splits, int epi, int ldo, int n_valid);
 int gemm_default_splits(const TiledW& w, int m);
 
+// ---- per-XCD fused layer kernels ----------------------------------------------------------
+// Counters of the XCD-local barriers.  rank_ctr / bar_ctr: one word per XCD, 64 words apart.
+// A launch that uses n barriers advances every bar_ctr by 32 * n; bar_base is its value before.
+struct FusedSync {
+    unsigned* rank_ctr;
+    unsigned* bar_ctr;
+    int* err;  // host-visible: 1 = a barrier timed out, 2 = unexpected XCD id
+    unsigned bar_base;
+};
+// Residual add + RMSNorm inputs stage shared by the fused kernels.
+struct NormStage {
+    const float* x_in;     // [16][hidden]
+    float* x_out;          // a different buffer: other XCDs may still be reading x_in
+    const float* partial;  // [n_partials][16][hidden] partial sums to add (n_partials <= 8)
+    int n_partials;
+    const float* norm_w;
+    uint8_t* frag;         // 8 private copies of the activation fragments, frag_stride bytes apart
+    size_t frag_stride;
+    float* ssq;            // [8][16][32] sums of squares per workgroup
+    int hidden;
+    float eps;
+};
+struct FfnBlockArgs {
+    FusedSync sync;
+    NormStage norm;
+    const VerifyParams* vp;
+    const uint8_t* w_gate_up;
+    int gu_tiles, gu_kchunks;
+    uint4* frag_c;  // silu(gate) * up as fragments, K = ffn
+    int ffn;
+    const uint8_t* w_down;
+    int down_tiles, down_kchunks;
+    float* partial_out;  // [8][16][hidden]
+};
+bool fused_ffn_supported(const TiledW& gate_up, const TiledW& down, int hidden, int ffn);
+int fused_ffn_barriers();
+int launch_ffn_block(hipStream_t s, int fmt, FfnBlockArgs& a, int m);
+
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
                  const VerifyParams* vp, int m);
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,

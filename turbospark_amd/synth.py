@@ -12,6 +12,12 @@ CONFIGS = {
     # a small Q4_K stand-in with the 8B model's head geometry (GQA 4, head_dim 128)
     "small_q4_k": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
                        vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
+    # the smallest shapes the per-XCD fused layer kernels take (8 KV heads, widths divisible
+    # into eight chunk-aligned slices); norm weights are not all ones here
+    "xcd_q4_k": dict(n_layers=2, hidden=1024, n_q_heads=32, n_kv_heads=8, head_dim=64, ffn=2048,
+                     vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K, norm_jitter=0.25),
+    "xcd_q8_0": dict(n_layers=2, hidden=1024, n_q_heads=16, n_kv_heads=8, head_dim=64, ffn=1024,
+                     vocab=4096, rms_eps=1e-5, rope_theta=10000.0, dtype=ffi.Q8_0, norm_jitter=0.25),
     # Llama-3-8B shape
     "llama3_8b_q4_k": dict(n_layers=32, hidden=4096, n_q_heads=32, n_kv_heads=8, head_dim=128,
                            ffn=14336, vocab=128256, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
@@ -24,7 +30,15 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
     dt = cfg["dtype"]
     H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
     qd, kvd = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
-    ones = lambda n: (ffi.F32, np.ones((1, n), np.float32).view(np.uint8).reshape(1, -1), 1, n)
+    jitter = float(cfg.get("norm_jitter", 0.0))
+    nrng = np.random.default_rng(seed + 99)
+
+    def ones(n):
+        v = np.ones((1, n), np.float32)
+        if jitter:
+            v = (v + jitter * nrng.uniform(-1.0, 1.0, (1, n))).astype(np.float32)
+        return (ffi.F32, v.view(np.uint8).reshape(1, -1), 1, n)
+
     stream = [0]
 
     def t(rows, cols):
