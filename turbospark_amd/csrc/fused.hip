@@ -64,10 +64,11 @@ __device__ __forceinline__ bool xcd_enter(XcdCtx& c, const FusedSync& s, int* ld
     return true;
 }
 
-// Barrier over the 32 workgroups of this XCD.  Every wave first waits for its own stores to be
-// acknowledged by the L2.
-__device__ __forceinline__ bool xcd_barrier(XcdCtx& c, int* lds_i) {
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+// Barrier over the 32 workgroups of this XCD.  A wave that stored something the other side of
+// the barrier will read first waits for its stores to be acknowledged by the L2 (drain); a wave
+// that only has weight prefetches in flight must not wait for those here.
+__device__ __forceinline__ bool xcd_barrier(XcdCtx& c, int* lds_i, bool drain = true) {
+    if (drain) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         __hip_atomic_fetch_add(c.bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -99,45 +100,51 @@ __device__ __forceinline__ float ld_sc1(const float* base, int idx) {
 // fp16 fragments of x * norm_w with their sub-block sums; and sum(x^2) over this workgroup's
 // columns.  Every XCD computes the same numbers; XCD 0 stores x, into a second buffer because
 // the other XCDs read the old rows at their own pace.
-__device__ __forceinline__ void norm_inputs(const NormStage& n, const XcdCtx& c, int M, float* lds_f) {
-    const int cpw = n.hidden / WGS_PER_XCD;  // columns per workgroup, a multiple of 32
+// Called by `nw` whole waves of the workgroup (wave index wi of nw): a wave takes rows wi,
+// wi + nw, ... and all of the workgroup's columns of each, so nothing is shared between waves
+// and the waves that are busy prefetching weights are not involved.
+__device__ __forceinline__ void norm_inputs(const NormStage& n, const XcdCtx& c, int M, int wi, int nw) {
+    const int cpw = n.hidden / WGS_PER_XCD;  // columns per workgroup, a multiple of 32, at most 256
     const int col0 = c.rank * cpw;
     _Float16* frag = (_Float16*)(n.frag + (size_t)c.xcc * n.frag_stride);
     float* sums = (float*)((char*)frag + xfrag_sum_offset(n.hidden));
     const int lane = threadIdx.x & 63;
-    const int nslot = cpw >> 5;
-    for (int idx = threadIdx.x; idx < cpw * 16; idx += 512) {
-        const int b = idx / cpw, cl = idx - b * cpw, col = col0 + cl;
-        float xv = 0.f;
-        if (b < M) {
-            xv = n.x_in[(size_t)b * n.hidden + col];
-            float p[8];
+    for (int b = wi; b < M; b += nw) {
+        float xin[4], wn[4], part[4][8];
 #pragma unroll
-            for (int s = 0; s < 8; s++) p[s] = s < n.n_partials ? n.partial[((size_t)s * 16 + b) * n.hidden + col] : 0.f;
+        for (int j = 0; j < 4; j++) {
+            const int cl = lane + 64 * j;
+            if (cl < cpw) {
+                xin[j] = n.x_in[(size_t)b * n.hidden + col0 + cl];
+                wn[j] = n.norm_w[col0 + cl];
 #pragma unroll
-            for (int s = 0; s < 8; s++) xv += p[s];
-            if (c.xcc == 0) n.x_out[(size_t)b * n.hidden + col] = xv;
+                for (int s = 0; s < 8; s++)
+                    if (s < n.n_partials) part[j][s] = n.partial[((size_t)s * 16 + b) * n.hidden + col0 + cl];
+            }
         }
-        const _Float16 h = (_Float16)(xv * n.norm_w[col]);
-        if (b < M) frag[frag_index(col, b)] = h;
-        float sum = (float)h, sq = xv * xv;
+        float sq = 0.f;
 #pragma unroll
-        for (int o = 1; o < 32; o <<= 1) {
-            sum += __shfl_xor(sum, o);
-            sq += __shfl_xor(sq, o);
+        for (int j = 0; j < 4; j++) {
+            const int cl = lane + 64 * j, col = col0 + cl;
+            if (cl < cpw) {  // cpw is a multiple of 32: half waves leave together
+                float xv = xin[j];
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+                    if (s < n.n_partials) xv += part[j][s];
+                if (c.xcc == 0) n.x_out[(size_t)b * n.hidden + col] = xv;
+                const _Float16 h = (_Float16)(xv * wn[j]);
+                frag[frag_index(col, b)] = h;
+                float sum = (float)h;
+#pragma unroll
+                for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
+                if ((lane & 31) == 0) sums[xsum_index(col >> 5, b)] = sum;
+                sq += xv * xv;
+            }
         }
-        if ((lane & 31) == 0) {
-            if (b < M) sums[xsum_index(col >> 5, b)] = sum;
-            lds_f[b * 8 + (cl >> 5)] = sq;
-        }
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) sq += __shfl_xor(sq, o);
+        if (lane == 0) n.ssq[((size_t)c.xcc * 16 + b) * WGS_PER_XCD + c.rank] = sq;
     }
-    __syncthreads();
-    if (threadIdx.x < 16) {
-        float ss = 0.f;
-        for (int s = 0; s < nslot; s++) ss += lds_f[threadIdx.x * 8 + s];
-        n.ssq[((size_t)c.xcc * 16 + threadIdx.x) * WGS_PER_XCD + c.rank] = ss;
-    }
-    __syncthreads();
 }
 
 // Row b's 1/rms from the XCD's 32 column partials, for all 16 rows, into LDS.
@@ -155,53 +162,90 @@ __device__ __forceinline__ void norm_factors(const NormStage& n, const XcdCtx& c
 }
 
 // ---- matmul items -----------------------------------------------------------------------------
-// One wave's share of a tile: chunks [c0, c0 + nc) of the weight tile row `tile` (kchunks per
-// row), against the activations whose chunk index is the weight's.  `prefetch` issues the first
-// two weight stages and can run before the activations exist; `run` finishes the job.
-template <class F, int NG>
-struct TileJob {
-    Stage<F, NG> st[2];
-    const uint8_t* wt;
+// One wave's share of a tile: chunks [c0, c0 + nc) of a weight tile row, against the activations
+// whose chunk index is the weight's.
+struct JobDesc {
+    const uint8_t* wt;  // chunk 0 of the tile row
     int c0, nc;
+};
 
-    __device__ __forceinline__ void prefetch(const uint8_t* w, int kchunks, int tile, int c0_, int nc_, int lane) {
-        wt = w + (size_t)tile * kchunks * F::TILE_BYTES;
-        c0 = c0_;
-        nc = nc_;
-        if (nc <= 0) return;
+// The weights of a job can be requested long before its activations exist -- that is what keeps
+// HBM busy across the barriers.  Per wave, two chunks wait in registers and two more in LDS
+// (copied there by the memory pipeline); a job's last chunks are the LDS ones, the earlier ones
+// stream through the two register stages.
+template <class F, int NG>
+struct WaveJob {
+    typename F::Regs wr[2];
+    XRegs<F, NG> xr[2];
+    uint32_t lds0, lds1;  // LDS addresses of this wave's two tile buffers
+    int lane;
+
+    static __device__ __forceinline__ int n_lds(int nc) { return nc >= 3 ? min(2, nc - 2) : 0; }
+
+    __device__ __forceinline__ void issue_regs(const JobDesc& j) {
+        if (j.nc <= 0) return;
         __builtin_amdgcn_sched_barrier(0);
-        F::load(st[0].w, wt + (size_t)c0 * F::TILE_BYTES, lane);
-        F::load(st[1].w, wt + (size_t)(c0 + min(1, nc - 1)) * F::TILE_BYTES, lane);
+        F::load(wr[0], j.wt + (size_t)j.c0 * F::TILE_BYTES, lane);
+        F::load(wr[1], j.wt + (size_t)(j.c0 + min(1, j.nc - 1)) * F::TILE_BYTES, lane);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __device__ __forceinline__ void issue_lds(const JobDesc& j) {
+        const int nl = n_lds(j.nc);
+        __builtin_amdgcn_sched_barrier(0);
+        if (nl >= 1) F::load_to_lds(lds0, j.wt + (size_t)(j.c0 + j.nc - nl) * F::TILE_BYTES, lane);
+        if (nl >= 2) F::load_to_lds(lds1, j.wt + (size_t)(j.c0 + j.nc - 1) * F::TILE_BYTES, lane);
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    __device__ __forceinline__ void run(const ActLoader<true>& x, const Consts& k, float4v (&acc)[NG], int lane) {
+    // after_regs() runs once both register stages are free again (the next job's issue_regs)
+    template <class Fn>
+    __device__ __forceinline__ void run(const JobDesc& j, const ActLoader<true>& x, const Consts& k,
+                                        float4v (&acc)[NG], Fn&& after_regs) {
 #pragma unroll
         for (int g = 0; g < NG; g++) acc[g] = float4v{0.f, 0.f, 0.f, 0.f};
-        if (nc <= 0) return;
+        if (j.nc <= 0) {
+            after_regs();
+            return;
+        }
+        const int nl = n_lds(j.nc), nr = j.nc - nl, c0 = j.c0;
+        auto fetch = [&](int s, int c) {
+            __builtin_amdgcn_sched_barrier(0);
+            load_x(xr[s], x, c, lane);
+            F::load(wr[s], j.wt + (size_t)c * F::TILE_BYTES, lane);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto mul = [&](int s) { compute_tile<NG>(F{}, RegSrc<F>{wr[s]}, xr[s], k, acc); };
         __builtin_amdgcn_sched_barrier(0);
-        load_x(st[0], x, c0, lane);
-        load_x(st[1], x, c0 + min(1, nc - 1), lane);
+        load_x(xr[0], x, c0, lane);
+        load_x(xr[1], x, c0 + min(1, nr - 1), lane);
         __builtin_amdgcn_sched_barrier(0);
         int c = 0;
-        for (; c + 4 <= nc; c += 2) {
+        for (; c + 4 <= nr; c += 2) {
 #pragma unroll
             for (int s = 0; s < 2; s++) {
-                compute(st[s], k, acc);
-                load_stage(st[s], x, wt + (size_t)(c0 + c + s + 2) * F::TILE_BYTES, c0 + c + s + 2, lane);
+                mul(s);
+                fetch(s, c0 + c + s + 2);
             }
         }
 #pragma unroll
         for (int s = 0; s < 2; s++) {
-            if (c + s < nc) {
-                compute(st[s], k, acc);
-                if (c + s + 2 < nc) load_stage(st[s], x, wt + (size_t)(c0 + c + s + 2) * F::TILE_BYTES, c0 + c + s + 2, lane);
+            if (c + s < nr) {
+                mul(s);
+                if (c + s + 2 < nr) fetch(s, c0 + c + s + 2);
             }
         }
         c += 2;
 #pragma unroll
         for (int s = 0; s < 2; s++)
-            if (c + s < nc) compute(st[s], k, acc);
+            if (c + s < nr) mul(s);
+        // the LDS chunks: their activations first, then whatever the caller wants in flight next
+        __builtin_amdgcn_sched_barrier(0);
+        if (nl >= 1) load_x(xr[0], x, c0 + nr, lane);
+        if (nl >= 2) load_x(xr[1], x, c0 + nr + 1, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        after_regs();
+        if (nl >= 1) compute_tile<NG>(F{}, LdsSrc<F>{lds_after(lds0, xr[0].xs[NG - 1]), lane}, xr[0], k, acc);
+        if (nl >= 2) compute_tile<NG>(F{}, LdsSrc<F>{lds_after(lds1, xr[1].xs[NG - 1]), lane}, xr[1], k, acc);
     }
 };
 
@@ -213,8 +257,11 @@ __device__ __forceinline__ void quarter_split(int kchunks_lo, int kchunks_n, int
     nc = min(per, kchunks_lo + kchunks_n - c0);
 }
 
+// `red` shares LDS with the waves' weight buffers, which every wave has finished reading
+// once it arrives here.
 template <int NG>
 __device__ __forceinline__ bool fold_quarters(float4v (&acc)[NG], float4v* red, int wave, int lane, float4v& v) {
+    __syncthreads();
 #pragma unroll
     for (int g = 0; g < NG; g++) red[(wave * NG + g) * 64 + lane] = acc[g];
     __syncthreads();
@@ -243,52 +290,79 @@ __device__ long long g_trace[64 * 16];
 
 template <class F, int NG>
 __global__ __launch_bounds__(512) void k_ffn_block(FfnBlockArgs a) {
-    extern __shared__ float4v red[];
+    extern __shared__ uint8_t wbuf[];  // [8 waves][2][tile bytes]; the fold buffer overlays its start
     __shared__ float s_inv[16];
-    __shared__ float s_sq[16 * 8];
     __shared__ int s_i[4];
+    float4v* red = (float4v*)wbuf;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     XcdCtx ctx;
     if (!xcd_enter(ctx, a.sync, s_i)) return;
     TRACE(0);
-    const int M = a.vp->m;
+    const int M = a.m;
     Consts k;
     k.k6400 = 0x64006400u;
     k.k5400 = 0x54005400u;
     k.k64 = 0x64646464u;
     asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
+    WaveJob<F, NG> job;
+    job.lane = lane;
+    job.lds0 = __builtin_amdgcn_readfirstlane(lds_addr(wbuf) + wave * 2 * F::TILE_BYTES);
+    job.lds1 = job.lds0 + F::TILE_BYTES;
 
-    // gate/up tiles of this XCD: a contiguous run, two per workgroup and round
-    const int gu_per = a.gu_tiles / XCDS, gu0 = ctx.xcc * gu_per;
+    // The workgroup's eight waves work on two tiles at a time, four K quarters each.
     const int q = wave & 3, tw = wave >> 2;
-    TileJob<F, NG> job;
-    int c0, nc;
-    quarter_split(0, a.gu_kchunks, q, c0, nc);
-    {
-        const int t = 2 * ctx.rank + tw;
-        job.prefetch(a.w_gate_up, a.gu_kchunks, gu0 + min(t, gu_per - 1), c0, t < gu_per ? nc : 0, lane);
-    }
+    // gate/up: this XCD's tiles are a contiguous run
+    const int gu_per = a.gu_tiles / XCDS, gu0 = ctx.xcc * gu_per;
+    int gc0, gnc;
+    quarter_split(0, a.gu_kchunks, q, gc0, gnc);
+    auto gu_job = [&](int t0) {
+        const int t = t0 + tw;
+        return JobDesc{a.w_gate_up + (size_t)(gu0 + min(t, gu_per - 1)) * a.gu_kchunks * F::TILE_BYTES, gc0,
+                       t < gu_per ? gnc : 0};
+    };
+    // down: every tile, this XCD's K slice
+    const int dk = a.down_kchunks / XCDS;
+    int dc0, dnc;
+    quarter_split(ctx.xcc * dk, dk, q, dc0, dnc);
+    auto down_job = [&](int t0) {
+        const int t = t0 + tw;
+        return JobDesc{a.w_down + (size_t)min(t, a.down_tiles - 1) * a.down_kchunks * F::TILE_BYTES, dc0,
+                       t < a.down_tiles ? dnc : 0};
+    };
+    const int first = 2 * ctx.rank, stride = 2 * WGS_PER_XCD;
 
-    TRACE(1);
-    norm_inputs(a.norm, ctx, M, s_sq);
+    // Waves 3 and 7 prepare the RMSNorm inputs; the others request the weights of their first
+    // gate/up job at once (loads complete in issue order, so a wave's own small loads would
+    // otherwise queue behind its 36 KB of weights).
+    JobDesc cur = gu_job(first);
+    const bool norm_wave = q == 3;
+    if (norm_wave) {
+        norm_inputs(a.norm, ctx, M, tw, 2);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    job.issue_regs(cur);
+    job.issue_lds(cur);
     TRACE(2);
-    if (!xcd_barrier(ctx, s_i)) return;
+    if (!xcd_barrier(ctx, s_i, false)) return;
     TRACE(3);
-    norm_factors(a.norm, ctx, s_inv);
-    TRACE(4);
 
     {
         const uint8_t* fa = a.norm.frag + (size_t)ctx.xcc * a.norm.frag_stride;
         const ActLoader<true> xa(fa, fa + xfrag_sum_offset(a.norm.hidden));
         _Float16* fc = (_Float16*)a.frag_c;
         float* fc_sums = (float*)((char*)a.frag_c + xfrag_sum_offset(a.ffn));
-        for (int t0 = 2 * ctx.rank; t0 < gu_per; t0 += 2 * WGS_PER_XCD) {
+        for (int t0 = first; t0 < gu_per; t0 += stride) {
             const int t = t0 + tw;
-            if (t0 != 2 * ctx.rank) job.prefetch(a.w_gate_up, a.gu_kchunks, gu0 + min(t, gu_per - 1), c0, t < gu_per ? nc : 0, lane);
+            const bool more = t0 + stride < gu_per;
+            const JobDesc next = more ? gu_job(t0 + stride) : down_job(first);
             float4v acc[NG];
-            job.run(xa, k, acc, lane);
+            job.run(cur, xa, k, acc, [&] { job.issue_regs(next); });
             float4v v;
-            if (fold_quarters<NG>(acc, red, wave, lane, v) && t < gu_per) {
+            const bool mine = fold_quarters<NG>(acc, red, wave, lane, v);
+            job.issue_lds(next);
+            cur = next;
+            if (t0 == first) norm_factors(a.norm, ctx, s_inv);  // everything this wave asked for has arrived by now
+            if (mine && t < gu_per) {
                 // lanes 0..31: gate rows, lanes 32..63: up rows of the same 32 columns
                 const int g = wave & 3, col = (gu0 + t) * 32 + (lane & 31);
 #pragma unroll
@@ -308,29 +382,30 @@ __global__ __launch_bounds__(512) void k_ffn_block(FfnBlockArgs a) {
                 }
             }
         }
+        if (first >= gu_per) {  // this workgroup had no gate/up tile: its first down job starts here
+            cur = down_job(first);
+            job.issue_regs(cur);
+            job.issue_lds(cur);
+        }
     }
-
     TRACE(5);
-    // down projection over this XCD's K slice; its first weights are requested before the barrier
-    const int dk = a.down_kchunks / XCDS, dk0 = ctx.xcc * dk;
-    quarter_split(dk0, dk, q, c0, nc);
-    {
-        const int t = 2 * ctx.rank + tw;
-        job.prefetch(a.w_down, a.down_kchunks, min(t, a.down_tiles - 1), c0, t < a.down_tiles ? nc : 0, lane);
-    }
     TRACE(6);
     if (!xcd_barrier(ctx, s_i)) return;
     TRACE(7);
     {
         const ActLoader<true> xc(a.frag_c, (const char*)a.frag_c + xfrag_sum_offset(a.ffn));
         float* out = a.partial_out + (size_t)ctx.xcc * 16 * a.norm.hidden;
-        for (int t0 = 2 * ctx.rank; t0 < a.down_tiles; t0 += 2 * WGS_PER_XCD) {
+        for (int t0 = first; t0 < a.down_tiles; t0 += stride) {
             const int t = t0 + tw;
-            if (t0 != 2 * ctx.rank) job.prefetch(a.w_down, a.down_kchunks, min(t, a.down_tiles - 1), c0, t < a.down_tiles ? nc : 0, lane);
+            const bool more = t0 + stride < a.down_tiles;
+            const JobDesc next = more ? down_job(t0 + stride) : JobDesc{nullptr, 0, 0};
             float4v acc[NG];
-            job.run(xc, k, acc, lane);
+            job.run(cur, xc, k, acc, [&] { job.issue_regs(next); });
             float4v v;
-            if (fold_quarters<NG>(acc, red, wave, lane, v) && t < a.down_tiles) {
+            const bool mine = fold_quarters<NG>(acc, red, wave, lane, v);
+            job.issue_lds(next);
+            cur = next;
+            if (mine && t < a.down_tiles) {
                 const int g = wave & 3, n = t * 64 + lane;
                 if (n < a.norm.hidden) {
 #pragma unroll
@@ -349,7 +424,12 @@ int launch_ffn_t(hipStream_t s, FfnBlockArgs& a) {
     // (one per compute unit, at most) are dispatched and all of them become resident together.
     // (A cooperative launch would guarantee that, but goes through a separate queue whose
     // hand-over costs tens of microseconds per launch.)  The bounded barrier waits are the net.
-    const size_t lds = (size_t)8 * NG * 1024;
+    const size_t lds = (size_t)8 * 2 * F::TILE_BYTES;  // >= the fold buffer, 8 * NG KiB
+    static bool configured = false;
+    if (!configured) {
+        TSV_HIP(hipFuncSetAttribute((const void*)k_ffn_block<F, NG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        configured = true;
+    }
     hipLaunchKernelGGL((k_ffn_block<F, NG>), dim3(XCDS * WGS_PER_XCD), dim3(512), lds, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;

@@ -51,6 +51,34 @@ struct Consts {
     uint32_t k6400, k5400, k64;
 };
 
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// 32-bit LDS address of a generic pointer into shared memory
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+// One wave-wide global -> LDS transfer, 16 (or 4) bytes per lane to lds + lane * size, done by the
+// memory pipeline without passing through registers; vmcnt counts it like a load.  Written as
+// inline assembly on purpose: the compiler then neither sees an LDS write (it would otherwise
+// drain the whole load queue before the next LDS access) nor counts the transfer, which only
+// makes its own s_waitcnt values wait for a few more, older, operations.  Readers of the
+// buffer order themselves after a later load with lds_after().
+__device__ __forceinline__ void dma_to_lds_b128(const void* g, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(g) : "memory");
+}
+__device__ __forceinline__ void dma_to_lds_b32(const void* g, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds), "v"(g) : "memory");
+}
+// An LDS address the compiler believes to depend on `loaded`, a register filled by a load that
+// was issued after the transfers into that buffer: loads complete in issue order, so once the
+// compiler has waited for `loaded`, the buffer is complete, and no read through the returned
+// address can be scheduled before that wait.
+__device__ __forceinline__ uint32_t lds_after(uint32_t lds, float loaded) {
+    asm volatile("" : "+v"(lds) : "v"(loaded));
+    return lds;
+}
+
 // ------------------------------------------------------------------------------- formats
 struct Q4K {
     static constexpr int NSUB = 8, NPAIR = 4, TILE_BYTES = 9216;
@@ -63,6 +91,12 @@ struct Q4K {
 #pragma unroll
         for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
         r.s = __builtin_nontemporal_load(p + 512);
+    }
+    // the same tile copied byte for byte into LDS by the memory pipeline (no registers involved);
+    // completion is counted by vmcnt like any other load
+    static __device__ __forceinline__ void load_to_lds(uint32_t lds, const uint8_t* tile, int lane) {
+#pragma unroll
+        for (int u = 0; u < 9; u++) dma_to_lds_b128(tile + u * 1024 + lane * 16, lds + u * 1024);
     }
     // float index of this lane's sub-block sums for row group g of chunk c
     static __device__ __forceinline__ int xs_index(int c, int g, int lane) { return (c * 4 + g) * 32 + (lane & 31); }
@@ -80,17 +114,51 @@ struct Q80 {
         for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
         r.s = __builtin_nontemporal_load((const u32x2*)(tile + 8192) + lane);
     }
+    static __device__ __forceinline__ void load_to_lds(uint32_t lds, const uint8_t* tile, int lane) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) dma_to_lds_b128(tile + u * 1024 + lane * 16, lds + u * 1024);
+        // the 512-byte scale block: 8 bytes per lane, as two 4-byte transfers of 256 bytes
+#pragma unroll
+        for (int h = 0; h < 2; h++) dma_to_lds_b32(tile + 8192 + h * 256 + lane * 4, lds + 8192 + h * 256);
+    }
     // a 128-element chunk is half of a 256-element sum group: its four sub-blocks go to blocks 0..3
     static __device__ __forceinline__ int xs_index(int c, int g, int lane) {
         return ((c >> 1) * 4 + g) * 32 + (c & 1) * 16 + (lane & 15);
     }
 };
 
+// activation registers of one K chunk
+template <class F, int NG>
+struct XRegs {
+    u32x2 xa[F::NPAIR][NG];
+    float xs[NG];
+};
+
 template <class F, int NG>
 struct Stage {
     typename F::Regs w;
-    u32x2 xa[F::NPAIR][NG];
-    float xs[NG];
+    XRegs<F, NG> x;
+};
+
+// Where a tile's bytes are read from while it is being multiplied: the registers of a stage, or
+// the LDS copy made by load_to_lds (16 bytes per lane and unit, read just before use).
+template <class F>
+struct RegSrc {
+    const typename F::Regs& r;
+    __device__ __forceinline__ u32x4 unit(int u) const { return r.q[u]; }
+    __device__ __forceinline__ auto scales() const { return r.s; }
+};
+template <class F>
+struct LdsSrc {
+    uint32_t base;  // LDS address (see lds_after)
+    int lane;
+    typedef decltype(typename F::Regs{}.s) Scales;
+    __device__ __forceinline__ u32x4 unit(int u) const {
+        return *(__attribute__((address_space(3))) const u32x4*)(uintptr_t)(base + (u * 64 + lane) * 16);
+    }
+    __device__ __forceinline__ Scales scales() const {
+        return *(__attribute__((address_space(3))) const Scales*)(uintptr_t)(base + 8192 + lane * sizeof(Scales));
+    }
 };
 
 // Cache policy of the activation loads: plain, or device-coherent (sc1) for activations that
@@ -120,13 +188,13 @@ struct ActLoader {
 
 // activations of K chunk c (chunk index in the activation's own K axis)
 template <class F, int NG, bool COH>
-__device__ __forceinline__ void load_x(Stage<F, NG>& st, const ActLoader<COH>& x, int c, int lane) {
+__device__ __forceinline__ void load_x(XRegs<F, NG>& xr, const ActLoader<COH>& x, int c, int lane) {
 #pragma unroll
     for (int p = 0; p < F::NPAIR; p++)
 #pragma unroll
-        for (int g = 0; g < NG; g++) st.xa[p][g] = x.frag_at(((c * F::NPAIR + p) * 4 + g) * 64 + lane);
+        for (int g = 0; g < NG; g++) xr.xa[p][g] = x.frag_at(((c * F::NPAIR + p) * 4 + g) * 64 + lane);
 #pragma unroll
-    for (int g = 0; g < NG; g++) st.xs[g] = x.sum_at(F::xs_index(c, g, lane));
+    for (int g = 0; g < NG; g++) xr.xs[g] = x.sum_at(F::xs_index(c, g, lane));
 }
 
 // The loads of one stage stay together and in program order (scheduling fences on both sides),
@@ -135,7 +203,7 @@ template <class F, int NG, bool COH>
 __device__ __forceinline__ void load_stage(Stage<F, NG>& st, const ActLoader<COH>& x, const uint8_t* tile_chunk, int c,
                                            int lane) {
     __builtin_amdgcn_sched_barrier(0);
-    load_x(st, x, c, lane);
+    load_x(st.x, x, c, lane);
     F::load(st.w, tile_chunk, lane);
     __builtin_amdgcn_sched_barrier(0);
 }
@@ -152,14 +220,15 @@ __device__ __forceinline__ void fma4(float4v& t, float s, const float4v& d) {
 //   t += sum_j d*sc_j * (X_j . (off_j + q_j))                  64 fp16 MFMAs per group
 // Both parts are summed per tile first so the large code offsets cancel before they reach the
 // running accumulator.
-template <int NG>
-__device__ __forceinline__ void compute(const Stage<Q4K, NG>& st, const Consts& k, float4v (&acc)[NG]) {
-    const Q4K::Regs& r = st.w;
-    const float d = h2f_lo(r.s.x), dmin = h2f_hi(r.s.x);
+template <int NG, class Src>
+__device__ __forceinline__ void compute_tile(Q4K, const Src& w, const XRegs<Q4K, NG>& x, const Consts& k,
+                                             float4v (&acc)[NG]) {
+    const u32x4 hs = w.scales();
+    const float d = h2f_lo(hs.x), dmin = h2f_hi(hs.x);
     // 6-bit scale / min unpack (q4_k.rs:43-54), four sub-blocks per 32-bit word
-    const uint32_t sl = r.s.y & 0x3F3F3F3Fu, ml = r.s.z & 0x3F3F3F3Fu;
-    const uint32_t sh = (r.s.w & 0x0F0F0F0Fu) | ((r.s.y >> 2) & 0x30303030u);
-    const uint32_t mh = ((r.s.w >> 4) & 0x0F0F0F0Fu) | ((r.s.z >> 2) & 0x30303030u);
+    const uint32_t sl = hs.y & 0x3F3F3F3Fu, ml = hs.z & 0x3F3F3F3Fu;
+    const uint32_t sh = (hs.w & 0x0F0F0F0Fu) | ((hs.y >> 2) & 0x30303030u);
+    const uint32_t mh = ((hs.w >> 4) & 0x0F0F0F0Fu) | ((hs.z >> 2) & 0x30303030u);
     float sc[8], cf[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -174,23 +243,24 @@ __device__ __forceinline__ void compute(const Stage<Q4K, NG>& st, const Consts& 
     static_for<8>([&](auto J) {
         constexpr int j = decltype(J)::value;
 #pragma unroll
-        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(st.xs[g], cf[j], t[g]);
+        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(x.xs[g], cf[j], t[g]);
     });
 #pragma unroll
     for (int p = 0; p < 4; p++) {
+        const u32x4 qa = w.unit(2 * p), qb = w.unit(2 * p + 1);
         float4v dlo[NG], dhi[NG];
 #pragma unroll
         for (int g = 0; g < NG; g++) dlo[g] = dhi[g] = float4v{0.f, 0.f, 0.f, 0.f};
         static_for<8>([&](auto W) {
-            constexpr int w = decltype(W)::value;
-            const uint32_t word = r.q[2 * p + w / 4][w % 4];
+            constexpr int wi = decltype(W)::value;
+            const uint32_t word = wi < 4 ? qa[wi % 4] : qb[wi % 4];
             const uint32_t v = word >> 8;
             const u32x2 blo = {and_or(word, 0x000F000Fu, k.k6400), and_or(v, 0x000F000Fu, k.k6400)};
             const u32x2 bhi = {and_or(word, 0x00F000F0u, k.k5400), and_or(v, 0x00F000F0u, k.k5400)};
 #pragma unroll
             for (int g = 0; g < NG; g++) {
-                dlo[g] = mfma_f16<w>(st.xa[p][g], blo, dlo[g]);
-                dhi[g] = mfma_f16<w + 8>(st.xa[p][g], bhi, dhi[g]);
+                dlo[g] = mfma_f16<wi>(x.xa[p][g], blo, dlo[g]);
+                dhi[g] = mfma_f16<wi + 8>(x.xa[p][g], bhi, dhi[g]);
             }
         });
 #pragma unroll
@@ -205,34 +275,36 @@ __device__ __forceinline__ void compute(const Stage<Q4K, NG>& st, const Consts& 
 
 // One Q8_0 tile (64 rows x 128 K = four 32-element blocks).  Codes go in as 1024 + (q + 128);
 // the 1152 offset comes back out through the activation sums on the fp32 matrix pipe.
-template <int NG>
-__device__ __forceinline__ void compute(const Stage<Q80, NG>& st, const Consts& k, float4v (&acc)[NG]) {
-    const Q80::Regs& r = st.w;
-    float dj[4] = {h2f_lo(r.s.x), h2f_hi(r.s.x), h2f_lo(r.s.y), h2f_hi(r.s.y)};
+template <int NG, class Src>
+__device__ __forceinline__ void compute_tile(Q80, const Src& w, const XRegs<Q80, NG>& x, const Consts& k,
+                                             float4v (&acc)[NG]) {
+    const u32x2 hs = w.scales();
+    float dj[4] = {h2f_lo(hs.x), h2f_hi(hs.x), h2f_lo(hs.y), h2f_hi(hs.y)};
     float4v t[NG];
 #pragma unroll
     for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
     static_for<4>([&](auto J) {
         constexpr int j = decltype(J)::value;
 #pragma unroll
-        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(st.xs[g], dj[j] * -1152.0f, t[g]);
+        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(x.xs[g], dj[j] * -1152.0f, t[g]);
     });
 #pragma unroll
     for (int p = 0; p < 2; p++) {
+        const u32x4 qa0 = w.unit(4 * p), qa1 = w.unit(4 * p + 1), qb0 = w.unit(4 * p + 2), qb1 = w.unit(4 * p + 3);
         float4v da[NG], db[NG];
 #pragma unroll
         for (int g = 0; g < NG; g++) da[g] = db[g] = float4v{0.f, 0.f, 0.f, 0.f};
         static_for<8>([&](auto W) {
-            constexpr int w = decltype(W)::value;
+            constexpr int wi = decltype(W)::value;
             // bytes -> fp16 1024 + (q + 128): interleave each byte with 0x64
-            const uint32_t wa = r.q[4 * p + w / 4][w % 4] ^ 0x80808080u;
-            const uint32_t wb = r.q[4 * p + 2 + w / 4][w % 4] ^ 0x80808080u;
+            const uint32_t wa = (wi < 4 ? qa0[wi % 4] : qa1[wi % 4]) ^ 0x80808080u;
+            const uint32_t wb = (wi < 4 ? qb0[wi % 4] : qb1[wi % 4]) ^ 0x80808080u;
             const u32x2 ba = {__builtin_amdgcn_perm(k.k64, wa, 0x04020400u), __builtin_amdgcn_perm(k.k64, wa, 0x04030401u)};
             const u32x2 bb = {__builtin_amdgcn_perm(k.k64, wb, 0x04020400u), __builtin_amdgcn_perm(k.k64, wb, 0x04030401u)};
 #pragma unroll
             for (int g = 0; g < NG; g++) {
-                da[g] = mfma_f16<w>(st.xa[p][g], ba, da[g]);
-                db[g] = mfma_f16<w + 8>(st.xa[p][g], bb, db[g]);
+                da[g] = mfma_f16<wi>(x.xa[p][g], ba, da[g]);
+                db[g] = mfma_f16<wi + 8>(x.xa[p][g], bb, db[g]);
             }
         });
 #pragma unroll
@@ -243,6 +315,12 @@ __device__ __forceinline__ void compute(const Stage<Q80, NG>& st, const Consts& 
     }
 #pragma unroll
     for (int g = 0; g < NG; g++) acc[g] += t[g];
+}
+
+// a register stage
+template <class F, int NG>
+__device__ __forceinline__ void compute(const Stage<F, NG>& st, const Consts& k, float4v (&acc)[NG]) {
+    compute_tile<NG>(F{}, RegSrc<F>{st.w}, st.x, k, acc);
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }

@@ -416,7 +416,7 @@ int launch_pass(tsv_ctx* c, int m) {
             fa.norm.ssq = c->ssq8;
             fa.norm.hidden = c->hidden;
             fa.norm.eps = c->eps;
-            fa.vp = c->vp_dev;
+            fa.m = m;
             fa.w_gate_up = L.gate_up.tiles;
             fa.gu_tiles = L.gate_up.n_tiles;
             fa.gu_kchunks = L.gate_up.kchunks;
@@ -644,8 +644,11 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         // per-XCD fused kernels: every layer must fit their sharding; they need all 256
         // workgroups resident at once (cooperative launch) and a fresh barrier base per launch
         // (so not inside a captured graph)
-        bool ok = !c->use_graph;
-        if (const char* e = getenv("TSV_FUSED")) ok = ok && e[0] != '0';
+        // Opt-in (TSV_FUSED=1): at the 8B shape the fused FFN block measured 36-42 us per layer
+        // against 31 us for the three separate kernels -- the block is bandwidth-bound, and its
+        // early bulk prefetch delays the small loads of the RMSNorm stage.
+        const char* fe = getenv("TSV_FUSED");
+        bool ok = !c->use_graph && fe && fe[0] == '1';
         int coop = 0, ncu = 0;
         if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, 0) != hipSuccess) coop = 0;
         if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) ncu = 0;

@@ -126,7 +126,7 @@ struct NormStage {
 struct FfnBlockArgs {
     FusedSync sync;
     NormStage norm;
-    const VerifyParams* vp;
+    int m;  // rows of the pass
     const uint8_t* w_gate_up;
     int gu_tiles, gu_kchunks;
     uint4* frag_c;  // silu(gate) * up as fragments, K = ffn
