@@ -74,10 +74,68 @@ def trace_summary(path):
     print(f"total kernel time in verify steps: {total / 1e6:.3f} ms over the traced steps")
 
 
+# HBM bytes per launch of the dominant kernel (gate/up matmul of the headline workload), measured
+# with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over `bench.py --traffic-probe` and
+# scaled by the copy kernel of known size (`bench.py --traffic-summary`): 66 938 785 B read +
+# 258 048 B written, against 66 060 288 algorithmic bytes.
+MEASURED_TRAFFIC = {"llama3_8b_q4_k_k4_ctx4096": 67196833}
+
+GATE_UP_8B = dict(dtype=12, rows=28672, cols=4096, m=5, epi=1)   # the dominant kernel of the headline workload
+COPY_BYTES = 256 << 20
+
+
+def traffic_probe():
+    """What `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` is pointed at: the plain copy kernel
+    of known size (COPY_BYTES read, COPY_BYTES written per launch), then the gate/up matmul of the
+    headline workload on weights cycled through HBM."""
+    from turbospark_amd import ffi
+    g = GATE_UP_8B
+    us = ffi.copy_time(COPY_BYTES, iters=10)
+    log(f"[traffic-probe] copy kernel {COPY_BYTES >> 20} MiB: {us:.1f} us, {2 * COPY_BYTES / us / 1e3:.0f} GB/s read+write")
+    us = ffi.matmul_time(g["dtype"], g["rows"], g["cols"], g["m"], g["epi"], 0, 20, 4)
+    nbytes = g["rows"] * ffi.row_bytes(g["dtype"], g["cols"])
+    log(f"[traffic-probe] gate/up matmul: {us:.2f} us, {nbytes / us / 1e3:.0f} GB/s of weight bytes")
+
+
+def traffic_summary(fetch_csv, write_csv):
+    """HBM bytes per launch of the gate/up matmul from two counter-collection CSVs of
+    `bench.py --traffic-probe` (FETCH_SIZE and WRITE_SIZE, KiB-like units per dispatch), each
+    scaled by what the same counter reads for the copy kernel of known size."""
+    import csv
+    from turbospark_amd import ffi
+
+    def per_kernel(path, counter):
+        acc = {}
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] != counter:
+                continue
+            key = "copy" if "k_copy_probe" in r["Kernel_Name"] else "gemm" if "k_gemm" in r["Kernel_Name"] else None
+            if key:
+                acc.setdefault(key, []).append(float(r["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}, {k: len(v) for k, v in acc.items()}
+
+    g = GATE_UP_8B
+    alg = g["rows"] * ffi.row_bytes(g["dtype"], g["cols"])
+    out = {"algorithmic_bytes_per_launch": alg}
+    for name, path, counter in (("read", fetch_csv, "FETCH_SIZE"), ("write", write_csv, "WRITE_SIZE")):
+        avg, n = per_kernel(path, counter)
+        factor = COPY_BYTES / avg["copy"]          # bytes per counter unit, from the copy kernel
+        out[name] = dict(counter=counter, copy_kernel_reading=round(avg["copy"], 1), bytes_per_unit=round(factor, 2),
+                         gemm_reading=round(avg["gemm"], 1), gemm_bytes=int(avg["gemm"] * factor),
+                         dispatches=n)
+    out["traffic_bytes_per_launch"] = out["read"]["gemm_bytes"] + out["write"]["gemm_bytes"]
+    out["traffic_over_algorithmic"] = round(out["traffic_bytes_per_launch"] / alg, 3)
+    print(json.dumps(out, indent=1))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--trace-summary", default=None, metavar="CSV",
                     help="summarise a rocprofv3 kernel-trace CSV of this script (verify steps only) and exit")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="run the copy kernel of known size and the dominant matmul (for rocprofv3 --pmc) and exit")
+    ap.add_argument("--traffic-summary", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="HBM bytes per launch of the dominant matmul from two --pmc runs of --traffic-probe")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -88,6 +146,12 @@ def main():
     args = ap.parse_args()
     if args.trace_summary:
         trace_summary(args.trace_summary)
+        return
+    if args.traffic_probe:
+        traffic_probe()
+        return
+    if args.traffic_summary:
+        traffic_summary(*args.traffic_summary)
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "
@@ -157,30 +221,50 @@ def main():
     min_margin = min(r.min_margin for r in results)
     ms_per_step = wall * 1000.0 / args.steps
 
-    # per-kernel-class durations, HIP events around every launch on the engine's stream
+    # Per-kernel durations inside the pipeline, with HIP events on the engine's stream around
+    # whole timed regions only: a region in which every launch of one kernel class is issued
+    # twice (same inputs, same outputs) takes longer than the plain region by exactly that
+    # class's launches.  (An event pair around each single launch adds ~2 us to a 5-20 us
+    # kernel; those readings are kept as profile_ms_per_step for the coarse breakdown.)
+    def timed_region(n):
+        hip.check(hip.rt().hipStreamSynchronize(stream), "sync")
+        a, b = hip.Event(), hip.Event()
+        a.record(stream)
+        for i in range(n):
+            step(args.warmup + (i % args.steps))
+        b.record(stream)
+        b.sync()
+        return b.ms_since(a) / n
+
+    nrep = min(10, args.steps)
+    plain_ms = timed_region(nrep)
+    ab = algorithmic_bytes(cfg, ctx, m)
+    L = cfg["n_layers"]
+    kern = {}
+    for name, nbytes, count in (("qkv", ab["per_layer"]["qkv"], L), ("wo", ab["per_layer"]["wo"], L),
+                                ("gate_up", ab["per_layer"]["gate_up"], L), ("down", ab["per_layer"]["down"], L),
+                                ("head", ab["head"], 1), ("attention", ab["kv"] // L, L), ("rope_kv", 0, L)):
+        eng.set_repeat(name, 2)
+        twice_ms = timed_region(nrep)
+        eng.set_repeat(name, 1)
+        avg_ms = (twice_ms - plain_ms) / count
+        kern[name] = dict(avg_us=round(avg_ms * 1000, 2), bytes=int(nbytes), launches_per_step=count,
+                          GBps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1) if nbytes and avg_ms > 0 else None)
+    gemm_ms = sum(kern[n]["avg_us"] * kern[n]["launches_per_step"] for n in ("qkv", "wo", "gate_up", "down", "head")) / 1000.0
+
+    # coarse breakdown: an event pair around every launch
     eng.set_profile(True)
     nprof = min(5, args.steps)
     for i in range(nprof):
         step(args.warmup + i)
     prof = eng.get_profile()
     eng.set_profile(False)
-    ab = algorithmic_bytes(cfg, ctx, m)
-    L = cfg["n_layers"]
-    kern = {}
-    for name, nbytes, count in (("qkv", ab["per_layer"]["qkv"], L), ("wo", ab["per_layer"]["wo"], L),
-                                ("gate_up", ab["per_layer"]["gate_up"], L), ("down", ab["per_layer"]["down"], L),
-                                ("head", ab["head"], 1), ("attention", ab["kv"] // L, L)):
-        ms, launches = prof[name]
-        if launches:
-            avg_ms = ms / launches
-            kern[name] = dict(avg_us=round(avg_ms * 1000, 2), GBps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
-                              bytes=int(nbytes), launches_per_step=launches // nprof)
-    gemm_ms = sum(prof[n][0] for n in ("qkv", "wo", "gate_up", "down", "head")) / nprof
     dom = kern.get("gate_up", {})
     peak = 8000.0
     roofline = dict(bound="hbm", kernel="k_gemm<Q4_K> gate/up (silu-mul epilogue)" if cfg["dtype"] == 12 else "k_gemm<Q8_0> gate/up",
                     achieved=dom.get("GBps"), peak=peak, unit="GB/s",
-                    frac=round(dom.get("GBps", 0.0) / peak, 4), traffic=None,
+                    frac=round((dom.get("GBps") or 0.0) / peak, 4),
+                    traffic=MEASURED_TRAFFIC.get(args.workload),
                     algorithmic_bytes_per_launch=dom.get("bytes"), avg_launch_us=dom.get("avg_us"),
                     all_matmuls_GBps=round(ab["weights"] / (gemm_ms * 1e-3) / 1e9, 1) if gemm_ms else None,
                     step_algorithmic_bytes=int(ab["total"]),
@@ -198,7 +282,9 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "q4_k weights x f16 activations, f32 accumulate; f64 acceptance" if cfg["dtype"] == 12 else "q8_0 x f16, f32 accumulate",
+        "dtype": "f16",
+        "dtype_detail": ("q4_k" if cfg["dtype"] == 12 else "q8_0") + " weight codes as exact f16 x f16 activations on MFMA, "
+                        "f32 accumulate; f64 acceptance",
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,
                    "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin},

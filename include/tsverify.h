@@ -192,11 +192,20 @@ int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int
 
 /* Per-kernel-class timing with HIP events on the handle's stream (one event pair per launch
  * while enabled).  Classes, in order: embed, norm, qkv matmul, rope+kv store, attention,
- * output projection, gate/up matmul, down matmul, output head, acceptance.  tsv_get_profile
- * sums the elapsed milliseconds and launch counts since the last call and clears them. */
-#define TSV_PROFILE_CLASSES 10
+ * output projection, gate/up matmul, down matmul, output head, acceptance, and "event pair":
+ * one pair per pass with nothing between the two events, i.e. what an event pair itself adds
+ * to every other reading.  tsv_get_profile sums the elapsed milliseconds and launch counts
+ * since the last call and clears them. */
+#define TSV_PROFILE_CLASSES 11
 int32_t tsv_set_profile(tsv_ctx* ctx, int32_t on);
 int32_t tsv_get_profile(tsv_ctx* ctx, float* ms, int32_t* counts, int32_t n_classes);
+
+/* Measurement hook (no reference counterpart): launch the kernels of one class `times` times
+ * in a row in every following pass (1 restores normal operation).  The extra launches redo the
+ * same work on the same buffers, so results do not change; timing a pass with and without the
+ * repeat gives the class's in-pipeline duration without an event pair around every launch.
+ * Classes that accumulate (norm, embed, acceptance) are refused. */
+int32_t tsv_set_repeat(tsv_ctx* ctx, int32_t profile_class, int32_t times);
 
 /* Measurement hook (no reference counterpart): average microseconds of `iters` back-to-back
  * launches of the verify matmul kernel on a rows x cols weight of `dtype` with m activation
@@ -204,6 +213,11 @@ int32_t tsv_get_profile(tsv_ctx* ctx, float* ms, int32_t* counts, int32_t n_clas
  * `rotate` weight copies are cycled so the bytes come from HBM. */
 int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
                         int32_t iters, int32_t rotate, float* avg_us);
+
+/* Measurement hook: average duration of `iters` launches of a plain device-to-device copy kernel
+ * over `bytes` bytes (read once, written once).  It is the copy kernel of known size that HBM
+ * traffic counters are scaled against, and the streaming rate the part actually reaches. */
+int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us);
 
 /* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
  * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache

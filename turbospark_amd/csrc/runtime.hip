@@ -75,6 +75,7 @@ struct tsv_ctx {
     hipGraphExec_t pass_graph[TSV_MAX_ROWS + 1] = {};
     // per-kernel-class timing (tsv_set_profile): one event pair per launch
     bool profile = false;
+    int repeat[TSV_PROFILE_CLASSES] = {1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1};  // tsv_set_repeat
     std::vector<hipEvent_t> ev;
     std::vector<int> ev_class;
     size_t ev_used = 0;
@@ -236,7 +237,8 @@ int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
     return TSV_OK;
 }
 
-enum { PC_EMBED = 0, PC_NORM, PC_QKV, PC_ROPE, PC_ATTN, PC_WO, PC_GATEUP, PC_DOWN, PC_HEAD, PC_ACCEPT, PC_COUNT };
+enum { PC_EMBED = 0, PC_NORM, PC_QKV, PC_ROPE, PC_ATTN, PC_WO, PC_GATEUP, PC_DOWN, PC_HEAD, PC_ACCEPT, PC_EVENTPAIR, PC_COUNT };
+static_assert(PC_COUNT == TSV_PROFILE_CLASSES, "profile classes");
 
 struct ProfScope {
     tsv_ctx* c;
@@ -331,6 +333,7 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
 int launch_pass(tsv_ctx* c, int m) {
     hipStream_t s = c->stream;
     int rc;
+    { PROF(PC_EVENTPAIR); }  // calibration: an event pair around nothing
     {
         PROF(PC_EMBED);
         rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m);
@@ -350,7 +353,8 @@ int launch_pass(tsv_ctx* c, int m) {
         int sp = splits_for(L.qkv, m, EPI_PARTIAL);
         {
             PROF(PC_QKV);
-            rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++) rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n);
         }
         if (rc) return rc;
         RopeKvArgs ra;
@@ -371,7 +375,8 @@ int launch_pass(tsv_ctx* c, int m) {
         ra.vp = c->vp_dev;
         {
             PROF(PC_ROPE);
-            rc = launch_rope_kv(s, ra, m);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_ROPE] && !rc; rep++) rc = launch_rope_kv(s, ra, m);
         }
         if (rc) return rc;
         AttnArgs aa;
@@ -390,13 +395,15 @@ int launch_pass(tsv_ctx* c, int m) {
         aa.vp = c->vp_dev;
         {
             PROF(PC_ATTN);
-            rc = launch_attention(s, aa, m);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_ATTN] && !rc; rep++) rc = launch_attention(s, aa, m);
         }
         if (rc) return rc;
         sp = splits_for(L.wo, m, EPI_PARTIAL);
         {
             PROF(PC_WO);
-            rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_WO] && !rc; rep++) rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
         }
         if (rc) return rc;
         if (c->fused_ffn) {
@@ -443,13 +450,17 @@ int launch_pass(tsv_ctx* c, int m) {
         if (rc) return rc;
         {
             PROF(PC_GATEUP);
-            rc = launch_gemm(s, L.gate_up, c->xf_a, c->xf_c, c->vp_dev, m, 1, EPI_SILU, 0, 0);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_GATEUP] && !rc; rep++)
+                rc = launch_gemm(s, L.gate_up, c->xf_a, c->xf_c, c->vp_dev, m, 1, EPI_SILU, 0, 0);
         }
         if (rc) return rc;
         sp = splits_for(L.down, m, EPI_PARTIAL);
         {
             PROF(PC_DOWN);
-            rc = launch_gemm(s, L.down, c->xf_c, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_DOWN] && !rc; rep++)
+                rc = launch_gemm(s, L.down, c->xf_c, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
         }
         if (rc) return rc;
         prev_partial = c->partial;
@@ -462,7 +473,9 @@ int launch_pass(tsv_ctx* c, int m) {
     if (rc) return rc;
     {
         PROF(PC_HEAD);
-        rc = launch_gemm(s, c->head, c->xf_a, c->logits, c->vp_dev, m, 1, EPI_LOGITS, c->vocab, c->vocab);
+        rc = 0;
+        for (int rep = 0; rep < c->repeat[PC_HEAD] && !rc; rep++)
+            rc = launch_gemm(s, c->head, c->xf_a, c->logits, c->vp_dev, m, 1, EPI_LOGITS, c->vocab, c->vocab);
     }
     return rc;
 }
@@ -705,6 +718,21 @@ extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
     TSV_HIP(hipStreamSynchronize(c->stream));
     c->profile = on != 0;
     c->ev_used = 0;
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_set_repeat(tsv_ctx* c, int32_t cls, int32_t times) {
+    if (cls != PC_QKV && cls != PC_ROPE && cls != PC_ATTN && cls != PC_WO && cls != PC_GATEUP && cls != PC_DOWN &&
+        cls != PC_HEAD) {
+        set_error("set_repeat: only the matmul, rope and attention classes can be repeated");
+        return TSV_ERR_INVALID;
+    }
+    if (times < 1 || times > 8) {
+        set_error("set_repeat: times must be 1..8");
+        return TSV_ERR_INVALID;
+    }
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    c->repeat[cls] = times;
     return TSV_OK;
 }
 
@@ -1116,6 +1144,52 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     (void)hipStreamSynchronize(c->stream);
     for (void* p : c->allocs) (void)hipFree(p);
     (void)hipStreamDestroy(c->stream);
+    return rc;
+}
+
+namespace {
+__global__ __launch_bounds__(256) void k_copy_probe(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+}  // namespace
+
+extern "C" int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us) {
+    if (bytes < 16 || bytes % 16 || iters < 1 || !avg_us) {
+        set_error("copy_time: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    hipStream_t s;
+    TSV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    uint4 *a = nullptr, *b = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = TSV_OK;
+    if (hipMalloc((void**)&a, (size_t)bytes) != hipSuccess || hipMalloc((void**)&b, (size_t)bytes) != hipSuccess ||
+        hipMemsetAsync(a, 1, (size_t)bytes, s) != hipSuccess || hipEventCreate(&e0) != hipSuccess ||
+        hipEventCreate(&e1) != hipSuccess) {
+        set_error("copy_time: allocation failed");
+        rc = TSV_ERR_DEVICE;
+    }
+    for (int pass = 0; pass < 2 && !rc; pass++) {
+        if (pass) (void)hipEventRecord(e0, s);
+        for (int i = 0; i < (pass ? iters : 2); i++)
+            hipLaunchKernelGGL(k_copy_probe, dim3(256 * 16), dim3(256), 0, s, a, b, (size_t)bytes / 16);
+        if (pass) (void)hipEventRecord(e1, s);
+    }
+    if (!rc) {
+        if (hipStreamSynchronize(s) != hipSuccess) {
+            set_error("copy_time: device execution failed");
+            rc = TSV_ERR_DEVICE;
+        } else {
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            *avg_us = ms * 1000.f / (float)iters;
+        }
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (a) (void)hipFree(a);
+    if (b) (void)hipFree(b);
+    (void)hipStreamDestroy(s);
     return rc;
 }
 

@@ -101,7 +101,7 @@ EXPORTS = [
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
-    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time",
+    "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
 ]
 
 _lib = None
@@ -149,6 +149,7 @@ def lib():
                                     C.c_int64, C.c_void_p, C.c_float, C.c_void_p]
         L.tsv_set_profile.argtypes = [C.c_void_p, C.c_int32]
         L.tsv_get_profile.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]
+        L.tsv_copy_time.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
         L.tsv_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                       C.c_int32, C.POINTER(C.c_float)]
         L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
@@ -226,6 +227,13 @@ def attention(q, k, v, base, parent=None, scale=0.0):
     check(lib().tsv_attention(q16.ctypes.data, k16.ctypes.data, v16.ctypes.data, m, nq, nkv, hd, base,
                               pa.ctypes.data if pa is not None else None, scale, out.ctypes.data))
     return out.astype(np.float32)
+
+
+def copy_time(nbytes, iters=20):
+    """Average microseconds per launch of a plain device copy kernel over nbytes (HIP events)."""
+    t = C.c_float()
+    check(lib().tsv_copy_time(nbytes, iters, C.byref(t)))
+    return t.value
 
 
 def matmul_time(dtype, rows, cols, m, epi=0, splits=0, iters=50, rotate=4):

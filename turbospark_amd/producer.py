@@ -206,10 +206,15 @@ class HipVerifier:
         ffi.check(ffi.lib().tsv_draft_chain(self._h, ptr, k, C.byref(cfg), C.byref(ds), props.ctypes.data))
         return props, ds.value
 
-    PROFILE_CLASSES = ("embed", "norm", "qkv", "rope_kv", "attention", "wo", "gate_up", "down", "head", "accept")
+    PROFILE_CLASSES = ("embed", "norm", "qkv", "rope_kv", "attention", "wo", "gate_up", "down", "head", "accept",
+                       "event_pair")
 
     def set_profile(self, on):
         ffi.check(ffi.lib().tsv_set_profile(self._h, int(bool(on))))
+
+    def set_repeat(self, profile_class, times):
+        """Launch the kernels of one class `times` times in a row per pass (measurement hook)."""
+        ffi.check(ffi.lib().tsv_set_repeat(self._h, self.PROFILE_CLASSES.index(profile_class), int(times)))
 
     def get_profile(self):
         """{class: (total ms, launches)} since the last call (HIP events around every launch)."""
