@@ -38,6 +38,7 @@ enum {
     TSV_Q8_0 = 8,  /* 34 B / 32 elems  (crates/compute/src/quant_gguf/q8_0.rs) */
     TSV_Q4_K = 12, /* 144 B / 256 elems (crates/compute/src/quant_gguf/q4_k.rs) */
     TSV_BF16 = 30,
+    TSV_MXFP4 = 39, /* 17 B / 32 elems: e8m0 scale + 32 e2m1 nibbles (crates/compute/src/quant_gguf_mxfp4.rs) */
 };
 
 /* A host tensor in GGUF layout: one byte run per output row, rows x cols elements. */

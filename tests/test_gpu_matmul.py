@@ -22,7 +22,8 @@ def _case(dtype, rows, cols, seed):
     return entry, x, x16, want
 
 
-@pytest.mark.parametrize("dtype,rows,cols", [(12, 64, 512), (12, 48, 2048), (8, 64, 512), (8, 32, 1408)])
+@pytest.mark.parametrize("dtype,rows,cols", [(12, 64, 512), (12, 48, 2048), (8, 64, 512), (8, 32, 1408),
+                                             (39, 64, 512), (39, 48, 2048), (39, 200, 768)])
 def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, rows, cols, 31)
@@ -42,7 +43,7 @@ def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
         assert np.array_equal(got[0], first), m
 
 
-@pytest.mark.parametrize("dtype", [12, 8])
+@pytest.mark.parametrize("dtype", [12, 8, 39])
 def test_split_k_changes_nothing_but_rounding_and_is_deterministic(dtype):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, 32, 2048, 77)
@@ -72,6 +73,30 @@ def test_q4k_hand_packed_superblock_through_the_kernel(golden):
     want = np.array([g["d"] * g["LS"][e // 32] * quants[e] - g["dmin"] * g["LM"][e // 32] for e in range(256)],
                     np.float32)
     for e0 in range(0, 256, 16):
+        x = np.zeros((16, 256), np.float32)
+        for b in range(16):
+            x[b, e0 + b] = 1.0
+        got = ffi.matmul(entry, x)
+        for b in range(16):
+            assert np.all(got[b] == want[e0 + b]), (e0 + b, got[b, 0], want[e0 + b])
+
+
+def test_mxfp4_ggml_golden_blocks_through_the_kernel(golden):
+    """The ggml-produced MXFP4 bytes -> floats fixture of the reference
+    (crates/compute/tests/generated/quant_gguf_mxfp4_oracle.rs) as a weight matrix: one-hot
+    activations read the decoded weights back out of the kernel, which must equal ggml's floats
+    exactly (every value is a codebook entry times a power of two)."""
+    import json, os
+    from turbospark_amd import ffi
+    g = json.load(open(os.path.join(golden, "mxfp4_ggml_oracle.json")))
+    blocks = np.array(g["bytes"], np.uint8).reshape(4, 17)
+    pad = np.zeros((4, 17), np.uint8)
+    pad[:, 0] = 127                                   # scale 2^-1, all codes zero
+    row = np.concatenate([blocks, pad]).reshape(1, -1)  # 8 blocks = one 256-element chunk
+    raw = np.tile(row, (16, 1))
+    entry = (ffi.MXFP4, np.ascontiguousarray(raw), 16, 256)
+    want = np.concatenate([np.array(g["floats"], np.float32), np.zeros(128, np.float32)])
+    for e0 in range(0, 128, 16):
         x = np.zeros((16, 256), np.float32)
         for b in range(16):
             x[b, e0 + b] = 1.0

@@ -80,12 +80,47 @@ __global__ void k_repack_q80(const uint8_t* __restrict__ raw, int n_rows, int kc
     }
 }
 
+// MXFP4: one thread per source block (17 bytes: scale, then 16 bytes whose low / high nibbles are
+// elements j and j + 16).  Nibble n of output word w is K element 8w + {0,2,1,3,4,6,5,7}[n].
+__global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)n_rows * kchunks * 8;
+    if (gid >= total) return;
+    const int u = (int)(gid % 8);
+    const long t = gid / 8;
+    const int c = (int)(t % kchunks);
+    const int r = (int)(t / kchunks);
+    const int drow = (r / grp) * stride + offset + r % grp;
+    const int tile = drow >> 6, lane = drow & 63;
+    const uint8_t* blk = raw + ((long)r * kchunks * 8 + (long)c * 8 + u) * 17;
+    uint8_t* tb = tiles + ((long)tile * kchunks + c) * 8704;
+    uint32_t words[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int n = 0; n < 8; n++) {
+            const int k = 8 * w + ((n & 4) | ((n & 1) << 1) | ((n >> 1) & 1));
+            const uint32_t code = k < 16 ? (blk[1 + k] & 0xFu) : (uint32_t)(blk[1 + k - 16] >> 4);
+            v |= code << (4 * n);
+        }
+        words[w] = v;
+    }
+    *(uint4*)(tb + (u * 64 + lane) * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+    tb[8192 + lane * 8 + u] = blk[0];
+}
+
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
                   int kchunks, int grp, int stride, int offset) {
     (void)k;
     const long total = (long)n_rows * kchunks * 9;
     if (total == 0) return TSV_OK;
-    if (fmt == FMT_Q4K)
+    if (fmt == FMT_MX4) {
+        const long blocks = (long)n_rows * kchunks * 8;
+        hipLaunchKernelGGL(k_repack_mx4, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
+                           tiles, grp, stride, offset);
+    } else if (fmt == FMT_Q4K)
         hipLaunchKernelGGL(k_repack_q4k, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, raw, n_rows,
                            kchunks, tiles, grp, stride, offset);
     else
@@ -283,7 +318,9 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
         }
         a.n_valid = w.n_rows / 2;  // K of the next matmul
     }
-    return w.fmt == FMT_Q4K ? launch_f<Q4K>(s, a, m, epi) : launch_f<Q80>(s, a, m, epi);
+    return w.fmt == FMT_Q4K   ? launch_f<Q4K>(s, a, m, epi)
+           : w.fmt == FMT_Q80 ? launch_f<Q80>(s, a, m, epi)
+                              : launch_f<MX4>(s, a, m, epi);
 }
 
 }  // namespace tsv

@@ -82,6 +82,7 @@ __device__ __forceinline__ uint32_t lds_after(uint32_t lds, float loaded) {
 // ------------------------------------------------------------------------------- formats
 struct Q4K {
     static constexpr int NSUB = 8, NPAIR = 4, TILE_BYTES = 9216;
+    static constexpr bool SUMS = true;  // the matmul needs the activations' sub-block sums
     struct Regs {
         u32x4 q[8];
         u32x4 s;
@@ -104,6 +105,7 @@ struct Q4K {
 
 struct Q80 {
     static constexpr int NSUB = 4, NPAIR = 2, TILE_BYTES = 8704;
+    static constexpr bool SUMS = true;
     struct Regs {
         u32x4 q[8];
         u32x2 s;
@@ -128,6 +130,24 @@ struct Q80 {
 };
 
 // activation registers of one K chunk
+// MXFP4 (ggml block_mxfp4: one e8m0 scale byte + 16 bytes of e2m1 nibbles per 32 elements;
+// crates/compute/src/quant_gguf_mxfp4.rs:76-141).  A tile is 64 rows x 256 K: unit u holds the
+// 32 nibbles of the lane's sub-block u, re-ordered at load time so that the four bytes of word w
+// are K elements (8w, 8w+2), (8w+1, 8w+3), (8w+4, 8w+6), (8w+5, 8w+7) -- what
+// v_cvt_scalef32_pk_f16_fp4 turns, byte by byte, into the fp16 pairs of two MFMA K steps in the
+// activations' element order; then the eight scale bytes per lane.  e2m1 values are exact in
+// fp16 and signed, so there is no code offset and no use for the activation sums.
+struct MX4 {
+    static constexpr int NSUB = 8, NPAIR = 4, TILE_BYTES = 8704;
+    static constexpr bool SUMS = false;
+    typedef Q80::Regs Regs;
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) { Q80::load(r, tile, lane); }
+    static __device__ __forceinline__ void load_to_lds(uint32_t lds, const uint8_t* tile, int lane) {
+        Q80::load_to_lds(lds, tile, lane);
+    }
+    static __device__ __forceinline__ int xs_index(int c, int g, int lane) { return Q4K::xs_index(c, g, lane); }
+};
+
 template <class F, int NG>
 struct XRegs {
     u32x2 xa[F::NPAIR][NG];
@@ -193,8 +213,10 @@ __device__ __forceinline__ void load_x(XRegs<F, NG>& xr, const ActLoader<COH>& x
     for (int p = 0; p < F::NPAIR; p++)
 #pragma unroll
         for (int g = 0; g < NG; g++) xr.xa[p][g] = x.frag_at(((c * F::NPAIR + p) * 4 + g) * 64 + lane);
+    if (F::SUMS) {
 #pragma unroll
-    for (int g = 0; g < NG; g++) xr.xs[g] = x.sum_at(F::xs_index(c, g, lane));
+        for (int g = 0; g < NG; g++) xr.xs[g] = x.sum_at(F::xs_index(c, g, lane));
+    }
 }
 
 // The loads of one stage stay together and in program order (scheduling fences on both sides),
@@ -315,6 +337,51 @@ __device__ __forceinline__ void compute_tile(Q80, const Src& w, const XRegs<Q80,
     }
 #pragma unroll
     for (int g = 0; g < NG; g++) acc[g] += t[g];
+}
+
+// One MXFP4 tile (64 rows x 256 K = eight 32-element blocks): value = e2m1(code) * 2^(e - 127).
+template <int NG, class Src>
+__device__ __forceinline__ void compute_tile(MX4, const Src& w, const XRegs<MX4, NG>& x, const Consts&,
+                                             float4v (&acc)[NG]) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const u32x2 hs = w.scales();
+    float sc[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t e = ((j < 4 ? hs.x : hs.y) >> (8 * (j & 3))) & 0xFFu;
+        sc[j] = __uint_as_float(e ? e << 23 : 0x00400000u);  // 2^(e-127); e = 0 is the subnormal 2^-127
+    }
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const u32x4 qa = w.unit(2 * p), qb = w.unit(2 * p + 1);
+        float4v da[NG], db[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) da[g] = db[g] = float4v{0.f, 0.f, 0.f, 0.f};
+        static_for<4>([&](auto W) {
+            constexpr int wi = decltype(W)::value;
+            const uint32_t wa = qa[wi], wb = qb[wi];
+            auto pair2 = [](uint32_t word, int lo) {
+                const half2v h0 = lo ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 2)
+                                     : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 0);
+                const half2v h1 = lo ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 3)
+                                     : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 1);
+                return u32x2{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1)};
+            };
+            const u32x2 a0 = pair2(wa, 0), a1 = pair2(wa, 1), b0 = pair2(wb, 0), b1 = pair2(wb, 1);
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                da[g] = mfma_f16<2 * wi>(x.xa[p][g], a0, da[g]);
+                da[g] = mfma_f16<2 * wi + 1>(x.xa[p][g], a1, da[g]);
+                db[g] = mfma_f16<8 + 2 * wi>(x.xa[p][g], b0, db[g]);
+                db[g] = mfma_f16<8 + 2 * wi + 1>(x.xa[p][g], b1, db[g]);
+            }
+        });
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            fma4(acc[g], sc[2 * p], da[g]);
+            fma4(acc[g], sc[2 * p + 1], db[g]);
+        }
+    }
 }
 
 // a register stage

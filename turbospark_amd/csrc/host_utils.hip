@@ -23,6 +23,7 @@ int64_t row_bytes(int dtype, int64_t cols) {
         case TSV_BF16: return cols * 2;
         case TSV_Q8_0: return cols % 32 ? -1 : cols / 32 * 34;
         case TSV_Q4_K: return cols % 256 ? -1 : cols / 256 * 144;
+        case TSV_MXFP4: return cols % 32 ? -1 : cols / 32 * 17;
     }
     return -1;
 }
@@ -130,6 +131,47 @@ void encode_q4_k(const float* row, int64_t n, uint8_t* out) {
     }
 }
 
+// MXFP4 install encoder.  The reference only decodes MXFP4 (quant_gguf_mxfp4.rs:114-141: value =
+// kvalues[code] * 2^(e-128) with kvalues = 0,1,2,3,4,6,8,12 and their negatives); this encoder
+// picks the smallest scale that keeps the block's largest magnitude within 12 * scale and then
+// the nearest code for every element (first of equals; the second zero, code 8, is never used).
+void encode_mxfp4(const float* row, int64_t n, uint8_t* out) {
+    static const float kvalues[16] = {0.0f, 1.0f, 2.0f, 3.0f, 4.0f, 6.0f, 8.0f, 12.0f,
+                                      0.0f, -1.0f, -2.0f, -3.0f, -4.0f, -6.0f, -8.0f, -12.0f};
+    for (int64_t b = 0; b < n / 32; b++) {
+        const float* block = row + b * 32;
+        float amax = 0.0f;
+        for (int k = 0; k < 32; k++) amax = std::fmax(amax, std::fabs(block[k]));
+        int e = 2;
+        if (amax > 0.0f) {
+            int ex;
+            (void)std::frexp(amax / 12.0f, &ex);
+            e = std::min(std::max(ex + 128, 2), 254);
+        }
+        const uint32_t bits = (uint32_t)(e - 1) << 23;  // 2^(e-128)
+        float d;
+        std::memcpy(&d, &bits, 4);
+        uint8_t* o = out + b * 17;
+        o[0] = (uint8_t)e;
+        uint8_t codes[32];
+        for (int k = 0; k < 32; k++) {
+            const float v = block[k] / d;
+            int best = 0;
+            float best_err = std::fabs(v - kvalues[0]);
+            for (int c = 1; c < 16; c++) {
+                if (c == 8) continue;
+                const float err = std::fabs(v - kvalues[c]);
+                if (err < best_err) {
+                    best_err = err;
+                    best = c;
+                }
+            }
+            codes[k] = (uint8_t)best;
+        }
+        for (int j = 0; j < 16; j++) o[1 + j] = (uint8_t)(codes[j] | (codes[j + 16] << 4));
+    }
+}
+
 int encode_row(int dtype, const float* src, int64_t cols, uint8_t* dst) {
     switch (dtype) {
         case TSV_F32: std::memcpy(dst, src, (size_t)cols * 4); return 0;
@@ -141,6 +183,7 @@ int encode_row(int dtype, const float* src, int64_t cols, uint8_t* dst) {
             return 0;
         case TSV_Q8_0: encode_q8_0(src, cols, dst); return 0;
         case TSV_Q4_K: encode_q4_k(src, cols, dst); return 0;
+        case TSV_MXFP4: encode_mxfp4(src, cols, dst); return 0;
     }
     return -1;
 }

@@ -22,7 +22,9 @@ struct LayerW {
     uint16_t *kc = nullptr, *vc = nullptr;
 };
 
-int dtype_fmt(int dtype) { return dtype == TSV_Q4_K ? FMT_Q4K : dtype == TSV_Q8_0 ? FMT_Q80 : -1; }
+int dtype_fmt(int dtype) {
+    return dtype == TSV_Q4_K ? FMT_Q4K : dtype == TSV_Q8_0 ? FMT_Q80 : dtype == TSV_MXFP4 ? FMT_MX4 : -1;
+}
 
 }  // namespace
 
@@ -149,11 +151,11 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
         return TSV_ERR_INVALID;
     }
     if (fmt < 0) {
-        set_error(std::string(what) + ": matmul weights must be Q4_K or Q8_0 in this build");
+        set_error(std::string(what) + ": matmul weights must be Q4_K, Q8_0 or MXFP4 in this build");
         return TSV_ERR_UNSUPPORTED;
     }
     if (cols % fmt_chunk_elems(fmt) || rows < 1) {
-        set_error(std::string(what) + ": K must be whole 256 (Q4_K) / 128 (Q8_0) chunks");
+        set_error(std::string(what) + ": K must be whole 256 (Q4_K, MXFP4) / 128 (Q8_0) chunks");
         return TSV_ERR_UNSUPPORTED;
     }
     return TSV_OK;
@@ -1235,8 +1237,10 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
                     sc[r * 16 + 1] = 0x20;
                     sc[r * 16 + 3] = 0x20;
                 }
-            else
+            else if (fmt == FMT_Q80)
                 for (int i = 0; i < 256; i++) sc[2 * i + 1] = 0x20;
+            else
+                for (int i = 0; i < 512; i++) sc[i] = 0x70 + (sc[i] & 7);  // e8m0 scales around 2^-12
         }
         for (int i = 0; i < rotate && !rc; i++) {
             rc = dev_alloc(c, &copies[i], w.bytes);

@@ -32,6 +32,9 @@ const std::string& get_error();
 //                      of each of the 64 superblocks, byte for byte, only re-ordered.
 //   Q8_0 tile, 8704 B: [unit 0..7][lane][16 B] int8 quants (unit u = bytes 16*(u%2).. of block
 //                      u/2 of the chunk), then [lane][4 x f16 d].
+//   MXFP4 tile, 8704 B (64 rows x 256 K): [unit 0..7][lane][16 B] the 32 e2m1 nibbles of the
+//                      lane's block u, nibbles re-ordered for the fp4 -> fp16 converter (see
+//                      gemm_core.h), then [lane][8 e8m0 scale bytes].
 // Rows past the matrix's last row are all-zero blocks (scale 0).
 //
 // Activation layout ("fragments").  The <=16 fp16 activation rows of a K-wide matmul input
@@ -42,7 +45,7 @@ const std::string& get_error();
 // every 32-element sub-block, [K/256][g][sub%8][i], which the matmul uses to take the
 // integer-code offsets and the Q4_K min term back out.
 // ---------------------------------------------------------------------------------------
-enum { FMT_Q4K = 0, FMT_Q80 = 1 };
+enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2 };
 
 struct TiledW {
     uint8_t* tiles = nullptr;  // device
@@ -54,9 +57,9 @@ struct TiledW {
     size_t bytes = 0;
 };
 
-inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q4K ? 256 : 128; }
+inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q80 ? 128 : 256; }
 inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : 8704; }
-inline int fmt_nsub(int fmt) { return fmt == FMT_Q4K ? 8 : 4; }
+inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : 8; }
 constexpr int TILE_ROWS = 64;
 
 // index (in halfs) of activation element (row, k) in the fragment layout
