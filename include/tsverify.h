@@ -53,6 +53,13 @@ typedef struct {
 typedef struct {
     tsv_tensor attn_norm, wq, wk, wv, wo, q_norm, k_norm;
     tsv_tensor ffn_norm, w_gate, w_up, w_down;
+    /* Routed experts in place of the dense FFN (crates/runtime/src/families/llama/moe.rs; router
+     * real_forward_dispatch.rs:1135-1158): n_experts == 0 means the dense matrices above are used.
+     * router: n_experts x hidden.  we_gate / we_up: all experts' matrices stacked,
+     * (n_experts * ffn) x hidden, expert e owning rows [e * ffn, (e + 1) * ffn); we_down:
+     * (n_experts * hidden) x ffn.  `ffn` of the model description is the expert width. */
+    int32_t n_experts, top_k;
+    tsv_tensor router, we_gate, we_up, we_down;
 } tsv_layer;
 
 typedef struct {

@@ -73,10 +73,13 @@ class Tensor(C.Structure):
     _fields_ = [("data", C.c_void_p), ("dtype", C.c_int32), ("rows", C.c_int64), ("cols", C.c_int64)]
 
 
+LAYER_TENSORS = ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up", "w_down")
+LAYER_MOE_TENSORS = ("router", "we_gate", "we_up", "we_down")
+
+
 class Layer(C.Structure):
-    _fields_ = [(n, Tensor) for n in
-                ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up",
-                 "w_down")]
+    _fields_ = ([(n, Tensor) for n in LAYER_TENSORS] + [("n_experts", C.c_int32), ("top_k", C.c_int32)] +
+                [(n, Tensor) for n in LAYER_MOE_TENSORS])
 
 
 class ModelDesc(C.Structure):
@@ -125,6 +128,7 @@ def lib():
         L.tso_dist_draw.restype = C.c_uint32
         L.tso_model_create.restype = C.c_void_p
         L.tso_model_position.restype = C.c_int64
+        L.tso_model_route_margin.restype = C.c_float
         L.tso_model_k.restype = C.POINTER(C.c_float)
         L.tso_model_v.restype = C.POINTER(C.c_float)
         L.tso_last_error.restype = C.c_char_p
@@ -401,8 +405,10 @@ class Model:
         n = cfg["n_layers"]
         self._layers = (Layer * n)()
         for i, lw in enumerate(weights["layers"]):
-            for name, _ in Layer._fields_:
+            for name in LAYER_TENSORS + LAYER_MOE_TENSORS:
                 setattr(self._layers[i], name, _tensor(lw.get(name)))
+            self._layers[i].n_experts = int(lw.get("n_experts", 0))
+            self._layers[i].top_k = int(lw.get("top_k", 0))
         d = ModelDesc()
         for key in ("n_layers", "hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab",
                     "max_context"):
@@ -434,6 +440,12 @@ class Model:
 
     def reset(self):
         lib().tso_model_reset(self._h)
+
+    @property
+    def route_margin(self):
+        """Smallest relative gap between the last chosen and the first rejected router logit
+        over the last verify call (1.0 for a dense model)."""
+        return float(lib().tso_model_route_margin(self._h))
 
     def rewind_to(self, position):
         lib().tso_model_rewind_to(self._h, C.c_int64(position))

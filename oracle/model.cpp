@@ -10,6 +10,7 @@
 // store (optional) and the logits store, the two dtype boundaries the engine fixes.
 #include "tsoracle.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <string>
@@ -27,6 +28,7 @@ struct tso_model {
     std::vector<float> rope_freqs;  // non-empty when rope_factors given
     std::vector<std::vector<float>> k, v;  // per layer [max_context][nkv*hd]
     int64_t position = 0;
+    float route_margin = 1.0f;
 };
 
 namespace {
@@ -51,6 +53,35 @@ void gemm_rows(const tso_tensor& w, const float* x, int m_rows, float* y, int th
                 y[(int64_t)m * rows + r] = acc;
             }
         }
+    }
+}
+
+// Rows [r0, r0 + n) of a stacked matrix as a tensor of their own.
+tso_tensor row_slice(const tso_tensor& t, int64_t r0, int64_t n) {
+    tso_tensor v = t;
+    v.data = (const uint8_t*)t.data + r0 * tso_row_bytes(t.dtype, t.cols);
+    v.rows = n;
+    return v;
+}
+
+// real_forward_dispatch.rs:1135-1158 (`router_topk_gemma4`, per_expert_scale all ones): top-k by
+// logit, ties to the lower index; softmax over the selected logits only.
+void route_topk(const float* logits, int n, int k, int* sel, float* w, float* margin) {
+    std::vector<int> order(n);
+    for (int i = 0; i < n; i++) order[i] = i;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return logits[a] > logits[b]; });
+    const float mx = logits[order[0]];
+    float sum = 0.0f, ex[8];
+    for (int i = 0; i < k; i++) {
+        sel[i] = order[i];
+        ex[i] = std::exp(logits[order[i]] - mx);
+        sum += ex[i];
+    }
+    for (int i = 0; i < k; i++) w[i] = ex[i] / sum * 1.0f;
+    if (k < n) {
+        const float range = mx - logits[order[n - 1]];
+        const float gap = (logits[order[k - 1]] - logits[order[k]]) / (range > 0.0f ? range : 1.0f);
+        if (gap < *margin) *margin = gap;
     }
 }
 
@@ -87,6 +118,7 @@ extern "C" tso_model* tso_model_create(const tso_model_desc* desc) {
 }
 
 extern "C" void tso_model_destroy(tso_model* m) { delete m; }
+extern "C" float tso_model_route_margin(const tso_model* m) { return m->route_margin; }
 extern "C" void tso_model_reset(tso_model* m) { m->position = 0; }
 extern "C" int64_t tso_model_position(const tso_model* m) { return m->position; }
 // kv_cache_rewind.rs:46-55: a cursor move; rows are addressed by absolute position and
@@ -149,6 +181,7 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
         att((size_t)M * qd), proj((size_t)M * H), gate((size_t)M * F), up((size_t)M * F);
 
     int L = n_layers_run < 0 ? d.n_layers : std::min(n_layers_run, (int)d.n_layers);
+    mdl->route_margin = 1.0f;
     for (int l = 0; l < L; l++) {
         const tso_layer& ly = d.layers[l];
         std::vector<float> wn = norm_weight(ly.attn_norm);
@@ -212,11 +245,32 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
         std::vector<float> wf = norm_weight(ly.ffn_norm);
         for (int m = 0; m < M; m++)
             tso_rms_norm(&x[(size_t)m * H], wf.data(), H, d.rms_eps, &xn[(size_t)m * H]);
-        gemm_rows(ly.w_gate, xn.data(), M, gate.data(), T);
-        gemm_rows(ly.w_up, xn.data(), M, up.data(), T);
-        for (size_t i = 0; i < (size_t)M * F; i++) gate[i] = tso_silu(gate[i]) * up[i];
-        gemm_rows(ly.w_down, gate.data(), M, proj.data(), T);
-        for (size_t i = 0; i < (size_t)M * H; i++) x[i] = x[i] + proj[i];
+        if (ly.n_experts > 0) {
+            // families/llama/moe.rs + compute/src/moe.rs:47-73: y = x + sum over slots, in the
+            // router's rank order, of w_slot * down_e(silu(gate_e xn) * up_e xn)
+            const int E = ly.n_experts, K = ly.top_k;
+            std::vector<float> rl((size_t)M * E);
+            gemm_rows(ly.router, xn.data(), M, rl.data(), T);
+            for (int m = 0; m < M; m++) {
+                int sel[8];
+                float w[8];
+                route_topk(&rl[(size_t)m * E], E, K, sel, w, &mdl->route_margin);
+                for (int s = 0; s < K; s++) {
+                    const int e = sel[s];
+                    gemm_rows(row_slice(ly.we_gate, (int64_t)e * F, F), &xn[(size_t)m * H], 1, gate.data(), T);
+                    gemm_rows(row_slice(ly.we_up, (int64_t)e * F, F), &xn[(size_t)m * H], 1, up.data(), T);
+                    for (int i = 0; i < F; i++) gate[i] = tso_silu(gate[i]) * up[i];
+                    gemm_rows(row_slice(ly.we_down, (int64_t)e * H, H), gate.data(), 1, proj.data(), T);
+                    for (int i = 0; i < H; i++) x[(size_t)m * H + i] += w[s] * proj[i];
+                }
+            }
+        } else {
+            gemm_rows(ly.w_gate, xn.data(), M, gate.data(), T);
+            gemm_rows(ly.w_up, xn.data(), M, up.data(), T);
+            for (size_t i = 0; i < (size_t)M * F; i++) gate[i] = tso_silu(gate[i]) * up[i];
+            gemm_rows(ly.w_down, gate.data(), M, proj.data(), T);
+            for (size_t i = 0; i < (size_t)M * H; i++) x[i] = x[i] + proj[i];
+        }
     }
 
     // head (verify_layers.rs:270-333): final norm, lm_head, raw logits (mod.rs:421-423)

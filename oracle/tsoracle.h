@@ -171,6 +171,10 @@ typedef struct {
 typedef struct {
     tso_tensor attn_norm, wq, wk, wv, wo, q_norm, k_norm; /* q_norm/k_norm data NULL when absent */
     tso_tensor ffn_norm, w_gate, w_up, w_down;
+    /* routed experts instead of the dense FFN when n_experts > 0: router n_experts x hidden;
+     * we_gate / we_up (n_experts * ffn) x hidden, we_down (n_experts * hidden) x ffn, stacked */
+    int32_t n_experts, top_k;
+    tso_tensor router, we_gate, we_up, we_down;
 } tso_layer;
 
 typedef struct {
@@ -184,6 +188,10 @@ typedef struct {
 } tso_model_desc;
 
 typedef struct tso_model tso_model;
+/* Smallest distance, over every routing decision of the last verify call, between the last
+ * selected and the first rejected router logit, relative to the row's logit range: a caller
+ * comparing against an implementation with different rounding can see that no choice was close. */
+float tso_model_route_margin(const tso_model* m);
 tso_model* tso_model_create(const tso_model_desc* desc);
 void tso_model_destroy(tso_model* m);
 void tso_model_reset(tso_model* m);

@@ -1,0 +1,93 @@
+"""GPU parity of the routed-expert (MoE) verify pass against the oracle: Q8_0 attention and
+router, MXFP4 experts, top-k routing with softmax over the selected logits (the arrangement of
+the Qwen3-30B-A3B configuration, crates/runtime/src/families/llama/moe.rs)."""
+import numpy as np
+import pytest
+
+from tests import gpu_common as gc
+
+pytestmark = pytest.mark.gpu
+
+MXFP4_TOL = 1e-2   # max-abs logit error relative to the logit range, MXFP4 / Q4_K bar
+
+
+def _prompt(n, vocab, seed):
+    return np.random.default_rng(seed).integers(0, vocab, n).astype(np.int32)
+
+
+def _clean_inputs(cfg, cpu, ctx, k, floor=2e-3):
+    """Seeded prompt + feed for which no routing decision of the reference run is a near tie (the
+    GPU's router logits carry fp16-activation rounding, a few 1e-4 of the logit range, so a
+    closer call could legitimately go the other way and the comparison would mean nothing).
+    Leaves the oracle advanced past both; returns its verify logits."""
+    for attempt in range(20):
+        prompt = _prompt(ctx, cfg["vocab"], 7 + 100 * attempt)
+        feed = _prompt(k + 1, cfg["vocab"], 8 + 100 * attempt)
+        cpu.reset()
+        margins = []
+        for i in range(0, ctx, 16):
+            cpu.verify(prompt[i:i + 16], i)
+            margins.append(cpu.route_margin)
+        want = cpu.verify(feed, ctx)
+        margins.append(cpu.route_margin)
+        if min(margins) > floor:
+            return prompt, feed, want, min(margins)
+    raise AssertionError("no seed without a near-tie routing decision in 20 tries")
+
+
+@pytest.mark.parametrize("ctx,k", [(40, 8), (21, 4), (33, 15), (16, 0)])
+def test_moe_verify_logits_match_the_oracle(ctx, k):
+    cfg, w, gpu, cpu = gc.build_pair("moe_small", max_context=ctx + 32)
+    prompt, feed, want, margin = _clean_inputs(cfg, cpu, ctx, k)
+    gpu.prefill(prompt, 0, want_logits=False)
+    got = gpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"moe_small ctx={ctx} m={k+1}: max-abs logit error / range = {err:.2e}, route margin {margin:.3e}")
+    assert err <= MXFP4_TOL, err
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gpu.read_kv(layer, 0, ctx)
+        kc, vc = cpu.kv(layer)
+        assert np.abs(kg.astype(np.float32) - kc[:ctx]).max() <= 2e-2 * np.abs(kc[:ctx]).max()
+
+
+def test_moe_batched_pass_equals_the_same_tokens_fed_one_at_a_time():
+    """Row invariance with routed experts: an expert multiplies only the rows that chose it, and a
+    row's result must not depend on which other rows share its experts."""
+    cfg, w, gpu, cpu = gc.build_pair("moe_small", max_context=96)
+    prompt = _prompt(30, cfg["vocab"], 3)
+    gpu.prefill(prompt, 0, want_logits=False)
+    feed = _prompt(9, cfg["vocab"], 4)
+    point = gpu.checkpoint()
+    batch = gpu.verify(feed, 30)
+    gpu.rollback(point)
+    seq = np.stack([gpu.produce(t, 30 + i) for i, t in enumerate(feed)])
+    assert np.array_equal(batch, seq)
+
+
+def test_moe_greedy_round_matches_the_oracle_walk():
+    """Configuration-4 style round: chain k=8, greedy acceptance on the MoE target's logits."""
+    import turbospark_amd as ts
+    from oracle import binding as ob
+    cfg, w, gpu, cpu = gc.build_pair("moe_small", max_context=96)
+    prompt = _prompt(24, cfg["vocab"], 5)
+    gpu.prefill(prompt[:-1], 0, want_logits=False)
+    cpu.verify(prompt[:-1], 0)
+    base = gpu.position
+    # proposals: the oracle's own greedy continuation for the first 3, then junk -> accepted == 3
+    point_tokens = [int(prompt[-1])]
+    for i in range(3):
+        lg = cpu.verify(point_tokens[-1:], base + i)
+        point_tokens.append(int(np.argmax(gc.f16(lg[0]))))
+    cpu.rewind_to(base)
+    feed = point_tokens + [1, 2, 3, 4, 5]
+    logits = gc.f16(cpu.verify(feed, base))
+    want_acc = 0
+    for i in range(8):
+        if int(np.argmax(logits[i])) == feed[i + 1]:
+            want_acc += 1
+        else:
+            break
+    res = gpu.verify_accept(feed, base, ts.shaping(0.0))
+    assert res.accepted == want_acc >= 3
+    assert res.next == int(np.argmax(logits[want_acc]))
+    assert res.kv_position == base + want_acc + 1

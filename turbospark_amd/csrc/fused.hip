@@ -348,7 +348,7 @@ __global__ __launch_bounds__(512) void k_ffn_block(FfnBlockArgs a) {
 
     {
         const uint8_t* fa = a.norm.frag + (size_t)ctx.xcc * a.norm.frag_stride;
-        const ActLoader<true> xa(fa, fa + xfrag_sum_offset(a.norm.hidden));
+        const ActLoader<true> xa(fa, fa + xfrag_sum_offset(a.norm.hidden), lane);
         _Float16* fc = (_Float16*)a.frag_c;
         float* fc_sums = (float*)((char*)a.frag_c + xfrag_sum_offset(a.ffn));
         for (int t0 = first; t0 < gu_per; t0 += stride) {
@@ -393,7 +393,7 @@ __global__ __launch_bounds__(512) void k_ffn_block(FfnBlockArgs a) {
     if (!xcd_barrier(ctx, s_i)) return;
     TRACE(7);
     {
-        const ActLoader<true> xc(a.frag_c, (const char*)a.frag_c + xfrag_sum_offset(a.ffn));
+        const ActLoader<true> xc(a.frag_c, (const char*)a.frag_c + xfrag_sum_offset(a.ffn), lane);
         float* out = a.partial_out + (size_t)ctx.xcc * 16 * a.norm.hidden;
         for (int t0 = first; t0 < a.down_tiles; t0 += stride) {
             const int t = t0 + tw;

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     // outstanding tile only (s_waitcnt vmcnt(n)) instead of draining the queue.
     if (nc > 0) {
         Stage<F, NG> st[STAGES];
-        const ActLoader<false> x(a.xfrag, a.xsum);
+        const ActLoader<false> x(a.xfrag, a.xsum, lane);
         const int last = c0 + nc - 1;
         auto fetch = [&](Stage<F, NG>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
 #pragma unroll

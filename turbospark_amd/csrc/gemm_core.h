@@ -99,8 +99,9 @@ struct Q4K {
 #pragma unroll
         for (int u = 0; u < 9; u++) dma_to_lds_b128(tile + u * 1024 + lane * 16, lds + u * 1024);
     }
-    // float index of this lane's sub-block sums for row group g of chunk c
-    static __device__ __forceinline__ int xs_index(int c, int g, int lane) { return (c * 4 + g) * 32 + (lane & 31); }
+    // float index of this lane's sub-block sums of chunk c, before the row's own offset
+    // (ActLoader::sumoff) is added: lane (b, i) reads sub-block b
+    static __device__ __forceinline__ int xs_base(int c, int lane) { return c * 128 + ((lane >> 2) & 7) * 4; }
 };
 
 struct Q80 {
@@ -124,8 +125,8 @@ struct Q80 {
         for (int h = 0; h < 2; h++) dma_to_lds_b32(tile + 8192 + h * 256 + lane * 4, lds + 8192 + h * 256);
     }
     // a 128-element chunk is half of a 256-element sum group: its four sub-blocks go to blocks 0..3
-    static __device__ __forceinline__ int xs_index(int c, int g, int lane) {
-        return ((c >> 1) * 4 + g) * 32 + (c & 1) * 16 + (lane & 15);
+    static __device__ __forceinline__ int xs_base(int c, int lane) {
+        return (c >> 1) * 128 + (c & 1) * 16 + ((lane >> 2) & 3) * 4;
     }
 };
 
@@ -145,7 +146,7 @@ struct MX4 {
     static __device__ __forceinline__ void load_to_lds(uint32_t lds, const uint8_t* tile, int lane) {
         Q80::load_to_lds(lds, tile, lane);
     }
-    static __device__ __forceinline__ int xs_index(int c, int g, int lane) { return Q4K::xs_index(c, g, lane); }
+    static __device__ __forceinline__ int xs_base(int c, int lane) { return Q4K::xs_base(c, lane); }
 };
 
 template <class F, int NG>
@@ -183,14 +184,23 @@ struct LdsSrc {
 
 // Cache policy of the activation loads: plain, or device-coherent (sc1) for activations that
 // another compute unit wrote earlier in the same kernel (they must not come from this CU's L1).
+// Which activation row feeds slot (g, i) of the MFMA A operand is a per-lane offset table: the
+// identity for a dense matmul, a gather for a routed expert that sees only its own rows.
 template <bool COHERENT>
 struct ActLoader {
     __amdgpu_buffer_rsrc_t frag, sums;
     const u32x2* fragp;
     const float* sump;
-    __device__ __forceinline__ ActLoader(const void* xfrag, const void* xsum) {
+    int rowoff[4], sumoff[4];  // offsets of row group g's row for this lane, in 8-byte units / floats
+    __device__ __forceinline__ void set_row(int g, int row) {
+        rowoff[g] = (row >> 2) * 64 + (row & 3);
+        sumoff[g] = (row >> 2) * 32 + (row & 3);
+    }
+    __device__ __forceinline__ ActLoader(const void* xfrag, const void* xsum, int lane) {
         fragp = (const u32x2*)xfrag;
         sump = (const float*)xsum;
+#pragma unroll
+        for (int g = 0; g < 4; g++) set_row(g, 4 * g + (lane & 3));
         if (COHERENT) {
             frag = __builtin_amdgcn_make_buffer_rsrc((void*)xfrag, 0, 0x7FFFFFFF, 0x00027000);
             sums = __builtin_amdgcn_make_buffer_rsrc((void*)xsum, 0, 0x7FFFFFFF, 0x00027000);
@@ -212,10 +222,10 @@ __device__ __forceinline__ void load_x(XRegs<F, NG>& xr, const ActLoader<COH>& x
 #pragma unroll
     for (int p = 0; p < F::NPAIR; p++)
 #pragma unroll
-        for (int g = 0; g < NG; g++) xr.xa[p][g] = x.frag_at(((c * F::NPAIR + p) * 4 + g) * 64 + lane);
+        for (int g = 0; g < NG; g++) xr.xa[p][g] = x.frag_at((c * F::NPAIR + p) * 256 + x.rowoff[g] + (lane >> 2) * 4);
     if (F::SUMS) {
 #pragma unroll
-        for (int g = 0; g < NG; g++) xr.xs[g] = x.sum_at(F::xs_index(c, g, lane));
+        for (int g = 0; g < NG; g++) xr.xs[g] = x.sum_at(F::xs_base(c, lane) + x.sumoff[g]);
     }
 }
 

@@ -77,7 +77,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // thread so every load of a row is issued before the first one is waited on.
 __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const float* __restrict__ partial,
                                                   int splits, int ldp, const float* __restrict__ w,
-                                                  float eps, int hidden, _Float16* __restrict__ xfrag) {
+                                                  float eps, int hidden, _Float16* __restrict__ xfrag,
+                                                  const float* __restrict__ weights) {
     __shared__ float red[16];
     const int m = blockIdx.x;
     float4* xr = (float4*)(x + (long)m * hidden);
@@ -87,11 +88,18 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
     for (int i = threadIdx.x; i < n4; i += 1024) {
         float4 v = xr[i];
         for (int s = 0; s < splits; s++) {
-            const float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
-            v.x += p.x;
-            v.y += p.y;
-            v.z += p.z;
-            v.w += p.w;
+            float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
+            if (weights) {  // routed experts: y += w_slot * out_slot, product and sum rounded apart
+                const float ws = weights[m * 8 + s];
+                p.x = __fmul_rn(ws, p.x);
+                p.y = __fmul_rn(ws, p.y);
+                p.z = __fmul_rn(ws, p.z);
+                p.w = __fmul_rn(ws, p.w);
+            }
+            v.x = __fadd_rn(v.x, p.x);
+            v.y = __fadd_rn(v.y, p.y);
+            v.z = __fadd_rn(v.z, p.z);
+            v.w = __fadd_rn(v.w, p.w);
         }
         xr[i] = v;
         ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
@@ -115,9 +123,9 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
 }
 
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
-                   float eps, int hidden, uint4* xfrag, int m) {
+                   float eps, int hidden, uint4* xfrag, int m, const float* weights) {
     hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
-                       (_Float16*)xfrag);
+                       (_Float16*)xfrag, weights);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -1,0 +1,255 @@
+// Routed-expert (MoE) FFN for a verify pass on gfx950.
+//
+// Replaces the reference's per-token expert dispatch (crates/runtime/src/families/llama/moe.rs,
+// router semantics real_forward_dispatch.rs:1135-1158, expert math
+// crates/gpu/src/shaders/moe_gguf.metal phase 1 / phase 2, CPU pattern crates/compute/src/moe.rs:22-73):
+//   logits = router . x_norm;  top-k by logit, ties to the lower expert index;  softmax over the
+//   selected logits only;  y = x + sum over slots IN RANK ORDER of w_slot * down_e(silu(gate_e x) * up_e x).
+// Here all rows of the pass are routed at once and the experts are grouped: every expert that at
+// least one row selected is multiplied ONCE, against just the rows that chose it (its weights are
+// read once however many rows share it), by the same 64-row-tile MFMA sequences as the dense
+// matmuls with a gathered activation operand.  The per-(row, slot) outputs are written apart and
+// the next residual kernel adds them in slot order, so the sum has the reference's order.
+#include <algorithm>
+
+#include "gemm_core.h"
+
+namespace tsv {
+
+namespace {
+
+// ---- router ---------------------------------------------------------------------------------
+// One workgroup.  Wave w routes rows w, w + 4, ...: the row's logits (split-K partials summed in
+// order) sit 'ne / 64' per lane; k rounds of a wave-wide arg-max (larger logit, then lower
+// index) pick the experts in rank order.  Then every expert's row list is built in row order.
+__global__ __launch_bounds__(256) void k_route(MoeRouteArgs a) {
+    __shared__ int s_sel[TSV_MAX_ROWS][8];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int M = a.vp->m, ne = a.n_experts, k = a.top_k;
+    for (int m = wave; m < M; m += 4) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int e = lane + 64 * j;
+            v[j] = -INFINITY;
+            if (e < ne) {
+                float s = 0.f;
+                for (int sp = 0; sp < a.splits; sp++) s += a.logits[((size_t)sp * 16 + m) * a.ld + e];
+                v[j] = s;
+            }
+        }
+        float top = 0.f, ex[8], sum = 0.f;
+        int sel[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            sel[r] = 0;
+            ex[r] = 0.f;
+            if (r < k) {
+                float best = -INFINITY;
+                int bi = 0x7FFFFFFF;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (v[j] > best) {  // ascending j is ascending index: the first maximum wins
+                        best = v[j];
+                        bi = lane + 64 * j;
+                    }
+                for (int o = 32; o > 0; o >>= 1) {
+                    const float ob = __shfl_xor(best, o);
+                    const int oi = __shfl_xor(bi, o);
+                    if (ob > best || (ob == best && oi < bi)) {
+                        best = ob;
+                        bi = oi;
+                    }
+                }
+                if (r == 0) top = best;
+                sel[r] = bi;
+                ex[r] = expf(best - top);
+                sum += ex[r];  // sequential in rank order, as `exps.iter().sum()`
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (lane + 64 * j == bi) v[j] = -INFINITY;
+            }
+        }
+        // lane r keeps slot r
+        float w = 0.f;
+        int e = 0;
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+            if (r == lane) {
+                w = ex[r] / sum;
+                e = sel[r];
+            }
+        if (lane < k) {
+            a.weights[m * 8 + lane] = w;
+            a.selected[m * 8 + lane] = e;
+            s_sel[m][lane] = e;
+        }
+    }
+    __syncthreads();
+    // expert e's rows, ascending (thread e)
+    for (int e = threadIdx.x; e < ne; e += 256) {
+        int n = 0;
+        for (int m = 0; m < M; m++)
+            for (int r = 0; r < k; r++)
+                if (s_sel[m][r] == e) {
+                    a.rows[e * 16 + n] = m;
+                    a.slots[e * 16 + n] = r;
+                    n++;
+                }
+        a.count[e] = n;
+    }
+}
+
+// ---- grouped expert matmul --------------------------------------------------------------------
+__device__ __forceinline__ float silu_moe(float x) { return x / (1.0f + __expf(-x)); }
+
+template <class F, int EPI, int NG>
+__device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, int e, int cnt, const int* rows, const int* slots,
+                                            float4v* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int tile = blockIdx.x;
+    const int per = (a.kchunks + nw - 1) / nw;
+    const int c0 = min(wave * per, a.kchunks), nc = min(per, a.kchunks - c0);
+    const uint8_t* wt = a.w + ((size_t)e * a.tiles_per_expert + tile) * a.kchunks * F::TILE_BYTES;
+    Consts k;
+    k.k6400 = 0x64006400u;
+    k.k5400 = 0x54005400u;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
+
+    // activation operand: gate/up reads the pass's rows this expert was chosen by (gathered); down
+    // reads the expert's own buffer, whose rows are already in the expert's order
+    const uint8_t* xbase = (const uint8_t*)a.xfrag + (EPI == EPI_SLOT ? (size_t)e * a.x_stride : 0);
+    ActLoader<false> x(xbase, xbase + xfrag_sum_offset(a.k), lane);
+    if (EPI == EPI_SILU) {
+#pragma unroll
+        for (int g = 0; g < NG; g++) x.set_row(g, rows[min(4 * g + (lane & 3), cnt - 1)]);
+    }
+
+    float4v acc[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) acc[g] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (nc > 0) {
+        Stage<F, NG> st[2];
+        const int last = c0 + nc - 1;
+        auto fetch = [&](Stage<F, NG>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
+        fetch(st[0], c0);
+        fetch(st[1], min(c0 + 1, last));
+        int c = 0;
+        for (; c + 4 <= nc; c += 2) {
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                compute(st[s], k, acc);
+                fetch(st[s], c0 + c + s + 2);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            if (c + s < nc) {
+                compute(st[s], k, acc);
+                if (c + s + 2 < nc) fetch(st[s], c0 + c + s + 2);
+            }
+        }
+        c += 2;
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+            if (c + s < nc) compute(st[s], k, acc);
+    }
+
+    // fold the waves in wave order, then wave w finishes row groups w, w + nw, ...
+#pragma unroll
+    for (int g = 0; g < NG; g++) red[(wave * NG + g) * 64 + lane] = acc[g];
+    __syncthreads();
+    for (int g = wave; g < NG; g += nw) {
+        float4v v = red[g * 64 + lane];
+        for (int w = 1; w < nw; w++) v += red[(w * NG + g) * 64 + lane];
+        if (EPI == EPI_SILU) {
+            // lanes 0..31: gate rows, lanes 32..63: up rows of the same 32 columns of this expert
+            const int col = tile * 32 + (lane & 31);
+            _Float16* out = (_Float16*)((uint8_t*)a.out + (size_t)e * a.out_stride);
+            float* sums = (float*)((uint8_t*)out + xfrag_sum_offset(a.n_out));
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float other = __shfl_xor(v[i], 32);
+                const float gate = lane < 32 ? v[i] : other, up = lane < 32 ? other : v[i];
+                const _Float16 h = (_Float16)(silu_moe(gate) * up);
+                float sum = (float)h;
+#pragma unroll
+                for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
+                const int b = 4 * g + i;  // the expert's own row order
+                if (b < cnt && lane < 32) {
+                    out[frag_index(col, b)] = h;
+                    if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
+                }
+            }
+        } else {
+            const int n = tile * 64 + lane;
+            if (n < a.n_out) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int b = 4 * g + i;
+                    if (b < cnt) ((float*)a.out)[((size_t)slots[b] * 16 + rows[b]) * a.n_out + n] = v[i];
+                }
+            }
+        }
+    }
+}
+
+// grid: (tiles per expert, experts).  Experts nobody chose leave at once.
+template <class F, int EPI>
+__global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
+    extern __shared__ float4v red[];
+    __shared__ int s_rows[16], s_slots[16];
+    const int e = blockIdx.y;
+    const int cnt = a.count[e];
+    if (cnt == 0) return;
+    if (threadIdx.x < 16) {
+        s_rows[threadIdx.x] = a.rows[e * 16 + threadIdx.x];
+        s_slots[threadIdx.x] = a.slots[e * 16 + threadIdx.x];
+    }
+    __syncthreads();
+    if (cnt <= 4)
+        expert_tile<F, EPI, 1>(a, e, cnt, s_rows, s_slots, red);
+    else if (cnt <= 8)
+        expert_tile<F, EPI, 2>(a, e, cnt, s_rows, s_slots, red);
+    else
+        expert_tile<F, EPI, 4>(a, e, cnt, s_rows, s_slots, red);
+}
+
+template <class F, int EPI>
+int launch_moe_t(hipStream_t s, const MoeGemmArgs& a, int n_experts) {
+    const int nw = std::min(8, std::max(1, a.kchunks));
+    const size_t lds = (size_t)nw * 4 * 1024;
+    hipLaunchKernelGGL((k_moe_gemm<F, EPI>), dim3(a.tiles_per_expert, n_experts), dim3(64 * nw), lds, s, a);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+template <int EPI>
+int launch_moe_f(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts) {
+    return fmt == FMT_Q4K   ? launch_moe_t<Q4K, EPI>(s, a, n_experts)
+           : fmt == FMT_Q80 ? launch_moe_t<Q80, EPI>(s, a, n_experts)
+                            : launch_moe_t<MX4, EPI>(s, a, n_experts);
+}
+
+}  // namespace
+
+int launch_route(hipStream_t s, const MoeRouteArgs& a) {
+    if (a.n_experts > 256 || a.top_k < 1 || a.top_k > 8 || a.top_k > a.n_experts) {
+        set_error("moe: at most 256 experts and top-k between 1 and 8");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(k_route, dim3(1), dim3(256), 0, s, a);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts) {
+    return launch_moe_f<EPI_SILU>(s, fmt, a, n_experts);
+}
+
+int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts) {
+    return launch_moe_f<EPI_SLOT>(s, fmt, a, n_experts);
+}
+
+}  // namespace tsv

@@ -18,6 +18,8 @@ namespace {
 
 struct LayerW {
     TiledW qkv, wo, gate_up, down;
+    int n_experts = 0, top_k = 0;     // routed experts: gate_up / down hold every expert's tiles
+    TiledW router;
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
     uint16_t *kc = nullptr, *vc = nullptr;
 };
@@ -43,6 +45,13 @@ struct tsv_ctx {
     uint4 *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
     float* partial = nullptr;
     size_t partial_floats = 0;
+    // routed experts: routing tables, per-expert activation fragments, per-slot outputs
+    int max_experts = 0;
+    float* route_w = nullptr;
+    int32_t *route_sel = nullptr, *route_cnt = nullptr, *route_rows = nullptr, *route_slots = nullptr;
+    uint8_t* frag_e = nullptr;
+    size_t frag_e_stride = 0;
+    float* moe_out = nullptr;
     // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
     // sum-of-squares partials, per-XCD partial sums, barrier counters
     bool fused_ffn = false;
@@ -343,13 +352,16 @@ int launch_pass(tsv_ctx* c, int m) {
     if (rc) return rc;
     int prev_splits = 0;
     const float* prev_partial = c->partial;
+    const float* prev_weights = nullptr;  // routed experts: the factors of the per-slot outputs
     float *x = c->x, *x_other = c->x2;  // the fused kernels write the residual rows to the other buffer
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
         {
             PROF(PC_NORM);
-            rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m);
+            rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m,
+                                prev_weights);
+            prev_weights = nullptr;
         }
         if (rc) return rc;
         int sp = splits_for(L.qkv, m, EPI_PARTIAL);
@@ -450,6 +462,62 @@ int launch_pass(tsv_ctx* c, int m) {
             rc = launch_addnorm(s, x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m);
         }
         if (rc) return rc;
+        if (L.n_experts) {
+            // router -> top-k -> grouped expert matmuls; the per-slot outputs are added, weighted
+            // and in slot order, by the next residual kernel
+            const int rsp = splits_for(L.router, m, EPI_PARTIAL);
+            MoeRouteArgs ra2;
+            ra2.logits = c->partial;
+            ra2.splits = rsp;
+            ra2.ld = L.n_experts;
+            ra2.n_experts = L.n_experts;
+            ra2.top_k = L.top_k;
+            ra2.vp = c->vp_dev;
+            ra2.weights = c->route_w;
+            ra2.selected = c->route_sel;
+            ra2.count = c->route_cnt;
+            ra2.rows = c->route_rows;
+            ra2.slots = c->route_slots;
+            MoeGemmArgs g1, g2;
+            g1.w = L.gate_up.tiles;
+            g1.tiles_per_expert = c->ffn / 32;
+            g1.kchunks = L.gate_up.kchunks;
+            g1.k = c->hidden;
+            g1.xfrag = c->xf_a;
+            g1.x_stride = 0;
+            g1.out = c->frag_e;
+            g1.out_stride = c->frag_e_stride;
+            g1.n_out = c->ffn;
+            g1.count = c->route_cnt;
+            g1.rows = c->route_rows;
+            g1.slots = c->route_slots;
+            g2 = g1;
+            g2.w = L.down.tiles;
+            g2.tiles_per_expert = c->hidden / 64;
+            g2.kchunks = L.down.kchunks;
+            g2.k = c->ffn;
+            g2.xfrag = c->frag_e;
+            g2.x_stride = c->frag_e_stride;
+            g2.out = c->moe_out;
+            g2.out_stride = 0;
+            g2.n_out = c->hidden;
+            {
+                PROF(PC_GATEUP);
+                rc = launch_gemm(s, L.router, c->xf_a, c->partial, c->vp_dev, m, rsp, EPI_PARTIAL, L.n_experts, L.n_experts);
+                if (!rc) rc = launch_route(s, ra2);
+                if (!rc) rc = launch_moe_gate_up(s, L.gate_up.fmt, g1, L.n_experts);
+            }
+            if (rc) return rc;
+            {
+                PROF(PC_DOWN);
+                rc = launch_moe_down(s, L.down.fmt, g2, L.n_experts);
+            }
+            if (rc) return rc;
+            prev_partial = c->moe_out;
+            prev_splits = L.top_k;
+            prev_weights = c->route_w;
+            continue;
+        }
         {
             PROF(PC_GATEUP);
             rc = 0;
@@ -470,7 +538,8 @@ int launch_pass(tsv_ctx* c, int m) {
     }
     {
         PROF(PC_NORM);
-        rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m);
+        rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m,
+                            prev_weights);
     }
     if (rc) return rc;
     {
@@ -572,18 +641,46 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         const tsv_layer& s = d->layers[l];
         LayerW& L = c->layers[l];
         if ((rc = check_matrix(s.wq, qd, c->hidden, "wq")) || (rc = check_matrix(s.wk, kvd, c->hidden, "wk")) ||
-            (rc = check_matrix(s.wv, kvd, c->hidden, "wv")) || (rc = check_matrix(s.wo, c->hidden, qd, "wo")) ||
-            (rc = check_matrix(s.w_gate, c->ffn, c->hidden, "w_gate")) ||
-            (rc = check_matrix(s.w_up, c->ffn, c->hidden, "w_up")) ||
-            (rc = check_matrix(s.w_down, c->hidden, c->ffn, "w_down")))
+            (rc = check_matrix(s.wv, kvd, c->hidden, "wv")) || (rc = check_matrix(s.wo, c->hidden, qd, "wo")))
             return fail(rc);
         const tsv_tensor* qkv[3] = {&s.wq, &s.wk, &s.wv};
-        const tsv_tensor* gu[2] = {&s.w_gate, &s.w_up};
         const tsv_tensor* wo[1] = {&s.wo};
-        const tsv_tensor* dn[1] = {&s.w_down};
-        if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv)) || (rc = make_tiled(c, st, wo, 1, false, &L.wo)) ||
-            (rc = make_tiled(c, st, gu, 2, true, &L.gate_up)) || (rc = make_tiled(c, st, dn, 1, false, &L.down)))
+        if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv)) || (rc = make_tiled(c, st, wo, 1, false, &L.wo)))
             return fail(rc);
+        const int ne = s.n_experts;
+        if (ne > 0) {
+            // every expert's gate/up rows interleave in runs of 32 inside the stacked matrix, so an
+            // expert owns ffn / 32 consecutive tiles; its down projection owns hidden / 64 tiles
+            if (ne > 256 || s.top_k < 1 || s.top_k > 8 || s.top_k > ne || c->ffn % 32 || c->hidden % 64) {
+                set_error("open: routed experts need <= 256 experts, top-k in 1..8, ffn % 32 == 0, hidden % 64 == 0");
+                return fail(TSV_ERR_UNSUPPORTED);
+            }
+            if ((rc = check_matrix(s.router, ne, c->hidden, "router")) ||
+                (rc = check_matrix(s.we_gate, (int64_t)ne * c->ffn, c->hidden, "we_gate")) ||
+                (rc = check_matrix(s.we_up, (int64_t)ne * c->ffn, c->hidden, "we_up")) ||
+                (rc = check_matrix(s.we_down, (int64_t)ne * c->hidden, c->ffn, "we_down")))
+                return fail(rc);
+            const tsv_tensor* rt[1] = {&s.router};
+            const tsv_tensor* gu[2] = {&s.we_gate, &s.we_up};
+            const tsv_tensor* dn[1] = {&s.we_down};
+            if ((rc = make_tiled(c, st, rt, 1, false, &L.router)) || (rc = make_tiled(c, st, gu, 2, true, &L.gate_up)) ||
+                (rc = make_tiled(c, st, dn, 1, false, &L.down)))
+                return fail(rc);
+            L.n_experts = ne;
+            L.top_k = s.top_k;
+            c->max_experts = std::max(c->max_experts, ne);
+            pneed = std::max(pneed, partial_need(L.router));
+        } else {
+            if ((rc = check_matrix(s.w_gate, c->ffn, c->hidden, "w_gate")) ||
+                (rc = check_matrix(s.w_up, c->ffn, c->hidden, "w_up")) ||
+                (rc = check_matrix(s.w_down, c->hidden, c->ffn, "w_down")))
+                return fail(rc);
+            const tsv_tensor* gu[2] = {&s.w_gate, &s.w_up};
+            const tsv_tensor* dn[1] = {&s.w_down};
+            if ((rc = make_tiled(c, st, gu, 2, true, &L.gate_up)) || (rc = make_tiled(c, st, dn, 1, false, &L.down)))
+                return fail(rc);
+            pneed = std::max(pneed, partial_need(L.down));
+        }
         if ((rc = upload_vector(c, s.attn_norm, c->hidden, &L.attn_norm, "attn_norm")) ||
             (rc = upload_vector(c, s.ffn_norm, c->hidden, &L.ffn_norm, "ffn_norm")))
             return fail(rc);
@@ -594,7 +691,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         }
         const size_t kvb = (size_t)c->nkv * c->ctx_alloc * c->hd * 2;
         if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) return fail(rc);
-        pneed = std::max(pneed, std::max(partial_need(L.qkv), std::max(partial_need(L.wo), partial_need(L.down))));
+        pneed = std::max(pneed, std::max(partial_need(L.qkv), partial_need(L.wo)));
     }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
@@ -641,7 +738,14 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->partial_floats = pneed;
     if ((rc = dev_alloc(c, &c->x, (size_t)16 * c->hidden * 4, true)) || (rc = dev_alloc(c, &c->xf_a, xfb, true)) ||
         (rc = dev_alloc(c, &c->xf_b, xfb, true)) || (rc = dev_alloc(c, &c->xf_c, xfb, true)) ||
-        (rc = dev_alloc(c, &c->partial, pneed * 4, true)) || (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
+        (rc = dev_alloc(c, &c->partial, pneed * 4, true)) ||
+        (c->max_experts &&
+         ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, 16 * 8 * 4, true)) ||
+          (rc = dev_alloc(c, &c->route_cnt, (size_t)c->max_experts * 4, true)) ||
+          (rc = dev_alloc(c, &c->route_rows, (size_t)c->max_experts * 16 * 4, true)) ||
+          (rc = dev_alloc(c, &c->route_slots, (size_t)c->max_experts * 16 * 4, true)) ||
+          (rc = dev_alloc(c, &c->frag_e, (size_t)c->max_experts * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
+          (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)))) || (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
         (rc = dev_alloc(c, &c->part_o, (size_t)c->nkv * c->nch * rows_max * c->hd * 4, true)) ||
         (rc = dev_alloc(c, &c->part_ml, (size_t)c->nkv * c->nch * rows_max * 2 * 4, true)) ||
         (rc = dev_alloc(c, &c->logits, (size_t)16 * c->vocab * 2, true)) ||
@@ -668,7 +772,8 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, 0) != hipSuccess) coop = 0;
         if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) ncu = 0;
         ok = ok && coop && ncu == 256;
-        for (const LayerW& L : c->layers) ok = ok && fused_ffn_supported(L.gate_up, L.down, c->hidden, c->ffn);
+        for (const LayerW& L : c->layers)
+            ok = ok && L.n_experts == 0 && fused_ffn_supported(L.gate_up, L.down, c->hidden, c->ffn);
         if (ok) {
             c->frag8_stride = (xfrag_bytes(c->hidden) + 255) & ~(size_t)255;
             if ((rc = dev_alloc(c, &c->x2, (size_t)16 * c->hidden * 4, true)) ||

@@ -84,7 +84,7 @@ struct VerifyParams {
     uint32_t anc[TSV_MAX_ROWS];  // bit s set: row i attends cache slot base+s
 };
 
-enum { EPI_PARTIAL = 0, EPI_SILU = 1, EPI_LOGITS = 2 };
+enum { EPI_PARTIAL = 0, EPI_SILU = 1, EPI_LOGITS = 2, EPI_SLOT = 3 };
 
 struct GemmArgs {
     const uint8_t* w;
@@ -103,6 +103,31 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
                 int m, int splits, int epi, int ldo, int n_valid);
 int gemm_default_splits(const TiledW& w, int m);
+
+// ---- routed experts (moe.hip) -----------------------------------------------------------------
+struct MoeRouteArgs {
+    const float* logits;  // router matmul partials [splits][16][ld]
+    int splits, ld, n_experts, top_k;
+    const VerifyParams* vp;
+    float* weights;   // [16][8] softmax over the selected logits, rank order
+    int32_t* selected;  // [16][8] expert ids, rank order
+    int32_t* count;     // [n_experts] rows that chose the expert
+    int32_t* rows;      // [n_experts][16] those rows, ascending
+    int32_t* slots;     // [n_experts][16] the rank slot the expert has in that row
+};
+struct MoeGemmArgs {
+    const uint8_t* w;      // tiled weights of all experts, tiles_per_expert x kchunks tiles each
+    int tiles_per_expert, kchunks, k;
+    const void* xfrag;     // gate/up: the pass's activation fragments; down: per-expert fragments
+    size_t x_stride;       // down: bytes between experts' fragment buffers
+    void* out;             // gate/up: per-expert fragments of silu(gate) * up; down: float [8 slots][16][n_out]
+    size_t out_stride;
+    int n_out;             // gate/up: expert FFN width; down: hidden
+    const int32_t *count, *rows, *slots;
+};
+int launch_route(hipStream_t s, const MoeRouteArgs& a);
+int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts);
+int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts);
 
 // ---- per-XCD fused layer kernels ----------------------------------------------------------
 // Counters of the XCD-local barriers.  rank_ctr / bar_ctr: one word per XCD, 64 words apart.
@@ -144,8 +169,9 @@ int launch_ffn_block(hipStream_t s, int fmt, FfnBlockArgs& a, int m);
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
                  const VerifyParams* vp, int m);
+// weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
-                   float eps, int hidden, uint4* xfrag, int m);
+                   float eps, int hidden, uint4* xfrag, int m, const float* weights = nullptr);
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
 
 struct RopeKvArgs {

@@ -22,10 +22,13 @@ class Tensor(C.Structure):
     _fields_ = [("data", C.c_void_p), ("dtype", C.c_int32), ("rows", C.c_int64), ("cols", C.c_int64)]
 
 
+LAYER_TENSORS = ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up", "w_down")
+LAYER_MOE_TENSORS = ("router", "we_gate", "we_up", "we_down")
+
+
 class Layer(C.Structure):
-    _fields_ = [(n, Tensor) for n in
-                ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up",
-                 "w_down")]
+    _fields_ = ([(n, Tensor) for n in LAYER_TENSORS] + [("n_experts", C.c_int32), ("top_k", C.c_int32)] +
+                [(n, Tensor) for n in LAYER_MOE_TENSORS])
 
 
 class ModelDesc(C.Structure):

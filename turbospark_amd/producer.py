@@ -39,8 +39,10 @@ class HipVerifier:
         n = len(weights["layers"])
         self._layers = (ffi.Layer * n)()
         for i, lw in enumerate(weights["layers"]):
-            for name, _ in ffi.Layer._fields_:
+            for name in ffi.LAYER_TENSORS + ffi.LAYER_MOE_TENSORS:
                 setattr(self._layers[i], name, ffi.tensor(lw.get(name)))
+            self._layers[i].n_experts = int(lw.get("n_experts", 0))
+            self._layers[i].top_k = int(lw.get("top_k", 0))
         d = ffi.ModelDesc()
         d.n_layers = n
         for key in ("hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_context"):

@@ -18,6 +18,11 @@ CONFIGS = {
                      vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K, norm_jitter=0.25),
     "xcd_q8_0": dict(n_layers=2, hidden=1024, n_q_heads=16, n_kv_heads=8, head_dim=64, ffn=1024,
                      vocab=4096, rms_eps=1e-5, rope_theta=10000.0, dtype=ffi.Q8_0, norm_jitter=0.25),
+    # a small routed-expert decoder in the arrangement of the Qwen3-30B-A3B configuration: Q8_0
+    # attention and router, MXFP4 experts, top-k routing with softmax over the selected logits
+    "moe_small": dict(n_layers=2, hidden=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=256,
+                      n_experts=16, top_k=4, vocab=4096, rms_eps=1e-6, rope_theta=1000000.0,
+                      dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08, norm_jitter=0.25),
     # Llama-3-8B shape
     "llama3_8b_q4_k": dict(n_layers=32, hidden=4096, n_q_heads=32, n_kv_heads=8, head_dim=128,
                            ffn=14336, vocab=128256, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
@@ -41,13 +46,21 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
 
     stream = [0]
 
-    def t(rows, cols):
+    def t(rows, cols, dtype=None, sig=None):
         stream[0] += 1
-        return ffi.synth_tensor(dt, seed, stream[0], sigma, rows, cols)
+        return ffi.synth_tensor(dt if dtype is None else dtype, seed, stream[0], sigma if sig is None else sig,
+                                rows, cols)
 
     L = cfg["n_layers"] if n_layers is None else n_layers
+    E = int(cfg.get("n_experts", 0))
     layers = []
     for _ in range(L):
-        layers.append(dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H), wo=t(H, qd),
-                           ffn_norm=ones(H), w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F)))
+        lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H), wo=t(H, qd), ffn_norm=ones(H))
+        if E:
+            xd = cfg.get("expert_dtype", dt)
+            lw.update(n_experts=E, top_k=int(cfg["top_k"]), router=t(E, H, sig=cfg.get("router_sigma", sigma)),
+                      we_gate=t(E * F, H, xd), we_up=t(E * F, H, xd), we_down=t(E * H, F, xd))
+        else:
+            lw.update(w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F))
+        layers.append(lw)
     return dict(embed=t(V, H), final_norm=ones(H), lm_head=t(V, H), layers=layers)
