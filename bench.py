@@ -24,6 +24,9 @@ WORKLOADS = {
     # BASELINE configs[0] (the reference's CPU-runnable plumbing case), greedy
     "tiny_q8_0_k4_ctx256": dict(model="tiny_q8_0", ctx=256, k=4, temperature=0.0),
     "small_q4_k_k4_ctx256": dict(model="small_q4_k", ctx=256, k=4, temperature=0.8),
+    # BASELINE configs[3]: routed experts (MXFP4) + Q8_0 attention, chain k=8, greedy
+    "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(model="qwen3_30b_a3b", ctx=8192, k=8, temperature=0.0),
+    "moe_small_k8_ctx256": dict(model="moe_small", ctx=256, k=8, temperature=0.0),
 }
 
 
@@ -37,8 +40,18 @@ def algorithmic_bytes(cfg, ctx, m):
     from turbospark_amd import ffi
     H, F, V, L = cfg["hidden"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
     qd, kvd = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
-    rb = lambda rows, cols: rows * ffi.row_bytes(cfg["dtype"], cols)
-    per_layer = dict(qkv=rb(qd + 2 * kvd, H), wo=rb(H, qd), gate_up=rb(2 * F, H), down=rb(H, F))
+    rb = lambda rows, cols, dt=None: rows * ffi.row_bytes(cfg["dtype"] if dt is None else dt, cols)
+    E = cfg.get("n_experts", 0)
+    if E:
+        # routed experts: an expert's matrices are read once if any of the m rows chose it; with
+        # independent uniform routing the expected number of distinct experts per layer is
+        # E * (1 - (1 - k/E)^m)  (the union actually routed is not read back)
+        union = E * (1.0 - (1.0 - cfg["top_k"] / E) ** m)
+        xd = cfg.get("expert_dtype", cfg["dtype"])
+        per_layer = dict(qkv=rb(qd + 2 * kvd, H), wo=rb(H, qd), gate_up=int(union * rb(2 * F, H, xd)) + rb(E, H),
+                         down=int(union * rb(H, F, xd)))
+    else:
+        per_layer = dict(qkv=rb(qd + 2 * kvd, H), wo=rb(H, qd), gate_up=rb(2 * F, H), down=rb(H, F))
     head = rb(V, H)
     weights = L * sum(per_layer.values()) + head
     kv = L * (ctx + m) * kvd * 2 * 2
@@ -261,7 +274,9 @@ def main():
     eng.set_profile(False)
     dom = kern.get("gate_up", {})
     peak = 8000.0
-    roofline = dict(bound="hbm", kernel="k_gemm<Q4_K> gate/up (silu-mul epilogue)" if cfg["dtype"] == 12 else "k_gemm<Q8_0> gate/up",
+    roofline = dict(bound="hbm",
+                    kernel="router + grouped expert gate/up matmuls (expected expert union)" if cfg.get("n_experts")
+                    else "k_gemm<Q4_K> gate/up (silu-mul epilogue)" if cfg["dtype"] == 12 else "k_gemm<Q8_0> gate/up",
                     achieved=dom.get("GBps"), peak=peak, unit="GB/s",
                     frac=round((dom.get("GBps") or 0.0) / peak, 4),
                     traffic=MEASURED_TRAFFIC.get(args.workload),
@@ -283,7 +298,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16",
-        "dtype_detail": ("q4_k" if cfg["dtype"] == 12 else "q8_0") + " weight codes as exact f16 x f16 activations on MFMA, "
+        "dtype_detail": ("q4_k" if cfg["dtype"] == 12 else "q8_0") + (" + mxfp4 experts" if cfg.get("n_experts") else "") +
+                        " weight codes as exact f16 x f16 activations on MFMA, "
                         "f32 accumulate; f64 acceptance",
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,

@@ -576,14 +576,25 @@ __global__ __launch_bounds__(1024) void k_argmax(const uint16_t* target, int voc
     float best = -INFINITY;
     int idx = 0x7FFFFFFF;
     bool bad = false;
-    for (int v = threadIdx.x; v < vocab; v += 1024) {
-        const uint16_t b = p[v];
+    auto take = [&](uint16_t b, int v) {
         bad |= (b & 0x7C00u) == 0x7C00u;
         const float f = h2f(b);
         if (f > best || (f == best && v < idx)) {
             best = f;
             idx = v;
         }
+    };
+    if ((((uintptr_t)p) & 15) == 0) {  // eight logits per 16-byte load
+        const int n8 = vocab >> 3;
+        for (int i = threadIdx.x; i < n8; i += 1024) {
+            const uint4 q = ((const uint4*)p)[i];
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 8; j++) take((uint16_t)(w[j >> 1] >> (16 * (j & 1))), 8 * i + j);
+        }
+        for (int v = (n8 << 3) + threadIdx.x; v < vocab; v += 1024) take(p[v], v);
+    } else {
+        for (int v = threadIdx.x; v < vocab; v += 1024) take(p[v], v);
     }
     if (bad) atomicOr(err, 1);
     for (int o = 32; o > 0; o >>= 1) {

@@ -11,6 +11,7 @@
 // matmuls with a gathered activation operand.  The per-(row, slot) outputs are written apart and
 // the next residual kernel adds them in slot order, so the sum has the reference's order.
 #include <algorithm>
+#include <cstdlib>
 
 #include "gemm_core.h"
 
@@ -19,14 +20,16 @@ namespace tsv {
 namespace {
 
 // ---- router ---------------------------------------------------------------------------------
-// One workgroup.  Wave w routes rows w, w + 4, ...: the row's logits (split-K partials summed in
-// order) sit 'ne / 64' per lane; k rounds of a wave-wide arg-max (larger logit, then lower
-// index) pick the experts in rank order.  Then every expert's row list is built in row order.
-__global__ __launch_bounds__(256) void k_route(MoeRouteArgs a) {
-    __shared__ int s_sel[TSV_MAX_ROWS][8];
+// One workgroup, one wave per row: the row's logits (split-K partials summed in order) sit
+// 'ne / 64' per lane; k rounds of a wave-wide arg-max (larger logit, then lower index) pick the
+// experts in rank order.  Then one thread per (row, slot) pair decides whether its expert
+// appears here for the first time and, if so, lists every pair that shares it, in row order.
+__global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
+    __shared__ int s_sel[TSV_MAX_ROWS * 8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int M = a.vp->m, ne = a.n_experts, k = a.top_k;
-    for (int m = wave; m < M; m += 4) {
+    if (wave < M) {
+        const int m = wave;
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -38,12 +41,10 @@ __global__ __launch_bounds__(256) void k_route(MoeRouteArgs a) {
                 v[j] = s;
             }
         }
-        float top = 0.f, ex[8], sum = 0.f;
-        int sel[8];
+        float top = 0.f, sum = 0.f, my_ex = 0.f;
+        int my_sel = 0;
 #pragma unroll
         for (int r = 0; r < 8; r++) {
-            sel[r] = 0;
-            ex[r] = 0.f;
             if (r < k) {
                 float best = -INFINITY;
                 int bi = 0x7FFFFFFF;
@@ -62,52 +63,51 @@ __global__ __launch_bounds__(256) void k_route(MoeRouteArgs a) {
                     }
                 }
                 if (r == 0) top = best;
-                sel[r] = bi;
-                ex[r] = expf(best - top);
-                sum += ex[r];  // sequential in rank order, as `exps.iter().sum()`
+                const float ex = expf(best - top);
+                sum += ex;  // sequential in rank order, as `exps.iter().sum()`
+                if (lane == r) {  // lane r keeps slot r
+                    my_ex = ex;
+                    my_sel = bi;
+                }
 #pragma unroll
                 for (int j = 0; j < 4; j++)
                     if (lane + 64 * j == bi) v[j] = -INFINITY;
             }
         }
-        // lane r keeps slot r
-        float w = 0.f;
-        int e = 0;
-#pragma unroll
-        for (int r = 0; r < 8; r++)
-            if (r == lane) {
-                w = ex[r] / sum;
-                e = sel[r];
-            }
         if (lane < k) {
-            a.weights[m * 8 + lane] = w;
-            a.selected[m * 8 + lane] = e;
-            s_sel[m][lane] = e;
+            a.weights[m * 8 + lane] = my_ex / sum;
+            a.selected[m * 8 + lane] = my_sel;
+            s_sel[m * k + lane] = my_sel;
         }
     }
     __syncthreads();
-    // expert e's rows, ascending (thread e)
-    for (int e = threadIdx.x; e < ne; e += 256) {
-        int n = 0;
-        for (int m = 0; m < M; m++)
-            for (int r = 0; r < k; r++)
-                if (s_sel[m][r] == e) {
-                    a.rows[e * 16 + n] = m;
-                    a.slots[e * 16 + n] = r;
-                    n++;
-                }
-        a.count[e] = n;
-    }
+    const int j = threadIdx.x, np = M * k;
+    if (j >= np) return;
+    const int e = s_sel[j];
+    bool leader = true;
+    for (int i = 0; i < j; i++) leader &= s_sel[i] != e;
+    MoeGroup* g = a.groups + j;
+    int n = 0;
+    if (leader)
+        for (int i = j; i < np; i++)
+            if (s_sel[i] == e) {
+                g->rows[n] = i / k;
+                g->slots[n] = i - (i / k) * k;
+                n++;
+            }
+    g->expert = e;
+    g->cnt = n;
 }
 
 // ---- grouped expert matmul --------------------------------------------------------------------
 __device__ __forceinline__ float silu_moe(float x) { return x / (1.0f + __expf(-x)); }
 
-template <class F, int EPI, int NG>
-__device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, int e, int cnt, const int* rows, const int* slots,
-                                            float4v* red) {
+// One 64-row weight tile of expert `e` against up to four of the group's rows (r0 .. r0 + 3).
+template <class F, int EPI>
+__device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup& grp, int gi, int r0, float4v* red) {
+    constexpr int NG = 1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int tile = blockIdx.x;
+    const int tile = blockIdx.x, e = grp.expert, cnt = grp.cnt;
     const int per = (a.kchunks + nw - 1) / nw;
     const int c0 = min(wave * per, a.kchunks), nc = min(per, a.kchunks - c0);
     const uint8_t* wt = a.w + ((size_t)e * a.tiles_per_expert + tile) * a.kchunks * F::TILE_BYTES;
@@ -117,18 +117,14 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, int e, int cnt
     k.k64 = 0x64646464u;
     asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
 
-    // activation operand: gate/up reads the pass's rows this expert was chosen by (gathered); down
-    // reads the expert's own buffer, whose rows are already in the expert's order
-    const uint8_t* xbase = (const uint8_t*)a.xfrag + (EPI == EPI_SLOT ? (size_t)e * a.x_stride : 0);
+    // activation operand: gate/up gathers the pass's rows this expert was chosen by; down reads
+    // the group's own buffer, whose rows are already in the group's order
+    const uint8_t* xbase = (const uint8_t*)a.xfrag + (EPI == EPI_SLOT ? (size_t)gi * a.x_stride : 0);
     ActLoader<false> x(xbase, xbase + xfrag_sum_offset(a.k), lane);
-    if (EPI == EPI_SILU) {
-#pragma unroll
-        for (int g = 0; g < NG; g++) x.set_row(g, rows[min(4 * g + (lane & 3), cnt - 1)]);
-    }
+    const int mine = min(r0 + (lane & 3), cnt - 1);
+    x.set_row(0, EPI == EPI_SILU ? grp.rows[mine] : mine);
 
-    float4v acc[NG];
-#pragma unroll
-    for (int g = 0; g < NG; g++) acc[g] = float4v{0.f, 0.f, 0.f, 0.f};
+    float4v acc[NG] = {float4v{0.f, 0.f, 0.f, 0.f}};
     if (nc > 0) {
         Stage<F, NG> st[2];
         const int last = c0 + nc - 1;
@@ -156,80 +152,77 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, int e, int cnt
             if (c + s < nc) compute(st[s], k, acc);
     }
 
-    // fold the waves in wave order, then wave w finishes row groups w, w + nw, ...
-#pragma unroll
-    for (int g = 0; g < NG; g++) red[(wave * NG + g) * 64 + lane] = acc[g];
+    // fold the waves in wave order; wave 0 finishes
     __syncthreads();
-    for (int g = wave; g < NG; g += nw) {
-        float4v v = red[g * 64 + lane];
-        for (int w = 1; w < nw; w++) v += red[(w * NG + g) * 64 + lane];
-        if (EPI == EPI_SILU) {
-            // lanes 0..31: gate rows, lanes 32..63: up rows of the same 32 columns of this expert
-            const int col = tile * 32 + (lane & 31);
-            _Float16* out = (_Float16*)((uint8_t*)a.out + (size_t)e * a.out_stride);
-            float* sums = (float*)((uint8_t*)out + xfrag_sum_offset(a.n_out));
+    red[wave * 64 + lane] = acc[0];
+    __syncthreads();
+    if (wave != 0) return;
+    float4v v = red[lane];
+    for (int w = 1; w < nw; w++) v += red[w * 64 + lane];
+    if (EPI == EPI_SILU) {
+        // lanes 0..31: gate rows, lanes 32..63: up rows of the same 32 columns of this expert
+        const int col = tile * 32 + (lane & 31);
+        _Float16* out = (_Float16*)((uint8_t*)a.out + (size_t)gi * a.out_stride);
+        float* sums = (float*)((uint8_t*)out + xfrag_sum_offset(a.n_out));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float other = __shfl_xor(v[i], 32);
+            const float gate = lane < 32 ? v[i] : other, up = lane < 32 ? other : v[i];
+            const _Float16 h = (_Float16)(silu_moe(gate) * up);
+            float sum = (float)h;
+#pragma unroll
+            for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
+            const int b = r0 + i;  // the group's own row order
+            if (b < cnt && lane < 32) {
+                out[frag_index(col, b)] = h;
+                if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
+            }
+        }
+    } else {
+        const int n = tile * 64 + lane;
+        if (n < a.n_out) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const float other = __shfl_xor(v[i], 32);
-                const float gate = lane < 32 ? v[i] : other, up = lane < 32 ? other : v[i];
-                const _Float16 h = (_Float16)(silu_moe(gate) * up);
-                float sum = (float)h;
-#pragma unroll
-                for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
-                const int b = 4 * g + i;  // the expert's own row order
-                if (b < cnt && lane < 32) {
-                    out[frag_index(col, b)] = h;
-                    if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
-                }
-            }
-        } else {
-            const int n = tile * 64 + lane;
-            if (n < a.n_out) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int b = 4 * g + i;
-                    if (b < cnt) ((float*)a.out)[((size_t)slots[b] * 16 + rows[b]) * a.n_out + n] = v[i];
-                }
+                const int b = r0 + i;
+                if (b < cnt) ((float*)a.out)[((size_t)grp.slots[b] * 16 + grp.rows[b]) * a.n_out + n] = v[i];
             }
         }
     }
 }
 
-// grid: (tiles per expert, experts).  Experts nobody chose leave at once.
+// grid: (tiles per expert, rows x top_k groups).  Groups that repeat an earlier expert leave at
+// once.  An expert chosen by more than four rows (rare at these batch widths) is multiplied in
+// several sweeps of four rows; its tile then comes from L2.
 template <class F, int EPI>
 __global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
     extern __shared__ float4v red[];
-    __shared__ int s_rows[16], s_slots[16];
-    const int e = blockIdx.y;
-    const int cnt = a.count[e];
-    if (cnt == 0) return;
-    if (threadIdx.x < 16) {
-        s_rows[threadIdx.x] = a.rows[e * 16 + threadIdx.x];
-        s_slots[threadIdx.x] = a.slots[e * 16 + threadIdx.x];
-    }
+    __shared__ MoeGroup grp;
+    const int gi = blockIdx.y;
+    if (threadIdx.x < sizeof(MoeGroup) / 4) ((int32_t*)&grp)[threadIdx.x] = ((const int32_t*)(a.groups + gi))[threadIdx.x];
     __syncthreads();
-    if (cnt <= 4)
-        expert_tile<F, EPI, 1>(a, e, cnt, s_rows, s_slots, red);
-    else if (cnt <= 8)
-        expert_tile<F, EPI, 2>(a, e, cnt, s_rows, s_slots, red);
-    else
-        expert_tile<F, EPI, 4>(a, e, cnt, s_rows, s_slots, red);
+    if (grp.cnt == 0) return;
+    for (int r0 = 0; r0 < grp.cnt; r0 += 4) expert_tile<F, EPI>(a, grp, gi, r0, red);
 }
 
 template <class F, int EPI>
-int launch_moe_t(hipStream_t s, const MoeGemmArgs& a, int n_experts) {
-    const int nw = std::min(8, std::max(1, a.kchunks));
-    const size_t lds = (size_t)nw * 4 * 1024;
-    hipLaunchKernelGGL((k_moe_gemm<F, EPI>), dim3(a.tiles_per_expert, n_experts), dim3(64 * nw), lds, s, a);
+int launch_moe_t(hipStream_t s, const MoeGemmArgs& a, int n_groups) {
+    // waves per workgroup: each takes `cpw` K chunks of the tile
+    static const int cpw = [] {
+        const char* e = getenv("TSV_MOE_CPW");
+        return e ? std::max(1, atoi(e)) : 2;
+    }();
+    const int nw = std::min(8, std::max(1, (a.kchunks + cpw - 1) / cpw));
+    const size_t lds = (size_t)nw * 1024;
+    hipLaunchKernelGGL((k_moe_gemm<F, EPI>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
 
 template <int EPI>
-int launch_moe_f(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts) {
-    return fmt == FMT_Q4K   ? launch_moe_t<Q4K, EPI>(s, a, n_experts)
-           : fmt == FMT_Q80 ? launch_moe_t<Q80, EPI>(s, a, n_experts)
-                            : launch_moe_t<MX4, EPI>(s, a, n_experts);
+int launch_moe_f(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
+    return fmt == FMT_Q4K   ? launch_moe_t<Q4K, EPI>(s, a, n_groups)
+           : fmt == FMT_Q80 ? launch_moe_t<Q80, EPI>(s, a, n_groups)
+                            : launch_moe_t<MX4, EPI>(s, a, n_groups);
 }
 
 }  // namespace
@@ -239,17 +232,17 @@ int launch_route(hipStream_t s, const MoeRouteArgs& a) {
         set_error("moe: at most 256 experts and top-k between 1 and 8");
         return TSV_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(k_route, dim3(1), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_route, dim3(1), dim3(1024), 0, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
 
-int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts) {
-    return launch_moe_f<EPI_SILU>(s, fmt, a, n_experts);
+int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
+    return launch_moe_f<EPI_SILU>(s, fmt, a, n_groups);
 }
 
-int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts) {
-    return launch_moe_f<EPI_SLOT>(s, fmt, a, n_experts);
+int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
+    return launch_moe_f<EPI_SLOT>(s, fmt, a, n_groups);
 }
 
 }  // namespace tsv

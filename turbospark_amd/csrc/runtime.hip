@@ -48,7 +48,8 @@ struct tsv_ctx {
     // routed experts: routing tables, per-expert activation fragments, per-slot outputs
     int max_experts = 0;
     float* route_w = nullptr;
-    int32_t *route_sel = nullptr, *route_cnt = nullptr, *route_rows = nullptr, *route_slots = nullptr;
+    int32_t* route_sel = nullptr;
+    MoeGroup* route_groups = nullptr;
     uint8_t* frag_e = nullptr;
     size_t frag_e_stride = 0;
     float* moe_out = nullptr;
@@ -475,9 +476,7 @@ int launch_pass(tsv_ctx* c, int m) {
             ra2.vp = c->vp_dev;
             ra2.weights = c->route_w;
             ra2.selected = c->route_sel;
-            ra2.count = c->route_cnt;
-            ra2.rows = c->route_rows;
-            ra2.slots = c->route_slots;
+            ra2.groups = c->route_groups;
             MoeGemmArgs g1, g2;
             g1.w = L.gate_up.tiles;
             g1.tiles_per_expert = c->ffn / 32;
@@ -488,9 +487,8 @@ int launch_pass(tsv_ctx* c, int m) {
             g1.out = c->frag_e;
             g1.out_stride = c->frag_e_stride;
             g1.n_out = c->ffn;
-            g1.count = c->route_cnt;
-            g1.rows = c->route_rows;
-            g1.slots = c->route_slots;
+            g1.groups = c->route_groups;
+            const int n_groups = m * L.top_k;
             g2 = g1;
             g2.w = L.down.tiles;
             g2.tiles_per_expert = c->hidden / 64;
@@ -503,14 +501,19 @@ int launch_pass(tsv_ctx* c, int m) {
             g2.n_out = c->hidden;
             {
                 PROF(PC_GATEUP);
-                rc = launch_gemm(s, L.router, c->xf_a, c->partial, c->vp_dev, m, rsp, EPI_PARTIAL, L.n_experts, L.n_experts);
-                if (!rc) rc = launch_route(s, ra2);
-                if (!rc) rc = launch_moe_gate_up(s, L.gate_up.fmt, g1, L.n_experts);
+                rc = 0;
+                for (int rep = 0; rep < c->repeat[PC_GATEUP] && !rc; rep++) {
+                    rc = launch_gemm(s, L.router, c->xf_a, c->partial, c->vp_dev, m, rsp, EPI_PARTIAL, L.n_experts,
+                                     L.n_experts);
+                    if (!rc) rc = launch_route(s, ra2);
+                    if (!rc) rc = launch_moe_gate_up(s, L.gate_up.fmt, g1, n_groups);
+                }
             }
             if (rc) return rc;
             {
                 PROF(PC_DOWN);
-                rc = launch_moe_down(s, L.down.fmt, g2, L.n_experts);
+                rc = 0;
+                for (int rep = 0; rep < c->repeat[PC_DOWN] && !rc; rep++) rc = launch_moe_down(s, L.down.fmt, g2, n_groups);
             }
             if (rc) return rc;
             prev_partial = c->moe_out;
@@ -741,10 +744,8 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->partial, pneed * 4, true)) ||
         (c->max_experts &&
          ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, 16 * 8 * 4, true)) ||
-          (rc = dev_alloc(c, &c->route_cnt, (size_t)c->max_experts * 4, true)) ||
-          (rc = dev_alloc(c, &c->route_rows, (size_t)c->max_experts * 16 * 4, true)) ||
-          (rc = dev_alloc(c, &c->route_slots, (size_t)c->max_experts * 16 * 4, true)) ||
-          (rc = dev_alloc(c, &c->frag_e, (size_t)c->max_experts * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
+          (rc = dev_alloc(c, &c->route_groups, (size_t)TSV_MAX_ROWS * 8 * sizeof(MoeGroup), true)) ||
+          (rc = dev_alloc(c, &c->frag_e, (size_t)TSV_MAX_ROWS * 8 * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
           (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)))) || (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
         (rc = dev_alloc(c, &c->part_o, (size_t)c->nkv * c->nch * rows_max * c->hd * 4, true)) ||
         (rc = dev_alloc(c, &c->part_ml, (size_t)c->nkv * c->nch * rows_max * 2 * 4, true)) ||

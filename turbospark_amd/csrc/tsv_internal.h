@@ -105,29 +105,35 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
 int gemm_default_splits(const TiledW& w, int m);
 
 // ---- routed experts (moe.hip) -----------------------------------------------------------------
+// One routed expert of a pass: the rows that chose it (ascending) and the rank slot it has in
+// each.  Groups are indexed by the (row, slot) pair at which the expert first appears; pairs that
+// repeat an earlier expert hold cnt == 0, so a launch over rows x top_k groups touches every
+// chosen expert exactly once and nothing else.
+struct MoeGroup {
+    int32_t expert, cnt;
+    int32_t rows[16], slots[16];
+};
 struct MoeRouteArgs {
     const float* logits;  // router matmul partials [splits][16][ld]
     int splits, ld, n_experts, top_k;
     const VerifyParams* vp;
-    float* weights;   // [16][8] softmax over the selected logits, rank order
+    float* weights;     // [16][8] softmax over the selected logits, rank order
     int32_t* selected;  // [16][8] expert ids, rank order
-    int32_t* count;     // [n_experts] rows that chose the expert
-    int32_t* rows;      // [n_experts][16] those rows, ascending
-    int32_t* slots;     // [n_experts][16] the rank slot the expert has in that row
+    MoeGroup* groups;   // [16 * 8]
 };
 struct MoeGemmArgs {
     const uint8_t* w;      // tiled weights of all experts, tiles_per_expert x kchunks tiles each
     int tiles_per_expert, kchunks, k;
-    const void* xfrag;     // gate/up: the pass's activation fragments; down: per-expert fragments
-    size_t x_stride;       // down: bytes between experts' fragment buffers
-    void* out;             // gate/up: per-expert fragments of silu(gate) * up; down: float [8 slots][16][n_out]
+    const void* xfrag;     // gate/up: the pass's activation fragments; down: per-group fragments
+    size_t x_stride;       // down: bytes between groups' fragment buffers
+    void* out;             // gate/up: per-group fragments of silu(gate) * up; down: float [8 slots][16][n_out]
     size_t out_stride;
     int n_out;             // gate/up: expert FFN width; down: hidden
-    const int32_t *count, *rows, *slots;
+    const MoeGroup* groups;
 };
 int launch_route(hipStream_t s, const MoeRouteArgs& a);
-int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts);
-int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_experts);
+int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
+int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 
 // ---- per-XCD fused layer kernels ----------------------------------------------------------
 // Counters of the XCD-local barriers.  rank_ctr / bar_ctr: one word per XCD, 64 words apart.

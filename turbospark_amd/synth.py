@@ -23,6 +23,10 @@ CONFIGS = {
     "moe_small": dict(n_layers=2, hidden=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=256,
                       n_experts=16, top_k=4, vocab=4096, rms_eps=1e-6, rope_theta=1000000.0,
                       dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08, norm_jitter=0.25),
+    # Qwen3-30B-A3B shape: 128 experts, top-8, MXFP4 experts, Q8_0 attention / router / head
+    "qwen3_30b_a3b": dict(n_layers=48, hidden=2048, n_q_heads=32, n_kv_heads=4, head_dim=128, ffn=768,
+                          n_experts=128, top_k=8, vocab=151936, rms_eps=1e-6, rope_theta=1000000.0,
+                          dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08),
     # Llama-3-8B shape
     "llama3_8b_q4_k": dict(n_layers=32, hidden=4096, n_q_heads=32, n_kv_heads=8, head_dim=128,
                            ffn=14336, vocab=128256, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
