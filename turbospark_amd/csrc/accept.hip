@@ -560,10 +560,123 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             res->next = dec.stopped ? -1 : token;
             res->draw_step = dec.draw_step;
             res->path_len = dec.accepted + 1;
-            for (int i = 0; i <= dec.accepted; i++) res->path[i] = i;
+            for (int i = 0; i <= dec.accepted; i++) res->path[i] = kind == 2 ? tokens_out[i] : i;
             res->min_margin = margin;
             res->error = *err;
         }
+    }
+}
+
+// ---- sampled acceptance over a draft tree ---------------------------------------------------
+// The reference has no multi-branch rejection sampler (speculative.rs:390-392 keeps tree rounds
+// greedy); this follows the oracle's definition: at node `at`, with p the target distribution of
+// row `at` and q the distribution its children were drawn from, the children are tried in slot
+// order -- child x is accepted when r * q(x) <= p(x) for a fresh uniform r; a rejection replaces
+// p by normalise(max(p - q, 0)) (kept as is when that mass is below 1e-12) -- and when no child
+// survives the next token is drawn from the p that is left.  No stop / budget bookkeeping.
+// One workgroup walks the tree; p and q live as dense f64 rows in the work area (job 0: slot 1
+// holds p, which is also what the final draw's histogram and in-bin walk read; slot 0 is scratch
+// for the residual; job 1 slot 0 holds q).
+__global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, const uint16_t* draft,
+                                                       const AcceptParams* app, double* scratch, double* work,
+                                                       unsigned long long* hist, Decision* dec_out,
+                                                       int32_t* path_out) {
+    __shared__ RowStat s_p, s_q;
+    __shared__ double red[16];
+    __shared__ int s_accept;
+    __shared__ double s_margin;
+    const AcceptParams& ap = *app;
+    const int tid = threadIdx.x, wave = tid >> 6;
+    const int vocab = ap.vocab, m = ap.m;
+    const double inv_t = 1.0 / ap.temperature;
+    Layout L = layout(scratch);
+    double* pc = work + vocab;          // job 0, slot 1
+    double* pr = work;                  // job 0, slot 0
+    double* qa = work + 2 * (long)vocab;  // job 1, slot 0
+    unsigned long long* hr = hist + 65536;
+    uint64_t ds = ap.draw_step;
+    int at = 0, plen = 1;
+    if (tid == 0) {
+        path_out[0] = 0;
+        s_margin = 1.0;
+    }
+    for (;;) {
+        if (wave == 0) {
+            const RowStat st = load_stat(L, at);
+            if (tid == 0) s_p = st;
+        } else if (wave == 1) {
+            const RowStat st = load_stat(L, m + at);
+            if ((tid & 63) == 0) s_q = st;
+        }
+        __syncthreads();
+        const uint16_t* lp = target + (long)at * vocab;
+        const uint16_t* lq = draft + (long)at * vocab;
+        for (int v = tid; v < vocab; v += 1024) {
+            pc[v] = prob_of(lp[v], s_p, inv_t);
+            qa[v] = prob_of(lq[v], s_q, inv_t);
+        }
+        __threadfence_block();
+        __syncthreads();
+        int hit = -1;
+        for (int s = 1; s < m && hit < 0; s++) {
+            if (ap.parent[s] != at) continue;
+            if (tid == 0) {
+                const int32_t x = ap.feed[s];
+                const double r = unit_draw(ap.seed, ds);
+                const double px = pc[x], qx = qa[x];
+                double mg = s_margin;
+                fold_margin(mg, r * qx, px);
+                s_margin = mg;
+                s_accept = r * qx <= px;
+            }
+            ds += 1;
+            __syncthreads();
+            if (s_accept) {
+                hit = s;
+                break;
+            }
+            // residual: p <- normalise(max(p - q, 0))
+            double acc = 0.0;
+            for (int v = tid; v < vocab; v += 1024) {
+                const double mv = fmax(pc[v] - qa[v], 0.0);
+                pr[v] = mv;
+                acc += mv;
+            }
+            const double total = block_sum_f64(acc, red);
+            if (total >= 1e-12)
+                for (int v = tid; v < vocab; v += 1024) pc[v] = pr[v] / total;
+            __threadfence_block();
+            __syncthreads();
+        }
+        if (hit >= 0) {
+            if (tid == 0) path_out[plen] = hit;
+            plen += 1;
+            at = hit;
+            __syncthreads();
+            continue;
+        }
+        // nothing accepted below `at`: the next token is drawn from what is left of p
+        const uint16_t* lpk = target + (long)at * vocab;
+        for (int v = tid; v < vocab; v += 1024) {
+            const double mv = pc[v];
+            if (mv > 0.0) atomicAdd(hr + bin_addr(rank_key(lpk[v])), (unsigned long long)(mv * FIX));
+        }
+        if (tid < NSEG * NSUB) L.segtot[tid] = tid == 0 ? 1.0 : 0.0;  // the masses are already normalised
+        if (tid == 0) {
+            Decision d;
+            d.job.mode = 2;
+            d.job.row_p = at;
+            d.job.row_q = 0;
+            d.job.u = unit_draw(ap.seed, ds);
+            d.accepted = plen - 1;
+            d.committed = plen - 1;
+            d.stopped = 0;
+            d.pad = 0;
+            d.draw_step = ds + 1;
+            d.margin = s_margin;
+            dec_out[0] = d;
+        }
+        return;
     }
 }
 
@@ -690,8 +803,20 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
         return TSV_OK;
     }
     if (ap.tree) {
-        set_error("sampled acceptance over a tree is not built yet (the reference has none: speculative.rs:390-392)");
-        return TSV_ERR_UNSUPPORTED;
+        // statistics of the m target rows and the m rows the children were drawn from
+        const int rows2 = 2 * ap.m;
+        const double it = 1.0 / ap.temperature;
+        int32_t* path = (int32_t*)sc.counters + 32;
+        hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err,
+                           (unsigned long long*)sc.hist, 2 * 65536);
+        hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
+        hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, it);
+        hipLaunchKernelGGL(k_tree_sampled, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                           (unsigned long long*)sc.hist, decisions(sc), path);
+        hipLaunchKernelGGL(k_pick, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                           (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);
+        TSV_HIP(hipGetLastError());
+        return TSV_OK;
     }
     const int rows = ap.m + ap.k;
     const double inv_t = 1.0 / ap.temperature;

@@ -1009,6 +1009,10 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
             set_error("accept: a sampled round needs the drafter's logits");
             return TSV_ERR_INVALID;
         }
+        if (r->parent && (r->n_stop > 0 || r->max_new_tokens > 0)) {
+            set_error("accept: sampled acceptance over a tree takes no stop tokens or budget");
+            return TSV_ERR_UNSUPPORTED;
+        }
         if ((rc = stage_draft(c, r->draft_logits, r->parent ? r->m : r->m - 1, &draft))) return rc;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));  // pinned parameter block is about to be rewritten
