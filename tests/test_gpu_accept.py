@@ -27,8 +27,13 @@ def _same(res, want, base):
     assert res.kv_position == base + want["committed"] + 1
 
 
-@pytest.mark.parametrize("temperature", [0.8, 1.0, 0.3])
-def test_sampled_chain_rounds_match_the_oracle_bit_for_bit(temperature):
+TRUNCATIONS = [dict(), dict(top_k=40), dict(top_p=0.9), dict(min_p=0.02), dict(top_k=50, top_p=0.95, min_p=0.01),
+               dict(top_k=1), dict(top_p=0.3), dict(top_k=256, top_p=0.999)]
+
+
+@pytest.mark.parametrize("temperature,kw", [(0.8, TRUNCATIONS[0]), (1.0, TRUNCATIONS[0]), (0.3, TRUNCATIONS[0])] +
+                         [(0.8, t) for t in TRUNCATIONS[1:]] + [(1.3, TRUNCATIONS[4])])
+def test_sampled_chain_rounds_match_the_oracle_bit_for_bit(temperature, kw):
     import turbospark_amd as ts
     cfg, gpu, prompt = _setup()
     V, k = cfg["vocab"], 4
@@ -44,11 +49,24 @@ def test_sampled_chain_rounds_match_the_oracle_bit_for_bit(temperature):
     history = history[:-1]
     for rnd in range(24):
         seed = 1000 + rnd
-        gcfg = ts.shaping(temperature, seed=seed)
-        ocfg = ob.shaping(temperature, seed=seed)
+        gcfg = ts.shaping(temperature, seed=seed, **kw)
+        ocfg = ob.shaping(temperature, seed=seed, **kw)
         draft = rng.standard_normal((k, V)).astype(np.float16)
         if rnd % 3 == 0:
             draft[0, :] = 0  # a flat drafter row
+        if rnd % 4 == 1:
+            draft[1] = np.round(draft[1] * 2) / 2  # many equal logits: the cut falls inside a rank bin
+        if rnd % 2 == 1:
+            # a drafter that resembles the target: its row i is the target's own row after the first i
+            # proposals, plus noise, so that truncated candidate sets overlap and proposals get accepted
+            here = gpu.checkpoint()
+            tok = nxt
+            for i in range(k):
+                row = gc.f16(gpu.produce(tok, gpu.position))
+                draft[i] = (row + rng.standard_normal(V) * 0.3).astype(np.float16)
+                one, _ = gpu.draft_chain(draft[i:i + 1], gcfg, draw_step + i)
+                tok = int(one[0])
+            gpu.rollback(here)
         # draft half on the device vs the oracle
         props, ds1 = gpu.draft_chain(draft, gcfg, draw_step)
         oprops, ods1 = ob.draft_chain(draft, ocfg, history + [nxt], len(history), draw_step)
@@ -67,7 +85,8 @@ def test_sampled_chain_rounds_match_the_oracle_bit_for_bit(temperature):
         assert gpu.position == len(history)
     print("accepted per round:", accepted_hist, " min margin:", min(margins))
     assert min(margins) > 1e-9          # no decision was anywhere near flipping
-    assert len(set(accepted_hist)) > 1  # the rounds really exercised different outcomes
+    if kw.get("top_k") != 1:
+        assert len(set(accepted_hist)) > 1  # the rounds really exercised different outcomes
 
 
 def test_identical_drafter_is_always_accepted_and_the_bonus_is_a_p_draw():
@@ -152,8 +171,9 @@ def test_greedy_tree_round_walks_compacts_and_truncates():
     assert gc.logit_error(nxt[None], ref[None]) <= 2e-3
 
 
-@pytest.mark.parametrize("name,temperature", [("tiny_q8_0", 1.0), ("small_q4_k", 0.8)])
-def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature):
+@pytest.mark.parametrize("name,temperature,kw", [("tiny_q8_0", 1.0, {}), ("small_q4_k", 0.8, {}),
+                                                 ("tiny_q8_0", 1.0, dict(top_k=64, top_p=0.9))])
+def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature, kw):
     """Multi-branch rejection over a 16-node tree.  The rule is the oracle's own (the reference
     keeps tree rounds greedy, speculative.rs:390-392), so this pins the device against the
     oracle only: parity with the reference is unpinned for this mode."""
@@ -165,9 +185,13 @@ def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature):
     parent = [-1, 0, 0, 0, 0, 1, 5, 6, 2, 8, 9, 3, 11, 12, 4, 14]
     rng = np.random.default_rng(17)
     depths, margins = [], []
+    row0 = gc.f16(gpu.verify([9], base))[0]
+    gpu.rollback(point)
+    likely = np.argsort(-row0)[:8]
     for rnd in range(12):
         feed = [int(t) for t in rng.integers(0, V, 16)]
         feed[0] = 9
+        feed[1:5] = [int(t) for t in rng.choice(likely, 4, replace=False)]  # children inside a truncated set
         logits = gpu.verify_tree(feed, parent, base)
         # drafter rows: the target's own rows plus noise, so that p(x) / q(x) scatters around one
         noise = rng.standard_normal((16, V)) * (0.25 if rnd % 2 else 1.5)
@@ -175,7 +199,7 @@ def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature):
         if rnd == 3:
             draft = gc.f16(logits).copy()      # q == p: the first child of every node is accepted
         seed = 500 + rnd
-        gcfg, ocfg = ts.shaping(temperature, seed=seed), ob.shaping(temperature, seed=seed)
+        gcfg, ocfg = ts.shaping(temperature, seed=seed, **kw), ob.shaping(temperature, seed=seed, **kw)
         res = gpu.accept(feed, base, gcfg, parent=parent, draft_logits=draft, draw_step=7 * rnd)
         want = ob.tree_round_sampled(logits, draft, feed, parent, ocfg, history=list(prompt), draw_step=7 * rnd)
         assert res.path == want["path"], (rnd, res, want)
@@ -189,7 +213,8 @@ def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature):
         gpu.rollback(point)
     print("accepted depth per round:", depths, " min margin:", min(margins))
     assert min(margins) > 1e-9
-    assert len(set(depths)) > 2
+    if not kw:  # (random deeper nodes fall outside both truncated sets, where 0 <= 0 accepts)
+        assert len(set(depths)) > 2
     # the compacted cache continues like a chain that fed the accepted path
     feed = [int(t) for t in rng.integers(0, V, 16)]
     logits = gpu.verify_tree(feed, parent, base)
@@ -213,7 +238,8 @@ def test_refusals_by_name():
     cfg, gpu, prompt = _setup()
     base = gpu.position
     with pytest.raises(TsvError, match="not built"):
-        gpu.verify_accept([1, 2], base, ts.shaping(0.8, top_k=40, seed=1), draft_logits=np.zeros((1, cfg["vocab"]), np.float16))
+        gpu.verify_accept([1, 2], base, ts.shaping(0.8, repetition_penalty=1.1, seed=1),
+                          draft_logits=np.zeros((1, cfg["vocab"]), np.float16))
     with pytest.raises(TsvError, match="seed"):
         gpu.verify_accept([1, 2], base, ts.shaping(0.8), draft_logits=np.zeros((1, cfg["vocab"]), np.float16))
     with pytest.raises(TsvError, match="drafter"):

@@ -30,25 +30,29 @@ constexpr double FIX = 4611686018427387904.0;  // 2^62
 
 struct RowStat {
     double mx, sum, total, top;
+    int32_t cut_key, cut_idx;  // last surviving candidate in rank order (truncation off: 65536, INT_MAX)
+};
+struct Cut {
+    int32_t key, idx;
 };
 
 // Scratch layout inside AcceptScratch::stats (doubles):
-//   [0, 4*32)                         RowStat per distribution row
-//   pmax / psum / ptot partials follow
+//   [0, 4*32)                         truncation cut per distribution row (8 bytes each)
+//   pmax / psum / ptot partials follow, then the residual pieces and the decisions
 struct Layout {
-    RowStat* stat;
     double* pmax;  // [rows][NSEG]
     double* psum;
     double* ptot;
     double* segtot;  // [jobs][NSEG * NSUB] residual mass per piece of a segment
+    Cut* cut;        // [rows] truncation cut
 };
 __host__ __device__ inline Layout layout(double* base) {
     Layout l;
-    l.stat = (RowStat*)base;
     l.pmax = base + 4 * MAX_DIST_ROWS;
     l.psum = l.pmax + MAX_DIST_ROWS * NSEG;
     l.ptot = l.psum + MAX_DIST_ROWS * NSEG;
     l.segtot = l.ptot + MAX_DIST_ROWS * NSEG;
+    l.cut = (Cut*)base;
     return l;
 }
 
@@ -94,8 +98,17 @@ __device__ __forceinline__ uint32_t bin_addr(uint32_t key) {
     return (key & 0xF000u) | ((key & 63u) << 6) | ((key >> 6) & 63u);
 }
 
+// Whether candidate v (logit `bits`) is inside the row's truncated candidate set: the set is a
+// prefix of the rank order (logit descending, index ascending), so it is described by its last
+// member.
+__device__ __forceinline__ bool survives(uint16_t bits, int v, const RowStat& s) {
+    const int key = (int)rank_key(bits);
+    return key < s.cut_key || (key == s.cut_key && v <= s.cut_idx);
+}
+
 // choose.rs:296-319 for one candidate of a row whose statistics are known
-__device__ __forceinline__ double prob_of(uint16_t bits, const RowStat& s, double inv_t) {
+__device__ __forceinline__ double prob_of(uint16_t bits, int v, const RowStat& s, double inv_t) {
+    if (!survives(bits, v, s)) return 0.0;
     const double e = exp((double)h2f(bits) - s.mx);
     const double p = e / s.sum;
     return pow(p / s.top, inv_t) / s.total;
@@ -165,7 +178,11 @@ __global__ __launch_bounds__(256) void k_row_max(const uint16_t* target, const u
     for (int o = 32; o > 0; o >>= 1) d = fmax(d, shfl_xor_t(d, o));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = d;
     __syncthreads();
-    if (threadIdx.x == 0) layout(scratch).pmax[row * NSEG + seg] = fmax(fmax(red[0], red[1]), fmax(red[2], red[3]));
+    if (threadIdx.x == 0) {
+        Layout L = layout(scratch);
+        L.pmax[row * NSEG + seg] = fmax(fmax(red[0], red[1]), fmax(red[2], red[3]));
+        if (seg == 0) L.cut[row] = Cut{65536, 0x7FFFFFFF};  // no truncation until a cut is computed
+    }
 }
 
 __global__ __launch_bounds__(256) void k_row_sum(const uint16_t* target, const uint16_t* draft, int m,
@@ -179,10 +196,7 @@ __global__ __launch_bounds__(256) void k_row_sum(const uint16_t* target, const u
     double acc = 0.0;
     for (int v = v0 + threadIdx.x; v < v1; v += 256) acc += exp((double)h2f(p[v]) - mx);
     acc = block_sum_f64(acc, red);
-    if (threadIdx.x == 0) {
-        L.psum[row * NSEG + seg] = acc;
-        if (seg == 0) L.stat[row].mx = mx;
-    }
+    if (threadIdx.x == 0) L.psum[row * NSEG + seg] = acc;
 }
 
 __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const uint16_t* draft, int m,
@@ -195,19 +209,18 @@ __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const
     const double top = 1.0 / sum;  // the arg-max candidate has e == exp(0) == 1
     const uint16_t* p = row_ptr(target, draft, m, vocab, row);
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    RowStat cs;
+    cs.cut_key = L.cut[row].key;
+    cs.cut_idx = L.cut[row].idx;
     double acc = 0.0;
     for (int v = v0 + threadIdx.x; v < v1; v += 256) {
-        const double e = exp((double)h2f(p[v]) - mx);
+        const uint16_t b = p[v];
+        if (!survives(b, v, cs)) continue;
+        const double e = exp((double)h2f(b) - mx);
         acc += pow((e / sum) / top, inv_t);
     }
     acc = block_sum_f64(acc, red);
-    if (threadIdx.x == 0) {
-        L.ptot[row * NSEG + seg] = acc;
-        if (seg == 0) {
-            L.stat[row].sum = sum;
-            L.stat[row].top = top;
-        }
-    }
+    if (threadIdx.x == 0) L.ptot[row * NSEG + seg] = acc;
 }
 
 // Called by one whole wave: the finished statistics of `row`, identical in every lane.
@@ -218,13 +231,15 @@ __device__ RowStat load_stat(const Layout& L, int row) {
     s.sum = wave_sum_f64(L.psum[row * NSEG + lane]);
     s.top = 1.0 / s.sum;
     s.total = wave_sum_f64(L.ptot[row * NSEG + lane]);
+    s.cut_key = L.cut[row].key;
+    s.cut_idx = L.cut[row].idx;
     return s;
 }
 
 __device__ __forceinline__ void fold_margin(double& margin, double a, double b) {
     const double scale = fmax(fabs(a), fabs(b));
-    const double rel = scale > 0.0 ? fabs(a - b) / scale : 0.0;
-    margin = fmin(margin, rel);
+    if (scale == 0.0) return;  // two exact zeros (a candidate outside both truncated sets): nothing can flip
+    margin = fmin(margin, fabs(a - b) / scale);
 }
 
 // TokenSink::commit restricted to what a token-id interface can see
@@ -253,8 +268,8 @@ __device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t*
     for (int i = 0; i < ap.k; i++) {
         const int32_t x = ap.feed[i + 1];
         const RowStat sp = stats[i], sq = stats[ap.m + i];
-        const double px = prob_of(target[(long)i * ap.vocab + x], sp, inv_t);
-        const double qx = prob_of(draft[(long)i * ap.vocab + x], sq, inv_t);
+        const double px = prob_of(target[(long)i * ap.vocab + x], x, sp, inv_t);
+        const double qx = prob_of(draft[(long)i * ap.vocab + x], x, sq, inv_t);
         const double r = unit_draw(ap.seed, ds);
         ds += 1;
         fold_margin(d.margin, r * qx, px);
@@ -334,12 +349,12 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     double racc = 0.0;
     for (int v = v0 + sub * 256 + threadIdx.x; v < v1; v += 256 * NSUB) {
         const uint16_t b = lp[v];
-        const double pv = prob_of(b, sp, inv_t);
+        const double pv = prob_of(b, v, sp, inv_t);
         const uint32_t key = bin_addr(rank_key(b));
         wp[v] = pv;
-        atomicAdd(hp + key, (unsigned long long)(pv * FIX));
+        if (pv > 0.0) atomicAdd(hp + key, (unsigned long long)(pv * FIX));
         if (job.mode == 2) {
-            const double mv = fmax(pv - prob_of(lq[v], sq, inv_t), 0.0);
+            const double mv = fmax(pv - prob_of(lq[v], v, sq, inv_t), 0.0);
             wr[v] = mv;
             racc += mv;
             if (mv > 0.0) atomicAdd(hr + key, (unsigned long long)(mv * FIX));
@@ -377,6 +392,214 @@ __device__ __forceinline__ void scan_chunk(const uint16_t* lp, int v0, int v1, u
             const uint32_t bits = (w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
             if (bits == want || (zero_bin && bits == 0x8000u)) on_match(g + j);
         }
+    }
+}
+
+// ---- truncation of the candidate set (top-k, top-p, min-p) ---------------------------------
+// choose.rs:111-228 / truncation.rs:79-236: candidates are ranked by softmax mass descending, ties
+// by ascending index; top-k keeps the first k, top-p the shortest prefix whose cumulative
+// `e / sum` reaches top_p, min-p those with e >= min_p * e_top.  All three keep a PREFIX of the
+// rank order, so the surviving set is described by its last member (rank bin, index); it is found
+// from per-row histograms over the 65536 rank bins (candidates per bin, fixed-point mass per
+// bin) instead of a sort, and the one bin the cut falls into is resolved in index order.
+__global__ __launch_bounds__(256) void k_trunc_clear(unsigned long long* tmass, uint32_t* tcount, int rows) {
+    const size_t n = (size_t)rows * 65536;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        tmass[i] = 0;
+        tcount[i] = 0;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_trunc_hist(const uint16_t* target, const uint16_t* draft, int m, int vocab,
+                                                    double* scratch, unsigned long long* tmass, uint32_t* tcount,
+                                                    int want_mass) {
+    const int row = blockIdx.y, seg = blockIdx.x, lane = threadIdx.x & 63;
+    Layout L = layout(scratch);
+    const double mx = wave_max_f64(L.pmax[row * NSEG + lane]);
+    const double sum = wave_sum_f64(L.psum[row * NSEG + lane]);
+    const uint16_t* p = row_ptr(target, draft, m, vocab, row);
+    const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    unsigned long long* hm = tmass + (size_t)row * 65536;
+    uint32_t* hc = tcount + (size_t)row * 65536;
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const uint16_t b = p[v];
+        const uint32_t key = bin_addr(rank_key(b));
+        unsigned long long mass = 0;
+        if (want_mass) mass = (unsigned long long)((exp((double)h2f(b) - mx) / sum) * FIX);
+        // a run of equal logits (a flat row) would serialise on one address: one lane adds for all
+        const uint32_t first = __builtin_amdgcn_readfirstlane(key);
+        const unsigned long long active = __ballot(1);
+        if (__ballot(key == first) == active) {
+            if (lane == (int)__builtin_ctzll(active)) {
+                const int n = __builtin_popcountll(active);
+                atomicAdd(hc + key, (uint32_t)n);
+                if (want_mass) atomicAdd(hm + key, mass * (unsigned long long)n);
+            }
+        } else {
+            atomicAdd(hc + key, 1u);
+            if (want_mass && mass) atomicAdd(hm + key, mass);
+        }
+    }
+}
+
+// fp16 bits whose rank key is `key` (inverse of rank_key; the zero bin maps to +0)
+__device__ __forceinline__ uint32_t key_bits(int key) {
+    const uint32_t asc = 0xFFFFu - (uint32_t)key;
+    return (asc & 0x8000u) ? (asc & 0x7FFFu) : (~asc & 0xFFFFu);
+}
+
+// Exclusive prefix of a 64-bit value over the 1024 threads of a workgroup; *total gets the sum.
+__device__ unsigned long long block_scan_u64(unsigned long long loc, unsigned long long* wsum,
+                                             unsigned long long* total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned long long inc = loc;
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t lo = __shfl_up((uint32_t)inc, o), hi = __shfl_up((uint32_t)(inc >> 32), o);
+        const unsigned long long up = ((unsigned long long)hi << 32) | lo;
+        if (lane >= o) inc += up;
+    }
+    __syncthreads();
+    if (lane == 63) wsum[wave] = inc;
+    __syncthreads();
+    unsigned long long wbase = 0, t = 0;
+    for (int i = 0; i < 16; i++) {
+        if (i < wave) wbase += wsum[i];
+        t += wsum[i];
+    }
+    *total = t;
+    return wbase + inc - loc;
+}
+
+// One workgroup per distribution row.
+__global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, const uint16_t* draft,
+                                                    const AcceptParams* app, int m, double* scratch,
+                                                    const unsigned long long* tmass, const uint32_t* tcount,
+                                                    AcceptResult* res) {
+    __shared__ unsigned long long wsum[16];
+    __shared__ unsigned long long s_before_p;
+    __shared__ int s_bin_k, s_j_k, s_bin_p, s_cnt_p, s_minp_key, s_bin, s_j, s_idx;
+    __shared__ double s_margin;
+    const AcceptParams& ap = *app;
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int vocab = ap.vocab;
+    Layout L = layout(scratch);
+    const double mx = wave_max_f64(L.pmax[row * NSEG + lane]);
+    const double sum = wave_sum_f64(L.psum[row * NSEG + lane]);
+    const uint32_t* cmine = tcount + (size_t)row * 65536 + (tid >> 6) * 4096 + (tid & 63);
+    const unsigned long long* mmine = tmass + (size_t)row * 65536 + (tid >> 6) * 4096 + (tid & 63);
+    if (tid == 0) {
+        s_bin_k = s_bin_p = s_minp_key = s_bin = -1;
+        s_idx = 0x7FFFFFFF;
+        s_margin = 1.0;
+    }
+    __syncthreads();
+    unsigned long long total, total_p = 0;
+    if (ap.top_k > 0) {
+        unsigned long long loc = 0;
+#pragma unroll 16
+        for (int i = 0; i < 64; i++) loc += cmine[i * 64];
+        const unsigned long long excl = block_scan_u64(loc, wsum, &total);
+        const unsigned long long K = (unsigned long long)ap.top_k;
+        if (excl < K && K <= excl + loc) {
+            unsigned long long c = excl;
+            for (int i = 0; i < 64; i++) {
+                const unsigned long long cv = cmine[i * 64];
+                if (K <= c + cv) {
+                    s_bin_k = tid * 64 + i;
+                    s_j_k = (int)(K - c);
+                    break;
+                }
+                c += cv;
+            }
+        }
+    }
+    if (ap.has_top_p) {
+        unsigned long long loc = 0;
+#pragma unroll 16
+        for (int i = 0; i < 64; i++) loc += mmine[i * 64];
+        const unsigned long long excl = block_scan_u64(loc, wsum, &total);
+        total_p = total;
+        const unsigned long long tgt = (unsigned long long)(ap.top_p * FIX);
+        if (excl < tgt && tgt <= excl + loc) {
+            unsigned long long c = excl;
+            for (int i = 0; i < 64; i++) {
+                const unsigned long long mv = mmine[i * 64];
+                if (mv > 0 && tgt <= c + mv) {
+                    s_bin_p = tid * 64 + i;
+                    s_before_p = c;
+                    s_cnt_p = (int)cmine[i * 64];
+                    break;
+                }
+                c += mv;
+            }
+        }
+    }
+    if (ap.has_min_p) {
+        int best = -1;
+        for (int i = 0; i < 64; i++) {
+            const int key = tid * 64 + i;
+            const uint32_t bits = key_bits(key);
+            if ((bits & 0x7C00u) == 0x7C00u) continue;  // no finite logit has this key
+            if (exp((double)h2f((uint16_t)bits) - mx) >= ap.min_p) best = key;  // e_top == exp(0) == 1
+        }
+        if (best >= 0) atomicMax(&s_minp_key, best);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int bin = s_bin_k, j = s_bin_k >= 0 ? s_j_k : 0;
+        if (s_bin_p >= 0) {
+            // how many candidates of the bin it takes to reach top_p: each carries the same mass
+            const double pm = exp((double)h2f((uint16_t)key_bits(s_bin_p)) - mx) / sum;
+            const double before = (double)s_before_p / FIX;
+            long jp = (long)ceil((ap.top_p - before) / pm);
+            jp = jp < 1 ? 1 : jp;
+            while (jp > 1 && before + (double)(jp - 1) * pm >= ap.top_p) jp--;
+            while (jp < s_cnt_p && before + (double)jp * pm < ap.top_p) jp++;
+            jp = jp > s_cnt_p ? s_cnt_p : jp;
+            double mg = 1.0;
+            fold_margin(mg, before + (double)jp * pm, ap.top_p);
+            if (jp > 1 || s_before_p > 0) fold_margin(mg, before + (double)(jp - 1) * pm, ap.top_p);
+            s_margin = mg;
+            if (bin < 0 || s_bin_p < bin || (s_bin_p == bin && jp < j)) {
+                bin = s_bin_p;
+                j = (int)jp;
+            }
+        }
+        if (ap.has_top_p && s_bin_p < 0) {  // the cumulative mass never reached top_p: everything ranked survives
+            double mg = 1.0;
+            fold_margin(mg, (double)total_p / FIX, ap.top_p);
+            s_margin = mg;
+        }
+        s_bin = bin;
+        s_j = j;
+    }
+    __syncthreads();
+    const int bin = s_bin, j = s_j;
+    if (bin >= 0 && j < (int)tcount[(size_t)row * 65536 + bin_addr(bin)]) {
+        // the j-th candidate of the bin in index order
+        const uint16_t* lp = row_ptr(target, draft, m, vocab, row);
+        const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = min(tid * per, vocab), v1 = min(v0 + per, vocab);
+        const bool vec = ((uintptr_t)lp & 15) == 0;
+        const uint32_t want = key_bits(bin);
+        const bool zero_bin = want == 0;
+        int n = 0;
+        scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int) { n++; });
+        const unsigned long long excl = block_scan_u64((unsigned long long)n, wsum, &total);
+        if ((int)excl < j && j <= (int)excl + n) {
+            int c = (int)excl;
+            scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int v) {
+                c++;
+                if (c == j) s_idx = v;
+            });
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        Cut cut{65536, 0x7FFFFFFF};
+        if (bin >= 0) cut = Cut{bin, s_idx};
+        if (ap.has_min_p && s_minp_key >= 0 && s_minp_key < cut.key) cut = Cut{s_minp_key, 0x7FFFFFFF};
+        L.cut[row] = cut;
+        atomicMin((unsigned long long*)&res->min_margin, __builtin_bit_cast(unsigned long long, s_margin));
     }
 }
 
@@ -561,7 +784,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             res->draw_step = dec.draw_step;
             res->path_len = dec.accepted + 1;
             for (int i = 0; i <= dec.accepted; i++) res->path[i] = kind == 2 ? tokens_out[i] : i;
-            res->min_margin = margin;
+            atomicMin((unsigned long long*)&res->min_margin, __builtin_bit_cast(unsigned long long, margin));
             res->error = *err;
         }
     }
@@ -612,8 +835,8 @@ __global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, c
         const uint16_t* lp = target + (long)at * vocab;
         const uint16_t* lq = draft + (long)at * vocab;
         for (int v = tid; v < vocab; v += 1024) {
-            pc[v] = prob_of(lp[v], s_p, inv_t);
-            qa[v] = prob_of(lq[v], s_q, inv_t);
+            pc[v] = prob_of(lp[v], v, s_p, inv_t);
+            qa[v] = prob_of(lq[v], v, s_q, inv_t);
         }
         __threadfence_block();
         __syncthreads();
@@ -791,6 +1014,20 @@ static Decision* decisions(const AcceptScratch& sc) {
     return (Decision*)(sc.stats + 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG * NSUB);
 }
 
+// Between the softmax sums and the reweighting totals: the truncation cut of every row.
+static void launch_trunc(hipStream_t s, const uint16_t* target, const uint16_t* draft, int m, int rows,
+                         const AcceptParams* ap_dev, const AcceptParams& ap, const AcceptScratch& sc) {
+    if (ap.top_k == 0 && !ap.has_top_p && !ap.has_min_p) return;
+    unsigned long long* tm = (unsigned long long*)sc.tmass;
+    if (ap.top_k != 0 || ap.has_top_p) {
+        hipLaunchKernelGGL(k_trunc_clear, dim3(64 * rows), dim3(256), 0, s, tm, sc.tcount, rows);
+        hipLaunchKernelGGL(k_trunc_hist, dim3(NSEG, rows), dim3(256), 0, s, target, draft, m, ap.vocab, sc.stats, tm,
+                           sc.tcount, ap.has_top_p);
+    }
+    hipLaunchKernelGGL(k_trunc_cut, dim3(rows), dim3(1024), 0, s, target, draft, ap_dev, m, sc.stats, tm, sc.tcount,
+                       sc.result);
+}
+
 int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
                   const AcceptParams& ap, const AcceptScratch& sc) {
     int32_t* err = (int32_t*)sc.counters;
@@ -810,6 +1047,7 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
         hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err,
                            (unsigned long long*)sc.hist, 2 * 65536);
         hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
+        launch_trunc(s, target, draft, ap.m, rows2, ap_dev, ap, sc);
         hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, it);
         hipLaunchKernelGGL(k_tree_sampled, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                            (unsigned long long*)sc.hist, decisions(sc), path);
@@ -823,6 +1061,7 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
     hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err,
                        (unsigned long long*)sc.hist, 2 * 65536);
     hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
+    launch_trunc(s, target, draft, ap.m, rows, ap_dev, ap, sc);
     hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, inv_t);
     hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, 1, NSUB), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), 0);
@@ -847,6 +1086,7 @@ int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams*
     hipLaunchKernelGGL(k_row_max, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, err,
                        (unsigned long long*)sc.hist, ap.k * 2 * 65536);
     hipLaunchKernelGGL(k_row_sum, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats);
+    launch_trunc(s, draft, draft, 0, ap.k, ap_dev, ap, sc);
     hipLaunchKernelGGL(k_row_total, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, inv_t);
     hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, ap.k, NSUB), dim3(256), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), 1);

@@ -241,9 +241,8 @@ int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
         return TSV_ERR_INVALID;
     }
     if (sampled_supported_only &&
-        (s.top_k != 0 || s.has_top_p || s.has_min_p || s.repetition_penalty != 1.0 || s.presence_penalty != 0.0 ||
-         s.frequency_penalty != 0.0)) {
-        set_error("device acceptance: top-k / top-p / min-p / penalties are not built; use temperature only");
+        (s.repetition_penalty != 1.0 || s.presence_penalty != 0.0 || s.frequency_penalty != 0.0)) {
+        set_error("device acceptance: repetition / presence / frequency penalties are not built");
         return TSV_ERR_UNSUPPORTED;
     }
     return TSV_OK;
@@ -758,6 +757,8 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->sc.work, (size_t)16 * 2 * c->vocab * 8, true)) ||
         (rc = dev_alloc(c, &c->sc.hist, (size_t)16 * 2 * 65536 * 8, true)) ||
         (rc = dev_alloc(c, &c->sc.counters, 64 * 4, true)) ||
+        (rc = dev_alloc(c, &c->sc.tmass, (size_t)32 * 65536 * 8, true)) ||
+        (rc = dev_alloc(c, &c->sc.tcount, (size_t)32 * 65536 * 4, true)) ||
         (rc = dev_alloc(c, &c->sc.result, sizeof(AcceptResult), true)))
         return fail(rc);
     {
@@ -960,6 +961,14 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
 
 namespace {
 
+void fill_truncation(AcceptParams* ap, const tsv_shaping& sh) {
+    ap->top_k = (int32_t)sh.top_k;
+    ap->has_top_p = sh.has_top_p != 0;
+    ap->top_p = sh.top_p;
+    ap->has_min_p = sh.has_min_p != 0;
+    ap->min_p = sh.min_p;
+}
+
 int fill_accept(tsv_ctx* c, const tsv_round* r, AcceptParams* ap) {
     std::memset(ap, 0, sizeof *ap);
     ap->m = r->m;
@@ -979,6 +988,7 @@ int fill_accept(tsv_ctx* c, const tsv_round* r, AcceptParams* ap) {
     for (int i = 0; i < r->n_stop; i++) ap->stop_tokens[i] = r->stop_tokens[i];
     ap->temperature = r->shaping.temperature;
     ap->seed = r->shaping.seed;
+    fill_truncation(ap, r->shaping);
     ap->draw_step = r->draw_step;
     ap->generated = r->generated;
     ap->max_new_tokens = r->max_new_tokens;
@@ -1095,6 +1105,7 @@ extern "C" int32_t tsv_draft_chain(tsv_ctx* c, const uint16_t* draft_logits, int
     ap->sampled = sh->temperature != 0.0;
     ap->temperature = sh->temperature;
     ap->seed = sh->seed;
+    fill_truncation(ap, *sh);
     ap->draw_step = *draw_step;
     TSV_HIP(hipMemcpyAsync(c->ap_dev, ap, sizeof *ap, hipMemcpyHostToDevice, c->stream));
     if ((rc = launch_draft_chain(c->stream, draft, c->ap_dev, *ap, c->sc, c->tok_dev))) return rc;

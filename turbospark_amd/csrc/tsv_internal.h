@@ -228,6 +228,9 @@ struct AcceptParams {
     int32_t stop_tokens[16];
     double temperature;
     uint64_t seed, draw_step, generated, max_new_tokens;
+    // truncation of the candidate set (crates/selection/src/choose.rs:111-228): 0 / false = off
+    int32_t top_k, has_top_p, has_min_p, pad0;
+    double top_p, min_p;
 };
 struct AcceptResult {
     int32_t accepted, committed, next, stopped;
@@ -242,6 +245,8 @@ struct AcceptScratch {
     double* work;        // [16 jobs][2][vocab] candidate masses (p, residual)
     uint64_t* hist;      // [16 jobs][2][65536] fixed-point mass per rank bin; a round clears what it uses first
     uint32_t* counters;  // 64 words: error flag, greedy arg-max per row
+    uint64_t* tmass;     // [32 rows][65536] fixed-point softmax mass per rank bin (top-p cut)
+    uint32_t* tcount;    // [32 rows][65536] candidates per rank bin (top-k / top-p cut)
     AcceptResult* result;  // device
 };
 size_t accept_stats_doubles();
