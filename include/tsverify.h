@@ -60,6 +60,17 @@ typedef struct {
      * (n_experts * hidden) x ffn.  `ffn` of the model description is the expert width. */
     int32_t n_experts, top_k;
     tsv_tensor router, we_gate, we_up, we_down;
+    /* gpt-oss layer additions (crates/runtime/src/families/gptoss/mod.rs:11-23); data == NULL when
+     * absent.  bq/bk/bv: projection biases, added BEFORE the rotation (gptoss/attn.rs:88-101); bo:
+     * output-projection bias; sinks: one attention sink logit per q head, joining the softmax
+     * maximum and denominator only (crates/compute/src/attention.rs:29-137); router_bias:
+     * n_experts values added to the router logits before the top-k (gptoss/moe.rs:82-87);
+     * be_gate / be_up (n_experts x ffn, added before the activation) and be_down (n_experts x
+     * hidden): per-expert biases (crates/gpu/src/shaders/moe_gguf.metal:592-600).  All f32 / f16 /
+     * bf16 vectors.  window > 0: a row sees only the last `window` positions of its sequence
+     * (gptoss/attn.rs:120-137); it must exceed TSV_MAX_ROWS. */
+    tsv_tensor bq, bk, bv, bo, sinks, router_bias, be_gate, be_up, be_down;
+    int32_t window, reserved;
 } tsv_layer;
 
 typedef struct {
@@ -68,6 +79,15 @@ typedef struct {
     const float* rope_factors;             /* NULL, or head_dim/2 llama-3 per-pair divisors */
     tsv_tensor embed, final_norm, lm_head; /* lm_head.data NULL: tied to embed */
     const tsv_layer* layers;
+    /* NULL, or head_dim/2 explicit per-pair rotation frequencies (a YaRN table from
+     * tsv_yarn_frequencies; overrides rope_theta / rope_factors), and the magnitude scale that
+     * multiplies cos and sin (<= 0 means 1): crates/compute/src/rope.rs:286-372. */
+    const float* rope_freqs;
+    float rope_mscale;
+    /* act_alpha > 0 selects gpt-oss's clamped SwiGLU for the routed experts,
+     * (min(g, limit) / (1 + exp(-alpha * min(g, limit)))) * (clamp(u, -limit, limit) + 1)
+     * (crates/gpu/src/shaders/moe_gguf.metal:528-556), instead of silu(g) * u. */
+    float act_alpha, act_limit;
 } tsv_model_desc;
 
 typedef struct tsv_ctx tsv_ctx;
@@ -184,6 +204,10 @@ int32_t tsv_draft_chain(tsv_ctx* ctx, const uint16_t* draft_logits, int32_t k,
 /* ---- install-time helpers (host) --------------------------------------------- */
 /* The reference's quantize-on-install encoders (q8_0.rs:56-77, q4_k.rs:126-204). */
 int64_t tsv_row_bytes(int32_t dtype, int64_t cols);
+/* yarn_frequencies (crates/compute/src/rope.rs:324-372): rotary_dim/2 per-pair frequencies and
+ * the magnitude scale 1 + 0.1 ln(factor); factor <= 0 gives the unscaled table and scale 1. */
+int32_t tsv_yarn_frequencies(int32_t rotary_dim, float base, float factor, int64_t original_context,
+                             float beta_fast, float beta_slow, float* freqs, float* mscale);
 int32_t tsv_quantize_rows(int32_t dtype, const float* src, int64_t rows, int64_t cols, void* dst);
 /* Seeded synthetic tensor: rows x cols of N(0, sigma) from a counter-based generator
  * keyed by (seed, stream), quantized to dtype row by row (the random-init installs of
@@ -233,10 +257,12 @@ int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us);
 /* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
  * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache
  * slot base+i and sees [0, base) plus the slots of its root path (parent NULL: chain).
+ * window > 0 keeps the last `window` positions of each row's sequence; sinks (nullable): one f32
+ * logit per q head (crates/compute/src/attention.rs:29-137).
  * out: m x nq x hd fp16.  (The per-kernel parity hook of crates/gpu/tests/attention_tree_parity.rs.) */
 int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
                       int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
-                      uint16_t* out);
+                      int32_t window, const float* sinks, uint16_t* out);
 
 #ifdef __cplusplus
 }

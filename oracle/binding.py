@@ -75,11 +75,13 @@ class Tensor(C.Structure):
 
 LAYER_TENSORS = ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up", "w_down")
 LAYER_MOE_TENSORS = ("router", "we_gate", "we_up", "we_down")
+LAYER_GPTOSS_TENSORS = ("bq", "bk", "bv", "bo", "sinks", "router_bias", "be_gate", "be_up", "be_down")
 
 
 class Layer(C.Structure):
     _fields_ = ([(n, Tensor) for n in LAYER_TENSORS] + [("n_experts", C.c_int32), ("top_k", C.c_int32)] +
-                [(n, Tensor) for n in LAYER_MOE_TENSORS])
+                [(n, Tensor) for n in LAYER_MOE_TENSORS] + [(n, Tensor) for n in LAYER_GPTOSS_TENSORS] +
+                [("window", C.c_int32)])
 
 
 class ModelDesc(C.Structure):
@@ -92,6 +94,8 @@ class ModelDesc(C.Structure):
         ("round_kv_f16", C.c_int32), ("threads", C.c_int32),
         ("embed", Tensor), ("final_norm", Tensor), ("lm_head", Tensor),
         ("layers", C.POINTER(Layer)),
+        ("rope_freqs", C.POINTER(C.c_float)), ("rope_mscale", C.c_float),
+        ("act_alpha", C.c_float), ("act_limit", C.c_float),
     ]
 
 
@@ -118,6 +122,7 @@ def lib():
         L.tso_mxfp4_scale.restype = C.c_float
         L.tso_silu.argtypes = [C.c_float]
         L.tso_silu.restype = C.c_float
+        L.tso_swiglu_oai.restype = C.c_float
         L.tso_mix.argtypes = [C.c_uint64]
         L.tso_mix.restype = C.c_uint64
         L.tso_derive_step_value.argtypes = [C.c_uint64, C.c_uint64]
@@ -221,6 +226,26 @@ def rope_neox_freqs(x, num_tokens, num_heads, head_dim, rotated_pairs, position,
     lib().tso_rope_neox_freqs(_p(x), num_tokens, num_heads, head_dim, rotated_pairs,
                               C.c_int64(position), _p(freqs))
     return x
+
+
+def yarn_frequencies(rotary_dim, base, factor, original_context, beta_fast, beta_slow):
+    f = np.empty(rotary_dim // 2, np.float32)
+    ms = C.c_float()
+    lib().tso_yarn_frequencies(rotary_dim, C.c_float(base), C.c_float(factor), C.c_int64(original_context),
+                               C.c_float(beta_fast), C.c_float(beta_slow), _p(f), C.byref(ms))
+    return f, float(ms.value)
+
+
+def rope_neox_freqs_scaled(x, num_tokens, num_heads, head_dim, rotated_pairs, position, freqs, mscale):
+    x = np.ascontiguousarray(x, np.float32).copy()
+    freqs = np.ascontiguousarray(freqs, np.float32)
+    lib().tso_rope_neox_freqs_scaled(_p(x), num_tokens, num_heads, head_dim, rotated_pairs,
+                                     C.c_int64(position), _p(freqs), C.c_float(mscale))
+    return x
+
+
+def swiglu_oai(gate, up, alpha, limit):
+    return float(lib().tso_swiglu_oai(C.c_float(gate), C.c_float(up), C.c_float(alpha), C.c_float(limit)))
 
 
 def llama3_rope_factors(rotary_dim, base, factor, low, high, original_context):
@@ -405,10 +430,11 @@ class Model:
         n = cfg["n_layers"]
         self._layers = (Layer * n)()
         for i, lw in enumerate(weights["layers"]):
-            for name in LAYER_TENSORS + LAYER_MOE_TENSORS:
+            for name in LAYER_TENSORS + LAYER_MOE_TENSORS + LAYER_GPTOSS_TENSORS:
                 setattr(self._layers[i], name, _tensor(lw.get(name)))
             self._layers[i].n_experts = int(lw.get("n_experts", 0))
             self._layers[i].top_k = int(lw.get("top_k", 0))
+            self._layers[i].window = int(lw.get("window", 0))
         d = ModelDesc()
         for key in ("n_layers", "hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab",
                     "max_context"):
@@ -420,6 +446,13 @@ class Model:
         if cfg.get("rope_factors") is not None:
             self._factors = np.ascontiguousarray(cfg["rope_factors"], np.float32)
             d.rope_factors = self._factors.ctypes.data_as(C.POINTER(C.c_float))
+        self._freqs = None
+        if cfg.get("rope_freqs") is not None:
+            self._freqs = np.ascontiguousarray(cfg["rope_freqs"], np.float32)
+            d.rope_freqs = self._freqs.ctypes.data_as(C.POINTER(C.c_float))
+        d.rope_mscale = cfg.get("rope_mscale", 0.0)
+        d.act_alpha = cfg.get("act_alpha", 0.0)
+        d.act_limit = cfg.get("act_limit", 0.0)
         d.round_kv_f16 = int(round_kv_f16)
         d.threads = threads
         d.embed = _tensor(weights["embed"])

@@ -93,6 +93,14 @@ std::vector<float> norm_weight(const tso_tensor& t) {
 
 inline float round_f16(float x) { return tso_f16_to_f32(tso_f32_to_f16(x)); }
 
+// y[m][i] += bias[i] for a one-row tensor of any dtype (absent: nothing)
+void add_bias(const tso_tensor& b, float* y, int m_rows, int n) {
+    if (!b.data) return;
+    std::vector<float> bias = norm_weight(b);
+    for (int m = 0; m < m_rows; m++)
+        for (int i = 0; i < n; i++) y[(size_t)m * n + i] += bias[i];
+}
+
 }  // namespace
 
 extern "C" tso_model* tso_model_create(const tso_model_desc* desc) {
@@ -108,12 +116,17 @@ extern "C" tso_model* tso_model_create(const tso_model_desc* desc) {
         m->k[l].assign((size_t)(desc->max_context * stride), 0.0f);
         m->v[l].assign((size_t)(desc->max_context * stride), 0.0f);
     }
-    if (desc->rope_factors) {
+    if (desc->rope_freqs) {
+        m->rope_freqs.assign(desc->rope_freqs, desc->rope_freqs + desc->head_dim / 2);
+        m->d.rope_freqs = nullptr;
+        m->d.rope_factors = nullptr;
+    } else if (desc->rope_factors) {
         m->rope_freqs.resize(desc->head_dim / 2);
         tso_rope_frequencies_with_factors(desc->head_dim, desc->rope_theta, desc->rope_factors,
                                           m->rope_freqs.data());
         m->d.rope_factors = nullptr;
     }
+    if (!(m->d.rope_mscale > 0.0f)) m->d.rope_mscale = 1.0f;
     return m;
 }
 
@@ -190,6 +203,10 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
         gemm_rows(ly.wq, xn.data(), M, q.data(), T);
         gemm_rows(ly.wk, xn.data(), M, kk.data(), T);
         gemm_rows(ly.wv, xn.data(), M, vv.data(), T);
+        // families/gptoss/attn.rs:88-101: the projection biases, before the rotation
+        add_bias(ly.bq, q.data(), M, qd);
+        add_bias(ly.bk, kk.data(), M, kvd);
+        add_bias(ly.bv, vv.data(), M, kvd);
         if (ly.q_norm.data) {  // per-head q/k RMSNorm (families/llama/state.rs:344-347)
             std::vector<float> qw = norm_weight(ly.q_norm), kw = norm_weight(ly.k_norm);
             std::vector<float> tmp(hd);
@@ -211,8 +228,10 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
         for (int m = 0; m < M; m++) {
             int64_t pos = base + depth[m];
             if (!mdl->rope_freqs.empty()) {
-                tso_rope_neox_freqs(&q[(size_t)m * qd], 1, nq, hd, hd / 2, pos, mdl->rope_freqs.data());
-                tso_rope_neox_freqs(&kk[(size_t)m * kvd], 1, nkv, hd, hd / 2, pos, mdl->rope_freqs.data());
+                tso_rope_neox_freqs_scaled(&q[(size_t)m * qd], 1, nq, hd, hd / 2, pos, mdl->rope_freqs.data(),
+                                           d.rope_mscale);
+                tso_rope_neox_freqs_scaled(&kk[(size_t)m * kvd], 1, nkv, hd, hd / 2, pos,
+                                           mdl->rope_freqs.data(), d.rope_mscale);
             } else {
                 tso_rope_neox(&q[(size_t)m * qd], 1, nq, hd, hd / 2, pos, d.rope_theta);
                 tso_rope_neox(&kk[(size_t)m * kvd], 1, nkv, hd, hd / 2, pos, d.rope_theta);
@@ -225,21 +244,31 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
                 vd[i] = d.round_kv_f16 ? round_f16(vv[(size_t)m * kvd + i]) : vv[(size_t)m * kvd + i];
             }
         }
+        std::vector<float> sinks;
+        if (ly.sinks.data) sinks = norm_weight(ly.sinks);
+        const float* sk = sinks.empty() ? nullptr : sinks.data();
 #pragma omp parallel for num_threads(T) schedule(static)
         for (int m = 0; m < M; m++) {
             if (!parent) {
-                tso_causal_attention(&q[(size_t)m * qd], kc, vc, hd, nq, nkv, base + m + 1, 0,
-                                     d.attn_scale, nullptr, &att[(size_t)m * qd]);
+                // window: families/gptoss/attn.rs:120-137 (kv_start = seq_len - window, saturating)
+                tso_causal_attention(&q[(size_t)m * qd], kc, vc, hd, nq, nkv, base + m + 1, ly.window,
+                                     d.attn_scale, sk, &att[(size_t)m * qd]);
             } else {
                 int64_t path[64];
                 int n = 0;
                 for (int s = m; s >= 0; s = parent[s]) path[n++] = base + s;
                 for (int i = 0; i < n / 2; i++) std::swap(path[i], path[n - 1 - i]);
-                tso_attention_core(&q[(size_t)m * qd], kc, vc, hd, nq, nkv, 0, base, path, n,
-                                   d.attn_scale, nullptr, &att[(size_t)m * qd]);
+                // the row's sequence is the committed prefix followed by its root path; a window
+                // keeps the last `window` members of that sequence
+                int64_t seq_len = base + n, kv_start = 0;
+                if (ly.window > 0 && seq_len > ly.window) kv_start = seq_len - ly.window;
+                int skip = kv_start > base ? (int)(kv_start - base) : 0;
+                tso_attention_core(&q[(size_t)m * qd], kc, vc, hd, nq, nkv, std::min(kv_start, base), base,
+                                   path + skip, n - skip, d.attn_scale, sk, &att[(size_t)m * qd]);
             }
         }
         gemm_rows(ly.wo, att.data(), M, proj.data(), T);
+        add_bias(ly.bo, proj.data(), M, H);
         for (size_t i = 0; i < (size_t)M * H; i++) x[i] = x[i] + proj[i];
 
         std::vector<float> wf = norm_weight(ly.ffn_norm);
@@ -251,18 +280,29 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
             const int E = ly.n_experts, K = ly.top_k;
             std::vector<float> rl((size_t)M * E);
             gemm_rows(ly.router, xn.data(), M, rl.data(), T);
+            add_bias(ly.router_bias, rl.data(), M, E);  // families/gptoss/moe.rs:82-87: before the top-k
+            std::vector<float> routed(H);
             for (int m = 0; m < M; m++) {
                 int sel[8];
                 float w[8];
                 route_topk(&rl[(size_t)m * E], E, K, sel, w, &mdl->route_margin);
+                // families/llama/moe.rs:193-198: the routed sum starts from zero, is accumulated in
+                // rank order, and is then added to the stream
+                std::fill(routed.begin(), routed.end(), 0.0f);
                 for (int s = 0; s < K; s++) {
                     const int e = sel[s];
                     gemm_rows(row_slice(ly.we_gate, (int64_t)e * F, F), &xn[(size_t)m * H], 1, gate.data(), T);
                     gemm_rows(row_slice(ly.we_up, (int64_t)e * F, F), &xn[(size_t)m * H], 1, up.data(), T);
-                    for (int i = 0; i < F; i++) gate[i] = tso_silu(gate[i]) * up[i];
+                    add_bias(row_slice(ly.be_gate, e, 1), gate.data(), 1, F);  // moe_gguf.metal:592-600
+                    add_bias(row_slice(ly.be_up, e, 1), up.data(), 1, F);
+                    for (int i = 0; i < F; i++)
+                        gate[i] = d.act_alpha > 0.0f ? tso_swiglu_oai(gate[i], up[i], d.act_alpha, d.act_limit)
+                                                     : tso_silu(gate[i]) * up[i];
                     gemm_rows(row_slice(ly.we_down, (int64_t)e * H, H), gate.data(), 1, proj.data(), T);
-                    for (int i = 0; i < H; i++) x[(size_t)m * H + i] += w[s] * proj[i];
+                    add_bias(row_slice(ly.be_down, e, 1), proj.data(), 1, H);
+                    for (int i = 0; i < H; i++) routed[i] += w[s] * proj[i];
                 }
+                for (int i = 0; i < H; i++) x[(size_t)m * H + i] += routed[i];
             }
         } else {
             gemm_rows(ly.w_gate, xn.data(), M, gate.data(), T);

@@ -58,6 +58,57 @@ extern "C" void tso_rope_neox_freqs(float* x, int num_tokens, int num_heads, int
     rotate_pairs(x, num_tokens, num_heads, head_dim, rotated_pairs, c.data(), s.data());
 }
 
+extern "C" void tso_rope_neox_freqs_scaled(float* x, int num_tokens, int num_heads, int head_dim,
+                                           int rotated_pairs, int64_t position, const float* freqs,
+                                           float mscale) {
+    float position_f = (float)position;
+    std::vector<float> c(rotated_pairs), s(rotated_pairs);
+    for (int i = 0; i < rotated_pairs; i++) {
+        float angle = position_f * freqs[i];
+        c[i] = std::cos(angle) * mscale;
+        s[i] = std::sin(angle) * mscale;
+    }
+    rotate_pairs(x, num_tokens, num_heads, head_dim, rotated_pairs, c.data(), s.data());
+}
+
+// crates/compute/src/rope.rs:296-372
+static float yarn_corr_dim(int n_dims, int64_t n_ctx_orig, float n_rot, float base) {
+    return (float)n_dims * std::log((float)n_ctx_orig / (n_rot * 2.0f * 3.14159265358979323846f)) /
+           (2.0f * std::log(base));
+}
+extern "C" void tso_yarn_frequencies(int rotary_dim, float base, float factor, int64_t original_context,
+                                     float beta_fast, float beta_slow, float* freqs, float* mscale) {
+    const int pairs = rotary_dim / 2;
+    const bool active = factor > 0.0f;
+    const float freq_scale = active ? 1.0f / factor : 1.0f;
+    float low = 0.0f, high = 0.0f;
+    if (active) {
+        float start = std::floor(yarn_corr_dim(rotary_dim, original_context, beta_fast, base));
+        float end = std::ceil(yarn_corr_dim(rotary_dim, original_context, beta_slow, base));
+        low = std::fmax(start, 0.0f);
+        high = std::fmin(end, (float)rotary_dim - 1.0f);
+    }
+    for (int p = 0; p < pairs; p++) {
+        int i0 = 2 * p;
+        float extrap = std::pow(base, -((float)i0) / (float)rotary_dim);
+        if (!active) {
+            freqs[p] = extrap;
+            continue;
+        }
+        float y = ((float)i0 / 2.0f - low) / std::fmax(high - low, 0.001f);
+        float mix = 1.0f - std::fmin(std::fmax(y, 0.0f), 1.0f);
+        freqs[p] = extrap * (freq_scale * (1.0f - mix) + mix);
+    }
+    *mscale = active ? 1.0f + 0.1f * std::log(factor) : 1.0f;
+}
+
+// crates/gpu/src/shaders/moe_gguf.metal:528-556
+extern "C" float tso_swiglu_oai(float gate, float up, float alpha, float limit) {
+    float x = std::fmin(gate, limit);
+    float y = std::fmin(std::fmax(up, -limit), limit);
+    return (x / (1.0f + std::exp(-alpha * x))) * (y + 1.0f);
+}
+
 // crates/compute/src/rope.rs:390-439
 extern "C" int tso_llama3_rope_factors(int rotary_dim, double base, double factor,
                                        double low_freq_factor, double high_freq_factor,

@@ -78,6 +78,15 @@ void tso_rope_neox_freqs(float* x, int num_tokens, int num_heads, int head_dim, 
 int tso_llama3_rope_factors(int rotary_dim, double base, double factor, double low_freq_factor,
                             double high_freq_factor, double original_context, float* out);
 void tso_rope_frequencies_with_factors(int rotary_dim, float base, const float* factors, float* out);
+/* crates/compute/src/rope.rs:324-372 (YaRN): per-pair frequencies and the magnitude scale. */
+void tso_yarn_frequencies(int rotary_dim, float base, float factor, int64_t original_context,
+                          float beta_fast, float beta_slow, float* freqs, float* mscale);
+/* The table rotation with a magnitude scale on cos and sin (crates/runtime/src/families/gptoss/
+ * attn.rs:104-118 binds crates/gpu's rope_neox_freqs with state.rope_mscale). */
+void tso_rope_neox_freqs_scaled(float* x, int num_tokens, int num_heads, int head_dim,
+                                int rotated_pairs, int64_t position, const float* freqs, float mscale);
+/* crates/gpu/src/shaders/moe_gguf.metal:528-556 (ggml's swiglu_oai). */
+float tso_swiglu_oai(float gate, float up, float alpha, float limit);
 /* window <= 0: full; sinks NULL: none; scale <= 0: 1/sqrt(head_dim). */
 void tso_causal_attention(const float* q, const float* k, const float* v, int head_dim, int nq,
                           int nkv, int64_t seq_len, int64_t window, float scale, const float* sinks,
@@ -175,6 +184,13 @@ typedef struct {
      * we_gate / we_up (n_experts * ffn) x hidden, we_down (n_experts * hidden) x ffn, stacked */
     int32_t n_experts, top_k;
     tso_tensor router, we_gate, we_up, we_down;
+    /* gpt-oss additions (families/gptoss/mod.rs:11-23); every data pointer may be NULL:
+     * projection biases added before the rotation (attn.rs:88-101) / after the output projection,
+     * one attention sink per q head, router bias added before the top-k (moe.rs:82-87), per-expert
+     * biases n_experts x ffn (gate, up; added before the activation) and n_experts x hidden (down).
+     * window > 0: the row sees only the last `window` positions of its sequence. */
+    tso_tensor bq, bk, bv, bo, sinks, router_bias, be_gate, be_up, be_down;
+    int32_t window;
 } tso_layer;
 
 typedef struct {
@@ -185,6 +201,9 @@ typedef struct {
     int32_t threads;                       /* OpenMP threads for the row loops; 1 = scalar reference */
     tso_tensor embed, final_norm, lm_head; /* lm_head.data NULL => tied to embed */
     const tso_layer* layers;
+    const float* rope_freqs; /* NULL, or head_dim/2 explicit per-pair frequencies (YaRN table) */
+    float rope_mscale;       /* multiplies cos and sin; <= 0 means 1 */
+    float act_alpha, act_limit; /* act_alpha > 0: gpt-oss clamped SwiGLU instead of silu(g) * u */
 } tso_model_desc;
 
 typedef struct tso_model tso_model;

@@ -30,7 +30,7 @@ def test_struct_layouts_match_the_header_sizes():
     import ctypes as C
     from turbospark_amd import ffi
     assert C.sizeof(ffi.Tensor) == 32
-    assert C.sizeof(ffi.Layer) == 11 * 32 + 8 + 4 * 32
+    assert C.sizeof(ffi.Layer) == 11 * 32 + 8 + 4 * 32 + 9 * 32 + 8
     assert C.sizeof(ffi.Shaping) == 80
     assert C.sizeof(ffi.RoundResultC) == 4 * 4 + 8 + 17 * 4 + 4 + 8 + 8
 

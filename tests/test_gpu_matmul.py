@@ -23,7 +23,9 @@ def _case(dtype, rows, cols, seed):
 
 
 @pytest.mark.parametrize("dtype,rows,cols", [(12, 64, 512), (12, 48, 2048), (8, 64, 512), (8, 32, 1408),
-                                             (39, 64, 512), (39, 48, 2048), (39, 200, 768)])
+                                             (39, 64, 512), (39, 48, 2048), (39, 200, 768),
+                                             (39, 64, 576), (39, 96, 2880),      # MXFP4 rows ending inside a 256-chunk
+                                             (30, 64, 512), (30, 40, 576), (30, 130, 2880)])  # bf16
 def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, rows, cols, 31)
@@ -43,7 +45,7 @@ def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
         assert np.array_equal(got[0], first), m
 
 
-@pytest.mark.parametrize("dtype", [12, 8, 39])
+@pytest.mark.parametrize("dtype", [12, 8, 39, 30])
 def test_split_k_changes_nothing_but_rounding_and_is_deterministic(dtype):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, 32, 2048, 77)

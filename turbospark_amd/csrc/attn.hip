@@ -40,21 +40,31 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
     const VerifyParams* vp = a.vp;
     const int M = vp->m, base = vp->base, kvlen = base + M;
     const int nblk = (kvlen + 15) >> 4;
-    const int bpc = (nblk + a.nch - 1) / a.nch;
-    const int b0 = chunk * bpc, b1 = min(b0 + bpc, nblk);
+    // sliding window (families/gptoss/attn.rs:120-137): a row at sequence length n sees positions
+    // n - window .. n - 1.  The window exceeds the pass width, so every row keeps its whole drafted
+    // suffix and the cut falls in the committed prefix: blocks before the first row's cut are not
+    // read at all, the few blocks where the rows' cuts differ are masked per row.
+    const int window = a.window;
+    const int bfirst = window > 0 ? max(base + 1 - window, 0) >> 4 : 0;
+    const int bpc = (nblk - bfirst + a.nch - 1) / a.nch;
+    const int b0 = bfirst + chunk * bpc, b1 = min(b0 + bpc, nblk);
+    const int cut_end = window > 0 ? base + M - window : 0;  // positions from here on are inside every row's window
     const float scale = a.scale;
     const uint32_t mmask = (1u << M) - 1u;  // slots that exist in this pass
 
     // query fragments and per-row ancestor sets
     uint4 qf[RT][KS];
     uint32_t anc[RT];
+    int lo[RT];  // first visible position of the row (window)
 #pragma unroll
     for (int t = 0; t < RT; t++) {
         const int r = (rt0 + t) * 16 + j;
         anc[t] = 0xFFFFu;
+        lo[t] = 0;
         if (r < R) {
             const int mrow = r / G, g = r - mrow * G;
             anc[t] = vp->anc[mrow];
+            if (window > 0) lo[t] = vp->pos[mrow] + 1 - window;
             const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
 #pragma unroll
             for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
@@ -101,6 +111,10 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
             if (tail) {
                 const uint64_t w = ((uint64_t)(anc[t] & mmask) << 16) | 0xFFFFull;
                 vis4 = (uint32_t)(w >> (p0 + 4 * kg - base + 16)) & 0xFu;  // shift in [1, 47]
+            }
+            if (p0 < cut_end) {  // some row's window starts inside or after this block
+                const int d = lo[t] - (p0 + 4 * kg);  // this lane's positions below index d are outside
+                vis4 &= d <= 0 ? 0xFu : d >= 4 ? 0u : (0xFu << d) & 0xFu;
             }
             float sc[4];
 #pragma unroll
@@ -206,9 +220,14 @@ __global__ void k_attn_combine(AttnArgs a, int G, int R) {
         }
         float mx = mc;
         for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        // the sink joins the maximum and the denominator, never the numerator
+        // (crates/compute/src/attention.rs:94-105)
+        const float sink = a.sinks ? a.sinks[qh] : -INFINITY;
+        mx = fmaxf(mx, sink);
         const float w = mc > -INFINITY ? __expf(mc - mx) : 0.f;
         float den = lc * w;
         for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+        if (a.sinks) den += __expf(sink - mx);
         wgt[d] = w;
         if (d == 0) s_den = den;
     }

@@ -83,7 +83,7 @@ __global__ void k_repack_q80(const uint8_t* __restrict__ raw, int n_rows, int kc
 // MXFP4: one thread per source block (17 bytes: scale, then 16 bytes whose low / high nibbles are
 // elements j and j + 16).  Nibble n of output word w is K element 8w + {0,2,1,3,4,6,5,7}[n].
 __global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
-                             uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, int nblk) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long total = (long)n_rows * kchunks * 8;
     if (gid >= total) return;
@@ -93,7 +93,8 @@ __global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kc
     const int r = (int)(t / kchunks);
     const int drow = (r / grp) * stride + offset + r % grp;
     const int tile = drow >> 6, lane = drow & 63;
-    const uint8_t* blk = raw + ((long)r * kchunks * 8 + (long)c * 8 + u) * 17;
+    if (c * 8 + u >= nblk) return;  // past the row's last block: the tile keeps its zero block
+    const uint8_t* blk = raw + ((long)r * nblk + (long)c * 8 + u) * 17;
     uint8_t* tb = tiles + ((long)tile * kchunks + c) * 8704;
     uint32_t words[4];
 #pragma unroll
@@ -111,15 +112,39 @@ __global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kc
     tb[8192 + lane * 8 + u] = blk[0];
 }
 
+// bf16: one thread per 16-byte unit (eight consecutive K values of a row, two MFMA steps).
+__global__ void k_repack_bf16(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
+                              uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)n_rows * kchunks * 8;
+    if (gid >= total) return;
+    const int u = (int)(gid % 8);
+    const long t = gid / 8;
+    const int c = (int)(t % kchunks);
+    const int r = (int)(t / kchunks);
+    const int drow = (r / grp) * stride + offset + r % grp;
+    const int tile = drow >> 6, lane = drow & 63;
+    const uint16_t* src = (const uint16_t*)raw + ((long)r * kchunks + c) * 64 + 8 * u;
+    uint16_t v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = src[(i & 4) | ((i & 1) << 1) | ((i >> 1) & 1)];
+    uint16_t* dst = (uint16_t*)(tiles + ((long)tile * kchunks + c) * 8192 + (u * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 8; i++) dst[i] = v[i];
+}
+
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
                   int kchunks, int grp, int stride, int offset) {
-    (void)k;
     const long total = (long)n_rows * kchunks * 9;
     if (total == 0) return TSV_OK;
-    if (fmt == FMT_MX4) {
+    if (fmt == FMT_BF16) {
+        const long units = (long)n_rows * kchunks * 8;
+        hipLaunchKernelGGL(k_repack_bf16, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
+                           tiles, grp, stride, offset);
+    } else if (fmt == FMT_MX4) {
         const long blocks = (long)n_rows * kchunks * 8;
         hipLaunchKernelGGL(k_repack_mx4, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
-                           tiles, grp, stride, offset);
+                           tiles, grp, stride, offset, k / 32);
     } else if (fmt == FMT_Q4K)
         hipLaunchKernelGGL(k_repack_q4k, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, raw, n_rows,
                            kchunks, tiles, grp, stride, offset);
@@ -291,7 +316,7 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
     if (epi != EPI_PARTIAL) splits = 1;
     if (splits < 1) splits = 1;
     if (splits > w.kchunks) splits = w.kchunks;
-    GemmArgs a;
+    GemmArgs a{};
     a.w = w.tiles;
     a.xfrag = (const uint2*)xfrag;
     a.xsum = (const float*)((const char*)xfrag + xfrag_sum_offset(w.k));
@@ -318,9 +343,10 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
         }
         a.n_valid = w.n_rows / 2;  // K of the next matmul
     }
-    return w.fmt == FMT_Q4K   ? launch_f<Q4K>(s, a, m, epi)
-           : w.fmt == FMT_Q80 ? launch_f<Q80>(s, a, m, epi)
-                              : launch_f<MX4>(s, a, m, epi);
+    return w.fmt == FMT_Q4K    ? launch_f<Q4K>(s, a, m, epi)
+           : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
+           : w.fmt == FMT_BF16 ? launch_f<BF16W>(s, a, m, epi)
+                               : launch_f<MX4>(s, a, m, epi);
 }
 
 }  // namespace tsv

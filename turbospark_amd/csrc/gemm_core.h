@@ -149,6 +149,32 @@ struct MX4 {
     static __device__ __forceinline__ int xs_base(int c, int lane) { return Q4K::xs_base(c, lane); }
 };
 
+// bf16 matrices (crates/compute/src/quant.rs:14-39: a bf16 is the upper half of the fp32 bits).
+// A tile is 64 rows x 64 K: unit u holds the lane's row at K steps 2u and 2u + 1, four values per
+// step in the activations' element order (k % 4 = 0, 2, 1, 3), i.e. exactly the B operand of
+// v_mfma_f32_4x4x4_16B_bf16.  The fp16 activations are split exactly into two bf16 terms
+// (upper eight significant bits + remainder), so the products are those of the fp16 values.
+struct BF16W {
+    static constexpr int NSUB = 2, NPAIR = 1, TILE_BYTES = 8192;
+    static constexpr bool SUMS = false;
+    struct Regs {
+        u32x4 q[8];
+    };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
+        const u32x4* p = (const u32x4*)tile + lane;
+#pragma unroll
+        for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
+    }
+    static __device__ __forceinline__ int xs_base(int, int) { return 0; }
+};
+
+template <int STEP>
+__device__ __forceinline__ float4v mfma_bf16(u32x2 a, u32x2 b, float4v c) {
+    typedef short short4v __attribute__((ext_vector_type(4)));
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4v, a), __builtin_bit_cast(short4v, b), c, 4,
+                                                  STEP, 0);
+}
+
 template <class F, int NG>
 struct XRegs {
     u32x2 xa[F::NPAIR][NG];
@@ -392,6 +418,35 @@ __device__ __forceinline__ void compute_tile(MX4, const Src& w, const XRegs<MX4,
             fma4(acc[g], sc[2 * p + 1], db[g]);
         }
     }
+}
+
+// One bf16 tile (64 rows x 64 K).
+template <int NG, class Src>
+__device__ __forceinline__ void compute_tile(BF16W, const Src& w, const XRegs<BF16W, NG>& x, const Consts&,
+                                             float4v (&acc)[NG]) {
+    u32x2 ahi[NG], alo[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t word = x.xa[0][g][h];
+            const float f0 = h2f_lo(word), f1 = h2f_hi(word);
+            const uint32_t b0 = __float_as_uint(f0) & 0xFFFF0000u, b1 = __float_as_uint(f1) & 0xFFFF0000u;
+            const uint32_t r0 = __float_as_uint(f0 - __uint_as_float(b0)), r1 = __float_as_uint(f1 - __uint_as_float(b1));
+            ahi[g][h] = (b0 >> 16) | b1;
+            alo[g][h] = (r0 >> 16) | (r1 & 0xFFFF0000u);
+        }
+    }
+    static_for<16>([&](auto S) {
+        constexpr int s = decltype(S)::value;
+        const u32x4 u = w.unit(s >> 1);
+        const u32x2 b = (s & 1) ? u32x2{u.z, u.w} : u32x2{u.x, u.y};
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            acc[g] = mfma_bf16<s>(ahi[g], b, acc[g]);
+            acc[g] = mfma_bf16<s>(alo[g], b, acc[g]);
+        }
+    });
 }
 
 // a register stage

@@ -229,6 +229,40 @@ void parallel_rows(int64_t rows, F f) {
 
 extern "C" int64_t tsv_row_bytes(int32_t dtype, int64_t cols) { return tsv::row_bytes(dtype, cols); }
 
+// crates/compute/src/rope.rs:296-372.  The two correction dimensions come from the wavelengths
+// that fit beta_fast / beta_slow times into the original context; pairs below the first keep
+// their frequency, pairs above the second are divided by the factor, linear mix between.
+extern "C" int32_t tsv_yarn_frequencies(int32_t rotary_dim, float base, float factor, int64_t original_context,
+                                        float beta_fast, float beta_slow, float* freqs, float* mscale) {
+    if (rotary_dim < 2 || rotary_dim % 2 || !freqs || !mscale || !(base > 1.0f)) {
+        tsv::set_error("yarn_frequencies: rotary_dim must be even and base > 1");
+        return TSV_ERR_INVALID;
+    }
+    const bool on = factor > 0.0f;
+    const float inv = on ? 1.0f / factor : 1.0f;
+    auto corr = [&](float n_rot) {
+        return (float)rotary_dim * logf((float)original_context / (n_rot * 2.0f * 3.14159265358979323846f)) /
+               (2.0f * logf(base));
+    };
+    float lo = 0.0f, hi = 0.0f;
+    if (on) {
+        lo = fmaxf(floorf(corr(beta_fast)), 0.0f);
+        hi = fminf(ceilf(corr(beta_slow)), (float)rotary_dim - 1.0f);
+    }
+    for (int p = 0; p < rotary_dim / 2; p++) {
+        const float plain = powf(base, -((float)(2 * p)) / (float)rotary_dim);
+        float f = plain;
+        if (on) {
+            const float y = ((float)p - lo) / fmaxf(hi - lo, 0.001f);
+            const float keep = 1.0f - fminf(fmaxf(y, 0.0f), 1.0f);
+            f = plain * (inv * (1.0f - keep) + keep);
+        }
+        freqs[p] = f;
+    }
+    *mscale = on ? 1.0f + 0.1f * logf(factor) : 1.0f;
+    return TSV_OK;
+}
+
 extern "C" int32_t tsv_quantize_rows(int32_t dtype, const float* src, int64_t rows, int64_t cols, void* dst) {
     const int64_t rb = tsv::row_bytes(dtype, cols);
     if (rb < 0 || !src || !dst) {

@@ -78,7 +78,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const float* __restrict__ partial,
                                                   int splits, int ldp, const float* __restrict__ w,
                                                   float eps, int hidden, _Float16* __restrict__ xfrag,
-                                                  const float* __restrict__ weights) {
+                                                  const float* __restrict__ weights,
+                                                  const float* __restrict__ bias) {
     __shared__ float red[16];
     const int m = blockIdx.x;
     float4* xr = (float4*)(x + (long)m * hidden);
@@ -87,19 +88,37 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
     float ss = 0.f;
     for (int i = threadIdx.x; i < n4; i += 1024) {
         float4 v = xr[i];
-        for (int s = 0; s < splits; s++) {
-            float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
-            if (weights) {  // routed experts: y += w_slot * out_slot, product and sum rounded apart
+        if (weights) {
+            // routed experts (families/llama/moe.rs:193-198): the slot outputs are weighted and summed
+            // in rank order starting from zero, then added to the stream; product and sum rounded apart
+            float4 r = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < splits; s++) {
+                const float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
                 const float ws = weights[m * 8 + s];
-                p.x = __fmul_rn(ws, p.x);
-                p.y = __fmul_rn(ws, p.y);
-                p.z = __fmul_rn(ws, p.z);
-                p.w = __fmul_rn(ws, p.w);
+                r.x = __fadd_rn(r.x, __fmul_rn(ws, p.x));
+                r.y = __fadd_rn(r.y, __fmul_rn(ws, p.y));
+                r.z = __fadd_rn(r.z, __fmul_rn(ws, p.z));
+                r.w = __fadd_rn(r.w, __fmul_rn(ws, p.w));
             }
-            v.x = __fadd_rn(v.x, p.x);
-            v.y = __fadd_rn(v.y, p.y);
-            v.z = __fadd_rn(v.z, p.z);
-            v.w = __fadd_rn(v.w, p.w);
+            v.x = __fadd_rn(v.x, r.x);
+            v.y = __fadd_rn(v.y, r.y);
+            v.z = __fadd_rn(v.z, r.z);
+            v.w = __fadd_rn(v.w, r.w);
+        } else {
+            for (int s = 0; s < splits; s++) {
+                const float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
+                v.x = __fadd_rn(v.x, p.x);
+                v.y = __fadd_rn(v.y, p.y);
+                v.z = __fadd_rn(v.z, p.z);
+                v.w = __fadd_rn(v.w, p.w);
+            }
+            if (bias) {  // the output projection's bias (families/gptoss/mod.rs:16)
+                const float4 b = *(const float4*)(bias + 4 * i);
+                v.x += b.x;
+                v.y += b.y;
+                v.z += b.z;
+                v.w += b.w;
+            }
         }
         xr[i] = v;
         ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
@@ -123,9 +142,9 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
 }
 
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
-                   float eps, int hidden, uint4* xfrag, int m, const float* weights) {
+                   float eps, int hidden, uint4* xfrag, int m, const float* weights, const float* bias) {
     hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
-                       (_Float16*)xfrag, weights);
+                       (_Float16*)xfrag, weights, bias);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -169,6 +188,10 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
             x0 += p[i];
             x1 += p[i + half];
         }
+        if (a.bias) {  // before the rotation (families/gptoss/attn.rs:88-101)
+            x0 += a.bias[col + i];
+            x1 += a.bias[col + i + half];
+        }
     }
     const float* nw = kind == 0 ? a.q_norm : kind == 1 ? a.k_norm : nullptr;
     if (nw) {
@@ -185,6 +208,8 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
         const float angle = (float)vp->pos[m] * a.freqs[i];
         float sn, cs;
         sincosf(angle, &sn, &cs);
+        sn *= a.mscale;
+        cs *= a.mscale;
         const float r0 = x0 * cs - x1 * sn;
         const float r1 = x0 * sn + x1 * cs;
         x0 = r0;

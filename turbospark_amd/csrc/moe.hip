@@ -38,6 +38,7 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
             if (e < ne) {
                 float s = 0.f;
                 for (int sp = 0; sp < a.splits; sp++) s += a.logits[((size_t)sp * 16 + m) * a.ld + e];
+                if (a.bias) s += a.bias[e];  // before the top-k (families/gptoss/moe.rs:82-87)
                 v[j] = s;
             }
         }
@@ -167,8 +168,19 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float other = __shfl_xor(v[i], 32);
-            const float gate = lane < 32 ? v[i] : other, up = lane < 32 ? other : v[i];
-            const _Float16 h = (_Float16)(silu_moe(gate) * up);
+            float gate = lane < 32 ? v[i] : other, up = lane < 32 ? other : v[i];
+            if (a.bias) {  // before the activation, where the clamp reads it too (moe_gguf.metal:585-600)
+                gate += a.bias[(size_t)e * a.n_out + col];
+                up += a.bias2[(size_t)e * a.n_out + col];
+            }
+            float act;
+            if (a.alpha > 0.0f) {
+                const float x = fminf(gate, a.limit), y = fminf(fmaxf(up, -a.limit), a.limit);
+                act = (x / (1.0f + __expf(-a.alpha * x))) * (y + 1.0f);
+            } else {
+                act = silu_moe(gate) * up;
+            }
+            const _Float16 h = (_Float16)act;
             float sum = (float)h;
 #pragma unroll
             for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
@@ -184,7 +196,9 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int b = r0 + i;
-                if (b < cnt) ((float*)a.out)[((size_t)grp.slots[b] * 16 + grp.rows[b]) * a.n_out + n] = v[i];
+                if (b < cnt)
+                    ((float*)a.out)[((size_t)grp.slots[b] * 16 + grp.rows[b]) * a.n_out + n] =
+                        a.bias ? v[i] + a.bias[(size_t)e * a.n_out + n] : v[i];
             }
         }
     }

@@ -21,18 +21,26 @@ struct LayerW {
     int n_experts = 0, top_k = 0;     // routed experts: gate_up / down hold every expert's tiles
     TiledW router;
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    // gpt-oss additions, all optional: fused q/k/v bias, output bias, sinks, router bias, expert biases
+    float *bqkv = nullptr, *bo = nullptr, *sinks = nullptr, *router_bias = nullptr;
+    float *be_gate = nullptr, *be_up = nullptr, *be_down = nullptr;
+    int window = 0;
     uint16_t *kc = nullptr, *vc = nullptr;
 };
 
 int dtype_fmt(int dtype) {
-    return dtype == TSV_Q4_K ? FMT_Q4K : dtype == TSV_Q8_0 ? FMT_Q80 : dtype == TSV_MXFP4 ? FMT_MX4 : -1;
+    return dtype == TSV_Q4_K    ? FMT_Q4K
+           : dtype == TSV_Q8_0  ? FMT_Q80
+           : dtype == TSV_MXFP4 ? FMT_MX4
+           : dtype == TSV_BF16  ? FMT_BF16
+                                : -1;
 }
 
 }  // namespace
 
 struct tsv_ctx {
     int n_layers = 0, hidden = 0, nq = 0, nkv = 0, hd = 0, ffn = 0, vocab = 0, max_context = 0, ctx_alloc = 0;
-    float eps = 0, attn_scale = 0;
+    float eps = 0, attn_scale = 0, rope_mscale = 1.0f, act_alpha = 0, act_limit = 0;
     hipStream_t stream = nullptr;
     std::vector<LayerW> layers;
     TiledW head;
@@ -161,11 +169,13 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
         return TSV_ERR_INVALID;
     }
     if (fmt < 0) {
-        set_error(std::string(what) + ": matmul weights must be Q4_K, Q8_0 or MXFP4 in this build");
+        set_error(std::string(what) + ": matmul weights must be Q4_K, Q8_0, MXFP4 or bf16 in this build");
         return TSV_ERR_UNSUPPORTED;
     }
-    if (cols % fmt_chunk_elems(fmt) || rows < 1) {
-        set_error(std::string(what) + ": K must be whole 256 (Q4_K, MXFP4) / 128 (Q8_0) chunks");
+    // MXFP4 rows may end inside a 256-element chunk (the tile is padded with zero blocks)
+    const int gran = fmt == FMT_MX4 ? 32 : fmt_chunk_elems(fmt);
+    if (cols % gran || rows < 1) {
+        set_error(std::string(what) + ": K must be whole 256 (Q4_K) / 128 (Q8_0) / 64 (bf16) / 32 (MXFP4) element runs");
         return TSV_ERR_UNSUPPORTED;
     }
     return TSV_OK;
@@ -190,7 +200,7 @@ int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_par
     }
     out->fmt = fmt;
     out->k = (int)parts[0]->cols;
-    out->kchunks = out->k / fmt_chunk_elems(fmt);
+    out->kchunks = (out->k + fmt_chunk_elems(fmt) - 1) / fmt_chunk_elems(fmt);
     out->n_rows = (int)total_rows;
     out->n_tiles = (int)((total_rows + TILE_ROWS - 1) / TILE_ROWS);
     out->bytes = (size_t)out->n_tiles * out->kchunks * fmt_tile_bytes(fmt);
@@ -371,11 +381,13 @@ int launch_pass(tsv_ctx* c, int m) {
             for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++) rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n);
         }
         if (rc) return rc;
-        RopeKvArgs ra;
+        RopeKvArgs ra{};
         ra.qkv = c->partial;
         ra.splits = sp;
         ra.ldq = qkv_n;
         ra.freqs = c->freqs;
+        ra.mscale = c->rope_mscale;
+        ra.bias = L.bqkv;
         ra.q_norm = L.q_norm;
         ra.k_norm = L.k_norm;
         ra.eps = c->eps;
@@ -393,7 +405,7 @@ int launch_pass(tsv_ctx* c, int m) {
             for (int rep = 0; rep < c->repeat[PC_ROPE] && !rc; rep++) rc = launch_rope_kv(s, ra, m);
         }
         if (rc) return rc;
-        AttnArgs aa;
+        AttnArgs aa{};
         aa.q16 = c->q16;
         aa.kc = L.kc;
         aa.vc = L.vc;
@@ -406,6 +418,8 @@ int launch_pass(tsv_ctx* c, int m) {
         aa.max_ctx = c->ctx_alloc;
         aa.nch = c->nch;
         aa.scale = c->attn_scale;
+        aa.window = L.window;
+        aa.sinks = L.sinks;
         aa.vp = c->vp_dev;
         {
             PROF(PC_ATTN);
@@ -421,7 +435,7 @@ int launch_pass(tsv_ctx* c, int m) {
         }
         if (rc) return rc;
         if (c->fused_ffn) {
-            FfnBlockArgs fa;
+            FfnBlockArgs fa{};
             fa.sync.rank_ctr = c->rank_ctr;
             fa.sync.bar_ctr = c->bar_ctr;
             fa.sync.err = c->fused_err;
@@ -459,14 +473,14 @@ int launch_pass(tsv_ctx* c, int m) {
         }
         {
             PROF(PC_NORM);
-            rc = launch_addnorm(s, x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m);
+            rc = launch_addnorm(s, x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo);
         }
         if (rc) return rc;
         if (L.n_experts) {
             // router -> top-k -> grouped expert matmuls; the per-slot outputs are added, weighted
             // and in slot order, by the next residual kernel
             const int rsp = splits_for(L.router, m, EPI_PARTIAL);
-            MoeRouteArgs ra2;
+            MoeRouteArgs ra2{};
             ra2.logits = c->partial;
             ra2.splits = rsp;
             ra2.ld = L.n_experts;
@@ -476,7 +490,8 @@ int launch_pass(tsv_ctx* c, int m) {
             ra2.weights = c->route_w;
             ra2.selected = c->route_sel;
             ra2.groups = c->route_groups;
-            MoeGemmArgs g1, g2;
+            ra2.bias = L.router_bias;
+            MoeGemmArgs g1{}, g2{};
             g1.w = L.gate_up.tiles;
             g1.tiles_per_expert = c->ffn / 32;
             g1.kchunks = L.gate_up.kchunks;
@@ -487,8 +502,14 @@ int launch_pass(tsv_ctx* c, int m) {
             g1.out_stride = c->frag_e_stride;
             g1.n_out = c->ffn;
             g1.groups = c->route_groups;
+            g1.bias = L.be_gate;
+            g1.bias2 = L.be_up;
+            g1.alpha = c->act_alpha;
+            g1.limit = c->act_limit;
             const int n_groups = m * L.top_k;
             g2 = g1;
+            g2.bias = L.be_down;
+            g2.bias2 = nullptr;
             g2.w = L.down.tiles;
             g2.tiles_per_expert = c->hidden / 64;
             g2.kchunks = L.down.kchunks;
@@ -628,6 +649,9 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->ctx_alloc = ((d->max_context + 15) / 16) * 16;
     c->eps = d->rms_eps;
     c->attn_scale = d->attn_scale > 0.f ? d->attn_scale : 1.0f / std::sqrt((float)d->head_dim);
+    c->rope_mscale = d->rope_mscale > 0.f ? d->rope_mscale : 1.0f;
+    c->act_alpha = d->act_alpha;
+    c->act_limit = d->act_limit;
     if (const char* e = getenv("TSV_GRAPH")) c->use_graph = e[0] == '1';
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("open: cannot create a HIP stream (no GPU?)");
@@ -691,6 +715,44 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
                 (rc = upload_vector(c, s.k_norm, c->hd, &L.k_norm, "k_norm")))
                 return fail(rc);
         }
+        // gpt-oss additions (families/gptoss/mod.rs:11-23)
+        if (s.bq.data || s.bk.data || s.bv.data) {
+            if (!s.bq.data || !s.bk.data || !s.bv.data) {
+                set_error("open: q, k and v projection biases come together");
+                return fail(TSV_ERR_INVALID);
+            }
+            float *bq = nullptr, *bk = nullptr, *bv = nullptr;  // one device vector in the fused row order
+            if ((rc = dev_alloc(c, &L.bqkv, (size_t)(qd + 2 * kvd) * 4))) return fail(rc);
+            if ((rc = upload_vector(c, s.bq, qd, &bq, "bq")) || (rc = upload_vector(c, s.bk, kvd, &bk, "bk")) ||
+                (rc = upload_vector(c, s.bv, kvd, &bv, "bv")))
+                return fail(rc);
+            if (hipMemcpy(L.bqkv, bq, (size_t)qd * 4, hipMemcpyDeviceToDevice) != hipSuccess ||
+                hipMemcpy(L.bqkv + qd, bk, (size_t)kvd * 4, hipMemcpyDeviceToDevice) != hipSuccess ||
+                hipMemcpy(L.bqkv + qd + kvd, bv, (size_t)kvd * 4, hipMemcpyDeviceToDevice) != hipSuccess)
+                return fail(TSV_ERR_DEVICE);
+        }
+        if (s.bo.data && (rc = upload_vector(c, s.bo, c->hidden, &L.bo, "bo"))) return fail(rc);
+        if (s.sinks.data && (rc = upload_vector(c, s.sinks, c->nq, &L.sinks, "sinks"))) return fail(rc);
+        if (s.window < 0 || (s.window > 0 && s.window <= TSV_MAX_ROWS)) {
+            set_error("open: a sliding window must be wider than one verify pass (16 rows)");
+            return fail(TSV_ERR_UNSUPPORTED);
+        }
+        L.window = s.window;
+        if (ne > 0) {
+            if (s.router_bias.data && (rc = upload_vector(c, s.router_bias, ne, &L.router_bias, "router_bias")))
+                return fail(rc);
+            if (s.be_gate.data || s.be_up.data) {
+                if (!s.be_gate.data || !s.be_up.data) {
+                    set_error("open: expert gate and up biases come together");
+                    return fail(TSV_ERR_INVALID);
+                }
+                if ((rc = upload_vector(c, s.be_gate, (int64_t)ne * c->ffn, &L.be_gate, "be_gate")) ||
+                    (rc = upload_vector(c, s.be_up, (int64_t)ne * c->ffn, &L.be_up, "be_up")))
+                    return fail(rc);
+            }
+            if (s.be_down.data && (rc = upload_vector(c, s.be_down, (int64_t)ne * c->hidden, &L.be_down, "be_down")))
+                return fail(rc);
+        }
         const size_t kvb = (size_t)c->nkv * c->ctx_alloc * c->hd * 2;
         if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) return fail(rc);
         pneed = std::max(pneed, std::max(partial_need(L.qkv), partial_need(L.wo)));
@@ -710,11 +772,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     {
         tsv_tensor head = d->lm_head.data ? d->lm_head : d->embed;
         // the head's row count need not be a multiple of 16: the last tile is zero padded
-        const int fmt = dtype_fmt(head.dtype);
-        if (head.rows != c->vocab || head.cols != c->hidden || fmt < 0 || c->hidden % fmt_chunk_elems(fmt)) {
-            set_error("open: output head must be a Q4_K / Q8_0 vocab x hidden matrix");
-            return fail(TSV_ERR_UNSUPPORTED);
-        }
+        if ((rc = check_matrix(head, c->vocab, c->hidden, "output head"))) return fail(rc);
         const tsv_tensor* hp[1] = {&head};
         if ((rc = make_tiled(c, st, hp, 1, false, &c->head))) return fail(rc);
     }
@@ -724,7 +782,9 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         // rope.rs:208-256 (scalar theta: exp(-(2i/hd) * ln theta)) or rope.rs:447-460 (per-pair divisors)
         std::vector<float> f((size_t)c->hd / 2);
         for (int i = 0; i < c->hd / 2; i++) {
-            if (d->rope_factors)
+            if (d->rope_freqs)
+                f[i] = d->rope_freqs[i];  // an explicit table (YaRN)
+            else if (d->rope_factors)
                 f[i] = std::pow(d->rope_theta, -((float)(2 * i)) / (float)c->hd) / d->rope_factors[i];
             else
                 f[i] = std::exp((-((float)(2 * i)) / (float)c->hd) * std::log(d->rope_theta));
@@ -1206,8 +1266,9 @@ extern "C" int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, fl
 
 extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
                                  int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
-                                 uint16_t* out) {
-    if (!q || !k || !v || !out || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0) {
+                                 int32_t window, const float* sinks, uint16_t* out) {
+    if (!q || !k || !v || !out || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0 || window < 0 ||
+        (window > 0 && window <= TSV_MAX_ROWS)) {
         set_error("attention: bad argument");
         return TSV_ERR_INVALID;
     }
@@ -1219,10 +1280,15 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv;
     const size_t kvb = (size_t)nkv * ctx * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
     uint16_t *kc = nullptr, *vc = nullptr, *kin = nullptr, *vin = nullptr, *q16 = nullptr;
-    float *po = nullptr, *pml = nullptr;
+    float *po = nullptr, *pml = nullptr, *sinks_dev = nullptr;
     uint4* xf = nullptr;
     VerifyParams* vpd = nullptr;
     const size_t xfb = xfrag_bytes(nq * hd);
+    if (!rc && sinks) {
+        rc = dev_alloc(c, &sinks_dev, (size_t)nq * 4);
+        if (!rc && hipMemcpyAsync(sinks_dev, sinks, (size_t)nq * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess)
+            rc = TSV_ERR_DEVICE;
+    }
     if (!rc) rc = dev_alloc(c, &kc, kvb, true);
     if (!rc) rc = dev_alloc(c, &vc, kvb, true);
     if (!rc) rc = dev_alloc(c, &kin, inb);
@@ -1239,7 +1305,7 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
         rc = TSV_ERR_DEVICE;
     if (!rc) rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, 0, seq, kin, vin);
     if (!rc) {
-        AttnArgs aa;
+        AttnArgs aa{};
         aa.q16 = q16;
         aa.kc = kc;
         aa.vc = vc;
@@ -1252,6 +1318,8 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
         aa.max_ctx = ctx;
         aa.nch = nch;
         aa.scale = scale > 0.f ? scale : 1.0f / std::sqrt((float)hd);
+        aa.window = window;
+        aa.sinks = sinks_dev;
         aa.vp = vpd;
         rc = launch_attention(c->stream, aa, m);
     }

@@ -35,6 +35,8 @@ const std::string& get_error();
 //   MXFP4 tile, 8704 B (64 rows x 256 K): [unit 0..7][lane][16 B] the 32 e2m1 nibbles of the
 //                      lane's block u, nibbles re-ordered for the fp4 -> fp16 converter (see
 //                      gemm_core.h), then [lane][8 e8m0 scale bytes].
+//   bf16 tile, 8192 B (64 rows x 64 K): [unit 0..7][lane][16 B] the lane's row at K steps 2u and
+//                      2u + 1, four values per step in the order k % 4 = 0, 2, 1, 3.
 // Rows past the matrix's last row are all-zero blocks (scale 0).
 //
 // Activation layout ("fragments").  The <=16 fp16 activation rows of a K-wide matmul input
@@ -45,7 +47,7 @@ const std::string& get_error();
 // every 32-element sub-block, [K/256][g][sub%8][i], which the matmul uses to take the
 // integer-code offsets and the Q4_K min term back out.
 // ---------------------------------------------------------------------------------------
-enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2 };
+enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2, FMT_BF16 = 3 };
 
 struct TiledW {
     uint8_t* tiles = nullptr;  // device
@@ -57,9 +59,9 @@ struct TiledW {
     size_t bytes = 0;
 };
 
-inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q80 ? 128 : 256; }
-inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : 8704; }
-inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : 8; }
+inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q80 ? 128 : fmt == FMT_BF16 ? 64 : 256; }
+inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : fmt == FMT_BF16 ? 8192 : 8704; }
+inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : fmt == FMT_BF16 ? 2 : 8; }
 constexpr int TILE_ROWS = 64;
 
 // index (in halfs) of activation element (row, k) in the fragment layout
@@ -67,7 +69,9 @@ __host__ __device__ inline int frag_index(int k, int row) {
     const int pos = ((k & 1) << 1) | ((k >> 1) & 1);  // k%4 = 0,1,2,3 -> slot 0,2,1,3
     return ((((k >> 6) * 4 + (row >> 2)) * 16 + ((k >> 2) & 15)) * 4 + (row & 3)) * 4 + pos;
 }
-__host__ __device__ inline size_t xfrag_sum_offset(int k) { return (size_t)((k + 63) / 64) * 2048; }
+// (K is rounded up to whole 256-element chunks: a matmul whose last chunk is only partly real
+// reads zeros there, never the sums)
+__host__ __device__ inline size_t xfrag_sum_offset(int k) { return (size_t)((k + 255) / 256) * 8192; }
 __host__ __device__ inline size_t xfrag_bytes(int k) { return xfrag_sum_offset(k) + (size_t)((k + 255) / 256) * 512; }
 // index (in floats) of the sum of sub-block `sub` (= k/32) of `row`
 __host__ __device__ inline int xsum_index(int sub, int row) {
@@ -120,6 +124,7 @@ struct MoeRouteArgs {
     float* weights;     // [16][8] softmax over the selected logits, rank order
     int32_t* selected;  // [16][8] expert ids, rank order
     MoeGroup* groups;   // [16 * 8]
+    const float* bias;  // nullable: n_experts values added to the logits before the top-k
 };
 struct MoeGemmArgs {
     const uint8_t* w;      // tiled weights of all experts, tiles_per_expert x kchunks tiles each
@@ -130,6 +135,11 @@ struct MoeGemmArgs {
     size_t out_stride;
     int n_out;             // gate/up: expert FFN width; down: hidden
     const MoeGroup* groups;
+    // nullable per-expert biases, [n_experts][n_out]: gate/up use bias (gate) and bias2 (up), added
+    // before the activation; down uses bias, added before the slot is weighted
+    const float* bias;
+    const float* bias2;
+    float alpha, limit;    // alpha > 0: clamped SwiGLU (moe_gguf.metal:528-556) instead of silu(g) * u
 };
 int launch_route(hipStream_t s, const MoeRouteArgs& a);
 int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
@@ -177,13 +187,16 @@ int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float
                  const VerifyParams* vp, int m);
 // weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
-                   float eps, int hidden, uint4* xfrag, int m, const float* weights = nullptr);
+                   float eps, int hidden, uint4* xfrag, int m, const float* weights = nullptr,
+                   const float* bias = nullptr);
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
 
 struct RopeKvArgs {
     const float* qkv;  // [splits][16][ldq]
     int splits, ldq;
     const float* freqs;   // head_dim/2
+    float mscale;         // multiplies cos and sin
+    const float* bias;    // nullable: [ldq] projection biases in the fused q, k, v row order
     const float* q_norm;  // nullable, head_dim
     const float* k_norm;
     float eps;
@@ -204,6 +217,8 @@ struct AttnArgs {
     uint4* xfrag;    // output, K index = qh*hd + d
     int nq, nkv, hd, max_ctx, nch;
     float scale;
+    int window;          // 0: full; else a row sees the last `window` positions of its sequence
+    const float* sinks;  // nullable: one logit per q head joining the softmax maximum and denominator
     const VerifyParams* vp;
 };
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);

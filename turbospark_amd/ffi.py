@@ -24,11 +24,13 @@ class Tensor(C.Structure):
 
 LAYER_TENSORS = ("attn_norm", "wq", "wk", "wv", "wo", "q_norm", "k_norm", "ffn_norm", "w_gate", "w_up", "w_down")
 LAYER_MOE_TENSORS = ("router", "we_gate", "we_up", "we_down")
+LAYER_GPTOSS_TENSORS = ("bq", "bk", "bv", "bo", "sinks", "router_bias", "be_gate", "be_up", "be_down")
 
 
 class Layer(C.Structure):
     _fields_ = ([(n, Tensor) for n in LAYER_TENSORS] + [("n_experts", C.c_int32), ("top_k", C.c_int32)] +
-                [(n, Tensor) for n in LAYER_MOE_TENSORS])
+                [(n, Tensor) for n in LAYER_MOE_TENSORS] + [(n, Tensor) for n in LAYER_GPTOSS_TENSORS] +
+                [("window", C.c_int32), ("reserved", C.c_int32)])
 
 
 class ModelDesc(C.Structure):
@@ -40,6 +42,8 @@ class ModelDesc(C.Structure):
         ("rope_factors", C.POINTER(C.c_float)),
         ("embed", Tensor), ("final_norm", Tensor), ("lm_head", Tensor),
         ("layers", C.POINTER(Layer)),
+        ("rope_freqs", C.POINTER(C.c_float)), ("rope_mscale", C.c_float),
+        ("act_alpha", C.c_float), ("act_limit", C.c_float),
     ]
 
 
@@ -105,6 +109,7 @@ EXPORTS = [
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
     "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
+    "tsv_yarn_frequencies",
 ]
 
 _lib = None
@@ -125,6 +130,8 @@ def lib():
         L.tsv_kv_position.argtypes = [C.c_void_p]
         L.tsv_row_bytes.restype = C.c_int64
         L.tsv_row_bytes.argtypes = [C.c_int32, C.c_int64]
+        L.tsv_yarn_frequencies.argtypes = [C.c_int32, C.c_float, C.c_float, C.c_int64, C.c_float, C.c_float,
+                                           C.c_void_p, C.POINTER(C.c_float)]
         L.tsv_close.restype = None
         L.tsv_close.argtypes = [C.c_void_p]
         L.tsv_open.argtypes = [C.POINTER(ModelDesc), C.POINTER(C.c_void_p)]
@@ -149,7 +156,7 @@ def lib():
         L.tsv_read_kv.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.tsv_matmul.argtypes = [C.POINTER(Tensor), C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
         L.tsv_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
-                                    C.c_int64, C.c_void_p, C.c_float, C.c_void_p]
+                                    C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_void_p, C.c_void_p]
         L.tsv_set_profile.argtypes = [C.c_void_p, C.c_int32]
         L.tsv_get_profile.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]
         L.tsv_copy_time.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
@@ -217,7 +224,7 @@ def matmul(entry, x, splits=0):
     return y
 
 
-def attention(q, k, v, base, parent=None, scale=0.0):
+def attention(q, k, v, base, parent=None, scale=0.0, window=0, sinks=None):
     """q [m, nq, hd], k/v [base+m, nkv, hd] (any float dtype; rounded to fp16) -> fp32 [m, nq, hd]."""
     q16 = np.ascontiguousarray(np.asarray(q, np.float32).astype(np.float16))
     k16 = np.ascontiguousarray(np.asarray(k, np.float32).astype(np.float16))
@@ -227,8 +234,11 @@ def attention(q, k, v, base, parent=None, scale=0.0):
     assert k16.shape[0] == base + m
     out = np.empty((m, nq, hd), np.float16)
     pa = np.ascontiguousarray(parent, np.int32) if parent is not None else None
-    check(lib().tsv_attention(q16.ctypes.data, k16.ctypes.data, v16.ctypes.data, m, nq, nkv, hd, base,
-                              pa.ctypes.data if pa is not None else None, scale, out.ctypes.data))
+    sk = np.ascontiguousarray(sinks, np.float32) if sinks is not None else None
+    check(lib().tsv_attention(C.c_void_p(q16.ctypes.data), C.c_void_p(k16.ctypes.data), C.c_void_p(v16.ctypes.data),
+                              m, nq, nkv, hd, C.c_int64(base), C.c_void_p(pa.ctypes.data) if pa is not None else None,
+                              C.c_float(scale), int(window), C.c_void_p(sk.ctypes.data) if sk is not None else None,
+                              C.c_void_p(out.ctypes.data)))
     return out.astype(np.float32)
 
 
@@ -244,3 +254,12 @@ def matmul_time(dtype, rows, cols, m, epi=0, splits=0, iters=50, rotate=4):
     t = C.c_float()
     check(lib().tsv_matmul_time(dtype, rows, cols, m, epi, splits, iters, rotate, C.byref(t)))
     return t.value
+
+
+def yarn_frequencies(rotary_dim, base, factor, original_context, beta_fast, beta_slow):
+    """(frequencies[rotary_dim // 2], mscale) of crates/compute/src/rope.rs:324-372."""
+    f = np.empty(rotary_dim // 2, np.float32)
+    ms = C.c_float()
+    check(lib().tsv_yarn_frequencies(rotary_dim, base, factor, original_context, beta_fast, beta_slow,
+                                     f.ctypes.data, C.byref(ms)))
+    return f, float(ms.value)

@@ -39,10 +39,11 @@ class HipVerifier:
         n = len(weights["layers"])
         self._layers = (ffi.Layer * n)()
         for i, lw in enumerate(weights["layers"]):
-            for name in ffi.LAYER_TENSORS + ffi.LAYER_MOE_TENSORS:
+            for name in ffi.LAYER_TENSORS + ffi.LAYER_MOE_TENSORS + ffi.LAYER_GPTOSS_TENSORS:
                 setattr(self._layers[i], name, ffi.tensor(lw.get(name)))
             self._layers[i].n_experts = int(lw.get("n_experts", 0))
             self._layers[i].top_k = int(lw.get("top_k", 0))
+            self._layers[i].window = int(lw.get("window", 0))
         d = ffi.ModelDesc()
         d.n_layers = n
         for key in ("hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_context"):
@@ -54,6 +55,13 @@ class HipVerifier:
         if cfg.get("rope_factors") is not None:
             self._factors = np.ascontiguousarray(cfg["rope_factors"], np.float32)
             d.rope_factors = self._factors.ctypes.data_as(C.POINTER(C.c_float))
+        self._freqs = None
+        if cfg.get("rope_freqs") is not None:
+            self._freqs = np.ascontiguousarray(cfg["rope_freqs"], np.float32)
+            d.rope_freqs = self._freqs.ctypes.data_as(C.POINTER(C.c_float))
+        d.rope_mscale = cfg.get("rope_mscale", 0.0)
+        d.act_alpha = cfg.get("act_alpha", 0.0)
+        d.act_limit = cfg.get("act_limit", 0.0)
         d.embed = ffi.tensor(weights["embed"])
         d.final_norm = ffi.tensor(weights["final_norm"])
         d.lm_head = ffi.tensor(weights.get("lm_head"))

@@ -23,6 +23,19 @@ CONFIGS = {
     "moe_small": dict(n_layers=2, hidden=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=256,
                       n_experts=16, top_k=4, vocab=4096, rms_eps=1e-6, rope_theta=1000000.0,
                       dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08, norm_jitter=0.25),
+    # a small decoder in the arrangement of the gpt-oss configuration: bf16 attention / router / head
+    # with projection biases, attention sinks, a sliding window on even layers, YaRN rotation,
+    # MXFP4 experts with biases and the clamped SwiGLU; hidden and expert width are NOT multiples
+    # of 256 (as 2880 is not), so the MXFP4 tiles end in zero-padded blocks
+    "gptoss_small": dict(n_layers=2, hidden=576, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=288,
+                         n_experts=8, top_k=4, vocab=4096, rms_eps=1e-5, rope_theta=150000.0, attn_scale=0.125,
+                         dtype=ffi.BF16, expert_dtype=ffi.MXFP4, router_sigma=0.08, norm_jitter=0.25,
+                         gptoss=dict(window=24, yarn=(32.0, 64, 32.0, 1.0), act_alpha=1.702, act_limit=7.0)),
+    # gpt-oss-120B shape (36 layers, 128 experts top-4, alternating 128-token window / full attention)
+    "gptoss_120b": dict(n_layers=36, hidden=2880, n_q_heads=64, n_kv_heads=8, head_dim=64, ffn=2880,
+                        n_experts=128, top_k=4, vocab=201088, rms_eps=1e-5, rope_theta=150000.0, attn_scale=0.125,
+                        dtype=ffi.BF16, expert_dtype=ffi.MXFP4, router_sigma=0.08,
+                        gptoss=dict(window=128, yarn=(32.0, 4096, 32.0, 1.0), act_alpha=1.702, act_limit=7.0)),
     # Qwen3-30B-A3B shape: 128 experts, top-8, MXFP4 experts, Q8_0 attention / router / head
     "qwen3_30b_a3b": dict(n_layers=48, hidden=2048, n_q_heads=32, n_kv_heads=4, head_dim=128, ffn=768,
                           n_experts=128, top_k=8, vocab=151936, rms_eps=1e-6, rope_theta=1000000.0,
@@ -57,8 +70,20 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
 
     L = cfg["n_layers"] if n_layers is None else n_layers
     E = int(cfg.get("n_experts", 0))
+    oss = cfg.get("gptoss")
+    brng = np.random.default_rng(seed + 7)
+
+    def vec(n, scale, dtype=ffi.F32):
+        """A small random vector (biases, sinks) stored as f32 or bf16."""
+        v = (brng.standard_normal((1, n)) * scale).astype(np.float32)
+        return ffi.quantize(dtype, v) if dtype != ffi.F32 else (ffi.F32, v.view(np.uint8).reshape(1, -1), 1, n)
+
+    if oss:
+        factor, octx, bf, bs = oss["yarn"]
+        cfg["rope_freqs"], cfg["rope_mscale"] = ffi.yarn_frequencies(cfg["head_dim"], cfg["rope_theta"], factor, octx, bf, bs)
+        cfg["act_alpha"], cfg["act_limit"] = oss["act_alpha"], oss["act_limit"]
     layers = []
-    for _ in range(L):
+    for li in range(L):
         lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H), wo=t(H, qd), ffn_norm=ones(H))
         if E:
             xd = cfg.get("expert_dtype", dt)
@@ -66,5 +91,16 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
                       we_gate=t(E * F, H, xd), we_up=t(E * F, H, xd), we_down=t(E * H, F, xd))
         else:
             lw.update(w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F))
+        if oss:
+            # attention biases and sinks are bf16 in the GGUF, expert and router biases f32
+            lw.update(bq=vec(qd, 0.05, ffi.BF16), bk=vec(kvd, 0.05, ffi.BF16), bv=vec(kvd, 0.05, ffi.BF16),
+                      bo=vec(H, 0.05, ffi.BF16), sinks=vec(cfg["n_q_heads"], 1.0, ffi.BF16),
+                      window=oss["window"] if li % 2 == 0 else 0)  # even layers slide (gptoss/attn.rs:20-23)
+            if E:
+                def mat(r, c, scale):
+                    v = (brng.standard_normal((r, c)) * scale).astype(np.float32)
+                    return (ffi.F32, v.view(np.uint8).reshape(r, -1), r, c)
+                lw.update(router_bias=vec(E, 0.05), be_gate=mat(E, F, 0.05), be_up=mat(E, F, 0.05),
+                          be_down=mat(E, H, 0.05))
         layers.append(lw)
     return dict(embed=t(V, H), final_norm=ones(H), lm_head=t(V, H), layers=layers)
