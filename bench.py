@@ -27,6 +27,9 @@ WORKLOADS = {
     # BASELINE configs[3]: routed experts (MXFP4) + Q8_0 attention, chain k=8, greedy
     "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(model="qwen3_30b_a3b", ctx=8192, k=8, temperature=0.0),
     "moe_small_k8_ctx256": dict(model="moe_small", ctx=256, k=8, temperature=0.0),
+    # BASELINE configs[4]: gpt-oss arrangement (bf16 + MXFP4 experts top-4, window / full layers), T = 1.0
+    "gptoss_120b_mxfp4_k8_ctx32768": dict(model="gptoss_120b", ctx=32768, k=8, temperature=1.0),
+    "gptoss_small_k8_ctx256": dict(model="gptoss_small", ctx=256, k=8, temperature=1.0),
 }
 
 
@@ -55,19 +58,22 @@ def algorithmic_bytes(cfg, ctx, m):
     head = rb(V, H)
     weights = L * sum(per_layer.values()) + head
     kv = L * (ctx + m) * kvd * 2 * 2
+    if cfg.get("gptoss"):  # even layers read only their window
+        win = (L + 1) // 2
+        kv = ((L - win) * (ctx + m) + win * min(cfg["gptoss"]["window"] + m, ctx + m)) * kvd * 2 * 2
     small = m * ffi.row_bytes(cfg["dtype"], H) + m * V * 2 + L * m * kvd * 2 * 2
     return dict(per_layer=per_layer, head=head, weights=weights, kv=kv, total=weights + kv + small)
 
 
 def trace_summary(path):
     """Per-kernel statistics of the verify STEPS in a `rocprofv3 --kernel-trace --output-format csv`
-    trace of this script: only dispatches after the first acceptance-statistics kernel are counted,
+    trace of this script: only dispatches from the first acceptance kernel on are counted,
     which leaves out weight re-tiling and the 16-row prefill passes that build the KV cache.
     Kernels are keyed by name and grid size, so the five matmul shapes show up separately."""
     import csv
     rows = list(csv.DictReader(open(path)))
     rows.sort(key=lambda r: int(r["Start_Timestamp"]))
-    start = next(i for i, r in enumerate(rows) if "k_row_max" in r["Kernel_Name"])
+    start = next(i for i, r in enumerate(rows) if "k_clear_result" in r["Kernel_Name"])
     stats = {}
     for r in rows[start:]:
         name = r["Kernel_Name"].replace("tsv::", "").replace("(anonymous namespace)::", "")
@@ -298,7 +304,7 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16",
-        "dtype_detail": ("q4_k" if cfg["dtype"] == 12 else "q8_0") + (" + mxfp4 experts" if cfg.get("n_experts") else "") +
+        "dtype_detail": {12: "q4_k", 8: "q8_0", 30: "bf16"}[cfg["dtype"]] + (" + mxfp4 experts" if cfg.get("n_experts") else "") +
                         " weight codes as exact f16 x f16 activations on MFMA, "
                         "f32 accumulate; f64 acceptance",
         "data": "synthetic",

@@ -201,6 +201,59 @@ int32_t tsv_verify_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result
 int32_t tsv_draft_chain(tsv_ctx* ctx, const uint16_t* draft_logits, int32_t k,
                         const tsv_shaping* shaping, uint64_t* draw_step, int32_t* proposals);
 
+/* ---- the generation loop (speculative.rs:194-900) and the adaptive depth ---------------- */
+/* Per-round draft depth controller, speculative_adaptive.rs:105-227: pure state.  A streak of
+ * fully accepted rounds (climb_low from depth 2-3, climb_mid from 4, climb_high from 5 up) climbs
+ * one step, `drop` accumulated missed proposals fall one step; never below floor or above cap. */
+typedef struct {
+    int32_t floor, cap, cur, climb, pressure;
+    int32_t climb_low, climb_mid, climb_high, drop;
+} tsv_adaptive;
+void tsv_adaptive_init(tsv_adaptive* a, int32_t floor, int32_t cap);       /* AdaptiveDepth::new, shipped tuning */
+int32_t tsv_adaptive_depth(const tsv_adaptive* a);                          /* depth() */
+void tsv_adaptive_observe(tsv_adaptive* a, int32_t offered, int32_t accepted); /* observe() */
+int32_t tsv_adaptive_tile_cap(int32_t cap, int32_t tile_rows);              /* tile_cap(); tile_rows <= 0: none */
+
+/* The draft side of SpeculativeProducer (producer.rs:164-260) as callbacks; non-zero = failure.
+ * prime(next, position): write the drafter's row for a token whose proposal is not needed;
+ * step(token, position, logits): the same and fill vocab fp16 logits (host memory);
+ * rewind(position): the drafter continues after the accepted prefix that ended at `position`. */
+typedef struct {
+    void* user;
+    int32_t (*prime)(void* user, int32_t next_token, int64_t position);
+    int32_t (*step)(void* user, int32_t token, int64_t position, uint16_t* logits);
+    int32_t (*rewind)(void* user, int64_t position);
+} tsv_drafter;
+
+typedef struct {
+    tsv_shaping shaping;
+    uint64_t max_new_tokens;     /* GenerationConfig::max_new_tokens, > 0 */
+    const int32_t* stop_tokens;  /* tokenizer stop ids + extra_stop_tokens */
+    int32_t n_stop;
+    int32_t block;               /* proposals per round (the cap when adaptive), 1..15 */
+    int32_t adaptive_floor;      /* 0: fixed block; else AdaptiveDepth(adaptive_floor, block) */
+} tsv_generation;
+
+typedef struct {
+    int32_t* tokens;   /* caller's buffer for the reported tokens */
+    int64_t capacity;  /* >= max_new_tokens */
+    int64_t n_tokens;
+    int32_t stop_reason; /* 1 stop token (not reported), 2 budget (its last token is reported) */
+    int32_t final_depth;
+    int64_t rounds, offered, accepted, rollbacks;
+    uint64_t draw_step;
+    int64_t kv_position;
+    double min_margin;
+} tsv_generation_result;
+
+/* run_speculative for the step-wise drafter and chain rounds: admission, headless prefill that
+ * primes the drafter, then rounds of draft -> verify + accept + truncate on the device ->
+ * rewind_drafter, never proposing past the budget or the context window (speculative.rs:448-459). */
+int32_t tsv_run_speculative(tsv_ctx* ctx, const tsv_drafter* drafter, const int32_t* prompt, int64_t n_prompt,
+                            const tsv_generation* config, tsv_generation_result* out);
+int64_t tsv_max_context(const tsv_ctx* ctx);
+int64_t tsv_vocab(const tsv_ctx* ctx);
+
 /* ---- install-time helpers (host) --------------------------------------------- */
 /* The reference's quantize-on-install encoders (q8_0.rs:56-77, q4_k.rs:126-204). */
 int64_t tsv_row_bytes(int32_t dtype, int64_t cols);

@@ -508,3 +508,104 @@ class Model:
     def compact_tree(self, base, path):
         p = np.ascontiguousarray(path, np.uint32)
         lib().tso_model_compact_tree(self._h, C.c_int64(base), _p(p), int(p.size))
+
+
+# ------------------------------------------------------- adaptive depth and the generation loop
+class Adaptive(C.Structure):
+    """crates/runtime/src/speculative_adaptive.rs:105-227."""
+    _fields_ = [("floor", C.c_int), ("cap", C.c_int), ("cur", C.c_int), ("climb", C.c_int),
+                ("pressure", C.c_int), ("params", C.c_int * 4)]
+
+    def __init__(self, floor, cap):
+        super().__init__()
+        lib().tso_adaptive_new(C.byref(self), floor, cap)
+
+    def depth(self):
+        return self.cur
+
+    def observe(self, offered, accepted):
+        lib().tso_adaptive_observe(C.byref(self), offered, accepted)
+
+    @staticmethod
+    def tile_cap(cap, tile_rows):
+        return lib().tso_adaptive_tile_cap(cap, tile_rows if tile_rows else 0)
+
+
+_CB_I = C.CFUNCTYPE(C.c_int, C.c_void_p)
+_CB_PRODUCE = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int32, C.c_int64, C.POINTER(C.c_uint16))
+_CB_TOKPOS = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int32, C.c_int64)
+_CB_VERIFY = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.c_int, C.c_int64, C.POINTER(C.c_uint16))
+_CB_ROLL = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64, C.c_int)
+_CB_POS = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64)
+
+
+class Producer(C.Structure):
+    _fields_ = [("user", C.c_void_p), ("reset", _CB_I), ("produce", _CB_PRODUCE), ("prefill", _CB_TOKPOS),
+                ("verify", _CB_VERIFY), ("rollback_retaining", _CB_ROLL), ("prime", _CB_TOKPOS),
+                ("step", _CB_PRODUCE), ("rewind", _CB_POS)]
+
+
+class Generation(C.Structure):
+    _fields_ = [("shaping", Shaping), ("max_new_tokens", C.c_uint64), ("stop_tokens", C.POINTER(C.c_int32)),
+                ("n_stop", C.c_int32), ("block", C.c_int32), ("adaptive_floor", C.c_int32)]
+
+
+class GenerationResult(C.Structure):
+    _fields_ = [("tokens", C.POINTER(C.c_int32)), ("n_tokens", C.c_int64), ("stop_reason", C.c_int32),
+                ("final_depth", C.c_int32), ("rounds", C.c_int64), ("offered", C.c_int64),
+                ("accepted", C.c_int64), ("rollbacks", C.c_int64), ("draw_step", C.c_uint64)]
+
+
+def run_speculative(target, drafter, prompt, cfg, max_new_tokens, block, vocab, max_context,
+                    stop_tokens=(), adaptive_floor=0):
+    """The reference loop over Python producers.  `target` offers reset(), produce(token, pos) ->
+    uint16[vocab], prefill(token, pos), verify(feed, base) -> uint16[m, vocab],
+    rollback_retaining(point, keep_rows); `drafter` offers prime(next, pos), step(token, pos) ->
+    uint16[vocab], rewind(pos)."""
+    def put(dst, arr, n):
+        C.memmove(dst, np.ascontiguousarray(arr, np.uint16).ctypes.data, n * 2)
+
+    def guard(fn):
+        def inner(*a):
+            try:
+                fn(*a)
+                return 0
+            except Exception as e:  # an exception cannot cross the C frame
+                errs.append(e)
+                return 1
+        return inner
+
+    errs = []
+    cbs = dict(
+        reset=_CB_I(guard(lambda u: target.reset())),
+        produce=_CB_PRODUCE(guard(lambda u, t, p, out: put(out, target.produce(t, p), vocab))),
+        prefill=_CB_TOKPOS(guard(lambda u, t, p: target.prefill(t, p))),
+        verify=_CB_VERIFY(guard(lambda u, f, m, b, out: put(out, target.verify([f[i] for i in range(m)], b), m * vocab))),
+        rollback_retaining=_CB_ROLL(guard(lambda u, pt, k: target.rollback_retaining(pt, k))),
+        prime=_CB_TOKPOS(guard(lambda u, t, p: drafter.prime(t, p))),
+        step=_CB_PRODUCE(guard(lambda u, t, p, out: put(out, drafter.step(t, p), vocab))),
+        rewind=_CB_POS(guard(lambda u, p: drafter.rewind(p))),
+    )
+    prod = Producer(None, *[cbs[k] for k in ("reset", "produce", "prefill", "verify", "rollback_retaining",
+                                             "prime", "step", "rewind")])
+    g = Generation()
+    g.shaping = cfg
+    g.max_new_tokens = max_new_tokens
+    st = np.ascontiguousarray(list(stop_tokens), np.int32)
+    g.stop_tokens = st.ctypes.data_as(C.POINTER(C.c_int32))
+    g.n_stop = st.size
+    g.block = block
+    g.adaptive_floor = adaptive_floor
+    toks = np.zeros(max_new_tokens + 1, np.int32)
+    res = GenerationResult()
+    res.tokens = toks.ctypes.data_as(C.POINTER(C.c_int32))
+    pr = np.ascontiguousarray(prompt, np.int32)
+    rc = lib().tso_run_speculative(C.byref(prod), _p(pr), C.c_int64(pr.size), C.byref(g), C.c_int64(max_context),
+                                   C.c_int64(vocab), C.byref(res))
+    if errs:
+        raise errs[0]
+    if rc < 0:
+        raise ValueError(f"run_speculative failed ({rc}): {last_error()}")
+    return dict(tokens=[int(t) for t in toks[: res.n_tokens]], stop_reason=res.stop_reason, rounds=res.rounds,
+                offered=res.offered, accepted=res.accepted, rollbacks=res.rollbacks, draw_step=res.draw_step,
+                final_depth=res.final_depth)

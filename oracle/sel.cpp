@@ -538,3 +538,179 @@ extern "C" int tso_tree_round_sampled(const uint16_t* target_logits, const uint1
     out->draw_step = draw_step;
     return 0;
 }
+
+// ---- adaptive depth: crates/runtime/src/speculative_adaptive.rs:105-227 ---------------------
+extern "C" void tso_adaptive_new(tso_adaptive* a, int floor, int cap) {
+    cap = std::max(cap, 1);
+    floor = std::min(std::max(floor, 1), cap);
+    *a = tso_adaptive{floor, cap, floor, 0, 0, {8, 6, 4, 2}};  // AdaptiveParams::default (:46-55)
+}
+extern "C" int tso_adaptive_tile_cap(int cap, int tile_rows) {
+    if (tile_rows <= 0) return cap;  // None
+    return std::min(cap, std::max(tile_rows - 1, 1));
+}
+static int adaptive_climb(const tso_adaptive* a, int depth) {  // AdaptiveParams::climb (:60-67)
+    if (depth <= 1) return 2;
+    if (depth == 2 || depth == 3) return a->params[0];
+    if (depth == 4) return a->params[1];
+    return a->params[2];
+}
+extern "C" void tso_adaptive_observe(tso_adaptive* a, int offered, int accepted) {
+    if (offered == 0) return;
+    accepted = std::min(accepted, offered);
+    if (accepted == offered) {
+        a->pressure = 0;
+        if (a->cur < a->cap) {
+            a->climb += 1;
+            if (a->climb >= adaptive_climb(a, a->cur)) {
+                a->cur += 1;
+                a->climb = 0;
+            }
+        }
+    } else {
+        a->climb = 0;
+        if (a->cur > a->floor) {
+            a->pressure += offered - accepted;
+            if (a->pressure >= a->params[3]) {
+                a->cur -= 1;
+                a->pressure = 0;
+            }
+        }
+    }
+}
+
+// ---- the loop: crates/runtime/src/speculative.rs:194-900, step-wise drafter, chain rounds ----
+// Generic over the producer, like the reference (`run_speculative<P: SpeculativeProducer>`): the
+// callbacks are the trait's methods.  Acceptance is the host code above.
+extern "C" int tso_run_speculative(const tso_producer* p, const int32_t* prompt, int64_t n,
+                                   const tso_generation* g, int64_t max_context, int64_t vocab,
+                                   tso_generation_result* out) {
+    // raw_completion.rs:126-146
+    if (n < 1) {
+        tso_set_error("empty prompt");
+        return -1;
+    }
+    if (g->max_new_tokens == 0) {
+        tso_set_error("zero budget");
+        return -1;
+    }
+    if ((uint64_t)n + g->max_new_tokens > (uint64_t)max_context) {
+        tso_set_error("context overflow");
+        return -1;
+    }
+    if (g->block == 0) {
+        tso_set_error("block size 0 proposes nothing");
+        return -1;
+    }
+    if (need_seed(&g->shaping)) return -3;
+    const tso_shaping* cfg = &g->shaping;
+    const bool sampled = !deterministic(cfg);
+    tso_adaptive ad;
+    const bool adaptive = g->adaptive_floor > 0;
+    if (adaptive) tso_adaptive_new(&ad, g->adaptive_floor, g->block);
+    std::memset(&out->n_tokens, 0, sizeof(*out) - offsetof(tso_generation_result, n_tokens));
+
+    p->reset(p->user);
+    std::vector<uint16_t> logits((size_t)vocab), draft_rows((size_t)g->block * vocab),
+        batch((size_t)(g->block + 1) * vocab);
+    int64_t position = 0;
+    std::vector<int32_t> history;
+    for (int64_t i = 0; i < n; i++) {  // :337-372
+        const bool last = i + 1 == n;
+        int rc = last ? p->produce(p->user, prompt[i], position, logits.data())
+                      : p->prefill(p->user, prompt[i], position);
+        if (rc) return -10;
+        if (i + 1 < n && p->prime(p->user, prompt[i + 1], i)) return -10;
+        position += 1;
+        history.push_back(prompt[i]);
+    }
+    Sink sink{history, 0, g->max_new_tokens, g->stop_tokens, g->n_stop};
+    uint64_t draw_step = 0;
+    int32_t next;
+    int rc = select_token(logits.data(), vocab, cfg, sink.history.data(), (int64_t)sink.history.size(),
+                          sink.generated, &next);
+    if (rc < 0) return rc;
+    auto report = [&](int32_t t) { out->tokens[out->n_tokens++] = t; };
+    std::vector<int32_t> proposals, feed;
+    for (;;) {
+        // TokenSink::commit reports every token but a stop token (token_sink.rs:64-124)
+        const bool stop_tok = std::find(g->stop_tokens, g->stop_tokens + g->n_stop, next) != g->stop_tokens + g->n_stop;
+        if (!stop_tok) report(next);
+        if (int why = sink.commit(next)) {
+            out->stop_reason = why;
+            break;
+        }
+        const int64_t base = (int64_t)sink.history.size() - 1;
+        position = (int64_t)sink.history.size();
+        // :448-459
+        const uint64_t budget_room = g->max_new_tokens - sink.generated;
+        const uint64_t context_room = (uint64_t)std::max<int64_t>(max_context - position, 0);
+        const uint64_t wanted = adaptive ? (uint64_t)std::min(ad.cur, g->block) : (uint64_t)g->block;
+        const int round_block = (int)std::min(std::min(wanted, budget_room), context_room);
+        const bool truncated = (uint64_t)round_block < wanted;
+        if (round_block == 0) {
+            tso_set_error("round_block is 0: no room after admission; invariant violation");
+            return -11;
+        }
+        // :606-660
+        proposals.clear();
+        int32_t chained = next;
+        for (int d = 0; d <= round_block; d++) {
+            if (d == round_block) {
+                if (p->prime(p->user, chained, base - 1 + d)) return -10;
+                if (sampled) draw_step += 1;
+                break;
+            }
+            uint16_t* row = draft_rows.data() + (size_t)d * vocab;
+            if (p->step(p->user, chained, base - 1 + d, row)) return -10;
+            if (sampled) {
+                Dist q;
+                rc = shaped(row, vocab, cfg, sink.history.data(), (int64_t)sink.history.size(), sink.generated, q);
+                if (rc < 0) return rc;
+                chained = (int32_t)draw(q, cfg->seed, draw_step);
+                draw_step += 1;
+            } else {
+                rc = select_token(row, vocab, cfg, sink.history.data(), (int64_t)sink.history.size(),
+                                  sink.generated, &chained);
+                if (rc < 0) return rc;
+            }
+            proposals.push_back(chained);
+        }
+        // :663-676
+        feed.assign(1, next);
+        feed.insert(feed.end(), proposals.begin(), proposals.end());
+        const int64_t point = base;
+        if (p->verify(p->user, feed.data(), (int)feed.size(), base, batch.data())) return -10;
+        // :694-754, 861-879
+        tso_round_result res;
+        rc = tso_chain_round(batch.data(), sampled ? draft_rows.data() : nullptr, proposals.data(), round_block,
+                             vocab, cfg, sink.history.data(), (int64_t)sink.history.size(), sink.generated,
+                             g->max_new_tokens, g->stop_tokens, g->n_stop, draw_step, &res);
+        if (rc < 0) return rc;
+        out->rounds += 1;
+        out->offered += round_block;
+        out->accepted += res.accepted;
+        if (adaptive && !truncated && !res.stopped) tso_adaptive_observe(&ad, round_block, res.accepted);
+        for (int i = 0; i < res.accepted; i++) {
+            const int32_t t = proposals[i];
+            const bool st = std::find(g->stop_tokens, g->stop_tokens + g->n_stop, t) != g->stop_tokens + g->n_stop;
+            if (!st) report(t);
+            sink.commit(t);  // the same calls the round made on its copy of the sink
+        }
+        const int committed = res.committed;
+        if (committed < round_block) {  // :800-814
+            out->rollbacks += 1;
+            if (p->rollback_retaining(p->user, point, committed + 1)) return -10;
+        }
+        if (p->rewind(p->user, base + committed)) return -10;  // :852-854
+        draw_step = res.draw_step;
+        if (res.stopped) {
+            out->stop_reason = res.stopped;
+            break;
+        }
+        next = res.next;
+    }
+    out->draw_step = draw_step;
+    out->final_depth = adaptive ? ad.cur : g->block;
+    return 0;
+}

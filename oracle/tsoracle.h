@@ -170,6 +170,47 @@ int tso_tree_round_sampled(const uint16_t* target_logits, const uint16_t* draft_
                            const tso_shaping* cfg, const int32_t* history, int64_t n_history,
                            uint64_t generated, uint64_t draw_step, tso_round_result* out);
 
+/* ---- adaptive depth and the generation loop ---------------------------------------- */
+/* crates/runtime/src/speculative_adaptive.rs:105-227; params = {climb_low, climb_mid, climb_high, drop} */
+typedef struct {
+    int floor, cap, cur, climb, pressure;
+    int params[4];
+} tso_adaptive;
+void tso_adaptive_new(tso_adaptive* a, int floor, int cap);
+void tso_adaptive_observe(tso_adaptive* a, int offered, int accepted);
+int tso_adaptive_tile_cap(int cap, int tile_rows); /* tile_rows <= 0: None */
+
+/* The producer traits of crates/runtime/src/producer.rs:17-387 as callbacks (non-zero = error). */
+typedef struct {
+    void* user;
+    int (*reset)(void* user);
+    int (*produce)(void* user, int32_t token, int64_t position, uint16_t* logits);
+    int (*prefill)(void* user, int32_t token, int64_t position); /* produce_prefill: no logits */
+    int (*verify)(void* user, const int32_t* feed, int m, int64_t base, uint16_t* logits);
+    int (*rollback_retaining)(void* user, int64_t point, int keep_rows);
+    int (*prime)(void* user, int32_t next_token, int64_t position);
+    int (*step)(void* user, int32_t token, int64_t position, uint16_t* logits);
+    int (*rewind)(void* user, int64_t position);
+} tso_producer;
+typedef struct {
+    tso_shaping shaping;
+    uint64_t max_new_tokens;
+    const int32_t* stop_tokens;
+    int32_t n_stop;
+    int32_t block, adaptive_floor; /* adaptive_floor 0: fixed block */
+} tso_generation;
+typedef struct {
+    int32_t* tokens; /* caller's buffer, >= max_new_tokens */
+    int64_t n_tokens;
+    int32_t stop_reason, final_depth; /* 1 stop token, 2 budget */
+    int64_t rounds, offered, accepted, rollbacks;
+    uint64_t draw_step;
+} tso_generation_result;
+/* crates/runtime/src/speculative.rs:194-900 for the step-wise drafter and chain rounds. */
+int tso_run_speculative(const tso_producer* p, const int32_t* prompt, int64_t n_prompt,
+                        const tso_generation* g, int64_t max_context, int64_t vocab,
+                        tso_generation_result* out);
+
 /* ---- Llama-style target model ------------------------------------------ */
 typedef struct {
     const void* data; /* row-major, one byte run per output row */

@@ -1,0 +1,94 @@
+"""The library's generation loop (device acceptance, device truncation) against the oracle's
+restatement of crates/runtime/src/speculative.rs:194-900 driving the SAME GPU target through
+`verify` + host acceptance: both see identical logits, so the reported tokens, the stop reason
+and every counter must agree exactly."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from tests import gpu_common as gc
+from tests.loop_common import GpuTarget, LmDrafter
+
+pytestmark = pytest.mark.gpu
+
+KEYS = ("tokens", "stop_reason", "rounds", "offered", "accepted", "rollbacks", "draw_step", "final_depth")
+
+
+def _pair(name="tiny_q8_0", max_context=200, draft_seed=1234):
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg, w, gpu, _ = gc.build_pair(name, max_context=max_context)
+    dcfg = dict(synth.CONFIGS[name], max_context=max_context)
+    dw = w if draft_seed == 1234 else synth.make_weights(dcfg, seed=draft_seed)
+    return cfg, gpu, ts.HipVerifier(dcfg, dw)
+
+
+@pytest.mark.parametrize("temperature,kw,block,floor,noise,draft_seed", [
+    (0.0, {}, 4, 0, 0.0, 77),          # greedy, a drafter that is usually wrong
+    (0.0, {}, 4, 0, 1.0, 1234),        # greedy, the target plus noise: mixed acceptance
+    (0.0, {}, 8, 2, 0.3, 1234),        # adaptive depth
+    (0.8, {}, 4, 0, 1.0, 1234),        # rejection sampling
+    (1.0, dict(top_p=0.95, top_k=50), 8, 2, 0.5, 1234),
+    (0.7, dict(min_p=0.02), 15, 0, 0.0, 1234),   # the widest block, a perfect drafter
+])
+def test_the_device_loop_reports_what_the_reference_loop_reports(temperature, kw, block, floor, noise, draft_seed):
+    import turbospark_amd as ts
+    cfg, gpu, lm = _pair(draft_seed=draft_seed)
+    V = cfg["vocab"]
+    prompt = np.random.default_rng(3).integers(0, V, 19).astype(np.int32)
+    seed = 41 if temperature else None
+    gcfg, ocfg = ts.shaping(temperature, seed=seed, **kw), ob.shaping(temperature, seed=seed, **kw)
+    new = 70
+    want = ob.run_speculative(GpuTarget(gpu), LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), prompt, ocfg, new, block,
+                              V, cfg["max_context"], adaptive_floor=floor)
+    got = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), gcfg, new, block,
+                              adaptive_floor=floor)
+    print({k: (got[k] if k != "tokens" else len(got[k])) for k in KEYS}, "min margin", got["min_margin"])
+    assert {k: got[k] for k in KEYS} == {k: want[k] for k in KEYS}
+    assert len(got["tokens"]) == new and got["stop_reason"] == 2
+    assert got["kv_position"] == len(prompt) + new - 1 == gpu.position
+    assert got["min_margin"] > 1e-9
+    if noise:
+        assert 0 < got["accepted"] < got["offered"]
+    # a stop token taken from the stream ends the run there, unreported
+    stop = got["tokens"][23]
+    first = got["tokens"].index(stop)
+    again = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), gcfg, new, block,
+                                stop_tokens=[stop], adaptive_floor=floor)
+    ref = ob.run_speculative(GpuTarget(gpu), LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), prompt, ocfg, new, block,
+                             V, cfg["max_context"], stop_tokens=[stop], adaptive_floor=floor)
+    assert {k: again[k] for k in KEYS} == {k: ref[k] for k in KEYS}
+    assert again["stop_reason"] == 1 and again["tokens"] == got["tokens"][:first]
+
+
+def test_greedy_speculation_on_the_device_equals_plain_decoding():
+    import turbospark_amd as ts
+    cfg, gpu, lm = _pair(draft_seed=77)
+    V = cfg["vocab"]
+    prompt = np.random.default_rng(5).integers(0, V, 12).astype(np.int32)
+    got = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V), ts.shaping(0.0), 50, 5)
+    gpu.reset()
+    gpu.prefill(prompt[:-1], 0, want_logits=False)
+    tok, plain = int(prompt[-1]), []
+    for i in range(50):
+        tok = int(np.argmax(gc.f16(gpu.produce(tok, len(prompt) - 1 + i))))
+        plain.append(tok)
+    assert got["tokens"] == plain
+
+
+def test_the_loop_stays_inside_the_context_window_and_refuses_bad_requests():
+    import turbospark_amd as ts
+    cfg, gpu, lm = _pair(max_context=64)
+    V = cfg["vocab"]
+    prompt = np.arange(3, 23).astype(np.int32)
+    got = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V), ts.shaping(0.0), 44, 15)
+    assert len(got["tokens"]) == 44 and got["kv_position"] == 63
+    for kwargs, text in ((dict(max_new_tokens=45), "overflow"), (dict(max_new_tokens=0), "zero"), (dict(block=0), "block"),
+                         (dict(block=16), "block")):
+        args = dict(max_new_tokens=10, block=4)
+        args.update(kwargs)
+        with pytest.raises(ts.TsvError, match=text):
+            gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V), ts.shaping(0.0), args["max_new_tokens"],
+                                args["block"])
+    with pytest.raises(ts.TsvError, match="empty"):
+        gpu.run_speculative([], LmDrafter(GpuTarget(lm), 0, V), ts.shaping(0.0), 4, 2)

@@ -1,0 +1,238 @@
+// Host loop of speculative generation over the device verify step, and the adaptive draft depth.
+//
+// Restates crates/runtime/src/speculative.rs:194-900 (`run_speculative`, step-wise drafter, chain
+// rounds) for a target that lives behind this library: admission (raw_completion.rs:126-146),
+// headless prefill priming the drafter, then rounds of  commit(next) -> cap the block by budget
+// and context (:448-459) -> draft_step x block + the row-only prime (:606-660) -> ONE call that
+// verifies, accepts on the device and truncates the KV -> observe (:760-765) -> rewind_drafter.
+// The token sink is the token-id part of crates/runtime/src/token_sink.rs:64-124: a stop token is
+// not reported, the token that exhausts the budget is; neither enters the history.
+// The controller is crates/runtime/src/speculative_adaptive.rs:105-227.
+#include <algorithm>
+#include <vector>
+
+#include "tsv_internal.h"
+
+using namespace tsv;
+
+// ---- adaptive depth ----------------------------------------------------------------------
+extern "C" void tsv_adaptive_init(tsv_adaptive* a, int32_t floor, int32_t cap) {
+    // shipped tuning (speculative_adaptive.rs:170-190): streaks of 8 / 6 / 4 clean rounds climb
+    // from depth 2-3 / 4 / 5+, two missed proposals drop a step
+    a->cap = std::max(cap, 1);
+    a->floor = std::min(std::max(floor, 1), a->cap);
+    a->cur = a->floor;
+    a->climb = a->pressure = 0;
+    a->climb_low = 8;
+    a->climb_mid = 6;
+    a->climb_high = 4;
+    a->drop = 2;
+}
+
+extern "C" int32_t tsv_adaptive_depth(const tsv_adaptive* a) { return a->cur; }
+
+extern "C" int32_t tsv_adaptive_tile_cap(int32_t cap, int32_t tile_rows) {
+    return tile_rows > 0 ? std::min(cap, std::max(tile_rows - 1, 1)) : cap;
+}
+
+static int climb_needed(const tsv_adaptive* a, int depth) {
+    return depth <= 1 ? 2 : depth <= 3 ? a->climb_low : depth == 4 ? a->climb_mid : a->climb_high;
+}
+
+extern "C" void tsv_adaptive_observe(tsv_adaptive* a, int32_t offered, int32_t accepted) {
+    if (offered <= 0) return;  // an empty round is not a signal
+    accepted = std::min(accepted, offered);
+    if (accepted == offered) {
+        a->pressure = 0;
+        if (a->cur < a->cap && ++a->climb >= climb_needed(a, a->cur)) {
+            a->cur += 1;
+            a->climb = 0;
+        }
+        return;
+    }
+    a->climb = 0;
+    if (a->cur > a->floor) {  // at the floor there is nowhere to fall and no pressure builds
+        a->pressure += offered - accepted;
+        if (a->pressure >= a->drop) {
+            a->cur -= 1;
+            a->pressure = 0;
+        }
+    }
+}
+
+// ---- the loop ------------------------------------------------------------------------------
+namespace {
+
+struct Emit {
+    tsv_generation_result* out;
+    int push(int32_t t) {
+        if (out->n_tokens >= out->capacity) {
+            set_error("run_speculative: the token buffer is smaller than the budget");
+            return TSV_ERR_INVALID;
+        }
+        out->tokens[out->n_tokens++] = t;
+        return TSV_OK;
+    }
+};
+
+bool is_stop(const tsv_generation* g, int32_t t) {
+    for (int i = 0; i < g->n_stop; i++)
+        if (g->stop_tokens[i] == t) return true;
+    return false;
+}
+
+// select() of one logits row at draw position `position` (choose.rs:61-98): arg-max, or a draw
+// from the shaped distribution
+int select_row(tsv_ctx* c, const uint16_t* row, const tsv_shaping* sh, uint64_t position, int32_t* token) {
+    uint64_t at = position;
+    return tsv_draft_chain(c, row, 1, sh, &at, token);
+}
+
+}  // namespace
+
+extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const int32_t* prompt, int64_t n,
+                                       const tsv_generation* g, tsv_generation_result* out) {
+    if (!c || !dr || !dr->prime || !dr->step || !dr->rewind || !prompt || !g || !out || !out->tokens) {
+        set_error("run_speculative: null argument");
+        return TSV_ERR_INVALID;
+    }
+    const int64_t max_context = tsv_max_context(c);
+    const int64_t vocab = tsv_vocab(c);
+    // check_admission
+    if (n < 1) {
+        set_error("run_speculative: empty prompt");
+        return TSV_ERR_INVALID;
+    }
+    if (g->max_new_tokens == 0) {
+        set_error("run_speculative: zero generation budget");
+        return TSV_ERR_INVALID;
+    }
+    if ((uint64_t)n + g->max_new_tokens > (uint64_t)max_context) {
+        set_error("run_speculative: prompt plus budget overflow the context window");
+        return TSV_ERR_INVALID;
+    }
+    if (g->block < 1 || g->block > TSV_MAX_ROWS - 1) {
+        set_error("run_speculative: block must be 1..15 (block size 0 proposes nothing)");
+        return TSV_ERR_INVALID;
+    }
+    if (g->n_stop < 0 || g->n_stop > 16 || (g->n_stop && !g->stop_tokens)) {
+        set_error("run_speculative: at most 16 stop tokens");
+        return TSV_ERR_INVALID;
+    }
+    const bool sampled = g->shaping.temperature != 0.0;
+    tsv_adaptive ad;
+    const bool adaptive = g->adaptive_floor > 0;
+    if (adaptive) tsv_adaptive_init(&ad, g->adaptive_floor, g->block);
+    out->n_tokens = 0;
+    out->stop_reason = 0;
+    out->rounds = out->offered = out->accepted = out->rollbacks = 0;
+    out->draw_step = 0;
+    out->min_margin = 1.0;
+    out->final_depth = adaptive ? ad.cur : g->block;
+    Emit emit{out};
+
+    int rc;
+    if ((rc = tsv_reset(c))) return rc;
+    std::vector<uint16_t> logits((size_t)vocab), rows((size_t)g->block * vocab);
+    // prefill: every prompt token but the last skips the output head; the drafter is primed with
+    // each known next token
+    if (n > 1 && (rc = tsv_prefill(c, prompt, n - 1, 0, nullptr))) return rc;
+    for (int64_t i = 0; i + 1 < n; i++)
+        if (dr->prime(dr->user, prompt[i + 1], i)) {
+            set_error("run_speculative: prime_drafter failed");
+            return TSV_ERR_INVALID;
+        }
+    if ((rc = tsv_produce(c, prompt[n - 1], n - 1, logits.data()))) return rc;
+    int64_t history = n;  // tokens backed by KV rows or about to be
+    uint64_t generated = 0, draw_step = 0;
+    int32_t next;
+    if ((rc = select_row(c, logits.data(), &g->shaping, generated, &next))) return rc;
+
+    int32_t feed[TSV_MAX_ROWS];
+    for (;;) {
+        // sink.commit(next)
+        generated += 1;
+        if (is_stop(g, next)) {
+            out->stop_reason = 1;
+            break;
+        }
+        if ((rc = emit.push(next))) return rc;
+        if (generated >= g->max_new_tokens) {
+            out->stop_reason = 2;
+            break;
+        }
+        history += 1;
+        const int64_t base = history - 1, position = history;
+        const uint64_t budget_room = g->max_new_tokens - generated;
+        const int64_t context_room = max_context - position;
+        const int wanted = adaptive ? std::min(tsv_adaptive_depth(&ad), g->block) : g->block;
+        const int round_block = (int)std::min<uint64_t>(std::min<uint64_t>((uint64_t)wanted, budget_room),
+                                                        (uint64_t)std::max<int64_t>(context_room, 0));
+        const bool truncated = round_block < wanted;
+        if (round_block == 0) {
+            set_error("run_speculative: round_block is 0: no room after admission; invariant violation");
+            return TSV_ERR_INVALID;
+        }
+        // draft: block steps, each proposal drawn from the drafter's own distribution (or its
+        // arg-max), then the row-only step that primes the drafter with the last proposal
+        feed[0] = next;
+        int32_t chained = next;
+        for (int d = 0; d <= round_block; d++) {
+            if (d == round_block) {
+                if (dr->prime(dr->user, chained, base - 1 + d)) {
+                    set_error("run_speculative: prime_drafter failed");
+                    return TSV_ERR_INVALID;
+                }
+                if (sampled) draw_step += 1;
+                break;
+            }
+            uint16_t* row = rows.data() + (size_t)d * vocab;
+            if (dr->step(dr->user, chained, base - 1 + d, row)) {
+                set_error("run_speculative: draft_step failed");
+                return TSV_ERR_INVALID;
+            }
+            if ((rc = select_row(c, row, &g->shaping, sampled ? draw_step : generated, &chained))) return rc;
+            if (sampled) draw_step += 1;
+            feed[1 + d] = chained;
+        }
+        // verify + accept + truncate
+        tsv_round r{};
+        r.feed = feed;
+        r.m = round_block + 1;
+        r.base = base;
+        r.shaping = g->shaping;
+        r.draft_logits = sampled ? rows.data() : nullptr;
+        r.draw_step = draw_step;
+        r.stop_tokens = g->stop_tokens;
+        r.n_stop = g->n_stop;
+        r.generated = generated;
+        r.max_new_tokens = g->max_new_tokens;
+        tsv_round_result res{};
+        if ((rc = tsv_verify_accept(c, &r, &res))) return rc;
+        out->rounds += 1;
+        out->offered += round_block;
+        out->accepted += res.accepted;
+        out->min_margin = std::min(out->min_margin, res.min_margin);
+        if (adaptive && !truncated && !res.stopped) tsv_adaptive_observe(&ad, round_block, res.accepted);
+        if (res.committed < round_block) out->rollbacks += 1;
+        for (int i = 0; i < res.committed; i++)
+            if ((rc = emit.push(feed[1 + i]))) return rc;
+        if (res.stopped == 2 && (rc = emit.push(feed[1 + res.committed]))) return rc;  // the budget's last token is reported
+        generated += (uint64_t)res.accepted;
+        history += res.committed;
+        draw_step = res.draw_step;
+        if (dr->rewind(dr->user, base + res.committed)) {
+            set_error("run_speculative: rewind_drafter failed");
+            return TSV_ERR_INVALID;
+        }
+        if (res.stopped) {
+            out->stop_reason = res.stopped;
+            break;
+        }
+        next = res.next;
+    }
+    out->draw_step = draw_step;
+    out->final_depth = adaptive ? ad.cur : g->block;
+    out->kv_position = tsv_kv_position(c);
+    return TSV_OK;
+}

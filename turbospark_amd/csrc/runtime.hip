@@ -933,6 +933,8 @@ extern "C" int32_t tsv_reset(tsv_ctx* c) {
 }
 
 extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c->position; }
+extern "C" int64_t tsv_max_context(const tsv_ctx* c) { return c->max_context; }
+extern "C" int64_t tsv_vocab(const tsv_ctx* c) { return c->vocab; }
 
 extern "C" int32_t tsv_verify(tsv_ctx* c, const int32_t* feed, int32_t m, int64_t base, uint16_t* logits) {
     int rc = enqueue_verify(c, feed, nullptr, m, base);

@@ -82,6 +82,49 @@ def shaping(temperature=0.0, top_k=0, top_p=None, repetition_penalty=1.0, seed=N
     return s
 
 
+class AdaptiveDepth(C.Structure):
+    """`AdaptiveDepth` of crates/runtime/src/speculative_adaptive.rs:105-227 (state lives here, the
+    transitions in the library)."""
+    _fields_ = [("floor", C.c_int32), ("cap", C.c_int32), ("cur", C.c_int32), ("climb", C.c_int32),
+                ("pressure", C.c_int32), ("climb_low", C.c_int32), ("climb_mid", C.c_int32),
+                ("climb_high", C.c_int32), ("drop", C.c_int32)]
+
+    def __init__(self, floor, cap):
+        super().__init__()
+        lib().tsv_adaptive_init(C.byref(self), floor, cap)
+
+    def depth(self):
+        return lib().tsv_adaptive_depth(C.byref(self))
+
+    def observe(self, offered, accepted):
+        lib().tsv_adaptive_observe(C.byref(self), offered, accepted)
+
+    @staticmethod
+    def tile_cap(cap, tile_rows=None):
+        return lib().tsv_adaptive_tile_cap(cap, tile_rows or 0)
+
+
+DRAFT_PRIME = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64)
+DRAFT_STEP = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.POINTER(C.c_uint16))
+DRAFT_REWIND = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int64)
+
+
+class Drafter(C.Structure):
+    _fields_ = [("user", C.c_void_p), ("prime", DRAFT_PRIME), ("step", DRAFT_STEP), ("rewind", DRAFT_REWIND)]
+
+
+class Generation(C.Structure):
+    _fields_ = [("shaping", Shaping), ("max_new_tokens", C.c_uint64), ("stop_tokens", C.POINTER(C.c_int32)),
+                ("n_stop", C.c_int32), ("block", C.c_int32), ("adaptive_floor", C.c_int32)]
+
+
+class GenerationResult(C.Structure):
+    _fields_ = [("tokens", C.POINTER(C.c_int32)), ("capacity", C.c_int64), ("n_tokens", C.c_int64),
+                ("stop_reason", C.c_int32), ("final_depth", C.c_int32), ("rounds", C.c_int64),
+                ("offered", C.c_int64), ("accepted", C.c_int64), ("rollbacks", C.c_int64),
+                ("draw_step", C.c_uint64), ("kv_position", C.c_int64), ("min_margin", C.c_double)]
+
+
 class Point(C.Structure):
     _fields_ = [("position", C.c_int64)]
 
@@ -109,7 +152,8 @@ EXPORTS = [
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
     "tsv_synth_tensor", "tsv_read_kv", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
-    "tsv_yarn_frequencies",
+    "tsv_yarn_frequencies", "tsv_adaptive_init", "tsv_adaptive_depth", "tsv_adaptive_observe", "tsv_adaptive_tile_cap",
+    "tsv_run_speculative", "tsv_max_context", "tsv_vocab",
 ]
 
 _lib = None
@@ -128,6 +172,14 @@ def lib():
         L.tsv_stream.argtypes = [C.c_void_p]
         L.tsv_kv_position.restype = C.c_int64
         L.tsv_kv_position.argtypes = [C.c_void_p]
+        L.tsv_max_context.restype = C.c_int64
+        L.tsv_max_context.argtypes = [C.c_void_p]
+        L.tsv_vocab.restype = C.c_int64
+        L.tsv_vocab.argtypes = [C.c_void_p]
+        L.tsv_adaptive_observe.restype = None
+        L.tsv_adaptive_init.restype = None
+        L.tsv_run_speculative.argtypes = [C.c_void_p, C.POINTER(Drafter), C.c_void_p, C.c_int64,
+                                          C.POINTER(Generation), C.POINTER(GenerationResult)]
         L.tsv_row_bytes.restype = C.c_int64
         L.tsv_row_bytes.argtypes = [C.c_int32, C.c_int64]
         L.tsv_yarn_frequencies.argtypes = [C.c_int32, C.c_float, C.c_float, C.c_int64, C.c_float, C.c_float,

@@ -216,6 +216,52 @@ class HipVerifier:
         ffi.check(ffi.lib().tsv_draft_chain(self._h, ptr, k, C.byref(cfg), C.byref(ds), props.ctypes.data))
         return props, ds.value
 
+    # ---- the generation loop --------------------------------------------------------------
+    def run_speculative(self, prompt, drafter, cfg, max_new_tokens, block, stop_tokens=(), adaptive_floor=0):
+        """`run_speculative` (crates/runtime/src/speculative.rs:194-900) for a step-wise drafter and
+        chain rounds, acceptance and truncation on the device.  `drafter` offers prime(next, pos),
+        step(token, pos) -> uint16[vocab] and rewind(pos).  Returns a dict with the reported tokens,
+        the stop reason (1 stop token, 2 budget) and the round statistics."""
+        vocab = self.vocab
+        failure = []
+
+        def guard(fn):
+            def inner(*a):
+                try:
+                    fn(*a)
+                    return 0
+                except Exception as e:  # an exception cannot cross the C frame
+                    failure.append(e)
+                    return 1
+            return inner
+
+        def step(user, token, pos, out):
+            row = np.ascontiguousarray(drafter.step(token, pos), np.uint16)
+            C.memmove(out, row.ctypes.data, vocab * 2)
+
+        d = ffi.Drafter(None, ffi.DRAFT_PRIME(guard(lambda u, t, p: drafter.prime(t, p))),
+                        ffi.DRAFT_STEP(guard(step)), ffi.DRAFT_REWIND(guard(lambda u, p: drafter.rewind(p))))
+        g = ffi.Generation()
+        g.shaping = cfg
+        g.max_new_tokens = int(max_new_tokens)
+        st = _i32(list(stop_tokens))
+        g.stop_tokens = st.ctypes.data_as(C.POINTER(C.c_int32))
+        g.n_stop = st.size
+        g.block = int(block)
+        g.adaptive_floor = int(adaptive_floor)
+        toks = np.zeros(int(max_new_tokens) + 1, np.int32)
+        res = ffi.GenerationResult()
+        res.tokens = toks.ctypes.data_as(C.POINTER(C.c_int32))
+        res.capacity = toks.size
+        pr = _i32(prompt)
+        rc = ffi.lib().tsv_run_speculative(self._h, C.byref(d), pr.ctypes.data, pr.size, C.byref(g), C.byref(res))
+        if failure:
+            raise failure[0]
+        ffi.check(rc)
+        return dict(tokens=[int(t) for t in toks[: res.n_tokens]], stop_reason=res.stop_reason, rounds=res.rounds,
+                    offered=res.offered, accepted=res.accepted, rollbacks=res.rollbacks, draw_step=res.draw_step,
+                    final_depth=res.final_depth, kv_position=res.kv_position, min_margin=res.min_margin)
+
     PROFILE_CLASSES = ("embed", "norm", "qkv", "rope_kv", "attention", "wo", "gate_up", "down", "head", "accept",
                        "event_pair")
 
