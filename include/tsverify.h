@@ -272,6 +272,10 @@ int32_t tsv_synth_tensor(int32_t dtype, uint64_t seed, uint64_t stream, float si
 /* Copies layer `layer`'s K and V rows [pos0, pos0+n) to host as fp16 in the reference
  * layout [position][kv_head][head_dim] (crates/gpu/src/kv_cache.rs:1-10). */
 int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v);
+/* The inverse: stores n rows of K and V (same host layout) at cache positions [pos0, pos0+n) of
+ * one layer and moves the cursor to at least pos0 + n -- a long context without the prefill that
+ * would build it (the full-size parity cases; also how a saved prefix would be restored). */
+int32_t tsv_write_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k, const uint16_t* v);
 /* One quantized small-M matmul through the same kernels the forward uses:
  * y[m][r] = sum_k W[r][k] x[m][k]; x is m x cols fp32 (rounded to fp16 on entry), y is
  * m x rows fp32.  W host tensor in GGUF layout (re-tiled per call).  `splits` <= 0 picks

@@ -1,0 +1,93 @@
+"""Parity at the benchmark configurations' real shapes: two layers + output head of the Llama-3-8B
+geometry (hidden 4096, 32q / 8kv x 128, ffn 14336, vocab 128256, Q4_K) at a 4096-token context,
+chain k = 4 and the 16-node tree; KV rows are seeded values written into both caches (prefilling
+4096 tokens through the CPU oracle is not feasible), the new rows come from the pass itself."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from tests import gpu_common as gc
+
+pytestmark = pytest.mark.gpu
+
+
+def _filled(name, ctx, n_layers, seed=3, **over):
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS[name])
+    cfg.update(n_layers=n_layers, max_context=ctx + 32, **over)
+    w = synth.make_weights(cfg, seed=seed, n_layers=n_layers)
+    gpu = ts.HipVerifier(cfg, w)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)
+    rng = np.random.default_rng(seed)
+    for layer in range(n_layers):
+        shape = (ctx, cfg["n_kv_heads"], cfg["head_dim"])
+        k = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+        v = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+        gpu.write_kv(layer, 0, k, v)
+        kc, vc = cpu.kv(layer)
+        kc[:ctx] = k.astype(np.float32)
+        vc[:ctx] = v.astype(np.float32)
+    cpu.rewind_to(ctx)
+    assert gpu.position == ctx
+    return cfg, gpu, cpu
+
+
+def test_llama3_8b_shape_chain_and_tree_at_4096_context():
+    import turbospark_amd as ts
+    ctx = 4096
+    cfg, gpu, cpu = _filled("llama3_8b_q4_k", ctx, 2)
+    V = cfg["vocab"]
+    rng = np.random.default_rng(1)
+    feed = rng.integers(0, V, 5).astype(np.int32)
+    point = gpu.checkpoint()
+    got = gpu.verify(feed, ctx)
+    want = cpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"8B shape, 2 layers, ctx 4096, m=5: max-abs logit error / range = {err:.2e}")
+    assert err <= 1e-2
+    # the new K rows of the pass agree too (rotation at positions 4096..4100)
+    kg, vg = gpu.read_kv(1, ctx, 5)
+    kc, vc = cpu.kv(1)
+    assert np.abs(kg.astype(np.float32) - kc[ctx:ctx + 5]).max() <= 2e-2 * np.abs(kc[ctx:ctx + 5]).max()
+    # acceptance at the full vocabulary on these logits, sampled T = 0.8: integers equal
+    draft = rng.standard_normal((4, V)).astype(np.float16)
+    gcfg, ocfg = ts.shaping(0.8, seed=9), ob.shaping(0.8, seed=9)
+    res = gpu.accept(feed, ctx, gcfg, draft_logits=draft, draw_step=3)
+    ref = ob.chain_round(got, draft, feed[1:], ocfg, history=[0] * ctx + [int(feed[0])], draw_step=3)
+    assert (res.accepted, res.committed, res.next, res.draw_step) == (ref["accepted"], ref["committed"], ref["next"], ref["draw_step"])
+    # the 16-node tree of configuration 3 on the same cache
+    gpu.rollback(point)
+    cpu.rewind_to(ctx)
+    parent = [-1, 0, 0, 0, 0, 1, 5, 6, 2, 8, 9, 3, 11, 12, 4, 14]
+    feed = rng.integers(0, V, 16).astype(np.int32)
+    got = gpu.verify_tree(feed, parent, ctx)
+    want = cpu.verify(feed, ctx, parent=parent)
+    err = gc.logit_error(got, want)
+    print(f"8B shape, 2 layers, ctx 4096, 16-node tree: max-abs logit error / range = {err:.2e}")
+    assert err <= 1e-2
+    draft = (gc.f16(got) + rng.standard_normal((16, V)).astype(np.float32)).astype(np.float16)
+    gcfg, ocfg = ts.shaping(1.0, seed=2), ob.shaping(1.0, seed=2)
+    res = gpu.accept(feed, ctx, gcfg, parent=parent, draft_logits=draft)
+    ref = ob.tree_round_sampled(got, draft, feed, parent, ocfg, history=[0] * ctx)
+    assert res.path == ref["path"] and res.next == ref["next"] and res.draw_step == ref["draw_step"]
+
+
+def test_gptoss_120b_shape_one_windowed_and_one_full_layer_at_long_context():
+    """Hidden 2880 (not whole 256-chunks), 64q / 8kv x 64, 128 experts top-4 with biases, window 128
+    on layer 0, full attention on layer 1, sinks, YaRN; vocabulary cut to 4096 to keep the CPU side short."""
+    ctx = 3000
+    cfg, gpu, cpu = _filled("gptoss_120b", ctx, 2, vocab=4096)
+    for attempt in range(8):
+        feed = np.random.default_rng(20 + attempt).integers(0, cfg["vocab"], 9).astype(np.int32)
+        cpu.rewind_to(ctx)
+        want = cpu.verify(feed, ctx)
+        if cpu.route_margin > 2e-3:
+            break
+    else:
+        raise AssertionError("no feed without a near-tie routing decision")
+    got = gpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"gpt-oss-120B shape, 2 layers, ctx {ctx}, m=9: max-abs logit error / range = {err:.2e}, "
+          f"route margin {cpu.route_margin:.2e}")
+    assert err <= 1e-2

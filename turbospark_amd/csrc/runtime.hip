@@ -1208,6 +1208,35 @@ extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t 
     return rc;
 }
 
+extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k,
+                                const uint16_t* v) {
+    if (!c || !k || !v || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->max_context) {
+        set_error("write_kv: range outside the cache");
+        return TSV_ERR_INVALID;
+    }
+    const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
+    uint16_t *kd = nullptr, *vd = nullptr;
+    TSV_HIP(hipMalloc((void**)&kd, bytes));
+    TSV_HIP(hipMalloc((void**)&vd, bytes));
+    int rc = TSV_OK;
+    if (hipMemcpyAsync(kd, k, bytes, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+        hipMemcpyAsync(vd, v, bytes, hipMemcpyHostToDevice, c->stream) != hipSuccess) {
+        set_error("write_kv: copy failed");
+        rc = TSV_ERR_DEVICE;
+    }
+    if (!rc)
+        rc = launch_kv_fill(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->ctx_alloc, (int)pos0,
+                            (int)n, kd, vd);
+    if (hipStreamSynchronize(c->stream) != hipSuccess && !rc) {
+        set_error("write_kv: device execution failed");
+        rc = TSV_ERR_DEVICE;
+    }
+    (void)hipFree(kd);
+    (void)hipFree(vd);
+    if (!rc && pos0 + n > c->position) c->position = pos0 + n;
+    return rc;
+}
+
 extern "C" int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits) {
     if (!w || !x || !y || m < 1 || m > TSV_MAX_ROWS) {
         set_error("matmul: bad argument");

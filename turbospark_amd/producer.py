@@ -281,6 +281,12 @@ class HipVerifier:
         return {k: (float(ms[i]), int(cnt[i])) for i, k in enumerate(self.PROFILE_CLASSES)}
 
     # ---- test introspection ------------------------------------------------------------------
+    def write_kv(self, layer, pos0, k, v):
+        """k, v: [n, n_kv_heads, head_dim] (rounded to fp16) stored at cache positions pos0.."""
+        k16 = np.ascontiguousarray(np.asarray(k).astype(np.float16))
+        v16 = np.ascontiguousarray(np.asarray(v).astype(np.float16))
+        ffi.check(ffi.lib().tsv_write_kv(self._h, layer, int(pos0), k16.shape[0], k16.ctypes.data, v16.ctypes.data))
+
     def read_kv(self, layer, pos0, n):
         c = self.cfg
         shape = (n, c["n_kv_heads"], c["head_dim"])
