@@ -12,6 +12,8 @@
 //    accumulator layout (lane: row j, positions 4*kg..4*kg+3) is exactly the B-operand layout
 //    of v_mfma_f32_16x16x16_f16, so O^T += V^T P^T needs no data movement; V is stored in the
 //    cache pre-arranged as that MFMA's A fragments.
+#include <algorithm>
+
 #include "tsv_internal.h"
 
 namespace tsv {
@@ -19,6 +21,8 @@ namespace tsv {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 int attn_chunks(int nkv) {
     int n = 256 / nkv;
@@ -27,12 +31,49 @@ int attn_chunks(int nkv) {
     return n;
 }
 
-template <int HD, int RT>
-__global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) {
+// One (m, l, O) running state merged into another (flash-decoding rescale).
+template <int RT, int VT>
+__device__ __forceinline__ void merge_state(float (&mrun)[RT], float (&lrun)[RT], float4v (&O)[RT][VT], const float* src) {
+    // `src` points at this lane's column of a [values][64 lanes] slot: consecutive lanes touch
+    // consecutive LDS banks
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const float m1 = src[64 * (2 * t)], l1 = src[64 * (2 * t + 1)];
+        const float mnew = fmaxf(mrun[t], m1);
+        if (mnew > -INFINITY) {
+            const float a0 = __expf(mrun[t] - mnew), a1 = __expf(m1 - mnew);
+            lrun[t] = lrun[t] * a0 + l1 * a1;
+#pragma unroll
+            for (int d = 0; d < VT; d++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) O[t][d][i] = O[t][d][i] * a0 + src[64 * (2 * RT + (t * VT + d) * 4 + i)] * a1;
+            mrun[t] = mnew;
+        }
+    }
+}
+template <int RT, int VT>
+__device__ __forceinline__ void store_state(const float (&mrun)[RT], const float (&lrun)[RT], const float4v (&O)[RT][VT],
+                                            float* dst) {
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        dst[64 * (2 * t)] = mrun[t];
+        dst[64 * (2 * t + 1)] = lrun[t];
+#pragma unroll
+        for (int d = 0; d < VT; d++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[64 * (2 * RT + (t * VT + d) * 4 + i)] = O[t][d][i];
+    }
+}
+
+// Eight waves per workgroup share a chunk of the context, each walking every eighth 16-position
+// block with up to STAGES blocks of K and V in flight.
+template <int HD, int RT, int STAGES>
+__global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) {
+    constexpr int NW = 8;
     constexpr int KS = HD / 32;  // K steps of the score MFMA
     constexpr int VT = HD / 16;  // output tiles along head_dim
     constexpr int PER_LANE = RT * VT * 4 + 2 * RT;
-    __shared__ float xch[64 * PER_LANE];
+    extern __shared__ float xch[];  // [4 slots][PER_LANE values][64 lanes]
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 15, kg = lane >> 4;
@@ -84,25 +125,36 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
         for (int d = 0; d < VT; d++) O[t][d] = float4v{0.f, 0.f, 0.f, 0.f};
     }
 
-    const _Float16* kbase = (const _Float16*)a.kc + (long)h * a.max_ctx * HD;
-    const _Float16* vbase = (const _Float16*)a.vc + (long)h * (a.max_ctx >> 4) * (HD * 16);
-    for (int b = b0 + wave; b < b1; b += 4) {
-        const int p0 = b << 4;
-        uint4 kf[KS];
-        uint2 vf[VT];
-        const _Float16* kp = kbase + (long)(p0 + j) * HD + 8 * kg;
+    // this head's K rows and V blocks as buffers that end after block b1 - 1
+    const uint32_t blk_bytes = 16 * HD * 2;
+    const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const _Float16*)a.kc + (long)h * a.max_ctx * HD), 0, (int)(b1 * blk_bytes), 0x00027000);
+    const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const _Float16*)a.vc + (long)h * (a.max_ctx >> 4) * (HD * 16)), 0, (int)(b1 * blk_bytes), 0x00027000);
+    struct Blk {
+        u32x4 kf[KS];
+        u32x2 vf[VT];
+    };
+    const uint32_t koff = (uint32_t)(j * HD + 8 * kg) * 2, voff = (uint32_t)lane * 8;
+    const int nb = b1 > b0 + wave ? (b1 - b0 - wave + NW - 1) / NW : 0;  // blocks of this wave
+    auto fetch = [&](Blk& st, int i) {  // block i of this wave's run
+        const uint32_t bo = (uint32_t)(b0 + wave + NW * i) * blk_bytes;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s = 0; s < KS; s++) kf[s] = *(const uint4*)(kp + 32 * s);
-        const _Float16* vpn = vbase + (long)b * (HD * 16) + lane * 4;
+        for (int s = 0; s < KS; s++) st.kf[s] = __builtin_amdgcn_raw_buffer_load_b128(krs, bo + koff + 64 * s, 0, 0);
 #pragma unroll
-        for (int d = 0; d < VT; d++) vf[d] = *(const uint2*)(vpn + d * 256);
+        for (int d = 0; d < VT; d++) st.vf[d] = __builtin_amdgcn_raw_buffer_load_b64(vrs, bo + voff + 512 * d, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto consume = [&](const Blk& st, int i) {
+        const int p0 = (b0 + wave + NW * i) << 4;
         const bool tail = p0 + 16 > base;
 #pragma unroll
         for (int t = 0; t < RT; t++) {
             float4v S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < KS; s++)
-                S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, kf[s]),
+                S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, st.kf[s]),
                                                            __builtin_bit_cast(half8, qf[t][s]), S, 0, 0, 0);
             // Visibility of this lane's four positions as a 4-bit word, computed without
             // branches: bit (slot + 16) of `w` says whether cache slot base+slot is visible
@@ -118,7 +170,7 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
             }
             float sc[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) sc[i] = ((vis4 >> i) & 1u) ? S[i] * scale : -INFINITY;
+            for (int i4 = 0; i4 < 4; i4++) sc[i4] = ((vis4 >> i4) & 1u) ? S[i4] * scale : -INFINITY;
             float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             mb = fmaxf(mb, __shfl_xor(mb, 16));
             mb = fmaxf(mb, __shfl_xor(mb, 32));
@@ -129,10 +181,10 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
                 alpha = __expf(mrun[t] - mnew);
                 float ps = 0.f;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float p = __expf(sc[i] - mnew);
+                for (int i4 = 0; i4 < 4; i4++) {
+                    const float p = __expf(sc[i4] - mnew);
                     ps += p;
-                    P[i] = (_Float16)p;
+                    P[i4] = (_Float16)p;
                 }
                 lrun[t] = lrun[t] * alpha + ps;
                 mrun[t] = mnew;
@@ -140,47 +192,58 @@ __global__ __launch_bounds__(256) void k_attn_partial(AttnArgs a, int G, int R) 
 #pragma unroll
             for (int d = 0; d < VT; d++) {
                 O[t][d] *= alpha;
-                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, vf[d]), P, O[t][d], 0, 0, 0);
+                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, st.vf[d]), P, O[t][d], 0, 0, 0);
             }
         }
+    };
+    // Short runs are straight-line code (every load issued before the first wait, no load the run
+    // does not need); longer ones keep STAGES blocks in flight, with unconditional loads in the
+    // steady state so the compiler waits on the oldest block only.
+    if (nb == 1) {
+        Blk st;
+        fetch(st, 0);
+        consume(st, 0);
+    } else if (nb == 2) {
+        Blk s0, s1;
+        fetch(s0, 0);
+        fetch(s1, 1);
+        consume(s0, 0);
+        consume(s1, 1);
+    } else if (nb >= STAGES) {
+        Blk st[STAGES];
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) fetch(st[s], s);
+        int i = 0;
+        for (; i + 2 * STAGES <= nb; i += STAGES) {
+#pragma unroll
+            for (int s = 0; s < STAGES; s++) {
+                consume(st[s], i + s);
+                fetch(st[s], i + s + STAGES);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) {
+            if (i + s < nb) {
+                consume(st[s], i + s);
+                if (i + s + STAGES < nb) fetch(st[s], i + s + STAGES);
+            }
+        }
+        i += STAGES;
+#pragma unroll
+        for (int s = 0; s < STAGES; s++)
+            if (i + s < nb) consume(st[s], i + s);
     }
 
-    // fold the four waves' running (m, l, O) into wave 0, one wave at a time
-    for (int w = 1; w < 4; w++) {
-        if (wave == w) {
-            float* dst = xch + lane * PER_LANE;
-#pragma unroll
-            for (int t = 0; t < RT; t++) {
-                dst[2 * t] = mrun[t];
-                dst[2 * t + 1] = lrun[t];
-#pragma unroll
-                for (int d = 0; d < VT; d++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) dst[2 * RT + (t * VT + d) * 4 + i] = O[t][d][i];
-            }
-        }
-        __syncthreads();
-        if (wave == 0) {
-            const float* src = xch + lane * PER_LANE;
-#pragma unroll
-            for (int t = 0; t < RT; t++) {
-                const float m1 = src[2 * t], l1 = src[2 * t + 1];
-                const float mnew = fmaxf(mrun[t], m1);
-                if (mnew > -INFINITY) {
-                    const float a0 = __expf(mrun[t] - mnew), a1 = __expf(m1 - mnew);
-                    lrun[t] = lrun[t] * a0 + l1 * a1;
-#pragma unroll
-                    for (int d = 0; d < VT; d++)
-#pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            O[t][d][i] = O[t][d][i] * a0 + src[2 * RT + (t * VT + d) * 4 + i] * a1;
-                    mrun[t] = mnew;
-                }
-            }
-        }
-        __syncthreads();
-    }
+    // fold the eight waves' running (m, l, O): 4..7 into 0..3, then 1..3 into 0
+    float* mine = xch + (wave & 3) * 64 * PER_LANE + lane;
+    if (wave >= 4) store_state<RT, VT>(mrun, lrun, O, mine);
+    __syncthreads();
+    if (wave < 4) merge_state<RT, VT>(mrun, lrun, O, mine);
+    __syncthreads();
+    if (wave >= 1 && wave < 4) store_state<RT, VT>(mrun, lrun, O, mine);
+    __syncthreads();
     if (wave != 0) return;
+    for (int w = 1; w < 4; w++) merge_state<RT, VT>(mrun, lrun, O, xch + w * 64 * PER_LANE + lane);
 #pragma unroll
     for (int t = 0; t < RT; t++) {
         float l = lrun[t];
@@ -247,17 +310,36 @@ __global__ void k_attn_combine(AttnArgs a, int G, int R) {
     if ((d & 31) == 0) ((float*)((char*)a.xfrag + xfrag_sum_offset(a.nq * hd)))[xsum_index(kk >> 5, m)] = sum;
 }
 
-template <int HD>
-static int launch_hd(hipStream_t s, const AttnArgs& a, int m, int G, int R) {
-    const int trt = (R + 15) / 16;
-    if (trt <= 1) {
-        hipLaunchKernelGGL((k_attn_partial<HD, 1>), dim3(a.nch, a.nkv, 1), dim3(256), 0, s, a, G, R);
-    } else if (trt <= 2) {
-        hipLaunchKernelGGL((k_attn_partial<HD, 2>), dim3(a.nch, a.nkv, 1), dim3(256), 0, s, a, G, R);
-    } else {
-        hipLaunchKernelGGL((k_attn_partial<HD, 4>), dim3(a.nch, a.nkv, (trt + 3) / 4), dim3(256), 0, s, a, G, R);
+template <int HD, int RT, int STAGES>
+static int launch_partial(hipStream_t s, const AttnArgs& a, int G, int R, int groups) {
+    constexpr int PER_LANE = RT * (HD / 16) * 4 + 2 * RT;
+    const size_t lds = (size_t)4 * 64 * PER_LANE * 4;
+    static bool raised = false;  // more than 64 KiB of dynamic LDS has to be allowed once per kernel
+    if (lds > 65536 && !raised) {
+        TSV_HIP(hipFuncSetAttribute((const void*)k_attn_partial<HD, RT, STAGES>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds));
+        raised = true;
     }
+    hipLaunchKernelGGL((k_attn_partial<HD, RT, STAGES>), dim3(a.nch, a.nkv, groups), dim3(512), lds, s, a, G, R);
     TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+template <int HD>
+static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
+    const int trt = (R + 15) / 16;
+    // more than 32 (row, q head) pairs: groups of 32 in grid z, each re-reading K and V (from L2)
+    const int groups = trt <= 2 ? 1 : (trt + 1) / 2;
+    // about one workgroup per compute unit: the chunk count shrinks as the row groups multiply
+    // (fewer, longer chunks also mean fewer partial results for the merge to read)
+    AttnArgs a = a0;
+    a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 256 / (a0.nkv * groups)));
+    int rc;
+    if (trt <= 1)
+        rc = launch_partial<HD, 1, 3>(s, a, G, R, 1);
+    else
+        rc = launch_partial<HD, 2, 3>(s, a, G, R, groups);
+    if (rc) return rc;
     hipLaunchKernelGGL(k_attn_combine, dim3(m, a.nq), dim3(HD < 64 ? 64 : HD), 0, s, a, G, R);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
