@@ -87,6 +87,7 @@ extern "C" int64_t tso_row_bytes(int dtype, int64_t n) {
         case TSO_BF16: return n * 2;
         case TSO_Q8_0: return n / 32 * 34;
         case TSO_Q4_K: return n / 256 * 144;
+        case TSO_Q6_K: return n / 256 * 210;
         case TSO_MXFP4: return (n + 31) / 32 * 17;
     }
     return -1;
@@ -302,7 +303,85 @@ extern "C" void tso_dequantize_row(int dtype, const uint8_t* row, int64_t n, flo
             break;
         case TSO_Q8_0: tso_dequantize_q8_0(row, n, out); break;
         case TSO_Q4_K: tso_dequantize_q4_k(row, n, out); break;
+        case TSO_Q6_K: tso_dequantize_q6_k(row, n, out); break;
         case TSO_MXFP4: tso_dequantize_mxfp4(row, n, out); break;
+    }
+}
+
+// crates/compute/src/quant_gguf/q6_k.rs:44-88.  A superblock is two halves of 128 elements; in a
+// half, byte l of `ql` (and l + 32) and byte l of `qh` serve the four elements l, l + 32, l + 64,
+// l + 96, each with its own scale (is, is + 2, is + 4, is + 6); stored levels carry a bias of 32.
+extern "C" void tso_dequantize_q6_k(const uint8_t* blocks, int64_t n, float* out) {
+    for (int64_t b = 0; b < n / 256; b++) {
+        const uint8_t* blk = blocks + b * 210;
+        uint16_t db;
+        std::memcpy(&db, blk + 208, 2);
+        const float d = tso_f16_to_f32(db);
+        for (int h = 0; h < 2; h++) {
+            const uint8_t* ql = blk + h * 64;
+            const uint8_t* qh = blk + 128 + h * 32;
+            const int8_t* sc = (const int8_t*)blk + 192 + h * 8;
+            float* o = out + b * 256 + h * 128;
+            for (int l = 0; l < 32; l++) {
+                const int is = l / 16;
+                const int q[4] = {(int)((ql[l] & 0xF) | ((qh[l] & 3) << 4)) - 32,
+                                  (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32,
+                                  (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32,
+                                  (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32};
+                for (int k = 0; k < 4; k++) o[l + k * 32] = d * (float)sc[is + k * 2] * (float)q[k];
+            }
+        }
+    }
+}
+
+// crates/compute/src/quant_gguf/q6_k.rs:101-194: per 16-element sub-block the signed element of
+// largest magnitude sets the scale (-extreme / 32), the scales are quantised to int8 against the
+// largest one through a negative iscale, d is rounded through f16 before the levels are chosen.
+extern "C" void tso_quantize_q6_k(const float* row, int64_t n, uint8_t* out) {
+    for (int64_t b = 0; b < n / 256; b++) {
+        const float* block = row + b * 256;
+        uint8_t* blk = out + b * 210;
+        float scales[16], max_scale = 0.0f;
+        for (int j = 0; j < 16; j++) {
+            float extreme = 0.0f;
+            for (int i = 0; i < 16; i++)
+                if (std::fabs(block[j * 16 + i]) > std::fabs(extreme)) extreme = block[j * 16 + i];
+            scales[j] = -extreme / 32.0f;
+            if (std::fabs(scales[j]) > std::fabs(max_scale)) max_scale = scales[j];
+        }
+        int8_t sc[16] = {0};
+        uint16_t dbits = tso_f32_to_f16(0.0f);
+        if (max_scale != 0.0f) {
+            const float iscale = -128.0f / max_scale;
+            for (int j = 0; j < 16; j++) {
+                int v = (int)std::round(iscale * scales[j]);  // f32::round: half away from zero
+                sc[j] = (int8_t)std::min(std::max(v, -128), 127);
+            }
+            dbits = tso_f32_to_f16(1.0f / iscale);
+        }
+        const float d = tso_f16_to_f32(dbits);
+        uint8_t levels[256];
+        std::memset(levels, 32, sizeof levels);
+        for (int j = 0; j < 16; j++) {
+            const float step = d * (float)sc[j];
+            if (step == 0.0f) continue;
+            for (int i = 0; i < 16; i++) {
+                float q = std::round(block[j * 16 + i] / step);
+                q = std::min(std::max(q, -32.0f), 31.0f);
+                levels[j * 16 + i] = (uint8_t)((int)q + 32);
+            }
+        }
+        std::memset(blk, 0, 210);
+        for (int h = 0; h < 2; h++)
+            for (int l = 0; l < 32; l++) {
+                const uint8_t* v = levels + h * 128 + l;
+                blk[h * 64 + l] = (uint8_t)((v[0] & 0xF) | ((v[64] & 0xF) << 4));
+                blk[h * 64 + l + 32] = (uint8_t)((v[32] & 0xF) | ((v[96] & 0xF) << 4));
+                blk[128 + h * 32 + l] =
+                    (uint8_t)((v[0] >> 4) | ((v[32] >> 4) << 2) | ((v[64] >> 4) << 4) | ((v[96] >> 4) << 6));
+            }
+        std::memcpy(blk + 192, sc, 16);
+        std::memcpy(blk + 208, &dbits, 2);
     }
 }
 

@@ -45,6 +45,7 @@ enum {
     TSO_F16 = 1,
     TSO_Q8_0 = 8,
     TSO_Q4_K = 12,
+    TSO_Q6_K = 14, /* 210 B / 256 elems: 4 low bits + 2 high bits per element, 16 signed int8 scales, f16 d */
     TSO_BF16 = 30,
     TSO_MXFP4 = 39,
 };
@@ -62,6 +63,9 @@ void tso_dequantize_q8_0(const uint8_t* blocks, int64_t n, float* out);
 void tso_quantize_q4_k(const float* row, int64_t n, uint8_t* out);
 void tso_dequantize_q4_k(const uint8_t* blocks, int64_t n, float* out);
 void tso_q4_k_scale_min(int j, const uint8_t* packed12, uint8_t* sc, uint8_t* mn);
+/* crates/compute/src/quant_gguf/q6_k.rs:44-88 (decode), :101-194 (largest-magnitude encoder) */
+void tso_dequantize_q6_k(const uint8_t* blocks, int64_t n, float* out);
+void tso_quantize_q6_k(const float* row, int64_t n, uint8_t* out);
 float tso_mxfp4_scale(uint8_t e);
 void tso_dequantize_mxfp4(const uint8_t* blocks, int64_t n, float* out);
 void tso_quantize_mxfp4(const float* row, int64_t n, uint8_t* out); /* ours: reference has no encoder */

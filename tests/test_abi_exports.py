@@ -41,7 +41,7 @@ def test_install_encoders_are_bit_identical_to_the_oracle():
     w = (rng.standard_normal((24, 1024)) * 0.02).astype(np.float32)
     w[3] = 0.0                      # an all-zero row: zero scales, no division
     w[5, :32] = 1e-9                # a nearly flat sub-block
-    for dt in (ffi.Q4_K, ffi.Q8_0, ffi.MXFP4, ffi.F16, ffi.BF16, ffi.F32):
+    for dt in (ffi.Q4_K, ffi.Q6_K, ffi.Q8_0, ffi.MXFP4, ffi.F16, ffi.BF16, ffi.F32):
         assert np.array_equal(ffi.quantize(dt, w)[1], ob.quantize(dt, w)), dt
     assert ffi.row_bytes(ffi.Q4_K, 4096) == 2304 and ffi.row_bytes(ffi.Q8_0, 4096) == 4352
     assert ffi.row_bytes(ffi.Q4_K, 100) < 0

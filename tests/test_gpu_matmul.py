@@ -25,7 +25,8 @@ def _case(dtype, rows, cols, seed):
 @pytest.mark.parametrize("dtype,rows,cols", [(12, 64, 512), (12, 48, 2048), (8, 64, 512), (8, 32, 1408),
                                              (39, 64, 512), (39, 48, 2048), (39, 200, 768),
                                              (39, 64, 576), (39, 96, 2880),      # MXFP4 rows ending inside a 256-chunk
-                                             (30, 64, 512), (30, 40, 576), (30, 130, 2880)])  # bf16
+                                             (30, 64, 512), (30, 40, 576), (30, 130, 2880),   # bf16
+                                             (14, 64, 512), (14, 48, 2048), (14, 200, 768)])   # Q6_K
 def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, rows, cols, 31)
@@ -45,7 +46,7 @@ def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
         assert np.array_equal(got[0], first), m
 
 
-@pytest.mark.parametrize("dtype", [12, 8, 39, 30])
+@pytest.mark.parametrize("dtype", [12, 8, 39, 30, 14])
 def test_split_k_changes_nothing_but_rounding_and_is_deterministic(dtype):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, 32, 2048, 77)
@@ -105,3 +106,26 @@ def test_mxfp4_ggml_golden_blocks_through_the_kernel(golden):
         got = ffi.matmul(entry, x)
         for b in range(16):
             assert np.all(got[b] == want[e0 + b]), (e0 + b, got[b, 0], want[e0 + b])
+
+
+def test_q6k_hand_packed_superblock_through_the_kernel(golden):
+    """The reference's literal Q6_K superblock (crates/compute/tests/quant_gguf.rs:413-445) as every row
+    of a weight matrix: one-hot activations read the decoded weights back out of the kernel, `==`."""
+    import json
+    import os
+    from turbospark_amd import ffi
+    g = json.load(open(os.path.join(golden, "q6k_handpacked.json")))
+    block = bytes([g["ql_byte"]] * 128 + [g["qh_byte"]] * 64 + [s & 0xFF for s in g["scales"]]) + \
+        int(g["d_bits"]).to_bytes(2, "little")
+    rows = 16
+    data = np.frombuffer(block * rows, np.uint8).reshape(rows, 210).copy()
+    entry = (ffi.Q6_K, data, rows, 256)
+    for k0 in range(0, 256, 16):
+        x = np.zeros((16, 256), np.float32)
+        x[np.arange(16), k0 + np.arange(16)] = 1.0
+        got = ffi.matmul(entry, x)
+        for b in range(16):
+            e = k0 + b
+            h, k, l = e // 128, (e % 128) // 32, e % 32
+            want = np.float32(g["d"]) * np.float32(g["scales"][h * 8 + l // 16 + 2 * k]) * np.float32(g["quants"][k])
+            assert np.all(got[b] == want), (e, got[b][0], want)

@@ -106,6 +106,47 @@ def test_q4k_quantizer_is_idempotent_on_its_own_output():
     assert np.max(np.abs(d2 - d1)) <= np.max(np.abs(d1 - w)) * 2 + 1e-6
 
 
+def _q6k_golden_block(golden):
+    g = json.load(open(os.path.join(golden, "q6k_handpacked.json")))
+    block = bytes([g["ql_byte"]] * 128 + [g["qh_byte"]] * 64 + [s & 0xFF for s in g["scales"]]) + \
+        int(g["d_bits"]).to_bytes(2, "little")
+    assert len(block) == 210
+    return g, np.frombuffer(block, np.uint8)
+
+
+def test_q6k_hand_packed_superblock_decodes_to_the_documented_formula(golden):
+    """crates/compute/tests/quant_gguf.rs:413-445: ql = 0x93, qh = 0xB1 give the levels 19, 3, 57, 41,
+    i.e. quants -13, -29, 25, 9; half of the sixteen signed scales are negative; `==` throughout."""
+    g, block = _q6k_golden_block(golden)
+    out = ob.dequantize(ob.Q6_K, block, 256)[0]
+    for h in range(2):
+        for k in range(4):
+            for l in range(32):
+                want = np.float32(g["d"]) * np.float32(g["scales"][h * 8 + l // 16 + 2 * k]) * np.float32(g["quants"][k])
+                assert out[h * 128 + k * 32 + l] == want, (h, k, l)
+    for at, want in g["spot"].items():
+        assert out[int(at)] == want
+
+
+def test_q6k_round_trip_signed_scales_and_zero_block():
+    # quant_gguf.rs:447-500: inside one quantization step; both scale signs occur and no element flips
+    w = lcg_weights(512, 41)
+    out = ob.dequantize(ob.Q6_K, ob.quantize(ob.Q6_K, w.reshape(1, -1)), 512)[0]
+    for j in range(32):
+        sub = w[16 * j:16 * j + 16]
+        amax = np.abs(sub).max()
+        assert np.abs(out[16 * j:16 * j + 16] - sub).max() <= amax / 32.0 * 0.5 + amax * 2e-2
+    e = np.arange(256)
+    w = (np.where((e // 16) % 2 == 0, 1.0, -1.0) * (1.0 + (e % 16) / 16.0)).astype(np.float32)
+    q = ob.quantize(ob.Q6_K, w.reshape(1, -1))[0]
+    scales = q[192:208].view(np.int8)
+    assert (scales < 0).any() and (scales > 0).any()
+    out = ob.dequantize(ob.Q6_K, q, 256)[0]
+    assert np.array_equal(np.sign(out), np.sign(w)) and np.abs(out - w).max() < 0.1
+    z = ob.quantize(ob.Q6_K, np.zeros((1, 256), np.float32))[0]
+    assert np.all(ob.dequantize(ob.Q6_K, z, 256) == 0.0) and ob.row_bytes(ob.Q6_K, 512) == 420
+
+
 def test_q8_0_round_trip_sign_zero_and_idempotence():
     w = lcg_weights(96, 7)
     q = ob.quantize(ob.Q8_0, w.reshape(1, -1))

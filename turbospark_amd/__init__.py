@@ -5,6 +5,6 @@ The compute lives in libtsverify.so (hand-written HIP for gfx950, C ABI in inclu
 this package is the thin host-side mirror of that interface.  There is no CPU fallback: if
 the library is missing, importing `turbospark_amd.ffi` raises.
 """
-from .ffi import F32, F16, Q8_0, Q4_K, BF16, TsvError, lib, shaping  # noqa: F401
+from .ffi import F32, F16, Q8_0, Q4_K, Q6_K, BF16, MXFP4, TsvError, lib, shaping  # noqa: F401
 from .producer import HipVerifier, RoundResult  # noqa: F401
 from . import synth  # noqa: F401

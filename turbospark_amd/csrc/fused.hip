@@ -455,7 +455,7 @@ extern "C" int tsv_fused_trace(long long* out) {
 // Shapes the FFN block kernel takes: both matrices in one format, the gate/up tiles and the
 // down projection's K chunks divisible by the XCD count, hidden a multiple of 32 * 32 columns.
 bool fused_ffn_supported(const TiledW& gate_up, const TiledW& down, int hidden, int ffn) {
-    if (gate_up.fmt != down.fmt) return false;
+    if (gate_up.fmt != down.fmt || (gate_up.fmt != FMT_Q4K && gate_up.fmt != FMT_Q80)) return false;
     if (gate_up.n_rows != 2 * ffn || down.k != ffn || gate_up.k != hidden || down.n_rows != hidden) return false;
     if (gate_up.n_tiles % XCDS || down.kchunks % XCDS) return false;
     if (hidden % (WGS_PER_XCD * 32) || hidden > 8192) return false;

@@ -112,6 +112,69 @@ __global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kc
     tb[8192 + lane * 8 + u] = blk[0];
 }
 
+// Q6_K: one thread per unit of a (row, chunk): 12 quant units, the scale unit, the d word.
+__device__ __forceinline__ uint32_t q6k_level(const uint8_t* blk, int e) {
+    // q6_k.rs:67-84: element e = 128 h + 32 k + l takes its low nibble from ql[64 h + l + 32 (k & 1)]
+    // (upper nibble when k >= 2) and its high pair from bits 2k.. of qh[32 h + l]
+    const int h = e >> 7, k = (e >> 5) & 3, l = e & 31;
+    const uint32_t lo = (blk[64 * h + l + 32 * (k & 1)] >> (4 * (k >> 1))) & 0xFu;
+    const uint32_t hi = (blk[128 + 32 * h + l] >> (2 * k)) & 3u;
+    return lo | (hi << 4);
+}
+__global__ void k_repack_q6k(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)n_rows * kchunks * 14;
+    if (gid >= total) return;
+    const int u = (int)(gid % 14);
+    const long t = gid / 14;
+    const int c = (int)(t % kchunks);
+    const int r = (int)(t / kchunks);
+    const int drow = (r / grp) * stride + offset + r % grp;
+    const int tile = drow >> 6, lane = drow & 63;
+    const uint8_t* blk = raw + ((long)r * kchunks + c) * 210;
+    uint8_t* tb = tiles + ((long)tile * kchunks + c) * 13568;
+    if (u == 13) {
+        *(uint32_t*)(tb + 13312 + lane * 4) = (uint32_t)blk[208] | ((uint32_t)blk[209] << 8);
+        return;
+    }
+    if (u == 12) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            w[i] = (uint32_t)blk[192 + 4 * i] | ((uint32_t)blk[193 + 4 * i] << 8) | ((uint32_t)blk[194 + 4 * i] << 16) |
+                   ((uint32_t)blk[195 + 4 * i] << 24);
+        *(uint4*)(tb + 12288 + lane * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        return;
+    }
+    const int p = u / 3, part = u % 3;
+    uint32_t w[4] = {0, 0, 0, 0};
+    if (part < 2) {
+        // word i: steps a = 8 part + 2i and a + 1; nibbles k0 k1 (a), k0 k1 (a + 1), k2 k3 (a), k2 k3 (a + 1)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int e0 = 64 * p + 4 * (8 * part + 2 * i);
+            const int order[8] = {e0, e0 + 1, e0 + 4, e0 + 5, e0 + 2, e0 + 3, e0 + 6, e0 + 7};
+#pragma unroll
+            for (int n = 0; n < 8; n++) w[i] |= (q6k_level(blk, order[n]) & 0xFu) << (4 * n);
+        }
+    } else {
+        // word i: steps 4i .. 4i + 3; extraction e = 2 * (step % 4) + ab holds (k0, k2) for ab = 0 and
+        // (k1, k3) for ab = 1: the first element's pair at bits 2e, the second's at bits 16 + 2e
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int si = 0; si < 4; si++)
+#pragma unroll
+                for (int ab = 0; ab < 2; ab++) {
+                    const int e0 = 64 * p + 4 * (4 * i + si), e = 2 * si + ab;
+                    w[i] |= (q6k_level(blk, e0 + ab) >> 4) << (2 * e);
+                    w[i] |= (q6k_level(blk, e0 + 2 + ab) >> 4) << (16 + 2 * e);
+                }
+    }
+    *(uint4*)(tb + (u * 64 + lane) * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // bf16: one thread per 16-byte unit (eight consecutive K values of a row, two MFMA steps).
 __global__ void k_repack_bf16(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
                               uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
@@ -137,7 +200,11 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
                   int kchunks, int grp, int stride, int offset) {
     const long total = (long)n_rows * kchunks * 9;
     if (total == 0) return TSV_OK;
-    if (fmt == FMT_BF16) {
+    if (fmt == FMT_Q6K) {
+        const long units = (long)n_rows * kchunks * 14;
+        hipLaunchKernelGGL(k_repack_q6k, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
+                           tiles, grp, stride, offset);
+    } else if (fmt == FMT_BF16) {
         const long units = (long)n_rows * kchunks * 8;
         hipLaunchKernelGGL(k_repack_bf16, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
                            tiles, grp, stride, offset);
@@ -346,6 +413,7 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
     return w.fmt == FMT_Q4K    ? launch_f<Q4K>(s, a, m, epi)
            : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
            : w.fmt == FMT_BF16 ? launch_f<BF16W>(s, a, m, epi)
+           : w.fmt == FMT_Q6K  ? launch_f<Q6K>(s, a, m, epi)
                                : launch_f<MX4>(s, a, m, epi);
 }
 

@@ -168,6 +168,28 @@ struct BF16W {
     static __device__ __forceinline__ int xs_base(int, int) { return 0; }
 };
 
+// Q6_K (crates/compute/src/quant_gguf/q6_k.rs:44-88): value = d * sc_j * (level - 32), level = 4 low
+// bits + 2 high bits, one signed int8 scale per 16 elements.  The level goes to the MFMA as the
+// exact fp16 integer level - 32: (low nibble | 0x6400) | (high pair << 4) is 1024 + level, and one
+// packed fp16 add of -1056 removes offset and bias together.
+struct Q6K {
+    static constexpr int NSUB = 16, NPAIR = 4, TILE_BYTES = 13568;
+    static constexpr bool SUMS = false;
+    struct Regs {
+        u32x4 q[12];
+        u32x4 s;
+        uint32_t d;
+    };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
+        const u32x4* p = (const u32x4*)tile + lane;
+#pragma unroll
+        for (int u = 0; u < 12; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
+        r.s = __builtin_nontemporal_load(p + 12 * 64);
+        r.d = __builtin_nontemporal_load((const uint32_t*)(tile + 13312) + lane);
+    }
+    static __device__ __forceinline__ int xs_base(int, int) { return 0; }
+};
+
 template <int STEP>
 __device__ __forceinline__ float4v mfma_bf16(u32x2 a, u32x2 b, float4v c) {
     typedef short short4v __attribute__((ext_vector_type(4)));
@@ -194,6 +216,7 @@ struct RegSrc {
     const typename F::Regs& r;
     __device__ __forceinline__ u32x4 unit(int u) const { return r.q[u]; }
     __device__ __forceinline__ auto scales() const { return r.s; }
+    __device__ __forceinline__ auto dval() const { return r.d; }
 };
 template <class F>
 struct LdsSrc {
@@ -417,6 +440,47 @@ __device__ __forceinline__ void compute_tile(MX4, const Src& w, const XRegs<MX4,
             fma4(acc[g], sc[2 * p], da[g]);
             fma4(acc[g], sc[2 * p + 1], db[g]);
         }
+    }
+}
+
+// One Q6_K superblock tile (64 rows x 256 K): sixteen 16-element sub-blocks, four K steps each.
+template <int NG, class Src>
+__device__ __forceinline__ void compute_tile(Q6K, const Src& w, const XRegs<Q6K, NG>& x, const Consts& k,
+                                             float4v (&acc)[NG]) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const u32x4 scw = w.scales();
+    const float d = h2f_lo(w.dval());
+    const half2v off = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const u32x4 n0 = w.unit(3 * p), n1 = w.unit(3 * p + 1), hh = w.unit(3 * p + 2);
+        static_for<4>([&](auto Q) {
+            constexpr int q = decltype(Q)::value;
+            const uint32_t H = hh[q];
+            float4v t[NG];
+#pragma unroll
+            for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
+            static_for<4>([&](auto SI) {
+                constexpr int si = decltype(SI)::value;
+                constexpr int s = 4 * q + si;
+                const uint32_t nw = s < 8 ? n0[(s & 7) >> 1] : n1[(s & 7) >> 1];
+                auto build = [&](int ab) {
+                    const int lo_sh = (s & 1) * 8 + 4 * ab, e = 2 * si + ab;
+                    const uint32_t lo = and_or(nw >> lo_sh, 0x000F000Fu, k.k6400);
+                    const uint32_t hi = 2 * e >= 4 ? H >> (2 * e - 4) : H << (4 - 2 * e);
+                    const uint32_t v = and_or(hi, 0x00300030u, lo);  // 1024 + level, twice
+                    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2v, v) + off);
+                };
+                const u32x2 b = {build(0), build(1)};
+#pragma unroll
+                for (int g = 0; g < NG; g++) t[g] = mfma_f16<s>(x.xa[p][g], b, t[g]);
+            });
+            constexpr int j = 4 * q;  // sub-block 4p + q: byte (4p + q) of the scale unit
+            const int sc8 = (int)(scw[p] << (24 - 8 * (j >> 2))) >> 24;
+            const float sc = d * (float)sc8;
+#pragma unroll
+            for (int g = 0; g < NG; g++) fma4(acc[g], sc, t[g]);
+        });
     }
 }
 

@@ -3,6 +3,7 @@
 // The encoders restate the reference's quantize-on-install routines
 // (crates/compute/src/quant_gguf/q8_0.rs:56-77, q4_k.rs:126-204); the generator plays the role
 // of the reference's random-weight synthetic installs (crates/repack/src/synthetic_*.rs).
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <thread>
@@ -23,6 +24,7 @@ int64_t row_bytes(int dtype, int64_t cols) {
         case TSV_BF16: return cols * 2;
         case TSV_Q8_0: return cols % 32 ? -1 : cols / 32 * 34;
         case TSV_Q4_K: return cols % 256 ? -1 : cols / 256 * 144;
+        case TSV_Q6_K: return cols % 256 ? -1 : cols / 256 * 210;
         case TSV_MXFP4: return cols % 32 ? -1 : cols / 32 * 17;
     }
     return -1;
@@ -131,6 +133,49 @@ void encode_q4_k(const float* row, int64_t n, uint8_t* out) {
     }
 }
 
+// Q6_K install encoder (crates/compute/src/quant_gguf/q6_k.rs:101-194): sub-block scale from the
+// signed element of largest magnitude, int8 scales against the largest through a negative
+// iscale, levels chosen against the f16-rounded d.
+void encode_q6_k(const float* row, int64_t n, uint8_t* out) {
+    for (int64_t sb = 0; sb < n / 256; sb++) {
+        const float* x = row + sb * 256;
+        uint8_t* blk = out + sb * 210;
+        float sub_scale[16], biggest = 0.f;
+        for (int j = 0; j < 16; j++) {
+            float ext = 0.f;
+            for (int i = 0; i < 16; i++)
+                if (fabsf(x[16 * j + i]) > fabsf(ext)) ext = x[16 * j + i];
+            sub_scale[j] = -ext / 32.0f;
+            if (fabsf(sub_scale[j]) > fabsf(biggest)) biggest = sub_scale[j];
+        }
+        int8_t sc[16] = {0};
+        _Float16 dh = (_Float16)0.0f;
+        if (biggest != 0.f) {
+            const float inv = -128.0f / biggest;
+            for (int j = 0; j < 16; j++) sc[j] = (int8_t)std::min(std::max((int)roundf(inv * sub_scale[j]), -128), 127);
+            dh = (_Float16)(1.0f / inv);
+        }
+        const float d = (float)dh;
+        uint8_t lv[256];
+        std::memset(lv, 32, sizeof lv);
+        for (int j = 0; j < 16; j++) {
+            const float step = d * (float)sc[j];
+            if (step == 0.f) continue;
+            for (int i = 0; i < 16; i++)
+                lv[16 * j + i] = (uint8_t)((int)fminf(fmaxf(roundf(x[16 * j + i] / step), -32.f), 31.f) + 32);
+        }
+        for (int h = 0; h < 2; h++)
+            for (int l = 0; l < 32; l++) {
+                const uint8_t a = lv[128 * h + l], b = lv[128 * h + 32 + l], c = lv[128 * h + 64 + l], e = lv[128 * h + 96 + l];
+                blk[64 * h + l] = (uint8_t)((a & 15) | ((c & 15) << 4));
+                blk[64 * h + 32 + l] = (uint8_t)((b & 15) | ((e & 15) << 4));
+                blk[128 + 32 * h + l] = (uint8_t)((a >> 4) | ((b >> 4) << 2) | ((c >> 4) << 4) | ((e >> 4) << 6));
+            }
+        std::memcpy(blk + 192, sc, 16);
+        std::memcpy(blk + 208, &dh, 2);
+    }
+}
+
 // MXFP4 install encoder.  The reference only decodes MXFP4 (quant_gguf_mxfp4.rs:114-141: value =
 // kvalues[code] * 2^(e-128) with kvalues = 0,1,2,3,4,6,8,12 and their negatives); this encoder
 // picks the smallest scale that keeps the block's largest magnitude within 12 * scale and then
@@ -183,6 +228,7 @@ int encode_row(int dtype, const float* src, int64_t cols, uint8_t* dst) {
             return 0;
         case TSV_Q8_0: encode_q8_0(src, cols, dst); return 0;
         case TSV_Q4_K: encode_q4_k(src, cols, dst); return 0;
+        case TSV_Q6_K: encode_q6_k(src, cols, dst); return 0;
         case TSV_MXFP4: encode_mxfp4(src, cols, dst); return 0;
     }
     return -1;

@@ -40,6 +40,13 @@ __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, 
             const uint8_t* blk = raw + (tok * (hidden / 32) + (e >> 5)) * 34;
             const float d = f16_bits_to_f32(*(const uint16_t*)blk);
             v = (float)(int8_t)blk[2 + (e & 31)] * d;
+        } else if (dtype == TSV_Q6_K) {  // q6_k.rs:44-88
+            const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 210;
+            const int w = e & 255, h = w >> 7, k = (w >> 5) & 3, l = w & 31;
+            const int lo = (blk[64 * h + l + 32 * (k & 1)] >> (4 * (k >> 1))) & 0xF;
+            const int hi = (blk[128 + 32 * h + l] >> (2 * k)) & 3;
+            const float d = f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+            v = d * (float)(int8_t)blk[192 + (w >> 4)] * (float)((lo | (hi << 4)) - 32);
         } else if (dtype == TSV_F16) {
             v = f16_bits_to_f32(((const uint16_t*)raw)[tok * hidden + e]);
         } else if (dtype == TSV_BF16) {

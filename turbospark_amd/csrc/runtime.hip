@@ -17,7 +17,10 @@ using namespace tsv;
 namespace {
 
 struct LayerW {
-    TiledW qkv, wo, gate_up, down;
+    // the fused q/k/v projection; when the value projection has a format of its own (Q4_K_M files
+    // keep attn_v in Q6_K) `qkv` holds q and k only and `v_only` the rest, written to the same
+    // partial buffer at its column offset
+    TiledW qkv, v_only, wo, gate_up, down;
     int n_experts = 0, top_k = 0;     // routed experts: gate_up / down hold every expert's tiles
     TiledW router;
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
@@ -33,6 +36,7 @@ int dtype_fmt(int dtype) {
            : dtype == TSV_Q8_0  ? FMT_Q80
            : dtype == TSV_MXFP4 ? FMT_MX4
            : dtype == TSV_BF16  ? FMT_BF16
+           : dtype == TSV_Q6_K  ? FMT_Q6K
                                 : -1;
 }
 
@@ -169,13 +173,13 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
         return TSV_ERR_INVALID;
     }
     if (fmt < 0) {
-        set_error(std::string(what) + ": matmul weights must be Q4_K, Q8_0, MXFP4 or bf16 in this build");
+        set_error(std::string(what) + ": matmul weights must be Q4_K, Q6_K, Q8_0, MXFP4 or bf16 in this build");
         return TSV_ERR_UNSUPPORTED;
     }
     // MXFP4 rows may end inside a 256-element chunk (the tile is padded with zero blocks)
     const int gran = fmt == FMT_MX4 ? 32 : fmt_chunk_elems(fmt);
     if (cols % gran || rows < 1) {
-        set_error(std::string(what) + ": K must be whole 256 (Q4_K) / 128 (Q8_0) / 64 (bf16) / 32 (MXFP4) element runs");
+        set_error(std::string(what) + ": K must be whole 256 (Q4_K, Q6_K) / 128 (Q8_0) / 64 (bf16) / 32 (MXFP4) element runs");
         return TSV_ERR_UNSUPPORTED;
     }
     return TSV_OK;
@@ -375,10 +379,22 @@ int launch_pass(tsv_ctx* c, int m) {
         }
         if (rc) return rc;
         int sp = splits_for(L.qkv, m, EPI_PARTIAL);
+        if (L.v_only.tiles) {  // one split count for both pieces: the consumer adds `sp` partials per column
+            auto fits = [](const TiledW& w, int n) {
+                const int kslice = (w.kchunks + n - 1) / n;
+                return (w.kchunks + kslice - 1) / kslice == n;
+            };
+            while (sp > 1 && !(fits(L.qkv, sp) && fits(L.v_only, sp))) sp--;
+        }
         {
             PROF(PC_QKV);
             rc = 0;
-            for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++) rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, qkv_n);
+            for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++) {
+                rc = launch_gemm(s, L.qkv, c->xf_a, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n, L.qkv.n_rows);
+                if (!rc && L.v_only.tiles)
+                    rc = launch_gemm(s, L.v_only, c->xf_a, c->partial + L.qkv.n_rows, c->vp_dev, m, sp, EPI_PARTIAL, qkv_n,
+                                     L.v_only.n_rows);
+            }
         }
         if (rc) return rc;
         RopeKvArgs ra{};
@@ -671,8 +687,18 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             return fail(rc);
         const tsv_tensor* qkv[3] = {&s.wq, &s.wk, &s.wv};
         const tsv_tensor* wo[1] = {&s.wo};
-        if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv)) || (rc = make_tiled(c, st, wo, 1, false, &L.wo)))
-            return fail(rc);
+        if (s.wq.dtype != s.wk.dtype) {
+            set_error("open: the q and k projections must share a storage type");
+            return fail(TSV_ERR_UNSUPPORTED);
+        }
+        if (s.wv.dtype == s.wq.dtype) {
+            if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv))) return fail(rc);
+        } else {
+            const tsv_tensor* vonly[1] = {&s.wv};
+            if ((rc = make_tiled(c, st, qkv, 2, false, &L.qkv)) || (rc = make_tiled(c, st, vonly, 1, false, &L.v_only)))
+                return fail(rc);
+        }
+        if ((rc = make_tiled(c, st, wo, 1, false, &L.wo))) return fail(rc);
         const int ne = s.n_experts;
         if (ne > 0) {
             // every expert's gate/up rows interleave in runs of 32 inside the stacked matrix, so an
@@ -756,6 +782,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         const size_t kvb = (size_t)c->nkv * c->ctx_alloc * c->hd * 2;
         if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) return fail(rc);
         pneed = std::max(pneed, std::max(partial_need(L.qkv), partial_need(L.wo)));
+        pneed = std::max(pneed, (size_t)8 * 16 * ((size_t)(qd + 2 * kvd) + TILE_ROWS));
     }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
@@ -1459,8 +1486,12 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
                 }
             else if (fmt == FMT_Q80)
                 for (int i = 0; i < 256; i++) sc[2 * i + 1] = 0x20;
-            else
+            else if (fmt == FMT_MX4)
                 for (int i = 0; i < 512; i++) sc[i] = 0x70 + (sc[i] & 7);  // e8m0 scales around 2^-12
+            else if (fmt == FMT_Q6K)
+                for (int r = 0; r < 64; r++) host[t * tb + 13312 + r * 4 + 1] = 0x20;  // f16 d
+            else  // bf16: every value a small finite number
+                for (int i = 0; i < 4096; i++) host[t * tb + 2 * i + 1] = (uint8_t)(0x3C | (host[t * tb + 2 * i + 1] & 0x80));
         }
         for (int i = 0; i < rotate && !rc; i++) {
             rc = dev_alloc(c, &copies[i], w.bytes);

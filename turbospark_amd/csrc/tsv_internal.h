@@ -35,6 +35,13 @@ const std::string& get_error();
 //   MXFP4 tile, 8704 B (64 rows x 256 K): [unit 0..7][lane][16 B] the 32 e2m1 nibbles of the
 //                      lane's block u, nibbles re-ordered for the fp4 -> fp16 converter (see
 //                      gemm_core.h), then [lane][8 e8m0 scale bytes].
+//   Q6_K tile, 13568 B (64 rows x 256 K): per 64-K pair p three units [lane][16 B]: 3p and 3p + 1
+//                      hold the low nibbles of K steps 0..7 / 8..15 (one word per two steps, nibble
+//                      order k0 k1 of the first step, k0 k1 of the second, then k2 k3, k2 k3), 3p + 2
+//                      the high bit pairs (one word per four steps: pair e in bits 2e.. is the first,
+//                      pair e + 8 in bits 16 + 2e.. the second element of extraction e); then
+//                      [lane][16 int8 scales], then [lane][f16 d + 2 B pad] -- the 210 bytes of a
+//                      superblock, re-ordered.
 //   bf16 tile, 8192 B (64 rows x 64 K): [unit 0..7][lane][16 B] the lane's row at K steps 2u and
 //                      2u + 1, four values per step in the order k % 4 = 0, 2, 1, 3.
 // Rows past the matrix's last row are all-zero blocks (scale 0).
@@ -47,7 +54,7 @@ const std::string& get_error();
 // every 32-element sub-block, [K/256][g][sub%8][i], which the matmul uses to take the
 // integer-code offsets and the Q4_K min term back out.
 // ---------------------------------------------------------------------------------------
-enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2, FMT_BF16 = 3 };
+enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2, FMT_BF16 = 3, FMT_Q6K = 4 };
 
 struct TiledW {
     uint8_t* tiles = nullptr;  // device
@@ -60,8 +67,8 @@ struct TiledW {
 };
 
 inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q80 ? 128 : fmt == FMT_BF16 ? 64 : 256; }
-inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : fmt == FMT_BF16 ? 8192 : 8704; }
-inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : fmt == FMT_BF16 ? 2 : 8; }
+inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : fmt == FMT_BF16 ? 8192 : fmt == FMT_Q6K ? 13568 : 8704; }
+inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : fmt == FMT_BF16 ? 2 : fmt == FMT_Q6K ? 16 : 8; }
 constexpr int TILE_ROWS = 64;
 
 // index (in halfs) of activation element (row, k) in the fragment layout

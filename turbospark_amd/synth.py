@@ -12,6 +12,11 @@ CONFIGS = {
     # a small Q4_K stand-in with the 8B model's head geometry (GQA 4, head_dim 128)
     "small_q4_k": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
                        vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
+    # the tensor mix of a Q4_K_M file: Q4_K with the value and down projections of some layers, the
+    # output head (and here the embedding table) in Q6_K
+    "small_q4_k_m": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
+                         vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K,
+                         overrides={(0, "wv"): ffi.Q6_K, (0, "w_down"): ffi.Q6_K, "lm_head": ffi.Q6_K, "embed": ffi.Q6_K}),
     # the smallest shapes the per-XCD fused layer kernels take (8 KV heads, widths divisible
     # into eight chunk-aligned slices); norm weights are not all ones here
     "xcd_q4_k": dict(n_layers=2, hidden=1024, n_q_heads=32, n_kv_heads=8, head_dim=64, ffn=2048,
@@ -63,8 +68,12 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
 
     stream = [0]
 
-    def t(rows, cols, dtype=None, sig=None):
+    over = cfg.get("overrides", {})
+
+    def t(rows, cols, dtype=None, sig=None, name=None):
         stream[0] += 1
+        if name in over:
+            dtype = over[name]
         return ffi.synth_tensor(dt if dtype is None else dtype, seed, stream[0], sigma if sig is None else sig,
                                 rows, cols)
 
@@ -84,13 +93,14 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
         cfg["act_alpha"], cfg["act_limit"] = oss["act_alpha"], oss["act_limit"]
     layers = []
     for li in range(L):
-        lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H), wo=t(H, qd), ffn_norm=ones(H))
+        lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H, name=(li, "wv")), wo=t(H, qd),
+                  ffn_norm=ones(H))
         if E:
             xd = cfg.get("expert_dtype", dt)
             lw.update(n_experts=E, top_k=int(cfg["top_k"]), router=t(E, H, sig=cfg.get("router_sigma", sigma)),
                       we_gate=t(E * F, H, xd), we_up=t(E * F, H, xd), we_down=t(E * H, F, xd))
         else:
-            lw.update(w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F))
+            lw.update(w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F, name=(li, "w_down")))
         if oss:
             # attention biases and sinks are bf16 in the GGUF, expert and router biases f32
             lw.update(bq=vec(qd, 0.05, ffi.BF16), bk=vec(kvd, 0.05, ffi.BF16), bv=vec(kvd, 0.05, ffi.BF16),
@@ -103,4 +113,4 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
                 lw.update(router_bias=vec(E, 0.05), be_gate=mat(E, F, 0.05), be_up=mat(E, F, 0.05),
                           be_down=mat(E, H, 0.05))
         layers.append(lw)
-    return dict(embed=t(V, H), final_norm=ones(H), lm_head=t(V, H), layers=layers)
+    return dict(embed=t(V, H, name="embed"), final_norm=ones(H), lm_head=t(V, H, name="lm_head"), layers=layers)
