@@ -250,3 +250,32 @@ def test_refusals_by_name():
     gpu.rollback(ts.ffi.Point(base))
     with pytest.raises(TsvError, match="non-finite"):
         gpu.verify_accept([1, 2], base, ts.shaping(0.8, seed=3), draft_logits=bad)
+
+
+def test_a_vocabulary_that_is_not_a_multiple_of_anything_convenient():
+    """4099 rows in the head (a padded last tile) and logit rows that start at odd byte offsets (no
+    16-byte loads in the acceptance walks): forward parity and sampled rounds equal to the oracle."""
+    import turbospark_amd as ts
+    cfg, w, gpu, cpu = gc.build_pair("tiny_q8_0", max_context=96, vocab=4099)
+    V = cfg["vocab"]
+    prompt = np.random.default_rng(5).integers(0, V, 33).astype(np.int32)
+    gpu.prefill(prompt, 0, want_logits=False)
+    for i in range(0, 33, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    rng = np.random.default_rng(6)
+    feed = rng.integers(0, V, 5).astype(np.int32)
+    point = gpu.checkpoint()
+    assert gc.logit_error(gpu.verify(feed, 33), cpu.verify(feed, 33)) <= 2e-3
+    gpu.rollback(point)
+    for seed, kw in enumerate([{}, dict(top_k=40), dict(top_p=0.9), dict(min_p=0.05)]):
+        gcfg, ocfg = ts.shaping(0.8, seed=seed, **kw), ob.shaping(0.8, seed=seed, **kw)
+        draft = rng.standard_normal((4, V)).astype(np.float16)
+        draft[2] = np.round(draft[2] * 2) / 2
+        props, ds = gpu.draft_chain(draft, gcfg, 0)
+        oprops, ods = ob.draft_chain(draft, ocfg, list(prompt) + [7], len(prompt), 0)
+        assert list(props) == list(oprops) and ds == ods
+        res, logits = gpu.verify_accept([7] + [int(t) for t in props], 33, gcfg, draft_logits=draft, draw_step=ds,
+                                        want_logits=True)
+        want = ob.chain_round(logits, draft, props, ocfg, history=list(prompt) + [7], draw_step=ds)
+        _same(res, want, 33)
+        gpu.rollback(point)
