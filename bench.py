@@ -30,7 +30,12 @@ WORKLOADS = {
     # BASELINE configs[4]: gpt-oss arrangement (bf16 + MXFP4 experts top-4, window / full layers), T = 1.0
     "gptoss_120b_mxfp4_k8_ctx32768": dict(model="gptoss_120b", ctx=32768, k=8, temperature=1.0),
     "gptoss_small_k8_ctx256": dict(model="gptoss_small", ctx=256, k=8, temperature=1.0),
+    # BASELINE configs[2]: the 16-node tree (root, four children, chains below them), 16 384-token
+    # context, multi-branch rejection at T = 1.0
+    "llama3_8b_q4_k_tree16_ctx16384": dict(model="llama3_8b_q4_k", ctx=16384, k=15, temperature=1.0, tree=True),
+    "small_q4_k_tree16_ctx256": dict(model="small_q4_k", ctx=256, k=15, temperature=1.0, tree=True),
 }
+TREE16 = [-1, 0, 0, 0, 0, 1, 5, 6, 2, 8, 9, 3, 11, 12, 4, 14]
 
 
 def log(*a):
@@ -206,17 +211,23 @@ def main():
     # drafter logits N(0,1) per round, resident on the device; proposals drawn on the device
     rounds = args.warmup + args.steps
     shaping = [ts.shaping(T, seed=args.seed + r) if T > 0 else ts.shaping(0.0) for r in range(rounds)]
-    draft_host = rng.standard_normal((rounds, k, V)).astype(np.float16)
+    tree = TREE16 if wl.get("tree") else None
+    drows = m if tree else k      # a tree round needs the drafter's row of every node
+    draft_host = rng.standard_normal((rounds, drows, V)).astype(np.float16)
     draft_dev = hip.DeviceBuffer(draft_host.nbytes).upload(draft_host)
-    row_bytes = k * V * 2
+    row_bytes = drows * V * 2
     feeds, draw_steps = [], []
     for r in range(rounds):
+        if tree:   # node tokens uniform over the vocabulary
+            feeds.append([anchor] + [int(t) for t in rng.integers(0, V, k)])
+            draw_steps.append(0)
+            continue
         props, ds = eng.draft_chain((draft_dev.address(r * row_bytes), k), shaping[r], 0)
         feeds.append([anchor] + [int(t) for t in props])
         draw_steps.append(ds)
 
     def step(r):
-        res = eng.verify_accept(feeds[r], base, shaping[r],
+        res = eng.verify_accept(feeds[r], base, shaping[r], parent=tree,
                                 draft_logits=draft_dev.address(r * row_bytes) if T > 0 else None,
                                 draw_step=draw_steps[r])
         eng.rollback(point)   # every step verifies at exactly `ctx` tokens of context
@@ -295,7 +306,7 @@ def main():
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(cfg, weights, eng, base, feeds[args.warmup], mean_acc)
+        cpu = cpu_baseline(cfg, weights, eng, base, feeds[args.warmup], mean_acc, tree)
 
     out = {
         "metric": "verified tokens/s + verify-step latency (8B Q4_K, k=4, 4K ctx); % HBM roofline",
@@ -315,7 +326,7 @@ def main():
     print(json.dumps(out), flush=True)
 
 
-def cpu_baseline(cfg, weights, eng, base, feed, mean_acc):
+def cpu_baseline(cfg, weights, eng, base, feed, mean_acc, parent=None):
     """The oracle (the CPU restatement of the reference path) timed on this host, one thread, on
     a bounded sample: the first two layers plus the output head of the same verify step, and
     the head alone; the full-stack time is extrapolated linearly in the layer count."""
@@ -330,11 +341,11 @@ def cpu_baseline(cfg, weights, eng, base, feed, mean_acc):
         vc[:base] = vg.astype(np.float32)
     cpu.rewind_to(base)
     t0 = time.perf_counter()
-    cpu.verify(feed, base, n_layers_run=0)
+    cpu.verify(feed, base, parent=parent, n_layers_run=0)
     t_head = time.perf_counter() - t0
     cpu.rewind_to(base)
     t0 = time.perf_counter()
-    cpu.verify(feed, base, n_layers_run=sample_layers)
+    cpu.verify(feed, base, parent=parent, n_layers_run=sample_layers)
     t_sample = time.perf_counter() - t0
     t_full = t_head + (t_sample - t_head) * L / sample_layers
     return {"value": round((mean_acc + 1.0) / t_full, 4), "unit": "verified tokens/s", "cores": 1, "kind": "port",

@@ -642,7 +642,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         }
         unsigned long long* hp = hist + (long)jobi * 2 * 65536;
         unsigned long long* hsel = mode == 2 ? hp + 65536 : hp;
-        const double* w = work + (long)jobi * 2 * vocab + (mode == 2 ? vocab : 0);
+        const double* w = kind == 2 ? work + (long)dec.pad * vocab : work + (long)jobi * 2 * vocab + (mode == 2 ? vocab : 0);
         const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, dec.job.row_p);
 
         // 64 consecutive rank bins per thread (see bin_addr); integer sums are exact and order
@@ -797,25 +797,42 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
 // order -- child x is accepted when r * q(x) <= p(x) for a fresh uniform r; a rejection replaces
 // p by normalise(max(p - q, 0)) (kept as is when that mass is below 1e-12) -- and when no child
 // survives the next token is drawn from the p that is left.  No stop / budget bookkeeping.
-// One workgroup walks the tree; p and q live as dense f64 rows in the work area (job 0: slot 1
-// holds p, which is also what the final draw's histogram and in-bin walk read; slot 0 is scratch
-// for the residual; job 1 slot 0 holds q).
-__global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, const uint16_t* draft,
-                                                       const AcceptParams* app, double* scratch, double* work,
-                                                       unsigned long long* hist, Decision* dec_out,
-                                                       int32_t* path_out) {
-    __shared__ RowStat s_p, s_q;
+//
+// First every node's p and q are written out as dense f64 rows by the whole chip (work slots
+// 0..m-1 and m..2m-1); then one workgroup walks the tree.  A child test is two lookups; only a
+// rejection costs a pass over the vocabulary (slots 32 and 33 alternate as the residual, whose
+// normalising division is applied when it is read, so a pass reads two rows and writes one).
+__global__ __launch_bounds__(256) void k_tree_probs(const uint16_t* target, const uint16_t* draft,
+                                                    const AcceptParams* app, double* scratch, double* work) {
+    __shared__ RowStat st;
+    const AcceptParams& ap = *app;
+    const int seg = blockIdx.x, row = blockIdx.y, vocab = ap.vocab;
+    Layout L = layout(scratch);
+    if (threadIdx.x < 64) {
+        const RowStat s0 = load_stat(L, row);
+        if (threadIdx.x == 0) st = s0;
+    }
+    __syncthreads();
+    const RowStat s0 = st;
+    const double inv_t = 1.0 / ap.temperature;
+    const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, row);
+    double* out = work + (long)row * vocab;
+    const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) out[v] = prob_of(lp[v], v, s0, inv_t);
+}
+
+constexpr int TREE_SCRATCH_SLOT = 2 * TSV_MAX_ROWS;  // two residual rows behind the 32 distribution rows
+
+__global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, const AcceptParams* app,
+                                                       double* scratch, double* work, unsigned long long* hist,
+                                                       Decision* dec_out, int32_t* path_out) {
     __shared__ double red[16];
     __shared__ int s_accept;
     __shared__ double s_margin;
     const AcceptParams& ap = *app;
-    const int tid = threadIdx.x, wave = tid >> 6;
+    const int tid = threadIdx.x;
     const int vocab = ap.vocab, m = ap.m;
-    const double inv_t = 1.0 / ap.temperature;
     Layout L = layout(scratch);
-    double* pc = work + vocab;          // job 0, slot 1
-    double* pr = work;                  // job 0, slot 0
-    double* qa = work + 2 * (long)vocab;  // job 1, slot 0
     unsigned long long* hr = hist + 65536;
     uint64_t ds = ap.draw_step;
     int at = 0, plen = 1;
@@ -823,30 +840,18 @@ __global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, c
         path_out[0] = 0;
         s_margin = 1.0;
     }
+    __syncthreads();
     for (;;) {
-        if (wave == 0) {
-            const RowStat st = load_stat(L, at);
-            if (tid == 0) s_p = st;
-        } else if (wave == 1) {
-            const RowStat st = load_stat(L, m + at);
-            if ((tid & 63) == 0) s_q = st;
-        }
-        __syncthreads();
-        const uint16_t* lp = target + (long)at * vocab;
-        const uint16_t* lq = draft + (long)at * vocab;
-        for (int v = tid; v < vocab; v += 1024) {
-            pc[v] = prob_of(lp[v], v, s_p, inv_t);
-            qa[v] = prob_of(lq[v], v, s_q, inv_t);
-        }
-        __threadfence_block();
-        __syncthreads();
-        int hit = -1;
+        const double* src = work + (long)at * vocab;  // the node's p; its values are src[v] / Z
+        const double* q = work + (long)(m + at) * vocab;
+        double Z = 1.0;
+        int which = 0, hit = -1;
         for (int s = 1; s < m && hit < 0; s++) {
             if (ap.parent[s] != at) continue;
             if (tid == 0) {
                 const int32_t x = ap.feed[s];
                 const double r = unit_draw(ap.seed, ds);
-                const double px = pc[x], qx = qa[x];
+                const double px = src[x] / Z, qx = q[x];
                 double mg = s_margin;
                 fold_margin(mg, r * qx, px);
                 s_margin = mg;
@@ -854,37 +859,43 @@ __global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, c
             }
             ds += 1;
             __syncthreads();
-            if (s_accept) {
+            const bool ok = s_accept != 0;
+            __syncthreads();
+            if (ok) {
                 hit = s;
                 break;
             }
-            // residual: p <- normalise(max(p - q, 0))
+            // residual: max(p - q, 0), normalised later by its total
+            double* dst = work + (long)(TREE_SCRATCH_SLOT + which) * vocab;
             double acc = 0.0;
             for (int v = tid; v < vocab; v += 1024) {
-                const double mv = fmax(pc[v] - qa[v], 0.0);
-                pr[v] = mv;
+                const double mv = fmax(src[v] / Z - q[v], 0.0);
+                dst[v] = mv;
                 acc += mv;
             }
             const double total = block_sum_f64(acc, red);
-            if (total >= 1e-12)
-                for (int v = tid; v < vocab; v += 1024) pc[v] = pr[v] / total;
             __threadfence_block();
             __syncthreads();
+            if (total >= 1e-12) {  // distribution.rs:96-126: below that the distribution is kept
+                src = dst;
+                Z = total;
+                which ^= 1;
+            }
         }
         if (hit >= 0) {
             if (tid == 0) path_out[plen] = hit;
             plen += 1;
             at = hit;
-            __syncthreads();
             continue;
         }
         // nothing accepted below `at`: the next token is drawn from what is left of p
         const uint16_t* lpk = target + (long)at * vocab;
         for (int v = tid; v < vocab; v += 1024) {
-            const double mv = pc[v];
+            const double mv = src[v] / Z;
             if (mv > 0.0) atomicAdd(hr + bin_addr(rank_key(lpk[v])), (unsigned long long)(mv * FIX));
         }
-        if (tid < NSEG * NSUB) L.segtot[tid] = tid == 0 ? 1.0 : 0.0;  // the masses are already normalised
+        // the draw divides the stored values by the fold of these pieces: Z, exactly
+        if (tid < NSEG * NSUB) L.segtot[tid] = tid == 0 ? Z : 0.0;
         if (tid == 0) {
             Decision d;
             d.job.mode = 2;
@@ -894,7 +905,7 @@ __global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, c
             d.accepted = plen - 1;
             d.committed = plen - 1;
             d.stopped = 0;
-            d.pad = 0;
+            d.pad = (int32_t)((src - work) / vocab);  // the work slot the draw reads
             d.draw_step = ds + 1;
             d.margin = s_margin;
             dec_out[0] = d;
@@ -1049,7 +1060,8 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
         hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
         launch_trunc(s, target, draft, ap.m, rows2, ap_dev, ap, sc);
         hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, it);
-        hipLaunchKernelGGL(k_tree_sampled, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+        hipLaunchKernelGGL(k_tree_probs, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
+        hipLaunchKernelGGL(k_tree_sampled, dim3(1), dim3(1024), 0, s, target, ap_dev, sc.stats, sc.work,
                            (unsigned long long*)sc.hist, decisions(sc), path);
         hipLaunchKernelGGL(k_pick, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                            (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);

@@ -264,7 +264,7 @@ struct AcceptResult {
 };
 struct AcceptScratch {
     double* stats;       // accept_stats_doubles() doubles: row statistics, partials, decisions
-    double* work;        // [16 jobs][2][vocab] candidate masses (p, residual)
+    double* work;        // [16 jobs][2][vocab] candidate masses (p, residual) + two more rows (tree residuals)
     uint64_t* hist;      // [16 jobs][2][65536] fixed-point mass per rank bin; a round clears what it uses first
     uint32_t* counters;  // 64 words: error flag, greedy arg-max per row
     uint64_t* tmass;     // [32 rows][65536] fixed-point softmax mass per rank bin (top-p cut)
