@@ -79,7 +79,7 @@ __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) 
     const int j = lane & 15, kg = lane >> 4;
     const int chunk = blockIdx.x, h = blockIdx.y, rt0 = blockIdx.z * RT;
     const VerifyParams* vp = a.vp;
-    const int M = vp->m, base = vp->base, kvlen = base + M;
+    const int M = a.base_hint >= 0 ? a.m_hint : vp->m, base = a.base_hint >= 0 ? a.base_hint : vp->base, kvlen = base + M;
     const int nblk = (kvlen + 15) >> 4;
     // sliding window (families/gptoss/attn.rs:120-137): a row at sequence length n sees positions
     // n - window .. n - 1.  The window exceeds the pass width, so every row keeps its whole drafted

@@ -285,6 +285,7 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     float4v acc[NG];
 #pragma unroll
     for (int g = 0; g < NG; g++) acc[g] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int M = a.vp->m;  // asked for before the K loop, needed after it
 
     // Software pipeline over the K chunks, STAGES tiles in flight per wave.  Every load in the
     // steady state is unconditional (straight-line code), so the compiler can wait on the oldest
@@ -318,7 +319,6 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
             if (c + s < nc) compute(st[s], k, acc);
     }
 
-    const int M = a.vp->m;
     if (a.kparts == 1) {
 #pragma unroll
         for (int g = 0; g < NG; g++) epilogue<EPI>(a, tile, split, g, acc[g], lane, M);

@@ -437,6 +437,8 @@ int launch_pass(tsv_ctx* c, int m) {
         aa.window = L.window;
         aa.sinks = L.sinks;
         aa.vp = c->vp_dev;
+        aa.m_hint = m;
+        aa.base_hint = c->use_graph ? -1 : c->vp_host->base;  // a captured launch must read the position at replay
         {
             PROF(PC_ATTN);
             rc = 0;
@@ -1379,6 +1381,8 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
         aa.window = window;
         aa.sinks = sinks_dev;
         aa.vp = vpd;
+        aa.m_hint = m;
+        aa.base_hint = (int)base;
         rc = launch_attention(c->stream, aa, m);
     }
     std::vector<uint16_t> frag(xfb / 2);

@@ -227,6 +227,9 @@ struct AttnArgs {
     int window;          // 0: full; else a row sees the last `window` positions of its sequence
     const float* sinks;  // nullable: one logit per q head joining the softmax maximum and denominator
     const VerifyParams* vp;
+    // row count and base position by value when the launch knows them (saves the kernel one
+    // dependent memory round trip before its first K/V load); base_hint < 0: read them from vp
+    int m_hint, base_hint;
 };
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
