@@ -179,7 +179,7 @@ def main():
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "
-                 "supported (see DESIGN.md, 'how the path would shard').")
+                 "supported: every number here is one GPU's throughput.")
 
     import turbospark_amd as ts
     from turbospark_amd import hip, synth
