@@ -122,3 +122,37 @@ def test_refusals_by_name():
     with pytest.raises(TsvError, match="parent"):
         gpu.verify_tree([1, 2], [-1, 1], 16)
     assert gpu.position == 16
+
+
+def test_graph_replay_of_the_pass_equals_plain_launches():
+    """The opt-in captured launch sequence (one graph per row count; positions, tokens and the tree
+    shape are read from device memory at replay): every replay, with eager work and
+    synchronisations between them, must give the bits the plain launches give."""
+    import os
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS["small_q4_k"], max_context=160)
+    w = synth.make_weights(cfg, seed=5)
+    plain = ts.HipVerifier(cfg, w)
+    os.environ["TSV_GRAPH"] = "1"
+    try:
+        graph = ts.HipVerifier(cfg, w)
+    finally:
+        os.environ["TSV_GRAPH"] = "0"
+    prompt = _prompt(37, cfg["vocab"], 3)
+    for eng in (plain, graph):
+        eng.prefill(prompt, 0, want_logits=False)
+    rng = np.random.default_rng(9)
+    base = 37
+    for rnd, m in enumerate([5, 5, 3, 5, 16, 5, 3]):
+        feed = rng.integers(0, cfg["vocab"], m).astype(np.int32)
+        a = plain.verify(feed, base)
+        b = graph.verify(feed, base)
+        assert np.array_equal(a, b), (rnd, m)
+        keep = 1 + rnd % 3                      # eager work between replays: a partial rollback
+        for eng in (plain, graph):
+            eng.rollback(ts.ffi.Point(base + keep))
+        base += keep
+    parent = [-1, 0, 0, 1, 1]
+    feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    assert np.array_equal(plain.verify_tree(feed, parent, base), graph.verify_tree(feed, parent, base))
