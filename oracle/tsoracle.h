@@ -21,6 +21,19 @@
  *                                        only tests invariants; its mixer is that textbook routine)
  *   - rejection round .................. distributional law (first emitted token ~ target p,
  *                                        acceptance rate = sum min(p,q)) over thousands of seeds
+ *   - Q6_K decode / encode ............. the reference's hand-packed superblock literal; round-trip
+ *                                        bound, both scale signs, zero block
+ *   - YaRN table ....................... the reference's gpt-oss scalars -> mscale 1.3465736, untouched
+ *                                        fast end, fully interpolated slow end, ramp between ggml's
+ *                                        correction dimensions, swapped betas differ
+ *   - swiglu_oai ....................... closed forms on both sides of every clamp, the (up + 1) term
+ *   - gpt-oss layer graph .............. an independent float64 numpy forward (biases, sinks, window,
+ *                                        YaRN, router bias, expert biases, clamped SwiGLU), 2e-4; each
+ *                                        term's removal moves the logits
+ *   - adaptive depth ................... the reference's unit scenarios, one by one
+ *   - generation loop .................. greedy output == plain greedy decoding for any drafter, exact
+ *                                        budget, stop tokens, context cap, a self-drafting target is
+ *                                        always accepted, draw counter = 2 offered + 2 rounds - 1
  * PARITY UNPINNED (no golden value exists anywhere in the reference):
  *   - tso_tree_round_sampled: multi-branch rejection sampling on a tree is not
  *     defined by the reference at all; the definition here is this project's own
