@@ -16,7 +16,7 @@ __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, 
     const int m = blockIdx.x;
     if (m >= vp->m) return;
     const long tok = vp->feed[m];
-    for (int e = threadIdx.x; e < hidden; e += blockDim.x) {
+    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < hidden; e += blockDim.x * gridDim.y) {
         float v;
         if (dtype == TSV_Q4_K) {
             const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 144;
@@ -60,7 +60,7 @@ __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, 
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
                  const VerifyParams* vp, int m) {
-    hipLaunchKernelGGL(k_embed, dim3(m), dim3(256), 0, s, raw, dtype, hidden, x, vp);
+    hipLaunchKernelGGL(k_embed, dim3(m, (hidden + 511) / 512), dim3(256), 0, s, raw, dtype, hidden, x, vp);  // two elements per thread
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
