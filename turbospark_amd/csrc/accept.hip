@@ -254,8 +254,10 @@ __device__ int sink_commit(const AcceptParams& ap, int32_t token, uint64_t& gene
 }
 
 // speculative.rs:694-754: the sequential walk over the proposals of a sampled chain round.
-__device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t* target,
-                                         const uint16_t* draft, const RowStat* stats) {
+// tbits / dbits: the target's and the drafter's logit of proposal i in its own row, fetched by
+// the caller for all proposals at once (one memory latency instead of one per proposal).
+__device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t* tbits, const uint16_t* dbits,
+                                         const RowStat* stats) {
     Decision d;
     d.job.mode = 0;
     d.job.row_p = d.job.row_q = 0;
@@ -268,8 +270,8 @@ __device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t*
     for (int i = 0; i < ap.k; i++) {
         const int32_t x = ap.feed[i + 1];
         const RowStat sp = stats[i], sq = stats[ap.m + i];
-        const double px = prob_of(target[(long)i * ap.vocab + x], x, sp, inv_t);
-        const double qx = prob_of(draft[(long)i * ap.vocab + x], x, sq, inv_t);
+        const double px = prob_of(tbits[i], x, sp, inv_t);
+        const double qx = prob_of(dbits[i], x, sq, inv_t);
         const double r = unit_draw(ap.seed, ds);
         ds += 1;
         fold_margin(d.margin, r * qx, px);
@@ -306,9 +308,16 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     __shared__ Decision dec;
     __shared__ double red[4];
     __shared__ RowStat stats[MAX_DIST_ROWS];
+    __shared__ uint16_t s_tb[TSV_MAX_ROWS], s_db[TSV_MAX_ROWS];
     const AcceptParams& ap = *app;
     const int seg = blockIdx.x, jobi = blockIdx.y, sub = blockIdx.z;
     Layout L = layout(scratch);
+    if (kind == 0 && (int)threadIdx.x < ap.k) {
+        const int i = threadIdx.x;
+        const int32_t x = ap.feed[i + 1];
+        s_tb[i] = target[(long)i * ap.vocab + x];
+        s_db[i] = draft[(long)i * ap.vocab + x];
+    }
     {
         // every row's statistics, one wave per row at a time
         const int rows = kind == 0 ? ap.m + ap.k : ap.k;
@@ -320,7 +329,7 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     __syncthreads();
     if (threadIdx.x == 0) {
         if (kind == 0) {
-            dec = decide_chain_sampled(ap, target, draft, stats);
+            dec = decide_chain_sampled(ap, s_tb, s_db, stats);
         } else {
             dec.job.mode = 1;
             dec.job.row_p = ap.m + jobi;

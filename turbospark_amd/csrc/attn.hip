@@ -268,12 +268,23 @@ __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) 
 // q_head*hd + d).  The first
 // wave turns the (m_c, l_c) pairs into per-chunk weights once; every thread then sums its
 // output element over the chunks with independent loads.
+// NCH > 0: the chunk count as a compile-time constant -- every thread then asks for its output
+// element of all chunks before the (m, l) pairs are looked at (the two groups of loads do not
+// depend on each other), and the kernel is one memory latency instead of two.  NCH == 0: any count.
+template <int NCH>
 __global__ void k_attn_combine(AttnArgs a, int G, int R) {
     __shared__ float wgt[64];
     __shared__ float s_den;
     const int m = blockIdx.x, qh = blockIdx.y, d = threadIdx.x;
-    const int hd = a.hd, nch = a.nch;
+    const int hd = a.hd, nch = NCH > 0 ? NCH : a.nch;
     const int h = qh / G, g = qh - h * G, r = m * G + g;
+    const float* po = a.part_o + ((long)h * nch * R + r) * hd + min(d, hd - 1);
+    const long stride = (long)R * hd;
+    float pre[NCH > 0 ? NCH : 1];
+    if (NCH > 0) {
+#pragma unroll
+        for (int c = 0; c < NCH; c++) pre[c] = po[c * stride];
+    }
     if (d < 64) {
         float mc = -INFINITY, lc = 0.f;
         if (d < nch) {
@@ -296,11 +307,14 @@ __global__ void k_attn_combine(AttnArgs a, int G, int R) {
     }
     __syncthreads();
     if (d >= hd) return;
-    const float* po = a.part_o + ((long)h * nch * R + r) * hd + d;
-    const long stride = (long)R * hd;
     float num = 0.f;
+    if (NCH > 0) {
+#pragma unroll
+        for (int c = 0; c < NCH; c++) num += wgt[c] * pre[c];
+    } else {
 #pragma unroll 8
-    for (int c = 0; c < nch; c++) num += wgt[c] * po[c * stride];
+        for (int c = 0; c < nch; c++) num += wgt[c] * po[c * stride];
+    }
     const _Float16 o16 = (_Float16)(num / s_den);
     const int kk = qh * hd + d;
     ((_Float16*)a.xfrag)[frag_index(kk, m)] = o16;
@@ -340,7 +354,13 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     else
         rc = launch_partial<HD, 2, 3>(s, a, G, R, groups);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_attn_combine, dim3(m, a.nq), dim3(HD < 64 ? 64 : HD), 0, s, a, G, R);
+    const dim3 cgrid(m, a.nq), cblock(HD < 64 ? 64 : HD);
+    switch (a.nch) {
+        case 8: hipLaunchKernelGGL(k_attn_combine<8>, cgrid, cblock, 0, s, a, G, R); break;
+        case 16: hipLaunchKernelGGL(k_attn_combine<16>, cgrid, cblock, 0, s, a, G, R); break;
+        case 32: hipLaunchKernelGGL(k_attn_combine<32>, cgrid, cblock, 0, s, a, G, R); break;
+        default: hipLaunchKernelGGL(k_attn_combine<0>, cgrid, cblock, 0, s, a, G, R); break;
+    }
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

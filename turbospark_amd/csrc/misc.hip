@@ -1,5 +1,7 @@
 // Small per-row kernels of the verify pass: embedding lookup, residual-add + RMSNorm,
 // q/k rotation + KV-cache store, KV row gather / read-back.
+#include <type_traits>
+
 #include "tsv_internal.h"
 
 namespace tsv {
@@ -92,49 +94,75 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
     float4* xr = (float4*)(x + (long)m * hidden);
     const float4* wr = (const float4*)w;
     const int n4 = hidden >> 2;
+    // the norm weights of a thread's first group are asked for now: they come from HBM (nothing
+    // else reads them in a step) and would otherwise be waited for after the reduction
+    const float4 g_first = (int)threadIdx.x < n4 ? wr[threadIdx.x] : float4{0.f, 0.f, 0.f, 0.f};
+    float4 v_first = {0.f, 0.f, 0.f, 0.f};
     float ss = 0.f;
-    for (int i = threadIdx.x; i < n4; i += 1024) {
-        float4 v = xr[i];
-        if (weights) {
-            // routed experts (families/llama/moe.rs:193-198): the slot outputs are weighted and summed
-            // in rank order starting from zero, then added to the stream; product and sum rounded apart
-            float4 r = {0.f, 0.f, 0.f, 0.f};
-            for (int s = 0; s < splits; s++) {
-                const float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
-                const float ws = weights[m * 8 + s];
-                r.x = __fadd_rn(r.x, __fmul_rn(ws, p.x));
-                r.y = __fadd_rn(r.y, __fmul_rn(ws, p.y));
-                r.z = __fadd_rn(r.z, __fmul_rn(ws, p.z));
-                r.w = __fadd_rn(r.w, __fmul_rn(ws, p.w));
+    // The partial sums of a group are loaded with a compile-time count (one of nine straight-line
+    // variants, chosen by a uniform branch): all loads are in flight before the first add, where a
+    // counted loop would wait for each in turn.
+    auto run = [&](auto S) {
+        constexpr int NS = decltype(S)::value;
+        for (int i = threadIdx.x; i < n4; i += 1024) {
+            float4 v = xr[i];
+            float4 p[NS > 0 ? NS : 1];
+#pragma unroll
+            for (int s = 0; s < NS; s++) p[s] = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
+            if (weights) {
+                // routed experts (families/llama/moe.rs:193-198): the slot outputs are weighted and summed
+                // in rank order starting from zero, then added to the stream; product and sum rounded apart
+                float4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < NS; s++) {
+                    const float ws = weights[m * 8 + s];
+                    r.x = __fadd_rn(r.x, __fmul_rn(ws, p[s].x));
+                    r.y = __fadd_rn(r.y, __fmul_rn(ws, p[s].y));
+                    r.z = __fadd_rn(r.z, __fmul_rn(ws, p[s].z));
+                    r.w = __fadd_rn(r.w, __fmul_rn(ws, p[s].w));
+                }
+                v.x = __fadd_rn(v.x, r.x);
+                v.y = __fadd_rn(v.y, r.y);
+                v.z = __fadd_rn(v.z, r.z);
+                v.w = __fadd_rn(v.w, r.w);
+            } else {
+#pragma unroll
+                for (int s = 0; s < NS; s++) {
+                    v.x = __fadd_rn(v.x, p[s].x);
+                    v.y = __fadd_rn(v.y, p[s].y);
+                    v.z = __fadd_rn(v.z, p[s].z);
+                    v.w = __fadd_rn(v.w, p[s].w);
+                }
+                if (bias) {  // the output projection's bias (families/gptoss/mod.rs:16)
+                    const float4 b = *(const float4*)(bias + 4 * i);
+                    v.x += b.x;
+                    v.y += b.y;
+                    v.z += b.z;
+                    v.w += b.w;
+                }
             }
-            v.x = __fadd_rn(v.x, r.x);
-            v.y = __fadd_rn(v.y, r.y);
-            v.z = __fadd_rn(v.z, r.z);
-            v.w = __fadd_rn(v.w, r.w);
-        } else {
-            for (int s = 0; s < splits; s++) {
-                const float4 p = *(const float4*)(partial + ((long)s * 16 + m) * ldp + 4 * i);
-                v.x = __fadd_rn(v.x, p.x);
-                v.y = __fadd_rn(v.y, p.y);
-                v.z = __fadd_rn(v.z, p.z);
-                v.w = __fadd_rn(v.w, p.w);
-            }
-            if (bias) {  // the output projection's bias (families/gptoss/mod.rs:16)
-                const float4 b = *(const float4*)(bias + 4 * i);
-                v.x += b.x;
-                v.y += b.y;
-                v.z += b.z;
-                v.w += b.w;
-            }
+            xr[i] = v;
+            if (i == (int)threadIdx.x) v_first = v;
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
         }
-        xr[i] = v;
-        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    };
+    switch (splits) {
+        case 0: run(std::integral_constant<int, 0>{}); break;
+        case 1: run(std::integral_constant<int, 1>{}); break;
+        case 2: run(std::integral_constant<int, 2>{}); break;
+        case 3: run(std::integral_constant<int, 3>{}); break;
+        case 4: run(std::integral_constant<int, 4>{}); break;
+        case 5: run(std::integral_constant<int, 5>{}); break;
+        case 6: run(std::integral_constant<int, 6>{}); break;
+        case 7: run(std::integral_constant<int, 7>{}); break;
+        default: run(std::integral_constant<int, 8>{}); break;
     }
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
     float* sums = (float*)((char*)xfrag + xfrag_sum_offset(hidden));
     for (int i = threadIdx.x; i < n4; i += 1024) {
-        const float4 v = xr[i], g = wr[i];
+        const bool first = i == (int)threadIdx.x;
+        const float4 v = first ? v_first : xr[i], g = first ? g_first : wr[i];
         // elements 4i..4i+3 are one K step of the fragment layout, stored in the order (0, 2, 1, 3)
         typedef _Float16 half4 __attribute__((ext_vector_type(4)));
         half4 h = {(_Float16)(v.x * g.x * inv), (_Float16)(v.z * g.z * inv), (_Float16)(v.y * g.y * inv),
@@ -150,6 +178,10 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
 
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
                    float eps, int hidden, uint4* xfrag, int m, const float* weights, const float* bias) {
+    if (splits < 0 || splits > 8) {
+        set_error("residual add: at most eight partial sums");
+        return TSV_ERR_UNSUPPORTED;
+    }
     hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
                        (_Float16*)xfrag, weights, bias);
     TSV_HIP(hipGetLastError());
@@ -183,17 +215,41 @@ int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int 
 __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
     const int m = blockIdx.x, head = blockIdx.y;
     const VerifyParams* vp = a.vp;
-    if (m >= vp->m) return;
+    // everything the kernel needs from the parameter block is asked for at once
+    const int rows = vp->m, rot_pos = vp->pos[m], base = vp->base;
+    if (m >= rows) return;
     const int hd = a.hd, half = hd >> 1, i = threadIdx.x;
     const int kind = head < a.nq ? 0 : head < a.nq + a.nkv ? 1 : 2;
     const int h = kind == 0 ? head : kind == 1 ? head - a.nq : head - a.nq - a.nkv;
     const int col = head * hd;  // q heads, then k heads, then v heads: the fused projection's row order
     float x0 = 0.f, x1 = 0.f;
     if (i < half) {
-        for (int s = 0; s < a.splits; s++) {
-            const float* p = a.qkv + ((long)s * 16 + m) * a.ldq + col;
-            x0 += p[i];
-            x1 += p[i + half];
+        // compile-time split count (a uniform branch picks the variant): every partial is in flight
+        // before the first add
+        auto sum_splits = [&](auto S) {
+            constexpr int NS = decltype(S)::value;
+            float p0[NS], p1[NS];
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                const float* p = a.qkv + ((long)s * 16 + m) * a.ldq + col;
+                p0[s] = p[i];
+                p1[s] = p[i + half];
+            }
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                x0 += p0[s];
+                x1 += p1[s];
+            }
+        };
+        switch (a.splits) {
+            case 1: sum_splits(std::integral_constant<int, 1>{}); break;
+            case 2: sum_splits(std::integral_constant<int, 2>{}); break;
+            case 3: sum_splits(std::integral_constant<int, 3>{}); break;
+            case 4: sum_splits(std::integral_constant<int, 4>{}); break;
+            case 5: sum_splits(std::integral_constant<int, 5>{}); break;
+            case 6: sum_splits(std::integral_constant<int, 6>{}); break;
+            case 7: sum_splits(std::integral_constant<int, 7>{}); break;
+            default: sum_splits(std::integral_constant<int, 8>{}); break;
         }
         if (a.bias) {  // before the rotation (families/gptoss/attn.rs:88-101)
             x0 += a.bias[col + i];
@@ -212,7 +268,7 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
     }
     if (i >= half) return;
     if (kind != 2) {
-        const float angle = (float)vp->pos[m] * a.freqs[i];
+        const float angle = (float)rot_pos * a.freqs[i];
         float sn, cs;
         sincosf(angle, &sn, &cs);
         sn *= a.mscale;
@@ -228,7 +284,7 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
         q[i] = h0;
         q[i + half] = h1;
     } else {
-        const int pos = vp->base + m;  // the cache slot of row m
+        const int pos = base + m;  // the cache slot of row m
         if (kind == 1) {
             _Float16* k = (_Float16*)a.kc + ((long)h * a.max_ctx + pos) * hd;
             k[i] = h0;
@@ -244,6 +300,10 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
 }
 
 int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m) {
+    if (a.splits < 1 || a.splits > 8) {
+        set_error("rope: one to eight partial sums");
+        return TSV_ERR_UNSUPPORTED;
+    }
     hipLaunchKernelGGL(k_rope_kv, dim3(m, a.nq + 2 * a.nkv), dim3(64), 0, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;

@@ -36,8 +36,12 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
             const int e = lane + 64 * j;
             v[j] = -INFINITY;
             if (e < ne) {
-                float s = 0.f;
-                for (int sp = 0; sp < a.splits; sp++) s += a.logits[((size_t)sp * 16 + m) * a.ld + e];
+                float part[8], s = 0.f;  // all partials in flight together, added in split order
+#pragma unroll
+                for (int sp = 0; sp < 8; sp++) part[sp] = a.logits[((size_t)min(sp, a.splits - 1) * 16 + m) * a.ld + e];
+#pragma unroll
+                for (int sp = 0; sp < 8; sp++)
+                    if (sp < a.splits) s += part[sp];
                 if (a.bias) s += a.bias[e];  // before the top-k (families/gptoss/moe.rs:82-87)
                 v[j] = s;
             }
