@@ -254,10 +254,9 @@ __device__ int sink_commit(const AcceptParams& ap, int32_t token, uint64_t& gene
 }
 
 // speculative.rs:694-754: the sequential walk over the proposals of a sampled chain round.
-// tbits / dbits: the target's and the drafter's logit of proposal i in its own row, fetched by
-// the caller for all proposals at once (one memory latency instead of one per proposal).
-__device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t* tbits, const uint16_t* dbits,
-                                         const RowStat* stats) {
+// pxs / qxs: p_i(x_i) and q_i(x_i) of every proposal, computed by the caller in parallel (one lane
+// per proposal: an f64 exp + pow chain per value is long for a single thread to walk k times).
+__device__ Decision decide_chain_sampled(const AcceptParams& ap, const double* pxs, const double* qxs) {
     Decision d;
     d.job.mode = 0;
     d.job.row_p = d.job.row_q = 0;
@@ -265,13 +264,10 @@ __device__ Decision decide_chain_sampled(const AcceptParams& ap, const uint16_t*
     d.accepted = d.committed = d.stopped = d.pad = 0;
     d.margin = 1.0;
     uint64_t ds = ap.draw_step, gen = ap.generated;
-    const double inv_t = 1.0 / ap.temperature;
     int reject = -1;
     for (int i = 0; i < ap.k; i++) {
         const int32_t x = ap.feed[i + 1];
-        const RowStat sp = stats[i], sq = stats[ap.m + i];
-        const double px = prob_of(tbits[i], x, sp, inv_t);
-        const double qx = prob_of(dbits[i], x, sq, inv_t);
+        const double px = pxs[i], qx = qxs[i];
         const double r = unit_draw(ap.seed, ds);
         ds += 1;
         fold_margin(d.margin, r * qx, px);
@@ -309,6 +305,7 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     __shared__ double red[4];
     __shared__ RowStat stats[MAX_DIST_ROWS];
     __shared__ uint16_t s_tb[TSV_MAX_ROWS], s_db[TSV_MAX_ROWS];
+    __shared__ double s_px[TSV_MAX_ROWS], s_qx[TSV_MAX_ROWS];
     const AcceptParams& ap = *app;
     const int seg = blockIdx.x, jobi = blockIdx.y, sub = blockIdx.z;
     Layout L = layout(scratch);
@@ -327,9 +324,16 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
         }
     }
     __syncthreads();
+    if (kind == 0 && (int)threadIdx.x < ap.k) {
+        const int i = threadIdx.x;
+        const double it = 1.0 / ap.temperature;
+        s_px[i] = prob_of(s_tb[i], ap.feed[i + 1], stats[i], it);
+        s_qx[i] = prob_of(s_db[i], ap.feed[i + 1], stats[ap.m + i], it);
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
         if (kind == 0) {
-            dec = decide_chain_sampled(ap, s_tb, s_db, stats);
+            dec = decide_chain_sampled(ap, s_px, s_qx);
         } else {
             dec.job.mode = 1;
             dec.job.row_p = ap.m + jobi;
