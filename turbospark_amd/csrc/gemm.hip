@@ -37,7 +37,7 @@ namespace tsv {
 // ------------------------------------------------------------------------------- re-tiling
 // One thread per 16-byte unit of a source row's chunk (unit 8 = the scale header).
 __global__ void k_repack_q4k(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
-                             uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, const int32_t* __restrict__ rowmap) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long total = (long)n_rows * kchunks * 9;
     if (gid >= total) return;
@@ -45,7 +45,7 @@ __global__ void k_repack_q4k(const uint8_t* __restrict__ raw, int n_rows, int kc
     const long t = gid / 9;
     const int c = (int)(t % kchunks);
     const int r = (int)(t / kchunks);
-    const int drow = (r / grp) * stride + offset + r % grp;
+    const int drow = rowmap ? rowmap[r] : (r / grp) * stride + offset + r % grp;
     const int tile = drow >> 6, lane = drow & 63;
     const uint8_t* blk = raw + ((long)r * kchunks + c) * 144;
     uint8_t* dst = tiles + ((long)tile * kchunks + c) * 9216 + (u < 8 ? (u * 64 + lane) * 16 : 8192 + lane * 16);
@@ -53,7 +53,7 @@ __global__ void k_repack_q4k(const uint8_t* __restrict__ raw, int n_rows, int kc
 }
 
 __global__ void k_repack_q80(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
-                             uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, const int32_t* __restrict__ rowmap) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long total = (long)n_rows * kchunks * 9;
     if (gid >= total) return;
@@ -61,7 +61,7 @@ __global__ void k_repack_q80(const uint8_t* __restrict__ raw, int n_rows, int kc
     const long t = gid / 9;
     const int c = (int)(t % kchunks);
     const int r = (int)(t / kchunks);
-    const int drow = (r / grp) * stride + offset + r % grp;
+    const int drow = rowmap ? rowmap[r] : (r / grp) * stride + offset + r % grp;
     const int tile = drow >> 6, lane = drow & 63;
     const uint8_t* row = raw + (long)r * kchunks * 4 * 34 + (long)c * 4 * 34;
     uint8_t* tb = tiles + ((long)tile * kchunks + c) * 8704;
@@ -83,7 +83,8 @@ __global__ void k_repack_q80(const uint8_t* __restrict__ raw, int n_rows, int kc
 // MXFP4: one thread per source block (17 bytes: scale, then 16 bytes whose low / high nibbles are
 // elements j and j + 16).  Nibble n of output word w is K element 8w + {0,2,1,3,4,6,5,7}[n].
 __global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
-                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, int nblk) {
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, int nblk,
+                             const int32_t* __restrict__ rowmap) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long total = (long)n_rows * kchunks * 8;
     if (gid >= total) return;
@@ -91,7 +92,7 @@ __global__ void k_repack_mx4(const uint8_t* __restrict__ raw, int n_rows, int kc
     const long t = gid / 8;
     const int c = (int)(t % kchunks);
     const int r = (int)(t / kchunks);
-    const int drow = (r / grp) * stride + offset + r % grp;
+    const int drow = rowmap ? rowmap[r] : (r / grp) * stride + offset + r % grp;
     const int tile = drow >> 6, lane = drow & 63;
     if (c * 8 + u >= nblk) return;  // past the row's last block: the tile keeps its zero block
     const uint8_t* blk = raw + ((long)r * nblk + (long)c * 8 + u) * 17;
@@ -122,7 +123,7 @@ __device__ __forceinline__ uint32_t q6k_level(const uint8_t* blk, int e) {
     return lo | (hi << 4);
 }
 __global__ void k_repack_q6k(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
-                             uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, const int32_t* __restrict__ rowmap) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long total = (long)n_rows * kchunks * 14;
     if (gid >= total) return;
@@ -130,7 +131,7 @@ __global__ void k_repack_q6k(const uint8_t* __restrict__ raw, int n_rows, int kc
     const long t = gid / 14;
     const int c = (int)(t % kchunks);
     const int r = (int)(t / kchunks);
-    const int drow = (r / grp) * stride + offset + r % grp;
+    const int drow = rowmap ? rowmap[r] : (r / grp) * stride + offset + r % grp;
     const int tile = drow >> 6, lane = drow & 63;
     const uint8_t* blk = raw + ((long)r * kchunks + c) * 210;
     uint8_t* tb = tiles + ((long)tile * kchunks + c) * 13568;
@@ -177,7 +178,7 @@ __global__ void k_repack_q6k(const uint8_t* __restrict__ raw, int n_rows, int kc
 
 // bf16: one thread per 16-byte unit (eight consecutive K values of a row, two MFMA steps).
 __global__ void k_repack_bf16(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
-                              uint8_t* __restrict__ tiles, int grp, int stride, int offset) {
+                              uint8_t* __restrict__ tiles, int grp, int stride, int offset, const int32_t* __restrict__ rowmap) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long total = (long)n_rows * kchunks * 8;
     if (gid >= total) return;
@@ -185,7 +186,7 @@ __global__ void k_repack_bf16(const uint8_t* __restrict__ raw, int n_rows, int k
     const long t = gid / 8;
     const int c = (int)(t % kchunks);
     const int r = (int)(t / kchunks);
-    const int drow = (r / grp) * stride + offset + r % grp;
+    const int drow = rowmap ? rowmap[r] : (r / grp) * stride + offset + r % grp;
     const int tile = drow >> 6, lane = drow & 63;
     const uint16_t* src = (const uint16_t*)raw + ((long)r * kchunks + c) * 64 + 8 * u;
     uint16_t v[8];
@@ -197,34 +198,86 @@ __global__ void k_repack_bf16(const uint8_t* __restrict__ raw, int n_rows, int k
 }
 
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
-                  int kchunks, int grp, int stride, int offset) {
+                  int kchunks, int grp, int stride, int offset, const int32_t* rowmap) {
     const long total = (long)n_rows * kchunks * 9;
     if (total == 0) return TSV_OK;
     if (fmt == FMT_Q6K) {
         const long units = (long)n_rows * kchunks * 14;
         hipLaunchKernelGGL(k_repack_q6k, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
-                           tiles, grp, stride, offset);
+                           tiles, grp, stride, offset, rowmap);
     } else if (fmt == FMT_BF16) {
         const long units = (long)n_rows * kchunks * 8;
         hipLaunchKernelGGL(k_repack_bf16, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
-                           tiles, grp, stride, offset);
+                           tiles, grp, stride, offset, rowmap);
     } else if (fmt == FMT_MX4) {
         const long blocks = (long)n_rows * kchunks * 8;
         hipLaunchKernelGGL(k_repack_mx4, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
-                           tiles, grp, stride, offset, k / 32);
+                           tiles, grp, stride, offset, k / 32, rowmap);
     } else if (fmt == FMT_Q4K)
         hipLaunchKernelGGL(k_repack_q4k, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, raw, n_rows,
-                           kchunks, tiles, grp, stride, offset);
+                           kchunks, tiles, grp, stride, offset, rowmap);
     else
         hipLaunchKernelGGL(k_repack_q80, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, raw, n_rows,
-                           kchunks, tiles, grp, stride, offset);
+                           kchunks, tiles, grp, stride, offset, rowmap);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
 
 // Stores one row group's finished sums.  v[i] is output column n of activation row 4g+i.
+// The fused q/k/v projection finishing its own rows (no split-K: the sums are complete here).
+// A tile of the rotated sections holds dims i (lanes 0..31) and i + hd/2 (lanes 32..63) of one
+// head: the NeoX pair of a lane is lane ^ 32 (crates/compute/src/rope.rs:208-256).  Bias first,
+// then the rotation (families/gptoss/attn.rs:88-118); q goes to the fp16 q buffer, K and V
+// straight into the cache slot of the row (families/qwen/batched_layers.rs:84-113).
+__device__ __forceinline__ void rope_epilogue(const GemmArgs& a, int tile, int g, float4v v, int lane, int M) {
+    const RopeEpi& e = a.rope;
+    const VerifyParams* vp = a.vp;
+    const int hd = e.hd, half = hd >> 1, tph = hd >> 6;  // tiles per head
+    const int tq = e.nq * tph, tk = e.nkv * tph;
+    const int kind = tile < tq ? 0 : tile < tq + tk ? 1 : 2;
+    const int st = kind == 0 ? tile : kind == 1 ? tile - tq : tile - tq - tk;
+    const int head = st / tph, t = st - head * tph;
+    const bool hi = lane >= 32;
+    const int idim = (tph == 2 ? 32 * t : 0) + (lane & 31);     // rotation pair index, 0 .. hd/2
+    const int d = kind == 2 ? t * 64 + lane : (hi ? idim + half : idim);  // this lane's head dimension
+    const int col = (kind == 0 ? 0 : kind == 1 ? e.nq * hd : (e.nq + e.nkv) * hd) + head * hd + d;
+    const float bias = e.bias ? e.bias[col] : 0.f;
+    const int base = vp->base;
+    float2 cs[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) cs[i] = kind != 2 && 4 * g + i < M ? e.cs[(4 * g + i) * half + idim] : float2{1.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int b = 4 * g + i;
+        float x = v[i] + bias;
+        const float other = __shfl_xor(x, 32);
+        if (b >= M) continue;
+        if (kind != 2) {
+            const float x0 = hi ? other : x, x1 = hi ? x : other;
+            x = hi ? x0 * cs[i].y + x1 * cs[i].x : x0 * cs[i].x - x1 * cs[i].y;
+        }
+        const _Float16 h = (_Float16)x;
+        if (kind == 0) {
+            ((_Float16*)e.q16)[((long)b * e.nq + head) * hd + d] = h;
+        } else {
+            const int pos = base + b;  // the cache slot of row b
+            if (kind == 1) {
+                ((_Float16*)e.kc)[((long)head * e.max_ctx + pos) * hd + d] = h;
+            } else {
+                _Float16* vb = (_Float16*)e.vc + ((long)head * (e.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
+                const int po = pos & 15;
+                vb[(((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3)] = h;
+            }
+        }
+    }
+}
+
 template <int EPI>
 __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split, int g, float4v v, int lane, int M) {
+    if (EPI == EPI_ROPE) {
+        rope_epilogue(a, tile, g, v, lane, M);
+        return;
+    }
     if (EPI == EPI_SILU) {
         // Lanes 0..31 hold the gate rows and lanes 32..63 the up rows of the same 32 columns;
         // silu(gate) * up becomes the next matmul's fp16 activation, stored in fragment order
@@ -369,13 +422,14 @@ template <class F>
 static int launch_f(hipStream_t s, const GemmArgs& a, int m, int epi) {
     switch (epi) {
         case EPI_PARTIAL: return launch_e<F, EPI_PARTIAL>(s, a, m);
+        case EPI_ROPE: return launch_e<F, EPI_ROPE>(s, a, m);
         case EPI_SILU: return launch_e<F, EPI_SILU>(s, a, m);
         default: return launch_e<F, EPI_LOGITS>(s, a, m);
     }
 }
 
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
-                int m, int splits, int epi, int ldo, int n_valid) {
+                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
     if (m < 1 || m > TSV_MAX_ROWS) {
         set_error("matmul: row count outside 1..16");
         return TSV_ERR_INVALID;
@@ -403,6 +457,13 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
     a.kparts = (a.kslice + a.per - 1) / a.per;
     a.ldo = ldo;
     a.n_valid = n_valid;
+    if (epi == EPI_ROPE) {
+        if (!rope || (rope->hd != 64 && rope->hd != 128) || w.n_rows != (rope->nq + 2 * rope->nkv) * rope->hd) {
+            set_error("matmul: the rotating epilogue needs the fused q/k/v projection of a 64- or 128-wide head");
+            return TSV_ERR_INVALID;
+        }
+        a.rope = *rope;
+    }
     if (epi == EPI_SILU) {
         if (w.n_rows % 64) {
             set_error("matmul: gate/up rows must fill whole 64-row tiles");

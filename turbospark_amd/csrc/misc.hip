@@ -13,12 +13,24 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
 // ---------------------------------------------------------------- embedding lookup
 // One dequantized table row per fed token (crates/runtime/src/real_forward_dispatch.rs:154),
 // arithmetic of dequantize_q4_k / dequantize_q8_0.
+// The last workgroup of a row (when `cs` is given) fills the row's rotation table instead:
+// (cos, sin) of pos * freq, scaled, for every pair index - the same for all layers of the step.
 __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, float* __restrict__ x,
-                        const VerifyParams* __restrict__ vp) {
+                        const VerifyParams* __restrict__ vp, const float* __restrict__ freqs, float mscale,
+                        int half, float2* __restrict__ cs, int nblk) {
     const int m = blockIdx.x;
     if (m >= vp->m) return;
+    if ((int)blockIdx.y == nblk) {
+        const float pos = (float)vp->pos[m];
+        for (int i = threadIdx.x; i < half; i += blockDim.x) {
+            float sn, c;
+            sincosf(pos * freqs[i], &sn, &c);
+            cs[m * half + i] = float2{c * mscale, sn * mscale};
+        }
+        return;
+    }
     const long tok = vp->feed[m];
-    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < hidden; e += blockDim.x * gridDim.y) {
+    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < hidden; e += blockDim.x * nblk) {
         float v;
         if (dtype == TSV_Q4_K) {
             const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 144;
@@ -61,8 +73,10 @@ __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, 
 }
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
-                 const VerifyParams* vp, int m) {
-    hipLaunchKernelGGL(k_embed, dim3(m, (hidden + 511) / 512), dim3(256), 0, s, raw, dtype, hidden, x, vp);  // two elements per thread
+                 const VerifyParams* vp, int m, const float* freqs, float mscale, int half, float2* cs) {
+    const int nblk = (hidden + 511) / 512;  // two elements per thread
+    hipLaunchKernelGGL(k_embed, dim3(m, nblk + (cs ? 1 : 0)), dim3(256), 0, s, raw, dtype, hidden, x, vp, freqs, mscale,
+                       half, cs, nblk);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -28,6 +28,7 @@ struct LayerW {
     float *bqkv = nullptr, *bo = nullptr, *sinks = nullptr, *router_bias = nullptr;
     float *be_gate = nullptr, *be_up = nullptr, *be_down = nullptr;
     int window = 0;
+    bool rope_fused = false;  // the q/k/v projection rotates and stores its own rows
     uint16_t *kc = nullptr, *vc = nullptr;
 };
 
@@ -46,12 +47,14 @@ struct tsv_ctx {
     int n_layers = 0, hidden = 0, nq = 0, nkv = 0, hd = 0, ffn = 0, vocab = 0, max_context = 0, ctx_alloc = 0;
     float eps = 0, attn_scale = 0, rope_mscale = 1.0f, act_alpha = 0, act_limit = 0;
     hipStream_t stream = nullptr;
+    bool rope_fused_ok = true;  // TSV_ROPE_FUSED=0 keeps the projection and the rotation apart
     std::vector<LayerW> layers;
     TiledW head;
     uint8_t* embed_raw = nullptr;
     int embed_dtype = 0;
     float* final_norm = nullptr;
     float* freqs = nullptr;
+    float2* rope_cs = nullptr;  // [16][hd / 2] rotation table of the step's rows (fused q/k/v projection)
     // scratch
     float* x = nullptr;
     uint4 *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
@@ -188,7 +191,11 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
 // Allocates a tiled matrix of `total_rows` rows and re-tiles `parts` into it: concatenated row
 // by row (interleave == false) or alternating in runs of 32 rows (gate / up: each 64-row tile
 // holds 32 gate rows in its low lanes and the matching 32 up rows in its high lanes).
-int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_parts, bool interleave, TiledW* out) {
+// pair_parts > 0 (128-wide heads feeding the rotating epilogue): inside every head of the first
+// `pair_parts` parts the rows are reordered so that a 64-row tile holds dims 32t..32t+31 in its low
+// lanes and their rotation partners, dims 64+32t.., in its high lanes.
+int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_parts, bool interleave, TiledW* out,
+               int pair_parts = 0) {
     const int fmt = dtype_fmt(parts[0]->dtype);
     int64_t total_rows = 0;
     for (int i = 0; i < n_parts; i++) {
@@ -214,6 +221,29 @@ int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_par
     for (int i = 0; i < n_parts; i++) {
         if ((rc = stage_raw(c, st, *parts[i]))) return rc;
         const int rows = (int)parts[i]->rows;
+        if (i < pair_parts) {
+            if (interleave || rows % 128) {
+                set_error("paired row order needs whole 128-wide heads");
+                return TSV_ERR_INVALID;
+            }
+            std::vector<int32_t> map((size_t)rows);
+            for (int r = 0; r < rows; r++) {
+                const int hl = r & 127, half = hl >> 6, w = hl & 63, t = w >> 5, j = w & 31;
+                map[(size_t)r] = row_off + (r & ~127) + t * 64 + half * 32 + j;
+            }
+            int32_t* map_dev = nullptr;
+            TSV_HIP(hipMalloc((void**)&map_dev, map.size() * 4));
+            hipError_t e = hipMemcpyAsync(map_dev, map.data(), map.size() * 4, hipMemcpyHostToDevice, c->stream);
+            if (e == hipSuccess) {
+                rc = launch_repack(c->stream, fmt, st.dev, rows, out->k, out->tiles, out->kchunks, rows, 0, row_off, map_dev);
+                e = hipStreamSynchronize(c->stream);
+            }
+            (void)hipFree(map_dev);
+            TSV_HIP(e);
+            if (rc) return rc;
+            row_off += rows;
+            continue;
+        }
         rc = interleave ? launch_repack(c->stream, fmt, st.dev, rows, out->k, out->tiles, out->kchunks, 32, 32 * n_parts, 32 * i)
                         : launch_repack(c->stream, fmt, st.dev, rows, out->k, out->tiles, out->kchunks, rows, 0, row_off);
         if (rc) return rc;
@@ -361,7 +391,8 @@ int launch_pass(tsv_ctx* c, int m) {
     { PROF(PC_EVENTPAIR); }  // calibration: an event pair around nothing
     {
         PROF(PC_EMBED);
-        rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m);
+        rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m, c->freqs, c->rope_mscale,
+                          c->hd / 2, c->rope_cs);
     }
     if (rc) return rc;
     int prev_splits = 0;
@@ -386,7 +417,22 @@ int launch_pass(tsv_ctx* c, int m) {
             };
             while (sp > 1 && !(fits(L.qkv, sp) && fits(L.v_only, sp))) sp--;
         }
-        {
+        if (L.rope_fused) {
+            RopeEpi re{};
+            re.cs = c->rope_cs;
+            re.bias = L.bqkv;
+            re.q16 = c->q16;
+            re.kc = L.kc;
+            re.vc = L.vc;
+            re.nq = c->nq;
+            re.nkv = c->nkv;
+            re.hd = c->hd;
+            re.max_ctx = c->ctx_alloc;
+            PROF(PC_QKV);
+            rc = 0;
+            for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++)
+                rc = launch_gemm(s, L.qkv, c->xf_a, nullptr, c->vp_dev, m, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re);
+        } else {
             PROF(PC_QKV);
             rc = 0;
             for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++) {
@@ -415,7 +461,7 @@ int launch_pass(tsv_ctx* c, int m) {
         ra.hd = c->hd;
         ra.max_ctx = c->ctx_alloc;
         ra.vp = c->vp_dev;
-        {
+        if (!L.rope_fused) {
             PROF(PC_ROPE);
             rc = 0;
             for (int rep = 0; rep < c->repeat[PC_ROPE] && !rc; rep++) rc = launch_rope_kv(s, ra, m);
@@ -671,6 +717,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->act_alpha = d->act_alpha;
     c->act_limit = d->act_limit;
     if (const char* e = getenv("TSV_GRAPH")) c->use_graph = e[0] == '1';
+    if (const char* e = getenv("TSV_ROPE_FUSED")) c->rope_fused_ok = e[0] != '0';
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("open: cannot create a HIP stream (no GPU?)");
         delete c;
@@ -693,8 +740,12 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             set_error("open: the q and k projections must share a storage type");
             return fail(TSV_ERR_UNSUPPORTED);
         }
+        // One launch that projects, rotates and stores (no split-K partials, no separate rotation
+        // kernel) where the head needs no per-head norm in between and q/k/v share a storage type.
+        L.rope_fused = c->rope_fused_ok && s.wv.dtype == s.wq.dtype && !s.q_norm.data && !s.k_norm.data &&
+                       (c->hd == 64 || c->hd == 128);
         if (s.wv.dtype == s.wq.dtype) {
-            if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv))) return fail(rc);
+            if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv, L.rope_fused && c->hd == 128 ? 2 : 0))) return fail(rc);
         } else {
             const tsv_tensor* vonly[1] = {&s.wv};
             if ((rc = make_tiled(c, st, qkv, 2, false, &L.qkv)) || (rc = make_tiled(c, st, vonly, 1, false, &L.v_only)))
@@ -820,6 +871,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         }
         if ((rc = dev_alloc(c, &c->freqs, f.size() * 4))) return fail(rc);
         if (hipMemcpy(c->freqs, f.data(), f.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail(TSV_ERR_DEVICE);
+        if ((rc = dev_alloc(c, &c->rope_cs, (size_t)TSV_MAX_ROWS * f.size() * sizeof(float2), true))) return fail(rc);
     }
     // scratch
     const int kmax = std::max(std::max(c->hidden, qd), c->ffn);

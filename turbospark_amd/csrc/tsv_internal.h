@@ -95,7 +95,19 @@ struct VerifyParams {
     uint32_t anc[TSV_MAX_ROWS];  // bit s set: row i attends cache slot base+s
 };
 
-enum { EPI_PARTIAL = 0, EPI_SILU = 1, EPI_LOGITS = 2, EPI_SLOT = 3 };
+enum { EPI_PARTIAL = 0, EPI_SILU = 1, EPI_LOGITS = 2, EPI_SLOT = 3, EPI_ROPE = 4 };
+
+// What the fused q/k/v projection needs to finish its rows itself (EPI_ROPE): bias, NeoX rotation
+// and the stores into the q buffer and the K / V cache slots.  The projection's rows are re-tiled
+// so that the two halves of a rotation pair sit in lanes l and l + 32 of one tile.
+struct RopeEpi {
+    const float2* cs;    // [16][head_dim / 2] (cos, sin) of the rows' rotation angles, scaled
+    const float* bias;   // nullable, fused q, k, v row order
+    uint16_t* q16;       // [16][nq][hd] fp16
+    uint16_t* kc;        // [nkv][max_ctx][hd]
+    uint16_t* vc;        // [nkv][max_ctx/16][hd/16][64][4]
+    int nq, nkv, hd, max_ctx;
+};
 
 struct GemmArgs {
     const uint8_t* w;
@@ -105,14 +117,16 @@ struct GemmArgs {
                          // next matmul; EPI_LOGITS: half [m][ldo]
     const VerifyParams* vp;
     int n_tiles, kchunks, kslice, splits, kparts, per, ldo, n_valid;
+    RopeEpi rope;  // EPI_ROPE only
 };
 
 // Re-tiles n_rows GGUF rows of `raw` into `tiles`; source row r lands in tiled row
 // (r / grp) * stride + offset + r % grp.
+// (rowmap, when given, names the tiled row of every source row instead)
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
-                  int kchunks, int grp, int stride, int offset);
+                  int kchunks, int grp, int stride, int offset, const int32_t* rowmap = nullptr);
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
-                int m, int splits, int epi, int ldo, int n_valid);
+                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
 int gemm_default_splits(const TiledW& w, int m);
 
 // ---- routed experts (moe.hip) -----------------------------------------------------------------
@@ -191,7 +205,8 @@ int fused_ffn_barriers();
 int launch_ffn_block(hipStream_t s, int fmt, FfnBlockArgs& a, int m);
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
-                 const VerifyParams* vp, int m);
+                 const VerifyParams* vp, int m, const float* freqs = nullptr, float mscale = 1.0f, int half = 0,
+                 float2* cs = nullptr);
 // weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
                    float eps, int hidden, uint4* xfrag, int m, const float* weights = nullptr,
