@@ -131,6 +131,12 @@ typedef struct {
     uint64_t generated;      /* tokens reported so far (TokenSink::generated) */
     uint64_t max_new_tokens; /* budget; 0 = unbounded */
     uint16_t* logits_out;    /* optional: m x vocab fp16 copy of the verify logits */
+    /* TokenSink::history when the round starts (prompt + every reported token, feed[0] last), host
+     * memory; read only when a repetition / presence / frequency penalty is set at temperature > 0
+     * (crates/selection/src/penalty.rs:15-82).  Its last min(generated, n_history) tokens are the
+     * generated suffix the presence / frequency penalties count over (choose.rs:138-154). */
+    const int32_t* history;
+    int64_t n_history;
 } tsv_round;
 
 typedef struct {
@@ -200,7 +206,8 @@ int32_t tsv_verify_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result
  * from each row of draft_logits (k x vocab fp16, host or device), advancing *draw_step by
  * k + 1; greedy: argmax per row. */
 int32_t tsv_draft_chain(tsv_ctx* ctx, const uint16_t* draft_logits, int32_t k,
-                        const tsv_shaping* shaping, uint64_t* draw_step, int32_t* proposals);
+                        const tsv_shaping* shaping, uint64_t* draw_step, int32_t* proposals,
+                        const int32_t* history, int64_t n_history, uint64_t generated);
 
 /* ---- the generation loop (speculative.rs:194-900) and the adaptive depth ---------------- */
 /* Per-round draft depth controller, speculative_adaptive.rs:105-227: pure state.  A streak of

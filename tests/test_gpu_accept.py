@@ -89,6 +89,109 @@ def test_sampled_chain_rounds_match_the_oracle_bit_for_bit(temperature, kw):
         assert len(set(accepted_hist)) > 1  # the rounds really exercised different outcomes
 
 
+PENALTIES = [dict(repetition_penalty=1.3), dict(presence_penalty=0.6, frequency_penalty=0.25),
+             dict(repetition_penalty=1.2, presence_penalty=0.4, frequency_penalty=0.1, top_k=50, top_p=0.95, min_p=0.01),
+             dict(repetition_penalty=0.7, top_p=0.9), dict(repetition_penalty=1.15, top_k=40),
+             dict(repetition_penalty=1.1, min_p=0.02), dict(presence_penalty=2.0, top_p=0.6),
+             dict(frequency_penalty=0.5, top_k=8)]
+
+
+@pytest.mark.parametrize("dense", [False, True])
+@pytest.mark.parametrize("kw", PENALTIES)
+def test_penalised_chain_rounds_match_the_oracle_bit_for_bit(kw, dense):
+    """Repetition / presence / frequency penalties (crates/selection/src/penalty.rs:15-82) in the draft
+    draws and in the acceptance of a sampled chain round: each target row is shaped with the history
+    a sequential decode would have had there (the proposals accepted before it included).  `dense`
+    hands over a long synthetic history that touches a third of the vocabulary, so penalised scores
+    sit between fp16 values in most rank bins, the truncation cuts' and the draws' bins included."""
+    import turbospark_amd as ts
+    cfg, gpu, prompt = _setup()
+    V, k = cfg["vocab"], 4
+    rng = np.random.default_rng(23)
+    gpu.rollback(ts.ffi.Point(len(prompt) - 1))
+    nxt = int(prompt[-1])
+    if dense:
+        history = [int(t) for t in rng.integers(-3, V + 3, 2500)]  # ids outside the vocabulary are skipped
+        n_prompt = 700
+    else:
+        history = [int(t) for t in prompt[:-1]]
+        n_prompt = len(history)
+    draw_step = 0
+    margins, accepted_hist = [], []
+    for rnd in range(16):
+        seed = 500 + rnd
+        gcfg = ts.shaping(0.8 if rnd % 2 else 1.0, seed=seed, **kw)
+        ocfg = ob.shaping(0.8 if rnd % 2 else 1.0, seed=seed, **kw)
+        hist_now = history + [nxt]
+        generated = len(hist_now) - n_prompt
+        draft = rng.standard_normal((k, V)).astype(np.float16)
+        if rnd % 4 == 1:
+            draft[1] = np.round(draft[1] * 2) / 2
+        if rnd % 2 == 1:  # a drafter that resembles the target, so that proposals get accepted
+            here = gpu.checkpoint()
+            tok = nxt
+            for i in range(k):
+                row = gc.f16(gpu.produce(tok, gpu.position))
+                draft[i] = (row + rng.standard_normal(V) * 0.3).astype(np.float16)
+                one, _ = gpu.draft_chain(draft[i:i + 1], gcfg, draw_step + i, history=hist_now, generated=generated)
+                tok = int(one[0])
+            gpu.rollback(here)
+        if rnd % 5 == 2:  # the proposals repeat themselves: later rows count the earlier ones
+            draft[1:] = draft[0]
+        props, ds1 = gpu.draft_chain(draft, gcfg, draw_step, history=hist_now, generated=generated)
+        oprops, ods1 = ob.draft_chain(draft, ocfg, hist_now, generated, draw_step)
+        assert list(props) == list(oprops) and ds1 == ods1
+        feed = [nxt] + [int(t) for t in props]
+        base = gpu.position
+        res, logits = gpu.verify_accept(feed, base, gcfg, draft_logits=draft, draw_step=ds1, want_logits=True,
+                                        history=hist_now, generated=generated)
+        want = ob.chain_round(logits, draft, props, ocfg, history=hist_now, generated=generated, draw_step=ds1)
+        _same(res, want, base)
+        margins.append(res.min_margin)
+        accepted_hist.append(res.accepted)
+        history = hist_now + feed[1: 1 + want["committed"]]
+        nxt = want["next"]
+        draw_step = want["draw_step"]
+    print("accepted per round:", accepted_hist, " min margin:", min(margins))
+    assert min(margins) > 1e-9
+    assert len(set(accepted_hist)) > 1
+
+
+def test_penalties_change_the_outcome_and_greedy_ignores_them():
+    """The penalised rounds are not the plain ones in disguise: with the proposal in the history a
+    strong penalty flips decisions the plain round makes; at temperature 0 the arg-max ignores
+    penalties (choose.rs:84-88)."""
+    import turbospark_amd as ts
+    cfg, gpu, prompt = _setup()
+    V = cfg["vocab"]
+    rng = np.random.default_rng(3)
+    base = gpu.position
+    point = gpu.checkpoint()
+    differs = 0
+    for seed in range(12):
+        draft = rng.standard_normal((3, V)).astype(np.float16)
+        plain = ts.shaping(0.9, seed=seed)
+        props, ds = gpu.draft_chain(draft, plain, 0)
+        feed = [5] + [int(t) for t in props]
+        hist = list(prompt) + feed  # every proposal is already in the history
+        a = gpu.verify_accept(feed, base, plain, draft_logits=draft, draw_step=ds)
+        gpu.rollback(point)
+        pen = ts.shaping(0.9, seed=seed, repetition_penalty=3.0, presence_penalty=4.0)
+        b, logits = gpu.verify_accept(feed, base, pen, draft_logits=draft, draw_step=ds, history=hist, generated=3,
+                                      want_logits=True)
+        gpu.rollback(point)
+        want = ob.chain_round(logits, draft, props, ob.shaping(0.9, seed=seed, repetition_penalty=3.0, presence_penalty=4.0),
+                              history=hist, generated=3, draw_step=ds)
+        _same(b, want, base)
+        differs += (a.accepted, a.next) != (b.accepted, b.next)
+    assert differs > 0
+    g = gpu.verify_accept([5, 6, 7], base, ts.shaping(0.0, repetition_penalty=2.0, presence_penalty=1.0),
+                          history=list(prompt), generated=2)
+    gpu.rollback(point)
+    h = gpu.verify_accept([5, 6, 7], base, ts.shaping(0.0))
+    assert (g.accepted, g.next) == (h.accepted, h.next)
+
+
 def test_identical_drafter_is_always_accepted_and_the_bonus_is_a_p_draw():
     import turbospark_amd as ts
     cfg, gpu, prompt = _setup()
@@ -237,9 +340,10 @@ def test_refusals_by_name():
     from turbospark_amd import TsvError
     cfg, gpu, prompt = _setup()
     base = gpu.position
-    with pytest.raises(TsvError, match="not built"):
-        gpu.verify_accept([1, 2], base, ts.shaping(0.8, repetition_penalty=1.1, seed=1),
-                          draft_logits=np.zeros((1, cfg["vocab"]), np.float16))
+    with pytest.raises(TsvError, match="not built"):  # penalties over a sampled tree
+        gpu.verify_accept([1, 2, 3], base, ts.shaping(0.8, repetition_penalty=1.1, seed=1), parent=[-1, 0, 0],
+                          draft_logits=np.zeros((3, cfg["vocab"]), np.float16), history=[1, 2])
+    assert gpu.position == base
     with pytest.raises(TsvError, match="seed"):
         gpu.verify_accept([1, 2], base, ts.shaping(0.8), draft_logits=np.zeros((1, cfg["vocab"]), np.float16))
     with pytest.raises(TsvError, match="drafter"):

@@ -30,6 +30,8 @@ def _pair(name="tiny_q8_0", max_context=200, draft_seed=1234):
     (0.8, {}, 4, 0, 1.0, 1234),        # rejection sampling
     (1.0, dict(top_p=0.95, top_k=50), 8, 2, 0.5, 1234),
     (0.7, dict(min_p=0.02), 15, 0, 0.0, 1234),   # the widest block, a perfect drafter
+    (0.9, dict(repetition_penalty=1.3, presence_penalty=0.5, frequency_penalty=0.2), 4, 0, 0.5, 1234),  # penalties see the growing history
+    (0.8, dict(repetition_penalty=1.1, top_p=0.9, top_k=64), 6, 2, 0.3, 1234),
 ])
 def test_the_device_loop_reports_what_the_reference_loop_reports(temperature, kw, block, floor, noise, draft_seed):
     import turbospark_amd as ts

@@ -16,6 +16,10 @@
 // distance from flipping is folded into `min_margin` so a caller can see that it never was.
 // Bin masses are accumulated as 2^-62 fixed point with integer atomics: order independent,
 // hence bit-reproducible run to run.
+//
+// Repetition / presence / frequency penalties (sampled chain rounds and the draft draws) are
+// applied per candidate as it is read, from a per-token table of the history (see score_of);
+// the kernels are compiled twice, and the variant without penalties is the code it always was.
 #include "tsv_internal.h"
 
 namespace tsv {
@@ -30,14 +34,17 @@ constexpr double FIX = 4611686018427387904.0;  // 2^62
 
 struct RowStat {
     double mx, sum, total, top;
+    double minp;               // penalised rounds: candidates with e < minp are out (0: off)
     int32_t cut_key, cut_idx;  // last surviving candidate in rank order (truncation off: 65536, INT_MAX)
+    float cut_w;               // its score (penalised rounds: a rank bin can hold several values)
 };
 struct Cut {
     int32_t key, idx;
+    float w, pad;
 };
 
 // Scratch layout inside AcceptScratch::stats (doubles):
-//   [0, 4*32)                         truncation cut per distribution row (8 bytes each)
+//   [0, 4*32)                         truncation cut per distribution row (16 bytes each)
 //   pmax / psum / ptot partials follow, then the residual pieces and the decisions
 struct Layout {
     double* pmax;  // [rows][NSEG]
@@ -114,6 +121,83 @@ __device__ __forceinline__ double prob_of(uint16_t bits, int v, const RowStat& s
     return pow(p / s.top, inv_t) / s.total;
 }
 
+// ---- penalised scores -------------------------------------------------------------------------
+// crates/selection/src/penalty.rs:15-82 through choose.rs:138-154: the repetition penalty divides
+// (positive) or multiplies (other) the f32 score of every distinct token of the history once; the
+// presence / frequency penalties subtract presence + frequency * count for every token of the
+// generated suffix.  `pen_cnt[v]` holds, for the history the round started with, bit 31 = seen and
+// the low bits = occurrences in the generated suffix; target row i of a chain round adds the i
+// proposals committed before it was judged (speculative.rs:694-716: each accepted proposal goes
+// through the sink before the next row is shaped), drafter rows add nothing (speculative.rs:636-641).
+//
+// A penalised score is an f32 that need not be an fp16 value.  Its rank bin is the bin of the
+// largest fp16 value not above it, so bins stay ordered; inside a bin the candidates with a score
+// above the bin's own value come first (score descending, index ascending: the few "side"
+// candidates), then the candidates exactly on the value in index order.
+template <bool PEN>
+__device__ __forceinline__ float score_of(const AcceptParams& ap, int row, int v, uint16_t bits) {
+    float w = h2f(bits);
+    if constexpr (PEN) {
+        const uint32_t c = ap.pen_cnt[v];
+        bool seen = (c >> 31) != 0;
+        uint32_t gen = c & 0x7FFFFFFFu;
+        const int extra = row < ap.m ? row : 0;
+        for (int j = 0; j < extra; j++)
+            if (ap.feed[j + 1] == v) {
+                seen = true;
+                gen += 1;
+            }
+        if (ap.pen_has_rep && seen) {
+            const float a = w > 0.0f ? __fdiv_rn(w, ap.pen_rep) : __fmul_rn(w, ap.pen_rep);
+            w = fminf(fmaxf(a, -3.40282347e+38f), 3.40282347e+38f);
+        }
+        if (ap.pen_has_pf && gen != 0)
+            w = __fsub_rn(w, (float)__dadd_rn(ap.pen_presence, __dmul_rn(ap.pen_frequency, (double)gen)));
+    }
+    return w;
+}
+
+// The largest fp16 value not above w (w clamped into the fp16 range first).
+__device__ __forceinline__ uint16_t floor16(float w) {
+    const float c = fminf(fmaxf(w, -65504.0f), 65504.0f);
+    const _Float16 h = (_Float16)c;
+    uint16_t b = __builtin_bit_cast(uint16_t, h);
+    if ((float)h > c) {
+        if ((b & 0x7FFFu) == 0)
+            b = 0x8001u;  // below zero: the smallest negative value
+        else if (b & 0x8000u)
+            b += 1;
+        else
+            b -= 1;
+    }
+    return b;
+}
+
+template <bool PEN>
+__device__ __forceinline__ uint32_t key_of(float w, uint16_t bits) {
+    if constexpr (PEN) return rank_key(floor16(w));
+    return rank_key(bits);
+}
+
+template <bool PEN>
+__device__ __forceinline__ bool survives_w(float w, int key, int v, const RowStat& s) {
+    if constexpr (PEN)
+        return key < s.cut_key || (key == s.cut_key && (w > s.cut_w || (w == s.cut_w && v <= s.cut_idx)));
+    return key < s.cut_key || (key == s.cut_key && v <= s.cut_idx);
+}
+
+// choose.rs:296-319 for a candidate given by its score
+template <bool PEN>
+__device__ __forceinline__ double prob_of_w(float w, int key, int v, const RowStat& s, double inv_t) {
+    if (!survives_w<PEN>(w, key, v, s)) return 0.0;
+    const double e = exp((double)w - s.mx);
+    if constexpr (PEN) {
+        if (e < s.minp) return 0.0;
+    }
+    const double p = e / s.sum;
+    return pow(p / s.top, inv_t) / s.total;
+}
+
 template <typename T>
 __device__ __forceinline__ T shfl_xor_t(T v, int o) {
     static_assert(sizeof(T) == 8, "64-bit only");
@@ -153,9 +237,11 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 static_assert(NSEG == 64, "one lane per segment");
 
 // ---- statistics, three short passes over every distribution row -------------------------
+template <bool PEN>
 __global__ __launch_bounds__(256) void k_row_max(const uint16_t* target, const uint16_t* draft, int m,
                                                  int vocab, double* scratch, int32_t* err,
-                                                 unsigned long long* hist, int hist_words) {
+                                                 unsigned long long* hist, int hist_words,
+                                                 const AcceptParams* app) {
     __shared__ double red[4];
     const int row = blockIdx.y, seg = blockIdx.x;
     {
@@ -168,12 +254,20 @@ __global__ __launch_bounds__(256) void k_row_max(const uint16_t* target, const u
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
     float mx = -INFINITY;
     bool bad = false;
+    bool low = false;
     for (int v = v0 + threadIdx.x; v < v1; v += 256) {
         const uint16_t b = p[v];
         bad |= (b & 0x7C00u) == 0x7C00u;
-        mx = fmaxf(mx, h2f(b));
+        if constexpr (PEN) {
+            const float w = score_of<true>(*app, row, v, b);
+            low |= !(w >= -65504.0f);
+            mx = fmaxf(mx, w);
+        } else {
+            mx = fmaxf(mx, h2f(b));
+        }
     }
     if (bad) atomicOr(err, 1);
+    if (low) atomicOr(err, 4);  // a penalised score below every fp16 value: no rank bin to put it in
     double d = (double)mx;
     for (int o = 32; o > 0; o >>= 1) d = fmax(d, shfl_xor_t(d, o));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = d;
@@ -181,12 +275,13 @@ __global__ __launch_bounds__(256) void k_row_max(const uint16_t* target, const u
     if (threadIdx.x == 0) {
         Layout L = layout(scratch);
         L.pmax[row * NSEG + seg] = fmax(fmax(red[0], red[1]), fmax(red[2], red[3]));
-        if (seg == 0) L.cut[row] = Cut{65536, 0x7FFFFFFF};  // no truncation until a cut is computed
+        if (seg == 0) L.cut[row] = Cut{65536, 0x7FFFFFFF, 0.f, 0.f};  // no truncation until a cut is computed
     }
 }
 
+template <bool PEN>
 __global__ __launch_bounds__(256) void k_row_sum(const uint16_t* target, const uint16_t* draft, int m,
-                                                 int vocab, double* scratch) {
+                                                 int vocab, double* scratch, const AcceptParams* app) {
     __shared__ double red[4];
     const int row = blockIdx.y, seg = blockIdx.x;
     Layout L = layout(scratch);
@@ -194,13 +289,22 @@ __global__ __launch_bounds__(256) void k_row_sum(const uint16_t* target, const u
     const uint16_t* p = row_ptr(target, draft, m, vocab, row);
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
     double acc = 0.0;
-    for (int v = v0 + threadIdx.x; v < v1; v += 256) acc += exp((double)h2f(p[v]) - mx);
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        float w;
+        if constexpr (PEN)
+            w = score_of<true>(*app, row, v, p[v]);
+        else
+            w = h2f(p[v]);
+        acc += exp((double)w - mx);
+    }
     acc = block_sum_f64(acc, red);
     if (threadIdx.x == 0) L.psum[row * NSEG + seg] = acc;
 }
 
+template <bool PEN>
 __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const uint16_t* draft, int m,
-                                                   int vocab, double* scratch, double inv_t) {
+                                                   int vocab, double* scratch, double inv_t,
+                                                   const AcceptParams* app) {
     __shared__ double red[4];
     const int row = blockIdx.y, seg = blockIdx.x;
     Layout L = layout(scratch);
@@ -212,12 +316,21 @@ __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const
     RowStat cs;
     cs.cut_key = L.cut[row].key;
     cs.cut_idx = L.cut[row].idx;
+    cs.cut_w = L.cut[row].w;
     double acc = 0.0;
     for (int v = v0 + threadIdx.x; v < v1; v += 256) {
         const uint16_t b = p[v];
-        if (!survives(b, v, cs)) continue;
-        const double e = exp((double)h2f(b) - mx);
-        acc += pow((e / sum) / top, inv_t);
+        if constexpr (PEN) {
+            const float w = score_of<true>(*app, row, v, b);
+            if (!survives_w<true>(w, (int)key_of<true>(w, b), v, cs)) continue;
+            const double e = exp((double)w - mx);
+            if (app->has_min_p && e < app->min_p) continue;
+            acc += pow((e / sum) / top, inv_t);
+        } else {
+            if (!survives(b, v, cs)) continue;
+            const double e = exp((double)h2f(b) - mx);
+            acc += pow((e / sum) / top, inv_t);
+        }
     }
     acc = block_sum_f64(acc, red);
     if (threadIdx.x == 0) L.ptot[row * NSEG + seg] = acc;
@@ -233,6 +346,8 @@ __device__ RowStat load_stat(const Layout& L, int row) {
     s.total = wave_sum_f64(L.ptot[row * NSEG + lane]);
     s.cut_key = L.cut[row].key;
     s.cut_idx = L.cut[row].idx;
+    s.cut_w = L.cut[row].w;
+    s.minp = 0.0;
     return s;
 }
 
@@ -298,6 +413,7 @@ __device__ Decision decide_chain_sampled(const AcceptParams& ap, const double* p
 // ---- masses + rank histogram --------------------------------------------------------------
 // kind 0: the job comes out of the chain decision (every workgroup re-derives it: a few
 // dozen f64 ops).  kind 1: jobs are "draw from drafter row j at position draw_step + j".
+template <bool PEN>
 __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const uint16_t* draft,
                                                    const AcceptParams* app, double* scratch, double* work,
                                                    unsigned long long* hist, Decision* dec_out, int kind) {
@@ -319,7 +435,8 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
         // every row's statistics, one wave per row at a time
         const int rows = kind == 0 ? ap.m + ap.k : ap.k;
         for (int r = threadIdx.x >> 6; r < rows; r += 4) {
-            const RowStat st = load_stat(L, r);
+            RowStat st = load_stat(L, r);
+            if (PEN && ap.has_min_p) st.minp = ap.min_p;
             if ((threadIdx.x & 63) == 0) stats[r] = st;
         }
     }
@@ -327,8 +444,10 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     if (kind == 0 && (int)threadIdx.x < ap.k) {
         const int i = threadIdx.x;
         const double it = 1.0 / ap.temperature;
-        s_px[i] = prob_of(s_tb[i], ap.feed[i + 1], stats[i], it);
-        s_qx[i] = prob_of(s_db[i], ap.feed[i + 1], stats[ap.m + i], it);
+        const int32_t x = ap.feed[i + 1];
+        const float wt = score_of<PEN>(ap, i, x, s_tb[i]), wd = score_of<PEN>(ap, ap.m + i, x, s_db[i]);
+        s_px[i] = prob_of_w<PEN>(wt, (int)key_of<PEN>(wt, s_tb[i]), x, stats[i], it);
+        s_qx[i] = prob_of_w<PEN>(wd, (int)key_of<PEN>(wd, s_db[i]), x, stats[ap.m + i], it);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -362,12 +481,16 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
     double racc = 0.0;
     for (int v = v0 + sub * 256 + threadIdx.x; v < v1; v += 256 * NSUB) {
         const uint16_t b = lp[v];
-        const double pv = prob_of(b, v, sp, inv_t);
-        const uint32_t key = bin_addr(rank_key(b));
+        const float w = score_of<PEN>(ap, job.row_p, v, b);
+        const uint32_t rk = key_of<PEN>(w, b);
+        const double pv = prob_of_w<PEN>(w, (int)rk, v, sp, inv_t);
+        const uint32_t key = bin_addr(rk);
         wp[v] = pv;
         if (pv > 0.0) atomicAdd(hp + key, (unsigned long long)(pv * FIX));
         if (job.mode == 2) {
-            const double mv = fmax(pv - prob_of(lq[v], v, sq, inv_t), 0.0);
+            const uint16_t bq = lq[v];
+            const float wq = score_of<PEN>(ap, job.row_q, v, bq);
+            const double mv = fmax(pv - prob_of_w<PEN>(wq, (int)key_of<PEN>(wq, bq), v, sq, inv_t), 0.0);
             wr[v] = mv;
             racc += mv;
             if (mv > 0.0) atomicAdd(hr + key, (unsigned long long)(mv * FIX));
@@ -423,9 +546,10 @@ __global__ __launch_bounds__(256) void k_trunc_clear(unsigned long long* tmass, 
     }
 }
 
+template <bool PEN>
 __global__ __launch_bounds__(256) void k_trunc_hist(const uint16_t* target, const uint16_t* draft, int m, int vocab,
                                                     double* scratch, unsigned long long* tmass, uint32_t* tcount,
-                                                    int want_mass) {
+                                                    int want_mass, const AcceptParams* app) {
     const int row = blockIdx.y, seg = blockIdx.x, lane = threadIdx.x & 63;
     Layout L = layout(scratch);
     const double mx = wave_max_f64(L.pmax[row * NSEG + lane]);
@@ -436,13 +560,18 @@ __global__ __launch_bounds__(256) void k_trunc_hist(const uint16_t* target, cons
     uint32_t* hc = tcount + (size_t)row * 65536;
     for (int v = v0 + threadIdx.x; v < v1; v += 256) {
         const uint16_t b = p[v];
-        const uint32_t key = bin_addr(rank_key(b));
+        float w;
+        if constexpr (PEN)
+            w = score_of<true>(*app, row, v, b);
+        else
+            w = h2f(b);
+        const uint32_t key = bin_addr(key_of<PEN>(w, b));
         unsigned long long mass = 0;
-        if (want_mass) mass = (unsigned long long)((exp((double)h2f(b) - mx) / sum) * FIX);
+        if (want_mass) mass = (unsigned long long)((exp((double)w - mx) / sum) * FIX);
         // a run of equal logits (a flat row) would serialise on one address: one lane adds for all
         const uint32_t first = __builtin_amdgcn_readfirstlane(key);
         const unsigned long long active = __ballot(1);
-        if (__ballot(key == first) == active) {
+        if (!PEN && __ballot(key == first) == active) {  // (equal keys are equal masses only without penalties)
             if (lane == (int)__builtin_ctzll(active)) {
                 const int n = __builtin_popcountll(active);
                 atomicAdd(hc + key, (uint32_t)n);
@@ -459,6 +588,63 @@ __global__ __launch_bounds__(256) void k_trunc_hist(const uint16_t* target, cons
 __device__ __forceinline__ uint32_t key_bits(int key) {
     const uint32_t asc = 0xFFFFu - (uint32_t)key;
     return (asc & 0x8000u) ? (asc & 0x7FFFu) : (~asc & 0xFFFFu);
+}
+
+// The candidates of rank bin `bin` that sit exactly on the bin's value, in index order over
+// [v0, v1).  Without penalties they are found by their fp16 bits.
+template <bool PEN, class Fn>
+__device__ __forceinline__ void scan_on(const AcceptParams& ap, int row, const uint16_t* lp, int v0, int v1, int bin,
+                                        bool vec, Fn&& on_match) {
+    const uint32_t want = key_bits(bin);
+    if constexpr (PEN) {
+        const float g = h2f((uint16_t)want);
+        for (int v = v0; v < v1; v++)
+            if (score_of<true>(ap, row, v, lp[v]) == g) on_match(v);
+    } else {
+        scan_chunk(lp, v0, v1, want, want == 0, vec, on_match);
+    }
+}
+
+// Penalised rounds, whole workgroup of 1024 threads: the candidates of `row` whose score falls
+// into rank bin `bin` without being the bin's own value, ordered by score descending, index
+// ascending, in sorted[0 .. n).  They precede the bin's on-value candidates in rank order.
+constexpr int SIDE_CAP = 1024;
+struct SideEnt {
+    float w;
+    int32_t v;
+};
+__device__ int collect_side(const AcceptParams& ap, int row, const uint16_t* lp, int bin, SideEnt* raw,
+                            SideEnt* sorted, int* counter, int32_t* err) {
+    const int tid = threadIdx.x;
+    const float g = h2f((uint16_t)key_bits(bin));
+    const int extra = row < ap.m ? row : 0;
+    __syncthreads();
+    if (tid == 0) *counter = 0;
+    __syncthreads();
+    for (int v = tid; v < ap.vocab; v += 1024) {
+        bool flagged = ap.pen_cnt[v] != 0;
+        for (int j = 0; j < extra; j++) flagged |= ap.feed[j + 1] == v;
+        if (!flagged) continue;  // an untouched score is an fp16 value: on its bin's value
+        const float w = score_of<true>(ap, row, v, lp[v]);
+        if (w != g && (int)rank_key(floor16(w)) == bin) {
+            const int i = atomicAdd(counter, 1);
+            if (i < SIDE_CAP) raw[i] = SideEnt{w, v};
+        }
+    }
+    __syncthreads();
+    int n = *counter;
+    if (n > SIDE_CAP) {  // refused: more penalised candidates between two neighbouring fp16 values than the list holds
+        if (tid == 0) atomicOr(err, 8);
+        n = SIDE_CAP;
+    }
+    for (int i = tid; i < n; i += 1024) {
+        const SideEnt me = raw[i];
+        int rank = 0;
+        for (int j = 0; j < n; j++) rank += raw[j].w > me.w || (raw[j].w == me.w && raw[j].v < me.v);
+        sorted[rank] = me;
+    }
+    __syncthreads();
+    return n;
 }
 
 // Exclusive prefix of a 64-bit value over the 1024 threads of a workgroup; *total gets the sum.
@@ -484,10 +670,13 @@ __device__ unsigned long long block_scan_u64(unsigned long long loc, unsigned lo
 }
 
 // One workgroup per distribution row.
+template <bool PEN>
 __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, const uint16_t* draft,
                                                     const AcceptParams* app, int m, double* scratch,
                                                     const unsigned long long* tmass, const uint32_t* tcount,
-                                                    AcceptResult* res) {
+                                                    AcceptResult* res, int32_t* err) {
+    __shared__ SideEnt s_raw[PEN ? SIDE_CAP : 1], s_sorted[PEN ? SIDE_CAP : 1];
+    __shared__ int s_nside;
     __shared__ unsigned long long wsum[16];
     __shared__ unsigned long long s_before_p;
     __shared__ int s_bin_k, s_j_k, s_bin_p, s_cnt_p, s_minp_key, s_bin, s_j, s_idx;
@@ -547,7 +736,7 @@ __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, cons
             }
         }
     }
-    if (ap.has_min_p) {
+    if (!PEN && ap.has_min_p) {  // (penalised rounds test e >= min_p per candidate instead)
         int best = -1;
         for (int i = 0; i < 64; i++) {
             const int key = tid * 64 + i;
@@ -558,24 +747,51 @@ __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, cons
         if (best >= 0) atomicMax(&s_minp_key, best);
     }
     __syncthreads();
+    const uint16_t* lp = row_ptr(target, draft, m, vocab, row);
+    int ns_p = 0;  // penalised rounds: the top-p bin's candidates above the bin's own value
+    if constexpr (PEN) {
+        if (s_bin_p >= 0) ns_p = collect_side(ap, row, lp, s_bin_p, s_raw, s_sorted, &s_nside, err);
+    }
     if (tid == 0) {
         int bin = s_bin_k, j = s_bin_k >= 0 ? s_j_k : 0;
         if (s_bin_p >= 0) {
             // how many candidates of the bin it takes to reach top_p: each carries the same mass
             const double pm = exp((double)h2f((uint16_t)key_bits(s_bin_p)) - mx) / sum;
-            const double before = (double)s_before_p / FIX;
-            long jp = (long)ceil((ap.top_p - before) / pm);
-            jp = jp < 1 ? 1 : jp;
-            while (jp > 1 && before + (double)(jp - 1) * pm >= ap.top_p) jp--;
-            while (jp < s_cnt_p && before + (double)jp * pm < ap.top_p) jp++;
-            jp = jp > s_cnt_p ? s_cnt_p : jp;
-            double mg = 1.0;
-            fold_margin(mg, before + (double)jp * pm, ap.top_p);
-            if (jp > 1 || s_before_p > 0) fold_margin(mg, before + (double)(jp - 1) * pm, ap.top_p);
-            s_margin = mg;
-            if (bin < 0 || s_bin_p < bin || (s_bin_p == bin && jp < j)) {
-                bin = s_bin_p;
-                j = (int)jp;
+            double before = (double)s_before_p / FIX;
+            long taken = 0;  // candidates above the bin's value, each with a mass of its own
+            bool reached = false;
+            double mg_side = 1.0;
+            if constexpr (PEN) {
+                for (int i = 0; i < ns_p && !reached; i++) {
+                    before += exp((double)s_sorted[i].w - mx) / sum;
+                    taken += 1;
+                    fold_margin(mg_side, before, ap.top_p);
+                    reached = before >= ap.top_p;
+                }
+                s_cnt_p -= ns_p;
+            }
+            long jp = reached || s_cnt_p <= 0 ? 0 : (long)ceil((ap.top_p - before) / pm);
+            if (reached || s_cnt_p <= 0) {
+                s_margin = mg_side;
+                jp = taken;
+                if (bin < 0 || s_bin_p < bin || (s_bin_p == bin && jp < j)) {
+                    bin = s_bin_p;
+                    j = (int)jp;
+                }
+            } else {
+                jp = jp < 1 ? 1 : jp;
+                while (jp > 1 && before + (double)(jp - 1) * pm >= ap.top_p) jp--;
+                while (jp < s_cnt_p && before + (double)jp * pm < ap.top_p) jp++;
+                jp = jp > s_cnt_p ? s_cnt_p : jp;
+                double mg = 1.0;
+                fold_margin(mg, before + (double)jp * pm, ap.top_p);
+                if (jp > 1 || s_before_p > 0) fold_margin(mg, before + (double)(jp - 1) * pm, ap.top_p);
+                s_margin = fmin(mg, mg_side);
+                jp += taken;
+                if (bin < 0 || s_bin_p < bin || (s_bin_p == bin && jp < j)) {
+                    bin = s_bin_p;
+                    j = (int)jp;
+                }
             }
         }
         if (ap.has_top_p && s_bin_p < 0) {  // the cumulative mass never reached top_p: everything ranked survives
@@ -587,30 +803,43 @@ __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, cons
         s_j = j;
     }
     __syncthreads();
-    const int bin = s_bin, j = s_j;
+    const int bin = s_bin;
+    int j = s_j;
+    float cut_w = bin >= 0 ? h2f((uint16_t)key_bits(bin)) : 0.f;
     if (bin >= 0 && j < (int)tcount[(size_t)row * 65536 + bin_addr(bin)]) {
-        // the j-th candidate of the bin in index order
-        const uint16_t* lp = row_ptr(target, draft, m, vocab, row);
-        const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = min(tid * per, vocab), v1 = min(v0 + per, vocab);
-        const bool vec = ((uintptr_t)lp & 15) == 0;
-        const uint32_t want = key_bits(bin);
-        const bool zero_bin = want == 0;
-        int n = 0;
-        scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int) { n++; });
-        const unsigned long long excl = block_scan_u64((unsigned long long)n, wsum, &total);
-        if ((int)excl < j && j <= (int)excl + n) {
-            int c = (int)excl;
-            scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int v) {
-                c++;
-                if (c == j) s_idx = v;
-            });
+        bool on_value = true;
+        if constexpr (PEN) {
+            // the bin's candidates above its own value come first in rank order
+            const int ns = bin == s_bin_p ? ns_p : collect_side(ap, row, lp, bin, s_raw, s_sorted, &s_nside, err);
+            if (j <= ns) {
+                if (tid == 0) s_idx = s_sorted[j - 1].v;
+                cut_w = s_sorted[j - 1].w;
+                on_value = false;
+            } else {
+                j -= ns;
+            }
+        }
+        if (on_value) {
+            // the j-th candidate on the bin's value in index order
+            const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = min(tid * per, vocab), v1 = min(v0 + per, vocab);
+            const bool vec = ((uintptr_t)lp & 15) == 0;
+            int n = 0;
+            scan_on<PEN>(ap, row, lp, v0, v1, bin, vec, [&](int) { n++; });
+            const unsigned long long excl = block_scan_u64((unsigned long long)n, wsum, &total);
+            if ((int)excl < j && j <= (int)excl + n) {
+                int c = (int)excl;
+                scan_on<PEN>(ap, row, lp, v0, v1, bin, vec, [&](int v) {
+                    c++;
+                    if (c == j) s_idx = v;
+                });
+            }
         }
         __syncthreads();
     }
     if (tid == 0) {
-        Cut cut{65536, 0x7FFFFFFF};
-        if (bin >= 0) cut = Cut{bin, s_idx};
-        if (ap.has_min_p && s_minp_key >= 0 && s_minp_key < cut.key) cut = Cut{s_minp_key, 0x7FFFFFFF};
+        Cut cut{65536, 0x7FFFFFFF, 0.f, 0.f};
+        if (bin >= 0) cut = Cut{bin, s_idx, cut_w, 0.f};
+        if (!PEN && ap.has_min_p && s_minp_key >= 0 && s_minp_key < cut.key) cut = Cut{s_minp_key, 0x7FFFFFFF, 0.f, 0.f};
         L.cut[row] = cut;
         atomicMin((unsigned long long*)&res->min_margin, __builtin_bit_cast(unsigned long long, s_margin));
     }
@@ -620,11 +849,15 @@ __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, cons
 // One workgroup per job.  Finds the rank bin in which the cumulative mass first exceeds the
 // uniform (exact integer prefix over the fixed-point bins, cleared as they are read), then
 // walks that bin's candidates in index order in f64.
+template <bool PEN>
 __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uint16_t* draft,
                                                const AcceptParams* app, double* scratch, const double* work,
                                                unsigned long long* hist, const Decision* dec_in,
-                                               AcceptResult* res, int32_t* tokens_out, const int32_t* err,
+                                               AcceptResult* res, int32_t* tokens_out, int32_t* err,
                                                int kind) {
+    __shared__ SideEnt s_raw[PEN ? SIDE_CAP : 1], s_sorted[PEN ? SIDE_CAP : 1];
+    __shared__ int s_nside, s_side_last;
+    __shared__ double s_side_sum;
     __shared__ unsigned long long wsum[16];
     __shared__ double dsum[16];
     __shared__ unsigned long long s_total, s_before;
@@ -717,15 +950,41 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             bin = s_bin;
         }
         const bool fallback = s_fallback != 0;
+        const double norm = (double)s_total;  // fixed-point total <-> 1.0 (p mode) or R (residual)
+        const double cum0 = (double)s_before / norm;  // cumulative mass before this bin
+        double side_sum = 0.0;
+        if constexpr (PEN) {
+            // the bin's candidates above its own value come first: few, walked by one thread
+            const int ns = collect_side(ap, dec.job.row_p, lp, bin, s_raw, s_sorted, &s_nside, err);
+            if (tid == 0) {
+                double c = cum0;
+                int last = -1;
+                bool found = false;
+                for (int i = 0; i < ns; i++) {
+                    const int v = s_sorted[i].v;
+                    const double wv = mode == 2 ? w[v] / R : w[v];
+                    if (mode == 2 && !(wv > 0.0)) continue;
+                    if (!fallback && !found && dec.job.u < c + wv) {
+                        s_token = v;
+                        s_cum_before = c;
+                        s_cum_at = c + wv;
+                        found = true;
+                    }
+                    c += wv;
+                    last = v;
+                }
+                s_side_sum = c - cum0;
+                s_side_last = last;
+            }
+            __syncthreads();
+            side_sum = s_side_sum;
+        }
         // walk the bin in index order: contiguous index chunk per thread
-        const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = tid * per, v1 = min(v0 + per, vocab);
+        const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = min(tid * per, vocab), v1 = min(v0 + per, vocab);
         const bool vec = ((uintptr_t)lp & 15) == 0;
-        const uint32_t asc = 0xFFFFu - (uint32_t)bin;  // inverse of rank_key
-        const uint32_t want = (asc & 0x8000u) ? (asc & 0x7FFFu) : (~asc & 0xFFFFu);
-        const bool zero_bin = want == 0;
         double lsum = 0.0;
         int lastv = -1;
-        scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int v) {
+        scan_on<PEN>(ap, dec.job.row_p, lp, v0, v1, bin, vec, [&](int v) {
             const double wv = mode == 2 ? w[v] / R : w[v];
             if (mode != 2 || wv > 0.0) {
                 lsum += wv;
@@ -743,9 +1002,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         __syncthreads();
         double dbase = 0.0;
         for (int i = 0; i < wave; i++) dbase += dsum[i];
-        const double norm = (double)s_total;  // fixed-point total <-> 1.0 (p mode) or R (residual)
-        const double cum0 = (double)s_before / norm;  // cumulative mass before this bin
-        const double before = cum0 + (dbase + incd - lsum);
+        const double before = PEN ? cum0 + side_sum + (dbase + incd - lsum) : cum0 + (dbase + incd - lsum);
         if (fallback) {
             if (lastv >= 0) atomicMax(&s_token, lastv);
         } else {
@@ -753,7 +1010,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             if (lsum > 0.0 && !(u < before) && u < before + lsum) {
                 double c = before;
                 bool found = false;
-                scan_chunk(lp, v0, v1, want, zero_bin, vec, [&](int v) {
+                scan_on<PEN>(ap, dec.job.row_p, lp, v0, v1, bin, vec, [&](int v) {
                     if (found) return;
                     const double wv = mode == 2 ? w[v] / R : w[v];
                     if (mode == 2 && !(wv > 0.0)) return;
@@ -770,6 +1027,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         }
         __syncthreads();
         token = s_token;
+        if (PEN && fallback && token < 0) token = s_side_last;  // no on-value candidate: the last of the others
         if (token < 0) {
             // the f64 walk and the fixed-point bin search disagreed by a rounding: the uniform
             // sits on a bin edge.  Take the bin's first (u below) or last candidate and report
@@ -777,6 +1035,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             if (lastv >= 0) atomicMax(&s_token, lastv);
             __syncthreads();
             token = s_token;
+            if (PEN && token < 0) token = s_side_last;
             margin = 0.0;
         } else if (!fallback) {
             margin = fmin(margin, fmin(dec.job.u - s_cum_before, s_cum_at - dec.job.u));
@@ -1039,17 +1298,56 @@ static Decision* decisions(const AcceptScratch& sc) {
 }
 
 // Between the softmax sums and the reweighting totals: the truncation cut of every row.
+template <bool PEN>
 static void launch_trunc(hipStream_t s, const uint16_t* target, const uint16_t* draft, int m, int rows,
                          const AcceptParams* ap_dev, const AcceptParams& ap, const AcceptScratch& sc) {
-    if (ap.top_k == 0 && !ap.has_top_p && !ap.has_min_p) return;
+    if (ap.top_k == 0 && !ap.has_top_p) {
+        if (PEN || !ap.has_min_p) return;  // (penalised rounds test min-p per candidate)
+    }
     unsigned long long* tm = (unsigned long long*)sc.tmass;
     if (ap.top_k != 0 || ap.has_top_p) {
         hipLaunchKernelGGL(k_trunc_clear, dim3(64 * rows), dim3(256), 0, s, tm, sc.tcount, rows);
-        hipLaunchKernelGGL(k_trunc_hist, dim3(NSEG, rows), dim3(256), 0, s, target, draft, m, ap.vocab, sc.stats, tm,
-                           sc.tcount, ap.has_top_p);
+        hipLaunchKernelGGL(k_trunc_hist<PEN>, dim3(NSEG, rows), dim3(256), 0, s, target, draft, m, ap.vocab, sc.stats, tm,
+                           sc.tcount, ap.has_top_p, ap_dev);
     }
-    hipLaunchKernelGGL(k_trunc_cut, dim3(rows), dim3(1024), 0, s, target, draft, ap_dev, m, sc.stats, tm, sc.tcount,
-                       sc.result);
+    hipLaunchKernelGGL(k_trunc_cut<PEN>, dim3(rows), dim3(1024), 0, s, target, draft, ap_dev, m, sc.stats, tm, sc.tcount,
+                       sc.result, (int32_t*)sc.counters);
+}
+
+// The statistics of `rows` distribution rows, their truncation cuts and reweighting totals.
+template <bool PEN>
+static void launch_stats(hipStream_t s, const uint16_t* target, const uint16_t* draft, int m, int rows, int hist_words,
+                         const AcceptParams* ap_dev, const AcceptParams& ap, const AcceptScratch& sc) {
+    int32_t* err = (int32_t*)sc.counters;
+    const double inv_t = 1.0 / ap.temperature;
+    hipLaunchKernelGGL(k_row_max<PEN>, dim3(NSEG, rows), dim3(256), 0, s, target, draft, m, ap.vocab, sc.stats, err,
+                       (unsigned long long*)sc.hist, hist_words, ap_dev);
+    hipLaunchKernelGGL(k_row_sum<PEN>, dim3(NSEG, rows), dim3(256), 0, s, target, draft, m, ap.vocab, sc.stats, ap_dev);
+    launch_trunc<PEN>(s, target, draft, m, rows, ap_dev, ap, sc);
+    hipLaunchKernelGGL(k_row_total<PEN>, dim3(NSEG, rows), dim3(256), 0, s, target, draft, m, ap.vocab, sc.stats, inv_t,
+                       ap_dev);
+}
+
+template <bool PEN>
+static void launch_chain_sampled(hipStream_t s, const uint16_t* target, const uint16_t* draft,
+                                 const AcceptParams* ap_dev, const AcceptParams& ap, const AcceptScratch& sc) {
+    int32_t* err = (int32_t*)sc.counters;
+    launch_stats<PEN>(s, target, draft, ap.m, ap.m + ap.k, 2 * 65536, ap_dev, ap, sc);
+    hipLaunchKernelGGL(k_mass_hist<PEN>, dim3(NSEG, 1, NSUB), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), 0);
+    hipLaunchKernelGGL(k_pick<PEN>, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), sc.result, (int32_t*)nullptr, err, 0);
+}
+
+template <bool PEN>
+static void launch_draft_sampled(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,
+                                 const AcceptParams& ap, const AcceptScratch& sc, int32_t* proposals_dev) {
+    int32_t* err = (int32_t*)sc.counters;
+    launch_stats<PEN>(s, draft, draft, 0, ap.k, ap.k * 2 * 65536, ap_dev, ap, sc);
+    hipLaunchKernelGGL(k_mass_hist<PEN>, dim3(NSEG, ap.k, NSUB), dim3(256), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), 1);
+    hipLaunchKernelGGL(k_pick<PEN>, dim3(ap.k), dim3(1024), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), sc.result, proposals_dev, err, 1);
 }
 
 int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
@@ -1057,41 +1355,32 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
     int32_t* err = (int32_t*)sc.counters;
     int32_t* amax = (int32_t*)sc.counters + 16;
     hipLaunchKernelGGL(k_clear_result, dim3(1), dim3(64), 0, s, sc.result, err);
-    if (!ap.sampled) {
+    if (!ap.sampled) {  // (the arg-max ignores penalties and truncation: choose.rs:84-88)
         hipLaunchKernelGGL(k_argmax, dim3(ap.m), dim3(1024), 0, s, target, ap.vocab, amax, err);
         hipLaunchKernelGGL(k_walk_greedy, dim3(1), dim3(64), 0, s, ap_dev, amax, sc.result, err);
         TSV_HIP(hipGetLastError());
         return TSV_OK;
     }
     if (ap.tree) {
+        if (ap.pen) {
+            set_error("device acceptance: penalties are not built for a sampled tree round");
+            return TSV_ERR_UNSUPPORTED;
+        }
         // statistics of the m target rows and the m rows the children were drawn from
-        const int rows2 = 2 * ap.m;
-        const double it = 1.0 / ap.temperature;
         int32_t* path = (int32_t*)sc.counters + 32;
-        hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err,
-                           (unsigned long long*)sc.hist, 2 * 65536);
-        hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
-        launch_trunc(s, target, draft, ap.m, rows2, ap_dev, ap, sc);
-        hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, it);
-        hipLaunchKernelGGL(k_tree_probs, dim3(NSEG, rows2), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
+        launch_stats<false>(s, target, draft, ap.m, 2 * ap.m, 2 * 65536, ap_dev, ap, sc);
+        hipLaunchKernelGGL(k_tree_probs, dim3(NSEG, 2 * ap.m), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
         hipLaunchKernelGGL(k_tree_sampled, dim3(1), dim3(1024), 0, s, target, ap_dev, sc.stats, sc.work,
                            (unsigned long long*)sc.hist, decisions(sc), path);
-        hipLaunchKernelGGL(k_pick, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+        hipLaunchKernelGGL(k_pick<false>, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                            (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);
         TSV_HIP(hipGetLastError());
         return TSV_OK;
     }
-    const int rows = ap.m + ap.k;
-    const double inv_t = 1.0 / ap.temperature;
-    hipLaunchKernelGGL(k_row_max, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, err,
-                       (unsigned long long*)sc.hist, 2 * 65536);
-    hipLaunchKernelGGL(k_row_sum, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats);
-    launch_trunc(s, target, draft, ap.m, rows, ap_dev, ap, sc);
-    hipLaunchKernelGGL(k_row_total, dim3(NSEG, rows), dim3(256), 0, s, target, draft, ap.m, ap.vocab, sc.stats, inv_t);
-    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, 1, NSUB), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work,
-                       (unsigned long long*)sc.hist, decisions(sc), 0);
-    hipLaunchKernelGGL(k_pick, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
-                       (unsigned long long*)sc.hist, decisions(sc), sc.result, (int32_t*)nullptr, err, 0);
+    if (ap.pen)
+        launch_chain_sampled<true>(s, target, draft, ap_dev, ap, sc);
+    else
+        launch_chain_sampled<false>(s, target, draft, ap_dev, ap, sc);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -1107,16 +1396,38 @@ int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams*
         TSV_HIP(hipGetLastError());
         return TSV_OK;
     }
-    const double inv_t = 1.0 / ap.temperature;
-    hipLaunchKernelGGL(k_row_max, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, err,
-                       (unsigned long long*)sc.hist, ap.k * 2 * 65536);
-    hipLaunchKernelGGL(k_row_sum, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats);
-    launch_trunc(s, draft, draft, 0, ap.k, ap_dev, ap, sc);
-    hipLaunchKernelGGL(k_row_total, dim3(NSEG, ap.k), dim3(256), 0, s, draft, draft, 0, ap.vocab, sc.stats, inv_t);
-    hipLaunchKernelGGL(k_mass_hist, dim3(NSEG, ap.k, NSUB), dim3(256), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
-                       (unsigned long long*)sc.hist, decisions(sc), 1);
-    hipLaunchKernelGGL(k_pick, dim3(ap.k), dim3(1024), 0, s, draft, draft, ap_dev, sc.stats, sc.work,
-                       (unsigned long long*)sc.hist, decisions(sc), sc.result, proposals_dev, err, 1);
+    if (ap.pen)
+        launch_draft_sampled<true>(s, draft, ap_dev, ap, sc, proposals_dev);
+    else
+        launch_draft_sampled<false>(s, draft, ap_dev, ap, sc, proposals_dev);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+// The history's token statistics for a penalised round: cnt[v] bit 31 = v occurs in history[0, n),
+// low bits = occurrences in history[suffix_start, n).  Token ids outside [0, vocab) are skipped
+// (penalty.rs:27-33,73-78).
+namespace {
+__global__ void k_pen_clear(uint32_t* cnt, int vocab) {
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    if (v < vocab) cnt[v] = 0;
+}
+__global__ void k_pen_count(const int32_t* history, long n, long suffix_start, int vocab, uint32_t* cnt) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const int32_t t = history[i];
+        if (t < 0 || t >= vocab) continue;
+        atomicOr(cnt + t, 0x80000000u);
+        if (i >= suffix_start) atomicAdd(cnt + t, 1u);
+    }
+}
+}  // namespace
+
+int launch_pen_counts(hipStream_t s, const int32_t* history_dev, long n, long suffix_start, int vocab, uint32_t* cnt) {
+    hipLaunchKernelGGL(k_pen_clear, dim3((vocab + 255) / 256), dim3(256), 0, s, cnt, vocab);
+    if (n > 0) {
+        const int blocks = (int)std::min<long>((n + 255) / 256, 256);
+        hipLaunchKernelGGL(k_pen_count, dim3(blocks), dim3(256), 0, s, history_dev, n, suffix_start, vocab, cnt);
+    }
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -83,9 +83,10 @@ bool is_stop(const tsv_generation* g, int32_t t) {
 
 // select() of one logits row at draw position `position` (choose.rs:61-98): arg-max, or a draw
 // from the shaped distribution
-int select_row(tsv_ctx* c, const uint16_t* row, const tsv_shaping* sh, uint64_t position, int32_t* token) {
+int select_row(tsv_ctx* c, const uint16_t* row, const tsv_shaping* sh, uint64_t position, int32_t* token,
+               const std::vector<int32_t>& hist, uint64_t generated) {
     uint64_t at = position;
-    return tsv_draft_chain(c, row, 1, sh, &at, token);
+    return tsv_draft_chain(c, row, 1, sh, &at, token, hist.data(), (int64_t)hist.size(), generated);
 }
 
 }  // namespace
@@ -144,9 +145,10 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         }
     if ((rc = tsv_produce(c, prompt[n - 1], n - 1, logits.data()))) return rc;
     int64_t history = n;  // tokens backed by KV rows or about to be
+    std::vector<int32_t> hist(prompt, prompt + n);  // TokenSink::history: what the penalties look at
     uint64_t generated = 0, draw_step = 0;
     int32_t next;
-    if ((rc = select_row(c, logits.data(), &g->shaping, generated, &next))) return rc;
+    if ((rc = select_row(c, logits.data(), &g->shaping, generated, &next, hist, generated))) return rc;
 
     int32_t feed[TSV_MAX_ROWS];
     for (;;) {
@@ -162,6 +164,7 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
             break;
         }
         history += 1;
+        hist.push_back(next);
         const int64_t base = history - 1, position = history;
         const uint64_t budget_room = g->max_new_tokens - generated;
         const int64_t context_room = max_context - position;
@@ -191,7 +194,8 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
                 set_error("run_speculative: draft_step failed");
                 return TSV_ERR_INVALID;
             }
-            if ((rc = select_row(c, row, &g->shaping, sampled ? draw_step : generated, &chained))) return rc;
+            if ((rc = select_row(c, row, &g->shaping, sampled ? draw_step : generated, &chained, hist, generated)))
+                return rc;
             if (sampled) draw_step += 1;
             feed[1 + d] = chained;
         }
@@ -207,6 +211,8 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         r.n_stop = g->n_stop;
         r.generated = generated;
         r.max_new_tokens = g->max_new_tokens;
+        r.history = hist.data();
+        r.n_history = (int64_t)hist.size();
         tsv_round_result res{};
         if ((rc = tsv_verify_accept(c, &r, &res))) return rc;
         out->rounds += 1;
@@ -220,6 +226,7 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         if (res.stopped == 2 && (rc = emit.push(feed[1 + res.committed]))) return rc;  // the budget's last token is reported
         generated += (uint64_t)res.accepted;
         history += res.committed;
+        hist.insert(hist.end(), feed + 1, feed + 1 + res.committed);
         draw_step = res.draw_step;
         if (dr->rewind(dr->user, base + res.committed)) {
             set_error("run_speculative: rewind_drafter failed");

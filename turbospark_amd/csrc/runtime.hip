@@ -86,6 +86,9 @@ struct tsv_ctx {
     uint16_t* draft_stage = nullptr;  // [16][vocab] fp16, device
     VerifyParams *vp_dev = nullptr, *vp_host = nullptr;
     AcceptParams *ap_dev = nullptr, *ap_host = nullptr;
+    int32_t* hist_dev = nullptr;  // the token history of a penalised round (grows on demand)
+    size_t hist_cap = 0;
+    uint32_t* pen_cnt = nullptr;  // [vocab] seen flag + generated-suffix count per token
     AcceptResult* res_host = nullptr;
     int32_t *tok_dev = nullptr, *tok_host = nullptr;
     AcceptScratch sc{};
@@ -284,12 +287,17 @@ int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
         set_error("a sampled round needs an explicit seed");
         return TSV_ERR_INVALID;
     }
-    if (sampled_supported_only &&
-        (s.repetition_penalty != 1.0 || s.presence_penalty != 0.0 || s.frequency_penalty != 0.0)) {
-        set_error("device acceptance: repetition / presence / frequency penalties are not built");
-        return TSV_ERR_UNSUPPORTED;
+    (void)sampled_supported_only;
+    if (!(s.repetition_penalty > 0.0) || !std::isfinite(s.repetition_penalty) || !std::isfinite(s.presence_penalty) ||
+        !std::isfinite(s.frequency_penalty)) {
+        set_error("penalties must be finite, the repetition penalty positive");
+        return TSV_ERR_INVALID;
     }
     return TSV_OK;
+}
+
+bool has_penalties(const tsv_shaping& s) {
+    return s.temperature != 0.0 && (s.repetition_penalty != 1.0 || s.presence_penalty != 0.0 || s.frequency_penalty != 0.0);
 }
 
 enum { PC_EMBED = 0, PC_NORM, PC_QKV, PC_ROPE, PC_ATTN, PC_WO, PC_GATEUP, PC_DOWN, PC_HEAD, PC_ACCEPT, PC_EVENTPAIR, PC_COUNT };
@@ -893,6 +901,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->draft_stage, (size_t)16 * c->vocab * 2, true)) ||
         (rc = dev_alloc(c, &c->vp_dev, sizeof(VerifyParams), true)) ||
         (rc = dev_alloc(c, &c->ap_dev, sizeof(AcceptParams), true)) ||
+        (rc = dev_alloc(c, &c->pen_cnt, (size_t)c->vocab * 4, true)) ||
         (rc = dev_alloc(c, &c->tok_dev, 64 * 4, true)) ||
         (rc = dev_alloc(c, &c->sc.stats, accept_stats_doubles() * 8, true)) ||
         (rc = dev_alloc(c, &c->sc.work, (size_t)(16 * 2 + 2) * c->vocab * 8, true)) ||
@@ -952,6 +961,7 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (!c) return;
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (void* p : c->allocs) (void)hipFree(p);
+    if (c->hist_dev) (void)hipFree(c->hist_dev);
     if (c->vp_host) (void)hipHostFree(c->vp_host);
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
@@ -1138,6 +1148,47 @@ int fill_accept(tsv_ctx* c, const tsv_round* r, AcceptParams* ap) {
     return TSV_OK;
 }
 
+// Penalised sampled rounds (choose.rs:138-154): uploads the history, counts its tokens on the device
+// and fills the penalty fields of the parameter block.  `generated` is the sink's count of reported
+// tokens: the last min(generated, n) tokens of the history are the generated suffix.
+int setup_penalties(tsv_ctx* c, const tsv_shaping& sh, const int32_t* history, int64_t n, uint64_t generated,
+                    AcceptParams* ap) {
+    ap->pen = 0;
+    if (!has_penalties(sh)) return TSV_OK;
+    if (n < 0 || (n > 0 && !history)) {
+        set_error("penalties: the round carries no token history");
+        return TSV_ERR_INVALID;
+    }
+    if ((size_t)n > c->hist_cap) {
+        if (c->hist_dev) TSV_HIP(hipFree(c->hist_dev));
+        c->hist_dev = nullptr;
+        c->hist_cap = 0;
+        const size_t cap = ((size_t)n + 4095) & ~(size_t)4095;
+        TSV_HIP(hipMalloc((void**)&c->hist_dev, cap * 4));
+        c->hist_cap = cap;
+    }
+    if (n > 0) TSV_HIP(hipMemcpyAsync(c->hist_dev, history, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
+    const int64_t suffix = (int64_t)std::min<uint64_t>(generated, (uint64_t)n);
+    int rc = launch_pen_counts(c->stream, c->hist_dev, (long)n, (long)(n - suffix), c->vocab, c->pen_cnt);
+    if (rc) return rc;
+    if (n > 0) TSV_HIP(hipStreamSynchronize(c->stream));  // the caller's history buffer is free again
+    ap->pen = 1;
+    ap->pen_has_rep = sh.repetition_penalty != 1.0;
+    // penalty.rs:20-25: the f64 setting as an f32 kept inside the normal range
+    ap->pen_rep = std::min(std::max((float)sh.repetition_penalty, 1.17549435e-38f), 3.40282347e+38f);
+    ap->pen_has_pf = sh.presence_penalty != 0.0 || sh.frequency_penalty != 0.0;
+    ap->pen_presence = sh.presence_penalty;
+    ap->pen_frequency = sh.frequency_penalty;
+    ap->pen_cnt = c->pen_cnt;
+    return TSV_OK;
+}
+
+const char* accept_error_text(int bits) {
+    if (bits & 1) return "score vector must not contain a non-finite entry";
+    if (bits & 4) return "a penalised score lies below every fp16 value (not built)";
+    return "too many penalised candidates between two neighbouring fp16 values (not built)";
+}
+
 int stage_draft(tsv_ctx* c, const uint16_t* draft, int rows, const uint16_t** dev) {
     if (is_device_pointer(draft)) {
         *dev = draft;
@@ -1148,8 +1199,18 @@ int stage_draft(tsv_ctx* c, const uint16_t* draft, int rows, const uint16_t** de
     return TSV_OK;
 }
 
-int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
+int check_round(const tsv_round* r) {
     int rc = check_shaping(r->shaping, true);
+    if (rc) return rc;
+    if (r->parent && has_penalties(r->shaping)) {
+        set_error("device acceptance: penalties are not built for a sampled tree round");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    return TSV_OK;
+}
+
+int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
+    int rc = check_round(r);
     if (rc) return rc;
     if (r->m != c->last_m || r->base != c->last_base) {
         set_error("accept: the round does not describe the last verify pass");
@@ -1170,6 +1231,7 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     }
     TSV_HIP(hipStreamSynchronize(c->stream));  // pinned parameter block is about to be rewritten
     if ((rc = fill_accept(c, r, c->ap_host))) return rc;
+    if ((rc = setup_penalties(c, r->shaping, r->history, r->n_history, r->generated, c->ap_host))) return rc;
     TSV_HIP(hipMemcpyAsync(c->ap_dev, c->ap_host, sizeof(AcceptParams), hipMemcpyHostToDevice, c->stream));
     {
         PROF(PC_ACCEPT);
@@ -1183,8 +1245,8 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     if ((rc = check_fused(c))) return rc;
     const AcceptResult& a = *c->res_host;
     if (a.error) {
-        set_error("accept: score vector must not contain a non-finite entry");
-        return TSV_ERR_INVALID;
+        set_error(std::string("accept: ") + accept_error_text(a.error));
+        return (a.error & 1) ? TSV_ERR_INVALID : TSV_ERR_UNSUPPORTED;
     }
     std::memset(out, 0, sizeof *out);
     out->accepted = a.accepted;
@@ -1223,14 +1285,15 @@ extern "C" int32_t tsv_verify_accept(tsv_ctx* c, const tsv_round* r, tsv_round_r
         set_error("verify_accept: null argument");
         return TSV_ERR_INVALID;
     }
-    int rc = check_shaping(r->shaping, true);
+    int rc = check_round(r);
     if (rc) return rc;
     if ((rc = enqueue_verify(c, r->feed, r->parent, r->m, r->base))) return rc;
     return accept_impl(c, r, out);
 }
 
 extern "C" int32_t tsv_draft_chain(tsv_ctx* c, const uint16_t* draft_logits, int32_t k, const tsv_shaping* sh,
-                                   uint64_t* draw_step, int32_t* proposals) {
+                                   uint64_t* draw_step, int32_t* proposals, const int32_t* history,
+                                   int64_t n_history, uint64_t generated) {
     if (!c || !draft_logits || !sh || !draw_step || !proposals || k < 1 || k > TSV_MAX_ROWS - 1) {
         set_error("draft_chain: bad argument");
         return TSV_ERR_INVALID;
@@ -1250,14 +1313,15 @@ extern "C" int32_t tsv_draft_chain(tsv_ctx* c, const uint16_t* draft_logits, int
     ap->seed = sh->seed;
     fill_truncation(ap, *sh);
     ap->draw_step = *draw_step;
+    if ((rc = setup_penalties(c, *sh, history, n_history, generated, ap))) return rc;
     TSV_HIP(hipMemcpyAsync(c->ap_dev, ap, sizeof *ap, hipMemcpyHostToDevice, c->stream));
     if ((rc = launch_draft_chain(c->stream, draft, c->ap_dev, *ap, c->sc, c->tok_dev))) return rc;
     TSV_HIP(hipMemcpyAsync(c->tok_host, c->tok_dev, (size_t)k * 4, hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipMemcpyAsync(c->res_host, c->sc.result, sizeof(AcceptResult), hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipStreamSynchronize(c->stream));
     if (c->res_host->error) {
-        set_error("draft_chain: score vector must not contain a non-finite entry");
-        return TSV_ERR_INVALID;
+        set_error(std::string("draft_chain: ") + accept_error_text(c->res_host->error));
+        return (c->res_host->error & 1) ? TSV_ERR_INVALID : TSV_ERR_UNSUPPORTED;
     }
     for (int i = 0; i < k; i++) proposals[i] = c->tok_host[i];
     if (ap->sampled) *draw_step += (uint64_t)k + 1;  // k draws + the row-only step (speculative.rs:618-624)

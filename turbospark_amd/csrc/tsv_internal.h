@@ -271,6 +271,12 @@ struct AcceptParams {
     // truncation of the candidate set (crates/selection/src/choose.rs:111-228): 0 / false = off
     int32_t top_k, has_top_p, has_min_p, pad0;
     double top_p, min_p;
+    // penalties (crates/selection/src/penalty.rs:15-82); pen == 0: none.  pen_cnt[v]: bit 31 = token v
+    // is in the history, low bits = its occurrences in the generated suffix of the history.
+    int32_t pen, pen_has_rep, pen_has_pf;
+    float pen_rep;  // the repetition penalty as the clamped f32 the reference divides / multiplies by
+    double pen_presence, pen_frequency;
+    const uint32_t* pen_cnt;
 };
 struct AcceptResult {
     int32_t accepted, committed, next, stopped;
@@ -294,6 +300,7 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
                   const AcceptParams& ap_host, const AcceptScratch& sc);
 int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,
                        const AcceptParams& ap_host, const AcceptScratch& sc, int32_t* proposals_dev);
+int launch_pen_counts(hipStream_t s, const int32_t* history_dev, long n, long suffix_start, int vocab, uint32_t* cnt);
 
 // ---- host utilities ----------------------------------------------------------------------
 int64_t row_bytes(int dtype, int64_t cols);

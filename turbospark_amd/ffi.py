@@ -135,6 +135,7 @@ class Round(C.Structure):
         ("base", C.c_int64), ("shaping", Shaping), ("draft_logits", C.c_void_p),
         ("draw_step", C.c_uint64), ("stop_tokens", C.POINTER(C.c_int32)), ("n_stop", C.c_int32),
         ("generated", C.c_uint64), ("max_new_tokens", C.c_uint64), ("logits_out", C.c_void_p),
+        ("history", C.POINTER(C.c_int32)), ("n_history", C.c_int64),
     ]
 
 
@@ -201,7 +202,7 @@ def lib():
         L.tsv_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
         L.tsv_verify_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
         L.tsv_draft_chain.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(Shaping),
-                                      C.POINTER(C.c_uint64), C.c_void_p]
+                                      C.POINTER(C.c_uint64), C.c_void_p, C.c_void_p, C.c_int64, C.c_uint64]
         L.tsv_quantize_rows.argtypes = [C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
         L.tsv_synth_tensor.argtypes = [C.c_int32, C.c_uint64, C.c_uint64, C.c_float, C.c_int64, C.c_int64,
                                        C.c_void_p]

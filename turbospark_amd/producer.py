@@ -145,9 +145,13 @@ class HipVerifier:
 
     # ---- device-side acceptance -----------------------------------------------------------
     def _round(self, feed, base, cfg, parent, draft_logits, draw_step, stop_tokens, generated,
-               max_new_tokens, want_logits):
+               max_new_tokens, want_logits, history=None):
         keep = {}
         r = ffi.Round()
+        if history is not None and len(history):
+            keep["history"] = _i32(history)
+            r.history = keep["history"].ctypes.data_as(C.POINTER(C.c_int32))
+            r.n_history = keep["history"].size
         keep["feed"] = _i32(feed)
         r.feed = keep["feed"].ctypes.data_as(C.POINTER(C.c_int32))
         r.m = keep["feed"].size
@@ -183,26 +187,28 @@ class HipVerifier:
                            list(c.path[: c.path_len]), c.kv_position, c.min_margin)
 
     def accept(self, feed, base, cfg, parent=None, draft_logits=None, draw_step=0, stop_tokens=None,
-               generated=0, max_new_tokens=0):
-        """Acceptance + truncation over the logits the last verify left on the device."""
+               generated=0, max_new_tokens=0, history=None):
+        """Acceptance + truncation over the logits the last verify left on the device.  `history`
+        (the sink's tokens when the round starts) is what the penalties of `cfg` look at."""
         r, keep = self._round(feed, base, cfg, parent, draft_logits, draw_step, stop_tokens, generated,
-                              max_new_tokens, False)
+                              max_new_tokens, False, history)
         out = ffi.RoundResultC()
         ffi.check(ffi.lib().tsv_accept(self._h, C.byref(r), C.byref(out)))
         return self._result(out)
 
     def verify_accept(self, feed, base, cfg, parent=None, draft_logits=None, draw_step=0,
-                      stop_tokens=None, generated=0, max_new_tokens=0, want_logits=False):
+                      stop_tokens=None, generated=0, max_new_tokens=0, want_logits=False, history=None):
         """The whole verify step: target forward, acceptance, KV truncation."""
         r, keep = self._round(feed, base, cfg, parent, draft_logits, draw_step, stop_tokens, generated,
-                              max_new_tokens, want_logits)
+                              max_new_tokens, want_logits, history)
         out = ffi.RoundResultC()
         ffi.check(ffi.lib().tsv_verify_accept(self._h, C.byref(r), C.byref(out)))
         res = self._result(out)
         return (res, keep["logits"]) if want_logits else res
 
-    def draft_chain(self, draft_logits, cfg, draw_step=0):
-        """Draw the k proposals of a chain round from the drafter's rows; returns (proposals, draw_step)."""
+    def draft_chain(self, draft_logits, cfg, draw_step=0, history=None, generated=0):
+        """Draw the k proposals of a chain round from the drafter's rows; returns (proposals, draw_step).
+        `history` / `generated`: the sink's state, read by the penalties of `cfg`."""
         if isinstance(draft_logits, tuple):  # (device pointer, k)
             ptr, k = draft_logits
         else:
@@ -213,7 +219,10 @@ class HipVerifier:
             ptr, k = a.ctypes.data, a.shape[0]
         ds = C.c_uint64(int(draw_step))
         props = np.empty(k, np.int32)
-        ffi.check(ffi.lib().tsv_draft_chain(self._h, ptr, k, C.byref(cfg), C.byref(ds), props.ctypes.data))
+        hist = _i32(history) if history is not None and len(history) else None
+        ffi.check(ffi.lib().tsv_draft_chain(self._h, ptr, k, C.byref(cfg), C.byref(ds), props.ctypes.data,
+                                            hist.ctypes.data if hist is not None else None,
+                                            hist.size if hist is not None else 0, int(generated)))
         return props, ds.value
 
     # ---- the generation loop --------------------------------------------------------------
