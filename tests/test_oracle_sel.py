@@ -161,6 +161,40 @@ def test_penalties():
     assert np.allclose(got, want, rtol=1e-6)
 
 
+def _shaped_scores(scores, cfg, history, position):
+    """The penalised scores behind a shaped distribution at temperature 1 with no truncation: p is the
+    softmax of them, so log p differences give them back."""
+    sup, pr = ob.shaped_distribution(np.array(scores, np.float16), cfg, history, position)
+    got = np.zeros(len(scores))
+    got[sup] = pr
+    return got
+
+
+@pytest.mark.parametrize("scores,history,position,kw,want", [
+    # crates/selection/src/penalty.rs:105-119: a repeated entry is attenuated once; positive scores
+    # divide, negative ones multiply
+    ([4.0, 1.0], [0, 0, 0], 0, dict(repetition_penalty=2.0), [2.0, 1.0]),
+    ([4.0, -4.0], [0, 1], 0, dict(repetition_penalty=2.0), [2.0, -8.0]),
+    # :143-160: presence once whatever the count, frequency per occurrence, both add
+    ([10.0, 7.0], [0, 0, 0], 3, dict(presence_penalty=1.5), [8.5, 7.0]),
+    ([10.0, 7.0], [0, 0, 0], 3, dict(frequency_penalty=1.5), [5.5, 7.0]),
+    ([10.0, 7.0], [0, 0], 2, dict(presence_penalty=1.0, frequency_penalty=0.5), [8.0, 7.0]),
+    ([10.0, 10.0], [0, 0], 2, dict(presence_penalty=1.0, frequency_penalty=1.0), [7.0, 10.0]),
+    # tests/presence_frequency.rs:80-116: a candidate that only appears in the prompt half is untouched
+    ([2.0, 2.0, 2.0, 2.0], [0, 0, 0], 0, dict(presence_penalty=2.0, frequency_penalty=2.0), [2.0, 2.0, 2.0, 2.0]),
+    # choose.rs:147-148: a position beyond the history counts all of it as generated
+    ([2.0, 2.0], [0], 7, dict(presence_penalty=1.5), [0.5, 2.0]),
+    # ids outside the candidate domain are skipped (penalty.rs:27-33)
+    ([3.0, 1.0], [-1, 5, 1], 3, dict(repetition_penalty=2.0, frequency_penalty=0.25), [3.0, 0.25]),
+])
+def test_penalties_reproduce_the_reference_unit_vectors(scores, history, position, kw, want):
+    cfg = ob.shaping(1.0, seed=1, **kw)
+    got = _shaped_scores(scores, cfg, history, position)
+    w = np.array(want, np.float64)
+    ref = np.exp(w - w.max()) / np.exp(w - w.max()).sum()
+    assert np.allclose(got, ref, rtol=1e-12, atol=0)
+
+
 def test_residual_unit_cases():
     # Leviathan worked example
     r = ob.residual(([0, 1], [0.5, 0.5]), ([0], [1.0]))
