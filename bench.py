@@ -289,6 +289,10 @@ def main():
         step(args.warmup + i)
     prof = eng.get_profile()
     eng.set_profile(False)
+    if prof.get("rope_kv", (0.0, 0))[1] == 0:  # the q/k/v projection rotates and stores its own rows: no such launch
+        kern.pop("rope_kv", None)
+        prof.pop("rope_kv", None)
+        kern["qkv"]["epilogue"] = "bias + rotation + fp16 q / KV-cache stores"
     dom = kern.get("gate_up", {})
     peak = 8000.0
     roofline = dict(bound="hbm",

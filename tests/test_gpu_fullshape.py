@@ -56,6 +56,19 @@ def test_llama3_8b_shape_chain_and_tree_at_4096_context():
     res = gpu.accept(feed, ctx, gcfg, draft_logits=draft, draw_step=3)
     ref = ob.chain_round(got, draft, feed[1:], ocfg, history=[0] * ctx + [int(feed[0])], draw_step=3)
     assert (res.accepted, res.committed, res.next, res.draw_step) == (ref["accepted"], ref["committed"], ref["next"], ref["draw_step"])
+    # the same with penalties over a 4097-token history that touches a few thousand vocabulary entries,
+    # a drafter close to the target (so proposals are accepted and later rows count them) and truncation
+    hist = [int(t) for t in rng.integers(0, V, ctx)] + [int(feed[0])]
+    near = (gc.f16(got)[:4] + rng.standard_normal((4, V)).astype(np.float32) * 0.3).astype(np.float16)
+    for seed, kw in enumerate([dict(repetition_penalty=1.3), dict(presence_penalty=0.7, frequency_penalty=0.3, top_p=0.9),
+                               dict(repetition_penalty=1.1, frequency_penalty=0.2, top_k=50, min_p=0.01)]):
+        gcfg, ocfg = ts.shaping(0.8, seed=seed, **kw), ob.shaping(0.8, seed=seed, **kw)
+        props, ds = gpu.draft_chain(near, gcfg, 7, history=hist, generated=600)
+        oprops, ods = ob.draft_chain(near, ocfg, hist, 600, 7)
+        assert list(props) == list(oprops) and ds == ods
+        res = gpu.accept(feed, ctx, gcfg, draft_logits=near, draw_step=3, history=hist, generated=600)
+        ref = ob.chain_round(got, near, feed[1:], ocfg, history=hist, generated=600, draw_step=3)
+        assert (res.accepted, res.committed, res.next, res.draw_step) == (ref["accepted"], ref["committed"], ref["next"], ref["draw_step"])
     # the 16-node tree of configuration 3 on the same cache
     gpu.rollback(point)
     cpu.rewind_to(ctx)
