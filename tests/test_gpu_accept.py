@@ -192,6 +192,30 @@ def test_penalties_change_the_outcome_and_greedy_ignores_them():
     assert (g.accepted, g.next) == (h.accepted, h.next)
 
 
+@pytest.mark.parametrize("kw", [dict(), dict(top_p=0.8), dict(repetition_penalty=1.4, frequency_penalty=0.3)])
+def test_a_round_without_proposals_is_one_draw_from_the_target(kw):
+    """m = 1 (nothing offered: the budget or the context left room for no proposal): the round is the
+    bonus draw from row 0 (speculative.rs:861-879), sampled or arg-max; penalties with an empty
+    history are no-ops (penalty.rs:16-18,66-69)."""
+    import turbospark_amd as ts
+    cfg, gpu, prompt = _setup()
+    V = cfg["vocab"]
+    base = gpu.position
+    point = gpu.checkpoint()
+    none = np.zeros((0, V), np.float16)
+    for seed, hist in enumerate([[], [int(t) for t in prompt] + [9], [9] * 30]):
+        gcfg, ocfg = ts.shaping(0.8, seed=seed, **kw), ob.shaping(0.8, seed=seed, **kw)
+        res, logits = gpu.verify_accept([9], base, gcfg, draft_logits=np.zeros((1, V), np.float16), draw_step=5,
+                                        want_logits=True, history=hist, generated=min(len(hist), 12))
+        want = ob.chain_round(logits, none, [], ocfg, history=hist, generated=min(len(hist), 12), draw_step=5)
+        _same(res, want, base)
+        assert res.accepted == 0 and res.draw_step == 6
+        gpu.rollback(point)
+    res, logits = gpu.verify_accept([9], base, ts.shaping(0.0), want_logits=True)
+    assert res.next == int(np.argmax(gc.f16(logits)[0])) and res.accepted == 0
+    gpu.rollback(point)
+
+
 def test_identical_drafter_is_always_accepted_and_the_bonus_is_a_p_draw():
     import turbospark_amd as ts
     cfg, gpu, prompt = _setup()
