@@ -30,6 +30,26 @@ def test_gptoss_verify_logits_match_the_oracle(ctx, k):
         assert np.abs(vg.astype(np.float32) - vc[:ctx]).max() <= 2e-2 * np.abs(vc[:ctx]).max()
 
 
+def test_projection_biases_and_yarn_with_128_wide_heads():
+    """The same arrangement with 128-wide heads: the fused q/k/v projection then holds the rows of
+    q and k in rotation-pair order (a load-time row map), and its biases, the YaRN table and the K / V
+    cache stores must follow that order (families/gptoss/attn.rs:88-118)."""
+    over = dict(head_dim=128, n_q_heads=4, n_kv_heads=1, hidden=576)
+    cfg, w, gpu, cpu = gc.build_pair("gptoss_small", max_context=96, **over)
+    ctx = 40
+    prompt, feed, want, margin = _clean_inputs(cfg, cpu, ctx, 8)
+    gpu.prefill(prompt, 0, want_logits=False)
+    got = gpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"gptoss_small with 128-wide heads: max-abs logit error / range = {err:.2e}")
+    assert err <= TOL, err
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gpu.read_kv(layer, 0, ctx + 9)
+        kc, vc = cpu.kv(layer)
+        assert np.abs(kg.astype(np.float32) - kc[:ctx + 9]).max() <= 2e-2 * np.abs(kc[:ctx + 9]).max()
+        assert np.abs(vg.astype(np.float32) - vc[:ctx + 9]).max() <= 2e-2 * np.abs(vc[:ctx + 9]).max()
+
+
 def test_gptoss_tree_rows_and_batch_invariance():
     cfg, w, gpu, cpu = gc.build_pair("gptoss_small", max_context=96)
     ctx = 37
