@@ -314,14 +314,19 @@ __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split,
     }
 }
 
+// Tiles in flight per wave.  One: up to eight activation rows then fit 128 VGPRs, so four waves
+// per SIMD are resident instead of two, and inside a verify step (cold L2 and TLB at every launch)
+// that hides more latency than a second register stage does -- the 8B step went from 2.31 to
+// 2.23 ms on the same box, the 16-row tree step from 3.62 to 3.51 ms (there the kernel stays at two
+// waves per SIMD either way), although an isolated launch on warm caches times the same.
 #ifndef TSV_GEMM_STAGES
-#define TSV_GEMM_STAGES 2
+#define TSV_GEMM_STAGES 1
 #endif
 
 template <class F, int EPI, int NG>
 __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     extern __shared__ float4v red[];
-    constexpr int STAGES = NG <= 2 ? TSV_GEMM_STAGES : 2;  // what fits 256 VGPRs at two waves per SIMD
+    constexpr int STAGES = TSV_GEMM_STAGES;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
     // this wave's run of chunks inside the workgroup's K slice
