@@ -1,0 +1,114 @@
+"""Seeded sweep over decoder shapes the verify path accepts: head width, GQA group, hidden / ffn /
+vocabulary sizes that are not round, layer count, context length, rows per pass, chain or random
+tree.  Each case checks the pass's logits and new K/V rows against the oracle's forward
+(families/qwen/batched.rs:92-456 semantics: row i sees the prefix plus its own root path) and then
+one sampled round -- random truncation and penalties -- against the oracle's acceptance on the
+GPU's own logits (speculative.rs:694-754), integers equal."""
+import numpy as np
+import pytest
+
+from oracle import binding as ob
+from tests import gpu_common as gc
+from turbospark_amd import ffi
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed):
+    r = np.random.default_rng(1000 + seed)
+    q4 = bool(r.integers(0, 2))
+    hd = int(r.choice([64, 128]))
+    nkv = int(r.choice([1, 2, 4, 8]))
+    group = int(r.choice([1, 2, 4, 8]))
+    while nkv * group > 32:
+        group //= 2
+    unit = 256 if q4 else 128            # K of a matmul is whole superblocks (Q4_K) / 128-element chunks (Q8_0)
+    hidden = unit * int(r.integers(1, 5 if q4 else 9))
+    while (nkv * group * hd) % unit:     # K of the output projection
+        group *= 2
+    ffn = unit * int(r.integers(1, 7 if q4 else 13))
+    cfg = dict(n_layers=int(r.integers(1, 4)), hidden=hidden, n_q_heads=nkv * group, n_kv_heads=nkv, head_dim=hd, ffn=ffn,
+               vocab=int(r.integers(700, 5000)), rms_eps=1e-5, rope_theta=float(r.choice([10000.0, 500000.0])),
+               dtype=ffi.Q4_K if q4 else ffi.Q8_0, norm_jitter=0.25)
+    ctx = int(r.integers(1, 90))
+    m = int(r.integers(1, 17))
+    tree = bool(r.integers(0, 2)) and m > 2
+    parent = None
+    if tree:
+        parent = [-1] + [int(r.integers(0, s)) for s in range(1, m)]
+    return cfg, ctx, m, parent, r
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_shape(seed):
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg, ctx, m, parent, r = _case(seed)
+    synth.CONFIGS["_random"] = cfg
+    try:
+        cfg, w, gpu, cpu = gc.build_pair("_random", max_context=ctx + 40, seed=77 + seed)
+    finally:
+        del synth.CONFIGS["_random"]
+    V = cfg["vocab"]
+    print(f"seed {seed}: {'q4_k' if cfg['dtype'] == ffi.Q4_K else 'q8_0'} L={cfg['n_layers']} H={cfg['hidden']} "
+          f"q/kv={cfg['n_q_heads']}/{cfg['n_kv_heads']}x{cfg['head_dim']} F={cfg['ffn']} V={V} ctx={ctx} m={m} "
+          f"{'tree' if parent else 'chain'}", flush=True)
+    prompt = r.integers(0, V, ctx).astype(np.int32)
+    feed = r.integers(0, V, m).astype(np.int32)
+    gpu.prefill(prompt, 0, want_logits=False)
+    for i in range(0, ctx, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    tol = gc.TOL[cfg["dtype"]]
+    if parent:
+        got = gpu.verify_tree(feed, parent, ctx)
+    else:
+        got = gpu.verify(feed, ctx)
+    want = cpu.verify(feed, ctx, parent=parent)
+    err = gc.logit_error(got, want)
+    print(f"   max-abs logit error / range = {err:.2e}", flush=True)
+    assert err <= tol, err
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gpu.read_kv(layer, 0, ctx + m)
+        kc, vc = cpu.kv(layer)
+        assert np.abs(kg.astype(np.float32) - kc[:ctx + m]).max() <= 2e-2 * np.abs(kc[:ctx + m]).max()
+        assert np.abs(vg.astype(np.float32) - vc[:ctx + m]).max() <= 2e-2 * np.abs(vc[:ctx + m]).max()
+    # one round of acceptance on these logits
+    kw = {}
+    if r.integers(0, 2):
+        kw["top_k"] = int(r.integers(1, 200))
+    if r.integers(0, 2):
+        kw["top_p"] = float(r.uniform(0.3, 1.0))
+    if r.integers(0, 2):
+        kw["min_p"] = float(r.uniform(0.001, 0.2))
+    temperature = float(r.choice([0.0, 0.6, 1.0, 1.4]))
+    hist = [int(t) for t in prompt] + [int(feed[0])]
+    if parent:
+        draft = (gc.f16(got) + r.standard_normal((m, V)).astype(np.float32) * 0.5).astype(np.float16)
+        gcfg = ts.shaping(temperature, seed=seed if temperature else None, **kw)
+        ocfg = ob.shaping(temperature, seed=seed if temperature else None, **kw)
+        res = gpu.accept(feed, ctx, gcfg, parent=parent, draft_logits=draft if temperature else None, draw_step=11)
+        if temperature:
+            ref = ob.tree_round_sampled(got, draft, feed, parent, ocfg, history=hist[:-1], draw_step=11)
+        else:
+            ref = ob.tree_round_greedy(got, feed, parent, ocfg, history=hist[:-1])
+        assert res.path == ref["path"] and res.next == ref["next"], (res, ref)
+        assert res.draw_step == (ref["draw_step"] if temperature else 11)  # the arg-max walk draws nothing
+        assert gpu.position == ctx + len(ref["path"])
+    else:
+        if r.integers(0, 2):
+            kw["repetition_penalty"] = float(r.uniform(0.8, 1.5))
+        if r.integers(0, 2):
+            kw["presence_penalty"] = float(r.uniform(-0.5, 1.5))
+            kw["frequency_penalty"] = float(r.uniform(-0.2, 0.6))
+        gcfg = ts.shaping(temperature, seed=seed if temperature else None, **kw)
+        ocfg = ob.shaping(temperature, seed=seed if temperature else None, **kw)
+        k = m - 1
+        draft = (gc.f16(got)[:k] + r.standard_normal((k, V)).astype(np.float32) * 0.5).astype(np.float16)
+        generated = int(r.integers(0, len(hist) + 3))
+        res = gpu.accept(feed, ctx, gcfg, draft_logits=draft if temperature else None, draw_step=11, history=hist,
+                         generated=generated, max_new_tokens=generated + 40)
+        ref = ob.chain_round(got, draft if temperature else None, feed[1:], ocfg, history=hist, generated=generated,
+                             max_new_tokens=generated + 40, draw_step=11)
+        assert (res.accepted, res.committed, res.next, res.stopped, res.draw_step) == \
+            (ref["accepted"], ref["committed"], ref["next"], ref["stopped"], ref["draw_step"]), (res, ref)
+        assert gpu.position == ctx + ref["committed"] + 1
