@@ -29,7 +29,7 @@ def _case(seed):
     ffn = unit * int(r.integers(1, 7 if q4 else 13))
     cfg = dict(n_layers=int(r.integers(1, 4)), hidden=hidden, n_q_heads=nkv * group, n_kv_heads=nkv, head_dim=hd, ffn=ffn,
                vocab=int(r.integers(700, 5000)), rms_eps=1e-5, rope_theta=float(r.choice([10000.0, 500000.0])),
-               dtype=ffi.Q4_K if q4 else ffi.Q8_0, norm_jitter=0.25)
+               dtype=ffi.Q4_K if q4 else ffi.Q8_0, norm_jitter=0.25, qk_norm=bool(r.integers(0, 2)))
     ctx = int(r.integers(1, 90))
     m = int(r.integers(1, 17))
     tree = bool(r.integers(0, 2)) and m > 2
@@ -52,7 +52,7 @@ def test_random_shape(seed):
     V = cfg["vocab"]
     print(f"seed {seed}: {'q4_k' if cfg['dtype'] == ffi.Q4_K else 'q8_0'} L={cfg['n_layers']} H={cfg['hidden']} "
           f"q/kv={cfg['n_q_heads']}/{cfg['n_kv_heads']}x{cfg['head_dim']} F={cfg['ffn']} V={V} ctx={ctx} m={m} "
-          f"{'tree' if parent else 'chain'}", flush=True)
+          f"{'tree' if parent else 'chain'}{' qk-norm' if cfg['qk_norm'] else ''}", flush=True)
     prompt = r.integers(0, V, ctx).astype(np.int32)
     feed = r.integers(0, V, m).astype(np.int32)
     gpu.prefill(prompt, 0, want_logits=False)
@@ -112,3 +112,56 @@ def test_random_shape(seed):
         assert (res.accepted, res.committed, res.next, res.stopped, res.draw_step) == \
             (ref["accepted"], ref["committed"], ref["next"], ref["stopped"], ref["draw_step"]), (res, ref)
         assert gpu.position == ctx + ref["committed"] + 1
+
+
+def _moe_case(seed):
+    r = np.random.default_rng(5000 + seed)
+    oss = bool(r.integers(0, 2))
+    hd = int(r.choice([64, 128]))
+    nkv = int(r.choice([1, 2, 4]))
+    group = int(r.choice([1, 2, 4, 8]))
+    hidden = 64 * int(r.integers(3, 13))           # MXFP4 / bf16 widths need not be whole 256-element chunks
+    if not oss:
+        hidden = 128 * int(r.integers(2, 7))       # Q8_0 attention: whole 128-element chunks
+        while (nkv * group * hd) % 128:
+            group *= 2
+    n_experts = int(r.choice([4, 8, 16]))
+    cfg = dict(n_layers=int(r.integers(1, 4)), hidden=hidden, n_q_heads=nkv * group, n_kv_heads=nkv, head_dim=hd,
+               ffn=32 * int(r.integers(2, 13)), n_experts=n_experts, top_k=int(r.choice([1, 2, 4])),
+               vocab=int(r.integers(700, 4000)), rms_eps=1e-6, rope_theta=150000.0,
+               dtype=ffi.BF16 if oss else ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08, norm_jitter=0.25)
+    cfg["qk_norm"] = not oss and bool(r.integers(0, 2))
+    if oss:
+        cfg["attn_scale"] = float(r.choice([0.125, 0.1]))
+        cfg["gptoss"] = dict(window=int(r.integers(17, 60)), yarn=(32.0, 64, 32.0, 1.0), act_alpha=1.702, act_limit=7.0)
+    return cfg, int(r.integers(1, 40)), int(r.integers(0, 16)), r
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_routed_expert_shape(seed):
+    """The same sweep over routed-expert decoders (families/llama/moe.rs:1-17, families/gptoss/mod.rs:11-23):
+    expert count, top-k, widths that are not whole chunks, and for the gpt-oss arrangement a random
+    window, biases, sinks and YaRN.  Inputs whose routing is a near tie in the oracle are skipped by
+    re-drawing (the GPU's router logits carry fp16-activation rounding)."""
+    from turbospark_amd import synth
+    from tests.test_gpu_moe import _clean_inputs
+    cfg, ctx, k, r = _moe_case(seed)
+    synth.CONFIGS["_random"] = cfg
+    try:
+        cfg, w, gpu, cpu = gc.build_pair("_random", max_context=ctx + 40, seed=31 + seed)
+    finally:
+        del synth.CONFIGS["_random"]
+    print(f"seed {seed}: {'gpt-oss' if cfg.get('gptoss') else 'qwen-moe'} L={cfg['n_layers']} H={cfg['hidden']} "
+          f"q/kv={cfg['n_q_heads']}/{cfg['n_kv_heads']}x{cfg['head_dim']} F={cfg['ffn']} E={cfg['n_experts']} top{cfg['top_k']} "
+          f"V={cfg['vocab']} ctx={ctx} m={k + 1}{' qk-norm' if cfg['qk_norm'] else ''}", flush=True)
+    prompt, feed, want, margin = _clean_inputs(cfg, cpu, ctx, k, floor=1e-3)
+    gpu.prefill(prompt, 0, want_logits=False)
+    got = gpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"   max-abs logit error / range = {err:.2e}, route margin {margin:.2e}", flush=True)
+    assert err <= 1e-2, err
+    for layer in range(cfg["n_layers"]):
+        kg, vg = gpu.read_kv(layer, 0, ctx + k + 1)
+        kc, vc = cpu.kv(layer)
+        assert np.abs(kg.astype(np.float32) - kc[:ctx + k + 1]).max() <= 2e-2 * np.abs(kc[:ctx + k + 1]).max()
+        assert np.abs(vg.astype(np.float32) - vc[:ctx + k + 1]).max() <= 2e-2 * np.abs(vc[:ctx + k + 1]).max()

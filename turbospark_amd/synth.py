@@ -24,9 +24,10 @@ CONFIGS = {
     "xcd_q8_0": dict(n_layers=2, hidden=1024, n_q_heads=16, n_kv_heads=8, head_dim=64, ffn=1024,
                      vocab=4096, rms_eps=1e-5, rope_theta=10000.0, dtype=ffi.Q8_0, norm_jitter=0.25),
     # a small routed-expert decoder in the arrangement of the Qwen3-30B-A3B configuration: Q8_0
-    # attention and router, MXFP4 experts, top-k routing with softmax over the selected logits
+    # attention and router, per-head q / k RMSNorm, MXFP4 experts, top-k routing with softmax over the
+    # selected logits
     "moe_small": dict(n_layers=2, hidden=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=256,
-                      n_experts=16, top_k=4, vocab=4096, rms_eps=1e-6, rope_theta=1000000.0,
+                      n_experts=16, top_k=4, vocab=4096, rms_eps=1e-6, rope_theta=1000000.0, qk_norm=True,
                       dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08, norm_jitter=0.25),
     # a small decoder in the arrangement of the gpt-oss configuration: bf16 attention / router / head
     # with projection biases, attention sinks, a sliding window on even layers, YaRN rotation,
@@ -43,7 +44,7 @@ CONFIGS = {
                         gptoss=dict(window=128, yarn=(32.0, 4096, 32.0, 1.0), act_alpha=1.702, act_limit=7.0)),
     # Qwen3-30B-A3B shape: 128 experts, top-8, MXFP4 experts, Q8_0 attention / router / head
     "qwen3_30b_a3b": dict(n_layers=48, hidden=2048, n_q_heads=32, n_kv_heads=4, head_dim=128, ffn=768,
-                          n_experts=128, top_k=8, vocab=151936, rms_eps=1e-6, rope_theta=1000000.0,
+                          n_experts=128, top_k=8, vocab=151936, rms_eps=1e-6, rope_theta=1000000.0, qk_norm=True,
                           dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08),
     # Llama-3-8B shape
     "llama3_8b_q4_k": dict(n_layers=32, hidden=4096, n_q_heads=32, n_kv_heads=8, head_dim=128,
@@ -95,6 +96,8 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
     for li in range(L):
         lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H, name=(li, "wv")), wo=t(H, qd),
                   ffn_norm=ones(H))
+        if cfg.get("qk_norm"):  # Qwen3: RMSNorm over each q / k head before the rotation
+            lw.update(q_norm=ones(cfg["head_dim"]), k_norm=ones(cfg["head_dim"]))
         if E:
             xd = cfg.get("expert_dtype", dt)
             lw.update(n_experts=E, top_k=int(cfg["top_k"]), router=t(E, H, sig=cfg.get("router_sigma", sigma)),
