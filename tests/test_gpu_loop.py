@@ -94,3 +94,45 @@ def test_the_loop_stays_inside_the_context_window_and_refuses_bad_requests():
                                 args["block"])
     with pytest.raises(ts.TsvError, match="empty"):
         gpu.run_speculative([], LmDrafter(GpuTarget(lm), 0, V), ts.shaping(0.0), 4, 2)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_generation_settings(seed):
+    """Seeded sweep over the loop's settings: temperature, truncation, penalties, block, adaptive floor,
+    drafter quality, budget, prompt length, and a stop token drawn from the vocabulary's frequent ids
+    (so that some runs end on it and some on the budget)."""
+    import turbospark_amd as ts
+    r = np.random.default_rng(900 + seed)
+    cfg, gpu, lm = _pair(draft_seed=1234)
+    V = cfg["vocab"]
+    temperature = float(r.choice([0.0, 0.5, 0.9, 1.2]))
+    kw = {}
+    if r.integers(0, 2):
+        kw["top_k"] = int(r.integers(2, 120))
+    if r.integers(0, 2):
+        kw["top_p"] = float(r.uniform(0.5, 1.0))
+    if r.integers(0, 2):
+        kw["min_p"] = float(r.uniform(0.001, 0.1))
+    if r.integers(0, 2):
+        kw["repetition_penalty"] = float(r.uniform(0.9, 1.6))
+    if r.integers(0, 2):
+        kw["presence_penalty"] = float(r.uniform(0.0, 1.5))
+        kw["frequency_penalty"] = float(r.uniform(0.0, 0.8))
+    block = int(r.integers(1, 16))
+    floor = int(r.integers(0, min(block, 3) + 1))
+    noise = float(r.choice([0.0, 0.3, 1.0]))
+    new = int(r.integers(5, 60))
+    prompt = r.integers(0, V, int(r.integers(1, 40))).astype(np.int32)
+    sd = 7 + seed if temperature else None
+    gcfg, ocfg = ts.shaping(temperature, seed=sd, **kw), ob.shaping(temperature, seed=sd, **kw)
+    print(f"seed {seed}: T={temperature} {kw} block={block} floor={floor} noise={noise} budget={new} prompt={len(prompt)}", flush=True)
+    free = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), gcfg, new, block, adaptive_floor=floor)
+    stops = [int(free["tokens"][len(free["tokens"]) // 2]), int(r.integers(0, V))]
+    for stop_tokens in ([], stops):
+        want = ob.run_speculative(GpuTarget(gpu), LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), prompt, ocfg, new, block,
+                                  V, cfg["max_context"], stop_tokens=stop_tokens, adaptive_floor=floor)
+        got = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V, noise, 9), gcfg, new, block,
+                                  stop_tokens=stop_tokens, adaptive_floor=floor)
+        assert {k: got[k] for k in KEYS} == {k: want[k] for k in KEYS}
+        assert got["min_margin"] > 1e-10
+    assert got["stop_reason"] == 1 and got["tokens"] == free["tokens"][: free["tokens"].index(stops[0])]
