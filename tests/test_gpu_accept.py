@@ -299,7 +299,10 @@ def test_greedy_tree_round_walks_compacts_and_truncates():
 
 
 @pytest.mark.parametrize("name,temperature,kw", [("tiny_q8_0", 1.0, {}), ("small_q4_k", 0.8, {}),
-                                                 ("tiny_q8_0", 1.0, dict(top_k=64, top_p=0.9))])
+                                                 ("tiny_q8_0", 1.0, dict(top_k=64, top_p=0.9)),
+                                                 ("tiny_q8_0", 1.0, dict(repetition_penalty=1.3, presence_penalty=0.5,
+                                                                         frequency_penalty=0.2)),
+                                                 ("small_q4_k", 0.8, dict(repetition_penalty=1.15, top_p=0.9, min_p=0.01))])
 def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature, kw):
     """Multi-branch rejection over a 16-node tree.  The rule is the oracle's own (the reference
     keeps tree rounds greedy, speculative.rs:390-392), so this pins the device against the
@@ -327,8 +330,12 @@ def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature, kw)
             draft = gc.f16(logits).copy()      # q == p: the first child of every node is accepted
         seed = 500 + rnd
         gcfg, ocfg = ts.shaping(temperature, seed=seed, **kw), ob.shaping(temperature, seed=seed, **kw)
-        res = gpu.accept(feed, base, gcfg, parent=parent, draft_logits=draft, draw_step=7 * rnd)
-        want = ob.tree_round_sampled(logits, draft, feed, parent, ocfg, history=list(prompt), draw_step=7 * rnd)
+        # (with penalties every node is shaped with the history of its own root path; the history
+        # handed over holds the likely children, so the penalties bite where decisions are made)
+        hist = list(prompt) + [int(t) for t in likely[:5]] + [9]
+        res = gpu.accept(feed, base, gcfg, parent=parent, draft_logits=draft, draw_step=7 * rnd, history=hist,
+                         generated=6)
+        want = ob.tree_round_sampled(logits, draft, feed, parent, ocfg, history=hist, generated=6, draw_step=7 * rnd)
         assert res.path == want["path"], (rnd, res, want)
         assert (res.accepted, res.committed, res.next, res.draw_step, res.stopped) == \
             (want["accepted"], want["committed"], want["next"], want["draw_step"], 0), (rnd, res, want)
@@ -340,7 +347,7 @@ def test_sampled_tree_rounds_match_the_oracle_bit_for_bit(name, temperature, kw)
         gpu.rollback(point)
     print("accepted depth per round:", depths, " min margin:", min(margins))
     assert min(margins) > 1e-9
-    if not kw:  # (random deeper nodes fall outside both truncated sets, where 0 <= 0 accepts)
+    if not (kw.get("top_k") or kw.get("top_p")):  # (random deeper nodes fall outside both truncated sets, where 0 <= 0 accepts)
         assert len(set(depths)) > 2
     # the compacted cache continues like a chain that fed the accepted path
     feed = [int(t) for t in rng.integers(0, V, 16)]
@@ -364,10 +371,6 @@ def test_refusals_by_name():
     from turbospark_amd import TsvError
     cfg, gpu, prompt = _setup()
     base = gpu.position
-    with pytest.raises(TsvError, match="not built"):  # penalties over a sampled tree
-        gpu.verify_accept([1, 2, 3], base, ts.shaping(0.8, repetition_penalty=1.1, seed=1), parent=[-1, 0, 0],
-                          draft_logits=np.zeros((3, cfg["vocab"]), np.float16), history=[1, 2])
-    assert gpu.position == base
     with pytest.raises(TsvError, match="seed"):
         gpu.verify_accept([1, 2], base, ts.shaping(0.8), draft_logits=np.zeros((1, cfg["vocab"]), np.float16))
     with pytest.raises(TsvError, match="drafter"):

@@ -82,29 +82,30 @@ def test_random_shape(seed):
         kw["min_p"] = float(r.uniform(0.001, 0.2))
     temperature = float(r.choice([0.0, 0.6, 1.0, 1.4]))
     hist = [int(t) for t in prompt] + [int(feed[0])]
+    if temperature and r.integers(0, 2):
+        kw["repetition_penalty"] = float(r.uniform(0.8, 1.5))
+    if temperature and r.integers(0, 2):
+        kw["presence_penalty"] = float(r.uniform(-0.5, 1.5))
+        kw["frequency_penalty"] = float(r.uniform(-0.2, 0.6))
+    generated = int(r.integers(0, len(hist) + 3))
     if parent:
         draft = (gc.f16(got) + r.standard_normal((m, V)).astype(np.float32) * 0.5).astype(np.float16)
         gcfg = ts.shaping(temperature, seed=seed if temperature else None, **kw)
         ocfg = ob.shaping(temperature, seed=seed if temperature else None, **kw)
-        res = gpu.accept(feed, ctx, gcfg, parent=parent, draft_logits=draft if temperature else None, draw_step=11)
+        res = gpu.accept(feed, ctx, gcfg, parent=parent, draft_logits=draft if temperature else None, draw_step=11,
+                         history=hist, generated=generated)
         if temperature:
-            ref = ob.tree_round_sampled(got, draft, feed, parent, ocfg, history=hist[:-1], draw_step=11)
+            ref = ob.tree_round_sampled(got, draft, feed, parent, ocfg, history=hist, generated=generated, draw_step=11)
         else:
             ref = ob.tree_round_greedy(got, feed, parent, ocfg, history=hist[:-1])
         assert res.path == ref["path"] and res.next == ref["next"], (res, ref)
         assert res.draw_step == (ref["draw_step"] if temperature else 11)  # the arg-max walk draws nothing
         assert gpu.position == ctx + len(ref["path"])
     else:
-        if r.integers(0, 2):
-            kw["repetition_penalty"] = float(r.uniform(0.8, 1.5))
-        if r.integers(0, 2):
-            kw["presence_penalty"] = float(r.uniform(-0.5, 1.5))
-            kw["frequency_penalty"] = float(r.uniform(-0.2, 0.6))
         gcfg = ts.shaping(temperature, seed=seed if temperature else None, **kw)
         ocfg = ob.shaping(temperature, seed=seed if temperature else None, **kw)
         k = m - 1
         draft = (gc.f16(got)[:k] + r.standard_normal((k, V)).astype(np.float32) * 0.5).astype(np.float16)
-        generated = int(r.integers(0, len(hist) + 3))
         res = gpu.accept(feed, ctx, gcfg, draft_logits=draft if temperature else None, draw_step=11, history=hist,
                          generated=generated, max_new_tokens=generated + 40)
         ref = ob.chain_round(got, draft if temperature else None, feed[1:], ocfg, history=hist, generated=generated,

@@ -128,7 +128,8 @@ __device__ __forceinline__ double prob_of(uint16_t bits, int v, const RowStat& s
 // generated suffix.  `pen_cnt[v]` holds, for the history the round started with, bit 31 = seen and
 // the low bits = occurrences in the generated suffix; target row i of a chain round adds the i
 // proposals committed before it was judged (speculative.rs:694-716: each accepted proposal goes
-// through the sink before the next row is shaped), drafter rows add nothing (speculative.rs:636-641).
+// through the sink before the next row is shaped) -- in general the tokens on the row's root path,
+// which is the same rule for a tree node -- and drafter rows add nothing (speculative.rs:636-641).
 //
 // A penalised score is an f32 that need not be an fp16 value.  Its rank bin is the bin of the
 // largest fp16 value not above it, so bins stay ordered; inside a bin the candidates with a score
@@ -141,9 +142,9 @@ __device__ __forceinline__ float score_of(const AcceptParams& ap, int row, int v
         const uint32_t c = ap.pen_cnt[v];
         bool seen = (c >> 31) != 0;
         uint32_t gen = c & 0x7FFFFFFFu;
-        const int extra = row < ap.m ? row : 0;
-        for (int j = 0; j < extra; j++)
-            if (ap.feed[j + 1] == v) {
+        // the tokens committed on the way to this row: its root path without the root (chain: rows 1..row)
+        for (int s = row < ap.m ? row : 0; s > 0; s = ap.parent[s])
+            if (ap.feed[s] == v) {
                 seen = true;
                 gen += 1;
             }
@@ -617,13 +618,12 @@ __device__ int collect_side(const AcceptParams& ap, int row, const uint16_t* lp,
                             SideEnt* sorted, int* counter, int32_t* err) {
     const int tid = threadIdx.x;
     const float g = h2f((uint16_t)key_bits(bin));
-    const int extra = row < ap.m ? row : 0;
     __syncthreads();
     if (tid == 0) *counter = 0;
     __syncthreads();
     for (int v = tid; v < ap.vocab; v += 1024) {
         bool flagged = ap.pen_cnt[v] != 0;
-        for (int j = 0; j < extra; j++) flagged |= ap.feed[j + 1] == v;
+        for (int s = row < ap.m ? row : 0; s > 0; s = ap.parent[s]) flagged |= ap.feed[s] == v;
         if (!flagged) continue;  // an untouched score is an fp16 value: on its bin's value
         const float w = score_of<true>(ap, row, v, lp[v]);
         if (w != g && (int)rank_key(floor16(w)) == bin) {
@@ -1074,6 +1074,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
 // 0..m-1 and m..2m-1); then one workgroup walks the tree.  A child test is two lookups; only a
 // rejection costs a pass over the vocabulary (slots 32 and 33 alternate as the residual, whose
 // normalising division is applied when it is read, so a pass reads two rows and writes one).
+template <bool PEN>
 __global__ __launch_bounds__(256) void k_tree_probs(const uint16_t* target, const uint16_t* draft,
                                                     const AcceptParams* app, double* scratch, double* work) {
     __shared__ RowStat st;
@@ -1085,16 +1086,22 @@ __global__ __launch_bounds__(256) void k_tree_probs(const uint16_t* target, cons
         if (threadIdx.x == 0) st = s0;
     }
     __syncthreads();
-    const RowStat s0 = st;
+    RowStat s0 = st;
+    if (PEN && ap.has_min_p) s0.minp = ap.min_p;
     const double inv_t = 1.0 / ap.temperature;
     const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, row);
     double* out = work + (long)row * vocab;
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
-    for (int v = v0 + threadIdx.x; v < v1; v += 256) out[v] = prob_of(lp[v], v, s0, inv_t);
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const uint16_t b = lp[v];
+        const float w = score_of<PEN>(ap, row, v, b);
+        out[v] = prob_of_w<PEN>(w, (int)key_of<PEN>(w, b), v, s0, inv_t);
+    }
 }
 
 constexpr int TREE_SCRATCH_SLOT = 2 * TSV_MAX_ROWS;  // two residual rows behind the 32 distribution rows
 
+template <bool PEN>
 __global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, const AcceptParams* app,
                                                        double* scratch, double* work, unsigned long long* hist,
                                                        Decision* dec_out, int32_t* path_out) {
@@ -1164,7 +1171,10 @@ __global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, c
         const uint16_t* lpk = target + (long)at * vocab;
         for (int v = tid; v < vocab; v += 1024) {
             const double mv = src[v] / Z;
-            if (mv > 0.0) atomicAdd(hr + bin_addr(rank_key(lpk[v])), (unsigned long long)(mv * FIX));
+            if (mv > 0.0) {
+                const uint16_t b = lpk[v];
+                atomicAdd(hr + bin_addr(key_of<PEN>(score_of<PEN>(ap, at, v, b), b)), (unsigned long long)(mv * FIX));
+            }
         }
         // the draw divides the stored values by the fold of these pieces: Z, exactly
         if (tid < NSEG * NSUB) L.segtot[tid] = tid == 0 ? Z : 0.0;
@@ -1340,6 +1350,20 @@ static void launch_chain_sampled(hipStream_t s, const uint16_t* target, const ui
 }
 
 template <bool PEN>
+static void launch_tree_sampled(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
+                                const AcceptParams& ap, const AcceptScratch& sc) {
+    int32_t* err = (int32_t*)sc.counters;
+    int32_t* path = (int32_t*)sc.counters + 32;
+    // statistics of the m target rows and the m rows the children were drawn from
+    launch_stats<PEN>(s, target, draft, ap.m, 2 * ap.m, 2 * 65536, ap_dev, ap, sc);
+    hipLaunchKernelGGL(k_tree_probs<PEN>, dim3(NSEG, 2 * ap.m), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
+    hipLaunchKernelGGL(k_tree_sampled<PEN>, dim3(1), dim3(1024), 0, s, target, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), path);
+    hipLaunchKernelGGL(k_pick<PEN>, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);
+}
+
+template <bool PEN>
 static void launch_draft_sampled(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,
                                  const AcceptParams& ap, const AcceptScratch& sc, int32_t* proposals_dev) {
     int32_t* err = (int32_t*)sc.counters;
@@ -1362,18 +1386,10 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
         return TSV_OK;
     }
     if (ap.tree) {
-        if (ap.pen) {
-            set_error("device acceptance: penalties are not built for a sampled tree round");
-            return TSV_ERR_UNSUPPORTED;
-        }
-        // statistics of the m target rows and the m rows the children were drawn from
-        int32_t* path = (int32_t*)sc.counters + 32;
-        launch_stats<false>(s, target, draft, ap.m, 2 * ap.m, 2 * 65536, ap_dev, ap, sc);
-        hipLaunchKernelGGL(k_tree_probs, dim3(NSEG, 2 * ap.m), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
-        hipLaunchKernelGGL(k_tree_sampled, dim3(1), dim3(1024), 0, s, target, ap_dev, sc.stats, sc.work,
-                           (unsigned long long*)sc.hist, decisions(sc), path);
-        hipLaunchKernelGGL(k_pick<false>, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
-                           (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);
+        if (ap.pen)
+            launch_tree_sampled<true>(s, target, draft, ap_dev, ap, sc);
+        else
+            launch_tree_sampled<false>(s, target, draft, ap_dev, ap, sc);
         TSV_HIP(hipGetLastError());
         return TSV_OK;
     }

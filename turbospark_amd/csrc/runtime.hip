@@ -1202,10 +1202,6 @@ int stage_draft(tsv_ctx* c, const uint16_t* draft, int rows, const uint16_t** de
 int check_round(const tsv_round* r) {
     int rc = check_shaping(r->shaping, true);
     if (rc) return rc;
-    if (r->parent && has_penalties(r->shaping)) {
-        set_error("device acceptance: penalties are not built for a sampled tree round");
-        return TSV_ERR_UNSUPPORTED;
-    }
     return TSV_OK;
 }
 
