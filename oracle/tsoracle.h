@@ -16,6 +16,10 @@
  *   - attention, rms_norm .............. closed-form small cases and brute-force restatements
  *   - whole fp32 Llama-style forward ... MLX known-answer logits (three fixtures), 2e-4
  *   - residual, shaped distribution .... the reference's exact unit cases; brute-force enumeration
+ *   - penalties ........................ the reference's unit vectors (attenuated once per distinct id,
+ *                                        divide / multiply by sign, presence once, frequency per
+ *                                        occurrence, both additive, prompt-only ids untouched, ids
+ *                                        outside the domain skipped, position beyond the history)
  *   - greedy tree walk ................. the reference's unit case
  *   - mix / derive_step_value .......... the published splitmix64 output vectors (the reference
  *                                        only tests invariants; its mixer is that textbook routine)
@@ -37,7 +41,8 @@
  * PARITY UNPINNED (no golden value exists anywhere in the reference):
  *   - tso_tree_round_sampled: multi-branch rejection sampling on a tree is not
  *     defined by the reference at all; the definition here is this project's own
- *     (checked only against the chain round on chain-shaped trees and in law).
+ *     (checked only against the chain round on chain-shaped trees and in law).  With penalties
+ *     a node is shaped with the history of its own root path, the chain round's rule.
  *   - tso_quantize_mxfp4: the reference has no MXFP4 encoder; checked by brute force
  *     against "nearest codebook value under the tightest covering exponent".
  */

@@ -17,7 +17,7 @@
 // Bin masses are accumulated as 2^-62 fixed point with integer atomics: order independent,
 // hence bit-reproducible run to run.
 //
-// Repetition / presence / frequency penalties (sampled chain rounds and the draft draws) are
+// Repetition / presence / frequency penalties (sampled chain and tree rounds, the draft draws) are
 // applied per candidate as it is read, from a per-token table of the history (see score_of);
 // the kernels are compiled twice, and the variant without penalties is the code it always was.
 #include "tsv_internal.h"
