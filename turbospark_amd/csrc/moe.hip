@@ -105,10 +105,15 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
 }
 
 // ---- grouped expert matmul --------------------------------------------------------------------
+
 __device__ __forceinline__ float silu_moe(float x) { return x / (1.0f + __expf(-x)); }
 
 // One 64-row weight tile of expert `e` against up to four of the group's rows (r0 .. r0 + 3).
-template <class F, int EPI>
+// STAGES: tiles in flight per wave.  Two when a wave has at most two K chunks to walk (both are then
+// requested at once); one otherwise (90-100 VGPRs instead of 150-230, so twice the resident waves,
+// which is worth more over a longer walk): the 120B-shaped step 5.86 -> 5.24 ms, the 30B-shaped one
+// 4.43 ms either way.
+template <class F, int EPI, int STAGES>
 __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup& grp, int gi, int r0, float4v* red) {
     constexpr int NG = 1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -131,29 +136,29 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
 
     float4v acc[NG] = {float4v{0.f, 0.f, 0.f, 0.f}};
     if (nc > 0) {
-        Stage<F, NG> st[2];
+        Stage<F, NG> st[STAGES];
         const int last = c0 + nc - 1;
         auto fetch = [&](Stage<F, NG>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
-        fetch(st[0], c0);
-        fetch(st[1], min(c0 + 1, last));
-        int c = 0;
-        for (; c + 4 <= nc; c += 2) {
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
+        for (int s = 0; s < STAGES; s++) fetch(st[s], min(c0 + s, last));
+        int c = 0;
+        for (; c + 2 * STAGES <= nc; c += STAGES) {
+#pragma unroll
+            for (int s = 0; s < STAGES; s++) {
                 compute(st[s], k, acc);
-                fetch(st[s], c0 + c + s + 2);
+                fetch(st[s], c0 + c + s + STAGES);
             }
         }
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
+        for (int s = 0; s < STAGES; s++) {
             if (c + s < nc) {
                 compute(st[s], k, acc);
-                if (c + s + 2 < nc) fetch(st[s], c0 + c + s + 2);
+                if (c + s + STAGES < nc) fetch(st[s], c0 + c + s + STAGES);
             }
         }
-        c += 2;
+        c += STAGES;
 #pragma unroll
-        for (int s = 0; s < 2; s++)
+        for (int s = 0; s < STAGES; s++)
             if (c + s < nc) compute(st[s], k, acc);
     }
 
@@ -211,7 +216,7 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
 // grid: (tiles per expert, rows x top_k groups).  Groups that repeat an earlier expert leave at
 // once.  An expert chosen by more than four rows (rare at these batch widths) is multiplied in
 // several sweeps of four rows; its tile then comes from L2.
-template <class F, int EPI>
+template <class F, int EPI, int STAGES>
 __global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
     extern __shared__ float4v red[];
     __shared__ MoeGroup grp;
@@ -219,19 +224,24 @@ __global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
     if (threadIdx.x < sizeof(MoeGroup) / 4) ((int32_t*)&grp)[threadIdx.x] = ((const int32_t*)(a.groups + gi))[threadIdx.x];
     __syncthreads();
     if (grp.cnt == 0) return;
-    for (int r0 = 0; r0 < grp.cnt; r0 += 4) expert_tile<F, EPI>(a, grp, gi, r0, red);
+    for (int r0 = 0; r0 < grp.cnt; r0 += 4) expert_tile<F, EPI, STAGES>(a, grp, gi, r0, red);
 }
 
 template <class F, int EPI>
 int launch_moe_t(hipStream_t s, const MoeGemmArgs& a, int n_groups) {
-    // waves per workgroup: each takes `cpw` K chunks of the tile
-    static const int cpw = [] {
+    // waves per workgroup: about four, each with at least two K chunks of the tile to walk (measured on
+    // the two routed configurations: 12 chunks -> 4 waves x 3, 8 chunks -> 4 x 2, 3 chunks -> 2 waves)
+    static const int forced = [] {
         const char* e = getenv("TSV_MOE_CPW");
-        return e ? std::max(1, atoi(e)) : 2;
+        return e ? std::max(1, atoi(e)) : 0;
     }();
+    const int cpw = forced ? forced : std::max(2, (a.kchunks + 3) / 4);
     const int nw = std::min(8, std::max(1, (a.kchunks + cpw - 1) / cpw));
     const size_t lds = (size_t)nw * 1024;
-    hipLaunchKernelGGL((k_moe_gemm<F, EPI>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);
+    if ((a.kchunks + nw - 1) / nw <= 2)
+        hipLaunchKernelGGL((k_moe_gemm<F, EPI, 2>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);
+    else
+        hipLaunchKernelGGL((k_moe_gemm<F, EPI, 1>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
