@@ -167,6 +167,10 @@ void* tsv_stream(tsv_ctx* ctx);
 /* ---- LogitProducer (producer.rs:17-104) ------------------------------------ */
 int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset */
 int64_t tsv_kv_position(const tsv_ctx* ctx);   /* kv.position() */
+/* KvCacheManager::max_safe_rewind (crates/gpu/src/kv_cache_rewind.rs:26-35): how many rows a rollback
+ * may drop.  INT64_MAX here: every layer, windowed ones included, stores position p at slot p, so
+ * "nothing rings" and any rewind down to position 0 is safe. */
+int64_t tsv_max_safe_rewind(const tsv_ctx* ctx);
 /* LogitProducer::produce: one token at `position`; logits: vocab fp16. */
 int32_t tsv_produce(tsv_ctx* ctx, int32_t token, int64_t position, uint16_t* logits);
 /* produce_prefill / ChunkedPrefillRunner::prefill_chunk: feeds n tokens from pos0 in

@@ -89,3 +89,23 @@ def test_gptoss_sampled_round_on_the_device():
             (want["accepted"], want["committed"], want["next"], want["draw_step"])
         assert res.min_margin > 1e-9
         gpu.rollback(ts.ffi.Point(base))
+
+
+def test_a_rewind_deeper_than_the_window_is_safe_in_the_linear_layout():
+    """`KvCacheManager::max_safe_rewind` (crates/gpu/src/kv_cache_rewind.rs:26-35) bounds a rollback by
+    the ring's slack; the windowed layers here store position p at slot p, so it is unbounded: after
+    rolling back 40 rows (the window is 24) the continuation equals, by bits, a run that never went
+    further."""
+    import turbospark_amd as ts
+    cfg, w, gpu, cpu = gc.build_pair("gptoss_small", max_context=128)
+    assert gpu.max_safe_rewind() == 2 ** 63 - 1
+    prompt = _prompt(80, cfg["vocab"], 5)
+    tail = _prompt(6, cfg["vocab"], 6)
+    gpu.prefill(prompt, 0, want_logits=False)
+    gpu.rollback(ts.ffi.Point(40))
+    assert gpu.position == 40
+    a = gpu.verify(tail, 40)
+    gpu.reset()
+    gpu.prefill(prompt[:40], 0, want_logits=False)
+    b = gpu.verify(tail, 40)
+    assert np.array_equal(a, b)

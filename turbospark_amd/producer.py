@@ -87,6 +87,10 @@ class HipVerifier:
     def position(self):
         return ffi.lib().tsv_kv_position(self._h)
 
+    def max_safe_rewind(self):
+        """`KvCacheManager::max_safe_rewind`: unbounded (2**63 - 1), the cache is linear in every layer."""
+        return ffi.lib().tsv_max_safe_rewind(self._h)
+
     @property
     def stream(self):
         """The hipStream_t (as an integer) every kernel of this handle runs on."""
