@@ -235,6 +235,10 @@ typedef struct {
     int32_t (*prime)(void* user, int32_t next_token, int64_t position);
     int32_t (*step)(void* user, int32_t token, int64_t position, uint16_t* logits);
     int32_t (*rewind)(void* user, int64_t position);
+    /* non-zero: `step` is handed DEVICE memory (a buffer of the loop's) and fills it on the GPU, finished
+     * by the time it returns; the draws and the round then read the drafter's rows where they are.  No
+     * counterpart in the reference, whose draft_step hands back host logits (producer.rs:196-204). */
+    int32_t device_logits;
 } tsv_drafter;
 
 typedef struct {
@@ -263,6 +267,10 @@ typedef struct {
  * rewind_drafter, never proposing past the budget or the context window (speculative.rs:448-459). */
 int32_t tsv_run_speculative(tsv_ctx* ctx, const tsv_drafter* drafter, const int32_t* prompt, int64_t n_prompt,
                             const tsv_generation* config, tsv_generation_result* out);
+/* Device address of the logits the last pass left on the GPU (rows x vocab fp16, valid until the next
+ * pass of this handle, written on tsv_stream): lets a second handle be the drafter of a loop without a
+ * host round trip. */
+const uint16_t* tsv_device_logits(tsv_ctx* ctx);
 int64_t tsv_max_context(const tsv_ctx* ctx);
 int64_t tsv_vocab(const tsv_ctx* ctx);
 

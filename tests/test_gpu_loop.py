@@ -136,3 +136,37 @@ def test_random_generation_settings(seed):
         assert {k: got[k] for k in KEYS} == {k: want[k] for k in KEYS}
         assert got["min_margin"] > 1e-10
     assert got["stop_reason"] == 1 and got["tokens"] == free["tokens"][: free["tokens"].index(stops[0])]
+
+
+class DeviceLmDrafter(LmDrafter):
+    """The same drafter leaving its logits on the GPU: a pass of the drafter's own handle, then a
+    device-to-device copy into the row the loop hands over."""
+
+    def step_device(self, token, position, address):
+        import ctypes as C
+        from turbospark_amd import hip
+        idx = position + 1
+        if self.pos == 0:
+            self.t.prefill(self.first, 0)
+            self.pos = 1
+        assert idx == self.pos, (idx, self.pos)
+        eng = self.t.e
+        eng.verify([int(token)], idx, want_logits=False)
+        self.pos = idx + 1
+        hip.check(hip.rt().hipStreamSynchronize(C.c_void_p(eng.stream)), "sync")
+        hip.check(hip.rt().hipMemcpy(C.c_void_p(address), C.c_void_p(eng.device_logits), self.vocab * 2, 3), "copy D2D")
+
+
+@pytest.mark.parametrize("temperature,kw", [(0.0, {}), (0.9, dict(top_p=0.95, repetition_penalty=1.2))])
+def test_a_drafter_that_leaves_its_logits_on_the_device(temperature, kw):
+    """tsv_drafter.device_logits: the draws and the round read the drafter's rows in device memory;
+    the run equals the one whose drafter hands back host logits."""
+    import turbospark_amd as ts
+    cfg, gpu, lm = _pair(draft_seed=77 if temperature == 0.0 else 1234)
+    V = cfg["vocab"]
+    prompt = np.random.default_rng(4).integers(0, V, 14).astype(np.int32)
+    gcfg = ts.shaping(temperature, seed=5 if temperature else None, **kw)
+    host = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V), gcfg, 40, 5)
+    dev = gpu.run_speculative(prompt, DeviceLmDrafter(GpuTarget(lm), prompt[0], V), gcfg, 40, 5, device_logits=True)
+    assert {k: dev[k] for k in KEYS} == {k: host[k] for k in KEYS}
+    assert len(dev["tokens"]) == 40

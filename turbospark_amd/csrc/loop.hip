@@ -134,7 +134,26 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
 
     int rc;
     if ((rc = tsv_reset(c))) return rc;
-    std::vector<uint16_t> logits((size_t)vocab), rows((size_t)g->block * vocab);
+    std::vector<uint16_t> logits((size_t)vocab), rows_host;
+    // the drafter's rows of a round: host memory, or a device buffer a GPU drafter fills in place
+    struct DeviceRows {
+        uint16_t* p = nullptr;
+        ~DeviceRows() {
+            if (p) (void)hipFree(p);
+        }
+    } rows_dev;
+    uint16_t* rows;
+    if (dr->device_logits) {
+        if (hipMalloc((void**)&rows_dev.p, (size_t)g->block * vocab * 2) != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("run_speculative: cannot allocate the drafter's device rows");
+            return TSV_ERR_DEVICE;
+        }
+        rows = rows_dev.p;
+    } else {
+        rows_host.resize((size_t)g->block * vocab);
+        rows = rows_host.data();
+    }
     // prefill: every prompt token but the last skips the output head; the drafter is primed with
     // each known next token
     if (n > 1 && (rc = tsv_prefill(c, prompt, n - 1, 0, nullptr))) return rc;
@@ -189,7 +208,7 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
                 if (sampled) draw_step += 1;
                 break;
             }
-            uint16_t* row = rows.data() + (size_t)d * vocab;
+            uint16_t* row = rows + (size_t)d * vocab;
             if (dr->step(dr->user, chained, base - 1 + d, row)) {
                 set_error("run_speculative: draft_step failed");
                 return TSV_ERR_INVALID;
@@ -205,7 +224,7 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         r.m = round_block + 1;
         r.base = base;
         r.shaping = g->shaping;
-        r.draft_logits = sampled ? rows.data() : nullptr;
+        r.draft_logits = sampled ? rows : nullptr;
         r.draw_step = draw_step;
         r.stop_tokens = g->stop_tokens;
         r.n_stop = g->n_stop;

@@ -1025,6 +1025,7 @@ extern "C" int32_t tsv_reset(tsv_ctx* c) {
 
 extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c->position; }
 extern "C" int64_t tsv_max_safe_rewind(const tsv_ctx*) { return INT64_MAX; }  // linear layout: nothing rings
+extern "C" const uint16_t* tsv_device_logits(tsv_ctx* c) { return c ? c->logits : nullptr; }
 extern "C" int64_t tsv_max_context(const tsv_ctx* c) { return c->max_context; }
 extern "C" int64_t tsv_vocab(const tsv_ctx* c) { return c->vocab; }
 

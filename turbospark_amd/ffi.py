@@ -110,7 +110,8 @@ DRAFT_REWIND = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int64)
 
 
 class Drafter(C.Structure):
-    _fields_ = [("user", C.c_void_p), ("prime", DRAFT_PRIME), ("step", DRAFT_STEP), ("rewind", DRAFT_REWIND)]
+    _fields_ = [("user", C.c_void_p), ("prime", DRAFT_PRIME), ("step", DRAFT_STEP), ("rewind", DRAFT_REWIND),
+                ("device_logits", C.c_int32)]
 
 
 class Generation(C.Structure):
@@ -148,7 +149,7 @@ class RoundResultC(C.Structure):
 
 
 EXPORTS = [
-    "tsv_open", "tsv_close", "tsv_last_error", "tsv_stream", "tsv_reset", "tsv_kv_position", "tsv_max_safe_rewind",
+    "tsv_open", "tsv_close", "tsv_last_error", "tsv_stream", "tsv_reset", "tsv_kv_position", "tsv_max_safe_rewind", "tsv_device_logits",
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
@@ -175,6 +176,8 @@ def lib():
         L.tsv_kv_position.argtypes = [C.c_void_p]
         L.tsv_max_safe_rewind.restype = C.c_int64
         L.tsv_max_safe_rewind.argtypes = [C.c_void_p]
+        L.tsv_device_logits.restype = C.c_void_p
+        L.tsv_device_logits.argtypes = [C.c_void_p]
         L.tsv_max_context.restype = C.c_int64
         L.tsv_max_context.argtypes = [C.c_void_p]
         L.tsv_vocab.restype = C.c_int64

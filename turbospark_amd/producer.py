@@ -87,6 +87,11 @@ class HipVerifier:
     def position(self):
         return ffi.lib().tsv_kv_position(self._h)
 
+    @property
+    def device_logits(self):
+        """Device address of the logits the last pass left on the GPU (rows x vocab fp16)."""
+        return ffi.lib().tsv_device_logits(self._h)
+
     def max_safe_rewind(self):
         """`KvCacheManager::max_safe_rewind`: unbounded (2**63 - 1), the cache is linear in every layer."""
         return ffi.lib().tsv_max_safe_rewind(self._h)
@@ -230,11 +235,14 @@ class HipVerifier:
         return props, ds.value
 
     # ---- the generation loop --------------------------------------------------------------
-    def run_speculative(self, prompt, drafter, cfg, max_new_tokens, block, stop_tokens=(), adaptive_floor=0):
+    def run_speculative(self, prompt, drafter, cfg, max_new_tokens, block, stop_tokens=(), adaptive_floor=0,
+                        device_logits=False):
         """`run_speculative` (crates/runtime/src/speculative.rs:194-900) for a step-wise drafter and
         chain rounds, acceptance and truncation on the device.  `drafter` offers prime(next, pos),
-        step(token, pos) -> uint16[vocab] and rewind(pos).  Returns a dict with the reported tokens,
-        the stop reason (1 stop token, 2 budget) and the round statistics."""
+        step(token, pos) -> uint16[vocab] and rewind(pos); with `device_logits` it offers
+        step_device(token, pos, device_address) instead and fills vocab fp16 values there on the GPU.
+        Returns a dict with the reported tokens, the stop reason (1 stop token, 2 budget) and the
+        round statistics."""
         vocab = self.vocab
         failure = []
 
@@ -249,11 +257,15 @@ class HipVerifier:
             return inner
 
         def step(user, token, pos, out):
+            if device_logits:
+                drafter.step_device(token, pos, C.cast(out, C.c_void_p).value)
+                return
             row = np.ascontiguousarray(drafter.step(token, pos), np.uint16)
             C.memmove(out, row.ctypes.data, vocab * 2)
 
         d = ffi.Drafter(None, ffi.DRAFT_PRIME(guard(lambda u, t, p: drafter.prime(t, p))),
-                        ffi.DRAFT_STEP(guard(step)), ffi.DRAFT_REWIND(guard(lambda u, p: drafter.rewind(p))))
+                        ffi.DRAFT_STEP(guard(step)), ffi.DRAFT_REWIND(guard(lambda u, p: drafter.rewind(p))),
+                        1 if device_logits else 0)
         g = ffi.Generation()
         g.shaping = cfg
         g.max_new_tokens = int(max_new_tokens)
