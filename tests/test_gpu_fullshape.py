@@ -104,3 +104,48 @@ def test_gptoss_120b_shape_one_windowed_and_one_full_layer_at_long_context():
     print(f"gpt-oss-120B shape, 2 layers, ctx {ctx}, m=9: max-abs logit error / range = {err:.2e}, "
           f"route margin {cpu.route_margin:.2e}")
     assert err <= 1e-2
+
+
+def test_llama3_8b_all_32_layers_size_independent_properties():
+    """The headline configuration at its real depth (32 layers, 4096-token context, vocabulary 128256),
+    where the oracle cannot follow: properties that hold at any size.  A pass is deterministic by bits;
+    a batched pass equals the same tokens fed one at a time by bits (families/qwen/batched.rs:92-110:
+    verify == sequential decode); a chain-shaped tree equals the chain; a rollback to the checkpoint
+    followed by the same pass reproduces it; the fused round equals verify followed by accept."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    ctx = 4096
+    cfg = dict(synth.CONFIGS["llama3_8b_q4_k"], max_context=ctx + 32)
+    gpu = ts.HipVerifier(cfg, synth.make_weights(cfg, seed=3))
+    rng = np.random.default_rng(3)
+    shape = (ctx, cfg["n_kv_heads"], cfg["head_dim"])
+    for layer in range(cfg["n_layers"]):
+        gpu.write_kv(layer, 0, (rng.standard_normal(shape) * 0.5).astype(np.float16),
+                     (rng.standard_normal(shape) * 0.5).astype(np.float16))
+    assert gpu.position == ctx
+    V = cfg["vocab"]
+    feed = rng.integers(0, V, 5).astype(np.int32)
+    point = gpu.checkpoint()
+    a = gpu.verify(feed, ctx)
+    gpu.rollback(point)
+    b = gpu.verify(feed, ctx)
+    assert np.array_equal(a, b)                       # deterministic, and the rollback left nothing behind
+    gpu.rollback(point)
+    seq = np.stack([gpu.produce(int(t), ctx + i) for i, t in enumerate(feed)])
+    assert np.array_equal(a, seq)                     # batched == sequential
+    gpu.rollback(point)
+    t = gpu.verify_tree(feed, [-1, 0, 1, 2, 3], ctx)
+    assert np.array_equal(a, t)                       # a chain-shaped tree is the chain
+    gpu.rollback(point)
+    draft = rng.standard_normal((4, V)).astype(np.float16)
+    cfg_s = ts.shaping(0.8, seed=11, top_p=0.95, repetition_penalty=1.1)
+    hist = [int(x) for x in rng.integers(0, V, 200)] + [int(feed[0])]
+    fused = gpu.verify_accept(feed, ctx, cfg_s, draft_logits=draft, draw_step=9, history=hist, generated=50)
+    gpu.rollback(point)
+    gpu.verify(feed, ctx, want_logits=False)
+    split = gpu.accept(feed, ctx, cfg_s, draft_logits=draft, draw_step=9, history=hist, generated=50)
+    assert fused == split and fused.kv_position == ctx + fused.committed + 1
+    ref = ob.chain_round(a, draft, feed[1:], ob.shaping(0.8, seed=11, top_p=0.95, repetition_penalty=1.1), history=hist,
+                         generated=50, draw_step=9)
+    assert (fused.accepted, fused.committed, fused.next, fused.draw_step) == \
+        (ref["accepted"], ref["committed"], ref["next"], ref["draw_step"])

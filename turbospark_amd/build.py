@@ -12,7 +12,10 @@ OPT = {"host_utils.hip": "-O2"}
 # MFMA results straight into VGPRs (no v_accvgpr_read copies before the scaling FMAs)
 EXTRA = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_GEMM_DEFS", "").split(),
          "fused.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),
-         "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+         "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+         # attention is instantiated per row-tile count, which depends on the rows of the pass: contraction is
+         # written out there (fmaf) instead of left to the compiler, so every instantiation rounds alike
+         "attn.hip": ["-ffp-contract=off"]}
 FLAGS = [
     "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed-fp32 VALU forms are switched off for every kernel in this library

@@ -31,6 +31,10 @@ int attn_chunks(int nkv) {
     return n;
 }
 
+// This file is compiled with -ffp-contract=off and every fused multiply-add is written out: left to
+// itself the compiler contracts a * b + c * d one way in one template instantiation and the other
+// way in the next, and a row's bits would then depend on how many rows share its pass.
+//
 // One (m, l, O) running state merged into another (flash-decoding rescale).
 template <int RT, int VT>
 __device__ __forceinline__ void merge_state(float (&mrun)[RT], float (&lrun)[RT], float4v (&O)[RT][VT], const float* src) {
@@ -42,11 +46,11 @@ __device__ __forceinline__ void merge_state(float (&mrun)[RT], float (&lrun)[RT]
         const float mnew = fmaxf(mrun[t], m1);
         if (mnew > -INFINITY) {
             const float a0 = __expf(mrun[t] - mnew), a1 = __expf(m1 - mnew);
-            lrun[t] = lrun[t] * a0 + l1 * a1;
+            lrun[t] = fmaf(lrun[t], a0, l1 * a1);
 #pragma unroll
             for (int d = 0; d < VT; d++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) O[t][d][i] = O[t][d][i] * a0 + src[64 * (2 * RT + (t * VT + d) * 4 + i)] * a1;
+                for (int i = 0; i < 4; i++) O[t][d][i] = fmaf(O[t][d][i], a0, src[64 * (2 * RT + (t * VT + d) * 4 + i)] * a1);
             mrun[t] = mnew;
         }
     }
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) 
                     ps += p;
                     P[i4] = (_Float16)p;
                 }
-                lrun[t] = lrun[t] * alpha + ps;
+                lrun[t] = fmaf(lrun[t], alpha, ps);
                 mrun[t] = mnew;
             }
 #pragma unroll
@@ -310,10 +314,10 @@ __global__ void k_attn_combine(AttnArgs a, int G, int R) {
     float num = 0.f;
     if (NCH > 0) {
 #pragma unroll
-        for (int c = 0; c < NCH; c++) num += wgt[c] * pre[c];
+        for (int c = 0; c < NCH; c++) num = fmaf(wgt[c], pre[c], num);
     } else {
 #pragma unroll 8
-        for (int c = 0; c < nch; c++) num += wgt[c] * po[c * stride];
+        for (int c = 0; c < nch; c++) num = fmaf(wgt[c], po[c * stride], num);
     }
     const _Float16 o16 = (_Float16)(num / s_den);
     const int kk = qh * hd + d;
