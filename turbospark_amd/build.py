@@ -12,12 +12,13 @@ OPT = {"host_utils.hip": "-O2"}
 # MFMA results straight into VGPRs (no v_accvgpr_read copies before the scaling FMAs)
 EXTRA = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_GEMM_DEFS", "").split(),
          "fused.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),
-         "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
-         # attention is instantiated per row-tile count, which depends on the rows of the pass: contraction is
-         # written out there (fmaf) instead of left to the compiler, so every instantiation rounds alike
-         "attn.hip": ["-ffp-contract=off"]}
+         "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 FLAGS = [
     "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # no implicit multiply-add fusion: the compiler picks the fused operand per template instantiation, and
+    # kernels are instantiated by row count, so a row's bits would depend on the width of its pass; the
+    # hot loops write their fmaf out, everything else rounds like the reference's unfused f32 / f64 code
+    "-ffp-contract=off",
     # packed-fp32 VALU forms are switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-pthread",

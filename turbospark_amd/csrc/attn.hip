@@ -31,9 +31,9 @@ int attn_chunks(int nkv) {
     return n;
 }
 
-// This file is compiled with -ffp-contract=off and every fused multiply-add is written out: left to
-// itself the compiler contracts a * b + c * d one way in one template instantiation and the other
-// way in the next, and a row's bits would then depend on how many rows share its pass.
+// The library is compiled with -ffp-contract=off and every fused multiply-add here is written out:
+// left to itself the compiler contracts a * b + c * d one way in one template instantiation and the
+// other way in the next, and a row's bits would then depend on how many rows share its pass.
 //
 // One (m, l, O) running state merged into another (flash-decoding rescale).
 template <int RT, int VT>
