@@ -149,3 +149,51 @@ def test_llama3_8b_all_32_layers_size_independent_properties():
                          generated=50, draw_step=9)
     assert (fused.accepted, fused.committed, fused.next, fused.draw_step) == \
         (ref["accepted"], ref["committed"], ref["next"], ref["draw_step"])
+
+
+def test_llama3_8b_all_32_layers_tree_of_16_at_16384_context():
+    """Configuration 3 at its real size (32 layers, 16384-token context, the 16-node tree, T = 1.0): a
+    chain-shaped tree of 16 rows equals the chain by bits; the pass is deterministic; multi-branch
+    rejection on the device equals the oracle's walk over the GPU's own logits; after compaction the
+    cache continues like one that was only ever fed the accepted path (families/qwen/dflash_tree.rs:106-207)."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    ctx = 16384
+    cfg = dict(synth.CONFIGS["llama3_8b_q4_k"], max_context=ctx + 32)
+    gpu = ts.HipVerifier(cfg, synth.make_weights(cfg, seed=3))
+    rng = np.random.default_rng(4)
+    shape = (ctx, cfg["n_kv_heads"], cfg["head_dim"])
+    for layer in range(cfg["n_layers"]):
+        k = (rng.standard_normal(shape, dtype=np.float32) * 0.5).astype(np.float16)
+        gpu.write_kv(layer, 0, k, k[::-1].copy())
+    V = cfg["vocab"]
+    feed = rng.integers(0, V, 16).astype(np.int32)
+    point = gpu.checkpoint()
+    chain = gpu.verify(feed, ctx)
+    gpu.rollback(point)
+    as_tree = gpu.verify_tree(feed, list(range(-1, 15)), ctx)
+    assert np.array_equal(chain, as_tree)
+    gpu.rollback(point)
+    parent = [-1, 0, 0, 0, 0, 1, 5, 6, 2, 8, 9, 3, 11, 12, 4, 14]
+    a = gpu.verify_tree(feed, parent, ctx)
+    gpu.rollback(point)
+    b = gpu.verify_tree(feed, parent, ctx)
+    assert np.array_equal(a, b)
+    # rows on the first root path see what the chain's rows saw: slots 0, 1, 5, 6, 7 are chain rows 0..4
+    # of a chain that fed those tokens
+    path = [0, 1, 5, 6, 7]
+    gpu.rollback(point)
+    alone = gpu.verify(feed[path], ctx)
+    assert gc.logit_error(a[path], alone) <= 2e-3
+    gpu.rollback(point)
+    gpu.verify_tree(feed, parent, ctx, want_logits=False)
+    draft = (gc.f16(a) + rng.standard_normal((16, V)).astype(np.float32) * 0.4).astype(np.float16)
+    res = gpu.accept(feed, ctx, ts.shaping(1.0, seed=6), parent=parent, draft_logits=draft, draw_step=2)
+    ref = ob.tree_round_sampled(a, draft, feed, parent, ob.shaping(1.0, seed=6), history=[0] * 8, draw_step=2)
+    assert res.path == ref["path"] and res.next == ref["next"] and res.draw_step == ref["draw_step"]
+    assert gpu.position == ctx + len(res.path)
+    # the compacted cache against a cache that only ever saw the accepted path
+    nxt = gpu.produce(res.next, gpu.position)
+    gpu.rollback(point)
+    gpu.verify(feed[res.path], ctx, want_logits=False)
+    assert gc.logit_error(nxt[None], gpu.produce(res.next, gpu.position)[None]) <= 2e-3
