@@ -197,3 +197,32 @@ def test_llama3_8b_all_32_layers_tree_of_16_at_16384_context():
     gpu.rollback(point)
     gpu.verify(feed[res.path], ctx, want_logits=False)
     assert gc.logit_error(nxt[None], gpu.produce(res.next, gpu.position)[None]) <= 2e-3
+
+
+def test_llama3_8b_all_32_layers_generation_loop_properties():
+    """The generation loop at the headline configuration's real depth and vocabulary: greedy
+    speculation reports exactly what plain greedy decoding reports whatever the drafter proposes
+    (speculative.rs:736-754), and a drafter that is the target itself has every proposal accepted,
+    greedy and sampled (r * q(x) <= p(x) with q == p)."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    from tests.loop_common import GpuTarget, LmDrafter
+    cfg = dict(synth.CONFIGS["llama3_8b_q4_k"], max_context=128)
+    w = synth.make_weights(cfg, seed=3)
+    gpu, twin = ts.HipVerifier(cfg, w), ts.HipVerifier(cfg, w)
+    V = cfg["vocab"]
+    prompt = np.random.default_rng(8).integers(0, V, 9).astype(np.int32)
+    new = 24
+    noisy = gpu.run_speculative(prompt, LmDrafter(GpuTarget(twin), prompt[0], V, noise=2.0, seed=3), ts.shaping(0.0), new, 4)
+    exact = gpu.run_speculative(prompt, LmDrafter(GpuTarget(twin), prompt[0], V), ts.shaping(0.0), new, 4)
+    gpu.reset()
+    gpu.prefill(prompt[:-1], 0, want_logits=False)
+    tok, plain = int(prompt[-1]), []
+    for i in range(new):
+        tok = int(np.argmax(gc.f16(gpu.produce(tok, len(prompt) - 1 + i))))
+        plain.append(tok)
+    assert noisy["tokens"] == plain == exact["tokens"]
+    assert exact["accepted"] == exact["offered"] and noisy["accepted"] < noisy["offered"]
+    sampled = gpu.run_speculative(prompt, LmDrafter(GpuTarget(twin), prompt[0], V), ts.shaping(0.8, seed=2, top_p=0.95), new, 4)
+    assert sampled["accepted"] == sampled["offered"] and len(sampled["tokens"]) == new
+    assert sampled["min_margin"] >= 0.0
