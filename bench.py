@@ -152,12 +152,27 @@ def traffic_summary(fetch_csv, write_csv):
     print(json.dumps(out, indent=1))
 
 
+def counter_summary(path):
+    """Per-dispatch averages of every counter in a `rocprofv3 --pmc ... --output-format csv` collection of
+    `bench.py --traffic-probe`, for the gate/up matmul launches (the copy kernel is left out)."""
+    import csv
+    acc = {}
+    for r in csv.DictReader(open(path)):
+        if "k_gemm" not in r["Kernel_Name"]:
+            continue
+        acc.setdefault(r["Counter_Name"], []).append(float(r["Counter_Value"]))
+    print(json.dumps({k: round(sum(v) / len(v), 1) for k, v in sorted(acc.items())} | {"dispatches": len(next(iter(acc.values())))},
+                     indent=1))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--trace-summary", default=None, metavar="CSV",
                     help="summarise a rocprofv3 kernel-trace CSV of this script (verify steps only) and exit")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run the copy kernel of known size and the dominant matmul (for rocprofv3 --pmc) and exit")
+    ap.add_argument("--counter-summary", default=None, metavar="CSV",
+                    help="per-dispatch averages of the counters a rocprofv3 --pmc run of --traffic-probe collected")
     ap.add_argument("--traffic-summary", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="HBM bytes per launch of the dominant matmul from two --pmc runs of --traffic-probe")
     ap.add_argument("--gpus", type=int, default=1)
@@ -173,6 +188,9 @@ def main():
         return
     if args.traffic_probe:
         traffic_probe()
+        return
+    if args.counter_summary:
+        counter_summary(args.counter_summary)
         return
     if args.traffic_summary:
         traffic_summary(*args.traffic_summary)
