@@ -296,6 +296,10 @@ int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16
  * one layer and moves the cursor to at least pos0 + n -- a long context without the prefill that
  * would build it (the full-size parity cases; also how a saved prefix would be restored). */
 int32_t tsv_write_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k, const uint16_t* v);
+/* Stores m x vocab fp16 logits (host memory) as if a verify pass of m rows at `base` had just left them on
+ * the device: tsv_accept then judges exactly these scores (acceptance cases no model would produce: ties,
+ * flat rows, the fp16 extremes).  The KV cache and the cursor are not touched. */
+int32_t tsv_write_logits(tsv_ctx* ctx, const uint16_t* logits, int32_t m, int64_t base);
 /* One quantized small-M matmul through the same kernels the forward uses:
  * y[m][r] = sum_k W[r][k] x[m][k]; x is m x cols fp32 (rounded to fp16 on entry), y is
  * m x rows fp32.  W host tensor in GGUF layout (re-tiled per call).  `splits` <= 0 picks

@@ -1351,6 +1351,18 @@ extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t 
     return rc;
 }
 
+extern "C" int32_t tsv_write_logits(tsv_ctx* c, const uint16_t* logits, int32_t m, int64_t base) {
+    if (!c || !logits || m < 1 || m > TSV_MAX_ROWS || base < 0) {
+        set_error("write_logits: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    TSV_HIP(hipMemcpyAsync(c->logits, logits, (size_t)m * c->vocab * 2, hipMemcpyHostToDevice, c->stream));
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    c->last_m = m;
+    c->last_base = base;
+    return TSV_OK;
+}
+
 extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k,
                                 const uint16_t* v) {
     if (!c || !k || !v || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->max_context) {

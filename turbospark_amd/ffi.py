@@ -153,7 +153,7 @@ EXPORTS = [
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
-    "tsv_synth_tensor", "tsv_read_kv", "tsv_write_kv", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
+    "tsv_synth_tensor", "tsv_read_kv", "tsv_write_kv", "tsv_write_logits", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
     "tsv_yarn_frequencies", "tsv_adaptive_init", "tsv_adaptive_depth", "tsv_adaptive_observe", "tsv_adaptive_tile_cap",
     "tsv_run_speculative", "tsv_max_context", "tsv_vocab",
 ]
@@ -213,6 +213,7 @@ def lib():
                                        C.c_void_p]
         L.tsv_read_kv.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.tsv_write_kv.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
+        L.tsv_write_logits.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64]
         L.tsv_matmul.argtypes = [C.POINTER(Tensor), C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
         L.tsv_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                     C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_void_p, C.c_void_p]

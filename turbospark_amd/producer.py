@@ -312,6 +312,14 @@ class HipVerifier:
         v16 = np.ascontiguousarray(np.asarray(v).astype(np.float16))
         ffi.check(ffi.lib().tsv_write_kv(self._h, layer, int(pos0), k16.shape[0], k16.ctypes.data, v16.ctypes.data))
 
+    def write_logits(self, logits, base):
+        """logits [m, vocab] (uint16 fp16 bits, or floats rounded to fp16) become what `accept` judges."""
+        a = np.asarray(logits)
+        if a.dtype != np.uint16:
+            a = a.astype(np.float16).view(np.uint16)
+        a = np.ascontiguousarray(a)
+        ffi.check(ffi.lib().tsv_write_logits(self._h, a.ctypes.data, a.shape[0], int(base)))
+
     def read_kv(self, layer, pos0, n):
         c = self.cfg
         shape = (n, c["n_kv_heads"], c["head_dim"])
