@@ -67,16 +67,18 @@ def _shaping(r, seed, penalties):
     return ts.shaping(t, seed=seed, **kw), ob.shaping(t, seed=seed, **kw), kw
 
 
-@pytest.mark.parametrize("vocab", [4096, 1000, 37, 2])
+@pytest.mark.parametrize("vocab", [4096, 1000, 37, 2, 128256, 201088])
 def test_adversarial_chain_rounds(vocab):
+    """(128256 and 201088: the vocabularies of the benchmark configurations, fewer and narrower rounds.)"""
     cfg, w, gpu, cpu = gc.build_pair("tiny_q8_0", max_context=64, vocab=vocab)
     V = vocab
     r = np.random.default_rng(77 + vocab)
     base = 20
     compared = skipped = 0
     outcomes = set()
-    for case in range(60):
-        k = int(r.integers(0, 16))
+    big = V > 100000
+    for case in range(14 if big else 60):
+        k = int(r.integers(0, 6 if big else 16))
         kind_t, kind_d = r.choice(KINDS), r.choice(KINDS)
         target = np.stack([_row(r, V, kind_t) for _ in range(k + 1)]).astype(np.float16)
         # the drafter: adversarial rows of its own, or the target's rows nudged (so that proposals get accepted)
@@ -123,7 +125,7 @@ def test_adversarial_chain_rounds(vocab):
         compared += 1
         outcomes.add((res.accepted == k, res.stopped))
     print(f"vocab {vocab}: {compared} rounds compared, {skipped} too close to call or refused by name; outcomes {sorted(outcomes)}")
-    assert compared >= 45 and len(outcomes) >= 2
+    assert compared >= (10 if big else 45) and len(outcomes) >= 2
 
 
 @pytest.mark.parametrize("vocab", [4096, 333])
