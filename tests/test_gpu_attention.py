@@ -106,3 +106,30 @@ def test_tree_attention_with_a_window():
         got = ffi.attention(q, k, v, base, parent, scale=0.125, window=window, sinks=sinks)
         want = _oracle(q, k, v, base, parent, 0.125, window, sinks)
         assert np.abs(got - want).max() <= 5e-3 * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_attention_shapes_and_long_contexts(seed):
+    """Seeded sweep: head width, GQA group 1..8, 1..16 rows, chain or random tree, contexts up to 20000
+    positions (several 16-position blocks per wave: the pipelined walk), optional window (wider than
+    the pass) and sinks, a scale of its own."""
+    from turbospark_amd import ffi
+    r = np.random.default_rng(4000 + seed)
+    hd = int(r.choice([64, 128]))
+    nkv = int(r.choice([1, 2, 4, 8]))
+    g = int(r.choice([1, 2, 3, 4, 8]))
+    nq = nkv * g
+    m = int(r.integers(1, 17))
+    base = int(r.choice([0, 1, 15, 16, 17, int(r.integers(18, 600)), int(r.integers(600, 5000)), int(r.integers(5000, 20000))]))
+    tree = bool(r.integers(0, 2)) and m > 2
+    parent = [-1] + [int(r.integers(0, s)) for s in range(1, m)] if tree else None
+    window = int(r.integers(17, 300)) if r.integers(0, 3) == 0 else 0
+    sinks = (r.standard_normal(nq) * 2).astype(np.float32) if r.integers(0, 3) == 0 else None
+    scale = float(r.choice([0.0, 0.1, 0.2]))
+    q, k, v = _rand(m, nq, nkv, hd, base, 9000 + seed)
+    print(f"seed {seed}: hd={hd} q/kv={nq}/{nkv} m={m} base={base} {'tree' if tree else 'chain'} window={window} "
+          f"sinks={'yes' if sinks is not None else 'no'} scale={scale}", flush=True)
+    got = ffi.attention(q, k, v, base, parent=parent, scale=scale, window=window, sinks=sinks)
+    want = _oracle(q, k, v, base, parent, scale=scale, window=window, sinks=sinks)
+    err = np.abs(got - want).max()
+    assert err <= 5e-3 * max(1.0, np.abs(want).max()), err

@@ -129,3 +129,31 @@ def test_q6k_hand_packed_superblock_through_the_kernel(golden):
             h, k, l = e // 128, (e % 128) // 32, e % 32
             want = np.float32(g["d"]) * np.float32(g["scales"][h * 8 + l // 16 + 2 * k]) * np.float32(g["quants"][k])
             assert np.all(got[b] == want), (e, got[b][0], want)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_matmul_shapes(seed):
+    """Seeded sweep over format, row count (padded last tiles), K (one chunk to dozens, MXFP4 / bf16 rows
+    that end inside a chunk), batch width and split-K count."""
+    from turbospark_amd import ffi
+    r = np.random.default_rng(6000 + seed)
+    dtype = int(r.choice([12, 8, 39, 30, 14]))
+    unit = {12: 256, 14: 256, 8: 128, 39: 32, 30: 64}[dtype]
+    cols = unit * int(r.integers(1, {12: 24, 14: 24, 8: 48, 39: 120, 30: 60}[dtype]))
+    rows = int(r.integers(1, 400))
+    m = int(r.integers(1, 17))
+    kchunks = -(-cols // {12: 256, 14: 256, 8: 128, 39: 256, 30: 64}[dtype])
+    splits = int(r.integers(0, min(8, kchunks) + 1))
+    w = (r.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+    entry = ffi.quantize(dtype, w)
+    x = r.standard_normal((m, cols)).astype(np.float32)
+    x16 = x.astype(np.float16).astype(np.float32)
+    want = np.stack([ob.gemv(dtype, entry[1], rows, cols, x16[b]) for b in range(m)])
+    print(f"seed {seed}: dtype {dtype} {rows} x {cols}, m={m}, splits={splits}", flush=True)
+    try:
+        got = ffi.matmul(entry, x, splits=splits)
+    except Exception as e:  # a split count that leaves an empty K slice is refused by name
+        assert "empty K slice" in str(e), e
+        got = ffi.matmul(entry, x)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= scale * 2e-4 + 1e-5
