@@ -12,7 +12,7 @@ import numpy as np
 _DIR = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_DIR, "libtsoracle.so")
 
-F32, F16, Q8_0, Q4_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 14, 30, 39
+F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 13, 14, 30, 39
 
 
 def build():
@@ -175,7 +175,8 @@ def quantize(dtype, w):
         for i in range(flat.size):
             o[i] = lib().tso_f32_to_bf16(float(flat[i]))
         return out.view(np.uint8).reshape(rows, cols * 2)
-    fn = {Q8_0: lib().tso_quantize_q8_0, Q4_K: lib().tso_quantize_q4_k, Q6_K: lib().tso_quantize_q6_k,
+    fn = {Q8_0: lib().tso_quantize_q8_0, Q4_K: lib().tso_quantize_q4_k, Q5_K: lib().tso_quantize_q5_k,
+          Q6_K: lib().tso_quantize_q6_k,
           MXFP4: lib().tso_quantize_mxfp4}[dtype]
     rb = row_bytes(dtype, cols)
     out = np.empty((rows, rb), np.uint8)

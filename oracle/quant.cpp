@@ -87,6 +87,7 @@ extern "C" int64_t tso_row_bytes(int dtype, int64_t n) {
         case TSO_BF16: return n * 2;
         case TSO_Q8_0: return n / 32 * 34;
         case TSO_Q4_K: return n / 256 * 144;
+        case TSO_Q5_K: return n / 256 * 176;
         case TSO_Q6_K: return n / 256 * 210;
         case TSO_MXFP4: return (n + 31) / 32 * 17;
     }
@@ -230,6 +231,101 @@ extern "C" void tso_quantize_q4_k(const float* row, int64_t n, uint8_t* out) {
     }
 }
 
+// crates/compute/src/quant_gguf/q5_k.rs:47-96.  Q4_K plus a fifth bit per element: d, dmin, the same
+// 12 packed 6-bit scales / mins, then 32 bytes `qh` and 128 nibble bytes.  Byte qh[l] serves the
+// elements l, l + 32, l + 64, ... of the superblock; group g (64 elements) reads bit 2g for its low
+// nibbles and bit 2g + 1 for its high ones.
+extern "C" void tso_dequantize_q5_k(const uint8_t* blocks, int64_t n, float* out) {
+    for (int64_t b = 0; b < n / 256; b++) {
+        const uint8_t* p = blocks + b * 176;
+        float d = tso_f16_to_f32((uint16_t)(p[0] | (p[1] << 8)));
+        float dmin = tso_f16_to_f32((uint16_t)(p[2] | (p[3] << 8)));
+        const uint8_t* packed = p + 4;
+        const uint8_t* qh = p + 16;
+        const uint8_t* ql = p + 48;
+        for (int g = 0; g < 4; g++) {
+            uint8_t sc_lo, m_lo, sc_hi, m_hi;
+            tso_q4_k_scale_min(2 * g, packed, &sc_lo, &m_lo);
+            tso_q4_k_scale_min(2 * g + 1, packed, &sc_hi, &m_hi);
+            float d_lo = d * (float)sc_lo, min_lo = dmin * (float)m_lo;
+            float d_hi = d * (float)sc_hi, min_hi = dmin * (float)m_hi;
+            const uint8_t* group = ql + g * 32;
+            float* at = out + b * 256 + g * 64;
+            for (int l = 0; l < 32; l++) {
+                uint8_t byte = group[l], hb = qh[l];
+                uint8_t q_lo = (uint8_t)((byte & 0xF) + (((hb >> (2 * g)) & 1) << 4));
+                uint8_t q_hi = (uint8_t)((byte >> 4) + (((hb >> (2 * g + 1)) & 1) << 4));
+                at[l] = d_lo * (float)q_lo - min_lo;
+                at[32 + l] = d_hi * (float)q_hi - min_hi;
+            }
+        }
+    }
+}
+
+// NOT IN THE REFERENCE (it only decodes Q5_K): the Q4_K min/max fitter of q4_k.rs:126-204 with 31
+// levels per sub-block instead of 15, so that synthetic weights can be stored in this format.
+extern "C" void tso_quantize_q5_k(const float* row, int64_t n, uint8_t* out) {
+    for (int64_t b = 0; b < n / 256; b++) {
+        const float* block = row + b * 256;
+        float scales[8], mins[8];
+        for (int j = 0; j < 8; j++) {
+            const float* sub = block + j * 32;
+            float lo = 0.0f;
+            for (int i = 0; i < 32; i++) lo = fold_min(lo, sub[i]);
+            float hi = lo;
+            for (int i = 0; i < 32; i++) hi = fold_max(hi, sub[i]);
+            scales[j] = (hi - lo) / 31.0f;
+            mins[j] = -lo;
+        }
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 8; j++) {
+            max_scale = fold_max(max_scale, scales[j]);
+            max_min = fold_max(max_min, mins[j]);
+        }
+        float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+        float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+        uint8_t packed[12] = {0};
+        for (int j = 0; j < 8; j++) {
+            uint8_t ls = (uint8_t)clampf(roundf(scales[j] * inv_scale), 0.0f, 63.0f);
+            uint8_t lm = (uint8_t)clampf(roundf(mins[j] * inv_min), 0.0f, 63.0f);
+            if (j < 4) {
+                packed[j] |= ls;
+                packed[j + 4] |= lm;
+            } else {
+                packed[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                packed[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                packed[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        uint16_t d = tso_f32_to_f16(max_scale / 63.0f);
+        uint16_t dmin = tso_f32_to_f16(max_min / 63.0f);
+        float d_f = tso_f16_to_f32(d), dmin_f = tso_f16_to_f32(dmin);
+        uint8_t quants[256] = {0};
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            tso_q4_k_scale_min(j, packed, &sc, &m);
+            float step = d_f * (float)sc;
+            if (step == 0.0f) continue;
+            float bias = dmin_f * (float)m;
+            for (int i = 0; i < 32; i++)
+                quants[j * 32 + i] = (uint8_t)clampf(roundf((block[j * 32 + i] + bias) / step), 0.0f, 31.0f);
+        }
+        uint8_t* o = out + b * 176;
+        std::memset(o, 0, 176);
+        o[0] = (uint8_t)(d & 0xFF);
+        o[1] = (uint8_t)(d >> 8);
+        o[2] = (uint8_t)(dmin & 0xFF);
+        o[3] = (uint8_t)(dmin >> 8);
+        std::memcpy(o + 4, packed, 12);
+        for (int g = 0; g < 4; g++)
+            for (int l = 0; l < 32; l++) {
+                const uint8_t q_lo = quants[g * 64 + l], q_hi = quants[g * 64 + 32 + l];
+                o[48 + g * 32 + l] = (uint8_t)((q_lo & 0xF) | ((q_hi & 0xF) << 4));
+                o[16 + l] |= (uint8_t)(((q_lo >> 4) << (2 * g)) | ((q_hi >> 4) << (2 * g + 1)));
+            }
+    }
+}
+
 // crates/compute/src/quant_gguf_mxfp4.rs:76-78
 static const float MXFP4_VALUES[16] = {0.0f, 1.0f, 2.0f,  3.0f,  4.0f,  6.0f,  8.0f,  12.0f,
                                        0.0f, -1.0f, -2.0f, -3.0f, -4.0f, -6.0f, -8.0f, -12.0f};
@@ -303,6 +399,7 @@ extern "C" void tso_dequantize_row(int dtype, const uint8_t* row, int64_t n, flo
             break;
         case TSO_Q8_0: tso_dequantize_q8_0(row, n, out); break;
         case TSO_Q4_K: tso_dequantize_q4_k(row, n, out); break;
+        case TSO_Q5_K: tso_dequantize_q5_k(row, n, out); break;
         case TSO_Q6_K: tso_dequantize_q6_k(row, n, out); break;
         case TSO_MXFP4: tso_dequantize_mxfp4(row, n, out); break;
     }

@@ -27,6 +27,8 @@
  *                                        acceptance rate = sum min(p,q)) over thousands of seeds
  *   - Q6_K decode / encode ............. the reference's hand-packed superblock literal; round-trip
  *                                        bound, both scale signs, zero block
+ *   - Q5_K decode ...................... ggml-produced bytes -> floats fixture (two superblocks), ==; dropping
+ *                                        the fifth-bit run changes the values
  *   - YaRN table ....................... the reference's gpt-oss scalars -> mscale 1.3465736, untouched
  *                                        fast end, fully interpolated slow end, ramp between ggml's
  *                                        correction dimensions, swapped betas differ
@@ -45,6 +47,8 @@
  *     a node is shaped with the history of its own root path, the chain round's rule.
  *   - tso_quantize_mxfp4: the reference has no MXFP4 encoder; checked by brute force
  *     against "nearest codebook value under the tightest covering exponent".
+ *   - tso_quantize_q5_k: the reference only decodes Q5_K; the encoder is Q4_K's min/max fitter with 31
+ *     levels, checked by decode(encode(x)) within half a step.
  */
 #ifndef TSORACLE_H
 #define TSORACLE_H
@@ -63,6 +67,7 @@ enum {
     TSO_F16 = 1,
     TSO_Q8_0 = 8,
     TSO_Q4_K = 12,
+    TSO_Q5_K = 13, /* 176 B / 256 elems: Q4_K's header, 32 bytes of fifth bits, 128 nibble bytes */
     TSO_Q6_K = 14, /* 210 B / 256 elems: 4 low bits + 2 high bits per element, 16 signed int8 scales, f16 d */
     TSO_BF16 = 30,
     TSO_MXFP4 = 39,
@@ -82,6 +87,8 @@ void tso_quantize_q4_k(const float* row, int64_t n, uint8_t* out);
 void tso_dequantize_q4_k(const uint8_t* blocks, int64_t n, float* out);
 void tso_q4_k_scale_min(int j, const uint8_t* packed12, uint8_t* sc, uint8_t* mn);
 /* crates/compute/src/quant_gguf/q6_k.rs:44-88 (decode), :101-194 (largest-magnitude encoder) */
+void tso_dequantize_q5_k(const uint8_t* blocks, int64_t n, float* out); /* crates/compute/src/quant_gguf/q5_k.rs:47-96 */
+void tso_quantize_q5_k(const float* row, int64_t n, uint8_t* out);      /* not in the reference: Q4_K's fitter, 31 levels */
 void tso_dequantize_q6_k(const uint8_t* blocks, int64_t n, float* out);
 void tso_quantize_q6_k(const float* row, int64_t n, uint8_t* out);
 float tso_mxfp4_scale(uint8_t e);

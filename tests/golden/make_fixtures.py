@@ -3,6 +3,8 @@
 Reads files below /root/reference as text / data only (nothing is imported or run):
   * the literal arrays of crates/compute/tests/generated/quant_gguf_mxfp4_oracle.rs
     (bytes ggml produced and the floats ggml decoded from them)  -> mxfp4_ggml_oracle.json
+  * the literal arrays of crates/compute/tests/generated/quant_gguf_q5_k_oracle.rs (two Q5_K superblocks
+    ggml quantized and the floats ggml decoded from them)  -> q5k_ggml_oracle.json
   * the hand-packed Q4_K superblock constants of crates/compute/tests/quant_gguf.rs:226-267
     -> q4k_handpacked.json
   * the llama-3 rope factor profile of crates/compute/src/rope.rs:471-482 -> llama3_rope_profile.json
@@ -41,6 +43,15 @@ def main():
     assert len(fixture["codebook"]) == 16 and len(fixture["e8m0_times_codebook1"]) == 256
     assert len(fixture["bytes"]) == 68 and len(fixture["floats"]) == 128
     json.dump(fixture, open(f"{OUT}/mxfp4_ggml_oracle.json", "w"))
+
+    src = open(f"{REF}/crates/compute/tests/generated/quant_gguf_q5_k_oracle.rs").read()
+    q5 = {
+        "source": "crates/compute/tests/generated/quant_gguf_q5_k_oracle.rs",
+        "bytes": [int(v) for v in rust_array(src, "Q5_K_ORACLE_BYTES")],
+        "floats": [float(v) for v in rust_array(src, "Q5_K_ORACLE_FLOATS")],
+    }
+    assert len(q5["bytes"]) == 352 and len(q5["floats"]) == 512
+    json.dump(q5, open(f"{OUT}/q5k_ggml_oracle.json", "w"))
 
     src = open(f"{REF}/crates/compute/tests/quant_gguf.rs").read()
     q4 = {

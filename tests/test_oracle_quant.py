@@ -218,3 +218,34 @@ def test_gemv_is_dequantize_then_sequential_dot():
                 acc = np.float32(acc + np.float32(deq[r, k] * x[k]))
             want[r] = acc
         assert np.array_equal(ob.gemv(dt, qb, 4, 256, x), want)
+
+
+def test_q5k_decodes_exactly_what_ggml_decodes(golden):
+    """crates/compute/tests/quant_gguf.rs:548-600: two superblocks ggml quantized, the floats ggml decoded
+    from them, `==`; without the fifth-bit run the values change (the bit carries 16 quant levels)."""
+    import json
+    g = json.load(open(os.path.join(golden, "q5k_ggml_oracle.json")))
+    raw = np.array(g["bytes"], np.uint8)
+    want = np.array(g["floats"], np.float32)
+    assert raw.size == 2 * 176 and want.size == 512 and ob.row_bytes(ob.Q5_K, 512) == 352
+    got = ob.dequantize(ob.Q5_K, raw, 512)[0]
+    assert np.array_equal(got, want)
+    stripped = raw.copy()
+    for b in range(2):
+        stripped[b * 176 + 16:b * 176 + 48] = 0
+    assert not np.array_equal(ob.dequantize(ob.Q5_K, stripped, 512)[0], want)
+
+
+def test_q5k_encoder_round_trip():
+    """The encoder is this project's (the reference only decodes Q5_K): decode(encode(x)) stays inside
+    half a quantization step of each sub-block plus the 6-bit scale / min rounding; a zero block is zeros."""
+    w = lcg_weights(1024, 43)
+    out = ob.dequantize(ob.Q5_K, ob.quantize(ob.Q5_K, w.reshape(1, -1)), 1024)[0]
+    for j in range(32):
+        sub = w[32 * j:32 * j + 32]
+        span = max(sub.max(), 0.0) - min(sub.min(), 0.0)
+        assert np.abs(out[32 * j:32 * j + 32] - sub).max() <= span / 31.0 * 0.5 + span * 3e-2
+    q4 = ob.dequantize(ob.Q4_K, ob.quantize(ob.Q4_K, w.reshape(1, -1)), 1024)[0]
+    assert np.abs(out - w).mean() < 0.7 * np.abs(q4 - w).mean()   # the fifth bit buys precision
+    z = ob.quantize(ob.Q5_K, np.zeros((1, 256), np.float32))[0]
+    assert np.all(ob.dequantize(ob.Q5_K, z, 256) == 0.0)
