@@ -37,6 +37,7 @@ enum {
     TSV_F16 = 1,
     TSV_Q8_0 = 8,  /* 34 B / 32 elems  (crates/compute/src/quant_gguf/q8_0.rs) */
     TSV_Q4_K = 12, /* 144 B / 256 elems (crates/compute/src/quant_gguf/q4_k.rs) */
+    TSV_Q5_K = 13, /* 176 B / 256 elems: Q4_K's header, 32 bytes of fifth bits, 128 nibble bytes (q5_k.rs) */
     TSV_Q6_K = 14, /* 210 B / 256 elems (crates/compute/src/quant_gguf/q6_k.rs): the other half of a Q4_K_M file */
     TSV_BF16 = 30,
     TSV_MXFP4 = 39, /* 17 B / 32 elems: e8m0 scale + 32 e2m1 nibbles (crates/compute/src/quant_gguf_mxfp4.rs) */

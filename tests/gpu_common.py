@@ -31,4 +31,4 @@ def logit_error(got_bits, want_bits):
     return float(np.abs(g - w).max() / rng)
 
 
-TOL = {ffi.Q8_0: 2e-3, ffi.Q4_K: 1e-2}
+TOL = {ffi.Q8_0: 2e-3, ffi.Q4_K: 1e-2, ffi.Q5_K: 1e-2}

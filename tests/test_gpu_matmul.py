@@ -26,7 +26,8 @@ def _case(dtype, rows, cols, seed):
                                              (39, 64, 512), (39, 48, 2048), (39, 200, 768),
                                              (39, 64, 576), (39, 96, 2880),      # MXFP4 rows ending inside a 256-chunk
                                              (30, 64, 512), (30, 40, 576), (30, 130, 2880),   # bf16
-                                             (14, 64, 512), (14, 48, 2048), (14, 200, 768)])   # Q6_K
+                                             (14, 64, 512), (14, 48, 2048), (14, 200, 768),    # Q6_K
+                                             (13, 64, 512), (13, 48, 2048), (13, 200, 768)])   # Q5_K
 def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, rows, cols, 31)
@@ -46,7 +47,7 @@ def test_matmul_matches_dequantize_then_dot_for_every_width(dtype, rows, cols):
         assert np.array_equal(got[0], first), m
 
 
-@pytest.mark.parametrize("dtype", [12, 8, 39, 30, 14])
+@pytest.mark.parametrize("dtype", [12, 8, 39, 30, 14, 13])
 def test_split_k_changes_nothing_but_rounding_and_is_deterministic(dtype):
     from turbospark_amd import ffi
     entry, x, x16, want = _case(dtype, 32, 2048, 77)
@@ -137,12 +138,12 @@ def test_random_matmul_shapes(seed):
     that end inside a chunk), batch width and split-K count."""
     from turbospark_amd import ffi
     r = np.random.default_rng(6000 + seed)
-    dtype = int(r.choice([12, 8, 39, 30, 14]))
-    unit = {12: 256, 14: 256, 8: 128, 39: 32, 30: 64}[dtype]
-    cols = unit * int(r.integers(1, {12: 24, 14: 24, 8: 48, 39: 120, 30: 60}[dtype]))
+    dtype = int(r.choice([12, 8, 39, 30, 14, 13]))
+    unit = {12: 256, 13: 256, 14: 256, 8: 128, 39: 32, 30: 64}[dtype]
+    cols = unit * int(r.integers(1, {12: 24, 13: 24, 14: 24, 8: 48, 39: 120, 30: 60}[dtype]))
     rows = int(r.integers(1, 400))
     m = int(r.integers(1, 17))
-    kchunks = -(-cols // {12: 256, 14: 256, 8: 128, 39: 256, 30: 64}[dtype])
+    kchunks = -(-cols // {12: 256, 13: 256, 14: 256, 8: 128, 39: 256, 30: 64}[dtype])
     splits = int(r.integers(0, min(8, kchunks) + 1))
     w = (r.standard_normal((rows, cols)) * 0.05).astype(np.float32)
     entry = ffi.quantize(dtype, w)
@@ -157,3 +158,21 @@ def test_random_matmul_shapes(seed):
         got = ffi.matmul(entry, x)
     scale = np.abs(want).max()
     assert np.abs(got - want).max() <= scale * 2e-4 + 1e-5
+
+
+def test_q5k_ggml_golden_superblocks_through_the_kernel(golden):
+    """The two Q5_K superblocks ggml quantized (crates/compute/tests/generated/quant_gguf_q5_k_oracle.rs), as
+    a one-row matrix, multiplied by unit vectors through the kernel: every weight reads back as the
+    float ggml decoded (fp16 unit activations select one weight each; products are exact in fp32)."""
+    import json
+    import os
+    from turbospark_amd import ffi
+    g = json.load(open(os.path.join(golden, "q5k_ggml_oracle.json")))
+    raw = np.array(g["bytes"], np.uint8).reshape(1, -1)
+    want = np.array(g["floats"], np.float32)
+    entry = (13, raw, 1, 512)
+    for k0 in range(0, 512, 16):
+        x = np.zeros((16, 512), np.float32)
+        x[np.arange(16), k0 + np.arange(16)] = 1.0
+        got = ffi.matmul(entry, x)[:, 0]
+        assert np.allclose(got, want[k0:k0 + 16], rtol=0, atol=2e-6), (k0, got, want[k0:k0 + 16])

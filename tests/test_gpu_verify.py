@@ -14,7 +14,8 @@ def _prompt(n, vocab, seed):
 @pytest.mark.parametrize("name,ctx,k", [("tiny_q8_0", 256, 4), ("small_q4_k", 70, 4), ("small_q4_k", 33, 15),
                                         ("xcd_q4_k", 70, 4), ("xcd_q4_k", 33, 7), ("xcd_q4_k", 40, 0),
                                         ("xcd_q8_0", 70, 4), ("xcd_q4_k", 33, 15),
-                                        ("small_q4_k_m", 70, 4), ("small_q4_k_m", 21, 15)])
+                                        ("small_q4_k_m", 70, 4), ("small_q4_k_m", 21, 15),
+                                        ("small_q5_k_m", 70, 4), ("small_q5_k_m", 21, 15)])
 def test_verify_logits_match_the_oracle(name, ctx, k):
     cfg, w, gpu, cpu = gc.build_pair(name, max_context=ctx + 32)
     prompt = _prompt(ctx, cfg["vocab"], 7)
@@ -36,7 +37,7 @@ def test_verify_logits_match_the_oracle(name, ctx, k):
     assert gpu.position == ctx + k + 1
 
 
-@pytest.mark.parametrize("name", ["small_q4_k", "xcd_q4_k", "xcd_q8_0", "small_q4_k_m"])
+@pytest.mark.parametrize("name", ["small_q4_k", "xcd_q4_k", "xcd_q8_0", "small_q4_k_m", "small_q5_k_m"])
 def test_a_batched_pass_equals_the_same_tokens_fed_one_at_a_time(name):
     """crates/runtime/tests/real_forward_qwen35_mtp.rs:962-1032: the row-invariance gate."""
     cfg, w, gpu, cpu = gc.build_pair(name, max_context=96)

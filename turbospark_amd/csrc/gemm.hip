@@ -52,6 +52,23 @@ __global__ void k_repack_q4k(const uint8_t* __restrict__ raw, int n_rows, int kc
     *(uint4*)dst = *(const uint4*)(u < 8 ? blk + 16 + 16 * u : blk);
 }
 
+// Q5_K: units 0..7 the nibble bytes, 8 the scale header (both as in Q4_K), 9 and 10 the fifth bits.
+__global__ void k_repack_q5k(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
+                             uint8_t* __restrict__ tiles, int grp, int stride, int offset, const int32_t* __restrict__ rowmap) {
+    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)n_rows * kchunks * 11;
+    if (gid >= total) return;
+    const int u = (int)(gid % 11);
+    const long t = gid / 11;
+    const int c = (int)(t % kchunks);
+    const int r = (int)(t / kchunks);
+    const int drow = rowmap ? rowmap[r] : (r / grp) * stride + offset + r % grp;
+    const int tile = drow >> 6, lane = drow & 63;
+    const uint8_t* blk = raw + ((long)r * kchunks + c) * 176;
+    uint8_t* dst = tiles + ((long)tile * kchunks + c) * 11264 + (u * 64 + lane) * 16;
+    *(uint4*)dst = *(const uint4*)(u < 8 ? blk + 48 + 16 * u : u == 8 ? blk : blk + 16 + 16 * (u - 9));
+}
+
 __global__ void k_repack_q80(const uint8_t* __restrict__ raw, int n_rows, int kchunks,
                              uint8_t* __restrict__ tiles, int grp, int stride, int offset, const int32_t* __restrict__ rowmap) {
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -213,6 +230,10 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
         const long blocks = (long)n_rows * kchunks * 8;
         hipLaunchKernelGGL(k_repack_mx4, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
                            tiles, grp, stride, offset, k / 32, rowmap);
+    } else if (fmt == FMT_Q5K) {
+        const long units = (long)n_rows * kchunks * 11;
+        hipLaunchKernelGGL(k_repack_q5k, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, raw, n_rows, kchunks,
+                           tiles, grp, stride, offset, rowmap);
     } else if (fmt == FMT_Q4K)
         hipLaunchKernelGGL(k_repack_q4k, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, raw, n_rows,
                            kchunks, tiles, grp, stride, offset, rowmap);
@@ -480,6 +501,7 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
            : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
            : w.fmt == FMT_BF16 ? launch_f<BF16W>(s, a, m, epi)
            : w.fmt == FMT_Q6K  ? launch_f<Q6K>(s, a, m, epi)
+           : w.fmt == FMT_Q5K  ? launch_f<Q5K>(s, a, m, epi)
                                : launch_f<MX4>(s, a, m, epi);
 }
 

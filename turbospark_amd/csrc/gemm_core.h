@@ -104,6 +104,27 @@ struct Q4K {
     static __device__ __forceinline__ int xs_base(int c, int lane) { return c * 128 + ((lane >> 2) & 7) * 4; }
 };
 
+// Q5_K (crates/compute/src/quant_gguf/q5_k.rs:47-96): the Q4_K tile followed by the fifth bits,
+// [2 units][64 lanes][16 B] = the lane's 32 qh bytes.
+struct Q5K {
+    static constexpr int NSUB = 8, NPAIR = 4, TILE_BYTES = 11264;
+    static constexpr bool SUMS = true;
+    struct Regs {
+        u32x4 q[8];
+        u32x4 s;
+        u32x4 h[2];
+    };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* tile, int lane) {
+        const u32x4* p = (const u32x4*)tile + lane;
+#pragma unroll
+        for (int u = 0; u < 8; u++) r.q[u] = __builtin_nontemporal_load(p + u * 64);
+        r.s = __builtin_nontemporal_load(p + 512);
+        r.h[0] = __builtin_nontemporal_load(p + 576);
+        r.h[1] = __builtin_nontemporal_load(p + 640);
+    }
+    static __device__ __forceinline__ int xs_base(int c, int lane) { return c * 128 + ((lane >> 2) & 7) * 4; }
+};
+
 struct Q80 {
     static constexpr int NSUB = 4, NPAIR = 2, TILE_BYTES = 8704;
     static constexpr bool SUMS = true;
@@ -217,6 +238,7 @@ struct RegSrc {
     __device__ __forceinline__ u32x4 unit(int u) const { return r.q[u]; }
     __device__ __forceinline__ auto scales() const { return r.s; }
     __device__ __forceinline__ auto dval() const { return r.d; }
+    __device__ __forceinline__ u32x4 high(int u) const { return r.h[u]; }
 };
 template <class F>
 struct LdsSrc {
@@ -350,6 +372,70 @@ __device__ __forceinline__ void compute_tile(Q4K, const Src& w, const XRegs<Q4K,
             fma4(t[g], sc[2 * p + 1], dhi[g]);
         }
     }
+#pragma unroll
+    for (int g = 0; g < NG; g++) acc[g] += t[g];
+}
+
+// One Q5_K superblock tile: Q4_K's sequence with the fifth bit of every code OR-ed into the fp16
+// integer before the MFMA (bit 4 of 1024 + q for the low-nibble elements, bit 8 of the 1/16-ulp
+// 64 + q form for the high-nibble ones).  Byte l of the lane's 32 qh bytes serves elements l of all
+// eight sub-blocks: sub-block pair p reads bit 2p (low nibbles) and bit 2p + 1 (high nibbles).
+template <int NG, class Src>
+__device__ __forceinline__ void compute_tile(Q5K, const Src& w, const XRegs<Q5K, NG>& x, const Consts& k,
+                                             float4v (&acc)[NG]) {
+    const u32x4 hs = w.scales();
+    const float d = h2f_lo(hs.x), dmin = h2f_hi(hs.x);
+    const uint32_t sl = hs.y & 0x3F3F3F3Fu, ml = hs.z & 0x3F3F3F3Fu;
+    const uint32_t sh = (hs.w & 0x0F0F0F0Fu) | ((hs.y >> 2) & 0x30303030u);
+    const uint32_t mh = ((hs.w >> 4) & 0x0F0F0F0Fu) | ((hs.z >> 2) & 0x30303030u);
+    float sc[8], cf[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        sc[j] = d * ubyte(j < 4 ? sl : sh, j & 3);
+        const float mn = dmin * ubyte(j < 4 ? ml : mh, j & 3);
+        cf[j] = -__builtin_fmaf(sc[j], (j & 1) ? 64.0f : 1024.0f, mn);
+    }
+    float4v t[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) t[g] = float4v{0.f, 0.f, 0.f, 0.f};
+    static_for<8>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+#pragma unroll
+        for (int g = 0; g < NG; g++) t[g] = mfma_f32<j>(x.xs[g], cf[j], t[g]);
+    });
+    const u32x4 h0 = w.high(0), h1 = w.high(1);
+    static_for<4>([&](auto P) {
+        constexpr int p = decltype(P)::value;
+        const u32x4 qa = w.unit(2 * p), qb = w.unit(2 * p + 1);
+        float4v dlo[NG], dhi[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) dlo[g] = dhi[g] = float4v{0.f, 0.f, 0.f, 0.f};
+        static_for<8>([&](auto W) {
+            constexpr int wi = decltype(W)::value;
+            const uint32_t word = wi < 4 ? qa[wi % 4] : qb[wi % 4];
+            const uint32_t hw = wi < 4 ? h0[wi % 4] : h1[wi % 4];
+            const uint32_t v = word >> 8, hv = hw >> 8;
+            // bit 2p of a qh byte -> bit 4 of its fp16 half; bit 2p + 1 -> bit 8
+            constexpr int slo = 4 - 2 * p, shi = 7 - 2 * p;
+            const uint32_t l0 = slo >= 0 ? hw << (slo >= 0 ? slo : 0) : hw >> (slo < 0 ? -slo : 0);
+            const uint32_t l1 = slo >= 0 ? hv << (slo >= 0 ? slo : 0) : hv >> (slo < 0 ? -slo : 0);
+            const uint32_t u0 = hw << shi, u1 = hv << shi;
+            const u32x2 blo = {and_or(l0, 0x00100010u, and_or(word, 0x000F000Fu, k.k6400)),
+                               and_or(l1, 0x00100010u, and_or(v, 0x000F000Fu, k.k6400))};
+            const u32x2 bhi = {and_or(u0, 0x01000100u, and_or(word, 0x00F000F0u, k.k5400)),
+                               and_or(u1, 0x01000100u, and_or(v, 0x00F000F0u, k.k5400))};
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                dlo[g] = mfma_f16<wi>(x.xa[p][g], blo, dlo[g]);
+                dhi[g] = mfma_f16<wi + 8>(x.xa[p][g], bhi, dhi[g]);
+            }
+        });
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            fma4(t[g], sc[2 * p], dlo[g]);
+            fma4(t[g], sc[2 * p + 1], dhi[g]);
+        }
+    });
 #pragma unroll
     for (int g = 0; g < NG; g++) acc[g] += t[g];
 }

@@ -24,6 +24,7 @@ int64_t row_bytes(int dtype, int64_t cols) {
         case TSV_BF16: return cols * 2;
         case TSV_Q8_0: return cols % 32 ? -1 : cols / 32 * 34;
         case TSV_Q4_K: return cols % 256 ? -1 : cols / 256 * 144;
+        case TSV_Q5_K: return cols % 256 ? -1 : cols / 256 * 176;
         case TSV_Q6_K: return cols % 256 ? -1 : cols / 256 * 210;
         case TSV_MXFP4: return cols % 32 ? -1 : cols / 32 * 17;
     }
@@ -133,6 +134,61 @@ void encode_q4_k(const float* row, int64_t n, uint8_t* out) {
     }
 }
 
+// Q5_K: the reference only decodes it (crates/compute/src/quant_gguf/q5_k.rs:47-96); this encoder is
+// Q4_K's fitter with 31 levels per sub-block, for synthetic weights in that format.
+void encode_q5_k(const float* row, int64_t n, uint8_t* out) {
+    for (int64_t b = 0; b < n / 256; b++, row += 256, out += 176) {
+        float scale[8], mn[8], smax = 0.0f, mmax = 0.0f;
+        for (int j = 0; j < 8; j++) {
+            const float* s = row + 32 * j;
+            float lo = 0.0f;
+            for (int i = 0; i < 32; i++) lo = keep_min(lo, s[i]);
+            float hi = lo;
+            for (int i = 0; i < 32; i++) hi = keep_max(hi, s[i]);
+            scale[j] = (hi - lo) / 31.0f;
+            mn[j] = -lo;
+            smax = keep_max(smax, scale[j]);
+            mmax = keep_max(mmax, mn[j]);
+        }
+        const float is = smax > 0.0f ? 63.0f / smax : 0.0f;
+        const float im = mmax > 0.0f ? 63.0f / mmax : 0.0f;
+        uint8_t* packed = out + 4;
+        std::memset(packed, 0, 12);
+        for (int j = 0; j < 8; j++) {
+            const uint8_t ls = round_clamp_u8(scale[j] * is, 63.0f), lm = round_clamp_u8(mn[j] * im, 63.0f);
+            if (j < 4) {
+                packed[j] |= ls;
+                packed[j + 4] |= lm;
+            } else {
+                packed[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                packed[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                packed[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        const uint16_t db = f16_bits(smax / 63.0f), mb = f16_bits(mmax / 63.0f);
+        std::memcpy(out, &db, 2);
+        std::memcpy(out + 2, &mb, 2);
+        const float d = f16_value(db), dmin = f16_value(mb);
+        uint8_t q[256];
+        std::memset(q, 0, sizeof q);
+        for (int j = 0; j < 8; j++) {  // quants from the scales as a decoder will read them back
+            int sc, m;
+            unpack_scale_min(packed, j, sc, m);
+            const float step = d * (float)sc;
+            if (step == 0.0f) continue;
+            const float bias = dmin * (float)m;
+            for (int i = 0; i < 32; i++) q[32 * j + i] = round_clamp_u8((row[32 * j + i] + bias) / step, 31.0f);
+        }
+        std::memset(out + 16, 0, 32);  // qh: byte l serves element l of every sub-block (q5_k.rs:27-33)
+        for (int g = 0; g < 4; g++)
+            for (int l = 0; l < 32; l++) {
+                const uint8_t lo = q[64 * g + l], hi = q[64 * g + 32 + l];
+                out[48 + 32 * g + l] = (uint8_t)((lo & 0xF) | ((hi & 0xF) << 4));
+                out[16 + l] |= (uint8_t)(((lo >> 4) << (2 * g)) | ((hi >> 4) << (2 * g + 1)));
+            }
+    }
+}
+
 // Q6_K install encoder (crates/compute/src/quant_gguf/q6_k.rs:101-194): sub-block scale from the
 // signed element of largest magnitude, int8 scales against the largest through a negative
 // iscale, levels chosen against the f16-rounded d.
@@ -228,6 +284,7 @@ int encode_row(int dtype, const float* src, int64_t cols, uint8_t* dst) {
             return 0;
         case TSV_Q8_0: encode_q8_0(src, cols, dst); return 0;
         case TSV_Q4_K: encode_q4_k(src, cols, dst); return 0;
+        case TSV_Q5_K: encode_q5_k(src, cols, dst); return 0;
         case TSV_Q6_K: encode_q6_k(src, cols, dst); return 0;
         case TSV_MXFP4: encode_mxfp4(src, cols, dst); return 0;
     }

@@ -54,6 +54,24 @@ __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, 
             const uint8_t* blk = raw + (tok * (hidden / 32) + (e >> 5)) * 34;
             const float d = f16_bits_to_f32(*(const uint16_t*)blk);
             v = (float)(int8_t)blk[2 + (e & 31)] * d;
+        } else if (dtype == TSV_Q5_K) {  // q5_k.rs:47-96
+            const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 176;
+            const float d = f16_bits_to_f32(*(const uint16_t*)blk);
+            const float dmin = f16_bits_to_f32(*(const uint16_t*)(blk + 2));
+            const uint8_t* packed = blk + 4;
+            const int w = e & 255, g = w >> 6, hi = (w >> 5) & 1, l = w & 31, j = 2 * g + hi;
+            int sc, mn;
+            if (j < 4) {
+                sc = packed[j] & 63;
+                mn = packed[j + 4] & 63;
+            } else {
+                sc = (packed[j + 4] & 0xF) | ((packed[j - 4] >> 6) << 4);
+                mn = (packed[j + 4] >> 4) | ((packed[j] >> 6) << 4);
+            }
+            const uint8_t byte = blk[48 + 32 * g + l];
+            const int q = (hi ? (byte >> 4) : (byte & 0xF)) + (((blk[16 + l] >> j) & 1) << 4);
+            const float dl = d * (float)sc, ml = dmin * (float)mn;
+            v = __fsub_rn(__fmul_rn(dl, (float)q), ml);
         } else if (dtype == TSV_Q6_K) {  // q6_k.rs:44-88
             const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 210;
             const int w = e & 255, h = w >> 7, k = (w >> 5) & 3, l = w & 31;

@@ -251,6 +251,7 @@ int launch_moe_f(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
     return fmt == FMT_Q4K    ? launch_moe_t<Q4K, EPI>(s, a, n_groups)
            : fmt == FMT_Q80  ? launch_moe_t<Q80, EPI>(s, a, n_groups)
            : fmt == FMT_Q6K  ? launch_moe_t<Q6K, EPI>(s, a, n_groups)
+           : fmt == FMT_Q5K  ? launch_moe_t<Q5K, EPI>(s, a, n_groups)
            : fmt == FMT_BF16 ? launch_moe_t<BF16W, EPI>(s, a, n_groups)
                              : launch_moe_t<MX4, EPI>(s, a, n_groups);
 }

@@ -38,6 +38,7 @@ int dtype_fmt(int dtype) {
            : dtype == TSV_MXFP4 ? FMT_MX4
            : dtype == TSV_BF16  ? FMT_BF16
            : dtype == TSV_Q6_K  ? FMT_Q6K
+           : dtype == TSV_Q5_K  ? FMT_Q5K
                                 : -1;
 }
 
@@ -179,13 +180,13 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
         return TSV_ERR_INVALID;
     }
     if (fmt < 0) {
-        set_error(std::string(what) + ": matmul weights must be Q4_K, Q6_K, Q8_0, MXFP4 or bf16 in this build");
+        set_error(std::string(what) + ": matmul weights must be Q4_K, Q5_K, Q6_K, Q8_0, MXFP4 or bf16 in this build");
         return TSV_ERR_UNSUPPORTED;
     }
     // MXFP4 rows may end inside a 256-element chunk (the tile is padded with zero blocks)
     const int gran = fmt == FMT_MX4 ? 32 : fmt_chunk_elems(fmt);
     if (cols % gran || rows < 1) {
-        set_error(std::string(what) + ": K must be whole 256 (Q4_K, Q6_K) / 128 (Q8_0) / 64 (bf16) / 32 (MXFP4) element runs");
+        set_error(std::string(what) + ": K must be whole 256 (Q4_K, Q5_K, Q6_K) / 128 (Q8_0) / 64 (bf16) / 32 (MXFP4) element runs");
         return TSV_ERR_UNSUPPORTED;
     }
     return TSV_OK;
@@ -1609,7 +1610,7 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
         const int tb = fmt_tile_bytes(fmt);
         for (size_t t = 0; t < w.bytes / tb; t++) {
             uint8_t* sc = &host[t * tb + 8192];
-            if (fmt == FMT_Q4K)
+            if (fmt == FMT_Q4K || fmt == FMT_Q5K)
                 for (int r = 0; r < 64; r++) {
                     sc[r * 16 + 1] = 0x20;
                     sc[r * 16 + 3] = 0x20;

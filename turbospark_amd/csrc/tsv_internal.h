@@ -54,7 +54,7 @@ const std::string& get_error();
 // every 32-element sub-block, [K/256][g][sub%8][i], which the matmul uses to take the
 // integer-code offsets and the Q4_K min term back out.
 // ---------------------------------------------------------------------------------------
-enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2, FMT_BF16 = 3, FMT_Q6K = 4 };
+enum { FMT_Q4K = 0, FMT_Q80 = 1, FMT_MX4 = 2, FMT_BF16 = 3, FMT_Q6K = 4, FMT_Q5K = 5 };
 
 struct TiledW {
     uint8_t* tiles = nullptr;  // device
@@ -67,7 +67,9 @@ struct TiledW {
 };
 
 inline int fmt_chunk_elems(int fmt) { return fmt == FMT_Q80 ? 128 : fmt == FMT_BF16 ? 64 : 256; }
-inline int fmt_tile_bytes(int fmt) { return fmt == FMT_Q4K ? 9216 : fmt == FMT_BF16 ? 8192 : fmt == FMT_Q6K ? 13568 : 8704; }
+inline int fmt_tile_bytes(int fmt) {
+    return fmt == FMT_Q4K ? 9216 : fmt == FMT_Q5K ? 11264 : fmt == FMT_BF16 ? 8192 : fmt == FMT_Q6K ? 13568 : 8704;
+}
 inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : fmt == FMT_BF16 ? 2 : fmt == FMT_Q6K ? 16 : 8; }
 constexpr int TILE_ROWS = 64;
 

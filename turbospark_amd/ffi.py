@@ -7,7 +7,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
 
-F32, F16, Q8_0, Q4_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 14, 30, 39
+F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 13, 14, 30, 39
 MAX_ROWS = 16
 
 

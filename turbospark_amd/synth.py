@@ -17,6 +17,10 @@ CONFIGS = {
     "small_q4_k_m": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
                          vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K,
                          overrides={(0, "wv"): ffi.Q6_K, (0, "w_down"): ffi.Q6_K, "lm_head": ffi.Q6_K, "embed": ffi.Q6_K}),
+    # the mix of a Q5_K_M file: Q5_K, with Q6_K on the value / down projections of a layer and on the head
+    "small_q5_k_m": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
+                         vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q5_K,
+                         overrides={(1, "wv"): ffi.Q6_K, (1, "w_down"): ffi.Q6_K, "lm_head": ffi.Q6_K}),
     # the smallest shapes the per-XCD fused layer kernels take (8 KV heads, widths divisible
     # into eight chunk-aligned slices); norm weights are not all ones here
     "xcd_q4_k": dict(n_layers=2, hidden=1024, n_q_heads=32, n_kv_heads=8, head_dim=64, ffn=2048,
