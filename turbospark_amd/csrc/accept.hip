@@ -1071,9 +1071,32 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
 // survives the next token is drawn from the p that is left.  No stop / budget bookkeeping.
 //
 // First every node's p and q are written out as dense f64 rows by the whole chip (work slots
-// 0..m-1 and m..2m-1); then one workgroup walks the tree.  A child test is two lookups; only a
-// rejection costs a pass over the vocabulary (slots 32 and 33 alternate as the residual, whose
-// normalising division is applied when it is read, so a pass reads two rows and writes one).
+// 0..m-1 and m..2m-1); then the tree is walked one child test per launch.  A test is two lookups;
+// only a rejection costs a pass over the vocabulary (slots 32 and 33 alternate as the residual,
+// whose normalising division is applied when it is read, so a pass reads two rows and writes one).
+constexpr int TREE_SCRATCH_SLOT = 2 * TSV_MAX_ROWS;  // two residual rows behind the 32 distribution rows
+
+// The walk as a sequence of short chip-wide launches (one per child test there can be, then the
+// finish): every workgroup re-derives the step's decision from the walk state (two lookups), a
+// rejection's residual pass is spread over all of them, and the pass's total is folded by the next
+// launch.  The state and the partial sums are double-buffered: launch k reads copy k & 1 and writes the
+// other one, so a workgroup that starts late still sees what the previous launch left.
+constexpr int TREE_WGS = 256;
+struct TreeWalk {
+    int32_t at, next_s, plen, which, done, pending, src_slot, pend_slot;
+    double Z, margin;
+    uint64_t ds;
+    int32_t path[TSV_MAX_ROWS + 1];
+    int32_t pad;
+};
+static_assert(sizeof(TreeWalk) % 8 == 0 && sizeof(TreeWalk) <= 32 * 8, "fits its slot of the statistics block");
+
+// behind the decisions: two copies of the state (32 doubles each), then two sets of TREE_WGS partial sums
+constexpr int STATS_DOUBLES = 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG * NSUB + MAX_JOBS * 16;
+constexpr int TREE_STATE_DOUBLES = 2 * 32 + 2 * TREE_WGS;
+__device__ TreeWalk* tree_walk(double* scratch, int copy) { return (TreeWalk*)(scratch + STATS_DOUBLES + 32 * copy); }
+__device__ double* tree_partials(double* scratch, int copy) { return scratch + STATS_DOUBLES + 64 + TREE_WGS * copy; }
+
 template <bool PEN>
 __global__ __launch_bounds__(256) void k_tree_probs(const uint16_t* target, const uint16_t* draft,
                                                     const AcceptParams* app, double* scratch, double* work) {
@@ -1091,6 +1114,18 @@ __global__ __launch_bounds__(256) void k_tree_probs(const uint16_t* target, cons
     const double inv_t = 1.0 / ap.temperature;
     const uint16_t* lp = row_ptr(target, draft, ap.m, vocab, row);
     double* out = work + (long)row * vocab;
+    if (seg == 0 && row == 0 && threadIdx.x == 0) {  // the walk starts at the root
+        TreeWalk w;
+        w.at = 0;
+        w.next_s = 1;
+        w.plen = 1;
+        w.which = w.done = w.pending = w.src_slot = w.pend_slot = w.pad = 0;
+        w.Z = 1.0;
+        w.margin = 1.0;
+        w.ds = ap.draw_step;
+        w.path[0] = 0;
+        *tree_walk(scratch, 0) = w;
+    }
     const int per = (vocab + NSEG - 1) / NSEG, v0 = seg * per, v1 = min(v0 + per, vocab);
     for (int v = v0 + threadIdx.x; v < v1; v += 256) {
         const uint16_t b = lp[v];
@@ -1099,100 +1134,116 @@ __global__ __launch_bounds__(256) void k_tree_probs(const uint16_t* target, cons
     }
 }
 
-constexpr int TREE_SCRATCH_SLOT = 2 * TSV_MAX_ROWS;  // two residual rows behind the 32 distribution rows
+// The state launch k starts from: copy k & 1 with the previous launch's residual pass resolved
+// (its total decides whether the residual replaces the node's distribution: distribution.rs:96-126).
+__device__ TreeWalk tree_state(double* scratch, int k, double* red) {
+    TreeWalk w = *tree_walk(scratch, k & 1);
+    if (w.pending) {
+        const double part = (int)threadIdx.x < TREE_WGS ? tree_partials(scratch, k & 1)[threadIdx.x] : 0.0;
+        const double total = block_sum_f64(part, red);
+        if (total >= 1e-12) {
+            w.src_slot = w.pend_slot;
+            w.Z = total;
+            w.which ^= 1;
+        }
+        w.pending = 0;
+    }
+    return w;
+}
 
 template <bool PEN>
-__global__ __launch_bounds__(1024) void k_tree_sampled(const uint16_t* target, const AcceptParams* app,
-                                                       double* scratch, double* work, unsigned long long* hist,
-                                                       Decision* dec_out, int32_t* path_out) {
-    __shared__ double red[16];
-    __shared__ int s_accept;
-    __shared__ double s_margin;
+__global__ __launch_bounds__(256) void k_tree_step(const AcceptParams* app, double* scratch, double* work, int k) {
+    __shared__ double red[4];
     const AcceptParams& ap = *app;
-    const int tid = threadIdx.x;
     const int vocab = ap.vocab, m = ap.m;
-    Layout L = layout(scratch);
-    unsigned long long* hr = hist + 65536;
-    uint64_t ds = ap.draw_step;
-    int at = 0, plen = 1;
-    if (tid == 0) {
-        path_out[0] = 0;
-        s_margin = 1.0;
-    }
-    __syncthreads();
-    for (;;) {
-        const double* src = work + (long)at * vocab;  // the node's p; its values are src[v] / Z
-        const double* q = work + (long)(m + at) * vocab;
-        double Z = 1.0;
-        int which = 0, hit = -1;
-        for (int s = 1; s < m && hit < 0; s++) {
-            if (ap.parent[s] != at) continue;
-            if (tid == 0) {
-                const int32_t x = ap.feed[s];
-                const double r = unit_draw(ap.seed, ds);
-                const double px = src[x] / Z, qx = q[x];
-                double mg = s_margin;
-                fold_margin(mg, r * qx, px);
-                s_margin = mg;
-                s_accept = r * qx <= px;
-            }
-            ds += 1;
-            __syncthreads();
-            const bool ok = s_accept != 0;
-            __syncthreads();
-            if (ok) {
-                hit = s;
+    TreeWalk w = tree_state(scratch, k, red);
+    TreeWalk* out = tree_walk(scratch, (k + 1) & 1);
+    const bool writer = blockIdx.x == 0 && threadIdx.x == 0;
+    int s = -1;
+    if (!w.done)
+        for (int c = w.next_s; c < m; c++)
+            if (ap.parent[c] == w.at) {
+                s = c;
                 break;
             }
-            // residual: max(p - q, 0), normalised later by its total
-            double* dst = work + (long)(TREE_SCRATCH_SLOT + which) * vocab;
-            double acc = 0.0;
-            for (int v = tid; v < vocab; v += 1024) {
-                const double mv = fmax(src[v] / Z - q[v], 0.0);
-                dst[v] = mv;
-                acc += mv;
-            }
-            const double total = block_sum_f64(acc, red);
-            __threadfence_block();
-            __syncthreads();
-            if (total >= 1e-12) {  // distribution.rs:96-126: below that the distribution is kept
-                src = dst;
-                Z = total;
-                which ^= 1;
-            }
-        }
-        if (hit >= 0) {
-            if (tid == 0) path_out[plen] = hit;
-            plen += 1;
-            at = hit;
-            continue;
-        }
-        // nothing accepted below `at`: the next token is drawn from what is left of p
-        const uint16_t* lpk = target + (long)at * vocab;
-        for (int v = tid; v < vocab; v += 1024) {
-            const double mv = src[v] / Z;
-            if (mv > 0.0) {
-                const uint16_t b = lpk[v];
-                atomicAdd(hr + bin_addr(key_of<PEN>(score_of<PEN>(ap, at, v, b), b)), (unsigned long long)(mv * FIX));
-            }
-        }
-        // the draw divides the stored values by the fold of these pieces: Z, exactly
-        if (tid < NSEG * NSUB) L.segtot[tid] = tid == 0 ? Z : 0.0;
-        if (tid == 0) {
-            Decision d;
-            d.job.mode = 2;
-            d.job.row_p = at;
-            d.job.row_q = 0;
-            d.job.u = unit_draw(ap.seed, ds);
-            d.accepted = plen - 1;
-            d.committed = plen - 1;
-            d.stopped = 0;
-            d.pad = (int32_t)((src - work) / vocab);  // the work slot the draw reads
-            d.draw_step = ds + 1;
-            d.margin = s_margin;
-            dec_out[0] = d;
-        }
+    if (s < 0) {  // nothing left to try below this node (or the walk had ended already)
+        w.done = 1;
+        if (writer) *out = w;
         return;
+    }
+    const double* src = work + (long)w.src_slot * vocab;  // the node's p; its values are src[v] / Z
+    const double* q = work + (long)(m + w.at) * vocab;
+    const int32_t x = ap.feed[s];
+    const double r = unit_draw(ap.seed, w.ds);
+    const double px = src[x] / w.Z, qx = q[x];
+    fold_margin(w.margin, r * qx, px);
+    w.ds += 1;
+    w.next_s = s + 1;
+    if (r * qx <= px) {
+        w.path[w.plen] = s;
+        w.plen += 1;
+        w.at = s;
+        w.src_slot = s;
+        w.Z = 1.0;
+        w.which = 0;
+        if (writer) *out = w;
+        return;
+    }
+    // residual max(p - q, 0) of this workgroup's slice; the next launch folds the totals
+    double* dst = work + (long)(TREE_SCRATCH_SLOT + w.which) * vocab;
+    const int per = (vocab + TREE_WGS - 1) / TREE_WGS, v0 = blockIdx.x * per, v1 = min(v0 + per, vocab);
+    double acc = 0.0;
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const double mv = fmax(src[v] / w.Z - q[v], 0.0);
+        dst[v] = mv;
+        acc += mv;
+    }
+    acc = block_sum_f64(acc, red);
+    if (threadIdx.x == 0) tree_partials(scratch, (k + 1) & 1)[blockIdx.x] = acc;
+    w.pending = 1;
+    w.pend_slot = TREE_SCRATCH_SLOT + w.which;
+    if (writer) *out = w;
+}
+
+// After the last step: the rank histogram of what is left of p at the node the walk ended on, and the
+// round's decision; the draw itself is k_pick's.
+template <bool PEN>
+__global__ __launch_bounds__(256) void k_tree_finish(const uint16_t* target, const AcceptParams* app, double* scratch,
+                                                     double* work, unsigned long long* hist, Decision* dec_out,
+                                                     int32_t* path_out, int k) {
+    __shared__ double red[4];
+    const AcceptParams& ap = *app;
+    const int vocab = ap.vocab;
+    const TreeWalk w = tree_state(scratch, k, red);
+    Layout L = layout(scratch);
+    unsigned long long* hr = hist + 65536;
+    const double* src = work + (long)w.src_slot * vocab;
+    const uint16_t* lpk = target + (long)w.at * vocab;
+    const int per = (vocab + TREE_WGS - 1) / TREE_WGS, v0 = blockIdx.x * per, v1 = min(v0 + per, vocab);
+    for (int v = v0 + threadIdx.x; v < v1; v += 256) {
+        const double mv = src[v] / w.Z;
+        if (mv > 0.0) {
+            const uint16_t b = lpk[v];
+            atomicAdd(hr + bin_addr(key_of<PEN>(score_of<PEN>(ap, w.at, v, b), b)), (unsigned long long)(mv * FIX));
+        }
+    }
+    if (blockIdx.x != 0) return;
+    // the draw divides the stored values by the fold of these pieces: Z, exactly
+    if (threadIdx.x < NSEG * NSUB) L.segtot[threadIdx.x] = threadIdx.x == 0 ? w.Z : 0.0;
+    if (threadIdx.x == 0) {
+        for (int i = 0; i < w.plen; i++) path_out[i] = w.path[i];
+        Decision d;
+        d.job.mode = 2;
+        d.job.row_p = w.at;
+        d.job.row_q = 0;
+        d.job.u = unit_draw(ap.seed, w.ds);
+        d.accepted = w.plen - 1;
+        d.committed = w.plen - 1;
+        d.stopped = 0;
+        d.pad = w.src_slot;  // the work slot the draw reads
+        d.draw_step = w.ds + 1;
+        d.margin = w.margin;
+        dec_out[0] = d;
     }
 }
 
@@ -1299,9 +1350,7 @@ __global__ void k_clear_result(AcceptResult* res, int32_t* err) {
 
 // scratch.counters: [0] error flag, [16..32) greedy arg-max per row; decisions live after the
 // statistics block; histograms and work arrays are separate allocations in AcceptScratch.
-size_t accept_stats_doubles() {
-    return 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG * NSUB + MAX_JOBS * 16;
-}
+size_t accept_stats_doubles() { return STATS_DOUBLES + TREE_STATE_DOUBLES; }
 
 static Decision* decisions(const AcceptScratch& sc) {
     return (Decision*)(sc.stats + 4 * MAX_DIST_ROWS + 3 * MAX_DIST_ROWS * NSEG + MAX_JOBS * NSEG * NSUB);
@@ -1357,8 +1406,11 @@ static void launch_tree_sampled(hipStream_t s, const uint16_t* target, const uin
     // statistics of the m target rows and the m rows the children were drawn from
     launch_stats<PEN>(s, target, draft, ap.m, 2 * ap.m, 2 * 65536, ap_dev, ap, sc);
     hipLaunchKernelGGL(k_tree_probs<PEN>, dim3(NSEG, 2 * ap.m), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
-    hipLaunchKernelGGL(k_tree_sampled<PEN>, dim3(1), dim3(1024), 0, s, target, ap_dev, sc.stats, sc.work,
-                       (unsigned long long*)sc.hist, decisions(sc), path);
+    // every slot behind the root is tested at most once: m - 1 steps cover any walk
+    for (int k = 0; k < ap.m - 1; k++)
+        hipLaunchKernelGGL(k_tree_step<PEN>, dim3(TREE_WGS), dim3(256), 0, s, ap_dev, sc.stats, sc.work, k);
+    hipLaunchKernelGGL(k_tree_finish<PEN>, dim3(TREE_WGS), dim3(256), 0, s, target, ap_dev, sc.stats, sc.work,
+                       (unsigned long long*)sc.hist, decisions(sc), path, ap.m - 1);
     hipLaunchKernelGGL(k_pick<PEN>, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);
 }

@@ -350,9 +350,12 @@ __device__ __forceinline__ long v_index(int h, int pos, int d, int hd, int max_c
 
 // Tree compaction (families/qwen/dflash_tree.rs:106-207): rows of slots path[0..n) move to
 // base..base+n.  path is strictly increasing with path[i] >= i, so walking i upward never
-// overwrites a row that is still to be read.  One workgroup per kv head, sequential over i.
-__global__ void k_kv_gather(uint16_t* kc, uint16_t* vc, int hd, int max_ctx, const int32_t* path, int n,
-                            int base) {
+// overwrites a row that is still to be read.  One workgroup per (kv head, layer), sequential over i:
+// every layer's cache in one launch.
+__global__ void k_kv_gather(uint16_t* const* caches, int hd, int max_ctx, const int32_t* path, int n, int base) {
+    // grid (kv heads, layers): caches[2 * layer] is the layer's K buffer, [2 * layer + 1] its V buffer
+    uint16_t* kc = caches[2 * blockIdx.y];
+    uint16_t* vc = caches[2 * blockIdx.y + 1];
     const int h = blockIdx.x, d = threadIdx.x;
     for (int i = 0; i < n; i++) {
         const int src = base + path[i], dst = base + i;
@@ -364,9 +367,9 @@ __global__ void k_kv_gather(uint16_t* kc, uint16_t* vc, int hd, int max_ctx, con
     }
 }
 
-int launch_kv_gather(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx,
+int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, int n_layers, int nkv, int hd, int max_ctx,
                      const int32_t* path_dev, int n, int base) {
-    hipLaunchKernelGGL(k_kv_gather, dim3(nkv), dim3(128), 0, s, kc, vc, hd, max_ctx, path_dev, n, base);
+    hipLaunchKernelGGL(k_kv_gather, dim3(nkv, n_layers), dim3(128), 0, s, caches_dev, hd, max_ctx, path_dev, n, base);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -87,6 +87,7 @@ struct tsv_ctx {
     uint16_t* draft_stage = nullptr;  // [16][vocab] fp16, device
     VerifyParams *vp_dev = nullptr, *vp_host = nullptr;
     AcceptParams *ap_dev = nullptr, *ap_host = nullptr;
+    uint16_t** kv_ptrs = nullptr;  // device: [2 * layer] = K buffer, [2 * layer + 1] = V buffer (tree compaction)
     int32_t* hist_dev = nullptr;  // the token history of a penalised round (grows on demand)
     size_t hist_cap = 0;
     uint32_t* pen_cnt = nullptr;  // [vocab] seen flag + generated-suffix count per token
@@ -846,6 +847,16 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         pneed = std::max(pneed, std::max(partial_need(L.qkv), partial_need(L.wo)));
         pneed = std::max(pneed, (size_t)8 * 16 * ((size_t)(qd + 2 * kvd) + TILE_ROWS));
     }
+    {
+        std::vector<uint16_t*> ptrs;
+        for (auto& L : c->layers) {
+            ptrs.push_back(L.kc);
+            ptrs.push_back(L.vc);
+        }
+        if ((rc = dev_alloc(c, &c->kv_ptrs, ptrs.size() * sizeof(uint16_t*)))) return fail(rc);
+        if (hipMemcpy(c->kv_ptrs, ptrs.data(), ptrs.size() * sizeof(uint16_t*), hipMemcpyHostToDevice) != hipSuccess)
+            return fail(TSV_ERR_DEVICE);
+    }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
     if (!d->embed.data || d->embed.rows != c->vocab || d->embed.cols != c->hidden || erb < 0) {
@@ -1108,11 +1119,7 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
     TSV_HIP(hipStreamSynchronize(c->stream));
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
-    for (auto& L : c->layers) {
-        int rc = launch_kv_gather(c->stream, L.kc, L.vc, c->nkv, c->hd, c->ctx_alloc, c->tok_dev + 32, n, (int)base);
-        if (rc) return rc;
-    }
-    return TSV_OK;
+    return launch_kv_gather(c->stream, c->kv_ptrs, c->n_layers, c->nkv, c->hd, c->ctx_alloc, c->tok_dev + 32, n, (int)base);
 }
 
 namespace {

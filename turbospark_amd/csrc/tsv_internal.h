@@ -251,7 +251,7 @@ struct AttnArgs {
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
 
-int launch_kv_gather(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx,
+int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, int n_layers, int nkv, int hd, int max_ctx,
                      const int32_t* path_dev, int n, int base);
 int launch_kv_fill(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0, int n,
                    const uint16_t* k_in, const uint16_t* v_in);
