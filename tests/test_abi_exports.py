@@ -80,3 +80,46 @@ def test_product_sources_never_touch_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(base, f), errors="replace").read()
                 assert "tsoracle" not in text and "from oracle" not in text and "import oracle" not in text, f
+
+
+def test_null_handles_are_refused_by_name_without_a_gpu():
+    """Every entry point that takes a handle answers a null one with an error (or -1 / null for the plain
+    getters) before any device call is made; a descriptor with a zero head count is refused by tsv_open."""
+    import ctypes as C
+    from turbospark_amd import ffi
+    L = ffi.lib()
+    assert L.tsv_kv_position(None) == -1 and L.tsv_max_context(None) == -1 and L.tsv_vocab(None) == -1
+    assert L.tsv_stream(None) is None and L.tsv_device_logits(None) is None
+    L.tsv_close(None)
+    point = ffi.Point()
+    tok = (C.c_int32 * 4)(1, 2, 3, 4)
+    out = (C.c_uint16 * 8)()
+    calls = [
+        lambda: L.tsv_reset(None),
+        lambda: L.tsv_set_profile(None, 1),
+        lambda: L.tsv_set_repeat(None, 0, 1),
+        lambda: L.tsv_get_profile(None, None, None, 0),
+        lambda: L.tsv_checkpoint(None, C.byref(point)),
+        lambda: L.tsv_rollback(None, C.byref(point)),
+        lambda: L.tsv_rollback_retaining(None, C.byref(point), 0),
+        lambda: L.tsv_verify(None, tok, 4, 0, out),
+        lambda: L.tsv_verify_tree(None, tok, tok, 4, 0, out),
+        lambda: L.tsv_produce(None, 1, 0, out),
+        lambda: L.tsv_prefill(None, tok, 4, 0, out),
+        lambda: L.tsv_compact_tree(None, 0, tok, 1),
+        lambda: L.tsv_accept(None, None, None),
+        lambda: L.tsv_verify_accept(None, None, None),
+        lambda: L.tsv_read_kv(None, 0, 0, 1, out, out),
+        lambda: L.tsv_write_kv(None, 0, 0, 1, out, out),
+        lambda: L.tsv_write_logits(None, out, 1, 0),
+    ]
+    for i, call in enumerate(calls):
+        assert call() != 0, i
+        assert ffi.last_error(), i
+    desc = ffi.ModelDesc()
+    layers = (ffi.Layer * 1)()
+    desc.layers = C.cast(layers, type(desc.layers))
+    desc.n_layers, desc.hidden, desc.n_q_heads, desc.n_kv_heads, desc.head_dim = 1, 64, 4, 0, 64
+    desc.ffn, desc.vocab, desc.max_context = 64, 100, 16
+    handle = C.c_void_p()
+    assert L.tsv_open(C.byref(desc), C.byref(handle)) != 0 and "positive" in ffi.last_error()

@@ -361,6 +361,7 @@ int run_pass(tsv_ctx* c, int m);
 
 // One verify pass: enqueue everything on the handle's stream; no synchronisation.
 int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m, int64_t base) {
+    TSV_NEED(c, "verify: null handle");
     // batched.rs:106-185 refusals
     if (!feed || m < 1) {
         set_error("verify: empty feed");
@@ -699,6 +700,11 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         set_error("open: null argument");
         return TSV_ERR_INVALID;
     }
+    if (d->n_layers < 1 || !d->layers || d->hidden < 1 || d->n_q_heads < 1 || d->n_kv_heads < 1 || d->ffn < 1 ||
+        d->vocab < 1 || d->max_context < 1) {
+        set_error("open: layer count, widths, head counts, vocabulary and context must all be positive");
+        return TSV_ERR_INVALID;
+    }
     if (d->head_dim != 64 && d->head_dim != 128) {
         set_error("open: head_dim must be 64 or 128");
         return TSV_ERR_UNSUPPORTED;
@@ -987,6 +993,7 @@ extern "C" void tsv_close(tsv_ctx* c) {
 }
 
 extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
+    TSV_NEED(c, "set_profile: null handle");
     TSV_HIP(hipStreamSynchronize(c->stream));
     c->profile = on != 0;
     c->ev_used = 0;
@@ -994,6 +1001,7 @@ extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
 }
 
 extern "C" int32_t tsv_set_repeat(tsv_ctx* c, int32_t cls, int32_t times) {
+    TSV_NEED(c, "set_repeat: null handle");
     if (cls != PC_QKV && cls != PC_ROPE && cls != PC_ATTN && cls != PC_WO && cls != PC_GATEUP && cls != PC_DOWN &&
         cls != PC_HEAD) {
         set_error("set_repeat: only the matmul, rope and attention classes can be repeated");
@@ -1009,6 +1017,7 @@ extern "C" int32_t tsv_set_repeat(tsv_ctx* c, int32_t cls, int32_t times) {
 }
 
 extern "C" int32_t tsv_get_profile(tsv_ctx* c, float* ms, int32_t* counts, int32_t n_classes) {
+    TSV_NEED(c && ms && counts && n_classes >= 0, "get_profile: null handle or output");
     TSV_HIP(hipStreamSynchronize(c->stream));
     for (int i = 0; i < n_classes; i++) {
         ms[i] = 0.f;
@@ -1030,16 +1039,17 @@ extern "C" int32_t tsv_get_profile(tsv_ctx* c, float* ms, int32_t* counts, int32
 extern "C" void* tsv_stream(tsv_ctx* c) { return c ? (void*)c->stream : nullptr; }
 
 extern "C" int32_t tsv_reset(tsv_ctx* c) {
+    TSV_NEED(c, "reset: null handle");
     c->position = 0;
     c->last_m = 0;
     return TSV_OK;
 }
 
-extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c->position; }
+extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c ? c->position : -1; }
 extern "C" int64_t tsv_max_safe_rewind(const tsv_ctx*) { return INT64_MAX; }  // linear layout: nothing rings
 extern "C" const uint16_t* tsv_device_logits(tsv_ctx* c) { return c ? c->logits : nullptr; }
-extern "C" int64_t tsv_max_context(const tsv_ctx* c) { return c->max_context; }
-extern "C" int64_t tsv_vocab(const tsv_ctx* c) { return c->vocab; }
+extern "C" int64_t tsv_max_context(const tsv_ctx* c) { return c ? c->max_context : -1; }
+extern "C" int64_t tsv_vocab(const tsv_ctx* c) { return c ? c->vocab : -1; }
 
 extern "C" int32_t tsv_verify(tsv_ctx* c, const int32_t* feed, int32_t m, int64_t base, uint16_t* logits) {
     int rc = enqueue_verify(c, feed, nullptr, m, base);
@@ -1061,6 +1071,7 @@ extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint
 }
 
 extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
+    TSV_NEED(c && ids, "prefill: null handle or token list");
     if (n < 1) {
         set_error("prefill: empty token list");
         return TSV_ERR_INVALID;
@@ -1079,6 +1090,7 @@ extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_
 }
 
 extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {
+    TSV_NEED(c && out, "checkpoint: null handle or output");
     out->position = c->position;
     return TSV_OK;
 }
@@ -1086,6 +1098,7 @@ extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {
 // real_forward_rollback.rs:153-209 for a target without recurrent state: kv.rewind_by, a
 // cursor move (kv_cache_rewind.rs:46-55); rows past the cursor become unreachable.
 extern "C" int32_t tsv_rollback(tsv_ctx* c, const tsv_point* p) {
+    TSV_NEED(c && p, "rollback: null handle or point");
     if (p->position < 0 || p->position > c->position) {
         set_error("rollback: point is ahead of the KV cursor");
         return TSV_ERR_INVALID;
@@ -1095,7 +1108,8 @@ extern "C" int32_t tsv_rollback(tsv_ctx* c, const tsv_point* p) {
 }
 
 extern "C" int32_t tsv_rollback_retaining(tsv_ctx* c, const tsv_point* p, int32_t keep_rows) {
-    if (keep_rows < 0 || p->position + keep_rows > c->position) {
+    TSV_NEED(c && p, "rollback_retaining: null handle or point");
+    if (keep_rows < 0 || p->position < 0 || p->position + keep_rows > c->position) {
         set_error("rollback_retaining: keep_rows exceeds the rows the last verify wrote");
         return TSV_ERR_INVALID;
     }
@@ -1107,6 +1121,7 @@ extern "C" int32_t tsv_commit_pending(tsv_ctx*, int32_t) { return TSV_OK; }
 extern "C" int32_t tsv_discard_pending(tsv_ctx*) { return TSV_OK; }
 
 extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* path, int32_t n) {
+    TSV_NEED(c && path, "compact_tree: null handle or path");
     if (n < 1 || n > TSV_MAX_ROWS || path[0] != 0) {
         set_error("compact_tree: path must start at slot 0 and hold 1..16 slots");
         return TSV_ERR_INVALID;
@@ -1116,6 +1131,10 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
             set_error("compact_tree: path must be strictly increasing");
             return TSV_ERR_INVALID;
         }
+    if (base < 0 || base + (int64_t)path[n - 1] >= c->ctx_alloc) {
+        set_error("compact_tree: the block at `base` lies outside the KV cache");
+        return TSV_ERR_INVALID;
+    }
     TSV_HIP(hipStreamSynchronize(c->stream));
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
@@ -1335,14 +1354,18 @@ extern "C" int32_t tsv_draft_chain(tsv_ctx* c, const uint16_t* draft_logits, int
 }
 
 extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v) {
-    if (layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
-        set_error("read_kv: range outside the cache");
+    if (!c || !k || !v || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
+        set_error("read_kv: null argument or range outside the cache");
         return TSV_ERR_INVALID;
     }
     const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
     uint16_t *kd = nullptr, *vd = nullptr;
     TSV_HIP(hipMalloc((void**)&kd, bytes));
-    TSV_HIP(hipMalloc((void**)&vd, bytes));
+    if (hipMalloc((void**)&vd, bytes) != hipSuccess) {
+        (void)hipFree(kd);
+        set_error("KV staging buffer: out of device memory");
+        return TSV_ERR_DEVICE;
+    }
     int rc = launch_kv_read(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->ctx_alloc,
                             (int)pos0, (int)n, kd, vd);
     if (!rc) {
@@ -1380,7 +1403,11 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
     const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
     uint16_t *kd = nullptr, *vd = nullptr;
     TSV_HIP(hipMalloc((void**)&kd, bytes));
-    TSV_HIP(hipMalloc((void**)&vd, bytes));
+    if (hipMalloc((void**)&vd, bytes) != hipSuccess) {
+        (void)hipFree(kd);
+        set_error("KV staging buffer: out of device memory");
+        return TSV_ERR_DEVICE;
+    }
     int rc = TSV_OK;
     if (hipMemcpyAsync(kd, k, bytes, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
         hipMemcpyAsync(vd, v, bytes, hipMemcpyHostToDevice, c->stream) != hipSuccess) {

@@ -21,6 +21,14 @@ const std::string& get_error();
         }                                                                                   \
     } while (0)
 
+#define TSV_NEED(cond, msg)          \
+    do {                             \
+        if (!(cond)) {               \
+            tsv::set_error(msg);     \
+            return TSV_ERR_INVALID;  \
+        }                            \
+    } while (0)
+
 // ---------------------------------------------------------------------------------------
 // Device weight layout ("row tiles").  A matrix W[N][K] is cut into tiles of 64 output rows
 // by one K-chunk (256 elements for Q4_K, 128 for Q8_0); tiles are stored [row tile][chunk]
