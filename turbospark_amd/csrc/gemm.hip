@@ -29,6 +29,7 @@
 //    Neither split depends on the number of activation rows, so a row's result is the same
 //    bits whether it is verified alone or in a block.
 #include <algorithm>
+#include <cstdlib>
 
 #include "gemm_core.h"
 
@@ -414,6 +415,246 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     }
 }
 
+// ------------------------------------------------------------------------------- nine to sixteen rows
+// Passes of more than eight rows (draft trees, prompt blocks) over Q4_K weights run on
+// v_mfma_f32_16x16x32_f16 instead: one instruction multiplies sixteen activation rows by sixteen
+// weight rows over a whole 32-element sub-block, where the 4x4x4 form needs four row groups x
+// eight K steps.  The tile bytes are the same; only the lane mapping differs:
+//   lane (r, kg) = (lane % 16, lane / 16) of row block rb holds weight row 16 rb + r, elements
+//   8 kg .. 8 kg + 7 of a sub-block (the B operand), and activation row r, same elements (the A
+//   operand; rows past m multiply whatever the fragment buffer holds into output rows nobody
+//   stores);  the result registers of the lane are activation rows 4 kg .. 4 kg + 3 of weight
+//   row 16 rb + r.
+// The two nibbles of a tile byte are the same element of sub-blocks 2p and 2p + 1, so one 8-byte
+// load per (rb, p) feeds two MFMAs.  The code-offset / min term is one v_mfma_f32_16x16x4_f32 per
+// four sub-blocks: lane (r, kg) supplies the sum of sub-block kg (kg + 4) of activation row r and
+// the coefficient of weight row r for that sub-block.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+struct Stage16 {
+    u32x2 q[4][4];  // [row block][sub-block pair]
+    u32x4 h[4];     // scale header of the lane's weight row in each row block
+    u32x2 x[8][2];  // [sub-block][K step] activation fragments
+    float xs[2];    // activation sums of sub-blocks kg and kg + 4
+};
+
+__device__ __forceinline__ void load_stage16(Stage16& st, const GemmArgs& a, const uint8_t* tile_chunk, int c, int lane) {
+    const int r = lane & 15, kg = lane >> 4;
+    __builtin_amdgcn_sched_barrier(0);
+    // fragment units (8 bytes) of chunk c: [64-element block][row group][K step][row in group]
+    const u32x2* xp = (const u32x2*)a.xfrag + (size_t)c * 1024 + (r >> 2) * 64 + (r & 3) + kg * 8;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) st.x[j][t] = xp[(j >> 1) * 256 + ((j & 1) * 8 + t) * 4];
+    const float* sp = a.xsum + (size_t)c * 128 + (r >> 2) * 32 + (r & 3) + kg * 4;
+    st.xs[0] = sp[0];
+    st.xs[1] = sp[16];
+    const uint8_t* wp = tile_chunk + ((kg >> 1) * 64 + r) * 16 + (kg & 1) * 8;
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++)
+#pragma unroll
+        for (int p = 0; p < 4; p++) st.q[rb][p] = __builtin_nontemporal_load((const u32x2*)(wp + (2 * p * 64 + 16 * rb) * 16));
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) st.h[rb] = __builtin_nontemporal_load((const u32x4*)(tile_chunk + 8192 + (16 * rb + r) * 16));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void compute16(const Stage16& st, const Consts& k, float4v (&acc)[4], int kg) {
+    const float4v zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+        const u32x4 hs = st.h[rb];
+        const float d = h2f_lo(hs.x), dmin = h2f_hi(hs.x);
+        const uint32_t sl = hs.y & 0x3F3F3F3Fu, ml = hs.z & 0x3F3F3F3Fu;
+        const uint32_t sh = (hs.w & 0x0F0F0F0Fu) | ((hs.y >> 2) & 0x30303030u);
+        const uint32_t mh = ((hs.w >> 4) & 0x0F0F0F0Fu) | ((hs.z >> 2) & 0x30303030u);
+        float sc[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) sc[j] = d * ubyte(j < 4 ? sl : sh, j & 3);
+        // the lane's two coefficients of the offset term (sub-blocks kg and kg + 4 have kg's parity:
+        // even ones carry the 1024 code offset, odd ones 64)
+        const int sft = 8 * kg;
+        const float off = (kg & 1) ? 64.0f : 1024.0f;
+        const float cf_lo = -__builtin_fmaf(d * (float)((sl >> sft) & 0xFF), off, dmin * (float)((ml >> sft) & 0xFF));
+        const float cf_hi = -__builtin_fmaf(d * (float)((sh >> sft) & 0xFF), off, dmin * (float)((mh >> sft) & 0xFF));
+        float4v t = __builtin_amdgcn_mfma_f32_16x16x4f32(st.xs[0], cf_lo, zero, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_16x16x4f32(st.xs[1], cf_hi, t, 0, 0, 0);
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const u32x2 w = st.q[rb][p];
+            const uint32_t w0 = w.x, w1 = w.x >> 8, w2 = w.y, w3 = w.y >> 8;
+            const u32x4 blo = {and_or(w0, 0x000F000Fu, k.k6400), and_or(w1, 0x000F000Fu, k.k6400),
+                               and_or(w2, 0x000F000Fu, k.k6400), and_or(w3, 0x000F000Fu, k.k6400)};
+            const u32x4 bhi = {and_or(w0, 0x00F000F0u, k.k5400), and_or(w1, 0x00F000F0u, k.k5400),
+                               and_or(w2, 0x00F000F0u, k.k5400), and_or(w3, 0x00F000F0u, k.k5400)};
+            const u32x4 alo = {st.x[2 * p][0].x, st.x[2 * p][0].y, st.x[2 * p][1].x, st.x[2 * p][1].y};
+            const u32x4 ahi = {st.x[2 * p + 1][0].x, st.x[2 * p + 1][0].y, st.x[2 * p + 1][1].x, st.x[2 * p + 1][1].y};
+            const float4v dlo = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, alo),
+                                                                       __builtin_bit_cast(half8, blo), zero, 0, 0, 0);
+            const float4v dhi = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ahi),
+                                                                       __builtin_bit_cast(half8, bhi), zero, 0, 0, 0);
+            fma4(t, sc[2 * p], dlo);
+            fma4(t, sc[2 * p + 1], dhi);
+        }
+        acc[rb] += t;
+    }
+}
+
+// v0 / v1: the finished sums of row blocks pr and pr + 2 (weight rows 16 pr + r and 32 + 16 pr + r of
+// the tile); register i is activation row 4 kg + i.
+template <int EPI>
+__device__ __forceinline__ void epilogue16(const GemmArgs& a, int tile, int split, int pr, float4v v0, float4v v1,
+                                           int lane, int M, float* ssum) {
+    const int r = lane & 15, kg = lane >> 4;
+    if (EPI == EPI_SILU) {
+        // gate rows are the tile's first 32 rows, up rows the other 32: a lane holds both of a column
+        const int col = tile * 32 + 16 * pr + r;  // K index of the down projection
+        _Float16* out = (_Float16*)a.out;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const _Float16 h = (_Float16)(silu_f(v0[i]) * v1[i]);
+            float sum = (float)h;
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o);
+            const int b = 4 * kg + i;
+            if (b < M) out[frag_index(col, b)] = h;
+            if (r == 0) ssum[pr * 16 + b] = sum;  // this half of the sub-block's sum
+        }
+        return;
+    }
+    if (EPI == EPI_ROPE) {
+        const RopeEpi& e = a.rope;
+        const int hd = e.hd, half = hd >> 1, tph = hd >> 6;
+        const int tq = e.nq * tph, tk = e.nkv * tph;
+        const int kind = tile < tq ? 0 : tile < tq + tk ? 1 : 2;
+        const int st = kind == 0 ? tile : kind == 1 ? tile - tq : tile - tq - tk;
+        const int head = st / tph, t = st - head * tph;
+        const int idim = (tph == 2 ? 32 * t : 0) + 16 * pr + r;  // rotation pair index, 0 .. hd/2
+        const int d0 = kind == 2 ? t * 64 + 16 * pr + r : idim, d1 = kind == 2 ? d0 + 32 : idim + half;
+        const int sec = (kind == 0 ? 0 : kind == 1 ? e.nq * hd : (e.nq + e.nkv) * hd) + head * hd;
+        const float b0 = e.bias ? e.bias[sec + d0] : 0.f, b1 = e.bias ? e.bias[sec + d1] : 0.f;
+        const int base = a.vp->base;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int b = 4 * kg + i;
+            if (b >= M) continue;
+            const float x0 = v0[i] + b0, x1 = v1[i] + b1;
+            float y0 = x0, y1 = x1;
+            if (kind != 2) {
+                const float2 cs = e.cs[b * half + idim];
+                y0 = x0 * cs.x - x1 * cs.y;
+                y1 = x0 * cs.y + x1 * cs.x;
+            }
+            const _Float16 h0 = (_Float16)y0, h1 = (_Float16)y1;
+            if (kind == 0) {
+                _Float16* q = (_Float16*)e.q16 + ((long)b * e.nq + head) * hd;
+                q[d0] = h0;
+                q[d1] = h1;
+            } else {
+                const int pos = base + b;
+                if (kind == 1) {
+                    _Float16* kc = (_Float16*)e.kc + ((long)head * e.max_ctx + pos) * hd;
+                    kc[d0] = h0;
+                    kc[d1] = h1;
+                } else {
+                    _Float16* vb = (_Float16*)e.vc + ((long)head * (e.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
+                    const int po = pos & 15;
+                    vb[(((d0 >> 4) * 64) + (po >> 2) * 16 + (d0 & 15)) * 4 + (po & 3)] = h0;
+                    vb[(((d1 >> 4) * 64) + (po >> 2) * 16 + (d1 & 15)) * 4 + (po & 3)] = h1;
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+        const float4v v = hf ? v1 : v0;
+        const int n = tile * 64 + 16 * (pr + 2 * hf) + r;
+        if (n >= a.n_valid) continue;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int b = 4 * kg + i;
+            if (b >= M) continue;
+            if (EPI == EPI_PARTIAL)
+                ((float*)a.out)[((size_t)split * 16 + b) * a.ldo + n] = v[i];
+            else
+                ((_Float16*)a.out)[(size_t)b * a.ldo + n] = (_Float16)v[i];
+        }
+    }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(512) void k_gemm16(GemmArgs a) {
+    extern __shared__ float4v red[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
+    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
+    const int c0 = min(s0 + wave * a.per, s1);
+    const int nc = min(a.per, s1 - c0);
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q4K::TILE_BYTES;
+    Consts k;
+    k.k6400 = 0x64006400u;
+    k.k5400 = 0x54005400u;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400));
+    float4v acc[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int M = a.vp->m;
+    if (nc > 0) {
+        Stage16 st;
+        load_stage16(st, a, wt + (size_t)c0 * Q4K::TILE_BYTES, c0, lane);
+        for (int c = 1; c < nc; c++) {
+            compute16(st, k, acc, lane >> 4);
+            load_stage16(st, a, wt + (size_t)(c0 + c) * Q4K::TILE_BYTES, c0 + c, lane);
+        }
+        compute16(st, k, acc, lane >> 4);
+    }
+    // fold the waves' accumulators in wave order; wave w finishes the row-block pairs w, w + kparts
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) red[(wave * 4 + rb) * 64 + lane] = acc[rb];
+    __syncthreads();
+    float* ssum = (float*)(red + a.kparts * 256);
+    for (int pr = wave; pr < 2; pr += a.kparts) {
+        float4v v0 = red[pr * 64 + lane], v1 = red[(pr + 2) * 64 + lane];
+        for (int w = 1; w < a.kparts; w++) {
+            v0 += red[(w * 4 + pr) * 64 + lane];
+            v1 += red[(w * 4 + pr + 2) * 64 + lane];
+        }
+        epilogue16<EPI>(a, tile, split, pr, v0, v1, lane, M, ssum);
+    }
+    if (EPI == EPI_SILU) {
+        // a sub-block of the down projection is this tile's 32 columns: both halves' sums, then one store
+        __syncthreads();
+        if (threadIdx.x < 16 && (int)threadIdx.x < M) {
+            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
+            sums[xsum_index(tile, threadIdx.x)] = ssum[threadIdx.x] + ssum[16 + threadIdx.x];
+        }
+    }
+}
+
+static bool gemm16_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("TSV_GEMM16");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+static int launch16(hipStream_t s, const GemmArgs& a, int epi) {
+    const size_t lds = (size_t)a.kparts * 4096 + 128;
+    const dim3 grid(a.n_tiles * a.splits), block(64 * a.kparts);
+    switch (epi) {
+        case EPI_PARTIAL: hipLaunchKernelGGL(k_gemm16<EPI_PARTIAL>, grid, block, lds, s, a); break;
+        case EPI_ROPE: hipLaunchKernelGGL(k_gemm16<EPI_ROPE>, grid, block, lds, s, a); break;
+        case EPI_SILU: hipLaunchKernelGGL(k_gemm16<EPI_SILU>, grid, block, lds, s, a); break;
+        default: hipLaunchKernelGGL(k_gemm16<EPI_LOGITS>, grid, block, lds, s, a); break;
+    }
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
 // Chunks one wave should walk at least, by the amount of work there is to spread.
 static int pref_chunks_per_wave(const TiledW& w) {
     const long total = (long)w.n_tiles * w.kchunks;
@@ -497,6 +738,7 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
         }
         a.n_valid = w.n_rows / 2;  // K of the next matmul
     }
+    if (w.fmt == FMT_Q4K && m > 8 && gemm16_enabled()) return launch16(s, a, epi);
     return w.fmt == FMT_Q4K    ? launch_f<Q4K>(s, a, m, epi)
            : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
            : w.fmt == FMT_BF16 ? launch_f<BF16W>(s, a, m, epi)
