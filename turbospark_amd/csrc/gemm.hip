@@ -634,12 +634,15 @@ __global__ __launch_bounds__(512) void k_gemm16(GemmArgs a) {
     }
 }
 
-static bool gemm16_enabled() {
-    static const bool on = [] {
+// Fewest rows that go to the 16x16x32 form (TSV_GEMM16=0: never; TSV_GEMM16=<n>: from n rows on).
+static int gemm16_min_rows() {
+    static const int n = [] {
         const char* e = getenv("TSV_GEMM16");
-        return !(e && e[0] == '0');
+        if (!e) return 9;
+        const int v = atoi(e);
+        return v <= 0 ? TSV_MAX_ROWS + 1 : v;
     }();
-    return on;
+    return n;
 }
 
 static int launch16(hipStream_t s, const GemmArgs& a, int epi) {
@@ -738,7 +741,7 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
         }
         a.n_valid = w.n_rows / 2;  // K of the next matmul
     }
-    if (w.fmt == FMT_Q4K && m > 8 && gemm16_enabled()) return launch16(s, a, epi);
+    if (w.fmt == FMT_Q4K && m >= gemm16_min_rows()) return launch16(s, a, epi);
     return w.fmt == FMT_Q4K    ? launch_f<Q4K>(s, a, m, epi)
            : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
            : w.fmt == FMT_BF16 ? launch_f<BF16W>(s, a, m, epi)
