@@ -185,6 +185,38 @@ int32_t tsv_rollback(tsv_ctx* ctx, const tsv_point* point);        /* rollback()
 int32_t tsv_rollback_retaining(tsv_ctx* ctx, const tsv_point* point, int32_t keep_rows);
 int32_t tsv_commit_pending(tsv_ctx* ctx, int32_t keep_rows); /* no-op without recurrent state */
 int32_t tsv_discard_pending(tsv_ctx* ctx);
+
+/* ---- what the KV rows were built from (crates/runtime/src/kv_prefix.rs:49-137) ---------
+ * The record on its own: pure host state, no GPU.  fed[0..len) are the token ids behind positions
+ * [0, len); a state that took in anything the ids do not describe is tainted until cleared. */
+typedef struct tsv_prefix tsv_prefix;
+tsv_prefix* tsv_prefix_new(void);
+void tsv_prefix_free(tsv_prefix* p);
+void tsv_prefix_clear(tsv_prefix* p);                                     /* clear() :60-63 */
+void tsv_prefix_taint(tsv_prefix* p);                                     /* taint() :68-70 */
+/* record(tokens, pos0) :79-92: starting inside the record replaces its tail, past its end taints. */
+void tsv_prefix_record(tsv_prefix* p, const int32_t* tokens, int64_t n, int64_t pos0);
+void tsv_prefix_rewind_to(tsv_prefix* p, int64_t position);               /* rewind_to() :96-100 */
+int64_t tsv_prefix_untainted_len(const tsv_prefix* p);                    /* untainted_len() :104-106; -1 = None */
+/* common_prefix(prompt) :129-137: longest common prefix, at most n - 1 (one token is always left to feed). */
+int64_t tsv_prefix_common(const tsv_prefix* p, const int32_t* prompt, int64_t n);
+
+/* The same record behind a handle.  It is written where tokens are fed: tsv_produce and
+ * tsv_prefill on success (real_forward_traits.rs:135-152, :395-402; a failed pass taints),
+ * tsv_record_committed after a verify round; tsv_reset clears it, the rollbacks and the fused
+ * round's truncation shorten it, tsv_write_kv taints it (rows no ids describe).
+ * RealForwardRunner::set_prefix_reuse: reuse answers 0 until the host opts in. */
+int32_t tsv_set_prefix_reuse(tsv_ctx* ctx, int32_t on);
+/* LogitProducer::try_reuse_prefix (producer.rs:24-47, real_forward_traits.rs:173-289): commits to
+ * continuing from the current state for the leading N tokens of the prompt and returns N (0: no
+ * reuse, the caller resets; < 0: error).  A cursor that runs past the agreed prefix is moved back
+ * to it, within tsv_max_safe_rewind. */
+int64_t tsv_try_reuse_prefix(tsv_ctx* ctx, const int32_t* prompt, int64_t n);
+/* SpeculativeProducer::record_committed(tokens, pos0) (producer.rs:322-330): the rows of a verify
+ * pass that the round committed, `feed[..committed + 1]` at `base` (speculative.rs:828-836). */
+int32_t tsv_record_committed(tsv_ctx* ctx, const int32_t* tokens, int64_t n, int64_t pos0);
+/* Positions the handle's record describes; -1 when tainted. */
+int64_t tsv_prefix_len(const tsv_ctx* ctx);
 /* verify(feed, base, logits): m rows at base..base+m, row i sees [0, base+i].
  * logits nullable (m x vocab fp16): NULL keeps them on the device for tsv_accept. */
 int32_t tsv_verify(tsv_ctx* ctx, const int32_t* feed, int32_t m, int64_t base, uint16_t* logits);
@@ -240,6 +272,10 @@ typedef struct {
      * by the time it returns; the draws and the round then read the drafter's rows where they are.  No
      * counterpart in the reference, whose draft_step hands back host logits (producer.rs:196-204). */
     int32_t device_logits;
+    /* optional (may be NULL): how many positions the drafter's own context covers.  The loop reuses
+     * a prefix only when this is within one row of it (the drafter continuity guard of
+     * real_forward_traits.rs:199-239); without it a run always starts from an empty state. */
+    int64_t (*position)(void* user);
 } tsv_drafter;
 
 typedef struct {
@@ -261,11 +297,13 @@ typedef struct {
     uint64_t draw_step;
     int64_t kv_position;
     double min_margin;
+    int64_t reused;      /* leading prompt tokens taken over from the previous run's state */
 } tsv_generation_result;
 
-/* run_speculative for the step-wise drafter and chain rounds: admission, headless prefill that
- * primes the drafter, then rounds of draft -> verify + accept + truncate on the device ->
- * rewind_drafter, never proposing past the budget or the context window (speculative.rs:448-459). */
+/* run_speculative for the step-wise drafter and chain rounds: admission, prefix reuse or reset
+ * (speculative.rs:240-251), headless prefill that primes the drafter, then rounds of draft ->
+ * verify + accept + truncate on the device -> record_committed -> rewind_drafter, never proposing
+ * past the budget or the context window (speculative.rs:448-459). */
 int32_t tsv_run_speculative(tsv_ctx* ctx, const tsv_drafter* drafter, const int32_t* prompt, int64_t n_prompt,
                             const tsv_generation* config, tsv_generation_result* out);
 /* Device address of the logits the last pass left on the GPU (rows x vocab fp16, valid until the next

@@ -133,7 +133,30 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
     Emit emit{out};
 
     int rc;
-    if ((rc = tsv_reset(c))) return rc;
+    // The reuse contract (speculative.rs:240-251): ask how much of this prompt the state already
+    // covers and reset only when the answer is none.  The drafter's context is not part of the
+    // target's state, so a prefix is taken over only as a pure continuation -- nothing rewound, and
+    // the drafter within one row of the reuse point (real_forward_traits.rs:199-239); a drafter
+    // that cannot say where it stands never reuses.
+    int64_t reused = 0, drafter_at = 0;
+    if (dr->position) {
+        const int64_t cursor = tsv_kv_position(c);
+        int64_t keep = tsv_try_reuse_prefix(c, prompt, n);
+        if (keep < 0) return TSV_ERR_INVALID;
+        keep = std::min<int64_t>(keep, n - 1);
+        if (keep > 0) {
+            drafter_at = dr->position(dr->user);
+            if (tsv_kv_position(c) != cursor || drafter_at < 0 || keep - drafter_at > 1) keep = 0;
+        }
+        reused = keep;
+    }
+    if (reused == 0) {
+        if ((rc = tsv_reset(c))) return rc;
+    } else if (drafter_at > reused && dr->rewind(dr->user, reused)) {
+        set_error("run_speculative: rewind_drafter failed");
+        return TSV_ERR_INVALID;
+    }
+    out->reused = reused;
     std::vector<uint16_t> logits((size_t)vocab), rows_host;
     // the drafter's rows of a round: host memory, or a device buffer a GPU drafter fills in place
     struct DeviceRows {
@@ -156,8 +179,10 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
     }
     // prefill: every prompt token but the last skips the output head; the drafter is primed with
     // each known next token
-    if (n > 1 && (rc = tsv_prefill(c, prompt, n - 1, 0, nullptr))) return rc;
-    for (int64_t i = 0; i + 1 < n; i++)
+    // the reused positions are already in the cache (and, by the guard above, in the drafter's
+    // context up to at most the one row it lags by, which is primed here with its known next token)
+    if (n - 1 > reused && (rc = tsv_prefill(c, prompt + reused, n - 1 - reused, reused, nullptr))) return rc;
+    for (int64_t i = reused ? std::min(drafter_at, reused) : 0; i + 1 < n; i++)
         if (dr->prime(dr->user, prompt[i + 1], i)) {
             set_error("run_speculative: prime_drafter failed");
             return TSV_ERR_INVALID;
@@ -247,6 +272,9 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         history += res.committed;
         hist.insert(hist.end(), feed + 1, feed + 1 + res.committed);
         draw_step = res.draw_step;
+        // the record that lets the next turn reuse: the confirmed token plus every committed
+        // proposal, rows base .. base + committed + 1 (speculative.rs:828-836)
+        if ((rc = tsv_record_committed(c, feed, res.committed + 1, base))) return rc;
         if (dr->rewind(dr->user, base + res.committed)) {
             set_error("run_speculative: rewind_drafter failed");
             return TSV_ERR_INVALID;

@@ -8,9 +8,11 @@
 // fixed (KV cache, logits) and as the MFMA operand type of the matmuls.
 #include <cmath>
 #include <cstring>
+#include <new>
 #include <vector>
 
 #include "tsv_internal.h"
+#include "kv_prefix.h"
 
 using namespace tsv;
 
@@ -96,6 +98,8 @@ struct tsv_ctx {
     AcceptScratch sc{};
     std::vector<void*> allocs;
     int64_t position = 0;
+    tsv_prefix prefix;          // the ids behind rows [0, prefix length): kv_prefix.rs
+    bool prefix_reuse = false;  // RealForwardRunner::set_prefix_reuse: off unless the host opts in
     int last_m = 0;
     int64_t last_base = -1;
     // The launch sequence of a pass depends on the row count only (positions, tokens and the
@@ -1042,6 +1046,7 @@ extern "C" int32_t tsv_reset(tsv_ctx* c) {
     TSV_NEED(c, "reset: null handle");
     c->position = 0;
     c->last_m = 0;
+    c->prefix.clear();  // cleared beside the cache it describes (real_forward_traits.rs:33-35)
     return TSV_OK;
 }
 
@@ -1066,16 +1071,18 @@ extern "C" int32_t tsv_verify_tree(tsv_ctx* c, const int32_t* feed, const int32_
     return rc ? rc : finish_verify(c, m, logits);
 }
 
+// The one recording point of the token-by-token walk (real_forward_traits.rs:135-152): recorded
+// after the call and on success only; a failed pass may have left rows half written.
 extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint16_t* logits) {
-    return tsv_verify(c, &token, 1, position, logits);
+    const int rc = tsv_verify(c, &token, 1, position, logits);
+    if (c) {
+        if (rc == TSV_OK) c->prefix.record(&token, 1, position);
+        else c->prefix.taint();
+    }
+    return rc;
 }
 
-extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
-    TSV_NEED(c && ids, "prefill: null handle or token list");
-    if (n < 1) {
-        set_error("prefill: empty token list");
-        return TSV_ERR_INVALID;
-    }
+static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
     for (int64_t i = 0; i < n; i += TSV_MAX_ROWS) {
         const int m = (int)std::min<int64_t>(TSV_MAX_ROWS, n - i);
         int rc = enqueue_verify(c, ids + i, nullptr, m, pos0 + i);
@@ -1087,6 +1094,20 @@ extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
     return check_fused(c);
+}
+
+extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
+    TSV_NEED(c && ids, "prefill: null handle or token list");
+    if (n < 1) {
+        set_error("prefill: empty token list");
+        return TSV_ERR_INVALID;
+    }
+    // the chunk is recorded once it has run to completion, and taints the record when it has
+    // not (real_forward_traits.rs:395-402)
+    int rc = prefill_passes(c, ids, n, pos0, logits);
+    if (rc == TSV_OK) c->prefix.record(ids, n, pos0);
+    else c->prefix.taint();
+    return rc;
 }
 
 extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {
@@ -1104,6 +1125,7 @@ extern "C" int32_t tsv_rollback(tsv_ctx* c, const tsv_point* p) {
         return TSV_ERR_INVALID;
     }
     c->position = p->position;
+    c->prefix.rewind_to(p->position);  // real_forward_rollback.rs:203
     return TSV_OK;
 }
 
@@ -1114,11 +1136,68 @@ extern "C" int32_t tsv_rollback_retaining(tsv_ctx* c, const tsv_point* p, int32_
         return TSV_ERR_INVALID;
     }
     c->position = p->position + keep_rows;
+    c->prefix.rewind_to(c->position);  // real_forward_rollback.rs:406
     return TSV_OK;
 }
 
 extern "C" int32_t tsv_commit_pending(tsv_ctx*, int32_t) { return TSV_OK; }
 extern "C" int32_t tsv_discard_pending(tsv_ctx*) { return TSV_OK; }
+
+// ---- the record of what the rows were built from, on its own and behind the handle ----
+extern "C" tsv_prefix* tsv_prefix_new(void) { return new (std::nothrow) tsv_prefix(); }
+extern "C" void tsv_prefix_free(tsv_prefix* p) { delete p; }
+extern "C" void tsv_prefix_clear(tsv_prefix* p) {
+    if (p) p->clear();
+}
+extern "C" void tsv_prefix_taint(tsv_prefix* p) {
+    if (p) p->taint();
+}
+extern "C" void tsv_prefix_record(tsv_prefix* p, const int32_t* tokens, int64_t n, int64_t pos0) {
+    if (p && (tokens || n <= 0)) p->record(tokens, n, pos0);
+}
+extern "C" void tsv_prefix_rewind_to(tsv_prefix* p, int64_t position) {
+    if (p) p->rewind_to(position);
+}
+extern "C" int64_t tsv_prefix_untainted_len(const tsv_prefix* p) { return p ? p->untainted_len() : -1; }
+extern "C" int64_t tsv_prefix_common(const tsv_prefix* p, const int32_t* prompt, int64_t n) {
+    return p && prompt ? p->common_prefix(prompt, n) : 0;
+}
+
+extern "C" int32_t tsv_set_prefix_reuse(tsv_ctx* c, int32_t on) {
+    TSV_NEED(c, "set_prefix_reuse: null handle");
+    c->prefix_reuse = on != 0;
+    return TSV_OK;
+}
+
+// real_forward_traits.rs:173-289 for a target without recurrent state, session pool or drafter of
+// its own: the longest common prefix of the record and the prompt; a state that runs past it is
+// moved back there (kv.rewind_by + kv_prefix.rewind_to), as far as the cache can go back.
+extern "C" int64_t tsv_try_reuse_prefix(tsv_ctx* c, const int32_t* prompt, int64_t n) {
+    if (!c || (!prompt && n > 0)) {
+        set_error("try_reuse_prefix: null handle or prompt");
+        return -1;
+    }
+    if (!c->prefix_reuse) return 0;
+    const int64_t keep = c->prefix.common_prefix(prompt, n);
+    if (keep == 0 || keep > c->position) return 0;
+    const int64_t back = c->position - keep;
+    if (back > 0) {
+        if (back > tsv_max_safe_rewind(c)) return 0;
+        c->position = keep;
+        c->prefix.rewind_to(keep);
+    }
+    return keep;
+}
+
+// record_committed(tokens, pos0) (real_forward_traits.rs:567-569): a verify feeds a block and only
+// the caller knows how much of it survived, so the loop reports the surviving rows after the round.
+extern "C" int32_t tsv_record_committed(tsv_ctx* c, const int32_t* tokens, int64_t n, int64_t pos0) {
+    TSV_NEED(c && (tokens || n <= 0), "record_committed: null handle or token list");
+    c->prefix.record(tokens, n, pos0);
+    return TSV_OK;
+}
+
+extern "C" int64_t tsv_prefix_len(const tsv_ctx* c) { return c ? c->prefix.untainted_len() : -1; }
 
 extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* path, int32_t n) {
     TSV_NEED(c && path, "compact_tree: null handle or path");
@@ -1291,6 +1370,7 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
         if ((rc = tsv_compact_tree(c, r->base, path, keep))) return rc;
     }
     c->position = r->base + keep;
+    c->prefix.rewind_to(c->position);
     out->kv_position = c->position;
     return TSV_OK;
 }
@@ -1424,6 +1504,7 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
     (void)hipFree(kd);
     (void)hipFree(vd);
     if (!rc && pos0 + n > c->position) c->position = pos0 + n;
+    c->prefix.taint();  // rows no token ids describe
     return rc;
 }
 

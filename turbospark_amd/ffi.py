@@ -104,14 +104,53 @@ class AdaptiveDepth(C.Structure):
         return lib().tsv_adaptive_tile_cap(cap, tile_rows or 0)
 
 
+class KvPrefix:
+    """`KvPrefix` of crates/runtime/src/kv_prefix.rs:49-137: the token ids behind the cache rows
+    (pure host state inside the library; no GPU involved)."""
+
+    def __init__(self, ids=None):
+        self._p = lib().tsv_prefix_new()
+        if not self._p:
+            raise MemoryError("tsv_prefix_new")
+        if ids is not None:
+            self.record(ids, 0)
+
+    def __del__(self):
+        if getattr(self, "_p", None):
+            lib().tsv_prefix_free(self._p)
+            self._p = None
+
+    def clear(self):
+        lib().tsv_prefix_clear(self._p)
+
+    def taint(self):
+        lib().tsv_prefix_taint(self._p)
+
+    def record(self, tokens, pos0):
+        t = np.ascontiguousarray(tokens, np.int32)
+        lib().tsv_prefix_record(self._p, t.ctypes.data, t.size, int(pos0))
+
+    def rewind_to(self, position):
+        lib().tsv_prefix_rewind_to(self._p, int(position))
+
+    def untainted_len(self):
+        n = lib().tsv_prefix_untainted_len(self._p)
+        return None if n < 0 else int(n)
+
+    def common_prefix(self, prompt):
+        t = np.ascontiguousarray(prompt, np.int32)
+        return int(lib().tsv_prefix_common(self._p, t.ctypes.data, t.size))
+
+
 DRAFT_PRIME = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64)
 DRAFT_STEP = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.POINTER(C.c_uint16))
 DRAFT_REWIND = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int64)
+DRAFT_POSITION = C.CFUNCTYPE(C.c_int64, C.c_void_p)
 
 
 class Drafter(C.Structure):
     _fields_ = [("user", C.c_void_p), ("prime", DRAFT_PRIME), ("step", DRAFT_STEP), ("rewind", DRAFT_REWIND),
-                ("device_logits", C.c_int32)]
+                ("device_logits", C.c_int32), ("position", DRAFT_POSITION)]
 
 
 class Generation(C.Structure):
@@ -123,7 +162,8 @@ class GenerationResult(C.Structure):
     _fields_ = [("tokens", C.POINTER(C.c_int32)), ("capacity", C.c_int64), ("n_tokens", C.c_int64),
                 ("stop_reason", C.c_int32), ("final_depth", C.c_int32), ("rounds", C.c_int64),
                 ("offered", C.c_int64), ("accepted", C.c_int64), ("rollbacks", C.c_int64),
-                ("draw_step", C.c_uint64), ("kv_position", C.c_int64), ("min_margin", C.c_double)]
+                ("draw_step", C.c_uint64), ("kv_position", C.c_int64), ("min_margin", C.c_double),
+                ("reused", C.c_int64)]
 
 
 class Point(C.Structure):
@@ -156,6 +196,9 @@ EXPORTS = [
     "tsv_synth_tensor", "tsv_read_kv", "tsv_write_kv", "tsv_write_logits", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
     "tsv_yarn_frequencies", "tsv_adaptive_init", "tsv_adaptive_depth", "tsv_adaptive_observe", "tsv_adaptive_tile_cap",
     "tsv_run_speculative", "tsv_max_context", "tsv_vocab",
+    "tsv_prefix_new", "tsv_prefix_free", "tsv_prefix_clear", "tsv_prefix_taint", "tsv_prefix_record",
+    "tsv_prefix_rewind_to", "tsv_prefix_untainted_len", "tsv_prefix_common",
+    "tsv_set_prefix_reuse", "tsv_try_reuse_prefix", "tsv_record_committed", "tsv_prefix_len",
 ]
 
 _lib = None
@@ -223,6 +266,25 @@ def lib():
         L.tsv_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                       C.c_int32, C.POINTER(C.c_float)]
         L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
+        L.tsv_prefix_new.restype = C.c_void_p
+        L.tsv_prefix_new.argtypes = []
+        for name in ("tsv_prefix_free", "tsv_prefix_clear", "tsv_prefix_taint"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [C.c_void_p]
+        L.tsv_prefix_record.restype = None
+        L.tsv_prefix_record.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]
+        L.tsv_prefix_rewind_to.restype = None
+        L.tsv_prefix_rewind_to.argtypes = [C.c_void_p, C.c_int64]
+        L.tsv_prefix_untainted_len.restype = C.c_int64
+        L.tsv_prefix_untainted_len.argtypes = [C.c_void_p]
+        L.tsv_prefix_common.restype = C.c_int64
+        L.tsv_prefix_common.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.tsv_set_prefix_reuse.argtypes = [C.c_void_p, C.c_int32]
+        L.tsv_try_reuse_prefix.restype = C.c_int64
+        L.tsv_try_reuse_prefix.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.tsv_record_committed.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]
+        L.tsv_prefix_len.restype = C.c_int64
+        L.tsv_prefix_len.argtypes = [C.c_void_p]
         _lib = L
     return _lib
 

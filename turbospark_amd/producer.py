@@ -114,6 +114,30 @@ class HipVerifier:
         return out
 
     # ---- SpeculativeProducer ----------------------------------------------------------
+    # ---- prefix reuse (LogitProducer::try_reuse_prefix, SpeculativeProducer::record_committed) ----
+    def set_prefix_reuse(self, on):
+        """RealForwardRunner::set_prefix_reuse: reuse answers 0 until the host opts in."""
+        ffi.check(ffi.lib().tsv_set_prefix_reuse(self._h, int(bool(on))))
+
+    def try_reuse_prefix(self, prompt_ids):
+        """producer.rs:24-47: commits to continuing from the current state for the leading N tokens
+        of the prompt (moving the cursor back to them when it ran past) and returns N; 0 = reset."""
+        p = _i32(prompt_ids)
+        n = ffi.lib().tsv_try_reuse_prefix(self._h, p.ctypes.data, p.size)
+        if n < 0:
+            raise ffi.TsvError(-1, ffi.last_error())
+        return int(n)
+
+    def record_committed(self, tokens, pos0):
+        """producer.rs:322-330: the rows of a verify pass that the round committed."""
+        t = _i32(tokens)
+        ffi.check(ffi.lib().tsv_record_committed(self._h, t.ctypes.data, t.size, int(pos0)))
+
+    def prefix_len(self):
+        """Positions the record describes; None when tainted."""
+        n = ffi.lib().tsv_prefix_len(self._h)
+        return None if n < 0 else int(n)
+
     def checkpoint(self):
         p = ffi.Point()
         ffi.check(ffi.lib().tsv_checkpoint(self._h, C.byref(p)))
@@ -266,6 +290,14 @@ class HipVerifier:
         d = ffi.Drafter(None, ffi.DRAFT_PRIME(guard(lambda u, t, p: drafter.prime(t, p))),
                         ffi.DRAFT_STEP(guard(step)), ffi.DRAFT_REWIND(guard(lambda u, p: drafter.rewind(p))),
                         1 if device_logits else 0)
+        if hasattr(drafter, "context_position"):  # lets the loop take over a prefix (the continuity guard)
+            def where(user):
+                try:
+                    return int(drafter.context_position())
+                except Exception as e:
+                    failure.append(e)
+                    return -1
+            d.position = ffi.DRAFT_POSITION(where)
         g = ffi.Generation()
         g.shaping = cfg
         g.max_new_tokens = int(max_new_tokens)
@@ -285,7 +317,8 @@ class HipVerifier:
         ffi.check(rc)
         return dict(tokens=[int(t) for t in toks[: res.n_tokens]], stop_reason=res.stop_reason, rounds=res.rounds,
                     offered=res.offered, accepted=res.accepted, rollbacks=res.rollbacks, draw_step=res.draw_step,
-                    final_depth=res.final_depth, kv_position=res.kv_position, min_margin=res.min_margin)
+                    final_depth=res.final_depth, kv_position=res.kv_position, min_margin=res.min_margin,
+                    reused=res.reused)
 
     PROFILE_CLASSES = ("embed", "norm", "qkv", "rope_kv", "attention", "wo", "gate_up", "down", "head", "accept",
                        "event_pair")
