@@ -106,63 +106,84 @@ MEASURED_TRAFFIC = {"llama3_8b_q4_k_k4_ctx4096": 67051534}
 
 GATE_UP_8B = dict(dtype=12, rows=28672, cols=4096, m=5, epi=1)   # the dominant kernel of the headline workload
 COPY_BYTES = 256 << 20
+# What a counter run can be pointed at (--probe): `match` picks the kernel's dispatches out of the
+# collection, `alg` is its algorithmic bytes per launch.
+ATTN_8B = dict(m=5, nq=32, nkv=8, hd=128, base=4096)             # one layer's attention of the headline workload
+PROBES = {
+    "gate_up": dict(match="k_gemm<", what="gate/up matmul, 28672 x 4096 Q4_K, M = 5", **GATE_UP_8B),
+    # the same weights under sixteen rows (the 16-node tree): the 16x16x32 MFMA form
+    "gemm16": dict(match="k_gemm16<", what="gate/up matmul, 28672 x 4096 Q4_K, M = 16", **dict(GATE_UP_8B, m=16)),
+    "attention": dict(match="k_attn_partial", what="attention partial pass, 32 q / 8 kv heads x 128, M = 5, 4096-token context",
+                      **ATTN_8B),
+}
 
 
-def traffic_probe():
-    """What `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` is pointed at: the plain copy kernel
-    of known size (COPY_BYTES read, COPY_BYTES written per launch), then the gate/up matmul of the
-    headline workload on weights cycled through HBM."""
+def probe_bytes(pr):
     from turbospark_amd import ffi
-    g = GATE_UP_8B
+    if "rows" in pr:
+        return pr["rows"] * ffi.row_bytes(pr["dtype"], pr["cols"])
+    return (pr["base"] + pr["m"]) * pr["nkv"] * pr["hd"] * 2 * 2    # K and V rows [0, base + m), fp16, read once
+
+
+def traffic_probe(which):
+    """What `rocprofv3 --pmc ...` is pointed at: the plain copy kernel of known size (COPY_BYTES
+    read, COPY_BYTES written per launch), then the probed kernel at the headline workload's shape
+    (matmuls: on weights cycled through HBM; attention: fresh seeded K/V per launch)."""
+    import numpy as np
+    from turbospark_amd import ffi
+    pr = PROBES[which]
     us = ffi.copy_time(COPY_BYTES, iters=10)
     log(f"[traffic-probe] copy kernel {COPY_BYTES >> 20} MiB: {us:.1f} us, {2 * COPY_BYTES / us / 1e3:.0f} GB/s read+write")
-    us = ffi.matmul_time(g["dtype"], g["rows"], g["cols"], g["m"], g["epi"], 0, 20, 4)
-    nbytes = g["rows"] * ffi.row_bytes(g["dtype"], g["cols"])
-    log(f"[traffic-probe] gate/up matmul: {us:.2f} us, {nbytes / us / 1e3:.0f} GB/s of weight bytes")
+    if "rows" in pr:
+        us = ffi.matmul_time(pr["dtype"], pr["rows"], pr["cols"], pr["m"], pr["epi"], 0, 20, 4)
+        log(f"[traffic-probe] {pr['what']}: {us:.2f} us, {probe_bytes(pr) / us / 1e3:.0f} GB/s of weight bytes")
+        return
+    rng = np.random.default_rng(1)
+    for it in range(8):
+        q = rng.standard_normal((pr["m"], pr["nq"], pr["hd"]), np.float32)
+        k = rng.standard_normal((pr["base"] + pr["m"], pr["nkv"], pr["hd"]), np.float32)
+        v = rng.standard_normal((pr["base"] + pr["m"], pr["nkv"], pr["hd"]), np.float32)
+        out = ffi.attention(q, k, v, pr["base"])
+        assert np.isfinite(out).all()
+    log(f"[traffic-probe] {pr['what']}: 8 launches, {probe_bytes(pr)} algorithmic bytes each")
 
 
-def traffic_summary(fetch_csv, write_csv):
-    """HBM bytes per launch of the gate/up matmul from two counter-collection CSVs of
+def per_kernel_counters(path, which):
+    """{counter: {"copy" | "kernel": [value per dispatch]}} from a counter-collection CSV of --traffic-probe."""
+    import csv
+    match = PROBES[which]["match"]
+    acc = {}
+    for r in csv.DictReader(open(path)):
+        key = "copy" if "k_copy_probe" in r["Kernel_Name"] else "kernel" if match in r["Kernel_Name"] else None
+        if key:
+            acc.setdefault(r["Counter_Name"], {}).setdefault(key, []).append(float(r["Counter_Value"]))
+    return acc
+
+
+def traffic_summary(fetch_csv, write_csv, which):
+    """HBM bytes per launch of the probed kernel from two counter-collection CSVs of
     `bench.py --traffic-probe` (FETCH_SIZE and WRITE_SIZE, KiB-like units per dispatch), each
     scaled by what the same counter reads for the copy kernel of known size."""
-    import csv
-    from turbospark_amd import ffi
-
-    def per_kernel(path, counter):
-        acc = {}
-        for r in csv.DictReader(open(path)):
-            if r["Counter_Name"] != counter:
-                continue
-            key = "copy" if "k_copy_probe" in r["Kernel_Name"] else "gemm" if "k_gemm" in r["Kernel_Name"] else None
-            if key:
-                acc.setdefault(key, []).append(float(r["Counter_Value"]))
-        return {k: sum(v) / len(v) for k, v in acc.items()}, {k: len(v) for k, v in acc.items()}
-
-    g = GATE_UP_8B
-    alg = g["rows"] * ffi.row_bytes(g["dtype"], g["cols"])
-    out = {"algorithmic_bytes_per_launch": alg}
+    alg = probe_bytes(PROBES[which])
+    out = {"kernel": PROBES[which]["what"], "algorithmic_bytes_per_launch": alg}
     for name, path, counter in (("read", fetch_csv, "FETCH_SIZE"), ("write", write_csv, "WRITE_SIZE")):
-        avg, n = per_kernel(path, counter)
+        acc = per_kernel_counters(path, which)[counter]
+        avg = {k: sum(v) / len(v) for k, v in acc.items()}
         factor = COPY_BYTES / avg["copy"]          # bytes per counter unit, from the copy kernel
         out[name] = dict(counter=counter, copy_kernel_reading=round(avg["copy"], 1), bytes_per_unit=round(factor, 2),
-                         gemm_reading=round(avg["gemm"], 1), gemm_bytes=int(avg["gemm"] * factor),
-                         dispatches=n)
-    out["traffic_bytes_per_launch"] = out["read"]["gemm_bytes"] + out["write"]["gemm_bytes"]
+                         kernel_reading=round(avg["kernel"], 1), kernel_bytes=int(avg["kernel"] * factor),
+                         dispatches={k: len(v) for k, v in acc.items()})
+    out["traffic_bytes_per_launch"] = out["read"]["kernel_bytes"] + out["write"]["kernel_bytes"]
     out["traffic_over_algorithmic"] = round(out["traffic_bytes_per_launch"] / alg, 3)
     print(json.dumps(out, indent=1))
 
 
-def counter_summary(path):
+def counter_summary(path, which):
     """Per-dispatch averages of every counter in a `rocprofv3 --pmc ... --output-format csv` collection of
-    `bench.py --traffic-probe`, for the gate/up matmul launches (the copy kernel is left out)."""
-    import csv
-    acc = {}
-    for r in csv.DictReader(open(path)):
-        if "k_gemm" not in r["Kernel_Name"]:
-            continue
-        acc.setdefault(r["Counter_Name"], []).append(float(r["Counter_Value"]))
-    print(json.dumps({k: round(sum(v) / len(v), 1) for k, v in sorted(acc.items())} | {"dispatches": len(next(iter(acc.values())))},
-                     indent=1))
+    `bench.py --traffic-probe`, for the probed kernel's launches (the copy kernel is left out)."""
+    acc = {c: d["kernel"] for c, d in per_kernel_counters(path, which).items() if "kernel" in d}
+    print(json.dumps({"kernel": PROBES[which]["what"]} | {k: round(sum(v) / len(v), 1) for k, v in sorted(acc.items())} |
+                     {"dispatches": len(next(iter(acc.values())))}, indent=1))
 
 
 def main():
@@ -175,6 +196,8 @@ def main():
                     help="per-dispatch averages of the counters a rocprofv3 --pmc run of --traffic-probe collected")
     ap.add_argument("--traffic-summary", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="HBM bytes per launch of the dominant matmul from two --pmc runs of --traffic-probe")
+    ap.add_argument("--probe", default="gate_up", choices=sorted(PROBES),
+                    help="which kernel --traffic-probe runs and the two summaries read")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -187,13 +210,13 @@ def main():
         trace_summary(args.trace_summary)
         return
     if args.traffic_probe:
-        traffic_probe()
+        traffic_probe(args.probe)
         return
     if args.counter_summary:
-        counter_summary(args.counter_summary)
+        counter_summary(args.counter_summary, args.probe)
         return
     if args.traffic_summary:
-        traffic_summary(*args.traffic_summary)
+        traffic_summary(*args.traffic_summary, args.probe)
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "
