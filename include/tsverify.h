@@ -175,7 +175,9 @@ int64_t tsv_max_safe_rewind(const tsv_ctx* ctx);
 /* LogitProducer::produce: one token at `position`; logits: vocab fp16. */
 int32_t tsv_produce(tsv_ctx* ctx, int32_t token, int64_t position, uint16_t* logits);
 /* produce_prefill / ChunkedPrefillRunner::prefill_chunk: feeds n tokens from pos0 in
- * passes of TSV_MAX_ROWS rows; logits (nullable) receives the LAST token's row. */
+ * passes of TSV_MAX_ROWS rows; logits (nullable) receives the LAST token's row.  Passes whose
+ * logits nobody reads skip the final norm and the output head (producer.rs:92-103): every pass but
+ * the last, and the last too when logits is NULL -- then no rows are left for tsv_accept. */
 int32_t tsv_prefill(tsv_ctx* ctx, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits);
 
 /* ---- SpeculativeProducer (producer.rs:164-387) ------------------------------ */

@@ -121,3 +121,31 @@ def test_a_second_turn_continues_from_the_first_turns_cache(temperature):
     # and a drafter that does not say where it stands never reuses
     four = gpu.run_speculative(prompt3, LmDrafter(GpuTarget(lm), prompt3[0], V, 0.5, 9), shaping, 8, 4)
     assert four["reused"] == 0 and four["tokens"] == three["tokens"]
+
+
+def test_headless_prefill_passes_leave_the_rows_of_full_passes():
+    """produce_prefill (producer.rs:92-103): skipping the output head must not change any other side
+    effect of the pass -- the cache rows and the cursor are those of a pass that paid for the head."""
+    import turbospark_amd as ts
+    cfg, w, gpu, _ = _target()
+    V = cfg["vocab"]
+    ids = np.random.default_rng(4).integers(0, V, 45).astype(np.int32)
+    gpu.reset()
+    gpu.prefill(ids, 0, want_logits=False)                     # three passes, none of them runs the head
+    assert gpu.position == 45
+    rows_a = [gpu.read_kv(layer, 0, 45) for layer in range(cfg["n_layers"])]
+    with pytest.raises(ts.ffi.TsvError):                       # no rows on the device to judge
+        gpu.accept(ids[:5], 40, ts.shaping(0.0))
+    after_a = gpu.produce(7, 45)
+    gpu.reset()
+    last = gpu.prefill(ids, 0)                                 # the last pass pays for the head
+    rows_b = [gpu.read_kv(layer, 0, 45) for layer in range(cfg["n_layers"])]
+    for (ka, va), (kb, vb) in zip(rows_a, rows_b):
+        assert np.array_equal(ka.view(np.uint16), kb.view(np.uint16))
+        assert np.array_equal(va.view(np.uint16), vb.view(np.uint16))
+    assert np.array_equal(after_a, gpu.produce(7, 45))
+    # and the row handed out is the row token-by-token decoding gives for the last prompt token
+    gpu.reset()
+    gpu.prefill(ids[:-1], 0, want_logits=False)
+    one = gpu.produce(int(ids[-1]), 44)
+    assert gc.logit_error(last, one) <= 2e-3

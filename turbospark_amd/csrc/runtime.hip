@@ -100,6 +100,7 @@ struct tsv_ctx {
     int64_t position = 0;
     tsv_prefix prefix;          // the ids behind rows [0, prefix length): kv_prefix.rs
     bool prefix_reuse = false;  // RealForwardRunner::set_prefix_reuse: off unless the host opts in
+    bool headless = false;      // the pass in flight is a prefill pass nobody reads the logits of
     int last_m = 0;
     int64_t last_base = -1;
     // The launch sequence of a pass depends on the row count only (positions, tokens and the
@@ -638,6 +639,10 @@ int launch_pass(tsv_ctx* c, int m) {
         prev_partial = c->partial;
         prev_splits = sp;
     }
+    // produce_prefill (producer.rs:92-103, real_forward_traits.rs:291-300): a prompt token whose
+    // logits nobody reads skips the final norm and the output head; every other side effect of
+    // the pass (the rows in the cache, the cursor) is that of a full pass.
+    if (c->headless) return TSV_OK;
     {
         PROF(PC_NORM);
         rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m,
@@ -654,7 +659,7 @@ int launch_pass(tsv_ctx* c, int m) {
 }
 
 int run_pass(tsv_ctx* c, int m) {
-    if (!c->use_graph || c->profile) return launch_pass(c, m);
+    if (!c->use_graph || c->profile || c->headless) return launch_pass(c, m);
     if (!c->pass_graph[m]) {
         hipGraph_t g = nullptr;
         TSV_HIP(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
@@ -1085,7 +1090,13 @@ extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint
 static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
     for (int64_t i = 0; i < n; i += TSV_MAX_ROWS) {
         const int m = (int)std::min<int64_t>(TSV_MAX_ROWS, n - i);
+        // only the last row's logits are ever handed out: every earlier pass is headless, and so
+        // is the last one when the caller takes no logits
+        c->headless = i + m < n || !logits;
         int rc = enqueue_verify(c, ids + i, nullptr, m, pos0 + i);
+        const bool skipped = c->headless;
+        c->headless = false;
+        if (skipped) c->last_m = 0;  // no rows on the device for tsv_accept to judge
         if (rc) return rc;
         if (i + m >= n && logits) {
             TSV_HIP(hipMemcpyAsync(logits, c->logits + (size_t)(m - 1) * c->vocab, (size_t)c->vocab * 2,
