@@ -315,6 +315,32 @@ const uint16_t* tsv_device_logits(tsv_ctx* ctx);
 int64_t tsv_max_context(const tsv_ctx* ctx);
 int64_t tsv_vocab(const tsv_ctx* ctx);
 
+/* ---- GGUF intake (host) -------------------------------------------------------- */
+/* The header parser of crates/repack/src/gguf_header/parser.rs:124-239 over a read-only mapping of
+ * the file: version 3 only, metadata keys and tensor names unique, at most four non-zero
+ * dimensions, every offset a multiple of general.alignment (default 32, a power of two); the data
+ * region starts at the aligned end of the tensor table.  Refusals are by name (tsv_last_error). */
+typedef struct tsv_gguf tsv_gguf;
+int32_t tsv_gguf_open(const char* path, tsv_gguf** out);
+void tsv_gguf_close(tsv_gguf* g);
+int64_t tsv_gguf_tensor_count(const tsv_gguf* g);
+int64_t tsv_gguf_data_start(const tsv_gguf* g);
+/* A tensor where it lies in the mapping (valid until tsv_gguf_close): dtype is the ggml type id,
+ * cols the first dimension, rows the product of the others (stacked experts are expert-major row
+ * runs); bounds-checked against the file. */
+int32_t tsv_gguf_tensor(const tsv_gguf* g, const char* name, tsv_tensor* out);
+int32_t tsv_gguf_meta_number(const tsv_gguf* g, const char* key, double* out);
+int32_t tsv_gguf_meta_string(const tsv_gguf* g, const char* key, char* buf, int32_t cap);
+/* Opens a llama-family GGUF as a verify target: tensor names of crates/repack/src/gguf_names/
+ * llama.rs:14-60 (`llama`; `qwen2` adds the q / k / v biases; `qwen3` / `qwen3moe` the per-head
+ * q / k norms; routed experts as the stacked *_exps tensors), sizes from the `<arch>.*` metadata,
+ * the q / k rows of a `llama` file un-permuted from llama.cpp's adjacent-pair order
+ * (crates/repack/src/gguf_checkpoint/conventions.rs:133-243).  rope_freqs.weight, which the
+ * reference refuses for this family, is taken as the llama-3 per-pair divisors; any other context
+ * extension (rope.scaling.type) and partial rotation are refused.  max_context <= 0: the file's
+ * context_length.  The mapping is dropped before the call returns. */
+int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx** out);
+
 /* ---- install-time helpers (host) --------------------------------------------- */
 /* The reference's quantize-on-install encoders (q8_0.rs:56-77, q4_k.rs:126-204). */
 int64_t tsv_row_bytes(int32_t dtype, int64_t cols);

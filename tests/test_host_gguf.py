@@ -1,0 +1,134 @@
+"""The GGUF header parser behind the C ABI (crates/repack/src/gguf_header/parser.rs:124-239) on
+files a test writer lays out as the public format says: what it reads back, and what it refuses
+by name.  No GPU is touched."""
+import os
+
+import numpy as np
+import pytest
+
+from tests.gguf_writer import permute_rotary_rows, write_gguf
+from turbospark_amd import ffi
+
+
+def _tensors():
+    rng = np.random.default_rng(0)
+    w = (rng.standard_normal((8, 256)) * 0.02).astype(np.float32)
+    q4 = ffi.quantize(ffi.Q4_K, w)
+    q8 = ffi.quantize(ffi.Q8_0, w)
+    norm = np.arange(256, dtype=np.float32)
+    experts = ffi.quantize(ffi.MXFP4, (rng.standard_normal((3 * 4, 64))).astype(np.float32))
+    return [("a.weight", [256, 8], ffi.Q4_K, q4[1].tobytes()), ("b.weight", [256, 8], ffi.Q8_0, q8[1].tobytes()),
+            ("n.weight", [256], ffi.F32, norm.tobytes()), ("e_exps.weight", [64, 4, 3], ffi.MXFP4, experts[1].tobytes())], q4, q8, norm, experts
+
+
+META = [("general.architecture", "str", "llama"), ("llama.block_count", "u32", 2), ("llama.rope.freq_base", "f32", 500000.0),
+        ("x.i64", "i64", -5), ("x.f64", "f64", 2.5), ("x.bool", "bool", 1), ("x.u8", "u8", 200),
+        ("tokenizer.ggml.tokens", "arr", ("str", ["a", "bc", ""])), ("nested", "arr", ("arr", [("u16", [1, 2]), ("u16", [])]))]
+
+
+def test_a_written_file_reads_back(tmp_path):
+    tensors, q4, q8, norm, experts = _tensors()
+    for alignment in (None, 64, 4096):
+        path = os.path.join(tmp_path, f"m{alignment}.gguf")
+        start = write_gguf(path, META, tensors, alignment=alignment)
+        g = ffi.Gguf(path)
+        assert g.tensor_count == 4 and g.data_start == start and start % (alignment or 32) == 0
+        assert g.string("general.architecture") == "llama"
+        assert g.number("llama.block_count") == 2 and g.number("llama.rope.freq_base") == 500000.0
+        assert g.number("x.i64") == -5 and g.number("x.f64") == 2.5 and g.number("x.bool") == 1 and g.number("x.u8") == 200
+        dt, raw, rows, cols = g.tensor("a.weight")
+        assert (dt, rows, cols) == (ffi.Q4_K, 8, 256) and np.array_equal(raw, q4[1])
+        dt, raw, rows, cols = g.tensor("b.weight")
+        assert (dt, rows, cols) == (ffi.Q8_0, 8, 256) and np.array_equal(raw, q8[1])
+        dt, raw, rows, cols = g.tensor("n.weight")
+        assert (dt, rows, cols) == (ffi.F32, 1, 256) and np.array_equal(raw.view(np.float32)[0], norm)
+        # stacked experts: every dimension past the first folds into expert-major rows
+        dt, raw, rows, cols = g.tensor("e_exps.weight")
+        assert (dt, rows, cols) == (ffi.MXFP4, 12, 64) and np.array_equal(raw, experts[1])
+        with pytest.raises(ffi.TsvError, match="no tensor"):
+            g.tensor("missing.weight")
+        with pytest.raises(ffi.TsvError, match="no numeric metadata"):
+            g.number("general.architecture")
+        g.close()
+
+
+def _refused(tmp_path, match, **kw):
+    tensors = kw.pop("tensors", None) or _tensors()[0]
+    meta = kw.pop("meta", META)
+    cut = kw.pop("cut", None)
+    path = os.path.join(tmp_path, "bad.gguf")
+    write_gguf(path, meta, tensors, **kw)
+    if cut is not None:
+        data = open(path, "rb").read()
+        open(path, "wb").write(data[:cut] if cut > 0 else data[:len(data) + cut])
+    with pytest.raises(ffi.TsvError, match=match):
+        ffi.Gguf(path).close()
+
+
+def test_the_parsers_refusals(tmp_path):
+    _refused(tmp_path, "bad magic", magic=b"GGML")
+    _refused(tmp_path, "version 2", version=2)
+    _refused(tmp_path, "too short", cut=250)                       # the header itself is cut
+    _refused(tmp_path, "shorter than a GGUF header", cut=10)
+    _refused(tmp_path, "duplicate metadata key", meta=META + [("x.u8", "u8", 1)])
+    t = _tensors()[0]
+    _refused(tmp_path, "duplicate tensor", tensors=t + [t[0]])
+    _refused(tmp_path, "a zero dimension", tensors=[("z", [256, 0], ffi.F32, b"")])
+    _refused(tmp_path, "5 dimensions", tensors=[("z", [2, 2, 2, 2, 2], ffi.F32, b"\0" * 128)])
+    _refused(tmp_path, "not a multiple of the file's alignment", misalign="b.weight")
+    _refused(tmp_path, "not a power of two", alignment=48)
+    with pytest.raises(ffi.TsvError, match="cannot read"):
+        ffi.Gguf(os.path.join(tmp_path, "absent.gguf"))
+
+
+def test_a_bad_value_type_and_deep_nesting_are_refused(tmp_path):
+    import struct
+    from tests import gguf_writer as gw
+    # a value type id the format does not define
+    gw.TYPE_IDS["bogus"], gw.PACK["bogus"] = 13, "<B"
+    try:
+        _refused(tmp_path, "is not a GGUF type", meta=[("k", "bogus", 1)])
+    finally:
+        del gw.TYPE_IDS["bogus"], gw.PACK["bogus"]
+    # arrays nested deeper than the parser walks: 70 array headers of one element each
+    body = b"".join(struct.pack("<IQ", 9, 1) for _ in range(70)) + struct.pack("<IQ", 0, 0)
+    head = b"GGUF" + struct.pack("<IQQ", 3, 0, 1) + struct.pack("<Q", 1) + b"k" + struct.pack("<I", 9) + body
+    path = os.path.join(tmp_path, "deep.gguf")
+    open(path, "wb").write(head + b"\0" * 64)
+    with pytest.raises(ffi.TsvError, match="nested deeper"):
+        ffi.Gguf(path)
+    # counts no file of this size could hold
+    open(path, "wb").write(b"GGUF" + struct.pack("<IQQ", 3, 1 << 40, 0) + b"\0" * 64)
+    with pytest.raises(ffi.TsvError, match="counts larger"):
+        ffi.Gguf(path)
+
+
+def test_tensor_views_are_checked_against_the_file(tmp_path):
+    tensors = _tensors()[0]
+    path = os.path.join(tmp_path, "cut.gguf")
+    write_gguf(path, META, tensors)
+    data = open(path, "rb").read()
+    open(path, "wb").write(data[:-40])                             # the last tensor's tail is gone
+    g = ffi.Gguf(path)
+    assert g.tensor("a.weight")[2] == 8
+    with pytest.raises(ffi.TsvError, match="runs past the end"):
+        g.tensor("e_exps.weight")
+    g.close()
+    # a block type without a kernel here (Q4_0) and a row length that is not whole blocks
+    write_gguf(path, META, [("q40.weight", [256, 2], 2, b"\0" * 288), ("odd.weight", [100, 2], ffi.Q4_K, b"\0" * 288)])
+    g = ffi.Gguf(path)
+    for name in ("q40.weight", "odd.weight"):
+        with pytest.raises(ffi.TsvError, match="no kernel here"):
+            g.tensor(name)
+    g.close()
+
+
+def test_the_writers_permutation_is_the_converters():
+    # conventions.rs:133-143: GGUF row j of a head holds the original row (j % 2) * (D/2) + j // 2,
+    # so the original row i is found at GGUF row (i % (D/2)) * 2 + i // (D/2)
+    D = 8
+    rows = np.arange(2 * D).reshape(2 * D, 1)
+    perm = permute_rotary_rows(rows, D)[:, 0]
+    assert perm[:D].tolist() == [0, 4, 1, 5, 2, 6, 3, 7] and perm[D:].tolist() == [8, 12, 9, 13, 10, 14, 11, 15]
+    for i in range(D):
+        assert perm[(i % (D // 2)) * 2 + i // (D // 2)] == i

@@ -6,9 +6,9 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
-SOURCES = ["gemm.hip", "fused.hip", "moe.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip"]
+SOURCES = ["gemm.hip", "fused.hip", "moe.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
 # host_utils.hip is host-only code; clang 22 -O3 does not terminate on it, -O2 does.
-OPT = {"host_utils.hip": "-O2"}
+OPT = {"host_utils.hip": "-O2", "gguf.hip": "-O2"}
 # MFMA results straight into VGPRs (no v_accvgpr_read copies before the scaling FMAs)
 EXTRA = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_GEMM_DEFS", "").split(),
          "fused.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),

@@ -142,6 +142,48 @@ class KvPrefix:
         return int(lib().tsv_prefix_common(self._p, t.ctypes.data, t.size))
 
 
+class Gguf:
+    """A GGUF file's header and tensors through the library's parser (read-only mapping)."""
+
+    def __init__(self, path):
+        h = C.c_void_p()
+        check(lib().tsv_gguf_open(os.fsencode(path), C.byref(h)))
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().tsv_gguf_close(self._h)
+            self._h = None
+
+    __del__ = close
+
+    @property
+    def tensor_count(self):
+        return int(lib().tsv_gguf_tensor_count(self._h))
+
+    @property
+    def data_start(self):
+        return int(lib().tsv_gguf_data_start(self._h))
+
+    def number(self, key):
+        v = C.c_double()
+        check(lib().tsv_gguf_meta_number(self._h, key.encode(), C.byref(v)))
+        return v.value
+
+    def string(self, key):
+        buf = C.create_string_buffer(256)
+        check(lib().tsv_gguf_meta_string(self._h, key.encode(), buf, 256))
+        return buf.value.decode()
+
+    def tensor(self, name):
+        """(dtype, bytes as uint8 [rows, row_bytes] -- a copy --, rows, cols)"""
+        t = Tensor()
+        check(lib().tsv_gguf_tensor(self._h, name.encode(), C.byref(t)))
+        rb = row_bytes(t.dtype, t.cols)
+        raw = np.ctypeslib.as_array(C.cast(t.data, C.POINTER(C.c_uint8)), shape=(t.rows * rb,)).copy()
+        return t.dtype, raw.reshape(t.rows, rb), int(t.rows), int(t.cols)
+
+
 DRAFT_PRIME = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64)
 DRAFT_STEP = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.POINTER(C.c_uint16))
 DRAFT_REWIND = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int64)
@@ -199,6 +241,8 @@ EXPORTS = [
     "tsv_prefix_new", "tsv_prefix_free", "tsv_prefix_clear", "tsv_prefix_taint", "tsv_prefix_record",
     "tsv_prefix_rewind_to", "tsv_prefix_untainted_len", "tsv_prefix_common",
     "tsv_set_prefix_reuse", "tsv_try_reuse_prefix", "tsv_record_committed", "tsv_prefix_len",
+    "tsv_gguf_open", "tsv_gguf_close", "tsv_gguf_tensor_count", "tsv_gguf_data_start", "tsv_gguf_tensor",
+    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf",
 ]
 
 _lib = None
@@ -266,6 +310,17 @@ def lib():
         L.tsv_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                       C.c_int32, C.POINTER(C.c_float)]
         L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
+        L.tsv_gguf_open.argtypes = [C.c_char_p, C.POINTER(C.c_void_p)]
+        L.tsv_gguf_close.restype = None
+        L.tsv_gguf_close.argtypes = [C.c_void_p]
+        L.tsv_gguf_tensor_count.restype = C.c_int64
+        L.tsv_gguf_tensor_count.argtypes = [C.c_void_p]
+        L.tsv_gguf_data_start.restype = C.c_int64
+        L.tsv_gguf_data_start.argtypes = [C.c_void_p]
+        L.tsv_gguf_tensor.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(Tensor)]
+        L.tsv_gguf_meta_number.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
+        L.tsv_gguf_meta_string.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_int32]
+        L.tsv_open_gguf.argtypes = [C.c_char_p, C.c_int32, C.POINTER(C.c_void_p)]
         L.tsv_prefix_new.restype = C.c_void_p
         L.tsv_prefix_new.argtypes = []
         for name in ("tsv_prefix_free", "tsv_prefix_clear", "tsv_prefix_taint"):

@@ -71,6 +71,34 @@ class HipVerifier:
         self._h = h
         self.vocab = cfg["vocab"]
 
+    @classmethod
+    def from_gguf(cls, path, max_context=0):
+        """Opens a llama-family GGUF file (llama, qwen2, qwen3, qwen3moe) as the target; the sizes
+        come from the file's metadata.  max_context 0: the file's context_length."""
+        import os
+        self = cls.__new__(cls)
+        h = C.c_void_p()
+        ffi.check(ffi.lib().tsv_open_gguf(os.fsencode(path), int(max_context), C.byref(h)))
+        self._h = h
+        self._keep = None
+        self.vocab = int(ffi.lib().tsv_vocab(h))
+        g = ffi.Gguf(path)
+        arch = g.string("general.architecture")
+        heads = int(g.number(arch + ".attention.head_count"))
+        hidden = int(g.number(arch + ".embedding_length"))
+
+        def opt(key, default):
+            try:
+                return g.number(arch + "." + key)
+            except ffi.TsvError:
+                return default
+        self.cfg = dict(n_layers=int(g.number(arch + ".block_count")), hidden=hidden, n_q_heads=heads,
+                        n_kv_heads=int(opt("attention.head_count_kv", heads)),
+                        head_dim=int(opt("attention.key_length", hidden // heads)), vocab=self.vocab,
+                        max_context=int(ffi.lib().tsv_max_context(h)))
+        g.close()
+        return self
+
     def close(self):
         if getattr(self, "_h", None):
             ffi.lib().tsv_close(self._h)
