@@ -333,11 +333,12 @@ int32_t tsv_gguf_meta_number(const tsv_gguf* g, const char* key, double* out);
 int32_t tsv_gguf_meta_string(const tsv_gguf* g, const char* key, char* buf, int32_t cap);
 /* Opens a llama-family GGUF as a verify target: tensor names of crates/repack/src/gguf_names/
  * llama.rs:14-60 (`llama`; `qwen2` adds the q / k / v biases; `qwen3` / `qwen3moe` the per-head
- * q / k norms; routed experts as the stacked *_exps tensors), sizes from the `<arch>.*` metadata,
+ * q / k norms; routed experts as the stacked *_exps tensors; `gpt-oss` by gguf_names/gpt_oss.rs:30-72
+ * with its biases, sinks, YaRN keys and the window on even layers), sizes from the `<arch>.*` metadata,
  * the q / k rows of a `llama` file un-permuted from llama.cpp's adjacent-pair order
  * (crates/repack/src/gguf_checkpoint/conventions.rs:133-243).  rope_freqs.weight, which the
  * reference refuses for this family, is taken as the llama-3 per-pair divisors; any other context
- * extension (rope.scaling.type) and partial rotation are refused.  max_context <= 0: the file's
+ * extension (rope.scaling.type, but gpt-oss's yarn) and partial rotation are refused.  max_context <= 0: the file's
  * context_length.  The mapping is dropped before the call returns. */
 int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx** out);
 

@@ -77,6 +77,12 @@ def llama_gguf(path, cfg, weights, arch="llama", permute=True):
                  (f"{arch}.expert_feed_forward_length", "u32", cfg["ffn"])]
     else:
         meta.append((f"{arch}.feed_forward_length", "u32", cfg["ffn"]))
+    oss = cfg.get("gptoss")
+    if oss:
+        factor, octx, bf, bs = oss["yarn"]
+        meta += [(f"{arch}.attention.sliding_window", "u32", oss["window"]), (f"{arch}.rope.scaling.type", "str", "yarn"),
+                 (f"{arch}.rope.scaling.factor", "f32", factor), (f"{arch}.rope.scaling.original_context_length", "u32", octx),
+                 (f"{arch}.rope.scaling.yarn_beta_fast", "f32", bf), (f"{arch}.rope.scaling.yarn_beta_slow", "f32", bs)]
     out = []
 
     def add(name, t, rot=False, expert_rows=0):
@@ -98,7 +104,10 @@ def llama_gguf(path, cfg, weights, arch="llama", permute=True):
         out.append(("rope_freqs.weight", [f.size], 0, f.tobytes()))
     names = dict(attn_norm="attn_norm.weight", wv="attn_v.weight", wo="attn_output.weight", ffn_norm="ffn_norm.weight",
                  q_norm="attn_q_norm.weight", k_norm="attn_k_norm.weight", w_gate="ffn_gate.weight", w_up="ffn_up.weight",
-                 w_down="ffn_down.weight", router="ffn_gate_inp.weight", bq="attn_q.bias", bk="attn_k.bias", bv="attn_v.bias")
+                 w_down="ffn_down.weight", router="ffn_gate_inp.weight", bq="attn_q.bias", bk="attn_k.bias", bv="attn_v.bias",
+                 bo="attn_output.bias", sinks="attn_sinks.weight", router_bias="ffn_gate_inp.bias")
+    if oss:
+        names["ffn_norm"] = "post_attention_norm.weight"
     for li, lw in enumerate(weights["layers"]):
         p = f"blk.{li}."
         add(p + "attn_q.weight", lw["wq"], rot=permute)
@@ -110,4 +119,7 @@ def llama_gguf(path, cfg, weights, arch="llama", permute=True):
             add(p + "ffn_gate_exps.weight", lw["we_gate"], expert_rows=cfg["ffn"])
             add(p + "ffn_up_exps.weight", lw["we_up"], expert_rows=cfg["ffn"])
             add(p + "ffn_down_exps.weight", lw["we_down"], expert_rows=H)
+            for key, name in (("be_gate", "ffn_gate_exps.bias"), ("be_up", "ffn_up_exps.bias"), ("be_down", "ffn_down_exps.bias")):
+                if lw.get(key) is not None:
+                    add(p + name, lw[key])
     return write_gguf(path, meta, out)

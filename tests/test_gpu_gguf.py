@@ -27,6 +27,7 @@ def _both(tmp_path, name, arch, permute, max_context=96, **over):
     ("small_q4_k_m", "llama", True),       # the Q4_K + Q6_K mix of a Q4_K_M file, 128-wide heads
     ("small_q5_k_m", "llama", True),
     ("moe_small", "qwen3moe", False),      # per-head q / k norms, stacked MXFP4 experts, Q8_0 router
+    ("gptoss_small", "gpt-oss", False),    # bf16 attention with biases and sinks, window on even layers, YaRN, expert biases
 ])
 def test_a_gguf_target_equals_the_directly_installed_one(tmp_path, name, arch, permute):
     cfg, w, path, direct, filed = _both(tmp_path, name, arch, permute)

@@ -351,7 +351,8 @@ extern "C" int32_t tsv_gguf_meta_string(const tsv_gguf* g, const char* key, char
 }
 
 // Opens a dense or routed-expert llama-family GGUF as a verify target: `llama` (q / k rows
-// un-permuted), `qwen2` (q / k / v biases), `qwen3` and `qwen3moe` (per-head q / k norms).
+// un-permuted), `qwen2` (q / k / v biases), `qwen3` and `qwen3moe` (per-head q / k norms),
+// `gpt-oss` (biases, sinks, alternating window, YaRN, clamped SwiGLU).
 extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx** out) {
     if (!out) {
         set_error("open_gguf: null output");
@@ -370,8 +371,9 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
     }
     const std::string arch = av->s;
     const bool is_llama = arch == "llama", is_qwen2 = arch == "qwen2", is_qwen3 = arch == "qwen3" || arch == "qwen3moe";
-    if (!is_llama && !is_qwen2 && !is_qwen3) {
-        set_error("open_gguf: architecture '" + arch + "' is not one this intake maps (llama, qwen2, qwen3, qwen3moe)");
+    const bool is_oss = arch == "gpt-oss";
+    if (!is_llama && !is_qwen2 && !is_qwen3 && !is_oss) {
+        set_error("open_gguf: architecture '" + arch + "' is not one this intake maps (llama, qwen2, qwen3, qwen3moe, gpt-oss)");
         return TSV_ERR_UNSUPPORTED;
     }
     auto need = [&](const char* suffix, double* v) {
@@ -399,10 +401,14 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
     }
     // a context-extension scheme this intake cannot express must refuse, not load a model that is
     // only wrong at long context
+    bool yarn = false;
     if (const Value* st = meta(*g, arch + ".rope.scaling.type"))
         if (st->kind == Value::STRING && st->s != "none" && !st->s.empty()) {
-            set_error("open_gguf: rope scaling '" + st->s + "' is not mapped");
-            return TSV_ERR_UNSUPPORTED;
+            yarn = is_oss && st->s == "yarn";
+            if (!yarn) {
+                set_error("open_gguf: rope scaling '" + st->s + "' is not mapped");
+                return TSV_ERR_UNSUPPORTED;
+            }
         }
 
     tsv_model_desc d{};
@@ -423,6 +429,36 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
     if (opt("rope.dimension_count", d.head_dim) != d.head_dim) {
         set_error("open_gguf: partial rotation (rope.dimension_count below the head width) is not mapped");
         return TSV_ERR_UNSUPPORTED;
+    }
+
+    // gpt-oss: YaRN frequency table and magnitude scale (crates/repack/src/gguf_config/mod.rs:396-440:
+    // factor and original context are required once the type says yarn, the betas default to
+    // llama.cpp's 32 and 1), the clamped SwiGLU's constants (crates/gpu/src/shaders/moe_gguf.metal:528-556),
+    // and a sliding window on EVEN layers (crates/runtime/src/families/gptoss/attn.rs:20-23).
+    std::vector<float> yarn_freqs;
+    double window = 0;
+    if (is_oss) {
+        if (yarn) {
+            double factor, octx;
+            if (!need("rope.scaling.factor", &factor) || !need("rope.scaling.original_context_length", &octx)) return TSV_ERR_INVALID;
+            if (factor <= 0) {
+                set_error("open_gguf: yarn factor is not usable");
+                return TSV_ERR_INVALID;
+            }
+            if (meta(*g, arch + ".rope.scaling.yarn_log_multiplier")) {
+                set_error("open_gguf: a yarn_log_multiplier other than the plain one is not mapped");
+                return TSV_ERR_UNSUPPORTED;
+            }
+            yarn_freqs.resize((size_t)d.head_dim / 2);
+            if ((rc = tsv_yarn_frequencies(d.head_dim, d.rope_theta, (float)factor, (int64_t)octx,
+                                           (float)opt("rope.scaling.yarn_beta_fast", 32.0),
+                                           (float)opt("rope.scaling.yarn_beta_slow", 1.0), yarn_freqs.data(), &d.rope_mscale)))
+                return rc;
+            d.rope_freqs = yarn_freqs.data();
+        }
+        d.act_alpha = 1.702f;
+        d.act_limit = 7.0f;
+        if (!need("attention.sliding_window", &window)) return TSV_ERR_INVALID;
     }
 
     std::vector<std::vector<uint8_t>> owned;  // un-permuted q / k rows
@@ -463,17 +499,26 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
         const Slot slots[] = {
             {"attn_norm.weight", &L.attn_norm, true}, {"attn_q.weight", &L.wq, true}, {"attn_k.weight", &L.wk, true},
             {"attn_v.weight", &L.wv, true}, {"attn_output.weight", &L.wo, true},
-            {"ffn_norm.weight", &L.ffn_norm, true},  // the pre-FFN norm (HF: post_attention_layernorm)
+            // the pre-FFN norm (HF: post_attention_layernorm); gpt-oss files spell it post_attention_norm
+            {is_oss ? "post_attention_norm.weight" : "ffn_norm.weight", &L.ffn_norm, true},
             {"attn_q_norm.weight", &L.q_norm, is_qwen3}, {"attn_k_norm.weight", &L.k_norm, is_qwen3},
-            {"attn_q.bias", &L.bq, is_qwen2}, {"attn_k.bias", &L.bk, is_qwen2}, {"attn_v.bias", &L.bv, is_qwen2},
+            {"attn_q.bias", &L.bq, is_qwen2 || is_oss}, {"attn_k.bias", &L.bk, is_qwen2 || is_oss},
+            {"attn_v.bias", &L.bv, is_qwen2 || is_oss},
+            // gpt-oss (crates/repack/src/gguf_names/gpt_oss.rs:30-72): every projection and the router
+            // carry a bias, one sink logit per q head, per-expert biases
+            {"attn_output.bias", &L.bo, is_oss}, {"attn_sinks.weight", &L.sinks, is_oss},
+            {"ffn_gate_inp.bias", &L.router_bias, is_oss}, {"ffn_gate_exps.bias", &L.be_gate, is_oss},
+            {"ffn_up_exps.bias", &L.be_up, is_oss}, {"ffn_down_exps.bias", &L.be_down, is_oss},
             {"ffn_gate.weight", &L.w_gate, !routed}, {"ffn_up.weight", &L.w_up, !routed}, {"ffn_down.weight", &L.w_down, !routed},
             {"ffn_gate_inp.weight", &L.router, routed}, {"ffn_gate_exps.weight", &L.we_gate, routed},
             {"ffn_up_exps.weight", &L.we_up, routed}, {"ffn_down_exps.weight", &L.we_down, routed},
         };
         for (const Slot& s : slots) {
-            if (!s.required && !g->tensors.count(p + s.suffix)) continue;
+            // a slot another family owns is not read even when a file carries the name
+            if (!s.required) continue;
             if ((rc = get(p + s.suffix, s.t, s.required))) return rc;
         }
+        if (is_oss && l % 2 == 0) L.window = (int32_t)window;
         if (routed) {
             L.n_experts = (int32_t)n_experts;
             L.top_k = (int32_t)opt("expert_used_count", 0);
