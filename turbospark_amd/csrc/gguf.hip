@@ -395,8 +395,11 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
     } else if (!need("feed_forward_length", &ffn)) {
         return TSV_ERR_INVALID;
     }
-    if (n_layers < 1 || n_layers > 4096 || hidden < 1 || n_heads < 1 || ffn < 1) {
-        set_error("open_gguf: the model sizes in the metadata are not positive");
+    const double kv_heads = opt("attention.head_count_kv", n_heads), key_len = opt("attention.key_length", hidden / n_heads);
+    auto sane = [](double v, double hi) { return v >= 1 && v <= hi && v == (double)(int64_t)v; };
+    if (!sane(n_layers, 4096) || !sane(hidden, 1 << 20) || !sane(n_heads, 1 << 16) || !sane(ffn, 1 << 24) ||
+        !sane(kv_heads, 1 << 16) || !sane(key_len, 1024) || (n_experts != 0 && !sane(n_experts, 1 << 16))) {
+        set_error("open_gguf: the model sizes in the metadata are not usable (layers, widths, head counts, experts)");
         return TSV_ERR_INVALID;
     }
     // a context-extension scheme this intake cannot express must refuse, not load a model that is
@@ -415,8 +418,8 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
     d.n_layers = (int32_t)n_layers;
     d.hidden = (int32_t)hidden;
     d.n_q_heads = (int32_t)n_heads;
-    d.n_kv_heads = (int32_t)opt("attention.head_count_kv", n_heads);
-    d.head_dim = (int32_t)opt("attention.key_length", hidden / n_heads);
+    d.n_kv_heads = (int32_t)kv_heads;
+    d.head_dim = (int32_t)key_len;
     d.ffn = (int32_t)ffn;
     d.rms_eps = (float)opt("attention.layer_norm_rms_epsilon", 1e-5);
     d.rope_theta = (float)opt("rope.freq_base", 10000.0);
@@ -459,6 +462,10 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
         d.act_alpha = 1.702f;
         d.act_limit = 7.0f;
         if (!need("attention.sliding_window", &window)) return TSV_ERR_INVALID;
+        if (!sane(window, 1 << 30)) {
+            set_error("open_gguf: attention.sliding_window is not usable");
+            return TSV_ERR_INVALID;
+        }
     }
 
     std::vector<std::vector<uint8_t>> owned;  // un-permuted q / k rows
@@ -521,7 +528,8 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
         if (is_oss && l % 2 == 0) L.window = (int32_t)window;
         if (routed) {
             L.n_experts = (int32_t)n_experts;
-            L.top_k = (int32_t)opt("expert_used_count", 0);
+            const double used = opt("expert_used_count", 0);
+            L.top_k = used >= 1 && used <= n_experts ? (int32_t)used : 0;  // 0 is refused by tsv_open
         }
         if (is_llama)
             for (tsv_tensor* t : {&L.wq, &L.wk}) {
