@@ -132,3 +132,52 @@ def test_the_writers_permutation_is_the_converters():
     assert perm[:D].tolist() == [0, 4, 1, 5, 2, 6, 3, 7] and perm[D:].tolist() == [8, 12, 9, 13, 10, 14, 11, 15]
     for i in range(D):
         assert perm[(i % (D // 2)) * 2 + i // (D // 2)] == i
+
+
+def _nested(depth):
+    """`depth` array headers of one element each around a u32 7 (crates/repack/tests/gguf_header.rs:191-216)."""
+    import struct
+    body = b"".join(struct.pack("<IQ", 9, 1) for _ in range(depth - 1)) + struct.pack("<IQ", 4, 1) + struct.pack("<I", 7)
+    return b"GGUF" + struct.pack("<IQQ", 3, 0, 1) + struct.pack("<Q", 6) + b"nested" + struct.pack("<I", 9) + body + b"\0" * 64
+
+
+def test_the_array_nesting_limit_is_exact(tmp_path):
+    # crates/repack/tests/gguf_header.rs:259-285: 64 levels parse, 65 are refused
+    path = os.path.join(tmp_path, "n.gguf")
+    open(path, "wb").write(_nested(64))
+    g = ffi.Gguf(path)
+    assert g.tensor_count == 0
+    g.close()
+    open(path, "wb").write(_nested(65))
+    with pytest.raises(ffi.TsvError, match="nested deeper than 64"):
+        ffi.Gguf(path)
+
+
+def test_the_references_own_fixture_scenario(tmp_path):
+    # crates/repack/tests/gguf_header.rs:18-110: mixed metadata kinds, a 3-D stacked tensor, the
+    # default alignment, and tensor ranges that are the writer's own
+    rng = np.random.default_rng(1)
+    gate = rng.integers(0, 256, 512 // 32 * 34, dtype=np.uint8).tobytes()
+    q = rng.integers(0, 256, 64 * 32 // 32 * 34, dtype=np.uint8).tobytes()
+    meta = [("general.architecture", "str", "gemma4"), ("gemma4.block_count", "u32", 2),
+            ("gemma4.attention.layer_norm_rms_epsilon", "f32", 1e-6), ("general.file_type", "u8", 7),
+            ("truncated", "bool", 1), ("signed", "i32", -3), ("wide", "u64", 1 << 40),
+            ("tokenizer.ggml.tokens", "arr", ("str", ["<pad>", "hi"])), ("nested", "arr", ("arr", [("u32", [1, 2])]))]
+    path = os.path.join(tmp_path, "f.gguf")
+    start = write_gguf(path, meta, [("blk.0.ffn_gate_exps.weight", [64, 2, 4], 8, gate),
+                                    ("blk.0.attn_q.weight", [64, 32], 8, q), ("output_norm.weight", [8], 0, b"\0" * 32)])
+    g = ffi.Gguf(path)
+    assert g.string("general.architecture") == "gemma4" and g.number("gemma4.block_count") == 2
+    assert g.number("wide") == float(1 << 40) and g.number("signed") == -3 and g.number("truncated") == 1
+    assert g.number("gemma4.attention.layer_norm_rms_epsilon") == float(np.float32(1e-6))
+    assert g.data_start == start and start % 32 == 0 and g.tensor_count == 3
+    dt, raw, rows, cols = g.tensor("blk.0.ffn_gate_exps.weight")
+    assert (dt, rows, cols) == (8, 8, 64) and raw.size == 512 // 32 * 34 and raw.tobytes() == gate
+    dt, raw, rows, cols = g.tensor("blk.0.attn_q.weight")
+    assert (dt, rows, cols) == (8, 32, 64) and raw.tobytes() == q
+    # block sizes of the types this library has kernels for, as the format's table gives them
+    # (crates/repack/tests/gguf_header.rs:548-560): (elements, bytes) per block
+    for tid, (elems, nbytes) in {0: (1, 4), 1: (1, 2), 8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210),
+                                 30: (1, 2), 39: (32, 17)}.items():
+        assert ffi.row_bytes(tid, 256) == 256 // elems * nbytes, tid
+    g.close()
