@@ -21,20 +21,57 @@ namespace {
 
 // ---- router ---------------------------------------------------------------------------------
 // One workgroup, one wave per row: the row's logits (split-K partials summed in order) sit
-// 'ne / 64' per lane; k rounds of a wave-wide arg-max (larger logit, then lower index) pick the
-// experts in rank order.  Then one thread per (row, slot) pair decides whether its expert
-// appears here for the first time and, if so, lists every pair that shares it, in row order.
+// 'ne / 64' per lane as order-preserving integer keys; k rounds of two wave-wide reductions on the
+// DPP network (the largest key, then the lowest index that holds it: larger logit, then lower
+// index) pick the experts in rank order.  Then one thread per (row, slot) pair finds the first
+// pair that chose its expert -- the group's leader -- and its own place among that group's
+// members, which are listed in pair order.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_from(uint32_t v) {  // a lane without a source keeps its own value
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+// quad swaps, shifts by four and eight inside a row of sixteen, then the rows' last lanes handed
+// on to the next row(s): lane 63 ends up with the reduction of all 64 (max and min are idempotent,
+// so lanes that see a value twice do no harm)
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+    v = max(v, dpp_from<0xb1, 0xf>(v));
+    v = max(v, dpp_from<0x4e, 0xf>(v));
+    v = max(v, dpp_from<0x114, 0xf>(v));
+    v = max(v, dpp_from<0x118, 0xf>(v));
+    v = max(v, dpp_from<0x142, 0xa>(v));
+    v = max(v, dpp_from<0x143, 0xc>(v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+__device__ __forceinline__ uint32_t wave_umin(uint32_t v) {
+    v = min(v, dpp_from<0xb1, 0xf>(v));
+    v = min(v, dpp_from<0x4e, 0xf>(v));
+    v = min(v, dpp_from<0x114, 0xf>(v));
+    v = min(v, dpp_from<0x118, 0xf>(v));
+    v = min(v, dpp_from<0x142, 0xa>(v));
+    v = min(v, dpp_from<0x143, 0xc>(v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+// float -> unsigned key with the same order (-0 is folded into +0 first, so equal floats have equal
+// keys); key 0 is below every float's key and marks an expert that is taken or absent
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = __float_as_uint(f + 0.0f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key);
+}
+
 __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
-    __shared__ int s_sel[TSV_MAX_ROWS * 8];
+    __shared__ int s_sel[TSV_MAX_ROWS * 8];    // the selected experts, pair index = row * k + slot
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int M = a.vp->m, ne = a.n_experts, k = a.top_k;
+    const int M = a.m, ne = a.n_experts, k = a.top_k;
     if (wave < M) {
         const int m = wave;
-        float v[4];
+        uint32_t key[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int e = lane + 64 * j;
-            v[j] = -INFINITY;
+            key[j] = 0;
             if (e < ne) {
                 float part[8], s = 0.f;  // all partials in flight together, added in split order
 #pragma unroll
@@ -43,7 +80,7 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
                 for (int sp = 0; sp < 8; sp++)
                     if (sp < a.splits) s += part[sp];
                 if (a.bias) s += a.bias[e];  // before the top-k (families/gptoss/moe.rs:82-87)
-                v[j] = s;
+                key[j] = order_key(s);
             }
         }
         float top = 0.f, sum = 0.f, my_ex = 0.f;
@@ -51,22 +88,14 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
 #pragma unroll
         for (int r = 0; r < 8; r++) {
             if (r < k) {
-                float best = -INFINITY;
-                int bi = 0x7FFFFFFF;
+                const uint32_t mine = max(max(key[0], key[1]), max(key[2], key[3]));
+                const uint32_t kbest = wave_umax(mine);
+                uint32_t idx = 0xFFFFFFFFu;  // ascending j is ascending index: the first maximum wins
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (v[j] > best) {  // ascending j is ascending index: the first maximum wins
-                        best = v[j];
-                        bi = lane + 64 * j;
-                    }
-                for (int o = 32; o > 0; o >>= 1) {
-                    const float ob = __shfl_xor(best, o);
-                    const int oi = __shfl_xor(bi, o);
-                    if (ob > best || (ob == best && oi < bi)) {
-                        best = ob;
-                        bi = oi;
-                    }
-                }
+                for (int j = 3; j >= 0; j--)
+                    if (key[j] == kbest) idx = (uint32_t)(lane + 64 * j);
+                const int bi = (int)min(wave_umin(idx), (uint32_t)(ne - 1));
+                const float best = key_value(kbest);
                 if (r == 0) top = best;
                 const float ex = expf(best - top);
                 sum += ex;  // sequential in rank order, as `exps.iter().sum()`
@@ -76,7 +105,7 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
                 }
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    if (lane + 64 * j == bi) v[j] = -INFINITY;
+                    if (lane + 64 * j == bi) key[j] = 0;
             }
         }
         if (lane < k) {
@@ -86,22 +115,30 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
         }
     }
     __syncthreads();
+    // Groups: pair j leads the group of its expert when no earlier pair chose it; the members of a
+    // group are listed in pair order.  Every pair finds its own place (how many earlier pairs share
+    // its expert, and which of them is the first) in one pass over the selections.
     const int j = threadIdx.x, np = M * k;
     if (j >= np) return;
     const int e = s_sel[j];
-    bool leader = true;
-    for (int i = 0; i < j; i++) leader &= s_sel[i] != e;
+    int first = j, pos = 0, cnt = 0;
+    for (int i = 0; i < np; i++) {
+        const bool same = s_sel[i] == e;
+        cnt += same ? 1 : 0;
+        if (same && i < j) {
+            pos++;
+            first = min(first, i);
+        }
+    }
+    const int row = j / k;
+    if (pos < TSV_MAX_ROWS) {  // a row chooses an expert once, so a group never has more members than rows
+        MoeGroup* lead = a.groups + first;
+        lead->rows[pos] = row;
+        lead->slots[pos] = j - row * k;
+    }
     MoeGroup* g = a.groups + j;
-    int n = 0;
-    if (leader)
-        for (int i = j; i < np; i++)
-            if (s_sel[i] == e) {
-                g->rows[n] = i / k;
-                g->slots[n] = i - (i / k) * k;
-                n++;
-            }
     g->expert = e;
-    g->cnt = n;
+    g->cnt = first == j ? min(cnt, TSV_MAX_ROWS) : 0;
 }
 
 // ---- grouped expert matmul --------------------------------------------------------------------

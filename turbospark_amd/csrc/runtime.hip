@@ -566,7 +566,7 @@ int launch_pass(tsv_ctx* c, int m) {
             ra2.ld = L.n_experts;
             ra2.n_experts = L.n_experts;
             ra2.top_k = L.top_k;
-            ra2.vp = c->vp_dev;
+            ra2.m = m;
             ra2.weights = c->route_w;
             ra2.selected = c->route_sel;
             ra2.groups = c->route_groups;

@@ -151,7 +151,7 @@ struct MoeGroup {
 struct MoeRouteArgs {
     const float* logits;  // router matmul partials [splits][16][ld]
     int splits, ld, n_experts, top_k;
-    const VerifyParams* vp;
+    int m;              // rows of the pass (the launch sequence is per row count)
     float* weights;     // [16][8] softmax over the selected logits, rank order
     int32_t* selected;  // [16][8] expert ids, rank order
     MoeGroup* groups;   // [16 * 8]
