@@ -91,3 +91,31 @@ def test_moe_greedy_round_matches_the_oracle_walk():
     assert res.accepted == want_acc >= 3
     assert res.next == int(np.argmax(logits[want_acc]))
     assert res.kv_position == base + want_acc + 1
+
+
+@pytest.mark.parametrize("top_k", [1, 3, 5])
+def test_exactly_tied_router_logits_go_to_the_lower_expert(top_k):
+    """real_forward_dispatch.rs:1135-1158: experts sort by logit, ties to the lower index.  Every odd
+    expert's router row is a copy of its even neighbour's, so each logit comes twice, bit for bit,
+    and with an odd top-k the last selection is always one half of a tied pair.  The experts
+    themselves differ, so taking the wrong half changes the logits far beyond the tolerance."""
+    import turbospark_amd as ts
+    from oracle import binding as ob
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS["moe_small"], max_context=64, top_k=top_k)
+    w = synth.make_weights(cfg, seed=77)
+    for lw in w["layers"]:
+        dt, raw, rows, cols = lw["router"]
+        raw = raw.copy()
+        raw[1::2] = raw[0::2]
+        lw["router"] = (dt, raw, rows, cols)
+    gpu = ts.HipVerifier(cfg, w)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=8)
+    prompt, feed = _prompt(24, cfg["vocab"], 3), _prompt(9, cfg["vocab"], 4)
+    for i in range(0, 24, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    want = cpu.verify(feed, 24)
+    gpu.prefill(prompt, 0, want_logits=False)
+    err = gc.logit_error(gpu.verify(feed, 24), want)
+    print(f"tied router, top-{top_k}: max-abs logit error / range = {err:.2e}")
+    assert err <= MXFP4_TOL, err
