@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from tests import gpu_common as gc
+from turbospark_amd import ffi
 from tests.loop_common import GpuTarget, LmDrafter
 
 pytestmark = pytest.mark.gpu
@@ -49,10 +50,10 @@ def test_reuse_answers_nothing_until_the_host_opts_in_and_keys_on_what_was_fed()
     assert gpu.position == 24 and gpu.prefix_len() == 19
     gpu.record_committed(feed[:3], 19)
     assert gpu.prefix_len() == 22
-    gpu.rollback_retaining(__import__("turbospark_amd").ffi.Point(19), 3)
+    gpu.rollback_retaining(ffi.Point(19), 3)
     assert gpu.position == 22 and gpu.try_reuse_prefix(ids) == 22
     # a plain rollback shortens the record with the cache
-    gpu.rollback(__import__("turbospark_amd").ffi.Point(10))
+    gpu.rollback(ffi.Point(10))
     assert gpu.prefix_len() == 10 and gpu.try_reuse_prefix(ids) == 10
     # rows written without token ids describe nothing reusable until the next reset
     k, v = gpu.read_kv(0, 0, 4)
