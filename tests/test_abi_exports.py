@@ -112,10 +112,27 @@ def test_null_handles_are_refused_by_name_without_a_gpu():
         lambda: L.tsv_read_kv(None, 0, 0, 1, out, out),
         lambda: L.tsv_write_kv(None, 0, 0, 1, out, out),
         lambda: L.tsv_write_logits(None, out, 1, 0),
+        lambda: L.tsv_set_prefix_reuse(None, 1),
+        lambda: L.tsv_record_committed(None, tok, 4, 0),
+        lambda: L.tsv_try_reuse_prefix(None, tok, 4),          # -1
+        lambda: L.tsv_gguf_open(None, None),
+        lambda: L.tsv_gguf_tensor(None, b"x", None),
+        lambda: L.tsv_gguf_meta_number(None, b"x", None),
+        lambda: L.tsv_gguf_meta_string(None, b"x", None, 0),
+        lambda: L.tsv_open_gguf(None, 0, C.byref(C.c_void_p())),
     ]
     for i, call in enumerate(calls):
         assert call() != 0, i
         assert ffi.last_error(), i
+    assert L.tsv_prefix_len(None) == -1 and L.tsv_gguf_tensor_count(None) == -1 and L.tsv_gguf_data_start(None) == -1
+    # the record on its own tolerates null and empty arguments
+    L.tsv_prefix_free(None)
+    L.tsv_prefix_clear(None)
+    L.tsv_prefix_record(None, tok, 4, 0)
+    assert L.tsv_prefix_common(None, tok, 4) == 0 and L.tsv_prefix_untainted_len(None) == -1
+    rec = ffi.KvPrefix([1, 2, 3])
+    L.tsv_prefix_record(rec._p, None, 0, 3)                    # nothing fed at the end: no change
+    assert rec.untainted_len() == 3 and L.tsv_prefix_common(rec._p, None, 0) == 0
     desc = ffi.ModelDesc()
     layers = (ffi.Layer * 1)()
     desc.layers = C.cast(layers, type(desc.layers))
