@@ -359,12 +359,19 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
         rc = launch_partial<HD, 2, 3>(s, a, G, R, groups);
     if (rc) return rc;
     const dim3 cgrid(m, a.nq), cblock(HD < 64 ? 64 : HD);
+    // the chunk count as a compile-time constant puts every partial's load in flight before the
+    // first add (a counted loop waits on each in turn); the sum runs in the same order either way
+#define TSV_COMBINE(N) \
+    case N: hipLaunchKernelGGL(k_attn_combine<N>, cgrid, cblock, 0, s, a, G, R); break;
     switch (a.nch) {
-        case 8: hipLaunchKernelGGL(k_attn_combine<8>, cgrid, cblock, 0, s, a, G, R); break;
-        case 16: hipLaunchKernelGGL(k_attn_combine<16>, cgrid, cblock, 0, s, a, G, R); break;
-        case 32: hipLaunchKernelGGL(k_attn_combine<32>, cgrid, cblock, 0, s, a, G, R); break;
+        TSV_COMBINE(1) TSV_COMBINE(2) TSV_COMBINE(3) TSV_COMBINE(4) TSV_COMBINE(5) TSV_COMBINE(6) TSV_COMBINE(7) TSV_COMBINE(8)
+        TSV_COMBINE(9) TSV_COMBINE(10) TSV_COMBINE(11) TSV_COMBINE(12) TSV_COMBINE(13) TSV_COMBINE(14) TSV_COMBINE(15)
+        TSV_COMBINE(16) TSV_COMBINE(17) TSV_COMBINE(18) TSV_COMBINE(19) TSV_COMBINE(20) TSV_COMBINE(21) TSV_COMBINE(22)
+        TSV_COMBINE(23) TSV_COMBINE(24) TSV_COMBINE(25) TSV_COMBINE(26) TSV_COMBINE(27) TSV_COMBINE(28) TSV_COMBINE(29)
+        TSV_COMBINE(30) TSV_COMBINE(31) TSV_COMBINE(32)
         default: hipLaunchKernelGGL(k_attn_combine<0>, cgrid, cblock, 0, s, a, G, R); break;
     }
+#undef TSV_COMBINE
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
