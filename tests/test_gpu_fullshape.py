@@ -226,3 +226,125 @@ def test_llama3_8b_all_32_layers_generation_loop_properties():
     sampled = gpu.run_speculative(prompt, LmDrafter(GpuTarget(twin), prompt[0], V), ts.shaping(0.8, seed=2, top_p=0.95), new, 4)
     assert sampled["accepted"] == sampled["offered"] and len(sampled["tokens"]) == new
     assert sampled["min_margin"] >= 0.0
+
+
+def test_qwen3_30b_a3b_shape_two_layers_at_long_context():
+    """Configuration 4 at its own geometry: hidden 2048, 32q / 4kv x 128 with the per-head q / k norm,
+    128 MXFP4 experts of width 768 routed top-8, Q8_0 attention / router / head, the full 151 936-row
+    vocabulary, nine rows (72 (row, q head) pairs per KV head: three attention row groups), two layers
+    at a 3000-token context.  Logits, the new cache rows and the greedy round against the oracle."""
+    import turbospark_amd as ts
+    ctx = 3000
+    cfg, gpu, cpu = _filled("qwen3_30b_a3b", ctx, 2)
+    V = cfg["vocab"]
+    for attempt in range(8):
+        rng = np.random.default_rng(40 + attempt)
+        # proposals: the oracle's own greedy continuation for three tokens, then junk
+        toks = [int(rng.integers(0, V))]
+        margins = []
+        for i in range(3):
+            cpu.rewind_to(ctx + i)
+            row = cpu.verify(toks[-1:], ctx + i)
+            margins.append(cpu.route_margin)
+            toks.append(int(np.argmax(gc.f16(row[0]))))
+        feed = np.array(toks + [int(t) for t in rng.integers(0, V, 5)], np.int32)
+        cpu.rewind_to(ctx)
+        want = cpu.verify(feed, ctx)
+        margins.append(cpu.route_margin)
+        if min(margins) > 2e-3:
+            break
+    else:
+        raise AssertionError("no feed without a near-tie routing decision")
+    got = gpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"Qwen3-30B-A3B shape, 2 layers, ctx {ctx}, m=9, vocab {V}: max-abs logit error / range = {err:.2e}, "
+          f"route margin {min(margins):.2e}")
+    assert err <= 1e-2
+    for layer in range(2):
+        kg, vg = gpu.read_kv(layer, ctx, 9)
+        kc, vc = cpu.kv(layer)
+        assert np.abs(kg.astype(np.float32) - kc[ctx:ctx + 9]).max() <= 2e-2 * np.abs(kc[ctx:ctx + 9]).max()
+        assert np.abs(vg.astype(np.float32) - vc[ctx:ctx + 9]).max() <= 2e-2 * np.abs(vc[ctx:ctx + 9]).max()
+    # the greedy round on the device: integers equal to the oracle's walk over the same fp16 logits ...
+    res = gpu.accept(feed, ctx, ts.shaping(0.0))
+    ref = ob.chain_round(got, None, feed[1:], ob.shaping(0.0))
+    assert (res.accepted, res.committed, res.next, res.stopped) == (ref["accepted"], ref["committed"], ref["next"], 0)
+    assert res.kv_position == ctx + ref["committed"] + 1 == gpu.position
+    # ... and, the routing decisions being clear of ties, to the walk over the oracle's own logits
+    own = ob.chain_round(want, None, feed[1:], ob.shaping(0.0))
+    assert res.accepted == own["accepted"] >= 3 and res.next == own["next"]
+
+
+def _cycled(name, ctx, distinct, seed=3):
+    """The configuration at its full depth with `distinct` seeded layers repeated down the stack (the
+    size-independent properties below do not care that layers repeat; synthesizing 128 experts for every
+    one of 36-48 layers would take minutes of host time).  Every layer still gets its own copy on the device."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS[name], max_context=ctx + 32)
+    w = synth.make_weights(cfg, seed=seed, n_layers=distinct)
+    w["layers"] = [w["layers"][i % distinct] for i in range(cfg["n_layers"])]
+    gpu = ts.HipVerifier(cfg, w)
+    rng = np.random.default_rng(seed)
+    shape = (ctx, cfg["n_kv_heads"], cfg["head_dim"])
+    k = (rng.standard_normal(shape, dtype=np.float32) * 0.5).astype(np.float16)
+    v = (rng.standard_normal(shape, dtype=np.float32) * 0.5).astype(np.float16)
+    for layer in range(cfg["n_layers"]):
+        s = 37 * layer % ctx
+        gpu.write_kv(layer, 0, np.roll(k, s, axis=0), np.roll(v, -s, axis=0))
+    assert gpu.position == ctx
+    return cfg, gpu
+
+
+def _size_independent_properties(cfg, gpu, ctx, m, shaping_kw, temperature):
+    """Deterministic by bits; a rollback leaves nothing behind; a chain-shaped tree is the chain by bits;
+    the fused round equals verify followed by accept and the oracle's walk over the same logits; rows
+    fed one at a time agree with the batched pass (by tolerance where the attention splits differ with
+    the row count, see families/qwen/batched.rs:92-110 for the contract)."""
+    import turbospark_amd as ts
+    V = cfg["vocab"]
+    rng = np.random.default_rng(5)
+    feed = rng.integers(0, V, m).astype(np.int32)
+    point = gpu.checkpoint()
+    a = gpu.verify(feed, ctx)
+    gpu.rollback(point)
+    b = gpu.verify(feed, ctx)
+    assert np.array_equal(a, b)
+    gpu.rollback(point)
+    t = gpu.verify_tree(feed, list(range(-1, m - 1)), ctx)
+    assert np.array_equal(a, t)
+    gpu.rollback(point)
+    seq = np.stack([gpu.produce(int(tok), ctx + i) for i, tok in enumerate(feed)])
+    err = gc.logit_error(seq, a)
+    print(f"{cfg['n_layers']} layers, ctx {ctx}, m={m}: batched vs one row at a time, max-abs / range = {err:.2e}")
+    assert err <= 2e-3
+    gpu.rollback(point)
+    draft = rng.standard_normal((m - 1, V)).astype(np.float16) if temperature else None
+    gs = ts.shaping(temperature, seed=11 if temperature else None, **shaping_kw)
+    os_ = ob.shaping(temperature, seed=11 if temperature else None, **shaping_kw)
+    fused = gpu.verify_accept(feed, ctx, gs, draft_logits=draft, draw_step=9)
+    gpu.rollback(point)
+    gpu.verify(feed, ctx, want_logits=False)
+    split = gpu.accept(feed, ctx, gs, draft_logits=draft, draw_step=9)
+    assert fused == split and fused.kv_position == ctx + fused.committed + 1
+    ref = ob.chain_round(a, draft, feed[1:], os_, history=[int(feed[0])], draw_step=9)
+    assert (fused.accepted, fused.committed, fused.next) == (ref["accepted"], ref["committed"], ref["next"])
+    if temperature:
+        assert fused.draw_step == ref["draw_step"]
+
+
+def test_qwen3_30b_a3b_all_48_layers_size_independent_properties():
+    """Configuration 4 at its real depth, context and vocabulary (48 layers, 8192 tokens, 151 936 rows,
+    chain k = 8, greedy), where the oracle cannot follow."""
+    ctx = 8192
+    cfg, gpu = _cycled("qwen3_30b_a3b", ctx, 6)
+    _size_independent_properties(cfg, gpu, ctx, 9, {}, 0.0)
+
+
+def test_gptoss_120b_all_36_layers_size_independent_properties():
+    """Configuration 5 at its real depth, context and vocabulary (36 layers alternating a 128-token
+    window with full attention, 32 768 tokens, 201 088 rows, 128 experts top-4 resident, chain k = 8,
+    rejection sampling at T = 1.0)."""
+    ctx = 32768
+    cfg, gpu = _cycled("gptoss_120b", ctx, 4)
+    _size_independent_properties(cfg, gpu, ctx, 9, {}, 1.0)

@@ -123,6 +123,18 @@ def test_refusals_by_name():
     with pytest.raises(TsvError, match="parent"):
         gpu.verify_tree([1, 2], [-1, 1], 16)
     assert gpu.position == 16
+    # a rollback retires the pass: its logits must not be judged at a position behind the cursor's past
+    import turbospark_amd as ts
+    gpu.rollback(ts.ffi.Point(8))
+    with pytest.raises(TsvError, match="last verify pass"):
+        gpu.accept(list(range(16)), 0, ts.shaping(0.0))
+    assert gpu.position == 8
+    point = gpu.checkpoint()
+    gpu.verify([1, 2, 3], 8, want_logits=False)
+    gpu.rollback_retaining(point, 1)
+    with pytest.raises(TsvError, match="last verify pass"):
+        gpu.accept([1, 2, 3], 8, ts.shaping(0.0))
+    assert gpu.position == 9
 
 
 def test_graph_replay_of_the_pass_equals_plain_launches():

@@ -123,6 +123,23 @@ def test_tensor_views_are_checked_against_the_file(tmp_path):
     g.close()
 
 
+def test_dimensions_that_would_wrap_the_byte_count_are_refused(tmp_path):
+    """A hostile tensor table: bf16 with a first dimension of 2^61 and four rows makes rows * row_bytes
+    wrap to zero in 64 bits, which would pass an end-of-file check done after the multiplication."""
+    path = os.path.join(tmp_path, "wrap.gguf")
+    write_gguf(path, META, [("wrap.weight", [1 << 61, 4], ffi.BF16, b"\0" * 64),
+                            ("tall.weight", [64, 1 << 39], ffi.BF16, b"\0" * 64),
+                            ("ok.weight", [64, 2], ffi.BF16, b"\1" * 256)])
+    g = ffi.Gguf(path)
+    with pytest.raises(ffi.TsvError, match="first dimension outside"):
+        g.tensor("wrap.weight")
+    with pytest.raises(ffi.TsvError, match="runs past the end"):
+        g.tensor("tall.weight")
+    dt, raw, rows, cols = g.tensor("ok.weight")
+    assert (dt, rows, cols) == (ffi.BF16, 2, 64)
+    g.close()
+
+
 def test_the_writers_permutation_is_the_converters():
     # conventions.rs:133-143: GGUF row j of a head holds the original row (j % 2) * (D/2) + j // 2,
     # so the original row i is found at GGUF row (i % (D/2)) * 2 + i // (D/2)

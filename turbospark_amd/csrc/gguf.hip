@@ -9,6 +9,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <climits>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -220,14 +221,21 @@ int tensor_view(const tsv_gguf& g, const std::string& name, tsv_tensor* out) {
         }
         rows *= t.dims[d];
     }
+    // a row longer than any matmul's K cannot be a real tensor; past 2^31 the element count would
+    // also wrap the signed arithmetic of the row-size helper
+    if (t.dims[0] == 0 || t.dims[0] > (uint64_t)INT32_MAX) {
+        set_error("gguf: tensor '" + name + "': first dimension outside 1..2^31-1");
+        return TSV_ERR_INVALID;
+    }
     const int64_t rb = tsv_row_bytes((int32_t)t.type, (int64_t)t.dims[0]);
     if (rb <= 0) {
         set_error("gguf: tensor '" + name + "': ggml type " + std::to_string(t.type) + " with rows of " +
                   std::to_string((unsigned long long)t.dims[0]) + " has no kernel here");
         return TSV_ERR_UNSUPPORTED;
     }
-    const uint64_t begin = g.data_start + t.offset, bytes = rows * (uint64_t)rb;
-    if (begin > g.size || bytes > g.size - begin) {
+    // no product before the bound is known: rows * rb must fit what is left of the file
+    const uint64_t begin = g.data_start + t.offset;
+    if (begin < g.data_start || begin > g.size || rows > (g.size - begin) / (uint64_t)rb) {
         set_error("gguf: tensor '" + name + "' runs past the end of the file");
         return TSV_ERR_INVALID;
     }

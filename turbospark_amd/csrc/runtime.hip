@@ -1136,6 +1136,7 @@ extern "C" int32_t tsv_rollback(tsv_ctx* c, const tsv_point* p) {
         return TSV_ERR_INVALID;
     }
     c->position = p->position;
+    c->last_m = 0;  // the logits on the device no longer describe rows behind the cursor
     c->prefix.rewind_to(p->position);  // real_forward_rollback.rs:203
     return TSV_OK;
 }
@@ -1147,6 +1148,7 @@ extern "C" int32_t tsv_rollback_retaining(tsv_ctx* c, const tsv_point* p, int32_
         return TSV_ERR_INVALID;
     }
     c->position = p->position + keep_rows;
+    c->last_m = 0;
     c->prefix.rewind_to(c->position);  // real_forward_rollback.rs:406
     return TSV_OK;
 }
@@ -1226,6 +1228,7 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
         return TSV_ERR_INVALID;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
+    if (int frc = check_fused(c)) return frc;  // rows a fused kernel gave up on must not be gathered
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
     return launch_kv_gather(c->stream, c->kv_ptrs, c->n_layers, c->nkv, c->hd, c->ctx_alloc, c->tok_dev + 32, n, (int)base);
