@@ -265,6 +265,16 @@ def test_qwen3_30b_a3b_shape_two_layers_at_long_context():
         kc, vc = cpu.kv(layer)
         assert np.abs(kg.astype(np.float32) - kc[ctx:ctx + 9]).max() <= 2e-2 * np.abs(kc[ctx:ctx + 9]).max()
         assert np.abs(vg.astype(np.float32) - vc[ctx:ctx + 9]).max() <= 2e-2 * np.abs(vc[ctx:ctx + 9]).max()
+    # the same rows fed one at a time (families/qwen/batched.rs:92-110: verify == sequential decode): the
+    # attention chunks differ with the row count at eight q heads per KV head, so to tolerance
+    point = ts.ffi.Point(ctx)
+    gpu.rollback(point)
+    seq = np.stack([gpu.produce(int(t), ctx + i) for i, t in enumerate(feed)])
+    err = gc.logit_error(seq, got)
+    print(f"  batched vs one row at a time: max-abs / range = {err:.2e}")
+    assert err <= 2e-3
+    gpu.rollback(point)
+    assert np.array_equal(gpu.verify(feed, ctx), got)
     # the greedy round on the device: integers equal to the oracle's walk over the same fp16 logits ...
     res = gpu.accept(feed, ctx, ts.shaping(0.0))
     ref = ob.chain_round(got, None, feed[1:], ob.shaping(0.0))
@@ -298,9 +308,7 @@ def _cycled(name, ctx, distinct, seed=3):
 
 def _size_independent_properties(cfg, gpu, ctx, m, shaping_kw, temperature):
     """Deterministic by bits; a rollback leaves nothing behind; a chain-shaped tree is the chain by bits;
-    the fused round equals verify followed by accept and the oracle's walk over the same logits; rows
-    fed one at a time agree with the batched pass (by tolerance where the attention splits differ with
-    the row count, see families/qwen/batched.rs:92-110 for the contract)."""
+    the fused round equals verify followed by accept and the oracle's walk over the same logits."""
     import turbospark_amd as ts
     V = cfg["vocab"]
     rng = np.random.default_rng(5)
@@ -314,10 +322,17 @@ def _size_independent_properties(cfg, gpu, ctx, m, shaping_kw, temperature):
     t = gpu.verify_tree(feed, list(range(-1, m - 1)), ctx)
     assert np.array_equal(a, t)
     gpu.rollback(point)
+    # Rows fed one at a time: with eight q heads per KV head a nine-row pass splits the context into other
+    # attention chunks than a one-row pass does, so the two agree to rounding per layer, not by bits --
+    # and through 36-48 random-init routed layers one router decision that sits within that rounding of
+    # a tie sends a row to another expert, after which its logits have little in common.  The
+    # comparison that means something is therefore made where the routing is known to be clear of ties
+    # (the two-layer cases at the same geometry, against the oracle); here only row 0 of the next token
+    # is checked to come out finite and the figure is printed.
     seq = np.stack([gpu.produce(int(tok), ctx + i) for i, tok in enumerate(feed)])
     err = gc.logit_error(seq, a)
     print(f"{cfg['n_layers']} layers, ctx {ctx}, m={m}: batched vs one row at a time, max-abs / range = {err:.2e}")
-    assert err <= 2e-3
+    assert np.isfinite(gc.f16(seq)).all()
     gpu.rollback(point)
     draft = rng.standard_normal((m - 1, V)).astype(np.float16) if temperature else None
     gs = ts.shaping(temperature, seed=11 if temperature else None, **shaping_kw)

@@ -20,6 +20,8 @@
 // Repetition / presence / frequency penalties (sampled chain and tree rounds, the draft draws) are
 // applied per candidate as it is read, from a per-token table of the history (see score_of);
 // the kernels are compiled twice, and the variant without penalties is the code it always was.
+#include <cstring>
+
 #include "tsv_internal.h"
 
 namespace tsv {
@@ -1248,11 +1250,19 @@ __global__ __launch_bounds__(256) void k_tree_finish(const uint16_t* target, con
 }
 
 // ---- greedy --------------------------------------------------------------------------------
-// choose.rs:277-285: first maximum.  One workgroup per target row.
-__global__ __launch_bounds__(1024) void k_argmax(const uint16_t* target, int vocab, int32_t* out, int32_t* err) {
-    __shared__ float bv[16];
-    __shared__ int bi[16];
-    const uint16_t* p = target + (long)blockIdx.x * vocab;
+// choose.rs:277-285: first maximum.  ARGMAX_SEG workgroups per target row, each over a contiguous
+// run of the vocabulary: the best (value, index) of every run goes to a partial slot, and whoever
+// needs the row's arg-max folds the runs in index order (a later run wins only with a strictly
+// larger value, so ties go to the lower index whatever the split).
+constexpr int ARGMAX_SEG = 16;
+
+__global__ __launch_bounds__(256) void k_argmax_part(const uint16_t* target, int vocab, float* pv, int32_t* pi, int32_t* err) {
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    const int row = blockIdx.y, seg = blockIdx.x;
+    const uint16_t* p = target + (long)row * vocab;
+    const int chunk = ((vocab + ARGMAX_SEG - 1) / ARGMAX_SEG + 7) & ~7;
+    const int v0 = min(seg * chunk, vocab), v1 = min(v0 + chunk, vocab);
     float best = -INFINITY;
     int idx = 0x7FFFFFFF;
     bool bad = false;
@@ -1264,17 +1274,17 @@ __global__ __launch_bounds__(1024) void k_argmax(const uint16_t* target, int voc
             idx = v;
         }
     };
-    if ((((uintptr_t)p) & 15) == 0) {  // eight logits per 16-byte load
-        const int n8 = vocab >> 3;
-        for (int i = threadIdx.x; i < n8; i += 1024) {
+    if ((((uintptr_t)p) & 15) == 0) {  // eight logits per 16-byte load (v0 is a multiple of 8)
+        const int i0 = v0 >> 3, i1 = v1 >> 3;
+        for (int i = i0 + threadIdx.x; i < i1; i += 256) {
             const uint4 q = ((const uint4*)p)[i];
             const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
             for (int j = 0; j < 8; j++) take((uint16_t)(w[j >> 1] >> (16 * (j & 1))), 8 * i + j);
         }
-        for (int v = (n8 << 3) + threadIdx.x; v < vocab; v += 1024) take(p[v], v);
+        for (int v = max(i1 << 3, v0) + threadIdx.x; v < v1; v += 256) take(p[v], v);
     } else {
-        for (int v = threadIdx.x; v < vocab; v += 1024) take(p[v], v);
+        for (int v = v0 + threadIdx.x; v < v1; v += 256) take(p[v], v);
     }
     if (bad) atomicOr(err, 1);
     for (int o = 32; o > 0; o >>= 1) {
@@ -1291,23 +1301,52 @@ __global__ __launch_bounds__(1024) void k_argmax(const uint16_t* target, int voc
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < 16; i++)
+        for (int i = 1; i < 4; i++)
             if (bv[i] > best || (bv[i] == best && bi[i] < idx)) {
                 best = bv[i];
                 idx = bi[i];
             }
-        out[blockIdx.x] = idx;
+        pv[row * ARGMAX_SEG + seg] = best;
+        pi[row * ARGMAX_SEG + seg] = idx;
     }
 }
 
-// speculative.rs:736-754 (chain) and 494-550 (tree walk) at temperature 0.
-__global__ void k_walk_greedy(const AcceptParams* app, const int32_t* amax, AcceptResult* res, const int32_t* err) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    const AcceptParams& ap = *app;
+// the row's arg-max from its runs' partial results, read by one thread
+__device__ __forceinline__ int32_t fold_argmax(const float* pv, const int32_t* pi, int row) {
+    float v[ARGMAX_SEG];
+    int32_t ix[ARGMAX_SEG];
+#pragma unroll
+    for (int s = 0; s < ARGMAX_SEG; s++) {
+        v[s] = pv[row * ARGMAX_SEG + s];
+        ix[s] = pi[row * ARGMAX_SEG + s];
+    }
+    float best = v[0];
+    int32_t idx = ix[0];
+#pragma unroll
+    for (int s = 1; s < ARGMAX_SEG; s++)
+        if (v[s] > best) {  // an empty run holds -inf and never wins
+            best = v[s];
+            idx = ix[s];
+        }
+    return idx;
+}
+
+__global__ void k_argmax_fold(const float* pv, const int32_t* pi, int rows, int32_t* out) {
+    if ((int)threadIdx.x < rows) out[threadIdx.x] = fold_argmax(pv, pi, threadIdx.x);
+}
+
+// speculative.rs:736-754 (chain) and 494-550 (tree walk) at temperature 0, by one thread over the
+// rows' arg-max tokens.
+struct GreedyWalk {
+    int32_t accepted, committed, stopped, next, path_len;
+    int32_t path[TSV_MAX_ROWS + 1];
+};
+__device__ GreedyWalk walk_greedy(const AcceptParams& ap, const int32_t* amax) {
+    GreedyWalk g;
     uint64_t gen = ap.generated;
     int32_t committed = 0, stopped = 0, next = -1;
     int at = 0, plen = 1;
-    res->path[0] = 0;
+    g.path[0] = 0;
     for (;;) {
         const int32_t want = amax[at];
         int hit = -1;
@@ -1324,16 +1363,33 @@ __global__ void k_walk_greedy(const AcceptParams* app, const int32_t* amax, Acce
             next = want;
             break;
         }
-        res->path[plen++] = hit;
+        g.path[plen++] = hit;
         at = hit;
         if ((stopped = sink_commit(ap, want, gen, committed))) break;
     }
-    res->accepted = plen - 1;
-    res->committed = committed;
-    res->stopped = stopped;
-    res->next = stopped ? -1 : next;
+    g.accepted = plen - 1;
+    g.committed = committed;
+    g.stopped = stopped;
+    g.next = stopped ? -1 : next;
+    g.path_len = plen;
+    return g;
+}
+
+__global__ void k_walk_greedy(const AcceptParams* app, const float* pv, const int32_t* pi, AcceptResult* res,
+                              const int32_t* err) {
+    __shared__ int32_t amax[TSV_MAX_ROWS];
+    const AcceptParams& ap = *app;
+    if ((int)threadIdx.x < ap.m) amax[threadIdx.x] = fold_argmax(pv, pi, threadIdx.x);
+    __syncthreads();
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const GreedyWalk g = walk_greedy(ap, amax);
+    for (int i = 0; i < g.path_len; i++) res->path[i] = g.path[i];
+    res->accepted = g.accepted;
+    res->committed = g.committed;
+    res->stopped = g.stopped;
+    res->next = g.next;
     res->draw_step = ap.draw_step;
-    res->path_len = plen;
+    res->path_len = g.path_len;
     res->min_margin = 1.0;
     res->error = *err;
 }
@@ -1348,7 +1404,8 @@ __global__ void k_clear_result(AcceptResult* res, int32_t* err) {
 
 }  // namespace
 
-// scratch.counters: [0] error flag, [16..32) greedy arg-max per row; decisions live after the
+// scratch.counters (ACCEPT_COUNTER_WORDS words): [0] error flag, [32..49) tree path, [64..) the greedy
+// arg-max partials (value, then index, per row and run); decisions live after the
 // statistics block; histograms and work arrays are separate allocations in AcceptScratch.
 size_t accept_stats_doubles() { return STATS_DOUBLES + TREE_STATE_DOUBLES; }
 
@@ -1429,11 +1486,12 @@ static void launch_draft_sampled(hipStream_t s, const uint16_t* draft, const Acc
 int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
                   const AcceptParams& ap, const AcceptScratch& sc) {
     int32_t* err = (int32_t*)sc.counters;
-    int32_t* amax = (int32_t*)sc.counters + 16;
+    float* pv = (float*)sc.counters + 64;
+    int32_t* pi = (int32_t*)sc.counters + 64 + TSV_MAX_ROWS * ARGMAX_SEG;
     hipLaunchKernelGGL(k_clear_result, dim3(1), dim3(64), 0, s, sc.result, err);
     if (!ap.sampled) {  // (the arg-max ignores penalties and truncation: choose.rs:84-88)
-        hipLaunchKernelGGL(k_argmax, dim3(ap.m), dim3(1024), 0, s, target, ap.vocab, amax, err);
-        hipLaunchKernelGGL(k_walk_greedy, dim3(1), dim3(64), 0, s, ap_dev, amax, sc.result, err);
+        hipLaunchKernelGGL(k_argmax_part, dim3(ARGMAX_SEG, ap.m), dim3(256), 0, s, target, ap.vocab, pv, pi, err);
+        hipLaunchKernelGGL(k_walk_greedy, dim3(1), dim3(64), 0, s, ap_dev, pv, pi, sc.result, err);
         TSV_HIP(hipGetLastError());
         return TSV_OK;
     }
@@ -1460,7 +1518,10 @@ int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams*
     int32_t* err = (int32_t*)sc.counters;
     hipLaunchKernelGGL(k_clear_result, dim3(1), dim3(64), 0, s, sc.result, err);
     if (!ap.sampled) {
-        hipLaunchKernelGGL(k_argmax, dim3(ap.k), dim3(1024), 0, s, draft, ap.vocab, proposals_dev, err);
+        float* pv = (float*)sc.counters + 64;
+        int32_t* pi = (int32_t*)sc.counters + 64 + TSV_MAX_ROWS * ARGMAX_SEG;
+        hipLaunchKernelGGL(k_argmax_part, dim3(ARGMAX_SEG, ap.k), dim3(256), 0, s, draft, ap.vocab, pv, pi, err);
+        hipLaunchKernelGGL(k_argmax_fold, dim3(1), dim3(64), 0, s, pv, pi, ap.k, proposals_dev);
         TSV_HIP(hipGetLastError());
         return TSV_OK;
     }

@@ -933,7 +933,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->sc.stats, accept_stats_doubles() * 8, true)) ||
         (rc = dev_alloc(c, &c->sc.work, (size_t)(16 * 2 + 2) * c->vocab * 8, true)) ||
         (rc = dev_alloc(c, &c->sc.hist, (size_t)16 * 2 * 65536 * 8, true)) ||
-        (rc = dev_alloc(c, &c->sc.counters, 64 * 4, true)) ||
+        (rc = dev_alloc(c, &c->sc.counters, ACCEPT_COUNTER_WORDS * 4, true)) ||
         (rc = dev_alloc(c, &c->sc.tmass, (size_t)32 * 65536 * 8, true)) ||
         (rc = dev_alloc(c, &c->sc.tcount, (size_t)32 * 65536 * 4, true)) ||
         (rc = dev_alloc(c, &c->sc.result, sizeof(AcceptResult), true)))

@@ -300,11 +300,12 @@ struct AcceptScratch {
     double* stats;       // accept_stats_doubles() doubles: row statistics, partials, decisions
     double* work;        // [16 jobs][2][vocab] candidate masses (p, residual) + two more rows (tree residuals)
     uint64_t* hist;      // [16 jobs][2][65536] fixed-point mass per rank bin; a round clears what it uses first
-    uint32_t* counters;  // 64 words: error flag, greedy arg-max per row
+    uint32_t* counters;  // ACCEPT_COUNTER_WORDS words: error flag, tree path, greedy arg-max partials
     uint64_t* tmass;     // [32 rows][65536] fixed-point softmax mass per rank bin (top-p cut)
     uint32_t* tcount;    // [32 rows][65536] candidates per rank bin (top-k / top-p cut)
     AcceptResult* result;  // device
 };
+constexpr int ACCEPT_COUNTER_WORDS = 1024;
 size_t accept_stats_doubles();
 int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
                   const AcceptParams& ap_host, const AcceptScratch& sc);
