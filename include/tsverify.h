@@ -241,6 +241,20 @@ int32_t tsv_compact_tree(tsv_ctx* ctx, int64_t base, const uint32_t* path, int32
 int32_t tsv_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result* out);
 /* verify + accept + truncate in one call: the whole verify step. */
 int32_t tsv_verify_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result* out);
+/* The greedy round of tsv_accept for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Nothing
+ * is allocated, copied from the host or waited for: the logits (m x vocab fp16) and the result are
+ * DEVICE memory of the caller's, `stream` is the caller's hipStream_t (NULL: the default stream),
+ * and the arg-max partial results live in a 4 KiB static device array that every GPU the library
+ * runs on holds until the process ends.  Limits: 1..TSV_MAX_ROWS rows (more is refused by name),
+ * at most 16 stop tokens.  There is no handle, so no KV truncation: result->kv_position = base +
+ * committed + 1 is where the caller moves its cursor.  A non-finite logit is reported in band
+ * (stopped = -1, next = -1, path_len = 0).  Calls on one GPU share that GPU's array: two calls that
+ * overlap in time on one GPU race. */
+int32_t tsv_accept_greedy_noalloc(void* stream, const uint16_t* logits_dev, int32_t vocab, const int32_t* feed,
+                                  const int32_t* parent, int32_t m, int64_t base, const int32_t* stop_tokens,
+                                  int32_t n_stop, uint64_t generated, uint64_t max_new_tokens,
+                                  tsv_round_result* result_dev);
 /* Draft half of a sampled chain round (speculative.rs:606-660): draws k proposals, one
  * from each row of draft_logits (k x vocab fp16, host or device), advancing *draw_step by
  * k + 1; greedy: argmax per row. */

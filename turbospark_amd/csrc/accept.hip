@@ -1562,3 +1562,133 @@ int launch_pen_counts(hipStream_t s, const int32_t* history_dev, long n, long su
 }
 
 }  // namespace tsv
+
+// ---- greedy acceptance for callers that cannot allocate ----------------------------------------
+// The greedy round of tsv_accept (arg-max per row, the walk, the stop ladder and budget) over logits
+// the caller holds on the device, writing the result to device memory of the caller's, on the
+// caller's stream, with no handle behind it: nothing is allocated, copied from the host or waited
+// for.  The partial results of the arg-max (one value / index pair per row and vocabulary run) and
+// the error flag live in a static device array; every GPU the library runs on holds its own copy
+// until the process ends, and every call on a GPU shares that GPU's copy, so two calls that overlap
+// on one GPU race.
+static __device__ __align__(256) unsigned char scratch[4096];
+
+namespace tsv {
+namespace {
+
+struct NoAllocScratch {
+    int32_t err;
+    int32_t pad[63];
+    float pv[TSV_MAX_ROWS * ARGMAX_SEG];
+    int32_t pi[TSV_MAX_ROWS * ARGMAX_SEG];
+};
+static_assert(sizeof(NoAllocScratch) <= sizeof(scratch), "the static array holds the greedy round's partial results");
+
+// the flag must start at zero; a fill kernel rather than a memset node, so a caller may capture the call
+__global__ void k_noalloc_clear(int32_t* err) {
+    if (threadIdx.x == 0) *err = 0;
+}
+
+__global__ void k_walk_greedy_value(AcceptParams ap, int64_t base, const float* pv, const int32_t* pi, const int32_t* err,
+                                    tsv_round_result* out) {
+    __shared__ int32_t amax[TSV_MAX_ROWS];
+    if ((int)threadIdx.x < ap.m) amax[threadIdx.x] = fold_argmax(pv, pi, threadIdx.x);
+    __syncthreads();
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    for (int i = 0; i <= TSV_MAX_ROWS; i++) out->path[i] = 0;
+    if (*err) {  // a non-finite logit (choose.rs:122-132 refuses the row): no round was judged
+        out->accepted = out->committed = 0;
+        out->next = -1;
+        out->stopped = -1;
+        out->draw_step = ap.draw_step;
+        out->path_len = 0;
+        out->kv_position = base;
+        out->min_margin = 0.0;
+        return;
+    }
+    const GreedyWalk g = walk_greedy(ap, amax);
+    for (int i = 0; i < g.path_len; i++) out->path[i] = g.path[i];
+    out->accepted = g.accepted;
+    out->committed = g.committed;
+    out->next = g.next;
+    out->stopped = g.stopped;
+    out->draw_step = ap.draw_step;
+    out->path_len = g.path_len;
+    out->kv_position = base + g.committed + 1;
+    out->min_margin = 1.0;
+}
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+// device address of `scratch` on each GPU (the array's name is only a host-side handle of the symbol)
+NoAllocScratch* g_noalloc_scratch[NOALLOC_MAX_DEVICES];
+
+int noalloc_scratch(NoAllocScratch** out) {
+    int dev = -1;
+    TSV_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) {
+        set_error("accept_greedy_noalloc: device ordinal outside 0..63");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    NoAllocScratch* p = __atomic_load_n(&g_noalloc_scratch[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        void* sym = nullptr;
+        TSV_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)));
+        if (!sym) {
+            set_error("accept_greedy_noalloc: the scratch symbol has no device address");
+            return TSV_ERR_DEVICE;
+        }
+        p = (NoAllocScratch*)sym;
+        __atomic_store_n(&g_noalloc_scratch[dev], p, __ATOMIC_RELEASE);
+    }
+    *out = p;
+    return TSV_OK;
+}
+
+}  // namespace
+}  // namespace tsv
+
+extern "C" int32_t tsv_accept_greedy_noalloc(void* stream, const uint16_t* logits_dev, int32_t vocab, const int32_t* feed,
+                                             const int32_t* parent, int32_t m, int64_t base, const int32_t* stop_tokens,
+                                             int32_t n_stop, uint64_t generated, uint64_t max_new_tokens,
+                                             tsv_round_result* result_dev) {
+    using namespace tsv;
+    if (!logits_dev || !feed || !result_dev || (n_stop > 0 && !stop_tokens)) {
+        set_error("accept_greedy_noalloc: null argument");
+        return TSV_ERR_INVALID;
+    }
+    if (m < 1 || m > TSV_MAX_ROWS) {
+        set_error("accept_greedy_noalloc: 1..16 rows (the static scratch holds the partial results of 16 rows)");
+        return TSV_ERR_INVALID;
+    }
+    if (vocab < 1 || base < 0 || n_stop < 0 || n_stop > 16) {
+        set_error("accept_greedy_noalloc: vocabulary and base must be positive / non-negative, at most 16 stop tokens");
+        return TSV_ERR_INVALID;
+    }
+    AcceptParams ap;
+    std::memset(&ap, 0, sizeof ap);
+    ap.m = m;
+    ap.k = m - 1;
+    ap.vocab = vocab;
+    ap.tree = parent != nullptr;
+    ap.n_stop = n_stop;
+    for (int i = 0; i < m; i++) {
+        if (parent && (i == 0 ? parent[0] != -1 : (parent[i] < 0 || parent[i] >= i))) {
+            set_error("accept_greedy_noalloc: parent[0] must be -1 and parent[s] in [0, s)");
+            return TSV_ERR_INVALID;
+        }
+        ap.feed[i] = feed[i];
+        ap.parent[i] = parent ? parent[i] : i - 1;
+    }
+    for (int i = 0; i < n_stop; i++) ap.stop_tokens[i] = stop_tokens[i];
+    ap.generated = generated;
+    ap.max_new_tokens = max_new_tokens;
+    NoAllocScratch* sc = nullptr;
+    int rc = noalloc_scratch(&sc);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_noalloc_clear, dim3(1), dim3(64), 0, s, &sc->err);
+    hipLaunchKernelGGL(k_argmax_part, dim3(ARGMAX_SEG, m), dim3(256), 0, s, logits_dev, vocab, sc->pv, sc->pi, &sc->err);
+    hipLaunchKernelGGL(k_walk_greedy_value, dim3(1), dim3(64), 0, s, ap, base, sc->pv, sc->pi, &sc->err, result_dev);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}

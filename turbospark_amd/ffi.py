@@ -234,7 +234,7 @@ EXPORTS = [
     "tsv_open", "tsv_close", "tsv_last_error", "tsv_stream", "tsv_reset", "tsv_kv_position", "tsv_max_safe_rewind", "tsv_device_logits",
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
-    "tsv_accept", "tsv_verify_accept", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
+    "tsv_accept", "tsv_verify_accept", "tsv_accept_greedy_noalloc", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
     "tsv_synth_tensor", "tsv_read_kv", "tsv_write_kv", "tsv_write_logits", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
     "tsv_yarn_frequencies", "tsv_adaptive_init", "tsv_adaptive_depth", "tsv_adaptive_observe", "tsv_adaptive_tile_cap",
     "tsv_run_speculative", "tsv_max_context", "tsv_vocab",
@@ -292,6 +292,8 @@ def lib():
         L.tsv_verify_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
         L.tsv_compact_tree.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int32]
         L.tsv_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
+        L.tsv_accept_greedy_noalloc.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32,
+                                                C.c_int64, C.c_void_p, C.c_int32, C.c_uint64, C.c_uint64, C.c_void_p]
         L.tsv_verify_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
         L.tsv_draft_chain.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(Shaping),
                                       C.POINTER(C.c_uint64), C.c_void_p, C.c_void_p, C.c_int64, C.c_uint64]
