@@ -42,9 +42,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def algorithmic_bytes(cfg, ctx, m):
+def algorithmic_bytes(cfg, ctx, m, union=None):
     """Bytes one verify step has to move: every quantized weight once, the KV rows [0, ctx+m)
-    once per layer, m embedding rows, m x vocab fp16 logits, m new KV rows."""
+    once per layer, m embedding rows, m x vocab fp16 logits, m new KV rows.  Routed experts: an
+    expert's matrices count once per layer in which any row chose it; `union` is the mean number of
+    distinct experts per layer actually routed (read back from the device), None the expectation
+    under independent uniform routing."""
     from turbospark_amd import ffi
     H, F, V, L = cfg["hidden"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
     qd, kvd = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
@@ -53,8 +56,9 @@ def algorithmic_bytes(cfg, ctx, m):
     if E:
         # routed experts: an expert's matrices are read once if any of the m rows chose it; with
         # independent uniform routing the expected number of distinct experts per layer is
-        # E * (1 - (1 - k/E)^m)  (the union actually routed is not read back)
-        union = E * (1.0 - (1.0 - cfg["top_k"] / E) ** m)
+        # E * (1 - (1 - k/E)^m)
+        if union is None:
+            union = E * (1.0 - (1.0 - cfg["top_k"] / E) ** m)
         xd = cfg.get("expert_dtype", cfg["dtype"])
         per_layer = dict(qkv=rb(qd + 2 * kvd, H), wo=rb(H, qd), gate_up=int(union * rb(2 * F, H, xd)) + rb(E, H),
                          down=int(union * rb(H, F, xd)))
@@ -98,11 +102,14 @@ def trace_summary(path):
     print(f"total kernel time in verify steps: {total / 1e6:.3f} ms over the traced steps")
 
 
-# HBM bytes per launch of the dominant kernel (gate/up matmul of the headline workload), measured
-# with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over `bench.py --traffic-probe` and
-# scaled by the copy kernel of known size (`bench.py --traffic-summary`): 66 793 486 B read +
-# 258 048 B written, against 66 060 288 algorithmic bytes.
-MEASURED_TRAFFIC = {"llama3_8b_q4_k_k4_ctx4096": 67051534}
+# Figures RECORDED from committed counter / trace runs (a bench run does not collect counters): HBM
+# bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# over `bench.py --traffic-probe`, scaled by the copy kernel of known size (`bench.py
+# --traffic-summary`): 66 793 486 B read + 258 048 B written against 66 060 288 algorithmic bytes;
+# and the same kernel's average duration in the committed rocprofv3 kernel trace of this script.
+RECORDED = {"llama3_8b_q4_k_k4_ctx4096": dict(
+    traffic=67051534, traffic_source="recorded: profiles/gate_up_matmul_llama3_8b_q4k_hbm_traffic.txt",
+    trace_avg_us=16.13, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt")}
 
 GATE_UP_8B = dict(dtype=12, rows=28672, cols=4096, m=5, epi=1)   # the dominant kernel of the headline workload
 COPY_BYTES = 256 << 20
@@ -309,7 +316,17 @@ def main():
 
     nrep = min(10, args.steps)
     plain_ms = timed_region(nrep)
-    ab = algorithmic_bytes(cfg, ctx, m)
+    # routed experts: the experts the timed steps actually chose, read back from the device in a pass
+    # of their own (the same feeds route the same way: the pass is deterministic)
+    union = None
+    if cfg.get("n_experts"):
+        per_step = []
+        for i in range(min(args.steps, 20)):
+            step(args.warmup + i)
+            sel = eng.route_selected()[:, :m, :cfg["top_k"]]
+            per_step.append(np.mean([len(np.unique(sel[l])) for l in range(sel.shape[0])]))
+        union = float(np.mean(per_step))
+    ab = algorithmic_bytes(cfg, ctx, m, union)
     L = cfg["n_layers"]
     kern = {}
     for name, nbytes, count in (("qkv", ab["per_layer"]["qkv"], L), ("wo", ab["per_layer"]["wo"], L),
@@ -336,12 +353,20 @@ def main():
         kern["qkv"]["epilogue"] = "bias + rotation + fp16 q / KV-cache stores"
     dom = kern.get("gate_up", {})
     peak = 8000.0
+    rec = RECORDED.get(args.workload, {})
     roofline = dict(bound="hbm",
-                    kernel="router + grouped expert gate/up matmuls (expected expert union)" if cfg.get("n_experts")
+                    kernel=f"router + grouped expert gate/up matmuls (experts actually routed: {union:.1f} of {cfg['n_experts']} per layer)"
+                    if cfg.get("n_experts")
                     else "k_gemm<Q4_K> gate/up (silu-mul epilogue)" if cfg["dtype"] == 12 else "k_gemm<Q8_0> gate/up",
                     achieved=dom.get("GBps"), peak=peak, unit="GB/s",
                     frac=round((dom.get("GBps") or 0.0) / peak, 4),
-                    traffic=MEASURED_TRAFFIC.get(args.workload),
+                    timing="live: HIP events on the engine's stream around timed regions, the region with this kernel class "
+                           "launched twice minus the plain region, per launch",
+                    traffic=rec.get("traffic"), traffic_source=rec.get("traffic_source", "not measured for this workload"),
+                    # the same kernel in the committed rocprofv3 kernel trace (begin-to-end of the dispatch, which
+                    # includes what overlaps with its neighbours in the pipeline): the lower of the two fractions
+                    trace_avg_launch_us=rec.get("trace_avg_us"), trace_source=rec.get("trace_source"),
+                    trace_frac=round(dom["bytes"] / (rec["trace_avg_us"] * 1e-6) / 1e9 / peak, 4) if rec.get("trace_avg_us") and dom.get("bytes") else None,
                     algorithmic_bytes_per_launch=dom.get("bytes"), avg_launch_us=dom.get("avg_us"),
                     all_matmuls_GBps=round(ab["weights"] / (gemm_ms * 1e-3) / 1e9, 1) if gemm_ms else None,
                     step_algorithmic_bytes=int(ab["total"]),
@@ -365,7 +390,8 @@ def main():
                         "f32 accumulate; f64 acceptance",
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,
-                   "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin},
+                   "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin,
+                   **({"experts_routed_per_layer": round(union, 2)} if union is not None else {})},
         "roofline": roofline, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

@@ -72,7 +72,11 @@ typedef struct {
      * bf16 vectors.  window > 0: a row sees only the last `window` positions of its sequence
      * (gptoss/attn.rs:120-137); it must exceed TSV_MAX_ROWS. */
     tsv_tensor bq, bk, bv, bo, sinks, router_bias, be_gate, be_up, be_down;
-    int32_t window, reserved;
+    /* ring != 0 (window > 0 only): the layer keeps a ring of window + 2 * TSV_MAX_ROWS positions
+     * (rounded to 16) instead of the whole context, position p in slot p % capacity -- the
+     * reference's fp16 ring for sliding-window layers (crates/gpu/src/kv_cache.rs:122-131,360-378).
+     * Rollbacks are then bounded by tsv_max_safe_rewind. */
+    int32_t window, ring;
 } tsv_layer;
 
 typedef struct {
@@ -169,8 +173,10 @@ void* tsv_stream(tsv_ctx* ctx);
 int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset */
 int64_t tsv_kv_position(const tsv_ctx* ctx);   /* kv.position() */
 /* KvCacheManager::max_safe_rewind (crates/gpu/src/kv_cache_rewind.rs:26-35): how many rows a rollback
- * may drop.  INT64_MAX here: every layer, windowed ones included, stores position p at slot p, so
- * "nothing rings" and any rewind down to position 0 is safe. */
+ * may drop and still leave every ring layer's window intact: the smallest capacity - window over the
+ * layers opened with `ring`; INT64_MAX when nothing rings (every layer stores position p at slot p).
+ * tsv_rollback, tsv_rollback_retaining and tsv_try_reuse_prefix refuse by name (:46-55) a cursor that
+ * would land more than this many rows behind the last row ever written. */
 int64_t tsv_max_safe_rewind(const tsv_ctx* ctx);
 /* LogitProducer::produce: one token at `position`; logits: vocab fp16. */
 int32_t tsv_produce(tsv_ctx* ctx, int32_t token, int64_t position, uint16_t* logits);
@@ -369,63 +375,6 @@ int32_t tsv_quantize_rows(int32_t dtype, const float* src, int64_t rows, int64_t
  * crates/repack/src/synthetic_*.rs).  dst holds rows * tsv_row_bytes(dtype, cols) bytes. */
 int32_t tsv_synth_tensor(int32_t dtype, uint64_t seed, uint64_t stream, float sigma, int64_t rows,
                          int64_t cols, void* dst);
-
-/* ---- introspection for tests -------------------------------------------------- */
-/* Copies layer `layer`'s K and V rows [pos0, pos0+n) to host as fp16 in the reference
- * layout [position][kv_head][head_dim] (crates/gpu/src/kv_cache.rs:1-10). */
-int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v);
-/* The inverse: stores n rows of K and V (same host layout) at cache positions [pos0, pos0+n) of
- * one layer and moves the cursor to at least pos0 + n -- a long context without the prefill that
- * would build it (the full-size parity cases; also how a saved prefix would be restored). */
-int32_t tsv_write_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k, const uint16_t* v);
-/* Stores m x vocab fp16 logits (host memory) as if a verify pass of m rows at `base` had just left them on
- * the device: tsv_accept then judges exactly these scores (acceptance cases no model would produce: ties,
- * flat rows, the fp16 extremes).  The KV cache and the cursor are not touched. */
-int32_t tsv_write_logits(tsv_ctx* ctx, const uint16_t* logits, int32_t m, int64_t base);
-/* One quantized small-M matmul through the same kernels the forward uses:
- * y[m][r] = sum_k W[r][k] x[m][k]; x is m x cols fp32 (rounded to fp16 on entry), y is
- * m x rows fp32.  W host tensor in GGUF layout (re-tiled per call).  `splits` <= 0 picks
- * the engine's own split-K factor. */
-int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits);
-
-/* Per-kernel-class timing with HIP events on the handle's stream (one event pair per launch
- * while enabled).  Classes, in order: embed, norm, qkv matmul, rope+kv store, attention,
- * output projection, gate/up matmul, down matmul, output head, acceptance, and "event pair":
- * one pair per pass with nothing between the two events, i.e. what an event pair itself adds
- * to every other reading.  tsv_get_profile sums the elapsed milliseconds and launch counts
- * since the last call and clears them. */
-#define TSV_PROFILE_CLASSES 11
-int32_t tsv_set_profile(tsv_ctx* ctx, int32_t on);
-int32_t tsv_get_profile(tsv_ctx* ctx, float* ms, int32_t* counts, int32_t n_classes);
-
-/* Measurement hook (no reference counterpart): launch the kernels of one class `times` times
- * in a row in every following pass (1 restores normal operation).  The extra launches redo the
- * same work on the same buffers, so results do not change; timing a pass with and without the
- * repeat gives the class's in-pipeline duration without an event pair around every launch.
- * Classes that accumulate (norm, embed, acceptance) are refused. */
-int32_t tsv_set_repeat(tsv_ctx* ctx, int32_t profile_class, int32_t times);
-
-/* Measurement hook (no reference counterpart): average microseconds of `iters` back-to-back
- * launches of the verify matmul kernel on a rows x cols weight of `dtype` with m activation
- * rows; epi 0 = split-K partials, 1 = silu(gate)*up over interleaved tiles, 2 = fp16 logits;
- * `rotate` weight copies are cycled so the bytes come from HBM. */
-int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
-                        int32_t iters, int32_t rotate, float* avg_us);
-
-/* Measurement hook: average duration of `iters` launches of a plain device-to-device copy kernel
- * over `bytes` bytes (read once, written once).  It is the copy kernel of known size that HBM
- * traffic counters are scaled against, and the streaming rate the part actually reaches. */
-int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us);
-
-/* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
- * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache
- * slot base+i and sees [0, base) plus the slots of its root path (parent NULL: chain).
- * window > 0 keeps the last `window` positions of each row's sequence; sinks (nullable): one f32
- * logit per q head (crates/compute/src/attention.rs:29-137).
- * out: m x nq x hd fp16.  (The per-kernel parity hook of crates/gpu/tests/attention_tree_parity.rs.) */
-int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
-                      int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
-                      int32_t window, const float* sinks, uint16_t* out);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,83 @@
+/*
+ * tsverify_testing.h -- test and measurement hooks of libtsverify.so.
+ *
+ * Nothing here belongs to the drop-in surface (include/tsverify.h maps the reference's producer
+ * traits); these entry points exist for the parity tests and for bench.py: reading and writing the
+ * KV cache and the logits directly, single kernels in isolation, per-kernel timing, and the routing
+ * decisions of the last pass.  A host that embeds the library needs none of them.
+ */
+#ifndef TSVERIFY_TESTING_H
+#define TSVERIFY_TESTING_H
+
+#include "tsverify.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Copies layer `layer`'s K and V rows [pos0, pos0+n) to host as fp16 in the reference
+ * layout [position][kv_head][head_dim] (crates/gpu/src/kv_cache.rs:1-10). */
+int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v);
+/* The inverse: stores n rows of K and V (same host layout) at cache positions [pos0, pos0+n) of
+ * one layer and moves the cursor to at least pos0 + n -- a long context without the prefill that
+ * would build it (the full-size parity cases; also how a saved prefix would be restored). */
+int32_t tsv_write_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k, const uint16_t* v);
+/* Stores m x vocab fp16 logits (host memory) as if a verify pass of m rows at `base` had just left them on
+ * the device: tsv_accept then judges exactly these scores (acceptance cases no model would produce: ties,
+ * flat rows, the fp16 extremes).  The KV cache and the cursor are not touched. */
+int32_t tsv_write_logits(tsv_ctx* ctx, const uint16_t* logits, int32_t m, int64_t base);
+/* One quantized small-M matmul through the same kernels the forward uses:
+ * y[m][r] = sum_k W[r][k] x[m][k]; x is m x cols fp32 (rounded to fp16 on entry), y is
+ * m x rows fp32.  W host tensor in GGUF layout (re-tiled per call).  `splits` <= 0 picks
+ * the engine's own split-K factor. */
+int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits);
+
+/* Per-kernel-class timing with HIP events on the handle's stream (one event pair per launch
+ * while enabled).  Classes, in order: embed, norm, qkv matmul, rope+kv store, attention,
+ * output projection, gate/up matmul, down matmul, output head, acceptance, and "event pair":
+ * one pair per pass with nothing between the two events, i.e. what an event pair itself adds
+ * to every other reading.  tsv_get_profile sums the elapsed milliseconds and launch counts
+ * since the last call and clears them. */
+#define TSV_PROFILE_CLASSES 11
+int32_t tsv_set_profile(tsv_ctx* ctx, int32_t on);
+int32_t tsv_get_profile(tsv_ctx* ctx, float* ms, int32_t* counts, int32_t n_classes);
+
+/* Measurement hook (no reference counterpart): launch the kernels of one class `times` times
+ * in a row in every following pass (1 restores normal operation).  The extra launches redo the
+ * same work on the same buffers, so results do not change; timing a pass with and without the
+ * repeat gives the class's in-pipeline duration without an event pair around every launch.
+ * Classes that accumulate (norm, embed, acceptance) are refused. */
+int32_t tsv_set_repeat(tsv_ctx* ctx, int32_t profile_class, int32_t times);
+
+/* Measurement hook (no reference counterpart): average microseconds of `iters` back-to-back
+ * launches of the verify matmul kernel on a rows x cols weight of `dtype` with m activation
+ * rows; epi 0 = split-K partials, 1 = silu(gate)*up over interleaved tiles, 2 = fp16 logits;
+ * `rotate` weight copies are cycled so the bytes come from HBM. */
+int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
+                        int32_t iters, int32_t rotate, float* avg_us);
+
+/* Measurement hook: average duration of `iters` launches of a plain device-to-device copy kernel
+ * over `bytes` bytes (read once, written once).  It is the copy kernel of known size that HBM
+ * traffic counters are scaled against, and the streaming rate the part actually reaches. */
+int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us);
+
+/* One verify-pass attention through the same kernels the forward uses.  q: m x nq x hd,
+ * k, v: (base + m) x nkv x hd in the reference cache layout, all fp16; row i sits at cache
+ * slot base+i and sees [0, base) plus the slots of its root path (parent NULL: chain).
+ * window > 0 keeps the last `window` positions of each row's sequence; sinks (nullable): one f32
+ * logit per q head (crates/compute/src/attention.rs:29-137).
+ * out: m x nq x hd fp16.  (The per-kernel parity hook of crates/gpu/tests/attention_tree_parity.rs.) */
+int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
+                      int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
+                      int32_t window, const float* sinks, uint16_t* out);
+
+/* The experts every row of the last pass chose in every routed layer: out is [n_layers][16][8] expert
+ * ids in rank order (row r of the pass at [layer][r], the first top_k entries of a row are valid).
+ * What the bench counts the expert bytes actually read from, and what the routing tests compare with
+ * the oracle's ranking (real_forward_dispatch.rs:1135-1158). */
+int32_t tsv_route_selected(tsv_ctx* ctx, int32_t* out, int32_t n_layers);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -134,6 +134,8 @@ def lib():
         L.tso_model_create.restype = C.c_void_p
         L.tso_model_position.restype = C.c_int64
         L.tso_model_route_margin.restype = C.c_float
+        L.tso_model_route_record.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.tso_model_force_route.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
         L.tso_model_k.restype = C.POINTER(C.c_float)
         L.tso_model_v.restype = C.POINTER(C.c_float)
         L.tso_last_error.restype = C.c_char_p
@@ -480,6 +482,23 @@ class Model:
         """Smallest relative gap between the last chosen and the first rejected router logit
         over the last verify call (1.0 for a dense model)."""
         return float(lib().tso_model_route_margin(self._h))
+
+    def route_record(self):
+        """(selected [layers, 16, 8] expert ids in rank order, -1 past top_k; gap [layers, 16]) of the last verify."""
+        n = self.cfg["n_layers"]
+        sel = np.full((n, 16, 8), -1, np.int32)
+        gap = np.ones((n, 16), np.float32)
+        if lib().tso_model_route_record(self._h, _p(sel), _p(gap)) != 0:
+            raise ValueError("no routed layer has run")
+        return sel, gap
+
+    def force_route(self, sel=None):
+        """Test hook: take these experts ([layers, 16, 8]) instead of the top-k; None restores the ranking."""
+        if sel is None:
+            lib().tso_model_force_route(self._h, None, 0)
+        else:
+            a = np.ascontiguousarray(sel, np.int32)
+            lib().tso_model_force_route(self._h, _p(a), a.size)
 
     def rewind_to(self, position):
         lib().tso_model_rewind_to(self._h, C.c_int64(position))

@@ -29,6 +29,12 @@ struct tso_model {
     std::vector<std::vector<float>> k, v;  // per layer [max_context][nkv*hd]
     int64_t position = 0;
     float route_margin = 1.0f;
+    // the routing of the last verify call: [layer][row][8] expert ids in rank order (-1 past top_k) and
+    // [layer][row] the relative gap between the last chosen and the first rejected logit
+    std::vector<int32_t> route_sel;
+    std::vector<float> route_gap;
+    // test hook: expert ids to take instead of the top-k, same shape (empty: route normally)
+    std::vector<int32_t> forced_sel;
 };
 
 namespace {
@@ -66,22 +72,30 @@ tso_tensor row_slice(const tso_tensor& t, int64_t r0, int64_t n) {
 
 // real_forward_dispatch.rs:1135-1158 (`router_topk_gemma4`, per_expert_scale all ones): top-k by
 // logit, ties to the lower index; softmax over the selected logits only.
-void route_topk(const float* logits, int n, int k, int* sel, float* w, float* margin) {
+// `forced` (test hook, nullable): k expert ids to take, in this order, instead of the top-k -- the
+// weights are still the softmax of this row's own logits over them.  `gap_out` (nullable): the
+// relative gap between the last chosen and the first rejected logit of the unforced ranking.
+void route_topk(const float* logits, int n, int k, int* sel, float* w, float* margin, const int32_t* forced = nullptr,
+                float* gap_out = nullptr) {
     std::vector<int> order(n);
     for (int i = 0; i < n; i++) order[i] = i;
     std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return logits[a] > logits[b]; });
-    const float mx = logits[order[0]];
+    for (int i = 0; i < k; i++) sel[i] = forced ? forced[i] : order[i];
+    float mx = logits[sel[0]];
+    for (int i = 1; i < k; i++) mx = std::max(mx, logits[sel[i]]);
     float sum = 0.0f, ex[8];
     for (int i = 0; i < k; i++) {
-        sel[i] = order[i];
-        ex[i] = std::exp(logits[order[i]] - mx);
+        ex[i] = std::exp(logits[sel[i]] - mx);
         sum += ex[i];
     }
     for (int i = 0; i < k; i++) w[i] = ex[i] / sum * 1.0f;
     if (k < n) {
-        const float range = mx - logits[order[n - 1]];
+        const float range = logits[order[0]] - logits[order[n - 1]];
         const float gap = (logits[order[k - 1]] - logits[order[k]]) / (range > 0.0f ? range : 1.0f);
         if (gap < *margin) *margin = gap;
+        if (gap_out) *gap_out = gap;
+    } else if (gap_out) {
+        *gap_out = 1.0f;
     }
 }
 
@@ -132,6 +146,15 @@ extern "C" tso_model* tso_model_create(const tso_model_desc* desc) {
 
 extern "C" void tso_model_destroy(tso_model* m) { delete m; }
 extern "C" float tso_model_route_margin(const tso_model* m) { return m->route_margin; }
+extern "C" int tso_model_route_record(const tso_model* m, int32_t* sel, float* gap) {
+    if (m->route_sel.empty()) return -1;
+    std::copy(m->route_sel.begin(), m->route_sel.end(), sel);
+    std::copy(m->route_gap.begin(), m->route_gap.end(), gap);
+    return 0;
+}
+extern "C" void tso_model_force_route(tso_model* m, const int32_t* sel, int64_t n) {
+    m->forced_sel.assign(sel, sel + (sel ? n : 0));
+}
 extern "C" void tso_model_reset(tso_model* m) { m->position = 0; }
 extern "C" int64_t tso_model_position(const tso_model* m) { return m->position; }
 // kv_cache_rewind.rs:46-55: a cursor move; rows are addressed by absolute position and
@@ -283,9 +306,22 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
             add_bias(ly.router_bias, rl.data(), M, E);  // families/gptoss/moe.rs:82-87: before the top-k
             std::vector<float> routed(H);
             for (int m = 0; m < M; m++) {
-                int sel[8];
+                int sel[8] = {0};
                 float w[8];
-                route_topk(&rl[(size_t)m * E], E, K, sel, w, &mdl->route_margin);
+                // the record (and the forced routing of the test hook) covers the first 16 rows of a call
+                const bool rec = m < 16;
+                const size_t slot = (size_t)l * 16 + (size_t)(rec ? m : 0);
+                const int32_t* forced = rec && mdl->forced_sel.size() >= (slot + 1) * 8 ? &mdl->forced_sel[slot * 8] : nullptr;
+                if (mdl->route_sel.size() < (size_t)d.n_layers * 16 * 8) {
+                    mdl->route_sel.assign((size_t)d.n_layers * 16 * 8, -1);
+                    mdl->route_gap.assign((size_t)d.n_layers * 16, 1.0f);
+                }
+                float gap_row = 1.0f;
+                route_topk(&rl[(size_t)m * E], E, K, sel, w, &mdl->route_margin, forced, &gap_row);
+                if (rec) {
+                    mdl->route_gap[slot] = gap_row;
+                    for (int s2 = 0; s2 < 8; s2++) mdl->route_sel[slot * 8 + s2] = s2 < K ? sel[s2] : -1;
+                }
                 // families/llama/moe.rs:193-198: the routed sum starts from zero, is accumulated in
                 // rank order, and is then added to the stream
                 std::fill(routed.begin(), routed.end(), 0.0f);

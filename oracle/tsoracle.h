@@ -281,6 +281,15 @@ typedef struct tso_model tso_model;
  * selected and the first rejected router logit, relative to the row's logit range: a caller
  * comparing against an implementation with different rounding can see that no choice was close. */
 float tso_model_route_margin(const tso_model* m);
+/* The routing of the last verify call: sel [n_layers][16][8] expert ids in rank order (-1 past
+ * top_k), gap [n_layers][16] the relative gap between the last chosen and the first rejected router
+ * logit (real_forward_dispatch.rs:1135-1158 ranks by logit, ties to the lower index).  -1: no routed
+ * layer has run. */
+int tso_model_route_record(const tso_model* m, int32_t* sel, float* gap);
+/* Test hook: expert ids to take in place of the top-k ([n_layers][16][8], n values; n = 0 restores
+ * the ranking).  The weights remain the softmax of the row's own logits over the forced experts: how
+ * the logits come out had the router decided a near tie the other way. */
+void tso_model_force_route(tso_model* m, const int32_t* sel, int64_t n);
 tso_model* tso_model_create(const tso_model_desc* desc);
 void tso_model_destroy(tso_model* m);
 void tso_model_reset(tso_model* m);

@@ -1,4 +1,4 @@
-"""The C-ABI library loads and exports every symbol include/tsverify.h declares (no GPU needed),
+"""The C-ABI library loads and exports every symbol include/*.h declares (no GPU needed),
 and the host-side install helpers agree with the oracle bit for bit."""
 import os
 import re
@@ -11,9 +11,20 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared():
-    text = open(os.path.join(ROOT, "include", "tsverify.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(tsv_[a-z_0-9]+)\s*\(", text)))
+    """Every entry point the two headers declare: the drop-in surface and the test / measurement hooks."""
+    names = set()
+    for header in ("tsverify.h", "tsverify_testing.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(tsv_[a-z_0-9]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_the_hooks_live_in_their_own_header():
+    surface = open(os.path.join(ROOT, "include", "tsverify.h")).read()
+    for hook in ("tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat", "tsv_write_logits", "tsv_write_kv", "tsv_read_kv",
+                 "tsv_set_profile", "tsv_route_selected"):
+        assert hook + "(" not in surface, hook
 
 
 def test_every_declared_entry_point_is_exported():

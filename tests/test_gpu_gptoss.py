@@ -93,7 +93,7 @@ def test_gptoss_sampled_round_on_the_device():
 
 def test_a_rewind_deeper_than_the_window_is_safe_in_the_linear_layout():
     """`KvCacheManager::max_safe_rewind` (crates/gpu/src/kv_cache_rewind.rs:26-35) bounds a rollback by
-    the ring's slack; the windowed layers here store position p at slot p, so it is unbounded: after
+    the ring's slack; without `ring` the windowed layers store position p at slot p, so it is unbounded: after
     rolling back 40 rows (the window is 24) the continuation equals, by bits, a run that never went
     further."""
     import turbospark_amd as ts
@@ -109,3 +109,95 @@ def test_a_rewind_deeper_than_the_window_is_safe_in_the_linear_layout():
     gpu.prefill(prompt[:40], 0, want_logits=False)
     b = gpu.verify(tail, 40)
     assert np.array_equal(a, b)
+
+
+def _ring_pair(name, max_context, n_layers=None, seed=1234, **over):
+    """The same weights twice: windowed layers as rings (kv_cache.rs:122-131) and in the linear layout."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS[name], max_context=max_context, **over)
+    if n_layers:
+        cfg["n_layers"] = n_layers
+    w = synth.make_weights(cfg, seed=seed, n_layers=n_layers)
+    linear = ts.HipVerifier(cfg, w)
+    ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
+    return cfg, linear, ts.HipVerifier(cfg, ringed)
+
+
+def test_windowed_layers_as_rings_equal_the_linear_layout_by_bits():
+    """N rows fed through both layouts, far past the ring's capacity (window 24 -> a ring of 64 slots):
+    prompt passes, verify passes, rollbacks inside the budget, a tree pass with compaction across the
+    ring's seam -- every logit equal by bits; the budget is capacity - window
+    (kv_cache_rewind.rs:26-35) and a rollback beyond it is refused by name (:46-55)."""
+    import turbospark_amd as ts
+    from turbospark_amd import TsvError
+    cfg, lin, ring = _ring_pair("gptoss_small", 400)
+    V = cfg["vocab"]
+    assert lin.max_safe_rewind() == 2 ** 63 - 1 and ring.max_safe_rewind() == 64 - 24
+    prompt = _prompt(150, V, 5)
+    a = lin.prefill(prompt, 0)
+    b = ring.prefill(prompt, 0)
+    assert np.array_equal(a, b)
+    rng = np.random.default_rng(2)
+    base = 150
+    for rnd in range(30):                       # verify, keep a few rows, continue: crosses the seam several times
+        m = int(rng.integers(1, 17))
+        feed = rng.integers(0, V, m).astype(np.int32)
+        pa, pb = lin.checkpoint(), ring.checkpoint()
+        assert np.array_equal(lin.verify(feed, base), ring.verify(feed, base)), rnd
+        keep = int(rng.integers(1, m + 1))
+        lin.rollback_retaining(pa, keep)
+        ring.rollback_retaining(pb, keep)
+        base += keep
+        assert lin.position == ring.position == base
+    # a tree pass whose rows straddle the seam, compacted
+    parent = [-1, 0, 0, 1, 1, 2, 3, 5]
+    feed = rng.integers(0, V, 8).astype(np.int32)
+    for eng in (lin, ring):
+        eng.verify_tree(feed, parent, base, want_logits=False)
+        eng.compact_tree(base, [0, 2, 5, 7])
+        eng.rollback_retaining(ts.ffi.Point(base), 4)
+    nxt = rng.integers(0, V, 3).astype(np.int32)
+    assert np.array_equal(lin.verify(nxt, base + 4), ring.verify(nxt, base + 4))
+    base += 8                                   # one past the last row ever written (the tree's eighth row)
+    # the budget: 40 rows behind the last row written is the limit
+    ring.rollback(ts.ffi.Point(base - 40))
+    lin.rollback(ts.ffi.Point(base - 40))
+    assert np.array_equal(lin.verify(nxt, base - 40), ring.verify(nxt, base - 40))
+    with pytest.raises(TsvError, match="exceeds the ring slack"):
+        ring.rollback(ts.ffi.Point(base - 41))
+    assert ring.position == base - 37
+    with pytest.raises(TsvError, match="no longer holds"):
+        ring.read_kv(0, 0, 4)                   # layer 0 slides: its first rows are long overwritten
+    k_full, _ = ring.read_kv(1, 0, 4)           # layer 1 is full attention: everything is there
+    assert np.array_equal(k_full, lin.read_kv(1, 0, 4)[0])
+    k_ring, v_ring = ring.read_kv(0, base - 60, 20)
+    k_lin, v_lin = lin.read_kv(0, base - 60, 20)
+    assert np.array_equal(k_ring, k_lin) and np.array_equal(v_ring, v_lin)
+    # a reset starts the ring over
+    ring.reset()
+    lin.reset()
+    assert np.array_equal(lin.prefill(prompt[:70], 0), ring.prefill(prompt[:70], 0))
+
+
+def test_gptoss_120b_geometry_ring_equals_linear_at_long_context():
+    """The gpt-oss-120B geometry (window 128 -> a ring of 160 slots beside a 3000-token context): seeded
+    rows written into both layouts, a nine-row pass, a rollback and a second pass, equal by bits."""
+    import turbospark_amd as ts
+    ctx = 3000
+    cfg, lin, ring = _ring_pair("gptoss_120b", ctx + 64, n_layers=2, vocab=4096)
+    rng = np.random.default_rng(3)
+    shape = (ctx, cfg["n_kv_heads"], cfg["head_dim"])
+    for layer in range(2):
+        k = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+        v = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+        lin.write_kv(layer, 0, k, v)
+        ring.write_kv(layer, 0, k, v)
+    assert ring.position == lin.position == ctx and ring.max_safe_rewind() == 160 - 128
+    feed = rng.integers(0, cfg["vocab"], 9).astype(np.int32)
+    pa, pb = lin.checkpoint(), ring.checkpoint()
+    assert np.array_equal(lin.verify(feed, ctx), ring.verify(feed, ctx))
+    lin.rollback_retaining(pa, 3)
+    ring.rollback_retaining(pb, 3)
+    feed2 = rng.integers(0, cfg["vocab"], 9).astype(np.int32)
+    assert np.array_equal(lin.verify(feed2, ctx + 3), ring.verify(feed2, ctx + 3))

@@ -1,0 +1,265 @@
+// Device-side core of the split-KV GQA attention of a verify pass: one workgroup's pass over its
+// chunk of the context (crates/gpu/src/attention_decode.rs:1092-1363; arithmetic contract
+// crates/compute/src/attention.rs:53-137).  Shared by the stand-alone attention kernel and the
+// per-XCD fused attention block.
+#pragma once
+#include "tsv_internal.h"
+
+namespace tsv {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// The library is compiled with -ffp-contract=off and every fused multiply-add here is written out:
+// left to itself the compiler contracts a * b + c * d one way in one template instantiation and the
+// other way in the next, and a row's bits would then depend on how many rows share its pass.
+//
+// One (m, l, O) running state merged into another (flash-decoding rescale).
+template <int RT, int VT>
+__device__ __forceinline__ void merge_state(float (&mrun)[RT], float (&lrun)[RT], float4v (&O)[RT][VT], const float* src) {
+    // `src` points at this lane's column of a [values][64 lanes] slot: consecutive lanes touch
+    // consecutive LDS banks
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const float m1 = src[64 * (2 * t)], l1 = src[64 * (2 * t + 1)];
+        const float mnew = fmaxf(mrun[t], m1);
+        if (mnew > -INFINITY) {
+            const float a0 = __expf(mrun[t] - mnew), a1 = __expf(m1 - mnew);
+            lrun[t] = fmaf(lrun[t], a0, l1 * a1);
+#pragma unroll
+            for (int d = 0; d < VT; d++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) O[t][d][i] = fmaf(O[t][d][i], a0, src[64 * (2 * RT + (t * VT + d) * 4 + i)] * a1);
+            mrun[t] = mnew;
+        }
+    }
+}
+template <int RT, int VT>
+__device__ __forceinline__ void store_state(const float (&mrun)[RT], const float (&lrun)[RT], const float4v (&O)[RT][VT],
+                                            float* dst) {
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        dst[64 * (2 * t)] = mrun[t];
+        dst[64 * (2 * t + 1)] = lrun[t];
+#pragma unroll
+        for (int d = 0; d < VT; d++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[64 * (2 * RT + (t * VT + d) * 4 + i)] = O[t][d][i];
+    }
+}
+
+// Eight waves per workgroup share a chunk of the context, each walking every eighth 16-position
+// block with up to STAGES blocks of K and V in flight.
+// COH: the query rows and the K / V blocks are read device-coherently (sc1), for a caller whose
+// other compute units wrote them earlier in the same kernel.
+// xch: [4 slots][PER_LANE values][64 lanes] floats of LDS.
+template <int HD, int RT, int STAGES, bool COH>
+__device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int R, int chunk, int h, int rt0, float* xch) {
+    constexpr int NW = 8;
+    constexpr int KS = HD / 32;  // K steps of the score MFMA
+    constexpr int VT = HD / 16;  // output tiles along head_dim
+    constexpr int PER_LANE = RT * VT * 4 + 2 * RT;
+    constexpr int POLICY = COH ? 16 : 0;  // buffer-load cache policy: sc1
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 15, kg = lane >> 4;
+    const VerifyParams* vp = a.vp;
+    const int M = a.base_hint >= 0 ? a.m_hint : vp->m, base = a.base_hint >= 0 ? a.base_hint : vp->base, kvlen = base + M;
+    const int nblk = (kvlen + 15) >> 4;
+    // sliding window (families/gptoss/attn.rs:120-137): a row at sequence length n sees positions
+    // n - window .. n - 1.  The window exceeds the pass width, so every row keeps its whole drafted
+    // suffix and the cut falls in the committed prefix: blocks before the first row's cut are not
+    // read at all, the few blocks where the rows' cuts differ are masked per row.
+    const int window = a.window;
+    const int bfirst = window > 0 ? max(base + 1 - window, 0) >> 4 : 0;
+    const int bpc = (nblk - bfirst + a.nch - 1) / a.nch;
+    const int b0 = bfirst + chunk * bpc, b1 = min(b0 + bpc, nblk);
+    const int cut_end = window > 0 ? base + M - window : 0;  // positions from here on are inside every row's window
+    const float scale = a.scale;
+    const uint32_t mmask = (1u << M) - 1u;  // slots that exist in this pass
+
+    // query fragments and per-row ancestor sets
+    uint4 qf[RT][KS];
+    uint32_t anc[RT];
+    int lo[RT];  // first visible position of the row (window)
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const int r = (rt0 + t) * 16 + j;
+        anc[t] = 0xFFFFu;
+        lo[t] = 0;
+        if (r < R) {
+            const int mrow = r / G, g = r - mrow * G;
+            anc[t] = vp->anc[mrow];
+            if (window > 0) lo[t] = vp->pos[mrow] + 1 - window;
+            const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
+            if (COH) {
+                const __amdgpu_buffer_rsrc_t qrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.q16, 0, 0x7FFFFFFF, 0x00027000);
+                const uint32_t qo = (uint32_t)((const char*)q - (const char*)a.q16);
+#pragma unroll
+                for (int s = 0; s < KS; s++)
+                    qf[t][s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qrs, qo + 64 * s, 0, 16));
+            } else {
+#pragma unroll
+                for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < KS; s++) qf[t][s] = make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    float mrun[RT], lrun[RT];
+    float4v O[RT][VT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        mrun[t] = -INFINITY;
+        lrun[t] = 0.f;
+#pragma unroll
+        for (int d = 0; d < VT; d++) O[t][d] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // this head's K rows and V blocks as buffers that end after block b1 - 1; a ring layer
+    // (kv_cache.rs:360-378: position p lives in slot p % capacity) keeps block b in slot b % nbc
+    const bool ring = a.ring != 0;
+    const int nbc = a.max_ctx >> 4;
+    const uint32_t blk_bytes = 16 * HD * 2;
+    const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const _Float16*)a.kc + (long)h * a.max_ctx * HD), 0, (int)((ring ? nbc : b1) * blk_bytes), 0x00027000);
+    const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const _Float16*)a.vc + (long)h * (a.max_ctx >> 4) * (HD * 16)), 0, (int)((ring ? nbc : b1) * blk_bytes), 0x00027000);
+    struct Blk {
+        u32x4 kf[KS];
+        u32x2 vf[VT];
+    };
+    const uint32_t koff = (uint32_t)(j * HD + 8 * kg) * 2, voff = (uint32_t)lane * 8;
+    const int nb = b1 > b0 + wave ? (b1 - b0 - wave + NW - 1) / NW : 0;  // blocks of this wave
+    auto fetch = [&](Blk& st, int i) {  // block i of this wave's run
+        const int blk = b0 + wave + NW * i;
+        const uint32_t bo = (uint32_t)(ring ? blk % nbc : blk) * blk_bytes;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; s++) st.kf[s] = __builtin_amdgcn_raw_buffer_load_b128(krs, bo + koff + 64 * s, 0, POLICY);
+#pragma unroll
+        for (int d = 0; d < VT; d++) st.vf[d] = __builtin_amdgcn_raw_buffer_load_b64(vrs, bo + voff + 512 * d, 0, POLICY);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto consume = [&](const Blk& st, int i) {
+        const int p0 = (b0 + wave + NW * i) << 4;
+        const bool tail = p0 + 16 > base;
+#pragma unroll
+        for (int t = 0; t < RT; t++) {
+            float4v S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; s++)
+                S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, st.kf[s]),
+                                                           __builtin_bit_cast(half8, qf[t][s]), S, 0, 0, 0);
+            // Visibility of this lane's four positions as a 4-bit word, computed without
+            // branches: bit (slot + 16) of `w` says whether cache slot base+slot is visible
+            // (the 16 low bits stand for prefix positions, always visible).
+            uint32_t vis4 = 0xFu;
+            if (tail) {
+                const uint64_t w = ((uint64_t)(anc[t] & mmask) << 16) | 0xFFFFull;
+                vis4 = (uint32_t)(w >> (p0 + 4 * kg - base + 16)) & 0xFu;  // shift in [1, 47]
+            }
+            if (p0 < cut_end) {  // some row's window starts inside or after this block
+                const int d = lo[t] - (p0 + 4 * kg);  // this lane's positions below index d are outside
+                vis4 &= d <= 0 ? 0xFu : d >= 4 ? 0u : (0xFu << d) & 0xFu;
+            }
+            float sc[4];
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++) sc[i4] = ((vis4 >> i4) & 1u) ? S[i4] * scale : -INFINITY;
+            float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            mb = fmaxf(mb, __shfl_xor(mb, 16));
+            mb = fmaxf(mb, __shfl_xor(mb, 32));
+            const float mnew = fmaxf(mrun[t], mb);
+            float alpha = 1.f;
+            half4 P = {0, 0, 0, 0};
+            if (mnew > -INFINITY) {
+                alpha = __expf(mrun[t] - mnew);
+                float ps = 0.f;
+#pragma unroll
+                for (int i4 = 0; i4 < 4; i4++) {
+                    const float p = __expf(sc[i4] - mnew);
+                    ps += p;
+                    P[i4] = (_Float16)p;
+                }
+                lrun[t] = fmaf(lrun[t], alpha, ps);
+                mrun[t] = mnew;
+            }
+#pragma unroll
+            for (int d = 0; d < VT; d++) {
+                O[t][d] *= alpha;
+                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, st.vf[d]), P, O[t][d], 0, 0, 0);
+            }
+        }
+    };
+    // Short runs are straight-line code (every load issued before the first wait, no load the run
+    // does not need); longer ones keep STAGES blocks in flight, with unconditional loads in the
+    // steady state so the compiler waits on the oldest block only.
+    if (nb == 1) {
+        Blk st;
+        fetch(st, 0);
+        consume(st, 0);
+    } else if (nb == 2) {
+        Blk s0, s1;
+        fetch(s0, 0);
+        fetch(s1, 1);
+        consume(s0, 0);
+        consume(s1, 1);
+    } else if (nb >= STAGES) {
+        Blk st[STAGES];
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) fetch(st[s], s);
+        int i = 0;
+        for (; i + 2 * STAGES <= nb; i += STAGES) {
+#pragma unroll
+            for (int s = 0; s < STAGES; s++) {
+                consume(st[s], i + s);
+                fetch(st[s], i + s + STAGES);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) {
+            if (i + s < nb) {
+                consume(st[s], i + s);
+                if (i + s + STAGES < nb) fetch(st[s], i + s + STAGES);
+            }
+        }
+        i += STAGES;
+#pragma unroll
+        for (int s = 0; s < STAGES; s++)
+            if (i + s < nb) consume(st[s], i + s);
+    }
+
+    // fold the eight waves' running (m, l, O): 4..7 into 0..3, then 1..3 into 0
+    float* mine = xch + (wave & 3) * 64 * PER_LANE + lane;
+    if (wave >= 4) store_state<RT, VT>(mrun, lrun, O, mine);
+    __syncthreads();
+    if (wave < 4) merge_state<RT, VT>(mrun, lrun, O, mine);
+    __syncthreads();
+    if (wave >= 1 && wave < 4) store_state<RT, VT>(mrun, lrun, O, mine);
+    __syncthreads();
+    if (wave != 0) return;
+    for (int w = 1; w < 4; w++) merge_state<RT, VT>(mrun, lrun, O, xch + w * 64 * PER_LANE + lane);
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        float l = lrun[t];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        const int r = (rt0 + t) * 16 + j;
+        if (r >= R) continue;
+        const long slot = ((long)h * a.nch + chunk) * R + r;
+        if (kg == 0) {
+            a.part_ml[slot * 2] = mrun[t];
+            a.part_ml[slot * 2 + 1] = l;
+        }
+        float* o = a.part_o + slot * HD + 4 * kg;
+#pragma unroll
+        for (int d = 0; d < VT; d++) *(float4v*)(o + 16 * d) = O[t][d];
+    }
+}
+
+}  // namespace tsv

@@ -21,79 +21,11 @@
 // Every wait is bounded: a barrier that does not complete within its spin budget raises the
 // error flag and the workgroup returns, so the grid always drains.
 #include "gemm_core.h"
+#include "xcd_sync.h"
 
 namespace tsv {
 
 namespace {
-
-constexpr int XCDS = 8;
-constexpr int WGS_PER_XCD = 32;
-constexpr unsigned SPIN_LIMIT = 1u << 22;
-
-struct XcdCtx {
-    int xcc, rank;
-    unsigned* bar;
-    unsigned next_target;
-    int* err;
-};
-
-// Identifies the workgroup's XCD and its rank among that XCD's workgroups.  The rank counter
-// only ever grows by 32 per launch, so the low five bits are the rank.
-__device__ __forceinline__ bool xcd_enter(XcdCtx& c, const FusedSync& s, int* lds_i) {
-    if (threadIdx.x == 0) {
-        unsigned xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        xcc &= 0xFu;
-        lds_i[0] = (int)xcc;
-        lds_i[1] = xcc < XCDS ? (int)(__hip_atomic_fetch_add(s.rank_ctr + xcc * 64, 1u, __ATOMIC_RELAXED,
-                                                            __HIP_MEMORY_SCOPE_AGENT) &
-                                      (WGS_PER_XCD - 1))
-                              : -1;
-    }
-    __syncthreads();
-    c.xcc = lds_i[0];
-    c.rank = lds_i[1];
-    c.err = s.err;
-    if (c.rank < 0) {
-        if (threadIdx.x == 0) *s.err = 2;
-        return false;
-    }
-    c.bar = s.bar_ctr + c.xcc * 64;
-    c.next_target = s.bar_base + WGS_PER_XCD;
-    __syncthreads();
-    return true;
-}
-
-// Barrier over the 32 workgroups of this XCD.  A wave that stored something the other side of
-// the barrier will read first waits for its stores to be acknowledged by the L2 (drain); a wave
-// that only has weight prefetches in flight must not wait for those here.
-__device__ __forceinline__ bool xcd_barrier(XcdCtx& c, int* lds_i, bool drain = true) {
-    if (drain) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(c.bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned n = 0;
-        int ok = 1;
-        while ((int)(__hip_atomic_load(c.bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - c.next_target) < 0) {
-            if (++n > SPIN_LIMIT) {
-                ok = 0;
-                *c.err = 1;
-                break;
-            }
-        }
-        lds_i[2] = ok;
-    }
-    __syncthreads();
-    c.next_target += WGS_PER_XCD;
-    const bool ok = lds_i[2] != 0;
-    __syncthreads();
-    return ok;
-}
-
-__device__ __forceinline__ float ld_sc1(const float* base, int idx) {
-    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7FFFFFFF, 0x00027000);
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, idx * 4, 0, 16));
-}
 
 // ---- P0: residual add + RMSNorm inputs, spread over the XCD's workgroups ---------------------
 // x[b][:] += sum of the incoming partial sums (fixed order); this XCD's private copy of the

@@ -246,58 +246,10 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
 }
 
 // Stores one row group's finished sums.  v[i] is output column n of activation row 4g+i.
-// The fused q/k/v projection finishing its own rows (no split-K: the sums are complete here).
-// A tile of the rotated sections holds dims i (lanes 0..31) and i + hd/2 (lanes 32..63) of one
-// head: the NeoX pair of a lane is lane ^ 32 (crates/compute/src/rope.rs:208-256).  Bias first,
-// then the rotation (families/gptoss/attn.rs:88-118); q goes to the fp16 q buffer, K and V
-// straight into the cache slot of the row (families/qwen/batched_layers.rs:84-113).
-__device__ __forceinline__ void rope_epilogue(const GemmArgs& a, int tile, int g, float4v v, int lane, int M) {
-    const RopeEpi& e = a.rope;
-    const VerifyParams* vp = a.vp;
-    const int hd = e.hd, half = hd >> 1, tph = hd >> 6;  // tiles per head
-    const int tq = e.nq * tph, tk = e.nkv * tph;
-    const int kind = tile < tq ? 0 : tile < tq + tk ? 1 : 2;
-    const int st = kind == 0 ? tile : kind == 1 ? tile - tq : tile - tq - tk;
-    const int head = st / tph, t = st - head * tph;
-    const bool hi = lane >= 32;
-    const int idim = (tph == 2 ? 32 * t : 0) + (lane & 31);     // rotation pair index, 0 .. hd/2
-    const int d = kind == 2 ? t * 64 + lane : (hi ? idim + half : idim);  // this lane's head dimension
-    const int col = (kind == 0 ? 0 : kind == 1 ? e.nq * hd : (e.nq + e.nkv) * hd) + head * hd + d;
-    const float bias = e.bias ? e.bias[col] : 0.f;
-    const int base = vp->base;
-    float2 cs[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) cs[i] = kind != 2 && 4 * g + i < M ? e.cs[(4 * g + i) * half + idim] : float2{1.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int b = 4 * g + i;
-        float x = v[i] + bias;
-        const float other = __shfl_xor(x, 32);
-        if (b >= M) continue;
-        if (kind != 2) {
-            const float x0 = hi ? other : x, x1 = hi ? x : other;
-            x = hi ? x0 * cs[i].y + x1 * cs[i].x : x0 * cs[i].x - x1 * cs[i].y;
-        }
-        const _Float16 h = (_Float16)x;
-        if (kind == 0) {
-            ((_Float16*)e.q16)[((long)b * e.nq + head) * hd + d] = h;
-        } else {
-            const int pos = base + b;  // the cache slot of row b
-            if (kind == 1) {
-                ((_Float16*)e.kc)[((long)head * e.max_ctx + pos) * hd + d] = h;
-            } else {
-                _Float16* vb = (_Float16*)e.vc + ((long)head * (e.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
-                const int po = pos & 15;
-                vb[(((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3)] = h;
-            }
-        }
-    }
-}
-
 template <int EPI>
 __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split, int g, float4v v, int lane, int M) {
     if (EPI == EPI_ROPE) {
-        rope_epilogue(a, tile, g, v, lane, M);
+        rope_epilogue(a.rope, a.vp, tile, g, v, lane, M);
         return;
     }
     if (EPI == EPI_SILU) {
@@ -552,7 +504,7 @@ __device__ __forceinline__ void epilogue16(const GemmArgs& a, int tile, int spli
                 q[d0] = h0;
                 q[d1] = h1;
             } else {
-                const int pos = base + b;
+                const int pos = (base + b) % e.max_ctx;
                 if (kind == 1) {
                     _Float16* kc = (_Float16*)e.kc + ((long)head * e.max_ctx + pos) * hd;
                     kc[d0] = h0;

@@ -10,6 +10,7 @@
 #include <unistd.h>
 
 #include <climits>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -533,7 +534,13 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
             if (!s.required) continue;
             if ((rc = get(p + s.suffix, s.t, s.required))) return rc;
         }
-        if (is_oss && l % 2 == 0) L.window = (int32_t)window;
+        if (is_oss && l % 2 == 0) {
+            L.window = (int32_t)window;
+            // the reference's fp16 ring for windowed layers is a session option there too
+            // (kv_cache.rs:122-131 fp16_ring_enabled); here the process environment asks for it
+            const char* ring = getenv("TSV_KV_RING");
+            L.ring = ring && ring[0] == '1';
+        }
         if (routed) {
             L.n_experts = (int32_t)n_experts;
             const double used = opt("expert_used_count", 0);

@@ -316,7 +316,7 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
         q[i] = h0;
         q[i + half] = h1;
     } else {
-        const int pos = base + m;  // the cache slot of row m
+        const int pos = (base + m) % a.max_ctx;  // the cache slot of row m (a ring layer wraps at its capacity)
         if (kind == 1) {
             _Float16* k = (_Float16*)a.kc + ((long)h * a.max_ctx + pos) * hd;
             k[i] = h0;
@@ -352,13 +352,15 @@ __device__ __forceinline__ long v_index(int h, int pos, int d, int hd, int max_c
 // base..base+n.  path is strictly increasing with path[i] >= i, so walking i upward never
 // overwrites a row that is still to be read.  One workgroup per (kv head, layer), sequential over i:
 // every layer's cache in one launch.
-__global__ void k_kv_gather(uint16_t* const* caches, int hd, int max_ctx, const int32_t* path, int n, int base) {
-    // grid (kv heads, layers): caches[2 * layer] is the layer's K buffer, [2 * layer + 1] its V buffer
+__global__ void k_kv_gather(uint16_t* const* caches, const int32_t* caps, int hd, const int32_t* path, int n, int base) {
+    // grid (kv heads, layers): caches[2 * layer] is the layer's K buffer, [2 * layer + 1] its V buffer,
+    // caps[layer] the positions it holds (a ring layer wraps there)
     uint16_t* kc = caches[2 * blockIdx.y];
     uint16_t* vc = caches[2 * blockIdx.y + 1];
+    const int max_ctx = caps[blockIdx.y];
     const int h = blockIdx.x, d = threadIdx.x;
     for (int i = 0; i < n; i++) {
-        const int src = base + path[i], dst = base + i;
+        const int src = (base + path[i]) % max_ctx, dst = (base + i) % max_ctx;
         if (src == dst) continue;
         if (d < hd) {
             kc[((long)h * max_ctx + dst) * hd + d] = kc[((long)h * max_ctx + src) * hd + d];
@@ -367,9 +369,9 @@ __global__ void k_kv_gather(uint16_t* const* caches, int hd, int max_ctx, const 
     }
 }
 
-int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, int n_layers, int nkv, int hd, int max_ctx,
+int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, const int32_t* caps_dev, int n_layers, int nkv, int hd,
                      const int32_t* path_dev, int n, int base) {
-    hipLaunchKernelGGL(k_kv_gather, dim3(nkv, n_layers), dim3(128), 0, s, caches_dev, hd, max_ctx, path_dev, n, base);
+    hipLaunchKernelGGL(k_kv_gather, dim3(nkv, n_layers), dim3(128), 0, s, caches_dev, caps_dev, hd, path_dev, n, base);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -379,8 +381,9 @@ __global__ void k_kv_read(const uint16_t* kc, const uint16_t* vc, int nkv, int h
     const int p = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
     if (d >= hd) return;
     const long o = ((long)p * nkv + h) * hd + d;
-    k_out[o] = kc[((long)h * max_ctx + pos0 + p) * hd + d];
-    v_out[o] = vc[v_index(h, pos0 + p, d, hd, max_ctx)];
+    const int pos = (pos0 + p) % max_ctx;
+    k_out[o] = kc[((long)h * max_ctx + pos) * hd + d];
+    v_out[o] = vc[v_index(h, pos, d, hd, max_ctx)];
 }
 
 __global__ void k_kv_fill(uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0,
@@ -388,8 +391,9 @@ __global__ void k_kv_fill(uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_c
     const int p = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
     if (d >= hd) return;
     const long o = ((long)p * nkv + h) * hd + d;
-    kc[((long)h * max_ctx + pos0 + p) * hd + d] = k_in[o];
-    vc[v_index(h, pos0 + p, d, hd, max_ctx)] = v_in[o];
+    const int pos = (pos0 + p) % max_ctx;
+    kc[((long)h * max_ctx + pos) * hd + d] = k_in[o];
+    vc[v_index(h, pos, d, hd, max_ctx)] = v_in[o];
 }
 
 int launch_kv_fill(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0, int n,

@@ -30,6 +30,7 @@ struct LayerW {
     float *bqkv = nullptr, *bo = nullptr, *sinks = nullptr, *router_bias = nullptr;
     float *be_gate = nullptr, *be_up = nullptr, *be_down = nullptr;
     int window = 0;
+    int cap = 0;        // positions the layer's cache holds: the context, or a ring of window + slack
     bool rope_fused = false;  // the q/k/v projection rotates and stores its own rows
     uint16_t *kc = nullptr, *vc = nullptr;
 };
@@ -73,7 +74,9 @@ struct tsv_ctx {
     float* moe_out = nullptr;
     // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
     // sum-of-squares partials, per-XCD partial sums, barrier counters
-    bool fused_ffn = false;
+    bool fused_ffn = false, fused_attn = false;
+    int attn_stages = 5;  // TSV_FUSED_ATTN_STAGES: how far the attention block goes before the separate kernels take over
+    float* partial8a = nullptr;  // the attention block's per-XCD partial sums
     float* x2 = nullptr;
     uint8_t* frag8 = nullptr;
     size_t frag8_stride = 0;
@@ -98,6 +101,9 @@ struct tsv_ctx {
     AcceptScratch sc{};
     std::vector<void*> allocs;
     int64_t position = 0;
+    int64_t high_water = 0;     // one past the last position any pass has written since the last reset
+    int64_t rewind_budget = INT64_MAX;  // KvCacheManager::max_safe_rewind: min over ring layers of capacity - window
+    int32_t* kv_caps = nullptr;  // device: positions each layer's cache holds (tree compaction)
     tsv_prefix prefix;          // the ids behind rows [0, prefix length): kv_prefix.rs
     bool prefix_reuse = false;  // RealForwardRunner::set_prefix_reuse: off unless the host opts in
     bool headless = false;      // the pass in flight is a prefill pass nobody reads the logits of
@@ -395,9 +401,22 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     int rc = run_pass(c, m);
     if (rc) return rc;
     c->position = base + m;
+    c->high_water = std::max(c->high_water, c->position);
     c->last_m = m;
     c->last_base = base;
     return TSV_OK;
+}
+
+// kv_cache_rewind.rs:46-55: a cursor may move back only as far as every ring layer still holds the
+// window of the position it lands on.  Rows are overwritten up to the high-water mark, so the test
+// is made against it (the reference tests each rewind's own count, which is the same thing in a
+// loop that never rolls back past its last checkpoint).
+int check_rewind(tsv_ctx* c, int64_t new_position, const char* who) {
+    if (c->rewind_budget == INT64_MAX || c->high_water - new_position <= c->rewind_budget) return TSV_OK;
+    set_error(std::string(who) + ": rewind of " + std::to_string((long long)(c->high_water - new_position)) +
+              " rows exceeds the ring slack of " + std::to_string((long long)c->rewind_budget) +
+              ": a sliding-window layer would read rows that have already been overwritten");
+    return TSV_ERR_INVALID;
 }
 
 // The kernels of one pass over m rows, in order, on the handle's stream.
@@ -416,8 +435,86 @@ int launch_pass(tsv_ctx* c, int m) {
     const float* prev_weights = nullptr;  // routed experts: the factors of the per-slot outputs
     float *x = c->x, *x_other = c->x2;  // the fused kernels write the residual rows to the other buffer
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
+    // the attention half as one per-XCD kernel: passes of at most eight rows and 32 (row, q head) pairs
+    const bool attn_block = c->fused_attn && m <= 8 && m * (c->nq / c->nkv) <= 32;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
+        int attn_splits = 0;  // partial sums the attention half leaves for the FFN norm
+        const float* attn_partial = c->partial;
+        if (attn_block && !prev_weights) {
+            AttnBlockArgs ba{};
+            ba.sync.rank_ctr = c->rank_ctr;
+            ba.sync.bar_ctr = c->bar_ctr;
+            ba.sync.err = c->fused_err;
+            ba.sync.bar_base = c->bar_count;
+            c->bar_count += 32u * (unsigned)attn_block_barriers();
+            ba.x_in = x;
+            ba.x_out = x_other;
+            ba.partial = prev_partial;
+            ba.n_partials = prev_splits;
+            ba.bias_in = nullptr;
+            ba.norm_w = L.attn_norm;
+            ba.frag = c->frag8;
+            ba.frag_stride = c->frag8_stride;
+            ba.ssq = c->ssq8;
+            ba.hidden = c->hidden;
+            ba.eps = c->eps;
+            ba.m = m;
+            ba.w_qkv = L.qkv.tiles;
+            ba.qkv_kchunks = L.qkv.kchunks;
+            ba.rope.cs = c->rope_cs;
+            ba.rope.bias = L.bqkv;
+            ba.rope.q16 = c->q16;
+            ba.rope.kc = L.kc;
+            ba.rope.vc = L.vc;
+            ba.rope.nq = c->nq;
+            ba.rope.nkv = c->nkv;
+            ba.rope.hd = c->hd;
+            ba.rope.max_ctx = L.cap;
+            ba.vp = c->vp_dev;
+            ba.attn.q16 = c->q16;
+            ba.attn.kc = L.kc;
+            ba.attn.vc = L.vc;
+            ba.attn.part_o = c->part_o;
+            ba.attn.part_ml = c->part_ml;
+            ba.attn.xfrag = c->xf_b;
+            ba.attn.nq = c->nq;
+            ba.attn.nkv = c->nkv;
+            ba.attn.hd = c->hd;
+            ba.attn.max_ctx = L.cap;
+            ba.attn.nch = c->nch;
+            ba.attn.scale = c->attn_scale;
+            ba.attn.window = 0;
+            ba.attn.sinks = nullptr;
+            ba.attn.vp = c->vp_dev;
+            ba.attn.m_hint = m;
+            ba.attn.base_hint = c->vp_host->base;
+            ba.w_o = L.wo.tiles;
+            ba.wo_tiles = L.wo.n_tiles;
+            ba.wo_kchunks = L.wo.kchunks;
+            ba.partial_out = c->partial8a;
+            ba.stages = c->attn_stages;
+            {
+                PROF(PC_ATTN);
+                rc = launch_attn_block(s, L.qkv.fmt, ba);
+            }
+            if (rc) return rc;
+            std::swap(x, x_other);
+            attn_splits = 8;
+            attn_partial = c->partial8a;
+            if (c->attn_stages < 5) {  // the remaining stages as separate kernels
+                if (c->attn_stages < 4) {
+                    AttnArgs aa = ba.attn;
+                    aa.nch = c->nch;
+                    if ((rc = c->attn_stages == 3 ? launch_attention_merge(s, aa, m) : launch_attention(s, aa, m))) return rc;
+                }
+                attn_splits = splits_for(L.wo, m, EPI_PARTIAL);
+                attn_partial = c->partial;
+                if ((rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, attn_splits, EPI_PARTIAL, c->hidden, c->hidden)))
+                    return rc;
+            }
+        }
+        if (!attn_splits) {
         {
             PROF(PC_NORM);
             rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m,
@@ -443,7 +540,7 @@ int launch_pass(tsv_ctx* c, int m) {
             re.nq = c->nq;
             re.nkv = c->nkv;
             re.hd = c->hd;
-            re.max_ctx = c->ctx_alloc;
+            re.max_ctx = L.cap;
             PROF(PC_QKV);
             rc = 0;
             for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++)
@@ -475,7 +572,7 @@ int launch_pass(tsv_ctx* c, int m) {
         ra.nq = c->nq;
         ra.nkv = c->nkv;
         ra.hd = c->hd;
-        ra.max_ctx = c->ctx_alloc;
+        ra.max_ctx = L.cap;
         ra.vp = c->vp_dev;
         if (!L.rope_fused) {
             PROF(PC_ROPE);
@@ -493,7 +590,8 @@ int launch_pass(tsv_ctx* c, int m) {
         aa.nq = c->nq;
         aa.nkv = c->nkv;
         aa.hd = c->hd;
-        aa.max_ctx = c->ctx_alloc;
+        aa.max_ctx = L.cap;
+        aa.ring = L.cap < c->ctx_alloc;
         aa.nch = c->nch;
         aa.scale = c->attn_scale;
         aa.window = L.window;
@@ -514,6 +612,9 @@ int launch_pass(tsv_ctx* c, int m) {
             for (int rep = 0; rep < c->repeat[PC_WO] && !rc; rep++) rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
         }
         if (rc) return rc;
+        attn_splits = sp;
+        }  // the separate kernels of the attention half
+        int sp = attn_splits;
         if (c->fused_ffn) {
             FfnBlockArgs fa{};
             fa.sync.rank_ctr = c->rank_ctr;
@@ -523,7 +624,7 @@ int launch_pass(tsv_ctx* c, int m) {
             c->bar_count += 32u * (unsigned)fused_ffn_barriers();
             fa.norm.x_in = x;
             fa.norm.x_out = x_other;
-            fa.norm.partial = c->partial;
+            fa.norm.partial = attn_partial;
             fa.norm.n_partials = sp;
             fa.norm.norm_w = L.ffn_norm;
             fa.norm.frag = c->frag8;
@@ -553,7 +654,7 @@ int launch_pass(tsv_ctx* c, int m) {
         }
         {
             PROF(PC_NORM);
-            rc = launch_addnorm(s, x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo);
+            rc = launch_addnorm(s, x, attn_partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo);
         }
         if (rc) return rc;
         if (L.n_experts) {
@@ -568,7 +669,7 @@ int launch_pass(tsv_ctx* c, int m) {
             ra2.top_k = L.top_k;
             ra2.m = m;
             ra2.weights = c->route_w;
-            ra2.selected = c->route_sel;
+            ra2.selected = c->route_sel + (size_t)l * 16 * 8;  // kept per layer: tsv_route_selected reads them back
             ra2.groups = c->route_groups;
             ra2.bias = L.router_bias;
             MoeGemmArgs g1{}, g2{};
@@ -690,6 +791,7 @@ int check_fused(tsv_ctx* c) {
                                  : "fused layer kernel: XCD barrier timed out; fused path disabled, repeat the call");
     *c->fused_err = 0;
     c->fused_ffn = false;
+    c->fused_attn = false;
     return TSV_ERR_DEVICE;
 }
 
@@ -857,7 +959,23 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             if (s.be_down.data && (rc = upload_vector(c, s.be_down, (int64_t)ne * c->hidden, &L.be_down, "be_down")))
                 return fail(rc);
         }
-        const size_t kvb = (size_t)c->nkv * c->ctx_alloc * c->hd * 2;
+        // kv_cache.rs:122-131,194-198: a windowed layer may keep a ring of window + chunk positions
+        // instead of the whole context (position p in slot p % capacity); the slack beyond the window
+        // is what a rollback may take back (kv_cache_rewind.rs:26-35).  Here the chunk is two passes
+        // wide so that a pass can follow a rollback of a whole pass.
+        L.cap = c->ctx_alloc;
+        if (s.ring) {
+            if (s.window <= 0) {
+                set_error("open: only a layer with a sliding window can keep its cache as a ring");
+                return fail(TSV_ERR_INVALID);
+            }
+            const int ring_cap = ((s.window + 15) / 16) * 16 + 2 * TSV_MAX_ROWS;
+            if (ring_cap < c->ctx_alloc) {
+                L.cap = ring_cap;
+                c->rewind_budget = std::min<int64_t>(c->rewind_budget, ring_cap - s.window);
+            }
+        }
+        const size_t kvb = (size_t)c->nkv * L.cap * c->hd * 2;
         if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) return fail(rc);
         pneed = std::max(pneed, std::max(partial_need(L.qkv), partial_need(L.wo)));
         pneed = std::max(pneed, (size_t)8 * 16 * ((size_t)(qd + 2 * kvd) + TILE_ROWS));
@@ -871,6 +989,10 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         if ((rc = dev_alloc(c, &c->kv_ptrs, ptrs.size() * sizeof(uint16_t*)))) return fail(rc);
         if (hipMemcpy(c->kv_ptrs, ptrs.data(), ptrs.size() * sizeof(uint16_t*), hipMemcpyHostToDevice) != hipSuccess)
             return fail(TSV_ERR_DEVICE);
+        std::vector<int32_t> caps;
+        for (auto& L : c->layers) caps.push_back(L.cap);
+        if ((rc = dev_alloc(c, &c->kv_caps, caps.size() * 4))) return fail(rc);
+        if (hipMemcpy(c->kv_caps, caps.data(), caps.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail(TSV_ERR_DEVICE);
     }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
@@ -918,7 +1040,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->xf_b, xfb, true)) || (rc = dev_alloc(c, &c->xf_c, xfb, true)) ||
         (rc = dev_alloc(c, &c->partial, pneed * 4, true)) ||
         (c->max_experts &&
-         ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, 16 * 8 * 4, true)) ||
+         ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, true)) ||
           (rc = dev_alloc(c, &c->route_groups, (size_t)TSV_MAX_ROWS * 8 * sizeof(MoeGroup), true)) ||
           (rc = dev_alloc(c, &c->frag_e, (size_t)TSV_MAX_ROWS * 8 * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
           (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)))) || (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
@@ -946,14 +1068,21 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         // against 31 us for the three separate kernels -- the block is bandwidth-bound, and its
         // early bulk prefetch delays the small loads of the RMSNorm stage.
         const char* fe = getenv("TSV_FUSED");
-        bool ok = !c->use_graph && fe && fe[0] == '1';
-        int coop = 0, ncu = 0;
-        if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, 0) != hipSuccess) coop = 0;
+        const char* fa = getenv("TSV_FUSED_ATTN");
+        int ncu = 0;
         if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) ncu = 0;
-        ok = ok && coop && ncu == 256;
-        for (const LayerW& L : c->layers)
+        bool ok = !c->use_graph && fe && fe[0] == '1' && ncu == 256;
+        // the attention half of a layer as one kernel (attn_block.hip)
+        bool ok_attn = !c->use_graph && fa && fa[0] == '1' && ncu == 256;
+        for (const LayerW& L : c->layers) {
             ok = ok && L.n_experts == 0 && fused_ffn_supported(L.gate_up, L.down, c->hidden, c->ffn);
-        if (ok) {
+            ok_attn = ok_attn && L.n_experts == 0 && !L.v_only.tiles && !L.sinks && L.window == 0 &&
+                      attn_block_supported(L.qkv, L.wo, c->hidden, c->nq, c->nkv, c->hd, L.rope_fused);
+        }
+        c->fused_attn = ok_attn;
+        if (const char* e = getenv("TSV_FUSED_ATTN_STAGES")) c->attn_stages = std::max(2, std::min(5, atoi(e)));
+        if (ok_attn && (rc = dev_alloc(c, &c->partial8a, (size_t)8 * 16 * c->hidden * 4, true))) return fail(rc);
+        if (ok || ok_attn) {
             c->frag8_stride = (xfrag_bytes(c->hidden) + 255) & ~(size_t)255;
             if ((rc = dev_alloc(c, &c->x2, (size_t)16 * c->hidden * 4, true)) ||
                 (rc = dev_alloc(c, &c->frag8, 8 * c->frag8_stride, true)) ||
@@ -966,7 +1095,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
                 return fail(TSV_ERR_DEVICE);
             }
             *c->fused_err = 0;
-            c->fused_ffn = true;
+            c->fused_ffn = ok;
         }
     }
     if (hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
@@ -1050,13 +1179,14 @@ extern "C" void* tsv_stream(tsv_ctx* c) { return c ? (void*)c->stream : nullptr;
 extern "C" int32_t tsv_reset(tsv_ctx* c) {
     TSV_NEED(c, "reset: null handle");
     c->position = 0;
+    c->high_water = 0;
     c->last_m = 0;
     c->prefix.clear();  // cleared beside the cache it describes (real_forward_traits.rs:33-35)
     return TSV_OK;
 }
 
 extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c ? c->position : -1; }
-extern "C" int64_t tsv_max_safe_rewind(const tsv_ctx*) { return INT64_MAX; }  // linear layout: nothing rings
+extern "C" int64_t tsv_max_safe_rewind(const tsv_ctx* c) { return c ? c->rewind_budget : -1; }
 extern "C" const uint16_t* tsv_device_logits(tsv_ctx* c) { return c ? c->logits : nullptr; }
 extern "C" int64_t tsv_max_context(const tsv_ctx* c) { return c ? c->max_context : -1; }
 extern "C" int64_t tsv_vocab(const tsv_ctx* c) { return c ? c->vocab : -1; }
@@ -1135,6 +1265,7 @@ extern "C" int32_t tsv_rollback(tsv_ctx* c, const tsv_point* p) {
         set_error("rollback: point is ahead of the KV cursor");
         return TSV_ERR_INVALID;
     }
+    if (int rrc = check_rewind(c, p->position, "rollback")) return rrc;
     c->position = p->position;
     c->last_m = 0;  // the logits on the device no longer describe rows behind the cursor
     c->prefix.rewind_to(p->position);  // real_forward_rollback.rs:203
@@ -1147,6 +1278,7 @@ extern "C" int32_t tsv_rollback_retaining(tsv_ctx* c, const tsv_point* p, int32_
         set_error("rollback_retaining: keep_rows exceeds the rows the last verify wrote");
         return TSV_ERR_INVALID;
     }
+    if (int rrc = check_rewind(c, p->position + keep_rows, "rollback_retaining")) return rrc;
     c->position = p->position + keep_rows;
     c->last_m = 0;
     c->prefix.rewind_to(c->position);  // real_forward_rollback.rs:406
@@ -1195,7 +1327,7 @@ extern "C" int64_t tsv_try_reuse_prefix(tsv_ctx* c, const int32_t* prompt, int64
     if (keep == 0 || keep > c->position) return 0;
     const int64_t back = c->position - keep;
     if (back > 0) {
-        if (back > tsv_max_safe_rewind(c)) return 0;
+        if (c->rewind_budget != INT64_MAX && c->high_water - keep > c->rewind_budget) return 0;  // real_forward_traits.rs:241-262: as far as the cache can go back
         c->position = keep;
         c->prefix.rewind_to(keep);
     }
@@ -1231,7 +1363,7 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
     if (int frc = check_fused(c)) return frc;  // rows a fused kernel gave up on must not be gathered
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
-    return launch_kv_gather(c->stream, c->kv_ptrs, c->n_layers, c->nkv, c->hd, c->ctx_alloc, c->tok_dev + 32, n, (int)base);
+    return launch_kv_gather(c->stream, c->kv_ptrs, c->kv_caps, c->n_layers, c->nkv, c->hd, c->tok_dev + 32, n, (int)base);
 }
 
 namespace {
@@ -1460,7 +1592,13 @@ extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t 
         set_error("KV staging buffer: out of device memory");
         return TSV_ERR_DEVICE;
     }
-    int rc = launch_kv_read(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->ctx_alloc,
+    if (c->layers[layer].cap < c->ctx_alloc && pos0 < c->high_water - c->layers[layer].cap) {
+        (void)hipFree(kd);
+        (void)hipFree(vd);
+        set_error("read_kv: the ring of this layer no longer holds the first rows asked for");
+        return TSV_ERR_INVALID;
+    }
+    int rc = launch_kv_read(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->layers[layer].cap,
                             (int)pos0, (int)n, kd, vd);
     if (!rc) {
         hipError_t e1 = hipMemcpyAsync(k, kd, bytes, hipMemcpyDeviceToHost, c->stream);
@@ -1474,6 +1612,20 @@ extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t 
     (void)hipFree(kd);
     (void)hipFree(vd);
     return rc;
+}
+
+extern "C" int32_t tsv_route_selected(tsv_ctx* c, int32_t* out, int32_t n_layers) {
+    if (!c || !out || n_layers != c->n_layers) {
+        set_error("route_selected: null argument or layer count mismatch");
+        return TSV_ERR_INVALID;
+    }
+    if (!c->route_sel) {
+        set_error("route_selected: the model has no routed layers");
+        return TSV_ERR_INVALID;
+    }
+    TSV_HIP(hipMemcpyAsync(out, c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    return TSV_OK;
 }
 
 extern "C" int32_t tsv_write_logits(tsv_ctx* c, const uint16_t* logits, int32_t m, int64_t base) {
@@ -1508,9 +1660,14 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
         set_error("write_kv: copy failed");
         rc = TSV_ERR_DEVICE;
     }
-    if (!rc)
-        rc = launch_kv_fill(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->ctx_alloc, (int)pos0,
-                            (int)n, kd, vd);
+    if (!rc) {
+        // a ring layer keeps the last `cap` of the rows (earlier ones would only be overwritten, by
+        // rows of the same launch)
+        const int64_t cap = c->layers[layer].cap, skip = n > cap ? n - cap : 0;
+        const size_t off = (size_t)skip * c->nkv * c->hd;
+        rc = launch_kv_fill(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, (int)cap,
+                            (int)(pos0 + skip), (int)(n - skip), kd + off, vd + off);
+    }
     if (hipStreamSynchronize(c->stream) != hipSuccess && !rc) {
         set_error("write_kv: device execution failed");
         rc = TSV_ERR_DEVICE;
@@ -1518,6 +1675,7 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
     (void)hipFree(kd);
     (void)hipFree(vd);
     if (!rc && pos0 + n > c->position) c->position = pos0 + n;
+    if (!rc) c->high_water = std::max(c->high_water, pos0 + n);
     c->prefix.taint();  // rows no token ids describe
     return rc;
 }

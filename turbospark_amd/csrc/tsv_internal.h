@@ -6,6 +6,7 @@
 #include <string>
 
 #include "../../include/tsverify.h"
+#include "../../include/tsverify_testing.h"
 
 namespace tsv {
 
@@ -210,9 +211,18 @@ struct FfnBlockArgs {
     int down_tiles, down_kchunks;
     float* partial_out;  // [8][16][hidden]
 };
+// The per-XCD fused kernels are an experiment that measured slower than the separate kernels they
+// replace; they are compiled only when the library is built with TSV_WITH_FUSED (build.py:
+// TSV_BUILD_FUSED=1) and are opt-in at run time even then.
+#ifdef TSV_WITH_FUSED
 bool fused_ffn_supported(const TiledW& gate_up, const TiledW& down, int hidden, int ffn);
 int fused_ffn_barriers();
 int launch_ffn_block(hipStream_t s, int fmt, FfnBlockArgs& a, int m);
+#else
+inline bool fused_ffn_supported(const TiledW&, const TiledW&, int, int) { return false; }
+inline int fused_ffn_barriers() { return 0; }
+inline int launch_ffn_block(hipStream_t, int, FfnBlockArgs&, int) { return TSV_ERR_UNSUPPORTED; }
+#endif
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
                  const VerifyParams* vp, int m, const float* freqs = nullptr, float mscale = 1.0f, int half = 0,
@@ -247,7 +257,8 @@ struct AttnArgs {
     float* part_o;   // [nkv][nch][rows][hd]
     float* part_ml;  // [nkv][nch][rows][2]
     uint4* xfrag;    // output, K index = qh*hd + d
-    int nq, nkv, hd, max_ctx, nch;
+    int nq, nkv, hd, max_ctx, nch;  // max_ctx: positions the layer's cache holds
+    int ring;            // non-zero: the cache is a ring, position p in slot p % max_ctx (a windowed layer)
     float scale;
     int window;          // 0: full; else a row sees the last `window` positions of its sequence
     const float* sinks;  // nullable: one logit per q head joining the softmax maximum and denominator
@@ -257,9 +268,51 @@ struct AttnArgs {
     int m_hint, base_hint;
 };
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);
+int launch_attention_merge(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
 
-int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, int n_layers, int nkv, int hd, int max_ctx,
+// The attention half of a layer as one per-XCD kernel (attn_block.hip): residual add + RMSNorm
+// inputs, the q/k/v projection with its rotating epilogue, split-KV attention, the merge of the chunk
+// partials and the output projection; leaves one partial sum of the output projection per XCD.
+struct AttnBlockArgs {
+    FusedSync sync;
+    // residual add + norm inputs
+    const float* x_in;     // [16][hidden]
+    float* x_out;          // a different buffer: other XCDs may still be reading x_in
+    const float* partial;  // [n_partials][16][hidden] partial sums to add (n_partials <= 8)
+    int n_partials;
+    const float* bias_in;  // nullable: hidden values added with the partial sums
+    const float* norm_w;
+    uint8_t* frag;         // 8 private copies of the activation fragments, frag_stride bytes apart
+    size_t frag_stride;
+    float* ssq;            // [8][16][32] sums of squares per norm workgroup
+    int hidden;
+    float eps;
+    int m;
+    // q/k/v projection (the fused matrix of the rotating epilogue)
+    const uint8_t* w_qkv;
+    int qkv_kchunks;
+    RopeEpi rope;
+    const VerifyParams* vp;
+    // attention: q16, caches, partials, the output projection's input fragments, nch == 32
+    AttnArgs attn;
+    // output projection
+    const uint8_t* w_o;
+    int wo_tiles, wo_kchunks;
+    float* partial_out;  // [8][16][hidden]
+    int stages;          // 5: everything; 2: stop after the projection; 3: after attention; 4: after the merge
+};
+#ifdef TSV_WITH_FUSED
+bool attn_block_supported(const TiledW& qkv, const TiledW& wo, int hidden, int nq, int nkv, int hd, bool rope_fused);
+int attn_block_barriers();
+int launch_attn_block(hipStream_t s, int fmt, const AttnBlockArgs& a);
+#else
+inline bool attn_block_supported(const TiledW&, const TiledW&, int, int, int, int, bool) { return false; }
+inline int attn_block_barriers() { return 0; }
+inline int launch_attn_block(hipStream_t, int, const AttnBlockArgs&) { return TSV_ERR_UNSUPPORTED; }
+#endif
+
+int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, const int32_t* caps_dev, int n_layers, int nkv, int hd,
                      const int32_t* path_dev, int n, int base);
 int launch_kv_fill(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0, int n,
                    const uint16_t* k_in, const uint16_t* v_in);

@@ -1,4 +1,4 @@
-"""ctypes binding of include/tsverify.h."""
+"""ctypes binding of include/tsverify.h and include/tsverify_testing.h."""
 import ctypes as C
 import os
 
@@ -30,7 +30,7 @@ LAYER_GPTOSS_TENSORS = ("bq", "bk", "bv", "bo", "sinks", "router_bias", "be_gate
 class Layer(C.Structure):
     _fields_ = ([(n, Tensor) for n in LAYER_TENSORS] + [("n_experts", C.c_int32), ("top_k", C.c_int32)] +
                 [(n, Tensor) for n in LAYER_MOE_TENSORS] + [(n, Tensor) for n in LAYER_GPTOSS_TENSORS] +
-                [("window", C.c_int32), ("reserved", C.c_int32)])
+                [("window", C.c_int32), ("ring", C.c_int32)])
 
 
 class ModelDesc(C.Structure):
@@ -242,7 +242,7 @@ EXPORTS = [
     "tsv_prefix_rewind_to", "tsv_prefix_untainted_len", "tsv_prefix_common",
     "tsv_set_prefix_reuse", "tsv_try_reuse_prefix", "tsv_record_committed", "tsv_prefix_len",
     "tsv_gguf_open", "tsv_gguf_close", "tsv_gguf_tensor_count", "tsv_gguf_data_start", "tsv_gguf_tensor",
-    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf",
+    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected",
 ]
 
 _lib = None
@@ -292,6 +292,7 @@ def lib():
         L.tsv_verify_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
         L.tsv_compact_tree.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int32]
         L.tsv_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
+        L.tsv_route_selected.argtypes = [C.c_void_p, C.c_void_p, C.c_int32]
         L.tsv_accept_greedy_noalloc.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32,
                                                 C.c_int64, C.c_void_p, C.c_int32, C.c_uint64, C.c_uint64, C.c_void_p]
         L.tsv_verify_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]

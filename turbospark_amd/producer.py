@@ -44,6 +44,7 @@ class HipVerifier:
             self._layers[i].n_experts = int(lw.get("n_experts", 0))
             self._layers[i].top_k = int(lw.get("top_k", 0))
             self._layers[i].window = int(lw.get("window", 0))
+            self._layers[i].ring = int(bool(lw.get("ring", 0)))
         d = ffi.ModelDesc()
         d.n_layers = n
         for key in ("hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_context"):
@@ -121,7 +122,7 @@ class HipVerifier:
         return ffi.lib().tsv_device_logits(self._h)
 
     def max_safe_rewind(self):
-        """`KvCacheManager::max_safe_rewind`: unbounded (2**63 - 1), the cache is linear in every layer."""
+        """`KvCacheManager::max_safe_rewind`: rows a rollback may drop; 2**63 - 1 when no layer keeps a ring."""
         return ffi.lib().tsv_max_safe_rewind(self._h)
 
     @property
@@ -380,6 +381,14 @@ class HipVerifier:
             a = a.astype(np.float16).view(np.uint16)
         a = np.ascontiguousarray(a)
         ffi.check(ffi.lib().tsv_write_logits(self._h, a.ctypes.data, a.shape[0], int(base)))
+
+    def route_selected(self):
+        """[n_layers, 16, 8] expert ids every row of the last pass chose per routed layer, rank order
+        (the first top_k entries of a row are valid)."""
+        n = len(self._layers) if getattr(self, "_layers", None) is not None else self.cfg["n_layers"]
+        out = np.zeros((n, 16, 8), np.int32)
+        ffi.check(ffi.lib().tsv_route_selected(self._h, out.ctypes.data, n))
+        return out
 
     def read_kv(self, layer, pos0, n):
         c = self.cfg

@@ -44,12 +44,13 @@ CONFIGS = {
     # gpt-oss-120B shape (36 layers, 128 experts top-4, alternating 128-token window / full attention)
     "gptoss_120b": dict(n_layers=36, hidden=2880, n_q_heads=64, n_kv_heads=8, head_dim=64, ffn=2880,
                         n_experts=128, top_k=4, vocab=201088, rms_eps=1e-5, rope_theta=150000.0, attn_scale=0.125,
-                        dtype=ffi.BF16, expert_dtype=ffi.MXFP4, router_sigma=0.08,
+                        dtype=ffi.BF16, expert_dtype=ffi.MXFP4, router_sigma=0.02,  # "all random-init N(0, 0.02)"
                         gptoss=dict(window=128, yarn=(32.0, 4096, 32.0, 1.0), act_alpha=1.702, act_limit=7.0)),
     # Qwen3-30B-A3B shape: 128 experts, top-8, MXFP4 experts, Q8_0 attention / router / head
     "qwen3_30b_a3b": dict(n_layers=48, hidden=2048, n_q_heads=32, n_kv_heads=4, head_dim=128, ffn=768,
                           n_experts=128, top_k=8, vocab=151936, rms_eps=1e-6, rope_theta=1000000.0, qk_norm=True,
-                          dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=0.08),
+                          # router logits N(0, 1): the normalised input has unit mean square, so sigma = hidden ** -0.5
+                          dtype=ffi.Q8_0, expert_dtype=ffi.MXFP4, router_sigma=2048 ** -0.5),
     # Llama-3-8B shape
     "llama3_8b_q4_k": dict(n_layers=32, hidden=4096, n_q_heads=32, n_kv_heads=8, head_dim=128,
                            ffn=14336, vocab=128256, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K),
