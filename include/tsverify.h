@@ -298,6 +298,14 @@ typedef struct {
      * a prefix only when this is within one row of it (the drafter continuity guard of
      * real_forward_traits.rs:199-239); without it a run always starts from an empty state. */
     int64_t (*position)(void* user);
+    /* optional (0 / NULL: chain rounds only): a drafter that offers TREES (producer.rs:253-274).
+     * tree_nodes: nodes per tree round.  draft_tree(anchor, base, nodes, node_parent, tokens): a tree
+     * anchored at `anchor` (the token at `base`), parents before children; node_parent[i] is the index
+     * of the node under which node i hangs, -1 for a child of the anchor (DflashTreeNode::parent,
+     * dflash_tree.rs:12-17), tokens[i] its token.  A round is a tree round when it is greedy, the
+     * depth is fixed, nothing shortened it and tree_nodes == block (speculative.rs:386-392). */
+    int32_t tree_nodes;
+    int32_t (*draft_tree)(void* user, int32_t anchor, int64_t base, int32_t nodes, int32_t* node_parent, int32_t* tokens);
 } tsv_drafter;
 
 typedef struct {
@@ -322,7 +330,9 @@ typedef struct {
     int64_t reused;      /* leading prompt tokens taken over from the previous run's state */
 } tsv_generation_result;
 
-/* run_speculative for the step-wise drafter and chain rounds: admission, prefix reuse or reset
+/* run_speculative for the step-wise drafter: chain rounds, and greedy tree rounds (speculative.rs:
+ * 467-575: draft_tree -> verify_tree -> the walk -> compact_tree -> rollback_retaining, all of it but
+ * the draft inside one tsv_verify_accept) for a drafter that offers trees: admission, prefix reuse or reset
  * (speculative.rs:240-251), headless prefill that primes the drafter, then rounds of draft ->
  * verify + accept + truncate on the device -> record_committed -> rewind_drafter, never proposing
  * past the budget or the context window (speculative.rs:448-459). */

@@ -559,10 +559,17 @@ _CB_ROLL = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64, C.c_int)
 _CB_POS = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64)
 
 
+_CB_DRAFT_TREE = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int32, C.c_int64, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_int32))
+_CB_VERIFY_TREE = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.c_int, C.c_int64,
+                              C.POINTER(C.c_uint16))
+_CB_COMPACT = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64, C.POINTER(C.c_uint32), C.c_int)
+
+
 class Producer(C.Structure):
     _fields_ = [("user", C.c_void_p), ("reset", _CB_I), ("produce", _CB_PRODUCE), ("prefill", _CB_TOKPOS),
                 ("verify", _CB_VERIFY), ("rollback_retaining", _CB_ROLL), ("prime", _CB_TOKPOS),
-                ("step", _CB_PRODUCE), ("rewind", _CB_POS)]
+                ("step", _CB_PRODUCE), ("rewind", _CB_POS), ("tree_nodes", C.c_int),
+                ("draft_tree", _CB_DRAFT_TREE), ("verify_tree", _CB_VERIFY_TREE), ("compact_tree", _CB_COMPACT)]
 
 
 class Generation(C.Structure):
@@ -581,7 +588,9 @@ def run_speculative(target, drafter, prompt, cfg, max_new_tokens, block, vocab, 
     """The reference loop over Python producers.  `target` offers reset(), produce(token, pos) ->
     uint16[vocab], prefill(token, pos), verify(feed, base) -> uint16[m, vocab],
     rollback_retaining(point, keep_rows); `drafter` offers prime(next, pos), step(token, pos) ->
-    uint16[vocab], rewind(pos)."""
+    uint16[vocab], rewind(pos).  A drafter with `tree_nodes` > 0 also offers draft_tree(anchor, base,
+    nodes) -> (node parents, tokens), and the target then verify_tree(feed, slot_parents, base) and
+    compact_tree(base, path)."""
     def put(dst, arr, n):
         C.memmove(dst, np.ascontiguousarray(arr, np.uint16).ctypes.data, n * 2)
 
@@ -608,6 +617,19 @@ def run_speculative(target, drafter, prompt, cfg, max_new_tokens, block, vocab, 
     )
     prod = Producer(None, *[cbs[k] for k in ("reset", "produce", "prefill", "verify", "rollback_retaining",
                                              "prime", "step", "rewind")])
+    if getattr(drafter, "tree_nodes", 0):  # a drafter that offers trees (producer.rs:253-294)
+        def draft_tree(u, anchor, base, nodes, parent_out, tokens_out):
+            parent, tokens = drafter.draft_tree(anchor, base, nodes)
+            assert len(parent) == len(tokens) == nodes
+            for i in range(nodes):
+                parent_out[i], tokens_out[i] = int(parent[i]), int(tokens[i])
+
+        cbs["draft_tree"] = _CB_DRAFT_TREE(guard(draft_tree))
+        cbs["verify_tree"] = _CB_VERIFY_TREE(guard(lambda u, f, par, m, b, out: put(
+            out, target.verify_tree([f[i] for i in range(m)], [par[i] for i in range(m)], b), m * vocab)))
+        cbs["compact_tree"] = _CB_COMPACT(guard(lambda u, b, path, n: target.compact_tree(b, [path[i] for i in range(n)])))
+        prod.tree_nodes = int(drafter.tree_nodes)
+        prod.draft_tree, prod.verify_tree, prod.compact_tree = cbs["draft_tree"], cbs["verify_tree"], cbs["compact_tree"]
     g = Generation()
     g.shaping = cfg
     g.max_new_tokens = max_new_tokens

@@ -652,6 +652,61 @@ extern "C" int tso_run_speculative(const tso_producer* p, const int32_t* prompt,
             tso_set_error("round_block is 0: no room after admission; invariant violation");
             return -11;
         }
+        // :386-392, :467-575: a TREE round -- greedy, fixed depth, the full block, a producer that drafts
+        // trees of exactly `block` nodes.  The walk is the chain's acceptance generalised: at the current
+        // node's row the target's pick is accepted when a child of that node carries it.
+        if (p->draft_tree && p->tree_nodes == g->block && !sampled && round_block == g->block && !adaptive) {
+            const int nodes = p->tree_nodes;
+            std::vector<int32_t> node_parent((size_t)nodes), tokens((size_t)nodes), parents((size_t)nodes + 1);
+            if (p->draft_tree(p->user, next, base, nodes, node_parent.data(), tokens.data())) return -10;
+            parents[0] = -1;  // dflash_tree.rs:119-123: slot 0 is the anchor, node i sits at slot i + 1
+            for (int i = 0; i < nodes; i++) parents[(size_t)i + 1] = node_parent[(size_t)i] < 0 ? 0 : node_parent[(size_t)i] + 1;
+            feed.assign(1, next);
+            feed.insert(feed.end(), tokens.begin(), tokens.end());
+            const int64_t point = base;
+            if (p->verify_tree(p->user, feed.data(), parents.data(), (int)feed.size(), base, batch.data())) return -10;
+            out->rounds += 1;
+            out->offered += nodes;
+            std::vector<uint32_t> path(1, 0u);
+            int at = -1, stopped = 0;
+            int32_t bonus = -1;
+            for (;;) {
+                const int slot = at + 1;
+                int32_t target;
+                rc = select_token(batch.data() + (size_t)slot * vocab, vocab, cfg, sink.history.data(),
+                                  (int64_t)sink.history.size(), sink.generated, &target);
+                if (rc < 0) return rc;
+                int hit = -1;
+                for (int id = 0; id < nodes; id++)
+                    if (node_parent[(size_t)id] == at && tokens[(size_t)id] == target) {
+                        hit = id;
+                        break;
+                    }
+                if (hit < 0) {
+                    bonus = target;
+                    break;
+                }
+                path.push_back((uint32_t)hit + 1u);
+                at = hit;
+                const bool st = std::find(g->stop_tokens, g->stop_tokens + g->n_stop, target) != g->stop_tokens + g->n_stop;
+                if (!st) report(target);
+                if ((stopped = sink.commit(target))) break;
+            }
+            out->accepted += (int64_t)path.size() - 1;
+            const int committed = (int)((int64_t)sink.history.size() - (base + 1));
+            if (p->compact_tree(p->user, base, path.data(), committed + 1)) return -10;
+            if (committed + 1 < (int)feed.size()) {
+                out->rollbacks += 1;
+                if (p->rollback_retaining(p->user, point, committed + 1)) return -10;
+            }
+            if (p->rewind(p->user, base + committed)) return -10;
+            if (stopped) {
+                out->stop_reason = stopped;
+                break;
+            }
+            next = bonus;
+            continue;
+        }
         // :606-660
         proposals.clear();
         int32_t chained = next;

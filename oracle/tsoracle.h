@@ -220,6 +220,15 @@ typedef struct {
     int (*prime)(void* user, int32_t next_token, int64_t position);
     int (*step)(void* user, int32_t token, int64_t position, uint16_t* logits);
     int (*rewind)(void* user, int64_t position);
+    /* Tree rounds (producer.rs:253-294), all NULL / 0 for a producer that verifies chains only.
+     * tree_nodes: nodes per tree round; draft_tree fills node_parent[i] (the node index under which
+     * node i hangs, -1 for a child of the anchor; parents before children) and tokens[i];
+     * verify_tree takes slot parents (slot 0 = the anchor, node i at slot i + 1); compact_tree moves
+     * the accepted path's slots to rows 0 .. n. */
+    int tree_nodes;
+    int (*draft_tree)(void* user, int32_t anchor, int64_t base, int nodes, int32_t* node_parent, int32_t* tokens);
+    int (*verify_tree)(void* user, const int32_t* feed, const int32_t* parent, int m, int64_t base, uint16_t* logits);
+    int (*compact_tree)(void* user, int64_t base, const uint32_t* path, int n);
 } tso_producer;
 typedef struct {
     tso_shaping shaping;
@@ -235,7 +244,8 @@ typedef struct {
     int64_t rounds, offered, accepted, rollbacks;
     uint64_t draw_step;
 } tso_generation_result;
-/* crates/runtime/src/speculative.rs:194-900 for the step-wise drafter and chain rounds. */
+/* crates/runtime/src/speculative.rs:194-900 for the step-wise drafter: chain rounds, and greedy tree
+ * rounds (:467-575) when the producer drafts trees of `block` nodes and the depth is fixed. */
 int tso_run_speculative(const tso_producer* p, const int32_t* prompt, int64_t n_prompt,
                         const tso_generation* g, int64_t max_context, int64_t vocab,
                         tso_generation_result* out);

@@ -7,7 +7,7 @@ import pytest
 
 from oracle import binding as ob
 from tests import gpu_common as gc
-from tests.loop_common import GpuTarget, LmDrafter
+from tests.loop_common import GpuTarget, LmDrafter, TreeTwinDrafter
 
 pytestmark = pytest.mark.gpu
 
@@ -170,3 +170,41 @@ def test_a_drafter_that_leaves_its_logits_on_the_device(temperature, kw):
     dev = gpu.run_speculative(prompt, DeviceLmDrafter(GpuTarget(lm), prompt[0], V), gcfg, 40, 5, device_logits=True)
     assert {k: dev[k] for k in KEYS} == {k: host[k] for k in KEYS}
     assert len(dev["tokens"]) == 40
+
+
+@pytest.mark.parametrize("nodes,stop_at", [(7, None), (15, None), (7, 30)])
+def test_tree_rounds_in_the_loop_report_what_the_reference_loop_reports(nodes, stop_at):
+    """speculative.rs:467-575: greedy, fixed-depth rounds of a drafter that offers trees of `block` nodes
+    run as draft_tree -> verify_tree -> the walk -> compact_tree -> rollback_retaining.  The library does
+    everything after the draft in one device round; the oracle's restatement drives the same GPU target
+    through verify_tree / compact_tree with the walk on the host.  Tokens, stop reason and every counter
+    agree, the output is plain greedy decoding, and rounds that the budget shortens fall back to chains."""
+    import turbospark_amd as ts
+    cfg, gpu, lm = _pair()
+    V = cfg["vocab"]
+    prompt = np.random.default_rng(5).integers(0, V, 11).astype(np.int32)
+    new = 60
+
+    def drafter():
+        return TreeTwinDrafter(GpuTarget(lm), prompt[0], V, nodes, seed=2)
+
+    plain = gpu.run_speculative(prompt, LmDrafter(GpuTarget(lm), prompt[0], V), ts.shaping(0.0), new, 4)["tokens"]
+    stops = [plain[stop_at]] if stop_at is not None else []
+    want = ob.run_speculative(GpuTarget(gpu), drafter(), prompt, ob.shaping(0.0), new, nodes, V, cfg["max_context"],
+                              stop_tokens=stops)
+    got = gpu.run_speculative(prompt, drafter(), ts.shaping(0.0), new, nodes, stop_tokens=stops)
+    print({k: (got[k] if k != "tokens" else len(got[k])) for k in KEYS})
+    assert {k: got[k] for k in KEYS} == {k: want[k] for k in KEYS}
+    if stops:
+        cut = plain.index(stops[0])
+        assert got["tokens"] == plain[:cut] and got["stop_reason"] == 1
+    else:
+        assert got["tokens"] == plain and got["stop_reason"] == 2
+        assert got["kv_position"] == len(prompt) + new - 1 == gpu.position
+    assert 0 < got["accepted"] < got["offered"] and got["rollbacks"] > 0
+    # the next token after the run continues from a cache that only ever kept accepted paths
+    if not stops:
+        nxt = gpu.produce(got["tokens"][-1], gpu.position)
+        gpu.reset()
+        gpu.prefill(np.concatenate([prompt, np.array(got["tokens"][:-1], np.int32)]), 0, want_logits=False)
+        assert gc.logit_error(nxt[None], gpu.produce(got["tokens"][-1], gpu.position)[None]) <= 2e-3

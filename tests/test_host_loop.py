@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from oracle import binding as ob
-from tests.loop_common import LmDrafter, OracleTarget
+from tests.loop_common import LmDrafter, OracleTarget, TreeTwinDrafter
 
 
 def _oracle_adaptive(floor, cap):
@@ -194,6 +194,33 @@ def test_greedy_speculation_equals_plain_greedy_decoding(seed_draft, block, floo
     got = ob.run_speculative(OracleTarget(target), drafter, prompt, ob.shaping(0.0), 40, block, cfg["vocab"],
                              cfg["max_context"], stop_tokens=[stop], adaptive_floor=floor)
     assert got["tokens"] == want[:first] and got["stop_reason"] == 1
+
+
+@pytest.mark.parametrize("nodes", [7, 15])
+def test_greedy_tree_rounds_equal_plain_greedy_decoding(nodes):
+    """speculative.rs:467-575: a drafter that offers trees of `block` nodes; the walk accepts the child
+    that carries the target's pick, the accepted path is compacted, and what is reported is plain
+    greedy decoding whatever the tree held.  The tree hides the true continuation behind junk siblings
+    and cuts it at a seeded depth, so rounds accept anything from nothing to five nodes."""
+    cfg, target, lm = _models(seed_draft=None)
+    prompt = np.random.default_rng(2).integers(0, cfg["vocab"], 9).astype(np.int32)
+    want, why = _plain_greedy(target, prompt, 40)
+    drafter = TreeTwinDrafter(OracleTarget(lm), prompt[0], cfg["vocab"], nodes, seed=4)
+    got = ob.run_speculative(OracleTarget(target), drafter, prompt, ob.shaping(0.0), 40, nodes, cfg["vocab"], cfg["max_context"])
+    assert got["tokens"] == want and got["stop_reason"] == 2 == why
+    assert target.position == len(prompt) + 39
+    assert 0 < got["accepted"] < got["offered"] and got["rollbacks"] > 0 and got["rounds"] < 40
+    stop = want[21]
+    drafter = TreeTwinDrafter(OracleTarget(lm), prompt[0], cfg["vocab"], nodes, seed=4)
+    got = ob.run_speculative(OracleTarget(target), drafter, prompt, ob.shaping(0.0), 40, nodes, cfg["vocab"], cfg["max_context"],
+                             stop_tokens=[stop])
+    assert got["tokens"] == want[:want.index(stop)] and got["stop_reason"] == 1
+    # an adaptive run keeps the chain (speculative.rs:390-392): the drafter is then stepped, never asked for a tree
+    drafter = TreeTwinDrafter(OracleTarget(lm), prompt[0], cfg["vocab"], nodes, seed=4)
+    drafter.draft_tree = None
+    got = ob.run_speculative(OracleTarget(target), drafter, prompt, ob.shaping(0.0), 40, nodes, cfg["vocab"], cfg["max_context"],
+                             adaptive_floor=2)
+    assert got["tokens"] == want
 
 
 def test_the_loop_fills_the_context_window_exactly_and_refuses_past_it():

@@ -220,6 +220,64 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
             set_error("run_speculative: round_block is 0: no room after admission; invariant violation");
             return TSV_ERR_INVALID;
         }
+        // speculative.rs:386-392, 467-575: a TREE round -- greedy, fixed depth, the full block, a drafter
+        // whose trees have exactly `block` nodes.  Verify, the walk (at the current node's row the
+        // target's pick is accepted when a child of that node carries it), the compaction of the
+        // accepted path and the truncation are one tsv_verify_accept.
+        if (dr->draft_tree && dr->tree_nodes == g->block && !sampled && round_block == g->block && !adaptive) {
+            const int nodes = dr->tree_nodes;
+            int32_t node_parent[TSV_MAX_ROWS], parents[TSV_MAX_ROWS];
+            feed[0] = next;
+            if (dr->draft_tree(dr->user, next, base, nodes, node_parent, feed + 1)) {
+                set_error("run_speculative: draft_tree failed");
+                return TSV_ERR_INVALID;
+            }
+            parents[0] = -1;  // dflash_tree.rs:119-123: slot 0 is the anchor, node i sits at slot i + 1
+            for (int i = 0; i < nodes; i++) {
+                if (node_parent[i] < -1 || node_parent[i] >= i) {
+                    set_error("run_speculative: draft_tree must list parents before children");
+                    return TSV_ERR_INVALID;
+                }
+                parents[i + 1] = node_parent[i] < 0 ? 0 : node_parent[i] + 1;
+            }
+            tsv_round r{};
+            r.feed = feed;
+            r.parent = parents;
+            r.m = nodes + 1;
+            r.base = base;
+            r.shaping = g->shaping;
+            r.draw_step = draw_step;
+            r.stop_tokens = g->stop_tokens;
+            r.n_stop = g->n_stop;
+            r.generated = generated;
+            r.max_new_tokens = g->max_new_tokens;
+            tsv_round_result res{};
+            if ((rc = tsv_verify_accept(c, &r, &res))) return rc;
+            out->rounds += 1;
+            out->offered += nodes;
+            out->accepted += res.accepted;
+            if (res.committed < nodes) out->rollbacks += 1;
+            int32_t path_feed[TSV_MAX_ROWS + 1];
+            for (int i = 0; i <= res.committed; i++) path_feed[i] = feed[res.path[i]];
+            for (int i = 1; i <= res.committed; i++)
+                if ((rc = emit.push(path_feed[i]))) return rc;
+            // the budget's last token is reported: the node the walk accepted last
+            if (res.stopped == 2 && (rc = emit.push(feed[res.path[res.committed + 1]]))) return rc;
+            generated += (uint64_t)res.accepted;
+            history += res.committed;
+            hist.insert(hist.end(), path_feed + 1, path_feed + 1 + res.committed);
+            if ((rc = tsv_record_committed(c, path_feed, res.committed + 1, base))) return rc;
+            if (dr->rewind(dr->user, base + res.committed)) {
+                set_error("run_speculative: rewind_drafter failed");
+                return TSV_ERR_INVALID;
+            }
+            if (res.stopped) {
+                out->stop_reason = res.stopped;
+                break;
+            }
+            next = res.next;
+            continue;
+        }
         // draft: block steps, each proposal drawn from the drafter's own distribution (or its
         // arg-max), then the row-only step that primes the drafter with the last proposal
         feed[0] = next;

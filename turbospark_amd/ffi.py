@@ -190,9 +190,13 @@ DRAFT_REWIND = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int64)
 DRAFT_POSITION = C.CFUNCTYPE(C.c_int64, C.c_void_p)
 
 
+DRAFT_TREE = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32))
+
+
 class Drafter(C.Structure):
     _fields_ = [("user", C.c_void_p), ("prime", DRAFT_PRIME), ("step", DRAFT_STEP), ("rewind", DRAFT_REWIND),
-                ("device_logits", C.c_int32), ("position", DRAFT_POSITION)]
+                ("device_logits", C.c_int32), ("position", DRAFT_POSITION), ("tree_nodes", C.c_int32),
+                ("draft_tree", DRAFT_TREE)]
 
 
 class Generation(C.Structure):

@@ -327,6 +327,19 @@ class HipVerifier:
                     failure.append(e)
                     return -1
             d.position = ffi.DRAFT_POSITION(where)
+        if getattr(drafter, "tree_nodes", 0):  # a drafter that offers trees: draft_tree(anchor, base, nodes) -> (parents, tokens)
+            def draft_tree(user, anchor, base, nodes, parent_out, tokens_out):
+                try:
+                    parent, tokens = drafter.draft_tree(anchor, base, nodes)
+                    assert len(parent) == len(tokens) == nodes
+                    for i in range(nodes):
+                        parent_out[i], tokens_out[i] = int(parent[i]), int(tokens[i])
+                    return 0
+                except Exception as e:
+                    failure.append(e)
+                    return 1
+            d.tree_nodes = int(drafter.tree_nodes)
+            d.draft_tree = ffi.DRAFT_TREE(draft_tree)
         g = ffi.Generation()
         g.shaping = cfg
         g.max_new_tokens = int(max_new_tokens)
