@@ -8,8 +8,9 @@ Reads files below /root/reference as text / data only (nothing is imported or ru
   * the hand-packed Q4_K superblock constants of crates/compute/tests/quant_gguf.rs:226-267
     -> q4k_handpacked.json
   * the llama-3 rope factor profile of crates/compute/src/rope.rs:471-482 -> llama3_rope_profile.json
-  * three MLX known-answer fixtures (config.json, model.safetensors, traces.json) of
-    crates/audio/testdata/lm/{llama_default,llama_llama3_rope,qwen3_default}  -> lm/<name>/
+  * five MLX known-answer fixtures (config.json, model.safetensors, traces.json) of
+    crates/audio/testdata/lm/{llama_default,llama_llama3_rope,qwen3_default,llama_yarn_rope,qwen2_default}
+    -> lm/<name>/
 
 Run once in the authoring container:  python tests/golden/make_fixtures.py
 The outputs are committed; tests never read /root/reference.
@@ -80,7 +81,7 @@ def main():
         open(f"{OUT}/llama3_rope_profile.json", "w"),
     )
 
-    for name in ["llama_default", "llama_llama3_rope", "qwen3_default"]:
+    for name in ["llama_default", "llama_llama3_rope", "qwen3_default", "llama_yarn_rope", "qwen2_default"]:
         dst = f"{OUT}/lm/{name}"
         os.makedirs(dst, exist_ok=True)
         for f in ["config.json", "model.safetensors", "traces.json"]:

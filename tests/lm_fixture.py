@@ -29,11 +29,15 @@ def load(golden_dir, name, max_context=64):
                vocab=conf["vocab_size"], max_context=max_context, rms_eps=conf["rms_norm_eps"],
                rope_theta=conf["rope_theta"])
     rs = conf.get("rope_scaling")
-    if rs:
-        assert rs["type"] == "llama3"
+    if rs and rs["type"] == "llama3":
         cfg["rope_factors"] = ob.llama3_rope_factors(hd, conf["rope_theta"], rs["factor"],
                                                      rs["low_freq_factor"], rs["high_freq_factor"],
                                                      rs["original_max_position_embeddings"])
+    elif rs:
+        # YaRN (crates/compute/src/rope.rs:324-372): a per-pair frequency table and a magnitude scale
+        assert rs["type"] == "yarn" and rs.get("mscale", 1.0) == 1.0 and rs.get("mscale_all_dim", 0.0) == 0.0
+        cfg["rope_freqs"], cfg["rope_mscale"] = ob.yarn_frequencies(
+            hd, conf["rope_theta"], rs["factor"], rs["original_max_position_embeddings"], rs["beta_fast"], rs["beta_slow"])
     layers = []
     for i in range(cfg["n_layers"]):
         p = f"model.layers.{i}."
@@ -43,6 +47,9 @@ def load(golden_dir, name, max_context=64):
                   ffn_norm=_t(st[p + "post_attention_layernorm.weight"]),
                   w_gate=_t(st[p + "mlp.gate_proj.weight"]), w_up=_t(st[p + "mlp.up_proj.weight"]),
                   w_down=_t(st[p + "mlp.down_proj.weight"]))
+        if p + "self_attn.q_proj.bias" in st:  # qwen2: biases on the q / k / v projections, added before the rotation
+            lw.update(bq=_t(st[p + "self_attn.q_proj.bias"]), bk=_t(st[p + "self_attn.k_proj.bias"]),
+                      bv=_t(st[p + "self_attn.v_proj.bias"]))
         if p + "self_attn.q_norm.weight" in st:
             lw["q_norm"] = _t(st[p + "self_attn.q_norm.weight"])
             lw["k_norm"] = _t(st[p + "self_attn.k_norm.weight"])

@@ -91,3 +91,51 @@ def test_files_the_intake_cannot_express_are_refused_by_name(tmp_path):
         gw.write_gguf = orig
     with pytest.raises(ffi.TsvError, match="rope scaling 'yarn'"):
         ts.HipVerifier.from_gguf(path)
+
+
+@pytest.mark.parametrize("name,arch,permute,tol", [
+    ("tiny_q8_0", "llama", True, 2e-3),
+    ("small_q4_k_m", "llama", True, 1e-2),
+    ("moe_small", "qwen3moe", False, 1e-2),
+    ("gptoss_small", "gpt-oss", False, 1e-2),
+])
+def test_a_gguf_target_agrees_with_the_oracle_reading_the_same_file(tmp_path, name, arch, permute, tol):
+    """The engine opened by tsv_open_gguf against the ORACLE fed by an independent reader of the same file
+    (tests/gguf_reader.py: header, tensor table, the names of gguf_names/llama.rs:14-60 and
+    gpt_oss.rs:30-72, the q / k row un-permutation of conventions.rs:133-151, the YaRN keys): two readings
+    of one file that share no code, so a name, a size or a row order taken wrongly by either shows up as
+    a logit error.  (The file itself is laid out by this project's writer: no GGUF ships with the reference.)"""
+    from oracle import binding as ob
+    from tests import gguf_reader
+    from tests import gpu_common as gc
+    cfg = dict(synth.CONFIGS[name], max_context=96)
+    w = synth.make_weights(cfg, seed=4321)
+    path = os.path.join(tmp_path, f"{name}.gguf")
+    llama_gguf(path, cfg, w, arch=arch, permute=permute)
+    filed = ts.HipVerifier.from_gguf(path)
+    ocfg, ow = gguf_reader.load_model(path, max_context=96)
+    for key in ("n_layers", "hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab"):
+        assert ocfg[key] == cfg[key], key
+    cpu = ob.Model(ocfg, ow, round_kv_f16=True, threads=8)
+    for attempt in range(20):
+        rng = np.random.default_rng(8 + attempt)
+        prompt = rng.integers(0, cfg["vocab"], 37).astype(np.int32)
+        feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+        cpu.reset()
+        margins = []
+        for i in range(0, 37, 16):
+            cpu.verify(prompt[i:i + 16], i)
+            margins.append(cpu.route_margin)
+        want = cpu.verify(feed, 37)
+        margins.append(cpu.route_margin)
+        if min(margins) > 1e-3:        # (routed models: a prompt without a near-tie routing decision)
+            break
+    filed.prefill(prompt, 0, want_logits=False)
+    got = filed.verify(feed, 37)
+    err = gc.logit_error(got, want)
+    print(f"{name} from GGUF: GPU engine vs oracle over an independent reader, max-abs / range = {err:.2e}")
+    assert err <= tol
+    for layer in range(cfg["n_layers"]):
+        kg, vg = filed.read_kv(layer, 0, 42)
+        kc, vc = cpu.kv(layer)
+        assert np.abs(kg.astype(np.float32) - kc[:42]).max() <= 2e-2 * np.abs(kc[:42]).max()

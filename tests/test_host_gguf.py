@@ -198,3 +198,32 @@ def test_the_references_own_fixture_scenario(tmp_path):
                                  30: (1, 2), 39: (32, 17)}.items():
         assert ffi.row_bytes(tid, 256) == 256 // elems * nbytes, tid
     g.close()
+
+
+def test_the_independent_reader_recovers_what_the_writer_was_given(tmp_path):
+    """tests/gguf_reader.py (the oracle side of the GGUF parity tests) against tests/gguf_writer.py: every
+    tensor of a llama file (q / k rows permuted by the converter and un-permuted by the reader,
+    conventions.rs:133-151), a routed qwen3moe file and a gpt-oss file comes back byte for byte under the
+    names of gguf_names/llama.rs:14-60 and gpt_oss.rs:30-72, with the sizes read from the metadata."""
+    from tests import gguf_reader
+    from tests.gguf_writer import llama_gguf
+    from turbospark_amd import synth
+    for name, arch, permute in [("tiny_q8_0", "llama", True), ("moe_small", "qwen3moe", False), ("gptoss_small", "gpt-oss", False)]:
+        cfg = dict(synth.CONFIGS[name], max_context=96)
+        w = synth.make_weights(cfg, seed=4321)
+        path = os.path.join(tmp_path, name + ".gguf")
+        llama_gguf(path, cfg, w, arch=arch, permute=permute)
+        ocfg, ow = gguf_reader.load_model(path, 96)
+        for key in ("n_layers", "hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab"):
+            assert ocfg[key] == cfg[key], (name, key)
+        for a, b in zip(w["layers"], ow["layers"]):
+            for k, v in a.items():
+                if isinstance(v, tuple):
+                    assert v[0] == b[k][0] and v[2:] == b[k][2:], (name, k)
+                    assert np.array_equal(np.asarray(v[1]).reshape(-1), np.asarray(b[k][1]).reshape(-1)), (name, k)
+                elif k in ("n_experts", "top_k", "window"):
+                    assert b.get(k, 0) == v, (name, k)
+        for k in ("embed", "final_norm", "lm_head"):
+            assert np.array_equal(np.asarray(w[k][1]).reshape(-1), np.asarray(ow[k][1]).reshape(-1)), (name, k)
+        if arch == "gpt-oss":
+            assert np.allclose(ocfg["rope_freqs"], cfg["rope_freqs"]) and abs(ocfg["rope_mscale"] - cfg["rope_mscale"]) < 1e-7

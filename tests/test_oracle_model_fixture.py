@@ -2,7 +2,8 @@
 
 The fixtures (crates/audio/testdata/lm/*, tolerance 2e-4 at crates/audio/src/lm/tests.rs:70-71)
 are the only in-tree absolute logits for this graph.  They pin op order, NeoX rope, GQA head
-mapping, llama-3 rope scaling and per-head q/k norm -- and, because the decode tokens are also
+mapping, llama-3 rope scaling, the YaRN frequency table and magnitude scale, the q / k / v
+projection biases and per-head q/k norm -- and, because the decode tokens are also
 fed as ONE batched verify over the prefill's cache, that a verify pass equals sequential decode.
 """
 import numpy as np
@@ -14,7 +15,7 @@ from tests import lm_fixture
 TOL = 2e-4
 
 
-@pytest.mark.parametrize("name", ["llama_default", "llama_llama3_rope", "qwen3_default"])
+@pytest.mark.parametrize("name", ["llama_default", "llama_llama3_rope", "qwen3_default", "llama_yarn_rope", "qwen2_default"])
 def test_forward_matches_mlx_traces(golden, name):
     cfg, weights, tr = lm_fixture.load(golden, name)
     tokens, dec = tr["tokens"], tr["decode_tokens"]
