@@ -237,7 +237,7 @@ def test_qwen3_30b_a3b_shape_two_layers_at_long_context():
     ctx = 3000
     cfg, gpu, cpu = _filled("qwen3_30b_a3b", ctx, 2)
     V = cfg["vocab"]
-    for attempt in range(8):
+    for attempt in range(40):
         rng = np.random.default_rng(40 + attempt)
         # proposals: the oracle's own greedy continuation for three tokens, then junk
         toks = [int(rng.integers(0, V))]
@@ -251,7 +251,9 @@ def test_qwen3_30b_a3b_shape_two_layers_at_long_context():
         cpu.rewind_to(ctx)
         want = cpu.verify(feed, ctx)
         margins.append(cpu.route_margin)
-        if min(margins) > 2e-3:
+        # the GPU's router logits carry about 1e-4 of the logit range in fp16 rounding (the largest margin
+        # at which a decision was seen to differ from the oracle's at this router shape: 1.4e-4)
+        if min(margins) > 1e-3:
             break
     else:
         raise AssertionError("no feed without a near-tie routing decision")

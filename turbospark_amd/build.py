@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
-SOURCES = ["gemm.hip", "moe.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
+SOURCES = ["gemm.hip", "moe.hip", "moe_fp4.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
 # The per-XCD fused layer kernels (an experiment that measured slower than the kernels it replaces) are
 # built only on request: TSV_BUILD_FUSED=1.
 WITH_FUSED = os.environ.get("TSV_BUILD_FUSED", "0") == "1"
@@ -18,7 +18,8 @@ OPT = {"host_utils.hip": "-O2", "gguf.hip": "-O2"}
 EXTRA = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_GEMM_DEFS", "").split(),
          "fused.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),
          "attn_block.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),
-         "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+         "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+         "moe_fp4.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 FLAGS = [
     "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # no implicit multiply-add fusion: the compiler picks the fused operand per template instantiation, and

@@ -74,7 +74,7 @@ __device__ __forceinline__ void norm_stage(const AttnBlockArgs& a, int xcc, int 
                     if (s < a.n_partials) xv = __fadd_rn(xv, part[j][s]);
                 if (a.bias_in) xv += a.bias_in[col];
                 if (xcc == 0) a.x_out[(size_t)b * a.hidden + col] = xv;
-                const _Float16 h = (_Float16)(xv * wn[j]);
+                const _Float16 h = pinned_half((_Float16)(xv * wn[j]));
                 frag[frag_index(col, b)] = h;
                 float sum = (float)h;
 #pragma unroll

@@ -64,7 +64,7 @@ __device__ __forceinline__ void norm_inputs(const NormStage& n, const XcdCtx& c,
                 for (int s = 0; s < 8; s++)
                     if (s < n.n_partials) xv += part[j][s];
                 if (c.xcc == 0) n.x_out[(size_t)b * n.hidden + col] = xv;
-                const _Float16 h = (_Float16)(xv * wn[j]);
+                const _Float16 h = pinned_half((_Float16)(xv * wn[j]));
                 frag[frag_index(col, b)] = h;
                 float sum = (float)h;
 #pragma unroll
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(512) void k_ffn_block(FfnBlockArgs a) {
                     const float sv = v[i] * s_inv[b];
                     const float other = __shfl_xor(sv, 32);
                     const float gate = lane < 32 ? sv : other, up = lane < 32 ? other : sv;
-                    const _Float16 h = (_Float16)(silu_f(gate) * up);
+                    const _Float16 h = pinned_half((_Float16)(silu_f(gate) * up));
                     float sum = (float)h;
 #pragma unroll
                     for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);

@@ -263,7 +263,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split,
         for (int i = 0; i < 4; i++) {
             const float other = __shfl_xor(v[i], 32);
             const float gate = lane < 32 ? v[i] : other, up = lane < 32 ? other : v[i];
-            const _Float16 h = (_Float16)(silu_f(gate) * up);
+            const _Float16 h = pinned_half((_Float16)(silu_f(gate) * up));
             float sum = (float)h;
 #pragma unroll
             for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
@@ -465,7 +465,7 @@ __device__ __forceinline__ void epilogue16(const GemmArgs& a, int tile, int spli
         _Float16* out = (_Float16*)a.out;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const _Float16 h = (_Float16)(silu_f(v0[i]) * v1[i]);
+            const _Float16 h = pinned_half((_Float16)(silu_f(v0[i]) * v1[i]));
             float sum = (float)h;
 #pragma unroll
             for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o);

@@ -3,6 +3,7 @@
 #include <type_traits>
 
 #include "tsv_internal.h"
+#include "x8.h"
 
 namespace tsv {
 
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
                                                   int splits, int ldp, const float* __restrict__ w,
                                                   float eps, int hidden, _Float16* __restrict__ xfrag,
                                                   const float* __restrict__ weights,
-                                                  const float* __restrict__ bias) {
+                                                  const float* __restrict__ bias, X8 x8, int x8_terms) {
     __shared__ float red[16];
     const int m = blockIdx.x;
     float4* xr = (float4*)(x + (long)m * hidden);
@@ -197,25 +198,49 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
         const float4 v = first ? v_first : xr[i], g = first ? g_first : wr[i];
         // elements 4i..4i+3 are one K step of the fragment layout, stored in the order (0, 2, 1, 3)
         typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+        typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
         half4 h = {(_Float16)(v.x * g.x * inv), (_Float16)(v.z * g.z * inv), (_Float16)(v.y * g.y * inv),
                    (_Float16)(v.w * g.w * inv)};
+        // The sums must be those of the stored bits: the matmuls multiply them by the weights' code offsets
+        // (up to 1024), so one value rounded differently on the way to the sum than on the way to the store
+        // is an error a thousand times its size.  The compiler is free to convert the same product twice, by
+        // different instructions; pinning the packed halves in registers leaves it one copy to read.
+        u32x2_t hb = __builtin_bit_cast(u32x2_t, h);
+        asm volatile("" : "+v"(hb.x), "+v"(hb.y));
+        h = __builtin_bit_cast(half4, hb);
         *(half4*)(xfrag + frag_index(4 * i, m)) = h;
         float sum = ((float)h.x + (float)h.y) + ((float)h.z + (float)h.w);
         sum += __shfl_xor(sum, 1);
         sum += __shfl_xor(sum, 2);
         sum += __shfl_xor(sum, 4);
         if ((i & 7) == 0) sums[xsum_index(i >> 3, m)] = sum;
+        if (x8_terms) {
+            // the same row as block-scaled fp8 terms, from the unrounded values; the eight threads of a
+            // 32-element block are neighbours in one wave (hidden is a multiple of 32)
+            float r[4] = {v.x * g.x * inv, v.z * g.z * inv, v.y * g.y * inv, v.w * g.w * inv};
+            for (int t = 0; t < x8_terms; t++) {
+                float amax = x8_amax4(r);
+                amax = fmaxf(amax, __shfl_xor(amax, 1));
+                amax = fmaxf(amax, __shfl_xor(amax, 2));
+                amax = fmaxf(amax, __shfl_xor(amax, 4));
+                const int byte = x8_scale_byte(amax);
+                const uint32_t word = x8_term4(r, byte);
+                *(uint32_t*)(x8.q + ((size_t)t * 16 + m) * x8.kpad + 4 * i) = word;
+                if ((i & 7) == 0) x8.s[((size_t)t * 16 + m) * (x8.kpad >> 5) + (i >> 3)] = (uint8_t)byte;
+            }
+        }
     }
 }
 
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
-                   float eps, int hidden, uint4* xfrag, int m, const float* weights, const float* bias) {
+                   float eps, int hidden, uint4* xfrag, int m, const float* weights, const float* bias, const X8* x8,
+                   int x8_terms) {
     if (splits < 0 || splits > 8) {
         set_error("residual add: at most eight partial sums");
         return TSV_ERR_UNSUPPORTED;
     }
     hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
-                       (_Float16*)xfrag, weights, bias);
+                       (_Float16*)xfrag, weights, bias, x8 ? *x8 : X8{}, x8 ? x8_terms : 0);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -224,7 +249,7 @@ __global__ void k_f32_to_xfrag(const float* __restrict__ x, int k, _Float16* __r
     const int m = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= k) return;  // k is a multiple of 32: whole sub-blocks leave together
-    const _Float16 h = (_Float16)x[(long)m * k + i];
+    const _Float16 h = pinned_half((_Float16)x[(long)m * k + i]);
     xfrag[frag_index(i, m)] = h;
     float sum = (float)h;
     for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);

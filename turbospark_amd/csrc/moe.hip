@@ -62,27 +62,41 @@ __device__ __forceinline__ float key_value(uint32_t key) {
 }
 
 __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
-    __shared__ int s_sel[TSV_MAX_ROWS * 8];    // the selected experts, pair index = row * k + slot
+    __shared__ int s_sel[TSV_MAX_ROWS * 8];  // the selected experts, pair index = row * k + slot
+    __shared__ uint32_t s_mask[256 * 4];     // per expert: which of the (at most 128) pairs chose it
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int M = a.m, ne = a.n_experts, k = a.top_k;
+    for (int i = threadIdx.x; i < ne * 4; i += blockDim.x) s_mask[i] = 0;
+    __syncthreads();
     if (wave < M) {
         const int m = wave;
-        uint32_t key[4];
+        uint32_t key[4] = {0u, 0u, 0u, 0u};
+        // every partial sum of every expert this lane holds is asked for before the first add: the loads
+        // have no branch between them (a lane past the last expert reads the last expert's, a split past
+        // the last split the last split's again), so they are one round trip, not one per expert block
+        auto gather = [&](auto NJ) {
+            constexpr int nj = decltype(NJ)::value;
+            float part[nj][8], bias[nj];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int e = lane + 64 * j;
-            key[j] = 0;
-            if (e < ne) {
-                float part[8], s = 0.f;  // all partials in flight together, added in split order
+            for (int j = 0; j < nj; j++) {
+                const int e = min(lane + 64 * j, ne - 1);
 #pragma unroll
-                for (int sp = 0; sp < 8; sp++) part[sp] = a.logits[((size_t)min(sp, a.splits - 1) * 16 + m) * a.ld + e];
-#pragma unroll
-                for (int sp = 0; sp < 8; sp++)
-                    if (sp < a.splits) s += part[sp];
-                if (a.bias) s += a.bias[e];  // before the top-k (families/gptoss/moe.rs:82-87)
-                key[j] = order_key(s);
+                for (int sp = 0; sp < 8; sp++) part[j][sp] = a.logits[((size_t)min(sp, a.splits - 1) * 16 + m) * a.ld + e];
+                bias[j] = a.bias ? a.bias[e] : 0.f;  // before the top-k (families/gptoss/moe.rs:82-87)
             }
-        }
+#pragma unroll
+            for (int j = 0; j < nj; j++) {
+                float s = 0.f;  // added in split order
+#pragma unroll
+                for (int sp = 0; sp < 8; sp++) s += sp < a.splits ? part[j][sp] : 0.f;
+                if (a.bias) s += bias[j];
+                if (lane + 64 * j < ne) key[j] = order_key(s);
+            }
+        };
+        if (ne <= 128)
+            gather(std::integral_constant<int, 2>{});
+        else
+            gather(std::integral_constant<int, 4>{});
         float top = 0.f, sum = 0.f, my_ex = 0.f;
         int my_sel = 0;
 #pragma unroll
@@ -112,29 +126,37 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
             a.weights[m * 8 + lane] = my_ex / sum;
             a.selected[m * 8 + lane] = my_sel;
             s_sel[m * k + lane] = my_sel;
+            const int pair = m * k + lane;
+            atomicOr(&s_mask[my_sel * 4 + (pair >> 5)], 1u << (pair & 31));
         }
     }
     __syncthreads();
     // Groups: pair j leads the group of its expert when no earlier pair chose it; the members of a
-    // group are listed in pair order.  Every pair finds its own place (how many earlier pairs share
-    // its expert, and which of them is the first) in one pass over the selections.
+    // group are listed in pair order.  Every pair has set its bit in its expert's membership mask: a
+    // pair's place is the number of set bits below its own, the group's leader the lowest set bit,
+    // the group's size the number of set bits.
     const int j = threadIdx.x, np = M * k;
     if (j >= np) return;
     const int e = s_sel[j];
-    int first = j, pos = 0, cnt = 0;
-    for (int i = 0; i < np; i++) {
-        const bool same = s_sel[i] == e;
-        cnt += same ? 1 : 0;
-        if (same && i < j) {
-            pos++;
-            first = min(first, i);
-        }
-    }
+    const uint32_t m0 = s_mask[e * 4], m1 = s_mask[e * 4 + 1], m2 = s_mask[e * 4 + 2], m3 = s_mask[e * 4 + 3];
+    const int cnt = __popc(m0) + __popc(m1) + __popc(m2) + __popc(m3);
+    const int first = m0 ? __ffs(m0) - 1 : m1 ? 31 + __ffs(m1) : m2 ? 63 + __ffs(m2) : 95 + __ffs(m3);
+    const uint32_t below = (1u << (j & 31)) - 1u;
+    const int w = j >> 5;
+    const int pos = (w > 0 ? __popc(m0) : 0) + (w > 1 ? __popc(m1) : 0) + (w > 2 ? __popc(m2) : 0) +
+                    __popc((w == 0 ? m0 : w == 1 ? m1 : w == 2 ? m2 : m3) & below);
     const int row = j / k;
     if (pos < TSV_MAX_ROWS) {  // a row chooses an expert once, so a group never has more members than rows
         MoeGroup* lead = a.groups + first;
         lead->rows[pos] = row;
         lead->slots[pos] = j - row * k;
+        // the last member also fills the entries past the count: a reader that takes entry n without
+        // looking at the count first then finds a row of the group, never a stale one
+        if (pos == cnt - 1)
+            for (int p = cnt; p < TSV_MAX_ROWS; p++) {
+                lead->rows[p] = row;
+                lead->slots[p] = j - row * k;
+            }
     }
     MoeGroup* g = a.groups + j;
     g->expert = e;
@@ -226,7 +248,7 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
             } else {
                 act = silu_moe(gate) * up;
             }
-            const _Float16 h = (_Float16)act;
+            const _Float16 h = pinned_half((_Float16)act);
             float sum = (float)h;
 #pragma unroll
             for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
@@ -250,18 +272,20 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
     }
 }
 
-// grid: (tiles per expert, rows x top_k groups).  Groups that repeat an earlier expert leave at
-// once.  An expert chosen by more than four rows (rare at these batch widths) is multiplied in
-// several sweeps of four rows; its tile then comes from L2.
+// grid: (tiles per expert, rows x top_k groups, sweeps).  Groups that repeat an earlier expert leave
+// at once.  A workgroup multiplies its tile by four of the group's rows, 4 z .. 4 z + 3: an expert
+// chosen by more than four rows is covered by several workgroups side by side, and those past the
+// group's count leave at once.  With tiles x groups a multiple of eight the workgroups of one tile
+// run on the same XCD, so the tile comes from HBM once and from that XCD's L2 after.
 template <class F, int EPI, int STAGES>
 __global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
     extern __shared__ float4v red[];
     __shared__ MoeGroup grp;
-    const int gi = blockIdx.y;
+    const int gi = blockIdx.y, r0 = 4 * blockIdx.z;
     if (threadIdx.x < sizeof(MoeGroup) / 4) ((int32_t*)&grp)[threadIdx.x] = ((const int32_t*)(a.groups + gi))[threadIdx.x];
     __syncthreads();
-    if (grp.cnt == 0) return;
-    for (int r0 = 0; r0 < grp.cnt; r0 += 4) expert_tile<F, EPI, STAGES>(a, grp, gi, r0, red);
+    if (r0 >= grp.cnt) return;
+    expert_tile<F, EPI, STAGES>(a, grp, gi, r0, red);
 }
 
 template <class F, int EPI>
@@ -275,10 +299,11 @@ int launch_moe_t(hipStream_t s, const MoeGemmArgs& a, int n_groups) {
     const int cpw = forced ? forced : std::max(2, (a.kchunks + 3) / 4);
     const int nw = std::min(8, std::max(1, (a.kchunks + cpw - 1) / cpw));
     const size_t lds = (size_t)nw * 1024;
+    const dim3 grid(a.tiles_per_expert, n_groups, (std::max(1, a.rows) + 3) / 4);  // no group has more members than the pass has rows
     if ((a.kchunks + nw - 1) / nw <= 2)
-        hipLaunchKernelGGL((k_moe_gemm<F, EPI, 2>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);
+        hipLaunchKernelGGL((k_moe_gemm<F, EPI, 2>), grid, dim3(64 * nw), lds, s, a);
     else
-        hipLaunchKernelGGL((k_moe_gemm<F, EPI, 1>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);
+        hipLaunchKernelGGL((k_moe_gemm<F, EPI, 1>), grid, dim3(64 * nw), lds, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -300,7 +325,9 @@ int launch_route(hipStream_t s, const MoeRouteArgs& a) {
         set_error("moe: at most 256 experts and top-k between 1 and 8");
         return TSV_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(k_route, dim3(1), dim3(1024), 0, s, a);
+    // one wave per row for the top-k, one thread per (row, slot) pair for the groups
+    const int threads = std::max(64 * a.m, (a.m * a.top_k + 63) / 64 * 64);
+    hipLaunchKernelGGL(k_route, dim3(1), dim3(std::min(1024, threads)), 0, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

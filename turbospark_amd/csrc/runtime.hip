@@ -72,6 +72,11 @@ struct tsv_ctx {
     uint8_t* frag_e = nullptr;
     size_t frag_e_stride = 0;
     float* moe_out = nullptr;
+    // scaled-MFMA expert matmuls (moe_fp4.hip): activation terms (0 = the fp16 path), the pass's rows
+    // and the groups' gate/up outputs as block-scaled fp8
+    int moe_fp4_terms = 0;
+    X8 x8_h{}, x8_e{};
+    size_t x8_e_q_stride = 0, x8_e_s_stride = 0;
     // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
     // sum-of-squares partials, per-XCD partial sums, barrier counters
     bool fused_ffn = false, fused_attn = false;
@@ -654,7 +659,9 @@ int launch_pass(tsv_ctx* c, int m) {
         }
         {
             PROF(PC_NORM);
-            rc = launch_addnorm(s, x, attn_partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo);
+            const bool fp4 = L.n_experts && c->moe_fp4_terms;
+            rc = launch_addnorm(s, x, attn_partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo,
+                                fp4 ? &c->x8_h : nullptr, c->moe_fp4_terms);
         }
         if (rc) return rc;
         if (L.n_experts) {
@@ -677,6 +684,7 @@ int launch_pass(tsv_ctx* c, int m) {
             g1.tiles_per_expert = c->ffn / 32;
             g1.kchunks = L.gate_up.kchunks;
             g1.k = c->hidden;
+            g1.rows = m;
             g1.xfrag = c->xf_a;
             g1.x_stride = 0;
             g1.out = c->frag_e;
@@ -700,6 +708,18 @@ int launch_pass(tsv_ctx* c, int m) {
             g2.out = c->moe_out;
             g2.out_stride = 0;
             g2.n_out = c->hidden;
+            const bool fp4 = c->moe_fp4_terms != 0;
+            if (fp4) {
+                g1.x8_terms = g2.x8_terms = c->moe_fp4_terms;
+                g1.x8 = c->x8_h;
+                g1.o8 = c->x8_e;
+                g1.o8_q_stride = c->x8_e_q_stride;
+                g1.o8_s_stride = c->x8_e_s_stride;
+                g2.x8 = c->x8_e;
+                g2.x8_q_stride = c->x8_e_q_stride;
+                g2.x8_s_stride = c->x8_e_s_stride;
+                g2.o8 = X8{};
+            }
             {
                 PROF(PC_GATEUP);
                 rc = 0;
@@ -707,14 +727,15 @@ int launch_pass(tsv_ctx* c, int m) {
                     rc = launch_gemm(s, L.router, c->xf_a, c->partial, c->vp_dev, m, rsp, EPI_PARTIAL, L.n_experts,
                                      L.n_experts);
                     if (!rc) rc = launch_route(s, ra2);
-                    if (!rc) rc = launch_moe_gate_up(s, L.gate_up.fmt, g1, n_groups);
+                    if (!rc) rc = fp4 ? launch_moe_fp4_gate_up(s, g1, n_groups) : launch_moe_gate_up(s, L.gate_up.fmt, g1, n_groups);
                 }
             }
             if (rc) return rc;
             {
                 PROF(PC_DOWN);
                 rc = 0;
-                for (int rep = 0; rep < c->repeat[PC_DOWN] && !rc; rep++) rc = launch_moe_down(s, L.down.fmt, g2, n_groups);
+                for (int rep = 0; rep < c->repeat[PC_DOWN] && !rc; rep++)
+                    rc = fp4 ? launch_moe_fp4_down(s, g2, n_groups) : launch_moe_down(s, L.down.fmt, g2, n_groups);
             }
             if (rc) return rc;
             prev_partial = c->moe_out;
@@ -845,6 +866,9 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->act_limit = d->act_limit;
     if (const char* e = getenv("TSV_GRAPH")) c->use_graph = e[0] == '1';
     if (const char* e = getenv("TSV_ROPE_FUSED")) c->rope_fused_ok = e[0] != '0';
+    // MXFP4 experts on the block-scaled matrix instruction: activation terms, 0 = the fp16 path
+    c->moe_fp4_terms = MOE_FP4_DEFAULT_TERMS;
+    if (const char* e = getenv("TSV_MOE_FP4")) c->moe_fp4_terms = e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("open: cannot create a HIP stream (no GPU?)");
         delete c;
@@ -900,6 +924,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
                 return fail(rc);
             L.n_experts = ne;
             L.top_k = s.top_k;
+            if (L.gate_up.fmt != FMT_MX4 || L.down.fmt != FMT_MX4) c->moe_fp4_terms = 0;
             c->max_experts = std::max(c->max_experts, ne);
             pneed = std::max(pneed, partial_need(L.router));
         } else {
@@ -1036,6 +1061,8 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->nch = attn_chunks(c->nkv);
     const size_t rows_max = (size_t)TSV_MAX_ROWS * (c->nq / c->nkv);
     c->partial_floats = pneed;
+    c->x8_h.kpad = (c->hidden + 255) / 256 * 256;
+    c->x8_e.kpad = (c->ffn + 255) / 256 * 256;
     if ((rc = dev_alloc(c, &c->x, (size_t)16 * c->hidden * 4, true)) || (rc = dev_alloc(c, &c->xf_a, xfb, true)) ||
         (rc = dev_alloc(c, &c->xf_b, xfb, true)) || (rc = dev_alloc(c, &c->xf_c, xfb, true)) ||
         (rc = dev_alloc(c, &c->partial, pneed * 4, true)) ||
@@ -1043,7 +1070,12 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
          ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, true)) ||
           (rc = dev_alloc(c, &c->route_groups, (size_t)TSV_MAX_ROWS * 8 * sizeof(MoeGroup), true)) ||
           (rc = dev_alloc(c, &c->frag_e, (size_t)TSV_MAX_ROWS * 8 * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
-          (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)))) || (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
+          (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)) ||
+          (c->moe_fp4_terms &&
+           ((rc = dev_alloc(c, &c->x8_h.q, x8_q_bytes(c->hidden), true)) || (rc = dev_alloc(c, &c->x8_h.s, x8_s_bytes(c->hidden), true)) ||
+            (rc = dev_alloc(c, &c->x8_e.q, (size_t)TSV_MAX_ROWS * 8 * (c->x8_e_q_stride = x8_q_bytes(c->ffn)), true)) ||
+            (rc = dev_alloc(c, &c->x8_e.s, (size_t)TSV_MAX_ROWS * 8 * (c->x8_e_s_stride = x8_s_bytes(c->ffn)), true)))))) ||
+        (rc = dev_alloc(c, &c->q16, (size_t)16 * qd * 2, true)) ||
         (rc = dev_alloc(c, &c->part_o, (size_t)c->nkv * c->nch * rows_max * c->hd * 4, true)) ||
         (rc = dev_alloc(c, &c->part_ml, (size_t)c->nkv * c->nch * rows_max * 2 * 4, true)) ||
         (rc = dev_alloc(c, &c->logits, (size_t)16 * c->vocab * 2, true)) ||

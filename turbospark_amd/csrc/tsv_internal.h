@@ -82,6 +82,17 @@ inline int fmt_tile_bytes(int fmt) {
 inline int fmt_nsub(int fmt) { return fmt == FMT_Q80 ? 4 : fmt == FMT_BF16 ? 2 : fmt == FMT_Q6K ? 16 : 8; }
 constexpr int TILE_ROWS = 64;
 
+// An fp16 activation on its way to both the fragment store and the sub-block sum.  The matmuls multiply
+// the sums by the weights' code offsets (up to 1024), so the sum must be that of the stored bits exactly;
+// left alone, the compiler may convert the same fp32 value twice, with different instructions (a packed
+// convert for the store, a fused multiply-convert for the sum).  Pinning the half in a register leaves it
+// one copy to read.
+__device__ __forceinline__ _Float16 pinned_half(_Float16 h) {
+    uint32_t b = __builtin_bit_cast(uint16_t, h);
+    asm volatile("" : "+v"(b));
+    return __builtin_bit_cast(_Float16, (uint16_t)b);
+}
+
 // index (in halfs) of activation element (row, k) in the fragment layout
 __host__ __device__ inline int frag_index(int k, int row) {
     const int pos = ((k & 1) << 1) | ((k >> 1) & 1);  // k%4 = 0,1,2,3 -> slot 0,2,1,3
@@ -158,9 +169,30 @@ struct MoeRouteArgs {
     MoeGroup* groups;   // [16 * 8]
     const float* bias;  // nullable: n_experts values added to the logits before the top-k
 };
+// Block-scaled fp8 activations: the B operand of the scaled-MFMA expert matmuls (MXFP4 experts).  A
+// value is the sum of `terms` e4m3 numbers, each times the power-of-two scale of its 32-element
+// block; term t holds what the terms before it left over, so three terms carry about 2^-13 of the
+// block's largest element.  Byte i of word w of a block is element 4 w + {0, 2, 1, 3}[i]: the order
+// of the weight tiles' nibbles.
+struct X8 {
+    uint8_t* q;  // [terms][16 rows][kpad] e4m3
+    uint8_t* s;  // [terms][16 rows][kpad / 32] E8M0: scale = 2^(byte - 127)
+    int kpad;    // K rounded up to whole 256-element chunks; the tail stays zero from the allocation
+};
+constexpr int X8_MAX_TERMS = 3;
+constexpr int MOE_FP4_DEFAULT_TERMS = 2;  // what a context uses unless TSV_MOE_FP4 says otherwise
+inline size_t x8_q_bytes(int k) { return (size_t)X8_MAX_TERMS * 16 * ((k + 255) / 256 * 256); }
+inline size_t x8_s_bytes(int k) { return x8_q_bytes(k) / 32; }
+
 struct MoeGemmArgs {
     const uint8_t* w;      // tiled weights of all experts, tiles_per_expert x kchunks tiles each
     int tiles_per_expert, kchunks, k;
+    int rows;              // rows of the pass: the most members a group can have
+    // scaled-MFMA path (x8_terms > 0, MXFP4 experts only): x8 replaces xfrag, o8 replaces the gate/up
+    // output fragments; the strides are the bytes between the groups' buffers (0: one shared buffer)
+    int x8_terms;
+    X8 x8, o8;
+    size_t x8_q_stride, x8_s_stride, o8_q_stride, o8_s_stride;
     const void* xfrag;     // gate/up: the pass's activation fragments; down: per-group fragments
     size_t x_stride;       // down: bytes between groups' fragment buffers
     void* out;             // gate/up: per-group fragments of silu(gate) * up; down: float [8 slots][16][n_out]
@@ -176,6 +208,9 @@ struct MoeGemmArgs {
 int launch_route(hipStream_t s, const MoeRouteArgs& a);
 int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
+// the same two matmuls on v_mfma_scale_f32_16x16x128_f8f6f4 (moe_fp4.hip)
+int launch_moe_fp4_gate_up(hipStream_t s, const MoeGemmArgs& a, int n_groups);
+int launch_moe_fp4_down(hipStream_t s, const MoeGemmArgs& a, int n_groups);
 
 // ---- per-XCD fused layer kernels ----------------------------------------------------------
 // Counters of the XCD-local barriers.  rank_ctr / bar_ctr: one word per XCD, 64 words apart.
@@ -230,7 +265,7 @@ int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float
 // weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
                    float eps, int hidden, uint4* xfrag, int m, const float* weights = nullptr,
-                   const float* bias = nullptr);
+                   const float* bias = nullptr, const X8* x8 = nullptr, int x8_terms = 0);
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
 
 struct RopeKvArgs {
