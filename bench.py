@@ -74,15 +74,16 @@ def algorithmic_bytes(cfg, ctx, m, union=None):
     return dict(per_layer=per_layer, head=head, weights=weights, kv=kv, total=weights + kv + small)
 
 
-def trace_summary(path):
+def trace_summary(path, first="k_clear_result"):
     """Per-kernel statistics of the verify STEPS in a `rocprofv3 --kernel-trace --output-format csv`
     trace of this script: only dispatches from the first acceptance kernel on are counted,
-    which leaves out weight re-tiling and the 16-row prefill passes that build the KV cache.
+    which leaves out weight re-tiling and the prompt passes that build the KV cache (--trace-from
+    k_embed counts from the first pass on instead: the prompt passes of a --prefill-bench run).
     Kernels are keyed by name and grid size, so the five matmul shapes show up separately."""
     import csv
     rows = list(csv.DictReader(open(path)))
     rows.sort(key=lambda r: int(r["Start_Timestamp"]))
-    start = next(i for i, r in enumerate(rows) if "k_clear_result" in r["Kernel_Name"])
+    start = next(i for i, r in enumerate(rows) if first in r["Kernel_Name"])
     stats = {}
     for r in rows[start:]:
         name = r["Kernel_Name"].replace("tsv::", "").replace("(anonymous namespace)::", "")
@@ -99,7 +100,8 @@ def trace_summary(path):
     for (name, wgs, lds), v in sorted(stats.items(), key=lambda kv: -kv[1][1]):
         print(f"{name[:44]:44s} {wgs:6d} {lds:7d} {v[0]:7d} {v[1] / v[0] / 1e3:9.2f} {v[2] / 1e3:9.2f} {v[3] / 1e3:9.2f} "
               f"{100.0 * v[1] / total:6.2f}%")
-    print(f"total kernel time in verify steps: {total / 1e6:.3f} ms over the traced steps")
+    what = "verify steps" if first == "k_clear_result" else f"dispatches from the first {first} on"
+    print(f"total kernel time in {what}: {total / 1e6:.3f} ms over the traced steps")
 
 
 # Figures RECORDED from committed counter / trace runs (a bench run does not collect counters): HBM
@@ -205,6 +207,11 @@ def main():
                     help="HBM bytes per launch of the dominant matmul from two --pmc runs of --traffic-probe")
     ap.add_argument("--probe", default="gate_up", choices=sorted(PROBES),
                     help="which kernel --traffic-probe runs and the two summaries read")
+    ap.add_argument("--trace-from", default="k_clear_result", metavar="KERNEL",
+                    help="--trace-summary counts dispatches from the first one of this kernel on")
+    ap.add_argument("--prefill-bench", type=int, default=0, metavar="TOKENS",
+                    help="time tsv_prefill over a prompt of this many tokens (after one untimed run of the same), print one "
+                         "JSON line and exit")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -214,7 +221,7 @@ def main():
     ap.add_argument("--seed", type=int, default=20261125)
     args = ap.parse_args()
     if args.trace_summary:
-        trace_summary(args.trace_summary)
+        trace_summary(args.trace_summary, args.trace_from)
         return
     if args.traffic_probe:
         traffic_probe(args.probe)
@@ -248,6 +255,22 @@ def main():
     eng = ts.HipVerifier(cfg, weights)
     log(f"[bench] upload + re-tile in {time.time() - t0:.1f}s")
     rng = np.random.default_rng(args.seed)
+    if args.prefill_bench:
+        n = args.prefill_bench
+        if n >= cfg["max_context"]:
+            sys.exit(f"bench.py: --prefill-bench takes at most {cfg['max_context'] - 1} tokens at this workload")
+        prompt = rng.integers(0, V, n).astype(np.int32)
+        eng.prefill(prompt, 0, want_logits=False)     # untimed: first-use allocations, code objects
+        eng.reset()
+        t0 = time.perf_counter()
+        eng.prefill(prompt, 0, want_logits=False)     # returns after the stream has drained
+        dt = time.perf_counter() - t0
+        rows = 16 if os.environ.get("TSV_WIDE_PREFILL") == "0" or cfg["dtype"] != ts.ffi.Q4_K or cfg.get("n_experts") else 64
+        print(json.dumps({"metric": "prefill tokens/s", "value": round(n / dt, 1), "unit": "tokens/s", "n_gpus": 1,
+                          "higher_is_better": True, "dtype": "f16", "data": "synthetic", "seconds": round(dt, 4),
+                          "config": {"workload": args.workload, "layers": cfg["n_layers"], "prompt_tokens": n,
+                                     "rows_per_pass": rows, "logits": "none (headless passes)"}}))
+        return
     prompt = rng.integers(0, V, ctx).astype(np.int32)
     t0 = time.time()
     eng.prefill(prompt[:-1], 0, want_logits=False)   # the last prompt token is the round's confirmed token

@@ -1,0 +1,95 @@
+"""Prompt passes of 64 rows (crates/runtime/src/producer.rs:122-150, ChunkedPrefillRunner; families/llama/prefill.rs):
+the cache they fill and the logits that follow, against the oracle and against the 16-row passes of the same
+library.  The two GPU paths multiply the same integers by the same fp16 activations and differ in the order of
+the fp32 additions only, so they agree to a few fp16 ulps per layer, not by bits."""
+import os
+
+import numpy as np
+import pytest
+
+from tests import gpu_common as gc
+
+pytestmark = pytest.mark.gpu
+
+
+def _engine(cfg, weights, wide):
+    import turbospark_amd as ts
+    os.environ["TSV_WIDE_PREFILL"] = "1" if wide else "0"
+    try:
+        return ts.HipVerifier(cfg, weights)
+    finally:
+        del os.environ["TSV_WIDE_PREFILL"]
+
+
+@pytest.mark.parametrize("name,n_prompt", [("small_q4_k", 150), ("small_q4_k", 64), ("xcd_q4_k", 200), ("small_q4_k", 129)])
+def test_a_prompt_fed_in_blocks_of_64_fills_the_cache_the_oracle_fills(name, n_prompt):
+    from turbospark_amd import synth
+    from oracle import binding as ob
+    os.environ["TSV_FUSED"] = "0"
+    cfg = dict(synth.CONFIGS[name], max_context=n_prompt + 48)
+    w = synth.make_weights(cfg, seed=11)
+    wide, narrow = _engine(cfg, w, True), _engine(cfg, w, False)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)
+    rng = np.random.default_rng(2)
+    prompt = rng.integers(0, cfg["vocab"], n_prompt).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    wide.prefill(prompt, 0, want_logits=False)
+    narrow.prefill(prompt, 0, want_logits=False)
+    for i in range(0, n_prompt, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    assert wide.position == narrow.position == n_prompt
+    for layer in range(cfg["n_layers"]):
+        kw, vw = wide.read_kv(layer, 0, n_prompt)
+        kn, vn = narrow.read_kv(layer, 0, n_prompt)
+        kc, vc = cpu.kv(layer)
+        for got, other, want in ((kw, kn, kc), (vw, vn, vc)):
+            got, other, want = got.astype(np.float32), other.astype(np.float32), want[:n_prompt]
+            scale = np.abs(want).max()
+            assert np.abs(got - want).max() <= 2e-2 * scale
+            # the two GPU paths: a few fp16 ulps of the largest value
+            assert np.abs(got - other).max() <= 4e-3 * scale, (layer, np.abs(got - other).max() / scale)
+    want = cpu.verify(feed, n_prompt)
+    got_w, got_n = wide.verify(feed, n_prompt), narrow.verify(feed, n_prompt)
+    err_w, err_n, err_wn = gc.logit_error(got_w, want), gc.logit_error(got_n, want), gc.logit_error(got_w, got_n)
+    print(f"{name}, prompt of {n_prompt}: logits after 64-row passes vs oracle {err_w:.2e}, after 16-row passes {err_n:.2e}, "
+          f"the two GPU paths {err_wn:.2e}")
+    assert err_w <= 1e-2 and err_wn <= 2e-3
+
+
+def test_logits_of_the_last_prompt_token_after_wide_passes():
+    """tsv_prefill hands out the last row's logits: the rows before it go in blocks of 64, the tail in
+    16-row passes whose last one carries the output head."""
+    from turbospark_amd import synth
+    from oracle import binding as ob
+    os.environ["TSV_FUSED"] = "0"
+    cfg = dict(synth.CONFIGS["small_q4_k"], max_context=256)
+    w = synth.make_weights(cfg, seed=12)
+    wide = _engine(cfg, w, True)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)
+    prompt = np.random.default_rng(3).integers(0, cfg["vocab"], 128).astype(np.int32)  # exactly two blocks: the second is not wide
+    got = wide.prefill(prompt, 0, want_logits=True)
+    want = None
+    for i in range(0, 128, 16):
+        want = cpu.verify(prompt[i:i + 16], i)
+    err = gc.logit_error(got.reshape(1, -1), want[-1:])
+    print(f"last prompt row after wide passes: {err:.2e}")
+    assert err <= 1e-2
+    assert wide.position == 128
+
+
+def test_wide_passes_are_deterministic_and_leave_the_prefix_record_intact():
+    from turbospark_amd import synth
+    os.environ["TSV_FUSED"] = "0"
+    cfg = dict(synth.CONFIGS["small_q4_k"], max_context=256)
+    w = synth.make_weights(cfg, seed=13)
+    a, b = _engine(cfg, w, True), _engine(cfg, w, True)
+    prompt = np.random.default_rng(4).integers(0, cfg["vocab"], 200).astype(np.int32)
+    a.prefill(prompt, 0, want_logits=False)
+    b.prefill(prompt[:70], 0, want_logits=False)     # another split of the same prompt: 64 + 6, then 64 + 64 + 2
+    b.prefill(prompt[70:], 70, want_logits=False)
+    feed = prompt[:4]
+    la, lb = a.verify(feed, 200), b.verify(feed, 200)
+    assert gc.logit_error(la, lb) <= 2e-3
+    a.reset()
+    a.prefill(prompt, 0, want_logits=False)
+    assert np.array_equal(a.verify(feed, 200), la)

@@ -586,6 +586,211 @@ __global__ __launch_bounds__(512) void k_gemm16(GemmArgs a) {
     }
 }
 
+// ------------------------------------------------------------------------------- prompt blocks of 64 rows
+// A prompt pass of BLOCKS x 16 rows over Q4_K weights (crates/runtime/src/producer.rs:122-150: the
+// chunked prefill runner feeds the prompt in blocks; families/llama/prefill.rs).  One workgroup per
+// (tile, K slice), one wave per block of sixteen rows.  A tile chunk is unpacked ONCE per workgroup:
+// wave w turns row block w of the chunk (sixteen weight rows x 256 K) into the B operands of
+// v_mfma_f32_16x16x32_f16 and leaves them in LDS, in the lane order the 16-row kernel builds them in
+// registers; after a barrier every wave multiplies all four row blocks by its own sixteen
+// activation rows.  So the weight bytes, and the vector-ALU work of unpacking them, are spent once
+// per 64 rows, and what is left per row block is matrix instructions.
+//
+// The unpacked operand is the integer sc_j * q (at most 63 * 15, exact in fp16), made from the
+// offset codes by one packed fma: (1024 + q) * sc - 1024 * sc and (64 + q) * sc - 64 * sc are exact.
+// With the sub-block scale inside the operand the eight sub-blocks of a chunk accumulate in one
+// chain of matrix instructions, and the superblock scale d is applied once per chunk; the min term
+// -dmin * m_j * sum_k x_k goes through v_mfma_f32_16x16x4_f32 as in the 16-row kernel.  The products
+// are those of the same integers and the same fp16 activations as in the narrower kernels; only
+// the order of the fp32 additions differs.
+struct GemmWideArgs {
+    GemmArgs g;         // block 0's view; blocks b > 0 sit at the strides below
+    size_t x_stride;    // bytes between the blocks' activation fragments (sums included)
+    size_t out_stride;  // bytes between the blocks' outputs (partial sums or fragments); unused by EPI_ROPE
+    // g.vp: consecutive VerifyParams, one per block; g.rope.cs: [blocks * 16][hd / 2]; g.rope.q16: [blocks * 16][nq][hd]
+};
+
+constexpr int WIDE_BLOCKS = 4;
+constexpr int WIDE_B_BYTES = 32768;             // [row block][sub-block pair][low / high nibbles][64 lanes][16 B]
+constexpr int WIDE_BUF_BYTES = WIDE_B_BYTES + 4096;  // + [row block][64 lanes] (d, -dmin m_kg, -dmin m_(kg+4), 0)
+
+struct WideW {  // what the unpacking wave holds of one chunk: its row block's codes and scale header
+    u32x2 q[4];
+    u32x4 h;
+};
+struct WideX {  // a block's activations of one chunk
+    u32x2 x[8][2];
+    float xs[2];
+};
+
+__device__ __forceinline__ void wide_load_w(WideW& w, const uint8_t* tile_chunk, int rb, int lane) {
+    const int r = lane & 15, kg = lane >> 4;
+    const uint8_t* wp = tile_chunk + ((kg >> 1) * 64 + r) * 16 + (kg & 1) * 8;
+#pragma unroll
+    for (int p = 0; p < 4; p++) w.q[p] = __builtin_nontemporal_load((const u32x2*)(wp + (2 * p * 64 + 16 * rb) * 16));
+    w.h = __builtin_nontemporal_load((const u32x4*)(tile_chunk + 8192 + (16 * rb + r) * 16));
+}
+
+__device__ __forceinline__ void wide_load_x(WideX& x, const GemmArgs& a, int c, int lane) {
+    const int r = lane & 15, kg = lane >> 4;
+    const u32x2* xp = (const u32x2*)a.xfrag + (size_t)c * 1024 + (r >> 2) * 64 + (r & 3) + kg * 8;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) x.x[j][t] = xp[(j >> 1) * 256 + ((j & 1) * 8 + t) * 4];
+    const float* sp = a.xsum + (size_t)c * 128 + (r >> 2) * 32 + (r & 3) + kg * 4;
+    x.xs[0] = sp[0];
+    x.xs[1] = sp[16];
+}
+
+// Row block `rb` of a chunk into LDS buffer `buf`.
+__device__ __forceinline__ void wide_unpack(const WideW& w, const Consts& k, uint8_t* buf, int rb, int lane) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const int kg = lane >> 4;
+    const u32x4 hs = w.h;
+    const float d = h2f_lo(hs.x), dmin = h2f_hi(hs.x);
+    const uint32_t sl = hs.y & 0x3F3F3F3Fu, ml = hs.z & 0x3F3F3F3Fu;
+    const uint32_t sh = (hs.w & 0x0F0F0F0Fu) | ((hs.y >> 2) & 0x30303030u);
+    const uint32_t mh = ((hs.w >> 4) & 0x0F0F0F0Fu) | ((hs.z >> 2) & 0x30303030u);
+    const int sft = 8 * kg;
+    float4v coef;
+    coef.x = d;
+    coef.y = -(dmin * (float)((ml >> sft) & 0xFF));
+    coef.z = -(dmin * (float)((mh >> sft) & 0xFF));
+    coef.w = 0.f;
+    *(float4v*)(buf + WIDE_B_BYTES + (rb * 64 + lane) * 16) = coef;
+    const half2v m1024 = {(_Float16)-1024.0f, (_Float16)-1024.0f}, m64 = {(_Float16)-64.0f, (_Float16)-64.0f};
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        // the 6-bit scales of sub-blocks 2p (low nibbles) and 2p + 1 (high nibbles) as fp16 pairs
+        const uint32_t s_lo = ((2 * p < 4 ? sl : sh) >> (8 * ((2 * p) & 3))) & 0xFFu;
+        const uint32_t s_hi = ((2 * p + 1 < 4 ? sl : sh) >> (8 * ((2 * p + 1) & 3))) & 0xFFu;
+        const half2v sc_lo = __builtin_bit_cast(half2v, k.k6400 | s_lo | (s_lo << 16)) + m1024;
+        const half2v sc_hi = __builtin_bit_cast(half2v, k.k6400 | s_hi | (s_hi << 16)) + m1024;
+        const half2v off_lo = sc_lo * m1024, off_hi = sc_hi * m64;
+        const uint32_t w0 = w.q[p].x, w1 = w.q[p].x >> 8, w2 = w.q[p].y, w3 = w.q[p].y >> 8;
+        const uint32_t wv[4] = {w0, w1, w2, w3};
+        u32x4 blo, bhi;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const half2v lo = __builtin_bit_cast(half2v, and_or(wv[i], 0x000F000Fu, k.k6400));  // 1024 + q
+            const half2v hi = __builtin_bit_cast(half2v, and_or(wv[i], 0x00F000F0u, k.k5400));  // 64 + q
+            blo[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(lo, sc_lo, off_lo));
+            bhi[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(hi, sc_hi, off_hi));
+        }
+        *(u32x4*)(buf + (((rb * 4 + p) * 2 + 0) * 64 + lane) * 16) = blo;
+        *(u32x4*)(buf + (((rb * 4 + p) * 2 + 1) * 64 + lane) * 16) = bhi;
+    }
+}
+
+// One chunk from LDS buffer `buf` against this wave's block.  The four row blocks are four independent
+// accumulator chains, walked side by side (an activation operand is used four times in a row), and
+// the operands of sub-block pair p + 1 are asked of LDS before the matrix instructions of pair p
+// issue: a wave is alone on its SIMD here, so nothing else would cover the LDS latency.
+__device__ __forceinline__ void wide_compute(const WideX& x, const uint8_t* buf, float4v (&acc)[4], int lane) {
+    const float4v zero = {0.f, 0.f, 0.f, 0.f};
+    float4v coef[4], t[4], tq[4];
+    u32x4 blo[2][4], bhi[2][4];
+    auto fetch = [&](int slot, int p) {
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++) {
+            blo[slot][rb] = *(const u32x4*)(buf + (((rb * 4 + p) * 2 + 0) * 64 + lane) * 16);
+            bhi[slot][rb] = *(const u32x4*)(buf + (((rb * 4 + p) * 2 + 1) * 64 + lane) * 16);
+        }
+    };
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) coef[rb] = *(const float4v*)(buf + WIDE_B_BYTES + (rb * 64 + lane) * 16);
+    fetch(0, 0);
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+        t[rb] = __builtin_amdgcn_mfma_f32_16x16x4f32(x.xs[0], coef[rb].y, zero, 0, 0, 0);
+        tq[rb] = zero;
+    }
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) t[rb] = __builtin_amdgcn_mfma_f32_16x16x4f32(x.xs[1], coef[rb].z, t[rb], 0, 0, 0);
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        if (p < 3) fetch((p + 1) & 1, p + 1);
+        const u32x4 alo = {x.x[2 * p][0].x, x.x[2 * p][0].y, x.x[2 * p][1].x, x.x[2 * p][1].y};
+        const u32x4 ahi = {x.x[2 * p + 1][0].x, x.x[2 * p + 1][0].y, x.x[2 * p + 1][1].x, x.x[2 * p + 1][1].y};
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            tq[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, alo), __builtin_bit_cast(half8, blo[p & 1][rb]),
+                                                            tq[rb], 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            tq[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ahi), __builtin_bit_cast(half8, bhi[p & 1][rb]),
+                                                            tq[rb], 0, 0, 0);
+    }
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+        fma4(t[rb], coef[rb].x, tq[rb]);
+        acc[rb] += t[rb];
+    }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;  // wave = this wave's block = the row block it unpacks
+    GemmArgs a = wa.g;
+    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
+    a.xsum = (const float*)((const uint8_t*)a.xsum + (size_t)wave * wa.x_stride);
+    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
+    a.vp = a.vp + wave;
+    if (EPI == EPI_ROPE) {
+        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
+        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
+    }
+    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
+    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q4K::TILE_BYTES;
+    Consts k;
+    k.k6400 = 0x64006400u;
+    k.k5400 = 0x54005400u;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400));
+    float4v acc[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int M = a.vp->m;
+    // chunk c: unpack into buffer c & 1 -> ask for chunk c + 1 -> barrier -> multiply chunk c.  The
+    // barrier of chunk c also separates the reads of chunk c - 1 from the unpacking of chunk c + 1,
+    // which goes to the same buffer.
+    WideW w[2];
+    WideX x[2];
+    if (s0 < s1) {
+        wide_load_w(w[0], wt + (size_t)s0 * Q4K::TILE_BYTES, wave, lane);
+        wide_load_x(x[0], a, s0, lane);
+    }
+    for (int c = s0; c < s1; c += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            if (c + u < s1) {
+                uint8_t* buf = wide_lds + u * WIDE_BUF_BYTES;
+                wide_unpack(w[u], k, buf, wave, lane);
+                if (c + u + 1 < s1) {
+                    wide_load_w(w[u ^ 1], wt + (size_t)(c + u + 1) * Q4K::TILE_BYTES, wave, lane);
+                    wide_load_x(x[u ^ 1], a, c + u + 1, lane);
+                }
+                __syncthreads();
+                wide_compute(x[u], buf, acc, lane);
+            }
+        }
+    }
+    __syncthreads();  // the sums below reuse no chunk buffer, but every wave must be done with LDS ordering games
+    float* ssum = (float*)(wide_lds + 2 * WIDE_BUF_BYTES) + wave * 32;
+#pragma unroll
+    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
+    if (EPI == EPI_SILU) {
+        __syncthreads();
+        if (lane < 16 && lane < M) {
+            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
+            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
+        }
+    }
+}
+
 // Fewest rows that go to the 16x16x32 form (TSV_GEMM16=0: never; TSV_GEMM16=<n>: from n rows on).
 static int gemm16_min_rows() {
     static const int n = [] {
@@ -650,16 +855,12 @@ static int launch_f(hipStream_t s, const GemmArgs& a, int m, int epi) {
     }
 }
 
-int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
-                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
-    if (m < 1 || m > TSV_MAX_ROWS) {
-        set_error("matmul: row count outside 1..16");
-        return TSV_ERR_INVALID;
-    }
+static int fill_gemm_args(GemmArgs& a, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp, int splits,
+                          int epi, int ldo, int n_valid, const RopeEpi* rope) {
     if (epi != EPI_PARTIAL) splits = 1;
     if (splits < 1) splits = 1;
     if (splits > w.kchunks) splits = w.kchunks;
-    GemmArgs a{};
+    a = GemmArgs{};
     a.w = w.tiles;
     a.xfrag = (const uint2*)xfrag;
     a.xsum = (const float*)((const char*)xfrag + xfrag_sum_offset(w.k));
@@ -693,6 +894,17 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
         }
         a.n_valid = w.n_rows / 2;  // K of the next matmul
     }
+    return TSV_OK;
+}
+
+int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
+                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
+    if (m < 1 || m > TSV_MAX_ROWS) {
+        set_error("matmul: row count outside 1..16");
+        return TSV_ERR_INVALID;
+    }
+    GemmArgs a;
+    if (int rc = fill_gemm_args(a, w, xfrag, out, vp, splits, epi, ldo, n_valid, rope)) return rc;
     if (w.fmt == FMT_Q4K && m >= gemm16_min_rows()) return launch16(s, a, epi);
     return w.fmt == FMT_Q4K    ? launch_f<Q4K>(s, a, m, epi)
            : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
@@ -700,6 +912,40 @@ int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, c
            : w.fmt == FMT_Q6K  ? launch_f<Q6K>(s, a, m, epi)
            : w.fmt == FMT_Q5K  ? launch_f<Q5K>(s, a, m, epi)
                                : launch_f<MX4>(s, a, m, epi);
+}
+
+int gemm_wide_rows() { return 16 * WIDE_BLOCKS; }
+
+// The same matmul over gemm_wide_rows() rows in blocks of sixteen: block b reads its fragments at
+// xfrag + b * x_stride bytes, its parameters at vp + b, and writes at out + b * out_stride bytes
+// (EPI_ROPE: rope->cs and rope->q16 hold all blocks' rows one after the other).  Q4_K weights only.
+int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t x_stride, void* out, size_t out_stride,
+                     const VerifyParams* vp, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
+    if (w.fmt != FMT_Q4K) {
+        set_error("matmul: prompt blocks of 64 rows need Q4_K weights");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    GemmWideArgs wa{};
+    if (int rc = fill_gemm_args(wa.g, w, xfrag, out, vp, splits, epi, ldo, n_valid, rope)) return rc;
+    wa.x_stride = x_stride;
+    wa.out_stride = out_stride;
+    const size_t lds = 2 * (size_t)WIDE_BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
+    const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
+    static bool attr_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+    if (!attr_set) {
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_PARTIAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_SILU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    switch (epi) {
+        case EPI_PARTIAL: hipLaunchKernelGGL(k_gemm_wide<EPI_PARTIAL>, grid, block, lds, s, wa); break;
+        case EPI_ROPE: hipLaunchKernelGGL(k_gemm_wide<EPI_ROPE>, grid, block, lds, s, wa); break;
+        case EPI_SILU: hipLaunchKernelGGL(k_gemm_wide<EPI_SILU>, grid, block, lds, s, wa); break;
+        default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
+    }
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
 }
 
 }  // namespace tsv

@@ -121,9 +121,13 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
                                                   int splits, int ldp, const float* __restrict__ w,
                                                   float eps, int hidden, _Float16* __restrict__ xfrag,
                                                   const float* __restrict__ weights,
-                                                  const float* __restrict__ bias, X8 x8, int x8_terms) {
+                                                  const float* __restrict__ bias, X8 x8, int x8_terms, NormBlocks nb) {
     __shared__ float red[16];
     const int m = blockIdx.x;
+    // a prompt pass of several 16-row blocks: block blockIdx.y has its own rows, partial sums and fragments
+    x += (long)blockIdx.y * nb.x;
+    partial += (long)blockIdx.y * nb.partial;
+    xfrag = (_Float16*)((char*)xfrag + (long)blockIdx.y * nb.frag);
     float4* xr = (float4*)(x + (long)m * hidden);
     const float4* wr = (const float4*)w;
     const int n4 = hidden >> 2;
@@ -234,13 +238,13 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
 
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
                    float eps, int hidden, uint4* xfrag, int m, const float* weights, const float* bias, const X8* x8,
-                   int x8_terms) {
+                   int x8_terms, int blocks, const NormBlocks* nb) {
     if (splits < 0 || splits > 8) {
         set_error("residual add: at most eight partial sums");
         return TSV_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(k_addnorm, dim3(m), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
-                       (_Float16*)xfrag, weights, bias, x8 ? *x8 : X8{}, x8 ? x8_terms : 0);
+    hipLaunchKernelGGL(k_addnorm, dim3(m, blocks), dim3(1024), 0, s, x, partial, splits, ldp, w, eps, hidden,
+                       (_Float16*)xfrag, weights, bias, x8 ? *x8 : X8{}, x8 ? x8_terms : 0, nb ? *nb : NormBlocks{});
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

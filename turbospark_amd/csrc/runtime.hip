@@ -77,6 +77,18 @@ struct tsv_ctx {
     int moe_fp4_terms = 0;
     X8 x8_h{}, x8_e{};
     size_t x8_e_q_stride = 0, x8_e_s_stride = 0;
+    // prompt passes of 64 rows (four blocks of sixteen): every block's rows, fragments, partial sums,
+    // q rows, parameters and rotation table, block after block; allocated at the first such pass
+    struct Wide {
+        bool ok = false, ready = false;
+        float* x = nullptr;
+        uint8_t *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
+        size_t xfb = 0;
+        float* partial = nullptr;
+        uint16_t* q16 = nullptr;
+        VerifyParams *vp = nullptr, *vp_host = nullptr;
+        float2* rope_cs = nullptr;
+    } wide;
     // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
     // sum-of-squares partials, per-XCD partial sums, barrier counters
     bool fused_ffn = false, fused_attn = false;
@@ -780,6 +792,132 @@ int launch_pass(tsv_ctx* c, int m) {
     return rc;
 }
 
+// ---- prompt passes of 64 rows -------------------------------------------------------------
+// producer.rs:122-150 (ChunkedPrefillRunner) feeds a prompt in blocks; here a block of 64 tokens is
+// one pass whose matmuls read every weight tile once for all 64 rows (k_gemm_wide).  The rows are
+// kept as four blocks of sixteen so that everything else -- embedding, norms, the rotating epilogue's
+// cache stores, attention -- is the 16-row pass's own code on block-strided buffers: block b is
+// rows base + 16 b .. base + 16 b + 15, its attention sees the cache up to its own rows, which the
+// q/k/v projection of the same pass has already stored for every block before any block attends.
+// Only for headless passes (no logits wanted) of dense models whose four matmuls are Q4_K with the
+// rotating epilogue, and whose layers are linear caches: a ring layer's slack is 32 rows, fewer than
+// a 64-row pass writes ahead of its first block's window.
+constexpr int WIDE_B = 4;
+
+int wide_prepare(tsv_ctx* c) {
+    tsv_ctx::Wide& w = c->wide;
+    if (w.ready) return TSV_OK;
+    const int qd = c->nq * c->hd;
+    const int kmax = std::max(std::max(c->hidden, qd), c->ffn);
+    w.xfb = xfrag_bytes(kmax);
+    int rc;
+    if ((rc = dev_alloc(c, &w.x, (size_t)WIDE_B * 16 * c->hidden * 4, true)) || (rc = dev_alloc(c, &w.xf_a, WIDE_B * w.xfb, true)) ||
+        (rc = dev_alloc(c, &w.xf_b, WIDE_B * w.xfb, true)) || (rc = dev_alloc(c, &w.xf_c, WIDE_B * w.xfb, true)) ||
+        (rc = dev_alloc(c, &w.partial, (size_t)WIDE_B * c->partial_floats * 4, true)) ||
+        (rc = dev_alloc(c, &w.q16, (size_t)WIDE_B * 16 * qd * 2, true)) || (rc = dev_alloc(c, &w.vp, WIDE_B * sizeof(VerifyParams), true)) ||
+        (rc = dev_alloc(c, &w.rope_cs, (size_t)WIDE_B * 16 * (c->hd / 2) * sizeof(float2), true)))
+        return rc;
+    if (hipHostMalloc((void**)&w.vp_host, WIDE_B * sizeof(VerifyParams)) != hipSuccess) {
+        set_error("prefill: cannot allocate pinned staging memory");
+        return TSV_ERR_DEVICE;
+    }
+    w.ready = true;
+    return TSV_OK;
+}
+
+int launch_wide_pass(tsv_ctx* c, int64_t base) {
+    hipStream_t s = c->stream;
+    tsv_ctx::Wide& w = c->wide;
+    int rc;
+    const int qd = c->nq * c->hd, half = c->hd / 2;
+    for (int b = 0; b < WIDE_B; b++)
+        if ((rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, w.x + (size_t)b * 16 * c->hidden, w.vp + b, 16, c->freqs,
+                               c->rope_mscale, half, w.rope_cs + (size_t)b * 16 * half)))
+            return rc;
+    const NormBlocks nb{(long)16 * c->hidden, (long)c->partial_floats, (long)w.xfb};
+    const size_t pstride = c->partial_floats * 4;
+    const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
+    int prev_splits = 0;
+    for (int l = 0; l < c->n_layers; l++) {
+        LayerW& L = c->layers[l];
+        if ((rc = launch_addnorm(s, w.x, w.partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr,
+                                 nullptr, nullptr, 0, WIDE_B, &nb)))
+            return rc;
+        RopeEpi re{};
+        re.cs = w.rope_cs;
+        re.bias = L.bqkv;
+        re.q16 = w.q16;
+        re.kc = L.kc;
+        re.vc = L.vc;
+        re.nq = c->nq;
+        re.nkv = c->nkv;
+        re.hd = c->hd;
+        re.max_ctx = L.cap;
+        if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
+        for (int b = 0; b < WIDE_B; b++) {
+            AttnArgs aa{};
+            aa.q16 = w.q16 + (size_t)b * 16 * qd;
+            aa.kc = L.kc;
+            aa.vc = L.vc;
+            aa.part_o = c->part_o;
+            aa.part_ml = c->part_ml;
+            aa.xfrag = (uint4*)(w.xf_b + (size_t)b * w.xfb);
+            aa.nq = c->nq;
+            aa.nkv = c->nkv;
+            aa.hd = c->hd;
+            aa.max_ctx = L.cap;
+            aa.ring = false;
+            aa.nch = c->nch;
+            aa.scale = c->attn_scale;
+            aa.window = L.window;
+            aa.sinks = L.sinks;
+            aa.vp = w.vp + b;
+            aa.m_hint = 16;
+            aa.base_hint = (int)(base + 16 * b);
+            if ((rc = launch_attention(s, aa, 16))) return rc;
+        }
+        int sp = splits_for(L.wo, 16, EPI_PARTIAL);
+        if ((rc = launch_gemm_wide(s, L.wo, (const uint4*)w.xf_b, w.xfb, w.partial, pstride, w.vp, sp, EPI_PARTIAL, c->hidden, c->hidden)))
+            return rc;
+        if ((rc = launch_addnorm(s, w.x, w.partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr, L.bo, nullptr,
+                                 0, WIDE_B, &nb)))
+            return rc;
+        if ((rc = launch_gemm_wide(s, L.gate_up, (const uint4*)w.xf_a, w.xfb, w.xf_c, w.xfb, w.vp, 1, EPI_SILU, 0, 0))) return rc;
+        sp = splits_for(L.down, 16, EPI_PARTIAL);
+        if ((rc = launch_gemm_wide(s, L.down, (const uint4*)w.xf_c, w.xfb, w.partial, pstride, w.vp, sp, EPI_PARTIAL, c->hidden, c->hidden)))
+            return rc;
+        prev_splits = sp;
+    }
+    return TSV_OK;  // headless: the last layer's sums are never added, nobody reads these rows' logits
+}
+
+// One 64-row prompt pass at the cursor: parameters of the four blocks, then the kernels.
+int enqueue_wide_prefill(tsv_ctx* c, const int32_t* ids, int64_t base) {
+    const int rows = 16 * WIDE_B;
+    if (base != c->position) {
+        set_error("prefill: start position does not match the KV cursor");
+        return TSV_ERR_INVALID;
+    }
+    if (base + rows > c->max_context) {
+        set_error("prefill: block would write past the KV capacity");
+        return TSV_ERR_INVALID;
+    }
+    int rc = wide_prepare(c);
+    if (rc) return rc;
+    VerifyParams vp[WIDE_B];
+    for (int b = 0; b < WIDE_B; b++)
+        if ((rc = fill_params(vp[b], ids + 16 * b, nullptr, 16, base + 16 * b, c->vocab))) return rc;
+    hipStream_t s = c->stream;
+    TSV_HIP(hipStreamSynchronize(s));  // the pinned staging copy must not be rewritten while a copy is in flight
+    std::memcpy(c->wide.vp_host, vp, sizeof vp);
+    TSV_HIP(hipMemcpyAsync(c->wide.vp, c->wide.vp_host, sizeof vp, hipMemcpyHostToDevice, s));
+    if ((rc = launch_wide_pass(c, base))) return rc;
+    c->position = base + rows;
+    c->high_water = std::max(c->high_water, c->position);
+    c->last_m = 0;  // no logits on the device for tsv_accept to judge
+    return TSV_OK;
+}
+
 int run_pass(tsv_ctx* c, int m) {
     if (!c->use_graph || c->profile || c->headless) return launch_pass(c, m);
     if (!c->pass_graph[m]) {
@@ -1141,6 +1279,13 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         set_error("open: device initialisation failed");
         return fail(TSV_ERR_DEVICE);
     }
+    // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
+    c->wide.ok = c->rewind_budget == INT64_MAX && !c->fused_ffn && !c->fused_attn;
+    for (const LayerW& L : c->layers)
+        if (L.n_experts || !L.rope_fused || L.v_only.tiles || L.qkv.fmt != FMT_Q4K || L.wo.fmt != FMT_Q4K ||
+            L.gate_up.fmt != FMT_Q4K || L.down.fmt != FMT_Q4K)
+            c->wide.ok = false;
+    if (const char* e = getenv("TSV_WIDE_PREFILL")) c->wide.ok = c->wide.ok && e[0] != '0';
     *out = c;
     return TSV_OK;
 }
@@ -1151,6 +1296,7 @@ extern "C" void tsv_close(tsv_ctx* c) {
     for (void* p : c->allocs) (void)hipFree(p);
     if (c->hist_dev) (void)hipFree(c->hist_dev);
     if (c->vp_host) (void)hipHostFree(c->vp_host);
+    if (c->wide.vp_host) (void)hipHostFree(c->wide.vp_host);
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
@@ -1250,7 +1396,14 @@ extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint
 }
 
 static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
-    for (int64_t i = 0; i < n; i += TSV_MAX_ROWS) {
+    const int wide_rows = 16 * WIDE_B;
+    for (int64_t i = 0; i < n;) {
+        // 64 rows at a time while that many remain and nobody wants their logits
+        if (c->wide.ok && !c->profile && n - i >= wide_rows && (i + wide_rows < n || !logits)) {
+            if (int rc = enqueue_wide_prefill(c, ids + i, pos0 + i)) return rc;
+            i += wide_rows;
+            continue;
+        }
         const int m = (int)std::min<int64_t>(TSV_MAX_ROWS, n - i);
         // only the last row's logits are ever handed out: every earlier pass is headless, and so
         // is the last one when the caller takes no logits
@@ -1264,6 +1417,7 @@ static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos
             TSV_HIP(hipMemcpyAsync(logits, c->logits + (size_t)(m - 1) * c->vocab, (size_t)c->vocab * 2,
                                    hipMemcpyDeviceToHost, c->stream));
         }
+        i += m;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
     return check_fused(c);

@@ -150,6 +150,10 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
                 int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
 int gemm_default_splits(const TiledW& w, int m);
+// rows of a prompt-block pass, and the matmul over them in blocks of sixteen (Q4_K weights only)
+int gemm_wide_rows();
+int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t x_stride, void* out, size_t out_stride,
+                     const VerifyParams* vp, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
 
 // ---- routed experts (moe.hip) -----------------------------------------------------------------
 // One routed expert of a pass: the rows that chose it (ascending) and the rank slot it has in
@@ -262,10 +266,15 @@ inline int launch_ffn_block(hipStream_t, int, FfnBlockArgs&, int) { return TSV_E
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
                  const VerifyParams* vp, int m, const float* freqs = nullptr, float mscale = 1.0f, int half = 0,
                  float2* cs = nullptr);
+// Strides between the 16-row blocks of a prompt pass: rows and partial sums in floats, fragments in bytes.
+struct NormBlocks {
+    long x, partial, frag;
+};
 // weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
                    float eps, int hidden, uint4* xfrag, int m, const float* weights = nullptr,
-                   const float* bias = nullptr, const X8* x8 = nullptr, int x8_terms = 0);
+                   const float* bias = nullptr, const X8* x8 = nullptr, int x8_terms = 0, int blocks = 1,
+                   const NormBlocks* nb = nullptr);
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
 
 struct RopeKvArgs {
