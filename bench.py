@@ -122,6 +122,9 @@ PROBES = {
     "gate_up": dict(match="k_gemm<", what="gate/up matmul, 28672 x 4096 Q4_K, M = 5", **GATE_UP_8B),
     # the same weights under sixteen rows (the 16-node tree): the 16x16x32 MFMA form
     "gemm16": dict(match="k_gemm16<", what="gate/up matmul, 28672 x 4096 Q4_K, M = 16", **dict(GATE_UP_8B, m=16)),
+    # the same weights in a 64-row prompt pass (counters over a --prefill-bench run; --counter-summary only)
+    "gemm_wide": dict(match="k_gemm_wide<1>", what="gate/up matmul, 28672 x 4096 Q4_K, 64-row prompt pass",
+                      **dict(GATE_UP_8B, m=64)),
     "attention": dict(match="k_attn_partial", what="attention partial pass, 32 q / 8 kv heads x 128, M = 5, 4096-token context",
                       **ATTN_8B),
 }

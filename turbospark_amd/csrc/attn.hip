@@ -87,7 +87,7 @@ __global__ void k_attn_combine(AttnArgs a, int G, int R) {
     }
     const _Float16 o16 = (_Float16)(num / s_den);
     const int kk = qh * hd + d;
-    ((_Float16*)a.xfrag)[frag_index(kk, m)] = o16;
+    ((_Float16*)a.xfrag)[a.frag16 ? frag16_index(kk, m) : frag_index(kk, m)] = o16;
     // sum of each 32-element sub-block of the output projection's input (32 neighbouring threads)
     float sum = (float)o16;
     for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);

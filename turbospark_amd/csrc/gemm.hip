@@ -470,7 +470,7 @@ __device__ __forceinline__ void epilogue16(const GemmArgs& a, int tile, int spli
 #pragma unroll
             for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o);
             const int b = 4 * kg + i;
-            if (b < M) out[frag_index(col, b)] = h;
+            if (b < M) out[a.out16 ? frag16_index(col, b) : frag_index(col, b)] = h;
             if (r == 0) ssum[pr * 16 + b] = sum;  // this half of the sub-block's sum
         }
         return;
@@ -595,6 +595,9 @@ __global__ __launch_bounds__(512) void k_gemm16(GemmArgs a) {
 // registers; after a barrier every wave multiplies all four row blocks by its own sixteen
 // activation rows.  So the weight bytes, and the vector-ALU work of unpacking them, are spent once
 // per 64 rows, and what is left per row block is matrix instructions.
+// The activations come in the layout of frag16_index (a lane's sixteen bytes of a sub-block side by
+// side: a wave's load is one contiguous KiB; the 16-row kernels' layout costs this kernel four times
+// the bytes in partly used cache lines), which the producers of a prompt pass write on request.
 //
 // The unpacked operand is the integer sc_j * q (at most 63 * 15, exact in fp16), made from the
 // offset codes by one packed fma: (1024 + q) * sc - 1024 * sc and (64 + q) * sc - 64 * sc are exact.
@@ -618,29 +621,33 @@ struct WideW {  // what the unpacking wave holds of one chunk: its row block's c
     u32x2 q[4];
     u32x4 h;
 };
-struct WideX {  // a block's activations of one chunk
-    u32x2 x[8][2];
+struct WideX {  // a block's activations of one chunk: the lane's A operand of every sub-block, and two sums
+    u32x4 v[8];
     float xs[2];
 };
 
+// (the loads of a chunk stay where they are written, scheduling fences on both sides: left alone, the
+// scheduler sinks them to their first use, one chunk later, and nothing is in flight ahead of the math)
 __device__ __forceinline__ void wide_load_w(WideW& w, const uint8_t* tile_chunk, int rb, int lane) {
     const int r = lane & 15, kg = lane >> 4;
     const uint8_t* wp = tile_chunk + ((kg >> 1) * 64 + r) * 16 + (kg & 1) * 8;
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int p = 0; p < 4; p++) w.q[p] = __builtin_nontemporal_load((const u32x2*)(wp + (2 * p * 64 + 16 * rb) * 16));
     w.h = __builtin_nontemporal_load((const u32x4*)(tile_chunk + 8192 + (16 * rb + r) * 16));
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 __device__ __forceinline__ void wide_load_x(WideX& x, const GemmArgs& a, int c, int lane) {
     const int r = lane & 15, kg = lane >> 4;
-    const u32x2* xp = (const u32x2*)a.xfrag + (size_t)c * 1024 + (r >> 2) * 64 + (r & 3) + kg * 8;
-#pragma unroll
-    for (int j = 0; j < 8; j++)
-#pragma unroll
-        for (int t = 0; t < 2; t++) x.x[j][t] = xp[(j >> 1) * 256 + ((j & 1) * 8 + t) * 4];
+    const u32x4* xp = (const u32x4*)a.xfrag + (size_t)c * 512 + lane;  // frag16_index: [sub-block][lane][16 B]
     const float* sp = a.xsum + (size_t)c * 128 + (r >> 2) * 32 + (r & 3) + kg * 4;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; j++) x.v[j] = xp[j * 64];
     x.xs[0] = sp[0];
     x.xs[1] = sp[16];
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // Row block `rb` of a chunk into LDS buffer `buf`.
@@ -711,8 +718,7 @@ __device__ __forceinline__ void wide_compute(const WideX& x, const uint8_t* buf,
 #pragma unroll
     for (int p = 0; p < 4; p++) {
         if (p < 3) fetch((p + 1) & 1, p + 1);
-        const u32x4 alo = {x.x[2 * p][0].x, x.x[2 * p][0].y, x.x[2 * p][1].x, x.x[2 * p][1].y};
-        const u32x4 ahi = {x.x[2 * p + 1][0].x, x.x[2 * p + 1][0].y, x.x[2 * p + 1][1].x, x.x[2 * p + 1][1].y};
+        const u32x4 alo = x.v[2 * p], ahi = x.v[2 * p + 1];
 #pragma unroll
         for (int rb = 0; rb < 4; rb++)
             tq[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, alo), __builtin_bit_cast(half8, blo[p & 1][rb]),
@@ -754,29 +760,38 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa)
 #pragma unroll
     for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
     const int M = a.vp->m;
-    // chunk c: unpack into buffer c & 1 -> ask for chunk c + 1 -> barrier -> multiply chunk c.  The
+    // chunk c: unpack into buffer c & 1 -> ask for what comes next -> barrier -> multiply chunk c.  The
     // barrier of chunk c also separates the reads of chunk c - 1 from the unpacking of chunk c + 1,
-    // which goes to the same buffer.
+    // which goes to the same buffer.  The codes are asked for two chunks ahead, the activations (which
+    // come from L2) one.  No branch surrounds a load -- a chunk index past the slice is clamped to its
+    // last chunk and that chunk is simply asked for again -- so the loop body is one block and the
+    // wait before each use is a count the compiler can know, not "everything".
     WideW w[2];
     WideX x[2];
-    if (s0 < s1) {
-        wide_load_w(w[0], wt + (size_t)s0 * Q4K::TILE_BYTES, wave, lane);
-        wide_load_x(x[0], a, s0, lane);
+    uint8_t* const buf0 = wide_lds;
+    uint8_t* const buf1 = wide_lds + WIDE_BUF_BYTES;
+    const int last = s1 - 1;
+    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * Q4K::TILE_BYTES; };
+    wide_load_w(w[0], tile_at(s0), wave, lane);
+    wide_load_x(x[0], a, s0, lane);
+    wide_load_w(w[1], tile_at(s0 + 1), wave, lane);
+    int c = s0;
+    for (; c + 2 <= s1; c += 2) {
+        wide_unpack(w[0], k, buf0, wave, lane);
+        wide_load_w(w[0], tile_at(c + 2), wave, lane);
+        wide_load_x(x[1], a, min(c + 1, last), lane);
+        __syncthreads();
+        wide_compute(x[0], buf0, acc, lane);
+        wide_unpack(w[1], k, buf1, wave, lane);
+        wide_load_w(w[1], tile_at(c + 3), wave, lane);
+        wide_load_x(x[0], a, min(c + 2, last), lane);
+        __syncthreads();
+        wide_compute(x[1], buf1, acc, lane);
     }
-    for (int c = s0; c < s1; c += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            if (c + u < s1) {
-                uint8_t* buf = wide_lds + u * WIDE_BUF_BYTES;
-                wide_unpack(w[u], k, buf, wave, lane);
-                if (c + u + 1 < s1) {
-                    wide_load_w(w[u ^ 1], wt + (size_t)(c + u + 1) * Q4K::TILE_BYTES, wave, lane);
-                    wide_load_x(x[u ^ 1], a, c + u + 1, lane);
-                }
-                __syncthreads();
-                wide_compute(x[u], buf, acc, lane);
-            }
-        }
+    if (c < s1) {
+        wide_unpack(w[0], k, buf0, wave, lane);
+        __syncthreads();
+        wide_compute(x[0], buf0, acc, lane);
     }
     __syncthreads();  // the sums below reuse no chunk buffer, but every wave must be done with LDS ordering games
     float* ssum = (float*)(wide_lds + 2 * WIDE_BUF_BYTES) + wave * 32;
@@ -929,6 +944,7 @@ int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t 
     if (int rc = fill_gemm_args(wa.g, w, xfrag, out, vp, splits, epi, ldo, n_valid, rope)) return rc;
     wa.x_stride = x_stride;
     wa.out_stride = out_stride;
+    wa.g.out16 = 1;  // what this kernel reads is what it writes for the next one
     const size_t lds = 2 * (size_t)WIDE_BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
     const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
     static bool attr_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel

@@ -212,7 +212,7 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
         u32x2_t hb = __builtin_bit_cast(u32x2_t, h);
         asm volatile("" : "+v"(hb.x), "+v"(hb.y));
         h = __builtin_bit_cast(half4, hb);
-        *(half4*)(xfrag + frag_index(4 * i, m)) = h;
+        *(half4*)(xfrag + (nb.frag16 ? frag16_index(4 * i, m) : frag_index(4 * i, m))) = h;
         float sum = ((float)h.x + (float)h.y) + ((float)h.z + (float)h.w);
         sum += __shfl_xor(sum, 1);
         sum += __shfl_xor(sum, 2);

@@ -834,7 +834,7 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         if ((rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, w.x + (size_t)b * 16 * c->hidden, w.vp + b, 16, c->freqs,
                                c->rope_mscale, half, w.rope_cs + (size_t)b * 16 * half)))
             return rc;
-    const NormBlocks nb{(long)16 * c->hidden, (long)c->partial_floats, (long)w.xfb};
+    const NormBlocks nb{(long)16 * c->hidden, (long)c->partial_floats, (long)w.xfb, 1};
     const size_t pstride = c->partial_floats * 4;
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     int prev_splits = 0;
@@ -874,6 +874,7 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
             aa.vp = w.vp + b;
             aa.m_hint = 16;
             aa.base_hint = (int)(base + 16 * b);
+            aa.frag16 = 1;
             if ((rc = launch_attention(s, aa, 16))) return rc;
         }
         int sp = splits_for(L.wo, 16, EPI_PARTIAL);

@@ -98,6 +98,13 @@ __host__ __device__ inline int frag_index(int k, int row) {
     const int pos = ((k & 1) << 1) | ((k >> 1) & 1);  // k%4 = 0,1,2,3 -> slot 0,2,1,3
     return ((((k >> 6) * 4 + (row >> 2)) * 16 + ((k >> 2) & 15)) * 4 + (row & 3)) * 4 + pos;
 }
+// The same activations as the 64-row prompt kernel reads them: [K / 32][K % 32 / 8][row][8 halfs], the sixteen
+// bytes a lane of v_mfma_f32_16x16x32_f16 holds of its row, so a wave's load is one contiguous KiB.  Within
+// every four K the halfs keep the order above; the sums sit behind, unchanged.
+__host__ __device__ inline int frag16_index(int k, int row) {
+    const int pos = ((k & 1) << 1) | ((k >> 1) & 1);
+    return (((k >> 5) * 4 + ((k >> 3) & 3)) * 16 + row) * 8 + (k & 4) + pos;
+}
 // (K is rounded up to whole 256-element chunks: a matmul whose last chunk is only partly real
 // reads zeros there, never the sums)
 __host__ __device__ inline size_t xfrag_sum_offset(int k) { return (size_t)((k + 255) / 256) * 8192; }
@@ -139,6 +146,7 @@ struct GemmArgs {
                          // next matmul; EPI_LOGITS: half [m][ldo]
     const VerifyParams* vp;
     int n_tiles, kchunks, kslice, splits, kparts, per, ldo, n_valid;
+    int out16;     // EPI_SILU: write the fragments in the prompt kernel's layout (frag16_index)
     RopeEpi rope;  // EPI_ROPE only
 };
 
@@ -269,6 +277,7 @@ int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float
 // Strides between the 16-row blocks of a prompt pass: rows and partial sums in floats, fragments in bytes.
 struct NormBlocks {
     long x, partial, frag;
+    int frag16;  // write the fragments in the prompt kernel's layout (frag16_index)
 };
 // weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
@@ -310,6 +319,7 @@ struct AttnArgs {
     // row count and base position by value when the launch knows them (saves the kernel one
     // dependent memory round trip before its first K/V load); base_hint < 0: read them from vp
     int m_hint, base_hint;
+    int frag16;  // write the output fragments in the prompt kernel's layout (frag16_index)
 };
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);
 int launch_attention_merge(hipStream_t s, const AttnArgs& a, int m);
