@@ -220,6 +220,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="llama3_8b_q4_k_k4_ctx4096", choices=sorted(WORKLOADS))
     ap.add_argument("--layers", type=int, default=None, help="debug: build only this many layers")
+    ap.add_argument("--routing", default="model", choices=["model", "independent"],
+                    help="routed-expert workloads: 'independent' forces every row of every layer onto top_k experts drawn "
+                         "uniformly and independently (tsv_force_route) instead of the synthetic router's own, nearly "
+                         "row-independent choice; a secondary measurement, labelled in the line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=20261125)
     args = ap.parse_args()
@@ -281,6 +285,14 @@ def main():
     base = eng.position
     point = eng.checkpoint()
     anchor = int(prompt[-1])
+    if args.routing == "independent":
+        if not cfg.get("n_experts"):
+            sys.exit("bench.py: --routing independent needs a routed-expert workload")
+        forced = np.full((cfg["n_layers"], 16, 8), -1, np.int32)
+        for l in range(cfg["n_layers"]):
+            for r in range(16):
+                forced[l, r, :cfg["top_k"]] = rng.permutation(cfg["n_experts"])[:cfg["top_k"]]
+        eng.force_route(forced)
 
     # drafter logits N(0,1) per round, resident on the device; proposals drawn on the device
     rounds = args.warmup + args.steps
@@ -411,13 +423,19 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16",
-        "dtype_detail": {12: "q4_k", 8: "q8_0", 30: "bf16"}[cfg["dtype"]] + (" + mxfp4 experts" if cfg.get("n_experts") else "") +
-                        " weight codes as exact f16 x f16 activations on MFMA, "
-                        "f32 accumulate; f64 acceptance",
+        "dtype_detail": {12: "q4_k", 8: "q8_0", 30: "bf16"}[cfg["dtype"]] +
+                        " weight codes as exact f16 x f16 activations on MFMA, f32 accumulate" +
+                        ("" if not cfg.get("n_experts") else
+                         "; mxfp4 experts as f16 x f16 too (TSV_MOE_FP4=0)" if os.environ.get("TSV_MOE_FP4") == "0" else
+                         "; mxfp4 experts as stored on the block-scaled fp4 x fp8 MFMA, activations as " +
+                         ("three" if os.environ.get("TSV_MOE_FP4") == "3" else "two") + " block-scaled e4m3 terms") +
+                        "; f64 acceptance",
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,
                    "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin,
-                   **({"experts_routed_per_layer": round(union, 2)} if union is not None else {})},
+                   **({"experts_routed_per_layer": round(union, 2),
+                       "routing": "the synthetic router's own" if args.routing == "model" else
+                                  "forced: top_k experts per row drawn uniformly and independently"} if union is not None else {})},
         "roofline": roofline, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

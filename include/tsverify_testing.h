@@ -77,6 +77,15 @@ int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, i
  * the oracle's ranking (real_forward_dispatch.rs:1135-1158). */
 int32_t tsv_route_selected(tsv_ctx* ctx, int32_t* out, int32_t n_layers);
 
+/* Makes the routed layers take the experts given instead of each row's own top-k: sel is
+ * [n_layers][16][8] expert ids (row r of a pass at [layer][r], slot order as given; a row whose first
+ * entry is negative routes freely); the weights stay the softmax of the row's own router logits over
+ * the experts taken.  NULL restores free routing.  With the oracle's ranking forced onto the device
+ * (or the device's onto the oracle, tso_model_force_route) the two sides run the same experts on any
+ * input, also one whose ranking sits inside the fp16 rounding of a tie; the bench uses it to time the
+ * expert matmuls under routing that is independent from row to row. */
+int32_t tsv_force_route(tsv_ctx* ctx, const int32_t* sel, int32_t n_layers);
+
 #ifdef __cplusplus
 }
 #endif

@@ -175,3 +175,43 @@ def test_routing_agrees_with_the_oracle_except_within_rounding_of_a_tie(name, ov
     print(f"{name} router shape: {differ} of {rows} routing decisions (a row's expert set in a layer) differ from the oracle's, "
           f"largest margin among them {worst_gap:.2e} of the logit range (bound {bound:.0e})")
     assert differ <= rows // 50
+
+
+@pytest.mark.parametrize("name,over", [("moe_small", {}), ("gptoss_small", {}), ("qwen3_30b_a3b", dict(vocab=4096, n_layers=2)),
+                                       ("gptoss_120b", dict(vocab=4096, n_layers=2))])
+def test_parity_on_unfiltered_inputs_with_the_oracles_routing_forced_onto_the_device(name, over):
+    """No seed is re-drawn here: the oracle routes freely (real_forward_dispatch.rs:1135-1158), its expert
+    sets are forced onto the device (tsv_force_route), and the logits must agree on every input -- also on
+    those where the device's own ranking would have gone the other way inside the rounding of a tie."""
+    import turbospark_amd as ts
+    from oracle import binding as ob
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS[name], max_context=64, **over)
+    w = synth.make_weights(cfg, seed=33, n_layers=cfg["n_layers"])
+    gpu = ts.HipVerifier(cfg, w)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)
+    worst, flips = 0.0, 0
+    rounds = 24 if cfg["hidden"] <= 1024 else 10
+    for rnd in range(rounds):
+        feed = _prompt(1 + rnd % 16, cfg["vocab"], 5000 + rnd)
+        cpu.reset()
+        want = cpu.verify(feed, 0)
+        sel, _ = cpu.route_record()
+        gpu.reset()
+        gpu.force_route(None)
+        free = gpu.verify(feed, 0)
+        own = gpu.route_selected()
+        K = cfg["top_k"]
+        flips += int(np.any(np.sort(own[:, :len(feed), :K], -1) != np.sort(sel[:, :len(feed), :K], -1)))
+        forced = np.full((cfg["n_layers"], 16, 8), -1, np.int32)
+        forced[:, :len(feed), :K] = sel[:, :len(feed), :K]
+        gpu.reset()
+        gpu.force_route(forced)
+        got = gpu.verify(feed, 0)
+        assert np.array_equal(np.sort(gpu.route_selected()[:, :len(feed), :K], -1), np.sort(forced[:, :len(feed), :K], -1))
+        worst = max(worst, gc.logit_error(got, want))
+        assert gc.logit_error(got, want) <= MXFP4_TOL, (rnd, gc.logit_error(got, want))
+        del free
+    gpu.force_route(None)
+    print(f"{name}: {rounds} unfiltered passes under the oracle's routing, worst logit error / range {worst:.2e}; "
+          f"the device's own ranking differed somewhere in {flips} of them")

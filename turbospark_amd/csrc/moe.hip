@@ -99,9 +99,26 @@ __global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
             gather(std::integral_constant<int, 4>{});
         float top = 0.f, sum = 0.f, my_ex = 0.f;
         int my_sel = 0;
+        const bool forced = a.forced && a.forced[m * 8] >= 0;  // the same for the whole wave
+        if (forced) {
+            // lane r < k takes slot r's expert as given and fetches that expert's logit from the lane that holds it
+            const int e = min(max(lane < k ? a.forced[m * 8 + lane] : 0, 0), ne - 1);
+            float l = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float v = __shfl(key_value(key[j]), e & 63);
+                if ((e >> 6) == j) l = v;
+            }
+            top = key_value(wave_umax(lane < k ? order_key(l) : 0u));
+            my_ex = expf(l - top);
+            my_sel = e;
+#pragma unroll
+            for (int r = 0; r < 8; r++)
+                if (r < k) sum += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_ex), r));
+        }
 #pragma unroll
         for (int r = 0; r < 8; r++) {
-            if (r < k) {
+            if (r < k && !forced) {
                 const uint32_t mine = max(max(key[0], key[1]), max(key[2], key[3]));
                 const uint32_t kbest = wave_umax(mine);
                 uint32_t idx = 0xFFFFFFFFu;  // ascending j is ascending index: the first maximum wins

@@ -236,15 +236,15 @@ __global__ __launch_bounds__(512) void k_moe_fp4(MoeGemmArgs a) {
 
 template <int EPI, int TERMS>
 int launch_fp4_t(hipStream_t s, const MoeGemmArgs& a, int n_groups) {
-    // One chunk per wave up to eight chunks (these launches are short: the sooner the tile's bytes are
-    // all asked for, the sooner it is done), three per wave on a longer K (measured at 12 chunks: 4 waves
-    // x 3 beat 6 x 2 and 3 x 4).  One register stage: a second stage in flight (227 VGPRs against 124)
-    // halves the resident waves and measured slower at every shape.  TSV_MOE_FP4_CPW: chunks per wave.
+    // About four waves on a tile (measured at 3, 8 and 12 chunks, with few and with many experts in
+    // play: 3 x 1, 4 x 2 and 4 x 3 beat both more, shorter waves -- whose sums wave 0 then folds alone
+    // -- and fewer, longer ones).  One register stage: a second stage in flight (227 VGPRs against
+    // 124) halves the resident waves and measured slower at every shape.  TSV_MOE_FP4_CPW: chunks per wave.
     static const int forced = [] {
         const char* e = getenv("TSV_MOE_FP4_CPW");
         return e ? std::max(1, atoi(e)) : 0;
     }();
-    const int cpw = forced ? forced : a.kchunks <= 8 ? 1 : 3;
+    const int cpw = forced ? forced : (a.kchunks + 3) / 4;
     const int nw = std::min(8, std::max(1, (a.kchunks + cpw - 1) / cpw));
     const size_t lds = (size_t)std::max(1, nw - 1) * 4 * 1024;
     hipLaunchKernelGGL((k_moe_fp4<EPI, TERMS, 1>), dim3(a.tiles_per_expert, n_groups), dim3(64 * nw), lds, s, a);

@@ -68,6 +68,7 @@ struct tsv_ctx {
     int max_experts = 0;
     float* route_w = nullptr;
     int32_t* route_sel = nullptr;
+    int32_t* route_forced = nullptr;  // test hook (tsv_force_route): [n_layers][16][8], negative = route freely
     MoeGroup* route_groups = nullptr;
     uint8_t* frag_e = nullptr;
     size_t frag_e_stride = 0;
@@ -691,6 +692,7 @@ int launch_pass(tsv_ctx* c, int m) {
             ra2.selected = c->route_sel + (size_t)l * 16 * 8;  // kept per layer: tsv_route_selected reads them back
             ra2.groups = c->route_groups;
             ra2.bias = L.router_bias;
+            ra2.forced = c->route_forced + (size_t)l * 16 * 8;
             MoeGemmArgs g1{}, g2{};
             g1.w = L.gate_up.tiles;
             g1.tiles_per_expert = c->ffn / 32;
@@ -1207,6 +1209,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->partial, pneed * 4, true)) ||
         (c->max_experts &&
          ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, true)) ||
+          (rc = dev_alloc(c, &c->route_forced, (size_t)c->n_layers * 16 * 8 * 4)) ||
           (rc = dev_alloc(c, &c->route_groups, (size_t)TSV_MAX_ROWS * 8 * sizeof(MoeGroup), true)) ||
           (rc = dev_alloc(c, &c->frag_e, (size_t)TSV_MAX_ROWS * 8 * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
           (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)) ||
@@ -1269,6 +1272,8 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             c->fused_ffn = ok;
         }
     }
+    if (c->route_forced && hipMemsetAsync(c->route_forced, 0xFF, (size_t)c->n_layers * 16 * 8 * 4, c->stream) != hipSuccess)
+        return fail(TSV_ERR_DEVICE);  // every entry -1: rows route freely until tsv_force_route says otherwise
     if (hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
         hipHostMalloc((void**)&c->ap_host, sizeof(AcceptParams)) != hipSuccess ||
         hipHostMalloc((void**)&c->res_host, sizeof(AcceptResult)) != hipSuccess ||
@@ -1812,6 +1817,25 @@ extern "C" int32_t tsv_route_selected(tsv_ctx* c, int32_t* out, int32_t n_layers
     }
     TSV_HIP(hipMemcpyAsync(out, c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipStreamSynchronize(c->stream));
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_force_route(tsv_ctx* c, const int32_t* sel, int32_t n_layers) {
+    if (!c || (sel && n_layers != c->n_layers)) {
+        set_error("force_route: null handle or layer count mismatch");
+        return TSV_ERR_INVALID;
+    }
+    if (!c->route_forced) {
+        set_error("force_route: the model has no routed layers");
+        return TSV_ERR_INVALID;
+    }
+    const size_t bytes = (size_t)c->n_layers * 16 * 8 * 4;
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    if (sel) {
+        TSV_HIP(hipMemcpy(c->route_forced, sel, bytes, hipMemcpyHostToDevice));
+    } else {
+        TSV_HIP(hipMemset(c->route_forced, 0xFF, bytes));  // every entry -1: every row routes freely
+    }
     return TSV_OK;
 }
 

@@ -180,6 +180,10 @@ struct MoeRouteArgs {
     int32_t* selected;  // [16][8] expert ids, rank order
     MoeGroup* groups;   // [16 * 8]
     const float* bias;  // nullable: n_experts values added to the logits before the top-k
+    // nullable test hook: [16][8] expert ids a row is to take instead of its own top-k (slot order as
+    // given, the weights still the softmax of the row's own logits over them); a row whose first
+    // entry is negative routes freely
+    const int32_t* forced;
 };
 // Block-scaled fp8 activations: the B operand of the scaled-MFMA expert matmuls (MXFP4 experts).  A
 // value is the sum of `terms` e4m3 numbers, each times the power-of-two scale of its 32-element

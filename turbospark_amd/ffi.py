@@ -246,7 +246,7 @@ EXPORTS = [
     "tsv_prefix_rewind_to", "tsv_prefix_untainted_len", "tsv_prefix_common",
     "tsv_set_prefix_reuse", "tsv_try_reuse_prefix", "tsv_record_committed", "tsv_prefix_len",
     "tsv_gguf_open", "tsv_gguf_close", "tsv_gguf_tensor_count", "tsv_gguf_data_start", "tsv_gguf_tensor",
-    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected",
+    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected", "tsv_force_route",
 ]
 
 _lib = None
@@ -297,6 +297,7 @@ def lib():
         L.tsv_compact_tree.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int32]
         L.tsv_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]
         L.tsv_route_selected.argtypes = [C.c_void_p, C.c_void_p, C.c_int32]
+        L.tsv_force_route.argtypes = [C.c_void_p, C.c_void_p, C.c_int32]
         L.tsv_accept_greedy_noalloc.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32,
                                                 C.c_int64, C.c_void_p, C.c_int32, C.c_uint64, C.c_uint64, C.c_void_p]
         L.tsv_verify_accept.argtypes = [C.c_void_p, C.POINTER(Round), C.POINTER(RoundResultC)]

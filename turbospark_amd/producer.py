@@ -403,6 +403,17 @@ class HipVerifier:
         ffi.check(ffi.lib().tsv_route_selected(self._h, out.ctypes.data, n))
         return out
 
+    def force_route(self, sel):
+        """Test hook: the routed layers take the experts of `sel` ([n_layers, 16, 8], a row whose first entry
+        is negative routes freely) instead of each row's own top-k; None restores free routing."""
+        n = self.cfg["n_layers"]
+        if sel is None:
+            ffi.check(ffi.lib().tsv_force_route(self._h, None, n))
+            return
+        a = np.ascontiguousarray(np.asarray(sel, np.int32))
+        assert a.shape == (n, 16, 8), a.shape
+        ffi.check(ffi.lib().tsv_force_route(self._h, a.ctypes.data, n))
+
     def read_kv(self, layer, pos0, n):
         c = self.cfg
         shape = (n, c["n_kv_heads"], c["head_dim"])
