@@ -29,7 +29,14 @@ int attn_chunks(int nkv) {
 template <int HD, int RT, int STAGES>
 __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) {
     extern __shared__ float xch[];  // [4 slots][PER_LANE values][64 lanes]
-    attn_partial_body<HD, RT, STAGES, false>(a, G, R, blockIdx.x, blockIdx.y, blockIdx.z * RT, xch);
+    // grid z: row groups of the pass, times the 16-row blocks of a prompt pass
+    const int groups = gridDim.z / max(a.blocks, 1), blk = blockIdx.z / groups, grp = blockIdx.z - blk * groups;
+    if (a.blocks > 1) {
+        const AttnArgs v = attn_block_view(a, blk);
+        attn_partial_body<HD, RT, STAGES, false>(v, G, R, blockIdx.x, blockIdx.y, grp * RT, xch);
+        return;
+    }
+    attn_partial_body<HD, RT, STAGES, false>(a, G, R, blockIdx.x, blockIdx.y, grp * RT, xch);
 }
 
 // Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
@@ -42,7 +49,8 @@ __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) 
 // element of all chunks before the (m, l) pairs are looked at (the two groups of loads do not
 // depend on each other), and the kernel is one memory latency instead of two.  NCH == 0: any count.
 template <int NCH>
-__global__ void k_attn_combine(AttnArgs a, int G, int R) {
+__global__ void k_attn_combine(AttnArgs a0, int G, int R) {
+    const AttnArgs a = a0.blocks > 1 ? attn_block_view(a0, blockIdx.z) : a0;
     __shared__ float wgt[64];
     __shared__ float s_den;
     const int m = blockIdx.x, qh = blockIdx.y, d = threadIdx.x;
@@ -104,7 +112,7 @@ static int launch_partial(hipStream_t s, const AttnArgs& a, int G, int R, int gr
                                     (int)lds));
         raised = true;
     }
-    hipLaunchKernelGGL((k_attn_partial<HD, RT, STAGES>), dim3(a.nch, a.nkv, groups), dim3(512), lds, s, a, G, R);
+    hipLaunchKernelGGL((k_attn_partial<HD, RT, STAGES>), dim3(a.nch, a.nkv, groups * std::max(a.blocks, 1)), dim3(512), lds, s, a, G, R);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -120,7 +128,7 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     // about one workgroup per compute unit: the chunk count shrinks as the row groups multiply
     // (fewer, longer chunks also mean fewer partial results for the merge to read)
     AttnArgs a = a0;
-    a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 256 / (a0.nkv * groups)));
+    a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 256 / (a0.nkv * groups * std::max(a0.blocks, 1))));
     int rc;
     if (trt <= 1)
         rc = launch_partial<HD, 1, 3>(s, a, G, R, 1);
@@ -132,7 +140,7 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
 
 template <int HD>
 static int launch_combine(hipStream_t s, const AttnArgs& a, int m, int G, int R) {
-    const dim3 cgrid(m, a.nq), cblock(HD < 64 ? 64 : HD);
+    const dim3 cgrid(m, a.nq, std::max(a.blocks, 1)), cblock(HD < 64 ? 64 : HD);
     // the chunk count as a compile-time constant puts every partial's load in flight before the
     // first add (a counted loop waits on each in turn); the sum runs in the same order either way
 #define TSV_COMBINE(N) \

@@ -239,7 +239,7 @@ int launch_fp4_t(hipStream_t s, const MoeGemmArgs& a, int n_groups) {
     // About four waves on a tile (measured at 3, 8 and 12 chunks, with few and with many experts in
     // play: 3 x 1, 4 x 2 and 4 x 3 beat both more, shorter waves -- whose sums wave 0 then folds alone
     // -- and fewer, longer ones).  One register stage: a second stage in flight (227 VGPRs against
-    // 124) halves the resident waves and measured slower at every shape.  TSV_MOE_FP4_CPW: chunks per wave.
+    // 124) halves the resident waves and measured slower at every shape, also where a wave has exactly two chunks to walk.  TSV_MOE_FP4_CPW: chunks per wave.
     static const int forced = [] {
         const char* e = getenv("TSV_MOE_FP4_CPW");
         return e ? std::max(1, atoi(e)) : 0;

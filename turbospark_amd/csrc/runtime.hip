@@ -89,6 +89,8 @@ struct tsv_ctx {
         uint16_t* q16 = nullptr;
         VerifyParams *vp = nullptr, *vp_host = nullptr;
         float2* rope_cs = nullptr;
+        float *part_o = nullptr, *part_ml = nullptr;  // attention partials of every block
+        size_t part_o_stride = 0, part_ml_stride = 0;
     } wide;
     // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
     // sum-of-squares partials, per-XCD partial sums, barrier counters
@@ -819,6 +821,11 @@ int wide_prepare(tsv_ctx* c) {
         (rc = dev_alloc(c, &w.q16, (size_t)WIDE_B * 16 * qd * 2, true)) || (rc = dev_alloc(c, &w.vp, WIDE_B * sizeof(VerifyParams), true)) ||
         (rc = dev_alloc(c, &w.rope_cs, (size_t)WIDE_B * 16 * (c->hd / 2) * sizeof(float2), true)))
         return rc;
+    const size_t rows_max = (size_t)TSV_MAX_ROWS * (c->nq / c->nkv);
+    w.part_o_stride = (size_t)c->nkv * c->nch * rows_max * c->hd;
+    w.part_ml_stride = (size_t)c->nkv * c->nch * rows_max * 2;
+    if ((rc = dev_alloc(c, &w.part_o, WIDE_B * w.part_o_stride * 4, true)) || (rc = dev_alloc(c, &w.part_ml, WIDE_B * w.part_ml_stride * 4, true)))
+        return rc;
     if (hipHostMalloc((void**)&w.vp_host, WIDE_B * sizeof(VerifyParams)) != hipSuccess) {
         set_error("prefill: cannot allocate pinned staging memory");
         return TSV_ERR_DEVICE;
@@ -856,14 +863,15 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         re.hd = c->hd;
         re.max_ctx = L.cap;
         if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
-        for (int b = 0; b < WIDE_B; b++) {
+        {
+            // all four blocks in one launch: block b attends with its own base position base + 16 b
             AttnArgs aa{};
-            aa.q16 = w.q16 + (size_t)b * 16 * qd;
+            aa.q16 = w.q16;
             aa.kc = L.kc;
             aa.vc = L.vc;
-            aa.part_o = c->part_o;
-            aa.part_ml = c->part_ml;
-            aa.xfrag = (uint4*)(w.xf_b + (size_t)b * w.xfb);
+            aa.part_o = w.part_o;
+            aa.part_ml = w.part_ml;
+            aa.xfrag = (uint4*)w.xf_b;
             aa.nq = c->nq;
             aa.nkv = c->nkv;
             aa.hd = c->hd;
@@ -873,10 +881,15 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
             aa.scale = c->attn_scale;
             aa.window = L.window;
             aa.sinks = L.sinks;
-            aa.vp = w.vp + b;
+            aa.vp = w.vp;
             aa.m_hint = 16;
-            aa.base_hint = (int)(base + 16 * b);
+            aa.base_hint = (int)base;
             aa.frag16 = 1;
+            aa.blocks = WIDE_B;
+            aa.q_stride = (size_t)16 * qd;
+            aa.part_o_stride = w.part_o_stride;
+            aa.part_ml_stride = w.part_ml_stride;
+            aa.frag_stride = w.xfb;
             if ((rc = launch_attention(s, aa, 16))) return rc;
         }
         int sp = splits_for(L.wo, 16, EPI_PARTIAL);

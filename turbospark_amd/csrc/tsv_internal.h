@@ -324,7 +324,24 @@ struct AttnArgs {
     // dependent memory round trip before its first K/V load); base_hint < 0: read them from vp
     int m_hint, base_hint;
     int frag16;  // write the output fragments in the prompt kernel's layout (frag16_index)
+    // a prompt pass of several 16-row blocks in one launch (blocks > 1): block b has its parameters at vp + b,
+    // its base position at base_hint + 16 b, and its q rows, partial results and output fragments at the
+    // strides below
+    int blocks;
+    size_t q_stride, part_o_stride, part_ml_stride;  // elements
+    size_t frag_stride;                              // bytes
 };
+// the view of one block of such a launch
+__host__ __device__ inline AttnArgs attn_block_view(const AttnArgs& a, int b) {
+    AttnArgs v = a;
+    v.q16 = a.q16 + (size_t)b * a.q_stride;
+    v.part_o = a.part_o + (size_t)b * a.part_o_stride;
+    v.part_ml = a.part_ml + (size_t)b * a.part_ml_stride;
+    v.xfrag = (uint4*)((char*)a.xfrag + (size_t)b * a.frag_stride);
+    v.vp = a.vp + b;
+    if (a.base_hint >= 0) v.base_hint = a.base_hint + 16 * b;
+    return v;
+}
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);
 int launch_attention_merge(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
