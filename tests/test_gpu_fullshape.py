@@ -228,6 +228,40 @@ def test_llama3_8b_all_32_layers_generation_loop_properties():
     assert sampled["min_margin"] >= 0.0
 
 
+def test_llama3_8b_all_32_layers_prompt_in_blocks_of_64_against_16_row_passes():
+    """The headline configuration at its real depth: a 1000-token prompt fed in 64-row passes (producer.rs:122-150)
+    leaves the cache and the following logits of the same prompt fed in 16-row passes, which the smaller cases hold
+    to the oracle.  The two paths multiply the same integers by the same fp16 activations in another order of fp32
+    additions, so they agree to a few fp16 ulps per layer; the tail of 40 tokens goes in 16-row passes in both."""
+    import os
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS["llama3_8b_q4_k"], max_context=1088)
+    w = synth.make_weights(cfg, seed=3)
+    rng = np.random.default_rng(8)
+    prompt = rng.integers(0, cfg["vocab"], 1000).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    out = {}
+    for wide in (True, False):
+        os.environ["TSV_WIDE_PREFILL"] = "1" if wide else "0"
+        try:
+            gpu = ts.HipVerifier(cfg, w)
+        finally:
+            del os.environ["TSV_WIDE_PREFILL"]
+        gpu.prefill(prompt, 0, want_logits=False)
+        assert gpu.position == 1000
+        kv = [gpu.read_kv(layer, 0, 1000) for layer in (0, 15, 31)]
+        out[wide] = (kv, gpu.verify(feed, 1000))
+        del gpu
+    for (kw, vw), (kn, vn) in zip(out[True][0], out[False][0]):
+        for a, b in ((kw, kn), (vw, vn)):
+            a, b = a.astype(np.float32), b.astype(np.float32)
+            assert np.abs(a - b).max() <= 1e-2 * np.abs(b).max()
+    err = gc.logit_error(out[True][1], out[False][1])
+    print(f"8B shape, 32 layers, 1000-token prompt: logits after 64-row passes vs after 16-row passes {err:.2e}")
+    assert err <= 5e-3
+
+
 def test_qwen3_30b_a3b_shape_two_layers_at_long_context():
     """Configuration 4 at its own geometry: hidden 2048, 32q / 4kv x 128 with the per-head q / k norm,
     128 MXFP4 experts of width 768 routed top-8, Q8_0 attention / router / head, the full 151 936-row
