@@ -793,7 +793,7 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa)
         __syncthreads();
         wide_compute(x[0], buf0, acc, lane);
     }
-    __syncthreads();  // the sums below reuse no chunk buffer, but every wave must be done with LDS ordering games
+    __syncthreads();  // every wave is done with the chunk buffers before the epilogue's sums go to LDS behind them
     float* ssum = (float*)(wide_lds + 2 * WIDE_BUF_BYTES) + wave * 32;
 #pragma unroll
     for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
