@@ -277,6 +277,95 @@ def causal_attention(q, k, v, head_dim, nq, nkv, seq_len, window=0, scale=0.0, s
     return out
 
 
+# ----------------------------------------------------------------- TurboQuant KV codec (tq.cpp)
+TQ_KEY_SEED, TQ_VALUE_SEED = 0, 1   # kv_quant.rs:33-36
+
+
+def tq_sign_vector(dim, seed):
+    out = np.empty(dim, np.float32)
+    lib().tso_tq_sign_vector(dim, C.c_uint64(seed), _p(out))
+    return out
+
+
+def tq_wht(x):
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty_like(x)
+    lib().tso_tq_wht(_p(x), x.size, _p(y))
+    return y
+
+
+def tq_rht(x, signs, inverse=False):
+    x, signs = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(signs, np.float32)
+    y = np.empty_like(x)
+    (lib().tso_tq_rht_inverse if inverse else lib().tso_tq_rht_forward)(_p(x), _p(signs), x.size, _p(y))
+    return y
+
+
+def tq_codebook(dim, bits):
+    out = np.empty(max(1 << bits, 1), np.float32)
+    n = lib().tso_tq_codebook(dim, bits, _p(out))
+    return out[:n].copy()
+
+
+def tq_midpoints(codebook):
+    cb = np.ascontiguousarray(codebook, np.float32)
+    out = np.empty(max(cb.size - 1, 0), np.float32)
+    lib().tso_tq_midpoints(_p(cb), cb.size, _p(out))
+    return out
+
+
+def tq_packed_words(length, bits):
+    return lib().tso_tq_packed_words(length, bits)
+
+
+def tq_pack(indices, bits):
+    idx = np.ascontiguousarray(indices, np.uint32)
+    out = np.zeros(max(tq_packed_words(idx.size, bits), 1) + 1, np.uint32)
+    n = lib().tso_tq_pack(_p(idx), idx.size, bits, _p(out))
+    if n < 0:
+        raise ValueError("index does not fit, or bits outside 1..16")
+    return out[:n].copy()
+
+
+def tq_unpack(packed, bits, length):
+    pk = np.ascontiguousarray(np.concatenate([np.asarray(packed, np.uint32), np.zeros(1, np.uint32)]))
+    out = np.zeros(length, np.uint32)
+    if lib().tso_tq_unpack(_p(pk), bits, length, _p(out)) < 0:
+        raise ValueError("bits outside 1..16")
+    return out
+
+
+def tq_quantize_row(x, signs, midpoints, bits):
+    x, signs, mp = (np.ascontiguousarray(a, np.float32) for a in (x, signs, midpoints))
+    words = np.zeros(tq_packed_words(x.size, bits) + 1, np.uint32)
+    norm = C.c_float(0)
+    lib().tso_tq_quantize_row(_p(x), x.size, _p(signs), _p(mp), bits, C.byref(norm), _p(words))
+    return norm.value, words[:-1].copy()
+
+
+def tq_dequantize_row(norm, words, signs, codebook, bits, dim):
+    pk = np.ascontiguousarray(np.concatenate([np.asarray(words, np.uint32), np.zeros(1, np.uint32)]))
+    signs, cb = np.ascontiguousarray(signs, np.float32), np.ascontiguousarray(codebook, np.float32)
+    out = np.empty(dim, np.float32)
+    lib().tso_tq_dequantize_row(C.c_float(norm), _p(pk), _p(signs), _p(cb), bits, dim, _p(out))
+    return out
+
+
+def tq_attention(q, k_words, k_norms, v_words, v_norms, hd, nq, nkv, seq_len, bits, k_signs, k_cb, v_signs, v_cb,
+                 scale=0.0, sinks=None):
+    """kv_quant_attention.rs:58-136.  k / v words: [seq_len, nkv, words per row] uint32, norms [seq_len, nkv]."""
+    q = np.ascontiguousarray(q, np.float32)
+    kw = np.ascontiguousarray(np.concatenate([np.asarray(k_words, np.uint32).reshape(-1), np.zeros(1, np.uint32)]))
+    vw = np.ascontiguousarray(np.concatenate([np.asarray(v_words, np.uint32).reshape(-1), np.zeros(1, np.uint32)]))
+    kn, vn = np.ascontiguousarray(k_norms, np.float32), np.ascontiguousarray(v_norms, np.float32)
+    ks, kc, vs, vc = (np.ascontiguousarray(a, np.float32) for a in (k_signs, k_cb, v_signs, v_cb))
+    out = np.empty(nq * hd, np.float32)
+    sp = _p(np.ascontiguousarray(sinks, np.float32)) if sinks is not None else None
+    lib().tso_tq_attention(_p(q), _p(kw), _p(kn), _p(vw), _p(vn), hd, nq, nkv, seq_len, C.c_float(scale), sp,
+                           _p(ks), _p(kc), _p(vs), _p(vc), bits, _p(out))
+    return out
+
+
 # ----------------------------------------------------------------- selection
 def _hist(history):
     h = np.ascontiguousarray(history if history is not None else [], np.int32)

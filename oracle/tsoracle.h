@@ -125,6 +125,25 @@ void tso_attention_core(const float* q, const float* k, const float* v, int head
                         int n_extra, float scale, const float* sinks, float* out);
 float tso_silu(float x);
 
+/* ---- TurboQuant KV-cache codec (tq.cpp; crates/compute/src/kv_quant.rs, kv_quant_attention.rs, wht.rs) ---- */
+void tso_tq_sign_vector(int dim, uint64_t seed, float* out);                        /* kv_quant.rs:68-81 */
+void tso_tq_wht(const float* x, int n, float* y);                                   /* wht.rs:5-29, normalized */
+void tso_tq_rht_forward(const float* x, const float* signs, int n, float* y);       /* kv_quant.rs:90-94 */
+void tso_tq_rht_inverse(const float* x, const float* signs, int n, float* y);       /* kv_quant.rs:102-107 */
+int tso_tq_codebook(int dim, int bits, float* out);                                 /* kv_quant.rs:166-256 */
+void tso_tq_midpoints(const float* codebook, int levels, float* out);               /* kv_quant.rs:262-264 */
+int tso_tq_packed_words(int length, int bits);                                      /* kv_quant.rs:276-282 */
+int tso_tq_pack(const uint32_t* indices, int length, int bits, uint32_t* packed);   /* kv_quant.rs:289-312; -1: refused */
+int tso_tq_unpack(const uint32_t* packed, int bits, int length, uint32_t* indices); /* kv_quant.rs:315-334 */
+void tso_tq_quantize_row(const float* x, int dim, const float* signs, const float* midpoints, int bits, float* norm_out,
+                         uint32_t* words);                                           /* kv_quant.rs:349-362 */
+void tso_tq_dequantize_row(float norm, const uint32_t* words, const float* signs, const float* codebook, int bits, int dim,
+                           float* out);                                              /* kv_quant.rs:367-379 */
+void tso_tq_attention(const float* q, const uint32_t* k_words, const float* k_norms, const uint32_t* v_words,
+                      const float* v_norms, int hd, int nq, int nkv, int seq_len, float scale, const float* sinks,
+                      const float* k_signs, const float* k_codebook, const float* v_signs, const float* v_codebook, int bits,
+                      float* out);                                                   /* kv_quant_attention.rs:58-136 */
+
 /* ---- selection --------------------------------------------------------- */
 typedef struct {
     double temperature;

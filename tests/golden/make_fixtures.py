@@ -8,6 +8,8 @@ Reads files below /root/reference as text / data only (nothing is imported or ru
   * the hand-packed Q4_K superblock constants of crates/compute/tests/quant_gguf.rs:226-267
     -> q4k_handpacked.json
   * the llama-3 rope factor profile of crates/compute/src/rope.rs:471-482 -> llama3_rope_profile.json
+  * the literal arrays of crates/compute/tests/generated/kv_quant_oracle.rs (TurboQuant KV codec: sign
+    vectors, codebooks, input rows, norms and packed words of four (dim, bits) shapes)  -> kv_quant_oracle.json
   * five MLX known-answer fixtures (config.json, model.safetensors, traces.json) of
     crates/audio/testdata/lm/{llama_default,llama_llama3_rope,qwen3_default,llama_yarn_rope,qwen2_default}
     -> lm/<name>/
@@ -53,6 +55,18 @@ def main():
     }
     assert len(q5["bytes"]) == 352 and len(q5["floats"]) == 512
     json.dump(q5, open(f"{OUT}/q5k_ggml_oracle.json", "w"))
+
+    src = open(f"{REF}/crates/compute/tests/generated/kv_quant_oracle.rs").read()
+    tq = {"source": "crates/compute/tests/generated/kv_quant_oracle.rs", "rows_per_shape": 4, "shapes": []}
+    for dim, bits in ((64, 2), (64, 3), (128, 4), (256, 3)):
+        tag = f"D{dim}B{bits}"
+        f32 = lambda name: [float(v.replace("f32", "")) for v in rust_array(src, f"{tag}_{name}")]
+        shape = {"dim": dim, "bits": bits, "signs": f32("SIGNS"), "codebook": f32("CODEBOOK"), "input_rows": f32("INPUT_ROWS"),
+                 "norms": f32("NORMS"), "packed": [int(v.replace("u32", ""), 0) for v in rust_array(src, f"{tag}_PACKED")]}
+        assert len(shape["signs"]) == dim and len(shape["codebook"]) == 1 << bits and len(shape["input_rows"]) == 4 * dim
+        assert len(shape["packed"]) == 4 * ((dim * bits + 31) // 32)
+        tq["shapes"].append(shape)
+    json.dump(tq, open(f"{OUT}/kv_quant_oracle.json", "w"))
 
     src = open(f"{REF}/crates/compute/tests/quant_gguf.rs").read()
     q4 = {
