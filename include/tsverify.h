@@ -94,6 +94,13 @@ typedef struct {
      * (min(g, limit) / (1 + exp(-alpha * min(g, limit)))) * (clamp(u, -limit, limit) + 1)
      * (crates/gpu/src/shaders/moe_gguf.metal:528-556), instead of silu(g) * u. */
     float act_alpha, act_limit;
+    /* TurboQuant KV rows (crates/model-io/src/kv_quant.rs:25-72): bits per key and per value coordinate,
+     * both 0 for fp16 rows everywhere; the pairs --kv-bits can name are 2/2, 3/3, 3/4 ("3.5") and 4/4.
+     * Quantized are the full-attention layers (window == 0), all of them in a stack of at most two, else
+     * all but the last (kv_quant.rs:102-107); such a layer keeps one f32 norm and the packed codebook
+     * indices per position and kv head, 4 + 4 * ceil(head_dim * bits / 32) bytes (kv_quant.rs:141-144).
+     * tsv_compact_tree, and with it tree rounds, are refused on such a handle. */
+    int32_t kv_k_bits, kv_v_bits;
 } tsv_model_desc;
 
 typedef struct tsv_ctx tsv_ctx;

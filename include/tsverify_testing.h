@@ -71,6 +71,27 @@ int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, i
                       int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
                       int32_t window, const float* sinks, uint16_t* out);
 
+/* The tables the quantized KV rows are coded with, computed on the host (no GPU needed): head_dim signs
+ * (crates/compute/src/kv_quant.rs:68-81, seed 0 for keys and 1 for values), the 1 << bits Lloyd-Max levels
+ * (kv_quant.rs:166-256) and their (1 << bits) - 1 midpoints (kv_quant.rs:262-264). */
+int32_t tsv_kv_quant_tables(int32_t head_dim, int32_t bits, int32_t value_side, float* signs, float* codebook,
+                            float* midpoints);
+
+/* The stored rows of a quantized layer as they lie in memory: n x n_kv_heads x (1 + words) u32 per side,
+ * the f32 norm first, then ceil(head_dim * bits / 32) words of LSB-first codebook indices -- the row
+ * crates/gpu/tests/kv_quantize_parity.rs:22-38 reads back. */
+int32_t tsv_read_kv_quantized(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint32_t* k_rows, uint32_t* v_rows);
+
+/* One verify-pass attention over quantized rows through the kernels the forward uses (the parity hook
+ * of crates/gpu/tests/kv_quantize_parity.rs and attention_tq_parity.rs).  k, v: (base + m) x nkv x hd
+ * fp16 staging rows; every one is quantized (the first `base` ahead of the pass, then wiped from the
+ * fp16 side so that attention sees them only as decoded), row i of the pass sits at position base + i
+ * and sees positions 0 .. base + i.  out: m x nq x hd fp16; k_rows / v_rows: the stored rows of all
+ * base + m positions in tsv_read_kv_quantized's layout. */
+int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq, int32_t nkv,
+                                int32_t hd, int64_t base, int32_t k_bits, int32_t v_bits, float scale, const float* sinks,
+                                uint16_t* out, uint32_t* k_rows, uint32_t* v_rows);
+
 /* The experts every row of the last pass chose in every routed layer: out is [n_layers][16][8] expert
  * ids in rank order (row r of the pass at [layer][r], the first top_k entries of a row are valid).
  * What the bench counts the expert bytes actually read from, and what the routing tests compare with

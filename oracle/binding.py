@@ -96,6 +96,7 @@ class ModelDesc(C.Structure):
         ("layers", C.POINTER(Layer)),
         ("rope_freqs", C.POINTER(C.c_float)), ("rope_mscale", C.c_float),
         ("act_alpha", C.c_float), ("act_limit", C.c_float),
+        ("kv_k_bits", C.c_int32), ("kv_v_bits", C.c_int32),
     ]
 
 
@@ -352,8 +353,9 @@ def tq_dequantize_row(norm, words, signs, codebook, bits, dim):
 
 
 def tq_attention(q, k_words, k_norms, v_words, v_norms, hd, nq, nkv, seq_len, bits, k_signs, k_cb, v_signs, v_cb,
-                 scale=0.0, sinks=None):
-    """kv_quant_attention.rs:58-136.  k / v words: [seq_len, nkv, words per row] uint32, norms [seq_len, nkv]."""
+                 scale=0.0, sinks=None, v_bits=None):
+    """kv_quant_attention.rs:58-136.  k / v words: [seq_len, nkv, words per row] uint32, norms [seq_len, nkv];
+    bits is the key width and, unless v_bits is given, the value width too."""
     q = np.ascontiguousarray(q, np.float32)
     kw = np.ascontiguousarray(np.concatenate([np.asarray(k_words, np.uint32).reshape(-1), np.zeros(1, np.uint32)]))
     vw = np.ascontiguousarray(np.concatenate([np.asarray(v_words, np.uint32).reshape(-1), np.zeros(1, np.uint32)]))
@@ -362,7 +364,7 @@ def tq_attention(q, k_words, k_norms, v_words, v_norms, hd, nq, nkv, seq_len, bi
     out = np.empty(nq * hd, np.float32)
     sp = _p(np.ascontiguousarray(sinks, np.float32)) if sinks is not None else None
     lib().tso_tq_attention(_p(q), _p(kw), _p(kn), _p(vw), _p(vn), hd, nq, nkv, seq_len, C.c_float(scale), sp,
-                           _p(ks), _p(kc), _p(vs), _p(vc), bits, _p(out))
+                           _p(ks), _p(kc), _p(vs), _p(vc), bits, bits if v_bits is None else v_bits, _p(out))
     return out
 
 
@@ -517,7 +519,8 @@ class Model:
     (dtype, uint8 ndarray, rows, cols).  The arrays must outlive the model.
     """
 
-    def __init__(self, cfg, weights, round_kv_f16=True, threads=1):
+    def __init__(self, cfg, weights, round_kv_f16=True, threads=1, kv_bits=None):
+        """kv_bits: None (fp16 rows) or (key bits, value bits) of the TurboQuant KV codec."""
         self._keep = weights
         n = cfg["n_layers"]
         self._layers = (Layer * n)()
@@ -547,6 +550,7 @@ class Model:
         d.act_limit = cfg.get("act_limit", 0.0)
         d.round_kv_f16 = int(round_kv_f16)
         d.threads = threads
+        d.kv_k_bits, d.kv_v_bits = kv_bits if kv_bits else (0, 0)
         d.embed = _tensor(weights["embed"])
         d.final_norm = _tensor(weights["final_norm"])
         d.lm_head = _tensor(weights.get("lm_head"))
@@ -562,6 +566,9 @@ class Model:
     @property
     def position(self):
         return lib().tso_model_position(self._h)
+
+    def layer_quantized(self, layer):
+        return bool(lib().tso_model_layer_quantized(self._h, layer))
 
     def reset(self):
         lib().tso_model_reset(self._h)

@@ -35,6 +35,12 @@ struct tso_model {
     std::vector<float> route_gap;
     // test hook: expert ids to take instead of the top-k, same shape (empty: route normally)
     std::vector<int32_t> forced_sel;
+    // TurboQuant KV: sign vectors, codebooks and midpoints of the key and the value side
+    std::vector<float> tq_k_signs, tq_v_signs, tq_k_cb, tq_v_cb, tq_k_mid, tq_v_mid;
+    bool quantized(int layer) const {  // model-io/src/kv_quant.rs:102-107
+        if (d.kv_k_bits <= 0 || layers[layer].window != 0) return false;
+        return d.n_layers <= 2 || layer + 1 < d.n_layers;
+    }
 };
 
 namespace {
@@ -141,8 +147,23 @@ extern "C" tso_model* tso_model_create(const tso_model_desc* desc) {
         m->d.rope_factors = nullptr;
     }
     if (!(m->d.rope_mscale > 0.0f)) m->d.rope_mscale = 1.0f;
+    if (m->d.kv_k_bits > 0) {  // kv_quant_attention.rs:24-44: one table set per side, KEY_SEED 0 and VALUE_SEED 1
+        if (m->d.kv_v_bits <= 0) m->d.kv_v_bits = m->d.kv_k_bits;
+        const int hd = desc->head_dim;
+        auto side = [&](int bits, uint64_t seed, std::vector<float>& signs, std::vector<float>& cb, std::vector<float>& mid) {
+            signs.resize(hd);
+            tso_tq_sign_vector(hd, seed, signs.data());
+            cb.resize((size_t)1 << bits);
+            tso_tq_codebook(hd, bits, cb.data());
+            mid.resize(cb.size());  // one spare
+            tso_tq_midpoints(cb.data(), (int)cb.size(), mid.data());
+        };
+        side(m->d.kv_k_bits, 0, m->tq_k_signs, m->tq_k_cb, m->tq_k_mid);
+        side(m->d.kv_v_bits, 1, m->tq_v_signs, m->tq_v_cb, m->tq_v_mid);
+    }
     return m;
 }
+extern "C" int tso_model_layer_quantized(const tso_model* m, int layer) { return m->quantized(layer) ? 1 : 0; }
 
 extern "C" void tso_model_destroy(tso_model* m) { delete m; }
 extern "C" float tso_model_route_margin(const tso_model* m) { return m->route_margin; }
@@ -265,6 +286,26 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
             for (int i = 0; i < kvd; i++) {
                 kd[i] = d.round_kv_f16 ? round_f16(kk[(size_t)m * kvd + i]) : kk[(size_t)m * kvd + i];
                 vd[i] = d.round_kv_f16 ? round_f16(vv[(size_t)m * kvd + i]) : vv[(size_t)m * kvd + i];
+            }
+            if (mdl->quantized(l)) {
+                // kv_write.rs:66-118: the fp16 staging row is quantized into the slot, head by head;
+                // attention then sees what the codes decode to (kv_quant_attention.rs:58-136 computes
+                // the same sums in the rotated space)
+                std::vector<uint32_t> words((size_t)hd + 1);
+                std::vector<float> back((size_t)hd);
+                for (int h = 0; h < nkv; h++) {
+                    float norm;
+                    tso_tq_quantize_row(kd + (size_t)h * hd, hd, mdl->tq_k_signs.data(), mdl->tq_k_mid.data(), d.kv_k_bits, &norm,
+                                        words.data());
+                    tso_tq_dequantize_row(norm, words.data(), mdl->tq_k_signs.data(), mdl->tq_k_cb.data(), d.kv_k_bits, hd,
+                                          back.data());
+                    std::memcpy(kd + (size_t)h * hd, back.data(), sizeof(float) * hd);
+                    tso_tq_quantize_row(vd + (size_t)h * hd, hd, mdl->tq_v_signs.data(), mdl->tq_v_mid.data(), d.kv_v_bits, &norm,
+                                        words.data());
+                    tso_tq_dequantize_row(norm, words.data(), mdl->tq_v_signs.data(), mdl->tq_v_cb.data(), d.kv_v_bits, hd,
+                                          back.data());
+                    std::memcpy(vd + (size_t)h * hd, back.data(), sizeof(float) * hd);
+                }
             }
         }
         std::vector<float> sinks;

@@ -236,12 +236,13 @@ void tso_tq_dequantize_row(float norm, const uint32_t* words, const float* signs
 }
 
 // kv_quant_attention.rs:58-136: one query position over seq_len quantized rows.  q: [nq][hd]; k / v words:
-// [seq_len][nkv][words per row], norms [seq_len][nkv]; scale <= 0: 1 / sqrt(hd); sinks nullable [nq].
+// [seq_len][nkv][words per row], norms [seq_len][nkv]; scale <= 0: 1 / sqrt(hd); sinks nullable [nq].  The two
+// sides carry their own tables and widths (kv_quant_attention.rs:24-44).
 void tso_tq_attention(const float* q, const uint32_t* k_words, const float* k_norms, const uint32_t* v_words,
                       const float* v_norms, int hd, int nq, int nkv, int seq_len, float scale, const float* sinks,
-                      const float* k_signs, const float* k_codebook, const float* v_signs, const float* v_codebook, int bits,
-                      float* out) {
-    const int group = nq / nkv, wpr = tso_tq_packed_words(hd, bits);
+                      const float* k_signs, const float* k_codebook, const float* v_signs, const float* v_codebook, int k_bits,
+                      int v_bits, float* out) {
+    const int group = nq / nkv, k_wpr = tso_tq_packed_words(hd, k_bits), v_wpr = tso_tq_packed_words(hd, v_bits);
     if (!(scale > 0.0f)) scale = 1.0f / std::sqrt((float)hd);
     std::vector<float> q_rot((size_t)hd), scores((size_t)seq_len), acc_rot((size_t)hd), acc((size_t)hd);
     std::vector<uint32_t> idx((size_t)hd);
@@ -250,7 +251,7 @@ void tso_tq_attention(const float* q, const uint32_t* k_words, const float* k_no
         tso_tq_rht_forward(q + (size_t)qh * hd, k_signs, hd, q_rot.data());
         for (int p = 0; p < seq_len; p++) {
             const size_t row = (size_t)p * nkv + kvh;
-            tso_tq_unpack(k_words + row * wpr, bits, hd, idx.data());
+            tso_tq_unpack(k_words + row * k_wpr, k_bits, hd, idx.data());
             float dot = 0.0f;
             for (int d = 0; d < hd; d++) dot += q_rot[d] * k_codebook[idx[d]];
             scores[p] = dot * k_norms[row] * scale;
@@ -267,7 +268,7 @@ void tso_tq_attention(const float* q, const uint32_t* k_words, const float* k_no
         std::fill(acc_rot.begin(), acc_rot.end(), 0.0f);
         for (int p = 0; p < seq_len; p++) {
             const size_t row = (size_t)p * nkv + kvh;
-            tso_tq_unpack(v_words + row * wpr, bits, hd, idx.data());
+            tso_tq_unpack(v_words + row * v_wpr, v_bits, hd, idx.data());
             const float coeff = scores[p] * v_norms[row];
             for (int d = 0; d < hd; d++) acc_rot[d] += coeff * v_codebook[idx[d]];
         }

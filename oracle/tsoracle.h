@@ -141,8 +141,8 @@ void tso_tq_dequantize_row(float norm, const uint32_t* words, const float* signs
                            float* out);                                              /* kv_quant.rs:367-379 */
 void tso_tq_attention(const float* q, const uint32_t* k_words, const float* k_norms, const uint32_t* v_words,
                       const float* v_norms, int hd, int nq, int nkv, int seq_len, float scale, const float* sinks,
-                      const float* k_signs, const float* k_codebook, const float* v_signs, const float* v_codebook, int bits,
-                      float* out);                                                   /* kv_quant_attention.rs:58-136 */
+                      const float* k_signs, const float* k_codebook, const float* v_signs, const float* v_codebook, int k_bits,
+                      int v_bits, float* out);                                                   /* kv_quant_attention.rs:58-136 */
 
 /* ---- selection --------------------------------------------------------- */
 typedef struct {
@@ -303,6 +303,12 @@ typedef struct {
     const float* rope_freqs; /* NULL, or head_dim/2 explicit per-pair frequencies (YaRN table) */
     float rope_mscale;       /* multiplies cos and sin; <= 0 means 1 */
     float act_alpha, act_limit; /* act_alpha > 0: gpt-oss clamped SwiGLU instead of silu(g) * u */
+    /* TurboQuant KV (crates/model-io/src/kv_quant.rs:25-40,102-107): bits per key / value coordinate,
+     * 0 = fp16 rows.  Quantized are the full-attention layers (window == 0), all of them in a stack of
+     * at most two layers, else all but the last.  A quantized layer's row goes through fp16 (the staging
+     * row of crates/runtime/src/kv_write.rs:66-118), is quantized per head, and every later read sees
+     * the decoded row. */
+    int32_t kv_k_bits, kv_v_bits;
 } tso_model_desc;
 
 typedef struct tso_model tso_model;
@@ -327,6 +333,8 @@ void tso_model_rewind_to(tso_model* m, int64_t position); /* kv_cache_rewind.rs:
 /* Raw access to the fp32 KV store of one layer: [position][kv_head][head_dim]. */
 float* tso_model_k(tso_model* m, int layer);
 float* tso_model_v(tso_model* m, int layer);
+/* 1 when the layer's rows are kept quantized (the rule above). */
+int tso_model_layer_quantized(const tso_model* m, int layer);
 /* One batched pass over `m_rows` fed tokens at base (batched.rs:92-456 semantics for a
  * pure-attention target).  parent NULL => chain (row i at position base+i, sees [0, base+i]).
  * parent given => tree (row s rotated at base+depth[s], sees [0,base) + its root path; K/V of

@@ -1,0 +1,193 @@
+"""TurboQuant KV rows on the GPU against the oracle (oracle/tq.cpp, pinned on the reference's recorded vectors by
+tests/test_oracle_tq.py).
+
+Three layers of checks, because the codec is discontinuous: a coordinate that sits on a midpoint takes either
+neighbour, so two forwards whose K / V rows differ in the last fp16 bit store a few different indices, and the
+logits of a random-weight model move by percents (the oracle itself moves by 2-3 % of its largest logit at four bits
+when its staging rows are left in f32 instead of fp16).
+  1. the stored rows -- norm and packed words -- of given fp16 staging rows: equal to the oracle's by bits
+     (the bar of crates/gpu/tests/kv_quantize_parity.rs, whose two shapes and input formula are the first cases);
+  2. attention over those stored rows against the oracle's rotated-space attention
+     (crates/compute/src/kv_quant_attention.rs:58-136), to fp16 accuracy (crates/gpu/tests/attention_tq_parity.rs);
+  3. the model: a pass of m rows equals m single-row passes by bits -- the per-token semantics of
+     crates/runtime/src/kv_write.rs:66-118 -- rollback and replay by bits, and the logits against the oracle model with
+     the bound that the codec's own sensitivity allows."""
+import os
+
+import numpy as np
+import pytest
+
+from tests import gpu_common as gc
+
+pytestmark = pytest.mark.gpu
+
+
+def _sides(hd, kb, vb):
+    from oracle import binding as ob
+    ks, vs = ob.tq_sign_vector(hd, ob.TQ_KEY_SEED), ob.tq_sign_vector(hd, ob.TQ_VALUE_SEED)
+    kc, vc = ob.tq_codebook(hd, kb), ob.tq_codebook(hd, vb)
+    return ks, kc, ob.tq_midpoints(kc), vs, vc, ob.tq_midpoints(vc)
+
+
+def _check_rows(rows16, stored, signs, mid, bits):
+    """stored [n, heads, 1 + words] against the oracle's quantize_row of the same fp16 rows."""
+    from oracle import binding as ob
+    n, heads, hd = rows16.shape
+    for p in range(n):
+        for h in range(heads):
+            norm, words = ob.tq_quantize_row(rows16[p, h].astype(np.float32), signs, mid, bits)
+            assert np.array_equal(stored[p, h, 1:], words), (p, h)
+            assert stored[p, h, 0] == np.float32(norm).view(np.uint32), (p, h, stored[p, h, :1].view(np.float32), norm)
+
+
+@pytest.mark.parametrize("hd,bits,rows,heads", [(64, 2, 3, 2), (128, 3, 2, 3), (128, 4, 5, 1), (64, 4, 16, 8), (64, 3, 9, 2),
+                                               (128, 2, 16, 4)])
+def test_stored_rows_of_a_pass_equal_the_oracles_by_bits(hd, bits, rows, heads):
+    """crates/gpu/tests/kv_quantize_parity.rs:41-110: hashed, non-degenerate rows read through fp16."""
+    from turbospark_amd import ffi
+    total = rows * heads * hd
+    x = (np.sin(np.arange(total, dtype=np.float32) * np.float32(0.913) + np.float32(0.37)) * 3).astype(np.float16)
+    x = x.reshape(rows, heads, hd)
+    q = np.zeros((rows, heads, hd), np.float16)
+    _, kr, vr = ffi.attention_quantized(q, x, x[::-1].copy(), 0, bits, bits)
+    ks, _, km, vs, _, vm = _sides(hd, bits, bits)
+    _check_rows(x, kr, ks, km, bits)
+    _check_rows(x[::-1], vr, vs, vm, bits)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,m,base,kb,vb,sinks", [
+    (4, 1, 128, 7, 0, 4, 4, False), (8, 2, 64, 16, 37, 3, 4, False), (32, 8, 128, 5, 300, 4, 4, False),
+    (8, 2, 64, 1, 129, 2, 2, True), (16, 8, 64, 8, 1000, 3, 3, True), (32, 8, 128, 16, 2049, 3, 4, False)])
+def test_attention_over_stored_rows_matches_the_rotated_space_oracle(nq, nkv, hd, m, base, kb, vb, sinks):
+    from oracle import binding as ob
+    from turbospark_amd import ffi
+    rng = np.random.default_rng(nq * 1000 + base)
+    seq = base + m
+    q = rng.standard_normal((m, nq, hd)).astype(np.float16)
+    k = (rng.standard_normal((seq, nkv, hd)) * rng.uniform(0.2, 3.0, (seq, nkv, 1))).astype(np.float16)
+    v = (rng.standard_normal((seq, nkv, hd)) * rng.uniform(0.2, 3.0, (seq, nkv, 1))).astype(np.float16)
+    sk = rng.standard_normal(nq).astype(np.float32) if sinks else None
+    got, kr, vr = ffi.attention_quantized(q, k, v, base, kb, vb, sinks=sk)
+    ks, kc, km, vs, vc, vm = _sides(hd, kb, vb)
+    # the rows stored ahead of the pass and by the pass: a sample of them by bits (all of them when few)
+    pick = np.unique(np.concatenate([np.arange(min(seq, 24)), np.arange(max(0, base - 8), seq),
+                                     rng.integers(0, seq, 24)]))
+    _check_rows(k[pick], kr[pick], ks, km, kb)
+    _check_rows(v[pick], vr[pick], vs, vm, vb)
+    worst = 0.0
+    for i in range(m):
+        want = ob.tq_attention(q[i].astype(np.float32), kr[:, :, 1:], kr[:, :, 0].view(np.float32), vr[:, :, 1:],
+                               vr[:, :, 0].view(np.float32), hd, nq, nkv, base + i + 1, kb, ks, kc, vs, vc, sinks=sk,
+                               v_bits=vb).reshape(nq, hd)
+        worst = max(worst, float(np.abs(got[i] - want).max() / np.abs(want).max()))
+    print(f"nq {nq} nkv {nkv} hd {hd} m {m} base {base} K{kb}/V{vb}: worst relative error {worst:.2e}")
+    assert worst <= 4e-3
+
+
+def _open(name, kv_bits, max_context=96, seed=21, **over):
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    os.environ["TSV_FUSED"] = "0"
+    cfg = dict(synth.CONFIGS[name], max_context=max_context, **over)
+    w = synth.make_weights(cfg, seed=seed)
+    return cfg, w, ts.HipVerifier(cfg, w, kv_bits=kv_bits)
+
+
+@pytest.mark.parametrize("name,kv_bits,layers", [("small_q4_k", (4, 4), 3), ("xcd_q4_k", (3, 4), 2), ("tiny_q8_0", (2, 2), 4),
+                                                 ("gptoss_small", (4, 4), 4), ("moe_small", (3, 3), 3)])
+def test_a_pass_of_m_rows_is_m_single_row_passes_by_bits(name, kv_bits, layers):
+    """What the reference's per-token path does (kv_write.rs:66-118: stage, commit, attend over stored rows, the
+    token's own included) is what every row of a wider pass must see."""
+    cfg, w, a = _open(name, kv_bits, n_layers=layers)
+    import turbospark_amd as ts
+    b = ts.HipVerifier(cfg, w, kv_bits=kv_bits)
+    rng = np.random.default_rng(5)
+    prompt = rng.integers(0, cfg["vocab"], 37).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 8).astype(np.int32)
+    a.prefill(prompt, 0, want_logits=False)
+    b.prefill(prompt, 0, want_logits=False)
+    wide = a.verify(feed, 37)
+    narrow = np.concatenate([b.verify(feed[i:i + 1], 37 + i) for i in range(8)])
+    assert np.array_equal(wide, narrow)
+    quantized = [l for l in range(layers) if int(w["layers"][l].get("window", 0)) == 0 and (layers <= 2 or l + 1 < layers)]
+    assert quantized
+    for l in quantized:
+        ka, va = a.read_kv_quantized(l, 0, 45)
+        kb_, vb_ = b.read_kv_quantized(l, 0, 45)
+        assert np.array_equal(ka, kb_) and np.array_equal(va, vb_)
+    for l in set(range(layers)) - set(quantized):
+        with pytest.raises(ts.ffi.TsvError):
+            a.read_kv_quantized(l, 0, 1)
+        a.read_kv(l, 40, 4)
+    with pytest.raises(ts.ffi.TsvError):
+        a.read_kv(quantized[0], 0, 1)
+
+
+def test_rollback_and_replay_by_bits():
+    cfg, w, g = _open("small_q4_k", (3, 4), n_layers=3)
+    rng = np.random.default_rng(6)
+    prompt = rng.integers(0, cfg["vocab"], 20).astype(np.int32)
+    g.prefill(prompt, 0, want_logits=False)
+    cp = g.checkpoint()
+    f1 = rng.integers(0, cfg["vocab"], 8).astype(np.int32)
+    f2 = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    first = g.verify(f1, 20)
+    g.rollback(cp)
+    other = g.verify(f2, 20)          # other rows over the same slots
+    g.rollback(cp)
+    again = g.verify(f1, 20)
+    assert np.array_equal(first, again) and not np.array_equal(first[:5], other)
+    # keep three of the rows and go on: the kept rows are read from the store, the rest recomputed
+    g.rollback_retaining(cp, 3)
+    assert g.position == 23
+    assert np.array_equal(g.verify(f1[3:], 23), first[3:])
+
+
+@pytest.mark.parametrize("name,kv_bits,layers,bound", [("small_q4_k", (4, 4), 3, 8e-2), ("xcd_q4_k", (4, 4), 3, 8e-2),
+                                                       ("gptoss_small", (4, 4), 4, 8e-2), ("small_q4_k", (3, 4), 3, 1.2e-1)])
+def test_logits_against_the_oracle_model_within_the_codecs_own_sensitivity(name, kv_bits, layers, bound):
+    """The same forward with the same codec on both sides.  The bound is not fp16 accuracy: indices of coordinates
+    near a midpoint differ between any two forwards whose K / V rows differ in the last bit.  What is asserted is
+    that the GPU is no further from the oracle than the oracle is from itself under such a change (its own
+    f32-staging variant), and far closer than the codec's effect (the distance to the fp16-row oracle)."""
+    from oracle import binding as ob
+    cfg, w, g = _open(name, kv_bits, n_layers=layers)
+    rng = np.random.default_rng(7)
+    prompt = rng.integers(0, cfg["vocab"], 40).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 12).astype(np.int32)
+
+    def oracle(**kw):
+        m = ob.Model(cfg, w, threads=16, **kw)
+        for i in range(0, 40, 16):
+            m.verify(prompt[i:i + 16], i)
+        return m.verify(feed, 40)
+
+    want = oracle(round_kv_f16=True, kv_bits=kv_bits)
+    twin = oracle(round_kv_f16=False, kv_bits=kv_bits)
+    plain = oracle(round_kv_f16=True)
+    g.prefill(prompt, 0, want_logits=False)
+    got = g.verify(feed, 40)
+    err, self_err, effect = gc.logit_error(got, want), gc.logit_error(twin, want), gc.logit_error(plain, want)
+    print(f"{name} K{kv_bits[0]}/V{kv_bits[1]}: GPU vs oracle {err:.2e}; oracle vs its f32-staging twin {self_err:.2e}; "
+          f"codec vs fp16 rows {effect:.2e}")
+    assert err <= bound and err <= max(3 * self_err, 2e-2) and err < 0.6 * effect
+
+
+def test_what_a_quantized_handle_refuses():
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg, w, g = _open("small_q4_k", (4, 4))
+    g.verify(np.arange(6, dtype=np.int32), 0)
+    with pytest.raises(ts.ffi.TsvError, match="quantized"):
+        g.compact_tree(0, [0, 2, 3])
+    for bad in ((4, 3), (1, 1), (5, 5), (2, 4), (0, 4)):
+        with pytest.raises(ts.ffi.TsvError, match="widths"):
+            ts.HipVerifier(cfg, w, kv_bits=bad)
+    # gpt-oss with a window on every layer: nothing to quantize, refused by name
+    # (crates/runtime/src/real_forward_init.rs:186-197)
+    oss = dict(synth.CONFIGS["gptoss_small"], max_context=96)
+    wo = synth.make_weights(oss, seed=3)
+    for lw in wo["layers"]:
+        lw["window"] = 24
+    with pytest.raises(ts.ffi.TsvError, match="nothing to quantize"):
+        ts.HipVerifier(oss, wo, kv_bits=(4, 4))

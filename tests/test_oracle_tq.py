@@ -195,14 +195,14 @@ def _quantized(g, dim, seq, nkv, kbits, vbits):
 
 
 def test_rotated_space_attention_equals_attention_over_the_decoded_rows():
-    """kv_quant.rs (tests):381-440, widened to grouped heads and sinks.  Same bit width on both sides, as
-    TqTables-per-side allows; the decoded rows go through the plain attention the other tests pin."""
-    for dim, nq, nkv, seq, bits in ((64, 1, 1, 5, 4), (128, 4, 2, 9, 3), (64, 6, 3, 17, 2)):
+    """kv_quant.rs (tests):381-440, widened to grouped heads, sinks and the K3/V4 split; the decoded rows go
+    through the plain attention the other tests pin."""
+    for dim, nq, nkv, seq, bits, vbits in ((64, 1, 1, 5, 4, 4), (128, 4, 2, 9, 3, 3), (64, 6, 3, 17, 2, 2), (128, 4, 1, 11, 3, 4)):
         g = Lcg(321 + dim + bits)
         q = np.array([g.f32() for _ in range(nq * dim)], np.float32)
-        kw, kn, vw, vn, kd, vd, t = _quantized(g, dim, seq, nkv, bits, bits)
+        kw, kn, vw, vn, kd, vd, t = _quantized(g, dim, seq, nkv, bits, vbits)
         for sinks in (None, np.linspace(-1, 1, nq).astype(np.float32)):
-            got = ob.tq_attention(q, kw, kn, vw, vn, dim, nq, nkv, seq, bits, sinks=sinks, **t)
+            got = ob.tq_attention(q, kw, kn, vw, vn, dim, nq, nkv, seq, bits, sinks=sinks, v_bits=vbits, **t)
             want = ob.causal_attention(q.reshape(nq, dim), kd, vd, dim, nq, nkv, seq, 0, 0.0, sinks)
             assert np.abs(got - want).max() < 1e-3, (dim, nq, nkv, seq, bits)
 
@@ -216,3 +216,40 @@ def test_sinks_enter_the_denominator_only():
     assert np.linalg.norm(b) < 0.5 * np.linalg.norm(a)
     # and the direction is unchanged: only the scale moves
     assert np.abs(b / np.linalg.norm(b) - a / np.linalg.norm(a)).max() < 1e-4
+
+
+def test_the_oracle_model_keeps_decoded_rows_on_the_layers_the_policy_names():
+    """crates/model-io/src/kv_quant.rs:102-107 (every full-attention layer but the last, all of them in a stack
+    of two) and crates/runtime/src/kv_write.rs:66-118 (the fp16 staging row is what gets quantized).  Layer 0
+    sees the same inputs with and without the codec, so its cached rows must be the decoded fp16 rows of the
+    plain model; the last layer's rows stay fp16."""
+    from turbospark_amd import synth
+    two = dict(synth.CONFIGS["small_q4_k"], max_context=32)
+    m2 = ob.Model(two, synth.make_weights(two, seed=5), kv_bits=(4, 4))
+    assert [m2.layer_quantized(l) for l in range(2)] == [True, True]
+    cfg = dict(two, n_layers=3)
+    w = synth.make_weights(cfg, seed=5)
+    n, nkv, hd = cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"]
+    plain = ob.Model(cfg, w, round_kv_f16=True, threads=8)
+    quant = ob.Model(cfg, w, round_kv_f16=True, threads=8, kv_bits=(3, 4))
+    assert [quant.layer_quantized(l) for l in range(n)] == [True] * (n - 1) + [False]
+    assert not any(plain.layer_quantized(l) for l in range(n))
+    feed = np.arange(7, dtype=np.int32) * 11 % cfg["vocab"]
+    lp, lq = plain.verify(feed, 0, want_f32=True), quant.verify(feed, 0, want_f32=True)
+    kp, vp = plain.kv(0)
+    kq, vq = quant.kv(0)
+    for side, rows, got, bits, seed in (("k", kp, kq, 3, ob.TQ_KEY_SEED), ("v", vp, vq, 4, ob.TQ_VALUE_SEED)):
+        signs, cb = ob.tq_sign_vector(hd, seed), ob.tq_codebook(hd, bits)
+        mp = ob.tq_midpoints(cb)
+        for pos in range(7):
+            for h in range(nkv):
+                x = rows[pos, h]
+                norm, words = ob.tq_quantize_row(x, signs, mp, bits)
+                want = ob.tq_dequantize_row(norm, words, signs, cb, bits, hd)
+                assert np.array_equal(got[pos, h], want), (side, pos, h)
+    # the last layer keeps fp16 rows: every value is its own fp16 rounding
+    kl, _ = quant.kv(n - 1)
+    assert np.array_equal(kl[:7], kl[:7].astype(np.float16).astype(np.float32))
+    # and the codec does move the logits
+    a, b = np.asarray(lp[1], np.float32), np.asarray(lq[1], np.float32)
+    assert np.abs(a - b).max() / np.abs(a).max() > 1e-4

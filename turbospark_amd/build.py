@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
-SOURCES = ["gemm.hip", "moe.hip", "moe_fp4.hip", "misc.hip", "attn.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
+SOURCES = ["gemm.hip", "moe.hip", "moe_fp4.hip", "misc.hip", "attn.hip", "kvquant.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
 # The per-XCD fused layer kernels (an experiment that measured slower than the kernels it replaces) are
 # built only on request: TSV_BUILD_FUSED=1.
 WITH_FUSED = os.environ.get("TSV_BUILD_FUSED", "0") == "1"

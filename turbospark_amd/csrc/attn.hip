@@ -93,7 +93,22 @@ __global__ void k_attn_combine(AttnArgs a0, int G, int R) {
 #pragma unroll 8
         for (int c = 0; c < nch; c++) num = fmaf(wgt[c], po[c * stride], num);
     }
-    const _Float16 o16 = (_Float16)(num / s_den);
+    float res = num / s_den;
+    if (a.unrot) {
+        // the sum was taken over rotated value rows: back through the normalized Hadamard transform
+        // (crates/compute/src/wht.rs:15-29, stage h pairs d with d + h) and the value signs
+        __shared__ float s_h[128];
+        const float c = 0.70710678118654752440f;
+        for (int st = 1; st < hd; st <<= 1) {
+            s_h[d] = res;
+            __syncthreads();
+            const float other = s_h[d ^ st];
+            __syncthreads();
+            res = ((d & st) ? other - res : res + other) * c;
+        }
+        res *= a.unrot[d];
+    }
+    const _Float16 o16 = (_Float16)res;
     const int kk = qh * hd + d;
     ((_Float16*)a.xfrag)[a.frag16 ? frag16_index(kk, m) : frag_index(kk, m)] = o16;
     // sum of each 32-element sub-block of the output projection's input (32 neighbouring threads)

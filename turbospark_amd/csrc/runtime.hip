@@ -33,6 +33,9 @@ struct LayerW {
     int cap = 0;        // positions the layer's cache holds: the context, or a ring of window + slack
     bool rope_fused = false;  // the q/k/v projection rotates and stores its own rows
     uint16_t *kc = nullptr, *vc = nullptr;
+    // a quantized layer (TurboQuant): kc / vc are then the fp16 cache all such layers share, and these
+    // the layer's own rows, [position][kv head][1 + words] with the norm first
+    uint32_t *kq = nullptr, *vq = nullptr;
 };
 
 int dtype_fmt(int dtype) {
@@ -120,6 +123,11 @@ struct tsv_ctx {
     int32_t *tok_dev = nullptr, *tok_host = nullptr;
     AcceptScratch sc{};
     std::vector<void*> allocs;
+    // TurboQuant KV rows (crates/model-io/src/kv_quant.rs): widths (0 = every layer fp16), the tables of the two
+    // sides and the fp16 cache the quantized layers decode into before their attention
+    int kv_k_bits = 0, kv_v_bits = 0;
+    TqSide tq_k{}, tq_v{};
+    uint16_t *tq_kc = nullptr, *tq_vc = nullptr;
     int64_t position = 0;
     int64_t high_water = 0;     // one past the last position any pass has written since the last reset
     int64_t rewind_budget = INT64_MAX;  // KvCacheManager::max_safe_rewind: min over ring layers of capacity - window
@@ -456,7 +464,7 @@ int launch_pass(tsv_ctx* c, int m) {
     float *x = c->x, *x_other = c->x2;  // the fused kernels write the residual rows to the other buffer
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     // the attention half as one per-XCD kernel: passes of at most eight rows and 32 (row, q head) pairs
-    const bool attn_block = c->fused_attn && m <= 8 && m * (c->nq / c->nkv) <= 32;
+    const bool attn_block = c->fused_attn && !c->kv_k_bits && m <= 8 && m * (c->nq / c->nkv) <= 32;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
         int attn_splits = 0;  // partial sums the attention half leaves for the FFN norm
@@ -600,10 +608,34 @@ int launch_pass(tsv_ctx* c, int m) {
             for (int rep = 0; rep < c->repeat[PC_ROPE] && !rc; rep++) rc = launch_rope_kv(s, ra, m);
         }
         if (rc) return rc;
+        if (L.kq) {
+            // the pass's K / V rows sit in the shared fp16 cache (the staging rows of
+            // crates/runtime/src/kv_write.rs:66-118): quantize them into the layer's store, decode the rows
+            // before them, rotate q -- attention then runs in the rotated space (kv_quant_attention.rs:58-136)
+            TqArgs ta{};
+            ta.q16 = c->q16;
+            ta.kc = L.kc;
+            ta.vc = L.vc;
+            ta.kq = L.kq;
+            ta.vq = L.vq;
+            ta.k = c->tq_k;
+            ta.v = c->tq_v;
+            ta.nq = c->nq;
+            ta.nkv = c->nkv;
+            ta.hd = c->hd;
+            ta.cap = L.cap;
+            ta.vp = c->vp_dev;
+            ta.m_hint = m;
+            ta.base_hint = c->use_graph ? -1 : c->vp_host->base;
+            PROF(PC_ROPE);
+            rc = launch_tq_prepare(s, ta, c->ctx_alloc);
+            if (rc) return rc;
+        }
         AttnArgs aa{};
         aa.q16 = c->q16;
         aa.kc = L.kc;
         aa.vc = L.vc;
+        aa.unrot = L.kq ? c->tq_v.signs : nullptr;
         aa.part_o = c->part_o;
         aa.part_ml = c->part_ml;
         aa.xfrag = c->xf_b;
@@ -1029,6 +1061,30 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         return TSV_ERR_DEVICE;
     }
     int rc;
+    if (d->kv_k_bits || d->kv_v_bits) {
+        // crates/model-io/src/kv_quant.rs:48-72: the widths --kv-bits can name (2, 3, 3.5 = K3/V4, 4);
+        // crates/runtime/src/real_forward_init.rs:170-199: refused by name when no layer would be quantized
+        const int kb = d->kv_k_bits, vb = d->kv_v_bits;
+        if (!((kb == 2 && vb == 2) || (kb == 3 && vb == 3) || (kb == 3 && vb == 4) || (kb == 4 && vb == 4))) {
+            set_error("open: KV quantization widths must be one of K2/V2, K3/V3, K3/V4, K4/V4");
+            return fail(TSV_ERR_INVALID);
+        }
+        bool any = false;
+        for (int l = 0; l < d->n_layers; l++)
+            any = any || (d->layers[l].window == 0 && (d->n_layers <= 2 || l + 1 < d->n_layers));
+        if (!any) {
+            set_error("open: KV quantization has nothing to quantize here: every full-attention layer is excluded by "
+                      "the last-layer rule, or there are no full-attention layers at all");
+            return fail(TSV_ERR_UNSUPPORTED);
+        }
+        float* tables = nullptr;
+        if ((rc = dev_alloc(c, &tables, (size_t)2 * TQ_TABLE_FLOATS * 4)) ||
+            (rc = tq_upload_side(c->hd, kb, 0, tables, &c->tq_k)) ||
+            (rc = tq_upload_side(c->hd, vb, 1, tables + TQ_TABLE_FLOATS, &c->tq_v)))
+            return fail(rc);
+        c->kv_k_bits = kb;
+        c->kv_v_bits = vb;
+    }
     Stager st;
     const int qd = c->nq * c->hd, kvd = c->nkv * c->hd;
     c->layers.resize(c->n_layers);
@@ -1155,7 +1211,19 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             }
         }
         const size_t kvb = (size_t)c->nkv * L.cap * c->hd * 2;
-        if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) return fail(rc);
+        // crates/model-io/src/kv_quant.rs:102-107: every full-attention layer of a stack of at most two, else
+        // every one but the last; windowed layers keep fp16 rows
+        if (c->kv_k_bits && s.window == 0 && (c->n_layers <= 2 || l + 1 < c->n_layers)) {
+            if (!c->tq_kc && ((rc = dev_alloc(c, &c->tq_kc, kvb, true)) || (rc = dev_alloc(c, &c->tq_vc, kvb, true)))) return fail(rc);
+            L.kc = c->tq_kc;
+            L.vc = c->tq_vc;
+            const size_t rows = (size_t)L.cap * c->nkv;
+            if ((rc = dev_alloc(c, &L.kq, rows * (1 + c->tq_k.words) * 4, true)) ||
+                (rc = dev_alloc(c, &L.vq, rows * (1 + c->tq_v.words) * 4, true)))
+                return fail(rc);
+        } else if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) {
+            return fail(rc);
+        }
         pneed = std::max(pneed, std::max(partial_need(L.qkv), partial_need(L.wo)));
         pneed = std::max(pneed, (size_t)8 * 16 * ((size_t)(qd + 2 * kvd) + TILE_ROWS));
     }
@@ -1299,7 +1367,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         return fail(TSV_ERR_DEVICE);
     }
     // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
-    c->wide.ok = c->rewind_budget == INT64_MAX && !c->fused_ffn && !c->fused_attn;
+    c->wide.ok = c->rewind_budget == INT64_MAX && !c->fused_ffn && !c->fused_attn && !c->kv_k_bits;
     for (const LayerW& L : c->layers)
         if (L.n_experts || !L.rope_fused || L.v_only.tiles || L.qkv.fmt != FMT_Q4K || L.wo.fmt != FMT_Q4K ||
             L.gate_up.fmt != FMT_Q4K || L.down.fmt != FMT_Q4K)
@@ -1564,6 +1632,10 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
         set_error("compact_tree: the block at `base` lies outside the KV cache");
         return TSV_ERR_INVALID;
     }
+    if (c->kv_k_bits) {
+        set_error("compact_tree: tree rounds are not supported over quantized KV rows");
+        return TSV_ERR_UNSUPPORTED;
+    }
     TSV_HIP(hipStreamSynchronize(c->stream));
     if (int frc = check_fused(c)) return frc;  // rows a fused kernel gave up on must not be gathered
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
@@ -1789,6 +1861,10 @@ extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t 
         set_error("read_kv: null argument or range outside the cache");
         return TSV_ERR_INVALID;
     }
+    if (c->layers[layer].kq) {
+        set_error("read_kv: this layer keeps quantized rows (tsv_read_kv_quantized reads them)");
+        return TSV_ERR_UNSUPPORTED;
+    }
     const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
     uint16_t *kd = nullptr, *vd = nullptr;
     TSV_HIP(hipMalloc((void**)&kd, bytes));
@@ -1869,6 +1945,10 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
     if (!c || !k || !v || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->max_context) {
         set_error("write_kv: range outside the cache");
         return TSV_ERR_INVALID;
+    }
+    if (c->layers[layer].kq) {
+        set_error("write_kv: this layer keeps quantized rows");
+        return TSV_ERR_UNSUPPORTED;
     }
     const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
     uint16_t *kd = nullptr, *vd = nullptr;
@@ -2027,6 +2107,152 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     if (!rc && (hipMemcpyAsync(frag.data(), xf, xfb, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
                 hipStreamSynchronize(c->stream) != hipSuccess)) {
         set_error("attention: device execution failed");
+        rc = TSV_ERR_DEVICE;
+    }
+    if (!rc)
+        for (int b = 0; b < m; b++)
+            for (int kk = 0; kk < nq * hd; kk++) out[(size_t)b * nq * hd + kk] = frag[(size_t)frag_index(kk, b)];
+    (void)hipStreamSynchronize(c->stream);
+    for (void* p : c->allocs) (void)hipFree(p);
+    (void)hipStreamDestroy(c->stream);
+    return rc;
+}
+
+extern "C" int32_t tsv_kv_quant_tables(int32_t head_dim, int32_t bits, int32_t value_side, float* signs, float* codebook,
+                                       float* midpoints) {
+    if (head_dim < 32 || head_dim > 512 || (head_dim & (head_dim - 1)) || bits < 1 || bits > 4 || !signs || !codebook ||
+        !midpoints) {
+        set_error("kv_quant_tables: head_dim must be a power of two in 32..512 and bits in 1..4");
+        return TSV_ERR_INVALID;
+    }
+    tq_sign_vector(head_dim, value_side ? 1 : 0, signs);
+    const std::vector<float> cb = tq_codebook(head_dim, bits);
+    for (size_t i = 0; i < cb.size(); i++) codebook[i] = cb[i];
+    for (size_t i = 0; i + 1 < cb.size(); i++) midpoints[i] = 0.5f * (cb[i] + cb[i + 1]);
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_read_kv_quantized(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, uint32_t* k_rows,
+                                         uint32_t* v_rows) {
+    if (!c || !k_rows || !v_rows || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
+        set_error("read_kv_quantized: null argument or range outside the cache");
+        return TSV_ERR_INVALID;
+    }
+    const LayerW& L = c->layers[layer];
+    if (!L.kq) {
+        set_error("read_kv_quantized: this layer keeps fp16 rows");
+        return TSV_ERR_INVALID;
+    }
+    const size_t kw = (size_t)c->nkv * (1 + c->tq_k.words), vw = (size_t)c->nkv * (1 + c->tq_v.words);
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    TSV_HIP(hipMemcpy(k_rows, L.kq + (size_t)pos0 * kw, (size_t)n * kw * 4, hipMemcpyDeviceToHost));
+    TSV_HIP(hipMemcpy(v_rows, L.vq + (size_t)pos0 * vw, (size_t)n * vw * 4, hipMemcpyDeviceToHost));
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
+                                           int32_t nkv, int32_t hd, int64_t base, int32_t k_bits, int32_t v_bits,
+                                           float scale, const float* sinks, uint16_t* out, uint32_t* k_rows,
+                                           uint32_t* v_rows) {
+    if (!q || !k || !v || !out || !k_rows || !v_rows || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0 ||
+        k_bits < 1 || k_bits > 4 || v_bits < 1 || v_bits > 4 || (hd != 64 && hd != 128)) {
+        set_error("attention_quantized: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    tsv_ctx tmp;
+    tsv_ctx* c = &tmp;
+    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    VerifyParams vp;
+    int rc = fill_params(vp, nullptr, nullptr, m, base, 0);
+    const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv;
+    const size_t kvb = (size_t)nkv * ctx * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
+    const size_t kwb = (size_t)ctx * nkv * (1 + tq_words(hd, k_bits)) * 4, vwb = (size_t)ctx * nkv * (1 + tq_words(hd, v_bits)) * 4;
+    uint16_t *kc = nullptr, *vc = nullptr, *kin = nullptr, *vin = nullptr, *q16 = nullptr;
+    uint32_t *kq = nullptr, *vq = nullptr;
+    float *po = nullptr, *pml = nullptr, *sinks_dev = nullptr, *tables = nullptr;
+    uint4* xf = nullptr;
+    VerifyParams* vpd = nullptr;
+    const size_t xfb = xfrag_bytes(nq * hd);
+    TqArgs ta{};
+    if (!rc && sinks) {
+        rc = dev_alloc(c, &sinks_dev, (size_t)nq * 4);
+        if (!rc && hipMemcpyAsync(sinks_dev, sinks, (size_t)nq * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess)
+            rc = TSV_ERR_DEVICE;
+    }
+    if (!rc) rc = dev_alloc(c, &kc, kvb, true);
+    if (!rc) rc = dev_alloc(c, &vc, kvb, true);
+    if (!rc) rc = dev_alloc(c, &kq, kwb, true);
+    if (!rc) rc = dev_alloc(c, &vq, vwb, true);
+    if (!rc) rc = dev_alloc(c, &kin, inb);
+    if (!rc) rc = dev_alloc(c, &vin, inb);
+    if (!rc) rc = dev_alloc(c, &q16, qb);
+    if (!rc) rc = dev_alloc(c, &po, (size_t)nkv * nch * m * G * hd * 4, true);
+    if (!rc) rc = dev_alloc(c, &pml, (size_t)nkv * nch * m * G * 2 * 4, true);
+    if (!rc) rc = dev_alloc(c, &xf, xfb, true);
+    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
+    if (!rc) rc = dev_alloc(c, &tables, (size_t)2 * TQ_TABLE_FLOATS * 4);
+    if (!rc) rc = tq_upload_side(hd, k_bits, 0, tables, &ta.k);
+    if (!rc) rc = tq_upload_side(hd, v_bits, 1, tables + TQ_TABLE_FLOATS, &ta.v);
+    if (!rc && (hipMemcpyAsync(kin, k, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+                hipMemcpyAsync(vin, v, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+                hipMemcpyAsync(q16, q, qb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+                hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess))
+        rc = TSV_ERR_DEVICE;
+    ta.q16 = q16;
+    ta.kc = kc;
+    ta.vc = vc;
+    ta.kq = kq;
+    ta.vq = vq;
+    ta.nkv = nkv;
+    ta.hd = hd;
+    ta.cap = ctx;
+    ta.vp = vpd;
+    // the rows before the pass: staged, quantized as one wide "pass" at position 0, then wiped from the
+    // fp16 cache so that what attention reads of them is what the decoder wrote
+    if (!rc && base > 0) {
+        rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, 0, (int)base, kin, vin);
+        ta.nq = 0;
+        ta.m_hint = (int)base;
+        ta.base_hint = 0;
+        if (!rc) rc = launch_tq_prepare(c->stream, ta, 0);
+        if (!rc && (hipMemsetAsync(kc, 0, kvb, c->stream) != hipSuccess || hipMemsetAsync(vc, 0, kvb, c->stream) != hipSuccess))
+            rc = TSV_ERR_DEVICE;
+    }
+    // the pass itself, as the forward runs it
+    const size_t row = (size_t)nkv * hd;
+    if (!rc) rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, (int)base, m, kin + (size_t)base * row, vin + (size_t)base * row);
+    ta.nq = nq;
+    ta.m_hint = m;
+    ta.base_hint = (int)base;
+    if (!rc) rc = launch_tq_prepare(c->stream, ta, base);
+    if (!rc) {
+        AttnArgs aa{};
+        aa.q16 = q16;
+        aa.kc = kc;
+        aa.vc = vc;
+        aa.unrot = ta.v.signs;
+        aa.part_o = po;
+        aa.part_ml = pml;
+        aa.xfrag = xf;
+        aa.nq = nq;
+        aa.nkv = nkv;
+        aa.hd = hd;
+        aa.max_ctx = ctx;
+        aa.nch = nch;
+        aa.scale = scale > 0.f ? scale : 1.0f / std::sqrt((float)hd);
+        aa.sinks = sinks_dev;
+        aa.vp = vpd;
+        aa.m_hint = m;
+        aa.base_hint = (int)base;
+        rc = launch_attention(c->stream, aa, m);
+    }
+    std::vector<uint16_t> frag(xfb / 2);
+    const size_t kn = (size_t)seq * nkv * (1 + tq_words(hd, k_bits)) * 4, vn = (size_t)seq * nkv * (1 + tq_words(hd, v_bits)) * 4;
+    if (!rc && (hipMemcpyAsync(frag.data(), xf, xfb, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                hipMemcpyAsync(k_rows, kq, kn, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                hipMemcpyAsync(v_rows, vq, vn, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                hipStreamSynchronize(c->stream) != hipSuccess)) {
+        set_error("attention_quantized: device execution failed");
         rc = TSV_ERR_DEVICE;
     }
     if (!rc)

@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include <string>
+#include <vector>
 
 #include "../../include/tsverify.h"
 #include "../../include/tsverify_testing.h"
@@ -324,6 +325,10 @@ struct AttnArgs {
     // dependent memory round trip before its first K/V load); base_hint < 0: read them from vp
     int m_hint, base_hint;
     int frag16;  // write the output fragments in the prompt kernel's layout (frag16_index)
+    // nullable: head_dim signs.  The values were summed in a rotated space (a quantized KV layer); the merge
+    // applies the normalized Hadamard transform to each head's result and multiplies by these signs
+    // (crates/compute/src/kv_quant.rs:102-107) before it writes the fragments
+    const float* unrot;
     // a prompt pass of several 16-row blocks in one launch (blocks > 1): block b has its parameters at vp + b,
     // its base position at base_hint + 16 b, and its q rows, partial results and output fragments at the
     // strides below
@@ -343,6 +348,32 @@ __host__ __device__ inline AttnArgs attn_block_view(const AttnArgs& a, int b) {
     return v;
 }
 int launch_attention(hipStream_t s, const AttnArgs& a, int m);
+
+// ---- quantized KV rows (kvquant.hip)
+enum { TQ_TABLE_FLOATS = 512 + 16 + 16 };  // signs (head_dim <= 512), codebook and midpoints (<= 4 bits)
+struct TqSide {
+    const float* signs;  // head_dim
+    const float* cb;     // 1 << bits
+    const float* mid;    // (1 << bits) - 1
+    int bits, words;     // packed words per row: ceil(head_dim * bits / 32)
+};
+struct TqArgs {
+    uint16_t* q16;       // [m][nq][hd] fp16, rotated in place with the key signs
+    uint16_t *kc, *vc;   // the shared fp16 cache in the attention kernels' layouts, `cap` positions
+    uint32_t *kq, *vq;   // the layer's stored rows: [position][kv head][1 + words], norm first
+    TqSide k, v;
+    int nq, nkv, hd, cap;
+    const VerifyParams* vp;
+    int m_hint, base_hint;  // rows of the pass; positions already stored (< 0: read vp->base)
+    float inv_sqrt2;        // set by the launcher
+};
+void tq_sign_vector(int dim, uint64_t seed, float* out);
+std::vector<float> tq_codebook(int dim, int bits);
+int tq_words(int hd, int bits);
+int tq_upload_side(int hd, int bits, uint64_t seed, float* dev, TqSide* out);
+// q rotation, quantization of the pass's rows at base .. base + m - 1 and decoding of the rows before them
+// into the shared cache; max_base sizes a launch that reads its base on the device
+int launch_tq_prepare(hipStream_t s, const TqArgs& a, long max_base);
 int launch_attention_merge(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
 

@@ -44,6 +44,7 @@ class ModelDesc(C.Structure):
         ("layers", C.POINTER(Layer)),
         ("rope_freqs", C.POINTER(C.c_float)), ("rope_mscale", C.c_float),
         ("act_alpha", C.c_float), ("act_limit", C.c_float),
+        ("kv_k_bits", C.c_int32), ("kv_v_bits", C.c_int32),
     ]
 
 
@@ -247,6 +248,7 @@ EXPORTS = [
     "tsv_set_prefix_reuse", "tsv_try_reuse_prefix", "tsv_record_committed", "tsv_prefix_len",
     "tsv_gguf_open", "tsv_gguf_close", "tsv_gguf_tensor_count", "tsv_gguf_data_start", "tsv_gguf_tensor",
     "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected", "tsv_force_route",
+    "tsv_read_kv_quantized", "tsv_attention_quantized", "tsv_kv_quant_tables",
 ]
 
 _lib = None
@@ -312,6 +314,10 @@ def lib():
         L.tsv_matmul.argtypes = [C.POINTER(Tensor), C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
         L.tsv_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                     C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_void_p, C.c_void_p]
+        L.tsv_read_kv_quantized.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
+        L.tsv_attention_quantized.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                              C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_void_p, C.c_void_p,
+                                              C.c_void_p, C.c_void_p]
         L.tsv_set_profile.argtypes = [C.c_void_p, C.c_int32]
         L.tsv_get_profile.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]
         L.tsv_copy_time.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
@@ -425,6 +431,39 @@ def attention(q, k, v, base, parent=None, scale=0.0, window=0, sinks=None):
                               C.c_float(scale), int(window), C.c_void_p(sk.ctypes.data) if sk is not None else None,
                               C.c_void_p(out.ctypes.data)))
     return out.astype(np.float32)
+
+
+def kv_quant_tables(head_dim, bits, value_side=False):
+    """(signs, codebook, midpoints) of one side of the KV codec, as the library computes them on the host."""
+    signs = np.empty(head_dim, np.float32)
+    cb = np.empty(1 << bits, np.float32)
+    mid = np.empty((1 << bits) - 1, np.float32)
+    check(lib().tsv_kv_quant_tables(int(head_dim), int(bits), int(bool(value_side)), C.c_void_p(signs.ctypes.data),
+                                    C.c_void_p(cb.ctypes.data), C.c_void_p(mid.ctypes.data)))
+    return signs, cb, mid
+
+
+def packed_words(head_dim, bits):
+    """crates/model-io/src/kv_quant.rs:128-133."""
+    return (head_dim * bits + 31) // 32 if head_dim > 0 and bits > 0 else 0
+
+
+def attention_quantized(q, k, v, base, k_bits, v_bits, scale=0.0, sinks=None):
+    """q [m, nq, hd], k/v [base+m, nkv, hd] fp16 staging rows -> (fp32 [m, nq, hd], stored K rows, stored V rows);
+    a stored row is [norm bits, words...] u32 per (position, kv head)."""
+    q16, k16, v16 = (np.ascontiguousarray(np.asarray(a, np.float32).astype(np.float16)) for a in (q, k, v))
+    m, nq, hd = q16.shape
+    nkv = k16.shape[1]
+    assert k16.shape[0] == base + m
+    out = np.empty((m, nq, hd), np.float16)
+    kr = np.zeros((base + m, nkv, 1 + packed_words(hd, k_bits)), np.uint32)
+    vr = np.zeros((base + m, nkv, 1 + packed_words(hd, v_bits)), np.uint32)
+    sk = np.ascontiguousarray(sinks, np.float32) if sinks is not None else None
+    check(lib().tsv_attention_quantized(q16.ctypes.data, k16.ctypes.data, v16.ctypes.data, m, nq, nkv, hd, C.c_int64(base),
+                                        int(k_bits), int(v_bits), C.c_float(scale),
+                                        C.c_void_p(sk.ctypes.data) if sk is not None else None, out.ctypes.data,
+                                        kr.ctypes.data, vr.ctypes.data))
+    return out.astype(np.float32), kr, vr
 
 
 def copy_time(nbytes, iters=20):

@@ -30,10 +30,21 @@ def _i32(a):
     return np.ascontiguousarray(a, np.int32)
 
 
-class HipVerifier:
-    """One target model resident on the GPU with its fp16 KV cache."""
+def parse_kv_bits(text):
+    """`--kv-bits` as crates/model-io/src/kv_quant.rs:48-72 reads it: "off" -> None, "2" / "3" / "4" -> the same
+    width on both sides, "3.5" -> 3 bits for keys and 4 for values."""
+    table = {"off": None, "2": (2, 2), "3": (3, 3), "3.5": (3, 4), "4": (4, 4)}
+    if text not in table:
+        raise ValueError(f"--kv-bits must be one of off|2|3|3.5|4, got {text!r}")
+    return table[text]
 
-    def __init__(self, cfg, weights):
+
+class HipVerifier:
+    """One target model resident on the GPU with its KV cache: fp16 rows, or TurboQuant rows on the layers
+    crates/model-io/src/kv_quant.rs:102-107 names when kv_bits = (key bits, value bits) is given
+    (RealForwardRunner::open_with_kv_quant, crates/runtime/src/real_forward_api.rs:568-590)."""
+
+    def __init__(self, cfg, weights, kv_bits=None):
         self.cfg = dict(cfg)
         self._keep = weights
         n = len(weights["layers"])
@@ -63,6 +74,8 @@ class HipVerifier:
         d.rope_mscale = cfg.get("rope_mscale", 0.0)
         d.act_alpha = cfg.get("act_alpha", 0.0)
         d.act_limit = cfg.get("act_limit", 0.0)
+        d.kv_k_bits, d.kv_v_bits = kv_bits if kv_bits else (0, 0)
+        self.kv_bits = tuple(kv_bits) if kv_bits else None
         d.embed = ffi.tensor(weights["embed"])
         d.final_norm = ffi.tensor(weights["final_norm"])
         d.lm_head = ffi.tensor(weights.get("lm_head"))
@@ -82,6 +95,7 @@ class HipVerifier:
         ffi.check(ffi.lib().tsv_open_gguf(os.fsencode(path), int(max_context), C.byref(h)))
         self._h = h
         self._keep = None
+        self.kv_bits = None
         self.vocab = int(ffi.lib().tsv_vocab(h))
         g = ffi.Gguf(path)
         arch = g.string("general.architecture")
@@ -413,6 +427,15 @@ class HipVerifier:
         a = np.ascontiguousarray(np.asarray(sel, np.int32))
         assert a.shape == (n, 16, 8), a.shape
         ffi.check(ffi.lib().tsv_force_route(self._h, a.ctypes.data, n))
+
+    def read_kv_quantized(self, layer, pos0, n):
+        """The stored rows of a quantized layer: (K rows, V rows), each [n, kv heads, 1 + words] u32, norm bits first."""
+        c = self.cfg
+        kb, vb = self.kv_bits
+        k = np.zeros((n, c["n_kv_heads"], 1 + ffi.packed_words(c["head_dim"], kb)), np.uint32)
+        v = np.zeros((n, c["n_kv_heads"], 1 + ffi.packed_words(c["head_dim"], vb)), np.uint32)
+        ffi.check(ffi.lib().tsv_read_kv_quantized(self._h, layer, int(pos0), int(n), k.ctypes.data, v.ctypes.data))
+        return k, v
 
     def read_kv(self, layer, pos0, n):
         c = self.cfg
