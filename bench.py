@@ -224,6 +224,9 @@ def main():
                     help="routed-expert workloads: 'independent' forces every row of every layer onto top_k experts drawn "
                          "uniformly and independently (tsv_force_route) instead of the synthetic router's own, nearly "
                          "row-independent choice; a secondary measurement, labelled in the line")
+    ap.add_argument("--kv-bits", default="off", choices=["off", "2", "3", "3.5", "4"],
+                    help="TurboQuant KV rows on the layers the reference's policy names (crates/model-io/src/kv_quant.rs); "
+                         "a secondary measurement, labelled in the line -- the headline workloads keep fp16 rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=20261125)
     args = ap.parse_args()
@@ -259,7 +262,8 @@ def main():
     weights = synth.make_weights(cfg, seed=args.seed)
     log(f"[bench] synthetic {wl['model']} weights ({cfg['n_layers']} layers) in {time.time() - t0:.1f}s")
     t0 = time.time()
-    eng = ts.HipVerifier(cfg, weights)
+    kv_bits = ts.producer.parse_kv_bits(args.kv_bits)
+    eng = ts.HipVerifier(cfg, weights, kv_bits=kv_bits)
     log(f"[bench] upload + re-tile in {time.time() - t0:.1f}s")
     rng = np.random.default_rng(args.seed)
     if args.prefill_bench:
@@ -414,7 +418,7 @@ def main():
                     profile_ms_per_step={n: round(v[0] / nprof, 4) for n, v in prof.items()})
 
     cpu = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not kv_bits:   # the baseline leg is the headline workloads' (fp16 rows)
         cpu = cpu_baseline(cfg, weights, eng, base, feeds[args.warmup], mean_acc, tree)
 
     out = {
@@ -434,6 +438,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,
                    "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin,
+                   **({"kv_rows": f"TurboQuant K{kv_bits[0]}/V{kv_bits[1]} on every full-attention layer but the last; "
+                                  "algorithmic bytes below still count fp16 rows"} if kv_bits else {}),
                    **({"experts_routed_per_layer": round(union, 2),
                        "routing": "the synthetic router's own" if args.routing == "model" else
                                   "forced: top_k experts per row drawn uniformly and independently"} if union is not None else {})},

@@ -14,7 +14,7 @@
 //    cache pre-arranged as that MFMA's A fragments.
 #include <algorithm>
 
-#include "attn_core.h"
+#include "attn_tq_core.h"
 
 namespace tsv {
 
@@ -37,6 +37,17 @@ __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) 
         return;
     }
     attn_partial_body<HD, RT, STAGES, false>(a, G, R, blockIdx.x, blockIdx.y, grp * RT, xch);
+}
+
+// The same pass over a layer that keeps quantized rows (attn_tq_core.h)
+template <int HD, int RT, int KB, int VB>
+__global__ __launch_bounds__(512) void k_attn_partial_tq(AttnArgs a, int G, int R) {
+    extern __shared__ float xch[];
+    __shared__ uint32_t s_kpair[1 << (2 * KB)], s_vpair[1 << (2 * VB)];
+    tq_fill_pairs(s_kpair, a.tq.k_cb, KB, threadIdx.x, 512);
+    tq_fill_pairs(s_vpair, a.tq.v_cb, VB, threadIdx.x, 512);
+    __syncthreads();
+    attn_partial_body_tq<HD, RT, 3, KB, VB>(a, G, R, blockIdx.x, blockIdx.y, blockIdx.z * RT, xch, s_kpair, s_vpair);
 }
 
 // Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
@@ -135,6 +146,31 @@ static int launch_partial(hipStream_t s, const AttnArgs& a, int G, int R, int gr
 template <int HD>
 static int launch_combine(hipStream_t s, const AttnArgs& a, int m, int G, int R);
 
+template <int HD, int RT, int KB, int VB>
+static int launch_partial_tq(hipStream_t s, const AttnArgs& a, int G, int R, int groups) {
+    constexpr int PER_LANE = RT * (HD / 16) * 4 + 2 * RT;
+    const size_t lds = (size_t)4 * 64 * PER_LANE * 4;
+    static bool raised = false;
+    if (lds > 60000 && !raised) {  // with the pair tables beside it the exchange area passes 64 KiB
+        TSV_HIP(hipFuncSetAttribute((const void*)k_attn_partial_tq<HD, RT, KB, VB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((k_attn_partial_tq<HD, RT, KB, VB>), dim3(a.nch, a.nkv, groups), dim3(512), lds, s, a, G, R);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+template <int HD, int RT>
+static int launch_partial_tq_widths(hipStream_t s, const AttnArgs& a, int G, int R, int groups) {
+    const int kb = a.tq.k_bits, vb = a.tq.v_bits;
+    if (kb == 4 && vb == 4) return launch_partial_tq<HD, RT, 4, 4>(s, a, G, R, groups);
+    if (kb == 3 && vb == 4) return launch_partial_tq<HD, RT, 3, 4>(s, a, G, R, groups);
+    if (kb == 3 && vb == 3) return launch_partial_tq<HD, RT, 3, 3>(s, a, G, R, groups);
+    if (kb == 2 && vb == 2) return launch_partial_tq<HD, RT, 2, 2>(s, a, G, R, groups);
+    set_error("attention: no kernel for these KV quantization widths");
+    return TSV_ERR_UNSUPPORTED;
+}
+
 template <int HD>
 static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     const int trt = (R + 15) / 16;
@@ -145,7 +181,13 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     AttnArgs a = a0;
     a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 256 / (a0.nkv * groups * std::max(a0.blocks, 1))));
     int rc;
-    if (trt <= 1)
+    if (a.tq.k_bits) {
+        if (a.window || a.ring || a.blocks > 1 || !a.unrot) {
+            set_error("attention: quantized rows go with full attention, a linear cache and single passes");
+            return TSV_ERR_UNSUPPORTED;
+        }
+        rc = trt <= 1 ? launch_partial_tq_widths<HD, 1>(s, a, G, R, 1) : launch_partial_tq_widths<HD, 2>(s, a, G, R, groups);
+    } else if (trt <= 1)
         rc = launch_partial<HD, 1, 3>(s, a, G, R, 1);
     else
         rc = launch_partial<HD, 2, 3>(s, a, G, R, groups);

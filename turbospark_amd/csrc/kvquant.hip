@@ -2,25 +2,23 @@
 // quantized layer.
 //
 // A quantized layer keeps, per position and kv head, one f32 norm and the packed codebook indices of
-// the row's rotated unit vector (crates/compute/src/kv_quant.rs:340-382; the row layout of
-// crates/gpu/tests/kv_quantize_parity.rs:22-38: [norm][words]).  Attention runs in the rotated space
-// (crates/compute/src/kv_quant_attention.rs:58-136): q is rotated once with the key signs, scores are
-// <q_rot, codebook[idx]> * norm, the values are summed as norm * codebook[idx] and the sum is rotated
-// back once with the value signs.  Here the rows norm * codebook[idx] are written, as fp16, into an
-// fp16 cache of one layer's size that all quantized layers share, and the ordinary attention kernels
-// read that; the merge kernel rotates the result back.
+// the row's rotated unit vector (crates/compute/src/kv_quant.rs:340-382).  Attention runs in the
+// rotated space (crates/compute/src/kv_quant_attention.rs:58-136): q is rotated once with the key
+// signs, scores are <q_rot, codebook[idx]> * norm, the values are summed as norm * codebook[idx] and
+// the sum is rotated back once with the value signs.  The attention kernel reads the stores directly
+// (attn_tq_core.h, which also states their layout); the merge kernel rotates the result back.
 //
-// The pass's own rows arrive in that shared cache as fp16 (the staging row of
+// The pass's own rows arrive as fp16 in a sixteen-slot staging cache (the staging row of
 // crates/runtime/src/kv_write.rs:66-118) and are quantized from there: norm as the f32 sum of squares
 // in index order, unit = x * (1 / max(norm, 1e-6)), the butterflies of crates/compute/src/wht.rs:15-29
 // in their order with each stage scaled by 1/sqrt(2), one index per coordinate as the count of
-// midpoints below it, bits LSB first.  Every operation is a single rounded f32 operation in the
-// reference's order, so the words and the norm are the reference's by bits.
+// midpoints below it.  Every operation is a single rounded f32 operation in the reference's order, so
+// the indices and the norm are the reference's by bits.
 #include <algorithm>
 #include <cmath>
 #include <vector>
 
-#include "tsv_internal.h"
+#include "attn_tq_core.h"
 
 namespace tsv {
 
@@ -149,24 +147,10 @@ __device__ __forceinline__ void wht(float (&e)[EPL], int lane, float c) {
     }
 }
 
-__device__ __forceinline__ long k_at(const TqArgs& a, int head, int pos, int d) { return ((long)head * a.cap + pos) * a.hd + d; }
-__device__ __forceinline__ long v_at(const TqArgs& a, int head, int pos, int d) {
+__device__ __forceinline__ long k_at(int cap, int hd, int head, int pos, int d) { return ((long)head * cap + pos) * hd + d; }
+__device__ __forceinline__ long v_at(int cap, int hd, int head, int pos, int d) {
     const int po = pos & 15;
-    return ((long)head * (a.cap >> 4) + (pos >> 4)) * (a.hd * 16) + (((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3);
-}
-
-__device__ __forceinline__ uint32_t index_at(const uint32_t* words, int i, int bits) {
-    const uint32_t bit = (uint32_t)i * (uint32_t)bits, w = bit >> 5, off = bit & 31;
-    uint32_t v = words[w] >> off;
-    if (off + bits > 32) v |= words[w + 1] << (32 - off);
-    return v & ((1u << bits) - 1u);
-}
-
-// what a stored row reads as in the rotated space: fp16(norm * codebook[idx]), one rounded product
-__device__ __forceinline__ _Float16 decoded(float norm, float level) {
-    float p = __fmul_rn(norm, level);
-    asm volatile("" : "+v"(p));  // the product is rounded to f32 before it is rounded to fp16
-    return (_Float16)p;
+    return ((long)head * (cap >> 4) + (pos >> 4)) * (hd * 16) + (((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3);
 }
 
 // q row (b, qh): rotate with the key signs, in place
@@ -182,21 +166,21 @@ __device__ void rotate_q(const TqArgs& a, int b, int qh, int lane) {
     for (int j = 0; j < EPL; j++) row[lane + 64 * j] = (_Float16)e[j];
 }
 
-// the pass's row at `pos`, kv head `head`: fp16 row in the shared cache -> norm + words in the layer's
-// store, and the decoded row back into the shared cache
+// the pass's row at `pos`, kv head `head`: fp16 staging row -> norm and indices in the layer's stores
 template <int HD>
 __device__ void commit_row(const TqArgs& a, bool value, int pos, int head, int lane, float* s_row, uint32_t* s_words) {
     constexpr int EPL = HD / 64;
     const TqSide& t = value ? a.v : a.k;
-    _Float16* cache = (_Float16*)(value ? a.vc : a.kc);
+    const _Float16* stage = (const _Float16*)(value ? a.vc : a.kc);
+    const int slot = pos % a.stage_cap;
     float x[EPL];
 #pragma unroll
     for (int j = 0; j < EPL; j++) {
         const int d = lane + 64 * j;
-        x[j] = (float)cache[value ? v_at(a, head, pos, d) : k_at(a, head, pos, d)];
+        x[j] = (float)stage[value ? v_at(a.stage_cap, HD, head, slot, d) : k_at(a.stage_cap, HD, head, slot, d)];
         s_row[d] = x[j];
     }
-    if (lane < t.words + 1) s_words[lane] = 0;
+    if (!value && lane < t.words + 1) s_words[lane] = 0;
     lds_order();
     float ss = 0.f;
     for (int i = 0; i < HD; i++) ss = __fadd_rn(ss, __fmul_rn(s_row[i], s_row[i]));
@@ -207,118 +191,75 @@ __device__ void commit_row(const TqArgs& a, bool value, int pos, int head, int l
     for (int j = 0; j < EPL; j++) e[j] = __fmul_rn(__fmul_rn(x[j], inv), t.signs[lane + 64 * j]);
     wht<EPL>(e, lane, a.inv_sqrt2);
     const int n_mid = (1 << t.bits) - 1;
-    uint32_t idx[EPL];
+    if (lane == 0) (value ? a.store.vn : a.store.kn)[(long)head * a.cap + pos] = norm;
+    if (!value) {
+        // a K row: packed LSB first (kv_quant.rs:289-312), assembled in LDS
 #pragma unroll
-    for (int j = 0; j < EPL; j++) {
-        uint32_t c = 0;
-        for (int i = 0; i < n_mid; i++) c += e[j] > t.mid[i] ? 1u : 0u;
-        idx[j] = c;
-        const uint32_t bit = (uint32_t)(lane + 64 * j) * (uint32_t)t.bits, w = bit >> 5, off = bit & 31;
-        atomicOr(&s_words[w], c << off);
-        if (off + t.bits > 32) atomicOr(&s_words[w + 1], c >> (32 - off));
-    }
-    lds_order();
-    uint32_t* out = (value ? a.vq : a.kq) + ((long)pos * a.nkv + head) * (1 + t.words);
-    if (lane == 0) out[0] = __builtin_bit_cast(uint32_t, norm);
-    if (lane < t.words) out[1 + lane] = s_words[lane];
-#pragma unroll
-    for (int j = 0; j < EPL; j++) {
-        const int d = lane + 64 * j;
-        cache[value ? v_at(a, head, pos, d) : k_at(a, head, pos, d)] = decoded(norm, t.cb[idx[j]]);
-    }
-    lds_order();
-}
-
-// a stored key row back into the shared cache
-template <int HD>
-__device__ void expand_k(const TqArgs& a, int pos, int head, int lane) {
-    constexpr int EPL = HD / 64;
-    const uint32_t* row = a.kq + ((long)pos * a.nkv + head) * (1 + a.k.words);
-    const float norm = __builtin_bit_cast(float, row[0]);
-    _Float16 h[EPL];
-#pragma unroll
-    for (int j = 0; j < EPL; j++) h[j] = decoded(norm, a.k.cb[index_at(row + 1, EPL * lane + j, a.k.bits)]);
-    _Float16* dst = (_Float16*)a.kc + k_at(a, head, pos, EPL * lane);
-    if (EPL == 2) {
-        *(uint32_t*)dst = (uint32_t)__builtin_bit_cast(uint16_t, h[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, h[EPL - 1]) << 16);
+        for (int j = 0; j < EPL; j++) {
+            uint32_t c = 0;
+            for (int i = 0; i < n_mid; i++) c += e[j] > t.mid[i] ? 1u : 0u;
+            const uint32_t bit = (uint32_t)(lane + 64 * j) * (uint32_t)t.bits, w = bit >> 5, off = bit & 31;
+            atomicOr(&s_words[w], c << off);
+            if (off + t.bits > 32) atomicOr(&s_words[w + 1], c >> (32 - off));
+        }
+        lds_order();
+        if (lane < t.words) a.store.kq[((long)head * a.cap + pos) * t.words + lane] = s_words[lane];
     } else {
-        dst[0] = h[0];
-    }
-}
-
-// sixteen stored value rows back into the shared cache: lane (j, dl) holds positions 4j .. 4j+3 of
-// dimension 16 dh + dl, eight contiguous bytes of the block's layout
-template <int HD>
-__device__ void expand_v(const TqArgs& a, int blk, int head, int base, int lane) {
-    const int j = lane >> 4, dl = lane & 15, p0 = blk * 16 + 4 * j;
-    const uint32_t* rows[4];
-    float norm[4];
+        // a V row: index of dimension d into bits (pos % 16) * bits .. of that dimension's group of the block;
+        // other rows of the pass own other bits of the same words
+        const int gw = tq_v_group_words(t.bits);
+        const uint32_t off = (uint32_t)(pos & 15) * (uint32_t)t.bits;
+        const uint64_t mask = (uint64_t)n_mid << off;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        rows[i] = a.vq + ((long)min(p0 + i, base - 1) * a.nkv + head) * (1 + a.v.words);
-        norm[i] = __builtin_bit_cast(float, rows[i][0]);
-    }
-    _Float16* dst = (_Float16*)a.vc + ((long)head * (a.cap >> 4) + blk) * (HD * 16);
-    const bool whole = p0 + 4 <= base;
-#pragma unroll 2
-    for (int dh = 0; dh < HD / 16; dh++) {
-        const int d = dh * 16 + dl;
-        uint16_t h[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) h[i] = __builtin_bit_cast(uint16_t, decoded(norm[i], a.v.cb[index_at(rows[i] + 1, d, a.v.bits)]));
-        _Float16* at = dst + (dh * 64 + lane) * 4;
-        if (whole) {
-            *(uint2*)at = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-        } else {  // the block the pass's own rows start in: those are the other kernel section's to write
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (p0 + i < base) at[i] = __builtin_bit_cast(_Float16, h[i]);
+        for (int j = 0; j < EPL; j++) {
+            uint32_t c = 0;
+            for (int i = 0; i < n_mid; i++) c += e[j] > t.mid[i] ? 1u : 0u;
+            const uint64_t bits = (uint64_t)c << off;
+            uint32_t* g = a.store.vq + (((long)head * (a.cap >> 4) + (pos >> 4)) * HD + lane + 64 * j) * gw;
+            if ((uint32_t)mask) {
+                __hip_atomic_fetch_and(g, ~(uint32_t)mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_or(g, (uint32_t)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (gw == 2 && (uint32_t)(mask >> 32)) {
+                __hip_atomic_fetch_and(g + 1, ~(uint32_t)(mask >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_or(g + 1, (uint32_t)(bits >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
+    lds_order();
 }
 
-// One wave per unit of work, units in four classes: q rows to rotate, the pass's K and V rows to
-// quantize, stored K rows and stored blocks of sixteen V rows to decode.  The classes touch disjoint
-// bytes, so their order does not matter.
+// One wave per unit of work: the q rows to rotate, then the pass's K and V rows to quantize.
 template <int HD>
 __global__ __launch_bounds__(256) void k_tq_prepare(TqArgs a) {
     __shared__ float s_row[4][HD];
     __shared__ uint32_t s_words[4][HD / 2 + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = a.m_hint, base = a.base_hint >= 0 ? a.base_hint : a.vp->base;
-    const long n_q = (long)m * a.nq, n_commit = 2l * m * a.nkv, n_k = (long)base * a.nkv, n_v = (long)((base + 15) >> 4) * a.nkv;
-    const long total = n_q + n_commit + n_k + n_v;
-    for (long u = (long)blockIdx.x * 4 + wave; u < total; u += (long)gridDim.x * 4) {
+    const int n_q = m * a.nq, n_rows = m * a.nkv, total = n_q + 2 * n_rows;
+    for (int u = blockIdx.x * 4 + wave; u < total; u += gridDim.x * 4) {
         if (u < n_q) {
-            rotate_q<HD>(a, (int)(u / a.nq), (int)(u % a.nq), lane);
-        } else if (u < n_q + n_commit) {
-            const long r = u - n_q;
-            const bool value = r >= (long)m * a.nkv;
-            const int rr = (int)(value ? r - (long)m * a.nkv : r);
-            commit_row<HD>(a, value, (base + rr / a.nkv) % a.cap, rr % a.nkv, lane, s_row[wave], s_words[wave]);
-        } else if (u < n_q + n_commit + n_k) {
-            const long r = u - n_q - n_commit;
-            expand_k<HD>(a, (int)(r / a.nkv), (int)(r % a.nkv), lane);
+            rotate_q<HD>(a, u / a.nq, u % a.nq, lane);
         } else {
-            const long r = u - n_q - n_commit - n_k;
-            expand_v<HD>(a, (int)(r / a.nkv), (int)(r % a.nkv), base, lane);
+            const bool value = u - n_q >= n_rows;
+            const int r = u - n_q - (value ? n_rows : 0);
+            commit_row<HD>(a, value, base + r / a.nkv, r % a.nkv, lane, s_row[wave], s_words[wave]);
         }
     }
 }
 
 }  // namespace
 
-int launch_tq_prepare(hipStream_t s, const TqArgs& a0, long max_base) {
+int launch_tq_prepare(hipStream_t s, const TqArgs& a0) {
     TqArgs a = a0;
     a.inv_sqrt2 = 1.0f / std::sqrt(2.0f);
-    if ((a.hd != 64 && a.hd != 128) || a.cap % 16 || a.k.bits < 1 || a.k.bits > 4 || a.v.bits < 1 || a.v.bits > 4) {
-        set_error("quantized KV: head_dim must be 64 or 128 and the widths 1..4 bits");
+    if ((a.hd != 64 && a.hd != 128) || a.cap % 16 || a.stage_cap % 16 || a.m_hint > a.stage_cap || a.k.bits < 2 || a.k.bits > 4 ||
+        a.v.bits < 2 || a.v.bits > 4) {
+        set_error("quantized KV: head_dim must be 64 or 128 and the widths 2..4 bits");
         return TSV_ERR_UNSUPPORTED;
     }
-    // a launch that reads its base position on the device (a captured one) is sized for the longest prefix
-    const long base = a.base_hint >= 0 ? a.base_hint : max_base;
-    const long units = (long)a.m_hint * (a.nq + 2 * a.nkv) + base * a.nkv + ((base + 15) / 16) * a.nkv;
-    const int blocks = (int)std::max(1l, std::min((units + 3) / 4, 8192l));
+    const int units = a.m_hint * (a.nq + 2 * a.nkv);
+    const int blocks = std::max(1, (units + 3) / 4);
     if (a.hd == 128)
         hipLaunchKernelGGL(k_tq_prepare<128>, dim3(blocks), dim3(256), 0, s, a);
     else
@@ -326,5 +267,8 @@ int launch_tq_prepare(hipStream_t s, const TqArgs& a0, long max_base) {
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
+
+size_t tq_kq_bytes(int nkv, int cap, int hd, int k_bits) { return (size_t)nkv * cap * tq_words(hd, k_bits) * 4; }
+size_t tq_vq_bytes(int nkv, int cap, int hd, int v_bits) { return (size_t)nkv * (cap / 16) * hd * tq_v_group_words(v_bits) * 4; }
 
 }  // namespace tsv

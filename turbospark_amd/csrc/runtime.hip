@@ -33,9 +33,10 @@ struct LayerW {
     int cap = 0;        // positions the layer's cache holds: the context, or a ring of window + slack
     bool rope_fused = false;  // the q/k/v projection rotates and stores its own rows
     uint16_t *kc = nullptr, *vc = nullptr;
-    // a quantized layer (TurboQuant): kc / vc are then the fp16 cache all such layers share, and these
-    // the layer's own rows, [position][kv head][1 + words] with the norm first
-    uint32_t *kq = nullptr, *vq = nullptr;
+    // a quantized layer (TurboQuant): kc / vc are then the sixteen-slot fp16 staging cache all such layers
+    // share (kv_slots positions instead of cap), and tq the layer's own stores
+    int kv_slots = 0;
+    TqKv tq{};
 };
 
 int dtype_fmt(int dtype) {
@@ -124,7 +125,7 @@ struct tsv_ctx {
     AcceptScratch sc{};
     std::vector<void*> allocs;
     // TurboQuant KV rows (crates/model-io/src/kv_quant.rs): widths (0 = every layer fp16), the tables of the two
-    // sides and the fp16 cache the quantized layers decode into before their attention
+    // sides and the fp16 staging rows of the pass in flight (crates/runtime/src/kv_write.rs:36-60)
     int kv_k_bits = 0, kv_v_bits = 0;
     TqSide tq_k{}, tq_v{};
     uint16_t *tq_kc = nullptr, *tq_vc = nullptr;
@@ -568,7 +569,7 @@ int launch_pass(tsv_ctx* c, int m) {
             re.nq = c->nq;
             re.nkv = c->nkv;
             re.hd = c->hd;
-            re.max_ctx = L.cap;
+            re.max_ctx = L.kv_slots;
             PROF(PC_QKV);
             rc = 0;
             for (int rep = 0; rep < c->repeat[PC_QKV] && !rc; rep++)
@@ -600,7 +601,7 @@ int launch_pass(tsv_ctx* c, int m) {
         ra.nq = c->nq;
         ra.nkv = c->nkv;
         ra.hd = c->hd;
-        ra.max_ctx = L.cap;
+        ra.max_ctx = L.kv_slots;
         ra.vp = c->vp_dev;
         if (!L.rope_fused) {
             PROF(PC_ROPE);
@@ -608,16 +609,16 @@ int launch_pass(tsv_ctx* c, int m) {
             for (int rep = 0; rep < c->repeat[PC_ROPE] && !rc; rep++) rc = launch_rope_kv(s, ra, m);
         }
         if (rc) return rc;
-        if (L.kq) {
-            // the pass's K / V rows sit in the shared fp16 cache (the staging rows of
-            // crates/runtime/src/kv_write.rs:66-118): quantize them into the layer's store, decode the rows
-            // before them, rotate q -- attention then runs in the rotated space (kv_quant_attention.rs:58-136)
+        if (L.tq.k_bits) {
+            // the pass's K / V rows sit in the staging cache (crates/runtime/src/kv_write.rs:66-118): quantize them
+            // into the layer's stores and rotate q -- attention then runs in the rotated space, over the stores
+            // (kv_quant_attention.rs:58-136)
             TqArgs ta{};
             ta.q16 = c->q16;
             ta.kc = L.kc;
             ta.vc = L.vc;
-            ta.kq = L.kq;
-            ta.vq = L.vq;
+            ta.stage_cap = L.kv_slots;
+            ta.store = L.tq;
             ta.k = c->tq_k;
             ta.v = c->tq_v;
             ta.nq = c->nq;
@@ -628,14 +629,15 @@ int launch_pass(tsv_ctx* c, int m) {
             ta.m_hint = m;
             ta.base_hint = c->use_graph ? -1 : c->vp_host->base;
             PROF(PC_ROPE);
-            rc = launch_tq_prepare(s, ta, c->ctx_alloc);
+            rc = launch_tq_prepare(s, ta);
             if (rc) return rc;
         }
         AttnArgs aa{};
         aa.q16 = c->q16;
         aa.kc = L.kc;
         aa.vc = L.vc;
-        aa.unrot = L.kq ? c->tq_v.signs : nullptr;
+        aa.unrot = L.tq.k_bits ? c->tq_v.signs : nullptr;
+        aa.tq = L.tq;
         aa.part_o = c->part_o;
         aa.part_ml = c->part_ml;
         aa.xfrag = c->xf_b;
@@ -1213,13 +1215,21 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         const size_t kvb = (size_t)c->nkv * L.cap * c->hd * 2;
         // crates/model-io/src/kv_quant.rs:102-107: every full-attention layer of a stack of at most two, else
         // every one but the last; windowed layers keep fp16 rows
+        L.kv_slots = L.cap;
         if (c->kv_k_bits && s.window == 0 && (c->n_layers <= 2 || l + 1 < c->n_layers)) {
-            if (!c->tq_kc && ((rc = dev_alloc(c, &c->tq_kc, kvb, true)) || (rc = dev_alloc(c, &c->tq_vc, kvb, true)))) return fail(rc);
+            L.kv_slots = TSV_MAX_ROWS;
+            const size_t stage = (size_t)c->nkv * L.kv_slots * c->hd * 2;
+            if (!c->tq_kc && ((rc = dev_alloc(c, &c->tq_kc, stage, true)) || (rc = dev_alloc(c, &c->tq_vc, stage, true)))) return fail(rc);
             L.kc = c->tq_kc;
             L.vc = c->tq_vc;
-            const size_t rows = (size_t)L.cap * c->nkv;
-            if ((rc = dev_alloc(c, &L.kq, rows * (1 + c->tq_k.words) * 4, true)) ||
-                (rc = dev_alloc(c, &L.vq, rows * (1 + c->tq_v.words) * 4, true)))
+            L.tq.k_bits = c->kv_k_bits;
+            L.tq.v_bits = c->kv_v_bits;
+            L.tq.k_cb = c->tq_k.cb;
+            L.tq.v_cb = c->tq_v.cb;
+            const size_t norms = (size_t)c->nkv * L.cap * 4;
+            if ((rc = dev_alloc(c, &L.tq.kq, tq_kq_bytes(c->nkv, L.cap, c->hd, c->kv_k_bits), true)) ||
+                (rc = dev_alloc(c, &L.tq.vq, tq_vq_bytes(c->nkv, L.cap, c->hd, c->kv_v_bits), true)) ||
+                (rc = dev_alloc(c, &L.tq.kn, norms, true)) || (rc = dev_alloc(c, &L.tq.vn, norms, true)))
                 return fail(rc);
         } else if ((rc = dev_alloc(c, &L.kc, kvb, true)) || (rc = dev_alloc(c, &L.vc, kvb, true))) {
             return fail(rc);
@@ -1861,7 +1871,7 @@ extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t 
         set_error("read_kv: null argument or range outside the cache");
         return TSV_ERR_INVALID;
     }
-    if (c->layers[layer].kq) {
+    if (c->layers[layer].tq.k_bits) {
         set_error("read_kv: this layer keeps quantized rows (tsv_read_kv_quantized reads them)");
         return TSV_ERR_UNSUPPORTED;
     }
@@ -1946,7 +1956,7 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
         set_error("write_kv: range outside the cache");
         return TSV_ERR_INVALID;
     }
-    if (c->layers[layer].kq) {
+    if (c->layers[layer].tq.k_bits) {
         set_error("write_kv: this layer keeps quantized rows");
         return TSV_ERR_UNSUPPORTED;
     }
@@ -2132,6 +2142,43 @@ extern "C" int32_t tsv_kv_quant_tables(int32_t head_dim, int32_t bits, int32_t v
     return TSV_OK;
 }
 
+namespace {
+// The stores of positions [pos0, pos0 + n) as the rows the reference keeps, [position][kv head][norm, words]
+// (crates/gpu/tests/kv_quantize_parity.rs:22-38): K rows are stored that way but for the norm; V indices are
+// stored transposed per block of sixteen positions and are packed back LSB first (kv_quant.rs:289-312) here.
+int tq_rows_to_host(hipStream_t stream, const TqKv& t, int nkv, int hd, int cap, int64_t pos0, int64_t n, uint32_t* k_rows,
+                    uint32_t* v_rows) {
+    const int kw = tq_words(hd, t.k_bits), vw = tq_words(hd, t.v_bits), gw = t.v_bits == 2 ? 1 : 2;
+    std::vector<uint32_t> kq((size_t)nkv * cap * kw), vq(tq_vq_bytes(nkv, cap, hd, t.v_bits) / 4);
+    std::vector<float> kn((size_t)nkv * cap), vn((size_t)nkv * cap);
+    TSV_HIP(hipStreamSynchronize(stream));
+    TSV_HIP(hipMemcpy(kq.data(), t.kq, kq.size() * 4, hipMemcpyDeviceToHost));
+    TSV_HIP(hipMemcpy(vq.data(), t.vq, vq.size() * 4, hipMemcpyDeviceToHost));
+    TSV_HIP(hipMemcpy(kn.data(), t.kn, kn.size() * 4, hipMemcpyDeviceToHost));
+    TSV_HIP(hipMemcpy(vn.data(), t.vn, vn.size() * 4, hipMemcpyDeviceToHost));
+    for (int64_t i = 0; i < n; i++) {
+        const int64_t pos = pos0 + i;
+        for (int h = 0; h < nkv; h++) {
+            uint32_t* kr = k_rows + ((size_t)i * nkv + h) * (1 + kw);
+            std::memcpy(kr, &kn[(size_t)h * cap + pos], 4);
+            std::memcpy(kr + 1, &kq[((size_t)h * cap + pos) * kw], (size_t)kw * 4);
+            uint32_t* vr = v_rows + ((size_t)i * nkv + h) * (1 + vw);
+            std::memcpy(vr, &vn[(size_t)h * cap + pos], 4);
+            std::fill(vr + 1, vr + 1 + vw, 0u);
+            for (int d = 0; d < hd; d++) {
+                const uint32_t* g = &vq[(((size_t)h * (cap / 16) + pos / 16) * hd + d) * gw];
+                const uint64_t group = gw == 2 ? ((uint64_t)g[1] << 32) | g[0] : g[0];
+                const uint32_t idx = (uint32_t)(group >> ((pos & 15) * t.v_bits)) & ((1u << t.v_bits) - 1u);
+                const uint32_t bit = (uint32_t)d * t.v_bits, w = bit >> 5, off = bit & 31;
+                vr[1 + w] |= idx << off;
+                if (off + t.v_bits > 32) vr[1 + w + 1] |= idx >> (32 - off);
+            }
+        }
+    }
+    return TSV_OK;
+}
+}  // namespace
+
 extern "C" int32_t tsv_read_kv_quantized(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, uint32_t* k_rows,
                                          uint32_t* v_rows) {
     if (!c || !k_rows || !v_rows || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
@@ -2139,15 +2186,11 @@ extern "C" int32_t tsv_read_kv_quantized(tsv_ctx* c, int32_t layer, int64_t pos0
         return TSV_ERR_INVALID;
     }
     const LayerW& L = c->layers[layer];
-    if (!L.kq) {
+    if (!L.tq.k_bits) {
         set_error("read_kv_quantized: this layer keeps fp16 rows");
         return TSV_ERR_INVALID;
     }
-    const size_t kw = (size_t)c->nkv * (1 + c->tq_k.words), vw = (size_t)c->nkv * (1 + c->tq_v.words);
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    TSV_HIP(hipMemcpy(k_rows, L.kq + (size_t)pos0 * kw, (size_t)n * kw * 4, hipMemcpyDeviceToHost));
-    TSV_HIP(hipMemcpy(v_rows, L.vq + (size_t)pos0 * vw, (size_t)n * vw * 4, hipMemcpyDeviceToHost));
-    return TSV_OK;
+    return tq_rows_to_host(c->stream, L.tq, c->nkv, c->hd, L.cap, pos0, n, k_rows, v_rows);
 }
 
 extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
@@ -2155,7 +2198,7 @@ extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k,
                                            float scale, const float* sinks, uint16_t* out, uint32_t* k_rows,
                                            uint32_t* v_rows) {
     if (!q || !k || !v || !out || !k_rows || !v_rows || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0 ||
-        k_bits < 1 || k_bits > 4 || v_bits < 1 || v_bits > 4 || (hd != 64 && hd != 128)) {
+        k_bits < 2 || k_bits > 4 || v_bits < 2 || v_bits > 4 || (hd != 64 && hd != 128)) {
         set_error("attention_quantized: bad argument");
         return TSV_ERR_INVALID;
     }
@@ -2164,25 +2207,28 @@ extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k,
     TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
     VerifyParams vp;
     int rc = fill_params(vp, nullptr, nullptr, m, base, 0);
-    const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv;
-    const size_t kvb = (size_t)nkv * ctx * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
-    const size_t kwb = (size_t)ctx * nkv * (1 + tq_words(hd, k_bits)) * 4, vwb = (size_t)ctx * nkv * (1 + tq_words(hd, v_bits)) * 4;
+    const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv, slots = TSV_MAX_ROWS;
+    const size_t stb = (size_t)nkv * slots * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
     uint16_t *kc = nullptr, *vc = nullptr, *kin = nullptr, *vin = nullptr, *q16 = nullptr;
-    uint32_t *kq = nullptr, *vq = nullptr;
     float *po = nullptr, *pml = nullptr, *sinks_dev = nullptr, *tables = nullptr;
     uint4* xf = nullptr;
     VerifyParams* vpd = nullptr;
     const size_t xfb = xfrag_bytes(nq * hd);
     TqArgs ta{};
+    TqKv st{};
+    st.k_bits = k_bits;
+    st.v_bits = v_bits;
     if (!rc && sinks) {
         rc = dev_alloc(c, &sinks_dev, (size_t)nq * 4);
         if (!rc && hipMemcpyAsync(sinks_dev, sinks, (size_t)nq * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess)
             rc = TSV_ERR_DEVICE;
     }
-    if (!rc) rc = dev_alloc(c, &kc, kvb, true);
-    if (!rc) rc = dev_alloc(c, &vc, kvb, true);
-    if (!rc) rc = dev_alloc(c, &kq, kwb, true);
-    if (!rc) rc = dev_alloc(c, &vq, vwb, true);
+    if (!rc) rc = dev_alloc(c, &kc, stb, true);
+    if (!rc) rc = dev_alloc(c, &vc, stb, true);
+    if (!rc) rc = dev_alloc(c, &st.kq, tq_kq_bytes(nkv, ctx, hd, k_bits), true);
+    if (!rc) rc = dev_alloc(c, &st.vq, tq_vq_bytes(nkv, ctx, hd, v_bits), true);
+    if (!rc) rc = dev_alloc(c, &st.kn, (size_t)nkv * ctx * 4, true);
+    if (!rc) rc = dev_alloc(c, &st.vn, (size_t)nkv * ctx * 4, true);
     if (!rc) rc = dev_alloc(c, &kin, inb);
     if (!rc) rc = dev_alloc(c, &vin, inb);
     if (!rc) rc = dev_alloc(c, &q16, qb);
@@ -2198,39 +2244,35 @@ extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k,
                 hipMemcpyAsync(q16, q, qb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
                 hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess))
         rc = TSV_ERR_DEVICE;
+    st.k_cb = ta.k.cb;
+    st.v_cb = ta.v.cb;
     ta.q16 = q16;
     ta.kc = kc;
     ta.vc = vc;
-    ta.kq = kq;
-    ta.vq = vq;
+    ta.stage_cap = slots;
+    ta.store = st;
     ta.nkv = nkv;
     ta.hd = hd;
     ta.cap = ctx;
     ta.vp = vpd;
-    // the rows before the pass: staged, quantized as one wide "pass" at position 0, then wiped from the
-    // fp16 cache so that what attention reads of them is what the decoder wrote
-    if (!rc && base > 0) {
-        rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, 0, (int)base, kin, vin);
-        ta.nq = 0;
-        ta.m_hint = (int)base;
-        ta.base_hint = 0;
-        if (!rc) rc = launch_tq_prepare(c->stream, ta, 0);
-        if (!rc && (hipMemsetAsync(kc, 0, kvb, c->stream) != hipSuccess || hipMemsetAsync(vc, 0, kvb, c->stream) != hipSuccess))
-            rc = TSV_ERR_DEVICE;
-    }
-    // the pass itself, as the forward runs it
+    // every row goes through the staging slots and the quantizer, sixteen at a time as passes do; the last
+    // group is the pass itself, whose q rows are rotated with it
     const size_t row = (size_t)nkv * hd;
-    if (!rc) rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, (int)base, m, kin + (size_t)base * row, vin + (size_t)base * row);
-    ta.nq = nq;
-    ta.m_hint = m;
-    ta.base_hint = (int)base;
-    if (!rc) rc = launch_tq_prepare(c->stream, ta, base);
+    for (int64_t p = 0; !rc && p < seq;) {
+        const bool last = p >= base;
+        const int n = last ? m : (int)std::min<int64_t>(slots, base - p);
+        rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, slots, (int)p, n, kin + (size_t)p * row, vin + (size_t)p * row);
+        ta.nq = last ? nq : 0;
+        ta.m_hint = n;
+        ta.base_hint = (int)p;
+        if (!rc) rc = launch_tq_prepare(c->stream, ta);
+        p += n;
+    }
     if (!rc) {
         AttnArgs aa{};
         aa.q16 = q16;
-        aa.kc = kc;
-        aa.vc = vc;
         aa.unrot = ta.v.signs;
+        aa.tq = st;
         aa.part_o = po;
         aa.part_ml = pml;
         aa.xfrag = xf;
@@ -2247,14 +2289,12 @@ extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k,
         rc = launch_attention(c->stream, aa, m);
     }
     std::vector<uint16_t> frag(xfb / 2);
-    const size_t kn = (size_t)seq * nkv * (1 + tq_words(hd, k_bits)) * 4, vn = (size_t)seq * nkv * (1 + tq_words(hd, v_bits)) * 4;
     if (!rc && (hipMemcpyAsync(frag.data(), xf, xfb, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-                hipMemcpyAsync(k_rows, kq, kn, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-                hipMemcpyAsync(v_rows, vq, vn, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
                 hipStreamSynchronize(c->stream) != hipSuccess)) {
         set_error("attention_quantized: device execution failed");
         rc = TSV_ERR_DEVICE;
     }
+    if (!rc) rc = tq_rows_to_host(c->stream, st, nkv, hd, ctx, 0, seq, k_rows, v_rows);
     if (!rc)
         for (int b = 0; b < m; b++)
             for (int kk = 0; kk < nq * hd; kk++) out[(size_t)b * nq * hd + kk] = frag[(size_t)frag_index(kk, b)];

@@ -308,6 +308,17 @@ struct RopeKvArgs {
 };
 int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m);
 
+// The stores of a layer whose K / V rows are kept quantized (TurboQuant; layout in attn_tq_core.h)
+struct TqKv {
+    uint32_t* kq;   // [kv head][position][head_dim * k_bits / 32]
+    float* kn;      // [kv head][position]
+    uint32_t* vq;   // [kv head][position / 16][head_dim][1 or 2]
+    float* vn;      // [kv head][position]
+    const float* k_cb;  // codebook levels of the two sides
+    const float* v_cb;
+    int k_bits, v_bits;  // 0: the layer keeps fp16 rows
+};
+
 struct AttnArgs {
     const uint16_t* q16;
     const uint16_t* kc;
@@ -329,6 +340,7 @@ struct AttnArgs {
     // applies the normalized Hadamard transform to each head's result and multiplies by these signs
     // (crates/compute/src/kv_quant.rs:102-107) before it writes the fragments
     const float* unrot;
+    TqKv tq;  // k_bits != 0: K and V come from these stores instead of kc / vc (q already rotated, unrot set)
     // a prompt pass of several 16-row blocks in one launch (blocks > 1): block b has its parameters at vp + b,
     // its base position at base_hint + 16 b, and its q rows, partial results and output fragments at the
     // strides below
@@ -359,21 +371,26 @@ struct TqSide {
 };
 struct TqArgs {
     uint16_t* q16;       // [m][nq][hd] fp16, rotated in place with the key signs
-    uint16_t *kc, *vc;   // the shared fp16 cache in the attention kernels' layouts, `cap` positions
-    uint32_t *kq, *vq;   // the layer's stored rows: [position][kv head][1 + words], norm first
+    // the pass's K / V rows as the q/k/v projection left them: fp16 caches of `stage_cap` positions in the
+    // attention kernels' layouts, row b of the pass in slot (base + b) % stage_cap
+    const uint16_t *kc, *vc;
+    int stage_cap;
+    TqKv store;          // where the rows go, at position base + b
     TqSide k, v;
-    int nq, nkv, hd, cap;
+    int nq, nkv, hd, cap;  // cap: positions the stores hold
     const VerifyParams* vp;
-    int m_hint, base_hint;  // rows of the pass; positions already stored (< 0: read vp->base)
+    int m_hint, base_hint;  // rows of the pass; position of its first row (< 0: read vp->base)
     float inv_sqrt2;        // set by the launcher
 };
 void tq_sign_vector(int dim, uint64_t seed, float* out);
 std::vector<float> tq_codebook(int dim, int bits);
 int tq_words(int hd, int bits);
 int tq_upload_side(int hd, int bits, uint64_t seed, float* dev, TqSide* out);
-// q rotation, quantization of the pass's rows at base .. base + m - 1 and decoding of the rows before them
-// into the shared cache; max_base sizes a launch that reads its base on the device
-int launch_tq_prepare(hipStream_t s, const TqArgs& a, long max_base);
+// q rotation and quantization of the pass's rows into the stores
+int launch_tq_prepare(hipStream_t s, const TqArgs& a);
+// bytes of a layer's four stores for `cap` positions (cap a multiple of 16)
+size_t tq_kq_bytes(int nkv, int cap, int hd, int k_bits);
+size_t tq_vq_bytes(int nkv, int cap, int hd, int v_bits);
 int launch_attention_merge(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
 
