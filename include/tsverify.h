@@ -98,8 +98,8 @@ typedef struct {
      * both 0 for fp16 rows everywhere; the pairs --kv-bits can name are 2/2, 3/3, 3/4 ("3.5") and 4/4.
      * Quantized are the full-attention layers (window == 0), all of them in a stack of at most two, else
      * all but the last (kv_quant.rs:102-107); such a layer keeps one f32 norm and the packed codebook
-     * indices per position and kv head, 4 + 4 * ceil(head_dim * bits / 32) bytes (kv_quant.rs:141-144).
-     * tsv_compact_tree, and with it tree rounds, are refused on such a handle. */
+     * indices per position and kv head, 4 + 4 * ceil(head_dim * bits / 32) bytes (kv_quant.rs:141-144; the
+     * value side at 3 bits takes 4 + head_dim / 2 bytes here, its indices being kept 16 positions to 64 bits). */
     int32_t kv_k_bits, kv_v_bits;
 } tsv_model_desc;
 

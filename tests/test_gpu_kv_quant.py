@@ -143,8 +143,9 @@ def test_rollback_and_replay_by_bits():
     assert np.array_equal(g.verify(f1[3:], 23), first[3:])
 
 
-@pytest.mark.parametrize("name,kv_bits,layers,bound", [("small_q4_k", (4, 4), 3, 8e-2), ("xcd_q4_k", (4, 4), 3, 8e-2),
-                                                       ("gptoss_small", (4, 4), 4, 8e-2), ("small_q4_k", (3, 4), 3, 1.2e-1)])
+@pytest.mark.parametrize("name,kv_bits,layers,bound", [("small_q4_k", (4, 4), 3, 3e-2), ("xcd_q4_k", (4, 4), 3, 4e-2),
+                                                       ("gptoss_small", (4, 4), 4, 1e-2), ("small_q4_k", (3, 4), 3, 3e-2),
+                                                       ("xcd_q4_k", (2, 2), 3, 1.5e-1), ("tiny_q8_0", (3, 3), 4, 6e-2)])
 def test_logits_against_the_oracle_model_within_the_codecs_own_sensitivity(name, kv_bits, layers, bound):
     """The same forward with the same codec on both sides.  The bound is not fp16 accuracy: indices of coordinates
     near a midpoint differ between any two forwards whose K / V rows differ in the last bit.  What is asserted is
@@ -173,13 +174,52 @@ def test_logits_against_the_oracle_model_within_the_codecs_own_sensitivity(name,
     assert err <= bound and err <= max(3 * self_err, 2e-2) and err < 0.6 * effect
 
 
+@pytest.mark.parametrize("name,kv_bits", [("small_q4_k", (3, 4)), ("xcd_q4_k", (4, 4)), ("tiny_q8_0", (2, 2)), ("small_q4_k", (3, 3))])
+def test_tree_compaction_moves_the_stored_rows_by_bits_and_the_round_goes_on(name, kv_bits):
+    """crates/runtime/src/speculative.rs:518-536: after a tree pass the accepted path's rows become rows
+    base .. base + n - 1.  The stored rows must move unchanged; the continuation is then compared with a handle that
+    fed the path as a chain (its rows come from a narrower pass, so a few indices near midpoints differ)."""
+    import turbospark_amd as ts
+    cfg, w, g = _open(name, kv_bits, n_layers=3)
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, cfg["vocab"], 37).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 16).astype(np.int32)
+    parent = [-1, 0, 0, 0, 0, 1, 5, 6, 2, 8, 9, 3, 11, 12, 4, 14]
+    path = [0, 2, 8, 9]
+    g.prefill(prompt, 0, want_logits=False)
+    point = g.checkpoint()
+    g.verify_tree(feed, parent, 37)
+    before = [g.read_kv_quantized(l, 0, 53) for l in (0, 1)]
+    plain_before = g.read_kv(2, 37, 16)
+    g.compact_tree(37, path)
+    after = [g.read_kv_quantized(l, 0, 53) for l in (0, 1)]
+    plain_after = g.read_kv(2, 37, 4)
+    for (kb, vb), (ka, va) in zip(before, after):
+        assert np.array_equal(ka[:37], kb[:37]) and np.array_equal(va[:37], vb[:37])
+        assert np.array_equal(ka[37:41], kb[37 + np.array(path)]) and np.array_equal(va[37:41], vb[37 + np.array(path)])
+    assert np.array_equal(plain_after[0], plain_before[0][path]) and np.array_equal(plain_after[1], plain_before[1][path])
+    g.rollback_retaining(point, 4)
+    nxt = g.produce(int(feed[10]), 41)
+    ref = ts.HipVerifier(cfg, w, kv_bits=kv_bits)
+    ref.prefill(prompt, 0, want_logits=False)
+    ref.verify(feed[path], 37)
+    want = ref.produce(int(feed[10]), 41)
+    err = gc.logit_error(nxt[None], want[None])
+    same = np.mean([np.mean(a[0][37:41, :, 1:] == r[0][:, :, 1:]) for a, r in zip(after, [ref.read_kv_quantized(l, 37, 4) for l in (0, 1)])])
+    print(f"{name} K{kv_bits[0]}/V{kv_bits[1]}: continuation after compaction vs chain {err:.2e}; K words equal {same:.3f}")
+    assert err <= 3e-2 and same >= 0.8
+
+
 def test_what_a_quantized_handle_refuses():
     import turbospark_amd as ts
     from turbospark_amd import synth
     cfg, w, g = _open("small_q4_k", (4, 4))
     g.verify(np.arange(6, dtype=np.int32), 0)
     with pytest.raises(ts.ffi.TsvError, match="quantized"):
-        g.compact_tree(0, [0, 2, 3])
+        g.read_kv(0, 0, 1)
+    with pytest.raises(ts.ffi.TsvError, match="quantized"):
+        g.write_kv(0, 0, np.zeros((1, cfg["n_kv_heads"], cfg["head_dim"]), np.float16),
+                   np.zeros((1, cfg["n_kv_heads"], cfg["head_dim"]), np.float16))
     for bad in ((4, 3), (1, 1), (5, 5), (2, 4), (0, 4)):
         with pytest.raises(ts.ffi.TsvError, match="widths"):
             ts.HipVerifier(cfg, w, kv_bits=bad)

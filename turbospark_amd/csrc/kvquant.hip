@@ -268,6 +268,44 @@ int launch_tq_prepare(hipStream_t s, const TqArgs& a0) {
     return TSV_OK;
 }
 
+namespace {
+// Tree compaction over quantized rows (crates/runtime/src/speculative.rs:518-536: the accepted path's rows move to
+// consecutive positions): the row at base + path[i] to base + i, in path order.  path is increasing and path[i] >= i,
+// so a destination is never a source still to be read.  One thread owns dimension d of a kv head on the V side (its
+// groups are its own words, no atomics), word d of the K rows, or one of the two norms.
+__global__ void k_tq_gather(const TqKv* __restrict__ stores, int nkv, int hd, int cap, const int32_t* __restrict__ path, int n, int base) {
+    const TqKv t = stores[blockIdx.y];
+    if (!t.k_bits) return;
+    const int id = blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= nkv * hd) return;
+    const int head = id / hd, d = id - head * hd;
+    const int kw = (hd * t.k_bits + 31) / 32, gw = tq_v_group_words(t.v_bits);
+    const uint32_t vmask = (1u << t.v_bits) - 1u;
+    for (int i = 0; i < n; i++) {
+        const int src = base + path[i], dst = base + i;
+        if (src == dst) continue;
+        uint32_t* gs = t.vq + (((long)head * (cap >> 4) + (src >> 4)) * hd + d) * gw;
+        uint32_t* gd = t.vq + (((long)head * (cap >> 4) + (dst >> 4)) * hd + d) * gw;
+        const uint64_t from = gw == 2 ? ((uint64_t)gs[1] << 32) | gs[0] : gs[0];
+        uint64_t to = gw == 2 ? ((uint64_t)gd[1] << 32) | gd[0] : gd[0];
+        const uint32_t so = (uint32_t)(src & 15) * t.v_bits, dof = (uint32_t)(dst & 15) * t.v_bits;
+        to = (to & ~((uint64_t)vmask << dof)) | ((uint64_t)((uint32_t)(from >> so) & vmask) << dof);
+        gd[0] = (uint32_t)to;
+        if (gw == 2) gd[1] = (uint32_t)(to >> 32);
+        if (d < kw) t.kq[((long)head * cap + dst) * kw + d] = t.kq[((long)head * cap + src) * kw + d];
+        if (d == kw) t.kn[(long)head * cap + dst] = t.kn[(long)head * cap + src];
+        if (d == kw + 1) t.vn[(long)head * cap + dst] = t.vn[(long)head * cap + src];
+    }
+}
+}  // namespace
+
+int launch_tq_gather(hipStream_t s, const TqKv* stores_dev, int n_layers, int nkv, int hd, int cap, const int32_t* path_dev, int n,
+                     int base) {
+    hipLaunchKernelGGL(k_tq_gather, dim3((nkv * hd + 255) / 256, n_layers), dim3(256), 0, s, stores_dev, nkv, hd, cap, path_dev, n, base);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
 size_t tq_kq_bytes(int nkv, int cap, int hd, int k_bits) { return (size_t)nkv * cap * tq_words(hd, k_bits) * 4; }
 size_t tq_vq_bytes(int nkv, int cap, int hd, int v_bits) { return (size_t)nkv * (cap / 16) * hd * tq_v_group_words(v_bits) * 4; }
 

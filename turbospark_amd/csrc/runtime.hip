@@ -129,6 +129,7 @@ struct tsv_ctx {
     int kv_k_bits = 0, kv_v_bits = 0;
     TqSide tq_k{}, tq_v{};
     uint16_t *tq_kc = nullptr, *tq_vc = nullptr;
+    TqKv* tq_stores = nullptr;  // device: every layer's stores (tree compaction)
     int64_t position = 0;
     int64_t high_water = 0;     // one past the last position any pass has written since the last reset
     int64_t rewind_budget = INT64_MAX;  // KvCacheManager::max_safe_rewind: min over ring layers of capacity - window
@@ -1247,9 +1248,16 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         if (hipMemcpy(c->kv_ptrs, ptrs.data(), ptrs.size() * sizeof(uint16_t*), hipMemcpyHostToDevice) != hipSuccess)
             return fail(TSV_ERR_DEVICE);
         std::vector<int32_t> caps;
-        for (auto& L : c->layers) caps.push_back(L.cap);
+        for (auto& L : c->layers) caps.push_back(L.kv_slots);  // a quantized layer: its fp16 side is the staging slots
         if ((rc = dev_alloc(c, &c->kv_caps, caps.size() * 4))) return fail(rc);
         if (hipMemcpy(c->kv_caps, caps.data(), caps.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail(TSV_ERR_DEVICE);
+    }
+    if (c->kv_k_bits) {
+        std::vector<TqKv> stores;
+        for (auto& L : c->layers) stores.push_back(L.tq);
+        if ((rc = dev_alloc(c, &c->tq_stores, stores.size() * sizeof(TqKv)))) return fail(rc);
+        if (hipMemcpy(c->tq_stores, stores.data(), stores.size() * sizeof(TqKv), hipMemcpyHostToDevice) != hipSuccess)
+            return fail(TSV_ERR_DEVICE);
     }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
@@ -1642,15 +1650,14 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
         set_error("compact_tree: the block at `base` lies outside the KV cache");
         return TSV_ERR_INVALID;
     }
-    if (c->kv_k_bits) {
-        set_error("compact_tree: tree rounds are not supported over quantized KV rows");
-        return TSV_ERR_UNSUPPORTED;
-    }
     TSV_HIP(hipStreamSynchronize(c->stream));
     if (int frc = check_fused(c)) return frc;  // rows a fused kernel gave up on must not be gathered
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
-    return launch_kv_gather(c->stream, c->kv_ptrs, c->kv_caps, c->n_layers, c->nkv, c->hd, c->tok_dev + 32, n, (int)base);
+    int rc = launch_kv_gather(c->stream, c->kv_ptrs, c->kv_caps, c->n_layers, c->nkv, c->hd, c->tok_dev + 32, n, (int)base);
+    if (!rc && c->kv_k_bits)
+        rc = launch_tq_gather(c->stream, c->tq_stores, c->n_layers, c->nkv, c->hd, c->ctx_alloc, c->tok_dev + 32, n, (int)base);
+    return rc;
 }
 
 namespace {

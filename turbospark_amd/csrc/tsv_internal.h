@@ -388,6 +388,9 @@ int tq_words(int hd, int bits);
 int tq_upload_side(int hd, int bits, uint64_t seed, float* dev, TqSide* out);
 // q rotation and quantization of the pass's rows into the stores
 int launch_tq_prepare(hipStream_t s, const TqArgs& a);
+// rows base + path[i] -> base + i of every quantized layer (stores_dev: one entry per layer, k_bits 0 where rows are fp16)
+int launch_tq_gather(hipStream_t s, const TqKv* stores_dev, int n_layers, int nkv, int hd, int cap, const int32_t* path_dev, int n,
+                     int base);
 // bytes of a layer's four stores for `cap` positions (cap a multiple of 16)
 size_t tq_kq_bytes(int nkv, int cap, int hd, int k_bits);
 size_t tq_vq_bytes(int nkv, int cap, int hd, int v_bits);
