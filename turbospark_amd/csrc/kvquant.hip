@@ -182,8 +182,22 @@ __device__ void commit_row(const TqArgs& a, bool value, int pos, int head, int l
     }
     if (!value && lane < t.words + 1) s_words[lane] = 0;
     lds_order();
+    // every lane adds the squares in index order (the reference's sum); the row comes out of LDS sixteen
+    // values at a time so that the reads run ahead of the dependent additions
     float ss = 0.f;
-    for (int i = 0; i < HD; i++) ss = __fadd_rn(ss, __fmul_rn(s_row[i], s_row[i]));
+#pragma unroll
+    for (int i = 0; i < HD; i += 16) {
+        float4 r[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) r[u] = *(const float4*)(s_row + i + 4 * u);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            ss = __fadd_rn(ss, __fmul_rn(r[u].x, r[u].x));
+            ss = __fadd_rn(ss, __fmul_rn(r[u].y, r[u].y));
+            ss = __fadd_rn(ss, __fmul_rn(r[u].z, r[u].z));
+            ss = __fadd_rn(ss, __fmul_rn(r[u].w, r[u].w));
+        }
+    }
     const float norm = sqrtf(ss);  // correctly rounded, as is the division (the toolchain's default for f32)
     const float inv = 1.0f / fmaxf(norm, 1e-6f);
     float e[EPL];
@@ -191,13 +205,20 @@ __device__ void commit_row(const TqArgs& a, bool value, int pos, int head, int l
     for (int j = 0; j < EPL; j++) e[j] = __fmul_rn(__fmul_rn(x[j], inv), t.signs[lane + 64 * j]);
     wht<EPL>(e, lane, a.inv_sqrt2);
     const int n_mid = (1 << t.bits) - 1;
+    float mid[15];  // the side's midpoints, +inf past the last: the index is the count of midpoints below the coordinate
+#pragma unroll
+    for (int i = 0; i < 15; i++) {
+        const float v = t.mid[i];  // the table holds sixteen slots
+        mid[i] = i < n_mid ? v : INFINITY;
+    }
     if (lane == 0) (value ? a.store.vn : a.store.kn)[(long)head * a.cap + pos] = norm;
     if (!value) {
         // a K row: packed LSB first (kv_quant.rs:289-312), assembled in LDS
 #pragma unroll
         for (int j = 0; j < EPL; j++) {
             uint32_t c = 0;
-            for (int i = 0; i < n_mid; i++) c += e[j] > t.mid[i] ? 1u : 0u;
+#pragma unroll
+            for (int i = 0; i < 15; i++) c += e[j] > mid[i] ? 1u : 0u;
             const uint32_t bit = (uint32_t)(lane + 64 * j) * (uint32_t)t.bits, w = bit >> 5, off = bit & 31;
             atomicOr(&s_words[w], c << off);
             if (off + t.bits > 32) atomicOr(&s_words[w + 1], c >> (32 - off));
@@ -213,7 +234,8 @@ __device__ void commit_row(const TqArgs& a, bool value, int pos, int head, int l
 #pragma unroll
         for (int j = 0; j < EPL; j++) {
             uint32_t c = 0;
-            for (int i = 0; i < n_mid; i++) c += e[j] > t.mid[i] ? 1u : 0u;
+#pragma unroll
+            for (int i = 0; i < 15; i++) c += e[j] > mid[i] ? 1u : 0u;
             const uint64_t bits = (uint64_t)c << off;
             uint32_t* g = a.store.vq + (((long)head * (a.cap >> 4) + (pos >> 4)) * HD + lane + 64 * j) * gw;
             if ((uint32_t)mask) {
@@ -232,7 +254,7 @@ __device__ void commit_row(const TqArgs& a, bool value, int pos, int head, int l
 // One wave per unit of work: the q rows to rotate, then the pass's K and V rows to quantize.
 template <int HD>
 __global__ __launch_bounds__(256) void k_tq_prepare(TqArgs a) {
-    __shared__ float s_row[4][HD];
+    __shared__ __attribute__((aligned(16))) float s_row[4][HD];
     __shared__ uint32_t s_words[4][HD / 2 + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = a.m_hint, base = a.base_hint >= 0 ? a.base_hint : a.vp->base;
