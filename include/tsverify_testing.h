@@ -77,17 +77,20 @@ int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, i
 int32_t tsv_kv_quant_tables(int32_t head_dim, int32_t bits, int32_t value_side, float* signs, float* codebook,
                             float* midpoints);
 
-/* The stored rows of a quantized layer as they lie in memory: n x n_kv_heads x (1 + words) u32 per side,
+/* The stored rows of a quantized layer in the reference's row form: n x n_kv_heads x (1 + words) u32 per side,
  * the f32 norm first, then ceil(head_dim * bits / 32) words of LSB-first codebook indices -- the row
- * crates/gpu/tests/kv_quantize_parity.rs:22-38 reads back. */
+ * crates/gpu/tests/kv_quantize_parity.rs:22-38 reads back.  (In device memory the norms and the indices lie in
+ * separate arrays and the value indices are grouped by dimension, sixteen positions to a group; this call
+ * re-packs them.) */
 int32_t tsv_read_kv_quantized(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint32_t* k_rows, uint32_t* v_rows);
 
 /* One verify-pass attention over quantized rows through the kernels the forward uses (the parity hook
  * of crates/gpu/tests/kv_quantize_parity.rs and attention_tq_parity.rs).  k, v: (base + m) x nkv x hd
- * fp16 staging rows; every one is quantized (the first `base` ahead of the pass, then wiped from the
- * fp16 side so that attention sees them only as decoded), row i of the pass sits at position base + i
- * and sees positions 0 .. base + i.  out: m x nq x hd fp16; k_rows / v_rows: the stored rows of all
- * base + m positions in tsv_read_kv_quantized's layout. */
+ * fp16 staging rows; every one goes through the sixteen staging slots and the quantizer, sixteen rows
+ * at a time as passes do, the last m of them as the pass itself: row i of the pass sits at position
+ * base + i and sees positions 0 .. base + i, all of them as stored.  out: m x nq x hd fp16;
+ * k_rows / v_rows: the stored rows of all base + m positions in tsv_read_kv_quantized's form.
+ * k_bits / v_bits: 2, 3 or 4. */
 int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq, int32_t nkv,
                                 int32_t hd, int64_t base, int32_t k_bits, int32_t v_bits, float scale, const float* sinks,
                                 uint16_t* out, uint32_t* k_rows, uint32_t* v_rows);

@@ -47,7 +47,9 @@ __global__ __launch_bounds__(512) void k_attn_partial_tq(AttnArgs a, int G, int 
     tq_fill_pairs(s_kpair, a.tq.k_cb, KB, threadIdx.x, 512);
     tq_fill_pairs(s_vpair, a.tq.v_cb, VB, threadIdx.x, 512);
     __syncthreads();
-    attn_partial_body_tq<HD, RT, 3, KB, VB>(a, G, R, blockIdx.x, blockIdx.y, blockIdx.z * RT, xch, s_kpair, s_vpair);
+    // blocks in flight: three, two where the three-bit fields' extra words would push the registers past 256
+    constexpr int STAGES = (HD == 128 && RT == 2 && KB == 3 && VB == 3) ? 2 : 3;
+    attn_partial_body_tq<HD, RT, STAGES, KB, VB>(a, G, R, blockIdx.x, blockIdx.y, blockIdx.z * RT, xch, s_kpair, s_vpair);
 }
 
 // Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
