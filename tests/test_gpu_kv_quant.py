@@ -231,3 +231,30 @@ def test_what_a_quantized_handle_refuses():
         lw["window"] = 24
     with pytest.raises(ts.ffi.TsvError, match="nothing to quantize"):
         ts.HipVerifier(oss, wo, kv_bits=(4, 4))
+
+
+def test_a_gguf_target_takes_the_width_from_the_environment(tmp_path):
+    """The option is a session's, not the file's (crates/model-io/src/kv_quant.rs:48-72): TSV_KV_BITS carries it to
+    tsv_open_gguf, and the handle then equals the directly installed one with the same widths, by bits."""
+    import turbospark_amd as ts
+    from tests.gguf_writer import llama_gguf
+    cfg, w, direct = _open("tiny_q8_0", (3, 4), n_layers=3)
+    path = os.path.join(tmp_path, "kv.gguf")
+    llama_gguf(path, cfg, w, arch="llama", permute=True)
+    os.environ["TSV_KV_BITS"] = "3.5"
+    try:
+        filed = ts.HipVerifier.from_gguf(path, max_context=96)
+        os.environ["TSV_KV_BITS"] = "7"
+        with pytest.raises(ts.ffi.TsvError, match="TSV_KV_BITS"):
+            ts.HipVerifier.from_gguf(path, max_context=96)
+    finally:
+        del os.environ["TSV_KV_BITS"]
+    filed.kv_bits = (3, 4)
+    rng = np.random.default_rng(8)
+    prompt = rng.integers(0, cfg["vocab"], 21).astype(np.int32)
+    assert np.array_equal(direct.prefill(prompt, 0), filed.prefill(prompt, 0))
+    feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    assert np.array_equal(direct.verify(feed, 21), filed.verify(feed, 21))
+    for layer in (0, 1):
+        (ka, va), (kb, vb) = direct.read_kv_quantized(layer, 0, 26), filed.read_kv_quantized(layer, 0, 26)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)

@@ -555,5 +555,18 @@ extern "C" int32_t tsv_open_gguf(const char* path, int32_t max_context, tsv_ctx*
             }
     }
     d.layers = layers.data();
+    // --kv-bits is a session option of the reference (crates/model-io/src/kv_quant.rs:48-72), not a property of
+    // the file; here the process environment carries it: TSV_KV_BITS = off | 2 | 3 | 3.5 | 4
+    if (const char* kvb = getenv("TSV_KV_BITS")) {
+        const std::string v(kvb);
+        if (v == "2") d.kv_k_bits = d.kv_v_bits = 2;
+        else if (v == "3") d.kv_k_bits = d.kv_v_bits = 3;
+        else if (v == "3.5") d.kv_k_bits = 3, d.kv_v_bits = 4;
+        else if (v == "4") d.kv_k_bits = d.kv_v_bits = 4;
+        else if (v != "off" && !v.empty()) {
+            set_error("open_gguf: TSV_KV_BITS must be one of off|2|3|3.5|4");
+            return TSV_ERR_INVALID;
+        }
+    }
     return tsv_open(&d, out);
 }
