@@ -20,7 +20,8 @@ extern "C" {
 int32_t tsv_read_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v);
 /* The inverse: stores n rows of K and V (same host layout) at cache positions [pos0, pos0+n) of
  * one layer and moves the cursor to at least pos0 + n -- a long context without the prefill that
- * would build it (the full-size parity cases; also how a saved prefix would be restored). */
+ * would build it (the full-size parity cases; also how a saved prefix would be restored).  On a layer that
+ * keeps quantized rows the rows are quantized on the way in, as the forward's own rows are. */
 int32_t tsv_write_kv(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k, const uint16_t* v);
 /* Stores m x vocab fp16 logits (host memory) as if a verify pass of m rows at `base` had just left them on
  * the device: tsv_accept then judges exactly these scores (acceptance cases no model would produce: ties,

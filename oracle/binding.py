@@ -352,6 +352,17 @@ def tq_dequantize_row(norm, words, signs, codebook, bits, dim):
     return out
 
 
+def tq_roundtrip_rows(rows, bits, seed):
+    """rows [..., dim] -> what a quantized layer holds of them (decode of the stored norm and indices), same shape."""
+    x = np.ascontiguousarray(rows, np.float32)
+    dim = x.shape[-1]
+    signs, cb = tq_sign_vector(dim, seed), tq_codebook(dim, bits)
+    mid = tq_midpoints(cb)
+    out = np.empty_like(x)
+    lib().tso_tq_roundtrip_rows(_p(x), C.c_int64(x.size // dim), dim, _p(signs), _p(cb), _p(mid), bits, _p(out))
+    return out
+
+
 def tq_attention(q, k_words, k_norms, v_words, v_norms, hd, nq, nkv, seq_len, bits, k_signs, k_cb, v_signs, v_cb,
                  scale=0.0, sinks=None, v_bits=None):
     """kv_quant_attention.rs:58-136.  k / v words: [seq_len, nkv, words per row] uint32, norms [seq_len, nkv];

@@ -235,6 +235,17 @@ void tso_tq_dequantize_row(float norm, const uint32_t* words, const float* signs
     for (int i = 0; i < dim; i++) out[i] = out[i] * norm;
 }
 
+// n rows of `dim` values through quantize_row and dequantize_row: what a quantized layer's cache holds of them
+void tso_tq_roundtrip_rows(const float* x, int64_t n, int dim, const float* signs, const float* codebook, const float* midpoints,
+                           int bits, float* out) {
+    std::vector<uint32_t> words((size_t)tso_tq_packed_words(dim, bits) + 1);
+    for (int64_t r = 0; r < n; r++) {
+        float norm;
+        tso_tq_quantize_row(x + r * dim, dim, signs, midpoints, bits, &norm, words.data());
+        tso_tq_dequantize_row(norm, words.data(), signs, codebook, bits, dim, out + r * dim);
+    }
+}
+
 // kv_quant_attention.rs:58-136: one query position over seq_len quantized rows.  q: [nq][hd]; k / v words:
 // [seq_len][nkv][words per row], norms [seq_len][nkv]; scale <= 0: 1 / sqrt(hd); sinks nullable [nq].  The two
 // sides carry their own tables and widths (kv_quant_attention.rs:24-44).

@@ -139,6 +139,8 @@ void tso_tq_quantize_row(const float* x, int dim, const float* signs, const floa
                          uint32_t* words);                                           /* kv_quant.rs:349-362 */
 void tso_tq_dequantize_row(float norm, const uint32_t* words, const float* signs, const float* codebook, int bits, int dim,
                            float* out);                                              /* kv_quant.rs:367-379 */
+void tso_tq_roundtrip_rows(const float* x, int64_t n, int dim, const float* signs, const float* codebook, const float* midpoints,
+                           int bits, float* out);                                    /* dequantize(quantize(row)), n rows */
 void tso_tq_attention(const float* q, const uint32_t* k_words, const float* k_norms, const uint32_t* v_words,
                       const float* v_norms, int hd, int nq, int nkv, int seq_len, float scale, const float* sinks,
                       const float* k_signs, const float* k_codebook, const float* v_signs, const float* v_codebook, int k_bits,

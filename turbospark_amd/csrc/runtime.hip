@@ -1963,10 +1963,6 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
         set_error("write_kv: range outside the cache");
         return TSV_ERR_INVALID;
     }
-    if (c->layers[layer].tq.k_bits) {
-        set_error("write_kv: this layer keeps quantized rows");
-        return TSV_ERR_UNSUPPORTED;
-    }
     const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
     uint16_t *kd = nullptr, *vd = nullptr;
     TSV_HIP(hipMalloc((void**)&kd, bytes));
@@ -1981,7 +1977,30 @@ extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t
         set_error("write_kv: copy failed");
         rc = TSV_ERR_DEVICE;
     }
-    if (!rc) {
+    if (!rc && c->layers[layer].tq.k_bits) {
+        // a quantized layer: the rows go through the staging slots and the quantizer sixteen at a time, as the
+        // forward's own rows do (crates/runtime/src/kv_write.rs:66-118)
+        const LayerW& L = c->layers[layer];
+        TqArgs ta{};
+        ta.kc = L.kc;
+        ta.vc = L.vc;
+        ta.stage_cap = L.kv_slots;
+        ta.store = L.tq;
+        ta.k = c->tq_k;
+        ta.v = c->tq_v;
+        ta.nkv = c->nkv;
+        ta.hd = c->hd;
+        ta.cap = L.cap;
+        ta.vp = c->vp_dev;
+        const size_t row = (size_t)c->nkv * c->hd;
+        for (int64_t p = 0; !rc && p < n; p += L.kv_slots) {
+            const int cnt = (int)std::min<int64_t>(L.kv_slots, n - p);
+            rc = launch_kv_fill(c->stream, L.kc, L.vc, c->nkv, c->hd, L.kv_slots, (int)(pos0 + p), cnt, kd + p * row, vd + p * row);
+            ta.m_hint = cnt;
+            ta.base_hint = (int)(pos0 + p);
+            if (!rc) rc = launch_tq_prepare(c->stream, ta);
+        }
+    } else if (!rc) {
         // a ring layer keeps the last `cap` of the rows (earlier ones would only be overwritten, by
         // rows of the same launch)
         const int64_t cap = c->layers[layer].cap, skip = n > cap ? n - cap : 0;
