@@ -101,6 +101,13 @@ typedef struct {
      * indices per position and kv head, 4 + 4 * ceil(head_dim * bits / 32) bytes (kv_quant.rs:141-144; the
      * value side at 3 bits takes 4 + head_dim / 2 bytes here, its indices being kept 16 positions to 64 bits). */
     int32_t kv_k_bits, kv_v_bits;
+    /* --session-slots (crates/runtime/src/session_pool.rs; RealForwardRunner::open_with_session_slots,
+     * real_forward_api.rs:526-556): how many conversations' KV state the handle keeps, the live one included.
+     * 0 or 1: none parked.  With n > 1, n - 1 further sets of KV buffers are allocated at open; tsv_reset then
+     * parks the live conversation (promoting the least recently used slot) instead of overwriting it, and
+     * tsv_try_reuse_prefix first swaps in the parked conversation that continues the prompt furthest, if it
+     * beats the live one.  A swap exchanges buffer pointers, never rows. */
+    int32_t session_slots;
 } tsv_model_desc;
 
 typedef struct tsv_ctx tsv_ctx;
@@ -177,7 +184,14 @@ int32_t tsv_last_error(char* buf, int32_t cap);
 void* tsv_stream(tsv_ctx* ctx);
 
 /* ---- LogitProducer (producer.rs:17-104) ------------------------------------ */
-int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset */
+int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset (with a session pool: real_forward_traits.rs:12-31) */
+int32_t tsv_session_pool_size(const tsv_ctx* ctx);    /* RealForwardRunner::session_pool_size: parked slots + 1 */
+int32_t tsv_session_slot_evicted(const tsv_ctx* ctx); /* 1: the last tsv_reset overwrote a parked conversation */
+/* The pool's two selection rules on their own (host only; session_pool.rs:116-129): the index of the highest of n
+ * common-prefix scores and that score (-1 and 0 when n == 0 or every score is zero), and the index of the smallest
+ * of n parking ticks (-1 when n == 0). */
+int64_t tsv_session_best_match(const int64_t* scores, int64_t n, int64_t* score_out);
+int64_t tsv_session_lru(const uint64_t* ticks, int64_t n);
 int64_t tsv_kv_position(const tsv_ctx* ctx);   /* kv.position() */
 /* KvCacheManager::max_safe_rewind (crates/gpu/src/kv_cache_rewind.rs:26-35): how many rows a rollback
  * may drop and still leave every ring layer's window intact: the smallest capacity - window over the
@@ -225,7 +239,9 @@ int32_t tsv_set_prefix_reuse(tsv_ctx* ctx, int32_t on);
 /* LogitProducer::try_reuse_prefix (producer.rs:24-47, real_forward_traits.rs:173-289): commits to
  * continuing from the current state for the leading N tokens of the prompt and returns N (0: no
  * reuse, the caller resets; < 0: error).  A cursor that runs past the agreed prefix is moved back
- * to it, within tsv_max_safe_rewind. */
+ * to it, within tsv_max_safe_rewind.  With a session pool the best-matching parked conversation is swapped in
+ * first (select_session, :655-673), and a rewind deeper than the kept prefix on a live session nobody compared
+ * favorably is refused (:283) so that the caller's reset parks that conversation instead of overwriting it. */
 int64_t tsv_try_reuse_prefix(tsv_ctx* ctx, const int32_t* prompt, int64_t n);
 /* SpeculativeProducer::record_committed(tokens, pos0) (producer.rs:322-330): the rows of a verify
  * pass that the round committed, `feed[..committed + 1]` at `base` (speculative.rs:828-836). */

@@ -135,6 +135,21 @@ struct tsv_ctx {
     int64_t rewind_budget = INT64_MAX;  // KvCacheManager::max_safe_rewind: min over ring layers of capacity - window
     int32_t* kv_caps = nullptr;  // device: positions each layer's cache holds (tree compaction)
     tsv_prefix prefix;          // the ids behind rows [0, prefix length): kv_prefix.rs
+    // Parked sessions (crates/runtime/src/session_pool.rs): each one a full set of per-layer KV buffers of its own
+    // with its cursor and its record; the live session is the fields above and in `layers`.  A swap exchanges
+    // pointers, never rows.
+    struct Session {
+        std::vector<uint16_t*> kc, vc;  // per layer (a quantized layer: unused, its rows are in `tq`)
+        std::vector<TqKv> tq;
+        uint16_t** kv_ptrs = nullptr;   // device copies of the pointer tables tree compaction reads
+        TqKv* tq_stores = nullptr;
+        int64_t position = 0, high_water = 0;
+        tsv_prefix prefix;
+        uint64_t last_used = 0;         // the pool's tick at parking (session_pool.rs:110-114)
+    };
+    std::vector<Session> parked;
+    uint64_t session_clock = 0;
+    bool session_slot_evicted = false;  // the last reset overwrote a parked conversation (real_forward_traits.rs:20-31)
     bool prefix_reuse = false;  // RealForwardRunner::set_prefix_reuse: off unless the host opts in
     bool headless = false;      // the pass in flight is a prefill pass nobody reads the logits of
     int last_m = 0;
@@ -1259,6 +1274,50 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         if (hipMemcpy(c->tq_stores, stores.data(), stores.size() * sizeof(TqKv), hipMemcpyHostToDevice) != hipSuccess)
             return fail(TSV_ERR_DEVICE);
     }
+    // --session-slots (crates/runtime/src/real_forward_api.rs:526-556, real_forward_open.rs:674-716): slots - 1 parked
+    // sessions, every one with KV buffers of its own, allocated here and never again
+    if (d->session_slots > 1) {
+        if (c->use_graph) {
+            set_error("open: captured passes (TSV_GRAPH=1) hold the live session's buffers and cannot be used with a session pool");
+            return fail(TSV_ERR_UNSUPPORTED);
+        }
+        if (d->session_slots > 64) {
+            set_error("open: at most 64 session slots");
+            return fail(TSV_ERR_INVALID);
+        }
+        for (int slot = 1; slot < d->session_slots; slot++) {
+            tsv_ctx::Session ses;
+            std::vector<uint16_t*> ptrs;
+            for (auto& L : c->layers) {
+                uint16_t *kc = L.kc, *vc = L.vc;  // a quantized layer: the shared staging slots
+                TqKv tq = L.tq;
+                if (L.tq.k_bits) {
+                    const size_t norms = (size_t)c->nkv * L.cap * 4;
+                    if ((rc = dev_alloc(c, &tq.kq, tq_kq_bytes(c->nkv, L.cap, c->hd, c->kv_k_bits), true)) ||
+                        (rc = dev_alloc(c, &tq.vq, tq_vq_bytes(c->nkv, L.cap, c->hd, c->kv_v_bits), true)) ||
+                        (rc = dev_alloc(c, &tq.kn, norms, true)) || (rc = dev_alloc(c, &tq.vn, norms, true)))
+                        return fail(rc);
+                } else {
+                    const size_t kvb = (size_t)c->nkv * L.cap * c->hd * 2;
+                    if ((rc = dev_alloc(c, &kc, kvb, true)) || (rc = dev_alloc(c, &vc, kvb, true))) return fail(rc);
+                }
+                ses.kc.push_back(kc);
+                ses.vc.push_back(vc);
+                ses.tq.push_back(tq);
+                ptrs.push_back(kc);
+                ptrs.push_back(vc);
+            }
+            if ((rc = dev_alloc(c, &ses.kv_ptrs, ptrs.size() * sizeof(uint16_t*)))) return fail(rc);
+            if (hipMemcpy(ses.kv_ptrs, ptrs.data(), ptrs.size() * sizeof(uint16_t*), hipMemcpyHostToDevice) != hipSuccess)
+                return fail(TSV_ERR_DEVICE);
+            if (c->kv_k_bits) {
+                if ((rc = dev_alloc(c, &ses.tq_stores, ses.tq.size() * sizeof(TqKv)))) return fail(rc);
+                if (hipMemcpy(ses.tq_stores, ses.tq.data(), ses.tq.size() * sizeof(TqKv), hipMemcpyHostToDevice) != hipSuccess)
+                    return fail(TSV_ERR_DEVICE);
+            }
+            c->parked.push_back(std::move(ses));
+        }
+    }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
     if (!d->embed.data || d->embed.rows != c->vocab || d->embed.cols != c->hidden || erb < 0) {
@@ -1459,8 +1518,84 @@ extern "C" int32_t tsv_get_profile(tsv_ctx* c, float* ms, int32_t* counts, int32
 
 extern "C" void* tsv_stream(tsv_ctx* c) { return c ? (void*)c->stream : nullptr; }
 
+// session_pool.rs:116-121 best_scoring_index: the index of the highest score (the last one among equals, as
+// Iterator::max_by_key returns), none when the pool is empty or every score is zero
+extern "C" int64_t tsv_session_best_match(const int64_t* scores, int64_t n, int64_t* score_out) {
+    int64_t best = 0, idx = -1;
+    for (int64_t i = 0; scores && i < n; i++)
+        if (scores[i] > 0 && scores[i] >= best) {
+            best = scores[i];
+            idx = i;
+        }
+    if (score_out) *score_out = idx < 0 ? 0 : best;
+    return idx;
+}
+// session_pool.rs:124-129 lru_index: the index of the smallest tick (the first one among equals, as
+// Iterator::min_by_key returns), -1 on an empty pool
+extern "C" int64_t tsv_session_lru(const uint64_t* ticks, int64_t n) {
+    int64_t idx = -1;
+    for (int64_t i = 0; ticks && i < n; i++)
+        if (idx < 0 || ticks[i] < ticks[idx]) idx = i;
+    return idx;
+}
+
+namespace {
+// real_forward_traits.rs:686-724 swap_live_session: the incoming session's buffers, cursor and record become the
+// live ones; what was live is left in `s` for the caller to park.
+void swap_live_session(tsv_ctx* c, tsv_ctx::Session& s) {
+    for (int l = 0; l < c->n_layers; l++) {
+        LayerW& L = c->layers[l];
+        if (L.tq.k_bits) {
+            std::swap(L.tq, s.tq[l]);
+        } else {
+            std::swap(L.kc, s.kc[l]);
+            std::swap(L.vc, s.vc[l]);
+        }
+    }
+    std::swap(c->kv_ptrs, s.kv_ptrs);
+    std::swap(c->tq_stores, s.tq_stores);
+    std::swap(c->position, s.position);
+    std::swap(c->high_water, s.high_water);
+    std::swap(c->prefix, s.prefix);
+    c->last_m = 0;  // the logits on the device describe the outgoing conversation
+}
+void park_session(tsv_ctx* c, tsv_ctx::Session&& s) {  // session_pool.rs:110-114
+    s.last_used = ++c->session_clock;
+    c->parked.push_back(std::move(s));
+}
+// real_forward_traits.rs:655-673 select_session: the parked session that continues the prompt furthest, if it beats
+// the live one (a tie stays live, an all-zero pool offers nothing: session_pool.rs:78-85,116-121)
+bool select_session(tsv_ctx* c, const int32_t* prompt, int64_t n) {
+    if (c->parked.empty()) return false;
+    const int64_t live = c->prefix.common_prefix(prompt, n);
+    std::vector<int64_t> scores;
+    for (auto& ses : c->parked) scores.push_back(ses.prefix.common_prefix(prompt, n));
+    int64_t best = 0;
+    const int64_t idx = tsv_session_best_match(scores.data(), (int64_t)scores.size(), &best);
+    if (idx < 0 || best <= live) return false;
+    tsv_ctx::Session incoming = std::move(c->parked[idx]);
+    c->parked.erase(c->parked.begin() + (long)idx);
+    swap_live_session(c, incoming);
+    park_session(c, std::move(incoming));
+    return true;
+}
+}  // namespace
+
 extern "C" int32_t tsv_reset(tsv_ctx* c) {
     TSV_NEED(c, "reset: null handle");
+    // real_forward_traits.rs:12-31: with a pool, the live conversation is parked rather than overwritten and the
+    // least recently used parked one takes its place (an eviction if that one held a conversation)
+    c->session_slot_evicted = false;
+    if (!c->parked.empty() && c->position > 0) {
+        std::vector<uint64_t> ticks;
+        for (auto& ses : c->parked) ticks.push_back(ses.last_used);
+        const size_t lru = (size_t)tsv_session_lru(ticks.data(), (int64_t)ticks.size());
+        tsv_ctx::Session promoted = std::move(c->parked[lru]);
+        c->parked.erase(c->parked.begin() + (long)lru);
+        c->session_slot_evicted = promoted.position > 0;
+        swap_live_session(c, promoted);
+        park_session(c, std::move(promoted));
+    }
     c->position = 0;
     c->high_water = 0;
     c->last_m = 0;
@@ -1468,6 +1603,8 @@ extern "C" int32_t tsv_reset(tsv_ctx* c) {
     return TSV_OK;
 }
 
+extern "C" int32_t tsv_session_pool_size(const tsv_ctx* c) { return c ? (int32_t)c->parked.size() + 1 : -1; }
+extern "C" int32_t tsv_session_slot_evicted(const tsv_ctx* c) { return c ? (c->session_slot_evicted ? 1 : 0) : -1; }
 extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c ? c->position : -1; }
 extern "C" int64_t tsv_max_safe_rewind(const tsv_ctx* c) { return c ? c->rewind_budget : -1; }
 extern "C" const uint16_t* tsv_device_logits(tsv_ctx* c) { return c ? c->logits : nullptr; }
@@ -1614,10 +1751,14 @@ extern "C" int64_t tsv_try_reuse_prefix(tsv_ctx* c, const int32_t* prompt, int64
         return -1;
     }
     if (!c->prefix_reuse) return 0;
+    const bool swapped = select_session(c, prompt, n);  // real_forward_traits.rs:184
     const int64_t keep = c->prefix.common_prefix(prompt, n);
     if (keep == 0 || keep > c->position) return 0;
     const int64_t back = c->position - keep;
     if (back > 0) {
+        // real_forward_traits.rs:247-285: with a pool, a shallow match against a live session nobody compared with
+        // anything would overwrite that conversation in place instead of parking it; the caller's reset parks it
+        if (!c->parked.empty() && !swapped && back > keep) return 0;
         if (c->rewind_budget != INT64_MAX && c->high_water - keep > c->rewind_budget) return 0;  // real_forward_traits.rs:241-262: as far as the cache can go back
         c->position = keep;
         c->prefix.rewind_to(keep);

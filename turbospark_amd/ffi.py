@@ -44,7 +44,7 @@ class ModelDesc(C.Structure):
         ("layers", C.POINTER(Layer)),
         ("rope_freqs", C.POINTER(C.c_float)), ("rope_mscale", C.c_float),
         ("act_alpha", C.c_float), ("act_limit", C.c_float),
-        ("kv_k_bits", C.c_int32), ("kv_v_bits", C.c_int32),
+        ("kv_k_bits", C.c_int32), ("kv_v_bits", C.c_int32), ("session_slots", C.c_int32),
     ]
 
 
@@ -249,6 +249,7 @@ EXPORTS = [
     "tsv_gguf_open", "tsv_gguf_close", "tsv_gguf_tensor_count", "tsv_gguf_data_start", "tsv_gguf_tensor",
     "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected", "tsv_force_route",
     "tsv_read_kv_quantized", "tsv_attention_quantized", "tsv_kv_quant_tables",
+    "tsv_session_pool_size", "tsv_session_slot_evicted", "tsv_session_best_match", "tsv_session_lru",
 ]
 
 _lib = None
@@ -265,6 +266,12 @@ def lib():
         L = C.CDLL(LIB_PATH)
         L.tsv_stream.restype = C.c_void_p
         L.tsv_stream.argtypes = [C.c_void_p]
+        L.tsv_session_pool_size.argtypes = [C.c_void_p]
+        L.tsv_session_best_match.restype = C.c_int64
+        L.tsv_session_best_match.argtypes = [C.c_void_p, C.c_int64, C.POINTER(C.c_int64)]
+        L.tsv_session_lru.restype = C.c_int64
+        L.tsv_session_lru.argtypes = [C.c_void_p, C.c_int64]
+        L.tsv_session_slot_evicted.argtypes = [C.c_void_p]
         L.tsv_kv_position.restype = C.c_int64
         L.tsv_kv_position.argtypes = [C.c_void_p]
         L.tsv_max_safe_rewind.restype = C.c_int64

@@ -44,7 +44,7 @@ class HipVerifier:
     crates/model-io/src/kv_quant.rs:102-107 names when kv_bits = (key bits, value bits) is given
     (RealForwardRunner::open_with_kv_quant, crates/runtime/src/real_forward_api.rs:568-590)."""
 
-    def __init__(self, cfg, weights, kv_bits=None):
+    def __init__(self, cfg, weights, kv_bits=None, session_slots=1):
         self.cfg = dict(cfg)
         self._keep = weights
         n = len(weights["layers"])
@@ -76,6 +76,7 @@ class HipVerifier:
         d.act_limit = cfg.get("act_limit", 0.0)
         d.kv_k_bits, d.kv_v_bits = kv_bits if kv_bits else (0, 0)
         self.kv_bits = tuple(kv_bits) if kv_bits else None
+        d.session_slots = int(session_slots)
         d.embed = ffi.tensor(weights["embed"])
         d.final_norm = ffi.tensor(weights["final_norm"])
         d.lm_head = ffi.tensor(weights.get("lm_head"))
@@ -123,6 +124,16 @@ class HipVerifier:
         self.close()
 
     # ---- LogitProducer ----------------------------------------------------------------
+    @property
+    def session_pool_size(self):
+        """Conversations whose KV state the handle keeps, the live one included (RealForwardRunner::session_pool_size)."""
+        return int(ffi.lib().tsv_session_pool_size(self._h))
+
+    @property
+    def session_slot_evicted(self):
+        """Whether the last reset overwrote a parked conversation."""
+        return bool(ffi.lib().tsv_session_slot_evicted(self._h))
+
     def reset(self):
         ffi.check(ffi.lib().tsv_reset(self._h))
 
