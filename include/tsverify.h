@@ -187,6 +187,10 @@ void* tsv_stream(tsv_ctx* ctx);
 int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset (with a session pool: real_forward_traits.rs:12-31) */
 int32_t tsv_session_pool_size(const tsv_ctx* ctx);    /* RealForwardRunner::session_pool_size: parked slots + 1 */
 int32_t tsv_session_slot_evicted(const tsv_ctx* ctx); /* 1: the last tsv_reset overwrote a parked conversation */
+/* 1: the last tsv_try_reuse_prefix swapped a parked conversation in.  A caller that keeps state of its own beside
+ * the handle's (a drafter's context) must not treat such a reuse as a continuation of what it holds
+ * (real_forward_traits.rs:199-239: "nothing rewound, nothing swapped"); tsv_run_speculative starts over then. */
+int32_t tsv_session_swapped(const tsv_ctx* ctx);
 /* The pool's two selection rules on their own (host only; session_pool.rs:116-129): the index of the highest of n
  * common-prefix scores and that score (-1 and 0 when n == 0 or every score is zero), and the index of the smallest
  * of n parking ticks (-1 when n == 0). */

@@ -47,7 +47,7 @@ def test_two_conversations_alternate_without_losing_each_other(name, kv_bits, la
     g.prefill(b, 0, want_logits=False)
     # A comes back: the pool hands its state over and it goes on as if B had never been here
     assert g.try_reuse_prefix(np.concatenate([a, feed_a])) == 40
-    assert g.position == 40 and g.prefix_len() == 40
+    assert g.position == 40 and g.prefix_len() == 40 and ts.ffi.lib().tsv_session_swapped(g._h) == 1
     assert np.array_equal(g.verify(feed_a, 40), _fresh_continuation(cfg, w, a, feed_a, kv_bits))
     g.record_committed(feed_a, 40)
     # and B likewise, from where it stood
@@ -55,7 +55,8 @@ def test_two_conversations_alternate_without_losing_each_other(name, kv_bits, la
     assert np.array_equal(g.verify(feed_b, 33), _fresh_continuation(cfg, w, b, feed_b, kv_bits))
     # A again, now five rows longer
     longer = np.concatenate([a, feed_a, _ids(cfg, 3, 5)])
-    assert g.try_reuse_prefix(longer) == 45 and g.position == 45
+    assert g.try_reuse_prefix(longer) == 45 and g.position == 45 and ts.ffi.lib().tsv_session_swapped(g._h) == 1
+    assert g.try_reuse_prefix(longer) == 45 and ts.ffi.lib().tsv_session_swapped(g._h) == 0   # already live
 
 
 def test_a_full_pool_evicts_the_least_recently_used_conversation():
@@ -154,3 +155,49 @@ def test_what_a_pool_refuses():
             ts.HipVerifier(cfg, w, session_slots=2)
     finally:
         del os.environ["TSV_GRAPH"]
+
+
+def test_the_loop_with_a_pool_keeps_both_conversations_and_generates_what_a_fresh_handle_generates():
+    """speculative.rs:240-251 with real_forward_traits.rs:199-239: the loop's drafter holds context of its own, so a
+    conversation swapped in from the pool is not continued from -- the loop starts over (which parks what was live) --
+    while a plain second turn of the live conversation still is.  Either way the tokens are those of a handle that
+    never saw anything else."""
+    from tests.loop_common import GpuTarget, LmDrafter
+
+    class ContinuingDrafter(LmDrafter):
+        def context_position(self):
+            return self.pos - 1
+
+    cfg, w, g = _open(slots=2, max_context=256)
+    V = cfg["vocab"]
+    lm = ts.HipVerifier(cfg, w)
+    shaping = ts.shaping(0.0)
+    a, b = _ids(cfg, 14, 1), _ids(cfg, 11, 2)
+    da = ContinuingDrafter(GpuTarget(lm), a[0], V, 0.5, 9)
+    one = g.run_speculative(a, da, shaping, 16, 4)
+    held = one["kv_position"]
+    # the same conversation goes on: a pure continuation
+    a2 = np.concatenate([a, np.asarray(one["tokens"][: held - len(a)], np.int32), _ids(cfg, 5, 3)])
+    two = g.run_speculative(a2, da, shaping, 16, 4)
+    assert two["reused"] == held
+    # another conversation: nothing matches, the loop resets, A is parked
+    lm_b = ts.HipVerifier(cfg, w)
+    db = ContinuingDrafter(GpuTarget(lm_b), b[0], V, 0.5, 9)
+    other = g.run_speculative(b, db, shaping, 16, 4)
+    assert other["reused"] == 0 and not g.session_slot_evicted
+    # A's third turn: the pool has its rows, the drafter does not -- the loop starts over
+    a3 = np.concatenate([a2, np.asarray(two["tokens"][: two["kv_position"] - len(a2)], np.int32), _ids(cfg, 4, 5)])
+    da3 = ContinuingDrafter(GpuTarget(lm), a3[0], V, 0.5, 9)
+    three = g.run_speculative(a3, da3, shaping, 16, 4)
+    assert three["reused"] == 0
+    fresh = ts.HipVerifier(cfg, w)
+    fresh.set_prefix_reuse(True)
+    base = fresh.run_speculative(a3, ContinuingDrafter(GpuTarget(ts.HipVerifier(cfg, w)), a3[0], V, 0.5, 9), shaping, 16, 4)
+    for key in ("tokens", "stop_reason", "rounds", "offered", "accepted", "kv_position"):
+        assert three[key] == base[key], key
+    # that start-over re-parked the conversation the pool had just handed out and promoted the other slot: the
+    # cascade the reference describes for installs with a drafter (real_forward_traits.rs:268-281)
+    assert g.session_slot_evicted
+    # the new conversation's own rows explain its transcript: no swap
+    assert g.try_reuse_prefix(np.concatenate([a2, a2[:1]])) == len(a2)
+    assert ts.ffi.lib().tsv_session_swapped(g._h) == 0

@@ -146,7 +146,7 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         keep = std::min<int64_t>(keep, n - 1);
         if (keep > 0) {
             drafter_at = dr->position(dr->user);
-            if (tsv_kv_position(c) != cursor || drafter_at < 0 || keep - drafter_at > 1) keep = 0;
+            if (tsv_kv_position(c) != cursor || tsv_session_swapped(c) || drafter_at < 0 || keep - drafter_at > 1) keep = 0;
         }
         reused = keep;
     }

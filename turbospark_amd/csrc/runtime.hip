@@ -150,6 +150,7 @@ struct tsv_ctx {
     std::vector<Session> parked;
     uint64_t session_clock = 0;
     bool session_slot_evicted = false;  // the last reset overwrote a parked conversation (real_forward_traits.rs:20-31)
+    bool session_swapped = false;       // the last try_reuse_prefix swapped a parked conversation in
     bool prefix_reuse = false;  // RealForwardRunner::set_prefix_reuse: off unless the host opts in
     bool headless = false;      // the pass in flight is a prefill pass nobody reads the logits of
     int last_m = 0;
@@ -1604,6 +1605,7 @@ extern "C" int32_t tsv_reset(tsv_ctx* c) {
 }
 
 extern "C" int32_t tsv_session_pool_size(const tsv_ctx* c) { return c ? (int32_t)c->parked.size() + 1 : -1; }
+extern "C" int32_t tsv_session_swapped(const tsv_ctx* c) { return c ? (c->session_swapped ? 1 : 0) : -1; }
 extern "C" int32_t tsv_session_slot_evicted(const tsv_ctx* c) { return c ? (c->session_slot_evicted ? 1 : 0) : -1; }
 extern "C" int64_t tsv_kv_position(const tsv_ctx* c) { return c ? c->position : -1; }
 extern "C" int64_t tsv_max_safe_rewind(const tsv_ctx* c) { return c ? c->rewind_budget : -1; }
@@ -1750,8 +1752,9 @@ extern "C" int64_t tsv_try_reuse_prefix(tsv_ctx* c, const int32_t* prompt, int64
         set_error("try_reuse_prefix: null handle or prompt");
         return -1;
     }
+    c->session_swapped = false;
     if (!c->prefix_reuse) return 0;
-    const bool swapped = select_session(c, prompt, n);  // real_forward_traits.rs:184
+    const bool swapped = c->session_swapped = select_session(c, prompt, n);  // real_forward_traits.rs:184
     const int64_t keep = c->prefix.common_prefix(prompt, n);
     if (keep == 0 || keep > c->position) return 0;
     const int64_t back = c->position - keep;
