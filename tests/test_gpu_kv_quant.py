@@ -303,3 +303,35 @@ def test_llama3_8b_shape_two_layers_at_4096_context_with_four_bit_rows():
     gpu.rollback(point)
     single = np.concatenate([gpu.verify(feed[i:i + 1], ctx + i) for i in range(5)])
     assert np.array_equal(got, single)
+
+
+def test_graph_replay_over_quantized_rows_equals_plain_launches():
+    """The captured launch sequence reads its positions from device memory at replay; the quantizer and the pass
+    over the stores must do so too: every replay, with rollbacks between them, gives the bits of the plain launches,
+    logits and stored rows."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    os.environ["TSV_FUSED"] = "0"
+    cfg = dict(synth.CONFIGS["small_q4_k"], max_context=160, n_layers=3)
+    w = synth.make_weights(cfg, seed=5)
+    plain = ts.HipVerifier(cfg, w, kv_bits=(4, 4))
+    os.environ["TSV_GRAPH"] = "1"
+    try:
+        graph = ts.HipVerifier(cfg, w, kv_bits=(4, 4))
+    finally:
+        os.environ["TSV_GRAPH"] = "0"
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, cfg["vocab"], 37).astype(np.int32)
+    for eng in (plain, graph):
+        eng.prefill(prompt, 0, want_logits=False)
+    base = 37
+    for rnd, m in enumerate([5, 5, 3, 5, 16, 5, 3]):
+        feed = rng.integers(0, cfg["vocab"], m).astype(np.int32)
+        assert np.array_equal(plain.verify(feed, base), graph.verify(feed, base)), (rnd, m)
+        keep = 1 + rnd % 3
+        for eng in (plain, graph):
+            eng.rollback(ts.ffi.Point(base + keep))
+        base += keep
+    for layer in (0, 1):
+        (ka, va), (kb, vb) = plain.read_kv_quantized(layer, 0, base), graph.read_kv_quantized(layer, 0, base)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
