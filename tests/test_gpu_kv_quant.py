@@ -335,3 +335,53 @@ def test_graph_replay_over_quantized_rows_equals_plain_launches():
     for layer in (0, 1):
         (ka, va), (kb, vb) = plain.read_kv_quantized(layer, 0, base), graph.read_kv_quantized(layer, 0, base)
         assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+
+
+def test_gptoss_120b_shape_with_the_full_layers_rows_quantized():
+    """Hidden 2880, 64 q heads over 8 kv heads of 64 (eight q heads per kv head: the widest group), sinks, YaRN, a
+    windowed layer (fp16 rows) beside a full one (K3/V4 rows), 128 experts top-4; 3000 positions written through the
+    quantizer on both sides; vocabulary cut to 4096 to keep the CPU side short."""
+    import turbospark_amd as ts
+    from oracle import binding as ob
+    from turbospark_amd import synth
+    os.environ["TSV_FUSED"] = "0"
+    ctx, kv_bits = 3000, (3, 4)
+    cfg = dict(synth.CONFIGS["gptoss_120b"], n_layers=2, max_context=ctx + 32, vocab=4096)
+    w = synth.make_weights(cfg, seed=3, n_layers=2)
+    gpu = ts.HipVerifier(cfg, w, kv_bits=kv_bits)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16, kv_bits=kv_bits)
+    assert [cpu.layer_quantized(l) for l in range(2)] == [False, True]
+    rng = np.random.default_rng(3)
+    for layer in range(2):
+        shape = (ctx, cfg["n_kv_heads"], cfg["head_dim"])
+        k = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+        v = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+        gpu.write_kv(layer, 0, k, v)
+        kc, vc = cpu.kv(layer)
+        if layer == 1:
+            kc[:ctx] = ob.tq_roundtrip_rows(k, kv_bits[0], ob.TQ_KEY_SEED)
+            vc[:ctx] = ob.tq_roundtrip_rows(v, kv_bits[1], ob.TQ_VALUE_SEED)
+        else:
+            kc[:ctx] = k.astype(np.float32)
+            vc[:ctx] = v.astype(np.float32)
+    cpu.rewind_to(ctx)
+    for attempt in range(40):
+        feed = np.random.default_rng(20 + attempt).integers(0, cfg["vocab"], 9).astype(np.int32)
+        cpu.rewind_to(ctx)
+        want = cpu.verify(feed, ctx)
+        if cpu.route_margin > 1e-3:
+            break
+    else:
+        raise AssertionError("no feed without a near-tie routing decision")
+    point = gpu.checkpoint()
+    got = gpu.verify(feed, ctx)
+    err = gc.logit_error(got, want)
+    print(f"gpt-oss-120B shape, 2 layers, ctx {ctx}, m=9, K3/V4 rows on the full layer: max-abs logit error / range = {err:.2e}")
+    assert err <= 3e-2
+    gpu.rollback(point)
+    # with eight q heads per kv head a nine-row pass splits the context into other attention chunks than a one-row
+    # pass does (fp16 rows or not), so the two agree to rounding here, not by bits
+    single = np.concatenate([gpu.verify(feed[i:i + 1], ctx + i) for i in range(9)])
+    gap = gc.logit_error(single, got)
+    print(f"  the same nine rows one at a time: {gap:.2e}")
+    assert gap <= 2e-2

@@ -13,10 +13,13 @@ from turbospark_amd import synth
 pytestmark = pytest.mark.gpu
 
 
-def _open(name="tiny_q8_0", slots=2, kv_bits=None, max_context=160, **over):
+def _open(name="tiny_q8_0", slots=2, kv_bits=None, max_context=160, ring=False, **over):
     os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS[name], max_context=max_context, **over)
     w = synth.make_weights(cfg, seed=77)
+    if ring:   # the windowed layers keep rings (and the handle a finite rewind budget): they are swapped like the rest
+        for lw in w["layers"]:
+            lw["ring"] = 1 if lw.get("window", 0) else 0
     g = ts.HipVerifier(cfg, w, kv_bits=kv_bits, session_slots=slots)
     g.set_prefix_reuse(True)
     return cfg, w, g
@@ -32,9 +35,10 @@ def _fresh_continuation(cfg, w, prompt, feed, kv_bits=None):
     return ref.verify(feed, len(prompt))
 
 
-@pytest.mark.parametrize("name,kv_bits,layers", [("tiny_q8_0", None, 2), ("small_q4_k", (3, 4), 3), ("gptoss_small", None, 2)])
-def test_two_conversations_alternate_without_losing_each_other(name, kv_bits, layers):
-    cfg, w, g = _open(name, 2, kv_bits, n_layers=layers)
+@pytest.mark.parametrize("name,kv_bits,layers,ring", [("tiny_q8_0", None, 2, False), ("small_q4_k", (3, 4), 3, False),
+                                                      ("gptoss_small", None, 2, False), ("gptoss_small", None, 2, True)])
+def test_two_conversations_alternate_without_losing_each_other(name, kv_bits, layers, ring):
+    cfg, w, g = _open(name, 2, kv_bits, ring=ring, n_layers=layers)
     assert g.session_pool_size == 2
     a, b = _ids(cfg, 40, 1), _ids(cfg, 33, 2)
     feed_a, feed_b = _ids(cfg, 5, 3), _ids(cfg, 4, 4)
