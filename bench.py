@@ -127,6 +127,9 @@ PROBES = {
                       **dict(GATE_UP_8B, m=64)),
     "attention": dict(match="k_attn_partial", what="attention partial pass, 32 q / 8 kv heads x 128, M = 5, 4096-token context",
                       **ATTN_8B),
+    # the same pass over TurboQuant rows, four bits for keys and values: norms and packed indices instead of fp16 rows
+    "attention_tq": dict(match="k_attn_partial_tq", what="attention partial pass over 4-bit KV rows, 32 q / 8 kv heads x 128, "
+                                                         "M = 5, 4096-token context", kv_bits=4, **ATTN_8B),
 }
 
 
@@ -134,6 +137,8 @@ def probe_bytes(pr):
     from turbospark_amd import ffi
     if "rows" in pr:
         return pr["rows"] * ffi.row_bytes(pr["dtype"], pr["cols"])
+    if "kv_bits" in pr:   # per position and kv head and side: an f32 norm and head_dim * bits / 8 bytes of indices
+        return (pr["base"] + pr["m"]) * pr["nkv"] * 2 * (4 + pr["hd"] * pr["kv_bits"] // 8)
     return (pr["base"] + pr["m"]) * pr["nkv"] * pr["hd"] * 2 * 2    # K and V rows [0, base + m), fp16, read once
 
 
@@ -155,7 +160,10 @@ def traffic_probe(which):
         q = rng.standard_normal((pr["m"], pr["nq"], pr["hd"]), np.float32)
         k = rng.standard_normal((pr["base"] + pr["m"], pr["nkv"], pr["hd"]), np.float32)
         v = rng.standard_normal((pr["base"] + pr["m"], pr["nkv"], pr["hd"]), np.float32)
-        out = ffi.attention(q, k, v, pr["base"])
+        if "kv_bits" in pr:
+            out = ffi.attention_quantized(q, k, v, pr["base"], pr["kv_bits"], pr["kv_bits"])[0]
+        else:
+            out = ffi.attention(q, k, v, pr["base"])
         assert np.isfinite(out).all()
     log(f"[traffic-probe] {pr['what']}: 8 launches, {probe_bytes(pr)} algorithmic bytes each")
 
