@@ -87,7 +87,7 @@ int32_t tsv_read_kv_quantized(tsv_ctx* ctx, int32_t layer, int64_t pos0, int64_t
 
 /* One verify-pass attention over quantized rows through the kernels the forward uses (the parity hook
  * of crates/gpu/tests/kv_quantize_parity.rs and attention_tq_parity.rs).  k, v: (base + m) x nkv x hd
- * fp16 staging rows; every one goes through the sixteen staging slots and the quantizer, sixteen rows
+ * fp16 staging rows; every one goes through staging slots and the quantizer, sixteen rows
  * at a time as passes do, the last m of them as the pass itself: row i of the pass sits at position
  * base + i and sees positions 0 .. base + i, all of them as stored.  out: m x nq x hd fp16;
  * k_rows / v_rows: the stored rows of all base + m positions in tsv_read_kv_quantized's form.

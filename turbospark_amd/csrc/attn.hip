@@ -49,7 +49,14 @@ __global__ __launch_bounds__(512) void k_attn_partial_tq(AttnArgs a, int G, int 
     __syncthreads();
     // blocks in flight: three, two where the three-bit fields' extra words would push the registers past 256
     constexpr int STAGES = (HD == 128 && RT == 2 && KB == 3 && VB == 3) ? 2 : 3;
-    attn_partial_body_tq<HD, RT, STAGES, KB, VB>(a, G, R, blockIdx.x, blockIdx.y, blockIdx.z * RT, xch, s_kpair, s_vpair);
+    // grid z: row groups of the pass, times the 16-row blocks of a prompt pass
+    const int groups = gridDim.z / max(a.blocks, 1), blk = blockIdx.z / groups, grp = blockIdx.z - blk * groups;
+    if (a.blocks > 1) {
+        const AttnArgs v = attn_block_view(a, blk);
+        attn_partial_body_tq<HD, RT, STAGES, KB, VB>(v, G, R, blockIdx.x, blockIdx.y, grp * RT, xch, s_kpair, s_vpair);
+        return;
+    }
+    attn_partial_body_tq<HD, RT, STAGES, KB, VB>(a, G, R, blockIdx.x, blockIdx.y, grp * RT, xch, s_kpair, s_vpair);
 }
 
 // Merge the chunk partials (crates/gpu/src/shaders/attention.metal:122-140 semantics:
@@ -158,7 +165,7 @@ static int launch_partial_tq(hipStream_t s, const AttnArgs& a, int G, int R, int
                                     (int)lds));
         raised = true;
     }
-    hipLaunchKernelGGL((k_attn_partial_tq<HD, RT, KB, VB>), dim3(a.nch, a.nkv, groups), dim3(512), lds, s, a, G, R);
+    hipLaunchKernelGGL((k_attn_partial_tq<HD, RT, KB, VB>), dim3(a.nch, a.nkv, groups * std::max(a.blocks, 1)), dim3(512), lds, s, a, G, R);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -184,8 +191,8 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 256 / (a0.nkv * groups * std::max(a0.blocks, 1))));
     int rc;
     if (a.tq.k_bits) {
-        if (a.window || a.ring || a.blocks > 1 || !a.unrot) {
-            set_error("attention: quantized rows go with full attention, a linear cache and single passes");
+        if (a.window || a.ring || !a.unrot) {
+            set_error("attention: quantized rows go with full attention and a linear cache");
             return TSV_ERR_UNSUPPORTED;
         }
         rc = trt <= 1 ? launch_partial_tq_widths<HD, 1>(s, a, G, R, 1) : launch_partial_tq_widths<HD, 2>(s, a, G, R, groups);

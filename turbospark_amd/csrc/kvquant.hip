@@ -8,7 +8,7 @@
 // the sum is rotated back once with the value signs.  The attention kernel reads the stores directly
 // (attn_tq_core.h, which also states their layout); the merge kernel rotates the result back.
 //
-// The pass's own rows arrive as fp16 in a sixteen-slot staging cache (the staging row of
+// The pass's own rows arrive as fp16 in a small staging cache (the staging row of
 // crates/runtime/src/kv_write.rs:66-118) and are quantized from there: norm as the f32 sum of squares
 // in index order, unit = x * (1 / max(norm, 1e-6)), the butterflies of crates/compute/src/wht.rs:15-29
 // in their order with each stage scaled by 1/sqrt(2), one index per coordinate as the count of

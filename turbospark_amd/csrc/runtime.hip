@@ -33,7 +33,7 @@ struct LayerW {
     int cap = 0;        // positions the layer's cache holds: the context, or a ring of window + slack
     bool rope_fused = false;  // the q/k/v projection rotates and stores its own rows
     uint16_t *kc = nullptr, *vc = nullptr;
-    // a quantized layer (TurboQuant): kc / vc are then the sixteen-slot fp16 staging cache all such layers
+    // a quantized layer (TurboQuant): kc / vc are then the small fp16 staging cache all such layers
     // share (kv_slots positions instead of cap), and tq the layer's own stores
     int kv_slots = 0;
     TqKv tq{};
@@ -912,14 +912,34 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         re.nq = c->nq;
         re.nkv = c->nkv;
         re.hd = c->hd;
-        re.max_ctx = L.cap;
+        re.max_ctx = L.kv_slots;
         if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
+        if (L.tq.k_bits) {  // all 64 rows are quantized (and their q rows rotated) before any block attends
+            TqArgs ta{};
+            ta.q16 = w.q16;
+            ta.kc = L.kc;
+            ta.vc = L.vc;
+            ta.stage_cap = L.kv_slots;
+            ta.store = L.tq;
+            ta.k = c->tq_k;
+            ta.v = c->tq_v;
+            ta.nq = c->nq;
+            ta.nkv = c->nkv;
+            ta.hd = c->hd;
+            ta.cap = L.cap;
+            ta.vp = w.vp;
+            ta.m_hint = 16 * WIDE_B;
+            ta.base_hint = (int)base;
+            if ((rc = launch_tq_prepare(s, ta))) return rc;
+        }
         {
             // all four blocks in one launch: block b attends with its own base position base + 16 b
             AttnArgs aa{};
             aa.q16 = w.q16;
             aa.kc = L.kc;
             aa.vc = L.vc;
+            aa.unrot = L.tq.k_bits ? c->tq_v.signs : nullptr;
+            aa.tq = L.tq;
             aa.part_o = w.part_o;
             aa.part_ml = w.part_ml;
             aa.xfrag = (uint4*)w.xf_b;
@@ -1234,7 +1254,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         // every one but the last; windowed layers keep fp16 rows
         L.kv_slots = L.cap;
         if (c->kv_k_bits && s.window == 0 && (c->n_layers <= 2 || l + 1 < c->n_layers)) {
-            L.kv_slots = TSV_MAX_ROWS;
+            L.kv_slots = 4 * TSV_MAX_ROWS;  // a prompt pass of four 16-row blocks stages all of its rows
             const size_t stage = (size_t)c->nkv * L.kv_slots * c->hd * 2;
             if (!c->tq_kc && ((rc = dev_alloc(c, &c->tq_kc, stage, true)) || (rc = dev_alloc(c, &c->tq_vc, stage, true)))) return fail(rc);
             L.kc = c->tq_kc;
@@ -1445,7 +1465,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         return fail(TSV_ERR_DEVICE);
     }
     // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
-    c->wide.ok = c->rewind_budget == INT64_MAX && !c->fused_ffn && !c->fused_attn && !c->kv_k_bits;
+    c->wide.ok = c->rewind_budget == INT64_MAX && !c->fused_ffn && !c->fused_attn;
     for (const LayerW& L : c->layers)
         if (L.n_experts || !L.rope_fused || L.v_only.tiles || L.qkv.fmt != FMT_Q4K || L.wo.fmt != FMT_Q4K ||
             L.gate_up.fmt != FMT_Q4K || L.down.fmt != FMT_Q4K)
