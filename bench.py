@@ -19,18 +19,18 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 WORKLOADS = {
-    # BASELINE configs[1]
+    # the headline configuration: 8B-shaped Q4_K target, chain k = 4, 4096-token context, T = 0.8
     "llama3_8b_q4_k_k4_ctx4096": dict(model="llama3_8b_q4_k", ctx=4096, k=4, temperature=0.8),
-    # BASELINE configs[0] (the reference's CPU-runnable plumbing case), greedy
+    # the reference's CPU-runnable plumbing case, greedy
     "tiny_q8_0_k4_ctx256": dict(model="tiny_q8_0", ctx=256, k=4, temperature=0.0),
     "small_q4_k_k4_ctx256": dict(model="small_q4_k", ctx=256, k=4, temperature=0.8),
-    # BASELINE configs[3]: routed experts (MXFP4) + Q8_0 attention, chain k=8, greedy
+    # configuration 4: routed experts (MXFP4) + Q8_0 attention, chain k=8, greedy
     "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(model="qwen3_30b_a3b", ctx=8192, k=8, temperature=0.0),
     "moe_small_k8_ctx256": dict(model="moe_small", ctx=256, k=8, temperature=0.0),
-    # BASELINE configs[4]: gpt-oss arrangement (bf16 + MXFP4 experts top-4, window / full layers), T = 1.0
+    # configuration 5: gpt-oss arrangement (bf16 + MXFP4 experts top-4, window / full layers), T = 1.0
     "gptoss_120b_mxfp4_k8_ctx32768": dict(model="gptoss_120b", ctx=32768, k=8, temperature=1.0),
     "gptoss_small_k8_ctx256": dict(model="gptoss_small", ctx=256, k=8, temperature=1.0),
-    # BASELINE configs[2]: the 16-node tree (root, four children, chains below them), 16 384-token
+    # configuration 3: the 16-node tree (root, four children, chains below them), 16 384-token
     # context, multi-branch rejection at T = 1.0
     "llama3_8b_q4_k_tree16_ctx16384": dict(model="llama3_8b_q4_k", ctx=16384, k=15, temperature=1.0, tree=True),
     "small_q4_k_tree16_ctx256": dict(model="small_q4_k", ctx=256, k=15, temperature=1.0, tree=True),

@@ -4,7 +4,7 @@ import numpy as np
 
 from . import ffi
 
-# BASELINE configurations of the verify path (dense ones).
+# The benchmark configurations of the verify path (dense ones).
 CONFIGS = {
     # tiny Llama-style decoder, the reference's CPU-runnable plumbing case
     "tiny_q8_0": dict(n_layers=2, hidden=512, n_q_heads=8, n_kv_heads=8, head_dim=64, ffn=1408,
