@@ -68,7 +68,7 @@ __global__ __launch_bounds__(512) void k_attn_partial_tq(AttnArgs a, int G, int 
 // NCH > 0: the chunk count as a compile-time constant -- every thread then asks for its output
 // element of all chunks before the (m, l) pairs are looked at (the two groups of loads do not
 // depend on each other), and the kernel is one memory latency instead of two.  NCH == 0: any count.
-template <int NCH>
+template <int NCH, bool UNROT>
 __global__ void k_attn_combine(AttnArgs a0, int G, int R) {
     const AttnArgs a = a0.blocks > 1 ? attn_block_view(a0, blockIdx.z) : a0;
     __shared__ float wgt[64];
@@ -114,7 +114,7 @@ __global__ void k_attn_combine(AttnArgs a0, int G, int R) {
         for (int c = 0; c < nch; c++) num = fmaf(wgt[c], po[c * stride], num);
     }
     float res = num / s_den;
-    if (a.unrot) {
+    if (UNROT) {
         // the sum was taken over rotated value rows: back through the normalized Hadamard transform
         // (crates/compute/src/wht.rs:15-29, stage h pairs d with d + h) and the value signs
         __shared__ float s_h[128];
@@ -209,15 +209,26 @@ static int launch_combine(hipStream_t s, const AttnArgs& a, int m, int G, int R)
     const dim3 cgrid(m, a.nq, std::max(a.blocks, 1)), cblock(HD < 64 ? 64 : HD);
     // the chunk count as a compile-time constant puts every partial's load in flight before the
     // first add (a counted loop waits on each in turn); the sum runs in the same order either way
-#define TSV_COMBINE(N) \
-    case N: hipLaunchKernelGGL(k_attn_combine<N>, cgrid, cblock, 0, s, a, G, R); break;
+    // UNROT: the variant that rotates each head's result back (quantized KV rows); the other one is unchanged code
+#define TSV_COMBINE(N)                                                                         \
+    case N:                                                                                    \
+        if (a.unrot)                                                                           \
+            hipLaunchKernelGGL((k_attn_combine<N, true>), cgrid, cblock, 0, s, a, G, R);       \
+        else                                                                                   \
+            hipLaunchKernelGGL((k_attn_combine<N, false>), cgrid, cblock, 0, s, a, G, R);      \
+        break;
     switch (a.nch) {
         TSV_COMBINE(1) TSV_COMBINE(2) TSV_COMBINE(3) TSV_COMBINE(4) TSV_COMBINE(5) TSV_COMBINE(6) TSV_COMBINE(7) TSV_COMBINE(8)
         TSV_COMBINE(9) TSV_COMBINE(10) TSV_COMBINE(11) TSV_COMBINE(12) TSV_COMBINE(13) TSV_COMBINE(14) TSV_COMBINE(15)
         TSV_COMBINE(16) TSV_COMBINE(17) TSV_COMBINE(18) TSV_COMBINE(19) TSV_COMBINE(20) TSV_COMBINE(21) TSV_COMBINE(22)
         TSV_COMBINE(23) TSV_COMBINE(24) TSV_COMBINE(25) TSV_COMBINE(26) TSV_COMBINE(27) TSV_COMBINE(28) TSV_COMBINE(29)
         TSV_COMBINE(30) TSV_COMBINE(31) TSV_COMBINE(32)
-        default: hipLaunchKernelGGL(k_attn_combine<0>, cgrid, cblock, 0, s, a, G, R); break;
+        default:
+            if (a.unrot)
+                hipLaunchKernelGGL((k_attn_combine<0, true>), cgrid, cblock, 0, s, a, G, R);
+            else
+                hipLaunchKernelGGL((k_attn_combine<0, false>), cgrid, cblock, 0, s, a, G, R);
+            break;
     }
 #undef TSV_COMBINE
     TSV_HIP(hipGetLastError());

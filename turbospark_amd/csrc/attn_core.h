@@ -84,31 +84,31 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
     // query fragments and per-row ancestor sets
     uint4 qf[RT][KS];
     uint32_t anc[RT];
-    int lo[RT];  // first visible position of the row (window)
+    int lo[RT];  // the row's position: with a window it sees positions lo + 1 - window .. lo
 #pragma unroll
+    // Lanes past the last (row, q head) pair work on pair 0 (a column of the MFMAs of their own, never stored):
+    // loads under a divergent branch would be waited for, all of them, where the branches join -- a memory round
+    // trip per row tile before the first K / V load is even issued.
     for (int t = 0; t < RT; t++) {
         const int r = (rt0 + t) * 16 + j;
-        anc[t] = 0xFFFFu;
-        lo[t] = 0;
-        if (r < R) {
-            const int mrow = r / G, g = r - mrow * G;
-            anc[t] = vp->anc[mrow];
-            if (window > 0) lo[t] = vp->pos[mrow] + 1 - window;
-            const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
-            if (COH) {
-                const __amdgpu_buffer_rsrc_t qrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.q16, 0, 0x7FFFFFFF, 0x00027000);
-                const uint32_t qo = (uint32_t)((const char*)q - (const char*)a.q16);
+        const int rr = r < R ? r : 0;
+        const int mrow = rr / G, g = rr - mrow * G;
+        const uint32_t anc_row = vp->anc[mrow];
+        const int pos_row = vp->pos[mrow];
+        const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
+        if (COH) {
+            const __amdgpu_buffer_rsrc_t qrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.q16, 0, 0x7FFFFFFF, 0x00027000);
+            const uint32_t qo = (uint32_t)((const char*)q - (const char*)a.q16);
 #pragma unroll
-                for (int s = 0; s < KS; s++)
-                    qf[t][s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qrs, qo + 64 * s, 0, 16));
-            } else {
-#pragma unroll
-                for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
-            }
+            for (int s = 0; s < KS; s++)
+                qf[t][s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qrs, qo + 64 * s, 0, 16));
         } else {
 #pragma unroll
-            for (int s = 0; s < KS; s++) qf[t][s] = make_uint4(0, 0, 0, 0);
+            for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
         }
+        // taken as loaded (for a lane past the end: pair 0's), and not touched before the first K / V loads are out
+        anc[t] = anc_row;
+        lo[t] = pos_row;
     }
 
     float mrun[RT], lrun[RT];
@@ -165,7 +165,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
                 vis4 = (uint32_t)(w >> (p0 + 4 * kg - base + 16)) & 0xFu;  // shift in [1, 47]
             }
             if (p0 < cut_end) {  // some row's window starts inside or after this block
-                const int d = lo[t] - (p0 + 4 * kg);  // this lane's positions below index d are outside
+                const int d = lo[t] + 1 - window - (p0 + 4 * kg);  // this lane's positions below index d are outside
                 vis4 &= d <= 0 ? 0xFu : d >= 4 ? 0u : (0xFu << d) & 0xFu;
             }
             float sc[4];

@@ -62,19 +62,17 @@ __device__ __forceinline__ void attn_partial_body_tq(const AttnArgs& a, int G, i
     uint4 qf[RT][KS];
     uint32_t anc[RT];
 #pragma unroll
+    // lanes past the last (row, q head) pair work on pair 0 (their column is never stored): no loads under a
+    // divergent branch
     for (int t = 0; t < RT; t++) {
         const int r = (rt0 + t) * 16 + j;
-        anc[t] = 0xFFFFu;
-        if (r < R) {
-            const int mrow = r / G, g = r - mrow * G;
-            anc[t] = vp->anc[mrow];
-            const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
+        const int rr = r < R ? r : 0;
+        const int mrow = rr / G, g = rr - mrow * G;
+        const uint32_t anc_row = vp->anc[mrow];
+        const _Float16* q = (const _Float16*)a.q16 + ((long)mrow * a.nq + h * G + g) * HD + 8 * kg;
 #pragma unroll
-            for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
-        } else {
-#pragma unroll
-            for (int s = 0; s < KS; s++) qf[t][s] = make_uint4(0, 0, 0, 0);
-        }
+        for (int s = 0; s < KS; s++) qf[t][s] = *(const uint4*)(q + 32 * s);
+        anc[t] = anc_row;
     }
 
     float mrun[RT], lrun[RT];
