@@ -185,6 +185,13 @@ void* tsv_stream(tsv_ctx* ctx);
 
 /* ---- LogitProducer (producer.rs:17-104) ------------------------------------ */
 int32_t tsv_reset(tsv_ctx* ctx);               /* LogitProducer::reset (with a session pool: real_forward_traits.rs:12-31) */
+/* What KV rows cost, on the host and without a handle (crates/model-io/src/kv_quant.rs:146-205 kv_layer_strides;
+ * context_policy.rs:294-333 kv_bytes_for_context_with): bytes one position costs in one layer, K side and V side
+ * -- fp16 rows, or a norm and packed indices per kv head on the layers kv_k_bits / kv_v_bits quantize -- and the
+ * bytes one conversation's KV state takes at `context` positions (a ring layer stops growing at its capacity;
+ * a session pool multiplies it by session_slots).  -1 / an error code on a bad description. */
+int32_t tsv_kv_row_bytes(const tsv_model_desc* desc, int32_t layer, int64_t* k_bytes, int64_t* v_bytes);
+int64_t tsv_kv_bytes_for_context(const tsv_model_desc* desc, int64_t context);
 int32_t tsv_session_pool_size(const tsv_ctx* ctx);    /* RealForwardRunner::session_pool_size: parked slots + 1 */
 int32_t tsv_session_slot_evicted(const tsv_ctx* ctx); /* 1: the last tsv_reset overwrote a parked conversation */
 /* 1: the last tsv_try_reuse_prefix swapped a parked conversation in.  A caller that keeps state of its own beside

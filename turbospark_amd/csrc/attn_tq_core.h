@@ -25,7 +25,6 @@ template <int B>
 struct TqWidth {
     static constexpr int PAIR_BITS = 2 * B, PAIR_MASK = (1 << (2 * B)) - 1;
 };
-__host__ __device__ constexpr int tq_v_group_words(int vb) { return vb == 2 ? 1 : 2; }
 
 // two adjacent indices -> two fp16 levels, from a table in LDS
 __device__ __forceinline__ void tq_fill_pairs(uint32_t* table, const float* cb, int bits, int tid, int nthreads) {

@@ -2318,6 +2318,45 @@ extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uin
     return rc;
 }
 
+// crates/model-io/src/kv_quant.rs:146-205 kv_layer_strides, for the layer kinds of this path and as this library
+// lays the rows out: bytes one position costs in layer `layer`, K side and V side
+extern "C" int32_t tsv_kv_row_bytes(const tsv_model_desc* d, int32_t layer, int64_t* k_bytes, int64_t* v_bytes) {
+    if (!d || !d->layers || layer < 0 || layer >= d->n_layers || !k_bytes || !v_bytes || d->n_kv_heads < 1 || d->head_dim < 1) {
+        set_error("kv_row_bytes: null argument or layer outside the model");
+        return TSV_ERR_INVALID;
+    }
+    const bool quantized = d->kv_k_bits > 0 && d->layers[layer].window == 0 && (d->n_layers <= 2 || layer + 1 < d->n_layers);
+    if (!quantized) {
+        *k_bytes = *v_bytes = (int64_t)d->n_kv_heads * d->head_dim * 2;
+        return TSV_OK;
+    }
+    // one f32 norm and the packed indices per kv head (kv_quant.rs:141-144); the V indices are kept sixteen positions to
+    // a group of 32 or 64 bits per dimension, which at three bits is a third more than the packed row
+    *k_bytes = (int64_t)d->n_kv_heads * (4 + 4 * tq_words(d->head_dim, d->kv_k_bits));
+    *v_bytes = (int64_t)d->n_kv_heads * (4 + (int64_t)d->head_dim * tq_v_group_words(d->kv_v_bits) * 4 / 16);
+    return TSV_OK;
+}
+
+// crates/model-io/src/context_policy.rs:294-333 kv_bytes_for_context_with: what one conversation's KV state costs at
+// `context` positions (rounded up to whole blocks of sixteen, as allocated): a ring layer stops growing at its capacity
+extern "C" int64_t tsv_kv_bytes_for_context(const tsv_model_desc* d, int64_t context) {
+    if (!d || !d->layers || context < 1) {
+        set_error("kv_bytes_for_context: null description or empty context");
+        return -1;
+    }
+    const int64_t alloc = (context + 15) / 16 * 16;
+    int64_t total = 0;
+    for (int l = 0; l < d->n_layers; l++) {
+        int64_t k, v;
+        if (tsv_kv_row_bytes(d, l, &k, &v)) return -1;
+        int64_t cap = alloc;
+        if (d->layers[l].ring && d->layers[l].window > 0)
+            cap = std::min<int64_t>(alloc, (int64_t)((d->layers[l].window + 15) / 16) * 16 + 2 * TSV_MAX_ROWS);
+        total += cap * (k + v);
+    }
+    return total;
+}
+
 extern "C" int32_t tsv_kv_quant_tables(int32_t head_dim, int32_t bits, int32_t value_side, float* signs, float* codebook,
                                        float* midpoints) {
     if (head_dim < 32 || head_dim > 512 || (head_dim & (head_dim - 1)) || bits < 1 || bits > 4 || !signs || !codebook ||

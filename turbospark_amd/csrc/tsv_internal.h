@@ -382,6 +382,8 @@ struct TqArgs {
     int m_hint, base_hint;  // rows of the pass; position of its first row (< 0: read vp->base)
     float inv_sqrt2;        // set by the launcher
 };
+// words of a V group: the sixteen positions' indices of one dimension, 32 bits at two bits per index, else 64
+__host__ __device__ constexpr int tq_v_group_words(int vb) { return vb == 2 ? 1 : 2; }
 void tq_sign_vector(int dim, uint64_t seed, float* out);
 std::vector<float> tq_codebook(int dim, int bits);
 int tq_words(int hd, int bits);

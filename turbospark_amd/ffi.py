@@ -250,6 +250,7 @@ EXPORTS = [
     "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected", "tsv_force_route",
     "tsv_read_kv_quantized", "tsv_attention_quantized", "tsv_kv_quant_tables",
     "tsv_session_pool_size", "tsv_session_slot_evicted", "tsv_session_best_match", "tsv_session_lru", "tsv_session_swapped",
+    "tsv_kv_row_bytes", "tsv_kv_bytes_for_context",
 ]
 
 _lib = None
@@ -267,6 +268,9 @@ def lib():
         L.tsv_stream.restype = C.c_void_p
         L.tsv_stream.argtypes = [C.c_void_p]
         L.tsv_session_pool_size.argtypes = [C.c_void_p]
+        L.tsv_kv_row_bytes.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+        L.tsv_kv_bytes_for_context.restype = C.c_int64
+        L.tsv_kv_bytes_for_context.argtypes = [C.c_void_p, C.c_int64]
         L.tsv_session_swapped.argtypes = [C.c_void_p]
         L.tsv_session_best_match.restype = C.c_int64
         L.tsv_session_best_match.argtypes = [C.c_void_p, C.c_int64, C.POINTER(C.c_int64)]
