@@ -438,3 +438,41 @@ def test_prompt_passes_of_64_rows_over_quantized_rows(name, kv_bits, n_prompt):
           f"64-row passes vs oracle {err_w:.2e}, after 16-row passes {err_n:.2e}, the two GPU paths {err_wn:.2e}")
     bound = 1.5e-1 if kv_bits == (2, 2) else 5e-2
     assert min(same) >= 0.97 and err_w <= bound and err_wn <= bound
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes_of_attention_over_stored_rows(seed):
+    """A seeded sweep over head widths, head groupings, pass widths, prefix lengths (block boundaries, short and long
+    contexts), the four width pairs and sinks: stored rows by bits on a sample, the pass against the oracle."""
+    from oracle import binding as ob
+    from turbospark_amd import ffi
+    rng = np.random.default_rng(1000 + seed)
+    hd = int(rng.choice([64, 128]))
+    nkv = int(rng.choice([1, 2, 4, 8]))
+    g = int(rng.choice([1, 2, 4, 8]))
+    nq = nkv * g
+    m = int(rng.integers(1, 17))
+    base = int(rng.choice([0, 1, 15, 16, 17, 31, int(rng.integers(32, 600)), int(rng.integers(600, 7000))]))
+    kb, vb = [(2, 2), (3, 3), (3, 4), (4, 4)][int(rng.integers(0, 4))]
+    sinks = rng.standard_normal(nq).astype(np.float32) if rng.random() < 0.4 else None
+    scale = float(rng.choice([0.0, 0.1, 0.2]))
+    seq = base + m
+    q = rng.standard_normal((m, nq, hd)).astype(np.float16)
+    k = (rng.standard_normal((seq, nkv, hd)) * rng.uniform(0.1, 4.0, (seq, nkv, 1))).astype(np.float16)
+    v = (rng.standard_normal((seq, nkv, hd)) * rng.uniform(0.1, 4.0, (seq, nkv, 1))).astype(np.float16)
+    print(f"seed {seed}: hd={hd} q/kv={nq}/{nkv} m={m} base={base} K{kb}/V{vb} sinks={'yes' if sinks is not None else 'no'} scale={scale}",
+          flush=True)
+    got, kr, vr = ffi.attention_quantized(q, k, v, base, kb, vb, scale=scale, sinks=sinks)
+    ks, kc, km, vs, vc, vm = _sides(hd, kb, vb)
+    pick = np.unique(np.concatenate([np.arange(min(seq, 8)), np.arange(max(0, base - 3), seq), rng.integers(0, seq, 8)]))
+    _check_rows(k[pick], kr[pick], ks, km, kb)
+    _check_rows(v[pick], vr[pick], vs, vm, vb)
+    rows = sorted(set([0, m - 1, int(rng.integers(0, m))]))
+    worst = 0.0
+    for i in rows:
+        want = ob.tq_attention(q[i].astype(np.float32), kr[:, :, 1:], kr[:, :, 0].view(np.float32), vr[:, :, 1:],
+                               vr[:, :, 0].view(np.float32), hd, nq, nkv, base + i + 1, kb, ks, kc, vs, vc, scale=scale,
+                               sinks=sinks, v_bits=vb).reshape(nq, hd)
+        worst = max(worst, float(np.abs(got[i] - want).max() / np.abs(want).max()))
+    print(f"  worst relative error {worst:.2e}")
+    assert worst <= 5e-3
