@@ -42,12 +42,14 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def algorithmic_bytes(cfg, ctx, m, union=None):
+def algorithmic_bytes(cfg, ctx, m, union=None, kv_bits=None):
     """Bytes one verify step has to move: every quantized weight once, the KV rows [0, ctx+m)
     once per layer, m embedding rows, m x vocab fp16 logits, m new KV rows.  Routed experts: an
     expert's matrices count once per layer in which any row chose it; `union` is the mean number of
     distinct experts per layer actually routed (read back from the device), None the expectation
-    under independent uniform routing."""
+    under independent uniform routing.  kv_bits = (key bits, value bits): the layers the reference's policy
+    quantizes (full attention, all but the last of a stack of more than two) cost a norm and packed indices per
+    kv head instead of fp16 rows."""
     from turbospark_amd import ffi
     H, F, V, L = cfg["hidden"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
     qd, kvd = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
@@ -66,10 +68,15 @@ def algorithmic_bytes(cfg, ctx, m, union=None):
         per_layer = dict(qkv=rb(qd + 2 * kvd, H), wo=rb(H, qd), gate_up=rb(2 * F, H), down=rb(H, F))
     head = rb(V, H)
     weights = L * sum(per_layer.values()) + head
-    kv = L * (ctx + m) * kvd * 2 * 2
-    if cfg.get("gptoss"):  # even layers read only their window
-        win = (L + 1) // 2
-        kv = ((L - win) * (ctx + m) + win * min(cfg["gptoss"]["window"] + m, ctx + m)) * kvd * 2 * 2
+    fp16_row = kvd * 2 * 2
+    kv = 0
+    for l in range(L):
+        windowed = bool(cfg.get("gptoss")) and l % 2 == 0      # even layers read only their window
+        positions = min(cfg["gptoss"]["window"] + m, ctx + m) if windowed else ctx + m
+        row = fp16_row
+        if kv_bits and not windowed and (L <= 2 or l + 1 < L):
+            row = sum(cfg["n_kv_heads"] * (4 + 4 * ((cfg["head_dim"] * b + 31) // 32)) for b in kv_bits)
+        kv += positions * row
     small = m * ffi.row_bytes(cfg["dtype"], H) + m * V * 2 + L * m * kvd * 2 * 2
     return dict(per_layer=per_layer, head=head, weights=weights, kv=kv, total=weights + kv + small)
 
@@ -377,7 +384,7 @@ def main():
             sel = eng.route_selected()[:, :m, :cfg["top_k"]]
             per_step.append(np.mean([len(np.unique(sel[l])) for l in range(sel.shape[0])]))
         union = float(np.mean(per_step))
-    ab = algorithmic_bytes(cfg, ctx, m, union)
+    ab = algorithmic_bytes(cfg, ctx, m, union, kv_bits)
     L = cfg["n_layers"]
     kern = {}
     for name, nbytes, count in (("qkv", ab["per_layer"]["qkv"], L), ("wo", ab["per_layer"]["wo"], L),
@@ -446,8 +453,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "rows": m, "context": ctx,
                    "temperature": T, "mean_accepted": round(mean_acc, 3), "min_margin": min_margin,
-                   **({"kv_rows": f"TurboQuant K{kv_bits[0]}/V{kv_bits[1]} on every full-attention layer but the last; "
-                                  "algorithmic bytes below still count fp16 rows"} if kv_bits else {}),
+                   **({"kv_rows": f"TurboQuant K{kv_bits[0]}/V{kv_bits[1]} on every full-attention layer but the last"} if kv_bits else {}),
                    **({"experts_routed_per_layer": round(union, 2),
                        "routing": "the synthetic router's own" if args.routing == "model" else
                                   "forced: top_k experts per row drawn uniformly and independently"} if union is not None else {})},
