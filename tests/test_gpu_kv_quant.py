@@ -476,3 +476,44 @@ def test_random_shapes_of_attention_over_stored_rows(seed):
         worst = max(worst, float(np.abs(got[i] - want).max() / np.abs(want).max()))
     print(f"  worst relative error {worst:.2e}")
     assert worst <= 5e-3
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_model_shapes_with_quantized_rows(seed):
+    """The seeded decoder shapes of tests/test_gpu_random_shapes.py with a random width pair: the pass (chain or tree)
+    against the oracle with the same codec within the codec's sensitivity, determinism by bits, and -- for chains of at
+    most eight rows, where the fp16-row path holds it too -- the pass as single-row passes by bits."""
+    import turbospark_amd as ts
+    from oracle import binding as ob
+    from tests.test_gpu_random_shapes import _case
+    from turbospark_amd import ffi
+    os.environ["TSV_FUSED"] = "0"
+    cfg, ctx, m, parent, r = _case(seed)
+    kv_bits = [(2, 2), (3, 3), (3, 4), (4, 4)][int(r.integers(0, 4))]
+    cfg = dict(cfg, max_context=ctx + 40)
+    from turbospark_amd import synth
+    w = synth.make_weights(cfg, seed=77 + seed)
+    gpu = ts.HipVerifier(cfg, w, kv_bits=kv_bits)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16, kv_bits=kv_bits)
+    V = cfg["vocab"]
+    print(f"seed {seed}: {'q4_k' if cfg['dtype'] == ffi.Q4_K else 'q8_0'} L={cfg['n_layers']} H={cfg['hidden']} "
+          f"q/kv={cfg['n_q_heads']}/{cfg['n_kv_heads']}x{cfg['head_dim']} ctx={ctx} m={m} {'tree' if parent else 'chain'}"
+          f"{' qk-norm' if cfg['qk_norm'] else ''} K{kv_bits[0]}/V{kv_bits[1]}", flush=True)
+    prompt = r.integers(0, V, ctx).astype(np.int32)
+    feed = r.integers(0, V, m).astype(np.int32)
+    gpu.prefill(prompt, 0, want_logits=False)
+    for i in range(0, ctx, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    point = gpu.checkpoint()
+    got = gpu.verify_tree(feed, parent, ctx) if parent else gpu.verify(feed, ctx)
+    want = cpu.verify(feed, ctx, parent=parent)
+    err = gc.logit_error(got, want)
+    print(f"   max-abs logit error / range = {err:.2e}", flush=True)
+    assert err <= (2.5e-1 if kv_bits == (2, 2) else 1.2e-1)
+    gpu.rollback(point)
+    again = gpu.verify_tree(feed, parent, ctx) if parent else gpu.verify(feed, ctx)
+    assert np.array_equal(got, again)
+    if not parent and m <= 8 and m * (cfg["n_q_heads"] // cfg["n_kv_heads"]) <= 32:
+        gpu.rollback(point)
+        single = np.concatenate([gpu.verify(feed[i:i + 1], ctx + i) for i in range(m)])
+        assert np.array_equal(got, single)
