@@ -509,7 +509,7 @@ def test_random_model_shapes_with_quantized_rows(seed):
     want = cpu.verify(feed, ctx, parent=parent)
     err = gc.logit_error(got, want)
     print(f"   max-abs logit error / range = {err:.2e}", flush=True)
-    assert err <= (2.5e-1 if kv_bits == (2, 2) else 1.2e-1)
+    assert err <= (2e-1 if kv_bits == (2, 2) else 8e-2)
     gpu.rollback(point)
     again = gpu.verify_tree(feed, parent, ctx) if parent else gpu.verify(feed, ctx)
     assert np.array_equal(got, again)
