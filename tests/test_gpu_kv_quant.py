@@ -517,3 +517,40 @@ def test_random_model_shapes_with_quantized_rows(seed):
         gpu.rollback(point)
         single = np.concatenate([gpu.verify(feed[i:i + 1], ctx + i) for i in range(m)])
         assert np.array_equal(got, single)
+
+
+def _greedy_decode(eng, steps, vocab):
+    """crates/runtime/tests/real_forward_llama_kv_quant.rs:56-80: produce, take the arg-max, feed it back."""
+    eng.reset()
+    token, out = 5, []
+    for position in range(steps):
+        logits = gc.f16(eng.produce(token, position))
+        assert np.isfinite(logits).all(), position
+        out.append(logits)
+        token = int(np.argmax(logits))
+    return np.stack(out)
+
+
+def test_the_reference_runtime_scenarios_for_kv_bits():
+    """crates/runtime/tests/real_forward_llama_kv_quant.rs: `off` is the plain handle by bits; every width the option
+    names decodes finite and deterministic over several tokens; turning it on moves the output past the first token
+    (where a single key makes the key side invisible); an unsupported head width is refused by name."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    os.environ["TSV_FUSED"] = "0"
+    cfg = dict(synth.CONFIGS["tiny_q8_0"], max_context=64, n_layers=4)
+    w = synth.make_weights(cfg, seed=9)
+    V = cfg["vocab"]
+    plain = _greedy_decode(ts.HipVerifier(cfg, w), 6, V)
+    off = _greedy_decode(ts.HipVerifier(cfg, w, kv_bits=ts.producer.parse_kv_bits("off")), 6, V)
+    assert np.array_equal(plain, off)
+    for text in ("2", "3", "3.5", "4"):
+        bits = ts.producer.parse_kv_bits(text)
+        first = _greedy_decode(ts.HipVerifier(cfg, w, kv_bits=bits), 5, V)
+        second = _greedy_decode(ts.HipVerifier(cfg, w, kv_bits=bits), 5, V)
+        assert np.array_equal(first, second), text
+    on = _greedy_decode(ts.HipVerifier(cfg, w, kv_bits=(3, 4)), 5, V)
+    assert np.abs(on[1:] - plain[1:5]).max() > 1e-3
+    bad = dict(cfg, head_dim=32, n_q_heads=16, n_kv_heads=16)
+    with pytest.raises(ts.ffi.TsvError, match="head_dim"):
+        ts.HipVerifier(bad, synth.make_weights(bad, seed=9), kv_bits=(4, 4))
