@@ -178,9 +178,14 @@ __device__ __forceinline__ void attn_partial_body_tq(const AttnArgs& a, int G, i
                 lrun[t] = fmaf(lrun[t], alpha, ps);
                 mrun[t] = mnew;
             }
+            // once the running maximum has settled the factor is exactly 1 in every lane: the products are
+            // skipped then (the same bits), which is most blocks of a long context
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+                for (int d = 0; d < VT; d++) O[t][d] *= alpha;
+            }
 #pragma unroll
             for (int d = 0; d < VT; d++) {
-                O[t][d] *= alpha;
                 O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, vf[d]), P, O[t][d], 0, 0, 0);
             }
         }
