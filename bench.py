@@ -111,14 +111,34 @@ def trace_summary(path, first="k_clear_result"):
     print(f"total kernel time in {what}: {total / 1e6:.3f} ms over the traced steps")
 
 
-# Figures RECORDED from committed counter / trace runs (a bench run does not collect counters): HBM
-# bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
-# over `bench.py --traffic-probe`, scaled by the copy kernel of known size (`bench.py
-# --traffic-summary`): 66 793 486 B read + 258 048 B written against 66 060 288 algorithmic bytes;
-# and the same kernel's average duration in the committed rocprofv3 kernel trace of this script.
-RECORDED = {"llama3_8b_q4_k_k4_ctx4096": dict(
-    traffic=67051534, traffic_source="recorded: profiles/gate_up_matmul_llama3_8b_q4k_hbm_traffic.txt",
-    trace_avg_us=16.68, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt")}
+# Figures RECORDED from committed counter / trace runs (a bench run does not collect counters).  `traffic`: HBM
+# bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, scaled by the
+# copy kernel of known size (headline workload: over `bench.py --traffic-probe`, 66 793 486 B read + 258 048 B
+# written against 66 060 288 algorithmic bytes; the others: the kernel's rows of `bench.py --step-traffic`, for the
+# routed workloads router + top-k + grouped gate/up together, as `achieved` counts them).  `trace_avg_us`: the same
+# kernel(s) in the committed rocprofv3 kernel trace of this script.  `step_traffic`: bytes read + written per
+# verify pass over all its kernels, to set beside `step_algorithmic_bytes`.
+_TRAFFIC = "recorded: profiles/verify_step_hbm_traffic_by_kernel_all_workloads.txt"
+RECORDED = {
+    "llama3_8b_q4_k_k4_ctx4096": dict(
+        traffic=67051534, traffic_source="recorded: profiles/gate_up_matmul_llama3_8b_q4k_hbm_traffic.txt",
+        trace_avg_us=16.68, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt",
+        step_traffic=5057454669 + 166119858, step_traffic_source=_TRAFFIC),
+    "llama3_8b_q4_k_tree16_ctx16384": dict(
+        traffic=67348044 + 516096, traffic_source=_TRAFFIC,
+        trace_avg_us=20.31, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt",
+        step_traffic=6973116518 + 511734731, step_traffic_source=_TRAFFIC),
+    "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(
+        traffic=(526294 + 18432) + (38401 + 3978) + (17877765 + 139726), traffic_source=_TRAFFIC,
+        trace_avg_us=4.80 + 6.69 + 9.98, trace_source="recorded: profiles/verify_step_qwen3_30b_a3b_mxfp4_ctx8192_kernels.txt "
+                                                      "(router + k_route + k_moe_fp4<1, 2, 1>)",
+        step_traffic=3815633101 + 291355412, step_traffic_source=_TRAFFIC),
+    "gptoss_120b_mxfp4_k8_ctx32768": dict(
+        traffic=(917440 + 36864) + (57345 + 3680) + (175608367 + 262669), traffic_source=_TRAFFIC,
+        trace_avg_us=4.61 + 5.14 + 35.07, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
+                                                       "(router + k_route + k_moe_fp4<1, 2, 1>)",
+        step_traffic=14106062728 + 188963704, step_traffic_source=_TRAFFIC),
+}
 
 GATE_UP_8B = dict(dtype=12, rows=28672, cols=4096, m=5, epi=1)   # the dominant kernel of the headline workload
 COPY_BYTES = 256 << 20
@@ -205,6 +225,39 @@ def traffic_summary(fetch_csv, write_csv, which):
     print(json.dumps(out, indent=1))
 
 
+def step_traffic(fetch_csv, write_csv, first="k_clear_result"):
+    """HBM bytes per launch of every kernel of the verify passes, from two `rocprofv3 --pmc` collections (FETCH_SIZE,
+    then WRITE_SIZE) of `bench.py --copy-probe ...`: dispatches from the first acceptance kernel on, keyed by kernel
+    name and grid like --trace-summary, each counter scaled by what it reads for the copy kernel of known size that
+    --copy-probe launches in the same process.  The last line is the whole run's bytes over its passes (one k_embed
+    each)."""
+    import csv
+    tables, passes = {}, 0
+    for side, path, counter in (("read", fetch_csv, "FETCH_SIZE"), ("write", write_csv, "WRITE_SIZE")):
+        rows = [r for r in csv.DictReader(open(path)) if r["Counter_Name"] == counter]
+        rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+        copies = [float(r["Counter_Value"]) for r in rows if "k_copy_probe" in r["Kernel_Name"]]
+        factor = COPY_BYTES / (sum(copies) / len(copies))
+        start = next(i for i, r in enumerate(rows) if first in r["Kernel_Name"])
+        passes = sum("k_embed" in r["Kernel_Name"] for r in rows[start:])
+        for r in rows[start:]:
+            name = r["Kernel_Name"].replace("tsv::", "").replace("(anonymous namespace)::", "").split("(")[0].replace("void ", "")
+            key = (name, int(r["Grid_Size"]) // max(int(r["Workgroup_Size"]), 1))
+            st = tables.setdefault(key, {"read": [0, 0.0], "write": [0, 0.0]})[side]
+            st[0] += 1
+            st[1] += float(r["Counter_Value"]) * factor
+        print(f"# {counter}: {factor:.2f} bytes per unit ({len(copies)} copy launches of {COPY_BYTES} B)")
+    print(f"{'kernel':44s} {'wgs':>6s} {'calls':>7s} {'read_B/launch':>14s} {'written_B/launch':>17s}")
+    tot = [0.0, 0.0]
+    for (name, wgs), v in sorted(tables.items(), key=lambda kv: -(kv[1]["read"][1] + kv[1]["write"][1])):
+        rd, wr = v["read"], v["write"]
+        tot[0] += rd[1]
+        tot[1] += wr[1]
+        print(f"{name[:44]:44s} {wgs:6d} {rd[0]:7d} {rd[1] / max(rd[0], 1):14.0f} {wr[1] / max(wr[0], 1):17.0f}")
+    print(f"all dispatches from the first {first} on: {tot[0] / passes:.0f} B read + {tot[1] / passes:.0f} B written per pass "
+          f"({passes} passes)")
+
+
 def counter_summary(path, which):
     """Per-dispatch averages of every counter in a `rocprofv3 --pmc ... --output-format csv` collection of
     `bench.py --traffic-probe`, for the probed kernel's launches (the copy kernel is left out)."""
@@ -223,6 +276,12 @@ def main():
                     help="per-dispatch averages of the counters a rocprofv3 --pmc run of --traffic-probe collected")
     ap.add_argument("--traffic-summary", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="HBM bytes per launch of the dominant matmul from two --pmc runs of --traffic-probe")
+    ap.add_argument("--step-traffic", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="HBM bytes per launch of every kernel of the verify passes from two --pmc runs of this script "
+                         "with --copy-probe")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="for a --pmc run: launch the copy kernel of known size before the workload (it calibrates the "
+                         "counters) and leave out the per-kernel timing, whose passes launch one kernel class twice")
     ap.add_argument("--probe", default="gate_up", choices=sorted(PROBES),
                     help="which kernel --traffic-probe runs and the two summaries read")
     ap.add_argument("--trace-from", default="k_clear_result", metavar="KERNEL",
@@ -256,6 +315,9 @@ def main():
         return
     if args.traffic_summary:
         traffic_summary(*args.traffic_summary, args.probe)
+        return
+    if args.step_traffic:
+        step_traffic(*args.step_traffic, args.trace_from)
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "
@@ -300,6 +362,9 @@ def main():
     prompt = rng.integers(0, V, ctx).astype(np.int32)
     t0 = time.time()
     eng.prefill(prompt[:-1], 0, want_logits=False)   # the last prompt token is the round's confirmed token
+    if args.copy_probe:
+        us = ts.ffi.copy_time(COPY_BYTES, iters=3)
+        log(f"[bench] copy kernel {COPY_BYTES >> 20} MiB: {us:.1f} us")
     prefill_s = time.time() - t0                      # first use: includes one-time allocations (--prefill-bench times it properly)
     log(f"[bench] prefill of {ctx - 1} tokens in {prefill_s:.2f}s")
     base = eng.position
@@ -390,10 +455,13 @@ def main():
     for name, nbytes, count in (("qkv", ab["per_layer"]["qkv"], L), ("wo", ab["per_layer"]["wo"], L),
                                 ("gate_up", ab["per_layer"]["gate_up"], L), ("down", ab["per_layer"]["down"], L),
                                 ("head", ab["head"], 1), ("attention", ab["kv"] // L, L), ("rope_kv", 0, L)):
-        eng.set_repeat(name, 2)
-        twice_ms = timed_region(nrep)
-        eng.set_repeat(name, 1)
-        avg_ms = (twice_ms - plain_ms) / count
+        if args.copy_probe:   # a counter run: every pass plain, so that the collection divides evenly by its passes
+            avg_ms = 0.0
+        else:
+            eng.set_repeat(name, 2)
+            twice_ms = timed_region(nrep)
+            eng.set_repeat(name, 1)
+            avg_ms = (twice_ms - plain_ms) / count
         kern[name] = dict(avg_us=round(avg_ms * 1000, 2), bytes=int(nbytes), launches_per_step=count,
                           GBps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1) if nbytes and avg_ms > 0 else None)
     gemm_ms = sum(kern[n]["avg_us"] * kern[n]["launches_per_step"] for n in ("qkv", "wo", "gate_up", "down", "head")) / 1000.0
@@ -411,7 +479,8 @@ def main():
         kern["qkv"]["epilogue"] = "bias + rotation + fp16 q / KV-cache stores"
     dom = kern.get("gate_up", {})
     peak = 8000.0
-    rec = RECORDED.get(args.workload, {})
+    # the recorded figures are the workload's as named: not a variant's (other KV rows, forced routing, fewer layers)
+    rec = {} if (kv_bits or args.routing != "model" or args.layers) else RECORDED.get(args.workload, {})
     roofline = dict(bound="hbm",
                     kernel=f"router + grouped expert gate/up matmuls (experts actually routed: {union:.1f} of {cfg['n_experts']} per layer)"
                     if cfg.get("n_experts")
@@ -428,6 +497,7 @@ def main():
                     algorithmic_bytes_per_launch=dom.get("bytes"), avg_launch_us=dom.get("avg_us"),
                     all_matmuls_GBps=round(ab["weights"] / (gemm_ms * 1e-3) / 1e9, 1) if gemm_ms else None,
                     step_algorithmic_bytes=int(ab["total"]),
+                    step_traffic=rec.get("step_traffic"), step_traffic_source=rec.get("step_traffic_source"),
                     step_frac_of_hbm_roofline=round(ab["total"] / (ms_per_step * 1e-3) / 1e9 / peak, 4),
                     per_kernel=kern,
                     profile_ms_per_step={n: round(v[0] / nprof, 4) for n, v in prof.items()})

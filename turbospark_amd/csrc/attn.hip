@@ -29,6 +29,11 @@ int attn_chunks(int nkv) {
 template <int HD, int RT, int STAGES>
 __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) {
     extern __shared__ float xch[];  // [4 slots][PER_LANE values][64 lanes]
+    if (a.xcd_groups) {  // several row groups of a verify pass: placed by die
+        int chunk, kvh, grp;
+        if (attn_grid_place(a, blockIdx.x, chunk, kvh, grp)) attn_partial_body<HD, RT, STAGES, false>(a, G, R, chunk, kvh, grp * RT, xch);
+        return;
+    }
     // grid z: row groups of the pass, times the 16-row blocks of a prompt pass
     const int groups = gridDim.z / max(a.blocks, 1), blk = blockIdx.z / groups, grp = blockIdx.z - blk * groups;
     if (a.blocks > 1) {
@@ -49,6 +54,12 @@ __global__ __launch_bounds__(512) void k_attn_partial_tq(AttnArgs a, int G, int 
     __syncthreads();
     // blocks in flight: three, two where the three-bit fields' extra words would push the registers past 256
     constexpr int STAGES = (HD == 128 && RT == 2 && KB == 3 && VB == 3) ? 2 : 3;
+    if (a.xcd_groups) {
+        int chunk, kvh, grp;
+        if (attn_grid_place(a, blockIdx.x, chunk, kvh, grp))
+            attn_partial_body_tq<HD, RT, STAGES, KB, VB>(a, G, R, chunk, kvh, grp * RT, xch, s_kpair, s_vpair);
+        return;
+    }
     // grid z: row groups of the pass, times the 16-row blocks of a prompt pass
     const int groups = gridDim.z / max(a.blocks, 1), blk = blockIdx.z / groups, grp = blockIdx.z - blk * groups;
     if (a.blocks > 1) {
@@ -147,7 +158,8 @@ static int launch_partial(hipStream_t s, const AttnArgs& a, int G, int R, int gr
                                     (int)lds));
         raised = true;
     }
-    hipLaunchKernelGGL((k_attn_partial<HD, RT, STAGES>), dim3(a.nch, a.nkv, groups * std::max(a.blocks, 1)), dim3(512), lds, s, a, G, R);
+    const dim3 grid = a.xcd_groups ? dim3(attn_grid_size(a.nch * a.nkv, groups)) : dim3(a.nch, a.nkv, groups * std::max(a.blocks, 1));
+    hipLaunchKernelGGL((k_attn_partial<HD, RT, STAGES>), grid, dim3(512), lds, s, a, G, R);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -165,7 +177,8 @@ static int launch_partial_tq(hipStream_t s, const AttnArgs& a, int G, int R, int
                                     (int)lds));
         raised = true;
     }
-    hipLaunchKernelGGL((k_attn_partial_tq<HD, RT, KB, VB>), dim3(a.nch, a.nkv, groups * std::max(a.blocks, 1)), dim3(512), lds, s, a, G, R);
+    const dim3 grid = a.xcd_groups ? dim3(attn_grid_size(a.nch * a.nkv, groups)) : dim3(a.nch, a.nkv, groups * std::max(a.blocks, 1));
+    hipLaunchKernelGGL((k_attn_partial_tq<HD, RT, KB, VB>), grid, dim3(512), lds, s, a, G, R);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -183,12 +196,17 @@ static int launch_partial_tq_widths(hipStream_t s, const AttnArgs& a, int G, int
 template <int HD>
 static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     const int trt = (R + 15) / 16;
-    // more than 32 (row, q head) pairs: groups of 32 in grid z, each re-reading K and V (from L2)
+    // more than 32 (row, q head) pairs: groups of 32, each re-reading K and V (from L2)
     const int groups = trt <= 2 ? 1 : (trt + 1) / 2;
     // about one workgroup per compute unit: the chunk count shrinks as the row groups multiply
     // (fewer, longer chunks also mean fewer partial results for the merge to read)
     AttnArgs a = a0;
     a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 256 / (a0.nkv * groups * std::max(a0.blocks, 1))));
+    // Several row groups of a verify pass read the same K / V: they are placed on one die.  A workgroup fills a
+    // compute unit (eight waves at two per SIMD) and a die has 32 of them: no die may be handed more than 32
+    // workgroups, or its last one waits for a whole workgroup to end (26 against 18 us at 21 chunks x 4 heads x 3)
+    a.xcd_groups = (groups > 1 && a0.blocks <= 1) ? groups : 0;
+    if (a.xcd_groups) a.nch = std::max(std::min(a0.nch, 8), std::min(a0.nch, 8 * (32 / groups) / a0.nkv));
     int rc;
     if (a.tq.k_bits) {
         if (a.window || a.ring || !a.unrot) {

@@ -345,9 +345,26 @@ struct AttnArgs {
     // its base position at base_hint + 16 b, and its q rows, partial results and output fragments at the
     // strides below
     int blocks;
+    // set by the launcher.  Non-zero: a one-dimensional grid in which the row groups of one (chunk, kv head) pair
+    // take neighbouring slots of ONE of the eight dies (attn_grid_place), this many groups per pair
+    int xcd_groups;
     size_t q_stride, part_o_stride, part_ml_stride;  // elements
     size_t frag_stride;                              // bytes
 };
+// Which (chunk, kv head, row group) a workgroup of the one-dimensional grid works on.  Workgroups go round the
+// eight dies (XCDs, each with an L2 of its own) by linear index: index 8 s + x is slot s of die x.  A pair's row
+// groups sit in slots next to each other on one die, so they start together and the K / V bytes the first one
+// pulls in reach the others through that die's L2 instead of being fetched once per die.  False: a slot past the
+// last pair, nothing to do.
+__device__ inline bool attn_grid_place(const AttnArgs& a, int index, int& chunk, int& kvh, int& grp) {
+    const int die = index & 7, slot = index >> 3;
+    grp = slot % a.xcd_groups;
+    const int pair = (slot / a.xcd_groups) * 8 + die;
+    chunk = pair % a.nch;
+    kvh = pair / a.nch;
+    return pair < a.nch * a.nkv;
+}
+inline int attn_grid_size(int pairs, int groups) { return 8 * groups * ((pairs + 7) / 8); }
 // the view of one block of such a launch
 __host__ __device__ inline AttnArgs attn_block_view(const AttnArgs& a, int b) {
     AttnArgs v = a;
