@@ -20,6 +20,7 @@
 // Repetition / presence / frequency penalties (sampled chain and tree rounds, the draft draws) are
 // applied per candidate as it is read, from a per-token table of the history (see score_of);
 // the kernels are compiled twice, and the variant without penalties is the code it always was.
+#include <algorithm>
 #include <cstring>
 
 #include "tsv_internal.h"
@@ -115,12 +116,17 @@ __device__ __forceinline__ bool survives(uint16_t bits, int v, const RowStat& s)
     return key < s.cut_key || (key == s.cut_key && v <= s.cut_idx);
 }
 
+// (p / top)^(1/T), choose.rs:296-311.  At T = 1 the power is the identity -- the host library's pow returns its
+// argument exactly there -- and the device's software pow, the most expensive operation of these kernels, is skipped
+// (a branch every lane takes the same way).
+__device__ __forceinline__ double temper(double x, double inv_t) { return inv_t == 1.0 ? x : pow(x, inv_t); }
+
 // choose.rs:296-319 for one candidate of a row whose statistics are known
 __device__ __forceinline__ double prob_of(uint16_t bits, int v, const RowStat& s, double inv_t) {
     if (!survives(bits, v, s)) return 0.0;
     const double e = exp((double)h2f(bits) - s.mx);
     const double p = e / s.sum;
-    return pow(p / s.top, inv_t) / s.total;
+    return temper(p / s.top, inv_t) / s.total;
 }
 
 // ---- penalised scores -------------------------------------------------------------------------
@@ -198,7 +204,7 @@ __device__ __forceinline__ double prob_of_w(float w, int key, int v, const RowSt
         if (e < s.minp) return 0.0;
     }
     const double p = e / s.sum;
-    return pow(p / s.top, inv_t) / s.total;
+    return temper(p / s.top, inv_t) / s.total;
 }
 
 template <typename T>
@@ -328,11 +334,11 @@ __global__ __launch_bounds__(256) void k_row_total(const uint16_t* target, const
             if (!survives_w<true>(w, (int)key_of<true>(w, b), v, cs)) continue;
             const double e = exp((double)w - mx);
             if (app->has_min_p && e < app->min_p) continue;
-            acc += pow((e / sum) / top, inv_t);
+            acc += temper((e / sum) / top, inv_t);
         } else {
             if (!survives(b, v, cs)) continue;
             const double e = exp((double)h2f(b) - mx);
-            acc += pow((e / sum) / top, inv_t);
+            acc += temper((e / sum) / top, inv_t);
         }
     }
     acc = block_sum_f64(acc, red);
@@ -1455,6 +1461,25 @@ static void launch_chain_sampled(hipStream_t s, const uint16_t* target, const ui
                        (unsigned long long*)sc.hist, decisions(sc), sc.result, (int32_t*)nullptr, err, 0);
 }
 
+// The most child tests a walk can take before it stops.  At a node with children c_1 < ... < c_n (tested in slot
+// order) the walk either rejects all n, or rejects j - 1, accepts c_j and goes on from there: worst(node) =
+// max(n, max_j (j + worst(c_j))).  A parent's slot is below its children's, so one descending sweep fills the
+// table.  Never more than m - 1 (every slot behind the root is tested at most once); 6 for the 16-node tree of a
+// root with four chains, where m - 1 is 15.
+static int tree_walk_bound(const AcceptParams& ap) {
+    int worst[TSV_MAX_ROWS] = {0}, seen[TSV_MAX_ROWS] = {0};
+    // children in descending slot order: the j of child c is known once all of its parent's children are counted
+    int count[TSV_MAX_ROWS] = {0};
+    for (int c = 1; c < ap.m; c++) count[ap.parent[c]]++;
+    for (int c = ap.m - 1; c >= 1; c--) {
+        const int par = ap.parent[c];
+        const int j = count[par] - seen[par];  // c is the j-th child of its parent in ascending order
+        seen[par]++;
+        worst[par] = std::max(worst[par], std::max(count[par], j + worst[c]));
+    }
+    return std::min(worst[0], ap.m - 1);
+}
+
 template <bool PEN>
 static void launch_tree_sampled(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
                                 const AcceptParams& ap, const AcceptScratch& sc) {
@@ -1463,11 +1488,12 @@ static void launch_tree_sampled(hipStream_t s, const uint16_t* target, const uin
     // statistics of the m target rows and the m rows the children were drawn from
     launch_stats<PEN>(s, target, draft, ap.m, 2 * ap.m, 2 * 65536, ap_dev, ap, sc);
     hipLaunchKernelGGL(k_tree_probs<PEN>, dim3(NSEG, 2 * ap.m), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
-    // every slot behind the root is tested at most once: m - 1 steps cover any walk
-    for (int k = 0; k < ap.m - 1; k++)
+    // one child test per launch: as many launches as the longest walk through this tree can take
+    const int steps = tree_walk_bound(ap);
+    for (int k = 0; k < steps; k++)
         hipLaunchKernelGGL(k_tree_step<PEN>, dim3(TREE_WGS), dim3(256), 0, s, ap_dev, sc.stats, sc.work, k);
     hipLaunchKernelGGL(k_tree_finish<PEN>, dim3(TREE_WGS), dim3(256), 0, s, target, ap_dev, sc.stats, sc.work,
-                       (unsigned long long*)sc.hist, decisions(sc), path, ap.m - 1);
+                       (unsigned long long*)sc.hist, decisions(sc), path, steps);
     hipLaunchKernelGGL(k_pick<PEN>, dim3(1), dim3(1024), 0, s, target, draft, ap_dev, sc.stats, sc.work,
                        (unsigned long long*)sc.hist, decisions(sc), sc.result, path, err, 2);
 }
