@@ -516,6 +516,24 @@ __global__ __launch_bounds__(256) void k_mass_hist(const uint16_t* target, const
 template <class Fn>
 __device__ __forceinline__ void scan_chunk(const uint16_t* lp, int v0, int v1, uint32_t want, bool zero_bin, bool vec,
                                            Fn&& on_match) {
+    // sixty-four keys at a time while the range lasts: the eight loads are in flight together (the loop below, one
+    // load per turn with the matches' own loads behind it, waits out a memory round trip per eight keys)
+    if (vec) {
+        for (; v0 + 64 <= v1; v0 += 64) {
+            uint4 q[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = *(const uint4*)(lp + v0 + 8 * i);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint32_t w[4] = {q[i].x, q[i].y, q[i].z, q[i].w};
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const uint32_t bits = (w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+                    if (bits == want || (zero_bin && bits == 0x8000u)) on_match(v0 + 8 * i + j);
+                }
+            }
+        }
+    }
     for (int g = v0; g < v1; g += 8) {
         uint32_t w[4];
         if (vec && g + 8 <= v1) {
@@ -929,16 +947,26 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         const unsigned long long tgt = (unsigned long long)(dec.job.u * (double)total);
         if (loc > 0) atomicMax(&s_last_bin, tid * 64 + 63);
         if (excl <= tgt && tgt < excl + loc) {
-            unsigned long long c = excl;
-            for (int i = 0; i < 64; i++) {
-                const unsigned long long hv = hmine[i * 64];
-                if (tgt < c + hv) {
-                    s_bin = tid * 64 + i;
-                    s_before = c;
-                    break;
+            // the one thread whose 64 bins hold the target: first bin at which the running sum passes it.  The bins
+            // are fetched sixteen at a time (a loop that stops at the hit waits out one L2 round trip per bin)
+            unsigned long long c = excl, before = excl;
+            int hit = -1;
+            for (int b = 0; b < 4; b++) {
+                unsigned long long hv[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) hv[i] = hmine[(b * 16 + i) * 64];
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    if (hit < 0 && tgt < c + hv[i]) {
+                        hit = b * 16 + i;
+                        before = c;
+                    }
+                    c += hv[i];
                 }
-                c += hv;
+                if (hit >= 0) break;
             }
+            s_bin = tid * 64 + hit;
+            s_before = before;
         }
         if (tid == 0) s_total = total;
         __syncthreads();
