@@ -277,7 +277,9 @@ int32_t tsv_compact_tree(tsv_ctx* ctx, int64_t base, const uint32_t* path, int32
  * of that verify.  A tree at temperature > 0 runs multi-branch rejection (children in
  * slot order, r * q(x) <= p(x), residual max(p - q, 0) renormalised after a rejection);
  * the reference keeps tree rounds greedy (speculative.rs:390-392), so that mode has no
- * counterpart there, and it takes no stop tokens or budget. */
+ * counterpart there, and it takes no stop tokens or budget.  m, base and the tree
+ * (parent, or NULL for a chain) must be those of that verify: anything else is refused
+ * as TSV_ERR_INVALID before a kernel runs. */
 int32_t tsv_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result* out);
 /* verify + accept + truncate in one call: the whole verify step. */
 int32_t tsv_verify_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result* out);

@@ -381,6 +381,24 @@ def test_refusals_by_name():
     gpu.rollback(ts.ffi.Point(base))
     with pytest.raises(TsvError, match="non-finite"):
         gpu.verify_accept([1, 2], base, ts.shaping(0.8, seed=3), draft_logits=bad)
+    # the tree a round names has to be well formed, and the one the pass attended by
+    gpu.rollback(ts.ffi.Point(base))
+    feed = [1, 2, 3, 4]
+    gpu.verify(feed, base)                                   # a chain pass ...
+    with pytest.raises(TsvError, match="not the one the last verify pass attended by"):
+        gpu.accept(feed, base, ts.shaping(0.0), parent=[-1, 0, 0, 1])        # ... judged as a tree
+    with pytest.raises(TsvError, match=r"parent\[s\] in \[0, s\)"):
+        gpu.accept(feed, base, ts.shaping(0.0), parent=[-1, 0, 2, 1])        # a link that does not lead towards slot 0
+    with pytest.raises(TsvError, match=r"parent\[0\] must be -1"):
+        gpu.accept(feed, base, ts.shaping(0.0), parent=[0, 0, 1, 2])
+    assert gpu.accept(feed, base, ts.shaping(0.0), parent=[-1, 0, 1, 2]).committed >= 0   # the chain, spelled out
+    gpu.rollback(ts.ffi.Point(base))
+    gpu.verify_tree(feed, [-1, 0, 0, 1], base)               # a tree pass ...
+    with pytest.raises(TsvError, match="not the one the last verify pass attended by"):
+        gpu.accept(feed, base, ts.shaping(0.0))                               # ... judged as a chain
+    with pytest.raises(TsvError, match="not the one the last verify pass attended by"):
+        gpu.accept(feed, base, ts.shaping(0.0), parent=[-1, 0, 0, 2])
+    assert gpu.accept(feed, base, ts.shaping(0.0), parent=[-1, 0, 0, 1]).committed >= 0
 
 
 def test_a_vocabulary_that_is_not_a_multiple_of_anything_convenient():

@@ -155,6 +155,7 @@ struct tsv_ctx {
     bool headless = false;      // the pass in flight is a prefill pass nobody reads the logits of
     int last_m = 0;
     int64_t last_base = -1;
+    bool last_shape_known = false;  // vp_host holds the ancestor sets of the rows tsv_accept is about to judge
     // The launch sequence of a pass depends on the row count only (positions, tokens and the
     // tree shape are read from device memory), so it can be captured once per row count into a
     // HIP graph and replayed (environment TSV_GRAPH=1).  Off by default: the pass is bound by
@@ -450,6 +451,7 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     c->high_water = std::max(c->high_water, c->position);
     c->last_m = m;
     c->last_base = base;
+    c->last_shape_known = true;
     return TSV_OK;
 }
 
@@ -1924,6 +1926,21 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
         set_error("accept: the round does not describe the last verify pass");
         return TSV_ERR_INVALID;
     }
+    // the tree the round names: well formed (the walks on both sides follow parent links towards slot 0), and the
+    // one the pass attended by -- a chain pass judged as a tree, or the other way round, would accept rows that never
+    // saw their supposed ancestors
+    uint32_t anc[TSV_MAX_ROWS];
+    for (int i = 0; i < r->m; i++) {
+        if (r->parent && (i == 0 ? r->parent[0] != -1 : (r->parent[i] < 0 || r->parent[i] >= i))) {
+            set_error("accept: parent[0] must be -1 and parent[s] in [0, s)");
+            return TSV_ERR_INVALID;
+        }
+        anc[i] = r->parent ? (i == 0 ? 0u : anc[r->parent[i]]) | (1u << i) : (2u << i) - 1u;
+        if (c->last_shape_known && anc[i] != c->vp_host->anc[i]) {
+            set_error("accept: the round's tree is not the one the last verify pass attended by");
+            return TSV_ERR_INVALID;
+        }
+    }
     const bool sampled = r->shaping.temperature != 0.0;
     const uint16_t* draft = nullptr;
     if (sampled) {
@@ -2118,6 +2135,7 @@ extern "C" int32_t tsv_write_logits(tsv_ctx* c, const uint16_t* logits, int32_t 
     TSV_HIP(hipStreamSynchronize(c->stream));
     c->last_m = m;
     c->last_base = base;
+    c->last_shape_known = false;  // rows from the host: whatever tree the round names is taken at its word
     return TSV_OK;
 }
 
