@@ -122,11 +122,11 @@ _TRAFFIC = "recorded: profiles/verify_step_hbm_traffic_by_kernel_all_workloads.t
 RECORDED = {
     "llama3_8b_q4_k_k4_ctx4096": dict(
         traffic=67051534, traffic_source="recorded: profiles/gate_up_matmul_llama3_8b_q4k_hbm_traffic.txt",
-        trace_avg_us=16.68, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt",
+        trace_avg_us=16.33, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt",
         step_traffic=5057454669 + 166119858, step_traffic_source=_TRAFFIC),
     "llama3_8b_q4_k_tree16_ctx16384": dict(
         traffic=67348044 + 516096, traffic_source=_TRAFFIC,
-        trace_avg_us=20.41, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt",
+        trace_avg_us=20.40, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt",
         step_traffic=6973116518 + 511734731, step_traffic_source=_TRAFFIC),
     "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(
         traffic=(526294 + 18432) + (38401 + 3978) + (17877765 + 139726), traffic_source=_TRAFFIC,
@@ -135,7 +135,7 @@ RECORDED = {
         step_traffic=3815633101 + 291355412, step_traffic_source=_TRAFFIC),
     "gptoss_120b_mxfp4_k8_ctx32768": dict(
         traffic=(917440 + 36864) + (57345 + 3680) + (175608367 + 262669), traffic_source=_TRAFFIC,
-        trace_avg_us=4.61 + 5.28 + 35.20, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
+        trace_avg_us=4.61 + 5.19 + 35.13, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
                                                        "(router + k_route + k_moe_fp4<1, 2, 1>)",
         step_traffic=14106062728 + 188963704, step_traffic_source=_TRAFFIC),
 }
@@ -492,7 +492,7 @@ def main():
                     traffic=rec.get("traffic"), traffic_source=rec.get("traffic_source", "not measured for this workload"),
                     # the same kernel in the committed rocprofv3 kernel trace (begin-to-end of the dispatch, which
                     # includes what overlaps with its neighbours in the pipeline): the lower of the two fractions
-                    trace_avg_launch_us=rec.get("trace_avg_us"), trace_source=rec.get("trace_source"),
+                    trace_avg_launch_us=round(rec["trace_avg_us"], 2) if rec.get("trace_avg_us") else None, trace_source=rec.get("trace_source"),
                     trace_frac=round(dom["bytes"] / (rec["trace_avg_us"] * 1e-6) / 1e9 / peak, 4) if rec.get("trace_avg_us") and dom.get("bytes") else None,
                     algorithmic_bytes_per_launch=dom.get("bytes"), avg_launch_us=dom.get("avg_us"),
                     all_matmuls_GBps=round(ab["weights"] / (gemm_ms * 1e-3) / 1e9, 1) if gemm_ms else None,
