@@ -875,6 +875,7 @@ __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, cons
 // One workgroup per job.  Finds the rank bin in which the cumulative mass first exceeds the
 // uniform (exact integer prefix over the fixed-point bins, cleared as they are read), then
 // walks that bin's candidates in index order in f64.
+constexpr int PICK_MASK_GROUPS = 32;  // groups of eight entries per thread the match mask holds: vocabularies to 262 144
 template <bool PEN>
 __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uint16_t* draft,
                                                const AcceptParams* app, double* scratch, const double* work,
@@ -882,6 +883,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
                                                AcceptResult* res, int32_t* tokens_out, int32_t* err,
                                                int kind) {
     __shared__ SideEnt s_raw[PEN ? SIDE_CAP : 1], s_sorted[PEN ? SIDE_CAP : 1];
+    __shared__ uint32_t s_mask[PEN ? 1 : 1024 * PICK_MASK_GROUPS / 4];  // one bit per vocabulary entry: on the bin's value
     __shared__ int s_nside, s_side_last;
     __shared__ double s_side_sum;
     __shared__ unsigned long long wsum[16];
@@ -920,9 +922,23 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         // 64 consecutive rank bins per thread (see bin_addr); integer sums are exact and order
         // independent
         const unsigned long long* hmine = hsel + (tid >> 6) * 4096 + (tid & 63);
-        unsigned long long loc = 0;
-#pragma unroll 16
-        for (int i = 0; i < 64; i++) loc += hmine[i * 64];
+        // (one workgroup reads the whole histogram: what bounds it is how many loads a wave keeps in flight, so the 64
+        // bins come as two rounds of 32 loads)
+        unsigned long long quarter[4], loc = 0;  // the bins' sum in four runs of sixteen: the rescan below needs one run
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            unsigned long long hv[32];
+#pragma unroll
+            for (int i = 0; i < 32; i++) hv[i] = hmine[(half * 32 + i) * 64];
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                unsigned long long q = 0;
+#pragma unroll
+                for (int i = 0; i < 16; i++) q += hv[b * 16 + i];
+                quarter[half * 2 + b] = q;
+                loc += q;
+            }
+        }
         unsigned long long inc = loc;
         for (int o = 1; o < 64; o <<= 1) {
             const uint32_t lo = __shfl_up((uint32_t)inc, o), hi = __shfl_up((uint32_t)(inc >> 32), o);
@@ -947,23 +963,29 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         const unsigned long long tgt = (unsigned long long)(dec.job.u * (double)total);
         if (loc > 0) atomicMax(&s_last_bin, tid * 64 + 63);
         if (excl <= tgt && tgt < excl + loc) {
-            // the one thread whose 64 bins hold the target: first bin at which the running sum passes it.  The bins
-            // are fetched sixteen at a time (a loop that stops at the hit waits out one L2 round trip per bin)
-            unsigned long long c = excl, before = excl;
-            int hit = -1;
-            for (int b = 0; b < 4; b++) {
-                unsigned long long hv[16];
+            // the one thread whose 64 bins hold the target: first bin at which the running sum passes it.  Only the
+            // run of sixteen the target falls into is fetched again, all of it at once (a loop over the 64 bins that
+            // stops at the hit waits out one L2 round trip per bin)
+            unsigned long long c = excl;
+            int b = 0;
 #pragma unroll
-                for (int i = 0; i < 16; i++) hv[i] = hmine[(b * 16 + i) * 64];
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    if (hit < 0 && tgt < c + hv[i]) {
-                        hit = b * 16 + i;
-                        before = c;
-                    }
-                    c += hv[i];
+            for (int t = 0; t < 3; t++)
+                if (b == t && !(tgt < c + quarter[t])) {
+                    c += quarter[t];
+                    b = t + 1;
                 }
-                if (hit >= 0) break;
+            unsigned long long hv[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) hv[i] = hmine[(b * 16 + i) * 64];
+            unsigned long long before = c;
+            int hit = -1;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                if (hit < 0 && tgt < c + hv[i]) {
+                    hit = b * 16 + i;
+                    before = c;
+                }
+                c += hv[i];
             }
             s_bin = tid * 64 + hit;
             s_before = before;
@@ -1018,9 +1040,66 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
         // walk the bin in index order: contiguous index chunk per thread
         const int per = ((vocab + 1023) / 1024 + 7) & ~7, v0 = min(tid * per, vocab), v1 = min(v0 + per, vocab);
         const bool vec = ((uintptr_t)lp & 15) == 0;
+        // Without penalties a candidate of the bin is found by its fp16 bits.  The row is read ONCE, coalesced --
+        // neighbouring lanes take neighbouring groups of eight entries, where a lane reading its own contiguous chunk
+        // touches 64 cache lines per load -- and leaves one bit per entry in LDS; each thread then walks the bits of
+        // its own chunk, here and again in the walk below, in the index order the sums are defined in.
+        const int groups = per >> 3;
+        const bool masked = !PEN && vec && groups <= PICK_MASK_GROUPS;
+        if constexpr (!PEN) {
+            if (masked) {
+                uint8_t* mask8 = (uint8_t*)s_mask;
+                const uint32_t want = key_bits(bin);
+                const bool zero_bin = want == 0;
+                // sixteen loads in flight per lane: a group past the row's last whole one reads group 0 and is discarded
+                const int whole = vocab >> 3;  // groups of eight entries that lie wholly inside the row
+                for (int g0 = 0; g0 < groups; g0 += 16) {
+                    uint4 q[16];
+#pragma unroll
+                    for (int j = 0; j < 16; j++) {
+                        const int g = (g0 + j) * 1024 + tid;
+                        q[j] = *(const uint4*)(lp + (g0 + j < groups && g < whole ? (long)g * 8 : 0));
+                    }
+#pragma unroll
+                    for (int j = 0; j < 16; j++) {
+                        if (g0 + j >= groups) break;
+                        const int g = (g0 + j) * 1024 + tid;
+                        const uint32_t t[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
+                        uint32_t m = 0;
+#pragma unroll
+                        for (int h = 0; h < 8; h++) {
+                            const uint32_t bits = (t[h >> 1] >> (16 * (h & 1))) & 0xFFFFu;
+                            m |= (uint32_t)(bits == want || (zero_bin && bits == 0x8000u)) << h;
+                        }
+                        mask8[g] = g < whole ? (uint8_t)m : (uint8_t)0;
+                    }
+                }
+                if ((vocab & 7) && whole < groups * 1024 && tid == (whole & 1023)) {  // the row's last, partial group
+                    uint32_t m = 0;
+                    for (int h = 0; h < (vocab & 7); h++) {
+                        const uint32_t bits = lp[(long)whole * 8 + h];
+                        m |= (uint32_t)(bits == want || (zero_bin && bits == 0x8000u)) << h;
+                    }
+                    mask8[whole] = (uint8_t)m;
+                }
+                __syncthreads();
+            }
+        }
+        // on_match(v) for the candidates of this thread's chunk that sit on the bin's value, ascending
+        auto for_matches = [&](auto&& on_match) {
+            if constexpr (!PEN) {
+                if (masked) {
+                    const uint8_t* mine = (const uint8_t*)s_mask + tid * groups;
+                    for (int k = 0; k < groups; k++)
+                        for (uint32_t m = mine[k]; m; m &= m - 1) on_match(v0 + 8 * k + (__ffs(m) - 1));
+                    return;
+                }
+            }
+            scan_on<PEN>(ap, dec.job.row_p, lp, v0, v1, bin, vec, on_match);
+        };
         double lsum = 0.0;
         int lastv = -1;
-        scan_on<PEN>(ap, dec.job.row_p, lp, v0, v1, bin, vec, [&](int v) {
+        for_matches([&](int v) {
             const double wv = mode == 2 ? w[v] / R : w[v];
             if (mode != 2 || wv > 0.0) {
                 lsum += wv;
@@ -1046,7 +1125,7 @@ __global__ __launch_bounds__(1024) void k_pick(const uint16_t* target, const uin
             if (lsum > 0.0 && !(u < before) && u < before + lsum) {
                 double c = before;
                 bool found = false;
-                scan_on<PEN>(ap, dec.job.row_p, lp, v0, v1, bin, vec, [&](int v) {
+                for_matches([&](int v) {
                     if (found) return;
                     const double wv = mode == 2 ? w[v] / R : w[v];
                     if (mode == 2 && !(wv > 0.0)) return;
