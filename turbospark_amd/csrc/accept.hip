@@ -873,7 +873,7 @@ __global__ __launch_bounds__(1024) void k_trunc_cut(const uint16_t* target, cons
 
 // ---- the cumulative walk --------------------------------------------------------------------
 // One workgroup per job.  Finds the rank bin in which the cumulative mass first exceeds the
-// uniform (exact integer prefix over the fixed-point bins, cleared as they are read), then
+// uniform (exact integer prefix over the fixed-point bins, which the round's first kernel zeroed), then
 // walks that bin's candidates in index order in f64.
 constexpr int PICK_MASK_GROUPS = 32;  // groups of eight entries per thread the match mask holds: vocabularies to 262 144
 template <bool PEN>
