@@ -33,6 +33,11 @@ int32_t tsv_write_logits(tsv_ctx* ctx, const uint16_t* logits, int32_t m, int64_
  * the engine's own split-K factor. */
 int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits);
 
+/* Host arithmetic only: how many launches of the walk kernel a sampled tree round of this shape is given -- the most
+ * child tests any walk through the tree can take (children are tested in slot order; a walk rejects all n children of
+ * a node, or rejects j - 1, accepts the j-th and goes on below it).  -1 for a malformed tree. */
+int32_t tsv_tree_walk_bound(const int32_t* parent, int32_t m);
+
 /* Per-kernel-class timing with HIP events on the handle's stream (one event pair per launch
  * while enabled).  Classes, in order: embed, norm, qkv matmul, rope+kv store, attention,
  * output projection, gate/up matmul, down matmul, output head, acceptance, and "event pair":

@@ -1573,18 +1573,18 @@ static void launch_chain_sampled(hipStream_t s, const uint16_t* target, const ui
 // max(n, max_j (j + worst(c_j))).  A parent's slot is below its children's, so one descending sweep fills the
 // table.  Never more than m - 1 (every slot behind the root is tested at most once); 6 for the 16-node tree of a
 // root with four chains, where m - 1 is 15.
-static int tree_walk_bound(const AcceptParams& ap) {
+int tree_walk_bound(const int32_t* parent, int m) {
     int worst[TSV_MAX_ROWS] = {0}, seen[TSV_MAX_ROWS] = {0};
     // children in descending slot order: the j of child c is known once all of its parent's children are counted
     int count[TSV_MAX_ROWS] = {0};
-    for (int c = 1; c < ap.m; c++) count[ap.parent[c]]++;
-    for (int c = ap.m - 1; c >= 1; c--) {
-        const int par = ap.parent[c];
+    for (int c = 1; c < m; c++) count[parent[c]]++;
+    for (int c = m - 1; c >= 1; c--) {
+        const int par = parent[c];
         const int j = count[par] - seen[par];  // c is the j-th child of its parent in ascending order
         seen[par]++;
         worst[par] = std::max(worst[par], std::max(count[par], j + worst[c]));
     }
-    return std::min(worst[0], ap.m - 1);
+    return std::min(worst[0], m - 1);
 }
 
 template <bool PEN>
@@ -1596,7 +1596,7 @@ static void launch_tree_sampled(hipStream_t s, const uint16_t* target, const uin
     launch_stats<PEN>(s, target, draft, ap.m, 2 * ap.m, 2 * 65536, ap_dev, ap, sc);
     hipLaunchKernelGGL(k_tree_probs<PEN>, dim3(NSEG, 2 * ap.m), dim3(256), 0, s, target, draft, ap_dev, sc.stats, sc.work);
     // one child test per launch: as many launches as the longest walk through this tree can take
-    const int steps = tree_walk_bound(ap);
+    const int steps = tree_walk_bound(ap.parent, ap.m);
     for (int k = 0; k < steps; k++)
         hipLaunchKernelGGL(k_tree_step<PEN>, dim3(TREE_WGS), dim3(256), 0, s, ap_dev, sc.stats, sc.work, k);
     hipLaunchKernelGGL(k_tree_finish<PEN>, dim3(TREE_WGS), dim3(256), 0, s, target, ap_dev, sc.stats, sc.work,
@@ -1824,4 +1824,19 @@ extern "C" int32_t tsv_accept_greedy_noalloc(void* stream, const uint16_t* logit
     hipLaunchKernelGGL(k_walk_greedy_value, dim3(1), dim3(64), 0, s, ap, base, sc->pv, sc->pi, &sc->err, result_dev);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
+}
+
+// Test hook: the number of walk launches a sampled tree round of this shape gets (host arithmetic only).
+extern "C" int32_t tsv_tree_walk_bound(const int32_t* parent, int32_t m) {
+    using namespace tsv;
+    if (!parent || m < 1 || m > TSV_MAX_ROWS || parent[0] != -1) {
+        set_error("tree_walk_bound: 1..16 slots, parent[0] == -1");
+        return -1;
+    }
+    for (int i = 1; i < m; i++)
+        if (parent[i] < 0 || parent[i] >= i) {
+            set_error("tree_walk_bound: parent[s] must lie in [0, s)");
+            return -1;
+        }
+    return tree_walk_bound(parent, m);
 }

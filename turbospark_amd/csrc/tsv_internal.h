@@ -505,6 +505,8 @@ struct AcceptScratch {
 };
 constexpr int ACCEPT_COUNTER_WORDS = 1024;
 size_t accept_stats_doubles();
+// launches of the walk kernel a sampled tree round of this shape needs (parent[s] in [0, s), m <= TSV_MAX_ROWS)
+int tree_walk_bound(const int32_t* parent, int m);
 int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, const AcceptParams* ap_dev,
                   const AcceptParams& ap_host, const AcceptScratch& sc);
 int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,

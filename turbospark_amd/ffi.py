@@ -247,7 +247,7 @@ EXPORTS = [
     "tsv_prefix_rewind_to", "tsv_prefix_untainted_len", "tsv_prefix_common",
     "tsv_set_prefix_reuse", "tsv_try_reuse_prefix", "tsv_record_committed", "tsv_prefix_len",
     "tsv_gguf_open", "tsv_gguf_close", "tsv_gguf_tensor_count", "tsv_gguf_data_start", "tsv_gguf_tensor",
-    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected", "tsv_force_route",
+    "tsv_gguf_meta_number", "tsv_gguf_meta_string", "tsv_open_gguf", "tsv_route_selected", "tsv_force_route", "tsv_tree_walk_bound",
     "tsv_read_kv_quantized", "tsv_attention_quantized", "tsv_kv_quant_tables",
     "tsv_session_pool_size", "tsv_session_slot_evicted", "tsv_session_best_match", "tsv_session_lru", "tsv_session_swapped",
     "tsv_kv_row_bytes", "tsv_kv_bytes_for_context",
