@@ -30,14 +30,21 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-pthread",
 ] + (["-DTSV_WITH_FUSED"] if WITH_FUSED else [])
+# TSV_HOST_UBSAN=1: the host pass of every source under the undefined-behaviour sanitizer in trap mode (no runtime
+# to link; device code is compiled as always), objects kept apart.  With TSV_LIB_NAME=libtsverify_ubsan.so for both
+# the build and the tests, every host path the suites reach either is clean or stops the process where it is not.
+HOST_UBSAN = os.environ.get("TSV_HOST_UBSAN", "0") == "1"
+if HOST_UBSAN:
+    FLAGS += ["-Xarch_host", "-fsanitize=undefined,bounds", "-Xarch_host", "-fsanitize-trap=all", "-g"]
+OBJ_DIR = "build_ubsan" if HOST_UBSAN else "build"
 
 
 def build(verbose=False):
     objs = []
     procs = []
-    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    os.makedirs(os.path.join(HERE, OBJ_DIR), exist_ok=True)
     for src in SOURCES:
-        obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+        obj = os.path.join(HERE, OBJ_DIR, src.replace(".hip", ".o"))
         cmd = ["hipcc", OPT.get(src, "-O3"), *FLAGS, *EXTRA.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
