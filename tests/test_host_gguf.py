@@ -227,3 +227,55 @@ def test_the_independent_reader_recovers_what_the_writer_was_given(tmp_path):
             assert np.array_equal(np.asarray(w[k][1]).reshape(-1), np.asarray(ow[k][1]).reshape(-1)), (name, k)
         if arch == "gpt-oss":
             assert np.allclose(ocfg["rope_freqs"], cfg["rope_freqs"]) and abs(ocfg["rope_mscale"] - cfg["rope_mscale"]) < 1e-7
+
+
+def test_mutated_headers_are_refused_or_read_within_the_file(tmp_path):
+    """Seeded damage to a valid file's header -- flipped bytes, huge little-endian integers dropped onto 8-byte
+    fields, truncation -- must end in a refusal by name or in reads that stay inside the file: the process surviving
+    the loop is the assertion (a parser that trusts a count or an offset dies here)."""
+    tensors = _tensors()[0]
+    path = os.path.join(tmp_path, "base.gguf")
+    start = write_gguf(path, META, tensors)
+    good = open(path, "rb").read()
+    names = [t[0] for t in tensors]
+    rng = np.random.default_rng(11)
+    big = [2 ** 64 - 1, 2 ** 63, 2 ** 63 - 1, 2 ** 61, 2 ** 40, 2 ** 32, 2 ** 31, len(good), len(good) + 1, 0]
+    refused = opened = 0
+    for case in range(600):
+        data = bytearray(good)
+        kind = case % 3
+        if kind == 0:      # a few flipped bytes in the header
+            for _ in range(int(rng.integers(1, 5))):
+                data[int(rng.integers(4, start))] = int(rng.integers(0, 256))
+        elif kind == 1:    # a huge or boundary integer over an 8-byte field
+            at = int(rng.integers(8, start - 8))
+            data[at:at + 8] = int(big[int(rng.integers(0, len(big)))]).to_bytes(8, "little")
+        else:              # truncation anywhere, header or data
+            data = data[:int(rng.integers(0, len(good)))]
+        p = os.path.join(tmp_path, "m.gguf")
+        open(p, "wb").write(bytes(data))
+        try:
+            g = ffi.Gguf(p)
+        except ffi.TsvError:
+            refused += 1
+            continue
+        opened += 1
+        assert 0 <= g.tensor_count <= 4096
+        for name in names:
+            try:
+                dt, raw, rows, cols = g.tensor(name)
+                assert raw.nbytes <= len(data)
+            except ffi.TsvError:
+                pass
+        for key in ("llama.block_count", "x.i64", "general.architecture"):
+            try:
+                g.number(key)
+            except ffi.TsvError:
+                pass
+            try:
+                g.string(key)
+            except ffi.TsvError:
+                pass
+        g.close()
+    print(f"600 damaged files: {refused} refused at open, {opened} opened and read within bounds")
+    assert refused > 100 and opened > 20
