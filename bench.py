@@ -122,11 +122,11 @@ _TRAFFIC = "recorded: profiles/verify_step_hbm_traffic_by_kernel_all_workloads.t
 RECORDED = {
     "llama3_8b_q4_k_k4_ctx4096": dict(
         traffic=67051534, traffic_source="recorded: profiles/gate_up_matmul_llama3_8b_q4k_hbm_traffic.txt",
-        trace_avg_us=16.33, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt",
+        trace_avg_us=16.17, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt",
         step_traffic=5057454669 + 166119858, step_traffic_source=_TRAFFIC),
     "llama3_8b_q4_k_tree16_ctx16384": dict(
         traffic=67348044 + 516096, traffic_source=_TRAFFIC,
-        trace_avg_us=20.40, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt",
+        trace_avg_us=20.46, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt",
         step_traffic=6973116518 + 511734731, step_traffic_source=_TRAFFIC),
     "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(
         traffic=(526294 + 18432) + (38401 + 3978) + (17877765 + 139726), traffic_source=_TRAFFIC,
@@ -135,7 +135,7 @@ RECORDED = {
         step_traffic=3815633101 + 291355412, step_traffic_source=_TRAFFIC),
     "gptoss_120b_mxfp4_k8_ctx32768": dict(
         traffic=(917440 + 36864) + (57345 + 3680) + (175608367 + 262669), traffic_source=_TRAFFIC,
-        trace_avg_us=4.61 + 5.19 + 35.13, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
+        trace_avg_us=4.61 + 5.26 + 35.33, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
                                                        "(router + k_route + k_moe_fp4<1, 2, 1>)",
         step_traffic=14106062728 + 188963704, step_traffic_source=_TRAFFIC),
 }
