@@ -135,7 +135,7 @@ RECORDED = {
         step_traffic=3815633101 + 291355412, step_traffic_source=_TRAFFIC),
     "gptoss_120b_mxfp4_k8_ctx32768": dict(
         traffic=(917440 + 36864) + (57345 + 3680) + (175608367 + 262669), traffic_source=_TRAFFIC,
-        trace_avg_us=4.61 + 5.26 + 35.33, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
+        trace_avg_us=4.56 + 5.43 + 35.22, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
                                                        "(router + k_route + k_moe_fp4<1, 2, 1>)",
         step_traffic=14106062728 + 188963704, step_traffic_source=_TRAFFIC),
 }

@@ -55,7 +55,8 @@ struct tsv_ctx {
     int n_layers = 0, hidden = 0, nq = 0, nkv = 0, hd = 0, ffn = 0, vocab = 0, max_context = 0, ctx_alloc = 0;
     float eps = 0, attn_scale = 0, rope_mscale = 1.0f, act_alpha = 0, act_limit = 0;
     hipStream_t stream = nullptr;
-    bool rope_fused_ok = true;  // TSV_ROPE_FUSED=0 keeps the projection and the rotation apart
+    bool rope_fused_ok = true;     // TSV_ROPE_FUSED=0 keeps the projection and the rotation apart
+    bool rope_fused_force = false;  // TSV_ROPE_FUSED=1 fuses them whatever a tile weighs
     std::vector<LayerW> layers;
     TiledW head;
     uint8_t* embed_raw = nullptr;
@@ -1092,7 +1093,10 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     c->act_alpha = d->act_alpha;
     c->act_limit = d->act_limit;
     if (const char* e = getenv("TSV_GRAPH")) c->use_graph = e[0] == '1';
-    if (const char* e = getenv("TSV_ROPE_FUSED")) c->rope_fused_ok = e[0] != '0';
+    if (const char* e = getenv("TSV_ROPE_FUSED")) {
+        c->rope_fused_ok = e[0] != '0';
+        c->rope_fused_force = e[0] == '1';
+    }
     // MXFP4 experts on the block-scaled matrix instruction: activation terms, 0 = the fp16 path
     c->moe_fp4_terms = MOE_FP4_DEFAULT_TERMS;
     if (const char* e = getenv("TSV_MOE_FP4")) c->moe_fp4_terms = e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
@@ -1144,8 +1148,12 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         }
         // One launch that projects, rotates and stores (no split-K partials, no separate rotation
         // kernel) where the head needs no per-head norm in between and q/k/v share a storage type.
-        L.rope_fused = c->rope_fused_ok && s.wv.dtype == s.wq.dtype && !s.q_norm.data && !s.k_norm.data &&
-                       (c->hd == 64 || c->hd == 128);
+        // The fused launch has one workgroup per 64-row tile and no K split, and one compute unit draws only so much:
+        // it is taken while a tile's weights stay under 256 KiB (8B Q4_K: 147 KB per tile, a tie with the two
+        // launches; gpt-oss-120B bf16: 369 KB, 15.3 us fused against 7.9 + 3.1 us apart).
+        const bool light_tiles = 64 * row_bytes(s.wq.dtype, s.wq.cols) <= 256 * 1024;
+        L.rope_fused = c->rope_fused_ok && (light_tiles || c->rope_fused_force) && s.wv.dtype == s.wq.dtype &&
+                       !s.q_norm.data && !s.k_norm.data && (c->hd == 64 || c->hd == 128);
         if (s.wv.dtype == s.wq.dtype) {
             if ((rc = make_tiled(c, st, qkv, 3, false, &L.qkv, L.rope_fused && c->hd == 128 ? 2 : 0))) return fail(rc);
         } else {
