@@ -137,7 +137,7 @@ RECORDED = {
         traffic=(917440 + 36864) + (57345 + 3680) + (175608367 + 262669), traffic_source=_TRAFFIC,
         trace_avg_us=4.56 + 5.43 + 35.22, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
                                                        "(router + k_route + k_moe_fp4<1, 2, 1>)",
-        step_traffic=14106062728 + 188963704, step_traffic_source=_TRAFFIC),
+        step_traffic=14135922230 + 229660271, step_traffic_source=_TRAFFIC),
 }
 
 GATE_UP_8B = dict(dtype=12, rows=28672, cols=4096, m=5, epi=1)   # the dominant kernel of the headline workload
