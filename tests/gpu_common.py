@@ -1,6 +1,4 @@
 """Shared helpers of the GPU parity tests: model construction on both sides, tolerances."""
-import os
-
 import numpy as np
 
 import turbospark_amd as ts
@@ -13,8 +11,6 @@ def f16(bits):
 
 
 def build_pair(name, max_context, seed=1234, threads=8, **over):
-    # the XCD-shaped configurations exist to exercise the per-XCD fused kernels (opt-in)
-    os.environ["TSV_FUSED"] = "1" if name.startswith("xcd_") else "0"
     cfg = dict(synth.CONFIGS[name])
     cfg.update(over)
     cfg["max_context"] = max_context

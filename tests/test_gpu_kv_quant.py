@@ -95,7 +95,6 @@ def test_attention_over_stored_rows_matches_the_rotated_space_oracle(nq, nkv, hd
 def _open(name, kv_bits, max_context=96, seed=21, **over):
     import turbospark_amd as ts
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS[name], max_context=max_context, **over)
     w = synth.make_weights(cfg, seed=seed)
     return cfg, w, ts.HipVerifier(cfg, w, kv_bits=kv_bits)
@@ -272,7 +271,6 @@ def test_llama3_8b_shape_two_layers_at_4096_context_with_four_bit_rows():
     import turbospark_amd as ts
     from oracle import binding as ob
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     ctx, kv_bits = 4096, (4, 4)
     cfg = dict(synth.CONFIGS["llama3_8b_q4_k"], n_layers=2, max_context=ctx + 32)
     w = synth.make_weights(cfg, seed=3, n_layers=2)
@@ -316,7 +314,6 @@ def test_graph_replay_over_quantized_rows_equals_plain_launches():
     logits and stored rows."""
     import turbospark_amd as ts
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS["small_q4_k"], max_context=160, n_layers=3)
     w = synth.make_weights(cfg, seed=5)
     plain = ts.HipVerifier(cfg, w, kv_bits=(4, 4))
@@ -349,7 +346,6 @@ def test_gptoss_120b_shape_with_the_full_layers_rows_quantized():
     import turbospark_amd as ts
     from oracle import binding as ob
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     ctx, kv_bits = 3000, (3, 4)
     cfg = dict(synth.CONFIGS["gptoss_120b"], n_layers=2, max_context=ctx + 32, vocab=4096)
     w = synth.make_weights(cfg, seed=3, n_layers=2)
@@ -401,7 +397,6 @@ def test_prompt_passes_of_64_rows_over_quantized_rows(name, kv_bits, n_prompt):
     import turbospark_amd as ts
     from oracle import binding as ob
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS[name], max_context=n_prompt + 48, n_layers=3)
     w = synth.make_weights(cfg, seed=11)
 
@@ -487,7 +482,6 @@ def test_random_model_shapes_with_quantized_rows(seed):
     from oracle import binding as ob
     from tests.test_gpu_random_shapes import _case
     from turbospark_amd import ffi
-    os.environ["TSV_FUSED"] = "0"
     cfg, ctx, m, parent, r = _case(seed)
     kv_bits = [(2, 2), (3, 3), (3, 4), (4, 4)][int(r.integers(0, 4))]
     cfg = dict(cfg, max_context=ctx + 40)
@@ -537,7 +531,6 @@ def test_the_reference_runtime_scenarios_for_kv_bits():
     (where a single key makes the key side invisible); an unsupported head width is refused by name."""
     import turbospark_amd as ts
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS["tiny_q8_0"], max_context=64, n_layers=4)
     w = synth.make_weights(cfg, seed=9)
     V = cfg["vocab"]

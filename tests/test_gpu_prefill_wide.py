@@ -25,7 +25,6 @@ def _engine(cfg, weights, wide):
 def test_a_prompt_fed_in_blocks_of_64_fills_the_cache_the_oracle_fills(name, n_prompt):
     from turbospark_amd import synth
     from oracle import binding as ob
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS[name], max_context=n_prompt + 48)
     w = synth.make_weights(cfg, seed=11)
     wide, narrow = _engine(cfg, w, True), _engine(cfg, w, False)
@@ -61,7 +60,6 @@ def test_logits_of_the_last_prompt_token_after_wide_passes():
     16-row passes whose last one carries the output head."""
     from turbospark_amd import synth
     from oracle import binding as ob
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS["small_q4_k"], max_context=256)
     w = synth.make_weights(cfg, seed=12)
     wide = _engine(cfg, w, True)
@@ -79,7 +77,6 @@ def test_logits_of_the_last_prompt_token_after_wide_passes():
 
 def test_wide_passes_are_deterministic_and_leave_the_prefix_record_intact():
     from turbospark_amd import synth
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS["small_q4_k"], max_context=256)
     w = synth.make_weights(cfg, seed=13)
     a, b = _engine(cfg, w, True), _engine(cfg, w, True)

@@ -14,7 +14,6 @@ pytestmark = pytest.mark.gpu
 
 
 def _open(name="tiny_q8_0", slots=2, kv_bits=None, max_context=160, ring=False, **over):
-    os.environ["TSV_FUSED"] = "0"
     cfg = dict(synth.CONFIGS[name], max_context=max_context, **over)
     w = synth.make_weights(cfg, seed=77)
     if ring:   # the windowed layers keep rings (and the handle a finite rewind budget): they are swapped like the rest

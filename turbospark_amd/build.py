@@ -7,17 +7,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
 SOURCES = ["gemm.hip", "moe.hip", "moe_fp4.hip", "misc.hip", "attn.hip", "kvquant.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
-# The per-XCD fused layer kernels (an experiment that measured slower than the kernels it replaces) are
-# built only on request: TSV_BUILD_FUSED=1.
-WITH_FUSED = os.environ.get("TSV_BUILD_FUSED", "0") == "1"
-if WITH_FUSED:
-    SOURCES += ["fused.hip", "attn_block.hip"]
 # host_utils.hip is host-only code; clang 22 -O3 does not terminate on it, -O2 does.
 OPT = {"host_utils.hip": "-O2", "gguf.hip": "-O2"}
 # MFMA results straight into VGPRs (no v_accvgpr_read copies before the scaling FMAs)
 EXTRA = {"gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_GEMM_DEFS", "").split(),
-         "fused.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),
-         "attn_block.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] + os.environ.get("TSV_FUSED_DEFS", "").split(),
          "moe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
          "moe_fp4.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 FLAGS = [
@@ -29,7 +22,7 @@ FLAGS = [
     # packed-fp32 VALU forms are switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-pthread",
-] + (["-DTSV_WITH_FUSED"] if WITH_FUSED else [])
+]
 # TSV_HOST_UBSAN=1: the host pass of every source under the undefined-behaviour sanitizer in trap mode (no runtime
 # to link; device code is compiled as always), objects kept apart.  With TSV_LIB_NAME=libtsverify_ubsan.so for both
 # the build and the tests, every host path the suites reach either is clean or stops the process where it is not.

@@ -97,19 +97,15 @@ struct tsv_ctx {
         float *part_o = nullptr, *part_ml = nullptr;  // attention partials of every block
         size_t part_o_stride = 0, part_ml_stride = 0;
     } wide;
-    // per-XCD fused layer kernels (fused.hip): second residual buffer, private fragment copies,
-    // sum-of-squares partials, per-XCD partial sums, barrier counters
-    bool fused_ffn = false, fused_attn = false;
-    int attn_stages = 5;  // TSV_FUSED_ATTN_STAGES: how far the attention block goes before the separate kernels take over
-    float* partial8a = nullptr;  // the attention block's per-XCD partial sums
-    float* x2 = nullptr;
-    uint8_t* frag8 = nullptr;
-    size_t frag8_stride = 0;
-    float* ssq8 = nullptr;
-    float* partial8 = nullptr;
-    unsigned *rank_ctr = nullptr, *bar_ctr = nullptr;
-    int* fused_err = nullptr;  // pinned host memory the kernels can write
-    unsigned bar_count = 0;
+    // Overlapped passes (handoff.h): the kernels of a pass alternate between the handle's stream and a second
+    // one, so that each is started while its producer still runs, asks for its weights and waits for a flag.
+    bool overlap = false;
+    hipStream_t ov_stream = nullptr;
+    hipEvent_t ov_fork = nullptr, ov_join = nullptr;
+    unsigned* ov_slots = nullptr;  // OV_SLOTS hand-over slots, used round robin
+    unsigned ov_epoch = 0;         // the epoch of the last producer launch (one counter for all slots)
+    unsigned ov_launches = 0;
+    int* ov_err = nullptr;         // pinned host memory the kernels can write
     uint16_t* q16 = nullptr;
     float *part_o = nullptr, *part_ml = nullptr;
     int nch = 0;
@@ -482,88 +478,10 @@ int launch_pass(tsv_ctx* c, int m) {
     int prev_splits = 0;
     const float* prev_partial = c->partial;
     const float* prev_weights = nullptr;  // routed experts: the factors of the per-slot outputs
-    float *x = c->x, *x_other = c->x2;  // the fused kernels write the residual rows to the other buffer
+    float* x = c->x;
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
-    // the attention half as one per-XCD kernel: passes of at most eight rows and 32 (row, q head) pairs
-    const bool attn_block = c->fused_attn && !c->kv_k_bits && m <= 8 && m * (c->nq / c->nkv) <= 32;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
-        int attn_splits = 0;  // partial sums the attention half leaves for the FFN norm
-        const float* attn_partial = c->partial;
-        if (attn_block && !prev_weights) {
-            AttnBlockArgs ba{};
-            ba.sync.rank_ctr = c->rank_ctr;
-            ba.sync.bar_ctr = c->bar_ctr;
-            ba.sync.err = c->fused_err;
-            ba.sync.bar_base = c->bar_count;
-            c->bar_count += 32u * (unsigned)attn_block_barriers();
-            ba.x_in = x;
-            ba.x_out = x_other;
-            ba.partial = prev_partial;
-            ba.n_partials = prev_splits;
-            ba.bias_in = nullptr;
-            ba.norm_w = L.attn_norm;
-            ba.frag = c->frag8;
-            ba.frag_stride = c->frag8_stride;
-            ba.ssq = c->ssq8;
-            ba.hidden = c->hidden;
-            ba.eps = c->eps;
-            ba.m = m;
-            ba.w_qkv = L.qkv.tiles;
-            ba.qkv_kchunks = L.qkv.kchunks;
-            ba.rope.cs = c->rope_cs;
-            ba.rope.bias = L.bqkv;
-            ba.rope.q16 = c->q16;
-            ba.rope.kc = L.kc;
-            ba.rope.vc = L.vc;
-            ba.rope.nq = c->nq;
-            ba.rope.nkv = c->nkv;
-            ba.rope.hd = c->hd;
-            ba.rope.max_ctx = L.cap;
-            ba.vp = c->vp_dev;
-            ba.attn.q16 = c->q16;
-            ba.attn.kc = L.kc;
-            ba.attn.vc = L.vc;
-            ba.attn.part_o = c->part_o;
-            ba.attn.part_ml = c->part_ml;
-            ba.attn.xfrag = c->xf_b;
-            ba.attn.nq = c->nq;
-            ba.attn.nkv = c->nkv;
-            ba.attn.hd = c->hd;
-            ba.attn.max_ctx = L.cap;
-            ba.attn.nch = c->nch;
-            ba.attn.scale = c->attn_scale;
-            ba.attn.window = 0;
-            ba.attn.sinks = nullptr;
-            ba.attn.vp = c->vp_dev;
-            ba.attn.m_hint = m;
-            ba.attn.base_hint = c->vp_host->base;
-            ba.w_o = L.wo.tiles;
-            ba.wo_tiles = L.wo.n_tiles;
-            ba.wo_kchunks = L.wo.kchunks;
-            ba.partial_out = c->partial8a;
-            ba.stages = c->attn_stages;
-            {
-                PROF(PC_ATTN);
-                rc = launch_attn_block(s, L.qkv.fmt, ba);
-            }
-            if (rc) return rc;
-            std::swap(x, x_other);
-            attn_splits = 8;
-            attn_partial = c->partial8a;
-            if (c->attn_stages < 5) {  // the remaining stages as separate kernels
-                if (c->attn_stages < 4) {
-                    AttnArgs aa = ba.attn;
-                    aa.nch = c->nch;
-                    if ((rc = c->attn_stages == 3 ? launch_attention_merge(s, aa, m) : launch_attention(s, aa, m))) return rc;
-                }
-                attn_splits = splits_for(L.wo, m, EPI_PARTIAL);
-                attn_partial = c->partial;
-                if ((rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, attn_splits, EPI_PARTIAL, c->hidden, c->hidden)))
-                    return rc;
-            }
-        }
-        if (!attn_splits) {
         {
             PROF(PC_NORM);
             rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, c->xf_a, m,
@@ -686,50 +604,10 @@ int launch_pass(tsv_ctx* c, int m) {
             for (int rep = 0; rep < c->repeat[PC_WO] && !rc; rep++) rc = launch_gemm(s, L.wo, c->xf_b, c->partial, c->vp_dev, m, sp, EPI_PARTIAL, c->hidden, c->hidden);
         }
         if (rc) return rc;
-        attn_splits = sp;
-        }  // the separate kernels of the attention half
-        int sp = attn_splits;
-        if (c->fused_ffn) {
-            FfnBlockArgs fa{};
-            fa.sync.rank_ctr = c->rank_ctr;
-            fa.sync.bar_ctr = c->bar_ctr;
-            fa.sync.err = c->fused_err;
-            fa.sync.bar_base = c->bar_count;
-            c->bar_count += 32u * (unsigned)fused_ffn_barriers();
-            fa.norm.x_in = x;
-            fa.norm.x_out = x_other;
-            fa.norm.partial = attn_partial;
-            fa.norm.n_partials = sp;
-            fa.norm.norm_w = L.ffn_norm;
-            fa.norm.frag = c->frag8;
-            fa.norm.frag_stride = c->frag8_stride;
-            fa.norm.ssq = c->ssq8;
-            fa.norm.hidden = c->hidden;
-            fa.norm.eps = c->eps;
-            fa.m = m;
-            fa.w_gate_up = L.gate_up.tiles;
-            fa.gu_tiles = L.gate_up.n_tiles;
-            fa.gu_kchunks = L.gate_up.kchunks;
-            fa.frag_c = c->xf_c;
-            fa.ffn = c->ffn;
-            fa.w_down = L.down.tiles;
-            fa.down_tiles = L.down.n_tiles;
-            fa.down_kchunks = L.down.kchunks;
-            fa.partial_out = c->partial8;
-            {
-                PROF(PC_GATEUP);
-                rc = launch_ffn_block(s, L.gate_up.fmt, fa, m);
-            }
-            if (rc) return rc;
-            std::swap(x, x_other);
-            prev_partial = c->partial8;
-            prev_splits = 8;
-            continue;
-        }
         {
             PROF(PC_NORM);
             const bool fp4 = L.n_experts && c->moe_fp4_terms;
-            rc = launch_addnorm(s, x, attn_partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo,
+            rc = launch_addnorm(s, x, c->partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, c->xf_a, m, nullptr, L.bo,
                                 fp4 ? &c->x8_h : nullptr, c->moe_fp4_terms);
         }
         if (rc) return rc;
@@ -1032,15 +910,15 @@ int run_pass(tsv_ctx* c, int m) {
     return TSV_OK;
 }
 
-// After a stream synchronisation: did a fused kernel give up on a barrier?  Its results are then
-// incomplete; the handle switches to the unfused kernels for good and reports the failure.
-int check_fused(tsv_ctx* c) {
-    if (!c->fused_err || *c->fused_err == 0) return TSV_OK;
-    set_error(*c->fused_err == 2 ? "fused layer kernel: unexpected XCD id; fused path disabled, repeat the call"
-                                 : "fused layer kernel: XCD barrier timed out; fused path disabled, repeat the call");
-    *c->fused_err = 0;
-    c->fused_ffn = false;
-    c->fused_attn = false;
+// After a stream synchronisation: did a kernel of an overlapped pass give up waiting for its producer
+// (handoff.h)?  Its results are then garbage; the handle goes back to ordered launches for good and
+// reports the failure.
+int check_overlap(tsv_ctx* c) {
+    if (!c->ov_err || *c->ov_err == 0) return TSV_OK;
+    set_error("verify: a kernel of an overlapped pass waited for its producer in vain; overlapped passes are switched "
+              "off for this handle, repeat the call");
+    *c->ov_err = 0;
+    c->overlap = false;
     return TSV_ERR_DEVICE;
 }
 
@@ -1048,7 +926,7 @@ int finish_verify(tsv_ctx* c, int m, uint16_t* logits_out) {
     if (logits_out) {
         TSV_HIP(hipMemcpyAsync(logits_out, c->logits, (size_t)m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
         TSV_HIP(hipStreamSynchronize(c->stream));
-        return check_fused(c);
+        return check_overlap(c);
     }
     return TSV_OK;
 }
@@ -1423,44 +1301,6 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (rc = dev_alloc(c, &c->sc.tcount, (size_t)32 * 65536 * 4, true)) ||
         (rc = dev_alloc(c, &c->sc.result, sizeof(AcceptResult), true)))
         return fail(rc);
-    {
-        // per-XCD fused kernels: every layer must fit their sharding; they need all 256
-        // workgroups resident at once (cooperative launch) and a fresh barrier base per launch
-        // (so not inside a captured graph)
-        // Opt-in (TSV_FUSED=1): at the 8B shape the fused FFN block measured 36-42 us per layer
-        // against 31 us for the three separate kernels -- the block is bandwidth-bound, and its
-        // early bulk prefetch delays the small loads of the RMSNorm stage.
-        const char* fe = getenv("TSV_FUSED");
-        const char* fa = getenv("TSV_FUSED_ATTN");
-        int ncu = 0;
-        if (hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, 0) != hipSuccess) ncu = 0;
-        bool ok = !c->use_graph && fe && fe[0] == '1' && ncu == 256;
-        // the attention half of a layer as one kernel (attn_block.hip)
-        bool ok_attn = !c->use_graph && fa && fa[0] == '1' && ncu == 256;
-        for (const LayerW& L : c->layers) {
-            ok = ok && L.n_experts == 0 && fused_ffn_supported(L.gate_up, L.down, c->hidden, c->ffn);
-            ok_attn = ok_attn && L.n_experts == 0 && !L.v_only.tiles && !L.sinks && L.window == 0 &&
-                      attn_block_supported(L.qkv, L.wo, c->hidden, c->nq, c->nkv, c->hd, L.rope_fused);
-        }
-        c->fused_attn = ok_attn;
-        if (const char* e = getenv("TSV_FUSED_ATTN_STAGES")) c->attn_stages = std::max(2, std::min(5, atoi(e)));
-        if (ok_attn && (rc = dev_alloc(c, &c->partial8a, (size_t)8 * 16 * c->hidden * 4, true))) return fail(rc);
-        if (ok || ok_attn) {
-            c->frag8_stride = (xfrag_bytes(c->hidden) + 255) & ~(size_t)255;
-            if ((rc = dev_alloc(c, &c->x2, (size_t)16 * c->hidden * 4, true)) ||
-                (rc = dev_alloc(c, &c->frag8, 8 * c->frag8_stride, true)) ||
-                (rc = dev_alloc(c, &c->ssq8, (size_t)8 * 16 * 32 * 4, true)) ||
-                (rc = dev_alloc(c, &c->partial8, (size_t)8 * 16 * c->hidden * 4, true)) ||
-                (rc = dev_alloc(c, &c->rank_ctr, 8 * 64 * 4, true)) || (rc = dev_alloc(c, &c->bar_ctr, 8 * 64 * 4, true)))
-                return fail(rc);
-            if (hipHostMalloc((void**)&c->fused_err, sizeof(int)) != hipSuccess) {
-                set_error("open: pinned host allocation failed");
-                return fail(TSV_ERR_DEVICE);
-            }
-            *c->fused_err = 0;
-            c->fused_ffn = ok;
-        }
-    }
     if (c->route_forced && hipMemsetAsync(c->route_forced, 0xFF, (size_t)c->n_layers * 16 * 8 * 4, c->stream) != hipSuccess)
         return fail(TSV_ERR_DEVICE);  // every entry -1: rows route freely until tsv_force_route says otherwise
     if (hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
@@ -1475,7 +1315,7 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         return fail(TSV_ERR_DEVICE);
     }
     // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
-    c->wide.ok = c->rewind_budget == INT64_MAX && !c->fused_ffn && !c->fused_attn;
+    c->wide.ok = c->rewind_budget == INT64_MAX;
     for (const LayerW& L : c->layers)
         if (L.n_experts || !L.rope_fused || L.v_only.tiles || L.qkv.fmt != FMT_Q4K || L.wo.fmt != FMT_Q4K ||
             L.gate_up.fmt != FMT_Q4K || L.down.fmt != FMT_Q4K)
@@ -1495,7 +1335,10 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
-    if (c->fused_err) (void)hipHostFree(c->fused_err);
+    if (c->ov_err) (void)hipHostFree(c->ov_err);
+    if (c->ov_stream) (void)hipStreamDestroy(c->ov_stream);
+    for (hipEvent_t e : {c->ov_fork, c->ov_join})
+        if (e) (void)hipEventDestroy(e);
     for (hipGraphExec_t g : c->pass_graph)
         if (g) (void)hipGraphExecDestroy(g);
     for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
@@ -1694,7 +1537,7 @@ static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos
         i += m;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
-    return check_fused(c);
+    return check_overlap(c);
 }
 
 extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
@@ -1825,7 +1668,7 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
         return TSV_ERR_INVALID;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
-    if (int frc = check_fused(c)) return frc;  // rows a fused kernel gave up on must not be gathered
+    if (int frc = check_overlap(c)) return frc;  // rows of a pass that gave up must not be gathered
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
     int rc = launch_kv_gather(c->stream, c->kv_ptrs, c->kv_caps, c->n_layers, c->nkv, c->hd, c->tok_dev + 32, n, (int)base);
@@ -1975,7 +1818,7 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     if (r->logits_out)
         TSV_HIP(hipMemcpyAsync(r->logits_out, c->logits, (size_t)r->m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipStreamSynchronize(c->stream));
-    if ((rc = check_fused(c))) return rc;
+    if ((rc = check_overlap(c))) return rc;
     const AcceptResult& a = *c->res_host;
     if (a.error) {
         set_error(std::string("accept: ") + accept_error_text(a.error));
@@ -2703,5 +2546,137 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
     (void)hipStreamSynchronize(c->stream);
     for (void* p : c->allocs) (void)hipFree(p);
     (void)hipStreamDestroy(c->stream);
+    return rc;
+}
+
+// Measurement hook: `iters` times the FFN pair of a dense layer -- gate/up with the silu-mul
+// epilogue over a (2 ffn) x hidden weight, then down over a hidden x ffn weight, m activation rows,
+// both Q4_K, `rotate` weight copies cycled so the bytes come from HBM -- as a dependent chain
+// (every launch consumes what the one before it wrote).  mode 0: ordered launches on one stream, plain
+// kernels.  mode 1: ordered launches on one stream with the hand-over kernels (what coherent stores,
+// loads and the flags cost by themselves).  mode 2: the launches alternate between two streams
+// and every kernel waits for its producer's flag after asking for its first weight tiles (handoff.h).
+// Reports the average microseconds per pair.
+extern "C" int32_t tsv_ffn_pair_time(int64_t hidden, int64_t ffn, int32_t m, int32_t mode, int32_t iters, int32_t rotate,
+                                     float* avg_us) {
+    if (hidden % 256 || ffn % 256 || m < 1 || m > 8 || mode < 0 || mode > 2 || iters < 1 || rotate < 1 || !avg_us) {
+        set_error("ffn_pair_time: bad argument");
+        return TSV_ERR_INVALID;
+    }
+    tsv_ctx tmp;
+    tsv_ctx* c = &tmp;
+    hipStream_t s2 = nullptr;
+    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    TSV_HIP(hipStreamCreateWithFlags(&s2, hipStreamNonBlocking));
+    TiledW gu, dn;
+    gu.fmt = dn.fmt = FMT_Q4K;
+    gu.k = (int)hidden;
+    gu.kchunks = gu.k / 256;
+    gu.n_rows = (int)(2 * ffn);
+    gu.n_tiles = gu.n_rows / TILE_ROWS;
+    gu.bytes = (size_t)gu.n_tiles * gu.kchunks * 9216;
+    dn.k = (int)ffn;
+    dn.kchunks = dn.k / 256;
+    dn.n_rows = (int)hidden;
+    dn.n_tiles = dn.n_rows / TILE_ROWS;
+    dn.bytes = (size_t)dn.n_tiles * dn.kchunks * 9216;
+    std::vector<uint8_t*> gu_c((size_t)rotate), dn_c((size_t)rotate);
+    int rc = TSV_OK;
+    {
+        std::vector<uint8_t> host(std::max(gu.bytes, dn.bytes));
+        uint64_t sd = 88172645463325252ull;
+        for (size_t i = 0; i < host.size(); i += 8) {
+            sd ^= sd << 13;
+            sd ^= sd >> 7;
+            sd ^= sd << 17;
+            std::memcpy(&host[i], &sd, std::min<size_t>(8, host.size() - i));
+        }
+        for (size_t t = 0; t < host.size() / 9216; t++)  // small fp16 scales
+            for (int r = 0; r < 64; r++) host[t * 9216 + 8192 + r * 16 + 1] = host[t * 9216 + 8192 + r * 16 + 3] = 0x10;
+        for (int i = 0; i < rotate && !rc; i++) {
+            if (!(rc = dev_alloc(c, &gu_c[i], gu.bytes)) && !(rc = dev_alloc(c, &dn_c[i], dn.bytes)) &&
+                (hipMemcpy(gu_c[i], host.data(), gu.bytes, hipMemcpyHostToDevice) != hipSuccess ||
+                 hipMemcpy(dn_c[i], host.data(), dn.bytes, hipMemcpyHostToDevice) != hipSuccess))
+                rc = TSV_ERR_DEVICE;
+        }
+    }
+    VerifyParams vp;
+    std::memset(&vp, 0, sizeof vp);
+    vp.m = m;
+    uint4 *xf_a = nullptr, *xf_c = nullptr;
+    float* partial = nullptr;
+    VerifyParams* vpd = nullptr;
+    unsigned* slots = nullptr;
+    int* err = nullptr;
+    const int sp = gemm_default_splits(dn, m);
+    if (!rc) rc = dev_alloc(c, &xf_a, xfrag_bytes((int)hidden), true);
+    if (!rc) rc = dev_alloc(c, &xf_c, xfrag_bytes((int)ffn), true);
+    if (!rc) rc = dev_alloc(c, &partial, (size_t)sp * 16 * hidden * 4, true);
+    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
+    if (!rc) rc = dev_alloc(c, &slots, (size_t)4 * HANDOFF_SLOT_WORDS * 4, true);
+    if (!rc && hipHostMalloc((void**)&err, sizeof(int)) != hipSuccess) rc = TSV_ERR_DEVICE;
+    if (!rc) *err = 0;
+    if (!rc && hipMemcpy(vpd, &vp, sizeof vp, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
+    hipEvent_t e0 = nullptr, e1 = nullptr, ej = nullptr;
+    if (!rc && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess ||
+                hipEventCreateWithFlags(&ej, hipEventDisableTiming) != hipSuccess))
+        rc = TSV_ERR_DEVICE;
+    unsigned epoch = 0, launches = 0;
+    for (int pass = 0; pass < 2 && !rc; pass++) {  // pass 0 warms up
+        if (hipStreamSynchronize(c->stream) != hipSuccess || hipStreamSynchronize(s2) != hipSuccess) rc = TSV_ERR_DEVICE;
+        if (pass == 1) (void)hipEventRecord(e0, c->stream);
+        if (mode == 2) {
+            (void)hipEventRecord(ej, c->stream);
+            (void)hipStreamWaitEvent(s2, ej, 0);
+        }
+        const int n = pass ? iters : std::min(iters, 3);
+        for (int i = 0; i < 2 * n && !rc; i++) {
+            Handoff h{};
+            if (mode) {
+                if (launches) {
+                    h.wait = slots + (size_t)((launches - 1) & 3) * HANDOFF_SLOT_WORDS;
+                    h.wait_epoch = epoch;
+                }
+                h.sig = slots + (size_t)(launches & 3) * HANDOFF_SLOT_WORDS;
+                h.sig_epoch = ++epoch;
+                h.err = err;
+                launches++;
+            }
+            hipStream_t s = mode == 2 && (i & 1) ? s2 : c->stream;
+            if (i & 1) {
+                dn.tiles = dn_c[(size_t)((i / 2) % rotate)];
+                rc = launch_gemm(s, dn, xf_c, partial, vpd, m, sp, EPI_PARTIAL, (int)hidden, (int)hidden, nullptr, mode ? &h : nullptr);
+            } else {
+                gu.tiles = gu_c[(size_t)((i / 2) % rotate)];
+                rc = launch_gemm(s, gu, xf_a, xf_c, vpd, m, 1, EPI_SILU, 0, 0, nullptr, mode ? &h : nullptr);
+            }
+        }
+        if (mode == 2) {
+            (void)hipEventRecord(ej, s2);
+            (void)hipStreamWaitEvent(c->stream, ej, 0);
+        }
+        if (pass == 1) (void)hipEventRecord(e1, c->stream);
+    }
+    if (!rc) {
+        if (hipStreamSynchronize(c->stream) != hipSuccess || hipStreamSynchronize(s2) != hipSuccess) {
+            set_error("ffn_pair_time: device execution failed");
+            rc = TSV_ERR_DEVICE;
+        } else if (*err) {
+            set_error("ffn_pair_time: a hand-over wait ran out");
+            rc = TSV_ERR_DEVICE;
+        } else {
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            *avg_us = ms * 1000.f / (float)iters;
+        }
+    }
+    for (hipEvent_t e : {e0, e1, ej})
+        if (e) (void)hipEventDestroy(e);
+    (void)hipStreamSynchronize(c->stream);
+    (void)hipStreamSynchronize(s2);
+    for (void* p : c->allocs) (void)hipFree(p);
+    if (err) (void)hipHostFree(err);
+    (void)hipStreamDestroy(c->stream);
+    (void)hipStreamDestroy(s2);
     return rc;
 }

@@ -8,6 +8,7 @@
 
 #include "../../include/tsverify.h"
 #include "../../include/tsverify_testing.h"
+#include "handoff.h"
 
 namespace tsv {
 
@@ -149,6 +150,7 @@ struct GemmArgs {
     int n_tiles, kchunks, kslice, splits, kparts, per, ldo, n_valid;
     int out16;     // EPI_SILU: write the fragments in the prompt kernel's layout (frag16_index)
     RopeEpi rope;  // EPI_ROPE only
+    Handoff h;     // wait / sig non-null: the launch overlaps its neighbours in the pass (handoff.h)
 };
 
 // Re-tiles n_rows GGUF rows of `raw` into `tiles`; source row r lands in tiled row
@@ -157,7 +159,7 @@ struct GemmArgs {
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
                   int kchunks, int grp, int stride, int offset, const int32_t* rowmap = nullptr);
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
-                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
+                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr, const Handoff* h = nullptr);
 int gemm_default_splits(const TiledW& w, int m);
 // rows of a prompt-block pass, and the matmul over them in blocks of sixteen (Q4_K weights only)
 int gemm_wide_rows();
@@ -228,53 +230,6 @@ int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 // the same two matmuls on v_mfma_scale_f32_16x16x128_f8f6f4 (moe_fp4.hip)
 int launch_moe_fp4_gate_up(hipStream_t s, const MoeGemmArgs& a, int n_groups);
 int launch_moe_fp4_down(hipStream_t s, const MoeGemmArgs& a, int n_groups);
-
-// ---- per-XCD fused layer kernels ----------------------------------------------------------
-// Counters of the XCD-local barriers.  rank_ctr / bar_ctr: one word per XCD, 64 words apart.
-// A launch that uses n barriers advances every bar_ctr by 32 * n; bar_base is its value before.
-struct FusedSync {
-    unsigned* rank_ctr;
-    unsigned* bar_ctr;
-    int* err;  // host-visible: 1 = a barrier timed out, 2 = unexpected XCD id
-    unsigned bar_base;
-};
-// Residual add + RMSNorm inputs stage shared by the fused kernels.
-struct NormStage {
-    const float* x_in;     // [16][hidden]
-    float* x_out;          // a different buffer: other XCDs may still be reading x_in
-    const float* partial;  // [n_partials][16][hidden] partial sums to add (n_partials <= 8)
-    int n_partials;
-    const float* norm_w;
-    uint8_t* frag;         // 8 private copies of the activation fragments, frag_stride bytes apart
-    size_t frag_stride;
-    float* ssq;            // [8][16][32] sums of squares per workgroup
-    int hidden;
-    float eps;
-};
-struct FfnBlockArgs {
-    FusedSync sync;
-    NormStage norm;
-    int m;  // rows of the pass
-    const uint8_t* w_gate_up;
-    int gu_tiles, gu_kchunks;
-    uint4* frag_c;  // silu(gate) * up as fragments, K = ffn
-    int ffn;
-    const uint8_t* w_down;
-    int down_tiles, down_kchunks;
-    float* partial_out;  // [8][16][hidden]
-};
-// The per-XCD fused kernels are an experiment that measured slower than the separate kernels they
-// replace; they are compiled only when the library is built with TSV_WITH_FUSED (build.py:
-// TSV_BUILD_FUSED=1) and are opt-in at run time even then.
-#ifdef TSV_WITH_FUSED
-bool fused_ffn_supported(const TiledW& gate_up, const TiledW& down, int hidden, int ffn);
-int fused_ffn_barriers();
-int launch_ffn_block(hipStream_t s, int fmt, FfnBlockArgs& a, int m);
-#else
-inline bool fused_ffn_supported(const TiledW&, const TiledW&, int, int) { return false; }
-inline int fused_ffn_barriers() { return 0; }
-inline int launch_ffn_block(hipStream_t, int, FfnBlockArgs&, int) { return TSV_ERR_UNSUPPORTED; }
-#endif
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
                  const VerifyParams* vp, int m, const float* freqs = nullptr, float mscale = 1.0f, int half = 0,
@@ -415,47 +370,6 @@ size_t tq_kq_bytes(int nkv, int cap, int hd, int k_bits);
 size_t tq_vq_bytes(int nkv, int cap, int hd, int v_bits);
 int launch_attention_merge(hipStream_t s, const AttnArgs& a, int m);
 int attn_chunks(int nkv);
-
-// The attention half of a layer as one per-XCD kernel (attn_block.hip): residual add + RMSNorm
-// inputs, the q/k/v projection with its rotating epilogue, split-KV attention, the merge of the chunk
-// partials and the output projection; leaves one partial sum of the output projection per XCD.
-struct AttnBlockArgs {
-    FusedSync sync;
-    // residual add + norm inputs
-    const float* x_in;     // [16][hidden]
-    float* x_out;          // a different buffer: other XCDs may still be reading x_in
-    const float* partial;  // [n_partials][16][hidden] partial sums to add (n_partials <= 8)
-    int n_partials;
-    const float* bias_in;  // nullable: hidden values added with the partial sums
-    const float* norm_w;
-    uint8_t* frag;         // 8 private copies of the activation fragments, frag_stride bytes apart
-    size_t frag_stride;
-    float* ssq;            // [8][16][32] sums of squares per norm workgroup
-    int hidden;
-    float eps;
-    int m;
-    // q/k/v projection (the fused matrix of the rotating epilogue)
-    const uint8_t* w_qkv;
-    int qkv_kchunks;
-    RopeEpi rope;
-    const VerifyParams* vp;
-    // attention: q16, caches, partials, the output projection's input fragments, nch == 32
-    AttnArgs attn;
-    // output projection
-    const uint8_t* w_o;
-    int wo_tiles, wo_kchunks;
-    float* partial_out;  // [8][16][hidden]
-    int stages;          // 5: everything; 2: stop after the projection; 3: after attention; 4: after the merge
-};
-#ifdef TSV_WITH_FUSED
-bool attn_block_supported(const TiledW& qkv, const TiledW& wo, int hidden, int nq, int nkv, int hd, bool rope_fused);
-int attn_block_barriers();
-int launch_attn_block(hipStream_t s, int fmt, const AttnBlockArgs& a);
-#else
-inline bool attn_block_supported(const TiledW&, const TiledW&, int, int, int, int, bool) { return false; }
-inline int attn_block_barriers() { return 0; }
-inline int launch_attn_block(hipStream_t, int, const AttnBlockArgs&) { return TSV_ERR_UNSUPPORTED; }
-#endif
 
 int launch_kv_gather(hipStream_t s, uint16_t* const* caches_dev, const int32_t* caps_dev, int n_layers, int nkv, int hd,
                      const int32_t* path_dev, int n, int base);

@@ -21,8 +21,8 @@ CONFIGS = {
     "small_q5_k_m": dict(n_layers=2, hidden=512, n_q_heads=4, n_kv_heads=1, head_dim=128, ffn=1536,
                          vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q5_K,
                          overrides={(1, "wv"): ffi.Q6_K, (1, "w_down"): ffi.Q6_K, "lm_head": ffi.Q6_K}),
-    # the smallest shapes the per-XCD fused layer kernels take (8 KV heads, widths divisible
-    # into eight chunk-aligned slices); norm weights are not all ones here
+    # eight KV heads of 64-wide heads (the group sizes 4 and 2), widths that split into eight
+    # chunk-aligned slices; norm weights are not all ones here
     "xcd_q4_k": dict(n_layers=2, hidden=1024, n_q_heads=32, n_kv_heads=8, head_dim=64, ffn=2048,
                      vocab=4096, rms_eps=1e-5, rope_theta=500000.0, dtype=ffi.Q4_K, norm_jitter=0.25),
     "xcd_q8_0": dict(n_layers=2, hidden=1024, n_q_heads=16, n_kv_heads=8, head_dim=64, ffn=1024,
