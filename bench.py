@@ -289,9 +289,6 @@ def main():
     ap.add_argument("--prefill-bench", type=int, default=0, metavar="TOKENS",
                     help="time tsv_prefill over a prompt of this many tokens (after one untimed run of the same), print one "
                          "JSON line and exit")
-    ap.add_argument("--ffn-pair-probe", action="store_true",
-                    help="time the gate/up + down pair of the headline shape as ordered launches, as ordered launches of "
-                         "the flag hand-over kernels, and overlapped on two streams; print one JSON line and exit")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -321,14 +318,6 @@ def main():
         return
     if args.step_traffic:
         step_traffic(*args.step_traffic, args.trace_from)
-        return
-    if args.ffn_pair_probe:
-        from turbospark_amd import ffi
-        out = {}
-        for rep in range(2):
-            for mode, name in enumerate(("ordered_plain_us", "ordered_handover_us", "overlapped_two_streams_us")):
-                out.setdefault(name, []).append(round(ffi.ffn_pair_time(4096, 14336, 5, mode), 2))
-        print(json.dumps({"probe": "gate/up (28672 x 4096) + down (4096 x 14336), Q4_K, M = 5, chain of 64 pairs"} | out))
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the verify step on ONE GPU; --gpus N with N > 1 is not "

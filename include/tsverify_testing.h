@@ -62,13 +62,6 @@ int32_t tsv_set_repeat(tsv_ctx* ctx, int32_t profile_class, int32_t times);
 int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
                         int32_t iters, int32_t rotate, float* avg_us);
 
-/* Measurement hook (no reference counterpart): average microseconds of one gate/up + down pair of a dense
- * Q4_K layer (hidden, ffn, m rows) in a dependent chain of `iters` pairs.  mode 0: ordered launches, plain
- * kernels; 1: ordered launches of the kernels that hand over through flags and device-coherent stores;
- * 2: those kernels alternating between two streams, each started while its producer runs. */
-int32_t tsv_ffn_pair_time(int64_t hidden, int64_t ffn, int32_t m, int32_t mode, int32_t iters, int32_t rotate,
-                          float* avg_us);
-
 /* Measurement hook: average duration of `iters` launches of a plain device-to-device copy kernel
  * over `bytes` bytes (read once, written once).  It is the copy kernel of known size that HBM
  * traffic counters are scaled against, and the streaming rate the part actually reaches. */

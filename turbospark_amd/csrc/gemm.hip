@@ -246,11 +246,10 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
 }
 
 // Stores one row group's finished sums.  v[i] is output column n of activation row 4g+i.
-// (COH: the results go to a kernel that runs at the same time as this one -- device-coherent stores)
-template <int EPI, bool COH>
+template <int EPI>
 __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split, int g, float4v v, int lane, int M) {
     if (EPI == EPI_ROPE) {
-        rope_epilogue<COH>(a.rope, a.vp, tile, g, v, lane, M);
+        rope_epilogue(a.rope, a.vp, tile, g, v, lane, M);
         return;
     }
     if (EPI == EPI_SILU) {
@@ -270,13 +269,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split,
             for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
             const int b = 4 * g + i;
             if (b < M && lane < 32) {
-                if (COH) {
-                    coh_store_f16(out + frag_index(col, b), h);
-                    if (lane == 0) coh_store_f32(sums + xsum_index(col >> 5, b), sum);
-                } else {
-                    out[frag_index(col, b)] = h;
-                    if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
-                }
+                out[frag_index(col, b)] = h;
+                if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
             }
         }
         return;
@@ -287,11 +281,9 @@ __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split,
     for (int i = 0; i < 4; i++) {
         const int b = 4 * g + i;
         if (b >= M) continue;
-        if (EPI == EPI_PARTIAL) {
-            float* o = (float*)a.out + ((size_t)split * 16 + b) * a.ldo + n;
-            if (COH) coh_store_f32(o, v[i]);
-            else *o = v[i];
-        } else
+        if (EPI == EPI_PARTIAL)
+            ((float*)a.out)[((size_t)split * 16 + b) * a.ldo + n] = v[i];
+        else
             ((_Float16*)a.out)[(size_t)b * a.ldo + n] = (_Float16)v[i];
     }
 }
@@ -305,26 +297,10 @@ __device__ __forceinline__ void epilogue(const GemmArgs& a, int tile, int split,
 #define TSV_GEMM_STAGES 1
 #endif
 
-// OVL: the launch overlaps its producer (handoff.h).  The wave asks for the weights of its first
-// OVL_STAGES tiles, which depend on nobody, waits for the producer, and only then reads activations
-// (device-coherently, like everything else another kernel of the same pass wrote); its own results
-// are stored device-coherently and the workgroup counts itself into the slot of its consumer.
-#ifndef OVL_STAGES_N
-#define OVL_STAGES_N 2
-#endif
-constexpr int OVL_STAGES = OVL_STAGES_N;
-
-template <class F, int EPI, int NG, bool OVL>
+template <class F, int EPI, int NG>
 __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     extern __shared__ float4v red[];
-    constexpr int STAGES = OVL ? OVL_STAGES : TSV_GEMM_STAGES;
-#if defined(OVL_PLAIN_ST)
-    constexpr bool OVL_ST = false;
-#elif defined(OVL_ST_ONLY)
-    constexpr bool OVL_ST = OVL && EPI == OVL_ST_ONLY;
-#else
-    constexpr bool OVL_ST = OVL;
-#endif
+    constexpr int STAGES = TSV_GEMM_STAGES;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
     // this wave's run of chunks inside the workgroup's K slice
@@ -346,32 +322,13 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
     // Software pipeline over the K chunks, STAGES tiles in flight per wave.  Every load in the
     // steady state is unconditional (straight-line code), so the compiler can wait on the oldest
     // outstanding tile only (s_waitcnt vmcnt(n)) instead of draining the queue.
-    Stage<F, NG> st[STAGES];
-#ifdef OVL_PLAIN_X
-    const ActLoader<false> x(a.xfrag, a.xsum, lane);
-#else
-    const ActLoader<OVL> x(a.xfrag, a.xsum, lane);
-#endif
-    const int last = max(c0 + nc - 1, c0);
-    auto fetch = [&](Stage<F, NG>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
-    if (OVL) {
-        // (a wave without chunks asks for a tile all the same: the loads are cheap, a branch around
-        // them would make every later wait a full one)
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < STAGES; s++) F::load(st[s].w, wt + (size_t)min(min(c0 + s, last), a.kchunks - 1) * F::TILE_BYTES, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        handoff_wait(a.h);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < STAGES; s++) load_x(st[s].x, x, min(min(c0 + s, last), a.kchunks - 1), lane);
-        __builtin_amdgcn_sched_barrier(0);
-    }
     if (nc > 0) {
-        if (!OVL) {
+        Stage<F, NG> st[STAGES];
+        const ActLoader<false> x(a.xfrag, a.xsum, lane);
+        const int last = c0 + nc - 1;
+        auto fetch = [&](Stage<F, NG>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
 #pragma unroll
-            for (int s = 0; s < STAGES; s++) fetch(st[s], min(c0 + s, last));
-        }
+        for (int s = 0; s < STAGES; s++) fetch(st[s], min(c0 + s, last));
         int c = 0;
         for (; c + 2 * STAGES <= nc; c += STAGES) {
 #pragma unroll
@@ -396,21 +353,18 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs a) {
 
     if (a.kparts == 1) {
 #pragma unroll
-        for (int g = 0; g < NG; g++) epilogue<EPI, OVL_ST>(a, tile, split, g, acc[g], lane, M);
-    } else {
-        // fold the waves' accumulators in wave order; wave w finishes row groups w, w + kparts, ...
-#pragma unroll
-        for (int g = 0; g < NG; g++) red[(wave * NG + g) * 64 + lane] = acc[g];
-        __syncthreads();
-        for (int g = wave; g < NG; g += a.kparts) {
-            float4v v = red[g * 64 + lane];
-            for (int w = 1; w < a.kparts; w++) v += red[(w * NG + g) * 64 + lane];
-            epilogue<EPI, OVL_ST>(a, tile, split, g, v, lane, M);
-        }
+        for (int g = 0; g < NG; g++) epilogue<EPI>(a, tile, split, g, acc[g], lane, M);
+        return;
     }
-#ifndef OVL_NO_SIGNAL
-    if (OVL) handoff_signal(a.h);
-#endif
+    // fold the waves' accumulators in wave order; wave w finishes row groups w, w + kparts, ...
+#pragma unroll
+    for (int g = 0; g < NG; g++) red[(wave * NG + g) * 64 + lane] = acc[g];
+    __syncthreads();
+    for (int g = wave; g < NG; g += a.kparts) {
+        float4v v = red[g * 64 + lane];
+        for (int w = 1; w < a.kparts; w++) v += red[(w * NG + g) * 64 + lane];
+        epilogue<EPI>(a, tile, split, g, v, lane, M);
+    }
 }
 
 // ------------------------------------------------------------------------------- nine to sixteen rows
@@ -894,15 +848,7 @@ int gemm_default_splits(const TiledW& w, int) {
 template <class F, int EPI, int NG>
 static int launch_t(hipStream_t s, const GemmArgs& a) {
     const size_t lds = a.kparts > 1 ? (size_t)a.kparts * NG * 1024 : 0;
-    if (a.h.wait || a.h.sig) {
-        if (EPI == EPI_LOGITS) {
-            set_error("matmul: the logits epilogue has no overlapped form");
-            return TSV_ERR_UNSUPPORTED;
-        }
-        hipLaunchKernelGGL((k_gemm<F, EPI == EPI_LOGITS ? EPI_PARTIAL : EPI, NG, true>), dim3(a.n_tiles * a.splits),
-                           dim3(64 * a.kparts), lds, s, a);
-    } else
-        hipLaunchKernelGGL((k_gemm<F, EPI, NG, false>), dim3(a.n_tiles * a.splits), dim3(64 * a.kparts), lds, s, a);
+    hipLaunchKernelGGL((k_gemm<F, EPI, NG>), dim3(a.n_tiles * a.splits), dim3(64 * a.kparts), lds, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
@@ -967,15 +913,14 @@ static int fill_gemm_args(GemmArgs& a, const TiledW& w, const uint4* xfrag, void
 }
 
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
-                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope, const Handoff* h) {
+                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
     if (m < 1 || m > TSV_MAX_ROWS) {
         set_error("matmul: row count outside 1..16");
         return TSV_ERR_INVALID;
     }
     GemmArgs a;
     if (int rc = fill_gemm_args(a, w, xfrag, out, vp, splits, epi, ldo, n_valid, rope)) return rc;
-    if (h) a.h = *h;
-    if (w.fmt == FMT_Q4K && m >= gemm16_min_rows() && !h) return launch16(s, a, epi);
+    if (w.fmt == FMT_Q4K && m >= gemm16_min_rows()) return launch16(s, a, epi);
     return w.fmt == FMT_Q4K    ? launch_f<Q4K>(s, a, m, epi)
            : w.fmt == FMT_Q80  ? launch_f<Q80>(s, a, m, epi)
            : w.fmt == FMT_BF16 ? launch_f<BF16W>(s, a, m, epi)

@@ -612,7 +612,6 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)
 // head: the NeoX pair of a lane is lane ^ 32 (crates/compute/src/rope.rs:208-256).  Bias first,
 // then the rotation (families/gptoss/attn.rs:88-118); q goes to the fp16 q buffer, K and V
 // straight into the cache slot of the row (families/qwen/batched_layers.rs:84-113).
-template <bool COH>
 __device__ __forceinline__ void rope_epilogue(const RopeEpi& e, const VerifyParams* vp, int tile, int g, float4v v, int lane, int M) {
     const int hd = e.hd, half = hd >> 1, tph = hd >> 6;  // tiles per head
     const int tq = e.nq * tph, tk = e.nkv * tph;
@@ -639,21 +638,18 @@ __device__ __forceinline__ void rope_epilogue(const RopeEpi& e, const VerifyPara
             x = hi ? x0 * cs[i].y + x1 * cs[i].x : x0 * cs[i].x - x1 * cs[i].y;
         }
         const _Float16 h = (_Float16)x;
-        _Float16* dst;
         if (kind == 0) {
-            dst = (_Float16*)e.q16 + ((long)b * e.nq + head) * hd + d;
+            ((_Float16*)e.q16)[((long)b * e.nq + head) * hd + d] = h;
         } else {
             const int pos = (base + b) % e.max_ctx;  // the cache slot of row b (a ring layer wraps at its capacity)
             if (kind == 1) {
-                dst = (_Float16*)e.kc + ((long)head * e.max_ctx + pos) * hd + d;
+                ((_Float16*)e.kc)[((long)head * e.max_ctx + pos) * hd + d] = h;
             } else {
                 _Float16* vb = (_Float16*)e.vc + ((long)head * (e.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
                 const int po = pos & 15;
-                dst = vb + (((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3);
+                vb[(((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3)] = h;
             }
         }
-        if (COH) coh_store_f16(dst, h);
-        else *dst = h;
     }
 }
 

@@ -97,15 +97,6 @@ struct tsv_ctx {
         float *part_o = nullptr, *part_ml = nullptr;  // attention partials of every block
         size_t part_o_stride = 0, part_ml_stride = 0;
     } wide;
-    // Overlapped passes (handoff.h): the kernels of a pass alternate between the handle's stream and a second
-    // one, so that each is started while its producer still runs, asks for its weights and waits for a flag.
-    bool overlap = false;
-    hipStream_t ov_stream = nullptr;
-    hipEvent_t ov_fork = nullptr, ov_join = nullptr;
-    unsigned* ov_slots = nullptr;  // OV_SLOTS hand-over slots, used round robin
-    unsigned ov_epoch = 0;         // the epoch of the last producer launch (one counter for all slots)
-    unsigned ov_launches = 0;
-    int* ov_err = nullptr;         // pinned host memory the kernels can write
     uint16_t* q16 = nullptr;
     float *part_o = nullptr, *part_ml = nullptr;
     int nch = 0;
@@ -910,23 +901,10 @@ int run_pass(tsv_ctx* c, int m) {
     return TSV_OK;
 }
 
-// After a stream synchronisation: did a kernel of an overlapped pass give up waiting for its producer
-// (handoff.h)?  Its results are then garbage; the handle goes back to ordered launches for good and
-// reports the failure.
-int check_overlap(tsv_ctx* c) {
-    if (!c->ov_err || *c->ov_err == 0) return TSV_OK;
-    set_error("verify: a kernel of an overlapped pass waited for its producer in vain; overlapped passes are switched "
-              "off for this handle, repeat the call");
-    *c->ov_err = 0;
-    c->overlap = false;
-    return TSV_ERR_DEVICE;
-}
-
 int finish_verify(tsv_ctx* c, int m, uint16_t* logits_out) {
     if (logits_out) {
         TSV_HIP(hipMemcpyAsync(logits_out, c->logits, (size_t)m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
         TSV_HIP(hipStreamSynchronize(c->stream));
-        return check_overlap(c);
     }
     return TSV_OK;
 }
@@ -1335,10 +1313,6 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
-    if (c->ov_err) (void)hipHostFree(c->ov_err);
-    if (c->ov_stream) (void)hipStreamDestroy(c->ov_stream);
-    for (hipEvent_t e : {c->ov_fork, c->ov_join})
-        if (e) (void)hipEventDestroy(e);
     for (hipGraphExec_t g : c->pass_graph)
         if (g) (void)hipGraphExecDestroy(g);
     for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
@@ -1537,7 +1511,7 @@ static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos
         i += m;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
-    return check_overlap(c);
+    return TSV_OK;
 }
 
 extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
@@ -1668,7 +1642,6 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
         return TSV_ERR_INVALID;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
-    if (int frc = check_overlap(c)) return frc;  // rows of a pass that gave up must not be gathered
     for (int i = 0; i < n; i++) c->tok_host[32 + i] = (int32_t)path[i];
     TSV_HIP(hipMemcpyAsync(c->tok_dev + 32, c->tok_host + 32, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
     int rc = launch_kv_gather(c->stream, c->kv_ptrs, c->kv_caps, c->n_layers, c->nkv, c->hd, c->tok_dev + 32, n, (int)base);
@@ -1818,7 +1791,6 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     if (r->logits_out)
         TSV_HIP(hipMemcpyAsync(r->logits_out, c->logits, (size_t)r->m * c->vocab * 2, hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipStreamSynchronize(c->stream));
-    if ((rc = check_overlap(c))) return rc;
     const AcceptResult& a = *c->res_host;
     if (a.error) {
         set_error(std::string("accept: ") + accept_error_text(a.error));
@@ -2549,134 +2521,3 @@ extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, in
     return rc;
 }
 
-// Measurement hook: `iters` times the FFN pair of a dense layer -- gate/up with the silu-mul
-// epilogue over a (2 ffn) x hidden weight, then down over a hidden x ffn weight, m activation rows,
-// both Q4_K, `rotate` weight copies cycled so the bytes come from HBM -- as a dependent chain
-// (every launch consumes what the one before it wrote).  mode 0: ordered launches on one stream, plain
-// kernels.  mode 1: ordered launches on one stream with the hand-over kernels (what coherent stores,
-// loads and the flags cost by themselves).  mode 2: the launches alternate between two streams
-// and every kernel waits for its producer's flag after asking for its first weight tiles (handoff.h).
-// Reports the average microseconds per pair.
-extern "C" int32_t tsv_ffn_pair_time(int64_t hidden, int64_t ffn, int32_t m, int32_t mode, int32_t iters, int32_t rotate,
-                                     float* avg_us) {
-    if (hidden % 256 || ffn % 256 || m < 1 || m > 8 || mode < 0 || mode > 2 || iters < 1 || rotate < 1 || !avg_us) {
-        set_error("ffn_pair_time: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    tsv_ctx tmp;
-    tsv_ctx* c = &tmp;
-    hipStream_t s2 = nullptr;
-    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    TSV_HIP(hipStreamCreateWithFlags(&s2, hipStreamNonBlocking));
-    TiledW gu, dn;
-    gu.fmt = dn.fmt = FMT_Q4K;
-    gu.k = (int)hidden;
-    gu.kchunks = gu.k / 256;
-    gu.n_rows = (int)(2 * ffn);
-    gu.n_tiles = gu.n_rows / TILE_ROWS;
-    gu.bytes = (size_t)gu.n_tiles * gu.kchunks * 9216;
-    dn.k = (int)ffn;
-    dn.kchunks = dn.k / 256;
-    dn.n_rows = (int)hidden;
-    dn.n_tiles = dn.n_rows / TILE_ROWS;
-    dn.bytes = (size_t)dn.n_tiles * dn.kchunks * 9216;
-    std::vector<uint8_t*> gu_c((size_t)rotate), dn_c((size_t)rotate);
-    int rc = TSV_OK;
-    {
-        std::vector<uint8_t> host(std::max(gu.bytes, dn.bytes));
-        uint64_t sd = 88172645463325252ull;
-        for (size_t i = 0; i < host.size(); i += 8) {
-            sd ^= sd << 13;
-            sd ^= sd >> 7;
-            sd ^= sd << 17;
-            std::memcpy(&host[i], &sd, std::min<size_t>(8, host.size() - i));
-        }
-        for (size_t t = 0; t < host.size() / 9216; t++)  // small fp16 scales
-            for (int r = 0; r < 64; r++) host[t * 9216 + 8192 + r * 16 + 1] = host[t * 9216 + 8192 + r * 16 + 3] = 0x10;
-        for (int i = 0; i < rotate && !rc; i++) {
-            if (!(rc = dev_alloc(c, &gu_c[i], gu.bytes)) && !(rc = dev_alloc(c, &dn_c[i], dn.bytes)) &&
-                (hipMemcpy(gu_c[i], host.data(), gu.bytes, hipMemcpyHostToDevice) != hipSuccess ||
-                 hipMemcpy(dn_c[i], host.data(), dn.bytes, hipMemcpyHostToDevice) != hipSuccess))
-                rc = TSV_ERR_DEVICE;
-        }
-    }
-    VerifyParams vp;
-    std::memset(&vp, 0, sizeof vp);
-    vp.m = m;
-    uint4 *xf_a = nullptr, *xf_c = nullptr;
-    float* partial = nullptr;
-    VerifyParams* vpd = nullptr;
-    unsigned* slots = nullptr;
-    int* err = nullptr;
-    const int sp = gemm_default_splits(dn, m);
-    if (!rc) rc = dev_alloc(c, &xf_a, xfrag_bytes((int)hidden), true);
-    if (!rc) rc = dev_alloc(c, &xf_c, xfrag_bytes((int)ffn), true);
-    if (!rc) rc = dev_alloc(c, &partial, (size_t)sp * 16 * hidden * 4, true);
-    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
-    if (!rc) rc = dev_alloc(c, &slots, (size_t)4 * HANDOFF_SLOT_WORDS * 4, true);
-    if (!rc && hipHostMalloc((void**)&err, sizeof(int)) != hipSuccess) rc = TSV_ERR_DEVICE;
-    if (!rc) *err = 0;
-    if (!rc && hipMemcpy(vpd, &vp, sizeof vp, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
-    hipEvent_t e0 = nullptr, e1 = nullptr, ej = nullptr;
-    if (!rc && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess ||
-                hipEventCreateWithFlags(&ej, hipEventDisableTiming) != hipSuccess))
-        rc = TSV_ERR_DEVICE;
-    unsigned epoch = 0, launches = 0;
-    for (int pass = 0; pass < 2 && !rc; pass++) {  // pass 0 warms up
-        if (hipStreamSynchronize(c->stream) != hipSuccess || hipStreamSynchronize(s2) != hipSuccess) rc = TSV_ERR_DEVICE;
-        if (pass == 1) (void)hipEventRecord(e0, c->stream);
-        if (mode == 2) {
-            (void)hipEventRecord(ej, c->stream);
-            (void)hipStreamWaitEvent(s2, ej, 0);
-        }
-        const int n = pass ? iters : std::min(iters, 3);
-        for (int i = 0; i < 2 * n && !rc; i++) {
-            Handoff h{};
-            if (mode) {
-                if (launches) {
-                    h.wait = slots + (size_t)((launches - 1) & 3) * HANDOFF_SLOT_WORDS;
-                    h.wait_epoch = epoch;
-                }
-                h.sig = slots + (size_t)(launches & 3) * HANDOFF_SLOT_WORDS;
-                h.sig_epoch = ++epoch;
-                h.err = err;
-                launches++;
-            }
-            hipStream_t s = mode == 2 && (i & 1) ? s2 : c->stream;
-            if (i & 1) {
-                dn.tiles = dn_c[(size_t)((i / 2) % rotate)];
-                rc = launch_gemm(s, dn, xf_c, partial, vpd, m, sp, EPI_PARTIAL, (int)hidden, (int)hidden, nullptr, mode ? &h : nullptr);
-            } else {
-                gu.tiles = gu_c[(size_t)((i / 2) % rotate)];
-                rc = launch_gemm(s, gu, xf_a, xf_c, vpd, m, 1, EPI_SILU, 0, 0, nullptr, mode ? &h : nullptr);
-            }
-        }
-        if (mode == 2) {
-            (void)hipEventRecord(ej, s2);
-            (void)hipStreamWaitEvent(c->stream, ej, 0);
-        }
-        if (pass == 1) (void)hipEventRecord(e1, c->stream);
-    }
-    if (!rc) {
-        if (hipStreamSynchronize(c->stream) != hipSuccess || hipStreamSynchronize(s2) != hipSuccess) {
-            set_error("ffn_pair_time: device execution failed");
-            rc = TSV_ERR_DEVICE;
-        } else if (*err) {
-            set_error("ffn_pair_time: a hand-over wait ran out");
-            rc = TSV_ERR_DEVICE;
-        } else {
-            float ms = 0.f;
-            (void)hipEventElapsedTime(&ms, e0, e1);
-            *avg_us = ms * 1000.f / (float)iters;
-        }
-    }
-    for (hipEvent_t e : {e0, e1, ej})
-        if (e) (void)hipEventDestroy(e);
-    (void)hipStreamSynchronize(c->stream);
-    (void)hipStreamSynchronize(s2);
-    for (void* p : c->allocs) (void)hipFree(p);
-    if (err) (void)hipHostFree(err);
-    (void)hipStreamDestroy(c->stream);
-    (void)hipStreamDestroy(s2);
-    return rc;
-}

@@ -8,7 +8,6 @@
 
 #include "../../include/tsverify.h"
 #include "../../include/tsverify_testing.h"
-#include "handoff.h"
 
 namespace tsv {
 
@@ -150,7 +149,6 @@ struct GemmArgs {
     int n_tiles, kchunks, kslice, splits, kparts, per, ldo, n_valid;
     int out16;     // EPI_SILU: write the fragments in the prompt kernel's layout (frag16_index)
     RopeEpi rope;  // EPI_ROPE only
-    Handoff h;     // wait / sig non-null: the launch overlaps its neighbours in the pass (handoff.h)
 };
 
 // Re-tiles n_rows GGUF rows of `raw` into `tiles`; source row r lands in tiled row
@@ -159,7 +157,7 @@ struct GemmArgs {
 int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k, uint8_t* tiles,
                   int kchunks, int grp, int stride, int offset, const int32_t* rowmap = nullptr);
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
-                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr, const Handoff* h = nullptr);
+                int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
 int gemm_default_splits(const TiledW& w, int m);
 // rows of a prompt-block pass, and the matmul over them in blocks of sixteen (Q4_K weights only)
 int gemm_wide_rows();

@@ -240,7 +240,7 @@ EXPORTS = [
     "tsv_produce", "tsv_prefill", "tsv_checkpoint", "tsv_rollback", "tsv_rollback_retaining",
     "tsv_commit_pending", "tsv_discard_pending", "tsv_verify", "tsv_verify_tree", "tsv_compact_tree",
     "tsv_accept", "tsv_verify_accept", "tsv_accept_greedy_noalloc", "tsv_draft_chain", "tsv_row_bytes", "tsv_quantize_rows",
-    "tsv_synth_tensor", "tsv_read_kv", "tsv_write_kv", "tsv_write_logits", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat", "tsv_ffn_pair_time",
+    "tsv_synth_tensor", "tsv_read_kv", "tsv_write_kv", "tsv_write_logits", "tsv_matmul", "tsv_attention", "tsv_set_profile", "tsv_get_profile", "tsv_matmul_time", "tsv_copy_time", "tsv_set_repeat",
     "tsv_yarn_frequencies", "tsv_adaptive_init", "tsv_adaptive_depth", "tsv_adaptive_observe", "tsv_adaptive_tile_cap",
     "tsv_run_speculative", "tsv_max_context", "tsv_vocab",
     "tsv_prefix_new", "tsv_prefix_free", "tsv_prefix_clear", "tsv_prefix_taint", "tsv_prefix_record",
@@ -335,7 +335,6 @@ def lib():
         L.tsv_copy_time.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
         L.tsv_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                       C.c_int32, C.POINTER(C.c_float)]
-        L.tsv_ffn_pair_time.argtypes = [C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_float)]
         L.tsv_last_error.argtypes = [C.c_char_p, C.c_int32]
         L.tsv_gguf_open.argtypes = [C.c_char_p, C.POINTER(C.c_void_p)]
         L.tsv_gguf_close.restype = None
@@ -490,14 +489,6 @@ def matmul_time(dtype, rows, cols, m, epi=0, splits=0, iters=50, rotate=4):
     """Average microseconds per launch of the verify matmul kernel (HIP events)."""
     t = C.c_float()
     check(lib().tsv_matmul_time(dtype, rows, cols, m, epi, splits, iters, rotate, C.byref(t)))
-    return t.value
-
-
-def ffn_pair_time(hidden, ffn, m, mode, iters=64, rotate=6):
-    """Average microseconds of one gate/up + down pair in a dependent chain (mode 0: ordered launches, 1: ordered
-    launches of the kernels that hand over through flags, 2: those kernels overlapped on two streams)."""
-    t = C.c_float()
-    check(lib().tsv_ffn_pair_time(hidden, ffn, m, mode, iters, rotate, C.byref(t)))
     return t.value
 
 
