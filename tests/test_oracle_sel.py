@@ -345,3 +345,80 @@ def test_sampled_tree_round_matches_the_target_in_law_with_two_siblings():
     p = np.zeros(V)
     p[sup] = pr
     assert 0.5 * np.abs(counts / N - p).sum() < 0.03
+
+
+def _softmax(row):
+    e = np.exp(np.asarray(row, np.float64) - np.max(row))
+    return e / e.sum()
+
+
+def test_sampled_tree_round_matches_the_target_in_law_with_three_siblings():
+    """Three children drawn i.i.d. from q under the root.  The first emitted token must follow p whatever q is, and
+    the chance that one of the three is accepted has a closed form: stage s accepts with sum min(p_s, q), where
+    p_0 = p and p_{s+1} = normalise(max(p_s - q, 0)) -- so a residual that is not carried from sibling to sibling, or
+    is carried wrongly, moves both figures."""
+    V, N = 5, 6000
+    target = np.array([[1.2, 0.3, -0.5, 0.8, -1.5]] * 4, np.float16)
+    draft = np.array([[-0.8, 1.0, 0.6, -0.2, 0.4]] * 4, np.float16)
+    counts, accepted = np.zeros(V), 0
+    for seed in range(N):
+        cfg = ob.shaping(1.0, seed=seed)
+        sup, pr = ob.shaped_distribution(draft[0], cfg)
+        kids = [ob.dist_draw(sup, pr, seed, i) for i in range(3)]
+        r = ob.tree_round_sampled(target, draft, [0] + kids, [-1, 0, 0, 0], cfg, draw_step=3)
+        assert r["draw_step"] == 3 + (r["path"][1] if r["accepted"] else 3) + 1   # one uniform per child tried, one final draw
+        counts[([0] + kids)[r["path"][1]] if r["accepted"] else r["next"]] += 1
+        accepted += r["accepted"] > 0
+    p, q = _softmax(target[0].astype(np.float64)), _softmax(draft[0].astype(np.float64))
+    assert 0.5 * np.abs(counts / N - p).sum() < 0.03
+    miss, ps = 1.0, p.copy()
+    for _ in range(3):
+        miss *= 1.0 - np.minimum(ps, q).sum()
+        ps = np.maximum(ps - q, 0.0)
+        ps /= ps.sum()
+    assert abs(accepted / N - (1.0 - miss)) < 0.03
+
+
+def test_sampled_tree_round_matches_the_target_in_law_below_an_accepted_child():
+    """Depth two: two siblings under the root, two children under each of them, every node's children drawn i.i.d.
+    from the drafter's row of that node.  Target and drafter rows of a depth-one node depend on the node's token (as a
+    model's would), so the law to meet is the chain rule: the first token follows p0, and below an accepted child
+    holding x the second token follows p(. | x) -- freshly, not what the root's rejections left over, and also
+    where the first sibling's subtree was rejected and the second sibling accepted."""
+    V, N = 4, 40000
+    rng = np.random.default_rng(11)
+    p0, q0 = rng.standard_normal(V), rng.standard_normal(V)
+    pc, qc = rng.standard_normal((V, V)) * 1.3, rng.standard_normal((V, V))
+    parent = [-1, 0, 0, 1, 1, 2, 2]
+    first = np.zeros(V)
+    second = np.zeros((V, V))
+    second_via_sibling = np.zeros((V, V))
+    for seed in range(N):
+        cfg = ob.shaping(1.0, seed=seed)
+        sup, pr = ob.shaped_distribution(q0.astype(np.float16), cfg)
+        a, b = ob.dist_draw(sup, pr, seed, 0), ob.dist_draw(sup, pr, seed, 1)
+        feed, step = [0, a, b], 2
+        for x in (a, b):
+            sup, pr = ob.shaped_distribution(qc[x].astype(np.float16), cfg)
+            feed += [ob.dist_draw(sup, pr, seed, step), ob.dist_draw(sup, pr, seed, step + 1)]
+            step += 2
+        target = np.stack([p0, pc[a], pc[b]] + [p0] * 4).astype(np.float16)
+        draft = np.stack([q0, qc[a], qc[b]] + [q0] * 4).astype(np.float16)
+        r = ob.tree_round_sampled(target, draft, feed, parent, cfg, draw_step=step)
+        if not r["accepted"]:
+            first[r["next"]] += 1
+            continue
+        x = feed[r["path"][1]]
+        first[x] += 1
+        y = feed[r["path"][2]] if r["accepted"] >= 2 else r["next"]
+        second[x, y] += 1
+        if r["path"][1] == 2:
+            second_via_sibling[x, y] += 1
+    f16 = lambda v: np.asarray(v, np.float16).astype(np.float64)
+    assert 0.5 * np.abs(first / N - _softmax(f16(p0))).sum() < 0.03
+    for table, bound in ((second, 0.03), (second_via_sibling, 0.06)):
+        n = table.sum()
+        assert n > 1500
+        tv = sum(0.5 * np.abs(table[x] / table[x].sum() - _softmax(f16(pc[x]))).sum() * table[x].sum() / n
+                 for x in range(V) if table[x].sum() > 0)
+        assert tv < bound, tv

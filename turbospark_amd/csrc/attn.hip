@@ -25,6 +25,15 @@ int attn_chunks(int nkv) {
     return n;
 }
 
+// blocks in flight per wave when a workgroup holds two row tiles: two at 128-wide heads (a third block's
+// registers would spill), three at 64-wide ones
+#ifndef TSV_ATTN_STAGES2_HD128
+#define TSV_ATTN_STAGES2_HD128 2
+#endif
+#ifndef TSV_ATTN_STAGES2_HD64
+#define TSV_ATTN_STAGES2_HD64 3
+#endif
+
 // Eight waves per workgroup share a chunk of the context (attn_core.h).
 template <int HD, int RT, int STAGES>
 __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) {
@@ -217,7 +226,7 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
     } else if (trt <= 1)
         rc = launch_partial<HD, 1, 3>(s, a, G, R, 1);
     else
-        rc = launch_partial<HD, 2, 3>(s, a, G, R, groups);
+        rc = launch_partial<HD, 2, (HD == 128 ? TSV_ATTN_STAGES2_HD128 : TSV_ATTN_STAGES2_HD64)>(s, a, G, R, groups);
     if (rc) return rc;
     return launch_combine<HD>(s, a, m, G, R);
 }

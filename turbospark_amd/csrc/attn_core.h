@@ -3,6 +3,8 @@
 // crates/compute/src/attention.rs:53-137).  Shared by the stand-alone attention kernel and the
 // per-XCD fused attention block.
 #pragma once
+#include <type_traits>
+
 #include "tsv_internal.h"
 
 namespace tsv {
@@ -18,7 +20,8 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // other way in the next, and a row's bits would then depend on how many rows share its pass.
 //
 // One (m, l, O) running state merged into another (flash-decoding rescale).
-template <int RT, int VT>
+// (BASE2: the maxima are kept in units of log 2, the weights are powers of two)
+template <int RT, int VT, bool BASE2 = false>
 __device__ __forceinline__ void merge_state(float (&mrun)[RT], float (&lrun)[RT], float4v (&O)[RT][VT], const float* src) {
     // `src` points at this lane's column of a [values][64 lanes] slot: consecutive lanes touch
     // consecutive LDS banks
@@ -27,7 +30,8 @@ __device__ __forceinline__ void merge_state(float (&mrun)[RT], float (&lrun)[RT]
         const float m1 = src[64 * (2 * t)], l1 = src[64 * (2 * t + 1)];
         const float mnew = fmaxf(mrun[t], m1);
         if (mnew > -INFINITY) {
-            const float a0 = __expf(mrun[t] - mnew), a1 = __expf(m1 - mnew);
+            const float a0 = BASE2 ? __builtin_amdgcn_exp2f(mrun[t] - mnew) : __expf(mrun[t] - mnew);
+            const float a1 = BASE2 ? __builtin_amdgcn_exp2f(m1 - mnew) : __expf(m1 - mnew);
             lrun[t] = fmaf(lrun[t], a0, l1 * a1);
 #pragma unroll
             for (int d = 0; d < VT; d++)
@@ -51,6 +55,19 @@ __device__ __forceinline__ void store_state(const float (&mrun)[RT], const float
     }
 }
 
+// max over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the four position groups of one (row, q head) pair), in every
+// one of them, on the vector ALU: v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even
+// rows of its second, v_permlane32_swap the upper half of the first with the lower half of the second, so with the
+// same value in both operands the two results hold the value of lane l and of its partner.  (Written as assembly:
+// the compiler folds max(result 0, result 1) of the builtin with equal operands into result 0.)
+__device__ __forceinline__ float max_over_position_groups(float v) {
+    float w = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1" : "+v"(v), "+v"(w));
+    w = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1" : "+v"(v), "+v"(w));
+    return v;
+}
+
 // Eight waves per workgroup share a chunk of the context, each walking every eighth 16-position
 // block with up to STAGES blocks of K and V in flight.
 // COH: the query rows and the K / V blocks are read device-coherently (sc1), for a caller whose
@@ -64,7 +81,9 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
     constexpr int PER_LANE = RT * VT * 4 + 2 * RT;
     constexpr int POLICY = COH ? 16 : 0;  // buffer-load cache policy: sc1
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // (the wave index as a scalar: everything derived from it -- block numbers, the choice of variant -- then stays
+    // on the scalar unit)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, kg = lane >> 4;
     const VerifyParams* vp = a.vp;
     const int M = a.base_hint >= 0 ? a.m_hint : vp->m, base = a.base_hint >= 0 ? a.base_hint : vp->base, kvlen = base + M;
@@ -121,31 +140,37 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
         for (int d = 0; d < VT; d++) O[t][d] = float4v{0.f, 0.f, 0.f, 0.f};
     }
 
-    // this head's K rows and V blocks as buffers that end after block b1 - 1; a ring layer
+    // this head's K and V blocks (kcache_index / vcache_index: a block is KS, resp. VT / 2, runs of one KiB, each
+    // what one wave-wide 16-byte load takes) as buffers that end after block b1 - 1; a ring layer
     // (kv_cache.rs:360-378: position p lives in slot p % capacity) keeps block b in slot b % nbc
     const bool ring = a.ring != 0;
     const int nbc = a.max_ctx >> 4;
     const uint32_t blk_bytes = 16 * HD * 2;
     const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)((const _Float16*)a.kc + (long)h * a.max_ctx * HD), 0, (int)((ring ? nbc : b1) * blk_bytes), 0x00027000);
+        (void*)((const _Float16*)a.kc + (long)h * (a.max_ctx >> 4) * (HD * 16)), 0, (int)((ring ? nbc : b1) * blk_bytes), 0x00027000);
     const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)((const _Float16*)a.vc + (long)h * (a.max_ctx >> 4) * (HD * 16)), 0, (int)((ring ? nbc : b1) * blk_bytes), 0x00027000);
     struct Blk {
         u32x4 kf[KS];
-        u32x2 vf[VT];
+        u32x4 vf[VT / 2];  // two output tiles' operands per load
     };
-    const uint32_t koff = (uint32_t)(j * HD + 8 * kg) * 2, voff = (uint32_t)lane * 8;
+    const uint32_t loff = (uint32_t)lane * 16;
     const int nb = b1 > b0 + wave ? (b1 - b0 - wave + NW - 1) / NW : 0;  // blocks of this wave
     auto fetch = [&](Blk& st, int i) {  // block i of this wave's run
         const int blk = b0 + wave + NW * i;
         const uint32_t bo = (uint32_t)(ring ? blk % nbc : blk) * blk_bytes;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s = 0; s < KS; s++) st.kf[s] = __builtin_amdgcn_raw_buffer_load_b128(krs, bo + koff + 64 * s, 0, POLICY);
+        for (int s = 0; s < KS; s++) st.kf[s] = __builtin_amdgcn_raw_buffer_load_b128(krs, bo + loff + 1024 * s, 0, POLICY);
 #pragma unroll
-        for (int d = 0; d < VT; d++) st.vf[d] = __builtin_amdgcn_raw_buffer_load_b64(vrs, bo + voff + 512 * d, 0, POLICY);
+        for (int u = 0; u < VT / 2; u++) st.vf[u] = __builtin_amdgcn_raw_buffer_load_b128(vrs, bo + loff + 1024 * u, 0, POLICY);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // Scores are kept in units of log 2 (one multiply by scale * log2(e), then v_exp_f32 as it is), and a block that
+    // lies wholly inside the committed prefix and inside every row's window -- nearly all of a long context -- takes
+    // the variant without the visibility words (a wave-uniform choice; a visible position gets the same operations
+    // in the same order in both, so its bits do not depend on which variant its block took).
+    const float c2 = scale * 1.44269504088896340736f;
     auto consume = [&](const Blk& st, int i) {
         const int p0 = (b0 + wave + NW * i) << 4;
         const bool tail = p0 + 16 > base;
@@ -156,39 +181,41 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
             for (int s = 0; s < KS; s++)
                 S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, st.kf[s]),
                                                            __builtin_bit_cast(half8, qf[t][s]), S, 0, 0, 0);
-            // Visibility of this lane's four positions as a 4-bit word, computed without
-            // branches: bit (slot + 16) of `w` says whether cache slot base+slot is visible
-            // (the 16 low bits stand for prefix positions, always visible).
-            uint32_t vis4 = 0xFu;
-            if (tail) {
-                const uint64_t w = ((uint64_t)(anc[t] & mmask) << 16) | 0xFFFFull;
-                vis4 = (uint32_t)(w >> (p0 + 4 * kg - base + 16)) & 0xFu;  // shift in [1, 47]
-            }
-            if (p0 < cut_end) {  // some row's window starts inside or after this block
-                const int d = lo[t] + 1 - window - (p0 + 4 * kg);  // this lane's positions below index d are outside
-                vis4 &= d <= 0 ? 0xFu : d >= 4 ? 0u : (0xFu << d) & 0xFu;
-            }
             float sc[4];
 #pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) sc[i4] = ((vis4 >> i4) & 1u) ? S[i4] * scale : -INFINITY;
-            float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-            mb = fmaxf(mb, __shfl_xor(mb, 16));
-            mb = fmaxf(mb, __shfl_xor(mb, 32));
-            const float mnew = fmaxf(mrun[t], mb);
-            float alpha = 1.f;
-            half4 P = {0, 0, 0, 0};
-            if (mnew > -INFINITY) {
-                alpha = __expf(mrun[t] - mnew);
-                float ps = 0.f;
-#pragma unroll
-                for (int i4 = 0; i4 < 4; i4++) {
-                    const float p = __expf(sc[i4] - mnew);
-                    ps += p;
-                    P[i4] = (_Float16)p;
+            for (int i4 = 0; i4 < 4; i4++) sc[i4] = S[i4] * c2;
+            if (tail || p0 < cut_end) {  // (wave-uniform: a scalar branch)
+                // Visibility of this lane's four positions as a 4-bit word, computed without
+                // branches: bit (slot + 16) of `w` says whether cache slot base+slot is visible
+                // (the 16 low bits stand for prefix positions, always visible).
+                uint32_t vis4 = 0xFu;
+                if (tail) {
+                    const uint64_t w = ((uint64_t)(anc[t] & mmask) << 16) | 0xFFFFull;
+                    vis4 = (uint32_t)(w >> (p0 + 4 * kg - base + 16)) & 0xFu;  // shift in [1, 47]
                 }
-                lrun[t] = fmaf(lrun[t], alpha, ps);
-                mrun[t] = mnew;
+                if (p0 < cut_end) {  // some row's window starts inside or after this block
+                    const int d = lo[t] + 1 - window - (p0 + 4 * kg);  // this lane's positions below index d are outside
+                    vis4 &= d <= 0 ? 0xFu : d >= 4 ? 0u : (0xFu << d) & 0xFu;
+                }
+#pragma unroll
+                for (int i4 = 0; i4 < 4; i4++) sc[i4] = ((vis4 >> i4) & 1u) ? sc[i4] : -INFINITY;
             }
+            const float mb = max_over_position_groups(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
+            const float mnew = fmaxf(mrun[t], mb);
+            // a row that has seen nothing yet (every position so far masked) has mnew = -inf: the differences below are
+            // taken against a finite stand-in, which makes every weight and the factor zero and leaves the empty state
+            const float mref = fmaxf(mnew, -3.0e38f);
+            const float alpha = __builtin_amdgcn_exp2f(mrun[t] - mref);
+            half4 P;
+            float ps = 0.f;
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++) {
+                const float p = __builtin_amdgcn_exp2f(sc[i4] - mref);
+                ps += p;
+                P[i4] = (_Float16)p;
+            }
+            lrun[t] = fmaf(lrun[t], alpha, ps);
+            mrun[t] = mnew;
             // once the running maximum has settled the factor is exactly 1 in every lane: the products are
             // skipped then (the same bits), which is most blocks of a long context
             if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
@@ -197,7 +224,9 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
             }
 #pragma unroll
             for (int d = 0; d < VT; d++) {
-                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, st.vf[d]), P, O[t][d], 0, 0, 0);
+                const u32x4 v2 = st.vf[d >> 1];
+                const u32x2 vd = (d & 1) ? u32x2{v2.z, v2.w} : u32x2{v2.x, v2.y};
+                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, vd), P, O[t][d], 0, 0, 0);
             }
         }
     };
@@ -243,12 +272,12 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
     float* mine = xch + (wave & 3) * 64 * PER_LANE + lane;
     if (wave >= 4) store_state<RT, VT>(mrun, lrun, O, mine);
     __syncthreads();
-    if (wave < 4) merge_state<RT, VT>(mrun, lrun, O, mine);
+    if (wave < 4) merge_state<RT, VT, true>(mrun, lrun, O, mine);
     __syncthreads();
     if (wave >= 1 && wave < 4) store_state<RT, VT>(mrun, lrun, O, mine);
     __syncthreads();
     if (wave != 0) return;
-    for (int w = 1; w < 4; w++) merge_state<RT, VT>(mrun, lrun, O, xch + w * 64 * PER_LANE + lane);
+    for (int w = 1; w < 4; w++) merge_state<RT, VT, true>(mrun, lrun, O, xch + w * 64 * PER_LANE + lane);
 #pragma unroll
     for (int t = 0; t < RT; t++) {
         float l = lrun[t];
@@ -258,7 +287,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
         if (r >= R) continue;
         const long slot = ((long)h * a.nch + chunk) * R + r;
         if (kg == 0) {
-            a.part_ml[slot * 2] = mrun[t];
+            a.part_ml[slot * 2] = mrun[t] * 0.69314718055994530942f;  // the merge works with natural logarithms
             a.part_ml[slot * 2 + 1] = l;
         }
         float* o = a.part_o + slot * HD + 4 * kg;

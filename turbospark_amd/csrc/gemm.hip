@@ -506,14 +506,11 @@ __device__ __forceinline__ void epilogue16(const GemmArgs& a, int tile, int spli
             } else {
                 const int pos = (base + b) % e.max_ctx;
                 if (kind == 1) {
-                    _Float16* kc = (_Float16*)e.kc + ((long)head * e.max_ctx + pos) * hd;
-                    kc[d0] = h0;
-                    kc[d1] = h1;
+                    ((_Float16*)e.kc)[kcache_index(head, pos, d0, hd, e.max_ctx)] = h0;
+                    ((_Float16*)e.kc)[kcache_index(head, pos, d1, hd, e.max_ctx)] = h1;
                 } else {
-                    _Float16* vb = (_Float16*)e.vc + ((long)head * (e.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
-                    const int po = pos & 15;
-                    vb[(((d0 >> 4) * 64) + (po >> 2) * 16 + (d0 & 15)) * 4 + (po & 3)] = h0;
-                    vb[(((d1 >> 4) * 64) + (po >> 2) * 16 + (d1 & 15)) * 4 + (po & 3)] = h1;
+                    ((_Float16*)e.vc)[vcache_index(head, pos, d0, hd, e.max_ctx)] = h0;
+                    ((_Float16*)e.vc)[vcache_index(head, pos, d1, hd, e.max_ctx)] = h1;
                 }
             }
         }

@@ -642,13 +642,10 @@ __device__ __forceinline__ void rope_epilogue(const RopeEpi& e, const VerifyPara
             ((_Float16*)e.q16)[((long)b * e.nq + head) * hd + d] = h;
         } else {
             const int pos = (base + b) % e.max_ctx;  // the cache slot of row b (a ring layer wraps at its capacity)
-            if (kind == 1) {
-                ((_Float16*)e.kc)[((long)head * e.max_ctx + pos) * hd + d] = h;
-            } else {
-                _Float16* vb = (_Float16*)e.vc + ((long)head * (e.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
-                const int po = pos & 15;
-                vb[(((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3)] = h;
-            }
+            if (kind == 1)
+                ((_Float16*)e.kc)[kcache_index(head, pos, d, hd, e.max_ctx)] = h;
+            else
+                ((_Float16*)e.vc)[vcache_index(head, pos, d, hd, e.max_ctx)] = h;
         }
     }
 }

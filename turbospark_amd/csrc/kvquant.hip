@@ -147,11 +147,8 @@ __device__ __forceinline__ void wht(float (&e)[EPL], int lane, float c) {
     }
 }
 
-__device__ __forceinline__ long k_at(int cap, int hd, int head, int pos, int d) { return ((long)head * cap + pos) * hd + d; }
-__device__ __forceinline__ long v_at(int cap, int hd, int head, int pos, int d) {
-    const int po = pos & 15;
-    return ((long)head * (cap >> 4) + (pos >> 4)) * (hd * 16) + (((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3);
-}
+__device__ __forceinline__ long k_at(int cap, int hd, int head, int pos, int d) { return kcache_index(head, pos, d, hd, cap); }
+__device__ __forceinline__ long v_at(int cap, int hd, int head, int pos, int d) { return vcache_index(head, pos, d, hd, cap); }
 
 // q row (b, qh): rotate with the key signs, in place
 template <int HD>

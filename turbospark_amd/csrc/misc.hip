@@ -347,15 +347,11 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
     } else {
         const int pos = (base + m) % a.max_ctx;  // the cache slot of row m (a ring layer wraps at its capacity)
         if (kind == 1) {
-            _Float16* k = (_Float16*)a.kc + ((long)h * a.max_ctx + pos) * hd;
-            k[i] = h0;
-            k[i + half] = h1;
+            ((_Float16*)a.kc)[kcache_index(h, pos, i, hd, a.max_ctx)] = h0;
+            ((_Float16*)a.kc)[kcache_index(h, pos, i + half, hd, a.max_ctx)] = h1;
         } else {
-            _Float16* v = (_Float16*)a.vc + ((long)h * (a.max_ctx >> 4) + (pos >> 4)) * (hd * 16);
-            const int po = pos & 15, kg = po >> 2, pi = po & 3;
-            const int d0 = i, d1 = i + half;
-            v[(((d0 >> 4) * 64) + kg * 16 + (d0 & 15)) * 4 + pi] = h0;
-            v[(((d1 >> 4) * 64) + kg * 16 + (d1 & 15)) * 4 + pi] = h1;
+            ((_Float16*)a.vc)[vcache_index(h, pos, i, hd, a.max_ctx)] = h0;
+            ((_Float16*)a.vc)[vcache_index(h, pos, i + half, hd, a.max_ctx)] = h1;
         }
     }
 }
@@ -371,11 +367,6 @@ int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m) {
 }
 
 // ---------------------------------------------------------------- KV row gather / read
-__device__ __forceinline__ long v_index(int h, int pos, int d, int hd, int max_ctx) {
-    const int po = pos & 15;
-    return ((long)h * (max_ctx >> 4) + (pos >> 4)) * (hd * 16) +
-           ((((d >> 4) * 64) + (po >> 2) * 16 + (d & 15)) * 4 + (po & 3));
-}
 
 // Tree compaction (families/qwen/dflash_tree.rs:106-207): rows of slots path[0..n) move to
 // base..base+n.  path is strictly increasing with path[i] >= i, so walking i upward never
@@ -392,8 +383,8 @@ __global__ void k_kv_gather(uint16_t* const* caches, const int32_t* caps, int hd
         const int src = (base + path[i]) % max_ctx, dst = (base + i) % max_ctx;
         if (src == dst) continue;
         if (d < hd) {
-            kc[((long)h * max_ctx + dst) * hd + d] = kc[((long)h * max_ctx + src) * hd + d];
-            vc[v_index(h, dst, d, hd, max_ctx)] = vc[v_index(h, src, d, hd, max_ctx)];
+            kc[kcache_index(h, dst, d, hd, max_ctx)] = kc[kcache_index(h, src, d, hd, max_ctx)];
+            vc[vcache_index(h, dst, d, hd, max_ctx)] = vc[vcache_index(h, src, d, hd, max_ctx)];
         }
     }
 }
@@ -411,8 +402,8 @@ __global__ void k_kv_read(const uint16_t* kc, const uint16_t* vc, int nkv, int h
     if (d >= hd) return;
     const long o = ((long)p * nkv + h) * hd + d;
     const int pos = (pos0 + p) % max_ctx;
-    k_out[o] = kc[((long)h * max_ctx + pos) * hd + d];
-    v_out[o] = vc[v_index(h, pos, d, hd, max_ctx)];
+    k_out[o] = kc[kcache_index(h, pos, d, hd, max_ctx)];
+    v_out[o] = vc[vcache_index(h, pos, d, hd, max_ctx)];
 }
 
 __global__ void k_kv_fill(uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0,
@@ -421,8 +412,8 @@ __global__ void k_kv_fill(uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_c
     if (d >= hd) return;
     const long o = ((long)p * nkv + h) * hd + d;
     const int pos = (pos0 + p) % max_ctx;
-    kc[((long)h * max_ctx + pos) * hd + d] = k_in[o];
-    vc[v_index(h, pos, d, hd, max_ctx)] = v_in[o];
+    kc[kcache_index(h, pos, d, hd, max_ctx)] = k_in[o];
+    vc[vcache_index(h, pos, d, hd, max_ctx)] = v_in[o];
 }
 
 int launch_kv_fill(hipStream_t s, uint16_t* kc, uint16_t* vc, int nkv, int hd, int max_ctx, int pos0, int n,

@@ -115,6 +115,23 @@ __host__ __device__ inline int xsum_index(int sub, int row) {
     return (((sub >> 3) * 4 + (row >> 2)) * 8 + (sub & 7)) * 4 + (row & 3);
 }
 
+// KV cache layouts (fp16).  Both caches are cut into blocks of 16 positions, and inside a block the halfs sit
+// where the attention kernel's matrix instructions want them, so that every wave-wide load of that kernel is
+// one contiguous KiB (64 lanes x 16 bytes):
+//   K: [kv head][pos / 16][hd / 32][lane = 16 * ((d % 32) / 8) + pos % 16][8 halfs = d % 8] -- lane (j, kg) of
+//      K step s holds dims 32 s + 8 kg .. + 7 of position j: the A operand of v_mfma_f32_16x16x32_f16;
+//   V: [kv head][pos / 16][hd / 32][lane = 16 * ((pos % 16) / 4) + d % 16][(d / 16) % 2][4 halfs = pos % 4] -- the
+//      A operands (V^T: dims x positions) of two v_mfma_f32_16x16x16_f16 output tiles side by side.
+// `cap` is the number of positions the cache holds (a multiple of 16).
+__host__ __device__ inline long kcache_index(int h, int pos, int d, int hd, int cap) {
+    return (((long)h * (cap >> 4) + (pos >> 4)) * (hd >> 5) + (d >> 5)) * 512 + ((((d >> 3) & 3) * 16 + (pos & 15)) << 3) + (d & 7);
+}
+__host__ __device__ inline long vcache_index(int h, int pos, int d, int hd, int cap) {
+    const int po = pos & 15;
+    return (((long)h * (cap >> 4) + (pos >> 4)) * (hd >> 5) + (d >> 5)) * 512 +
+           ((((po >> 2) * 16 + (d & 15)) * 2 + ((d >> 4) & 1)) << 2) + (po & 3);
+}
+
 // Per-call parameters every kernel of a verify pass reads from device memory, so a captured
 // launch sequence can be replayed at another base position.
 struct VerifyParams {
