@@ -292,7 +292,10 @@ int32_t tsv_verify_accept(tsv_ctx* ctx, const tsv_round* round, tsv_round_result
  * at most 16 stop tokens.  There is no handle, so no KV truncation: result->kv_position = base +
  * committed + 1 is where the caller moves its cursor.  A non-finite logit is reported in band
  * (stopped = -1, next = -1, path_len = 0).  Calls on one GPU share that GPU's array: two calls that
- * overlap in time on one GPU race. */
+ * overlap in time on one GPU race.  Under stream capture: the stream must be one of the caller's own (the
+ * NULL stream cannot be captured), and the array's address must already be known on that GPU -- it is once
+ * tsv_open has run there, or after one call of this entry point outside capture (the first call on a GPU asks
+ * the runtime for the address, which is not a capturable operation). */
 int32_t tsv_accept_greedy_noalloc(void* stream, const uint16_t* logits_dev, int32_t vocab, const int32_t* feed,
                                   const int32_t* parent, int32_t m, int64_t base, const int32_t* stop_tokens,
                                   int32_t n_stop, uint64_t generated, uint64_t max_new_tokens,

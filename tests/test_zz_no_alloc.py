@@ -85,6 +85,45 @@ def test_the_allocation_free_greedy_round_equals_tsv_accept(vocab):
     assert (good.accepted, good.next, good.stopped) == (want.accepted, want.next, 0)
 
 
+def test_the_entry_point_captured_into_a_graph_replays_like_the_eager_round():
+    """The call recorded once into a HIP graph on a stream of the caller's own (a handle was opened first, so the
+    scratch address is known and the call makes no runtime query), then replayed three times with the program's own
+    eager work and synchronizations between the replays and new logits in the same device buffer each time: every
+    replay equals tsv_accept on those logits."""
+    import turbospark_amd as ts
+    from turbospark_amd import ffi, hip, synth
+    vocab, m, base = 4096, 6, 11
+    cfg = dict(synth.CONFIGS["tiny_q8_0"], max_context=64, vocab=vocab)
+    gpu = ts.HipVerifier(cfg, synth.make_weights(cfg, seed=5))
+    rng = np.random.default_rng(77)
+    dev = hip.DeviceBuffer(m * vocab * 2)
+    out_dev = hip.DeviceBuffer(C.sizeof(ffi.RoundResultC))
+    # the graph bakes the host arguments in (feed, tree, limits): the proposals stay, the logits change
+    feed = rng.integers(0, vocab, m).astype(np.int32)
+    stream = hip.Stream()
+
+    def record(s):
+        ffi.check(ffi.lib().tsv_accept_greedy_noalloc(s.h, dev.ptr, vocab, feed.ctypes.data, None, m, base, None, 0, 0, 0,
+                                                      out_dev.ptr))
+    graph = hip.CapturedGraph(stream, record)
+    outcomes = set()
+    for replay in range(3):
+        logits = rng.standard_normal((m, vocab)).astype(np.float16)
+        for row in range(replay + 1):                      # the first rows' arg-max is the next proposal: 1, 2, 3 hits
+            logits[row, feed[row + 1]] = np.float16(9.0)
+        gpu.write_logits(logits, base)                     # eager work on another stream, and its synchronization
+        want = gpu.accept(feed, base, ts.shaping(0.0))
+        dev.upload(np.ascontiguousarray(logits.view(np.uint16)))
+        graph.launch()
+        stream.sync()
+        got = ffi.RoundResultC()
+        hip.check(hip.rt().hipMemcpy(C.byref(got), out_dev.ptr, C.sizeof(got), 2), "copy back")
+        assert (got.accepted, got.committed, got.next, got.stopped, got.kv_position) == \
+            (want.accepted, want.committed, want.next, want.stopped, want.kv_position), (replay, want)
+        outcomes.add(got.accepted)
+    assert len(outcomes) == 3                              # the replays really judged different logits
+
+
 def test_sizes_beyond_the_static_scratch_are_refused_by_name():
     from turbospark_amd import ffi, hip
     buf = hip.DeviceBuffer(1 << 16)

@@ -1718,6 +1718,7 @@ struct NoAllocScratch {
 static_assert(sizeof(NoAllocScratch) <= sizeof(scratch), "the static array holds the greedy round's partial results");
 
 // the flag must start at zero; a fill kernel rather than a memset node, so a caller may capture the call
+// (on a stream of its own, with the scratch address already resolved on the device: noalloc_prepare_device)
 __global__ void k_noalloc_clear(int32_t* err) {
     if (threadIdx.x == 0) *err = 0;
 }
@@ -1778,6 +1779,13 @@ int noalloc_scratch(NoAllocScratch** out) {
 }
 
 }  // namespace
+
+// Resolves the scratch array's address on the current device, so that a later tsv_accept_greedy_noalloc makes no
+// runtime query (tsv_open calls this: after any handle was opened on a device the entry point can be captured).
+int noalloc_prepare_device() {
+    NoAllocScratch* sc = nullptr;
+    return noalloc_scratch(&sc);
+}
 }  // namespace tsv
 
 extern "C" int32_t tsv_accept_greedy_noalloc(void* stream, const uint16_t* logits_dev, int32_t vocab, const int32_t* feed,

@@ -53,6 +53,19 @@ __global__ __launch_bounds__(512) void k_attn_partial(AttnArgs a, int G, int R) 
     attn_partial_body<HD, RT, STAGES, false>(a, G, R, blockIdx.x, blockIdx.y, grp * RT, xch);
 }
 
+// A pass of more than two row tiles: TG tile groups side by side in one workgroup (attn_core.h), one read of the
+// chunk's K / V blocks out of the L2 for all of them.  Grid (chunks, kv heads, 16-row blocks of a prompt pass).
+template <int HD, int RT, int STAGES, int TG>
+__global__ __launch_bounds__(64 * TG * attn_phases(TG)) void k_attn_partial_groups(AttnArgs a, int G, int R) {
+    extern __shared__ float xch[];
+    if (a.blocks > 1) {
+        const AttnArgs v = attn_block_view(a, blockIdx.z);
+        attn_partial_body<HD, RT, STAGES, false, TG>(v, G, R, blockIdx.x, blockIdx.y, 0, xch);
+        return;
+    }
+    attn_partial_body<HD, RT, STAGES, false, TG>(a, G, R, blockIdx.x, blockIdx.y, 0, xch);
+}
+
 // The same pass over a layer that keeps quantized rows (attn_tq_core.h)
 template <int HD, int RT, int KB, int VB>
 __global__ __launch_bounds__(512) void k_attn_partial_tq(AttnArgs a, int G, int R) {
@@ -173,6 +186,22 @@ static int launch_partial(hipStream_t s, const AttnArgs& a, int G, int R, int gr
     return TSV_OK;
 }
 
+template <int HD, int RT, int STAGES, int TG>
+static int launch_partial_groups(hipStream_t s, const AttnArgs& a, int G, int R) {
+    constexpr int PER_LANE = RT * (HD / 16) * 4 + 2 * RT, NW = attn_phases(TG), SLOTS = NW < 4 ? NW : 4;
+    const size_t lds = (size_t)TG * SLOTS * 64 * PER_LANE * 4;
+    static bool raised = false;  // more than 64 KiB of dynamic LDS has to be allowed once per kernel
+    if (lds > 65536 && !raised) {
+        TSV_HIP(hipFuncSetAttribute((const void*)k_attn_partial_groups<HD, RT, STAGES, TG>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((k_attn_partial_groups<HD, RT, STAGES, TG>), dim3(a.nch, a.nkv, std::max(a.blocks, 1)), dim3(64 * TG * NW),
+                       lds, s, a, G, R);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
 template <int HD>
 static int launch_combine(hipStream_t s, const AttnArgs& a, int m, int G, int R);
 
@@ -225,8 +254,27 @@ static int launch_hd(hipStream_t s, const AttnArgs& a0, int m, int G, int R) {
         rc = trt <= 1 ? launch_partial_tq_widths<HD, 1>(s, a, G, R, 1) : launch_partial_tq_widths<HD, 2>(s, a, G, R, groups);
     } else if (trt <= 1)
         rc = launch_partial<HD, 1, 3>(s, a, G, R, 1);
-    else
-        rc = launch_partial<HD, 2, (HD == 128 ? TSV_ATTN_STAGES2_HD128 : TSV_ATTN_STAGES2_HD64)>(s, a, G, R, groups);
+    else if (trt <= 2)
+        rc = launch_partial<HD, 2, (HD == 128 ? TSV_ATTN_STAGES2_HD128 : TSV_ATTN_STAGES2_HD64)>(s, a, G, R, 1);
+    else {
+        // more row tiles than a wave holds: tile groups inside one workgroup, about one workgroup per compute unit
+        a.xcd_groups = 0;
+        a.nch = std::max(1, std::min(a0.nch, 256 / (a0.nkv * std::max(a0.blocks, 1))));
+        // (64 chunks at four KV heads would fill the chip, but what the partial pass wins the merge loses reading
+        // twice the partial results: 10.9 + 6.0 us against 12.9 + 4.1 us at the Qwen3-30B-A3B shape)
+        if (a.nch > 32) a.nch = 32;
+        constexpr int ST = HD == 128 ? TSV_ATTN_STAGES2_HD128 : TSV_ATTN_STAGES2_HD64;
+        if (HD == 64 && trt >= 7)
+            rc = launch_partial_groups<HD, (HD == 64 ? 4 : 2), 2, 2>(s, a, G, R);
+        else if (HD == 64 && trt >= 5)
+            rc = launch_partial_groups<HD, (HD == 64 ? 3 : 2), 2, 2>(s, a, G, R);
+        else if (trt <= 4)
+            rc = launch_partial_groups<HD, 2, ST, 2>(s, a, G, R);
+        else if (trt <= 6)
+            rc = launch_partial_groups<HD, 2, ST, 3>(s, a, G, R);
+        else
+            rc = launch_partial_groups<HD, 2, ST, 4>(s, a, G, R);
+    }
     if (rc) return rc;
     return launch_combine<HD>(s, a, m, G, R);
 }

@@ -60,6 +60,12 @@ __device__ __forceinline__ void store_state(const float (&mrun)[RT], const float
 // rows of its second, v_permlane32_swap the upper half of the first with the lower half of the second, so with the
 // same value in both operands the two results hold the value of lane l and of its partner.  (Written as assembly:
 // the compiler folds max(result 0, result 1) of the builtin with equal operands into result 0.)
+__device__ __forceinline__ float max4(float a, float b, float c, float d) {
+    float r;
+    asm("v_max_f32 %0, %1, %2\n\tv_max3_f32 %0, %0, %3, %4" : "=&v"(r) : "v"(a), "v"(b), "v"(c), "v"(d));
+    return r;
+}
+constexpr float REF_SLACK = 8.0f;
 __device__ __forceinline__ float max_over_position_groups(float v) {
     float w = v;
     asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1" : "+v"(v), "+v"(w));
@@ -68,14 +74,19 @@ __device__ __forceinline__ float max_over_position_groups(float v) {
     return v;
 }
 
-// Eight waves per workgroup share a chunk of the context, each walking every eighth 16-position
-// block with up to STAGES blocks of K and V in flight.
+// The waves of a workgroup share a chunk of the context.  A pass of more than RT row tiles is split into TG tile
+// groups: wave w works on group w % TG (row tiles RT * group ..) and walks every NW-th 16-position block of the
+// chunk, NW = attn_phases(TG), starting at block w / TG, with up to STAGES blocks of K and V in flight.  The waves of
+// different groups that walk the same blocks run side by side on one compute unit, so a block comes out of the L2
+// once for all (row, q head) pairs of the pass.  (Legacy callers pass TG = 1 and their own rt0: eight waves, one group.)
 // COH: the query rows and the K / V blocks are read device-coherently (sc1), for a caller whose
 // other compute units wrote them earlier in the same kernel.
-// xch: [4 slots][PER_LANE values][64 lanes] floats of LDS.
-template <int HD, int RT, int STAGES, bool COH>
-__device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int R, int chunk, int h, int rt0, float* xch) {
-    constexpr int NW = 8;
+// xch: [TG][min(NW, 4) slots][PER_LANE values][64 lanes] floats of LDS.
+__host__ __device__ constexpr int attn_phases(int tg) { return tg == 1 ? 8 : tg == 2 ? 4 : 2; }
+
+template <int HD, int RT, int STAGES, bool COH, int TG = 1>
+__device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int R, int chunk, int h, int rt_first, float* xch) {
+    constexpr int NW = attn_phases(TG);
     constexpr int KS = HD / 32;  // K steps of the score MFMA
     constexpr int VT = HD / 16;  // output tiles along head_dim
     constexpr int PER_LANE = RT * VT * 4 + 2 * RT;
@@ -83,7 +94,9 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
 
     // (the wave index as a scalar: everything derived from it -- block numbers, the choice of variant -- then stays
     // on the scalar unit)
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tg = TG == 1 ? 0 : wave_in_wg % TG, wave = TG == 1 ? wave_in_wg : wave_in_wg / TG;  // wave: the phase
+    const int rt0 = rt_first + tg * RT;
     const int j = lane & 15, kg = lane >> 4;
     const VerifyParams* vp = a.vp;
     const int M = a.base_hint >= 0 ? a.m_hint : vp->m, base = a.base_hint >= 0 ? a.base_hint : vp->base, kvlen = base + M;
@@ -174,16 +187,24 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
     auto consume = [&](const Blk& st, int i) {
         const int p0 = (b0 + wave + NW * i) << 4;
         const bool tail = p0 + 16 > base;
+        // Three phases over the row tiles -- all score products, then the softmax steps, then all value products --
+        // so that the matrix pipe works through one tile's chain while the vector ALU is busy with another's.
+        float4v Sx[RT];
+        half4 Px[RT];
+#pragma unroll
+        for (int t = 0; t < RT; t++) Sx[t] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+#pragma unroll
+            for (int t = 0; t < RT; t++)
+                Sx[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, st.kf[s]),
+                                                               __builtin_bit_cast(half8, qf[t][s]), Sx[t], 0, 0, 0);
 #pragma unroll
         for (int t = 0; t < RT; t++) {
-            float4v S = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < KS; s++)
-                S = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, st.kf[s]),
-                                                           __builtin_bit_cast(half8, qf[t][s]), S, 0, 0, 0);
-            float sc[4];
-#pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) sc[i4] = S[i4] * c2;
+            const float4v S = Sx[t];
+            // (raw scores; they are scaled where they are used: the block maximum once, the weights by one fused
+            // multiply-add each -- exp2(S * c2 - reference))
+            float sc[4] = {S[0], S[1], S[2], S[3]};
             if (tail || p0 < cut_end) {  // (wave-uniform: a scalar branch)
                 // Visibility of this lane's four positions as a 4-bit word, computed without
                 // branches: bit (slot + 16) of `w` says whether cache slot base+slot is visible
@@ -200,34 +221,43 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
 #pragma unroll
                 for (int i4 = 0; i4 < 4; i4++) sc[i4] = ((vis4 >> i4) & 1u) ? sc[i4] : -INFINITY;
             }
-            const float mb = max_over_position_groups(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
-            const float mnew = fmaxf(mrun[t], mb);
-            // a row that has seen nothing yet (every position so far masked) has mnew = -inf: the differences below are
-            // taken against a finite stand-in, which makes every weight and the factor zero and leaves the empty state
-            const float mref = fmaxf(mnew, -3.0e38f);
-            const float alpha = __builtin_amdgcn_exp2f(mrun[t] - mref);
+            const float mb = max_over_position_groups(max4(sc[0], sc[1], sc[2], sc[3])) * c2;
+            // The reference the weights are taken against follows the row's maximum lazily: it moves only when the
+            // block's maximum passes it by more than REF_SLACK (in units of log 2), so a weight never exceeds
+            // 2^REF_SLACK -- far inside fp16 -- and the running sums are rescaled a handful of times per row instead of
+            // at every new maximum (a wave that walks eight blocks of random scores would otherwise rescale in nearly
+            // every one of them).  Any reference gives the same quotient; the decision is per row, from the row's own
+            // scores, so a row's bits do not depend on what shares its pass.
+            const bool grow = mb > mrun[t] + REF_SLACK;
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+                // a row that has seen nothing yet and sees nothing here (every position masked) keeps mrun = -inf:
+                // its factor is taken against a finite stand-in and comes out as zero, on empty sums
+                const float mnew = grow ? mb : mrun[t];
+                const float alpha = __builtin_amdgcn_exp2f(mrun[t] - fmaxf(mnew, -3.0e38f));  // exactly 1 where the row kept its reference
+                lrun[t] *= alpha;
+#pragma unroll
+                for (int d = 0; d < VT; d++) O[t][d] *= alpha;
+                mrun[t] = mnew;
+            }
+            const float nref = -fmaxf(mrun[t], -3.0e38f);
             half4 P;
             float ps = 0.f;
 #pragma unroll
             for (int i4 = 0; i4 < 4; i4++) {
-                const float p = __builtin_amdgcn_exp2f(sc[i4] - mref);
+                const float p = __builtin_amdgcn_exp2f(fmaf(sc[i4], c2, nref));
                 ps += p;
                 P[i4] = (_Float16)p;
             }
-            lrun[t] = fmaf(lrun[t], alpha, ps);
-            mrun[t] = mnew;
-            // once the running maximum has settled the factor is exactly 1 in every lane: the products are
-            // skipped then (the same bits), which is most blocks of a long context
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+            lrun[t] += ps;
+            Px[t] = P;
+        }
 #pragma unroll
-                for (int d = 0; d < VT; d++) O[t][d] *= alpha;
-            }
+        for (int d = 0; d < VT; d++) {
+            const u32x4 v2 = st.vf[d >> 1];
+            const u32x2 vd = (d & 1) ? u32x2{v2.z, v2.w} : u32x2{v2.x, v2.y};
 #pragma unroll
-            for (int d = 0; d < VT; d++) {
-                const u32x4 v2 = st.vf[d >> 1];
-                const u32x2 vd = (d & 1) ? u32x2{v2.z, v2.w} : u32x2{v2.x, v2.y};
-                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, vd), P, O[t][d], 0, 0, 0);
-            }
+            for (int t = 0; t < RT; t++)
+                O[t][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, vd), Px[t], O[t][d], 0, 0, 0);
         }
     };
     // Short runs are straight-line code (every load issued before the first wait, no load the run
@@ -268,16 +298,19 @@ __device__ __forceinline__ void attn_partial_body(const AttnArgs& a, int G, int 
             if (i + s < nb) consume(st[s], i + s);
     }
 
-    // fold the eight waves' running (m, l, O): 4..7 into 0..3, then 1..3 into 0
-    float* mine = xch + (wave & 3) * 64 * PER_LANE + lane;
-    if (wave >= 4) store_state<RT, VT>(mrun, lrun, O, mine);
-    __syncthreads();
-    if (wave < 4) merge_state<RT, VT, true>(mrun, lrun, O, mine);
-    __syncthreads();
-    if (wave >= 1 && wave < 4) store_state<RT, VT>(mrun, lrun, O, mine);
+    // fold the group's running (m, l, O): with eight phases 4..7 into 0..3 first, then 1.. into 0
+    constexpr int SLOTS = NW < 4 ? NW : 4;
+    float* grp = xch + tg * SLOTS * 64 * PER_LANE + lane;
+    if (NW == 8) {
+        if (wave >= 4) store_state<RT, VT>(mrun, lrun, O, grp + (wave & 3) * 64 * PER_LANE);
+        __syncthreads();
+        if (wave < 4) merge_state<RT, VT, true>(mrun, lrun, O, grp + wave * 64 * PER_LANE);
+        __syncthreads();
+    }
+    if (wave >= 1 && wave < 4) store_state<RT, VT>(mrun, lrun, O, grp + wave * 64 * PER_LANE);
     __syncthreads();
     if (wave != 0) return;
-    for (int w = 1; w < 4; w++) merge_state<RT, VT, true>(mrun, lrun, O, xch + w * 64 * PER_LANE + lane);
+    for (int w = 1; w < SLOTS; w++) merge_state<RT, VT, true>(mrun, lrun, O, grp + w * 64 * PER_LANE);
 #pragma unroll
     for (int t = 0; t < RT; t++) {
         float l = lrun[t];

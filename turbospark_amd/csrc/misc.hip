@@ -378,6 +378,7 @@ __global__ void k_kv_gather(uint16_t* const* caches, const int32_t* caps, int hd
     uint16_t* kc = caches[2 * blockIdx.y];
     uint16_t* vc = caches[2 * blockIdx.y + 1];
     const int max_ctx = caps[blockIdx.y];
+    if (max_ctx == 0) return;  // a layer without fp16 rows (quantized KV)
     const int h = blockIdx.x, d = threadIdx.x;
     for (int i = 0; i < n; i++) {
         const int src = (base + path[i]) % max_ctx, dst = (base + i) % max_ctx;

@@ -61,123 +61,118 @@ __device__ __forceinline__ float key_value(uint32_t key) {
     return __uint_as_float((key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key);
 }
 
-__global__ __launch_bounds__(1024) void k_route(MoeRouteArgs a) {
-    __shared__ int s_sel[TSV_MAX_ROWS * 8];  // the selected experts, pair index = row * k + slot
-    __shared__ uint32_t s_mask[256 * 4];     // per expert: which of the (at most 128) pairs chose it
+// The top-k of one row, by one wave: key[j] is the order key of expert lane + 64 j (0: absent).  Writes the row's
+// weights and selections.
+__device__ __forceinline__ void route_row(const MoeRouteArgs& a, int m, uint32_t (&key)[4], int lane) {
+    const int ne = a.n_experts, k = a.top_k;
+    float top = 0.f, sum = 0.f, my_ex = 0.f;
+    int my_sel = 0;
+    const bool forced = a.forced && a.forced[m * 8] >= 0;  // the same for the whole wave
+    if (forced) {
+        // lane r < k takes slot r's expert as given and fetches that expert's logit from the lane that holds it
+        const int e = min(max(lane < k ? a.forced[m * 8 + lane] : 0, 0), ne - 1);
+        float l = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float v = __shfl(key_value(key[j]), e & 63);
+            if ((e >> 6) == j) l = v;
+        }
+        top = key_value(wave_umax(lane < k ? order_key(l) : 0u));
+        my_ex = expf(l - top);
+        my_sel = e;
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+            if (r < k) sum += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_ex), r));
+    }
+#pragma unroll
+    for (int r = 0; r < 8; r++) {
+        if (r < k && !forced) {
+            const uint32_t mine = max(max(key[0], key[1]), max(key[2], key[3]));
+            const uint32_t kbest = wave_umax(mine);
+            uint32_t idx = 0xFFFFFFFFu;  // ascending j is ascending index: the first maximum wins
+#pragma unroll
+            for (int j = 3; j >= 0; j--)
+                if (key[j] == kbest) idx = (uint32_t)(lane + 64 * j);
+            const int bi = (int)min(wave_umin(idx), (uint32_t)(ne - 1));
+            const float best = key_value(kbest);
+            if (r == 0) top = best;
+            const float ex = expf(best - top);
+            sum += ex;  // sequential in rank order, as `exps.iter().sum()`
+            if (lane == r) {  // lane r keeps slot r
+                my_ex = ex;
+                my_sel = bi;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (lane + 64 * j == bi) key[j] = 0;
+        }
+    }
+    if (lane < k) {
+        a.weights[m * 8 + lane] = my_ex / sum;
+        a.selected[m * 8 + lane] = my_sel;
+    }
+}
+
+// Router matmul and top-k in one kernel: a workgroup of sixteen waves per group of four rows.  The waves split
+// the router's tiles and K chunks among them (the dense matmul's own tile sequences, one row group), their sums
+// are folded through LDS in wave order, and wave i of the first four then ranks row 4 g + i.  The groups of
+// rows that share an expert are not built here: every expert matmul workgroup derives its own from the
+// selections (moe_derive_group), which takes a wave a few dozen instructions.
+template <class F>
+__global__ __launch_bounds__(1024) void k_route_fused(MoeRouteArgs a) {
+    __shared__ float4v red[16 * 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int M = a.m, ne = a.n_experts, k = a.top_k;
-    for (int i = threadIdx.x; i < ne * 4; i += blockDim.x) s_mask[i] = 0;
+    const int g = blockIdx.x, nt = a.n_tiles, parts = 16 / nt;
+    const int tile = wave % nt, part = wave / nt;
+    const int per = (a.kchunks + parts - 1) / parts;
+    const int c0 = min(part * per, a.kchunks), nc = min(per, a.kchunks - c0);
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * F::TILE_BYTES;
+    Consts k;
+    k.k6400 = 0x64006400u;
+    k.k5400 = 0x54005400u;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
+    ActLoader<false> x(a.xfrag, a.xsum, lane);
+    x.set_row(0, 4 * g + (lane & 3));
+    float4v acc[1] = {float4v{0.f, 0.f, 0.f, 0.f}};
+    if (nc > 0) {
+        Stage<F, 1> st[2];
+        const int last = c0 + nc - 1;
+        auto fetch = [&](Stage<F, 1>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
+        fetch(st[0], c0);
+        fetch(st[1], min(c0 + 1, last));
+        int c = 0;
+        for (; c + 4 <= nc; c += 2) {
+            compute(st[0], k, acc);
+            fetch(st[0], c0 + c + 2);
+            compute(st[1], k, acc);
+            fetch(st[1], c0 + c + 3);
+        }
+        for (int s2 = 0; s2 < 2; s2++)
+            if (c + s2 < nc) {
+                compute(st[s2], k, acc);
+                if (c + s2 + 2 < nc) fetch(st[s2], c0 + c + s2 + 2);
+            }
+        c += 2;
+        for (int s2 = 0; s2 < 2; s2++)
+            if (c + s2 < nc) compute(st[s2], k, acc);
+    }
+    red[wave * 64 + lane] = acc[0];
     __syncthreads();
-    if (wave < M) {
-        const int m = wave;
-        uint32_t key[4] = {0u, 0u, 0u, 0u};
-        // every partial sum of every expert this lane holds is asked for before the first add: the loads
-        // have no branch between them (a lane past the last expert reads the last expert's, a split past
-        // the last split the last split's again), so they are one round trip, not one per expert block
-        auto gather = [&](auto NJ) {
-            constexpr int nj = decltype(NJ)::value;
-            float part[nj][8], bias[nj];
+    const int m = 4 * g + wave;
+    if (wave >= 4 || m >= a.m) return;
+    uint32_t key[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int j = 0; j < nj; j++) {
-                const int e = min(lane + 64 * j, ne - 1);
-#pragma unroll
-                for (int sp = 0; sp < 8; sp++) part[j][sp] = a.logits[((size_t)min(sp, a.splits - 1) * 16 + m) * a.ld + e];
-                bias[j] = a.bias ? a.bias[e] : 0.f;  // before the top-k (families/gptoss/moe.rs:82-87)
-            }
-#pragma unroll
-            for (int j = 0; j < nj; j++) {
-                float s = 0.f;  // added in split order
-#pragma unroll
-                for (int sp = 0; sp < 8; sp++) s += sp < a.splits ? part[j][sp] : 0.f;
-                if (a.bias) s += bias[j];
-                if (lane + 64 * j < ne) key[j] = order_key(s);
-            }
-        };
-        if (ne <= 128)
-            gather(std::integral_constant<int, 2>{});
-        else
-            gather(std::integral_constant<int, 4>{});
-        float top = 0.f, sum = 0.f, my_ex = 0.f;
-        int my_sel = 0;
-        const bool forced = a.forced && a.forced[m * 8] >= 0;  // the same for the whole wave
-        if (forced) {
-            // lane r < k takes slot r's expert as given and fetches that expert's logit from the lane that holds it
-            const int e = min(max(lane < k ? a.forced[m * 8 + lane] : 0, 0), ne - 1);
-            float l = 0.f;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float v = __shfl(key_value(key[j]), e & 63);
-                if ((e >> 6) == j) l = v;
-            }
-            top = key_value(wave_umax(lane < k ? order_key(l) : 0u));
-            my_ex = expf(l - top);
-            my_sel = e;
-#pragma unroll
-            for (int r = 0; r < 8; r++)
-                if (r < k) sum += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_ex), r));
-        }
-#pragma unroll
-        for (int r = 0; r < 8; r++) {
-            if (r < k && !forced) {
-                const uint32_t mine = max(max(key[0], key[1]), max(key[2], key[3]));
-                const uint32_t kbest = wave_umax(mine);
-                uint32_t idx = 0xFFFFFFFFu;  // ascending j is ascending index: the first maximum wins
-#pragma unroll
-                for (int j = 3; j >= 0; j--)
-                    if (key[j] == kbest) idx = (uint32_t)(lane + 64 * j);
-                const int bi = (int)min(wave_umin(idx), (uint32_t)(ne - 1));
-                const float best = key_value(kbest);
-                if (r == 0) top = best;
-                const float ex = expf(best - top);
-                sum += ex;  // sequential in rank order, as `exps.iter().sum()`
-                if (lane == r) {  // lane r keeps slot r
-                    my_ex = ex;
-                    my_sel = bi;
-                }
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (lane + 64 * j == bi) key[j] = 0;
-            }
-        }
-        if (lane < k) {
-            a.weights[m * 8 + lane] = my_ex / sum;
-            a.selected[m * 8 + lane] = my_sel;
-            s_sel[m * k + lane] = my_sel;
-            const int pair = m * k + lane;
-            atomicOr(&s_mask[my_sel * 4 + (pair >> 5)], 1u << (pair & 31));
+    for (int j = 0; j < 4; j++) {
+        if (j < nt) {
+            float sum = 0.f;  // the K parts in order
+            for (int p = 0; p < parts; p++) sum += red[(p * nt + j) * 64 + lane][wave];
+            const int e = lane + 64 * j;
+            if (a.bias && e < a.n_experts) sum += a.bias[e];  // before the top-k (families/gptoss/moe.rs:82-87)
+            if (e < a.n_experts) key[j] = order_key(sum);
         }
     }
-    __syncthreads();
-    // Groups: pair j leads the group of its expert when no earlier pair chose it; the members of a
-    // group are listed in pair order.  Every pair has set its bit in its expert's membership mask: a
-    // pair's place is the number of set bits below its own, the group's leader the lowest set bit,
-    // the group's size the number of set bits.
-    const int j = threadIdx.x, np = M * k;
-    if (j >= np) return;
-    const int e = s_sel[j];
-    const uint32_t m0 = s_mask[e * 4], m1 = s_mask[e * 4 + 1], m2 = s_mask[e * 4 + 2], m3 = s_mask[e * 4 + 3];
-    const int cnt = __popc(m0) + __popc(m1) + __popc(m2) + __popc(m3);
-    const int first = m0 ? __ffs(m0) - 1 : m1 ? 31 + __ffs(m1) : m2 ? 63 + __ffs(m2) : 95 + __ffs(m3);
-    const uint32_t below = (1u << (j & 31)) - 1u;
-    const int w = j >> 5;
-    const int pos = (w > 0 ? __popc(m0) : 0) + (w > 1 ? __popc(m1) : 0) + (w > 2 ? __popc(m2) : 0) +
-                    __popc((w == 0 ? m0 : w == 1 ? m1 : w == 2 ? m2 : m3) & below);
-    const int row = j / k;
-    if (pos < TSV_MAX_ROWS) {  // a row chooses an expert once, so a group never has more members than rows
-        MoeGroup* lead = a.groups + first;
-        lead->rows[pos] = row;
-        lead->slots[pos] = j - row * k;
-        // the last member also fills the entries past the count: a reader that takes entry n without
-        // looking at the count first then finds a row of the group, never a stale one
-        if (pos == cnt - 1)
-            for (int p = cnt; p < TSV_MAX_ROWS; p++) {
-                lead->rows[p] = row;
-                lead->slots[p] = j - row * k;
-            }
-    }
-    MoeGroup* g = a.groups + j;
-    g->expert = e;
-    g->cnt = first == j ? min(cnt, TSV_MAX_ROWS) : 0;
+    route_row(a, m, key, lane);
 }
 
 // ---- grouped expert matmul --------------------------------------------------------------------
@@ -299,7 +294,7 @@ __global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
     extern __shared__ float4v red[];
     __shared__ MoeGroup grp;
     const int gi = blockIdx.y, r0 = 4 * blockIdx.z;
-    if (threadIdx.x < sizeof(MoeGroup) / 4) ((int32_t*)&grp)[threadIdx.x] = ((const int32_t*)(a.groups + gi))[threadIdx.x];
+    if (threadIdx.x < 64) moe_derive_group(&grp, a.selected, a.rows, a.top_k, gi, threadIdx.x);
     __syncthreads();
     if (r0 >= grp.cnt) return;
     expert_tile<F, EPI, STAGES>(a, grp, gi, r0, red);
@@ -337,14 +332,24 @@ int launch_moe_f(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
 
 }  // namespace
 
-int launch_route(hipStream_t s, const MoeRouteArgs& a) {
+int launch_route(hipStream_t s, int fmt, const MoeRouteArgs& a) {
     if (a.n_experts > 256 || a.top_k < 1 || a.top_k > 8 || a.top_k > a.n_experts) {
         set_error("moe: at most 256 experts and top-k between 1 and 8");
         return TSV_ERR_UNSUPPORTED;
     }
-    // one wave per row for the top-k, one thread per (row, slot) pair for the groups
-    const int threads = std::max(64 * a.m, (a.m * a.top_k + 63) / 64 * 64);
-    hipLaunchKernelGGL(k_route, dim3(1), dim3(std::min(1024, threads)), 0, s, a);
+    if (a.n_tiles != 1 && a.n_tiles != 2 && a.n_tiles != 4) {
+        set_error("moe: the router's experts must fill one, two or four 64-row tiles");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((a.m + 3) / 4), block(1024);
+    switch (fmt) {
+        case FMT_Q4K: hipLaunchKernelGGL(k_route_fused<Q4K>, grid, block, 0, s, a); break;
+        case FMT_Q80: hipLaunchKernelGGL(k_route_fused<Q80>, grid, block, 0, s, a); break;
+        case FMT_Q6K: hipLaunchKernelGGL(k_route_fused<Q6K>, grid, block, 0, s, a); break;
+        case FMT_Q5K: hipLaunchKernelGGL(k_route_fused<Q5K>, grid, block, 0, s, a); break;
+        case FMT_BF16: hipLaunchKernelGGL(k_route_fused<BF16W>, grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL(k_route_fused<MX4>, grid, block, 0, s, a); break;
+    }
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -109,10 +109,13 @@ __global__ __launch_bounds__(512) void k_moe_fp4(MoeGemmArgs a) {
     const int gi = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int n = lane & 15, g = lane >> 4;
-    // the group's header and this lane's member, asked for together.  Entries past the group's count
-    // repeat its last member (k_route fills them): such a lane multiplies that row again, from the
-    // same cache lines, and its column of D is dropped.
-    const MoeGroup* grp = a.groups + gi;
+    // the group of this workgroup's pair, derived from the rows' selections by the first wave.  Entries past the
+    // group's count repeat its last member: such a lane multiplies that row again, from the same cache lines,
+    // and its column of D is dropped.
+    __shared__ MoeGroup grp_s;
+    if (threadIdx.x < 64) moe_derive_group(&grp_s, a.selected, a.rows, a.top_k, gi, threadIdx.x);
+    __syncthreads();
+    const MoeGroup* grp = &grp_s;
     const int cnt = grp->cnt, e = grp->expert, my_row = grp->rows[n], my_slot = grp->slots[n];
     if (cnt == 0) return;
     const int tile = blockIdx.x;

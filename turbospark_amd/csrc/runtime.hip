@@ -74,7 +74,6 @@ struct tsv_ctx {
     float* route_w = nullptr;
     int32_t* route_sel = nullptr;
     int32_t* route_forced = nullptr;  // test hook (tsv_force_route): [n_layers][16][8], negative = route freely
-    MoeGroup* route_groups = nullptr;
     uint8_t* frag_e = nullptr;
     size_t frag_e_stride = 0;
     float* moe_out = nullptr;
@@ -92,7 +91,7 @@ struct tsv_ctx {
         size_t xfb = 0;
         float* partial = nullptr;
         uint16_t* q16 = nullptr;
-        VerifyParams *vp = nullptr, *vp_host = nullptr;
+        VerifyParams* vp = nullptr;
         float2* rope_cs = nullptr;
         float *part_o = nullptr, *part_ml = nullptr;  // attention partials of every block
         size_t part_o_stride = 0, part_ml_stride = 0;
@@ -103,6 +102,16 @@ struct tsv_ctx {
     uint16_t* logits = nullptr;       // [16][vocab] fp16, device
     uint16_t* draft_stage = nullptr;  // [16][vocab] fp16, device
     VerifyParams *vp_dev = nullptr, *vp_host = nullptr;
+    // Pinned staging slots of the per-pass parameters (four 16-row blocks each), used round robin: a slot is
+    // rewritten only once the copy that last read it has completed (its event), so consecutive passes queue
+    // without the host waiting for the stream.
+    struct ParamRing {
+        static constexpr int SLOTS = 8, PER_SLOT = 4;
+        VerifyParams* host = nullptr;
+        hipEvent_t ev[SLOTS] = {};
+        bool used[SLOTS] = {};
+        int next = 0;
+    } ring;
     AcceptParams *ap_dev = nullptr, *ap_host = nullptr;
     uint16_t** kv_ptrs = nullptr;  // device: [2 * layer] = K buffer, [2 * layer + 1] = V buffer (tree compaction)
     int32_t* hist_dev = nullptr;  // the token history of a penalised round (grows on demand)
@@ -405,6 +414,20 @@ int fill_params(VerifyParams& vp, const int32_t* feed, const int32_t* parent, in
 
 int run_pass(tsv_ctx* c, int m);
 
+// n parameter blocks to `dev` through the next pinned staging slot, on the handle's stream.
+int stage_params(tsv_ctx* c, const VerifyParams* vp, int n, VerifyParams* dev) {
+    auto& r = c->ring;
+    const int i = r.next;
+    r.next = (i + 1) % tsv_ctx::ParamRing::SLOTS;
+    if (r.used[i]) TSV_HIP(hipEventSynchronize(r.ev[i]));
+    VerifyParams* slot = r.host + (size_t)i * tsv_ctx::ParamRing::PER_SLOT;
+    std::memcpy(slot, vp, (size_t)n * sizeof(VerifyParams));
+    TSV_HIP(hipMemcpyAsync(dev, slot, (size_t)n * sizeof(VerifyParams), hipMemcpyHostToDevice, c->stream));
+    TSV_HIP(hipEventRecord(r.ev[i], c->stream));
+    r.used[i] = true;
+    return TSV_OK;
+}
+
 // One verify pass: enqueue everything on the handle's stream; no synchronisation.
 int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m, int64_t base) {
     TSV_NEED(c, "verify: null handle");
@@ -428,11 +451,9 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     VerifyParams vp;
     int prc = fill_params(vp, feed, parent, m, base, c->vocab);
     if (prc) return prc;
-    hipStream_t s = c->stream;
-    // the pinned staging copy must not be rewritten while an earlier copy is still in flight
-    TSV_HIP(hipStreamSynchronize(s));
-    *c->vp_host = vp;
-    TSV_HIP(hipMemcpyAsync(c->vp_dev, c->vp_host, sizeof vp, hipMemcpyHostToDevice, s));
+    *c->vp_host = vp;  // the host's own copy of the pass in flight
+    int prc2 = stage_params(c, &vp, 1, c->vp_dev);
+    if (prc2) return prc2;
     int rc = run_pass(c, m);
     if (rc) return rc;
     c->position = base + m;
@@ -605,17 +626,17 @@ int launch_pass(tsv_ctx* c, int m) {
         if (L.n_experts) {
             // router -> top-k -> grouped expert matmuls; the per-slot outputs are added, weighted
             // and in slot order, by the next residual kernel
-            const int rsp = splits_for(L.router, m, EPI_PARTIAL);
             MoeRouteArgs ra2{};
-            ra2.logits = c->partial;
-            ra2.splits = rsp;
-            ra2.ld = L.n_experts;
+            ra2.w = L.router.tiles;
+            ra2.n_tiles = L.router.n_tiles;
+            ra2.kchunks = L.router.kchunks;
+            ra2.xfrag = (const uint2*)c->xf_a;
+            ra2.xsum = (const float*)((const char*)c->xf_a + xfrag_sum_offset(c->hidden));
             ra2.n_experts = L.n_experts;
             ra2.top_k = L.top_k;
             ra2.m = m;
             ra2.weights = c->route_w;
             ra2.selected = c->route_sel + (size_t)l * 16 * 8;  // kept per layer: tsv_route_selected reads them back
-            ra2.groups = c->route_groups;
             ra2.bias = L.router_bias;
             ra2.forced = c->route_forced + (size_t)l * 16 * 8;
             MoeGemmArgs g1{}, g2{};
@@ -629,7 +650,8 @@ int launch_pass(tsv_ctx* c, int m) {
             g1.out = c->frag_e;
             g1.out_stride = c->frag_e_stride;
             g1.n_out = c->ffn;
-            g1.groups = c->route_groups;
+            g1.selected = ra2.selected;
+            g1.top_k = L.top_k;
             g1.bias = L.be_gate;
             g1.bias2 = L.be_up;
             g1.alpha = c->act_alpha;
@@ -663,9 +685,7 @@ int launch_pass(tsv_ctx* c, int m) {
                 PROF(PC_GATEUP);
                 rc = 0;
                 for (int rep = 0; rep < c->repeat[PC_GATEUP] && !rc; rep++) {
-                    rc = launch_gemm(s, L.router, c->xf_a, c->partial, c->vp_dev, m, rsp, EPI_PARTIAL, L.n_experts,
-                                     L.n_experts);
-                    if (!rc) rc = launch_route(s, ra2);
+                    rc = launch_route(s, L.router.fmt, ra2);
                     if (!rc) rc = fp4 ? launch_moe_fp4_gate_up(s, g1, n_groups) : launch_moe_gate_up(s, L.gate_up.fmt, g1, n_groups);
                 }
             }
@@ -749,10 +769,6 @@ int wide_prepare(tsv_ctx* c) {
     w.part_ml_stride = (size_t)c->nkv * c->nch * rows_max * 2;
     if ((rc = dev_alloc(c, &w.part_o, WIDE_B * w.part_o_stride * 4, true)) || (rc = dev_alloc(c, &w.part_ml, WIDE_B * w.part_ml_stride * 4, true)))
         return rc;
-    if (hipHostMalloc((void**)&w.vp_host, WIDE_B * sizeof(VerifyParams)) != hipSuccess) {
-        set_error("prefill: cannot allocate pinned staging memory");
-        return TSV_ERR_DEVICE;
-    }
     w.ready = true;
     return TSV_OK;
 }
@@ -866,10 +882,8 @@ int enqueue_wide_prefill(tsv_ctx* c, const int32_t* ids, int64_t base) {
     VerifyParams vp[WIDE_B];
     for (int b = 0; b < WIDE_B; b++)
         if ((rc = fill_params(vp[b], ids + 16 * b, nullptr, 16, base + 16 * b, c->vocab))) return rc;
-    hipStream_t s = c->stream;
-    TSV_HIP(hipStreamSynchronize(s));  // the pinned staging copy must not be rewritten while a copy is in flight
-    std::memcpy(c->wide.vp_host, vp, sizeof vp);
-    TSV_HIP(hipMemcpyAsync(c->wide.vp, c->wide.vp_host, sizeof vp, hipMemcpyHostToDevice, s));
+    static_assert(WIDE_B <= tsv_ctx::ParamRing::PER_SLOT, "a staging slot holds a prompt pass's blocks");
+    if ((rc = stage_params(c, vp, WIDE_B, c->wide.vp))) return rc;
     if ((rc = launch_wide_pass(c, base))) return rc;
     c->position = base + rows;
     c->high_water = std::max(c->high_water, c->position);
@@ -1041,7 +1055,6 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             L.top_k = s.top_k;
             if (L.gate_up.fmt != FMT_MX4 || L.down.fmt != FMT_MX4) c->moe_fp4_terms = 0;
             c->max_experts = std::max(c->max_experts, ne);
-            pneed = std::max(pneed, partial_need(L.router));
         } else {
             if ((rc = check_matrix(s.w_gate, c->ffn, c->hidden, "w_gate")) ||
                 (rc = check_matrix(s.w_up, c->ffn, c->hidden, "w_up")) ||
@@ -1150,7 +1163,9 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         if (hipMemcpy(c->kv_ptrs, ptrs.data(), ptrs.size() * sizeof(uint16_t*), hipMemcpyHostToDevice) != hipSuccess)
             return fail(TSV_ERR_DEVICE);
         std::vector<int32_t> caps;
-        for (auto& L : c->layers) caps.push_back(L.kv_slots);  // a quantized layer: its fp16 side is the staging slots
+        // a quantized layer holds no fp16 rows to move (its staging slots are shared by all such layers and are dead
+        // once the pass has quantized them; launch_tq_gather moves its stored rows): capacity 0, the gather skips it
+        for (auto& L : c->layers) caps.push_back(L.tq.k_bits ? 0 : L.kv_slots);
         if ((rc = dev_alloc(c, &c->kv_caps, caps.size() * 4))) return fail(rc);
         if (hipMemcpy(c->kv_caps, caps.data(), caps.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return fail(TSV_ERR_DEVICE);
     }
@@ -1255,7 +1270,6 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         (c->max_experts &&
          ((rc = dev_alloc(c, &c->route_w, 16 * 8 * 4, true)) || (rc = dev_alloc(c, &c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, true)) ||
           (rc = dev_alloc(c, &c->route_forced, (size_t)c->n_layers * 16 * 8 * 4)) ||
-          (rc = dev_alloc(c, &c->route_groups, (size_t)TSV_MAX_ROWS * 8 * sizeof(MoeGroup), true)) ||
           (rc = dev_alloc(c, &c->frag_e, (size_t)TSV_MAX_ROWS * 8 * (c->frag_e_stride = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255), true)) ||
           (rc = dev_alloc(c, &c->moe_out, (size_t)8 * 16 * c->hidden * 4, true)) ||
           (c->moe_fp4_terms &&
@@ -1281,13 +1295,20 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         return fail(rc);
     if (c->route_forced && hipMemsetAsync(c->route_forced, 0xFF, (size_t)c->n_layers * 16 * 8 * 4, c->stream) != hipSuccess)
         return fail(TSV_ERR_DEVICE);  // every entry -1: rows route freely until tsv_force_route says otherwise
-    if (hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
+    for (hipEvent_t& e : c->ring.ev)
+        if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+            set_error("open: event creation failed");
+            return fail(TSV_ERR_DEVICE);
+        }
+    if (hipHostMalloc((void**)&c->ring.host, sizeof(VerifyParams) * tsv_ctx::ParamRing::SLOTS * tsv_ctx::ParamRing::PER_SLOT) != hipSuccess ||
+        hipHostMalloc((void**)&c->vp_host, sizeof(VerifyParams)) != hipSuccess ||
         hipHostMalloc((void**)&c->ap_host, sizeof(AcceptParams)) != hipSuccess ||
         hipHostMalloc((void**)&c->res_host, sizeof(AcceptResult)) != hipSuccess ||
         hipHostMalloc((void**)&c->tok_host, 64 * 4) != hipSuccess) {
         set_error("open: pinned host allocation failed");
         return fail(TSV_ERR_DEVICE);
     }
+    if (int nrc = noalloc_prepare_device()) return fail(nrc);  // tsv_accept_greedy_noalloc is capturable from here on
     if (hipStreamSynchronize(c->stream) != hipSuccess) {
         set_error("open: device initialisation failed");
         return fail(TSV_ERR_DEVICE);
@@ -1309,7 +1330,9 @@ extern "C" void tsv_close(tsv_ctx* c) {
     for (void* p : c->allocs) (void)hipFree(p);
     if (c->hist_dev) (void)hipFree(c->hist_dev);
     if (c->vp_host) (void)hipHostFree(c->vp_host);
-    if (c->wide.vp_host) (void)hipHostFree(c->wide.vp_host);
+    if (c->ring.host) (void)hipHostFree(c->ring.host);
+    for (hipEvent_t e : c->ring.ev)
+        if (e) (void)hipEventDestroy(e);
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);

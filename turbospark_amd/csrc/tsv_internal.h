@@ -191,18 +191,53 @@ struct MoeGroup {
     int32_t rows[16], slots[16];
 };
 struct MoeRouteArgs {
-    const float* logits;  // router matmul partials [splits][16][ld]
-    int splits, ld, n_experts, top_k;
+    const uint8_t* w;     // the router's tiled weights: n_tiles tiles of 64 experts x kchunks
+    int n_tiles, kchunks;
+    const uint2* xfrag;   // the pass's activation fragments and their sub-block sums
+    const float* xsum;
+    int n_experts, top_k;
     int m;              // rows of the pass (the launch sequence is per row count)
     float* weights;     // [16][8] softmax over the selected logits, rank order
     int32_t* selected;  // [16][8] expert ids, rank order
-    MoeGroup* groups;   // [16 * 8]
     const float* bias;  // nullable: n_experts values added to the logits before the top-k
     // nullable test hook: [16][8] expert ids a row is to take instead of its own top-k (slot order as
     // given, the weights still the softmax of the row's own logits over them); a row whose first
     // entry is negative routes freely
     const int32_t* forced;
 };
+// The group of pair gi (row gi / k, slot gi % k) from the rows' selections, by one whole wave (lane = threadIdx.x
+// < 64) into *g: the expert, the rows that chose it in pair order with the slot it has in each, and cnt != 0 only
+// where pair gi is the first to name the expert.  Entries past the count repeat the last member, so a reader that
+// takes entry n without looking at the count finds a row of the group.
+__device__ __forceinline__ void moe_derive_group(MoeGroup* g, const int32_t* selected, int m, int k, int gi, int lane) {
+    const int np = m * k, p0 = lane, p1 = lane + 64;
+    const int e0 = p0 < np ? selected[(p0 / k) * 8 + p0 % k] : -1;
+    const int e1 = p1 < np ? selected[(p1 / k) * 8 + p1 % k] : -2;
+    const int ea = __builtin_amdgcn_readlane(e0, gi & 63), eb = __builtin_amdgcn_readlane(e1, gi & 63);
+    const int e = gi < 64 ? ea : eb;
+    const uint64_t m0 = __builtin_amdgcn_ballot_w64(e0 == e), m1 = __builtin_amdgcn_ballot_w64(e1 == e);
+    const int c0 = __popcll(m0), cnt = c0 + __popcll(m1);
+    const int first = m0 ? __ffsll((long long)m0) - 1 : 63 + __ffsll((long long)m1);
+    const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        if ((h ? e1 : e0) != e) continue;
+        const int p = h ? p1 : p0, pos = h ? c0 + __popcll(m1 & below) : __popcll(m0 & below);
+        if (pos >= TSV_MAX_ROWS) continue;  // a row chooses an expert once: never more members than rows
+        const int row = p / k, slot = p - row * k;
+        g->rows[pos] = row;
+        g->slots[pos] = slot;
+        if (pos == cnt - 1)
+            for (int q = cnt; q < TSV_MAX_ROWS; q++) {
+                g->rows[q] = row;
+                g->slots[q] = slot;
+            }
+    }
+    if (lane == 0) {
+        g->expert = e;
+        g->cnt = first == gi ? min(cnt, TSV_MAX_ROWS) : 0;
+    }
+}
 // Block-scaled fp8 activations: the B operand of the scaled-MFMA expert matmuls (MXFP4 experts).  A
 // value is the sum of `terms` e4m3 numbers, each times the power-of-two scale of its 32-element
 // block; term t holds what the terms before it left over, so three terms carry about 2^-13 of the
@@ -214,7 +249,10 @@ struct X8 {
     int kpad;    // K rounded up to whole 256-element chunks; the tail stays zero from the allocation
 };
 constexpr int X8_MAX_TERMS = 3;
-constexpr int MOE_FP4_DEFAULT_TERMS = 2;  // what a context uses unless TSV_MOE_FP4 says otherwise
+// What a context uses unless TSV_MOE_FP4 says otherwise.  Three: with two terms the Qwen3-30B-A3B configuration at its
+// full depth (48 layers) came out 1.2e-2 of the logit range away from the oracle under the oracle's own routing -- past
+// the 1e-2 the path is held to -- against 3.4e-3 with three terms and 5.5e-3 with fp16 activations.
+constexpr int MOE_FP4_DEFAULT_TERMS = 3;
 inline size_t x8_q_bytes(int k) { return (size_t)X8_MAX_TERMS * 16 * ((k + 255) / 256 * 256); }
 inline size_t x8_s_bytes(int k) { return x8_q_bytes(k) / 32; }
 
@@ -232,14 +270,15 @@ struct MoeGemmArgs {
     void* out;             // gate/up: per-group fragments of silu(gate) * up; down: float [8 slots][16][n_out]
     size_t out_stride;
     int n_out;             // gate/up: expert FFN width; down: hidden
-    const MoeGroup* groups;
+    const int32_t* selected;  // [16][8] expert ids the rows chose (k_route_fused): the groups are derived from them
+    int top_k;
     // nullable per-expert biases, [n_experts][n_out]: gate/up use bias (gate) and bias2 (up), added
     // before the activation; down uses bias, added before the slot is weighted
     const float* bias;
     const float* bias2;
     float alpha, limit;    // alpha > 0: clamped SwiGLU (moe_gguf.metal:528-556) instead of silu(g) * u
 };
-int launch_route(hipStream_t s, const MoeRouteArgs& a);
+int launch_route(hipStream_t s, int fmt, const MoeRouteArgs& a);
 int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 // the same two matmuls on v_mfma_scale_f32_16x16x128_f8f6f4 (moe_fp4.hip)
@@ -440,6 +479,7 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
                   const AcceptParams& ap_host, const AcceptScratch& sc);
 int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,
                        const AcceptParams& ap_host, const AcceptScratch& sc, int32_t* proposals_dev);
+int noalloc_prepare_device();
 int launch_pen_counts(hipStream_t s, const int32_t* history_dev, long n, long suffix_start, int vocab, uint32_t* cnt);
 
 // ---- host utilities ----------------------------------------------------------------------

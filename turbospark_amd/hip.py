@@ -21,6 +21,14 @@ def rt():
         L.hipEventDestroy.argtypes = [C.c_void_p]
         L.hipStreamSynchronize.argtypes = [C.c_void_p]
         L.hipGetDeviceCount.argtypes = [C.POINTER(C.c_int)]
+        L.hipStreamCreateWithFlags.argtypes = [C.POINTER(C.c_void_p), C.c_uint]
+        L.hipStreamDestroy.argtypes = [C.c_void_p]
+        L.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        L.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        L.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        L.hipGraphDestroy.argtypes = [C.c_void_p]
+        L.hipGraphExecDestroy.argtypes = [C.c_void_p]
         _rt = L
     return _rt
 
@@ -82,3 +90,43 @@ class Event:
     def __del__(self):
         if self.h:
             rt().hipEventDestroy(self.h)
+
+
+class Stream:
+    """A non-blocking stream of the caller's own (graph capture needs one: the NULL stream cannot be captured)."""
+
+    def __init__(self):
+        self.h = C.c_void_p()
+        check(rt().hipStreamCreateWithFlags(C.byref(self.h), 1), "hipStreamCreateWithFlags")
+
+    def sync(self):
+        check(rt().hipStreamSynchronize(self.h), "hipStreamSynchronize")
+
+    def __del__(self):
+        if self.h:
+            rt().hipStreamDestroy(self.h)
+
+
+class CapturedGraph:
+    """What `record(stream)` enqueues on `stream`, captured once (thread-local mode) and replayable."""
+
+    def __init__(self, stream, record):
+        g = C.c_void_p()
+        check(rt().hipStreamBeginCapture(stream.h, 1), "hipStreamBeginCapture")
+        try:
+            record(stream)
+        finally:
+            code = rt().hipStreamEndCapture(stream.h, C.byref(g))
+        check(code, "hipStreamEndCapture")
+        self.exe = C.c_void_p()
+        code = rt().hipGraphInstantiate(C.byref(self.exe), g, None, None, 0)
+        rt().hipGraphDestroy(g)
+        check(code, "hipGraphInstantiate")
+        self.stream = stream
+
+    def launch(self):
+        check(rt().hipGraphLaunch(self.exe, self.stream.h), "hipGraphLaunch")
+
+    def __del__(self):
+        if getattr(self, "exe", None):
+            rt().hipGraphExecDestroy(self.exe)
