@@ -63,14 +63,17 @@ __device__ __forceinline__ float key_value(uint32_t key) {
 
 // The top-k of one row, by one wave: key[j] is the order key of expert lane + 64 j (0: absent).  Writes the row's
 // weights and selections.
-__device__ __forceinline__ void route_row(const MoeRouteArgs& a, int m, uint32_t (&key)[4], int lane) {
+// `forced_first` / `forced_mine`: a.forced[m * 8] and a.forced[m * 8 + lane] (lane < k), asked for by the caller before its
+// matmul so that they are not one more memory round trip here.
+__device__ __forceinline__ void route_row(const MoeRouteArgs& a, int m, uint32_t (&key)[4], int lane, int forced_first,
+                                          int forced_mine) {
     const int ne = a.n_experts, k = a.top_k;
     float top = 0.f, sum = 0.f, my_ex = 0.f;
     int my_sel = 0;
-    const bool forced = a.forced && a.forced[m * 8] >= 0;  // the same for the whole wave
+    const bool forced = forced_first >= 0;  // the same for the whole wave
     if (forced) {
         // lane r < k takes slot r's expert as given and fetches that expert's logit from the lane that holds it
-        const int e = min(max(lane < k ? a.forced[m * 8 + lane] : 0, 0), ne - 1);
+        const int e = min(max(lane < k ? forced_mine : 0, 0), ne - 1);
         float l = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -134,6 +137,13 @@ __global__ __launch_bounds__(1024) void k_route_fused(MoeRouteArgs a) {
     asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
     ActLoader<false> x(a.xfrag, a.xsum, lane);
     x.set_row(0, 4 * g + (lane & 3));
+    // what the ranking needs besides the logits, asked for now (row 4 g + wave; waves past the fourth read row 4 g's)
+    const int mrow = min(4 * g + (wave & 3), TSV_MAX_ROWS - 1);
+    const int forced_first = a.forced ? a.forced[mrow * 8] : -1;
+    const int forced_mine = a.forced ? a.forced[mrow * 8 + (lane & 7)] : -1;
+    float bias[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) bias[j] = a.bias ? a.bias[min(lane + 64 * j, a.n_experts - 1)] : 0.f;
     float4v acc[1] = {float4v{0.f, 0.f, 0.f, 0.f}};
     if (nc > 0) {
         Stage<F, 1> st[2];
@@ -168,11 +178,11 @@ __global__ __launch_bounds__(1024) void k_route_fused(MoeRouteArgs a) {
             float sum = 0.f;  // the K parts in order
             for (int p = 0; p < parts; p++) sum += red[(p * nt + j) * 64 + lane][wave];
             const int e = lane + 64 * j;
-            if (a.bias && e < a.n_experts) sum += a.bias[e];  // before the top-k (families/gptoss/moe.rs:82-87)
+            if (a.bias) sum += bias[j];  // before the top-k (families/gptoss/moe.rs:82-87)
             if (e < a.n_experts) key[j] = order_key(sum);
         }
     }
-    route_row(a, m, key, lane);
+    route_row(a, m, key, lane, forced_first, forced_mine);
 }
 
 // ---- grouped expert matmul --------------------------------------------------------------------

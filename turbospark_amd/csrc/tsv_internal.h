@@ -249,10 +249,13 @@ struct X8 {
     int kpad;    // K rounded up to whole 256-element chunks; the tail stays zero from the allocation
 };
 constexpr int X8_MAX_TERMS = 3;
-// What a context uses unless TSV_MOE_FP4 says otherwise.  Three: with two terms the Qwen3-30B-A3B configuration at its
-// full depth (48 layers) came out 1.2e-2 of the logit range away from the oracle under the oracle's own routing -- past
-// the 1e-2 the path is held to -- against 3.4e-3 with three terms and 5.5e-3 with fp16 activations.
-constexpr int MOE_FP4_DEFAULT_TERMS = 3;
+// What a context uses unless TSV_MOE_FP4 says otherwise: 0, fp16 activations on the 4x4x4 MFMA (moe.hip).  The block-scaled
+// fp8 operand of moe_fp4.hip is opt-in (TSV_MOE_FP4=2 or 3 terms): against the oracle at full depth, under the oracle's own
+// routing, two terms came out 1.2e-2 of the logit range away at the Qwen3-30B-A3B configuration (48 layers) -- past the 1e-2
+// the path is held to -- and 6.5e-3 at the gpt-oss-120B one; three terms 3.4e-3 / 4.2e-3; fp16 activations 5.5e-3 / 3.9e-3.
+// Three terms cost what the instruction saves (gpt-oss-120B shape: 5.3 ms per step against 4.7), and where every row goes
+// to its own experts the fp16 form is the fastest of the three.
+constexpr int MOE_FP4_DEFAULT_TERMS = 0;
 inline size_t x8_q_bytes(int k) { return (size_t)X8_MAX_TERMS * 16 * ((k + 255) / 256 * 256); }
 inline size_t x8_s_bytes(int k) { return x8_q_bytes(k) / 32; }
 
