@@ -345,7 +345,66 @@ typedef struct {
      * depth is fixed, nothing shortened it and tree_nodes == block (speculative.rs:386-392). */
     int32_t tree_nodes;
     int32_t (*draft_tree)(void* user, int32_t anchor, int64_t base, int32_t nodes, int32_t* node_parent, int32_t* tokens);
+    /* optional (may be NULL): drafts_block_passes / draft_block (producer.rs:222-250, call site
+     * speculative.rs:596-603).  draft_block(anchor, base, block, proposals): `block` proposals for positions
+     * base + 1 .. base + block in ONE call, `anchor` being the token at `base`; the drafter keeps its own state
+     * (no prime follows) and picks its own tokens.  A drafter that has it is asked for blocks in every greedy
+     * round (the arg-max ignores penalties and truncation, crates/selection/src/choose.rs:84-88); sampled rounds
+     * need the proposal distributions and go step by step, which a drafter without `step` refuses. */
+    int32_t (*draft_block)(void* user, int32_t anchor, int64_t base, int32_t block, int32_t* proposals);
+    /* optional (may be NULL): supports_chunked_drafter_prefill / prefill_chunk_priming_drafter
+     * (producer.rs:193-211, call site speculative.rs:287-316).  prefill_chunk(tokens, n, start_position, logits,
+     * next_token): the target's prefill of one prompt chunk, priming the drafter over every position whose next
+     * token is known; next_token is the prompt token after the chunk, -1 when the chunk ends the prompt (that
+     * last position is left for the first draft step).  logits (host, vocab fp16): the row after the chunk's
+     * last token.  With it the loop hands the prompt to this callback instead of tsv_prefill + prime per token
+     * (the loop prefills the whole prompt before it primes: a drafter whose prime reads the target's state of
+     * the same position, as the head of tsv_mtp_open does, must offer this callback). */
+    int32_t (*prefill_chunk)(void* user, const int32_t* tokens, int64_t n, int64_t start_position, uint16_t* logits,
+                             int32_t next_token);
 } tsv_drafter;
+
+/* ---- a drafter inside the library: the head that predicts one token further from the target's own state ----
+ * docs/MTP.md:53-60, crates/runtime/src/families/qwen/mtp.rs:
+ *     x   = fc([ norm_embedding(embed(t_{i+1})) ; norm_hidden(target_final_norm(h_i)) ])     (embedding half first)
+ *     x   = x + attn(attn_norm(x))      -- over the head's OWN cache, at position i
+ *     x   = x + ffn(ffn_norm(x))
+ *     out = target_lm_head(head_norm(x))
+ * h_i is the target's residual stream at position i after its last layer (what its final norm consumes); a
+ * chained step (depth > 1) feeds the head's own x of the step before in its place (mtp.rs:85-91).  The norms
+ * are this family's plain RMSNorm (the reference's qwen3.5 head stores its norm weights as offsets from one,
+ * docs/MTP.md:82-90: a caller with such a file adds the one before handing the vectors over).
+ * `model`: n_layers == 1, that layer being the head's decoder block; final_norm the head's own norm; embed and
+ * lm_head left empty (data NULL): the head uses the target's, where they already are on the device; widths,
+ * head counts, vocabulary and rotation as the target's; max_context the positions the head's cache holds. */
+typedef struct {
+    tsv_model_desc model;
+    tsv_tensor fc;                          /* hidden x (2 * hidden), any matmul storage type */
+    tsv_tensor norm_embedding, norm_hidden; /* hidden-wide vectors */
+} tsv_mtp_desc;
+/* Opens the head on the target's device and stream and attaches it: from then on the target's prompt passes
+ * keep their final residual rows for the head.  Close the head before the target. */
+int32_t tsv_mtp_open(tsv_ctx* target, const tsv_mtp_desc* desc, tsv_ctx** head);
+/* mtp_draft_step / mtp_prime_step (mtp.rs:92-116): the head's row at `position` (which must be where its cache
+ * ends, mtp.rs:484-491) from next_token -- the token at position + 1 -- and the state at `position`: the
+ * target's, when the target's last pass holds a row for that position and the head has not stepped since its
+ * last rewind; else the head's own from the step before.  logits NULL: a priming step, cache row only.
+ * Otherwise vocab fp16, host memory, or device memory when logits_on_device is non-zero. */
+int32_t tsv_mtp_step(tsv_ctx* head, int32_t next_token, int64_t position, uint16_t* logits, int32_t logits_on_device);
+/* mtp_rewind_to (mtp.rs:422-436): the head continues after the accepted prefix that ended at `position`. */
+int32_t tsv_mtp_rewind(tsv_ctx* head, int64_t position);
+/* prefill_chunk_priming_drafter for this head (real_forward_traits.rs:361-402, mtp_prime_rows_batched
+ * mtp.rs:146-400): tsv_prefill of the target over the chunk, and after each pass the head's rows for every
+ * position of it whose next token is known, sixteen at a time.  The head must stand at start_position. */
+int32_t tsv_mtp_prefill_chunk(tsv_ctx* head, const int32_t* tokens, int64_t n, int64_t start_position, uint16_t* logits,
+                              int32_t next_token);
+/* `block` greedy proposals (1..15) chained on the device: the step at base - 1 from `anchor` and the target's
+ * state, then each arg-max fed to the next step as a device-side token, no host round trip in between; ends
+ * with the row-only step of the last proposal (speculative.rs:612-625), so the head stands at base + block. */
+int32_t tsv_mtp_draft_block(tsv_ctx* head, int32_t anchor, int64_t base, int32_t block, int32_t* proposals);
+/* Fills `out` with this head's callbacks (prime, step with device logits, rewind, position, draft_block,
+ * prefill_chunk) for tsv_run_speculative on the target the head is attached to. */
+int32_t tsv_mtp_drafter(tsv_ctx* head, tsv_drafter* out);
 
 typedef struct {
     tsv_shaping shaping;

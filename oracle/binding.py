@@ -137,6 +137,9 @@ def lib():
         L.tso_model_route_margin.restype = C.c_float
         L.tso_model_route_record.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.tso_model_force_route.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.tso_model_last_hidden.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+        L.tso_mtp_step.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_void_p,
+                                   C.c_void_p, C.c_void_p]
         L.tso_model_k.restype = C.POINTER(C.c_float)
         L.tso_model_v.restype = C.POINTER(C.c_float)
         L.tso_last_error.restype = C.c_char_p
@@ -624,6 +627,20 @@ class Model:
             raise ValueError(last_error())
         return (f16, f32) if want_f32 else f16
 
+    def prime(self, feed, base):
+        """A pass taken for its cache rows alone: no final norm, no output head."""
+        feed = np.ascontiguousarray(feed, np.int32)
+        rc = lib().tso_model_verify(self._h, _p(feed), None, int(feed.size), C.c_int64(base), None, None, -1)
+        if rc < 0:
+            raise ValueError(last_error())
+
+    def last_hidden(self, row):
+        """Row `row` of the last pass's residual stream after the last layer (what the final norm consumes)."""
+        out = np.empty(self.cfg["hidden"], np.float32)
+        if lib().tso_model_last_hidden(self._h, int(row), _p(out)) != 0:
+            raise ValueError(last_error())
+        return out
+
     def kv(self, layer):
         c = self.cfg
         n = c["max_context"] * c["n_kv_heads"] * c["head_dim"]
@@ -635,6 +652,53 @@ class Model:
     def compact_tree(self, base, path):
         p = np.ascontiguousarray(path, np.uint32)
         lib().tso_model_compact_tree(self._h, C.c_int64(base), _p(p), int(p.size))
+
+
+class MtpDesc(C.Structure):
+    _fields_ = [("fc", Tensor), ("norm_embedding", Tensor), ("norm_hidden", Tensor), ("trunk_norm", Tensor)]
+
+
+class MtpHead:
+    """The drafter head of docs/MTP.md:53-60 over host weight bytes: a one-layer Model (its final_norm the
+    head's own norm, embed / lm_head the trunk's) plus fc and the norms of fc's two halves.  `weights`
+    is a Model weights dict with the extra keys fc, norm_embedding, norm_hidden, trunk_norm."""
+
+    def __init__(self, cfg, weights, round_kv_f16=True, threads=1):
+        assert cfg["n_layers"] == 1
+        self.model = Model(cfg, weights, round_kv_f16=round_kv_f16, threads=threads)
+        self.cfg = cfg
+        self._d = MtpDesc()
+        for name in ("fc", "norm_embedding", "norm_hidden", "trunk_norm"):
+            setattr(self._d, name, _tensor(weights[name]))
+
+    @property
+    def position(self):
+        return self.model.position
+
+    def rewind_to(self, position):
+        self.model.rewind_to(position)
+
+    def reset(self):
+        self.model.reset()
+
+    def step(self, next_tokens, h_rows, position, want="f16", want_x0=False):
+        """Rows at position .. position + n - 1.  want: "f16", "f32" (both), or None (a priming step)."""
+        toks = np.ascontiguousarray(next_tokens, np.int32)
+        h = np.ascontiguousarray(h_rows, np.float32).reshape(toks.size, self.cfg["hidden"])
+        vocab = self.cfg["vocab"]
+        f16 = np.empty((toks.size, vocab), np.uint16) if want else None
+        f32 = np.empty((toks.size, vocab), np.float32) if want == "f32" else None
+        x0 = np.empty((toks.size, self.cfg["hidden"]), np.float32) if want_x0 else None
+        rc = lib().tso_mtp_step(self.model._h, C.byref(self._d), _p(toks), _p(h), int(toks.size), C.c_int64(position),
+                                _p(f16) if f16 is not None else None, _p(f32) if f32 is not None else None,
+                                _p(x0) if x0 is not None else None)
+        if rc < 0:
+            raise ValueError(last_error())
+        out = (f16, f32) if want == "f32" else f16
+        return (out, x0) if want_x0 else out
+
+    def last_hidden(self, row=0):
+        return self.model.last_hidden(row)
 
 
 # ------------------------------------------------------- adaptive depth and the generation loop

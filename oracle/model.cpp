@@ -37,6 +37,9 @@ struct tso_model {
     std::vector<int32_t> forced_sel;
     // TurboQuant KV: sign vectors, codebooks and midpoints of the key and the value side
     std::vector<float> tq_k_signs, tq_v_signs, tq_k_cb, tq_v_cb, tq_k_mid, tq_v_mid;
+    // the residual stream of the last pass's rows after the last layer, before the final norm: [rows][hidden]
+    std::vector<float> last_x;
+    int last_rows = 0;
     bool quantized(int layer) const {  // model-io/src/kv_quant.rs:102-107
         if (d.kv_k_bits <= 0 || layers[layer].window != 0) return false;
         return d.n_layers <= 2 || layer + 1 < d.n_layers;
@@ -184,9 +187,9 @@ extern "C" void tso_model_rewind_to(tso_model* m, int64_t position) { m->positio
 extern "C" float* tso_model_k(tso_model* m, int layer) { return m->k[layer].data(); }
 extern "C" float* tso_model_v(tso_model* m, int layer) { return m->v[layer].data(); }
 
-extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32_t* parent,
-                                int M, int64_t base, uint16_t* logits_f16, float* logits_f32,
-                                int n_layers_run) {
+// `x0` (nullable): the rows that enter the first layer, in place of the embedding lookup of `feed`.
+static int verify_impl(tso_model* mdl, const int32_t* feed, const int32_t* parent, int M, int64_t base,
+                       uint16_t* logits_f16, float* logits_f32, int n_layers_run, const float* x0) {
     const tso_model_desc& d = mdl->d;
     // batched.rs:106-185 refusals
     if (M <= 0) {
@@ -228,7 +231,9 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
     const int T = d.threads;
     std::vector<float> x((size_t)M * H), xn((size_t)M * H);
     // embed lookup (real_forward_dispatch.rs:154): one dequantized row per token
-    {
+    if (x0) {
+        std::memcpy(x.data(), x0, sizeof(float) * (size_t)M * H);
+    } else {
         int64_t rb = tso_row_bytes(d.embed.dtype, H);
         for (int m = 0; m < M; m++)
             tso_dequantize_row(d.embed.dtype, (const uint8_t*)d.embed.data + (int64_t)feed[m] * rb, H,
@@ -390,7 +395,13 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
         }
     }
 
+    mdl->last_x = x;
+    mdl->last_rows = M;
     // head (verify_layers.rs:270-333): final norm, lm_head, raw logits (mod.rs:421-423)
+    if (!logits_f16 && !logits_f32) {  // a pass taken for its cache rows alone (produce_prefill, mtp_prime_step)
+        mdl->position = base + M;
+        return 0;
+    }
     std::vector<float> wfin = norm_weight(d.final_norm);
     for (int m = 0; m < M; m++)
         tso_rms_norm(&x[(size_t)m * H], wfin.data(), H, d.rms_eps, &xn[(size_t)m * H]);
@@ -402,6 +413,64 @@ extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32
         for (size_t i = 0; i < logits.size(); i++) logits_f16[i] = tso_f32_to_f16(logits[i]);
     mdl->position = base + M;
     return 0;
+}
+
+extern "C" int tso_model_verify(tso_model* mdl, const int32_t* feed, const int32_t* parent, int M, int64_t base,
+                                uint16_t* logits_f16, float* logits_f32, int n_layers_run) {
+    return verify_impl(mdl, feed, parent, M, base, logits_f16, logits_f32, n_layers_run, nullptr);
+}
+
+extern "C" int tso_model_last_hidden(const tso_model* m, int row, float* out) {
+    if (row < 0 || row >= m->last_rows) {
+        tso_set_error("last_hidden: no such row in the last pass");
+        return -1;
+    }
+    std::memcpy(out, &m->last_x[(size_t)row * m->d.hidden], sizeof(float) * m->d.hidden);
+    return 0;
+}
+
+// The drafter head's recurrence (docs/MTP.md:53-60; families/qwen/mtp.rs:441-700, batched rows :146-400):
+//   x0 = fc([ norm_e(embed(t_{i+1})) ; norm_h(trunk_final_norm(h_i)) ])   embedding half first
+// then the head model's one decoder layer over its OWN cache at position i, its own final norm
+// (mtp.norm) and the trunk's output head.  h_i is a row of the trunk's residual stream (what its final
+// norm consumes), or -- a chained step -- the head's own residual of the step before, through the same
+// two norms.  The norms are the plain RMSNorm of this family's layers (the reference's qwen3.5 head keeps
+// its weights as offsets from one; a plain-norm file holds the effective scale).
+extern "C" int tso_mtp_step(tso_model* head, const tso_mtp_desc* mtp, const int32_t* next_tokens, const float* h_rows,
+                            int M, int64_t position, uint16_t* logits_f16, float* logits_f32, float* x0_out) {
+    const tso_model_desc& d = head->d;
+    const int H = d.hidden;
+    if (M <= 0) {
+        tso_set_error("mtp_step: no rows");
+        return -1;
+    }
+    if (mtp->fc.rows != H || mtp->fc.cols != 2 * H) {
+        tso_set_error("mtp_step: fc must be hidden x (2 * hidden)");
+        return -6;
+    }
+    for (int m = 0; m < M; m++)
+        if (next_tokens[m] < 0 || next_tokens[m] >= d.vocab) {  // mtp.rs:461-465
+            tso_set_error("mtp_step: draft token id outside the vocabulary");
+            return -4;
+        }
+    if (position != head->position) {  // mtp.rs:484-491
+        tso_set_error("mtp_step: the step's position is not where the head's cache ends");
+        return -2;
+    }
+    std::vector<float> we = norm_weight(mtp->norm_embedding), wh = norm_weight(mtp->norm_hidden),
+                       wt = norm_weight(mtp->trunk_norm);
+    std::vector<float> cat((size_t)M * 2 * H), e(H), t(H), x0((size_t)M * H);
+    const int64_t rb = tso_row_bytes(d.embed.dtype, H);
+    for (int m = 0; m < M; m++) {
+        tso_dequantize_row(d.embed.dtype, (const uint8_t*)d.embed.data + (int64_t)next_tokens[m] * rb, H, e.data());
+        tso_rms_norm(e.data(), we.data(), H, d.rms_eps, &cat[(size_t)m * 2 * H]);
+        tso_rms_norm(h_rows + (size_t)m * H, wt.data(), H, d.rms_eps, t.data());
+        tso_rms_norm(t.data(), wh.data(), H, d.rms_eps, &cat[(size_t)m * 2 * H + H]);
+    }
+    gemm_rows(mtp->fc, cat.data(), M, x0.data(), d.threads);
+    if (x0_out) std::memcpy(x0_out, x0.data(), sizeof(float) * x0.size());
+    std::vector<int32_t> feed(next_tokens, next_tokens + M);
+    return verify_impl(head, feed.data(), nullptr, M, position, logits_f16, logits_f32, -1, x0.data());
 }
 
 // families/qwen/dflash_tree.rs:106-207: gather the accepted path's rows into consecutive

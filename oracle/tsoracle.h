@@ -341,11 +341,31 @@ int tso_model_layer_quantized(const tso_model* m, int layer);
  * pure-attention target).  parent NULL => chain (row i at position base+i, sees [0, base+i]).
  * parent given => tree (row s rotated at base+depth[s], sees [0,base) + its root path; K/V of
  * slot s stored at cache position base+s).  logits_f16 (m_rows x vocab) and logits_f32 are
- * both optional.  n_layers_run < 0 => all layers (a positive value runs a prefix of the
+ * both optional; with neither, the pass stops after the last layer (produce_prefill, producer.rs:92-103).  n_layers_run < 0 => all layers (a positive value runs a prefix of the
  * stack and then the head; used only to bound the timed CPU baseline sample).
  * Advances the cursor by m_rows. */
 int tso_model_verify(tso_model* m, const int32_t* feed, const int32_t* parent, int m_rows,
                      int64_t base, uint16_t* logits_f16, float* logits_f32, int n_layers_run);
+/* Row `row` of the last pass's residual stream after the last layer -- what the final norm consumes
+ * (hidden floats).  -1: the last pass had no such row. */
+int tso_model_last_hidden(const tso_model* m, int row, float* out);
+
+/* The drafter head that predicts one token further from the trunk's own state (docs/MTP.md:53-60,
+ * crates/runtime/src/families/qwen/mtp.rs): `head` is a model of ONE decoder layer whose final_norm is
+ * the head's own norm, whose embed / lm_head are the trunk's, and whose cache is the head's own. */
+typedef struct {
+    tso_tensor fc;                          /* hidden x (2 * hidden) */
+    tso_tensor norm_embedding, norm_hidden; /* the norms of fc's two input halves */
+    tso_tensor trunk_norm;                  /* the TRUNK's final norm: h goes through it first */
+} tso_mtp_desc;
+/* m_rows steps at positions position .. position + m_rows - 1 (mtp.rs:146-400 batches them over a
+ * prompt; one row is mtp_step, :441-700): row r pairs next_tokens[r] -- the token at position + r + 1 --
+ * with h_rows[r], the residual-stream row of position + r (the trunk's, or for a chained step the
+ * head's own from the step before).  Both logits outputs NULL = a priming step: the cache rows alone
+ * (mtp_prime_step, :110-116).  x0_out (nullable): fc's output rows.  The head's residual after the
+ * block is then tso_model_last_hidden(head, r).  Advances the head's cursor by m_rows. */
+int tso_mtp_step(tso_model* head, const tso_mtp_desc* mtp, const int32_t* next_tokens, const float* h_rows,
+                 int m_rows, int64_t position, uint16_t* logits_f16, float* logits_f32, float* x0_out);
 /* Tree compaction (families/qwen/dflash_tree.rs:106-207): move the K/V rows of slots
  * path[0..n) to cache positions base..base+n. */
 void tso_model_compact_tree(tso_model* m, int64_t base, const uint32_t* path, int n);

@@ -6,5 +6,5 @@ this package is the thin host-side mirror of that interface.  There is no CPU fa
 the library is missing, importing `turbospark_amd.ffi` raises.
 """
 from .ffi import F32, F16, Q8_0, Q4_K, Q6_K, BF16, MXFP4, TsvError, lib, shaping  # noqa: F401
-from .producer import HipVerifier, RoundResult  # noqa: F401
+from .producer import HipVerifier, MtpHead, RoundResult  # noqa: F401
 from . import synth  # noqa: F401

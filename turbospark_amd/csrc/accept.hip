@@ -1666,6 +1666,21 @@ int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams*
     return TSV_OK;
 }
 
+// The arg-max of `rows` logit rows (select() at temperature 0, crates/selection/src/choose.rs:61-98: the
+// lowest index among equals, penalties and truncation ignored) into out[0, rows), nothing else touched but the error word, which is cleared only when
+// `clear_error` says so: a chain of such calls keeps the first non-finite row's flag until the host reads it.
+int launch_argmax_rows(hipStream_t s, const uint16_t* logits, int rows, int vocab, const AcceptScratch& sc, int32_t* out,
+                       bool clear_error) {
+    int32_t* err = (int32_t*)sc.counters;
+    if (clear_error) hipLaunchKernelGGL(k_clear_result, dim3(1), dim3(64), 0, s, sc.result, err);
+    float* pv = (float*)sc.counters + 64;
+    int32_t* pi = (int32_t*)sc.counters + 64 + TSV_MAX_ROWS * ARGMAX_SEG;
+    hipLaunchKernelGGL(k_argmax_part, dim3(ARGMAX_SEG, rows), dim3(256), 0, s, logits, vocab, pv, pi, err);
+    hipLaunchKernelGGL(k_argmax_fold, dim3(1), dim3(64), 0, s, pv, pi, rows, out);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
 // The history's token statistics for a penalised round: cnt[v] bit 31 = v occurs in history[0, n),
 // low bits = occurrences in history[suffix_start, n).  Token ids outside [0, vocab) are skipped
 // (penalty.rs:27-33,73-78).

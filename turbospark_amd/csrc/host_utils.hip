@@ -15,6 +15,7 @@ namespace tsv {
 
 static thread_local std::string g_error;
 void set_error(const std::string& s) { g_error = s; }
+bool error_is_empty() { return g_error.empty(); }
 const std::string& get_error() { return g_error; }
 
 int64_t row_bytes(int dtype, int64_t cols) {

@@ -93,8 +93,14 @@ int select_row(tsv_ctx* c, const uint16_t* row, const tsv_shaping* sh, uint64_t 
 
 extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const int32_t* prompt, int64_t n,
                                        const tsv_generation* g, tsv_generation_result* out) {
-    if (!c || !dr || !dr->prime || !dr->step || !dr->rewind || !prompt || !g || !out || !out->tokens) {
+    if (!c || !dr || !dr->rewind || !prompt || !g || !out || !out->tokens) {
         set_error("run_speculative: null argument");
+        return TSV_ERR_INVALID;
+    }
+    // a step-wise drafter steps and primes; a block drafter (producer.rs:222-250) may leave both out, and is
+    // then primed over the prompt by its own prefill_chunk
+    if (!(dr->step && dr->prime) && !(dr->draft_block && dr->prefill_chunk)) {
+        set_error("run_speculative: the drafter needs step and prime, or draft_block and prefill_chunk");
         return TSV_ERR_INVALID;
     }
     const int64_t max_context = tsv_max_context(c);
@@ -121,6 +127,10 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         return TSV_ERR_INVALID;
     }
     const bool sampled = g->shaping.temperature != 0.0;
+    if (sampled && !dr->step) {
+        set_error("run_speculative: this drafter is block-wise only; a sampled round needs draft_step's distributions");
+        return TSV_ERR_UNSUPPORTED;
+    }
     tsv_adaptive ad;
     const bool adaptive = g->adaptive_floor > 0;
     if (adaptive) tsv_adaptive_init(&ad, g->adaptive_floor, g->block);
@@ -147,11 +157,21 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         if (keep > 0) {
             drafter_at = dr->position(dr->user);
             if (tsv_kv_position(c) != cursor || tsv_session_swapped(c) || drafter_at < 0 || keep - drafter_at > 1) keep = 0;
+            // a drafter primed by the prefill itself needs the target's pass over the row it lags by: the
+            // target steps back that one row and both continue from the drafter's position
+            if (keep > drafter_at && dr->prefill_chunk) {
+                tsv_point back{drafter_at};
+                keep = drafter_at > 0 && tsv_rollback(c, &back) == TSV_OK ? drafter_at : 0;
+            }
         }
         reused = keep;
     }
     if (reused == 0) {
         if ((rc = tsv_reset(c))) return rc;
+        if (dr->position && dr->position(dr->user) > 0 && dr->rewind(dr->user, 0)) {
+            set_error("run_speculative: rewind_drafter failed");
+            return TSV_ERR_INVALID;
+        }
     } else if (drafter_at > reused && dr->rewind(dr->user, reused)) {
         set_error("run_speculative: rewind_drafter failed");
         return TSV_ERR_INVALID;
@@ -181,13 +201,23 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
     // each known next token
     // the reused positions are already in the cache (and, by the guard above, in the drafter's
     // context up to at most the one row it lags by, which is primed here with its known next token)
-    if (n - 1 > reused && (rc = tsv_prefill(c, prompt + reused, n - 1 - reused, reused, nullptr))) return rc;
-    for (int64_t i = reused ? std::min(drafter_at, reused) : 0; i + 1 < n; i++)
-        if (dr->prime(dr->user, prompt[i + 1], i)) {
-            set_error("run_speculative: prime_drafter failed");
+    if (dr->prefill_chunk) {
+        // speculative.rs:287-316: the whole prompt through the drafter-priming prefill; the last position is left
+        // for the first draft step
+        set_error("");
+        if (dr->prefill_chunk(dr->user, prompt + reused, n - reused, reused, logits.data(), -1)) {
+            if (error_is_empty()) set_error("run_speculative: prefill_chunk_priming_drafter failed");
             return TSV_ERR_INVALID;
         }
-    if ((rc = tsv_produce(c, prompt[n - 1], n - 1, logits.data()))) return rc;
+    } else {
+        if (n - 1 > reused && (rc = tsv_prefill(c, prompt + reused, n - 1 - reused, reused, nullptr))) return rc;
+        for (int64_t i = reused ? std::min(drafter_at, reused) : 0; i + 1 < n; i++)
+            if (dr->prime(dr->user, prompt[i + 1], i)) {
+                set_error("run_speculative: prime_drafter failed");
+                return TSV_ERR_INVALID;
+            }
+        if ((rc = tsv_produce(c, prompt[n - 1], n - 1, logits.data()))) return rc;
+    }
     int64_t history = n;  // tokens backed by KV rows or about to be
     std::vector<int32_t> hist(prompt, prompt + n);  // TokenSink::history: what the penalties look at
     uint64_t generated = 0, draw_step = 0;
@@ -282,6 +312,14 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
         // arg-max), then the row-only step that primes the drafter with the last proposal
         feed[0] = next;
         int32_t chained = next;
+        if (dr->draft_block && !sampled) {
+            // speculative.rs:596-603: the whole block from one call; the drafter keeps its own state
+            set_error("");
+            if (dr->draft_block(dr->user, next, base, round_block, feed + 1)) {
+                if (error_is_empty()) set_error("run_speculative: draft_block failed");
+                return TSV_ERR_INVALID;
+            }
+        } else
         for (int d = 0; d <= round_block; d++) {
             if (d == round_block) {
                 if (dr->prime(dr->user, chained, base - 1 + d)) {

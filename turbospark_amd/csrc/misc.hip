@@ -249,6 +249,63 @@ int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, in
     return TSV_OK;
 }
 
+// ---------------------------------------------------------------- the drafter head's input
+// fc's input rows (docs/MTP.md:53-60, families/qwen/mtp.rs:512-590): [ norm_e(e) ; norm_h(norm_t(h)) ] with e the
+// looked-up embedding of the row's next token and h the residual row of the row's position; every norm is
+// x * w / sqrt(mean x^2 + eps) (crates/compute/src/rms_norm.rs:5-14).  One workgroup per row.  The row of the
+// head's own residual stream `x_zero` is cleared last -- it may be the very row h was read from (a chained
+// step), and fc's partial sums are added onto it by the layer's first residual kernel.
+__global__ __launch_bounds__(1024) void k_mtp_cat(const float* __restrict__ e_rows, const float* h_rows,
+                                                  const float* __restrict__ w_e, const float* __restrict__ w_t,
+                                                  const float* __restrict__ w_h, float eps, int hidden,
+                                                  float* __restrict__ cat, float* x_zero) {
+    __shared__ float red[16];
+    const int m = blockIdx.x;
+    const float* e = e_rows + (long)m * hidden;
+    const float* h = h_rows + (long)m * hidden;
+    float se = 0.f, sh = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += 1024) {
+        se += e[i] * e[i];
+        sh += h[i] * h[i];
+    }
+    se = block_sum(se, red);
+    sh = block_sum(sh, red);
+    const float inv_e = 1.0f / sqrtf(se / (float)hidden + eps), inv_h = 1.0f / sqrtf(sh / (float)hidden + eps);
+    float st = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += 1024) {
+        const float t = h[i] * w_t[i] * inv_h;
+        st += t * t;
+    }
+    st = block_sum(st, red);
+    const float inv_t = 1.0f / sqrtf(st / (float)hidden + eps);
+    float* out = cat + (long)m * 2 * hidden;
+    for (int i = threadIdx.x; i < hidden; i += 1024) {
+        const float t = h[i] * w_t[i] * inv_h;
+        out[i] = e[i] * w_e[i] * inv_e;
+        out[hidden + i] = t * w_h[i] * inv_t;
+        x_zero[(long)m * hidden + i] = 0.f;
+    }
+}
+
+int launch_mtp_cat(hipStream_t s, const float* e_rows, const float* h_rows, const float* w_e, const float* w_t,
+                   const float* w_h, float eps, int hidden, float* cat, float* x_zero, int m) {
+    hipLaunchKernelGGL(k_mtp_cat, dim3(m), dim3(1024), 0, s, e_rows, h_rows, w_e, w_t, w_h, eps, hidden, cat, x_zero);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+// Row 0 of a pass takes its token from device memory (a proposal the step before picked on the GPU).
+__global__ void k_feed_token(VerifyParams* vp, const int32_t* token, int vocab) {
+    const int t = *token;
+    vp->feed[0] = t < 0 ? 0 : t >= vocab ? vocab - 1 : t;
+}
+
+int launch_feed_token(hipStream_t s, VerifyParams* vp, const int32_t* token, int vocab) {
+    hipLaunchKernelGGL(k_feed_token, dim3(1), dim3(1), 0, s, vp, token, vocab);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
 __global__ void k_f32_to_xfrag(const float* __restrict__ x, int k, _Float16* __restrict__ xfrag) {
     const int m = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;

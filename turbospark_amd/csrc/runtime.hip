@@ -166,6 +166,25 @@ struct tsv_ctx {
     std::vector<hipEvent_t> ev;
     std::vector<int> ev_class;
     size_t ev_used = 0;
+    // A drafter head (tsv_mtp_open; docs/MTP.md:53-60): a one-layer handle on the target's stream whose rows
+    // enter the layer as fc over [norm_e(embedding of the row's NEXT token) ; norm_h(target_final_norm(h))], h
+    // the residual row of the row's position.  Embedding table and output head are the target's buffers.
+    struct Mtp {
+        bool on = false;
+        tsv_ctx* target = nullptr;
+        TiledW fc;
+        float *norm_e = nullptr, *norm_h = nullptr;
+        float *e_rows = nullptr, *cat = nullptr;  // [16][hidden] looked-up embeddings, [16][2 hidden] fc's input
+        uint4* xf_cat = nullptr;                  // the same as matmul fragments
+        const float* h_src = nullptr;             // the pass in flight: its residual rows, hidden floats apart
+        bool own_valid = false;  // x row 0 is this head's own residual of the step at position - 1 (a chained step)
+        const int32_t* feed_dev = nullptr;  // the pass in flight takes row 0's token from device memory
+        int32_t *chain = nullptr, *chain_host = nullptr;  // the tokens of a block draft and the error word
+    } mtp;
+    int64_t x_base = -1;  // rows [0, x_rows) of x are the finished residual rows of positions x_base ..
+    int x_rows = 0;
+    tsv_ctx* mtp_head = nullptr;  // target side: the attached head; prompt passes then finish their residual rows
+    bool owns_stream = true;
 };
 
 namespace {
@@ -454,6 +473,7 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     *c->vp_host = vp;  // the host's own copy of the pass in flight
     int prc2 = stage_params(c, &vp, 1, c->vp_dev);
     if (prc2) return prc2;
+    if (c->mtp.feed_dev && (prc2 = launch_feed_token(c->stream, c->vp_dev, c->mtp.feed_dev, c->vocab))) return prc2;
     int rc = run_pass(c, m);
     if (rc) return rc;
     c->position = base + m;
@@ -461,6 +481,10 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     c->last_m = m;
     c->last_base = base;
     c->last_shape_known = true;
+    // whose residual rows x holds now: a chain pass that ran its last residual add leaves row r = position base + r
+    c->x_base = base;
+    c->x_rows = parent || (c->headless && !c->mtp_head) ? 0 : m;
+    if (c->mtp_head) c->mtp_head->mtp.own_valid = false;  // the head's next step reads the target's rows again
     return TSV_OK;
 }
 
@@ -481,13 +505,26 @@ int launch_pass(tsv_ctx* c, int m) {
     hipStream_t s = c->stream;
     int rc;
     { PROF(PC_EVENTPAIR); }  // calibration: an event pair around nothing
-    {
+    int prev_splits = 0;
+    if (c->mtp.on) {
+        // the head's rows: fc over the normed embedding of each row's next token and the normed state of its
+        // position; fc's split-K partial sums are added onto the cleared rows by the layer's first residual kernel
+        tsv_ctx::Mtp& h = c->mtp;
+        PROF(PC_EMBED);
+        if ((rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, h.e_rows, c->vp_dev, m, c->freqs, c->rope_mscale,
+                               c->hd / 2, c->rope_cs)) ||
+            (rc = launch_mtp_cat(s, h.e_rows, h.h_src, h.norm_e, h.target->final_norm, h.norm_h, c->eps, c->hidden, h.cat,
+                                 c->x, m)) ||
+            (rc = launch_f32_to_xfrag(s, h.cat, 2 * c->hidden, h.xf_cat, m)))
+            return rc;
+        prev_splits = splits_for(h.fc, m, EPI_PARTIAL);
+        rc = launch_gemm(s, h.fc, h.xf_cat, c->partial, c->vp_dev, m, prev_splits, EPI_PARTIAL, c->hidden, c->hidden);
+    } else {
         PROF(PC_EMBED);
         rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, c->x, c->vp_dev, m, c->freqs, c->rope_mscale,
                           c->hd / 2, c->rope_cs);
     }
     if (rc) return rc;
-    int prev_splits = 0;
     const float* prev_partial = c->partial;
     const float* prev_weights = nullptr;  // routed experts: the factors of the per-slot outputs
     float* x = c->x;
@@ -723,13 +760,14 @@ int launch_pass(tsv_ctx* c, int m) {
     // produce_prefill (producer.rs:92-103, real_forward_traits.rs:291-300): a prompt token whose
     // logits nobody reads skips the final norm and the output head; every other side effect of
     // the pass (the rows in the cache, the cursor) is that of a full pass.
-    if (c->headless) return TSV_OK;
+    // (With a drafter head attached the rows' last residual add still happens: the head reads them.)
+    if (c->headless && !c->mtp_head) return TSV_OK;
     {
         PROF(PC_NORM);
         rc = launch_addnorm(s, x, prev_partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, c->xf_a, m,
                             prev_weights);
     }
-    if (rc) return rc;
+    if (rc || c->headless) return rc;
     {
         PROF(PC_HEAD);
         rc = 0;
@@ -892,7 +930,7 @@ int enqueue_wide_prefill(tsv_ctx* c, const int32_t* ids, int64_t base) {
 }
 
 int run_pass(tsv_ctx* c, int m) {
-    if (!c->use_graph || c->profile || c->headless) return launch_pass(c, m);
+    if (!c->use_graph || c->profile || c->headless || c->mtp.on) return launch_pass(c, m);
     if (!c->pass_graph[m]) {
         hipGraph_t g = nullptr;
         TSV_HIP(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
@@ -925,7 +963,9 @@ int finish_verify(tsv_ctx* c, int m, uint16_t* logits_out) {
 
 }  // namespace
 
-extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
+// `share` / `md`: a drafter head opened on a target handle -- its stream, embedding table and output head are
+// the target's, and md names fc and the norms of fc's two halves.
+static int open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* md, tsv_ctx** out) {
     if (!d || !out || !d->layers) {
         set_error("open: null argument");
         return TSV_ERR_INVALID;
@@ -970,7 +1010,10 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     // MXFP4 experts on the block-scaled matrix instruction: activation terms, 0 = the fp16 path
     c->moe_fp4_terms = MOE_FP4_DEFAULT_TERMS;
     if (const char* e = getenv("TSV_MOE_FP4")) c->moe_fp4_terms = e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
-    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
+    if (share) {
+        c->stream = share->stream;
+        c->owns_stream = false;
+    } else if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("open: cannot create a HIP stream (no GPU?)");
         delete c;
         return TSV_ERR_DEVICE;
@@ -1222,17 +1265,32 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
     }
     // embedding table (raw GGUF rows for the lookup) and output head (tiled)
     const int64_t erb = row_bytes(d->embed.dtype, c->hidden);
-    if (!d->embed.data || d->embed.rows != c->vocab || d->embed.cols != c->hidden || erb < 0) {
+    if (share) {
+        if (d->embed.data || d->lm_head.data) {
+            set_error("mtp_open: the head takes the target's embedding table and output head; leave both empty");
+            return fail(TSV_ERR_INVALID);
+        }
+        c->embed_raw = share->embed_raw;
+        c->embed_dtype = share->embed_dtype;
+        c->head = share->head;
+        const tsv_tensor* fp[1] = {&md->fc};
+        if ((rc = check_matrix(md->fc, c->hidden, 2 * (int64_t)c->hidden, "fc")) || (rc = make_tiled(c, st, fp, 1, false, &c->mtp.fc)) ||
+            (rc = upload_vector(c, md->norm_embedding, c->hidden, &c->mtp.norm_e, "norm_embedding")) ||
+            (rc = upload_vector(c, md->norm_hidden, c->hidden, &c->mtp.norm_h, "norm_hidden")))
+            return fail(rc);
+        pneed = std::max(pneed, partial_need(c->mtp.fc));
+    } else if (!d->embed.data || d->embed.rows != c->vocab || d->embed.cols != c->hidden || erb < 0) {
         set_error("open: embedding table shape / dtype");
         return fail(TSV_ERR_INVALID);
+    } else {
+        c->embed_dtype = d->embed.dtype;
+        if ((rc = dev_alloc(c, &c->embed_raw, (size_t)(erb * c->vocab)))) return fail(rc);
+        if (hipMemcpy(c->embed_raw, d->embed.data, (size_t)(erb * c->vocab), hipMemcpyHostToDevice) != hipSuccess) {
+            set_error("open: embedding upload failed");
+            return fail(TSV_ERR_DEVICE);
+        }
     }
-    c->embed_dtype = d->embed.dtype;
-    if ((rc = dev_alloc(c, &c->embed_raw, (size_t)(erb * c->vocab)))) return fail(rc);
-    if (hipMemcpy(c->embed_raw, d->embed.data, (size_t)(erb * c->vocab), hipMemcpyHostToDevice) != hipSuccess) {
-        set_error("open: embedding upload failed");
-        return fail(TSV_ERR_DEVICE);
-    }
-    {
+    if (!share) {
         tsv_tensor head = d->lm_head.data ? d->lm_head : d->embed;
         // the head's row count need not be a multiple of 16: the last tile is zero padded
         if ((rc = check_matrix(head, c->vocab, c->hidden, "output head"))) return fail(rc);
@@ -1308,6 +1366,19 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
         set_error("open: pinned host allocation failed");
         return fail(TSV_ERR_DEVICE);
     }
+    if (share) {
+        tsv_ctx::Mtp& h = c->mtp;
+        if ((rc = dev_alloc(c, &h.e_rows, (size_t)16 * c->hidden * 4, true)) ||
+            (rc = dev_alloc(c, &h.cat, (size_t)16 * 2 * c->hidden * 4, true)) ||
+            (rc = dev_alloc(c, &h.xf_cat, xfrag_bytes(2 * c->hidden), true)) || (rc = dev_alloc(c, &h.chain, 32 * 4, true)))
+            return fail(rc);
+        if (hipHostMalloc((void**)&h.chain_host, 32 * 4) != hipSuccess) {
+            set_error("mtp_open: pinned host allocation failed");
+            return fail(TSV_ERR_DEVICE);
+        }
+        h.on = true;
+        h.target = share;
+    }
     if (int nrc = noalloc_prepare_device()) return fail(nrc);  // tsv_accept_greedy_noalloc is capturable from here on
     if (hipStreamSynchronize(c->stream) != hipSuccess) {
         set_error("open: device initialisation failed");
@@ -1320,9 +1391,12 @@ extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) {
             L.gate_up.fmt != FMT_Q4K || L.down.fmt != FMT_Q4K)
             c->wide.ok = false;
     if (const char* e = getenv("TSV_WIDE_PREFILL")) c->wide.ok = c->wide.ok && e[0] != '0';
+    if (share) c->wide.ok = false;  // the head's rows come sixteen at a time
     *out = c;
     return TSV_OK;
 }
+
+extern "C" int32_t tsv_open(const tsv_model_desc* d, tsv_ctx** out) { return open_impl(d, nullptr, nullptr, out); }
 
 extern "C" void tsv_close(tsv_ctx* c) {
     if (!c) return;
@@ -1336,10 +1410,12 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->ap_host) (void)hipHostFree(c->ap_host);
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
+    if (c->mtp.chain_host) (void)hipHostFree(c->mtp.chain_host);
+    if (c->mtp.on && c->mtp.target && c->mtp.target->mtp_head == c) c->mtp.target->mtp_head = nullptr;
     for (hipGraphExec_t g : c->pass_graph)
         if (g) (void)hipGraphExecDestroy(g);
     for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
-    if (c->stream) (void)hipStreamDestroy(c->stream);
+    if (c->stream && c->owns_stream) (void)hipStreamDestroy(c->stream);
     delete c;
 }
 
@@ -1509,7 +1585,12 @@ extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint
     return rc;
 }
 
-static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits) {
+static int mtp_pass(tsv_ctx* c, const int32_t* next_tokens, int m, int64_t position, const float* h_rows, bool want_logits);
+
+// `head` (nullable): the drafter head primed after each pass over every row whose next token is known
+// (mtp_prime_rows_batched, families/qwen/mtp.rs:146-400); next_token: the token after ids[n - 1], or -1.
+static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits, tsv_ctx* head = nullptr,
+                          int32_t next_token = -1) {
     const int wide_rows = 16 * WIDE_B;
     for (int64_t i = 0; i < n;) {
         // 64 rows at a time while that many remain and nobody wants their logits
@@ -1531,6 +1612,17 @@ static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos
             TSV_HIP(hipMemcpyAsync(logits, c->logits + (size_t)(m - 1) * c->vocab, (size_t)c->vocab * 2,
                                    hipMemcpyDeviceToHost, c->stream));
         }
+        if (head) {
+            int32_t nt[TSV_MAX_ROWS];
+            int rows = 0;
+            for (; rows < m; rows++) {
+                const int64_t j = i + rows + 1;
+                if (j < n) nt[rows] = ids[j];
+                else if (next_token >= 0) nt[rows] = next_token;
+                else break;
+            }
+            if (rows && (rc = mtp_pass(head, nt, rows, pos0 + i, c->x, false))) return rc;
+        }
         i += m;
     }
     TSV_HIP(hipStreamSynchronize(c->stream));
@@ -1549,6 +1641,166 @@ extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_
     if (rc == TSV_OK) c->prefix.record(ids, n, pos0);
     else c->prefix.taint();
     return rc;
+}
+
+// ---- the drafter head (docs/MTP.md:53-60, crates/runtime/src/families/qwen/mtp.rs) ------------------------
+// One pass of the head over m rows at position .. position + m - 1: row r pairs next_tokens[r] with h_rows' row r.
+static int mtp_pass(tsv_ctx* c, const int32_t* next_tokens, int m, int64_t position, const float* h_rows, bool want_logits) {
+    if (position != c->position) {  // mtp.rs:484-491
+        set_error("mtp: step at position " + std::to_string((long long)position) + " but the head's cache covers [0, " +
+                  std::to_string((long long)c->position) + "): prime the head over the prompt and rewind it after a rejected draft");
+        return TSV_ERR_INVALID;
+    }
+    c->mtp.h_src = h_rows;
+    c->headless = !want_logits;
+    const int rc = enqueue_verify(c, next_tokens, nullptr, m, position);
+    c->headless = false;
+    c->mtp.h_src = nullptr;
+    // after a full step row 0 of x is the head's own finished residual: what a chained step reads (mtp.rs:85-91)
+    c->mtp.own_valid = rc == TSV_OK && want_logits && m == 1;
+    return rc;
+}
+
+// Where the state of `position` is: the head's own row after a step of its own, else the target's last pass.
+static int mtp_source(tsv_ctx* c, int64_t position, const float** src) {
+    const tsv_ctx* t = c->mtp.target;
+    if (c->mtp.own_valid) {
+        *src = c->x;
+        return TSV_OK;
+    }
+    if (position >= t->x_base && position < t->x_base + t->x_rows) {
+        *src = t->x + (size_t)(position - t->x_base) * t->hidden;
+        return TSV_OK;
+    }
+    set_error("mtp: the target's last pass holds no row for position " + std::to_string((long long)position) +
+              " and the head has no step of its own to chain from");
+    return TSV_ERR_INVALID;
+}
+
+extern "C" int32_t tsv_mtp_open(tsv_ctx* target, const tsv_mtp_desc* d, tsv_ctx** out) {
+    TSV_NEED(target && d && out, "mtp_open: null argument");
+    if (target->mtp.on || target->mtp_head) {
+        set_error("mtp_open: the target is itself a head, or already has one");
+        return TSV_ERR_INVALID;
+    }
+    const tsv_model_desc& m = d->model;
+    if (m.n_layers != 1 || m.hidden != target->hidden || m.vocab != target->vocab) {
+        set_error("mtp_open: the head is ONE decoder layer of the target's width over the target's vocabulary");
+        return TSV_ERR_INVALID;
+    }
+    if (m.kv_k_bits || m.kv_v_bits || m.session_slots > 1 || (m.layers && m.layers[0].ring)) {
+        set_error("mtp_open: the head keeps one plain fp16 cache (no quantized rows, ring or session slots)");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    TSV_HIP(hipStreamSynchronize(target->stream));
+    const int rc = open_impl(&m, target, d, out);
+    if (rc) return rc;
+    target->mtp_head = *out;
+    target->wide.ok = false;  // the head reads each prompt pass's rows where the sixteen-row pass leaves them
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_mtp_step(tsv_ctx* c, int32_t next_token, int64_t position, uint16_t* logits, int32_t on_device) {
+    TSV_NEED(c && c->mtp.on, "mtp_step: not a drafter head");
+    const float* src = nullptr;
+    int rc = mtp_source(c, position, &src);
+    if (rc) return rc;
+    if ((rc = mtp_pass(c, &next_token, 1, position, src, logits != nullptr))) return rc;
+    if (!logits) return TSV_OK;
+    if (on_device) {  // stays in stream order: whoever reads the row does so on the target's stream
+        TSV_HIP(hipMemcpyAsync(logits, c->logits, (size_t)c->vocab * 2, hipMemcpyDeviceToDevice, c->stream));
+        return TSV_OK;
+    }
+    return finish_verify(c, 1, logits);
+}
+
+extern "C" int32_t tsv_mtp_rewind(tsv_ctx* c, int64_t position) {
+    TSV_NEED(c && c->mtp.on, "mtp_rewind: not a drafter head");
+    if (position < 0 || position > c->position) {  // mtp.rs:422-436
+        set_error("mtp_rewind: the head cannot be moved forward, or before position 0");
+        return TSV_ERR_INVALID;
+    }
+    c->position = position;
+    c->mtp.own_valid = false;
+    return TSV_OK;
+}
+
+extern "C" int32_t tsv_mtp_prefill_chunk(tsv_ctx* c, const int32_t* tokens, int64_t n, int64_t start_position,
+                                         uint16_t* logits, int32_t next_token) {
+    TSV_NEED(c && c->mtp.on && tokens, "mtp_prefill_chunk: not a drafter head, or no tokens");
+    if (n < 1) {
+        set_error("mtp_prefill_chunk: empty token list");
+        return TSV_ERR_INVALID;
+    }
+    if (c->position != start_position) {
+        set_error("mtp_prefill_chunk: the head's cache must end where the chunk starts");
+        return TSV_ERR_INVALID;
+    }
+    tsv_ctx* t = c->mtp.target;
+    // recorded once the chunk has run to completion, tainted when it has not (real_forward_traits.rs:395-402)
+    const int rc = prefill_passes(t, tokens, n, start_position, logits, c, next_token >= 0 && next_token < t->vocab ? next_token : -1);
+    if (rc == TSV_OK) t->prefix.record(tokens, n, start_position);
+    else t->prefix.taint();
+    return rc;
+}
+
+extern "C" int32_t tsv_mtp_draft_block(tsv_ctx* c, int32_t anchor, int64_t base, int32_t block, int32_t* proposals) {
+    TSV_NEED(c && c->mtp.on && proposals, "mtp_draft_block: not a drafter head, or no output");
+    if (block < 1 || block > TSV_MAX_ROWS - 1 || base < 1) {
+        set_error("mtp_draft_block: 1..15 proposals after a position the target has produced");
+        return TSV_ERR_INVALID;
+    }
+    tsv_ctx::Mtp& h = c->mtp;
+    int rc;
+    const int32_t none = 0;
+    for (int d = 0; d <= block; d++) {
+        // step d pairs the state of base - 1 + d with the token at base + d: the anchor, then each pick of the
+        // step before, read where the arg-max left it; the last step is the row-only one (speculative.rs:612-625)
+        const float* src = nullptr;
+        if ((rc = mtp_source(c, base - 1 + d, &src))) return rc;
+        h.feed_dev = d ? h.chain + d : nullptr;
+        rc = mtp_pass(c, d ? &none : &anchor, 1, base - 1 + d, src, d < block);
+        h.feed_dev = nullptr;
+        if (rc) return rc;
+        if (d < block && (rc = launch_argmax_rows(c->stream, c->logits, 1, c->vocab, c->sc, h.chain + d + 1, d == 0))) return rc;
+    }
+    h.own_valid = false;
+    TSV_HIP(hipMemcpyAsync(h.chain_host, h.chain + 1, (size_t)block * 4, hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipMemcpyAsync(h.chain_host + 31, c->sc.counters, 4, hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    if (h.chain_host[31]) {
+        set_error("mtp_draft_block: score vector must not contain a non-finite entry");
+        return TSV_ERR_INVALID;
+    }
+    for (int i = 0; i < block; i++) proposals[i] = h.chain_host[i];
+    return TSV_OK;
+}
+
+namespace {
+int32_t mtp_cb_prime(void* u, int32_t next, int64_t position) { return tsv_mtp_step((tsv_ctx*)u, next, position, nullptr, 0); }
+int32_t mtp_cb_step(void* u, int32_t tok, int64_t position, uint16_t* logits) { return tsv_mtp_step((tsv_ctx*)u, tok, position, logits, 1); }
+int32_t mtp_cb_rewind(void* u, int64_t position) { return tsv_mtp_rewind((tsv_ctx*)u, position); }
+int64_t mtp_cb_position(void* u) { return ((tsv_ctx*)u)->position; }
+int32_t mtp_cb_block(void* u, int32_t anchor, int64_t base, int32_t block, int32_t* proposals) {
+    return tsv_mtp_draft_block((tsv_ctx*)u, anchor, base, block, proposals);
+}
+int32_t mtp_cb_chunk(void* u, const int32_t* tokens, int64_t n, int64_t start, uint16_t* logits, int32_t next_token) {
+    return tsv_mtp_prefill_chunk((tsv_ctx*)u, tokens, n, start, logits, next_token);
+}
+}  // namespace
+
+extern "C" int32_t tsv_mtp_drafter(tsv_ctx* c, tsv_drafter* out) {
+    TSV_NEED(c && c->mtp.on && out, "mtp_drafter: not a drafter head, or no output");
+    std::memset(out, 0, sizeof *out);
+    out->user = c;
+    out->prime = mtp_cb_prime;
+    out->step = mtp_cb_step;
+    out->rewind = mtp_cb_rewind;
+    out->device_logits = 1;
+    out->position = mtp_cb_position;
+    out->draft_block = mtp_cb_block;
+    out->prefill_chunk = mtp_cb_chunk;
+    return TSV_OK;
 }
 
 extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {

@@ -12,6 +12,7 @@
 namespace tsv {
 
 void set_error(const std::string& s);
+bool error_is_empty();
 const std::string& get_error();
 
 #define TSV_HIP(call)                                                                       \
@@ -302,6 +303,10 @@ int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, in
                    const float* bias = nullptr, const X8* x8 = nullptr, int x8_terms = 0, int blocks = 1,
                    const NormBlocks* nb = nullptr);
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
+// the drafter head: fc's input rows [m][2 * hidden] from embedding rows and residual rows; clears x_zero's rows
+int launch_mtp_cat(hipStream_t s, const float* e_rows, const float* h_rows, const float* w_e, const float* w_t,
+                   const float* w_h, float eps, int hidden, float* cat, float* x_zero, int m);
+int launch_feed_token(hipStream_t s, VerifyParams* vp, const int32_t* token, int vocab);
 
 struct RopeKvArgs {
     const float* qkv;  // [splits][16][ldq]
@@ -482,6 +487,9 @@ int launch_accept(hipStream_t s, const uint16_t* target, const uint16_t* draft, 
                   const AcceptParams& ap_host, const AcceptScratch& sc);
 int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams* ap_dev,
                        const AcceptParams& ap_host, const AcceptScratch& sc, int32_t* proposals_dev);
+// arg-max of `rows` logit rows into out[0, rows); the error word (sc.counters[0]) is cleared first only on request
+int launch_argmax_rows(hipStream_t s, const uint16_t* logits, int rows, int vocab, const AcceptScratch& sc, int32_t* out,
+                       bool clear_error);
 int noalloc_prepare_device();
 int launch_pen_counts(hipStream_t s, const int32_t* history_dev, long n, long suffix_start, int vocab, uint32_t* cnt);
 

@@ -194,10 +194,19 @@ DRAFT_POSITION = C.CFUNCTYPE(C.c_int64, C.c_void_p)
 DRAFT_TREE = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32))
 
 
+DRAFT_BLOCK = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_int32))
+DRAFT_PREFILL_CHUNK = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.POINTER(C.c_int32), C.c_int64, C.c_int64, C.POINTER(C.c_uint16),
+                                  C.c_int32)
+
+
 class Drafter(C.Structure):
     _fields_ = [("user", C.c_void_p), ("prime", DRAFT_PRIME), ("step", DRAFT_STEP), ("rewind", DRAFT_REWIND),
                 ("device_logits", C.c_int32), ("position", DRAFT_POSITION), ("tree_nodes", C.c_int32),
-                ("draft_tree", DRAFT_TREE)]
+                ("draft_tree", DRAFT_TREE), ("draft_block", DRAFT_BLOCK), ("prefill_chunk", DRAFT_PREFILL_CHUNK)]
+
+
+class MtpDesc(C.Structure):
+    _fields_ = [("model", ModelDesc), ("fc", Tensor), ("norm_embedding", Tensor), ("norm_hidden", Tensor)]
 
 
 class Generation(C.Structure):
@@ -251,6 +260,7 @@ EXPORTS = [
     "tsv_read_kv_quantized", "tsv_attention_quantized", "tsv_kv_quant_tables",
     "tsv_session_pool_size", "tsv_session_slot_evicted", "tsv_session_best_match", "tsv_session_lru", "tsv_session_swapped",
     "tsv_kv_row_bytes", "tsv_kv_bytes_for_context",
+    "tsv_mtp_open", "tsv_mtp_step", "tsv_mtp_rewind", "tsv_mtp_prefill_chunk", "tsv_mtp_draft_block", "tsv_mtp_drafter",
 ]
 
 _lib = None
@@ -330,6 +340,12 @@ def lib():
         L.tsv_attention_quantized.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                               C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_void_p, C.c_void_p,
                                               C.c_void_p, C.c_void_p]
+        L.tsv_mtp_open.argtypes = [C.c_void_p, C.POINTER(MtpDesc), C.POINTER(C.c_void_p)]
+        L.tsv_mtp_step.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_void_p, C.c_int32]
+        L.tsv_mtp_rewind.argtypes = [C.c_void_p, C.c_int64]
+        L.tsv_mtp_prefill_chunk.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_int32]
+        L.tsv_mtp_draft_block.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_void_p]
+        L.tsv_mtp_drafter.argtypes = [C.c_void_p, C.POINTER(Drafter)]
         L.tsv_set_profile.argtypes = [C.c_void_p, C.c_int32]
         L.tsv_get_profile.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]
         L.tsv_copy_time.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]

@@ -39,6 +39,115 @@ def parse_kv_bits(text):
     return table[text]
 
 
+def model_desc(cfg, weights, kv_bits=None, session_slots=1, shared_tables=False):
+    """(tsv_model_desc, what must stay alive while it is used) for a weight dictionary; `shared_tables` leaves the
+    embedding table and the output head empty (a drafter head takes the target's)."""
+    n = len(weights["layers"])
+    layers = (ffi.Layer * n)()
+    for i, lw in enumerate(weights["layers"]):
+        for name in ffi.LAYER_TENSORS + ffi.LAYER_MOE_TENSORS + ffi.LAYER_GPTOSS_TENSORS:
+            setattr(layers[i], name, ffi.tensor(lw.get(name)))
+        layers[i].n_experts = int(lw.get("n_experts", 0))
+        layers[i].top_k = int(lw.get("top_k", 0))
+        layers[i].window = int(lw.get("window", 0))
+        layers[i].ring = int(bool(lw.get("ring", 0)))
+    d = ffi.ModelDesc()
+    d.n_layers = n
+    for key in ("hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_context"):
+        setattr(d, key, cfg[key])
+    d.rms_eps = cfg.get("rms_eps", 1e-5)
+    d.rope_theta = cfg.get("rope_theta", 10000.0)
+    d.attn_scale = cfg.get("attn_scale", 0.0)
+    factors = freqs = None
+    if cfg.get("rope_factors") is not None:
+        factors = np.ascontiguousarray(cfg["rope_factors"], np.float32)
+        d.rope_factors = factors.ctypes.data_as(C.POINTER(C.c_float))
+    if cfg.get("rope_freqs") is not None:
+        freqs = np.ascontiguousarray(cfg["rope_freqs"], np.float32)
+        d.rope_freqs = freqs.ctypes.data_as(C.POINTER(C.c_float))
+    d.rope_mscale = cfg.get("rope_mscale", 0.0)
+    d.act_alpha = cfg.get("act_alpha", 0.0)
+    d.act_limit = cfg.get("act_limit", 0.0)
+    d.kv_k_bits, d.kv_v_bits = kv_bits if kv_bits else (0, 0)
+    d.session_slots = int(session_slots)
+    if not shared_tables:
+        d.embed = ffi.tensor(weights["embed"])
+        d.lm_head = ffi.tensor(weights.get("lm_head"))
+    d.final_norm = ffi.tensor(weights["final_norm"])
+    d.layers = C.cast(layers, C.POINTER(ffi.Layer))
+    return d, (weights, layers, factors, freqs)
+
+
+class MtpHead:
+    """The drafter head that predicts one token further from the target's own state (docs/MTP.md:53-60,
+    crates/runtime/src/families/qwen/mtp.rs), resident beside a HipVerifier and attached to it: one decoder
+    layer with a cache of its own, fc over [norm(embedding of the next token); norm(target's final state)],
+    the target's embedding table and output head.  `weights`: a one-layer weight dictionary (final_norm the
+    head's own norm) with the extra keys fc, norm_embedding, norm_hidden.  Close it before the target."""
+
+    def __init__(self, target, cfg, weights):
+        md = ffi.MtpDesc()
+        md.model, self._keep = model_desc(cfg, weights, shared_tables=True)
+        md.fc = ffi.tensor(weights["fc"])
+        md.norm_embedding = ffi.tensor(weights["norm_embedding"])
+        md.norm_hidden = ffi.tensor(weights["norm_hidden"])
+        h = C.c_void_p()
+        ffi.check(ffi.lib().tsv_mtp_open(target._h, C.byref(md), C.byref(h)))
+        self._h = h
+        self.target = target
+        self.vocab = target.vocab
+        self.cfg = dict(cfg)
+
+    def close(self):
+        if getattr(self, "_h", None):
+            ffi.lib().tsv_close(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    @property
+    def position(self):
+        return int(ffi.lib().tsv_kv_position(self._h))
+
+    def step(self, next_token, position):
+        """mtp_draft_step: the head's logits (uint16[vocab] fp16 bits) for the token after `next_token`."""
+        out = np.empty(self.vocab, np.uint16)
+        ffi.check(ffi.lib().tsv_mtp_step(self._h, int(next_token), int(position), out.ctypes.data, 0))
+        return out
+
+    def step_device(self, next_token, position, address):
+        ffi.check(ffi.lib().tsv_mtp_step(self._h, int(next_token), int(position), C.c_void_p(address), 1))
+
+    def prime(self, next_token, position):
+        """mtp_prime_step: the cache row alone."""
+        ffi.check(ffi.lib().tsv_mtp_step(self._h, int(next_token), int(position), None, 0))
+
+    def rewind(self, position):
+        ffi.check(ffi.lib().tsv_mtp_rewind(self._h, int(position)))
+
+    def context_position(self):
+        return self.position
+
+    def prefill_chunk(self, tokens, start_position, next_token=None, want_logits=True):
+        """The target's prefill of the chunk, priming the head over every position whose next token is known."""
+        ids = _i32(tokens)
+        out = np.empty(self.vocab, np.uint16) if want_logits else None
+        ffi.check(ffi.lib().tsv_mtp_prefill_chunk(self._h, ids.ctypes.data, ids.size, int(start_position),
+                                                  out.ctypes.data if want_logits else None,
+                                                  -1 if next_token is None else int(next_token)))
+        return out
+
+    def draft_block(self, anchor, base, block):
+        """`block` greedy proposals chained on the device; the head then stands at base + block."""
+        out = np.empty(int(block), np.int32)
+        ffi.check(ffi.lib().tsv_mtp_draft_block(self._h, int(anchor), int(base), int(block), out.ctypes.data))
+        return [int(t) for t in out]
+
+    def read_kv(self, pos0, n):
+        return HipVerifier.read_kv(self, 0, pos0, n)
+
+
 class HipVerifier:
     """One target model resident on the GPU with its KV cache: fp16 rows, or TurboQuant rows on the layers
     crates/model-io/src/kv_quant.rs:102-107 names when kv_bits = (key bits, value bits) is given
@@ -46,41 +155,8 @@ class HipVerifier:
 
     def __init__(self, cfg, weights, kv_bits=None, session_slots=1):
         self.cfg = dict(cfg)
-        self._keep = weights
-        n = len(weights["layers"])
-        self._layers = (ffi.Layer * n)()
-        for i, lw in enumerate(weights["layers"]):
-            for name in ffi.LAYER_TENSORS + ffi.LAYER_MOE_TENSORS + ffi.LAYER_GPTOSS_TENSORS:
-                setattr(self._layers[i], name, ffi.tensor(lw.get(name)))
-            self._layers[i].n_experts = int(lw.get("n_experts", 0))
-            self._layers[i].top_k = int(lw.get("top_k", 0))
-            self._layers[i].window = int(lw.get("window", 0))
-            self._layers[i].ring = int(bool(lw.get("ring", 0)))
-        d = ffi.ModelDesc()
-        d.n_layers = n
-        for key in ("hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_context"):
-            setattr(d, key, cfg[key])
-        d.rms_eps = cfg.get("rms_eps", 1e-5)
-        d.rope_theta = cfg.get("rope_theta", 10000.0)
-        d.attn_scale = cfg.get("attn_scale", 0.0)
-        self._factors = None
-        if cfg.get("rope_factors") is not None:
-            self._factors = np.ascontiguousarray(cfg["rope_factors"], np.float32)
-            d.rope_factors = self._factors.ctypes.data_as(C.POINTER(C.c_float))
-        self._freqs = None
-        if cfg.get("rope_freqs") is not None:
-            self._freqs = np.ascontiguousarray(cfg["rope_freqs"], np.float32)
-            d.rope_freqs = self._freqs.ctypes.data_as(C.POINTER(C.c_float))
-        d.rope_mscale = cfg.get("rope_mscale", 0.0)
-        d.act_alpha = cfg.get("act_alpha", 0.0)
-        d.act_limit = cfg.get("act_limit", 0.0)
-        d.kv_k_bits, d.kv_v_bits = kv_bits if kv_bits else (0, 0)
+        d, self._keep = model_desc(cfg, weights, kv_bits, session_slots)
         self.kv_bits = tuple(kv_bits) if kv_bits else None
-        d.session_slots = int(session_slots)
-        d.embed = ffi.tensor(weights["embed"])
-        d.final_norm = ffi.tensor(weights["final_norm"])
-        d.lm_head = ffi.tensor(weights.get("lm_head"))
-        d.layers = C.cast(self._layers, C.POINTER(ffi.Layer))
         h = C.c_void_p()
         ffi.check(ffi.lib().tsv_open(C.byref(d), C.byref(h)))
         self._h = h
@@ -314,7 +390,7 @@ class HipVerifier:
 
     # ---- the generation loop --------------------------------------------------------------
     def run_speculative(self, prompt, drafter, cfg, max_new_tokens, block, stop_tokens=(), adaptive_floor=0,
-                        device_logits=False):
+                        device_logits=False, block_drafts=True, chunked_prefill=True):
         """`run_speculative` (crates/runtime/src/speculative.rs:194-900) for a step-wise drafter and
         chain rounds, acceptance and truncation on the device.  `drafter` offers prime(next, pos),
         step(token, pos) -> uint16[vocab] and rewind(pos); with `device_logits` it offers
@@ -341,9 +417,43 @@ class HipVerifier:
             row = np.ascontiguousarray(drafter.step(token, pos), np.uint16)
             C.memmove(out, row.ctypes.data, vocab * 2)
 
-        d = ffi.Drafter(None, ffi.DRAFT_PRIME(guard(lambda u, t, p: drafter.prime(t, p))),
-                        ffi.DRAFT_STEP(guard(step)), ffi.DRAFT_REWIND(guard(lambda u, p: drafter.rewind(p))),
-                        1 if device_logits else 0)
+        if isinstance(drafter, MtpHead):
+            # the library's own callbacks; `block_drafts` / `chunked_prefill` False hand the loop a drafter
+            # without that callback (the step-wise walk of the same head)
+            d = ffi.Drafter()
+            ffi.check(ffi.lib().tsv_mtp_drafter(drafter._h, C.byref(d)))
+            if not block_drafts:
+                d.draft_block = ffi.DRAFT_BLOCK()
+            if not chunked_prefill:
+                d.prefill_chunk = ffi.DRAFT_PREFILL_CHUNK()
+            drafter = None
+        else:
+            d = ffi.Drafter(None, ffi.DRAFT_PRIME(guard(lambda u, t, p: drafter.prime(t, p))),
+                            ffi.DRAFT_STEP(guard(step)), ffi.DRAFT_REWIND(guard(lambda u, p: drafter.rewind(p))),
+                            1 if device_logits else 0)
+        if hasattr(drafter, "draft_block"):  # a block drafter: draft_block(anchor, base, block) -> tokens
+            def draft_block(user, anchor, base, block, out):
+                try:
+                    toks = drafter.draft_block(anchor, base, block)
+                    for i in range(min(len(toks), block)):  # (a short answer is the loop's to refuse)
+                        out[i] = int(toks[i])
+                    return 0 if len(toks) == block else 1
+                except Exception as e:
+                    failure.append(e)
+                    return 1
+            d.draft_block = ffi.DRAFT_BLOCK(draft_block)
+        if hasattr(drafter, "prefill_chunk"):  # prefill_chunk(tokens, start, next_token or None) -> uint16[vocab]
+            def prefill_chunk(user, tokens, n, start, out, next_token):
+                try:
+                    row = drafter.prefill_chunk([int(tokens[i]) for i in range(n)], int(start),
+                                                None if next_token < 0 else int(next_token))
+                    row = np.ascontiguousarray(row, np.uint16)
+                    C.memmove(out, row.ctypes.data, vocab * 2)
+                    return 0
+                except Exception as e:
+                    failure.append(e)
+                    return 1
+            d.prefill_chunk = ffi.DRAFT_PREFILL_CHUNK(prefill_chunk)
         if hasattr(drafter, "context_position"):  # lets the loop take over a prefix (the continuity guard)
             def where(user):
                 try:

@@ -83,6 +83,9 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
         return ffi.synth_tensor(dt if dtype is None else dtype, seed, stream[0], sigma if sig is None else sig,
                                 rows, cols)
 
+    # weak_layers < 1 scales what each layer adds to the stream (the output and down projections): the logits
+    # then follow the last token's embedding more than its context
+    weak = float(cfg.get("weak_layers", 1.0)) * sigma
     L = cfg["n_layers"] if n_layers is None else n_layers
     E = int(cfg.get("n_experts", 0))
     oss = cfg.get("gptoss")
@@ -99,16 +102,16 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
         cfg["act_alpha"], cfg["act_limit"] = oss["act_alpha"], oss["act_limit"]
     layers = []
     for li in range(L):
-        lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H, name=(li, "wv")), wo=t(H, qd),
+        lw = dict(attn_norm=ones(H), wq=t(qd, H), wk=t(kvd, H), wv=t(kvd, H, name=(li, "wv")), wo=t(H, qd, sig=weak),
                   ffn_norm=ones(H))
         if cfg.get("qk_norm"):  # Qwen3: RMSNorm over each q / k head before the rotation
             lw.update(q_norm=ones(cfg["head_dim"]), k_norm=ones(cfg["head_dim"]))
         if E:
             xd = cfg.get("expert_dtype", dt)
             lw.update(n_experts=E, top_k=int(cfg["top_k"]), router=t(E, H, sig=cfg.get("router_sigma", sigma)),
-                      we_gate=t(E * F, H, xd), we_up=t(E * F, H, xd), we_down=t(E * H, F, xd))
+                      we_gate=t(E * F, H, xd), we_up=t(E * F, H, xd), we_down=t(E * H, F, xd, sig=weak))
         else:
-            lw.update(w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F, name=(li, "w_down")))
+            lw.update(w_gate=t(F, H), w_up=t(F, H), w_down=t(H, F, sig=weak, name=(li, "w_down")))
         if oss:
             # attention biases and sinks are bf16 in the GGUF, expert and router biases f32
             lw.update(bq=vec(qd, 0.05, ffi.BF16), bk=vec(kvd, 0.05, ffi.BF16), bv=vec(kvd, 0.05, ffi.BF16),
@@ -122,3 +125,29 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
                           be_down=mat(E, H, 0.05))
         layers.append(lw)
     return dict(embed=t(V, H, name="embed"), final_norm=ones(H), lm_head=t(V, H, name="lm_head"), layers=layers)
+
+
+def make_mtp_weights(cfg, trunk_weights, seed=4321, sigma=0.02, follow=0.0):
+    """A drafter head for `cfg`'s target (docs/MTP.md:53-60): (head cfg, head weights) -- one decoder layer of
+    the target's shapes, its own norm, fc (hidden x 2 hidden) and the norms of fc's two halves, with the target's
+    embedding table, output head and final norm by reference.  `follow` > 0 adds that multiple of the identity
+    to fc's embedding half: with a target whose layers add little to the stream, both then predict from the
+    embedding of the last token, and the head's proposals are often the target's picks."""
+    hcfg = dict(cfg, n_layers=1)
+    hcfg.pop("overrides", None)
+    base = make_weights(hcfg, seed=seed, sigma=sigma, n_layers=1)
+    base["layers"][0]["window"] = 0  # the head's one layer attends over everything (docs/MTP.md:76-78)
+    H = cfg["hidden"]
+    rng = np.random.default_rng(seed + 5)
+
+    def near_one(n):
+        v = (1.0 + 0.1 * rng.uniform(-1.0, 1.0, (1, n))).astype(np.float32)
+        return (ffi.F32, v.view(np.uint8).reshape(1, -1), 1, n)
+
+    fc = (rng.standard_normal((H, 2 * H)) * sigma).astype(np.float32)
+    if follow:
+        fc[:, :H] += follow * np.eye(H, dtype=np.float32)
+    fdt = cfg["dtype"] if cfg["dtype"] != ffi.MXFP4 else ffi.BF16
+    return hcfg, dict(embed=trunk_weights["embed"], lm_head=trunk_weights.get("lm_head"), final_norm=near_one(H),
+                      layers=base["layers"], fc=ffi.quantize(fdt, fc), norm_embedding=near_one(H),
+                      norm_hidden=near_one(H), trunk_norm=trunk_weights["final_norm"])
