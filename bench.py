@@ -289,6 +289,17 @@ def main():
     ap.add_argument("--prefill-bench", type=int, default=0, metavar="TOKENS",
                     help="time tsv_prefill over a prompt of this many tokens (after one untimed run of the same), print one "
                          "JSON line and exit")
+    ap.add_argument("--loop-bench", type=int, default=0, metavar="NEW_TOKENS",
+                    help="end to end instead of one step: generate this many tokens with the library's loop and its "
+                         "drafter head (one decoder layer of the workload's shape, draft cost inside the timed region); "
+                         "prints verified tokens/s with the acceptance the synthetic weights give")
+    ap.add_argument("--weak-layers", type=float, default=1.0,
+                    help="--loop-bench: scale of what each layer adds to the stream; below 1 the target's picks follow "
+                         "the last token's embedding, which the synthetic head predicts (sets the acceptance rate)")
+    ap.add_argument("--embed-scale", type=float, default=1.0,
+                    help="--loop-bench: scale of the embedding rows, to the same end (the final norm removes it)")
+    ap.add_argument("--greedy", action="store_true", help="--loop-bench: temperature 0 (block drafts chained on the device)")
+    ap.add_argument("--step-drafts", action="store_true", help="--loop-bench: draft step by step even when greedy")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -335,6 +346,10 @@ def main():
     cfg["max_context"] = ctx + 32
     V = cfg["vocab"]
 
+    if args.loop_bench and args.weak_layers != 1.0:
+        cfg["weak_layers"] = args.weak_layers
+    if args.loop_bench and args.embed_scale != 1.0:
+        cfg["embed_scale"] = args.embed_scale
     t0 = time.time()
     weights = synth.make_weights(cfg, seed=args.seed)
     log(f"[bench] synthetic {wl['model']} weights ({cfg['n_layers']} layers) in {time.time() - t0:.1f}s")
@@ -358,6 +373,9 @@ def main():
                           "higher_is_better": True, "dtype": "f16", "data": "synthetic", "seconds": round(dt, 4),
                           "config": {"workload": args.workload, "layers": cfg["n_layers"], "prompt_tokens": n,
                                      "rows_per_pass": rows, "logits": "none (headless passes)"}}))
+        return
+    if args.loop_bench:
+        loop_bench(args, ts, synth, cfg, weights, eng, wl, rng)
         return
     prompt = rng.integers(0, V, ctx).astype(np.int32)
     t0 = time.time()
@@ -532,6 +550,59 @@ def main():
         "prefill": {"tokens": ctx - 1, "seconds": round(prefill_s, 3), "tokens_per_s": round((ctx - 1) / prefill_s, 1)},
     }
     print(json.dumps(out), flush=True)
+
+
+def loop_bench(args, ts, synth, cfg, weights, eng, wl, rng):
+    """Verified tokens/s of the whole loop: prompt of ctx - NEW tokens, then NEW tokens generated by
+    tsv_run_speculative with the drafter head inside the library (chain rounds of the workload's k).  The timed
+    region is the difference of two runs of the same prompt, one generating 1 token and one 1 + NEW: every
+    draft step, verify pass, acceptance and truncation of the NEW tokens, and nothing of the prompt."""
+    k, ctx, V = wl["k"], wl["ctx"], cfg["vocab"]
+    T = 0.0 if args.greedy else wl["temperature"]
+    new = args.loop_bench
+    hcfg, hw = synth.make_mtp_weights(cfg, weights, seed=args.seed + 1, follow=256.0, norm_jitter=0.0)
+    head = ts.MtpHead(eng, hcfg, hw)
+    prompt = rng.integers(0, V, ctx - new).astype(np.int32)
+    sh = ts.shaping(T, seed=args.seed) if T > 0 else ts.shaping(0.0)
+
+    def run(n_new):
+        t0 = time.perf_counter()
+        r = eng.run_speculative(prompt, head, sh, n_new, k, block_drafts=not args.step_drafts)
+        return time.perf_counter() - t0, r
+
+    run(k + 2)   # untimed: first-use allocations, code objects
+    t_a, _ = run(1)
+    t_b, r = run(1 + new)
+    dt = t_b - t_a
+    log(f"[bench] prompt of {prompt.size} tokens + 1 token: {t_a:.2f}s; + {new} more: {t_b:.2f}s")
+    # the draft side alone: the block of k chained steps (plus the row-only step) from where the run ended
+    pos = eng.position
+    reps = 20
+    head.draft_block(r["tokens"][-1], pos, k)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        head.rewind(pos - 1)
+        head.draft_block(r["tokens"][-1], pos, k)
+    draft_ms = (time.perf_counter() - t0) * 1e3 / reps
+    head.rewind(pos - 1)
+    # plain decoding on the same handle at the same context: one-row rounds (pass, device arg-max, no draft)
+    tok, plain_n = int(r["tokens"][-1]), min(64, eng.cfg["max_context"] - pos - 1)
+    greedy = ts.shaping(0.0)
+    t0 = time.perf_counter()
+    for i in range(plain_n):
+        tok = eng.verify_accept([tok], pos + i, greedy).next
+    plain_s = time.perf_counter() - t0
+    print(json.dumps({
+        "metric": "verified tokens/s, end to end (drafter head inside the library)", "value": round(new / dt, 1),
+        "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "f16", "data": "synthetic",
+        "new_tokens": new, "seconds": round(dt, 4), "rounds": r["rounds"], "offered": r["offered"],
+        "accepted": r["accepted"], "tokens_per_round": round(new / max(r["rounds"], 1), 3),
+        "ms_per_round": round(dt * 1e3 / max(r["rounds"], 1), 3),
+        "prompt_tokens_per_s": round(prompt.size / t_a, 1), "draft_ms_per_block": round(draft_ms, 3),
+        "plain_decode_tokens_per_s": round(plain_n / plain_s, 1), "vs_plain_decode": round(new / dt / (plain_n / plain_s), 2),
+        "config": {"workload": args.workload, "layers": cfg["n_layers"], "block": k, "temperature": T,
+                   "drafts": "step by step" if (args.step_drafts or T > 0) else "block, chained on the device",
+                   "weak_layers": args.weak_layers, "embed_scale": args.embed_scale, "prompt_tokens": int(prompt.size)}}))
 
 
 def cpu_baseline(cfg, weights, eng, base, feed, mean_acc, parent=None):

@@ -124,10 +124,12 @@ def make_weights(cfg, seed=1234, sigma=0.02, n_layers=None):
                 lw.update(router_bias=vec(E, 0.05), be_gate=mat(E, F, 0.05), be_up=mat(E, F, 0.05),
                           be_down=mat(E, H, 0.05))
         layers.append(lw)
-    return dict(embed=t(V, H, name="embed"), final_norm=ones(H), lm_head=t(V, H, name="lm_head"), layers=layers)
+    # embed_scale > 1: embedding rows that dwarf what the layers add (the final norm takes the scale out again)
+    return dict(embed=t(V, H, sig=sigma * float(cfg.get("embed_scale", 1.0)), name="embed"), final_norm=ones(H),
+                lm_head=t(V, H, name="lm_head"), layers=layers)
 
 
-def make_mtp_weights(cfg, trunk_weights, seed=4321, sigma=0.02, follow=0.0):
+def make_mtp_weights(cfg, trunk_weights, seed=4321, sigma=0.02, follow=0.0, norm_jitter=0.1):
     """A drafter head for `cfg`'s target (docs/MTP.md:53-60): (head cfg, head weights) -- one decoder layer of
     the target's shapes, its own norm, fc (hidden x 2 hidden) and the norms of fc's two halves, with the target's
     embedding table, output head and final norm by reference.  `follow` > 0 adds that multiple of the identity
@@ -141,7 +143,7 @@ def make_mtp_weights(cfg, trunk_weights, seed=4321, sigma=0.02, follow=0.0):
     rng = np.random.default_rng(seed + 5)
 
     def near_one(n):
-        v = (1.0 + 0.1 * rng.uniform(-1.0, 1.0, (1, n))).astype(np.float32)
+        v = (1.0 + norm_jitter * rng.uniform(-1.0, 1.0, (1, n))).astype(np.float32)
         return (ffi.F32, v.view(np.uint8).reshape(1, -1), 1, n)
 
     fc = (rng.standard_normal((H, 2 * H)) * sigma).astype(np.float32)
