@@ -901,7 +901,12 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
             return rc;
         prev_splits = sp;
     }
-    return TSV_OK;  // headless: the last layer's sums are never added, nobody reads these rows' logits
+    // headless: nobody reads these rows' logits, and the last layer's sums are added only for a drafter head,
+    // which reads the finished rows (64 consecutive rows of w.x)
+    if (c->mtp_head)
+        return launch_addnorm(s, w.x, w.partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr,
+                              nullptr, nullptr, 0, WIDE_B, &nb);
+    return TSV_OK;
 }
 
 // One 64-row prompt pass at the cursor: parameters of the four blocks, then the kernels.
@@ -926,6 +931,8 @@ int enqueue_wide_prefill(tsv_ctx* c, const int32_t* ids, int64_t base) {
     c->position = base + rows;
     c->high_water = std::max(c->high_water, c->position);
     c->last_m = 0;  // no logits on the device for tsv_accept to judge
+    c->x_rows = 0;  // (the pass's rows are in the wide buffers, not in x)
+    if (c->mtp_head) c->mtp_head->mtp.own_valid = false;
     return TSV_OK;
 }
 
@@ -1594,8 +1601,16 @@ static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos
     const int wide_rows = 16 * WIDE_B;
     for (int64_t i = 0; i < n;) {
         // 64 rows at a time while that many remain and nobody wants their logits
-        if (c->wide.ok && !c->profile && n - i >= wide_rows && (i + wide_rows < n || !logits)) {
+        // (with a drafter head the last pass is a sixteen-row one: the first draft step reads its rows)
+        if (c->wide.ok && !c->profile && n - i >= wide_rows && (i + wide_rows < n || (!logits && !head))) {
             if (int rc = enqueue_wide_prefill(c, ids + i, pos0 + i)) return rc;
+            if (head) {
+                for (int b = 0; b < WIDE_B; b++) {
+                    int32_t nt[TSV_MAX_ROWS];
+                    for (int r = 0; r < 16; r++) nt[r] = ids[i + 16 * b + r + 1];  // (i + 64 < n: every row has a next token)
+                    if (int rc = mtp_pass(head, nt, 16, pos0 + i + 16 * b, c->wide.x + (size_t)b * 16 * c->hidden, false)) return rc;
+                }
+            }
             i += wide_rows;
             continue;
         }
@@ -1696,7 +1711,6 @@ extern "C" int32_t tsv_mtp_open(tsv_ctx* target, const tsv_mtp_desc* d, tsv_ctx*
     const int rc = open_impl(&m, target, d, out);
     if (rc) return rc;
     target->mtp_head = *out;
-    target->wide.ok = false;  // the head reads each prompt pass's rows where the sixteen-row pass leaves them
     return TSV_OK;
 }
 
