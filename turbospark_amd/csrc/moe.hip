@@ -116,71 +116,38 @@ __device__ __forceinline__ void route_row(const MoeRouteArgs& a, int m, uint32_t
     }
 }
 
-// Router matmul and top-k in one kernel: a workgroup of sixteen waves per group of four rows.  The waves split
-// the router's tiles and K chunks among them (the dense matmul's own tile sequences, one row group), their sums
-// are folded through LDS in wave order, and wave i of the first four then ranks row 4 g + i.  The groups of
-// rows that share an expert are not built here: every expert matmul workgroup derives its own from the
-// selections (moe_derive_group), which takes a wave a few dozen instructions.
-template <class F>
-__global__ __launch_bounds__(1024) void k_route_fused(MoeRouteArgs a) {
-    __shared__ float4v red[16 * 64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int g = blockIdx.x, nt = a.n_tiles, parts = 16 / nt;
-    const int tile = wave % nt, part = wave / nt;
-    const int per = (a.kchunks + parts - 1) / parts;
-    const int c0 = min(part * per, a.kchunks), nc = min(per, a.kchunks - c0);
-    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * F::TILE_BYTES;
-    Consts k;
-    k.k6400 = 0x64006400u;
-    k.k5400 = 0x54005400u;
-    k.k64 = 0x64646464u;
-    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
-    ActLoader<false> x(a.xfrag, a.xsum, lane);
-    x.set_row(0, 4 * g + (lane & 3));
-    // what the ranking needs besides the logits, asked for now (row 4 g + wave; waves past the fourth read row 4 g's)
-    const int mrow = min(4 * g + (wave & 3), TSV_MAX_ROWS - 1);
-    const int forced_first = a.forced ? a.forced[mrow * 8] : -1;
-    const int forced_mine = a.forced ? a.forced[mrow * 8 + (lane & 7)] : -1;
-    float bias[4];
+// The ranking of every row of a pass: one workgroup, wave m ranks row m.  The router matmul before it is the dense
+// one (split-K partial sums, a workgroup per tile and K slice): its sums are added here in split order.  The
+// groups of rows that share an expert are not built here: every expert matmul workgroup derives its own from
+// the selections (moe_derive_group), which takes a wave a few dozen instructions.
+// (One launch for matmul and ranking -- a workgroup of sixteen waves per four rows walking the whole router --
+// measured 12.3 us against 4.8 + 4.2 at 128 x 2048 Q8_0 and 19.5 against 4.6 + 4.3 at 128 x 2880 bf16: a
+// workgroup's 32 or 90 tile chunks are issue-bound on its one compute unit.)
+__global__ __launch_bounds__(1024) void k_route_rank(MoeRouteArgs a) {
+    const int lane = threadIdx.x & 63, m = threadIdx.x >> 6;
+    if (m >= a.m) return;
+    const int ne = a.n_experts;
+    // everything the row needs is asked for before the first add: the loads have no branch between them (a lane
+    // past the last expert reads the last expert's, a split past the last split the last split's again)
+    const int forced_first = a.forced ? a.forced[m * 8] : -1;
+    const int forced_mine = a.forced ? a.forced[m * 8 + (lane & 7)] : -1;
+    float part[4][8], bias[4];
+    const int nj = ne <= 128 ? 2 : 4;
 #pragma unroll
-    for (int j = 0; j < 4; j++) bias[j] = a.bias ? a.bias[min(lane + 64 * j, a.n_experts - 1)] : 0.f;
-    float4v acc[1] = {float4v{0.f, 0.f, 0.f, 0.f}};
-    if (nc > 0) {
-        Stage<F, 1> st[2];
-        const int last = c0 + nc - 1;
-        auto fetch = [&](Stage<F, 1>& sg, int c) { load_stage(sg, x, wt + (size_t)c * F::TILE_BYTES, c, lane); };
-        fetch(st[0], c0);
-        fetch(st[1], min(c0 + 1, last));
-        int c = 0;
-        for (; c + 4 <= nc; c += 2) {
-            compute(st[0], k, acc);
-            fetch(st[0], c0 + c + 2);
-            compute(st[1], k, acc);
-            fetch(st[1], c0 + c + 3);
-        }
-        for (int s2 = 0; s2 < 2; s2++)
-            if (c + s2 < nc) {
-                compute(st[s2], k, acc);
-                if (c + s2 + 2 < nc) fetch(st[s2], c0 + c + s2 + 2);
-            }
-        c += 2;
-        for (int s2 = 0; s2 < 2; s2++)
-            if (c + s2 < nc) compute(st[s2], k, acc);
+    for (int j = 0; j < 4; j++) {
+        const int e = min(lane + 64 * j, ne - 1);
+        bias[j] = a.bias && j < nj ? a.bias[e] : 0.f;  // before the top-k (families/gptoss/moe.rs:82-87)
+#pragma unroll
+        for (int sp = 0; sp < 8; sp++) part[j][sp] = j < nj ? a.logits[((size_t)min(sp, a.splits - 1) * 16 + m) * a.ld + e] : 0.f;
     }
-    red[wave * 64 + lane] = acc[0];
-    __syncthreads();
-    const int m = 4 * g + wave;
-    if (wave >= 4 || m >= a.m) return;
     uint32_t key[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        if (j < nt) {
-            float sum = 0.f;  // the K parts in order
-            for (int p = 0; p < parts; p++) sum += red[(p * nt + j) * 64 + lane][wave];
-            const int e = lane + 64 * j;
-            if (a.bias) sum += bias[j];  // before the top-k (families/gptoss/moe.rs:82-87)
-            if (e < a.n_experts) key[j] = order_key(sum);
-        }
+        float sum = 0.f;  // added in split order
+#pragma unroll
+        for (int sp = 0; sp < 8; sp++) sum += sp < a.splits ? part[j][sp] : 0.f;
+        if (a.bias) sum += bias[j];
+        if (j < nj && lane + 64 * j < ne) key[j] = order_key(sum);
     }
     route_row(a, m, key, lane, forced_first, forced_mine);
 }
@@ -342,24 +309,16 @@ int launch_moe_f(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
 
 }  // namespace
 
-int launch_route(hipStream_t s, int fmt, const MoeRouteArgs& a) {
+int launch_route(hipStream_t s, const MoeRouteArgs& a) {
     if (a.n_experts > 256 || a.top_k < 1 || a.top_k > 8 || a.top_k > a.n_experts) {
         set_error("moe: at most 256 experts and top-k between 1 and 8");
         return TSV_ERR_UNSUPPORTED;
     }
-    if (a.n_tiles != 1 && a.n_tiles != 2 && a.n_tiles != 4) {
-        set_error("moe: the router's experts must fill one, two or four 64-row tiles");
+    if (a.splits < 1 || a.splits > 8 || a.m < 1 || a.m > TSV_MAX_ROWS) {
+        set_error("moe: the router's logits come in one to eight partial sums of at most sixteen rows");
         return TSV_ERR_UNSUPPORTED;
     }
-    const dim3 grid((a.m + 3) / 4), block(1024);
-    switch (fmt) {
-        case FMT_Q4K: hipLaunchKernelGGL(k_route_fused<Q4K>, grid, block, 0, s, a); break;
-        case FMT_Q80: hipLaunchKernelGGL(k_route_fused<Q80>, grid, block, 0, s, a); break;
-        case FMT_Q6K: hipLaunchKernelGGL(k_route_fused<Q6K>, grid, block, 0, s, a); break;
-        case FMT_Q5K: hipLaunchKernelGGL(k_route_fused<Q5K>, grid, block, 0, s, a); break;
-        case FMT_BF16: hipLaunchKernelGGL(k_route_fused<BF16W>, grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL(k_route_fused<MX4>, grid, block, 0, s, a); break;
-    }
+    hipLaunchKernelGGL(k_route_rank, dim3(1), dim3(64 * a.m), 0, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -664,11 +664,10 @@ int launch_pass(tsv_ctx* c, int m) {
             // router -> top-k -> grouped expert matmuls; the per-slot outputs are added, weighted
             // and in slot order, by the next residual kernel
             MoeRouteArgs ra2{};
-            ra2.w = L.router.tiles;
-            ra2.n_tiles = L.router.n_tiles;
-            ra2.kchunks = L.router.kchunks;
-            ra2.xfrag = (const uint2*)c->xf_a;
-            ra2.xsum = (const float*)((const char*)c->xf_a + xfrag_sum_offset(c->hidden));
+            const int rsp = splits_for(L.router, m, EPI_PARTIAL);
+            ra2.logits = c->partial;
+            ra2.splits = rsp;
+            ra2.ld = L.n_experts;
             ra2.n_experts = L.n_experts;
             ra2.top_k = L.top_k;
             ra2.m = m;
@@ -722,7 +721,8 @@ int launch_pass(tsv_ctx* c, int m) {
                 PROF(PC_GATEUP);
                 rc = 0;
                 for (int rep = 0; rep < c->repeat[PC_GATEUP] && !rc; rep++) {
-                    rc = launch_route(s, L.router.fmt, ra2);
+                    rc = launch_gemm(s, L.router, c->xf_a, c->partial, c->vp_dev, m, rsp, EPI_PARTIAL, L.n_experts, L.n_experts);
+                    if (!rc) rc = launch_route(s, ra2);
                     if (!rc) rc = fp4 ? launch_moe_fp4_gate_up(s, g1, n_groups) : launch_moe_gate_up(s, L.gate_up.fmt, g1, n_groups);
                 }
             }
@@ -1101,6 +1101,7 @@ static int open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc
             if ((rc = make_tiled(c, st, rt, 1, false, &L.router)) || (rc = make_tiled(c, st, gu, 2, true, &L.gate_up)) ||
                 (rc = make_tiled(c, st, dn, 1, false, &L.down)))
                 return fail(rc);
+            pneed = std::max(pneed, partial_need(L.router));
             L.n_experts = ne;
             L.top_k = s.top_k;
             if (L.gate_up.fmt != FMT_MX4 || L.down.fmt != FMT_MX4) c->moe_fp4_terms = 0;

@@ -192,10 +192,8 @@ struct MoeGroup {
     int32_t rows[16], slots[16];
 };
 struct MoeRouteArgs {
-    const uint8_t* w;     // the router's tiled weights: n_tiles tiles of 64 experts x kchunks
-    int n_tiles, kchunks;
-    const uint2* xfrag;   // the pass's activation fragments and their sub-block sums
-    const float* xsum;
+    const float* logits;  // the router matmul's split-K partial sums: [splits][16][ld]
+    int splits, ld;
     int n_experts, top_k;
     int m;              // rows of the pass (the launch sequence is per row count)
     float* weights;     // [16][8] softmax over the selected logits, rank order
@@ -282,7 +280,7 @@ struct MoeGemmArgs {
     const float* bias2;
     float alpha, limit;    // alpha > 0: clamped SwiGLU (moe_gguf.metal:528-556) instead of silu(g) * u
 };
-int launch_route(hipStream_t s, int fmt, const MoeRouteArgs& a);
+int launch_route(hipStream_t s, const MoeRouteArgs& a);
 int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 // the same two matmuls on v_mfma_scale_f32_16x16x128_f8f6f4 (moe_fp4.hip)
