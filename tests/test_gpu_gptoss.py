@@ -180,6 +180,38 @@ def test_windowed_layers_as_rings_equal_the_linear_layout_by_bits():
     assert np.array_equal(lin.prefill(prompt[:70], 0), ring.prefill(prompt[:70], 0))
 
 
+def test_after_rejected_rounds_the_rewind_budget_counts_from_the_last_row_written():
+    """Rounds that write sixteen rows and keep one (everything else rejected) leave the cursor fifteen rows
+    behind the last row written; the rows of a ring are overwritten up to that row, so the budget
+    (capacity - window = 40, kv_cache_rewind.rs:26-35) is counted from it: a rollback may go 40 rows below the
+    last row written -- 25 committed rows here -- and one row more is refused by name.  The rings give the
+    linear layout's logits after that deepest rollback."""
+    import turbospark_amd as ts
+    from turbospark_amd import TsvError
+    cfg, lin, ring = _ring_pair("gptoss_small", 400)
+    V = cfg["vocab"]
+    prompt = _prompt(120, V, 9)
+    assert np.array_equal(lin.prefill(prompt, 0), ring.prefill(prompt, 0))
+    rng = np.random.default_rng(4)
+    base = 120
+    for rnd in range(30):
+        feed = rng.integers(0, V, 16).astype(np.int32)
+        pa, pb = lin.checkpoint(), ring.checkpoint()
+        assert np.array_equal(lin.verify(feed, base), ring.verify(feed, base)), rnd
+        lin.rollback_retaining(pa, 1)
+        ring.rollback_retaining(pb, 1)
+        base += 1
+    written = base + 15                          # one past the last row written: the last round's sixteenth row
+    assert ring.position == base
+    with pytest.raises(TsvError, match="exceeds the ring slack"):
+        ring.rollback(ts.ffi.Point(written - 41))
+    assert ring.position == base                 # a refused rollback moves nothing
+    ring.rollback(ts.ffi.Point(written - 40))    # 25 committed rows back
+    lin.rollback(ts.ffi.Point(written - 40))
+    nxt = rng.integers(0, V, 5).astype(np.int32)
+    assert np.array_equal(lin.verify(nxt, written - 40), ring.verify(nxt, written - 40))
+
+
 def test_gptoss_120b_geometry_ring_equals_linear_at_long_context():
     """The gpt-oss-120B geometry (window 128 -> a ring of 160 slots beside a 3000-token context): seeded
     rows written into both layouts, a nine-row pass, a rollback and a second pass, equal by bits."""
