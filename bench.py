@@ -17,6 +17,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+os.environ.setdefault("TSV_MEASUREMENT_HOOKS", "1")   # the per-class timing and repeated launches answer only under this
 
 WORKLOADS = {
     # the headline configuration: 8B-shaped Q4_K target, chain k = 4, 4096-token context, T = 0.8
@@ -111,34 +112,74 @@ def trace_summary(path, first="k_clear_result"):
     print(f"total kernel time in {what}: {total / 1e6:.3f} ms over the traced steps")
 
 
-# Figures RECORDED from committed counter / trace runs (a bench run does not collect counters).  `traffic`: HBM
-# bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, scaled by the
-# copy kernel of known size (headline workload: over `bench.py --traffic-probe`, 66 793 486 B read + 258 048 B
-# written against 66 060 288 algorithmic bytes; the others: the kernel's rows of `bench.py --step-traffic`, for the
-# routed workloads router + top-k + grouped gate/up together, as `achieved` counts them).  `trace_avg_us`: the same
-# kernel(s) in the committed rocprofv3 kernel trace of this script.  `step_traffic`: bytes read + written per
-# verify pass over all its kernels, to set beside `step_algorithmic_bytes`.
-_TRAFFIC = "recorded: profiles/verify_step_hbm_traffic_by_kernel_all_workloads.txt"
-RECORDED = {
+# Figures read from the committed counter / trace summaries under profiles/ (a bench run does not collect counters).
+# For each workload: the kernels `achieved` counts (the dominant launch: the gate/up matmul; for the routed workloads
+# router matmul + ranking + grouped gate/up together), named as the tables name them with the workgroup count that
+# tells same-named launches apart (None: the name is unique).  `traffic`: their HBM bytes per launch from
+# `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`, each counter scaled by the copy kernel of known size (the rows of
+# `bench.py --step-traffic`); `trace_avg_us`: the same kernels in the rocprofv3 kernel trace of this script;
+# `step_traffic`: bytes read + written per verify pass over all its kernels, to set beside `step_algorithmic_bytes`.
+_TRAFFIC = "profiles/verify_step_hbm_traffic_by_kernel_all_workloads.txt"
+PROFILED = {
     "llama3_8b_q4_k_k4_ctx4096": dict(
-        traffic=67051534, traffic_source="recorded: profiles/gate_up_matmul_llama3_8b_q4k_hbm_traffic.txt",
-        trace_avg_us=16.17, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt",
-        step_traffic=5057454669 + 166119858, step_traffic_source=_TRAFFIC),
+        trace="profiles/verify_step_llama3_8b_q4k_ctx4096_kernels.txt", kernels=[("k_gemm<Q4K, 1, 2>", 448, 448)]),
     "llama3_8b_q4_k_tree16_ctx16384": dict(
-        traffic=67348044 + 516096, traffic_source=_TRAFFIC,
-        trace_avg_us=20.46, trace_source="recorded: profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt",
-        step_traffic=6973116518 + 511734731, step_traffic_source=_TRAFFIC),
+        trace="profiles/verify_step_llama3_8b_q4k_tree16_ctx16384_kernels.txt", kernels=[("k_gemm16<1>", 448, 448)]),
     "qwen3_30b_a3b_mxfp4_k8_ctx8192": dict(
-        traffic=(526294 + 18432) + (38401 + 3978) + (17877765 + 139726), traffic_source=_TRAFFIC,
-        trace_avg_us=4.80 + 6.69 + 9.80, trace_source="recorded: profiles/verify_step_qwen3_30b_a3b_mxfp4_ctx8192_kernels.txt "
-                                                      "(router + k_route + k_moe_fp4<1, 2, 1>)",
-        step_traffic=3815633101 + 291355412, step_traffic_source=_TRAFFIC),
+        trace="profiles/verify_step_qwen3_30b_a3b_mxfp4_ctx8192_kernels.txt",
+        kernels=[("k_gemm<Q80, 0, 4>", 8, 8), ("k_route_rank", None, None), ("k_moe_gemm<MX4, 1, 2>", None, None)]),
     "gptoss_120b_mxfp4_k8_ctx32768": dict(
-        traffic=(917440 + 36864) + (57345 + 3680) + (175608367 + 262669), traffic_source=_TRAFFIC,
-        trace_avg_us=4.56 + 5.43 + 35.22, trace_source="recorded: profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt "
-                                                       "(router + k_route + k_moe_fp4<1, 2, 1>)",
-        step_traffic=14135922230 + 229660271, step_traffic_source=_TRAFFIC),
+        trace="profiles/verify_step_gptoss_120b_mxfp4_ctx32768_kernels.txt",
+        kernels=[("k_gemm<BF16W, 0, 4>", 16, 16), ("k_route_rank", None, None), ("k_moe_gemm<MX4, 1, 1>", None, None)]),
 }
+
+
+def _table_rows(lines, n_numbers):
+    """(kernel name, [numbers]) of every table line: the name, then `n_numbers` right-aligned numeric columns."""
+    import re
+    pat = re.compile(r"^(\S.*?)" + r"\s+(-?[\d.]+)%?" * n_numbers + r"\s*$")
+    for l in lines:
+        m = pat.match(l.rstrip("\n"))
+        if m and not l.startswith(("#", "kernel ")):
+            yield m.group(1), [float(g) for g in m.groups()[1:]]
+
+
+def recorded(workload):
+    """The workload's figures out of profiles/ (see PROFILED), or {} where a summary is missing or names none of the kernels."""
+    spec = PROFILED.get(workload)
+    if not spec:
+        return {}
+    try:
+        out = {}
+        trace = list(_table_rows(open(os.path.join(ROOT, spec["trace"])), 7))   # wgs lds calls avg min max share
+        section, per_pass = [], None
+        inside = False
+        for l in open(os.path.join(ROOT, _TRAFFIC)):
+            if l.startswith("## "):
+                inside = l[3:].strip() == workload
+            elif inside:
+                section.append(l)
+                if l.startswith("all dispatches from the first"):
+                    w = l.split()
+                    per_pass = int(w[w.index("B") - 1]) + int(w[w.index("written") - 2])
+        traffic = list(_table_rows(section, 4))                                   # wgs calls read written
+        us, nbytes = 0.0, 0
+        for name, trace_wgs, traffic_wgs in spec["kernels"]:
+            t = [v for n, v in trace if n == name and (trace_wgs is None or v[0] == trace_wgs)]
+            b = [v for n, v in traffic if n == name and (traffic_wgs is None or v[0] == traffic_wgs)]
+            if len(t) != 1 or len(b) != 1:
+                return {}
+            us += t[0][3]
+            nbytes += int(b[0][2] + b[0][3])
+        names = " + ".join(n for n, _, _ in spec["kernels"])
+        out.update(trace_avg_us=us, trace_source=f"recorded: {spec['trace']} ({names})", traffic=nbytes,
+                   traffic_source=f"recorded: {_TRAFFIC} ({names})")
+        if per_pass:
+            out.update(step_traffic=per_pass, step_traffic_source=f"recorded: {_TRAFFIC}")
+        return out
+    except (OSError, ValueError):
+        return {}
+
 
 GATE_UP_8B = dict(dtype=12, rows=28672, cols=4096, m=5, epi=1)   # the dominant kernel of the headline workload
 COPY_BYTES = 256 << 20
@@ -498,7 +539,7 @@ def main():
     dom = kern.get("gate_up", {})
     peak = 8000.0
     # the recorded figures are the workload's as named: not a variant's (other KV rows, forced routing, fewer layers)
-    rec = {} if (kv_bits or args.routing != "model" or args.layers) else RECORDED.get(args.workload, {})
+    rec = {} if (kv_bits or args.routing != "model" or args.layers) else recorded(args.workload)
     roofline = dict(bound="hbm",
                     kernel=f"router + grouped expert gate/up matmuls (experts actually routed: {union:.1f} of {cfg['n_experts']} per layer)"
                     if cfg.get("n_experts")
@@ -534,8 +575,8 @@ def main():
         "dtype_detail": {12: "q4_k", 8: "q8_0", 30: "bf16"}[cfg["dtype"]] +
                         " weight codes as exact f16 x f16 activations on MFMA, f32 accumulate" +
                         ("" if not cfg.get("n_experts") else
-                         "; mxfp4 experts as f16 x f16 too (TSV_MOE_FP4=0)" if os.environ.get("TSV_MOE_FP4") == "0" else
-                         "; mxfp4 experts as stored on the block-scaled fp4 x fp8 MFMA, activations as " +
+                         "; mxfp4 experts as f16 x f16 too" if os.environ.get("TSV_MOE_FP4", "0") not in ("2", "3") else
+                         "; mxfp4 experts as stored on the block-scaled fp4 x fp8 MFMA (TSV_MOE_FP4), activations as " +
                          ("three" if os.environ.get("TSV_MOE_FP4") == "3" else "two") + " block-scaled e4m3 terms") +
                         "; f64 acceptance",
         "data": "synthetic",

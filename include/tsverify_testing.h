@@ -38,6 +38,9 @@ int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int
  * a node, or rejects j - 1, accepts the j-th and goes on below it).  -1 for a malformed tree. */
 int32_t tsv_tree_walk_bound(const int32_t* parent, int32_t m);
 
+/* The four measurement hooks below (tsv_set_profile, tsv_set_repeat, tsv_matmul_time, tsv_copy_time) answer only in
+ * a process whose environment carries TSV_MEASUREMENT_HOOKS=1; anywhere else turning one on is refused by name
+ * (TSV_ERR_UNSUPPORTED) and the library runs exactly its serving path. */
 /* Per-kernel-class timing with HIP events on the handle's stream (one event pair per launch
  * while enabled).  Classes, in order: embed, norm, qkv matmul, rope+kv store, attention,
  * output projection, gate/up matmul, down matmul, output head, acceptance, and "event pair":

@@ -131,6 +131,12 @@ def test_null_handles_are_refused_by_name_without_a_gpu():
         lambda: L.tsv_gguf_meta_number(None, b"x", None),
         lambda: L.tsv_gguf_meta_string(None, b"x", None, 0),
         lambda: L.tsv_open_gguf(None, 0, C.byref(C.c_void_p())),
+        lambda: L.tsv_mtp_open(None, None, C.byref(C.c_void_p())),
+        lambda: L.tsv_mtp_step(None, 1, 0, None, 0),
+        lambda: L.tsv_mtp_rewind(None, 0),
+        lambda: L.tsv_mtp_prefill_chunk(None, tok, 4, 0, out, -1),
+        lambda: L.tsv_mtp_draft_block(None, 1, 1, 2, tok),
+        lambda: L.tsv_mtp_drafter(None, None),
     ]
     for i, call in enumerate(calls):
         assert call() != 0, i
@@ -151,3 +157,16 @@ def test_null_handles_are_refused_by_name_without_a_gpu():
     desc.ffn, desc.vocab, desc.max_context = 64, 100, 16
     handle = C.c_void_p()
     assert L.tsv_open(C.byref(desc), C.byref(handle)) != 0 and "positive" in ffi.last_error()
+
+
+def test_measurement_hooks_answer_only_under_their_switch(monkeypatch):
+    """The timing loops refuse by name in a process without TSV_MEASUREMENT_HOOKS=1 -- before any device call,
+    so this runs without a GPU."""
+    import ctypes as C
+    from turbospark_amd import ffi
+    L = ffi.lib()
+    monkeypatch.delenv("TSV_MEASUREMENT_HOOKS", raising=False)
+    t = C.c_float()
+    for call in (lambda: L.tsv_copy_time(1 << 20, 1, C.byref(t)),
+                 lambda: L.tsv_matmul_time(ffi.Q4_K, 64, 256, 4, 0, 0, 1, 1, C.byref(t))):
+        assert call() == -3 and "TSV_MEASUREMENT_HOOKS=1" in ffi.last_error()

@@ -1427,8 +1427,20 @@ extern "C" void tsv_close(tsv_ctx* c) {
     delete c;
 }
 
+// The measurement hooks (per-class event pairs, repeated launches, the timing loops) answer only in a process
+// whose environment carries TSV_MEASUREMENT_HOOKS=1: a serving process cannot be put into a measuring mode by
+// a stray call.
+static int measurement_hooks_on(const char* who) {
+    const char* e = getenv("TSV_MEASUREMENT_HOOKS");
+    if (e && e[0] == '1') return TSV_OK;
+    set_error(std::string(who) + ": measurement hooks are off (set TSV_MEASUREMENT_HOOKS=1 in the process environment)");
+    return TSV_ERR_UNSUPPORTED;
+}
+
 extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
     TSV_NEED(c, "set_profile: null handle");
+    if (on)
+        if (int rc = measurement_hooks_on("set_profile")) return rc;
     TSV_HIP(hipStreamSynchronize(c->stream));
     c->profile = on != 0;
     c->ev_used = 0;
@@ -1437,6 +1449,8 @@ extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
 
 extern "C" int32_t tsv_set_repeat(tsv_ctx* c, int32_t cls, int32_t times) {
     TSV_NEED(c, "set_repeat: null handle");
+    if (times != 1)
+        if (int rc = measurement_hooks_on("set_repeat")) return rc;
     if (cls != PC_QKV && cls != PC_ROPE && cls != PC_ATTN && cls != PC_WO && cls != PC_GATEUP && cls != PC_DOWN &&
         cls != PC_HEAD) {
         set_error("set_repeat: only the matmul, rope and attention classes can be repeated");
@@ -2671,6 +2685,7 @@ __global__ __launch_bounds__(256) void k_copy_probe(const uint4* __restrict__ sr
 }  // namespace
 
 extern "C" int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us) {
+    if (int hrc = measurement_hooks_on("copy_time")) return hrc;
     if (bytes < 16 || bytes % 16 || iters < 1 || !avg_us) {
         set_error("copy_time: bad argument");
         return TSV_ERR_INVALID;
@@ -2717,6 +2732,7 @@ extern "C" int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us) {
 // kernel streams from HBM rather than from cache.
 extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
                                    int32_t iters, int32_t rotate, float* avg_us) {
+    if (int hrc = measurement_hooks_on("matmul_time")) return hrc;
     const int fmt = dtype_fmt(dtype);
     if (fmt < 0 || rows % TILE_ROWS || cols % fmt_chunk_elems(fmt) || m < 1 || m > TSV_MAX_ROWS || iters < 1 || rotate < 1) {
         set_error("matmul_time: bad argument");
