@@ -420,7 +420,14 @@ def main():
         return
     prompt = rng.integers(0, V, ctx).astype(np.int32)
     t0 = time.time()
-    eng.prefill(prompt[:-1], 0, want_logits=False)   # the last prompt token is the round's confirmed token
+    if args.copy_probe:
+        # a counter run: the prompt goes one pass per call, each ending with the stream drained (with a few thousand
+        # launches queued ahead of the device the counter collection has crashed inside the profiler)
+        step = 64 if eng.cfg["dtype"] == ts.ffi.Q4_K and not eng.cfg.get("n_experts") else 16
+        for i in range(0, ctx - 1, step):
+            eng.prefill(prompt[i:min(i + step, ctx - 1)], i, want_logits=False)
+    else:
+        eng.prefill(prompt[:-1], 0, want_logits=False)   # the last prompt token is the round's confirmed token
     if args.copy_probe:
         us = ts.ffi.copy_time(COPY_BYTES, iters=3)
         log(f"[bench] copy kernel {COPY_BYTES >> 20} MiB: {us:.1f} us")

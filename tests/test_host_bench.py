@@ -119,3 +119,24 @@ def test_step_traffic_gives_bytes_per_launch_and_per_pass(tmp_path, capsys):
     assert embed[-4:] == ["5", "2", str(20 * 2048), str(2 * 1024)]
     assert out[-1].startswith(f"all dispatches from the first k_clear_result on: {(4000 + 40) * 2048 // 2} B read + "
                               f"{(400 + 4) * 1024 // 2} B written per pass (2 passes)")
+
+
+def test_the_recorded_figures_come_out_of_the_committed_profiles():
+    """bench.py reads the dominant launch's trace duration and HBM traffic from the tables under profiles/: every
+    measured workload finds its kernels there, the traffic is the algorithmic bytes plus a little, and a pass moves
+    more than its algorithmic bytes and less than half as much again."""
+    from turbospark_amd import synth
+    b = _bench()
+    assert set(b.PROFILED) == {"llama3_8b_q4_k_k4_ctx4096", "llama3_8b_q4_k_tree16_ctx16384",
+                               "qwen3_30b_a3b_mxfp4_k8_ctx8192", "gptoss_120b_mxfp4_k8_ctx32768"}
+    for w in b.PROFILED:
+        r = b.recorded(w)
+        assert r, w
+        assert 5.0 < r["trace_avg_us"] < 80.0 and r["trace_source"].startswith("recorded: profiles/")
+        wl = b.WORKLOADS[w]
+        cfg = synth.CONFIGS[wl["model"]]
+        if not cfg.get("n_experts"):
+            gate_up = b.algorithmic_bytes(cfg, wl["ctx"], wl["k"] + 1)["per_layer"]["gate_up"]
+            assert 1.0 <= r["traffic"] / gate_up < 1.05, (w, r["traffic"], gate_up)
+        assert r["step_traffic"] > 3e9
+    assert b.recorded("tiny_q8_0_k4_ctx256") == {}
