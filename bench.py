@@ -649,7 +649,7 @@ def loop_bench(args, ts, synth, cfg, weights, eng, wl, rng):
         "prompt_tokens_per_s": round(prompt.size / t_a, 1), "draft_ms_per_block": round(draft_ms, 3),
         "plain_decode_tokens_per_s": round(plain_n / plain_s, 1), "vs_plain_decode": round(new / dt / (plain_n / plain_s), 2),
         "config": {"workload": args.workload, "layers": cfg["n_layers"], "block": k, "temperature": T,
-                   "drafts": "step by step" if (args.step_drafts or T > 0) else "block, chained on the device",
+                   "drafts": "step by step" if args.step_drafts else "block, chained on the device" + (" (drawn there)" if T > 0 else ""),
                    "weak_layers": args.weak_layers, "embed_scale": args.embed_scale, "prompt_tokens": int(prompt.size)}}))
 
 

@@ -403,7 +403,10 @@ int32_t tsv_mtp_prefill_chunk(tsv_ctx* head, const int32_t* tokens, int64_t n, i
  * with the row-only step of the last proposal (speculative.rs:612-625), so the head stands at base + block. */
 int32_t tsv_mtp_draft_block(tsv_ctx* head, int32_t anchor, int64_t base, int32_t block, int32_t* proposals);
 /* Fills `out` with this head's callbacks (prime, step with device logits, rewind, position, draft_block,
- * prefill_chunk) for tsv_run_speculative on the target the head is attached to. */
+ * prefill_chunk) for tsv_run_speculative on the target the head is attached to.  With these callbacks in place the
+ * loop chains SAMPLED rounds on the device too: every step's row stays in the loop's device buffer (the proposal
+ * distributions of the rejection test) and its proposal is drawn there, at the draw positions the step-by-step
+ * walk would use -- same tokens, same counters, one host wait per block. */
 int32_t tsv_mtp_drafter(tsv_ctx* head, tsv_drafter* out);
 
 typedef struct {

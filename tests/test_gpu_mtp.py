@@ -136,7 +136,9 @@ class _HeadDrafter:
     (0.0, {}, 4, 0, {}),                                     # block drafts, chunked prefill
     (0.0, {}, 8, 2, {}),                                     # adaptive depth
     (0.0, {}, 5, 0, dict(block_drafts=False)),               # the same head step by step
-    (0.8, dict(top_p=0.95), 4, 0, {}),                       # sampled rounds go step by step on device rows
+    (0.8, dict(top_p=0.95), 4, 0, {}),                       # sampled rounds: the library's own head chains them on the device
+    (0.9, dict(repetition_penalty=1.3, presence_penalty=0.5, top_k=64), 6, 2, {}),   # ... with penalties over the growing history
+    (0.8, dict(min_p=0.02), 4, 0, dict(block_drafts=False)), # the same head step by step on device rows
     (0.0, dict(repetition_penalty=1.3), 4, 0, {}),           # the arg-max ignores penalties
 ])
 def test_the_loop_with_the_head_reports_what_the_reference_loop_reports(temperature, kw, block, floor, flags):

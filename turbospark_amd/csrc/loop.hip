@@ -319,6 +319,13 @@ extern "C" int32_t tsv_run_speculative(tsv_ctx* c, const tsv_drafter* dr, const 
                 if (error_is_empty()) set_error("run_speculative: draft_block failed");
                 return TSV_ERR_INVALID;
             }
+        } else if (tsv_ctx* own = sampled ? tsv_mtp_own_head(dr) : nullptr) {
+            // the library's own head chains a sampled round on the device as well: the rows stay in `rows`, the draws
+            // are the ones the steps below would make (positions draw_step .. draw_step + block - 1, then the row-only step)
+            if ((rc = tsv_mtp_draft_block_sampled(own, next, base, round_block, &g->shaping, draw_step, hist.data(), (int64_t)hist.size(),
+                                                  generated, rows, feed + 1)))
+                return rc;
+            draw_step += (uint64_t)round_block + 1;
         } else
         for (int d = 0; d <= round_block; d++) {
             if (d == round_block) {

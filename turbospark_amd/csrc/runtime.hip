@@ -180,6 +180,7 @@ struct tsv_ctx {
         bool own_valid = false;  // x row 0 is this head's own residual of the step at position - 1 (a chained step)
         const int32_t* feed_dev = nullptr;  // the pass in flight takes row 0's token from device memory
         int32_t *chain = nullptr, *chain_host = nullptr;  // the tokens of a block draft and the error word
+        AcceptParams *draw_dev = nullptr, *draw_host = nullptr;  // [16] the draw parameters of a sampled block's steps
     } mtp;
     int64_t x_base = -1;  // rows [0, x_rows) of x are the finished residual rows of positions x_base ..
     int x_rows = 0;
@@ -1378,9 +1379,11 @@ static int open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc
         tsv_ctx::Mtp& h = c->mtp;
         if ((rc = dev_alloc(c, &h.e_rows, (size_t)16 * c->hidden * 4, true)) ||
             (rc = dev_alloc(c, &h.cat, (size_t)16 * 2 * c->hidden * 4, true)) ||
-            (rc = dev_alloc(c, &h.xf_cat, xfrag_bytes(2 * c->hidden), true)) || (rc = dev_alloc(c, &h.chain, 32 * 4, true)))
+            (rc = dev_alloc(c, &h.xf_cat, xfrag_bytes(2 * c->hidden), true)) || (rc = dev_alloc(c, &h.chain, 32 * 4, true)) ||
+            (rc = dev_alloc(c, &h.draw_dev, TSV_MAX_ROWS * sizeof(AcceptParams), true)))
             return fail(rc);
-        if (hipHostMalloc((void**)&h.chain_host, 32 * 4) != hipSuccess) {
+        if (hipHostMalloc((void**)&h.chain_host, 32 * 4) != hipSuccess ||
+            hipHostMalloc((void**)&h.draw_host, TSV_MAX_ROWS * sizeof(AcceptParams)) != hipSuccess) {
             set_error("mtp_open: pinned host allocation failed");
             return fail(TSV_ERR_DEVICE);
         }
@@ -1419,6 +1422,7 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->res_host) (void)hipHostFree(c->res_host);
     if (c->tok_host) (void)hipHostFree(c->tok_host);
     if (c->mtp.chain_host) (void)hipHostFree(c->mtp.chain_host);
+    if (c->mtp.draw_host) (void)hipHostFree(c->mtp.draw_host);
     if (c->mtp.on && c->mtp.target && c->mtp.target->mtp_head == c) c->mtp.target->mtp_head = nullptr;
     for (hipGraphExec_t g : c->pass_graph)
         if (g) (void)hipGraphExecDestroy(g);
@@ -1805,6 +1809,65 @@ extern "C" int32_t tsv_mtp_draft_block(tsv_ctx* c, int32_t anchor, int64_t base,
     return TSV_OK;
 }
 
+namespace {  // (defined with the acceptance entry points below)
+void fill_truncation(AcceptParams* ap, const tsv_shaping& sh);
+int setup_penalties(tsv_ctx* c, const tsv_shaping& sh, const int32_t* history, int64_t n, uint64_t generated, AcceptParams* ap);
+const char* accept_error_text(int bits);
+}  // namespace
+
+// The sampled counterpart, for the library's own loop (no reference counterpart: its draft_block hands back tokens
+// only, so its sampled rounds go step by step, speculative.rs:612-660): every step's logits row stays in `rows`
+// (device, block x vocab fp16: the proposal distributions the rejection test needs), the proposal is DRAWN on
+// the device from the row's shaped distribution at draw position draw_step + d (the same kernels and parameters as
+// tsv_draft_chain for that row) and fed to the next step where it lies.  One host wait per block.
+int tsv_mtp_draft_block_sampled(tsv_ctx* c, int32_t anchor, int64_t base, int32_t block, const tsv_shaping* sh, uint64_t draw_step,
+                                const int32_t* history, int64_t n_history, uint64_t generated, uint16_t* rows, int32_t* proposals) {
+    TSV_NEED(c && c->mtp.on && sh && rows && proposals, "mtp_draft_block: not a drafter head, or a null argument");
+    if (block < 1 || block > TSV_MAX_ROWS - 1 || base < 1) {
+        set_error("mtp_draft_block: 1..15 proposals after a position the target has produced");
+        return TSV_ERR_INVALID;
+    }
+    int rc = check_shaping(*sh, true);
+    if (rc) return rc;
+    tsv_ctx::Mtp& h = c->mtp;
+    AcceptParams ap;
+    std::memset(&ap, 0, sizeof ap);
+    ap.m = 0;
+    ap.k = 1;
+    ap.vocab = c->vocab;
+    ap.sampled = sh->temperature != 0.0;
+    ap.temperature = sh->temperature;
+    ap.seed = sh->seed;
+    fill_truncation(&ap, *sh);
+    if ((rc = setup_penalties(c, *sh, history, n_history, generated, &ap))) return rc;  // the same history for every step of a round
+    const int32_t none = 0;
+    for (int d = 0; d <= block; d++) {
+        const float* src = nullptr;
+        if ((rc = mtp_source(c, base - 1 + d, &src))) return rc;
+        h.feed_dev = d ? h.chain + d : nullptr;
+        rc = mtp_pass(c, d ? &none : &anchor, 1, base - 1 + d, src, d < block);
+        h.feed_dev = nullptr;
+        if (rc) return rc;
+        if (d == block) break;
+        uint16_t* row = rows + (size_t)d * c->vocab;
+        TSV_HIP(hipMemcpyAsync(row, c->logits, (size_t)c->vocab * 2, hipMemcpyDeviceToDevice, c->stream));
+        h.draw_host[d] = ap;
+        h.draw_host[d].draw_step = draw_step + (uint64_t)d;
+        TSV_HIP(hipMemcpyAsync(h.draw_dev + d, h.draw_host + d, sizeof(AcceptParams), hipMemcpyHostToDevice, c->stream));
+        if ((rc = launch_draft_chain(c->stream, row, h.draw_dev + d, h.draw_host[d], c->sc, h.chain + d + 1))) return rc;
+    }
+    h.own_valid = false;
+    TSV_HIP(hipMemcpyAsync(h.chain_host, h.chain + 1, (size_t)block * 4, hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipMemcpyAsync(c->res_host, c->sc.result, sizeof(AcceptResult), hipMemcpyDeviceToHost, c->stream));
+    TSV_HIP(hipStreamSynchronize(c->stream));
+    if (c->res_host->error) {  // (each step's draw clears the flag first: this is the last step's)
+        set_error(std::string("mtp_draft_block: ") + accept_error_text(c->res_host->error));
+        return (c->res_host->error & 1) ? TSV_ERR_INVALID : TSV_ERR_UNSUPPORTED;
+    }
+    for (int i = 0; i < block; i++) proposals[i] = h.chain_host[i];
+    return TSV_OK;
+}
+
 namespace {
 int32_t mtp_cb_prime(void* u, int32_t next, int64_t position) { return tsv_mtp_step((tsv_ctx*)u, next, position, nullptr, 0); }
 int32_t mtp_cb_step(void* u, int32_t tok, int64_t position, uint16_t* logits) { return tsv_mtp_step((tsv_ctx*)u, tok, position, logits, 1); }
@@ -1817,6 +1880,12 @@ int32_t mtp_cb_chunk(void* u, const int32_t* tokens, int64_t n, int64_t start, u
     return tsv_mtp_prefill_chunk((tsv_ctx*)u, tokens, n, start, logits, next_token);
 }
 }  // namespace
+
+// Whether a drafter is this library's own head with its block callback in place (the loop then chains sampled rounds too).
+tsv_ctx* tsv_mtp_own_head(const tsv_drafter* d) {
+    return d && d->draft_block == mtp_cb_block && d->step == mtp_cb_step && d->user && ((tsv_ctx*)d->user)->mtp.on ? (tsv_ctx*)d->user
+                                                                                                                     : nullptr;
+}
 
 extern "C" int32_t tsv_mtp_drafter(tsv_ctx* c, tsv_drafter* out) {
     TSV_NEED(c && c->mtp.on && out, "mtp_drafter: not a drafter head, or no output");

@@ -489,6 +489,12 @@ int launch_draft_chain(hipStream_t s, const uint16_t* draft, const AcceptParams*
 int launch_argmax_rows(hipStream_t s, const uint16_t* logits, int rows, int vocab, const AcceptScratch& sc, int32_t* out,
                        bool clear_error);
 int noalloc_prepare_device();
+}  // namespace tsv
+// the library's own drafter head behind a tsv_drafter (NULL: someone else's), and its sampled block draft (runtime.hip)
+tsv_ctx* tsv_mtp_own_head(const tsv_drafter* d);
+int tsv_mtp_draft_block_sampled(tsv_ctx* head, int32_t anchor, int64_t base, int32_t block, const tsv_shaping* sh, uint64_t draw_step,
+                                const int32_t* history, int64_t n_history, uint64_t generated, uint16_t* rows, int32_t* proposals);
+namespace tsv {
 int launch_pen_counts(hipStream_t s, const int32_t* history_dev, long n, long suffix_start, int vocab, uint32_t* cnt);
 
 // ---- host utilities ----------------------------------------------------------------------
