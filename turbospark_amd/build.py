@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, os.environ.get("TSV_LIB_NAME", "libtsverify.so"))
-SOURCES = ["gemm.hip", "moe.hip", "moe_fp4.hip", "misc.hip", "attn.hip", "kvquant.hip", "accept.hip", "host_utils.hip", "runtime.hip", "loop.hip", "gguf.hip"]
+SOURCES = ["gemm.hip", "moe.hip", "moe_fp4.hip", "misc.hip", "attn.hip", "kvquant.hip", "accept.hip", "host_utils.hip", "runtime.hip", "mtp.hip", "testing.hip", "loop.hip", "gguf.hip"]
 # host_utils.hip is host-only code; clang 22 -O3 does not terminate on it, -O2 does.
 OPT = {"host_utils.hip": "-O2", "gguf.hip": "-O2"}
 # MFMA results straight into VGPRs (no v_accvgpr_read copies before the scaling FMAs)

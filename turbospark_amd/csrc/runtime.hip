@@ -6,38 +6,11 @@
 // batched-verify contract of crates/runtime/src/families/qwen/batched.rs:92-456.  Residual
 // stream and all intermediates are fp32; fp16 appears where the engine's storage dtype is
 // fixed (KV cache, logits) and as the MFMA operand type of the matmuls.
-#include <cmath>
-#include <cstring>
-#include <new>
-#include <vector>
-
-#include "tsv_internal.h"
-#include "kv_prefix.h"
+#include "ctx.h"
 
 using namespace tsv;
 
-namespace {
-
-struct LayerW {
-    // the fused q/k/v projection; when the value projection has a format of its own (Q4_K_M files
-    // keep attn_v in Q6_K) `qkv` holds q and k only and `v_only` the rest, written to the same
-    // partial buffer at its column offset
-    TiledW qkv, v_only, wo, gate_up, down;
-    int n_experts = 0, top_k = 0;     // routed experts: gate_up / down hold every expert's tiles
-    TiledW router;
-    float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
-    // gpt-oss additions, all optional: fused q/k/v bias, output bias, sinks, router bias, expert biases
-    float *bqkv = nullptr, *bo = nullptr, *sinks = nullptr, *router_bias = nullptr;
-    float *be_gate = nullptr, *be_up = nullptr, *be_down = nullptr;
-    int window = 0;
-    int cap = 0;        // positions the layer's cache holds: the context, or a ring of window + slack
-    bool rope_fused = false;  // the q/k/v projection rotates and stores its own rows
-    uint16_t *kc = nullptr, *vc = nullptr;
-    // a quantized layer (TurboQuant): kc / vc are then the small fp16 staging cache all such layers
-    // share (kv_slots positions instead of cap), and tq the layer's own stores
-    int kv_slots = 0;
-    TqKv tq{};
-};
+namespace tsv {
 
 int dtype_fmt(int dtype) {
     return dtype == TSV_Q4_K    ? FMT_Q4K
@@ -47,157 +20,6 @@ int dtype_fmt(int dtype) {
            : dtype == TSV_Q6_K  ? FMT_Q6K
            : dtype == TSV_Q5_K  ? FMT_Q5K
                                 : -1;
-}
-
-}  // namespace
-
-struct tsv_ctx {
-    int n_layers = 0, hidden = 0, nq = 0, nkv = 0, hd = 0, ffn = 0, vocab = 0, max_context = 0, ctx_alloc = 0;
-    float eps = 0, attn_scale = 0, rope_mscale = 1.0f, act_alpha = 0, act_limit = 0;
-    hipStream_t stream = nullptr;
-    bool rope_fused_ok = true;     // TSV_ROPE_FUSED=0 keeps the projection and the rotation apart
-    bool rope_fused_force = false;  // TSV_ROPE_FUSED=1 fuses them whatever a tile weighs
-    std::vector<LayerW> layers;
-    TiledW head;
-    uint8_t* embed_raw = nullptr;
-    int embed_dtype = 0;
-    float* final_norm = nullptr;
-    float* freqs = nullptr;
-    float2* rope_cs = nullptr;  // [16][hd / 2] rotation table of the step's rows (fused q/k/v projection)
-    // scratch
-    float* x = nullptr;
-    uint4 *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
-    float* partial = nullptr;
-    size_t partial_floats = 0;
-    // routed experts: routing tables, per-expert activation fragments, per-slot outputs
-    int max_experts = 0;
-    float* route_w = nullptr;
-    int32_t* route_sel = nullptr;
-    int32_t* route_forced = nullptr;  // test hook (tsv_force_route): [n_layers][16][8], negative = route freely
-    uint8_t* frag_e = nullptr;
-    size_t frag_e_stride = 0;
-    float* moe_out = nullptr;
-    // scaled-MFMA expert matmuls (moe_fp4.hip): activation terms (0 = the fp16 path), the pass's rows
-    // and the groups' gate/up outputs as block-scaled fp8
-    int moe_fp4_terms = 0;
-    X8 x8_h{}, x8_e{};
-    size_t x8_e_q_stride = 0, x8_e_s_stride = 0;
-    // prompt passes of 64 rows (four blocks of sixteen): every block's rows, fragments, partial sums,
-    // q rows, parameters and rotation table, block after block; allocated at the first such pass
-    struct Wide {
-        bool ok = false, ready = false;
-        float* x = nullptr;
-        uint8_t *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
-        size_t xfb = 0;
-        float* partial = nullptr;
-        uint16_t* q16 = nullptr;
-        VerifyParams* vp = nullptr;
-        float2* rope_cs = nullptr;
-        float *part_o = nullptr, *part_ml = nullptr;  // attention partials of every block
-        size_t part_o_stride = 0, part_ml_stride = 0;
-    } wide;
-    uint16_t* q16 = nullptr;
-    float *part_o = nullptr, *part_ml = nullptr;
-    int nch = 0;
-    uint16_t* logits = nullptr;       // [16][vocab] fp16, device
-    uint16_t* draft_stage = nullptr;  // [16][vocab] fp16, device
-    VerifyParams *vp_dev = nullptr, *vp_host = nullptr;
-    // Pinned staging slots of the per-pass parameters (four 16-row blocks each), used round robin: a slot is
-    // rewritten only once the copy that last read it has completed (its event), so consecutive passes queue
-    // without the host waiting for the stream.
-    struct ParamRing {
-        static constexpr int SLOTS = 8, PER_SLOT = 4;
-        VerifyParams* host = nullptr;
-        hipEvent_t ev[SLOTS] = {};
-        bool used[SLOTS] = {};
-        int next = 0;
-    } ring;
-    AcceptParams *ap_dev = nullptr, *ap_host = nullptr;
-    uint16_t** kv_ptrs = nullptr;  // device: [2 * layer] = K buffer, [2 * layer + 1] = V buffer (tree compaction)
-    int32_t* hist_dev = nullptr;  // the token history of a penalised round (grows on demand)
-    size_t hist_cap = 0;
-    uint32_t* pen_cnt = nullptr;  // [vocab] seen flag + generated-suffix count per token
-    AcceptResult* res_host = nullptr;
-    int32_t *tok_dev = nullptr, *tok_host = nullptr;
-    AcceptScratch sc{};
-    std::vector<void*> allocs;
-    // TurboQuant KV rows (crates/model-io/src/kv_quant.rs): widths (0 = every layer fp16), the tables of the two
-    // sides and the fp16 staging rows of the pass in flight (crates/runtime/src/kv_write.rs:36-60)
-    int kv_k_bits = 0, kv_v_bits = 0;
-    TqSide tq_k{}, tq_v{};
-    uint16_t *tq_kc = nullptr, *tq_vc = nullptr;
-    TqKv* tq_stores = nullptr;  // device: every layer's stores (tree compaction)
-    int64_t position = 0;
-    int64_t high_water = 0;     // one past the last position any pass has written since the last reset
-    int64_t rewind_budget = INT64_MAX;  // KvCacheManager::max_safe_rewind: min over ring layers of capacity - window
-    int32_t* kv_caps = nullptr;  // device: positions each layer's cache holds (tree compaction)
-    tsv_prefix prefix;          // the ids behind rows [0, prefix length): kv_prefix.rs
-    // Parked sessions (crates/runtime/src/session_pool.rs): each one a full set of per-layer KV buffers of its own
-    // with its cursor and its record; the live session is the fields above and in `layers`.  A swap exchanges
-    // pointers, never rows.
-    struct Session {
-        std::vector<uint16_t*> kc, vc;  // per layer (a quantized layer: unused, its rows are in `tq`)
-        std::vector<TqKv> tq;
-        uint16_t** kv_ptrs = nullptr;   // device copies of the pointer tables tree compaction reads
-        TqKv* tq_stores = nullptr;
-        int64_t position = 0, high_water = 0;
-        tsv_prefix prefix;
-        uint64_t last_used = 0;         // the pool's tick at parking (session_pool.rs:110-114)
-    };
-    std::vector<Session> parked;
-    uint64_t session_clock = 0;
-    bool session_slot_evicted = false;  // the last reset overwrote a parked conversation (real_forward_traits.rs:20-31)
-    bool session_swapped = false;       // the last try_reuse_prefix swapped a parked conversation in
-    bool prefix_reuse = false;  // RealForwardRunner::set_prefix_reuse: off unless the host opts in
-    bool headless = false;      // the pass in flight is a prefill pass nobody reads the logits of
-    int last_m = 0;
-    int64_t last_base = -1;
-    bool last_shape_known = false;  // vp_host holds the ancestor sets of the rows tsv_accept is about to judge
-    // The launch sequence of a pass depends on the row count only (positions, tokens and the
-    // tree shape are read from device memory), so it can be captured once per row count into a
-    // HIP graph and replayed (environment TSV_GRAPH=1).  Off by default: the pass is bound by
-    // the GPU-side cost of ~290 dependent kernels, not by host launch time, and replay measured
-    // the same step time as plain stream launches.
-    bool use_graph = false;
-    hipGraphExec_t pass_graph[TSV_MAX_ROWS + 1] = {};
-    // per-kernel-class timing (tsv_set_profile): one event pair per launch
-    bool profile = false;
-    int repeat[TSV_PROFILE_CLASSES] = {1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1};  // tsv_set_repeat
-    std::vector<hipEvent_t> ev;
-    std::vector<int> ev_class;
-    size_t ev_used = 0;
-    // A drafter head (tsv_mtp_open; docs/MTP.md:53-60): a one-layer handle on the target's stream whose rows
-    // enter the layer as fc over [norm_e(embedding of the row's NEXT token) ; norm_h(target_final_norm(h))], h
-    // the residual row of the row's position.  Embedding table and output head are the target's buffers.
-    struct Mtp {
-        bool on = false;
-        tsv_ctx* target = nullptr;
-        TiledW fc;
-        float *norm_e = nullptr, *norm_h = nullptr;
-        float *e_rows = nullptr, *cat = nullptr;  // [16][hidden] looked-up embeddings, [16][2 hidden] fc's input
-        uint4* xf_cat = nullptr;                  // the same as matmul fragments
-        const float* h_src = nullptr;             // the pass in flight: its residual rows, hidden floats apart
-        bool own_valid = false;  // x row 0 is this head's own residual of the step at position - 1 (a chained step)
-        const int32_t* feed_dev = nullptr;  // the pass in flight takes row 0's token from device memory
-        int32_t *chain = nullptr, *chain_host = nullptr;  // the tokens of a block draft and the error word
-        AcceptParams *draw_dev = nullptr, *draw_host = nullptr;  // [16] the draw parameters of a sampled block's steps
-    } mtp;
-    int64_t x_base = -1;  // rows [0, x_rows) of x are the finished residual rows of positions x_base ..
-    int x_rows = 0;
-    tsv_ctx* mtp_head = nullptr;  // target side: the attached head; prompt passes then finish their residual rows
-    bool owns_stream = true;
-};
-
-namespace {
-
-template <class T>
-int dev_alloc(tsv_ctx* c, T** p, size_t bytes, bool zero = false) {
-    void* q = nullptr;
-    TSV_HIP(hipMalloc(&q, bytes ? bytes : 16));
-    c->allocs.push_back(q);
-    if (zero) TSV_HIP(hipMemsetAsync(q, 0, bytes, c->stream));
-    *p = (T*)q;
-    return TSV_OK;
 }
 
 float to_f32(const tsv_tensor& t, int64_t i) {
@@ -230,11 +52,6 @@ int upload_vector(tsv_ctx* c, const tsv_tensor& t, int64_t n, float** out, const
     TSV_HIP(hipMemcpy(*out, h.data(), (size_t)n * 4, hipMemcpyHostToDevice));
     return TSV_OK;
 }
-
-struct Stager {
-    uint8_t* dev = nullptr;
-    size_t cap = 0;
-};
 
 int stage_raw(tsv_ctx* c, Stager& st, const tsv_tensor& t) {
     const int64_t rb = row_bytes(t.dtype, t.cols);
@@ -274,8 +91,7 @@ int check_matrix(const tsv_tensor& t, int64_t rows, int64_t cols, const char* wh
 // pair_parts > 0 (128-wide heads feeding the rotating epilogue): inside every head of the first
 // `pair_parts` parts the rows are reordered so that a 64-row tile holds dims 32t..32t+31 in its low
 // lanes and their rotation partners, dims 64+32t.., in its high lanes.
-int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_parts, bool interleave, TiledW* out,
-               int pair_parts = 0) {
+int make_tiled(tsv_ctx* c, Stager& st, const tsv_tensor* const* parts, int n_parts, bool interleave, TiledW* out, int pair_parts) {
     const int fmt = dtype_fmt(parts[0]->dtype);
     int64_t total_rows = 0;
     for (int i = 0; i < n_parts; i++) {
@@ -376,9 +192,6 @@ int check_shaping(const tsv_shaping& s, bool sampled_supported_only) {
 bool has_penalties(const tsv_shaping& s) {
     return s.temperature != 0.0 && (s.repetition_penalty != 1.0 || s.presence_penalty != 0.0 || s.frequency_penalty != 0.0);
 }
-
-enum { PC_EMBED = 0, PC_NORM, PC_QKV, PC_ROPE, PC_ATTN, PC_WO, PC_GATEUP, PC_DOWN, PC_HEAD, PC_ACCEPT, PC_EVENTPAIR, PC_COUNT };
-static_assert(PC_COUNT == TSV_PROFILE_CLASSES, "profile classes");
 
 struct ProfScope {
     tsv_ctx* c;
@@ -969,11 +782,11 @@ int finish_verify(tsv_ctx* c, int m, uint16_t* logits_out) {
     return TSV_OK;
 }
 
-}  // namespace
+}  // namespace tsv
 
 // `share` / `md`: a drafter head opened on a target handle -- its stream, embedding table and output head are
 // the target's, and md names fc and the norms of fc's two halves.
-static int open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* md, tsv_ctx** out) {
+int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* md, tsv_ctx** out) {
     if (!d || !out || !d->layers) {
         set_error("open: null argument");
         return TSV_ERR_INVALID;
@@ -1431,64 +1244,6 @@ extern "C" void tsv_close(tsv_ctx* c) {
     delete c;
 }
 
-// The measurement hooks (per-class event pairs, repeated launches, the timing loops) answer only in a process
-// whose environment carries TSV_MEASUREMENT_HOOKS=1: a serving process cannot be put into a measuring mode by
-// a stray call.
-static int measurement_hooks_on(const char* who) {
-    const char* e = getenv("TSV_MEASUREMENT_HOOKS");
-    if (e && e[0] == '1') return TSV_OK;
-    set_error(std::string(who) + ": measurement hooks are off (set TSV_MEASUREMENT_HOOKS=1 in the process environment)");
-    return TSV_ERR_UNSUPPORTED;
-}
-
-extern "C" int32_t tsv_set_profile(tsv_ctx* c, int32_t on) {
-    TSV_NEED(c, "set_profile: null handle");
-    if (on)
-        if (int rc = measurement_hooks_on("set_profile")) return rc;
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    c->profile = on != 0;
-    c->ev_used = 0;
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_set_repeat(tsv_ctx* c, int32_t cls, int32_t times) {
-    TSV_NEED(c, "set_repeat: null handle");
-    if (times != 1)
-        if (int rc = measurement_hooks_on("set_repeat")) return rc;
-    if (cls != PC_QKV && cls != PC_ROPE && cls != PC_ATTN && cls != PC_WO && cls != PC_GATEUP && cls != PC_DOWN &&
-        cls != PC_HEAD) {
-        set_error("set_repeat: only the matmul, rope and attention classes can be repeated");
-        return TSV_ERR_INVALID;
-    }
-    if (times < 1 || times > 8) {
-        set_error("set_repeat: times must be 1..8");
-        return TSV_ERR_INVALID;
-    }
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    c->repeat[cls] = times;
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_get_profile(tsv_ctx* c, float* ms, int32_t* counts, int32_t n_classes) {
-    TSV_NEED(c && ms && counts && n_classes >= 0, "get_profile: null handle or output");
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    for (int i = 0; i < n_classes; i++) {
-        ms[i] = 0.f;
-        counts[i] = 0;
-    }
-    for (size_t i = 0; i + 1 < c->ev_used; i += 2) {
-        float t = 0.f;
-        TSV_HIP(hipEventElapsedTime(&t, c->ev[i], c->ev[i + 1]));
-        const int cls = c->ev_class[i];
-        if (cls < n_classes) {
-            ms[cls] += t;
-            counts[cls] += 1;
-        }
-    }
-    c->ev_used = 0;
-    return TSV_OK;
-}
-
 extern "C" void* tsv_stream(tsv_ctx* c) { return c ? (void*)c->stream : nullptr; }
 
 // session_pool.rs:116-121 best_scoring_index: the index of the highest score (the last one among equals, as
@@ -1611,12 +1366,9 @@ extern "C" int32_t tsv_produce(tsv_ctx* c, int32_t token, int64_t position, uint
     return rc;
 }
 
-static int mtp_pass(tsv_ctx* c, const int32_t* next_tokens, int m, int64_t position, const float* h_rows, bool want_logits);
-
 // `head` (nullable): the drafter head primed after each pass over every row whose next token is known
 // (mtp_prime_rows_batched, families/qwen/mtp.rs:146-400); next_token: the token after ids[n - 1], or -1.
-static int prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits, tsv_ctx* head = nullptr,
-                          int32_t next_token = -1) {
+int tsv::prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0, uint16_t* logits, tsv_ctx* head, int32_t next_token) {
     const int wide_rows = 16 * WIDE_B;
     for (int64_t i = 0; i < n;) {
         // 64 rows at a time while that many remain and nobody wants their logits
@@ -1675,230 +1427,6 @@ extern "C" int32_t tsv_prefill(tsv_ctx* c, const int32_t* ids, int64_t n, int64_
     if (rc == TSV_OK) c->prefix.record(ids, n, pos0);
     else c->prefix.taint();
     return rc;
-}
-
-// ---- the drafter head (docs/MTP.md:53-60, crates/runtime/src/families/qwen/mtp.rs) ------------------------
-// One pass of the head over m rows at position .. position + m - 1: row r pairs next_tokens[r] with h_rows' row r.
-static int mtp_pass(tsv_ctx* c, const int32_t* next_tokens, int m, int64_t position, const float* h_rows, bool want_logits) {
-    if (position != c->position) {  // mtp.rs:484-491
-        set_error("mtp: step at position " + std::to_string((long long)position) + " but the head's cache covers [0, " +
-                  std::to_string((long long)c->position) + "): prime the head over the prompt and rewind it after a rejected draft");
-        return TSV_ERR_INVALID;
-    }
-    c->mtp.h_src = h_rows;
-    c->headless = !want_logits;
-    const int rc = enqueue_verify(c, next_tokens, nullptr, m, position);
-    c->headless = false;
-    c->mtp.h_src = nullptr;
-    // after a full step row 0 of x is the head's own finished residual: what a chained step reads (mtp.rs:85-91)
-    c->mtp.own_valid = rc == TSV_OK && want_logits && m == 1;
-    return rc;
-}
-
-// Where the state of `position` is: the head's own row after a step of its own, else the target's last pass.
-static int mtp_source(tsv_ctx* c, int64_t position, const float** src) {
-    const tsv_ctx* t = c->mtp.target;
-    if (c->mtp.own_valid) {
-        *src = c->x;
-        return TSV_OK;
-    }
-    if (position >= t->x_base && position < t->x_base + t->x_rows) {
-        *src = t->x + (size_t)(position - t->x_base) * t->hidden;
-        return TSV_OK;
-    }
-    set_error("mtp: the target's last pass holds no row for position " + std::to_string((long long)position) +
-              " and the head has no step of its own to chain from");
-    return TSV_ERR_INVALID;
-}
-
-extern "C" int32_t tsv_mtp_open(tsv_ctx* target, const tsv_mtp_desc* d, tsv_ctx** out) {
-    TSV_NEED(target && d && out, "mtp_open: null argument");
-    if (target->mtp.on || target->mtp_head) {
-        set_error("mtp_open: the target is itself a head, or already has one");
-        return TSV_ERR_INVALID;
-    }
-    const tsv_model_desc& m = d->model;
-    if (m.n_layers != 1 || m.hidden != target->hidden || m.vocab != target->vocab) {
-        set_error("mtp_open: the head is ONE decoder layer of the target's width over the target's vocabulary");
-        return TSV_ERR_INVALID;
-    }
-    if (m.kv_k_bits || m.kv_v_bits || m.session_slots > 1 || (m.layers && m.layers[0].ring)) {
-        set_error("mtp_open: the head keeps one plain fp16 cache (no quantized rows, ring or session slots)");
-        return TSV_ERR_UNSUPPORTED;
-    }
-    TSV_HIP(hipStreamSynchronize(target->stream));
-    const int rc = open_impl(&m, target, d, out);
-    if (rc) return rc;
-    target->mtp_head = *out;
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_mtp_step(tsv_ctx* c, int32_t next_token, int64_t position, uint16_t* logits, int32_t on_device) {
-    TSV_NEED(c && c->mtp.on, "mtp_step: not a drafter head");
-    const float* src = nullptr;
-    int rc = mtp_source(c, position, &src);
-    if (rc) return rc;
-    if ((rc = mtp_pass(c, &next_token, 1, position, src, logits != nullptr))) return rc;
-    if (!logits) return TSV_OK;
-    if (on_device) {  // stays in stream order: whoever reads the row does so on the target's stream
-        TSV_HIP(hipMemcpyAsync(logits, c->logits, (size_t)c->vocab * 2, hipMemcpyDeviceToDevice, c->stream));
-        return TSV_OK;
-    }
-    return finish_verify(c, 1, logits);
-}
-
-extern "C" int32_t tsv_mtp_rewind(tsv_ctx* c, int64_t position) {
-    TSV_NEED(c && c->mtp.on, "mtp_rewind: not a drafter head");
-    if (position < 0 || position > c->position) {  // mtp.rs:422-436
-        set_error("mtp_rewind: the head cannot be moved forward, or before position 0");
-        return TSV_ERR_INVALID;
-    }
-    c->position = position;
-    c->mtp.own_valid = false;
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_mtp_prefill_chunk(tsv_ctx* c, const int32_t* tokens, int64_t n, int64_t start_position,
-                                         uint16_t* logits, int32_t next_token) {
-    TSV_NEED(c && c->mtp.on && tokens, "mtp_prefill_chunk: not a drafter head, or no tokens");
-    if (n < 1) {
-        set_error("mtp_prefill_chunk: empty token list");
-        return TSV_ERR_INVALID;
-    }
-    if (c->position != start_position) {
-        set_error("mtp_prefill_chunk: the head's cache must end where the chunk starts");
-        return TSV_ERR_INVALID;
-    }
-    tsv_ctx* t = c->mtp.target;
-    // recorded once the chunk has run to completion, tainted when it has not (real_forward_traits.rs:395-402)
-    const int rc = prefill_passes(t, tokens, n, start_position, logits, c, next_token >= 0 && next_token < t->vocab ? next_token : -1);
-    if (rc == TSV_OK) t->prefix.record(tokens, n, start_position);
-    else t->prefix.taint();
-    return rc;
-}
-
-extern "C" int32_t tsv_mtp_draft_block(tsv_ctx* c, int32_t anchor, int64_t base, int32_t block, int32_t* proposals) {
-    TSV_NEED(c && c->mtp.on && proposals, "mtp_draft_block: not a drafter head, or no output");
-    if (block < 1 || block > TSV_MAX_ROWS - 1 || base < 1) {
-        set_error("mtp_draft_block: 1..15 proposals after a position the target has produced");
-        return TSV_ERR_INVALID;
-    }
-    tsv_ctx::Mtp& h = c->mtp;
-    int rc;
-    const int32_t none = 0;
-    for (int d = 0; d <= block; d++) {
-        // step d pairs the state of base - 1 + d with the token at base + d: the anchor, then each pick of the
-        // step before, read where the arg-max left it; the last step is the row-only one (speculative.rs:612-625)
-        const float* src = nullptr;
-        if ((rc = mtp_source(c, base - 1 + d, &src))) return rc;
-        h.feed_dev = d ? h.chain + d : nullptr;
-        rc = mtp_pass(c, d ? &none : &anchor, 1, base - 1 + d, src, d < block);
-        h.feed_dev = nullptr;
-        if (rc) return rc;
-        if (d < block && (rc = launch_argmax_rows(c->stream, c->logits, 1, c->vocab, c->sc, h.chain + d + 1, d == 0))) return rc;
-    }
-    h.own_valid = false;
-    TSV_HIP(hipMemcpyAsync(h.chain_host, h.chain + 1, (size_t)block * 4, hipMemcpyDeviceToHost, c->stream));
-    TSV_HIP(hipMemcpyAsync(h.chain_host + 31, c->sc.counters, 4, hipMemcpyDeviceToHost, c->stream));
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    if (h.chain_host[31]) {
-        set_error("mtp_draft_block: score vector must not contain a non-finite entry");
-        return TSV_ERR_INVALID;
-    }
-    for (int i = 0; i < block; i++) proposals[i] = h.chain_host[i];
-    return TSV_OK;
-}
-
-namespace {  // (defined with the acceptance entry points below)
-void fill_truncation(AcceptParams* ap, const tsv_shaping& sh);
-int setup_penalties(tsv_ctx* c, const tsv_shaping& sh, const int32_t* history, int64_t n, uint64_t generated, AcceptParams* ap);
-const char* accept_error_text(int bits);
-}  // namespace
-
-// The sampled counterpart, for the library's own loop (no reference counterpart: its draft_block hands back tokens
-// only, so its sampled rounds go step by step, speculative.rs:612-660): every step's logits row stays in `rows`
-// (device, block x vocab fp16: the proposal distributions the rejection test needs), the proposal is DRAWN on
-// the device from the row's shaped distribution at draw position draw_step + d (the same kernels and parameters as
-// tsv_draft_chain for that row) and fed to the next step where it lies.  One host wait per block.
-int tsv_mtp_draft_block_sampled(tsv_ctx* c, int32_t anchor, int64_t base, int32_t block, const tsv_shaping* sh, uint64_t draw_step,
-                                const int32_t* history, int64_t n_history, uint64_t generated, uint16_t* rows, int32_t* proposals) {
-    TSV_NEED(c && c->mtp.on && sh && rows && proposals, "mtp_draft_block: not a drafter head, or a null argument");
-    if (block < 1 || block > TSV_MAX_ROWS - 1 || base < 1) {
-        set_error("mtp_draft_block: 1..15 proposals after a position the target has produced");
-        return TSV_ERR_INVALID;
-    }
-    int rc = check_shaping(*sh, true);
-    if (rc) return rc;
-    tsv_ctx::Mtp& h = c->mtp;
-    AcceptParams ap;
-    std::memset(&ap, 0, sizeof ap);
-    ap.m = 0;
-    ap.k = 1;
-    ap.vocab = c->vocab;
-    ap.sampled = sh->temperature != 0.0;
-    ap.temperature = sh->temperature;
-    ap.seed = sh->seed;
-    fill_truncation(&ap, *sh);
-    if ((rc = setup_penalties(c, *sh, history, n_history, generated, &ap))) return rc;  // the same history for every step of a round
-    const int32_t none = 0;
-    for (int d = 0; d <= block; d++) {
-        const float* src = nullptr;
-        if ((rc = mtp_source(c, base - 1 + d, &src))) return rc;
-        h.feed_dev = d ? h.chain + d : nullptr;
-        rc = mtp_pass(c, d ? &none : &anchor, 1, base - 1 + d, src, d < block);
-        h.feed_dev = nullptr;
-        if (rc) return rc;
-        if (d == block) break;
-        uint16_t* row = rows + (size_t)d * c->vocab;
-        TSV_HIP(hipMemcpyAsync(row, c->logits, (size_t)c->vocab * 2, hipMemcpyDeviceToDevice, c->stream));
-        h.draw_host[d] = ap;
-        h.draw_host[d].draw_step = draw_step + (uint64_t)d;
-        TSV_HIP(hipMemcpyAsync(h.draw_dev + d, h.draw_host + d, sizeof(AcceptParams), hipMemcpyHostToDevice, c->stream));
-        if ((rc = launch_draft_chain(c->stream, row, h.draw_dev + d, h.draw_host[d], c->sc, h.chain + d + 1))) return rc;
-    }
-    h.own_valid = false;
-    TSV_HIP(hipMemcpyAsync(h.chain_host, h.chain + 1, (size_t)block * 4, hipMemcpyDeviceToHost, c->stream));
-    TSV_HIP(hipMemcpyAsync(c->res_host, c->sc.result, sizeof(AcceptResult), hipMemcpyDeviceToHost, c->stream));
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    if (c->res_host->error) {  // (each step's draw clears the flag first: this is the last step's)
-        set_error(std::string("mtp_draft_block: ") + accept_error_text(c->res_host->error));
-        return (c->res_host->error & 1) ? TSV_ERR_INVALID : TSV_ERR_UNSUPPORTED;
-    }
-    for (int i = 0; i < block; i++) proposals[i] = h.chain_host[i];
-    return TSV_OK;
-}
-
-namespace {
-int32_t mtp_cb_prime(void* u, int32_t next, int64_t position) { return tsv_mtp_step((tsv_ctx*)u, next, position, nullptr, 0); }
-int32_t mtp_cb_step(void* u, int32_t tok, int64_t position, uint16_t* logits) { return tsv_mtp_step((tsv_ctx*)u, tok, position, logits, 1); }
-int32_t mtp_cb_rewind(void* u, int64_t position) { return tsv_mtp_rewind((tsv_ctx*)u, position); }
-int64_t mtp_cb_position(void* u) { return ((tsv_ctx*)u)->position; }
-int32_t mtp_cb_block(void* u, int32_t anchor, int64_t base, int32_t block, int32_t* proposals) {
-    return tsv_mtp_draft_block((tsv_ctx*)u, anchor, base, block, proposals);
-}
-int32_t mtp_cb_chunk(void* u, const int32_t* tokens, int64_t n, int64_t start, uint16_t* logits, int32_t next_token) {
-    return tsv_mtp_prefill_chunk((tsv_ctx*)u, tokens, n, start, logits, next_token);
-}
-}  // namespace
-
-// Whether a drafter is this library's own head with its block callback in place (the loop then chains sampled rounds too).
-tsv_ctx* tsv_mtp_own_head(const tsv_drafter* d) {
-    return d && d->draft_block == mtp_cb_block && d->step == mtp_cb_step && d->user && ((tsv_ctx*)d->user)->mtp.on ? (tsv_ctx*)d->user
-                                                                                                                     : nullptr;
-}
-
-extern "C" int32_t tsv_mtp_drafter(tsv_ctx* c, tsv_drafter* out) {
-    TSV_NEED(c && c->mtp.on && out, "mtp_drafter: not a drafter head, or no output");
-    std::memset(out, 0, sizeof *out);
-    out->user = c;
-    out->prime = mtp_cb_prime;
-    out->step = mtp_cb_step;
-    out->rewind = mtp_cb_rewind;
-    out->device_logits = 1;
-    out->position = mtp_cb_position;
-    out->draft_block = mtp_cb_block;
-    out->prefill_chunk = mtp_cb_chunk;
-    return TSV_OK;
 }
 
 extern "C" int32_t tsv_checkpoint(tsv_ctx* c, tsv_point* out) {
@@ -2023,7 +1551,7 @@ extern "C" int32_t tsv_compact_tree(tsv_ctx* c, int64_t base, const uint32_t* pa
     return rc;
 }
 
-namespace {
+namespace tsv {
 
 void fill_truncation(AcceptParams* ap, const tsv_shaping& sh) {
     ap->top_k = (int32_t)sh.top_k;
@@ -2192,7 +1720,7 @@ int accept_impl(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     return TSV_OK;
 }
 
-}  // namespace
+}  // namespace tsv
 
 extern "C" int32_t tsv_accept(tsv_ctx* c, const tsv_round* r, tsv_round_result* out) {
     if (!c || !r || !out || !r->feed) {
@@ -2250,288 +1778,6 @@ extern "C" int32_t tsv_draft_chain(tsv_ctx* c, const uint16_t* draft_logits, int
     return TSV_OK;
 }
 
-extern "C" int32_t tsv_read_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, uint16_t* k, uint16_t* v) {
-    if (!c || !k || !v || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
-        set_error("read_kv: null argument or range outside the cache");
-        return TSV_ERR_INVALID;
-    }
-    if (c->layers[layer].tq.k_bits) {
-        set_error("read_kv: this layer keeps quantized rows (tsv_read_kv_quantized reads them)");
-        return TSV_ERR_UNSUPPORTED;
-    }
-    const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
-    uint16_t *kd = nullptr, *vd = nullptr;
-    TSV_HIP(hipMalloc((void**)&kd, bytes));
-    if (hipMalloc((void**)&vd, bytes) != hipSuccess) {
-        (void)hipFree(kd);
-        set_error("KV staging buffer: out of device memory");
-        return TSV_ERR_DEVICE;
-    }
-    if (c->layers[layer].cap < c->ctx_alloc && pos0 < c->high_water - c->layers[layer].cap) {
-        (void)hipFree(kd);
-        (void)hipFree(vd);
-        set_error("read_kv: the ring of this layer no longer holds the first rows asked for");
-        return TSV_ERR_INVALID;
-    }
-    int rc = launch_kv_read(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, c->layers[layer].cap,
-                            (int)pos0, (int)n, kd, vd);
-    if (!rc) {
-        hipError_t e1 = hipMemcpyAsync(k, kd, bytes, hipMemcpyDeviceToHost, c->stream);
-        hipError_t e2 = hipMemcpyAsync(v, vd, bytes, hipMemcpyDeviceToHost, c->stream);
-        hipError_t e3 = hipStreamSynchronize(c->stream);
-        if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) {
-            set_error("read_kv: copy failed");
-            rc = TSV_ERR_DEVICE;
-        }
-    }
-    (void)hipFree(kd);
-    (void)hipFree(vd);
-    return rc;
-}
-
-extern "C" int32_t tsv_route_selected(tsv_ctx* c, int32_t* out, int32_t n_layers) {
-    if (!c || !out || n_layers != c->n_layers) {
-        set_error("route_selected: null argument or layer count mismatch");
-        return TSV_ERR_INVALID;
-    }
-    if (!c->route_sel) {
-        set_error("route_selected: the model has no routed layers");
-        return TSV_ERR_INVALID;
-    }
-    TSV_HIP(hipMemcpyAsync(out, c->route_sel, (size_t)c->n_layers * 16 * 8 * 4, hipMemcpyDeviceToHost, c->stream));
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_force_route(tsv_ctx* c, const int32_t* sel, int32_t n_layers) {
-    if (!c || (sel && n_layers != c->n_layers)) {
-        set_error("force_route: null handle or layer count mismatch");
-        return TSV_ERR_INVALID;
-    }
-    if (!c->route_forced) {
-        set_error("force_route: the model has no routed layers");
-        return TSV_ERR_INVALID;
-    }
-    const size_t bytes = (size_t)c->n_layers * 16 * 8 * 4;
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    if (sel) {
-        TSV_HIP(hipMemcpy(c->route_forced, sel, bytes, hipMemcpyHostToDevice));
-    } else {
-        TSV_HIP(hipMemset(c->route_forced, 0xFF, bytes));  // every entry -1: every row routes freely
-    }
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_write_logits(tsv_ctx* c, const uint16_t* logits, int32_t m, int64_t base) {
-    if (!c || !logits || m < 1 || m > TSV_MAX_ROWS || base < 0) {
-        set_error("write_logits: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    TSV_HIP(hipMemcpyAsync(c->logits, logits, (size_t)m * c->vocab * 2, hipMemcpyHostToDevice, c->stream));
-    TSV_HIP(hipStreamSynchronize(c->stream));
-    c->last_m = m;
-    c->last_base = base;
-    c->last_shape_known = false;  // rows from the host: whatever tree the round names is taken at its word
-    return TSV_OK;
-}
-
-extern "C" int32_t tsv_write_kv(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, const uint16_t* k,
-                                const uint16_t* v) {
-    if (!c || !k || !v || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->max_context) {
-        set_error("write_kv: range outside the cache");
-        return TSV_ERR_INVALID;
-    }
-    const size_t bytes = (size_t)n * c->nkv * c->hd * 2;
-    uint16_t *kd = nullptr, *vd = nullptr;
-    TSV_HIP(hipMalloc((void**)&kd, bytes));
-    if (hipMalloc((void**)&vd, bytes) != hipSuccess) {
-        (void)hipFree(kd);
-        set_error("KV staging buffer: out of device memory");
-        return TSV_ERR_DEVICE;
-    }
-    int rc = TSV_OK;
-    if (hipMemcpyAsync(kd, k, bytes, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-        hipMemcpyAsync(vd, v, bytes, hipMemcpyHostToDevice, c->stream) != hipSuccess) {
-        set_error("write_kv: copy failed");
-        rc = TSV_ERR_DEVICE;
-    }
-    if (!rc && c->layers[layer].tq.k_bits) {
-        // a quantized layer: the rows go through the staging slots and the quantizer sixteen at a time, as the
-        // forward's own rows do (crates/runtime/src/kv_write.rs:66-118)
-        const LayerW& L = c->layers[layer];
-        TqArgs ta{};
-        ta.kc = L.kc;
-        ta.vc = L.vc;
-        ta.stage_cap = L.kv_slots;
-        ta.store = L.tq;
-        ta.k = c->tq_k;
-        ta.v = c->tq_v;
-        ta.nkv = c->nkv;
-        ta.hd = c->hd;
-        ta.cap = L.cap;
-        ta.vp = c->vp_dev;
-        const size_t row = (size_t)c->nkv * c->hd;
-        for (int64_t p = 0; !rc && p < n; p += L.kv_slots) {
-            const int cnt = (int)std::min<int64_t>(L.kv_slots, n - p);
-            rc = launch_kv_fill(c->stream, L.kc, L.vc, c->nkv, c->hd, L.kv_slots, (int)(pos0 + p), cnt, kd + p * row, vd + p * row);
-            ta.m_hint = cnt;
-            ta.base_hint = (int)(pos0 + p);
-            if (!rc) rc = launch_tq_prepare(c->stream, ta);
-        }
-    } else if (!rc) {
-        // a ring layer keeps the last `cap` of the rows (earlier ones would only be overwritten, by
-        // rows of the same launch)
-        const int64_t cap = c->layers[layer].cap, skip = n > cap ? n - cap : 0;
-        const size_t off = (size_t)skip * c->nkv * c->hd;
-        rc = launch_kv_fill(c->stream, c->layers[layer].kc, c->layers[layer].vc, c->nkv, c->hd, (int)cap,
-                            (int)(pos0 + skip), (int)(n - skip), kd + off, vd + off);
-    }
-    if (hipStreamSynchronize(c->stream) != hipSuccess && !rc) {
-        set_error("write_kv: device execution failed");
-        rc = TSV_ERR_DEVICE;
-    }
-    (void)hipFree(kd);
-    (void)hipFree(vd);
-    if (!rc && pos0 + n > c->position) c->position = pos0 + n;
-    if (!rc) c->high_water = std::max(c->high_water, pos0 + n);
-    c->prefix.taint();  // rows no token ids describe
-    return rc;
-}
-
-extern "C" int32_t tsv_matmul(const tsv_tensor* w, const float* x, int32_t m, float* y, int32_t splits) {
-    if (!w || !x || !y || m < 1 || m > TSV_MAX_ROWS) {
-        set_error("matmul: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    int rc = check_matrix(*w, w->rows, w->cols, "matmul weight");
-    if (rc) return rc;
-    tsv_ctx tmp;
-    tsv_ctx* c = &tmp;
-    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    Stager st;
-    TiledW tw;
-    const tsv_tensor* parts[1] = {w};
-    VerifyParams vp;
-    std::memset(&vp, 0, sizeof vp);
-    vp.m = m;
-    float *xd = nullptr, *pd = nullptr;
-    uint4* xf = nullptr;
-    VerifyParams* vpd = nullptr;
-    const int k = (int)w->cols, n = (int)w->rows;
-    std::vector<float> part;
-    int sp = 1;
-    rc = make_tiled(c, st, parts, 1, false, &tw);
-    if (!rc) {
-        sp = splits > 0 ? std::min(splits, tw.kchunks) : gemm_default_splits(tw, m);
-        const int kslice = (tw.kchunks + sp - 1) / sp;
-        sp = (tw.kchunks + kslice - 1) / kslice;
-    }
-    if (!rc) rc = dev_alloc(c, &xd, (size_t)m * k * 4);
-    if (!rc) rc = dev_alloc(c, &xf, xfrag_bytes(k), true);
-    if (!rc) rc = dev_alloc(c, &pd, (size_t)sp * 16 * n * 4, true);
-    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
-    if (!rc && hipMemcpyAsync(xd, x, (size_t)m * k * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess) rc = TSV_ERR_DEVICE;
-    if (!rc && hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess) rc = TSV_ERR_DEVICE;
-    if (!rc) rc = launch_f32_to_xfrag(c->stream, xd, k, xf, m);
-    if (!rc) rc = launch_gemm(c->stream, tw, xf, pd, vpd, m, sp, EPI_PARTIAL, n, n);
-    if (!rc) {
-        part.resize((size_t)sp * 16 * n);
-        if (hipMemcpyAsync(part.data(), pd, part.size() * 4, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-            hipStreamSynchronize(c->stream) != hipSuccess) {
-            set_error("matmul: device execution failed");
-            rc = TSV_ERR_DEVICE;
-        }
-    }
-    if (!rc)
-        for (int b = 0; b < m; b++)
-            for (int j = 0; j < n; j++) {
-                float acc = 0.f;
-                for (int s = 0; s < sp; s++) acc += part[((size_t)s * 16 + b) * n + j];
-                y[(size_t)b * n + j] = acc;
-            }
-    if (st.dev) (void)hipFree(st.dev);
-    (void)hipStreamSynchronize(c->stream);
-    for (void* p : c->allocs) (void)hipFree(p);
-    (void)hipStreamDestroy(c->stream);
-    return rc;
-}
-
-extern "C" int32_t tsv_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
-                                 int32_t nkv, int32_t hd, int64_t base, const int32_t* parent, float scale,
-                                 int32_t window, const float* sinks, uint16_t* out) {
-    if (!q || !k || !v || !out || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0 || window < 0 ||
-        (window > 0 && window <= TSV_MAX_ROWS)) {
-        set_error("attention: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    tsv_ctx tmp;
-    tsv_ctx* c = &tmp;
-    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    VerifyParams vp;
-    int rc = fill_params(vp, nullptr, parent, m, base, 0);
-    const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv;
-    const size_t kvb = (size_t)nkv * ctx * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
-    uint16_t *kc = nullptr, *vc = nullptr, *kin = nullptr, *vin = nullptr, *q16 = nullptr;
-    float *po = nullptr, *pml = nullptr, *sinks_dev = nullptr;
-    uint4* xf = nullptr;
-    VerifyParams* vpd = nullptr;
-    const size_t xfb = xfrag_bytes(nq * hd);
-    if (!rc && sinks) {
-        rc = dev_alloc(c, &sinks_dev, (size_t)nq * 4);
-        if (!rc && hipMemcpyAsync(sinks_dev, sinks, (size_t)nq * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess)
-            rc = TSV_ERR_DEVICE;
-    }
-    if (!rc) rc = dev_alloc(c, &kc, kvb, true);
-    if (!rc) rc = dev_alloc(c, &vc, kvb, true);
-    if (!rc) rc = dev_alloc(c, &kin, inb);
-    if (!rc) rc = dev_alloc(c, &vin, inb);
-    if (!rc) rc = dev_alloc(c, &q16, qb);
-    if (!rc) rc = dev_alloc(c, &po, (size_t)nkv * nch * m * G * hd * 4, true);
-    if (!rc) rc = dev_alloc(c, &pml, (size_t)nkv * nch * m * G * 2 * 4, true);
-    if (!rc) rc = dev_alloc(c, &xf, xfb, true);
-    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
-    if (!rc && (hipMemcpyAsync(kin, k, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-                hipMemcpyAsync(vin, v, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-                hipMemcpyAsync(q16, q, qb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-                hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess))
-        rc = TSV_ERR_DEVICE;
-    if (!rc) rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, ctx, 0, seq, kin, vin);
-    if (!rc) {
-        AttnArgs aa{};
-        aa.q16 = q16;
-        aa.kc = kc;
-        aa.vc = vc;
-        aa.part_o = po;
-        aa.part_ml = pml;
-        aa.xfrag = xf;
-        aa.nq = nq;
-        aa.nkv = nkv;
-        aa.hd = hd;
-        aa.max_ctx = ctx;
-        aa.nch = nch;
-        aa.scale = scale > 0.f ? scale : 1.0f / std::sqrt((float)hd);
-        aa.window = window;
-        aa.sinks = sinks_dev;
-        aa.vp = vpd;
-        aa.m_hint = m;
-        aa.base_hint = (int)base;
-        rc = launch_attention(c->stream, aa, m);
-    }
-    std::vector<uint16_t> frag(xfb / 2);
-    if (!rc && (hipMemcpyAsync(frag.data(), xf, xfb, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-                hipStreamSynchronize(c->stream) != hipSuccess)) {
-        set_error("attention: device execution failed");
-        rc = TSV_ERR_DEVICE;
-    }
-    if (!rc)
-        for (int b = 0; b < m; b++)
-            for (int kk = 0; kk < nq * hd; kk++) out[(size_t)b * nq * hd + kk] = frag[(size_t)frag_index(kk, b)];
-    (void)hipStreamSynchronize(c->stream);
-    for (void* p : c->allocs) (void)hipFree(p);
-    (void)hipStreamDestroy(c->stream);
-    return rc;
-}
-
 // crates/model-io/src/kv_quant.rs:146-205 kv_layer_strides, for the layer kinds of this path and as this library
 // lays the rows out: bytes one position costs in layer `layer`, K side and V side
 extern "C" int32_t tsv_kv_row_bytes(const tsv_model_desc* d, int32_t layer, int64_t* k_bytes, int64_t* v_bytes) {
@@ -2570,329 +1816,3 @@ extern "C" int64_t tsv_kv_bytes_for_context(const tsv_model_desc* d, int64_t con
     }
     return total;
 }
-
-extern "C" int32_t tsv_kv_quant_tables(int32_t head_dim, int32_t bits, int32_t value_side, float* signs, float* codebook,
-                                       float* midpoints) {
-    if (head_dim < 32 || head_dim > 512 || (head_dim & (head_dim - 1)) || bits < 1 || bits > 4 || !signs || !codebook ||
-        !midpoints) {
-        set_error("kv_quant_tables: head_dim must be a power of two in 32..512 and bits in 1..4");
-        return TSV_ERR_INVALID;
-    }
-    tq_sign_vector(head_dim, value_side ? 1 : 0, signs);
-    const std::vector<float> cb = tq_codebook(head_dim, bits);
-    for (size_t i = 0; i < cb.size(); i++) codebook[i] = cb[i];
-    for (size_t i = 0; i + 1 < cb.size(); i++) midpoints[i] = 0.5f * (cb[i] + cb[i + 1]);
-    return TSV_OK;
-}
-
-namespace {
-// The stores of positions [pos0, pos0 + n) as the rows the reference keeps, [position][kv head][norm, words]
-// (crates/gpu/tests/kv_quantize_parity.rs:22-38): K rows are stored that way but for the norm; V indices are
-// stored transposed per block of sixteen positions and are packed back LSB first (kv_quant.rs:289-312) here.
-int tq_rows_to_host(hipStream_t stream, const TqKv& t, int nkv, int hd, int cap, int64_t pos0, int64_t n, uint32_t* k_rows,
-                    uint32_t* v_rows) {
-    const int kw = tq_words(hd, t.k_bits), vw = tq_words(hd, t.v_bits), gw = t.v_bits == 2 ? 1 : 2;
-    std::vector<uint32_t> kq((size_t)nkv * cap * kw), vq(tq_vq_bytes(nkv, cap, hd, t.v_bits) / 4);
-    std::vector<float> kn((size_t)nkv * cap), vn((size_t)nkv * cap);
-    TSV_HIP(hipStreamSynchronize(stream));
-    TSV_HIP(hipMemcpy(kq.data(), t.kq, kq.size() * 4, hipMemcpyDeviceToHost));
-    TSV_HIP(hipMemcpy(vq.data(), t.vq, vq.size() * 4, hipMemcpyDeviceToHost));
-    TSV_HIP(hipMemcpy(kn.data(), t.kn, kn.size() * 4, hipMemcpyDeviceToHost));
-    TSV_HIP(hipMemcpy(vn.data(), t.vn, vn.size() * 4, hipMemcpyDeviceToHost));
-    for (int64_t i = 0; i < n; i++) {
-        const int64_t pos = pos0 + i;
-        for (int h = 0; h < nkv; h++) {
-            uint32_t* kr = k_rows + ((size_t)i * nkv + h) * (1 + kw);
-            std::memcpy(kr, &kn[(size_t)h * cap + pos], 4);
-            std::memcpy(kr + 1, &kq[((size_t)h * cap + pos) * kw], (size_t)kw * 4);
-            uint32_t* vr = v_rows + ((size_t)i * nkv + h) * (1 + vw);
-            std::memcpy(vr, &vn[(size_t)h * cap + pos], 4);
-            std::fill(vr + 1, vr + 1 + vw, 0u);
-            for (int d = 0; d < hd; d++) {
-                const uint32_t* g = &vq[(((size_t)h * (cap / 16) + pos / 16) * hd + d) * gw];
-                const uint64_t group = gw == 2 ? ((uint64_t)g[1] << 32) | g[0] : g[0];
-                const uint32_t idx = (uint32_t)(group >> ((pos & 15) * t.v_bits)) & ((1u << t.v_bits) - 1u);
-                const uint32_t bit = (uint32_t)d * t.v_bits, w = bit >> 5, off = bit & 31;
-                vr[1 + w] |= idx << off;
-                if (off + t.v_bits > 32) vr[1 + w + 1] |= idx >> (32 - off);
-            }
-        }
-    }
-    return TSV_OK;
-}
-}  // namespace
-
-extern "C" int32_t tsv_read_kv_quantized(tsv_ctx* c, int32_t layer, int64_t pos0, int64_t n, uint32_t* k_rows,
-                                         uint32_t* v_rows) {
-    if (!c || !k_rows || !v_rows || layer < 0 || layer >= c->n_layers || pos0 < 0 || n < 1 || pos0 + n > c->ctx_alloc) {
-        set_error("read_kv_quantized: null argument or range outside the cache");
-        return TSV_ERR_INVALID;
-    }
-    const LayerW& L = c->layers[layer];
-    if (!L.tq.k_bits) {
-        set_error("read_kv_quantized: this layer keeps fp16 rows");
-        return TSV_ERR_INVALID;
-    }
-    return tq_rows_to_host(c->stream, L.tq, c->nkv, c->hd, L.cap, pos0, n, k_rows, v_rows);
-}
-
-extern "C" int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k, const uint16_t* v, int32_t m, int32_t nq,
-                                           int32_t nkv, int32_t hd, int64_t base, int32_t k_bits, int32_t v_bits,
-                                           float scale, const float* sinks, uint16_t* out, uint32_t* k_rows,
-                                           uint32_t* v_rows) {
-    if (!q || !k || !v || !out || !k_rows || !v_rows || m < 1 || m > TSV_MAX_ROWS || nq % nkv || nq / nkv > 8 || base < 0 ||
-        k_bits < 2 || k_bits > 4 || v_bits < 2 || v_bits > 4 || (hd != 64 && hd != 128)) {
-        set_error("attention_quantized: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    tsv_ctx tmp;
-    tsv_ctx* c = &tmp;
-    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    VerifyParams vp;
-    int rc = fill_params(vp, nullptr, nullptr, m, base, 0);
-    const int seq = (int)base + m, ctx = (seq + 15) / 16 * 16, nch = attn_chunks(nkv), G = nq / nkv, slots = TSV_MAX_ROWS;
-    const size_t stb = (size_t)nkv * slots * hd * 2, inb = (size_t)seq * nkv * hd * 2, qb = (size_t)m * nq * hd * 2;
-    uint16_t *kc = nullptr, *vc = nullptr, *kin = nullptr, *vin = nullptr, *q16 = nullptr;
-    float *po = nullptr, *pml = nullptr, *sinks_dev = nullptr, *tables = nullptr;
-    uint4* xf = nullptr;
-    VerifyParams* vpd = nullptr;
-    const size_t xfb = xfrag_bytes(nq * hd);
-    TqArgs ta{};
-    TqKv st{};
-    st.k_bits = k_bits;
-    st.v_bits = v_bits;
-    if (!rc && sinks) {
-        rc = dev_alloc(c, &sinks_dev, (size_t)nq * 4);
-        if (!rc && hipMemcpyAsync(sinks_dev, sinks, (size_t)nq * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess)
-            rc = TSV_ERR_DEVICE;
-    }
-    if (!rc) rc = dev_alloc(c, &kc, stb, true);
-    if (!rc) rc = dev_alloc(c, &vc, stb, true);
-    if (!rc) rc = dev_alloc(c, &st.kq, tq_kq_bytes(nkv, ctx, hd, k_bits), true);
-    if (!rc) rc = dev_alloc(c, &st.vq, tq_vq_bytes(nkv, ctx, hd, v_bits), true);
-    if (!rc) rc = dev_alloc(c, &st.kn, (size_t)nkv * ctx * 4, true);
-    if (!rc) rc = dev_alloc(c, &st.vn, (size_t)nkv * ctx * 4, true);
-    if (!rc) rc = dev_alloc(c, &kin, inb);
-    if (!rc) rc = dev_alloc(c, &vin, inb);
-    if (!rc) rc = dev_alloc(c, &q16, qb);
-    if (!rc) rc = dev_alloc(c, &po, (size_t)nkv * nch * m * G * hd * 4, true);
-    if (!rc) rc = dev_alloc(c, &pml, (size_t)nkv * nch * m * G * 2 * 4, true);
-    if (!rc) rc = dev_alloc(c, &xf, xfb, true);
-    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
-    if (!rc) rc = dev_alloc(c, &tables, (size_t)2 * TQ_TABLE_FLOATS * 4);
-    if (!rc) rc = tq_upload_side(hd, k_bits, 0, tables, &ta.k);
-    if (!rc) rc = tq_upload_side(hd, v_bits, 1, tables + TQ_TABLE_FLOATS, &ta.v);
-    if (!rc && (hipMemcpyAsync(kin, k, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-                hipMemcpyAsync(vin, v, inb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-                hipMemcpyAsync(q16, q, qb, hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-                hipMemcpyAsync(vpd, &vp, sizeof vp, hipMemcpyHostToDevice, c->stream) != hipSuccess))
-        rc = TSV_ERR_DEVICE;
-    st.k_cb = ta.k.cb;
-    st.v_cb = ta.v.cb;
-    ta.q16 = q16;
-    ta.kc = kc;
-    ta.vc = vc;
-    ta.stage_cap = slots;
-    ta.store = st;
-    ta.nkv = nkv;
-    ta.hd = hd;
-    ta.cap = ctx;
-    ta.vp = vpd;
-    // every row goes through the staging slots and the quantizer, sixteen at a time as passes do; the last
-    // group is the pass itself, whose q rows are rotated with it
-    const size_t row = (size_t)nkv * hd;
-    for (int64_t p = 0; !rc && p < seq;) {
-        const bool last = p >= base;
-        const int n = last ? m : (int)std::min<int64_t>(slots, base - p);
-        rc = launch_kv_fill(c->stream, kc, vc, nkv, hd, slots, (int)p, n, kin + (size_t)p * row, vin + (size_t)p * row);
-        ta.nq = last ? nq : 0;
-        ta.m_hint = n;
-        ta.base_hint = (int)p;
-        if (!rc) rc = launch_tq_prepare(c->stream, ta);
-        p += n;
-    }
-    if (!rc) {
-        AttnArgs aa{};
-        aa.q16 = q16;
-        aa.unrot = ta.v.signs;
-        aa.tq = st;
-        aa.part_o = po;
-        aa.part_ml = pml;
-        aa.xfrag = xf;
-        aa.nq = nq;
-        aa.nkv = nkv;
-        aa.hd = hd;
-        aa.max_ctx = ctx;
-        aa.nch = nch;
-        aa.scale = scale > 0.f ? scale : 1.0f / std::sqrt((float)hd);
-        aa.sinks = sinks_dev;
-        aa.vp = vpd;
-        aa.m_hint = m;
-        aa.base_hint = (int)base;
-        rc = launch_attention(c->stream, aa, m);
-    }
-    std::vector<uint16_t> frag(xfb / 2);
-    if (!rc && (hipMemcpyAsync(frag.data(), xf, xfb, hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-                hipStreamSynchronize(c->stream) != hipSuccess)) {
-        set_error("attention_quantized: device execution failed");
-        rc = TSV_ERR_DEVICE;
-    }
-    if (!rc) rc = tq_rows_to_host(c->stream, st, nkv, hd, ctx, 0, seq, k_rows, v_rows);
-    if (!rc)
-        for (int b = 0; b < m; b++)
-            for (int kk = 0; kk < nq * hd; kk++) out[(size_t)b * nq * hd + kk] = frag[(size_t)frag_index(kk, b)];
-    (void)hipStreamSynchronize(c->stream);
-    for (void* p : c->allocs) (void)hipFree(p);
-    (void)hipStreamDestroy(c->stream);
-    return rc;
-}
-
-namespace {
-__global__ __launch_bounds__(256) void k_copy_probe(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
-}
-}  // namespace
-
-extern "C" int32_t tsv_copy_time(int64_t bytes, int32_t iters, float* avg_us) {
-    if (int hrc = measurement_hooks_on("copy_time")) return hrc;
-    if (bytes < 16 || bytes % 16 || iters < 1 || !avg_us) {
-        set_error("copy_time: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    hipStream_t s;
-    TSV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-    uint4 *a = nullptr, *b = nullptr;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    int rc = TSV_OK;
-    if (hipMalloc((void**)&a, (size_t)bytes) != hipSuccess || hipMalloc((void**)&b, (size_t)bytes) != hipSuccess ||
-        hipMemsetAsync(a, 1, (size_t)bytes, s) != hipSuccess || hipEventCreate(&e0) != hipSuccess ||
-        hipEventCreate(&e1) != hipSuccess) {
-        set_error("copy_time: allocation failed");
-        rc = TSV_ERR_DEVICE;
-    }
-    for (int pass = 0; pass < 2 && !rc; pass++) {
-        if (pass) (void)hipEventRecord(e0, s);
-        for (int i = 0; i < (pass ? iters : 2); i++)
-            hipLaunchKernelGGL(k_copy_probe, dim3(256 * 16), dim3(256), 0, s, a, b, (size_t)bytes / 16);
-        if (pass) (void)hipEventRecord(e1, s);
-    }
-    if (!rc) {
-        if (hipStreamSynchronize(s) != hipSuccess) {
-            set_error("copy_time: device execution failed");
-            rc = TSV_ERR_DEVICE;
-        } else {
-            float ms = 0.f;
-            (void)hipEventElapsedTime(&ms, e0, e1);
-            *avg_us = ms * 1000.f / (float)iters;
-        }
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    if (a) (void)hipFree(a);
-    if (b) (void)hipFree(b);
-    (void)hipStreamDestroy(s);
-    return rc;
-}
-
-// Measurement hook: average duration (HIP events on a private stream) of `iters` back-to-back
-// launches of the verify pass's matmul over a rows x cols weight of the given dtype filled with
-// pseudo-random block bytes, m activation rows, epilogue `epi` (0 split-K partials, 1 silu-mul over
-// interleaved gate/up tiles, 2 fp16 logits).  `rotate` distinct weight copies are cycled so the
-// kernel streams from HBM rather than from cache.
-extern "C" int32_t tsv_matmul_time(int32_t dtype, int64_t rows, int64_t cols, int32_t m, int32_t epi, int32_t splits,
-                                   int32_t iters, int32_t rotate, float* avg_us) {
-    if (int hrc = measurement_hooks_on("matmul_time")) return hrc;
-    const int fmt = dtype_fmt(dtype);
-    if (fmt < 0 || rows % TILE_ROWS || cols % fmt_chunk_elems(fmt) || m < 1 || m > TSV_MAX_ROWS || iters < 1 || rotate < 1) {
-        set_error("matmul_time: bad argument");
-        return TSV_ERR_INVALID;
-    }
-    tsv_ctx tmp;
-    tsv_ctx* c = &tmp;
-    TSV_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    TiledW w;
-    w.fmt = fmt;
-    w.k = (int)cols;
-    w.kchunks = w.k / fmt_chunk_elems(fmt);
-    w.n_rows = (int)rows;
-    w.n_tiles = (int)(rows / TILE_ROWS);
-    w.bytes = (size_t)w.n_tiles * w.kchunks * fmt_tile_bytes(fmt);
-    std::vector<uint8_t*> copies((size_t)rotate);
-    int rc = TSV_OK;
-    {
-        // block bytes: small fp16 scales (0x2xxx) and arbitrary quants
-        std::vector<uint8_t> host(w.bytes);
-        uint64_t sd = 88172645463325252ull;
-        for (size_t i = 0; i < host.size(); i += 8) {
-            sd ^= sd << 13;
-            sd ^= sd >> 7;
-            sd ^= sd << 17;
-            std::memcpy(&host[i], &sd, std::min<size_t>(8, host.size() - i));
-        }
-        const int tb = fmt_tile_bytes(fmt);
-        for (size_t t = 0; t < w.bytes / tb; t++) {
-            uint8_t* sc = &host[t * tb + 8192];
-            if (fmt == FMT_Q4K || fmt == FMT_Q5K)
-                for (int r = 0; r < 64; r++) {
-                    sc[r * 16 + 1] = 0x20;
-                    sc[r * 16 + 3] = 0x20;
-                }
-            else if (fmt == FMT_Q80)
-                for (int i = 0; i < 256; i++) sc[2 * i + 1] = 0x20;
-            else if (fmt == FMT_MX4)
-                for (int i = 0; i < 512; i++) sc[i] = 0x70 + (sc[i] & 7);  // e8m0 scales around 2^-12
-            else if (fmt == FMT_Q6K)
-                for (int r = 0; r < 64; r++) host[t * tb + 13312 + r * 4 + 1] = 0x20;  // f16 d
-            else  // bf16: every value a small finite number
-                for (int i = 0; i < 4096; i++) host[t * tb + 2 * i + 1] = (uint8_t)(0x3C | (host[t * tb + 2 * i + 1] & 0x80));
-        }
-        for (int i = 0; i < rotate && !rc; i++) {
-            rc = dev_alloc(c, &copies[i], w.bytes);
-            if (!rc && hipMemcpy(copies[i], host.data(), w.bytes, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
-        }
-    }
-    VerifyParams vp;
-    std::memset(&vp, 0, sizeof vp);
-    vp.m = m;
-    uint4* xf = nullptr;
-    float* out = nullptr;
-    VerifyParams* vpd = nullptr;
-    int sp = 1;
-    if (!rc) {
-        w.tiles = copies[0];
-        sp = epi == EPI_PARTIAL ? (splits > 0 ? splits : gemm_default_splits(w, m)) : 1;
-        const int kslice = (w.kchunks + sp - 1) / sp;
-        sp = (w.kchunks + kslice - 1) / kslice;
-    }
-    if (!rc) rc = dev_alloc(c, &xf, xfrag_bytes((int)cols), true);
-    if (!rc) rc = dev_alloc(c, &out, (size_t)sp * 16 * rows * 4 + xfrag_bytes((int)rows), true);
-    if (!rc) rc = dev_alloc(c, &vpd, sizeof vp);
-    if (!rc && hipMemcpy(vpd, &vp, sizeof vp, hipMemcpyHostToDevice) != hipSuccess) rc = TSV_ERR_DEVICE;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (!rc && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = TSV_ERR_DEVICE;
-    for (int pass = 0; pass < 2 && !rc; pass++) {  // pass 0 warms up
-        if (pass == 1) (void)hipEventRecord(e0, c->stream);
-        for (int i = 0; i < (pass ? iters : std::min(iters, 3)) && !rc; i++) {
-            w.tiles = copies[(size_t)(i % rotate)];
-            rc = launch_gemm(c->stream, w, xf, (void*)out, vpd, m, sp, epi, (int)rows, (int)rows);
-        }
-        if (pass == 1) (void)hipEventRecord(e1, c->stream);
-    }
-    if (!rc) {
-        if (hipStreamSynchronize(c->stream) != hipSuccess) {
-            set_error("matmul_time: device execution failed");
-            rc = TSV_ERR_DEVICE;
-        } else {
-            float ms = 0.f;
-            (void)hipEventElapsedTime(&ms, e0, e1);
-            *avg_us = ms * 1000.f / (float)iters;
-        }
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    (void)hipStreamSynchronize(c->stream);
-    for (void* p : c->allocs) (void)hipFree(p);
-    (void)hipStreamDestroy(c->stream);
-    return rc;
-}
-
