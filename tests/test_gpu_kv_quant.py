@@ -237,6 +237,44 @@ def test_what_a_quantized_handle_refuses():
         ts.HipVerifier(oss, wo, kv_bits=(4, 4))
 
 
+def test_rings_on_a_quantized_handle_equal_the_linear_layout_by_bits():
+    """gpt-oss arrangement with both options at once: the sliding layers as rings (kv_cache.rs:360-378), the full layers'
+    rows quantized (kv_quant.rs:102-107).  Prompt passes far past the rings' capacity, verify rounds with rollbacks
+    inside the budget, a tree round with compaction across a ring's seam: every logit equal to the same handle with
+    the sliding layers laid out linearly, and the rewind budget is the rings'."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    cfg = dict(synth.CONFIGS["gptoss_small"], max_context=400, n_layers=4)
+    w = synth.make_weights(cfg, seed=21)
+    ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
+    lin, ring = ts.HipVerifier(cfg, w, kv_bits=(4, 4)), ts.HipVerifier(cfg, ringed, kv_bits=(4, 4))
+    assert lin.max_safe_rewind() == 2 ** 63 - 1 and ring.max_safe_rewind() == 64 - 24
+    V = cfg["vocab"]
+    rng = np.random.default_rng(8)
+    prompt = rng.integers(0, V, 150).astype(np.int32)
+    assert np.array_equal(lin.prefill(prompt, 0), ring.prefill(prompt, 0))
+    base = 150
+    for rnd in range(20):
+        m = int(rng.integers(1, 17))
+        feed = rng.integers(0, V, m).astype(np.int32)
+        pa, pb = lin.checkpoint(), ring.checkpoint()
+        assert np.array_equal(lin.verify(feed, base), ring.verify(feed, base)), rnd
+        keep = int(rng.integers(1, m + 1))
+        lin.rollback_retaining(pa, keep)
+        ring.rollback_retaining(pb, keep)
+        base += keep
+    parent = [-1, 0, 0, 1, 1, 2, 3, 5]
+    feed = rng.integers(0, V, 8).astype(np.int32)
+    for eng in (lin, ring):
+        eng.verify_tree(feed, parent, base, want_logits=False)
+        eng.compact_tree(base, [0, 2, 5, 7])
+        eng.rollback_retaining(ts.ffi.Point(base), 4)
+    nxt = rng.integers(0, V, 3).astype(np.int32)
+    assert np.array_equal(lin.verify(nxt, base + 4), ring.verify(nxt, base + 4))
+    with pytest.raises(ts.ffi.TsvError, match="exceeds the ring slack"):
+        ring.rollback(ts.ffi.Point(base - 60))
+
+
 def test_a_gguf_target_takes_the_width_from_the_environment(tmp_path):
     """The option is a session's, not the file's (crates/model-io/src/kv_quant.rs:48-72): TSV_KV_BITS carries it to
     tsv_open_gguf, and the handle then equals the directly installed one with the same widths, by bits."""
