@@ -165,11 +165,12 @@ struct tsv_ctx {
         tsv_ctx* target = nullptr;
         TiledW fc;
         float *norm_e = nullptr, *norm_h = nullptr;
-        float *e_rows = nullptr, *cat = nullptr;  // [16][hidden] looked-up embeddings, [16][2 hidden] fc's input
-        uint4* xf_cat = nullptr;                  // the same as matmul fragments
+        uint4* xf_cat = nullptr;                  // fc's input rows as matmul fragments (K = 2 hidden)
         const float* h_src = nullptr;             // the pass in flight: its residual rows, hidden floats apart
         bool own_valid = false;  // x row 0 is this head's own residual of the step at position - 1 (a chained step)
         const int32_t* feed_dev = nullptr;  // the pass in flight takes row 0's token from device memory
+        bool params_staged = false;         // ... and finds its parameter block on the device already (vp_dev)
+        VerifyParams *vp_block = nullptr, *vp_block_host = nullptr;  // [16] the parameter blocks of a block draft's steps
         int32_t *chain = nullptr, *chain_host = nullptr;  // the tokens of a block draft and the error word
         AcceptParams *draw_dev = nullptr, *draw_host = nullptr;  // [16] the draw parameters of a sampled block's steps
     } mtp;

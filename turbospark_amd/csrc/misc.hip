@@ -11,6 +11,66 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// Element e of table row `tok`: the arithmetic of the reference's dequantize_* for the row's storage type.
+__device__ __forceinline__ float embed_elem(const uint8_t* __restrict__ raw, int dtype, int hidden, long tok, int e) {
+    float v;
+    if (dtype == TSV_Q4_K) {
+        const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 144;
+        const float d = f16_bits_to_f32(*(const uint16_t*)blk);
+        const float dmin = f16_bits_to_f32(*(const uint16_t*)(blk + 2));
+        const uint8_t* packed = blk + 4;
+        const int w = e & 255, g = w >> 6, hi = (w >> 5) & 1, l = w & 31, j = 2 * g + hi;
+        int sc, mn;
+        if (j < 4) {
+            sc = packed[j] & 63;
+            mn = packed[j + 4] & 63;
+        } else {
+            sc = (packed[j + 4] & 0xF) | ((packed[j - 4] >> 6) << 4);
+            mn = (packed[j + 4] >> 4) | ((packed[j] >> 6) << 4);
+        }
+        const uint8_t byte = blk[16 + 32 * g + l];
+        const int q = hi ? (byte >> 4) : (byte & 0xF);
+        const float dl = d * (float)sc, ml = dmin * (float)mn;
+        v = __fsub_rn(__fmul_rn(dl, (float)q), ml);
+    } else if (dtype == TSV_Q8_0) {
+        const uint8_t* blk = raw + (tok * (hidden / 32) + (e >> 5)) * 34;
+        const float d = f16_bits_to_f32(*(const uint16_t*)blk);
+        v = (float)(int8_t)blk[2 + (e & 31)] * d;
+    } else if (dtype == TSV_Q5_K) {  // q5_k.rs:47-96
+        const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 176;
+        const float d = f16_bits_to_f32(*(const uint16_t*)blk);
+        const float dmin = f16_bits_to_f32(*(const uint16_t*)(blk + 2));
+        const uint8_t* packed = blk + 4;
+        const int w = e & 255, g = w >> 6, hi = (w >> 5) & 1, l = w & 31, j = 2 * g + hi;
+        int sc, mn;
+        if (j < 4) {
+            sc = packed[j] & 63;
+            mn = packed[j + 4] & 63;
+        } else {
+            sc = (packed[j + 4] & 0xF) | ((packed[j - 4] >> 6) << 4);
+            mn = (packed[j + 4] >> 4) | ((packed[j] >> 6) << 4);
+        }
+        const uint8_t byte = blk[48 + 32 * g + l];
+        const int q = (hi ? (byte >> 4) : (byte & 0xF)) + (((blk[16 + l] >> j) & 1) << 4);
+        const float dl = d * (float)sc, ml = dmin * (float)mn;
+        v = __fsub_rn(__fmul_rn(dl, (float)q), ml);
+    } else if (dtype == TSV_Q6_K) {  // q6_k.rs:44-88
+        const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 210;
+        const int w = e & 255, h = w >> 7, k = (w >> 5) & 3, l = w & 31;
+        const int lo = (blk[64 * h + l + 32 * (k & 1)] >> (4 * (k >> 1))) & 0xF;
+        const int hi = (blk[128 + 32 * h + l] >> (2 * k)) & 3;
+        const float d = f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+        v = d * (float)(int8_t)blk[192 + (w >> 4)] * (float)((lo | (hi << 4)) - 32);
+    } else if (dtype == TSV_F16) {
+        v = f16_bits_to_f32(((const uint16_t*)raw)[tok * hidden + e]);
+    } else if (dtype == TSV_BF16) {
+        v = __uint_as_float((uint32_t)((const uint16_t*)raw)[tok * hidden + e] << 16);
+    } else {
+        v = ((const float*)raw)[tok * hidden + e];
+    }
+    return v;
+}
+
 // ---------------------------------------------------------------- embedding lookup
 // One dequantized table row per fed token (crates/runtime/src/real_forward_dispatch.rs:154),
 // arithmetic of dequantize_q4_k / dequantize_q8_0.
@@ -31,64 +91,8 @@ __global__ void k_embed(const uint8_t* __restrict__ raw, int dtype, int hidden, 
         return;
     }
     const long tok = vp->feed[m];
-    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < hidden; e += blockDim.x * nblk) {
-        float v;
-        if (dtype == TSV_Q4_K) {
-            const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 144;
-            const float d = f16_bits_to_f32(*(const uint16_t*)blk);
-            const float dmin = f16_bits_to_f32(*(const uint16_t*)(blk + 2));
-            const uint8_t* packed = blk + 4;
-            const int w = e & 255, g = w >> 6, hi = (w >> 5) & 1, l = w & 31, j = 2 * g + hi;
-            int sc, mn;
-            if (j < 4) {
-                sc = packed[j] & 63;
-                mn = packed[j + 4] & 63;
-            } else {
-                sc = (packed[j + 4] & 0xF) | ((packed[j - 4] >> 6) << 4);
-                mn = (packed[j + 4] >> 4) | ((packed[j] >> 6) << 4);
-            }
-            const uint8_t byte = blk[16 + 32 * g + l];
-            const int q = hi ? (byte >> 4) : (byte & 0xF);
-            const float dl = d * (float)sc, ml = dmin * (float)mn;
-            v = __fsub_rn(__fmul_rn(dl, (float)q), ml);
-        } else if (dtype == TSV_Q8_0) {
-            const uint8_t* blk = raw + (tok * (hidden / 32) + (e >> 5)) * 34;
-            const float d = f16_bits_to_f32(*(const uint16_t*)blk);
-            v = (float)(int8_t)blk[2 + (e & 31)] * d;
-        } else if (dtype == TSV_Q5_K) {  // q5_k.rs:47-96
-            const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 176;
-            const float d = f16_bits_to_f32(*(const uint16_t*)blk);
-            const float dmin = f16_bits_to_f32(*(const uint16_t*)(blk + 2));
-            const uint8_t* packed = blk + 4;
-            const int w = e & 255, g = w >> 6, hi = (w >> 5) & 1, l = w & 31, j = 2 * g + hi;
-            int sc, mn;
-            if (j < 4) {
-                sc = packed[j] & 63;
-                mn = packed[j + 4] & 63;
-            } else {
-                sc = (packed[j + 4] & 0xF) | ((packed[j - 4] >> 6) << 4);
-                mn = (packed[j + 4] >> 4) | ((packed[j] >> 6) << 4);
-            }
-            const uint8_t byte = blk[48 + 32 * g + l];
-            const int q = (hi ? (byte >> 4) : (byte & 0xF)) + (((blk[16 + l] >> j) & 1) << 4);
-            const float dl = d * (float)sc, ml = dmin * (float)mn;
-            v = __fsub_rn(__fmul_rn(dl, (float)q), ml);
-        } else if (dtype == TSV_Q6_K) {  // q6_k.rs:44-88
-            const uint8_t* blk = raw + (tok * (hidden / 256) + (e >> 8)) * 210;
-            const int w = e & 255, h = w >> 7, k = (w >> 5) & 3, l = w & 31;
-            const int lo = (blk[64 * h + l + 32 * (k & 1)] >> (4 * (k >> 1))) & 0xF;
-            const int hi = (blk[128 + 32 * h + l] >> (2 * k)) & 3;
-            const float d = f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
-            v = d * (float)(int8_t)blk[192 + (w >> 4)] * (float)((lo | (hi << 4)) - 32);
-        } else if (dtype == TSV_F16) {
-            v = f16_bits_to_f32(((const uint16_t*)raw)[tok * hidden + e]);
-        } else if (dtype == TSV_BF16) {
-            v = __uint_as_float((uint32_t)((const uint16_t*)raw)[tok * hidden + e] << 16);
-        } else {
-            v = ((const float*)raw)[tok * hidden + e];
-        }
-        x[(long)m * hidden + e] = v;
-    }
+    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < hidden; e += blockDim.x * nblk)
+        x[(long)m * hidden + e] = embed_elem(raw, dtype, hidden, tok, e);
 }
 
 int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float* x,
@@ -250,58 +254,90 @@ int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, in
 }
 
 // ---------------------------------------------------------------- the drafter head's input
-// fc's input rows (docs/MTP.md:53-60, families/qwen/mtp.rs:512-590): [ norm_e(e) ; norm_h(norm_t(h)) ] with e the
-// looked-up embedding of the row's next token and h the residual row of the row's position; every norm is
-// x * w / sqrt(mean x^2 + eps) (crates/compute/src/rms_norm.rs:5-14).  One workgroup per row.  The row of the
-// head's own residual stream `x_zero` is cleared last -- it may be the very row h was read from (a chained
-// step), and fc's partial sums are added onto it by the layer's first residual kernel.
-__global__ __launch_bounds__(1024) void k_mtp_cat(const float* __restrict__ e_rows, const float* h_rows,
-                                                  const float* __restrict__ w_e, const float* __restrict__ w_t,
-                                                  const float* __restrict__ w_h, float eps, int hidden,
-                                                  float* __restrict__ cat, float* x_zero) {
+// fc's input rows (docs/MTP.md:53-60, families/qwen/mtp.rs:512-590) as matmul fragments, one workgroup per row:
+//   [ norm_e(e) ; norm_h(norm_t(h)) ]   e = the embedding row of the row's NEXT token (from the parameter block, or
+//   for row 0 from device memory: a proposal the step before picked on the GPU), h = the residual row of the row's
+//   position; every norm is x * w / sqrt(mean x^2 + eps) (crates/compute/src/rms_norm.rs:5-14).
+// Also the row's rotation table (as the embedding kernel leaves it), and the row of the head's own residual
+// stream `x_zero` cleared LAST -- it may be the very row h was read from (a chained step), and fc's partial sums
+// are added onto it by the layer's first residual kernel.  Embedding lookup, three norms, the fragment conversion
+// and the token hand-over were four launches and a copy before.
+__global__ __launch_bounds__(1024) void k_mtp_input(const uint8_t* __restrict__ raw, int dtype, const VerifyParams* __restrict__ vp,
+                                                    const int32_t* __restrict__ token_dev, int vocab, const float* h_rows,
+                                                    const float* __restrict__ w_e, const float* __restrict__ w_t,
+                                                    const float* __restrict__ w_h, float eps, int hidden,
+                                                    _Float16* __restrict__ xfrag, float* x_zero,
+                                                    const float* __restrict__ freqs, float mscale, int half,
+                                                    float2* __restrict__ cs) {
     __shared__ float red[16];
     const int m = blockIdx.x;
-    const float* e = e_rows + (long)m * hidden;
+    if (m >= vp->m) return;
+    long tok = vp->feed[m];
+    if (token_dev && m == 0) {
+        const int t = *token_dev;
+        tok = t < 0 ? 0 : t >= vocab ? vocab - 1 : t;
+    }
+    const float pos = (float)vp->pos[m];
+    for (int i = threadIdx.x; i < half; i += 1024) {
+        float sn, c;
+        sincosf(pos * freqs[i], &sn, &c);
+        cs[m * half + i] = float2{c * mscale, sn * mscale};
+    }
     const float* h = h_rows + (long)m * hidden;
+    // at most eight elements per thread (hidden <= 8192): kept in registers across the reductions
+    float ev[8], hv[8];
     float se = 0.f, sh = 0.f;
-    for (int i = threadIdx.x; i < hidden; i += 1024) {
-        se += e[i] * e[i];
-        sh += h[i] * h[i];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int i = threadIdx.x + 1024 * j;
+        ev[j] = i < hidden ? embed_elem(raw, dtype, hidden, tok, i) : 0.f;
+        hv[j] = i < hidden ? h[i] : 0.f;
+        se += ev[j] * ev[j];
+        sh += hv[j] * hv[j];
     }
     se = block_sum(se, red);
     sh = block_sum(sh, red);
     const float inv_e = 1.0f / sqrtf(se / (float)hidden + eps), inv_h = 1.0f / sqrtf(sh / (float)hidden + eps);
     float st = 0.f;
-    for (int i = threadIdx.x; i < hidden; i += 1024) {
-        const float t = h[i] * w_t[i] * inv_h;
-        st += t * t;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int i = threadIdx.x + 1024 * j;
+        hv[j] = i < hidden ? hv[j] * w_t[i] * inv_h : 0.f;
+        st += hv[j] * hv[j];
     }
     st = block_sum(st, red);
     const float inv_t = 1.0f / sqrtf(st / (float)hidden + eps);
-    float* out = cat + (long)m * 2 * hidden;
-    for (int i = threadIdx.x; i < hidden; i += 1024) {
-        const float t = h[i] * w_t[i] * inv_h;
-        out[i] = e[i] * w_e[i] * inv_e;
-        out[hidden + i] = t * w_h[i] * inv_t;
+    float* sums = (float*)((char*)xfrag + xfrag_sum_offset(2 * hidden));
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int i = threadIdx.x + 1024 * j;  // hidden is a multiple of 32: whole sub-blocks stay or leave together
+        if (i >= hidden) continue;
+        const _Float16 he = pinned_half((_Float16)(ev[j] * w_e[i] * inv_e));
+        const _Float16 hh = pinned_half((_Float16)(hv[j] * w_h[i] * inv_t));
+        xfrag[frag_index(i, m)] = he;
+        xfrag[frag_index(hidden + i, m)] = hh;
+        float s0 = (float)he, s1 = (float)hh;
+        for (int o = 1; o < 32; o <<= 1) {
+            s0 += __shfl_xor(s0, o);
+            s1 += __shfl_xor(s1, o);
+        }
+        if ((i & 31) == 0) {
+            sums[xsum_index(i >> 5, m)] = s0;
+            sums[xsum_index((hidden + i) >> 5, m)] = s1;
+        }
         x_zero[(long)m * hidden + i] = 0.f;
     }
 }
 
-int launch_mtp_cat(hipStream_t s, const float* e_rows, const float* h_rows, const float* w_e, const float* w_t,
-                   const float* w_h, float eps, int hidden, float* cat, float* x_zero, int m) {
-    hipLaunchKernelGGL(k_mtp_cat, dim3(m), dim3(1024), 0, s, e_rows, h_rows, w_e, w_t, w_h, eps, hidden, cat, x_zero);
-    TSV_HIP(hipGetLastError());
-    return TSV_OK;
-}
-
-// Row 0 of a pass takes its token from device memory (a proposal the step before picked on the GPU).
-__global__ void k_feed_token(VerifyParams* vp, const int32_t* token, int vocab) {
-    const int t = *token;
-    vp->feed[0] = t < 0 ? 0 : t >= vocab ? vocab - 1 : t;
-}
-
-int launch_feed_token(hipStream_t s, VerifyParams* vp, const int32_t* token, int vocab) {
-    hipLaunchKernelGGL(k_feed_token, dim3(1), dim3(1), 0, s, vp, token, vocab);
+int launch_mtp_input(hipStream_t s, const uint8_t* raw, int dtype, const VerifyParams* vp, const int32_t* token_dev, int vocab,
+                     const float* h_rows, const float* w_e, const float* w_t, const float* w_h, float eps, int hidden, uint4* xfrag,
+                     float* x_zero, const float* freqs, float mscale, int half, float2* cs, int m) {
+    if (hidden > 8192 || hidden % 32) {
+        set_error("drafter head: hidden must be a multiple of 32, at most 8192");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(k_mtp_input, dim3(m), dim3(1024), 0, s, raw, dtype, vp, token_dev, vocab, h_rows, w_e, w_t, w_h, eps, hidden,
+                       (_Float16*)xfrag, x_zero, freqs, mscale, half, cs);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -106,6 +106,17 @@ extern "C" int32_t tsv_mtp_prefill_chunk(tsv_ctx* c, const int32_t* tokens, int6
     return rc;
 }
 
+// The parameter blocks of a block draft's steps (one row each at base - 1 + d, d = 0 .. block) to the device in ONE copy;
+// step d then runs with vp_dev naming its block and stages nothing.
+static int stage_block_params(tsv_ctx* c, int64_t base, int block) {
+    tsv_ctx::Mtp& h = c->mtp;
+    const int32_t none = 0;
+    for (int d = 0; d <= block; d++)
+        if (int rc = fill_params(h.vp_block_host[d], &none, nullptr, 1, base - 1 + d, c->vocab)) return rc;
+    TSV_HIP(hipMemcpyAsync(h.vp_block, h.vp_block_host, (size_t)(block + 1) * sizeof(VerifyParams), hipMemcpyHostToDevice, c->stream));
+    return TSV_OK;
+}
+
 extern "C" int32_t tsv_mtp_draft_block(tsv_ctx* c, int32_t anchor, int64_t base, int32_t block, int32_t* proposals) {
     TSV_NEED(c && c->mtp.on && proposals, "mtp_draft_block: not a drafter head, or no output");
     if (block < 1 || block > TSV_MAX_ROWS - 1 || base < 1) {
@@ -115,17 +126,31 @@ extern "C" int32_t tsv_mtp_draft_block(tsv_ctx* c, int32_t anchor, int64_t base,
     tsv_ctx::Mtp& h = c->mtp;
     int rc;
     const int32_t none = 0;
+    if (anchor < 0 || anchor >= c->vocab) {
+        set_error("mtp_draft_block: token id outside the vocabulary");
+        return TSV_ERR_INVALID;
+    }
+    // every step takes its token from chain[d] on the device: the anchor is put there with the parameter blocks
+    h.chain_host[30] = anchor;
+    TSV_HIP(hipMemcpyAsync(h.chain, h.chain_host + 30, 4, hipMemcpyHostToDevice, c->stream));
+    if ((rc = stage_block_params(c, base, block))) return rc;
+    VerifyParams* const vp_own = c->vp_dev;
     for (int d = 0; d <= block; d++) {
         // step d pairs the state of base - 1 + d with the token at base + d: the anchor, then each pick of the
         // step before, read where the arg-max left it; the last step is the row-only one (speculative.rs:612-625)
         const float* src = nullptr;
-        if ((rc = mtp_source(c, base - 1 + d, &src))) return rc;
-        h.feed_dev = d ? h.chain + d : nullptr;
-        rc = mtp_pass(c, d ? &none : &anchor, 1, base - 1 + d, src, d < block);
+        if ((rc = mtp_source(c, base - 1 + d, &src))) break;
+        h.feed_dev = h.chain + d;
+        h.params_staged = true;
+        c->vp_dev = h.vp_block + d;
+        rc = mtp_pass(c, &none, 1, base - 1 + d, src, d < block);
+        c->vp_dev = vp_own;
+        h.params_staged = false;
         h.feed_dev = nullptr;
         if (rc) return rc;
         if (d < block && (rc = launch_argmax_rows(c->stream, c->logits, 1, c->vocab, c->sc, h.chain + d + 1, d == 0))) return rc;
     }
+    if (rc) return rc;
     h.own_valid = false;
     TSV_HIP(hipMemcpyAsync(h.chain_host, h.chain + 1, (size_t)block * 4, hipMemcpyDeviceToHost, c->stream));
     TSV_HIP(hipMemcpyAsync(h.chain_host + 31, c->sc.counters, 4, hipMemcpyDeviceToHost, c->stream));
@@ -164,11 +189,23 @@ int tsv_mtp_draft_block_sampled(tsv_ctx* c, int32_t anchor, int64_t base, int32_
     fill_truncation(&ap, *sh);
     if ((rc = setup_penalties(c, *sh, history, n_history, generated, &ap))) return rc;  // the same history for every step of a round
     const int32_t none = 0;
+    if (anchor < 0 || anchor >= c->vocab) {
+        set_error("mtp_draft_block: token id outside the vocabulary");
+        return TSV_ERR_INVALID;
+    }
+    h.chain_host[30] = anchor;
+    TSV_HIP(hipMemcpyAsync(h.chain, h.chain_host + 30, 4, hipMemcpyHostToDevice, c->stream));
+    if ((rc = stage_block_params(c, base, block))) return rc;
+    VerifyParams* const vp_own = c->vp_dev;
     for (int d = 0; d <= block; d++) {
         const float* src = nullptr;
         if ((rc = mtp_source(c, base - 1 + d, &src))) return rc;
-        h.feed_dev = d ? h.chain + d : nullptr;
-        rc = mtp_pass(c, d ? &none : &anchor, 1, base - 1 + d, src, d < block);
+        h.feed_dev = h.chain + d;
+        h.params_staged = true;
+        c->vp_dev = h.vp_block + d;
+        rc = mtp_pass(c, &none, 1, base - 1 + d, src, d < block);
+        c->vp_dev = vp_own;
+        h.params_staged = false;
         h.feed_dev = nullptr;
         if (rc) return rc;
         if (d == block) break;

@@ -285,9 +285,9 @@ int enqueue_verify(tsv_ctx* c, const int32_t* feed, const int32_t* parent, int m
     int prc = fill_params(vp, feed, parent, m, base, c->vocab);
     if (prc) return prc;
     *c->vp_host = vp;  // the host's own copy of the pass in flight
-    int prc2 = stage_params(c, &vp, 1, c->vp_dev);
-    if (prc2) return prc2;
-    if (c->mtp.feed_dev && (prc2 = launch_feed_token(c->stream, c->vp_dev, c->mtp.feed_dev, c->vocab))) return prc2;
+    // (a block draft has put the parameter blocks of all its steps on the device in one copy: vp_dev names this step's)
+    if (!c->mtp.params_staged)
+        if (int prc2 = stage_params(c, &vp, 1, c->vp_dev)) return prc2;
     int rc = run_pass(c, m);
     if (rc) return rc;
     c->position = base + m;
@@ -325,11 +325,9 @@ int launch_pass(tsv_ctx* c, int m) {
         // position; fc's split-K partial sums are added onto the cleared rows by the layer's first residual kernel
         tsv_ctx::Mtp& h = c->mtp;
         PROF(PC_EMBED);
-        if ((rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, h.e_rows, c->vp_dev, m, c->freqs, c->rope_mscale,
-                               c->hd / 2, c->rope_cs)) ||
-            (rc = launch_mtp_cat(s, h.e_rows, h.h_src, h.norm_e, h.target->final_norm, h.norm_h, c->eps, c->hidden, h.cat,
-                                 c->x, m)) ||
-            (rc = launch_f32_to_xfrag(s, h.cat, 2 * c->hidden, h.xf_cat, m)))
+        if ((rc = launch_mtp_input(s, c->embed_raw, c->embed_dtype, c->vp_dev, h.feed_dev, c->vocab, h.h_src, h.norm_e,
+                                   h.target->final_norm, h.norm_h, c->eps, c->hidden, h.xf_cat, c->x, c->freqs, c->rope_mscale,
+                                   c->hd / 2, c->rope_cs, m)))
             return rc;
         prev_splits = splits_for(h.fc, m, EPI_PARTIAL);
         rc = launch_gemm(s, h.fc, h.xf_cat, c->partial, c->vp_dev, m, prev_splits, EPI_PARTIAL, c->hidden, c->hidden);
@@ -1190,13 +1188,13 @@ int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* 
     }
     if (share) {
         tsv_ctx::Mtp& h = c->mtp;
-        if ((rc = dev_alloc(c, &h.e_rows, (size_t)16 * c->hidden * 4, true)) ||
-            (rc = dev_alloc(c, &h.cat, (size_t)16 * 2 * c->hidden * 4, true)) ||
-            (rc = dev_alloc(c, &h.xf_cat, xfrag_bytes(2 * c->hidden), true)) || (rc = dev_alloc(c, &h.chain, 32 * 4, true)) ||
+        if ((rc = dev_alloc(c, &h.xf_cat, xfrag_bytes(2 * c->hidden), true)) || (rc = dev_alloc(c, &h.chain, 32 * 4, true)) ||
+            (rc = dev_alloc(c, &h.vp_block, TSV_MAX_ROWS * sizeof(VerifyParams), true)) ||
             (rc = dev_alloc(c, &h.draw_dev, TSV_MAX_ROWS * sizeof(AcceptParams), true)))
             return fail(rc);
         if (hipHostMalloc((void**)&h.chain_host, 32 * 4) != hipSuccess ||
-            hipHostMalloc((void**)&h.draw_host, TSV_MAX_ROWS * sizeof(AcceptParams)) != hipSuccess) {
+            hipHostMalloc((void**)&h.draw_host, TSV_MAX_ROWS * sizeof(AcceptParams)) != hipSuccess ||
+            hipHostMalloc((void**)&h.vp_block_host, TSV_MAX_ROWS * sizeof(VerifyParams)) != hipSuccess) {
             set_error("mtp_open: pinned host allocation failed");
             return fail(TSV_ERR_DEVICE);
         }
@@ -1236,6 +1234,7 @@ extern "C" void tsv_close(tsv_ctx* c) {
     if (c->tok_host) (void)hipHostFree(c->tok_host);
     if (c->mtp.chain_host) (void)hipHostFree(c->mtp.chain_host);
     if (c->mtp.draw_host) (void)hipHostFree(c->mtp.draw_host);
+    if (c->mtp.vp_block_host) (void)hipHostFree(c->mtp.vp_block_host);
     if (c->mtp.on && c->mtp.target && c->mtp.target->mtp_head == c) c->mtp.target->mtp_head = nullptr;
     for (hipGraphExec_t g : c->pass_graph)
         if (g) (void)hipGraphExecDestroy(g);

@@ -301,10 +301,11 @@ int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, in
                    const float* bias = nullptr, const X8* x8 = nullptr, int x8_terms = 0, int blocks = 1,
                    const NormBlocks* nb = nullptr);
 int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int m);
-// the drafter head: fc's input rows [m][2 * hidden] from embedding rows and residual rows; clears x_zero's rows
-int launch_mtp_cat(hipStream_t s, const float* e_rows, const float* h_rows, const float* w_e, const float* w_t,
-                   const float* w_h, float eps, int hidden, float* cat, float* x_zero, int m);
-int launch_feed_token(hipStream_t s, VerifyParams* vp, const int32_t* token, int vocab);
+// the drafter head: fc's input rows as fragments (K = 2 * hidden) from the rows' next tokens (row 0's from device memory when
+// token_dev is given) and residual rows; fills the rotation table, clears x_zero's rows
+int launch_mtp_input(hipStream_t s, const uint8_t* raw, int dtype, const VerifyParams* vp, const int32_t* token_dev, int vocab,
+                     const float* h_rows, const float* w_e, const float* w_t, const float* w_h, float eps, int hidden, uint4* xfrag,
+                     float* x_zero, const float* freqs, float mscale, int half, float2* cs, int m);
 
 struct RopeKvArgs {
     const float* qkv;  // [splits][16][ldq]
