@@ -330,6 +330,8 @@ def main():
     ap.add_argument("--prefill-bench", type=int, default=0, metavar="TOKENS",
                     help="time tsv_prefill over a prompt of this many tokens (after one untimed run of the same), print one "
                          "JSON line and exit")
+    ap.add_argument("--weights-dtype", default=None, choices=["q4_k", "q8_0", "bf16"],
+                    help="--prefill-bench: the dense workload's shape with its matrices in this storage type")
     ap.add_argument("--loop-bench", type=int, default=0, metavar="NEW_TOKENS",
                     help="end to end instead of one step: generate this many tokens with the library's loop and its "
                          "drafter head (one decoder layer of the workload's shape, draft cost inside the timed region); "
@@ -387,6 +389,10 @@ def main():
     cfg["max_context"] = ctx + 32
     V = cfg["vocab"]
 
+    if args.weights_dtype:
+        if not args.prefill_bench or cfg.get("n_experts"):
+            sys.exit("bench.py: --weights-dtype goes with --prefill-bench at a dense workload")
+        cfg["dtype"] = {"q4_k": ts.ffi.Q4_K, "q8_0": ts.ffi.Q8_0, "bf16": ts.ffi.BF16}[args.weights_dtype]
     if args.loop_bench and args.weak_layers != 1.0:
         cfg["weak_layers"] = args.weak_layers
     if args.loop_bench and args.embed_scale != 1.0:
@@ -409,10 +415,12 @@ def main():
         t0 = time.perf_counter()
         eng.prefill(prompt, 0, want_logits=False)     # returns after the stream has drained
         dt = time.perf_counter() - t0
-        rows = 16 if os.environ.get("TSV_WIDE_PREFILL") == "0" or cfg["dtype"] != ts.ffi.Q4_K or cfg.get("n_experts") else 64
+        wide = cfg["dtype"] in (ts.ffi.Q4_K, ts.ffi.Q8_0, ts.ffi.BF16) and not cfg.get("n_experts")
+        rows = 64 if wide and os.environ.get("TSV_WIDE_PREFILL") != "0" else 16
         print(json.dumps({"metric": "prefill tokens/s", "value": round(n / dt, 1), "unit": "tokens/s", "n_gpus": 1,
                           "higher_is_better": True, "dtype": "f16", "data": "synthetic", "seconds": round(dt, 4),
-                          "config": {"workload": args.workload, "layers": cfg["n_layers"], "prompt_tokens": n,
+                          "config": {"workload": args.workload, "weights": args.weights_dtype or "as the workload names",
+                                     "layers": cfg["n_layers"], "prompt_tokens": n,
                                      "rows_per_pass": rows, "logits": "none (headless passes)"}}))
         return
     if args.loop_bench:

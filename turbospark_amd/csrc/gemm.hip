@@ -803,6 +803,273 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa)
     }
 }
 
+// ---- the same pass over Q8_0 weights ---------------------------------------------------------
+// A chunk is 128 K = four 32-element blocks, each with its own fp16 scale per weight row, so a block is
+// one matrix instruction per row block whose result takes the block's scale in fp32 (fma4) on its way
+// into the accumulator.  The operand is the signed code itself: the bytes become 1024 + (q + 128) by a
+// byte permute against 0x64 as in the narrower kernel, and one packed add of -1152 -- exact -- leaves q;
+// the activations' sums are not needed.  Products are again those of the same integers and the same
+// fp16 activations as in the narrower kernels.
+constexpr int WIDE80_B_BYTES = 16384;                    // [row block][block j][64 lanes][16 B]
+constexpr int WIDE80_BUF_BYTES = WIDE80_B_BYTES + 4096;  // + [row block][64 lanes] the four scales as floats
+
+struct WideW80 {
+    u32x2 q[4];
+    u32x2 d;
+};
+struct WideX80 {
+    u32x4 v[4];
+};
+
+__device__ __forceinline__ void wide80_load_w(WideW80& w, const uint8_t* tile_chunk, int rb, int lane) {
+    const int r = lane & 15, kg = lane >> 4;
+    const uint8_t* wp = tile_chunk + ((kg >> 1) * 64 + 16 * rb + r) * 16 + (kg & 1) * 8;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) w.q[j] = __builtin_nontemporal_load((const u32x2*)(wp + 2 * j * 64 * 16));
+    w.d = __builtin_nontemporal_load((const u32x2*)(tile_chunk + 8192 + (16 * rb + r) * 8));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void wide80_load_x(WideX80& x, const GemmArgs& a, int c, int lane) {
+    const u32x4* xp = (const u32x4*)a.xfrag + (size_t)c * 256 + lane;  // frag16_index: [block of 32 K][lane][16 B]
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) x.v[j] = xp[j * 64];
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void wide80_unpack(const WideW80& w, const Consts& k, uint8_t* buf, int rb, int lane) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const half2v off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    const float4v d = {h2f_lo(w.d.x), h2f_hi(w.d.x), h2f_lo(w.d.y), h2f_hi(w.d.y)};
+    *(float4v*)(buf + WIDE80_B_BYTES + (rb * 64 + lane) * 16) = d;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t wa = w.q[j].x ^ 0x80808080u, wb = w.q[j].y ^ 0x80808080u;
+        const uint32_t sel[2] = {0x04020400u, 0x04030401u};  // bytes (0, 2) and (1, 3) under 0x64: 1024 + code
+        u32x4 b;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            b[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2v, __builtin_amdgcn_perm(k.k64, wa, sel[i])) + off);
+            b[2 + i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2v, __builtin_amdgcn_perm(k.k64, wb, sel[i])) + off);
+        }
+        *(u32x4*)(buf + ((rb * 4 + j) * 64 + lane) * 16) = b;
+    }
+}
+
+__device__ __forceinline__ void wide80_compute(const WideX80& x, const uint8_t* buf, float4v (&acc)[4], int lane) {
+    const float4v zero = {0.f, 0.f, 0.f, 0.f};
+    float4v d[4], t[4];
+    u32x4 b[2][4];
+    auto fetch = [&](int slot, int j) {
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++) b[slot][rb] = *(const u32x4*)(buf + ((rb * 4 + j) * 64 + lane) * 16);
+    };
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) d[rb] = *(const float4v*)(buf + WIDE80_B_BYTES + (rb * 64 + lane) * 16);
+    fetch(0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if (j < 3) fetch((j + 1) & 1, j + 1);
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            t[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, x.v[j]), __builtin_bit_cast(half8, b[j & 1][rb]),
+                                                           zero, 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++) fma4(acc[rb], d[rb][j], t[rb]);
+    }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_q80(GemmWideArgs wa) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    GemmArgs a = wa.g;
+    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
+    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
+    a.vp = a.vp + wave;
+    if (EPI == EPI_ROPE) {
+        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
+        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
+    }
+    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
+    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q80::TILE_BYTES;
+    Consts k;
+    k.k6400 = 0;
+    k.k5400 = 0;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k64));
+    float4v acc[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int M = a.vp->m;
+    // the chunk loop of k_gemm_wide: unpack c -> ask for what comes next -> barrier -> multiply c
+    WideW80 w[2];
+    WideX80 x[2];
+    uint8_t* const buf0 = wide_lds;
+    uint8_t* const buf1 = wide_lds + WIDE80_BUF_BYTES;
+    const int last = s1 - 1;
+    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * Q80::TILE_BYTES; };
+    wide80_load_w(w[0], tile_at(s0), wave, lane);
+    wide80_load_x(x[0], a, s0, lane);
+    wide80_load_w(w[1], tile_at(s0 + 1), wave, lane);
+    int c = s0;
+    for (; c + 2 <= s1; c += 2) {
+        wide80_unpack(w[0], k, buf0, wave, lane);
+        wide80_load_w(w[0], tile_at(c + 2), wave, lane);
+        wide80_load_x(x[1], a, min(c + 1, last), lane);
+        __syncthreads();
+        wide80_compute(x[0], buf0, acc, lane);
+        wide80_unpack(w[1], k, buf1, wave, lane);
+        wide80_load_w(w[1], tile_at(c + 3), wave, lane);
+        wide80_load_x(x[0], a, min(c + 2, last), lane);
+        __syncthreads();
+        wide80_compute(x[1], buf1, acc, lane);
+    }
+    if (c < s1) {
+        wide80_unpack(w[0], k, buf0, wave, lane);
+        __syncthreads();
+        wide80_compute(x[0], buf0, acc, lane);
+    }
+    __syncthreads();
+    float* ssum = (float*)(wide_lds + 2 * WIDE80_BUF_BYTES) + wave * 32;
+#pragma unroll
+    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
+    if (EPI == EPI_SILU) {
+        __syncthreads();
+        if (lane < 16 && lane < M) {
+            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
+            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
+        }
+    }
+}
+
+// ---- the same pass over bf16 weights ---------------------------------------------------------
+// A chunk is 64 K, and a tile's unit 4 s + kg already is what lane (r, kg) of v_mfma_f32_16x16x32_bf16
+// holds of weight row r in K step s, so "unpacking" is a copy into LDS.  The fp16 activations go in as
+// two bf16 terms, split exactly as in the narrower kernel (upper eight significant bits + remainder).
+constexpr int WIDEBF_BUF_BYTES = 8192;  // [row block][K step][64 lanes][16 B]
+
+struct WideWBf {
+    u32x4 q[2];
+};
+struct WideXBf {
+    u32x4 v[2];
+};
+
+__device__ __forceinline__ void widebf_load_w(WideWBf& w, const uint8_t* tile_chunk, int rb, int lane) {
+    const int r = lane & 15, kg = lane >> 4;
+    const uint8_t* wp = tile_chunk + (kg * 64 + 16 * rb + r) * 16;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int st = 0; st < 2; st++) w.q[st] = __builtin_nontemporal_load((const u32x4*)(wp + st * 4 * 64 * 16));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void widebf_load_x(WideXBf& x, const GemmArgs& a, int c, int lane) {
+    const u32x4* xp = (const u32x4*)a.xfrag + (size_t)c * 128 + lane;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int st = 0; st < 2; st++) x.v[st] = xp[st * 64];
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void widebf_store(const WideWBf& w, uint8_t* buf, int rb, int lane) {
+#pragma unroll
+    for (int st = 0; st < 2; st++) *(u32x4*)(buf + ((rb * 2 + st) * 64 + lane) * 16) = w.q[st];
+}
+
+__device__ __forceinline__ void widebf_compute(const WideXBf& x, const uint8_t* buf, float4v (&acc)[4], int lane) {
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    u32x4 b[2][4];
+#pragma unroll
+    for (int st = 0; st < 2; st++)
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++) b[st][rb] = *(const u32x4*)(buf + ((rb * 2 + st) * 64 + lane) * 16);
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+        u32x4 hi, lo;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t word = x.v[st][i];
+            const float f0 = h2f_lo(word), f1 = h2f_hi(word);
+            const uint32_t b0 = __float_as_uint(f0) & 0xFFFF0000u, b1 = __float_as_uint(f1) & 0xFFFF0000u;
+            const uint32_t r0 = __float_as_uint(f0 - __uint_as_float(b0)), r1 = __float_as_uint(f1 - __uint_as_float(b1));
+            hi[i] = (b0 >> 16) | b1;
+            lo[i] = (r0 >> 16) | (r1 & 0xFFFF0000u);
+        }
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, hi), __builtin_bit_cast(bf16x8, b[st][rb]),
+                                                              acc[rb], 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, lo), __builtin_bit_cast(bf16x8, b[st][rb]),
+                                                              acc[rb], 0, 0, 0);
+    }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_bf16(GemmWideArgs wa) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    GemmArgs a = wa.g;
+    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
+    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
+    a.vp = a.vp + wave;
+    if (EPI == EPI_ROPE) {
+        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
+        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
+    }
+    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
+    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * BF16W::TILE_BYTES;
+    float4v acc[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int M = a.vp->m;
+    WideWBf w[2];
+    WideXBf x[2];
+    uint8_t* const buf0 = wide_lds;
+    uint8_t* const buf1 = wide_lds + WIDEBF_BUF_BYTES;
+    const int last = s1 - 1;
+    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * BF16W::TILE_BYTES; };
+    widebf_load_w(w[0], tile_at(s0), wave, lane);
+    widebf_load_x(x[0], a, s0, lane);
+    widebf_load_w(w[1], tile_at(s0 + 1), wave, lane);
+    int c = s0;
+    for (; c + 2 <= s1; c += 2) {
+        widebf_store(w[0], buf0, wave, lane);
+        widebf_load_w(w[0], tile_at(c + 2), wave, lane);
+        widebf_load_x(x[1], a, min(c + 1, last), lane);
+        __syncthreads();
+        widebf_compute(x[0], buf0, acc, lane);
+        widebf_store(w[1], buf1, wave, lane);
+        widebf_load_w(w[1], tile_at(c + 3), wave, lane);
+        widebf_load_x(x[0], a, min(c + 2, last), lane);
+        __syncthreads();
+        widebf_compute(x[1], buf1, acc, lane);
+    }
+    if (c < s1) {
+        widebf_store(w[0], buf0, wave, lane);
+        __syncthreads();
+        widebf_compute(x[0], buf0, acc, lane);
+    }
+    __syncthreads();
+    float* ssum = (float*)(wide_lds + 2 * WIDEBF_BUF_BYTES) + wave * 32;
+#pragma unroll
+    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
+    if (EPI == EPI_SILU) {
+        __syncthreads();
+        if (lane < 16 && lane < M) {
+            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
+            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
+        }
+    }
+}
+
 // Fewest rows that go to the 16x16x32 form (TSV_GEMM16=0: never; TSV_GEMM16=<n>: from n rows on).
 static int gemm16_min_rows() {
     static const int n = [] {
@@ -930,11 +1197,11 @@ int gemm_wide_rows() { return 16 * WIDE_BLOCKS; }
 
 // The same matmul over gemm_wide_rows() rows in blocks of sixteen: block b reads its fragments at
 // xfrag + b * x_stride bytes, its parameters at vp + b, and writes at out + b * out_stride bytes
-// (EPI_ROPE: rope->cs and rope->q16 hold all blocks' rows one after the other).  Q4_K weights only.
+// (EPI_ROPE: rope->cs and rope->q16 hold all blocks' rows one after the other).  Q4_K, Q8_0 or bf16 weights.
 int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t x_stride, void* out, size_t out_stride,
                      const VerifyParams* vp, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
-    if (w.fmt != FMT_Q4K) {
-        set_error("matmul: prompt blocks of 64 rows need Q4_K weights");
+    if (w.fmt != FMT_Q4K && w.fmt != FMT_Q80 && w.fmt != FMT_BF16) {
+        set_error("matmul: prompt blocks of 64 rows need Q4_K, Q8_0 or bf16 weights");
         return TSV_ERR_UNSUPPORTED;
     }
     GemmWideArgs wa{};
@@ -942,6 +1209,28 @@ int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t 
     wa.x_stride = x_stride;
     wa.out_stride = out_stride;
     wa.g.out16 = 1;  // what this kernel reads is what it writes for the next one
+    if (w.fmt == FMT_Q80 || w.fmt == FMT_BF16) {
+        const bool q80 = w.fmt == FMT_Q80;
+        const size_t lds2 = 2 * (size_t)(q80 ? WIDE80_BUF_BYTES : WIDEBF_BUF_BYTES) + WIDE_BLOCKS * 32 * sizeof(float);
+        const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
+        switch (epi) {
+            case EPI_PARTIAL:
+                if (q80) hipLaunchKernelGGL(k_gemm_wide_q80<EPI_PARTIAL>, grid, block, lds2, s, wa);
+                else hipLaunchKernelGGL(k_gemm_wide_bf16<EPI_PARTIAL>, grid, block, lds2, s, wa);
+                break;
+            case EPI_ROPE:
+                if (q80) hipLaunchKernelGGL(k_gemm_wide_q80<EPI_ROPE>, grid, block, lds2, s, wa);
+                else hipLaunchKernelGGL(k_gemm_wide_bf16<EPI_ROPE>, grid, block, lds2, s, wa);
+                break;
+            case EPI_SILU:
+                if (q80) hipLaunchKernelGGL(k_gemm_wide_q80<EPI_SILU>, grid, block, lds2, s, wa);
+                else hipLaunchKernelGGL(k_gemm_wide_bf16<EPI_SILU>, grid, block, lds2, s, wa);
+                break;
+            default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
+        }
+        TSV_HIP(hipGetLastError());
+        return TSV_OK;
+    }
     const size_t lds = 2 * (size_t)WIDE_BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
     const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
     static bool attr_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel

@@ -596,10 +596,12 @@ int launch_pass(tsv_ctx* c, int m) {
 // cache stores, attention -- is the 16-row pass's own code on block-strided buffers: block b is
 // rows base + 16 b .. base + 16 b + 15, its attention sees the cache up to its own rows, which the
 // q/k/v projection of the same pass has already stored for every block before any block attends.
-// Only for headless passes (no logits wanted) of dense models whose four matmuls are Q4_K with the
-// rotating epilogue, and whose layers are linear caches: a ring layer's slack is 32 rows, fewer than
-// a 64-row pass writes ahead of its first block's window.
+// Only for headless passes (no logits wanted) of dense models whose four matmuls are Q4_K, Q8_0 or bf16
+// (the q/k/v projection with the rotating epilogue, or followed by the rotation kernel block by
+// block), and whose layers are linear caches: a ring layer's slack is 32 rows, fewer than a 64-row
+// pass writes ahead of its first block's window.
 constexpr int WIDE_B = 4;
+static bool wide_fmt(int fmt) { return fmt == FMT_Q4K || fmt == FMT_Q80 || fmt == FMT_BF16; }
 
 int wide_prepare(tsv_ctx* c) {
     tsv_ctx::Wide& w = c->wide;
@@ -651,7 +653,35 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         re.nkv = c->nkv;
         re.hd = c->hd;
         re.max_ctx = L.kv_slots;
-        if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
+        if (L.rope_fused) {
+            if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
+        } else {
+            // the projection's partial sums, then the 16-row pass's own norm / rotation / cache stores block by block
+            const int spq = splits_for(L.qkv, 16, EPI_PARTIAL);
+            if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, w.partial, pstride, w.vp, spq, EPI_PARTIAL, qkv_n, L.qkv.n_rows)))
+                return rc;
+            for (int b = 0; b < WIDE_B; b++) {
+                RopeKvArgs ra{};
+                ra.qkv = w.partial + (size_t)b * c->partial_floats;
+                ra.splits = spq;
+                ra.ldq = qkv_n;
+                ra.freqs = c->freqs;
+                ra.mscale = c->rope_mscale;
+                ra.bias = L.bqkv;
+                ra.q_norm = L.q_norm;
+                ra.k_norm = L.k_norm;
+                ra.eps = c->eps;
+                ra.q16 = w.q16 + (size_t)b * 16 * qd;
+                ra.kc = L.kc;
+                ra.vc = L.vc;
+                ra.nq = c->nq;
+                ra.nkv = c->nkv;
+                ra.hd = c->hd;
+                ra.max_ctx = L.kv_slots;
+                ra.vp = w.vp + b;
+                if ((rc = launch_rope_kv(s, ra, 16))) return rc;
+            }
+        }
         if (L.tq.k_bits) {  // all 64 rows are quantized (and their q rows rotated) before any block attends
             TqArgs ta{};
             ta.q16 = w.q16;
@@ -1209,8 +1239,8 @@ int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* 
     // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
     c->wide.ok = c->rewind_budget == INT64_MAX;
     for (const LayerW& L : c->layers)
-        if (L.n_experts || !L.rope_fused || L.v_only.tiles || L.qkv.fmt != FMT_Q4K || L.wo.fmt != FMT_Q4K ||
-            L.gate_up.fmt != FMT_Q4K || L.down.fmt != FMT_Q4K)
+        if (L.n_experts || L.v_only.tiles || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) ||
+            !wide_fmt(L.gate_up.fmt) || !wide_fmt(L.down.fmt))
             c->wide.ok = false;
     if (const char* e = getenv("TSV_WIDE_PREFILL")) c->wide.ok = c->wide.ok && e[0] != '0';
     if (share) c->wide.ok = false;  // the head's rows come sixteen at a time
