@@ -415,7 +415,7 @@ def main():
         t0 = time.perf_counter()
         eng.prefill(prompt, 0, want_logits=False)     # returns after the stream has drained
         dt = time.perf_counter() - t0
-        wide = cfg["dtype"] in (ts.ffi.Q4_K, ts.ffi.Q8_0, ts.ffi.BF16) and not cfg.get("n_experts")
+        wide = cfg["dtype"] in (ts.ffi.Q4_K, ts.ffi.Q8_0, ts.ffi.BF16) and not (cfg.get("n_experts") and os.environ.get("TSV_MOE_FP4"))
         rows = 64 if wide and os.environ.get("TSV_WIDE_PREFILL") != "0" else 16
         print(json.dumps({"metric": "prefill tokens/s", "value": round(n / dt, 1), "unit": "tokens/s", "n_gpus": 1,
                           "higher_is_better": True, "dtype": "f16", "data": "synthetic", "seconds": round(dt, 4),

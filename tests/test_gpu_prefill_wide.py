@@ -95,6 +95,44 @@ def test_wide_passes_where_the_rotation_is_a_kernel_of_its_own(name, over, monke
     assert err_w <= gc.TOL.get(cfg["dtype"], 1e-2) and err_wn <= 2e-3
 
 
+@pytest.mark.parametrize("name,n_prompt,seed", [("moe_small", 150, 31), ("gptoss_small", 150, 31), ("moe_small", 64, 32),
+                                                ("gptoss_small", 200, 33)])
+def test_routed_layers_in_passes_of_64_rows(name, n_prompt, seed):
+    """Routed experts over the 64 rows of a prompt pass: every expert is multiplied once against all the rows of the
+    pass that chose it (crates/runtime/src/families/llama/moe.rs, the grouping of moe.hip taken to 64 rows).  Held to
+    the oracle and to the 16-row passes of the same library.  (The rows' inputs to the router differ by rounding
+    between the two GPU paths, so a near tie can fall either way; these seeds have none inside that band, and the
+    selections of the following verify pass are compared to say so.)"""
+    from turbospark_amd import synth
+    from oracle import binding as ob
+    cfg = dict(synth.CONFIGS[name], max_context=n_prompt + 48)
+    w = synth.make_weights(cfg, seed=seed)
+    wide, narrow = _engine(cfg, w, True), _engine(cfg, w, False)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)
+    rng = np.random.default_rng(seed)
+    prompt = rng.integers(0, cfg["vocab"], n_prompt).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    wide.prefill(prompt, 0, want_logits=False)
+    narrow.prefill(prompt, 0, want_logits=False)
+    for i in range(0, n_prompt, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    assert wide.position == narrow.position == n_prompt
+    for layer in range(cfg["n_layers"]):
+        (kw, vw), (kn, vn), (kc, vc) = wide.read_kv(layer, 0, n_prompt), narrow.read_kv(layer, 0, n_prompt), cpu.kv(layer)
+        for got, other, want in ((kw, kn, kc), (vw, vn, vc)):
+            got, other, want = got.astype(np.float32), other.astype(np.float32), want[:n_prompt]
+            scale = np.abs(want).max()
+            assert np.abs(got - want).max() <= 2e-2 * scale, (layer, np.abs(got - want).max() / scale)
+            assert np.abs(got - other).max() <= 4e-3 * scale, (layer, np.abs(got - other).max() / scale)
+    want = cpu.verify(feed, n_prompt)
+    got_w, got_n = wide.verify(feed, n_prompt), narrow.verify(feed, n_prompt)
+    k = cfg["top_k"]
+    assert np.array_equal(wide.route_selected()[:, :5, :k], narrow.route_selected()[:, :5, :k])
+    err_w, err_wn = gc.logit_error(got_w, want), gc.logit_error(got_w, got_n)
+    print(f"{name}, prompt of {n_prompt}: logits after 64-row passes vs oracle {err_w:.2e}, the two GPU paths {err_wn:.2e}")
+    assert err_w <= 1e-2 and err_wn <= 2e-3
+
+
 def test_logits_of_the_last_prompt_token_after_wide_passes():
     """tsv_prefill hands out the last row's logits: the rows before it go in blocks of 64, the tail in
     16-row passes whose last one carries the output head."""

@@ -86,7 +86,16 @@ struct tsv_ctx {
         float2* rope_cs = nullptr;
         float *part_o = nullptr, *part_ml = nullptr;  // attention partials of every block
         size_t part_o_stride = 0, part_ml_stride = 0;
+        // routed layers: the 64 rows' factors and selections, every expert's members, the experts' gate/up outputs
+        // (four 16-member sub-buffers per expert) and the blocks' per-slot down outputs
+        float* route_w = nullptr;
+        int32_t* route_sel = nullptr;
+        MoeGroupW* groups = nullptr;
+        uint8_t* frag_e = nullptr;
+        size_t frag_e_sub = 0;
+        float* moe_out = nullptr;
     } wide;
+    bool route_forced_set = false;  // tsv_force_route holds selections: prompt passes stay at sixteen rows
     uint16_t* q16 = nullptr;
     float *part_o = nullptr, *part_ml = nullptr;
     int nch = 0;

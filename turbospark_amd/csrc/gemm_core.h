@@ -267,6 +267,12 @@ struct ActLoader {
         rowoff[g] = (row >> 2) * 64 + (row & 3);
         sumoff[g] = (row >> 2) * 32 + (row & 3);
     }
+    // row `row` of a buffer made of 16-row blocks `block_bytes` apart (fragments and sums move together)
+    __device__ __forceinline__ void set_row_blocked(int g, int row, size_t block_bytes) {
+        set_row(g, row & 15);
+        rowoff[g] += (int)((row >> 4) * (block_bytes >> 3));
+        sumoff[g] += (int)((row >> 4) * (block_bytes >> 2));
+    }
     __device__ __forceinline__ ActLoader(const void* xfrag, const void* xsum, int lane) {
         fragp = (const u32x2*)xfrag;
         sump = (const float*)xsum;

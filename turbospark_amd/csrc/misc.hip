@@ -156,7 +156,7 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
                 float4 r = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s = 0; s < NS; s++) {
-                    const float ws = weights[m * 8 + s];
+                    const float ws = weights[(blockIdx.y * 16 + m) * 8 + s];  // (block b's factors follow block b - 1's)
                     r.x = __fadd_rn(r.x, __fmul_rn(ws, p[s].x));
                     r.y = __fadd_rn(r.y, __fmul_rn(ws, p[s].y));
                     r.z = __fadd_rn(r.z, __fmul_rn(ws, p[s].z));
@@ -368,7 +368,10 @@ int launch_f32_to_xfrag(hipStream_t s, const float* x, int k, uint4* xfrag, int 
 // MFMA A-fragments: [hd/16][lane = (pos%16/4)*16 + d%16][pos%4].
 __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
     const int m = blockIdx.x, head = blockIdx.y;
-    const VerifyParams* vp = a.vp;
+    // a prompt pass of several 16-row blocks: block blockIdx.z has its own parameters, partial sums and q rows
+    const VerifyParams* vp = a.vp + blockIdx.z;
+    a.qkv += (long)blockIdx.z * a.qkv_block_stride;
+    a.q16 += (long)blockIdx.z * 16 * a.nq * a.hd;
     // everything the kernel needs from the parameter block is asked for at once
     const int rows = vp->m, rot_pos = vp->pos[m], base = vp->base;
     if (m >= rows) return;
@@ -454,7 +457,7 @@ int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m) {
         set_error("rope: one to eight partial sums");
         return TSV_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(k_rope_kv, dim3(m, a.nq + 2 * a.nkv), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(k_rope_kv, dim3(m, a.nq + 2 * a.nkv, std::max(1, a.blocks)), dim3(64), 0, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }

@@ -126,6 +126,12 @@ __device__ __forceinline__ void route_row(const MoeRouteArgs& a, int m, uint32_t
 __global__ __launch_bounds__(1024) void k_route_rank(MoeRouteArgs a) {
     const int lane = threadIdx.x & 63, m = threadIdx.x >> 6;
     if (m >= a.m) return;
+    if (a.blocks > 1) {  // a prompt pass: this workgroup's block of sixteen rows
+        a.logits += (long)blockIdx.x * a.logits_block_stride;
+        a.weights += blockIdx.x * 16 * 8;
+        a.selected += blockIdx.x * 16 * 8;
+        a.forced = nullptr;
+    }
     const int ne = a.n_experts;
     // everything the row needs is asked for before the first add: the loads have no branch between them (a lane
     // past the last expert reads the last expert's, a split past the last split the last split's again)
@@ -161,8 +167,11 @@ __device__ __forceinline__ float silu_moe(float x) { return x / (1.0f + __expf(-
 // requested at once); one otherwise (90-100 VGPRs instead of 150-230, so twice the resident waves,
 // which is worth more over a longer walk): the 120B-shaped step 5.86 -> 5.24 ms, the 30B-shaped one
 // 4.43 ms either way.
-template <class F, int EPI, int STAGES>
-__device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup& grp, int gi, int r0, float4v* red) {
+// WIDE: the group is an expert's members among the 64 rows of a prompt pass (MoeGroupW): rows and members are
+// addressed through their 16-row blocks, and every wave stays to the end so that the caller can go on to the
+// group's next four members.
+template <class F, int EPI, int STAGES, bool WIDE = false, class G = MoeGroup>
+__device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, int gi, int r0, float4v* red) {
     constexpr int NG = 1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int tile = blockIdx.x, e = grp.expert, cnt = grp.cnt;
@@ -180,7 +189,12 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
     const uint8_t* xbase = (const uint8_t*)a.xfrag + (EPI == EPI_SLOT ? (size_t)gi * a.x_stride : 0);
     ActLoader<false> x(xbase, xbase + xfrag_sum_offset(a.k), lane);
     const int mine = min(r0 + (lane & 3), cnt - 1);
-    x.set_row(0, EPI == EPI_SILU ? grp.rows[mine] : mine);
+    if (WIDE) {
+        if (EPI == EPI_SILU) x.set_row_blocked(0, grp.rows[mine], a.x_block_stride);
+        else x.set_row_blocked(0, mine, a.sub_stride);
+    } else {
+        x.set_row(0, EPI == EPI_SILU ? grp.rows[mine] : mine);
+    }
 
     float4v acc[NG] = {float4v{0.f, 0.f, 0.f, 0.f}};
     if (nc > 0) {
@@ -214,7 +228,7 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
     __syncthreads();
     red[wave * 64 + lane] = acc[0];
     __syncthreads();
-    if (wave != 0) return;
+    if (wave != 0) return;  // (WIDE: the caller's barrier is the next thing every wave meets)
     float4v v = red[lane];
     for (int w = 1; w < nw; w++) v += red[w * 64 + lane];
     if (EPI == EPI_SILU) {
@@ -243,8 +257,14 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
             for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
             const int b = r0 + i;  // the group's own row order
             if (b < cnt && lane < 32) {
-                out[frag_index(col, b)] = h;
-                if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
+                if (WIDE) {
+                    _Float16* ow = (_Float16*)((uint8_t*)out + (size_t)(b >> 4) * a.sub_stride);
+                    ow[frag_index(col, b & 15)] = h;
+                    if (lane == 0) ((float*)((uint8_t*)ow + xfrag_sum_offset(a.n_out)))[xsum_index(col >> 5, b & 15)] = sum;
+                } else {
+                    out[frag_index(col, b)] = h;
+                    if (lane == 0) sums[xsum_index(col >> 5, b)] = sum;
+                }
             }
         }
     } else {
@@ -253,9 +273,12 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const MoeGroup
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int b = r0 + i;
-                if (b < cnt)
-                    ((float*)a.out)[((size_t)grp.slots[b] * 16 + grp.rows[b]) * a.n_out + n] =
-                        a.bias ? v[i] + a.bias[(size_t)e * a.n_out + n] : v[i];
+                if (b < cnt) {
+                    const int row = grp.rows[b];
+                    const size_t at = WIDE ? (size_t)(row >> 4) * a.out_block_stride + ((size_t)grp.slots[b] * 16 + (row & 15)) * a.n_out
+                                           : ((size_t)grp.slots[b] * 16 + row) * a.n_out;
+                    ((float*)a.out)[at + n] = a.bias ? v[i] + a.bias[(size_t)e * a.n_out + n] : v[i];
+                }
             }
         }
     }
@@ -275,6 +298,89 @@ __global__ __launch_bounds__(512) void k_moe_gemm(MoeGemmArgs a) {
     __syncthreads();
     if (r0 >= grp.cnt) return;
     expert_tile<F, EPI, STAGES>(a, grp, gi, r0, red);
+}
+
+// ---- the 64 rows of a prompt pass ---------------------------------------------------------------
+// The members of every expert: one wave per expert walks the pass's (row, slot) pairs sixty-four at a time in
+// pair order; a ballot marks the pairs that name the expert and a lane's place in the list is the count of
+// marked pairs before it.  A row names an expert at most once, so a list has at most as many members as the
+// pass has rows.
+__global__ __launch_bounds__(1024) void k_moe_groups(const int32_t* __restrict__ selected, int rows, int top_k, int ne,
+                                                     MoeGroupW* __restrict__ groups) {
+    const int lane = threadIdx.x & 63, e = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (e >= ne) return;
+    MoeGroupW* g = groups + e;
+    const int np = rows * top_k;
+    int cnt = 0;
+    for (int p0 = 0; p0 < np; p0 += 64) {
+        const int p = p0 + lane;
+        const int row = p / top_k, slot = p - row * top_k;
+        const bool hit = p < np && selected[row * 8 + slot] == e;
+        const uint64_t mask = __builtin_amdgcn_ballot_w64(hit);
+        const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+        if (hit && pos < MOE_WIDE_ROWS) {
+            g->rows[pos] = row;
+            g->slots[pos] = slot;
+        }
+        cnt += __popcll(mask);
+    }
+    if (lane == 0) {
+        g->expert = e;
+        g->cnt = min(cnt, MOE_WIDE_ROWS);
+    }
+}
+
+// grid: (tiles per expert, experts, 4).  Workgroup z takes the expert's members 4 z .. 4 z + 3, then sixteen further
+// on, and so on: an expert few rows chose costs one workgroup per tile, one that many chose is spread over four.
+template <class F, int EPI, int STAGES>
+__global__ __launch_bounds__(512) void k_moe_gemm_wide(MoeGemmArgs a) {
+    extern __shared__ float4v red[];
+    __shared__ MoeGroupW grp;
+    const int e = blockIdx.y;
+    const MoeGroupW* src = a.groups + e;
+    const int cnt = min(src->cnt, MOE_WIDE_ROWS);
+    if (4 * (int)blockIdx.z >= cnt) return;
+    for (int i = threadIdx.x; i < MOE_WIDE_ROWS; i += blockDim.x) {
+        grp.rows[i] = min(max(src->rows[min(i, cnt - 1)], 0), MOE_WIDE_ROWS - 1);
+        grp.slots[i] = min(max(src->slots[min(i, cnt - 1)], 0), 7);
+    }
+    if (threadIdx.x == 0) {
+        grp.expert = e;
+        grp.cnt = cnt;
+    }
+    __syncthreads();
+    for (int r0 = 4 * blockIdx.z; r0 < cnt; r0 += 4 * gridDim.z) {
+        expert_tile<F, EPI, STAGES, true>(a, grp, e, r0, red);
+        __syncthreads();
+    }
+}
+
+template <class F, int EPI>
+int launch_moe_wide_t(hipStream_t s, const MoeGemmArgs& a) {
+    const int cpw = std::max(2, (a.kchunks + 3) / 4);
+    const int nw = std::min(8, std::max(1, (a.kchunks + cpw - 1) / cpw));
+    const size_t lds = (size_t)nw * 1024;
+    const dim3 grid(a.tiles_per_expert, a.n_experts, 4);
+    if ((a.kchunks + nw - 1) / nw <= 2)
+        hipLaunchKernelGGL((k_moe_gemm_wide<F, EPI, 2>), grid, dim3(64 * nw), lds, s, a);
+    else
+        hipLaunchKernelGGL((k_moe_gemm_wide<F, EPI, 1>), grid, dim3(64 * nw), lds, s, a);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+template <int EPI>
+int launch_moe_wide_f(hipStream_t s, int fmt, const MoeGemmArgs& a) {
+    if (!a.groups || a.n_experts < 1 || a.n_experts > 256 || a.rows != MOE_WIDE_ROWS || a.x8_terms) {
+        set_error("moe: a prompt pass lists its 64 rows' experts first and keeps fp16 activations");
+        return TSV_ERR_INVALID;
+    }
+    return fmt == FMT_Q4K    ? launch_moe_wide_t<Q4K, EPI>(s, a)
+           : fmt == FMT_Q80  ? launch_moe_wide_t<Q80, EPI>(s, a)
+           : fmt == FMT_Q6K  ? launch_moe_wide_t<Q6K, EPI>(s, a)
+           : fmt == FMT_Q5K  ? launch_moe_wide_t<Q5K, EPI>(s, a)
+           : fmt == FMT_BF16 ? launch_moe_wide_t<BF16W, EPI>(s, a)
+                             : launch_moe_wide_t<MX4, EPI>(s, a);
 }
 
 template <class F, int EPI>
@@ -318,10 +424,24 @@ int launch_route(hipStream_t s, const MoeRouteArgs& a) {
         set_error("moe: the router's logits come in one to eight partial sums of at most sixteen rows");
         return TSV_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(k_route_rank, dim3(1), dim3(64 * a.m), 0, s, a);
+    hipLaunchKernelGGL(k_route_rank, dim3(std::max(1, a.blocks)), dim3(64 * a.m), 0, s, a);
     TSV_HIP(hipGetLastError());
     return TSV_OK;
 }
+
+int launch_moe_groups(hipStream_t s, const int32_t* selected, int rows, int top_k, int n_experts, MoeGroupW* groups) {
+    if (rows < 1 || rows > MOE_WIDE_ROWS || n_experts < 1 || n_experts > 256 || top_k < 1 || top_k > 8) {
+        set_error("moe: at most 64 rows, 256 experts and top-k 8 in a prompt pass");
+        return TSV_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(k_moe_groups, dim3((n_experts + 15) / 16), dim3(1024), 0, s, selected, rows, top_k, n_experts, groups);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+int launch_moe_wide_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a) { return launch_moe_wide_f<EPI_SILU>(s, fmt, a); }
+
+int launch_moe_wide_down(hipStream_t s, int fmt, const MoeGemmArgs& a) { return launch_moe_wide_f<EPI_SLOT>(s, fmt, a); }
 
 int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups) {
     return launch_moe_f<EPI_SILU>(s, fmt, a, n_groups);

@@ -621,6 +621,16 @@ int wide_prepare(tsv_ctx* c) {
     w.part_ml_stride = (size_t)c->nkv * c->nch * rows_max * 2;
     if ((rc = dev_alloc(c, &w.part_o, WIDE_B * w.part_o_stride * 4, true)) || (rc = dev_alloc(c, &w.part_ml, WIDE_B * w.part_ml_stride * 4, true)))
         return rc;
+    int ne_max = 0;
+    for (const LayerW& L : c->layers) ne_max = std::max(ne_max, L.n_experts);
+    if (ne_max) {
+        w.frag_e_sub = (xfrag_bytes(c->ffn) + 255) & ~(size_t)255;
+        if ((rc = dev_alloc(c, &w.route_w, (size_t)WIDE_B * 16 * 8 * 4, true)) || (rc = dev_alloc(c, &w.route_sel, (size_t)WIDE_B * 16 * 8 * 4, true)) ||
+            (rc = dev_alloc(c, &w.groups, (size_t)ne_max * sizeof(MoeGroupW), true)) ||
+            (rc = dev_alloc(c, &w.frag_e, (size_t)ne_max * WIDE_B * w.frag_e_sub, true)) ||
+            (rc = dev_alloc(c, &w.moe_out, (size_t)WIDE_B * 8 * 16 * c->hidden * 4, true)))
+            return rc;
+    }
     w.ready = true;
     return TSV_OK;
 }
@@ -635,14 +645,21 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
                                c->rope_mscale, half, w.rope_cs + (size_t)b * 16 * half)))
             return rc;
     const NormBlocks nb{(long)16 * c->hidden, (long)c->partial_floats, (long)w.xfb, 1};
+    // after a routed layer the partial sums are the blocks' per-slot expert outputs and come with the rows' factors
+    const long moe_block = (long)8 * 16 * c->hidden;
+    const NormBlocks nb_moe{nb.x, moe_block, nb.frag, 1};
     const size_t pstride = c->partial_floats * 4;
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     int prev_splits = 0;
+    const float* prev_partial = w.partial;
+    const float* prev_weights = nullptr;
     for (int l = 0; l < c->n_layers; l++) {
         LayerW& L = c->layers[l];
-        if ((rc = launch_addnorm(s, w.x, w.partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr,
-                                 nullptr, nullptr, 0, WIDE_B, &nb)))
+        if ((rc = launch_addnorm(s, w.x, prev_partial, prev_splits, c->hidden, L.attn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, prev_weights,
+                                 nullptr, nullptr, 0, WIDE_B, prev_weights ? &nb_moe : &nb)))
             return rc;
+        prev_partial = w.partial;
+        prev_weights = nullptr;
         RopeEpi re{};
         re.cs = w.rope_cs;
         re.bias = L.bqkv;
@@ -656,13 +673,15 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         if (L.rope_fused) {
             if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
         } else {
-            // the projection's partial sums, then the 16-row pass's own norm / rotation / cache stores block by block
+            // the projection's partial sums, then the 16-row pass's own norm / rotation / cache stores over the four blocks
             const int spq = splits_for(L.qkv, 16, EPI_PARTIAL);
             if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, w.partial, pstride, w.vp, spq, EPI_PARTIAL, qkv_n, L.qkv.n_rows)))
                 return rc;
-            for (int b = 0; b < WIDE_B; b++) {
+            {
                 RopeKvArgs ra{};
-                ra.qkv = w.partial + (size_t)b * c->partial_floats;
+                ra.qkv = w.partial;
+                ra.blocks = WIDE_B;
+                ra.qkv_block_stride = (long)c->partial_floats;
                 ra.splits = spq;
                 ra.ldq = qkv_n;
                 ra.freqs = c->freqs;
@@ -671,14 +690,14 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
                 ra.q_norm = L.q_norm;
                 ra.k_norm = L.k_norm;
                 ra.eps = c->eps;
-                ra.q16 = w.q16 + (size_t)b * 16 * qd;
+                ra.q16 = w.q16;
                 ra.kc = L.kc;
                 ra.vc = L.vc;
                 ra.nq = c->nq;
                 ra.nkv = c->nkv;
                 ra.hd = c->hd;
                 ra.max_ctx = L.kv_slots;
-                ra.vp = w.vp + b;
+                ra.vp = w.vp;
                 if ((rc = launch_rope_kv(s, ra, 16))) return rc;
             }
         }
@@ -734,6 +753,73 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         int sp = splits_for(L.wo, 16, EPI_PARTIAL);
         if ((rc = launch_gemm_wide(s, L.wo, (const uint4*)w.xf_b, w.xfb, w.partial, pstride, w.vp, sp, EPI_PARTIAL, c->hidden, c->hidden)))
             return rc;
+        if (L.n_experts) {
+            // routed experts over the 64 rows: the router and the expert matmuls read the 16-row kernels' fragment
+            // layout; the router runs block by block (its matrix is small), its ranking as one launch of four
+            // workgroups; then every expert is multiplied once against all of the pass's rows that chose it
+            const NormBlocks nb4{nb.x, nb.partial, nb.frag, 0};
+            if ((rc = launch_addnorm(s, w.x, w.partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr, L.bo,
+                                     nullptr, 0, WIDE_B, &nb4)))
+                return rc;
+            const int rsp = splits_for(L.router, 16, EPI_PARTIAL);
+            for (int b = 0; b < WIDE_B; b++)
+                if ((rc = launch_gemm(s, L.router, (const uint4*)(w.xf_a + (size_t)b * w.xfb), w.partial + (size_t)b * c->partial_floats,
+                                      w.vp + b, 16, rsp, EPI_PARTIAL, L.n_experts, L.n_experts)))
+                    return rc;
+            MoeRouteArgs ra{};
+            ra.logits = w.partial;
+            ra.splits = rsp;
+            ra.ld = L.n_experts;
+            ra.n_experts = L.n_experts;
+            ra.top_k = L.top_k;
+            ra.m = 16;
+            ra.weights = w.route_w;
+            ra.selected = w.route_sel;
+            ra.bias = L.router_bias;
+            ra.forced = nullptr;
+            ra.blocks = WIDE_B;
+            ra.logits_block_stride = (long)c->partial_floats;
+            if ((rc = launch_route(s, ra)) || (rc = launch_moe_groups(s, w.route_sel, 16 * WIDE_B, L.top_k, L.n_experts, w.groups))) return rc;
+            MoeGemmArgs g1{};
+            g1.w = L.gate_up.tiles;
+            g1.tiles_per_expert = c->ffn / 32;
+            g1.kchunks = L.gate_up.kchunks;
+            g1.k = c->hidden;
+            g1.rows = 16 * WIDE_B;
+            g1.xfrag = w.xf_a;
+            g1.x_stride = 0;
+            g1.x_block_stride = w.xfb;
+            g1.out = w.frag_e;
+            g1.out_stride = WIDE_B * w.frag_e_sub;
+            g1.sub_stride = w.frag_e_sub;
+            g1.n_out = c->ffn;
+            g1.selected = w.route_sel;
+            g1.top_k = L.top_k;
+            g1.bias = L.be_gate;
+            g1.bias2 = L.be_up;
+            g1.alpha = c->act_alpha;
+            g1.limit = c->act_limit;
+            g1.groups = w.groups;
+            g1.n_experts = L.n_experts;
+            MoeGemmArgs g2 = g1;
+            g2.bias = L.be_down;
+            g2.bias2 = nullptr;
+            g2.w = L.down.tiles;
+            g2.tiles_per_expert = c->hidden / 64;
+            g2.kchunks = L.down.kchunks;
+            g2.k = c->ffn;
+            g2.xfrag = w.frag_e;
+            g2.x_stride = WIDE_B * w.frag_e_sub;
+            g2.out = w.moe_out;
+            g2.out_stride = 0;
+            g2.out_block_stride = (size_t)moe_block;
+            g2.n_out = c->hidden;
+            if ((rc = launch_moe_wide_gate_up(s, L.gate_up.fmt, g1)) || (rc = launch_moe_wide_down(s, L.down.fmt, g2))) return rc;
+            prev_partial = w.moe_out;
+            prev_splits = L.top_k;
+            prev_weights = w.route_w;
+            continue;
+        }
         if ((rc = launch_addnorm(s, w.x, w.partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr, L.bo, nullptr,
                                  0, WIDE_B, &nb)))
             return rc;
@@ -746,8 +832,8 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
     // headless: nobody reads these rows' logits, and the last layer's sums are added only for a drafter head,
     // which reads the finished rows (64 consecutive rows of w.x)
     if (c->mtp_head)
-        return launch_addnorm(s, w.x, w.partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr,
-                              nullptr, nullptr, 0, WIDE_B, &nb);
+        return launch_addnorm(s, w.x, prev_partial, prev_splits, c->hidden, c->final_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, prev_weights,
+                              nullptr, nullptr, 0, WIDE_B, prev_weights ? &nb_moe : &nb);
     return TSV_OK;
 }
 
@@ -1239,7 +1325,9 @@ int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* 
     // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
     c->wide.ok = c->rewind_budget == INT64_MAX;
     for (const LayerW& L : c->layers)
-        if (L.n_experts || L.v_only.tiles || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) ||
+        if (L.n_experts) {  // routed layers: the attention projections as below, the experts in any format, fp16 activations
+            if (c->moe_fp4_terms || L.v_only.tiles || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt)) c->wide.ok = false;
+        } else if (L.v_only.tiles || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) ||
             !wide_fmt(L.gate_up.fmt) || !wide_fmt(L.down.fmt))
             c->wide.ok = false;
     if (const char* e = getenv("TSV_WIDE_PREFILL")) c->wide.ok = c->wide.ok && e[0] != '0';
@@ -1402,7 +1490,7 @@ int tsv::prefill_passes(tsv_ctx* c, const int32_t* ids, int64_t n, int64_t pos0,
     for (int64_t i = 0; i < n;) {
         // 64 rows at a time while that many remain and nobody wants their logits
         // (with a drafter head the last pass is a sixteen-row one: the first draft step reads its rows)
-        if (c->wide.ok && !c->profile && n - i >= wide_rows && (i + wide_rows < n || (!logits && !head))) {
+        if (c->wide.ok && !c->profile && !c->route_forced_set && n - i >= wide_rows && (i + wide_rows < n || (!logits && !head))) {
             if (int rc = enqueue_wide_prefill(c, ids + i, pos0 + i)) return rc;
             if (head) {
                 for (int b = 0; b < WIDE_B; b++) {

@@ -127,6 +127,7 @@ extern "C" int32_t tsv_force_route(tsv_ctx* c, const int32_t* sel, int32_t n_lay
     }
     const size_t bytes = (size_t)c->n_layers * 16 * 8 * 4;
     TSV_HIP(hipStreamSynchronize(c->stream));
+    c->route_forced_set = sel != nullptr;
     if (sel) {
         TSV_HIP(hipMemcpy(c->route_forced, sel, bytes, hipMemcpyHostToDevice));
     } else {

@@ -191,6 +191,13 @@ struct MoeGroup {
     int32_t expert, cnt;
     int32_t rows[16], slots[16];
 };
+// Prompt passes of 64 rows: the members of every expert, listed once per layer (k_moe_groups) -- the rows that chose
+// it in pair order (row-major, then slot) and the slot it has in each.
+constexpr int MOE_WIDE_ROWS = 64;
+struct MoeGroupW {
+    int32_t expert, cnt;
+    int32_t rows[MOE_WIDE_ROWS], slots[MOE_WIDE_ROWS];
+};
 struct MoeRouteArgs {
     const float* logits;  // the router matmul's split-K partial sums: [splits][16][ld]
     int splits, ld;
@@ -203,6 +210,10 @@ struct MoeRouteArgs {
     // given, the weights still the softmax of the row's own logits over them); a row whose first
     // entry is negative routes freely
     const int32_t* forced;
+    // a prompt pass of several 16-row blocks (one workgroup each): floats between the blocks' logits; weights and
+    // selections of block b follow those of block b - 1; no forced routing
+    int blocks;
+    long logits_block_stride;
 };
 // The group of pair gi (row gi / k, slot gi % k) from the rows' selections, by one whole wave (lane = threadIdx.x
 // < 64) into *g: the expert, the rows that chose it in pair order with the slot it has in each, and cnt != 0 only
@@ -279,10 +290,22 @@ struct MoeGemmArgs {
     const float* bias;
     const float* bias2;
     float alpha, limit;    // alpha > 0: clamped SwiGLU (moe_gguf.metal:528-556) instead of silu(g) * u
+    // 64-row prompt passes (launch_moe_wide_*): one group per expert, listed in `groups`; a row r of the pass sits in
+    // block r / 16 of the activation fragments and of the down outputs, member b of a group in sub-buffer b / 16 of
+    // the group's own fragments
+    const MoeGroupW* groups;
+    int n_experts;
+    size_t x_block_stride;    // gate/up: bytes between the blocks' activation fragments
+    size_t sub_stride;        // bytes between the 16-member sub-buffers of a group's fragments
+    size_t out_block_stride;  // down: floats between the blocks' [8 slots][16][n_out] outputs
 };
 int launch_route(hipStream_t s, const MoeRouteArgs& a);
 int launch_moe_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
 int launch_moe_down(hipStream_t s, int fmt, const MoeGemmArgs& a, int n_groups);
+// the same two matmuls over the 64 rows of a prompt pass, and the listing of the experts' members before them
+int launch_moe_groups(hipStream_t s, const int32_t* selected, int rows, int top_k, int n_experts, MoeGroupW* groups);
+int launch_moe_wide_gate_up(hipStream_t s, int fmt, const MoeGemmArgs& a);
+int launch_moe_wide_down(hipStream_t s, int fmt, const MoeGemmArgs& a);
 // the same two matmuls on v_mfma_scale_f32_16x16x128_f8f6f4 (moe_fp4.hip)
 int launch_moe_fp4_gate_up(hipStream_t s, const MoeGemmArgs& a, int n_groups);
 int launch_moe_fp4_down(hipStream_t s, const MoeGemmArgs& a, int n_groups);
@@ -321,6 +344,10 @@ struct RopeKvArgs {
     uint16_t* vc;   // [nkv][max_ctx/16][hd/16][64][4]
     int nq, nkv, hd, max_ctx;
     const VerifyParams* vp;
+    // a prompt pass: `blocks` 16-row blocks (0 or 1: one), block b with parameters vp[b], partial sums qkv_block_stride
+    // floats further on and its sixteen q rows behind block b - 1's
+    int blocks;
+    long qkv_block_stride;
 };
 int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m);
 
