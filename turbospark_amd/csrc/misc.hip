@@ -222,6 +222,11 @@ __global__ __launch_bounds__(1024) void k_addnorm(float* __restrict__ x, const f
         sum += __shfl_xor(sum, 2);
         sum += __shfl_xor(sum, 4);
         if ((i & 7) == 0) sums[xsum_index(i >> 3, m)] = sum;
+        if (nb.frag2) {  // the same fragments once more, in the other of the two layouts (sums included)
+            _Float16* x2 = (_Float16*)((char*)nb.frag2 + (long)blockIdx.y * nb.frag);
+            *(half4*)(x2 + (nb.frag16 ? frag_index(4 * i, m) : frag16_index(4 * i, m))) = h;
+            if ((i & 7) == 0) ((float*)((char*)x2 + xfrag_sum_offset(hidden)))[xsum_index(i >> 3, m)] = sum;
+        }
         if (x8_terms) {
             // the same row as block-scaled fp8 terms, from the unrounded values; the eight threads of a
             // 32-element block are neighbours in one wave (hidden is a multiple of 32)

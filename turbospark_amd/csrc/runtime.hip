@@ -644,10 +644,10 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         if ((rc = launch_embed(s, c->embed_raw, c->embed_dtype, c->hidden, w.x + (size_t)b * 16 * c->hidden, w.vp + b, 16, c->freqs,
                                c->rope_mscale, half, w.rope_cs + (size_t)b * 16 * half)))
             return rc;
-    const NormBlocks nb{(long)16 * c->hidden, (long)c->partial_floats, (long)w.xfb, 1};
+    const NormBlocks nb{(long)16 * c->hidden, (long)c->partial_floats, (long)w.xfb, 1, nullptr};
     // after a routed layer the partial sums are the blocks' per-slot expert outputs and come with the rows' factors
     const long moe_block = (long)8 * 16 * c->hidden;
-    const NormBlocks nb_moe{nb.x, moe_block, nb.frag, 1};
+    const NormBlocks nb_moe{nb.x, moe_block, nb.frag, 1, nullptr};
     const size_t pstride = c->partial_floats * 4;
     const int qkv_n = (c->nq + 2 * c->nkv) * c->hd;
     int prev_splits = 0;
@@ -757,15 +757,24 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
             // routed experts over the 64 rows: the router and the expert matmuls read the 16-row kernels' fragment
             // layout; the router runs block by block (its matrix is small), its ranking as one launch of four
             // workgroups; then every expert is multiplied once against all of the pass's rows that chose it
-            const NormBlocks nb4{nb.x, nb.partial, nb.frag, 0};
+            // (where the router's format has a 64-row matmul the norm leaves its rows in that kernel's layout as well,
+            //  in the buffer the dense FFN would use, and the router is one launch; else one launch per block)
+            const bool wide_router = wide_fmt(L.router.fmt);
+            const NormBlocks nb4{nb.x, nb.partial, nb.frag, 0, wide_router ? (void*)w.xf_c : nullptr};
             if ((rc = launch_addnorm(s, w.x, w.partial, sp, c->hidden, L.ffn_norm, c->eps, c->hidden, (uint4*)w.xf_a, 16, nullptr, L.bo,
                                      nullptr, 0, WIDE_B, &nb4)))
                 return rc;
             const int rsp = splits_for(L.router, 16, EPI_PARTIAL);
-            for (int b = 0; b < WIDE_B; b++)
-                if ((rc = launch_gemm(s, L.router, (const uint4*)(w.xf_a + (size_t)b * w.xfb), w.partial + (size_t)b * c->partial_floats,
-                                      w.vp + b, 16, rsp, EPI_PARTIAL, L.n_experts, L.n_experts)))
+            if (wide_router) {
+                if ((rc = launch_gemm_wide(s, L.router, (const uint4*)w.xf_c, w.xfb, w.partial, pstride, w.vp, rsp, EPI_PARTIAL, L.n_experts,
+                                           L.n_experts)))
                     return rc;
+            } else {
+                for (int b = 0; b < WIDE_B; b++)
+                    if ((rc = launch_gemm(s, L.router, (const uint4*)(w.xf_a + (size_t)b * w.xfb), w.partial + (size_t)b * c->partial_floats,
+                                          w.vp + b, 16, rsp, EPI_PARTIAL, L.n_experts, L.n_experts)))
+                        return rc;
+            }
             MoeRouteArgs ra{};
             ra.logits = w.partial;
             ra.splits = rsp;

@@ -317,6 +317,7 @@ int launch_embed(hipStream_t s, const uint8_t* raw, int dtype, int hidden, float
 struct NormBlocks {
     long x, partial, frag;
     int frag16;  // write the fragments in the prompt kernel's layout (frag16_index)
+    void* frag2;  // nullable: a second fragment buffer (blocks `frag` bytes apart as well) that takes the other layout
 };
 // weights: NULL, or [16][8] factors of the partials (row m, partial s): the routed experts' sum
 int launch_addnorm(hipStream_t s, float* x, const float* partial, int splits, int ldp, const float* w,
