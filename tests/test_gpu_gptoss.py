@@ -91,12 +91,14 @@ def test_gptoss_sampled_round_on_the_device():
         gpu.rollback(ts.ffi.Point(base))
 
 
-def test_a_rewind_deeper_than_the_window_is_safe_in_the_linear_layout():
+def test_a_rewind_deeper_than_the_window_is_safe_in_the_linear_layout(monkeypatch):
     """`KvCacheManager::max_safe_rewind` (crates/gpu/src/kv_cache_rewind.rs:26-35) bounds a rollback by
     the ring's slack; without `ring` the windowed layers store position p at slot p, so it is unbounded: after
     rolling back 40 rows (the window is 24) the continuation equals, by bits, a run that never went
-    further."""
+    further.  (Both runs in 16-row passes: a 64-row pass sums in another order, so its rows differ from a
+    16-row pass's in the last bits and the comparison by bits would measure that instead.)"""
     import turbospark_amd as ts
+    monkeypatch.setenv("TSV_WIDE_PREFILL", "0")
     cfg, w, gpu, cpu = gc.build_pair("gptoss_small", max_context=128)
     assert gpu.max_safe_rewind() == 2 ** 63 - 1
     prompt = _prompt(80, cfg["vocab"], 5)
@@ -119,7 +121,14 @@ def _ring_pair(name, max_context, n_layers=None, seed=1234, **over):
     if n_layers:
         cfg["n_layers"] = n_layers
     w = synth.make_weights(cfg, seed=seed, n_layers=n_layers)
-    linear = ts.HipVerifier(cfg, w)
+    # (ring layers take their prompts in 16-row passes; the linear handle is held to them too, so that "equal by
+    #  bits" compares the two layouts and not the summation orders of 64-row and 16-row passes)
+    import os
+    os.environ["TSV_WIDE_PREFILL"] = "0"
+    try:
+        linear = ts.HipVerifier(cfg, w)
+    finally:
+        del os.environ["TSV_WIDE_PREFILL"]
     ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
     return cfg, linear, ts.HipVerifier(cfg, ringed)
 

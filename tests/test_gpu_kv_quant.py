@@ -247,7 +247,13 @@ def test_rings_on_a_quantized_handle_equal_the_linear_layout_by_bits():
     cfg = dict(synth.CONFIGS["gptoss_small"], max_context=400, n_layers=4)
     w = synth.make_weights(cfg, seed=21)
     ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
-    lin, ring = ts.HipVerifier(cfg, w, kv_bits=(4, 4)), ts.HipVerifier(cfg, ringed, kv_bits=(4, 4))
+    # (both handles in 16-row prompt passes, the only kind a ring layer takes: the comparison is of the layouts)
+    import os
+    os.environ["TSV_WIDE_PREFILL"] = "0"
+    try:
+        lin, ring = ts.HipVerifier(cfg, w, kv_bits=(4, 4)), ts.HipVerifier(cfg, ringed, kv_bits=(4, 4))
+    finally:
+        del os.environ["TSV_WIDE_PREFILL"]
     assert lin.max_safe_rewind() == 2 ** 63 - 1 and ring.max_safe_rewind() == 64 - 24
     V = cfg["vocab"]
     rng = np.random.default_rng(8)

@@ -72,10 +72,12 @@ def test_the_heads_logits_match_the_oracle_through_priming_steps_chained_steps_a
     assert max(errs) <= tol
 
 
-@pytest.mark.parametrize("n", [37, 171])   # the longer prompt goes through 64-row passes, which prime the head too
-def test_priming_by_the_prefill_equals_priming_token_by_token(n):
-    cfg, gpu_a, head_a = _build("xcd_q4_k", ctx=200, oracle=False)
-    _, gpu_b, head_b = _build("xcd_q4_k", ctx=200, oracle=False)
+# the longer prompts go through 64-row passes, which prime the head too (Q8_0: the rotation as a kernel of its own
+# under TSV_ROPE_FUSED=0 elsewhere, here the epilogue; routed layers: the experts' members over 64 rows)
+@pytest.mark.parametrize("name,n", [("xcd_q4_k", 37), ("xcd_q4_k", 171), ("xcd_q8_0", 171), ("moe_small", 171)])
+def test_priming_by_the_prefill_equals_priming_token_by_token(name, n):
+    cfg, gpu_a, head_a = _build(name, ctx=200, oracle=False)
+    _, gpu_b, head_b = _build(name, ctx=200, oracle=False)
     V = cfg["vocab"]
     prompt = np.random.default_rng(6).integers(0, V, n).astype(np.int32)
     la = head_a.prefill_chunk(prompt[:20], 0, next_token=int(prompt[20]))   # two chunks, the first names its next token
