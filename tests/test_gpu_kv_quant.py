@@ -432,7 +432,8 @@ def test_gptoss_120b_shape_with_the_full_layers_rows_quantized():
     assert gap <= 2e-2
 
 
-@pytest.mark.parametrize("name,kv_bits,n_prompt", [("small_q4_k", (4, 4), 150), ("xcd_q4_k", (3, 4), 129), ("small_q4_k", (2, 2), 64)])
+@pytest.mark.parametrize("name,kv_bits,n_prompt", [("small_q4_k", (4, 4), 150), ("xcd_q4_k", (3, 4), 129), ("small_q4_k", (2, 2), 64),
+                                                   ("xcd_q8_0", (4, 4), 150), ("moe_small", (4, 4), 150)])
 def test_prompt_passes_of_64_rows_over_quantized_rows(name, kv_bits, n_prompt):
     """crates/runtime/src/producer.rs:122-150 with --kv-bits: all 64 rows of a pass are quantized before any of its four
     blocks attends, so every row sees what sixteen-row passes would show it.  The two paths multiply the same integers
