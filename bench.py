@@ -330,7 +330,7 @@ def main():
     ap.add_argument("--prefill-bench", type=int, default=0, metavar="TOKENS",
                     help="time tsv_prefill over a prompt of this many tokens (after one untimed run of the same), print one "
                          "JSON line and exit")
-    ap.add_argument("--weights-dtype", default=None, choices=["q4_k", "q8_0", "bf16"],
+    ap.add_argument("--weights-dtype", default=None, choices=["q4_k", "q8_0", "bf16", "q4_k_m", "q5_k_m"],
                     help="--prefill-bench: the dense workload's shape with its matrices in this storage type")
     ap.add_argument("--loop-bench", type=int, default=0, metavar="NEW_TOKENS",
                     help="end to end instead of one step: generate this many tokens with the library's loop and its "
@@ -392,7 +392,16 @@ def main():
     if args.weights_dtype:
         if not args.prefill_bench or cfg.get("n_experts"):
             sys.exit("bench.py: --weights-dtype goes with --prefill-bench at a dense workload")
-        cfg["dtype"] = {"q4_k": ts.ffi.Q4_K, "q8_0": ts.ffi.Q8_0, "bf16": ts.ffi.BF16}[args.weights_dtype]
+        cfg["dtype"] = {"q4_k": ts.ffi.Q4_K, "q8_0": ts.ffi.Q8_0, "bf16": ts.ffi.BF16, "q4_k_m": ts.ffi.Q4_K,
+                        "q5_k_m": ts.ffi.Q5_K}[args.weights_dtype]
+        if args.weights_dtype.endswith("_m"):
+            # the tensor mix of a *_K_M file: value and down projections in Q6_K in the first and last eighth of the
+            # layers and every third layer between, and the output head
+            n = cfg["n_layers"]
+            more = [i for i in range(n) if i < n // 8 or i >= 7 * n // 8 or (i - n // 8) % 3 == 2]
+            cfg["overrides"] = {"lm_head": ts.ffi.Q6_K}
+            for i in more:
+                cfg["overrides"][(i, "wv")] = cfg["overrides"][(i, "w_down")] = ts.ffi.Q6_K
     if args.loop_bench and args.weak_layers != 1.0:
         cfg["weak_layers"] = args.weak_layers
     if args.loop_bench and args.embed_scale != 1.0:
@@ -415,7 +424,7 @@ def main():
         t0 = time.perf_counter()
         eng.prefill(prompt, 0, want_logits=False)     # returns after the stream has drained
         dt = time.perf_counter() - t0
-        wide = cfg["dtype"] in (ts.ffi.Q4_K, ts.ffi.Q8_0, ts.ffi.BF16) and not (cfg.get("n_experts") and os.environ.get("TSV_MOE_FP4"))
+        wide = cfg["dtype"] in (ts.ffi.Q4_K, ts.ffi.Q5_K, ts.ffi.Q8_0, ts.ffi.BF16) and not (cfg.get("n_experts") and os.environ.get("TSV_MOE_FP4"))
         rows = 64 if wide and os.environ.get("TSV_WIDE_PREFILL") != "0" else 16
         print(json.dumps({"metric": "prefill tokens/s", "value": round(n / dt, 1), "unit": "tokens/s", "n_gpus": 1,
                           "higher_is_better": True, "dtype": "f16", "data": "synthetic", "seconds": round(dt, 4),

@@ -22,7 +22,8 @@ def _engine(cfg, weights, wide):
 
 
 @pytest.mark.parametrize("name,n_prompt", [("small_q4_k", 150), ("small_q4_k", 64), ("xcd_q4_k", 200), ("small_q4_k", 129),
-                                           ("tiny_q8_0", 150), ("xcd_q8_0", 200), ("tiny_q8_0", 64)])
+                                           ("tiny_q8_0", 150), ("xcd_q8_0", 200), ("tiny_q8_0", 64),
+                                           ("small_q4_k_m", 150), ("small_q5_k_m", 150)])   # the K-quant mixes: Q6_K value / down matrices
 def test_a_prompt_fed_in_blocks_of_64_fills_the_cache_the_oracle_fills(name, n_prompt):
     from turbospark_amd import synth
     from oracle import binding as ob

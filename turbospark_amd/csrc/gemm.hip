@@ -584,8 +584,9 @@ __global__ __launch_bounds__(512) void k_gemm16(GemmArgs a) {
 }
 
 // ------------------------------------------------------------------------------- prompt blocks of 64 rows
-// A prompt pass of BLOCKS x 16 rows over Q4_K weights (crates/runtime/src/producer.rs:122-150: the
-// chunked prefill runner feeds the prompt in blocks; families/llama/prefill.rs).  One workgroup per
+// A prompt pass of BLOCKS x 16 rows, here over Q4_K / Q5_K weights and further down over Q8_0, bf16 and Q6_K
+// (crates/runtime/src/producer.rs:122-150: the chunked prefill runner feeds the prompt in blocks;
+// families/llama/prefill.rs).  One workgroup per
 // (tile, K slice), one wave per block of sixteen rows.  A tile chunk is unpacked ONCE per workgroup:
 // wave w turns row block w of the chunk (sixteen weight rows x 256 K) into the B operands of
 // v_mfma_f32_16x16x32_f16 and leaves them in LDS, in the lane order the 16-row kernel builds them in
@@ -617,6 +618,7 @@ constexpr int WIDE_BUF_BYTES = WIDE_B_BYTES + 4096;  // + [row block][64 lanes] 
 struct WideW {  // what the unpacking wave holds of one chunk: its row block's codes and scale header
     u32x2 q[4];
     u32x4 h;
+    u32x2 qh;  // Q5_K: the fifth bits of the lane's eight elements (bit 2 p / 2 p + 1 for pair p's low / high nibbles)
 };
 struct WideX {  // a block's activations of one chunk: the lane's A operand of every sub-block, and two sums
     u32x4 v[8];
@@ -625,6 +627,7 @@ struct WideX {  // a block's activations of one chunk: the lane's A operand of e
 
 // (the loads of a chunk stay where they are written, scheduling fences on both sides: left alone, the
 // scheduler sinks them to their first use, one chunk later, and nothing is in flight ahead of the math)
+template <bool Q5 = false>
 __device__ __forceinline__ void wide_load_w(WideW& w, const uint8_t* tile_chunk, int rb, int lane) {
     const int r = lane & 15, kg = lane >> 4;
     const uint8_t* wp = tile_chunk + ((kg >> 1) * 64 + r) * 16 + (kg & 1) * 8;
@@ -632,6 +635,8 @@ __device__ __forceinline__ void wide_load_w(WideW& w, const uint8_t* tile_chunk,
 #pragma unroll
     for (int p = 0; p < 4; p++) w.q[p] = __builtin_nontemporal_load((const u32x2*)(wp + (2 * p * 64 + 16 * rb) * 16));
     w.h = __builtin_nontemporal_load((const u32x4*)(tile_chunk + 8192 + (16 * rb + r) * 16));
+    if (Q5) w.qh = __builtin_nontemporal_load((const u32x2*)(wp + (9 * 64 + 16 * rb) * 16));  // units 9 and 10: byte l serves element l
+    else w.qh = u32x2{0u, 0u};
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -647,7 +652,10 @@ __device__ __forceinline__ void wide_load_x(WideX& x, const GemmArgs& a, int c, 
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// Row block `rb` of a chunk into LDS buffer `buf`.
+// Row block `rb` of a chunk into LDS buffer `buf`.  Q5_K (q5_k.rs:47-96): the fifth bit of a code is OR-ed into the
+// offset integer before the fma -- bit 4 of 1024 + q, bit 8 of the 1/16-ulp form of 64 + q -- and sc_j * q stays an
+// exact fp16 integer (at most 63 * 31).
+template <bool Q5 = false>
 __device__ __forceinline__ void wide_unpack(const WideW& w, const Consts& k, uint8_t* buf, int rb, int lane) {
     typedef _Float16 half2v __attribute__((ext_vector_type(2)));
     const int kg = lane >> 4;
@@ -674,11 +682,19 @@ __device__ __forceinline__ void wide_unpack(const WideW& w, const Consts& k, uin
         const half2v off_lo = sc_lo * m1024, off_hi = sc_hi * m64;
         const uint32_t w0 = w.q[p].x, w1 = w.q[p].x >> 8, w2 = w.q[p].y, w3 = w.q[p].y >> 8;
         const uint32_t wv[4] = {w0, w1, w2, w3};
+        const uint32_t hv[4] = {w.qh.x, w.qh.x >> 8, w.qh.y, w.qh.y >> 8};
         u32x4 blo, bhi;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const half2v lo = __builtin_bit_cast(half2v, and_or(wv[i], 0x000F000Fu, k.k6400));  // 1024 + q
-            const half2v hi = __builtin_bit_cast(half2v, and_or(wv[i], 0x00F000F0u, k.k5400));  // 64 + q
+            uint32_t lo_bits = and_or(wv[i], 0x000F000Fu, k.k6400), hi_bits = and_or(wv[i], 0x00F000F0u, k.k5400);
+            if (Q5) {
+                const int slo = 4 - 2 * p;
+                const uint32_t l5 = slo >= 0 ? hv[i] << (slo >= 0 ? slo : 0) : hv[i] >> (slo < 0 ? -slo : 0);
+                lo_bits = and_or(l5, 0x00100010u, lo_bits);
+                hi_bits = and_or(hv[i] << (7 - 2 * p), 0x01000100u, hi_bits);
+            }
+            const half2v lo = __builtin_bit_cast(half2v, lo_bits);  // 1024 + q
+            const half2v hi = __builtin_bit_cast(half2v, hi_bits);  // 64 + q
             blo[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(lo, sc_lo, off_lo));
             bhi[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(hi, sc_hi, off_hi));
         }
@@ -732,8 +748,9 @@ __device__ __forceinline__ void wide_compute(const WideX& x, const uint8_t* buf,
     }
 }
 
-template <int EPI>
+template <int EPI, bool Q5 = false>
 __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa) {
+    constexpr int TILE = Q5 ? Q5K::TILE_BYTES : Q4K::TILE_BYTES;
     extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;  // wave = this wave's block = the row block it unpacks
     GemmArgs a = wa.g;
@@ -747,7 +764,7 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa)
     }
     const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
     const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
-    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q4K::TILE_BYTES;
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * TILE;
     Consts k;
     k.k6400 = 0x64006400u;
     k.k5400 = 0x54005400u;
@@ -768,25 +785,25 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa)
     uint8_t* const buf0 = wide_lds;
     uint8_t* const buf1 = wide_lds + WIDE_BUF_BYTES;
     const int last = s1 - 1;
-    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * Q4K::TILE_BYTES; };
-    wide_load_w(w[0], tile_at(s0), wave, lane);
+    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * TILE; };
+    wide_load_w<Q5>(w[0], tile_at(s0), wave, lane);
     wide_load_x(x[0], a, s0, lane);
-    wide_load_w(w[1], tile_at(s0 + 1), wave, lane);
+    wide_load_w<Q5>(w[1], tile_at(s0 + 1), wave, lane);
     int c = s0;
     for (; c + 2 <= s1; c += 2) {
-        wide_unpack(w[0], k, buf0, wave, lane);
-        wide_load_w(w[0], tile_at(c + 2), wave, lane);
+        wide_unpack<Q5>(w[0], k, buf0, wave, lane);
+        wide_load_w<Q5>(w[0], tile_at(c + 2), wave, lane);
         wide_load_x(x[1], a, min(c + 1, last), lane);
         __syncthreads();
         wide_compute(x[0], buf0, acc, lane);
-        wide_unpack(w[1], k, buf1, wave, lane);
-        wide_load_w(w[1], tile_at(c + 3), wave, lane);
+        wide_unpack<Q5>(w[1], k, buf1, wave, lane);
+        wide_load_w<Q5>(w[1], tile_at(c + 3), wave, lane);
         wide_load_x(x[0], a, min(c + 2, last), lane);
         __syncthreads();
         wide_compute(x[1], buf1, acc, lane);
     }
     if (c < s1) {
-        wide_unpack(w[0], k, buf0, wave, lane);
+        wide_unpack<Q5>(w[0], k, buf0, wave, lane);
         __syncthreads();
         wide_compute(x[0], buf0, acc, lane);
     }
@@ -1070,6 +1087,187 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_bf16(GemmWideArg
     }
 }
 
+// ---- the same pass over Q6_K weights ---------------------------------------------------------
+// value = d * sc_j * (level - 32) with an int8 scale per 16 elements (crates/compute/src/quant_gguf/q6_k.rs:44-88).
+// level - 32 is exact in fp16, but its product with the scale (up to 32 * 128) is not, so the scale goes in as
+// sc = 16 a + b (a = sc >> 4 in -8..7, b = sc & 15): two operands (level - 32) * a and (level - 32) * b, both exact
+// integers below 512, two chains of matrix instructions, and d * (16 * hi + lo) per 128 K in fp32.  A lane's eight
+// K of a 32-K step lie inside one 16-element sub-block, so its scale is one byte.  The loop walks HALF chunks
+// (128 K, two 64-K pairs): the two operands of a whole chunk would not leave room for two workgroups' buffers on a
+// compute unit.  Lane (r, kg) finds its eight levels of step (pair p, half h) in word kg of unit 3 p + h (low
+// nibbles: k0 k1 of the first 4-K step, k0 k1 of the second, then k2 k3, k2 k3) and in word 2 h + kg / 2 of unit
+// 3 p + 2 (high bit pairs: extraction e = 4 (kg & 1) + 2 t + ab of 4-K step t in bits 2 e.. and 16 + 2 e..).
+constexpr int WIDE6_B_BYTES = 32768;                   // [row block][32-K step of the half chunk][a / b][64 lanes][16 B]
+constexpr int WIDE6_BUF_BYTES = WIDE6_B_BYTES + 1024;  // + [row block][64 lanes] d
+
+struct WideW6 {
+    uint32_t lo[2][2], hi[2][2];  // [pair of the half][h]
+    u32x2 sc;                     // the half chunk's eight scales
+    uint32_t d;
+};
+struct WideX6 {
+    u32x4 v[4];
+};
+
+__device__ __forceinline__ void wide6_load_w(WideW6& w, const uint8_t* tile_chunk, int half, int rb, int lane) {
+    const int r = lane & 15, kg = lane >> 4, row = 16 * rb + r;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int pp = 0; pp < 2; pp++) {
+        const int p = 2 * half + pp;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            w.lo[pp][h] = __builtin_nontemporal_load((const uint32_t*)(tile_chunk + ((3 * p + h) * 64 + row) * 16 + 4 * kg));
+            w.hi[pp][h] = __builtin_nontemporal_load((const uint32_t*)(tile_chunk + ((3 * p + 2) * 64 + row) * 16 + 4 * (2 * h + (kg >> 1))));
+        }
+    }
+    w.sc = __builtin_nontemporal_load((const u32x2*)(tile_chunk + 12288 + row * 16 + 8 * half));
+    w.d = __builtin_nontemporal_load((const uint32_t*)(tile_chunk + 13312 + row * 4));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void wide6_load_x(WideX6& x, const GemmArgs& a, int hc, int lane) {
+    const u32x4* xp = (const u32x4*)a.xfrag + (size_t)hc * 256 + lane;  // frag16_index: four 32-K steps per half chunk
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) x.v[j] = xp[j * 64];
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void wide6_unpack(const WideW6& w, const Consts& k, uint8_t* buf, int rb, int lane) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const int kg = lane >> 4;
+    const half2v off = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+    *(float*)(buf + WIDE6_B_BYTES + (rb * 64 + lane) * 4) = h2f_lo(w.d);
+#pragma unroll
+    for (int pp = 0; pp < 2; pp++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int sj = 4 * pp + 2 * h + (kg >> 1);  // the lane's sub-block among the half chunk's eight
+            const uint32_t scw = sj < 4 ? w.sc.x : w.sc.y;
+            const int sc8 = (int)(scw << (24 - 8 * (sj & 3))) >> 24;
+            const _Float16 fa = (_Float16)(float)(sc8 >> 4), fb = (_Float16)(float)(sc8 & 15);
+            const half2v a2 = {fa, fa}, b2 = {fb, fb};
+            const uint32_t nw = w.lo[pp][h], H = w.hi[pp][h];
+            u32x4 ba, bb;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int ab = 0; ab < 2; ab++) {
+                    const int e = 4 * (kg & 1) + 2 * t + ab;
+                    const uint32_t lo = and_or(nw >> (8 * t + 4 * ab), 0x000F000Fu, k.k6400);
+                    const uint32_t v = lo | (((H >> (2 * e)) << 4) & 0x00300030u);  // 1024 + level, twice
+                    const half2v lv = __builtin_bit_cast(half2v, v) + off;             // level - 32
+                    ba[2 * t + ab] = __builtin_bit_cast(uint32_t, lv * a2);
+                    bb[2 * t + ab] = __builtin_bit_cast(uint32_t, lv * b2);
+                }
+            const int jj = 2 * pp + h;
+            *(u32x4*)(buf + (((rb * 4 + jj) * 2 + 0) * 64 + lane) * 16) = ba;
+            *(u32x4*)(buf + (((rb * 4 + jj) * 2 + 1) * 64 + lane) * 16) = bb;
+        }
+}
+
+__device__ __forceinline__ void wide6_compute(const WideX6& x, const uint8_t* buf, float4v (&acc)[4], int lane) {
+    const float4v zero = {0.f, 0.f, 0.f, 0.f};
+    float d[4];
+    float4v thi[4], tlo[4];
+    u32x4 ba[2][4], bb[2][4];
+    auto fetch = [&](int slot, int jj) {
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++) {
+            ba[slot][rb] = *(const u32x4*)(buf + (((rb * 4 + jj) * 2 + 0) * 64 + lane) * 16);
+            bb[slot][rb] = *(const u32x4*)(buf + (((rb * 4 + jj) * 2 + 1) * 64 + lane) * 16);
+        }
+    };
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+        d[rb] = *(const float*)(buf + WIDE6_B_BYTES + (rb * 64 + lane) * 4);
+        thi[rb] = zero;
+        tlo[rb] = zero;
+    }
+    fetch(0, 0);
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) {
+        if (jj < 3) fetch((jj + 1) & 1, jj + 1);
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            thi[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, x.v[jj]), __builtin_bit_cast(half8, ba[jj & 1][rb]),
+                                                             thi[rb], 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++)
+            tlo[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, x.v[jj]), __builtin_bit_cast(half8, bb[jj & 1][rb]),
+                                                             tlo[rb], 0, 0, 0);
+    }
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+        fma4(tlo[rb], 16.0f, thi[rb]);
+        fma4(acc[rb], d[rb], tlo[rb]);
+    }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_q6k(GemmWideArgs wa) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two half-chunk buffers, then the blocks' sub-block sums
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    GemmArgs a = wa.g;
+    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
+    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
+    a.vp = a.vp + wave;
+    if (EPI == EPI_ROPE) {
+        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
+        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
+    }
+    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
+    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q6K::TILE_BYTES;
+    Consts k;
+    k.k6400 = 0x64006400u;
+    k.k5400 = 0;
+    k.k64 = 0;
+    asm volatile("" : "+v"(k.k6400));
+    float4v acc[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int M = a.vp->m;
+    // the chunk loop of k_gemm_wide over half chunks h0 .. h1 - 1 (half chunk hc = chunk hc / 2, half hc % 2)
+    WideW6 w[2];
+    WideX6 x[2];
+    uint8_t* const buf0 = wide_lds;
+    uint8_t* const buf1 = wide_lds + WIDE6_BUF_BYTES;
+    const int h0 = 2 * s0, h1 = 2 * s1, last = h1 - 1;
+    auto load_w = [&](WideW6& ww, int hc) {
+        const int c = min(hc, last);
+        wide6_load_w(ww, wt + (size_t)(c >> 1) * Q6K::TILE_BYTES, c & 1, wave, lane);
+    };
+    load_w(w[0], h0);
+    wide6_load_x(x[0], a, h0, lane);
+    load_w(w[1], h0 + 1);
+    int c = h0;
+    for (; c + 2 <= h1; c += 2) {
+        wide6_unpack(w[0], k, buf0, wave, lane);
+        load_w(w[0], c + 2);
+        wide6_load_x(x[1], a, min(c + 1, last), lane);
+        __syncthreads();
+        wide6_compute(x[0], buf0, acc, lane);
+        wide6_unpack(w[1], k, buf1, wave, lane);
+        load_w(w[1], c + 3);
+        wide6_load_x(x[0], a, min(c + 2, last), lane);
+        __syncthreads();
+        wide6_compute(x[1], buf1, acc, lane);
+    }
+    __syncthreads();  // (the half chunks of a slice come in pairs: nothing is left over)
+    float* ssum = (float*)(wide_lds + 2 * WIDE6_BUF_BYTES) + wave * 32;
+#pragma unroll
+    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
+    if (EPI == EPI_SILU) {
+        __syncthreads();
+        if (lane < 16 && lane < M) {
+            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
+            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
+        }
+    }
+}
+
 // Fewest rows that go to the 16x16x32 form (TSV_GEMM16=0: never; TSV_GEMM16=<n>: from n rows on).
 static int gemm16_min_rows() {
     static const int n = [] {
@@ -1197,11 +1395,11 @@ int gemm_wide_rows() { return 16 * WIDE_BLOCKS; }
 
 // The same matmul over gemm_wide_rows() rows in blocks of sixteen: block b reads its fragments at
 // xfrag + b * x_stride bytes, its parameters at vp + b, and writes at out + b * out_stride bytes
-// (EPI_ROPE: rope->cs and rope->q16 hold all blocks' rows one after the other).  Q4_K, Q8_0 or bf16 weights.
+// (EPI_ROPE: rope->cs and rope->q16 hold all blocks' rows one after the other).  Q4_K, Q5_K, Q6_K, Q8_0 or bf16 weights.
 int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t x_stride, void* out, size_t out_stride,
                      const VerifyParams* vp, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
-    if (w.fmt != FMT_Q4K && w.fmt != FMT_Q80 && w.fmt != FMT_BF16) {
-        set_error("matmul: prompt blocks of 64 rows need Q4_K, Q8_0 or bf16 weights");
+    if (w.fmt != FMT_Q4K && w.fmt != FMT_Q5K && w.fmt != FMT_Q80 && w.fmt != FMT_BF16 && w.fmt != FMT_Q6K) {
+        set_error("matmul: prompt blocks of 64 rows need Q4_K, Q5_K, Q6_K, Q8_0 or bf16 weights");
         return TSV_ERR_UNSUPPORTED;
     }
     GemmWideArgs wa{};
@@ -1209,6 +1407,25 @@ int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t 
     wa.x_stride = x_stride;
     wa.out_stride = out_stride;
     wa.g.out16 = 1;  // what this kernel reads is what it writes for the next one
+    if (w.fmt == FMT_Q6K) {
+        const size_t lds6 = 2 * (size_t)WIDE6_BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
+        const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
+        static bool attr6_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+        if (!attr6_set) {
+            TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide_q6k<EPI_PARTIAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds6));
+            TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide_q6k<EPI_ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds6));
+            TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide_q6k<EPI_SILU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds6));
+            attr6_set = true;
+        }
+        switch (epi) {
+            case EPI_PARTIAL: hipLaunchKernelGGL(k_gemm_wide_q6k<EPI_PARTIAL>, grid, block, lds6, s, wa); break;
+            case EPI_ROPE: hipLaunchKernelGGL(k_gemm_wide_q6k<EPI_ROPE>, grid, block, lds6, s, wa); break;
+            case EPI_SILU: hipLaunchKernelGGL(k_gemm_wide_q6k<EPI_SILU>, grid, block, lds6, s, wa); break;
+            default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
+        }
+        TSV_HIP(hipGetLastError());
+        return TSV_OK;
+    }
     if (w.fmt == FMT_Q80 || w.fmt == FMT_BF16) {
         const bool q80 = w.fmt == FMT_Q80;
         const size_t lds2 = 2 * (size_t)(q80 ? WIDE80_BUF_BYTES : WIDEBF_BUF_BYTES) + WIDE_BLOCKS * 32 * sizeof(float);
@@ -1238,12 +1455,25 @@ int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t 
         TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_PARTIAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_SILU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_PARTIAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_ROPE, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_SILU, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_set = true;
     }
+    const bool q5 = w.fmt == FMT_Q5K;
     switch (epi) {
-        case EPI_PARTIAL: hipLaunchKernelGGL(k_gemm_wide<EPI_PARTIAL>, grid, block, lds, s, wa); break;
-        case EPI_ROPE: hipLaunchKernelGGL(k_gemm_wide<EPI_ROPE>, grid, block, lds, s, wa); break;
-        case EPI_SILU: hipLaunchKernelGGL(k_gemm_wide<EPI_SILU>, grid, block, lds, s, wa); break;
+        case EPI_PARTIAL:
+            if (q5) hipLaunchKernelGGL((k_gemm_wide<EPI_PARTIAL, true>), grid, block, lds, s, wa);
+            else hipLaunchKernelGGL(k_gemm_wide<EPI_PARTIAL>, grid, block, lds, s, wa);
+            break;
+        case EPI_ROPE:
+            if (q5) hipLaunchKernelGGL((k_gemm_wide<EPI_ROPE, true>), grid, block, lds, s, wa);
+            else hipLaunchKernelGGL(k_gemm_wide<EPI_ROPE>, grid, block, lds, s, wa);
+            break;
+        case EPI_SILU:
+            if (q5) hipLaunchKernelGGL((k_gemm_wide<EPI_SILU, true>), grid, block, lds, s, wa);
+            else hipLaunchKernelGGL(k_gemm_wide<EPI_SILU>, grid, block, lds, s, wa);
+            break;
         default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
     }
     TSV_HIP(hipGetLastError());

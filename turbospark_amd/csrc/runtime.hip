@@ -596,12 +596,13 @@ int launch_pass(tsv_ctx* c, int m) {
 // cache stores, attention -- is the 16-row pass's own code on block-strided buffers: block b is
 // rows base + 16 b .. base + 16 b + 15, its attention sees the cache up to its own rows, which the
 // q/k/v projection of the same pass has already stored for every block before any block attends.
-// Only for headless passes (no logits wanted) of dense models whose four matmuls are Q4_K, Q8_0 or bf16
-// (the q/k/v projection with the rotating epilogue, or followed by the rotation kernel block by
-// block), and whose layers are linear caches: a ring layer's slack is 32 rows, fewer than a 64-row
-// pass writes ahead of its first block's window.
+// Only for headless passes (no logits wanted), in any of the storage types the 64-row matmuls read
+// (wide_fmt; the q/k/v projection with the rotating epilogue, or followed by the rotation kernel over
+// the four blocks; routed layers through the experts' member lists), and only where every layer is a
+// linear cache: a ring layer's slack is 32 rows, fewer than a 64-row pass writes ahead of its first
+// block's window.
 constexpr int WIDE_B = 4;
-static bool wide_fmt(int fmt) { return fmt == FMT_Q4K || fmt == FMT_Q80 || fmt == FMT_BF16; }
+static bool wide_fmt(int fmt) { return fmt == FMT_Q4K || fmt == FMT_Q5K || fmt == FMT_Q6K || fmt == FMT_Q80 || fmt == FMT_BF16; }
 
 int wide_prepare(tsv_ctx* c) {
     tsv_ctx::Wide& w = c->wide;
@@ -674,8 +675,18 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
             if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
         } else {
             // the projection's partial sums, then the 16-row pass's own norm / rotation / cache stores over the four blocks
-            const int spq = splits_for(L.qkv, 16, EPI_PARTIAL);
+            int spq = splits_for(L.qkv, 16, EPI_PARTIAL);
+            if (L.v_only.tiles) {  // (the value projection in a storage type of its own: one split count for both pieces)
+                auto fits = [](const TiledW& t, int n) {
+                    const int kslice = (t.kchunks + n - 1) / n;
+                    return (t.kchunks + kslice - 1) / kslice == n;
+                };
+                while (spq > 1 && !(fits(L.qkv, spq) && fits(L.v_only, spq))) spq--;
+            }
             if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, w.partial, pstride, w.vp, spq, EPI_PARTIAL, qkv_n, L.qkv.n_rows)))
+                return rc;
+            if (L.v_only.tiles && (rc = launch_gemm_wide(s, L.v_only, (const uint4*)w.xf_a, w.xfb, w.partial + L.qkv.n_rows, pstride, w.vp, spq,
+                                                         EPI_PARTIAL, qkv_n, L.v_only.n_rows)))
                 return rc;
             {
                 RopeKvArgs ra{};
@@ -1335,9 +1346,9 @@ int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* 
     c->wide.ok = c->rewind_budget == INT64_MAX;
     for (const LayerW& L : c->layers)
         if (L.n_experts) {  // routed layers: the attention projections as below, the experts in any format, fp16 activations
-            if (c->moe_fp4_terms || L.v_only.tiles || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt)) c->wide.ok = false;
-        } else if (L.v_only.tiles || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) ||
-            !wide_fmt(L.gate_up.fmt) || !wide_fmt(L.down.fmt))
+            if (c->moe_fp4_terms || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) || (L.v_only.tiles && !wide_fmt(L.v_only.fmt))) c->wide.ok = false;
+        } else if (!wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) || (L.v_only.tiles && !wide_fmt(L.v_only.fmt)) ||
+                   !wide_fmt(L.gate_up.fmt) || !wide_fmt(L.down.fmt))
             c->wide.ok = false;
     if (const char* e = getenv("TSV_WIDE_PREFILL")) c->wide.ok = c->wide.ok && e[0] != '0';
     if (share) c->wide.ok = false;  // the head's rows come sixteen at a time

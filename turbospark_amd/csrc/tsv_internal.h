@@ -177,7 +177,7 @@ int launch_repack(hipStream_t s, int fmt, const uint8_t* raw, int n_rows, int k,
 int launch_gemm(hipStream_t s, const TiledW& w, const uint4* xfrag, void* out, const VerifyParams* vp,
                 int m, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
 int gemm_default_splits(const TiledW& w, int m);
-// rows of a prompt-block pass, and the matmul over them in blocks of sixteen (Q4_K weights only)
+// rows of a prompt-block pass, and the matmul over them in blocks of sixteen (Q4_K, Q5_K, Q6_K, Q8_0 or bf16 weights)
 int gemm_wide_rows();
 int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t x_stride, void* out, size_t out_stride,
                      const VerifyParams* vp, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope = nullptr);
