@@ -134,6 +134,38 @@ def test_routed_layers_in_passes_of_64_rows(name, n_prompt, seed):
     assert err_w <= 1e-2 and err_wn <= 2e-3
 
 
+@pytest.mark.parametrize("name", ["small_q4_k", "xcd_q4_k", "tiny_q8_0"])
+def test_the_rotating_epilogue_in_64_row_passes(name, monkeypatch):
+    """TSV_WIDE_ROPE_FUSED=1 keeps the projection that rotates and stores its own rows (one workgroup per tile) in the
+    64-row passes as well; by default they split the projection along K and leave the rotation to its kernel."""
+    from turbospark_amd import synth
+    from oracle import binding as ob
+    cfg = dict(synth.CONFIGS[name], max_context=200)
+    w = synth.make_weights(cfg, seed=17)
+    monkeypatch.setenv("TSV_WIDE_ROPE_FUSED", "1")
+    fused = _engine(cfg, w, True)
+    monkeypatch.delenv("TSV_WIDE_ROPE_FUSED")
+    split = _engine(cfg, w, True)
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, cfg["vocab"], 150).astype(np.int32)
+    feed = rng.integers(0, cfg["vocab"], 5).astype(np.int32)
+    fused.prefill(prompt, 0, want_logits=False)
+    split.prefill(prompt, 0, want_logits=False)
+    for i in range(0, 150, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    for layer in range(cfg["n_layers"]):
+        (kf, vf), (ks, vs), (kc, vc) = fused.read_kv(layer, 0, 150), split.read_kv(layer, 0, 150), cpu.kv(layer)
+        for got, other, want in ((kf, ks, kc), (vf, vs, vc)):
+            got, other, want = got.astype(np.float32), other.astype(np.float32), want[:150]
+            scale = np.abs(want).max()
+            assert np.abs(got - want).max() <= 2e-2 * scale and np.abs(got - other).max() <= 4e-3 * scale
+    want = cpu.verify(feed, 150)
+    a, b = fused.verify(feed, 150), split.verify(feed, 150)
+    print(f"{name}: epilogue {gc.logit_error(a, want):.2e}, split {gc.logit_error(b, want):.2e}, between {gc.logit_error(a, b):.2e}")
+    assert gc.logit_error(a, want) <= gc.TOL.get(cfg["dtype"], 1e-2) and gc.logit_error(a, b) <= 2e-3
+
+
 def test_logits_of_the_last_prompt_token_after_wide_passes():
     """tsv_prefill hands out the last row's logits: the rows before it go in blocks of 64, the tail in
     16-row passes whose last one carries the output head."""

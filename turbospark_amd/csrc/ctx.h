@@ -77,6 +77,7 @@ struct tsv_ctx {
     // q rows, parameters and rotation table, block after block; allocated at the first such pass
     struct Wide {
         bool ok = false, ready = false;
+        bool keep_epilogue = false;  // TSV_WIDE_ROPE_FUSED=1: the 64-row q/k/v launch rotates its own rows (one workgroup per tile)
         float* x = nullptr;
         uint8_t *xf_a = nullptr, *xf_b = nullptr, *xf_c = nullptr;
         size_t xfb = 0;

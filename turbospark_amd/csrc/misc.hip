@@ -385,6 +385,11 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
     const int h = kind == 0 ? head : kind == 1 ? head - a.nq : head - a.nq - a.nkv;
     const int col = head * hd;  // q heads, then k heads, then v heads: the fused projection's row order
     float x0 = 0.f, x1 = 0.f;
+    // where dims i and i + half sit among the head's columns: side by side in the natural order, or -- q and k rows
+    // tiled for the rotating epilogue (128-wide heads) -- dims 32 t .. 32 t + 31 in the low half of 64-row tile t and
+    // their partners in its high half
+    const bool paired = a.paired && kind != 2;
+    const int c0 = paired ? (i >> 5) * 64 + (i & 31) : i, c1 = paired ? c0 + 32 : i + half;
     if (i < half) {
         // compile-time split count (a uniform branch picks the variant): every partial is in flight
         // before the first add
@@ -394,8 +399,8 @@ __global__ __launch_bounds__(64) void k_rope_kv(RopeKvArgs a) {
 #pragma unroll
             for (int s = 0; s < NS; s++) {
                 const float* p = a.qkv + ((long)s * 16 + m) * a.ldq + col;
-                p0[s] = p[i];
-                p1[s] = p[i + half];
+                p0[s] = p[c0];
+                p1[s] = p[c1];
             }
 #pragma unroll
             for (int s = 0; s < NS; s++) {

@@ -671,7 +671,10 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         re.nkv = c->nkv;
         re.hd = c->hd;
         re.max_ctx = L.kv_slots;
-        if (L.rope_fused) {
+        // The rotating epilogue needs whole sums, so its launch has one workgroup per tile (96 at the 8B shape, for 256
+        // compute units: 29.7 us); split along K it fills the chip and the rotation kernel finishes all four blocks in
+        // one launch.  TSV_WIDE_ROPE_FUSED=1 keeps the epilogue.
+        if (L.rope_fused && w.keep_epilogue) {
             if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
         } else {
             // the projection's partial sums, then the 16-row pass's own norm / rotation / cache stores over the four blocks
@@ -693,6 +696,7 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
                 ra.qkv = w.partial;
                 ra.blocks = WIDE_B;
                 ra.qkv_block_stride = (long)c->partial_floats;
+                ra.paired = L.rope_fused && c->hd == 128;
                 ra.splits = spq;
                 ra.ldq = qkv_n;
                 ra.freqs = c->freqs;
@@ -1351,6 +1355,7 @@ int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* 
                    !wide_fmt(L.gate_up.fmt) || !wide_fmt(L.down.fmt))
             c->wide.ok = false;
     if (const char* e = getenv("TSV_WIDE_PREFILL")) c->wide.ok = c->wide.ok && e[0] != '0';
+    if (const char* e = getenv("TSV_WIDE_ROPE_FUSED")) c->wide.keep_epilogue = e[0] == '1';
     if (share) c->wide.ok = false;  // the head's rows come sixteen at a time
     *out = c;
     return TSV_OK;

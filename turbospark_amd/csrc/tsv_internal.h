@@ -349,6 +349,7 @@ struct RopeKvArgs {
     // floats further on and its sixteen q rows behind block b - 1's
     int blocks;
     long qkv_block_stride;
+    int paired;  // the q and k columns of a head come in the rotating epilogue's tile order (128-wide heads)
 };
 int launch_rope_kv(hipStream_t s, const RopeKvArgs& a, int m);
 
