@@ -107,7 +107,8 @@ int32_t tsv_attention_quantized(const uint16_t* q, const uint16_t* k, const uint
 /* The experts every row of the last pass chose in every routed layer: out is [n_layers][16][8] expert
  * ids in rank order (row r of the pass at [layer][r], the first top_k entries of a row are valid).
  * What the bench counts the expert bytes actually read from, and what the routing tests compare with
- * the oracle's ranking (real_forward_dispatch.rs:1135-1158). */
+ * the oracle's ranking (real_forward_dispatch.rs:1135-1158).  Passes of at most sixteen rows are meant: the
+ * 64-row prompt passes keep their selections in buffers of their own. */
 int32_t tsv_route_selected(tsv_ctx* ctx, int32_t* out, int32_t n_layers);
 
 /* Makes the routed layers take the experts given instead of each row's own top-k: sel is
@@ -116,7 +117,8 @@ int32_t tsv_route_selected(tsv_ctx* ctx, int32_t* out, int32_t n_layers);
  * the experts taken.  NULL restores free routing.  With the oracle's ranking forced onto the device
  * (or the device's onto the oracle, tso_model_force_route) the two sides run the same experts on any
  * input, also one whose ranking sits inside the fp16 rounding of a tie; the bench uses it to time the
- * expert matmuls under routing that is independent from row to row. */
+ * expert matmuls under routing that is independent from row to row.  While selections are held, prompts go in
+ * 16-row passes (the 64-row passes route freely). */
 int32_t tsv_force_route(tsv_ctx* ctx, const int32_t* sel, int32_t n_layers);
 
 #ifdef __cplusplus

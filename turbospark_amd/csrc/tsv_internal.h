@@ -283,7 +283,7 @@ struct MoeGemmArgs {
     void* out;             // gate/up: per-group fragments of silu(gate) * up; down: float [8 slots][16][n_out]
     size_t out_stride;
     int n_out;             // gate/up: expert FFN width; down: hidden
-    const int32_t* selected;  // [16][8] expert ids the rows chose (k_route_fused): the groups are derived from them
+    const int32_t* selected;  // [rows][8] expert ids the rows chose (k_route_rank): the groups are derived from them
     int top_k;
     // nullable per-expert biases, [n_experts][n_out]: gate/up use bias (gate) and bias2 (up), added
     // before the activation; down uses bias, added before the slot is weighted
