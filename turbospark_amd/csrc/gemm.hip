@@ -748,78 +748,6 @@ __device__ __forceinline__ void wide_compute(const WideX& x, const uint8_t* buf,
     }
 }
 
-template <int EPI, bool Q5 = false>
-__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa) {
-    constexpr int TILE = Q5 ? Q5K::TILE_BYTES : Q4K::TILE_BYTES;
-    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;  // wave = this wave's block = the row block it unpacks
-    GemmArgs a = wa.g;
-    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
-    a.xsum = (const float*)((const uint8_t*)a.xsum + (size_t)wave * wa.x_stride);
-    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
-    a.vp = a.vp + wave;
-    if (EPI == EPI_ROPE) {
-        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
-        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
-    }
-    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
-    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
-    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * TILE;
-    Consts k;
-    k.k6400 = 0x64006400u;
-    k.k5400 = 0x54005400u;
-    k.k64 = 0x64646464u;
-    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400));
-    float4v acc[4];
-#pragma unroll
-    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
-    const int M = a.vp->m;
-    // chunk c: unpack into buffer c & 1 -> ask for what comes next -> barrier -> multiply chunk c.  The
-    // barrier of chunk c also separates the reads of chunk c - 1 from the unpacking of chunk c + 1,
-    // which goes to the same buffer.  The codes are asked for two chunks ahead, the activations (which
-    // come from L2) one.  No branch surrounds a load -- a chunk index past the slice is clamped to its
-    // last chunk and that chunk is simply asked for again -- so the loop body is one block and the
-    // wait before each use is a count the compiler can know, not "everything".
-    WideW w[2];
-    WideX x[2];
-    uint8_t* const buf0 = wide_lds;
-    uint8_t* const buf1 = wide_lds + WIDE_BUF_BYTES;
-    const int last = s1 - 1;
-    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * TILE; };
-    wide_load_w<Q5>(w[0], tile_at(s0), wave, lane);
-    wide_load_x(x[0], a, s0, lane);
-    wide_load_w<Q5>(w[1], tile_at(s0 + 1), wave, lane);
-    int c = s0;
-    for (; c + 2 <= s1; c += 2) {
-        wide_unpack<Q5>(w[0], k, buf0, wave, lane);
-        wide_load_w<Q5>(w[0], tile_at(c + 2), wave, lane);
-        wide_load_x(x[1], a, min(c + 1, last), lane);
-        __syncthreads();
-        wide_compute(x[0], buf0, acc, lane);
-        wide_unpack<Q5>(w[1], k, buf1, wave, lane);
-        wide_load_w<Q5>(w[1], tile_at(c + 3), wave, lane);
-        wide_load_x(x[0], a, min(c + 2, last), lane);
-        __syncthreads();
-        wide_compute(x[1], buf1, acc, lane);
-    }
-    if (c < s1) {
-        wide_unpack<Q5>(w[0], k, buf0, wave, lane);
-        __syncthreads();
-        wide_compute(x[0], buf0, acc, lane);
-    }
-    __syncthreads();  // every wave is done with the chunk buffers before the epilogue's sums go to LDS behind them
-    float* ssum = (float*)(wide_lds + 2 * WIDE_BUF_BYTES) + wave * 32;
-#pragma unroll
-    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
-    if (EPI == EPI_SILU) {
-        __syncthreads();
-        if (lane < 16 && lane < M) {
-            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
-            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
-        }
-    }
-}
-
 // ---- the same pass over Q8_0 weights ---------------------------------------------------------
 // A chunk is 128 K = four 32-element blocks, each with its own fp16 scale per weight row, so a block is
 // one matrix instruction per row block whose result takes the block's scale in fp32 (fma4) on its way
@@ -898,71 +826,6 @@ __device__ __forceinline__ void wide80_compute(const WideX80& x, const uint8_t* 
     }
 }
 
-template <int EPI>
-__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_q80(GemmWideArgs wa) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    GemmArgs a = wa.g;
-    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
-    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
-    a.vp = a.vp + wave;
-    if (EPI == EPI_ROPE) {
-        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
-        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
-    }
-    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
-    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
-    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q80::TILE_BYTES;
-    Consts k;
-    k.k6400 = 0;
-    k.k5400 = 0;
-    k.k64 = 0x64646464u;
-    asm volatile("" : "+v"(k.k64));
-    float4v acc[4];
-#pragma unroll
-    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
-    const int M = a.vp->m;
-    // the chunk loop of k_gemm_wide: unpack c -> ask for what comes next -> barrier -> multiply c
-    WideW80 w[2];
-    WideX80 x[2];
-    uint8_t* const buf0 = wide_lds;
-    uint8_t* const buf1 = wide_lds + WIDE80_BUF_BYTES;
-    const int last = s1 - 1;
-    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * Q80::TILE_BYTES; };
-    wide80_load_w(w[0], tile_at(s0), wave, lane);
-    wide80_load_x(x[0], a, s0, lane);
-    wide80_load_w(w[1], tile_at(s0 + 1), wave, lane);
-    int c = s0;
-    for (; c + 2 <= s1; c += 2) {
-        wide80_unpack(w[0], k, buf0, wave, lane);
-        wide80_load_w(w[0], tile_at(c + 2), wave, lane);
-        wide80_load_x(x[1], a, min(c + 1, last), lane);
-        __syncthreads();
-        wide80_compute(x[0], buf0, acc, lane);
-        wide80_unpack(w[1], k, buf1, wave, lane);
-        wide80_load_w(w[1], tile_at(c + 3), wave, lane);
-        wide80_load_x(x[0], a, min(c + 2, last), lane);
-        __syncthreads();
-        wide80_compute(x[1], buf1, acc, lane);
-    }
-    if (c < s1) {
-        wide80_unpack(w[0], k, buf0, wave, lane);
-        __syncthreads();
-        wide80_compute(x[0], buf0, acc, lane);
-    }
-    __syncthreads();
-    float* ssum = (float*)(wide_lds + 2 * WIDE80_BUF_BYTES) + wave * 32;
-#pragma unroll
-    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
-    if (EPI == EPI_SILU) {
-        __syncthreads();
-        if (lane < 16 && lane < M) {
-            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
-            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
-        }
-    }
-}
-
 // ---- the same pass over bf16 weights ---------------------------------------------------------
 // A chunk is 64 K, and a tile's unit 4 s + kg already is what lane (r, kg) of v_mfma_f32_16x16x32_bf16
 // holds of weight row r in K step s, so "unpacking" is a copy into LDS.  The fp16 activations go in as
@@ -1025,65 +888,6 @@ __device__ __forceinline__ void widebf_compute(const WideXBf& x, const uint8_t* 
         for (int rb = 0; rb < 4; rb++)
             acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, lo), __builtin_bit_cast(bf16x8, b[st][rb]),
                                                               acc[rb], 0, 0, 0);
-    }
-}
-
-template <int EPI>
-__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_bf16(GemmWideArgs wa) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two chunk buffers, then the blocks' sub-block sums
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    GemmArgs a = wa.g;
-    a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
-    a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
-    a.vp = a.vp + wave;
-    if (EPI == EPI_ROPE) {
-        a.rope.cs += (size_t)wave * 16 * (a.rope.hd >> 1);
-        a.rope.q16 += (size_t)wave * 16 * a.rope.nq * a.rope.hd;
-    }
-    const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
-    const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
-    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * BF16W::TILE_BYTES;
-    float4v acc[4];
-#pragma unroll
-    for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
-    const int M = a.vp->m;
-    WideWBf w[2];
-    WideXBf x[2];
-    uint8_t* const buf0 = wide_lds;
-    uint8_t* const buf1 = wide_lds + WIDEBF_BUF_BYTES;
-    const int last = s1 - 1;
-    auto tile_at = [&](int c) { return wt + (size_t)min(c, last) * BF16W::TILE_BYTES; };
-    widebf_load_w(w[0], tile_at(s0), wave, lane);
-    widebf_load_x(x[0], a, s0, lane);
-    widebf_load_w(w[1], tile_at(s0 + 1), wave, lane);
-    int c = s0;
-    for (; c + 2 <= s1; c += 2) {
-        widebf_store(w[0], buf0, wave, lane);
-        widebf_load_w(w[0], tile_at(c + 2), wave, lane);
-        widebf_load_x(x[1], a, min(c + 1, last), lane);
-        __syncthreads();
-        widebf_compute(x[0], buf0, acc, lane);
-        widebf_store(w[1], buf1, wave, lane);
-        widebf_load_w(w[1], tile_at(c + 3), wave, lane);
-        widebf_load_x(x[0], a, min(c + 2, last), lane);
-        __syncthreads();
-        widebf_compute(x[1], buf1, acc, lane);
-    }
-    if (c < s1) {
-        widebf_store(w[0], buf0, wave, lane);
-        __syncthreads();
-        widebf_compute(x[0], buf0, acc, lane);
-    }
-    __syncthreads();
-    float* ssum = (float*)(wide_lds + 2 * WIDEBF_BUF_BYTES) + wave * 32;
-#pragma unroll
-    for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
-    if (EPI == EPI_SILU) {
-        __syncthreads();
-        if (lane < 16 && lane < M) {
-            float* sums = (float*)((char*)a.out + xfrag_sum_offset(a.n_valid));
-            sums[xsum_index(tile, lane)] = ssum[lane] + ssum[16 + lane];
-        }
     }
 }
 
@@ -1205,12 +1009,59 @@ __device__ __forceinline__ void wide6_compute(const WideX6& x, const uint8_t* bu
     }
 }
 
-template <int EPI>
-__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_q6k(GemmWideArgs wa) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two half-chunk buffers, then the blocks' sub-block sums
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// ---- the pass itself, whatever the storage type ------------------------------------------------
+// What a storage type brings: its tile size, the size of an LDS buffer, how many loop units a K chunk
+// makes (one; two half chunks for Q6_K), and the four steps of a unit -- load the unpacking wave's share of
+// the tile, load a block's activations, unpack into LDS, multiply from LDS.
+struct WideQ4 {
+    static constexpr int TILE_BYTES = Q4K::TILE_BYTES, BUF_BYTES = WIDE_BUF_BYTES, UNITS = 1;
+    typedef WideW W;
+    typedef WideX X;
+    static __device__ __forceinline__ void load_w(W& w, const uint8_t* t, int, int rb, int lane) { wide_load_w<false>(w, t, rb, lane); }
+    static __device__ __forceinline__ void load_x(X& x, const GemmArgs& a, int u, int lane) { wide_load_x(x, a, u, lane); }
+    static __device__ __forceinline__ void unpack(const W& w, const Consts& k, uint8_t* buf, int rb, int lane) { wide_unpack<false>(w, k, buf, rb, lane); }
+    static __device__ __forceinline__ void compute(const X& x, const uint8_t* buf, float4v (&acc)[4], int lane) { wide_compute(x, buf, acc, lane); }
+};
+struct WideQ5 : WideQ4 {
+    static constexpr int TILE_BYTES = Q5K::TILE_BYTES;
+    static __device__ __forceinline__ void load_w(W& w, const uint8_t* t, int, int rb, int lane) { wide_load_w<true>(w, t, rb, lane); }
+    static __device__ __forceinline__ void unpack(const W& w, const Consts& k, uint8_t* buf, int rb, int lane) { wide_unpack<true>(w, k, buf, rb, lane); }
+};
+struct WideQ8 {
+    static constexpr int TILE_BYTES = Q80::TILE_BYTES, BUF_BYTES = WIDE80_BUF_BYTES, UNITS = 1;
+    typedef WideW80 W;
+    typedef WideX80 X;
+    static __device__ __forceinline__ void load_w(W& w, const uint8_t* t, int, int rb, int lane) { wide80_load_w(w, t, rb, lane); }
+    static __device__ __forceinline__ void load_x(X& x, const GemmArgs& a, int u, int lane) { wide80_load_x(x, a, u, lane); }
+    static __device__ __forceinline__ void unpack(const W& w, const Consts& k, uint8_t* buf, int rb, int lane) { wide80_unpack(w, k, buf, rb, lane); }
+    static __device__ __forceinline__ void compute(const X& x, const uint8_t* buf, float4v (&acc)[4], int lane) { wide80_compute(x, buf, acc, lane); }
+};
+struct WideBf {
+    static constexpr int TILE_BYTES = BF16W::TILE_BYTES, BUF_BYTES = WIDEBF_BUF_BYTES, UNITS = 1;
+    typedef WideWBf W;
+    typedef WideXBf X;
+    static __device__ __forceinline__ void load_w(W& w, const uint8_t* t, int, int rb, int lane) { widebf_load_w(w, t, rb, lane); }
+    static __device__ __forceinline__ void load_x(X& x, const GemmArgs& a, int u, int lane) { widebf_load_x(x, a, u, lane); }
+    static __device__ __forceinline__ void unpack(const W& w, const Consts&, uint8_t* buf, int rb, int lane) { widebf_store(w, buf, rb, lane); }
+    static __device__ __forceinline__ void compute(const X& x, const uint8_t* buf, float4v (&acc)[4], int lane) { widebf_compute(x, buf, acc, lane); }
+};
+struct WideQ6 {
+    static constexpr int TILE_BYTES = Q6K::TILE_BYTES, BUF_BYTES = WIDE6_BUF_BYTES, UNITS = 2;
+    typedef WideW6 W;
+    typedef WideX6 X;
+    static __device__ __forceinline__ void load_w(W& w, const uint8_t* t, int half, int rb, int lane) { wide6_load_w(w, t, half, rb, lane); }
+    static __device__ __forceinline__ void load_x(X& x, const GemmArgs& a, int u, int lane) { wide6_load_x(x, a, u, lane); }
+    static __device__ __forceinline__ void unpack(const W& w, const Consts& k, uint8_t* buf, int rb, int lane) { wide6_unpack(w, k, buf, rb, lane); }
+    static __device__ __forceinline__ void compute(const X& x, const uint8_t* buf, float4v (&acc)[4], int lane) { wide6_compute(x, buf, acc, lane); }
+};
+
+template <class P, int EPI>
+__global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide(GemmWideArgs wa) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];  // two unit buffers, then the blocks' sub-block sums
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;  // wave = this wave's block = the row block it unpacks
     GemmArgs a = wa.g;
     a.xfrag = (const uint2*)((const uint8_t*)a.xfrag + (size_t)wave * wa.x_stride);
+    a.xsum = (const float*)((const uint8_t*)a.xsum + (size_t)wave * wa.x_stride);
     a.out = a.out ? (uint8_t*)a.out + (size_t)wave * wa.out_stride : nullptr;
     a.vp = a.vp + wave;
     if (EPI == EPI_ROPE) {
@@ -1219,44 +1070,54 @@ __global__ __launch_bounds__(64 * WIDE_BLOCKS) void k_gemm_wide_q6k(GemmWideArgs
     }
     const int split = blockIdx.x % a.splits, tile = blockIdx.x / a.splits;
     const int s0 = split * a.kslice, s1 = min(s0 + a.kslice, a.kchunks);
-    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * Q6K::TILE_BYTES;
+    const uint8_t* wt = a.w + (size_t)tile * a.kchunks * P::TILE_BYTES;
     Consts k;
     k.k6400 = 0x64006400u;
-    k.k5400 = 0;
-    k.k64 = 0;
-    asm volatile("" : "+v"(k.k6400));
+    k.k5400 = 0x54005400u;
+    k.k64 = 0x64646464u;
+    asm volatile("" : "+v"(k.k6400), "+v"(k.k5400), "+v"(k.k64));
     float4v acc[4];
 #pragma unroll
     for (int rb = 0; rb < 4; rb++) acc[rb] = float4v{0.f, 0.f, 0.f, 0.f};
     const int M = a.vp->m;
-    // the chunk loop of k_gemm_wide over half chunks h0 .. h1 - 1 (half chunk hc = chunk hc / 2, half hc % 2)
-    WideW6 w[2];
-    WideX6 x[2];
+    // unit u: unpack into buffer u & 1 -> ask for what comes next -> barrier -> multiply unit u.  The
+    // barrier of unit u also separates the reads of unit u - 1 from the unpacking of unit u + 1,
+    // which goes to the same buffer.  The codes are asked for two units ahead, the activations (which
+    // come from L2) one.  No branch surrounds a load -- a unit index past the slice is clamped to its
+    // last unit and that unit is simply asked for again -- so the loop body is one block and the
+    // wait before each use is a count the compiler can know, not "everything".
+    typename P::W w[2];
+    typename P::X x[2];
     uint8_t* const buf0 = wide_lds;
-    uint8_t* const buf1 = wide_lds + WIDE6_BUF_BYTES;
-    const int h0 = 2 * s0, h1 = 2 * s1, last = h1 - 1;
-    auto load_w = [&](WideW6& ww, int hc) {
-        const int c = min(hc, last);
-        wide6_load_w(ww, wt + (size_t)(c >> 1) * Q6K::TILE_BYTES, c & 1, wave, lane);
+    uint8_t* const buf1 = wide_lds + P::BUF_BYTES;
+    const int u0 = P::UNITS * s0, u1 = P::UNITS * s1, last = u1 - 1;
+    auto load_w = [&](typename P::W& ww, int u) {
+        const int c = min(u, last);
+        P::load_w(ww, wt + (size_t)(c / P::UNITS) * P::TILE_BYTES, c % P::UNITS, wave, lane);
     };
-    load_w(w[0], h0);
-    wide6_load_x(x[0], a, h0, lane);
-    load_w(w[1], h0 + 1);
-    int c = h0;
-    for (; c + 2 <= h1; c += 2) {
-        wide6_unpack(w[0], k, buf0, wave, lane);
+    load_w(w[0], u0);
+    P::load_x(x[0], a, u0, lane);
+    load_w(w[1], u0 + 1);
+    int c = u0;
+    for (; c + 2 <= u1; c += 2) {
+        P::unpack(w[0], k, buf0, wave, lane);
         load_w(w[0], c + 2);
-        wide6_load_x(x[1], a, min(c + 1, last), lane);
+        P::load_x(x[1], a, min(c + 1, last), lane);
         __syncthreads();
-        wide6_compute(x[0], buf0, acc, lane);
-        wide6_unpack(w[1], k, buf1, wave, lane);
+        P::compute(x[0], buf0, acc, lane);
+        P::unpack(w[1], k, buf1, wave, lane);
         load_w(w[1], c + 3);
-        wide6_load_x(x[0], a, min(c + 2, last), lane);
+        P::load_x(x[0], a, min(c + 2, last), lane);
         __syncthreads();
-        wide6_compute(x[1], buf1, acc, lane);
+        P::compute(x[1], buf1, acc, lane);
     }
-    __syncthreads();  // (the half chunks of a slice come in pairs: nothing is left over)
-    float* ssum = (float*)(wide_lds + 2 * WIDE6_BUF_BYTES) + wave * 32;
+    if (c < u1) {
+        P::unpack(w[0], k, buf0, wave, lane);
+        __syncthreads();
+        P::compute(x[0], buf0, acc, lane);
+    }
+    __syncthreads();  // every wave is done with the unit buffers before the epilogue's sums go to LDS behind them
+    float* ssum = (float*)(wide_lds + 2 * P::BUF_BYTES) + wave * 32;
 #pragma unroll
     for (int pr = 0; pr < 2; pr++) epilogue16<EPI>(a, tile, split, pr, acc[pr], acc[pr + 2], lane, M, ssum);
     if (EPI == EPI_SILU) {
@@ -1396,6 +1257,29 @@ int gemm_wide_rows() { return 16 * WIDE_BLOCKS; }
 // The same matmul over gemm_wide_rows() rows in blocks of sixteen: block b reads its fragments at
 // xfrag + b * x_stride bytes, its parameters at vp + b, and writes at out + b * out_stride bytes
 // (EPI_ROPE: rope->cs and rope->q16 hold all blocks' rows one after the other).  Q4_K, Q5_K, Q6_K, Q8_0 or bf16 weights.
+template <class P, int EPI>
+static int launch_wide_pe(hipStream_t s, const GemmWideArgs& wa) {
+    const size_t lds = 2 * (size_t)P::BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
+    static bool attr_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+    if (!attr_set && lds > 65536) {
+        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<P, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((k_gemm_wide<P, EPI>), dim3(wa.g.n_tiles * wa.g.splits), dim3(64 * WIDE_BLOCKS), lds, s, wa);
+    TSV_HIP(hipGetLastError());
+    return TSV_OK;
+}
+
+template <class P>
+static int launch_wide_p(hipStream_t s, const GemmWideArgs& wa, int epi) {
+    switch (epi) {
+        case EPI_PARTIAL: return launch_wide_pe<P, EPI_PARTIAL>(s, wa);
+        case EPI_ROPE: return launch_wide_pe<P, EPI_ROPE>(s, wa);
+        case EPI_SILU: return launch_wide_pe<P, EPI_SILU>(s, wa);
+        default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
+    }
+}
+
 int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t x_stride, void* out, size_t out_stride,
                      const VerifyParams* vp, int splits, int epi, int ldo, int n_valid, const RopeEpi* rope) {
     if (w.fmt != FMT_Q4K && w.fmt != FMT_Q5K && w.fmt != FMT_Q80 && w.fmt != FMT_BF16 && w.fmt != FMT_Q6K) {
@@ -1407,77 +1291,11 @@ int launch_gemm_wide(hipStream_t s, const TiledW& w, const uint4* xfrag, size_t 
     wa.x_stride = x_stride;
     wa.out_stride = out_stride;
     wa.g.out16 = 1;  // what this kernel reads is what it writes for the next one
-    if (w.fmt == FMT_Q6K) {
-        const size_t lds6 = 2 * (size_t)WIDE6_BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
-        const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
-        static bool attr6_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-        if (!attr6_set) {
-            TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide_q6k<EPI_PARTIAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds6));
-            TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide_q6k<EPI_ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds6));
-            TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide_q6k<EPI_SILU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds6));
-            attr6_set = true;
-        }
-        switch (epi) {
-            case EPI_PARTIAL: hipLaunchKernelGGL(k_gemm_wide_q6k<EPI_PARTIAL>, grid, block, lds6, s, wa); break;
-            case EPI_ROPE: hipLaunchKernelGGL(k_gemm_wide_q6k<EPI_ROPE>, grid, block, lds6, s, wa); break;
-            case EPI_SILU: hipLaunchKernelGGL(k_gemm_wide_q6k<EPI_SILU>, grid, block, lds6, s, wa); break;
-            default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
-        }
-        TSV_HIP(hipGetLastError());
-        return TSV_OK;
-    }
-    if (w.fmt == FMT_Q80 || w.fmt == FMT_BF16) {
-        const bool q80 = w.fmt == FMT_Q80;
-        const size_t lds2 = 2 * (size_t)(q80 ? WIDE80_BUF_BYTES : WIDEBF_BUF_BYTES) + WIDE_BLOCKS * 32 * sizeof(float);
-        const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
-        switch (epi) {
-            case EPI_PARTIAL:
-                if (q80) hipLaunchKernelGGL(k_gemm_wide_q80<EPI_PARTIAL>, grid, block, lds2, s, wa);
-                else hipLaunchKernelGGL(k_gemm_wide_bf16<EPI_PARTIAL>, grid, block, lds2, s, wa);
-                break;
-            case EPI_ROPE:
-                if (q80) hipLaunchKernelGGL(k_gemm_wide_q80<EPI_ROPE>, grid, block, lds2, s, wa);
-                else hipLaunchKernelGGL(k_gemm_wide_bf16<EPI_ROPE>, grid, block, lds2, s, wa);
-                break;
-            case EPI_SILU:
-                if (q80) hipLaunchKernelGGL(k_gemm_wide_q80<EPI_SILU>, grid, block, lds2, s, wa);
-                else hipLaunchKernelGGL(k_gemm_wide_bf16<EPI_SILU>, grid, block, lds2, s, wa);
-                break;
-            default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
-        }
-        TSV_HIP(hipGetLastError());
-        return TSV_OK;
-    }
-    const size_t lds = 2 * (size_t)WIDE_BUF_BYTES + WIDE_BLOCKS * 32 * sizeof(float);
-    const dim3 grid(wa.g.n_tiles * wa.g.splits), block(64 * WIDE_BLOCKS);
-    static bool attr_set = false;  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    if (!attr_set) {
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_PARTIAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_SILU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_PARTIAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_ROPE, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        TSV_HIP(hipFuncSetAttribute((const void*)k_gemm_wide<EPI_SILU, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
-    }
-    const bool q5 = w.fmt == FMT_Q5K;
-    switch (epi) {
-        case EPI_PARTIAL:
-            if (q5) hipLaunchKernelGGL((k_gemm_wide<EPI_PARTIAL, true>), grid, block, lds, s, wa);
-            else hipLaunchKernelGGL(k_gemm_wide<EPI_PARTIAL>, grid, block, lds, s, wa);
-            break;
-        case EPI_ROPE:
-            if (q5) hipLaunchKernelGGL((k_gemm_wide<EPI_ROPE, true>), grid, block, lds, s, wa);
-            else hipLaunchKernelGGL(k_gemm_wide<EPI_ROPE>, grid, block, lds, s, wa);
-            break;
-        case EPI_SILU:
-            if (q5) hipLaunchKernelGGL((k_gemm_wide<EPI_SILU, true>), grid, block, lds, s, wa);
-            else hipLaunchKernelGGL(k_gemm_wide<EPI_SILU>, grid, block, lds, s, wa);
-            break;
-        default: set_error("matmul: prompt blocks have no logits epilogue"); return TSV_ERR_UNSUPPORTED;
-    }
-    TSV_HIP(hipGetLastError());
-    return TSV_OK;
+    return w.fmt == FMT_Q4K    ? launch_wide_p<WideQ4>(s, wa, epi)
+           : w.fmt == FMT_Q5K  ? launch_wide_p<WideQ5>(s, wa, epi)
+           : w.fmt == FMT_Q80  ? launch_wide_p<WideQ8>(s, wa, epi)
+           : w.fmt == FMT_BF16 ? launch_wide_p<WideBf>(s, wa, epi)
+                               : launch_wide_p<WideQ6>(s, wa, epi);
 }
 
 }  // namespace tsv
