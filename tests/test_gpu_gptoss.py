@@ -121,16 +121,16 @@ def _ring_pair(name, max_context, n_layers=None, seed=1234, **over):
     if n_layers:
         cfg["n_layers"] = n_layers
     w = synth.make_weights(cfg, seed=seed, n_layers=n_layers)
-    # (ring layers take their prompts in 16-row passes; the linear handle is held to them too, so that "equal by
-    #  bits" compares the two layouts and not the summation orders of 64-row and 16-row passes)
+    # (both handles are held to 16-row prompt passes, so that "equal by bits" compares the two layouts: inside a
+    #  64-row pass a ring layer attends block by block while a linear one attends the four blocks at once, and a
+    #  64-row matmul sums in another order than a 16-row one)
     import os
+    ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
     os.environ["TSV_WIDE_PREFILL"] = "0"
     try:
-        linear = ts.HipVerifier(cfg, w)
+        return cfg, ts.HipVerifier(cfg, w), ts.HipVerifier(cfg, ringed)
     finally:
         del os.environ["TSV_WIDE_PREFILL"]
-    ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
-    return cfg, linear, ts.HipVerifier(cfg, ringed)
 
 
 def test_windowed_layers_as_rings_equal_the_linear_layout_by_bits():

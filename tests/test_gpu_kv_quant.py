@@ -247,7 +247,7 @@ def test_rings_on_a_quantized_handle_equal_the_linear_layout_by_bits():
     cfg = dict(synth.CONFIGS["gptoss_small"], max_context=400, n_layers=4)
     w = synth.make_weights(cfg, seed=21)
     ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
-    # (both handles in 16-row prompt passes, the only kind a ring layer takes: the comparison is of the layouts)
+    # (both handles in 16-row prompt passes: the comparison is of the layouts, not of the passes' summation orders)
     import os
     os.environ["TSV_WIDE_PREFILL"] = "0"
     try:

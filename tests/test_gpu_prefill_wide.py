@@ -166,6 +166,55 @@ def test_the_rotating_epilogue_in_64_row_passes(name, monkeypatch):
     assert gc.logit_error(a, want) <= gc.TOL.get(cfg["dtype"], 1e-2) and gc.logit_error(a, b) <= 2e-3
 
 
+@pytest.mark.parametrize("kv_bits", [None, (4, 4)])
+def test_ring_layers_take_the_blocks_of_a_64_row_pass_one_after_the_other(kv_bits):
+    """Windowed layers as rings (kv_cache.rs:122-131: window 24 -> a ring of 64 slots, fewer than a 64-row pass would
+    write ahead of its first block's window): inside a 64-row pass such a layer stores and attends block by block, the
+    cache states of four 16-row passes.  A 300-token prompt wraps the ring several times; then verify passes and
+    rollbacks inside the budget, against the oracle and against the 16-row passes of the same library."""
+    import turbospark_amd as ts
+    from turbospark_amd import synth
+    from oracle import binding as ob
+    cfg = dict(synth.CONFIGS["gptoss_small"], max_context=400)
+    w = synth.make_weights(cfg, seed=41)
+    ringed = dict(w, layers=[dict(lw, ring=1 if lw.get("window") else 0) for lw in w["layers"]])
+    kw = dict(kv_bits=kv_bits) if kv_bits else {}
+
+    def engine(wide):
+        os.environ["TSV_WIDE_PREFILL"] = "1" if wide else "0"
+        try:
+            return ts.HipVerifier(cfg, ringed, **kw)
+        finally:
+            del os.environ["TSV_WIDE_PREFILL"]
+
+    wide, narrow = engine(True), engine(False)
+    assert wide.max_safe_rewind() == narrow.max_safe_rewind() == 64 - 24
+    cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16, **kw)
+    rng = np.random.default_rng(41)
+    n = 300
+    prompt = rng.integers(0, cfg["vocab"], n).astype(np.int32)
+    wide.prefill(prompt, 0, want_logits=False)
+    narrow.prefill(prompt, 0, want_logits=False)
+    for i in range(0, n, 16):
+        cpu.verify(prompt[i:i + 16], i)
+    base = n
+    bound = 5e-2 if kv_bits else 1e-2
+    errs = []
+    for rnd in range(6):
+        m = int(rng.integers(3, 17))
+        feed = rng.integers(0, cfg["vocab"], m).astype(np.int32)
+        pw, pn = wide.checkpoint(), narrow.checkpoint()
+        got_w, got_n, want = wide.verify(feed, base), narrow.verify(feed, base), cpu.verify(feed, base)
+        errs.append((gc.logit_error(got_w, want), gc.logit_error(got_w, got_n)))
+        keep = int(rng.integers(1, m + 1))
+        wide.rollback_retaining(pw, keep)
+        narrow.rollback_retaining(pn, keep)
+        cpu.rewind_to(base + keep)
+        base += keep
+    print(f"rings, kv_bits {kv_bits}: (vs oracle, vs 16-row passes) per round", [f"{a:.1e}/{b:.1e}" for a, b in errs])
+    assert max(a for a, _ in errs) <= bound and max(b for _, b in errs) <= (bound if kv_bits else 2e-3)
+
+
 def test_logits_of_the_last_prompt_token_after_wide_passes():
     """tsv_prefill hands out the last row's logits: the rows before it go in blocks of 64, the tail in
     16-row passes whose last one carries the output head."""

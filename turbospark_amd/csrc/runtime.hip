@@ -598,9 +598,8 @@ int launch_pass(tsv_ctx* c, int m) {
 // q/k/v projection of the same pass has already stored for every block before any block attends.
 // Only for headless passes (no logits wanted), in any of the storage types the 64-row matmuls read
 // (wide_fmt; the q/k/v projection with the rotating epilogue, or followed by the rotation kernel over
-// the four blocks; routed layers through the experts' member lists), and only where every layer is a
-// linear cache: a ring layer's slack is 32 rows, fewer than a 64-row pass writes ahead of its first
-// block's window.
+// the four blocks; routed layers through the experts' member lists).  A ring layer stores and attends
+// the four blocks one after the other (below).
 constexpr int WIDE_B = 4;
 static bool wide_fmt(int fmt) { return fmt == FMT_Q4K || fmt == FMT_Q5K || fmt == FMT_Q6K || fmt == FMT_Q80 || fmt == FMT_BF16; }
 
@@ -671,14 +670,21 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
         re.nkv = c->nkv;
         re.hd = c->hd;
         re.max_ctx = L.kv_slots;
+        // A ring layer (kv_cache.rs:360-378) holds window + 32 positions, fewer than a 64-row pass would write ahead of
+        // its first block's window: there the rows are stored and attended one block of sixteen after the other,
+        // exactly the cache states four 16-row passes go through; everywhere else all 64 rows are stored (and, where
+        // the layer keeps quantized rows, quantized) before any block attends, and the four blocks are one launch.
+        const bool ring = L.cap < c->ctx_alloc;
         // The rotating epilogue needs whole sums, so its launch has one workgroup per tile (96 at the 8B shape, for 256
         // compute units: 29.7 us); split along K it fills the chip and the rotation kernel finishes all four blocks in
-        // one launch.  TSV_WIDE_ROPE_FUSED=1 keeps the epilogue.
-        if (L.rope_fused && w.keep_epilogue) {
+        // one launch.  TSV_WIDE_ROPE_FUSED=1 keeps the epilogue (not on ring layers: it stores all 64 rows at once).
+        const bool epilogue = L.rope_fused && w.keep_epilogue && !ring;
+        int spq = 1;
+        if (epilogue) {
             if ((rc = launch_gemm_wide(s, L.qkv, (const uint4*)w.xf_a, w.xfb, nullptr, 0, w.vp, 1, EPI_ROPE, qkv_n, L.qkv.n_rows, &re))) return rc;
         } else {
-            // the projection's partial sums, then the 16-row pass's own norm / rotation / cache stores over the four blocks
-            int spq = splits_for(L.qkv, 16, EPI_PARTIAL);
+            // the projection's partial sums; the 16-row pass's own norm / rotation / cache stores follow
+            spq = splits_for(L.qkv, 16, EPI_PARTIAL);
             if (L.v_only.tiles) {  // (the value projection in a storage type of its own: one split count for both pieces)
                 auto fits = [](const TiledW& t, int n) {
                     const int kslice = (t.kchunks + n - 1) / n;
@@ -691,79 +697,87 @@ int launch_wide_pass(tsv_ctx* c, int64_t base) {
             if (L.v_only.tiles && (rc = launch_gemm_wide(s, L.v_only, (const uint4*)w.xf_a, w.xfb, w.partial + L.qkv.n_rows, pstride, w.vp, spq,
                                                          EPI_PARTIAL, qkv_n, L.v_only.n_rows)))
                 return rc;
-            {
-                RopeKvArgs ra{};
-                ra.qkv = w.partial;
-                ra.blocks = WIDE_B;
-                ra.qkv_block_stride = (long)c->partial_floats;
-                ra.paired = L.rope_fused && c->hd == 128;
-                ra.splits = spq;
-                ra.ldq = qkv_n;
-                ra.freqs = c->freqs;
-                ra.mscale = c->rope_mscale;
-                ra.bias = L.bqkv;
-                ra.q_norm = L.q_norm;
-                ra.k_norm = L.k_norm;
-                ra.eps = c->eps;
-                ra.q16 = w.q16;
-                ra.kc = L.kc;
-                ra.vc = L.vc;
-                ra.nq = c->nq;
-                ra.nkv = c->nkv;
-                ra.hd = c->hd;
-                ra.max_ctx = L.kv_slots;
-                ra.vp = w.vp;
-                if ((rc = launch_rope_kv(s, ra, 16))) return rc;
+        }
+        // rotation + cache stores, quantization and attention of blocks b0 .. b0 + nb - 1 (one launch each)
+        auto store_rows = [&](int b0, int nb) -> int {
+            if (epilogue) return TSV_OK;
+            RopeKvArgs ra{};
+            ra.qkv = w.partial + (size_t)b0 * c->partial_floats;
+            ra.blocks = nb;
+            ra.qkv_block_stride = (long)c->partial_floats;
+            ra.paired = L.rope_fused && c->hd == 128;
+            ra.splits = spq;
+            ra.ldq = qkv_n;
+            ra.freqs = c->freqs;
+            ra.mscale = c->rope_mscale;
+            ra.bias = L.bqkv;
+            ra.q_norm = L.q_norm;
+            ra.k_norm = L.k_norm;
+            ra.eps = c->eps;
+            ra.q16 = w.q16 + (size_t)b0 * 16 * qd;
+            ra.kc = L.kc;
+            ra.vc = L.vc;
+            ra.nq = c->nq;
+            ra.nkv = c->nkv;
+            ra.hd = c->hd;
+            ra.max_ctx = L.kv_slots;
+            ra.vp = w.vp + b0;
+            return launch_rope_kv(s, ra, 16);
+        };
+        auto attend = [&](int b0, int nb) -> int {
+            if (L.tq.k_bits) {  // the rows are quantized (and their q rows rotated) before they are attended
+                TqArgs ta{};
+                ta.q16 = w.q16 + (size_t)b0 * 16 * qd;
+                ta.kc = L.kc;
+                ta.vc = L.vc;
+                ta.stage_cap = L.kv_slots;
+                ta.store = L.tq;
+                ta.k = c->tq_k;
+                ta.v = c->tq_v;
+                ta.nq = c->nq;
+                ta.nkv = c->nkv;
+                ta.hd = c->hd;
+                ta.cap = L.cap;
+                ta.vp = w.vp + b0;
+                ta.m_hint = 16 * nb;
+                ta.base_hint = (int)base + 16 * b0;
+                if (int trc = launch_tq_prepare(s, ta)) return trc;
             }
-        }
-        if (L.tq.k_bits) {  // all 64 rows are quantized (and their q rows rotated) before any block attends
-            TqArgs ta{};
-            ta.q16 = w.q16;
-            ta.kc = L.kc;
-            ta.vc = L.vc;
-            ta.stage_cap = L.kv_slots;
-            ta.store = L.tq;
-            ta.k = c->tq_k;
-            ta.v = c->tq_v;
-            ta.nq = c->nq;
-            ta.nkv = c->nkv;
-            ta.hd = c->hd;
-            ta.cap = L.cap;
-            ta.vp = w.vp;
-            ta.m_hint = 16 * WIDE_B;
-            ta.base_hint = (int)base;
-            if ((rc = launch_tq_prepare(s, ta))) return rc;
-        }
-        {
-            // all four blocks in one launch: block b attends with its own base position base + 16 b
+            // the blocks in one launch: block b attends with its own base position base + 16 b
             AttnArgs aa{};
-            aa.q16 = w.q16;
+            aa.q16 = w.q16 + (size_t)b0 * 16 * qd;
             aa.kc = L.kc;
             aa.vc = L.vc;
             aa.unrot = L.tq.k_bits ? c->tq_v.signs : nullptr;
             aa.tq = L.tq;
-            aa.part_o = w.part_o;
-            aa.part_ml = w.part_ml;
-            aa.xfrag = (uint4*)w.xf_b;
+            aa.part_o = w.part_o + (size_t)b0 * w.part_o_stride;
+            aa.part_ml = w.part_ml + (size_t)b0 * w.part_ml_stride;
+            aa.xfrag = (uint4*)(w.xf_b + (size_t)b0 * w.xfb);
             aa.nq = c->nq;
             aa.nkv = c->nkv;
             aa.hd = c->hd;
             aa.max_ctx = L.cap;
-            aa.ring = false;
+            aa.ring = ring;
             aa.nch = c->nch;
             aa.scale = c->attn_scale;
             aa.window = L.window;
             aa.sinks = L.sinks;
-            aa.vp = w.vp;
+            aa.vp = w.vp + b0;
             aa.m_hint = 16;
-            aa.base_hint = (int)base;
+            aa.base_hint = (int)base + 16 * b0;
             aa.frag16 = 1;
-            aa.blocks = WIDE_B;
+            aa.blocks = nb;
             aa.q_stride = (size_t)16 * qd;
             aa.part_o_stride = w.part_o_stride;
             aa.part_ml_stride = w.part_ml_stride;
             aa.frag_stride = w.xfb;
-            if ((rc = launch_attention(s, aa, 16))) return rc;
+            return launch_attention(s, aa, 16);
+        };
+        if (ring) {
+            for (int b = 0; b < WIDE_B; b++)
+                if ((rc = store_rows(b, 1)) || (rc = attend(b, 1))) return rc;
+        } else if ((rc = store_rows(0, WIDE_B)) || (rc = attend(0, WIDE_B))) {
+            return rc;
         }
         int sp = splits_for(L.wo, 16, EPI_PARTIAL);
         if ((rc = launch_gemm_wide(s, L.wo, (const uint4*)w.xf_b, w.xfb, w.partial, pstride, w.vp, sp, EPI_PARTIAL, c->hidden, c->hidden)))
@@ -1347,7 +1361,7 @@ int tsv::open_impl(const tsv_model_desc* d, tsv_ctx* share, const tsv_mtp_desc* 
         return fail(TSV_ERR_DEVICE);
     }
     // 64-row prompt passes (TSV_WIDE_PREFILL=0 keeps every pass at sixteen rows)
-    c->wide.ok = c->rewind_budget == INT64_MAX;
+    c->wide.ok = true;
     for (const LayerW& L : c->layers)
         if (L.n_experts) {  // routed layers: the attention projections as below, the experts in any format, fp16 activations
             if (c->moe_fp4_terms || !wide_fmt(L.qkv.fmt) || !wide_fmt(L.wo.fmt) || (L.v_only.tiles && !wide_fmt(L.v_only.fmt))) c->wide.ok = false;
