@@ -96,9 +96,12 @@ def test_wide_passes_where_the_rotation_is_a_kernel_of_its_own(name, over, monke
     assert err_w <= gc.TOL.get(cfg["dtype"], 1e-2) and err_wn <= 2e-3
 
 
-@pytest.mark.parametrize("name,n_prompt,seed", [("moe_small", 150, 31), ("gptoss_small", 150, 31), ("moe_small", 64, 32),
-                                                ("gptoss_small", 200, 33)])
-def test_routed_layers_in_passes_of_64_rows(name, n_prompt, seed):
+@pytest.mark.parametrize("name,n_prompt,seed,over", [
+    ("moe_small", 150, 31, {}), ("gptoss_small", 150, 31, {}), ("moe_small", 64, 32, {}), ("gptoss_small", 200, 33, {}),
+    # many experts, few slots: an expert has two members on average (the four-members-at-a-time walk); the cases above
+    # give an expert sixteen or eight (the sixteen-at-a-time walk of an expert many rows chose, and the mix of both)
+    ("moe_small", 150, 35, dict(n_experts=64, top_k=2)), ("gptoss_small", 150, 36, dict(n_experts=128, top_k=4))])
+def test_routed_layers_in_passes_of_64_rows(name, n_prompt, seed, over):
     """Routed experts over the 64 rows of a prompt pass: every expert is multiplied once against all the rows of the
     pass that chose it (crates/runtime/src/families/llama/moe.rs, the grouping of moe.hip taken to 64 rows).  Held to
     the oracle and to the 16-row passes of the same library.  (The rows' inputs to the router differ by rounding
@@ -106,7 +109,7 @@ def test_routed_layers_in_passes_of_64_rows(name, n_prompt, seed):
     selections of the following verify pass are compared to say so.)"""
     from turbospark_amd import synth
     from oracle import binding as ob
-    cfg = dict(synth.CONFIGS[name], max_context=n_prompt + 48)
+    cfg = dict(synth.CONFIGS[name], max_context=n_prompt + 48, **over)
     w = synth.make_weights(cfg, seed=seed)
     wide, narrow = _engine(cfg, w, True), _engine(cfg, w, False)
     cpu = ob.Model(cfg, w, round_kv_f16=True, threads=16)

@@ -170,9 +170,10 @@ __device__ __forceinline__ float silu_moe(float x) { return x / (1.0f + __expf(-
 // WIDE: the group is an expert's members among the 64 rows of a prompt pass (MoeGroupW): rows and members are
 // addressed through their 16-row blocks, and every wave stays to the end so that the caller can go on to the
 // group's next four members.
-template <class F, int EPI, int STAGES, bool WIDE = false, class G = MoeGroup>
+// NG: row groups of four walked side by side (the 64-row passes take four where an expert has many members: the
+// tile is then unpacked once per sixteen rows instead of once per four).
+template <class F, int EPI, int STAGES, bool WIDE = false, class G = MoeGroup, int NG = 1>
 __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, int gi, int r0, float4v* red) {
-    constexpr int NG = 1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int tile = blockIdx.x, e = grp.expert, cnt = grp.cnt;
     const int per = (a.kchunks + nw - 1) / nw;
@@ -188,15 +189,20 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, 
     // the group's own buffer, whose rows are already in the group's order
     const uint8_t* xbase = (const uint8_t*)a.xfrag + (EPI == EPI_SLOT ? (size_t)gi * a.x_stride : 0);
     ActLoader<false> x(xbase, xbase + xfrag_sum_offset(a.k), lane);
-    const int mine = min(r0 + (lane & 3), cnt - 1);
-    if (WIDE) {
-        if (EPI == EPI_SILU) x.set_row_blocked(0, grp.rows[mine], a.x_block_stride);
-        else x.set_row_blocked(0, mine, a.sub_stride);
-    } else {
-        x.set_row(0, EPI == EPI_SILU ? grp.rows[mine] : mine);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int mine = min(r0 + 4 * g + (lane & 3), cnt - 1);
+        if (WIDE) {
+            if (EPI == EPI_SILU) x.set_row_blocked(g, grp.rows[mine], a.x_block_stride);
+            else x.set_row_blocked(g, mine, a.sub_stride);
+        } else {
+            x.set_row(g, EPI == EPI_SILU ? grp.rows[mine] : mine);
+        }
     }
 
-    float4v acc[NG] = {float4v{0.f, 0.f, 0.f, 0.f}};
+    float4v acc[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) acc[g] = float4v{0.f, 0.f, 0.f, 0.f};
     if (nc > 0) {
         Stage<F, NG> st[STAGES];
         const int last = c0 + nc - 1;
@@ -226,11 +232,16 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, 
 
     // fold the waves in wave order; wave 0 finishes
     __syncthreads();
-    red[wave * 64 + lane] = acc[0];
+#pragma unroll
+    for (int g = 0; g < NG; g++) red[(wave * NG + g) * 64 + lane] = acc[g];
     __syncthreads();
     if (wave != 0) return;  // (WIDE: the caller's barrier is the next thing every wave meets)
-    float4v v = red[lane];
-    for (int w = 1; w < nw; w++) v += red[w * 64 + lane];
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+    const int rg = r0 + 4 * g;
+    if (rg >= cnt) break;
+    float4v v = red[g * 64 + lane];
+    for (int w = 1; w < nw; w++) v += red[(w * NG + g) * 64 + lane];
     if (EPI == EPI_SILU) {
         // lanes 0..31: gate rows, lanes 32..63: up rows of the same 32 columns of this expert
         const int col = tile * 32 + (lane & 31);
@@ -255,7 +266,7 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, 
             float sum = (float)h;
 #pragma unroll
             for (int o = 1; o < 32; o <<= 1) sum += __shfl_xor(sum, o);
-            const int b = r0 + i;  // the group's own row order
+            const int b = rg + i;  // the group's own row order
             if (b < cnt && lane < 32) {
                 if (WIDE) {
                     _Float16* ow = (_Float16*)((uint8_t*)out + (size_t)(b >> 4) * a.sub_stride);
@@ -272,7 +283,7 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, 
         if (n < a.n_out) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int b = r0 + i;
+                const int b = rg + i;
                 if (b < cnt) {
                     const int row = grp.rows[b];
                     const size_t at = WIDE ? (size_t)(row >> 4) * a.out_block_stride + ((size_t)grp.slots[b] * 16 + (row & 15)) * a.n_out
@@ -281,6 +292,7 @@ __device__ __forceinline__ void expert_tile(const MoeGemmArgs& a, const G& grp, 
                 }
             }
         }
+    }
     }
 }
 
@@ -332,6 +344,9 @@ __global__ __launch_bounds__(1024) void k_moe_groups(const int32_t* __restrict__
 
 // grid: (tiles per expert, experts, 4).  Workgroup z takes the expert's members 4 z .. 4 z + 3, then sixteen further
 // on, and so on: an expert few rows chose costs one workgroup per tile, one that many chose is spread over four.
+// An expert with more than MOE_WIDE_HEAVY members is walked eight members at a time instead (workgroup z: members
+// 8 z .. 8 z + 7, then 32 further on), so its tiles are unpacked half as often.
+constexpr int MOE_WIDE_HEAVY = 8;
 template <class F, int EPI, int STAGES>
 __global__ __launch_bounds__(512) void k_moe_gemm_wide(MoeGemmArgs a) {
     extern __shared__ float4v red[];
@@ -349,8 +364,17 @@ __global__ __launch_bounds__(512) void k_moe_gemm_wide(MoeGemmArgs a) {
         grp.cnt = cnt;
     }
     __syncthreads();
+    if (cnt > MOE_WIDE_HEAVY) {
+        // many members: eight per walk of the tile, one stage in flight (sixteen per walk costs 209 registers where this
+        // costs 119-164, and the experts with few members, who share the kernel, lose their resident waves)
+        for (int r0 = 8 * blockIdx.z; r0 < cnt; r0 += 8 * gridDim.z) {
+            expert_tile<F, EPI, 1, true, MoeGroupW, 2>(a, grp, e, r0, red);
+            __syncthreads();
+        }
+        return;
+    }
     for (int r0 = 4 * blockIdx.z; r0 < cnt; r0 += 4 * gridDim.z) {
-        expert_tile<F, EPI, STAGES, true>(a, grp, e, r0, red);
+        expert_tile<F, EPI, STAGES, true, MoeGroupW, 1>(a, grp, e, r0, red);
         __syncthreads();
     }
 }
@@ -359,7 +383,7 @@ template <class F, int EPI>
 int launch_moe_wide_t(hipStream_t s, const MoeGemmArgs& a) {
     const int cpw = std::max(2, (a.kchunks + 3) / 4);
     const int nw = std::min(8, std::max(1, (a.kchunks + cpw - 1) / cpw));
-    const size_t lds = (size_t)nw * 1024;
+    const size_t lds = (size_t)nw * 2 * 1024;  // two row groups' sums per wave
     const dim3 grid(a.tiles_per_expert, a.n_experts, 4);
     if ((a.kchunks + nw - 1) / nw <= 2)
         hipLaunchKernelGGL((k_moe_gemm_wide<F, EPI, 2>), grid, dim3(64 * nw), lds, s, a);
